@@ -1,0 +1,203 @@
+/*
+ * ugache_hip.h — the thin C-ABI over the hand-written gfx950 kernels of the embedding-extraction path.
+ *
+ * Everything above this header (the coll_cache_lib-compatible facade, CacheContext, ExtractSession,
+ * RefreshSession, the collcache Python package) is host code that never includes a HIP header: it sees
+ * plain pointers, sizes and opaque `void*` streams/events.  Each entry point names the piece of the
+ * reference (SJTU-IPADS/ugache, paths relative to its root) whose job it takes over.
+ *
+ * Conventions
+ *   - every function returns 0 on success, non-zero on failure; ugk_last_error() then describes it
+ *     (thread-local, valid until the next failing call on the same thread);
+ *   - all launches are asynchronous on `stream` (NULL = the null stream) unless stated otherwise;
+ *   - `status` is a device word the kernels OR error bits into instead of faulting
+ *     (UGK_ST_*); the host reads it after synchronising;
+ *   - pointers named *_dev must be device-accessible (HBM, or pinned host memory from ugk_host_malloc).
+ */
+#ifndef UGACHE_HIP_H_
+#define UGACHE_HIP_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* ---- status bits written by kernels -------------------------------------------------------------- */
+#define UGK_ST_KEY_OUT_OF_RANGE 0x1u /* a key / source row index beyond the source's row count: row skipped */
+#define UGK_ST_TABLE_FULL 0x2u       /* hash insert found no free bucket */
+#define UGK_ST_DUP_KEY 0x4u          /* insert of a key that is already present (the reference asserts) */
+#define UGK_ST_EVICT_ABSENT 0x8u     /* evict of a key that is not present */
+
+/* ---- locations (cache_context.cu:2421-2422: GPUs are 0..G-1, the host is G; here G = 1) ---------- */
+#define UGK_LOC_LOCAL 0u
+#define UGK_LOC_HOST 1u
+#define UGK_EMPTY_U32 0xffffffffu /* cache_hashtable.h:17 kEmptyPos */
+
+/* One gather work item.  Takes the place of SrcKeyDstVal (cache_context.h:47-52); the location is not
+ * stored because every group holds one location only. */
+typedef struct {
+  uint32_t dst_off; /* output row */
+  uint32_t src_off; /* row inside the group's source (cache slot, or host row) */
+} ugk_idx_t;
+
+/* Bucket of the open-addressing table.  Takes the place of BucketO2N (cache_hashtable.h:44-49) with a
+ * 64-bit key and a 32-bit offset so sparse 2^40 ids and > 2^28 rows fit. */
+typedef struct {
+  uint64_t key;  /* UGK_HASH_EMPTY = never used, UGK_HASH_TOMB = evicted */
+  uint32_t off;  /* row inside the location */
+  uint32_t meta; /* bit 31 = valid, bits 0..3 = location */
+} ugk_bucket_t;
+#define UGK_HASH_EMPTY 0xffffffffffffffffull
+#define UGK_HASH_TOMB 0xfffffffffffffffeull
+#define UGK_META_VALID 0x80000000u
+
+/* Lookup table handle passed by value to kernels.
+ * kind 0: none (direct mapping, cache_context.h:309-317 IsDirectMapping)
+ * kind 1: flat  — uint32 per key of the key space, (loc << 28) + off, 0xffffffff = absent
+ *                 (DeviceFlatHashTable, cache_hashtable.cuh:224-251)
+ * kind 2: hash  — ugk_bucket_t[size], linear probing (replaces DeviceSimpleHashTable, cuh:154-222) */
+typedef struct {
+  int32_t kind;
+  int32_t reserved;
+  void *table;
+  uint64_t size; /* flat: number of keys; hash: number of buckets */
+} ugk_table_t;
+
+typedef struct {
+  char name[256];
+  char arch[64];
+  int32_t compute_units;
+  int32_t wavefront_size;
+  uint64_t total_mem;
+  uint64_t lds_per_block;
+} ugk_device_info_t;
+
+const char *ugk_last_error(void);
+/* version of this ABI; bumped on any signature change */
+int ugk_abi_version(void);
+
+/* ---- runtime plumbing: Device::{AllocDataSpace,FreeDataSpace,CopyDataFromTo,StreamSync,CreateStream}
+ *      (device.h:35-65; cuda/cuda_device.cc:36-135) ---------------------------------------------- */
+int ugk_device_count(int *count);
+int ugk_set_device(int dev);
+int ugk_get_device_info(int dev, ugk_device_info_t *info);
+int ugk_mem_info(size_t *free_bytes, size_t *total_bytes);
+int ugk_malloc(void **ptr, size_t nbytes);
+int ugk_free(void *ptr);
+/* pinned, GPU-mapped host memory (the reference page-locks the caller's table with cudaHostRegister,
+ * facade.cc:476; this platform needs the table to be allocated pinned instead) */
+int ugk_host_malloc(void **ptr, size_t nbytes);
+int ugk_host_free(void *ptr);
+/* kind: 0 = ordinary host memory (kernels cannot read it), 1 = pinned host, 2 = device */
+int ugk_pointer_kind(const void *ptr, int *kind);
+int ugk_stream_create(void **stream);
+int ugk_stream_destroy(void *stream);
+int ugk_stream_sync(void *stream);
+int ugk_device_sync(void);
+int ugk_event_create(void **event);
+int ugk_event_destroy(void *event);
+int ugk_event_record(void *event, void *stream);
+int ugk_event_sync(void *event);
+int ugk_stream_wait_event(void *stream, void *event);
+int ugk_event_elapsed_ms(void *start, void *stop, float *ms);
+/* async copy, direction inferred from the pointers */
+int ugk_memcpy_async(void *dst, const void *src, size_t nbytes, void *stream);
+/* fill kernel (not a memset node, so it is safe to capture and replay) */
+int ugk_fill_u32(uint32_t *dst_dev, uint32_t value, size_t nwords, void *stream);
+/* iota: cuda_utils.cu:29-34 arrange_array */
+int ugk_arange_u32(uint32_t *dst_dev, uint32_t start, size_t n, void *stream);
+/* streaming device copy used to calibrate counters and to measure the attainable HBM rate */
+int ugk_copy_rows(void *dst_dev, const void *src_dev, size_t nbytes, void *stream);
+
+/* ---- gather: extract_data + Combine (cache_context.cu:214-231, 1076-1100) -----------------------
+ * out[dst(i), :] = src[srcrow(i), :] for row_bytes bytes.  max_blocks = 0 lets the kernel fill the
+ * chip; a non-zero value caps the grid (the reference's limit_block / per-source SM budget). */
+/* IdxStoreDirect (cache_context.h:341-354): srcrow = keys[i], dst = i */
+int ugk_gather_direct_u32(const void *src_dev, uint64_t src_rows, const uint32_t *keys_dev, size_t n, void *out_dev,
+                          size_t row_bytes, unsigned max_blocks, uint32_t *status_dev, void *stream);
+int ugk_gather_direct_i64(const void *src_dev, uint64_t src_rows, const int64_t *keys_dev, size_t n, void *out_dev,
+                          size_t row_bytes, unsigned max_blocks, uint32_t *status_dev, void *stream);
+/* IdxStoreDst (cache_context.h:356-361): srcrow = keys[i], dst = dst_off[i] (cache fill / refresh insert) */
+int ugk_gather_scatter_u32(const void *src_dev, uint64_t src_rows, const uint32_t *keys_dev,
+                           const uint32_t *dst_off_dev, size_t n, void *out_dev, uint64_t out_rows, size_t row_bytes,
+                           unsigned max_blocks, uint32_t *status_dev, void *stream);
+int ugk_gather_scatter_i64(const void *src_dev, uint64_t src_rows, const int64_t *keys_dev,
+                           const uint32_t *dst_off_dev, size_t n, void *out_dev, uint64_t out_rows, size_t row_bytes,
+                           unsigned max_blocks, uint32_t *status_dev, void *stream);
+/* CombineOneGroup with DataIterPerLoc<IdxStoreCompact> (cache_context.cu:195-212, 855-859).
+ * The group is idx[begin, begin+count) where, with c = counts_dev (written by ugk_classify_*):
+ *   group UGK_LOC_LOCAL: begin = 0,            count = c[0]
+ *   group UGK_LOC_HOST : begin = n - c[1],     count = c[1]
+ * so no host round trip is needed between classify and gather.  n is the batch size (grid upper bound). */
+int ugk_gather_group(const void *src_dev, uint64_t src_rows, const ugk_idx_t *idx_dev, const uint32_t *counts_dev,
+                     uint32_t group, size_t n, void *out_dev, size_t row_bytes, unsigned max_blocks,
+                     uint32_t *status_dev, void *stream);
+/* same with an explicit list (count known on the host) */
+int ugk_gather_idx(const void *src_dev, uint64_t src_rows, const ugk_idx_t *idx_dev, size_t count, void *out_dev,
+                   size_t row_bytes, unsigned max_blocks, uint32_t *status_dev, void *stream);
+
+/* ---- lookup tables -------------------------------------------------------------------------------
+ * flat: FlatHashTable ctor memset 0xFF (cache_hashtable.cu:588-607) is ugk_fill_u32(table, 0xffffffff, nkeys). */
+/* number of buckets for n entries at the given load factor (replaces TableSize, cache_hashtable.cu:222-225) */
+size_t ugk_hash_buckets_for(size_t n_entries, double load_factor);
+int ugk_hash_init(ugk_bucket_t *table_dev, size_t nbuckets, void *stream);
+/* insert_hashmap_unique + InsertWithLoc / InsertSeqOffWithLoc (cache_hashtable.cu:249-268;
+ * cache_hashtable.cuh:601-608): value = (loc, offs ? offs[i] : seq_base + i).  Keys must be unique and absent. */
+int ugk_table_insert_u32(ugk_table_t t, const uint32_t *keys_dev, const uint32_t *offs_dev, uint32_t seq_base,
+                         uint32_t loc, size_t n, uint32_t *status_dev, void *stream);
+int ugk_table_insert_i64(ugk_table_t t, const int64_t *keys_dev, const uint32_t *offs_dev, uint32_t seq_base,
+                         uint32_t loc, size_t n, uint32_t *status_dev, void *stream);
+/* evict_hashmap_unique (cache_hashtable.cu:269-308) */
+int ugk_table_evict_u32(ugk_table_t t, const uint32_t *keys_dev, size_t n, uint32_t *status_dev, void *stream);
+int ugk_table_evict_i64(ugk_table_t t, const int64_t *keys_dev, size_t n, uint32_t *status_dev, void *stream);
+/* LookupValCustom with SepLocOffset (cache_hashtable.cuh:420-434): loc_out/off_out per key; a miss gives
+ * (fallback_loc, (uint32)key).  Either output may be NULL (OffsetOnly, cuh:396-407). */
+int ugk_table_lookup_u32(ugk_table_t t, const uint32_t *keys_dev, size_t n, uint32_t fallback_loc,
+                         uint32_t *loc_out_dev, uint32_t *off_out_dev, void *stream);
+int ugk_table_lookup_i64(ugk_table_t t, const int64_t *keys_dev, size_t n, uint32_t fallback_loc,
+                         uint32_t *loc_out_dev, uint32_t *off_out_dev, void *stream);
+/* CountEntries (cache_hashtable.cu:742-777): census_dev[3] = occupied, tombstoned, never used */
+int ugk_hash_census(const ugk_bucket_t *table_dev, size_t nbuckets, uint64_t *census_dev, void *stream);
+
+/* ---- classify + partition by source ---------------------------------------------------------------
+ * Replaces GetMissCacheIndex + CubSortDispatcher + SplitGroup/find_boundary
+ * (cache_context.cu:702-761, 825-847; cub_sort_wrapper.cuh:472-486) with ONE kernel:
+ * per key a table lookup (one probe per lane, wavefront-cooperative continuation on collisions), then a
+ * wavefront-ballot prefix scan and LDS-staged compaction into idx_dev[0..n):
+ *   local hits  fill idx[0, c[0])          as {dst_off = i, src_off = cache slot}
+ *   host misses fill idx[n - c[1], n)      as {dst_off = i, src_off = host row = key}
+ * counts_dev[0..1] must be zero on entry; the kernel also zeroes next_counts_dev[0..1] (may be NULL) so a
+ * caller can rotate two counter pairs and never launch a memset.  host_rows bounds the miss offsets.
+ * A key found with a location other than local/host sets UGK_ST_KEY_OUT_OF_RANGE (one GPU has two sources). */
+int ugk_classify_u32(ugk_table_t t, const uint32_t *keys_dev, size_t n, uint64_t host_rows, ugk_idx_t *idx_dev,
+                     uint32_t *counts_dev, uint32_t *next_counts_dev, uint32_t *status_dev, void *stream);
+int ugk_classify_i64(ugk_table_t t, const int64_t *keys_dev, size_t n, uint64_t host_rows, ugk_idx_t *idx_dev,
+                     uint32_t *counts_dev, uint32_t *next_counts_dev, uint32_t *status_dev, void *stream);
+
+/* ---- single-kernel mixed-source extraction: kDirectNoGroup with DataIterMixLoc
+ *      (cache_context.cu:137-159, 1295-1329): lookup and gather fused, source picked per row ---------- */
+int ugk_extract_mix_u32(ugk_table_t t, const uint32_t *keys_dev, size_t n, const void *cache_dev, uint64_t cache_rows,
+                        const void *host_dev, uint64_t host_rows, void *out_dev, size_t row_bytes,
+                        uint32_t *status_dev, void *stream);
+int ugk_extract_mix_i64(ugk_table_t t, const int64_t *keys_dev, size_t n, const void *cache_dev, uint64_t cache_rows,
+                        const void *host_dev, uint64_t host_rows, void *out_dev, size_t row_bytes,
+                        uint32_t *status_dev, void *stream);
+
+/* ---- key dedup (the caller-side array_ops.unique of
+ *      python_tf2/collcache_tf2/collcache_tf2/core/sparse_lookup_layer.py:197) ------------------------
+ * unique_out[0..*n_unique) = distinct keys (order unspecified), inverse_out[i] = position of keys[i] in it.
+ * workspace_dev: ugk_dedup_workspace_bytes(n) bytes, zero-filled once at allocation and then reused as is
+ * (slots are epoch-tagged, so no per-call clearing); epoch must be non-zero and different on every call
+ * that shares the workspace.  n_unique_dev must be zero on entry. */
+size_t ugk_dedup_workspace_bytes(size_t n);
+int ugk_dedup_u32(const uint32_t *keys_dev, size_t n, void *workspace_dev, uint32_t epoch, uint32_t *unique_out_dev,
+                  uint32_t *inverse_out_dev, uint32_t *n_unique_dev, void *stream);
+int ugk_dedup_i64(const int64_t *keys_dev, size_t n, void *workspace_dev, uint32_t epoch, int64_t *unique_out_dev,
+                  uint32_t *inverse_out_dev, uint32_t *n_unique_dev, void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* UGACHE_HIP_H_ */

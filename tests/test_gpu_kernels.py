@@ -1,0 +1,431 @@
+"""GPU parity tests of the HIP kernels, called through the C-ABI of libugache_hip.so and checked bit-for-bit
+against the CPU oracle (and against closed forms at full size)."""
+import ctypes as C
+
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+torch = pytest.importorskip("torch")
+
+from oracle_lib import IDX_DTYPE, Oracle  # noqa: E402
+from ugache_amd import hip  # noqa: E402
+
+if torch.cuda.is_available():
+    from gpu_util import (PinnedArray, dev_bytes, dev_zeros_u32, pinned_from, ptr, status_value, sync, to_dev,
+                          to_np)
+
+ORC = Oracle()
+
+
+def _rand_table(rng, rows, row_bytes):
+    return rng.integers(0, 256, size=(rows, row_bytes), dtype=np.uint8)
+
+
+def _gather_direct(table_np, keys_np, max_blocks=0):
+    rows, rb = table_np.shape
+    tbl = to_dev(table_np)
+    keys = to_dev(keys_np)
+    out = dev_bytes(len(keys_np) * rb, fill=0xEE)
+    st = dev_zeros_u32(1)
+    fn = "ugk_gather_direct_i64" if keys_np.dtype == np.int64 else "ugk_gather_direct_u32"
+    hip.call(fn, ptr(tbl), rows, ptr(keys), len(keys_np), ptr(out), rb, max_blocks, ptr(st), None)
+    return to_np(out)[: len(keys_np) * rb].reshape(len(keys_np), rb), status_value(st)
+
+
+# ------------------------------------------------------------------------------------------------------
+# direct gather (IsDirectMapping fast path)
+# ------------------------------------------------------------------------------------------------------
+@pytest.mark.parametrize("row_bytes", [512, 128, 16, 32, 400, 2048, 4096 + 16, 8, 24, 4, 12, 2, 6, 1, 3])
+@pytest.mark.parametrize("kdtype", [np.uint32, np.int64])
+def test_gather_direct_matches_oracle(row_bytes, kdtype):
+    rng = np.random.default_rng(row_bytes)
+    rows = 3001
+    table = _rand_table(rng, rows, row_bytes)
+    for n in (1, 63, 4099):
+        keys = rng.integers(0, rows, size=n).astype(kdtype)
+        got, st = _gather_direct(table, keys)
+        assert st == 0
+        assert got.tobytes() == ORC.gather(table, keys).tobytes(), (row_bytes, n)
+
+
+def test_gather_direct_empty_and_capped_grid():
+    rng = np.random.default_rng(1)
+    table = _rand_table(rng, 100, 512)
+    got, st = _gather_direct(table, np.zeros(0, np.uint32))
+    assert got.shape == (0, 512) and st == 0
+    keys = rng.integers(0, 100, size=20000).astype(np.uint32)
+    for cap in (1, 3, 16):
+        got, st = _gather_direct(table, keys, max_blocks=cap)
+        assert st == 0 and got.tobytes() == table[keys].tobytes()
+
+
+def test_gather_out_of_range_key_sets_status_and_skips_row():
+    rng = np.random.default_rng(2)
+    table = _rand_table(rng, 50, 128)
+    keys = np.array([1, 50, 2, 0xFFFFFFFF, 49], np.uint32)
+    got, st = _gather_direct(table, keys)
+    assert st & hip.ST_KEY_OUT_OF_RANGE
+    assert (got[[1, 3]] == 0xEE).all()
+    assert got[[0, 2, 4]].tobytes() == table[[1, 2, 49]].tobytes()
+    keys64 = np.array([3, -1, 1 << 40], np.int64)
+    got, st = _gather_direct(table, keys64)
+    assert st & hip.ST_KEY_OUT_OF_RANGE and got[0].tobytes() == table[3].tobytes() and (got[1:] == 0xEE).all()
+
+
+@pytest.mark.parametrize("kdtype", [np.uint32, np.int64])
+def test_gather_scatter(kdtype):
+    rng = np.random.default_rng(3)
+    table = _rand_table(rng, 500, 512)
+    n = 300
+    keys = rng.integers(0, 500, size=n).astype(kdtype)
+    dst = rng.permutation(400)[:n].astype(np.uint32)
+    out = dev_bytes(400 * 512, fill=0)
+    st = dev_zeros_u32(1)
+    fn = "ugk_gather_scatter_i64" if kdtype == np.int64 else "ugk_gather_scatter_u32"
+    d_table, d_keys, d_dst = to_dev(table), to_dev(keys), to_dev(dst)
+    hip.call(fn, ptr(d_table), 500, ptr(d_keys), ptr(d_dst), n, ptr(out), 400, 512, 0, ptr(st), None)
+    want = np.zeros((400, 512), np.uint8)
+    want[dst] = table[keys.astype(np.int64)]
+    assert status_value(st) == 0 and to_np(out).reshape(400, 512).tobytes() == want.tobytes()
+    # destination beyond the output is refused
+    bad = dst.copy()
+    bad[0] = 400
+    d_bad = to_dev(bad)
+    hip.call(fn, ptr(d_table), 500, ptr(d_keys), ptr(d_bad), n, ptr(out), 400, 512, 0, ptr(st), None)
+    assert status_value(st) & hip.ST_KEY_OUT_OF_RANGE
+
+
+def test_gather_from_pinned_host_memory():
+    rng = np.random.default_rng(4)
+    table = _rand_table(rng, 2000, 512)
+    pin = pinned_from(table)
+    try:
+        keys = rng.integers(0, 2000, size=5000).astype(np.uint32)
+        out = dev_bytes(5000 * 512)
+        st = dev_zeros_u32(1)
+        d_keys = to_dev(keys)
+        hip.call("ugk_gather_direct_u32", pin.ptr, 2000, ptr(d_keys), 5000, ptr(out), 512, 8, ptr(st), None)
+        assert status_value(st) == 0
+        assert to_np(out).reshape(5000, 512).tobytes() == table[keys].tobytes()
+        kind = C.c_int(-1)
+        hip.call("ugk_pointer_kind", pin.ptr, C.byref(kind))
+        assert kind.value == 1
+        hip.call("ugk_pointer_kind", ptr(out), C.byref(kind))
+        assert kind.value == 2
+        plain = np.zeros(64, np.uint8)
+        hip.call("ugk_pointer_kind", plain.ctypes.data, C.byref(kind))
+        assert kind.value == 0
+    finally:
+        sync()
+        pin.free()
+
+
+def test_gather_full_size_all_hit_closed_form():
+    """10M x 128 fp32 table resident in HBM, 262144 uniform uint32 keys (the all-hit configuration).
+    table[r, c] is a closed form of (r, c), so out[i, c] can be checked without a host copy of the table."""
+    rows, dim, n = 10_000_000, 128, 262_144
+    r = torch.arange(rows, device="cuda", dtype=torch.int32).unsqueeze(1)
+    c = torch.arange(dim, device="cuda", dtype=torch.int32).unsqueeze(0)
+    table = (r * 131 + c * 7919) ^ (r >> 3)  # int32 bit pattern, 4 bytes per element like fp32
+    del r
+    g = torch.Generator(device="cuda").manual_seed(4)
+    keys = torch.randint(0, rows, (n,), generator=g, device="cuda", dtype=torch.int32)
+    out = torch.empty((n, dim), dtype=torch.int32, device="cuda")
+    st = dev_zeros_u32(1)
+    hip.call("ugk_gather_direct_u32", table.data_ptr(), rows, keys.data_ptr(), n, out.data_ptr(), dim * 4, 0, ptr(st),
+             None)
+    assert status_value(st) == 0
+    k = keys.unsqueeze(1)
+    want = (k * 131 + c * 7919) ^ (k >> 3)
+    assert torch.equal(out, want)
+    # and a sample of rows against the oracle on the host
+    sample = keys[:4096].cpu().numpy().astype(np.uint32)
+    sub = table[keys[:4096].long()].cpu().numpy()
+    assert ORC.gather(sub, np.arange(4096, dtype=np.uint32)).tobytes() == out[:4096].cpu().numpy().tobytes()
+    assert sample.max() < rows
+
+
+# ------------------------------------------------------------------------------------------------------
+# lookup tables
+# ------------------------------------------------------------------------------------------------------
+def _make_flat(nkeys):
+    t = dev_zeros_u32(nkeys)
+    hip.call("ugk_fill_u32", ptr(t), hip.EMPTY_U32, nkeys, None)
+    return t, hip.table(hip.TABLE_FLAT, ptr(t), nkeys)
+
+
+def _make_hash(n_entries, load=0.7):
+    nb = hip.lib().ugk_hash_buckets_for(n_entries, load)
+    t = dev_bytes(nb * 16 + 128)
+    base = (ptr(t) + 127) // 128 * 128
+    hip.call("ugk_hash_init", base, nb, None)
+    return t, hip.table(hip.TABLE_HASH, base, nb), nb
+
+
+def _lookup(tb, keys_np, fallback=1):
+    n = len(keys_np)
+    loc = dev_zeros_u32(n)
+    off = dev_zeros_u32(n)
+    fn = "ugk_table_lookup_i64" if keys_np.dtype == np.int64 else "ugk_table_lookup_u32"
+    d_keys = to_dev(keys_np)
+    hip.call(fn, tb, ptr(d_keys), n, fallback, ptr(loc), ptr(off), None)
+    sync()
+    return to_np(loc, np.uint32)[:n], to_np(off, np.uint32)[:n]
+
+
+def _insert(tb, keys_np, offs_np=None, seq_base=0, loc=0):
+    st = dev_zeros_u32(1)
+    fn = "ugk_table_insert_i64" if keys_np.dtype == np.int64 else "ugk_table_insert_u32"
+    offs = None if offs_np is None else to_dev(offs_np)
+    d_keys = to_dev(keys_np)
+    hip.call(fn, tb, ptr(d_keys), ptr(offs), seq_base, loc, len(keys_np), ptr(st), None)
+    return status_value(st)
+
+
+def _evict(tb, keys_np):
+    st = dev_zeros_u32(1)
+    fn = "ugk_table_evict_i64" if keys_np.dtype == np.int64 else "ugk_table_evict_u32"
+    d_keys = to_dev(keys_np)
+    hip.call(fn, tb, ptr(d_keys), len(keys_np), ptr(st), None)
+    return status_value(st)
+
+
+def test_flat_table_matches_oracle_rule():
+    rng = np.random.default_rng(5)
+    nkeys = 200_000
+    cached = rng.choice(nkeys, 50_000, replace=False).astype(np.uint32)
+    mem, tb = _make_flat(nkeys)
+    assert _insert(tb, cached) == 0  # sequential slots, location 0 (InsertSeqOffWithLoc)
+    oflat = ORC.flat_table(nkeys)
+    ORC.lib.orc_flat_insert(oflat, cached, np.arange(len(cached), dtype=np.uint32), len(cached))
+    q = rng.integers(0, nkeys, size=100_003).astype(np.uint32)
+    loc, off = _lookup(tb, q)
+    want = ORC.lookup_src_dst(q, flat=oflat, fallback_loc=1)
+    assert np.array_equal(loc, want["src"] >> 28) and np.array_equal(off, want["src"] & 0x0FFFFFFF)
+    assert np.array_equal(to_np(mem, np.uint32)[:nkeys], oflat)
+    # evict
+    ev = cached[:10_000]
+    assert _evict(tb, ev) == 0
+    ORC.lib.orc_flat_evict(oflat, ev, len(ev))
+    assert np.array_equal(to_np(mem, np.uint32)[:nkeys], oflat)
+    assert _evict(tb, ev[:5]) & hip.ST_EVICT_ABSENT
+    assert _insert(tb, cached[10_000:10_001]) & hip.ST_DUP_KEY
+    assert _insert(tb, np.array([nkeys], np.uint32)) & hip.ST_KEY_OUT_OF_RANGE
+
+
+# uint32 keys stay below 2^28: the reference packs a missed key into the 28-bit offset field
+@pytest.mark.parametrize("kdtype,space", [(np.uint32, 1 << 28), (np.int64, 1 << 40)])
+@pytest.mark.parametrize("n", [10, 1000, 200_000])
+def test_hash_table_against_dict_and_oracle_table(kdtype, space, n):
+    rng = np.random.default_rng(n)
+    keys = np.unique(rng.integers(0, space, size=n * 2))[:n]
+    rng.shuffle(keys)
+    keys = keys.astype(kdtype)
+    n = len(keys)
+    offs = rng.integers(0, 1 << 28, size=n).astype(np.uint32)
+    mem, tb, nb = _make_hash(n)
+    assert _insert(tb, keys, offs, loc=0) == 0
+    absent = np.setdiff1d(rng.integers(0, space, size=n).astype(kdtype), keys)
+    q = np.concatenate([keys, absent, keys[::-1][: n // 2]])
+    loc, off = _lookup(tb, q)
+    model = dict(zip(keys.tolist(), offs.tolist()))
+    want_loc = np.array([0 if int(k) in model else 1 for k in q], np.uint32)
+    want_off = np.array([model.get(int(k), int(k) & 0xFFFFFFFF) for k in q], np.uint32)
+    assert np.array_equal(loc, want_loc) and np.array_equal(off, want_off)
+    if kdtype == np.uint32:
+        # same answers as the reference's simple table restated in the oracle
+        ot = ORC.simple_table(n)
+        ORC.simple_insert(ot, keys, offs)  # loc 0 => packed value == off
+        want = ORC.lookup_src_dst(q.astype(np.uint32), simple=ot, fallback_loc=1)
+        assert np.array_equal(loc, want["src"] >> 28) and np.array_equal(off, want["src"] & 0x0FFFFFFF)
+    # census: occupied / tombstones / never used
+    cen = torch.zeros(3, dtype=torch.int64, device="cuda")
+    hip.call("ugk_hash_census", tb.table, nb, cen.data_ptr(), None)
+    sync()
+    assert cen.cpu().tolist() == [n, 0, nb - n]
+    # evict half: they miss, the rest still hit; tombstones appear
+    ev = keys[: n // 2]
+    assert _evict(tb, ev) == 0
+    loc, off = _lookup(tb, keys)
+    assert (loc[: n // 2] == 1).all() and (loc[n // 2:] == 0).all()
+    assert np.array_equal(off[n // 2:], offs[n // 2:])
+    hip.call("ugk_hash_census", tb.table, nb, cen.data_ptr(), None)
+    sync()
+    assert cen.cpu().tolist() == [n - n // 2, n // 2, nb - n]
+    assert _evict(tb, ev[:1]) & hip.ST_EVICT_ABSENT
+    # re-insert with new offsets
+    new_offs = (offs[: n // 2] ^ 0x5555).astype(np.uint32)
+    assert _insert(tb, ev, new_offs) == 0
+    loc, off = _lookup(tb, keys)
+    assert (loc == 0).all() and np.array_equal(off[: n // 2], new_offs)
+    assert _insert(tb, keys[:1], offs[:1]) & hip.ST_DUP_KEY
+    hip.call("ugk_hash_census", tb.table, nb, cen.data_ptr(), None)
+    sync()
+    occ, tomb, empty = cen.cpu().tolist()
+    assert occ == n and occ + tomb + empty == nb
+
+
+def test_hash_table_dense_collisions_and_host_entries():
+    """Load factor 0.9 with sequential keys forces long probe runs; host-located entries carry explicit rows."""
+    n = 50_000
+    keys = (np.arange(n, dtype=np.int64) * 7 + 3)
+    mem, tb, nb = _make_hash(n, load=0.9)
+    locs_half = n // 2
+    assert _insert(tb, keys[:locs_half], seq_base=100, loc=hip.LOC_LOCAL) == 0
+    assert _insert(tb, keys[locs_half:], seq_base=0, loc=hip.LOC_HOST) == 0
+    loc, off = _lookup(tb, keys, fallback=9)
+    assert (loc[:locs_half] == 0).all() and (loc[locs_half:] == 1).all()
+    assert np.array_equal(off[:locs_half], 100 + np.arange(locs_half, dtype=np.uint32))
+    assert np.array_equal(off[locs_half:], np.arange(n - locs_half, dtype=np.uint32))
+    loc, off = _lookup(tb, keys + 1, fallback=9)
+    assert (loc == 9).all()
+    # table full
+    mem2, tb2, nb2 = _make_hash(10, load=0.9)
+    many = np.arange(nb2 + 5, dtype=np.int64)
+    assert _insert(tb2, many) & hip.ST_TABLE_FULL
+    loc, off = _lookup(tb2, np.array([10_000_000], np.int64), fallback=1)  # full lap without a free bucket ends
+    assert loc[0] == 1
+
+
+# ------------------------------------------------------------------------------------------------------
+# classify + partition + factored gather
+# ------------------------------------------------------------------------------------------------------
+def _classify(tb, keys_np, host_rows):
+    n = len(keys_np)
+    idx = dev_bytes(max(n, 1) * 8, fill=0xAB)
+    counts = dev_zeros_u32(4)
+    counts[2:] = 77  # the "next" pair must be cleared by the kernel
+    st = dev_zeros_u32(1)
+    fn = "ugk_classify_i64" if keys_np.dtype == np.int64 else "ugk_classify_u32"
+    keys = to_dev(keys_np)
+    hip.call(fn, tb, ptr(keys), n, host_rows, ptr(idx), ptr(counts), ptr(counts) + 8, ptr(st), None)
+    sync()
+    c = to_np(counts, np.uint32)
+    return idx, counts, c, status_value(st), keys
+
+
+@pytest.mark.parametrize("mode", ["flat", "hash"])
+@pytest.mark.parametrize("kdtype", [np.uint32, np.int64])
+@pytest.mark.parametrize("n", [0, 1, 1023, 1024, 1025, 70_001])
+def test_classify_partition_and_factored_gather(mode, kdtype, n):
+    rng = np.random.default_rng(n + (7 if mode == "hash" else 0))
+    nkeys, rb = 20_000, 512
+    host = _rand_table(rng, nkeys, rb)
+    cached = rng.choice(nkeys, 6_000, replace=False).astype(np.uint32)
+    cap = 6_100
+    cache = np.zeros((cap, rb), np.uint8)
+    cache[: len(cached)] = host[cached]
+    if mode == "flat":
+        mem, tb = _make_flat(nkeys)
+    else:
+        mem, tb, _ = _make_hash(len(cached))
+    assert _insert(tb, cached.astype(kdtype)) == 0
+    oflat = ORC.flat_table(nkeys)
+    ORC.lib.orc_flat_insert(oflat, cached, np.arange(len(cached), dtype=np.uint32), len(cached))
+    keys = (rng.zipf(1.1, size=n) % nkeys).astype(kdtype)
+
+    idx, counts, c, st, keys_dev = _classify(tb, keys, nkeys)
+    assert st == 0
+    assert c[2] == 0 and c[3] == 0
+    want_idx = ORC.sort_idx(ORC.lookup_src_dst(keys.astype(np.uint32), flat=oflat, fallback_loc=1))
+    g = ORC.find_boundary(want_idx, 2) if n else np.zeros(3, np.uint32)
+    assert c[0] == g[1] - g[0] and c[1] == g[2] - g[1] and c[0] + c[1] == n
+    got = to_np(idx, IDX_DTYPE)[:n] if n else np.zeros(0, IDX_DTYPE)
+    # same work items per group as the reference's sorted index, up to order inside a group
+    def canon(a):
+        return np.sort(a["dst_off"].astype(np.uint64) << 32 | a["src"].astype(np.uint64))
+    want_hits = want_idx[: g[1]].copy()
+    want_miss = want_idx[g[1]:].copy()
+    want_miss["src"] &= 0x0FFFFFFF
+    assert np.array_equal(canon(got[: c[0]]), canon(want_hits))
+    assert np.array_equal(canon(got[n - c[1]:]), canon(want_miss))
+
+    # factored extraction: host group and local group as two launches reading the device-side counts
+    pin = pinned_from(host)
+    try:
+        out = dev_bytes(n * rb, fill=0xCD)
+        st2 = dev_zeros_u32(1)
+        cache_dev = to_dev(cache)
+        hip.call("ugk_gather_group", pin.ptr, nkeys, ptr(idx), ptr(counts), hip.LOC_HOST, n, ptr(out), rb, 4, ptr(st2),
+                 None)
+        hip.call("ugk_gather_group", ptr(cache_dev), cap, ptr(idx), ptr(counts), hip.LOC_LOCAL, n, ptr(out), rb, 0,
+                 ptr(st2), None)
+        assert status_value(st2) == 0
+        want_out, _ = ORC.extract_feat(keys.astype(np.uint32), cache, host, flat=oflat)
+        assert to_np(out)[: n * rb].tobytes() == want_out.tobytes()
+        assert want_out.tobytes() == host[keys.astype(np.int64)].tobytes()
+
+        # fused single-kernel variant gives the same bytes
+        out2 = dev_bytes(n * rb, fill=0x11)
+        fn = "ugk_extract_mix_i64" if kdtype == np.int64 else "ugk_extract_mix_u32"
+        hip.call(fn, tb, ptr(keys_dev), n, ptr(cache_dev), cap, pin.ptr, nkeys, ptr(out2), rb, ptr(st2), None)
+        assert status_value(st2) == 0
+        assert to_np(out2)[: n * rb].tobytes() == want_out.tobytes()
+    finally:
+        sync()
+        pin.free()
+
+
+def test_classify_rejects_keys_beyond_the_host_table():
+    mem, tb = _make_flat(100)
+    keys = np.array([5, 100, 7, 1 << 33], np.int64)
+    idx, counts, c, st, _ = _classify(tb, keys, 100)
+    assert st & hip.ST_KEY_OUT_OF_RANGE
+    assert c[0] == 0 and c[1] == 2
+    got = to_np(idx, IDX_DTYPE)[:4]
+    assert sorted(got[2:]["dst_off"].tolist()) == [0, 2] and sorted(got[2:]["src"].tolist()) == [5, 7]
+
+
+@pytest.mark.parametrize("row_bytes", [128, 64, 1024])
+def test_extract_mix_other_row_sizes(row_bytes):
+    rng = np.random.default_rng(row_bytes)
+    nkeys = 5000
+    host = _rand_table(rng, nkeys, row_bytes)
+    cached = rng.choice(nkeys, 1500, replace=False).astype(np.uint32)
+    cache = host[cached].copy()
+    mem, tb, _ = _make_hash(len(cached))
+    assert _insert(tb, cached) == 0
+    keys = rng.integers(0, nkeys, size=10_001).astype(np.uint32)
+    pin = pinned_from(host)
+    try:
+        out = dev_bytes(len(keys) * row_bytes)
+        st = dev_zeros_u32(1)
+        d_keys, d_cache = to_dev(keys), to_dev(cache)
+        hip.call("ugk_extract_mix_u32", tb, ptr(d_keys), len(keys), ptr(d_cache), len(cached), pin.ptr,
+                 nkeys, ptr(out), row_bytes, ptr(st), None)
+        assert status_value(st) == 0
+        assert to_np(out)[: len(keys) * row_bytes].tobytes() == host[keys].tobytes()
+    finally:
+        sync()
+        pin.free()
+
+
+# ------------------------------------------------------------------------------------------------------
+# dedup
+# ------------------------------------------------------------------------------------------------------
+@pytest.mark.parametrize("kdtype", [np.uint32, np.int64])
+@pytest.mark.parametrize("n", [1, 255, 256, 257, 100_000])
+def test_dedup_matches_numpy_unique(kdtype, n):
+    rng = np.random.default_rng(n)
+    space = (1 << 31) if kdtype == np.uint32 else (1 << 40)
+    pool = rng.integers(0, space, size=max(n // 3, 1))
+    ws_bytes = hip.lib().ugk_dedup_workspace_bytes(n)
+    ws = dev_bytes(ws_bytes, fill=0)
+    for epoch in (1, 2, 3):  # the workspace is reused without clearing
+        keys = pool[rng.integers(0, len(pool), size=n)].astype(kdtype)
+        uniq = dev_bytes(n * np.dtype(kdtype).itemsize)
+        inv = dev_zeros_u32(n)
+        nu = dev_zeros_u32(1)
+        fn = "ugk_dedup_i64" if kdtype == np.int64 else "ugk_dedup_u32"
+        d_keys = to_dev(keys)
+        hip.call(fn, ptr(d_keys), n, ptr(ws), epoch, ptr(uniq), ptr(inv), ptr(nu), None)
+        sync()
+        k = int(to_np(nu, np.uint32)[0])
+        u = to_np(uniq, kdtype)[:k]
+        i = to_np(inv, np.uint32)[:n]
+        want_u, _ = ORC.dedup(keys.astype(np.int64))
+        assert k == len(want_u) == len(np.unique(keys))
+        assert np.array_equal(np.sort(u.astype(np.int64)), np.sort(want_u))
+        assert i.max() < k and np.array_equal(u[i], keys)

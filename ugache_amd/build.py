@@ -1,0 +1,90 @@
+"""Build recipe for the native libraries of this package (gfx950 only).
+
+  libugache_hip.so  — hand-written HIP kernels behind the C-ABI of include/ugache_hip.h   (hipcc)
+  libcoll_cache.so  — host C++ mirror of the reference's coll_cache_lib facade + extern "C" shim (g++),
+                      linked against libugache_hip.so; it never includes a HIP header.
+
+Both are built in-tree next to this file.  `python -m ugache_amd.build` rebuilds everything.
+"""
+import os
+import shutil
+import subprocess
+import sys
+
+PKG = os.path.dirname(os.path.abspath(__file__))
+ROOT = os.path.dirname(PKG)
+CSRC = os.path.join(PKG, "csrc")
+HOST = os.path.join(PKG, "coll_cache_lib")
+INCLUDE = os.path.join(ROOT, "include")
+
+HIP_LIB = os.path.join(PKG, "libugache_hip.so")
+HOST_LIB = os.path.join(PKG, "libcoll_cache.so")
+
+HIP_SOURCES = ["ugk_runtime.hip", "ugk_gather.hip", "ugk_table.hip", "ugk_partition.hip"]
+
+HIPCC_FLAGS = [
+    "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-shared",
+    # packed FP32 instructions are kept out of every code object of this library
+    "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    "-Wall", "-Wno-unused-function",
+]
+
+
+def _run(cmd, cwd=None):
+    proc = subprocess.run(cmd, cwd=cwd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    out = "\n".join(l for l in proc.stdout.splitlines() if "packed-fp32-ops' is not a recognized feature" not in l)
+    if proc.returncode != 0:
+        raise RuntimeError("command failed: %s\n%s" % (" ".join(cmd), out))
+    return out
+
+
+def hipcc_path():
+    for cand in (shutil.which("hipcc"), "/opt/rocm/bin/hipcc"):
+        if cand and os.path.exists(cand):
+            return cand
+    raise RuntimeError("hipcc not found")
+
+
+def build_hip(verbose=False):
+    cmd = [hipcc_path()] + HIPCC_FLAGS + ["-I", INCLUDE, "-I", CSRC]
+    cmd += [os.path.join(CSRC, s) for s in HIP_SOURCES]
+    cmd += ["-o", HIP_LIB]
+    out = _run(cmd)
+    if verbose and out.strip():
+        print(out)
+    return HIP_LIB
+
+
+def host_sources():
+    if not os.path.isdir(HOST):
+        return []
+    return sorted(os.path.join(HOST, f) for f in os.listdir(HOST) if f.endswith(".cc"))
+
+
+def build_host(verbose=False):
+    srcs = host_sources()
+    if not srcs:
+        return None
+    cmd = ["g++", "-O2", "-g", "-std=c++17", "-fPIC", "-shared", "-fopenmp", "-pthread", "-Wall", "-Wextra",
+           "-Wno-unused-parameter", "-I", INCLUDE, "-I", PKG]
+    cmd += srcs
+    cmd += ["-o", HOST_LIB, "-L", PKG, "-lugache_hip", "-Wl,-rpath,$ORIGIN", "-Wl,--no-undefined"]
+    out = _run(cmd)
+    if verbose and out.strip():
+        print(out)
+    return HOST_LIB
+
+
+def build_oracle():
+    _run(["make", "-B", "-C", os.path.join(ROOT, "oracle")])
+
+
+def build_all(verbose=False):
+    build_hip(verbose)
+    build_host(verbose)
+    build_oracle()
+
+
+if __name__ == "__main__":
+    build_all(verbose=True)
+    print("built:", HIP_LIB, HOST_LIB if os.path.exists(HOST_LIB) else "(no host lib yet)")

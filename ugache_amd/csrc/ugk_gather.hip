@@ -1,0 +1,234 @@
+// Row gather kernels for gfx950: out[dst(i), :] = src[srcrow(i), :].
+//
+// This is pure HBM (or host-link) traffic, so the kernel is built around 16-byte lanes and many rows in
+// flight rather than around arithmetic:
+//   * a row of V 16-byte vectors is copied by LPR = min(64, pow2ceil(V)) adjacent lanes, so one wavefront
+//     instruction moves 64/LPR whole rows as fully coalesced segments (512-B rows: 2 rows, 128-B rows: 8);
+//   * every lane keeps UNROLL independent rows in flight (all loads issued before the first store);
+//   * loads and stores carry the non-temporal hint: rows are touched once, the output is write-only;
+//   * the grid is a grid-stride launch sized from the CU count, or capped by the caller so a host-link
+//     gather occupies only a few CUs while the HBM gather runs next to it;
+//   * keys / index records are range-checked against the source's row count: a bad key sets a status bit
+//     and its row is skipped instead of faulting.
+#include "ugk_internal.h"
+
+namespace ugk {
+namespace {
+
+constexpr uint64_t kNoLimit = ~0ull;
+
+// ---- index functors (what the reference calls IdxStore*) -------------------------------------------
+struct DirectU32 {
+  const uint32_t *keys;
+  __device__ __forceinline__ void get(size_t i, uint64_t &s, uint64_t &d) const {
+    s = keys[i];
+    d = i;
+  }
+};
+struct DirectI64 {
+  const int64_t *keys;
+  __device__ __forceinline__ void get(size_t i, uint64_t &s, uint64_t &d) const {
+    s = (uint64_t)keys[i];  // negative keys become huge and fail the range check
+    d = i;
+  }
+};
+struct ScatterU32 {
+  const uint32_t *keys;
+  const uint32_t *dst;
+  __device__ __forceinline__ void get(size_t i, uint64_t &s, uint64_t &d) const {
+    s = keys[i];
+    d = dst[i];
+  }
+};
+struct ScatterI64 {
+  const int64_t *keys;
+  const uint32_t *dst;
+  __device__ __forceinline__ void get(size_t i, uint64_t &s, uint64_t &d) const {
+    s = (uint64_t)keys[i];
+    d = dst[i];
+  }
+};
+struct IdxList {
+  const ugk_idx_t *idx;
+  __device__ __forceinline__ void get(size_t i, uint64_t &s, uint64_t &d) const {
+    const uint2 e = *reinterpret_cast<const uint2 *>(idx + i);  // one 8-byte load
+    d = e.x;
+    s = e.y;
+  }
+};
+
+template <typename V>
+__device__ __forceinline__ V ld_stream(const V *p) {
+  return __builtin_nontemporal_load(p);
+}
+template <typename V>
+__device__ __forceinline__ void st_stream(V *p, V v) {
+  __builtin_nontemporal_store(v, p);
+}
+
+template <typename V, int LPR, int UNROLL, typename Idx>
+__global__ __launch_bounds__(kBlock) void gather_kernel(Idx ix, const V *__restrict__ src, uint64_t src_rows,
+                                                        V *__restrict__ out, uint64_t out_rows, uint32_t vpr,
+                                                        const uint32_t *__restrict__ counts, uint32_t group, size_t n,
+                                                        uint32_t *status) {
+  size_t begin = 0, count = n;
+  if (counts) {
+    const uint32_t c = counts[group];
+    count = c;
+    begin = (group == UGK_LOC_LOCAL) ? 0 : n - c;
+  }
+  constexpr int RPB = kBlock / LPR;  // rows copied by one block instruction
+  const uint32_t lane = threadIdx.x % LPR;
+  const uint32_t rib = threadIdx.x / LPR;
+  constexpr size_t kPerIter = (size_t)RPB * UNROLL;
+
+  for (size_t base = (size_t)blockIdx.x * kPerIter; base < count; base += (size_t)gridDim.x * kPerIter) {
+    uint64_t s[UNROLL], d[UNROLL];
+    bool ok[UNROLL];
+#pragma unroll
+    for (int u = 0; u < UNROLL; ++u) {
+      const size_t r = base + (size_t)u * RPB + rib;
+      ok[u] = r < count;
+      s[u] = 0;
+      d[u] = 0;
+      if (ok[u]) {
+        ix.get(begin + r, s[u], d[u]);
+        if (s[u] >= src_rows || d[u] >= out_rows) {
+          ok[u] = false;
+          if (lane == 0) atomicOr(status, UGK_ST_KEY_OUT_OF_RANGE);
+        }
+      }
+    }
+    for (uint32_t c0 = 0; c0 < vpr; c0 += LPR) {
+      const uint32_t col = c0 + lane;
+      if (col < vpr) {
+        V v[UNROLL];
+#pragma unroll
+        for (int u = 0; u < UNROLL; ++u)
+          if (ok[u]) v[u] = ld_stream(src + s[u] * vpr + col);
+#pragma unroll
+        for (int u = 0; u < UNROLL; ++u)
+          if (ok[u]) st_stream(out + d[u] * vpr + col, v[u]);
+      }
+    }
+  }
+}
+
+template <typename V, int LPR, typename Idx>
+int launch_one(Idx ix, const void *src, uint64_t src_rows, void *out, uint64_t out_rows, uint32_t vpr,
+               const uint32_t *counts, uint32_t group, size_t n, unsigned max_blocks, uint32_t *status,
+               hipStream_t stream) {
+  constexpr int UNROLL = 4;
+  constexpr size_t kPerIter = (size_t)(kBlock / LPR) * UNROLL;
+  const unsigned grid = clamp_grid((n + kPerIter - 1) / kPerIter, max_blocks);
+  hipLaunchKernelGGL((gather_kernel<V, LPR, UNROLL, Idx>), dim3(grid), dim3(kBlock), 0, stream, ix,
+                     reinterpret_cast<const V *>(src), src_rows, reinterpret_cast<V *>(out), out_rows, vpr, counts,
+                     group, n, status);
+  UGK_HIP(hipGetLastError());
+  return 0;
+}
+
+template <typename V, typename Idx, bool ALL_LPR>
+int launch_vec(Idx ix, const void *src, uint64_t src_rows, void *out, uint64_t out_rows, size_t row_bytes,
+               const uint32_t *counts, uint32_t group, size_t n, unsigned max_blocks, uint32_t *status,
+               hipStream_t stream) {
+  const uint32_t vpr = (uint32_t)(row_bytes / sizeof(V));
+#define UGK_GO(L) \
+  return launch_one<V, L, Idx>(ix, src, src_rows, out, out_rows, vpr, counts, group, n, max_blocks, status, stream)
+  if (ALL_LPR) {
+    if (vpr <= 1) UGK_GO(1);
+    if (vpr <= 2) UGK_GO(2);
+    if (vpr <= 4) UGK_GO(4);
+    if (vpr <= 8) UGK_GO(8);
+    if (vpr <= 16) UGK_GO(16);
+    if (vpr <= 32) UGK_GO(32);
+    UGK_GO(64);
+  } else {
+    if (vpr <= 1) UGK_GO(1);
+    if (vpr <= 16) UGK_GO(16);
+    UGK_GO(64);
+  }
+#undef UGK_GO
+}
+
+template <typename Idx>
+int launch_gather(Idx ix, const void *src, uint64_t src_rows, void *out, uint64_t out_rows, size_t row_bytes,
+                  const uint32_t *counts, uint32_t group, size_t n, unsigned max_blocks, uint32_t *status,
+                  void *stream) {
+  if (n == 0) return 0;
+  UGK_REQUIRE(src && out, "gather: null source or output");
+  UGK_REQUIRE(status, "gather: null status word");
+  UGK_REQUIRE(row_bytes > 0 && row_bytes <= (1u << 30), "gather: row_bytes %zu out of range", row_bytes);
+  UGK_REQUIRE(n <= 0xffffffffull, "gather: batch of %zu rows exceeds 2^32", n);
+  const uintptr_t align = (uintptr_t)src | (uintptr_t)out | (uintptr_t)row_bytes;
+  hipStream_t st = as_stream(stream);
+  if (align % 16 == 0)
+    return launch_vec<u32x4, Idx, true>(ix, src, src_rows, out, out_rows, row_bytes, counts, group, n, max_blocks,
+                                        status, st);
+  if (align % 8 == 0)
+    return launch_vec<unsigned long long, Idx, false>(ix, src, src_rows, out, out_rows, row_bytes, counts, group, n,
+                                                      max_blocks, status, st);
+  if (align % 4 == 0)
+    return launch_vec<uint32_t, Idx, false>(ix, src, src_rows, out, out_rows, row_bytes, counts, group, n,
+                                            max_blocks, status, st);
+  if (align % 2 == 0)
+    return launch_vec<uint16_t, Idx, false>(ix, src, src_rows, out, out_rows, row_bytes, counts, group, n,
+                                            max_blocks, status, st);
+  return launch_vec<uint8_t, Idx, false>(ix, src, src_rows, out, out_rows, row_bytes, counts, group, n, max_blocks,
+                                         status, st);
+}
+
+}  // namespace
+}  // namespace ugk
+
+using namespace ugk;
+
+extern "C" {
+
+int ugk_gather_direct_u32(const void *src_dev, uint64_t src_rows, const uint32_t *keys_dev, size_t n, void *out_dev,
+                          size_t row_bytes, unsigned max_blocks, uint32_t *status_dev, void *stream) {
+  UGK_REQUIRE(n == 0 || keys_dev, "ugk_gather_direct_u32: null keys");
+  return launch_gather(DirectU32{keys_dev}, src_dev, src_rows, out_dev, kNoLimit, row_bytes, nullptr, 0, n,
+                       max_blocks, status_dev, stream);
+}
+
+int ugk_gather_direct_i64(const void *src_dev, uint64_t src_rows, const int64_t *keys_dev, size_t n, void *out_dev,
+                          size_t row_bytes, unsigned max_blocks, uint32_t *status_dev, void *stream) {
+  UGK_REQUIRE(n == 0 || keys_dev, "ugk_gather_direct_i64: null keys");
+  return launch_gather(DirectI64{keys_dev}, src_dev, src_rows, out_dev, kNoLimit, row_bytes, nullptr, 0, n,
+                       max_blocks, status_dev, stream);
+}
+
+int ugk_gather_scatter_u32(const void *src_dev, uint64_t src_rows, const uint32_t *keys_dev,
+                           const uint32_t *dst_off_dev, size_t n, void *out_dev, uint64_t out_rows, size_t row_bytes,
+                           unsigned max_blocks, uint32_t *status_dev, void *stream) {
+  UGK_REQUIRE(n == 0 || (keys_dev && dst_off_dev), "ugk_gather_scatter_u32: null keys or destinations");
+  return launch_gather(ScatterU32{keys_dev, dst_off_dev}, src_dev, src_rows, out_dev, out_rows, row_bytes, nullptr, 0,
+                       n, max_blocks, status_dev, stream);
+}
+
+int ugk_gather_scatter_i64(const void *src_dev, uint64_t src_rows, const int64_t *keys_dev,
+                           const uint32_t *dst_off_dev, size_t n, void *out_dev, uint64_t out_rows, size_t row_bytes,
+                           unsigned max_blocks, uint32_t *status_dev, void *stream) {
+  UGK_REQUIRE(n == 0 || (keys_dev && dst_off_dev), "ugk_gather_scatter_i64: null keys or destinations");
+  return launch_gather(ScatterI64{keys_dev, dst_off_dev}, src_dev, src_rows, out_dev, out_rows, row_bytes, nullptr, 0,
+                       n, max_blocks, status_dev, stream);
+}
+
+int ugk_gather_group(const void *src_dev, uint64_t src_rows, const ugk_idx_t *idx_dev, const uint32_t *counts_dev,
+                     uint32_t group, size_t n, void *out_dev, size_t row_bytes, unsigned max_blocks,
+                     uint32_t *status_dev, void *stream) {
+  UGK_REQUIRE(n == 0 || (idx_dev && counts_dev), "ugk_gather_group: null index list or counts");
+  UGK_REQUIRE(group == UGK_LOC_LOCAL || group == UGK_LOC_HOST, "ugk_gather_group: group %u is not local/host", group);
+  return launch_gather(IdxList{idx_dev}, src_dev, src_rows, out_dev, n, row_bytes, counts_dev, group, n, max_blocks,
+                       status_dev, stream);
+}
+
+int ugk_gather_idx(const void *src_dev, uint64_t src_rows, const ugk_idx_t *idx_dev, size_t count, void *out_dev,
+                   size_t row_bytes, unsigned max_blocks, uint32_t *status_dev, void *stream) {
+  UGK_REQUIRE(count == 0 || idx_dev, "ugk_gather_idx: null index list");
+  return launch_gather(IdxList{idx_dev}, src_dev, src_rows, out_dev, kNoLimit, row_bytes, nullptr, 0, count,
+                       max_blocks, status_dev, stream);
+}
+
+}  // extern "C"

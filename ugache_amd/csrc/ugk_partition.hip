@@ -1,0 +1,350 @@
+// Classify + partition by source, fused mixed-source extraction, key dedup.
+//
+// classify: one kernel does what the reference spreads over a lookup kernel, a 64-bit radix sort, a
+// boundary kernel and four stream synchronisations.  A block takes a tile of 1024 keys (4 per lane, loaded
+// coalesced), looks each key up (wavefront-cooperative for the hash table), derives positions with a
+// wavefront ballot + popcount prefix and a 16-entry cross-wave table in LDS, reserves its output ranges with
+// ONE atomic per source, stages the compacted records in LDS and writes them out as contiguous, coalesced
+// runs: hits grow from the front of idx[], misses from the back, so idx[] and the two counters describe the
+// same (location-grouped) array the reference obtains by sorting.
+#include "ugk_internal.h"
+#include "ugk_table.cuh"
+
+namespace ugk {
+namespace {
+
+constexpr int kItems = 4;
+constexpr int kTile = kBlock * kItems;
+constexpr int kWavesPerBlock = kBlock / kWave;
+
+template <typename K, int KIND>
+__global__ __launch_bounds__(kBlock) void classify_kernel(ugk_table_t t, const K *__restrict__ keys, size_t n,
+                                                          uint64_t host_rows, ugk_idx_t *__restrict__ idx,
+                                                          uint32_t *counts, uint32_t *next_counts, uint32_t *status) {
+  __shared__ uint2 stage[kTile];
+  __shared__ uint32_t wave_tot[kItems][kWavesPerBlock][2];
+  __shared__ uint32_t base[2];
+  const int tid = threadIdx.x;
+  const int lane = tid & (kWave - 1), wave = tid / kWave;
+  const uint64_t lt_mask = (1ull << lane) - 1ull;
+
+  if (blockIdx.x == 0 && tid == 0 && next_counts) {
+    next_counts[0] = 0;
+    next_counts[1] = 0;
+  }
+
+  for (size_t tile0 = (size_t)blockIdx.x * kTile; tile0 < n; tile0 += (size_t)gridDim.x * kTile) {
+    uint32_t cls[kItems], off[kItems], pre[kItems];
+#pragma unroll
+    for (int j = 0; j < kItems; ++j) {
+      const size_t i = tile0 + (size_t)j * kBlock + tid;
+      const bool active = i < n;
+      const uint64_t key = active ? key_to_u64<K>(keys[i]) : 0;
+      const Found f = table_lookup<KIND>(t, key, active);
+      uint32_t c = 0, o = 0;
+      if (active) {
+        if (f.hit && f.loc == UGK_LOC_LOCAL) {
+          c = 1;
+          o = f.off;
+        } else if (f.hit && f.loc == UGK_LOC_HOST && f.off < host_rows) {
+          c = 2;
+          o = f.off;
+        } else if (!f.hit && key < host_rows && key <= 0xffffffffull) {
+          c = 2;
+          o = (uint32_t)key;
+        } else {
+          atomicOr(status, UGK_ST_KEY_OUT_OF_RANGE);
+        }
+      }
+      const uint64_t hb = __ballot(c == 1), mb = __ballot(c == 2);
+      cls[j] = c;
+      off[j] = o;
+      pre[j] = (c == 1) ? __popcll(hb & lt_mask) : __popcll(mb & lt_mask);
+      if (lane == 0) {
+        wave_tot[j][wave][0] = __popcll(hb);
+        wave_tot[j][wave][1] = __popcll(mb);
+      }
+    }
+    __syncthreads();
+    uint32_t H = 0, M = 0, hoff[kItems], moff[kItems];
+#pragma unroll
+    for (int j = 0; j < kItems; ++j) {
+#pragma unroll
+      for (int w = 0; w < kWavesPerBlock; ++w) {
+        if (w == wave) {
+          hoff[j] = H;
+          moff[j] = M;
+        }
+        H += wave_tot[j][w][0];
+        M += wave_tot[j][w][1];
+      }
+    }
+    if (tid == 0) {
+      base[0] = H ? atomicAdd(counts + 0, H) : 0u;
+      base[1] = M ? atomicAdd(counts + 1, M) : 0u;
+    }
+#pragma unroll
+    for (int j = 0; j < kItems; ++j) {
+      const uint32_t i32 = (uint32_t)(tile0 + (size_t)j * kBlock + tid);
+      if (cls[j] == 1) stage[hoff[j] + pre[j]] = make_uint2(i32, off[j]);
+      if (cls[j] == 2) stage[kTile - M + moff[j] + pre[j]] = make_uint2(i32, off[j]);
+    }
+    __syncthreads();
+    uint2 *out = reinterpret_cast<uint2 *>(idx);
+    const size_t hit0 = base[0];
+    const size_t miss0 = n - (size_t)base[1] - M;
+    for (uint32_t p = tid; p < H; p += kBlock) out[hit0 + p] = stage[p];
+    for (uint32_t q = tid; q < M; q += kBlock) out[miss0 + q] = stage[kTile - M + q];
+    __syncthreads();
+  }
+}
+
+// ---- fused lookup + gather: every wavefront resolves 64 keys, then copies their 64 rows ------------------
+template <typename K, int KIND, int LPR>
+__global__ __launch_bounds__(kBlock) void extract_mix_kernel(ugk_table_t t, const K *__restrict__ keys, size_t n,
+                                                             const u32x4 *__restrict__ cache, uint64_t cache_rows,
+                                                             const u32x4 *__restrict__ host, uint64_t host_rows,
+                                                             u32x4 *__restrict__ out, uint32_t vpr,
+                                                             uint32_t *status) {
+  constexpr int RPW = kWave / LPR;  // rows per wavefront instruction
+  constexpr int UNROLL = (RPW * 4 <= kWave) ? 4 : (kWave / RPW);
+  const int lane = (int)lane_id();
+  const int sub = lane % LPR, rg = lane / LPR;
+  const size_t wave_global = (size_t)blockIdx.x * kWavesPerBlock + threadIdx.x / kWave;
+  const size_t n_waves = (size_t)gridDim.x * kWavesPerBlock;
+  for (size_t b0 = wave_global * kWave; b0 < n; b0 += n_waves * kWave) {
+    const size_t i = b0 + lane;
+    const bool active = i < n;
+    const uint64_t key = active ? key_to_u64<K>(keys[i]) : 0;
+    const Found f = table_lookup<KIND>(t, key, active);
+    const u32x4 *rowp = nullptr;
+    if (active) {
+      if (f.hit && f.loc == UGK_LOC_LOCAL && f.off < cache_rows) rowp = cache + (uint64_t)f.off * vpr;
+      else if (f.hit && f.loc == UGK_LOC_HOST && f.off < host_rows) rowp = host + (uint64_t)f.off * vpr;
+      else if (!f.hit && key < host_rows) rowp = host + key * vpr;
+      else atomicOr(status, UGK_ST_KEY_OUT_OF_RANGE);
+    }
+    const uint64_t rowbits = reinterpret_cast<uint64_t>(rowp);
+    for (int r0 = 0; r0 < kWave; r0 += RPW * UNROLL) {
+      const u32x4 *p[UNROLL];
+#pragma unroll
+      for (int u = 0; u < UNROLL; ++u) p[u] = reinterpret_cast<const u32x4 *>(shfl64(rowbits, r0 + u * RPW + rg));
+      for (uint32_t c0 = 0; c0 < vpr; c0 += LPR) {
+        const uint32_t col = c0 + sub;
+        if (col < vpr) {
+          u32x4 v[UNROLL];
+#pragma unroll
+          for (int u = 0; u < UNROLL; ++u)
+            if (p[u]) v[u] = __builtin_nontemporal_load(p[u] + col);
+#pragma unroll
+          for (int u = 0; u < UNROLL; ++u)
+            if (p[u]) __builtin_nontemporal_store(v[u], out + (b0 + r0 + u * RPW + rg) * vpr + col);
+        }
+      }
+    }
+  }
+}
+
+// ---- dedup -----------------------------------------------------------------------------------------------
+// slot word = (epoch << 32) | index of the first occurrence that claimed the slot.  A slot whose epoch is not
+// the current one is free, so the set never needs clearing between batches.
+template <typename K>
+__global__ __launch_bounds__(kBlock) void dedup_claim_kernel(const K *__restrict__ keys, size_t n,
+                                                             unsigned long long *slots, size_t cap_mask,
+                                                             uint32_t epoch, uint32_t *uid_of, K *unique_out,
+                                                             uint32_t *inverse, uint32_t *n_unique) {
+  __shared__ uint32_t wave_tot[kWavesPerBlock];
+  __shared__ uint32_t base;
+  __shared__ K stage[kBlock];
+  const int tid = threadIdx.x;
+  const int lane = tid & (kWave - 1), wave = tid / kWave;
+  const size_t n_round = (n + kBlock - 1) / kBlock * kBlock;
+  for (size_t i = (size_t)blockIdx.x * kBlock + tid; i < n_round; i += (size_t)gridDim.x * kBlock) {
+    const bool active = i < n;
+    bool winner = false;
+    K key = 0;
+    if (active) {
+      key = keys[i];
+      size_t h = fmix64(key_to_u64<K>(key)) & cap_mask;
+      uint32_t rep = (uint32_t)i;
+      for (;;) {
+        unsigned long long s = __atomic_load_n(slots + h, __ATOMIC_RELAXED);
+        bool claimed = false;
+        while ((uint32_t)(s >> 32) != epoch) {
+          const unsigned long long want = ((unsigned long long)epoch << 32) | (uint32_t)i;
+          const unsigned long long seen = atomicCAS(slots + h, s, want);
+          if (seen == s) {
+            claimed = true;
+            break;
+          }
+          s = seen;
+        }
+        if (claimed) {
+          winner = true;
+          break;
+        }
+        const uint32_t j = (uint32_t)s;
+        if (keys[j] == key) {
+          rep = j;
+          break;
+        }
+        h = (h + 1) & cap_mask;
+      }
+      inverse[i] = rep;  // index of the representative; replaced by its unique id in the second kernel
+    }
+    const uint64_t wb = __ballot(winner);
+    const uint32_t pre = __popcll(wb & ((1ull << lane) - 1ull));
+    if (lane == 0) wave_tot[wave] = __popcll(wb);
+    __syncthreads();
+    uint32_t before = 0, total = 0;
+#pragma unroll
+    for (int w = 0; w < kWavesPerBlock; ++w) {
+      if (w == wave) before = total;
+      total += wave_tot[w];
+    }
+    if (tid == 0) base = total ? atomicAdd(n_unique, total) : 0u;
+    if (winner) stage[before + pre] = key;
+    __syncthreads();
+    if (winner) uid_of[i] = base + before + pre;
+    if ((uint32_t)tid < total) unique_out[base + tid] = stage[tid];
+    __syncthreads();
+  }
+}
+
+__global__ __launch_bounds__(kBlock) void dedup_resolve_kernel(size_t n, const uint32_t *__restrict__ uid_of,
+                                                               uint32_t *inverse) {
+  for (size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x; i < n; i += (size_t)gridDim.x * kBlock)
+    inverse[i] = uid_of[inverse[i]];
+}
+
+size_t dedup_capacity(size_t n) {
+  size_t cap = 1024;
+  while (cap < 2 * n) cap <<= 1;
+  return cap;
+}
+
+template <typename K>
+int classify(ugk_table_t t, const K *keys, size_t n, uint64_t host_rows, ugk_idx_t *idx, uint32_t *counts,
+             uint32_t *next_counts, uint32_t *status, void *stream) {
+  UGK_REQUIRE(counts && status, "ugk_classify: null counters or status");
+  UGK_REQUIRE(n <= 0xffffffffull, "ugk_classify: batch of %zu keys exceeds 2^32", n);
+  UGK_REQUIRE(t.kind == 1 || t.kind == 2, "ugk_classify: table kind %d is not flat(1) or hash(2)", t.kind);
+  UGK_REQUIRE(t.table && t.size, "ugk_classify: empty table");
+  if (t.kind == 2)
+    UGK_REQUIRE(t.size % 8 == 0 && (uintptr_t)t.table % 128 == 0,
+                "ugk_classify: hash table must be 128-byte aligned with a multiple of 8 buckets");
+  UGK_REQUIRE(n == 0 || (keys && idx), "ugk_classify: null keys or index list");
+  // n == 0 still launches one block so that next_counts is cleared
+  const unsigned grid = clamp_grid((n + kTile - 1) / kTile, 0);
+  if (t.kind == 1)
+    hipLaunchKernelGGL((classify_kernel<K, 1>), dim3(grid), dim3(kBlock), 0, as_stream(stream), t, keys, n, host_rows,
+                       idx, counts, next_counts, status);
+  else
+    hipLaunchKernelGGL((classify_kernel<K, 2>), dim3(grid), dim3(kBlock), 0, as_stream(stream), t, keys, n, host_rows,
+                       idx, counts, next_counts, status);
+  UGK_HIP(hipGetLastError());
+  return 0;
+}
+
+template <typename K, int KIND>
+int extract_mix_lpr(ugk_table_t t, const K *keys, size_t n, const void *cache, uint64_t cache_rows, const void *host,
+                    uint64_t host_rows, void *out, uint32_t vpr, uint32_t *status, hipStream_t st) {
+  const unsigned grid = clamp_grid((n + kBlock - 1) / kBlock, 0);
+#define UGK_GO(L)                                                                                                 \
+  hipLaunchKernelGGL((extract_mix_kernel<K, KIND, L>), dim3(grid), dim3(kBlock), 0, st, t, keys, n,               \
+                     (const u32x4 *)cache, cache_rows, (const u32x4 *)host, host_rows, (u32x4 *)out, vpr, status)
+  if (vpr <= 1) UGK_GO(1);
+  else if (vpr <= 2) UGK_GO(2);
+  else if (vpr <= 4) UGK_GO(4);
+  else if (vpr <= 8) UGK_GO(8);
+  else if (vpr <= 16) UGK_GO(16);
+  else if (vpr <= 32) UGK_GO(32);
+  else UGK_GO(64);
+#undef UGK_GO
+  UGK_HIP(hipGetLastError());
+  return 0;
+}
+
+template <typename K>
+int extract_mix(ugk_table_t t, const K *keys, size_t n, const void *cache, uint64_t cache_rows, const void *host,
+                uint64_t host_rows, void *out, size_t row_bytes, uint32_t *status, void *stream) {
+  if (n == 0) return 0;
+  UGK_REQUIRE(keys && out && status, "ugk_extract_mix: null keys, output or status");
+  UGK_REQUIRE(t.kind == 1 || t.kind == 2, "ugk_extract_mix: table kind %d is not flat(1) or hash(2)", t.kind);
+  UGK_REQUIRE(t.table && t.size, "ugk_extract_mix: empty table");
+  if (t.kind == 2)
+    UGK_REQUIRE(t.size % 8 == 0 && (uintptr_t)t.table % 128 == 0,
+                "ugk_extract_mix: hash table must be 128-byte aligned with a multiple of 8 buckets");
+  UGK_REQUIRE(cache_rows == 0 || cache, "ugk_extract_mix: null cache with %llu rows", (unsigned long long)cache_rows);
+  UGK_REQUIRE(host_rows == 0 || host, "ugk_extract_mix: null host table with %llu rows",
+              (unsigned long long)host_rows);
+  const uintptr_t align = (uintptr_t)cache | (uintptr_t)host | (uintptr_t)out | (uintptr_t)row_bytes;
+  UGK_REQUIRE(row_bytes > 0 && align % 16 == 0,
+              "ugk_extract_mix: rows and buffers must be multiples of 16 bytes (row_bytes=%zu)", row_bytes);
+  const uint32_t vpr = (uint32_t)(row_bytes / 16);
+  if (t.kind == 1)
+    return extract_mix_lpr<K, 1>(t, keys, n, cache, cache_rows, host, host_rows, out, vpr, status, as_stream(stream));
+  return extract_mix_lpr<K, 2>(t, keys, n, cache, cache_rows, host, host_rows, out, vpr, status, as_stream(stream));
+}
+
+template <typename K>
+int dedup(const K *keys, size_t n, void *workspace, uint32_t epoch, K *unique_out, uint32_t *inverse,
+          uint32_t *n_unique, void *stream) {
+  if (n == 0) return 0;
+  UGK_REQUIRE(keys && workspace && unique_out && inverse && n_unique, "ugk_dedup: null pointer");
+  UGK_REQUIRE(epoch != 0, "ugk_dedup: epoch must be non-zero");
+  UGK_REQUIRE(n <= 0x7fffffffull, "ugk_dedup: batch of %zu keys exceeds 2^31", n);
+  UGK_REQUIRE((uintptr_t)workspace % 8 == 0, "ugk_dedup: workspace must be 8-byte aligned");
+  const size_t cap = dedup_capacity(n);
+  unsigned long long *slots = reinterpret_cast<unsigned long long *>(workspace);
+  uint32_t *uid_of = reinterpret_cast<uint32_t *>(slots + cap);
+  const unsigned grid = clamp_grid((n + kBlock - 1) / kBlock, 0);
+  hipLaunchKernelGGL(dedup_claim_kernel<K>, dim3(grid), dim3(kBlock), 0, as_stream(stream), keys, n, slots, cap - 1,
+                     epoch, uid_of, unique_out, inverse, n_unique);
+  UGK_HIP(hipGetLastError());
+  hipLaunchKernelGGL(dedup_resolve_kernel, dim3(grid), dim3(kBlock), 0, as_stream(stream), n, uid_of, inverse);
+  UGK_HIP(hipGetLastError());
+  return 0;
+}
+
+}  // namespace
+}  // namespace ugk
+
+using namespace ugk;
+
+extern "C" {
+
+int ugk_classify_u32(ugk_table_t t, const uint32_t *keys_dev, size_t n, uint64_t host_rows, ugk_idx_t *idx_dev,
+                     uint32_t *counts_dev, uint32_t *next_counts_dev, uint32_t *status_dev, void *stream) {
+  return classify<uint32_t>(t, keys_dev, n, host_rows, idx_dev, counts_dev, next_counts_dev, status_dev, stream);
+}
+int ugk_classify_i64(ugk_table_t t, const int64_t *keys_dev, size_t n, uint64_t host_rows, ugk_idx_t *idx_dev,
+                     uint32_t *counts_dev, uint32_t *next_counts_dev, uint32_t *status_dev, void *stream) {
+  return classify<int64_t>(t, keys_dev, n, host_rows, idx_dev, counts_dev, next_counts_dev, status_dev, stream);
+}
+
+int ugk_extract_mix_u32(ugk_table_t t, const uint32_t *keys_dev, size_t n, const void *cache_dev, uint64_t cache_rows,
+                        const void *host_dev, uint64_t host_rows, void *out_dev, size_t row_bytes,
+                        uint32_t *status_dev, void *stream) {
+  return extract_mix<uint32_t>(t, keys_dev, n, cache_dev, cache_rows, host_dev, host_rows, out_dev, row_bytes,
+                               status_dev, stream);
+}
+int ugk_extract_mix_i64(ugk_table_t t, const int64_t *keys_dev, size_t n, const void *cache_dev, uint64_t cache_rows,
+                        const void *host_dev, uint64_t host_rows, void *out_dev, size_t row_bytes,
+                        uint32_t *status_dev, void *stream) {
+  return extract_mix<int64_t>(t, keys_dev, n, cache_dev, cache_rows, host_dev, host_rows, out_dev, row_bytes,
+                              status_dev, stream);
+}
+
+size_t ugk_dedup_workspace_bytes(size_t n) { return dedup_capacity(n) * 8 + ((n + 1) / 2 * 2) * 4 + 64; }
+
+int ugk_dedup_u32(const uint32_t *keys_dev, size_t n, void *workspace_dev, uint32_t epoch, uint32_t *unique_out_dev,
+                  uint32_t *inverse_out_dev, uint32_t *n_unique_dev, void *stream) {
+  return dedup<uint32_t>(keys_dev, n, workspace_dev, epoch, unique_out_dev, inverse_out_dev, n_unique_dev, stream);
+}
+int ugk_dedup_i64(const int64_t *keys_dev, size_t n, void *workspace_dev, uint32_t epoch, int64_t *unique_out_dev,
+                  uint32_t *inverse_out_dev, uint32_t *n_unique_dev, void *stream) {
+  return dedup<int64_t>(keys_dev, n, workspace_dev, epoch, unique_out_dev, inverse_out_dev, n_unique_dev, stream);
+}
+
+}  // extern "C"

@@ -1,0 +1,263 @@
+// Runtime plumbing of the C-ABI: memory, streams, events, copies, fill/iota kernels.
+#include <cstdlib>
+#include <cstring>
+
+#include "ugk_internal.h"
+
+static thread_local char g_err[1024] = "";
+
+int ugk_set_error(const char *fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_err, sizeof(g_err), fmt, ap);
+  va_end(ap);
+  return 1;
+}
+
+namespace ugk {
+
+int cu_count() {
+  static int cached[64] = {0};
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 256;
+  if (cached[dev] == 0) {
+    int n = 0;
+    if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
+    cached[dev] = n;
+  }
+  return cached[dev];
+}
+
+int blocks_per_cu() {
+  static int v = 0;
+  if (v == 0) {
+    const char *e = getenv("UGK_BLOCKS_PER_CU");
+    v = e ? atoi(e) : 0;
+    if (v <= 0) v = 16;
+  }
+  return v;
+}
+
+namespace {
+
+__global__ __launch_bounds__(kBlock) void fill_u32_kernel(uint32_t *dst, uint32_t v, size_t n) {
+  for (size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x; i < n; i += (size_t)gridDim.x * kBlock) dst[i] = v;
+}
+
+__global__ __launch_bounds__(kBlock) void arange_u32_kernel(uint32_t *dst, uint32_t start, size_t n) {
+  for (size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x; i < n; i += (size_t)gridDim.x * kBlock)
+    dst[i] = start + (uint32_t)i;
+}
+
+// plain streaming copy, 16 bytes per lane, 4 vectors in flight per lane
+__global__ __launch_bounds__(kBlock) void copy_v16_kernel(u32x4 *__restrict__ dst, const u32x4 *__restrict__ src,
+                                                          size_t nvec) {
+  const size_t stride = (size_t)gridDim.x * kBlock;
+  size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x;
+  for (; i + 3 * stride < nvec; i += 4 * stride) {
+    u32x4 a = __builtin_nontemporal_load(src + i);
+    u32x4 b = __builtin_nontemporal_load(src + i + stride);
+    u32x4 c = __builtin_nontemporal_load(src + i + 2 * stride);
+    u32x4 d = __builtin_nontemporal_load(src + i + 3 * stride);
+    __builtin_nontemporal_store(a, dst + i);
+    __builtin_nontemporal_store(b, dst + i + stride);
+    __builtin_nontemporal_store(c, dst + i + 2 * stride);
+    __builtin_nontemporal_store(d, dst + i + 3 * stride);
+  }
+  for (; i < nvec; i += stride) __builtin_nontemporal_store(__builtin_nontemporal_load(src + i), dst + i);
+}
+
+__global__ void copy_tail_kernel(uint8_t *dst, const uint8_t *src, size_t n) {
+  for (size_t i = threadIdx.x; i < n; i += blockDim.x) dst[i] = src[i];
+}
+
+}  // namespace
+}  // namespace ugk
+
+using namespace ugk;
+
+extern "C" {
+
+const char *ugk_last_error(void) { return g_err; }
+int ugk_abi_version(void) { return 1; }
+
+int ugk_device_count(int *count) {
+  UGK_REQUIRE(count, "ugk_device_count: null output");
+  UGK_HIP(hipGetDeviceCount(count));
+  return 0;
+}
+
+int ugk_set_device(int dev) {
+  UGK_HIP(hipSetDevice(dev));
+  return 0;
+}
+
+int ugk_get_device_info(int dev, ugk_device_info_t *info) {
+  UGK_REQUIRE(info, "ugk_get_device_info: null output");
+  hipDeviceProp_t p;
+  UGK_HIP(hipGetDeviceProperties(&p, dev));
+  memset(info, 0, sizeof(*info));
+  snprintf(info->name, sizeof(info->name), "%s", p.name);
+  snprintf(info->arch, sizeof(info->arch), "%s", p.gcnArchName);
+  info->compute_units = p.multiProcessorCount;
+  info->wavefront_size = p.warpSize;
+  info->total_mem = p.totalGlobalMem;
+  info->lds_per_block = p.sharedMemPerBlock;
+  return 0;
+}
+
+int ugk_mem_info(size_t *free_bytes, size_t *total_bytes) {
+  size_t f = 0, t = 0;
+  UGK_HIP(hipMemGetInfo(&f, &t));
+  if (free_bytes) *free_bytes = f;
+  if (total_bytes) *total_bytes = t;
+  return 0;
+}
+
+int ugk_malloc(void **ptr, size_t nbytes) {
+  UGK_REQUIRE(ptr, "ugk_malloc: null output");
+  *ptr = nullptr;
+  if (nbytes == 0) return 0;
+  UGK_HIP(hipMalloc(ptr, nbytes));
+  return 0;
+}
+
+int ugk_free(void *ptr) {
+  if (ptr) UGK_HIP(hipFree(ptr));
+  return 0;
+}
+
+int ugk_host_malloc(void **ptr, size_t nbytes) {
+  UGK_REQUIRE(ptr, "ugk_host_malloc: null output");
+  *ptr = nullptr;
+  if (nbytes == 0) return 0;
+  UGK_HIP(hipHostMalloc(ptr, nbytes, hipHostMallocMapped | hipHostMallocPortable));
+  return 0;
+}
+
+int ugk_host_free(void *ptr) {
+  if (ptr) UGK_HIP(hipHostFree(ptr));
+  return 0;
+}
+
+int ugk_pointer_kind(const void *ptr, int *kind) {
+  UGK_REQUIRE(kind, "ugk_pointer_kind: null output");
+  hipPointerAttribute_t a;
+  hipError_t e = hipPointerGetAttributes(&a, ptr);
+  if (e != hipSuccess) {
+    (void)hipGetLastError();  // ordinary host memory is reported as an error; clear it
+    *kind = 0;
+    return 0;
+  }
+  if (a.type == hipMemoryTypeDevice || a.type == hipMemoryTypeManaged || a.type == hipMemoryTypeArray)
+    *kind = 2;
+  else if (a.type == hipMemoryTypeHost)
+    *kind = 1;
+  else
+    *kind = 0;
+  return 0;
+}
+
+int ugk_stream_create(void **stream) {
+  UGK_REQUIRE(stream, "ugk_stream_create: null output");
+  hipStream_t s;
+  // default priority on purpose: mixed stream priorities are not used anywhere in this library
+  UGK_HIP(hipStreamCreateWithFlags(&s, hipStreamNonBlocking));
+  *stream = s;
+  return 0;
+}
+
+int ugk_stream_destroy(void *stream) {
+  if (stream) UGK_HIP(hipStreamDestroy(as_stream(stream)));
+  return 0;
+}
+
+int ugk_stream_sync(void *stream) {
+  UGK_HIP(hipStreamSynchronize(as_stream(stream)));
+  return 0;
+}
+
+int ugk_device_sync(void) {
+  UGK_HIP(hipDeviceSynchronize());
+  return 0;
+}
+
+int ugk_event_create(void **event) {
+  UGK_REQUIRE(event, "ugk_event_create: null output");
+  hipEvent_t e;
+  UGK_HIP(hipEventCreate(&e));
+  *event = e;
+  return 0;
+}
+
+int ugk_event_destroy(void *event) {
+  if (event) UGK_HIP(hipEventDestroy(reinterpret_cast<hipEvent_t>(event)));
+  return 0;
+}
+
+int ugk_event_record(void *event, void *stream) {
+  UGK_HIP(hipEventRecord(reinterpret_cast<hipEvent_t>(event), as_stream(stream)));
+  return 0;
+}
+
+int ugk_event_sync(void *event) {
+  UGK_HIP(hipEventSynchronize(reinterpret_cast<hipEvent_t>(event)));
+  return 0;
+}
+
+int ugk_stream_wait_event(void *stream, void *event) {
+  UGK_HIP(hipStreamWaitEvent(as_stream(stream), reinterpret_cast<hipEvent_t>(event), 0));
+  return 0;
+}
+
+int ugk_event_elapsed_ms(void *start, void *stop, float *ms) {
+  UGK_REQUIRE(ms, "ugk_event_elapsed_ms: null output");
+  UGK_HIP(hipEventElapsedTime(ms, reinterpret_cast<hipEvent_t>(start), reinterpret_cast<hipEvent_t>(stop)));
+  return 0;
+}
+
+int ugk_memcpy_async(void *dst, const void *src, size_t nbytes, void *stream) {
+  if (nbytes == 0) return 0;
+  UGK_HIP(hipMemcpyAsync(dst, src, nbytes, hipMemcpyDefault, as_stream(stream)));
+  return 0;
+}
+
+int ugk_fill_u32(uint32_t *dst_dev, uint32_t value, size_t nwords, void *stream) {
+  if (nwords == 0) return 0;
+  UGK_REQUIRE(dst_dev, "ugk_fill_u32: null destination");
+  const unsigned grid = clamp_grid((nwords + kBlock - 1) / kBlock, 0);
+  hipLaunchKernelGGL(fill_u32_kernel, dim3(grid), dim3(kBlock), 0, as_stream(stream), dst_dev, value, nwords);
+  UGK_HIP(hipGetLastError());
+  return 0;
+}
+
+int ugk_arange_u32(uint32_t *dst_dev, uint32_t start, size_t n, void *stream) {
+  if (n == 0) return 0;
+  UGK_REQUIRE(dst_dev, "ugk_arange_u32: null destination");
+  const unsigned grid = clamp_grid((n + kBlock - 1) / kBlock, 0);
+  hipLaunchKernelGGL(arange_u32_kernel, dim3(grid), dim3(kBlock), 0, as_stream(stream), dst_dev, start, n);
+  UGK_HIP(hipGetLastError());
+  return 0;
+}
+
+int ugk_copy_rows(void *dst_dev, const void *src_dev, size_t nbytes, void *stream) {
+  if (nbytes == 0) return 0;
+  UGK_REQUIRE(dst_dev && src_dev, "ugk_copy_rows: null pointer");
+  UGK_REQUIRE(((uintptr_t)dst_dev % 16 == 0) && ((uintptr_t)src_dev % 16 == 0), "ugk_copy_rows: pointers must be 16-byte aligned");
+  const size_t nvec = nbytes / 16;
+  if (nvec) {
+    const unsigned grid = clamp_grid((nvec + kBlock * 4 - 1) / (kBlock * 4), 0);
+    hipLaunchKernelGGL(copy_v16_kernel, dim3(grid), dim3(kBlock), 0, as_stream(stream), (u32x4 *)dst_dev,
+                       (const u32x4 *)src_dev, nvec);
+    UGK_HIP(hipGetLastError());
+  }
+  const size_t tail = nbytes - nvec * 16;
+  if (tail) {
+    hipLaunchKernelGGL(copy_tail_kernel, dim3(1), dim3(64), 0, as_stream(stream), (uint8_t *)dst_dev + nvec * 16,
+                       (const uint8_t *)src_dev + nvec * 16, tail);
+    UGK_HIP(hipGetLastError());
+  }
+  return 0;
+}
+
+}  // extern "C"

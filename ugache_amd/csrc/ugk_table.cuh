@@ -1,0 +1,179 @@
+// Device-side lookup tables shared by the table, classify and fused-extraction kernels.
+//
+// flat table  : one uint32 per key of the key space, (loc << 28) + off, 0xffffffff = absent.
+// hash table  : ugk_bucket_t[nbuckets] (16 bytes each, nbuckets a multiple of 8, base 128-byte aligned),
+//               linear probing from home(key) = mulhi64(fmix64(key), nbuckets).
+//               A search stops at a never-used bucket, walks over tombstones and other keys.
+//               A matching key only counts when its VALID bit is set; a key that is half-way through an
+//               insert or an evict therefore reads as a miss, which is always correct because the host
+//               table holds every row.
+//
+// Lookup is wavefront-cooperative.  Phase 1: every lane probes the home bucket of its own key with one
+// 16-byte load.  Phase 2: lanes that hit a foreign key are served eight at a time: eight 8-lane groups
+// each take one pending key and read one 128-byte line (eight adjacent buckets) per step, a wavefront
+// ballot decides match / never-used / continue.  A collision therefore costs one line per step, not
+// one dependent 16-byte load per bucket.
+#pragma once
+
+#include "ugk_internal.h"
+
+namespace ugk {
+
+__device__ __forceinline__ uint64_t fmix64(uint64_t x) {
+  x ^= x >> 33;
+  x *= 0xff51afd7ed558ccdull;
+  x ^= x >> 33;
+  x *= 0xc4ceb9fe1a85ec53ull;
+  x ^= x >> 33;
+  return x;
+}
+
+__device__ __forceinline__ uint64_t hash_home(uint64_t key, uint64_t nbuckets) {
+  return __umul64hi(fmix64(key), nbuckets);
+}
+
+struct Found {
+  bool hit;      // present and valid
+  uint32_t loc;  // location of the row
+  uint32_t off;  // row inside the location
+};
+
+__device__ __forceinline__ ugk_bucket_t load_bucket(const ugk_bucket_t *p) {
+  const u32x4 v = *reinterpret_cast<const u32x4 *>(p);
+  ugk_bucket_t b;
+  b.key = ((uint64_t)v.y << 32) | v.x;
+  b.off = v.z;
+  b.meta = v.w;
+  return b;
+}
+
+__device__ __forceinline__ uint64_t shfl64(uint64_t v, int src) {
+  const uint32_t lo = __shfl((uint32_t)v, src);
+  const uint32_t hi = __shfl((uint32_t)(v >> 32), src);
+  return ((uint64_t)hi << 32) | lo;
+}
+
+// Flat lookup: one dependent 4-byte read.  Keys beyond the key space read as absent.
+__device__ __forceinline__ Found flat_lookup(const uint32_t *table, uint64_t nkeys, uint64_t key, bool active) {
+  Found f{false, 0, 0};
+  if (active && key < nkeys) {
+    const uint32_t v = table[key];
+    if (v != UGK_EMPTY_U32) {
+      f.hit = true;
+      f.loc = (v >> 28) & 0xfu;
+      f.off = v & 0x0fffffffu;
+    }
+  }
+  return f;
+}
+
+// Wavefront-cooperative hash lookup.  Must be called by all 64 lanes of the wavefront (inactive lanes pass
+// active = false).
+__device__ __forceinline__ Found hash_lookup_wave(const ugk_bucket_t *table, uint64_t nb, uint64_t key, bool active) {
+  Found f{false, 0, 0};
+  uint64_t home = 0;
+  bool pending = false;
+  if (active) {
+    home = hash_home(key, nb);
+    const ugk_bucket_t b = load_bucket(table + home);
+    if (b.key == key) {
+      if (b.meta & UGK_META_VALID) {
+        f.hit = true;
+        f.loc = b.meta & 0xfu;
+        f.off = b.off;
+      }
+    } else if (b.key != UGK_HASH_EMPTY) {
+      pending = true;
+    }
+  }
+  uint64_t pend = __ballot(pending);
+  if (pend == 0) return f;
+
+  const int lane = (int)lane_id();
+  const int grp = lane >> 3, sub = lane & 7;
+  uint64_t win = home & ~7ull;              // next 8-bucket window this lane's key has to examine
+  int min_sub = (int)(home & 7);            // in the home window only buckets after the home bucket count
+  uint64_t steps = 0;
+  const uint64_t max_steps = nb / 8 + 1;    // a full lap: give up (table without a never-used bucket)
+
+  while (pend) {
+    // the g-th 8-lane group serves the g-th pending lane
+    const int rank = __popcll(pend & ((1ull << lane) - 1ull));
+    uint64_t m = pend;
+    for (int i = 0; i < grp; ++i) m &= m - 1;
+    const int src = m ? (__ffsll((unsigned long long)m) - 1) : -1;
+    const bool gactive = src >= 0;
+    const int from = gactive ? src : lane;
+    const uint64_t k = shfl64(key, from);
+    const uint64_t w = shfl64(win, from);
+    const int ms = __shfl(min_sub, from);
+
+    bool is_match = false, is_empty = false;
+    ugk_bucket_t bb{0, 0, 0};
+    if (gactive && sub > ms) {
+      bb = load_bucket(table + w + sub);
+      is_match = bb.key == k;
+      is_empty = bb.key == UGK_HASH_EMPTY;
+    }
+    const uint32_t mb = (uint32_t)((__ballot(is_match) >> (grp * 8)) & 0xffull);
+    const uint32_t eb = (uint32_t)((__ballot(is_empty) >> (grp * 8)) & 0xffull);
+    const int fm = mb ? (__ffs(mb) - 1) : 8;
+    const int fe = eb ? (__ffs(eb) - 1) : 8;
+    // linear probing keeps a key in front of the first never-used bucket of its probe sequence
+    const bool g_found = fm < fe;
+    const bool g_done = g_found || fe < 8;
+    const int hit_lane = grp * 8 + (g_found ? fm : 0);
+    const uint32_t h_off = __shfl(bb.off, hit_lane);
+    const uint32_t h_meta = __shfl(bb.meta, hit_lane);
+    // group-uniform result word: bit 0 done, bit 1 found
+    const uint32_t g_flags = (g_done ? 1u : 0u) | (g_found ? 2u : 0u);
+
+    // hand the result back to the lane that owns the key
+    const bool served = pending && rank < 8;
+    const int back = served ? rank * 8 : lane;
+    const uint32_t r_flags = __shfl(g_flags, back);
+    const uint32_t r_off = __shfl(h_off, back);
+    const uint32_t r_meta = __shfl(h_meta, back);
+    if (served) {
+      if (r_flags & 1u) {
+        pending = false;
+        if ((r_flags & 2u) && (r_meta & UGK_META_VALID)) {
+          f.hit = true;
+          f.loc = r_meta & 0xfu;
+          f.off = r_off;
+        }
+      } else {
+        win += 8;
+        if (win >= nb) win = 0;
+        min_sub = -1;
+        if (++steps > max_steps) pending = false;
+      }
+    }
+    pend = __ballot(pending);
+  }
+  return f;
+}
+
+// Table lookup dispatch.  KIND is ugk_table_t::kind.  All lanes of the wavefront must call it.
+template <int KIND>
+__device__ __forceinline__ Found table_lookup(const ugk_table_t &t, uint64_t key, bool active) {
+  if (KIND == 1) return flat_lookup(reinterpret_cast<const uint32_t *>(t.table), t.size, key, active);
+  if (KIND == 2) return hash_lookup_wave(reinterpret_cast<const ugk_bucket_t *>(t.table), t.size, key, active);
+  return Found{false, 0, 0};
+}
+
+template <typename K>
+__device__ __forceinline__ uint64_t key_to_u64(K k);
+template <>
+__device__ __forceinline__ uint64_t key_to_u64<uint32_t>(uint32_t k) {
+  return k;
+}
+template <>
+__device__ __forceinline__ uint64_t key_to_u64<int64_t>(int64_t k) {
+  return (uint64_t)k;
+}
+
+// keys that collide with the two reserved bucket states cannot live in the hash table
+__device__ __forceinline__ bool key_is_reserved(uint64_t k) { return k >= UGK_HASH_TOMB; }
+
+}  // namespace ugk

@@ -1,0 +1,271 @@
+// Table maintenance kernels: init, insert, evict, plain lookup, census.
+// Insert and evict run at cache-fill / refresh time only, so they use a simple per-lane probe loop; the
+// per-batch lookup is the wavefront-cooperative one in ugk_table.cuh.
+#include <cmath>
+
+#include "ugk_internal.h"
+#include "ugk_table.cuh"
+
+namespace ugk {
+namespace {
+
+__global__ __launch_bounds__(kBlock) void hash_init_kernel(ugk_bucket_t *table, size_t nb) {
+  const u32x4 empty = {0xffffffffu, 0xffffffffu, 0u, 0u};
+  for (size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x; i < nb; i += (size_t)gridDim.x * kBlock)
+    *reinterpret_cast<u32x4 *>(table + i) = empty;
+}
+
+template <typename K>
+__global__ __launch_bounds__(kBlock) void flat_insert_kernel(uint32_t *table, uint64_t nkeys, const K *keys,
+                                                             const uint32_t *offs, uint32_t seq_base, uint32_t loc,
+                                                             size_t n, uint32_t *status) {
+  for (size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x; i < n; i += (size_t)gridDim.x * kBlock) {
+    const uint64_t key = key_to_u64<K>(keys[i]);
+    const uint32_t off = offs ? offs[i] : seq_base + (uint32_t)i;
+    if (key >= nkeys || off > 0x0fffffffu) {
+      atomicOr(status, UGK_ST_KEY_OUT_OF_RANGE);
+      continue;
+    }
+    const uint32_t old = atomicExch(table + key, (loc << 28) + off);
+    if (old != UGK_EMPTY_U32) atomicOr(status, UGK_ST_DUP_KEY);
+  }
+}
+
+template <typename K>
+__global__ __launch_bounds__(kBlock) void flat_evict_kernel(uint32_t *table, uint64_t nkeys, const K *keys, size_t n,
+                                                            uint32_t *status) {
+  for (size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x; i < n; i += (size_t)gridDim.x * kBlock) {
+    const uint64_t key = key_to_u64<K>(keys[i]);
+    if (key >= nkeys) {
+      atomicOr(status, UGK_ST_KEY_OUT_OF_RANGE);
+      continue;
+    }
+    const uint32_t old = atomicExch(table + key, UGK_EMPTY_U32);
+    if (old == UGK_EMPTY_U32) atomicOr(status, UGK_ST_EVICT_ABSENT);
+  }
+}
+
+__device__ __forceinline__ uint64_t load_key_relaxed(const ugk_bucket_t *b) {
+  return __atomic_load_n(&b->key, __ATOMIC_RELAXED);
+}
+
+template <typename K>
+__global__ __launch_bounds__(kBlock) void hash_insert_kernel(ugk_bucket_t *table, uint64_t nb, const K *keys,
+                                                             const uint32_t *offs, uint32_t seq_base, uint32_t loc,
+                                                             size_t n, uint32_t *status) {
+  for (size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x; i < n; i += (size_t)gridDim.x * kBlock) {
+    const uint64_t key = key_to_u64<K>(keys[i]);
+    const uint32_t off = offs ? offs[i] : seq_base + (uint32_t)i;
+    if (key_is_reserved(key)) {
+      atomicOr(status, UGK_ST_KEY_OUT_OF_RANGE);
+      continue;
+    }
+    uint64_t pos = hash_home(key, nb);
+    bool placed = false;
+    for (uint64_t step = 0; step < nb && !placed; ++step) {
+      uint64_t cur = load_key_relaxed(table + pos);
+      while (cur == UGK_HASH_EMPTY || cur == UGK_HASH_TOMB) {
+        const uint64_t seen = atomicCAS(reinterpret_cast<unsigned long long *>(&table[pos].key),
+                                        (unsigned long long)cur, (unsigned long long)key);
+        if (seen == cur) {
+          // the bucket is ours: publish the value, then the valid bit
+          table[pos].off = off;
+          __threadfence();
+          __atomic_store_n(&table[pos].meta, UGK_META_VALID | (loc & 0xfu), __ATOMIC_RELEASE);
+          placed = true;
+          break;
+        }
+        cur = seen;  // somebody else took it; re-examine what is there now
+      }
+      if (placed) break;
+      if (cur == key) {
+        atomicOr(status, UGK_ST_DUP_KEY);
+        placed = true;
+        break;
+      }
+      if (++pos == nb) pos = 0;
+    }
+    if (!placed) atomicOr(status, UGK_ST_TABLE_FULL);
+  }
+}
+
+template <typename K>
+__global__ __launch_bounds__(kBlock) void hash_evict_kernel(ugk_bucket_t *table, uint64_t nb, const K *keys,
+                                                            size_t n, uint32_t *status) {
+  for (size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x; i < n; i += (size_t)gridDim.x * kBlock) {
+    const uint64_t key = key_to_u64<K>(keys[i]);
+    uint64_t pos = key_is_reserved(key) ? 0 : hash_home(key, nb);
+    bool done = key_is_reserved(key);
+    if (done) atomicOr(status, UGK_ST_EVICT_ABSENT);
+    for (uint64_t step = 0; step < nb && !done; ++step) {
+      const uint64_t cur = load_key_relaxed(table + pos);
+      if (cur == key) {
+        __atomic_store_n(&table[pos].meta, 0u, __ATOMIC_RELEASE);
+        __threadfence();
+        __atomic_store_n(&table[pos].key, UGK_HASH_TOMB, __ATOMIC_RELEASE);
+        done = true;
+      } else if (cur == UGK_HASH_EMPTY) {
+        atomicOr(status, UGK_ST_EVICT_ABSENT);
+        done = true;
+      } else if (++pos == nb) {
+        pos = 0;
+      }
+    }
+    if (!done) atomicOr(status, UGK_ST_EVICT_ABSENT);
+  }
+}
+
+template <typename K, int KIND>
+__global__ __launch_bounds__(kBlock) void lookup_kernel(ugk_table_t t, const K *keys, size_t n, uint32_t fallback_loc,
+                                                        uint32_t *loc_out, uint32_t *off_out) {
+  // whole wavefronts stay in the loop together: the hash lookup is cooperative
+  const size_t n_round = (n + kWave - 1) / kWave * kWave;
+  for (size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x; i < n_round; i += (size_t)gridDim.x * kBlock) {
+    const bool active = i < n;
+    const uint64_t key = active ? key_to_u64<K>(keys[i]) : 0;
+    const Found f = table_lookup<KIND>(t, key, active);
+    if (active) {
+      if (loc_out) loc_out[i] = f.hit ? f.loc : fallback_loc;
+      if (off_out) off_out[i] = f.hit ? f.off : (uint32_t)key;
+    }
+  }
+}
+
+__global__ __launch_bounds__(kBlock) void census_kernel(const ugk_bucket_t *table, size_t nb,
+                                                        unsigned long long *census) {
+  unsigned long long occ = 0, tomb = 0, empty = 0;
+  for (size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x; i < nb; i += (size_t)gridDim.x * kBlock) {
+    const uint64_t k = table[i].key;
+    if (k == UGK_HASH_EMPTY) ++empty;
+    else if (k == UGK_HASH_TOMB) ++tomb;
+    else ++occ;
+  }
+  __shared__ unsigned long long red[3];
+  if (threadIdx.x < 3) red[threadIdx.x] = 0;
+  __syncthreads();
+  atomicAdd(&red[0], occ);
+  atomicAdd(&red[1], tomb);
+  atomicAdd(&red[2], empty);
+  __syncthreads();
+  if (threadIdx.x < 3) atomicAdd(census + threadIdx.x, red[threadIdx.x]);
+}
+
+int check_table(const ugk_table_t &t, const char *who) {
+  UGK_REQUIRE(t.kind == 1 || t.kind == 2, "%s: table kind %d is not flat(1) or hash(2)", who, t.kind);
+  UGK_REQUIRE(t.table != nullptr && t.size > 0, "%s: empty table", who);
+  if (t.kind == 2) {
+    UGK_REQUIRE(t.size % 8 == 0, "%s: hash table needs a multiple of 8 buckets, got %llu", who,
+                (unsigned long long)t.size);
+    UGK_REQUIRE((uintptr_t)t.table % 128 == 0, "%s: hash table must be 128-byte aligned", who);
+  }
+  return 0;
+}
+
+template <typename K>
+int table_insert(ugk_table_t t, const K *keys, const uint32_t *offs, uint32_t seq_base, uint32_t loc, size_t n,
+                 uint32_t *status, void *stream) {
+  if (n == 0) return 0;
+  if (check_table(t, "ugk_table_insert")) return 1;
+  UGK_REQUIRE(keys && status, "ugk_table_insert: null keys or status");
+  UGK_REQUIRE(loc < 16, "ugk_table_insert: location %u does not fit 4 bits", loc);
+  const unsigned grid = clamp_grid((n + kBlock - 1) / kBlock, 0);
+  if (t.kind == 1)
+    hipLaunchKernelGGL(flat_insert_kernel<K>, dim3(grid), dim3(kBlock), 0, as_stream(stream), (uint32_t *)t.table,
+                       t.size, keys, offs, seq_base, loc, n, status);
+  else
+    hipLaunchKernelGGL(hash_insert_kernel<K>, dim3(grid), dim3(kBlock), 0, as_stream(stream),
+                       (ugk_bucket_t *)t.table, t.size, keys, offs, seq_base, loc, n, status);
+  UGK_HIP(hipGetLastError());
+  return 0;
+}
+
+template <typename K>
+int table_evict(ugk_table_t t, const K *keys, size_t n, uint32_t *status, void *stream) {
+  if (n == 0) return 0;
+  if (check_table(t, "ugk_table_evict")) return 1;
+  UGK_REQUIRE(keys && status, "ugk_table_evict: null keys or status");
+  const unsigned grid = clamp_grid((n + kBlock - 1) / kBlock, 0);
+  if (t.kind == 1)
+    hipLaunchKernelGGL(flat_evict_kernel<K>, dim3(grid), dim3(kBlock), 0, as_stream(stream), (uint32_t *)t.table,
+                       t.size, keys, n, status);
+  else
+    hipLaunchKernelGGL(hash_evict_kernel<K>, dim3(grid), dim3(kBlock), 0, as_stream(stream), (ugk_bucket_t *)t.table,
+                       t.size, keys, n, status);
+  UGK_HIP(hipGetLastError());
+  return 0;
+}
+
+template <typename K>
+int table_lookup_host(ugk_table_t t, const K *keys, size_t n, uint32_t fallback_loc, uint32_t *loc_out,
+                      uint32_t *off_out, void *stream) {
+  if (n == 0) return 0;
+  if (check_table(t, "ugk_table_lookup")) return 1;
+  UGK_REQUIRE(keys, "ugk_table_lookup: null keys");
+  const unsigned grid = clamp_grid((n + kBlock - 1) / kBlock, 0);
+  if (t.kind == 1)
+    hipLaunchKernelGGL((lookup_kernel<K, 1>), dim3(grid), dim3(kBlock), 0, as_stream(stream), t, keys, n,
+                       fallback_loc, loc_out, off_out);
+  else
+    hipLaunchKernelGGL((lookup_kernel<K, 2>), dim3(grid), dim3(kBlock), 0, as_stream(stream), t, keys, n,
+                       fallback_loc, loc_out, off_out);
+  UGK_HIP(hipGetLastError());
+  return 0;
+}
+
+}  // namespace
+}  // namespace ugk
+
+using namespace ugk;
+
+extern "C" {
+
+size_t ugk_hash_buckets_for(size_t n_entries, double load_factor) {
+  if (!(load_factor > 0.0) || load_factor > 0.95) load_factor = 0.7;
+  size_t nb = (size_t)std::ceil((double)n_entries / load_factor) + 1;
+  if (nb < 64) nb = 64;
+  return (nb + 7) / 8 * 8;
+}
+
+int ugk_hash_init(ugk_bucket_t *table_dev, size_t nbuckets, void *stream) {
+  UGK_REQUIRE(table_dev && nbuckets > 0, "ugk_hash_init: empty table");
+  UGK_REQUIRE(nbuckets % 8 == 0, "ugk_hash_init: bucket count must be a multiple of 8");
+  const unsigned grid = clamp_grid((nbuckets + kBlock - 1) / kBlock, 0);
+  hipLaunchKernelGGL(hash_init_kernel, dim3(grid), dim3(kBlock), 0, as_stream(stream), table_dev, nbuckets);
+  UGK_HIP(hipGetLastError());
+  return 0;
+}
+
+int ugk_table_insert_u32(ugk_table_t t, const uint32_t *keys_dev, const uint32_t *offs_dev, uint32_t seq_base,
+                         uint32_t loc, size_t n, uint32_t *status_dev, void *stream) {
+  return table_insert<uint32_t>(t, keys_dev, offs_dev, seq_base, loc, n, status_dev, stream);
+}
+int ugk_table_insert_i64(ugk_table_t t, const int64_t *keys_dev, const uint32_t *offs_dev, uint32_t seq_base,
+                         uint32_t loc, size_t n, uint32_t *status_dev, void *stream) {
+  return table_insert<int64_t>(t, keys_dev, offs_dev, seq_base, loc, n, status_dev, stream);
+}
+int ugk_table_evict_u32(ugk_table_t t, const uint32_t *keys_dev, size_t n, uint32_t *status_dev, void *stream) {
+  return table_evict<uint32_t>(t, keys_dev, n, status_dev, stream);
+}
+int ugk_table_evict_i64(ugk_table_t t, const int64_t *keys_dev, size_t n, uint32_t *status_dev, void *stream) {
+  return table_evict<int64_t>(t, keys_dev, n, status_dev, stream);
+}
+int ugk_table_lookup_u32(ugk_table_t t, const uint32_t *keys_dev, size_t n, uint32_t fallback_loc,
+                         uint32_t *loc_out_dev, uint32_t *off_out_dev, void *stream) {
+  return table_lookup_host<uint32_t>(t, keys_dev, n, fallback_loc, loc_out_dev, off_out_dev, stream);
+}
+int ugk_table_lookup_i64(ugk_table_t t, const int64_t *keys_dev, size_t n, uint32_t fallback_loc,
+                         uint32_t *loc_out_dev, uint32_t *off_out_dev, void *stream) {
+  return table_lookup_host<int64_t>(t, keys_dev, n, fallback_loc, loc_out_dev, off_out_dev, stream);
+}
+
+int ugk_hash_census(const ugk_bucket_t *table_dev, size_t nbuckets, uint64_t *census_dev, void *stream) {
+  UGK_REQUIRE(table_dev && census_dev, "ugk_hash_census: null pointer");
+  if (ugk_fill_u32(reinterpret_cast<uint32_t *>(census_dev), 0u, 6, stream)) return 1;
+  const unsigned grid = clamp_grid((nbuckets + kBlock - 1) / kBlock, 0);
+  hipLaunchKernelGGL(census_kernel, dim3(grid), dim3(kBlock), 0, as_stream(stream), table_dev, nbuckets,
+                     reinterpret_cast<unsigned long long *>(census_dev));
+  UGK_HIP(hipGetLastError());
+  return 0;
+}
+
+}  // extern "C"
