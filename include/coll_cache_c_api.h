@@ -1,0 +1,114 @@
+/*
+ * coll_cache_c_api.h — the drop-in C boundary of the embedding-extraction path (libcoll_cache.so).
+ *
+ * Section 1 is, name for name and argument for argument, the extern "C" surface of the reference's shim
+ * (SJTU-IPADS/ugache python/collcache/common/operation.h:31-61 and operation.cc:205-209), which its ctypes
+ * loader (python/collcache/common/__init__.py:173-262) and its PyTorch / TensorFlow bindings call.
+ * Section 2 holds C-callable forms of what the reference exposes only as C++ (the std::function allocator of
+ * coll_cache_init, the refresh driven by the TF LookupManager) plus wide-key siblings; each names what it
+ * stands for.
+ *
+ * Errors follow the reference: no return codes; a violated precondition or a failed GPU call prints a message
+ * and abort()s (coll_cache_lib/logging.h:32-34, logging.cc:69-73).
+ * Threading: one replica <-> one GPU <-> one caller thread; coll_cache_lookup is blocking and not re-entrant per
+ * replica; coll_cache_refresh may run on another thread concurrently with lookups.
+ * All key / output pointers of lookups are device pointers; `stream` is a hipStream_t passed as void*.
+ */
+#ifndef COLL_CACHE_C_API_H_
+#define COLL_CACHE_C_API_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef void *StreamHandle; /* coll_cache_lib/common.h:137 */
+
+/* ---------------- Section 1: the reference's extern "C" surface ---------------- */
+
+/* operation.h:35-36, operation.cc:154-167.  Required keys (operation.cc:72-78): cache_percentage, _cache_policy,
+ * num_device, num_global_step_per_epoch, num_epoch, num_total_item, omp_thread_num.  Once per process. */
+void coll_cache_config(const char **config_keys, const char **config_values, const size_t num_config_items);
+/* operation.h:42, operation.cc:177-180 */
+void coll_cache_log_step_by_key(uint64_t key, int item, double val);
+/* operation.h:44, operation.cc:182-186 */
+void coll_cache_report_step_by_key(uint64_t key);
+/* operation.h:46, operation.cc:188-202 */
+void coll_cache_report_step_average_by_key(uint64_t key);
+/* operation.h:49, operation.cc:211-213 */
+void coll_cache_train_barrier(void);
+/* operation.h:53, operation.cc:219-230: waitpid(-1); 1 if a child exited non-zero or by signal, else 0 */
+int coll_cache_wait_one_child(void);
+/* operation.h:55, operation.cc:258-261 */
+void coll_cache_print_memory_usage(void);
+/* operation.h:57, operation.cc:232-236: output[i, :] = table[key[i], :]; step key = steps[replica] * num_device + replica */
+void coll_cache_lookup(int replica_id, uint32_t *key, size_t num_keys, void *output, StreamHandle stream);
+/* operation.h:59, operation.cc:241-244: host pointer; counts hotness and tracks the largest batch */
+void coll_cache_record(int replica_id, uint32_t *key, size_t num_keys);
+/* operation.cc:205-209 (declared by the ctypes loader, __init__.py:201-202) */
+void coll_cache_record_init(int replica_id);
+
+/* ---------------- Section 2: C forms of the reference's C++-only entry points ---------------- */
+
+/* Device allocator callback pair standing for std::function<MemHandle(size_t)> (operation.h:28;
+ * coll_cache_lib/common.h:140-149): alloc returns device memory of at least nbytes, release frees it.
+ * Passing alloc == NULL makes the library use its own device allocator. */
+typedef void *(*coll_cache_alloc_fn)(size_t nbytes, void *user);
+typedef void (*coll_cache_release_fn)(void *ptr, void *user);
+
+/* coll_cache_init (operation.h:28, operation.cc:129-150): combine + rank the recorded hotness, place, build the
+ * cache of replica_id.  dtype is the DataType code of coll_cache_lib/common.h:39-49 (kF32 = 0, kF16 = 2 ...);
+ * fp16 tables may be passed as kF16 with their true dim.  cpu_data must be pinned GPU-mapped host memory
+ * (coll_cache_alloc_host_table) unless cache_percentage == 1. */
+void coll_cache_init_c(int replica_id, size_t key_space_size, coll_cache_alloc_fn alloc, coll_cache_release_fn release,
+                       void *user, void *cpu_data, int dtype, size_t dim, double cache_percentage,
+                       StreamHandle stream);
+/* the build_v2 overload taking an explicit rank list + frequency list over all keys
+ * (coll_cache_lib/facade.h:56-60) instead of recorded hotness */
+void coll_cache_init_ranked_c(int replica_id, size_t key_space_size, const uint32_t *rank_keys,
+                              const uint32_t *rank_freq, coll_cache_alloc_fn alloc, coll_cache_release_fn release,
+                              void *user, void *cpu_data, int dtype, size_t dim, double cache_percentage,
+                              StreamHandle stream);
+/* 64-bit (dense) keys: siblings of coll_cache_lookup / coll_cache_record.  The reference is uint32 end to end
+ * (coll_cache_lib/constant.h:28). */
+void coll_cache_lookup_i64(int replica_id, const int64_t *key, size_t num_keys, void *output, StreamHandle stream);
+void coll_cache_record_i64(int replica_id, const int64_t *key, size_t num_keys);
+/* LookupManager::refresh (python_tf2/collcache_tf2/collcache_tf2/core/lookup_manager.cc:317-333) ->
+ * CollCache::refresh (coll_cache_lib/facade.cc:513-557): re-rank by the hotness recorded since the last
+ * build/refresh, evict and insert.  foreground != 0 skips the wait for an in-flight lookup and the throttling. */
+void coll_cache_refresh(int replica_id, StreamHandle stream, int foreground);
+/* pinned, GPU-mapped host memory for the embedding table; stands for Tensor::CreateShm + cudaHostRegister
+ * (python/collcache/torch/adapter.cc:239-268; coll_cache_lib/facade.cc:476) */
+void *coll_cache_alloc_host_table(size_t nbytes);
+void coll_cache_free_host_table(void *ptr);
+/* `extern size_t max_num_keys` of operation.h:29 */
+size_t coll_cache_max_num_keys(void);
+void coll_cache_set_max_num_keys(size_t n);
+/* {0, #rows served from the GPU cache, num_keys} of the last lookup: the reference's group_offset
+ * (coll_cache_lib/cache_context.cu:825-847) */
+void coll_cache_last_group_offset(int replica_id, uint32_t out[3]);
+/* out[0] cache capacity in rows, [1] cached rows, [2] lookup table kind (0 none/direct, 1 flat, 2 open addressing),
+ * [3] row bytes, [4] key space, [5] completed lookups, [6] free cache slots, [7] reserved */
+void coll_cache_get_info(int replica_id, uint64_t out[8]);
+/* cached keys of replica_id (ascending): copies up to `capacity` keys, returns the number cached */
+size_t coll_cache_get_cached_keys(int replica_id, uint32_t *out, size_t capacity);
+/* value of one profiler item of the reference's LogStepItem enum at a step key (0 when not logged) */
+double coll_cache_get_step_value(uint64_t key, int item);
+/* host-only pieces of the build, callable without a GPU:
+ * rank the hotness recorded so far exactly as coll_cache_init_c would (LocalCombineToShared + GlobalCombine + Sort,
+ * operation.cc:138-147; this consumes the recorded counts): distinct keys in rank order with their counts, up to
+ * `capacity` entries are copied; returns the number of distinct keys */
+size_t coll_cache_rank_hotness(int replica_id, uint32_t *keys_out, uint32_t *cnts_out, size_t capacity);
+/* place num_node ranked keys for one GPU (the solver step of build_v2, facade.cc:93-160): nid_to_block_out[key] = 0
+ * (cached) or 1 (host); returns the number of cached keys */
+uint32_t coll_cache_place_ranked(const uint32_t *rank_keys, const uint32_t *rank_freq, uint32_t num_node,
+                                 double cache_percentage, uint32_t *nid_to_block_out);
+/* drop every global object so that coll_cache_config may be called again (the reference has no teardown) */
+void coll_cache_shutdown(void);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* COLL_CACHE_C_API_H_ */

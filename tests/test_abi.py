@@ -1,0 +1,74 @@
+"""CPU checks of the drop-in boundary: both shared libraries load, and export every symbol their headers declare
+(no compute call is made here)."""
+import ctypes
+import os
+import re
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def _declared(header, prefix):
+    text = open(os.path.join(ROOT, "include", header)).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    names = set(re.findall(r"\b(%s\w+)\s*\(" % prefix, text))
+    # function-pointer typedefs are not symbols
+    names -= set(re.findall(r"\(\s*\*\s*(%s\w+)\s*\)" % prefix, text))
+    return names
+
+
+def test_hip_library_exports_everything_ugache_hip_h_declares():
+    from ugache_amd import hip
+    lib = hip.lib()
+    declared = _declared("ugache_hip.h", "ugk_")
+    assert len(declared) > 40
+    for name in declared:
+        assert hasattr(lib, name), name
+    assert declared == set(hip.SIGNATURES), declared ^ set(hip.SIGNATURES)
+    assert hip.call("ugk_abi_version") == 1
+    assert lib.ugk_hash_buckets_for(50_000_000, 0.7) % 8 == 0
+    assert lib.ugk_hash_buckets_for(50_000_000, 0.7) >= 50_000_000 / 0.7
+    assert lib.ugk_dedup_workspace_bytes(1000) >= 2048 * 8 + 4000
+
+
+def test_host_library_exports_everything_coll_cache_c_api_h_declares():
+    import sys
+    sys.path.insert(0, os.path.join(ROOT, "ugache_amd"))
+    import collcache.common as cc
+    lib = cc._basics.C_LIB_CTYPES
+    declared = _declared("coll_cache_c_api.h", "coll_cache_")
+    for name in declared:
+        assert hasattr(lib, name), name
+    assert declared == set(cc.C_API), declared ^ set(cc.C_API)
+    # the reference's own extern "C" names (python/collcache/common/operation.h:31-61, operation.cc:205-209)
+    for name in ["coll_cache_config", "coll_cache_log_step_by_key", "coll_cache_report_step_by_key",
+                 "coll_cache_report_step_average_by_key", "coll_cache_train_barrier", "coll_cache_wait_one_child",
+                 "coll_cache_print_memory_usage", "coll_cache_lookup", "coll_cache_record", "coll_cache_record_init"]:
+        assert name in declared
+
+
+def test_host_library_has_no_hip_symbols_of_its_own():
+    """host C++ reaches the GPU only through the ugk_* C-ABI"""
+    import subprocess
+    out = subprocess.run(["nm", "-D", "--undefined-only", os.path.join(ROOT, "ugache_amd", "libcoll_cache.so")],
+                         stdout=subprocess.PIPE, text=True).stdout
+    undefined = [l.split()[-1] for l in out.splitlines() if l.strip()]
+    assert any(u.startswith("ugk_") for u in undefined)
+    assert not [u for u in undefined if u.startswith("hip") or u.startswith("__hip")]
+
+
+def test_python_surface_matches_reference_names():
+    import sys
+    sys.path.insert(0, os.path.join(ROOT, "ugache_amd"))
+    import collcache.common as cc
+    # policy ids and profiler item ids (python/collcache/common/__init__.py:47-171)
+    assert cc.kCollCacheAsymmLink == 13 and cc.kRepCache == 12 and cc.kCollFineGrain == 18
+    assert cc.cache_policies["coll_cache_asymm_link"] == 13
+    assert cc.kLogL1FeatureBytes == 9 and cc.kLogL1MissBytes == 13 and cc.kLogL1RemoteBytes == 14
+    assert cc.kLogL2CacheCopyTime == 27
+    assert cc.kLogL3CacheGetIndexTime == 46 and cc.kLogL3CacheCombineMissTime == 50
+    assert cc.kLogL3CacheCombineCacheTime == 51 and cc.kLogL3CacheCombineRemoteTime == 52
+    assert cc.kLogL3LabelExtractTime == 53
+    assert cc.kLogEpochFeatureBytes == 13 and cc.kLogEpochMissBytes == 14
+    assert cc.gpu(1) == "cuda:1" and cc.cpu() == "cpu:0"

@@ -1,0 +1,251 @@
+"""GPU parity tests through the drop-in boundary: the `collcache.torch` surface over libcoll_cache.so, used in the
+reference's call order (config -> record_init -> record* -> create_emb_shm -> init_t -> lookup*, see
+example/gnn/dgl_sample.py:238-259 of the reference) and checked bit-for-bit against the CPU oracle."""
+import os
+import sys
+import threading
+
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+torch = pytest.importorskip("torch")
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+sys.path.insert(0, os.path.join(ROOT, "ugache_amd"))
+
+from oracle_lib import Oracle  # noqa: E402
+
+ORC = Oracle()
+
+if torch.cuda.is_available():
+    import collcache.torch as co
+    from collcache.common import _basics, kLogL1FeatureBytes, kLogL1MissBytes, kLogL2CacheCopyTime
+
+
+def zipf_ranks(rng, n, space, s):
+    """bounded-Pareto inverse CDF used for the synthetic hotness (ranks in [0, space))"""
+    u = rng.random(n)
+    h = float(space)
+    r = np.floor(((h ** (1 - s) - 1) * u + 1) ** (1 / (1 - s))).astype(np.int64)
+    return np.clip(r - 1, 0, space - 1)
+
+
+def make_config(num_total_item, pct, threads=8):
+    return {"cache_percentage": pct, "_cache_policy": co.kCollCacheAsymmLink, "num_device": 1,
+            "num_global_step_per_epoch": 100, "num_epoch": 1, "num_total_item": num_total_item,
+            "omp_thread_num": threads}
+
+
+@pytest.fixture(autouse=True)
+def _fresh_cache(monkeypatch):
+    for v in ("COLL_HASH_TABLE", "SAMGRAPH_COLL_CACHE_CONCURRENT_LINK_IMPL", "SAMGRAPH_COLL_CACHE_NO_GROUP"):
+        monkeypatch.delenv(v, raising=False)
+    yield
+    if torch.cuda.is_available():
+        co.coll_torch_shutdown()
+
+
+def fill_table(emb, rng):
+    a = emb.numpy()
+    a.view(np.uint8)[...] = rng.integers(0, 256, size=a.view(np.uint8).shape, dtype=np.uint8)
+    if a.dtype == np.float32:
+        # keep the bit patterns, but avoid NaN payload surprises in printing only; bytes are compared anyway
+        pass
+    return a
+
+
+def expected_cached_set(stream_u32, n_item, pct):
+    rank_k, _ = ORC.full_rank(stream_u32, n_item)
+    nid, nc = ORC.rep_solve(rank_k, n_item, pct * 100)
+    return np.nonzero(nid == 0)[0].astype(np.uint32), nid
+
+
+def lookup_bytes(keys_t, n_item, pad=True):
+    out = co.coll_torch_lookup_key_t_val_ret(0, keys_t, pad)
+    return out
+
+
+@pytest.mark.parametrize("kdtype", [torch.int32, torch.int64])
+@pytest.mark.parametrize("pct", [1.0, 0.0])
+def test_direct_mapping_full_and_no_cache(kdtype, pct):
+    rng = np.random.default_rng(1)
+    n_item, dim = 20_000, 128
+    co.config(make_config(n_item, pct))
+    co.coll_cache_record_init(0)
+    emb = co.coll_torch_create_emb_shm(0, n_item, dim, torch.float32)
+    table = fill_table(emb, rng)
+    co.coll_torch_init_t(0, 0, emb, pct)
+    info = _basics.info(0)
+    assert info["table_kind"] == 0 and info["row_bytes"] == dim * 4
+    for n in (1, 13, 4096, 30_001):
+        keys = rng.integers(0, n_item, size=n)
+        kt = torch.from_numpy(keys).to(kdtype).cuda()
+        out = co.coll_torch_lookup_key_t_val_ret(0, kt, True)
+        assert out.shape == ((n + 7) // 8 * 8, dim) and out.dtype == torch.float32 and out.is_cuda
+        got = out[:n].cpu().numpy()
+        assert got.tobytes() == ORC.gather(table, keys.astype(np.int64)).tobytes()
+        g = _basics.last_group_offset(0)
+        assert g == ([0, n, n] if pct == 1.0 else [0, 0, n])
+        out2 = co.coll_torch_lookup_key_t_val_ret(0, kt, False)
+        assert out2.shape == (n, dim)
+        assert out2.data_ptr() == out.data_ptr() or n > 4096  # one reused buffer unless it had to grow
+    # profiler hooks of the lookup
+    assert _basics.step_value(0, kLogL1FeatureBytes) == 1 * dim * 4
+    assert _basics.step_value(0, kLogL2CacheCopyTime) > 0
+    assert _basics.info(0)["lookups"] == 8
+
+
+@pytest.mark.parametrize("table_kind", ["FLAT", "HASH"])
+@pytest.mark.parametrize("impl", ["", "DIRECT", "NONE"])
+@pytest.mark.parametrize("kdtype", [torch.int32, torch.int64])
+def test_partial_cache_matches_oracle(table_kind, impl, kdtype, monkeypatch):
+    monkeypatch.setenv("COLL_HASH_TABLE", table_kind)
+    if impl:
+        monkeypatch.setenv("SAMGRAPH_COLL_CACHE_CONCURRENT_LINK_IMPL", impl)
+    rng = np.random.default_rng(7)
+    n_item, dim, pct = 50_000, 128, 0.1
+    co.config(make_config(n_item, pct))
+    co.coll_cache_record_init(0)
+    perm = rng.permutation(n_item)
+    stream = []
+    for _ in range(4):  # presample epochs
+        keys = perm[zipf_ranks(rng, 40_000, n_item, 1.1)]
+        stream.append(keys)
+        co.coll_torch_record(0, torch.from_numpy(keys).to(kdtype))
+    emb = co.coll_torch_create_emb_shm(0, n_item, dim, torch.float32)
+    table = fill_table(emb, rng)
+    co.coll_torch_init_t(0, 0, emb, pct)
+
+    want_cached, nid = expected_cached_set(np.concatenate(stream).astype(np.uint32), n_item, pct)
+    info = _basics.info(0)
+    assert info["table_kind"] == (1 if table_kind == "FLAT" else 2)
+    assert info["capacity_rows"] == ORC.lib.orc_cache_capacity(n_item, pct)
+    assert info["cached_rows"] == len(want_cached) == int(n_item * (pct * 100 / 100.0))
+    assert info["free_slots"] == info["capacity_rows"] - info["cached_rows"]
+    got_cached = np.zeros(len(want_cached), np.uint32)
+    assert _basics.C_LIB_CTYPES.coll_cache_get_cached_keys(0, got_cached.ctypes.data, len(got_cached)) == len(want_cached)
+    assert np.array_equal(got_cached, want_cached)
+
+    for n in (1, 1000, 65_536):
+        keys = perm[zipf_ranks(rng, n, n_item, 1.1)]
+        kt = torch.from_numpy(keys).to(kdtype).cuda()
+        out = co.coll_torch_lookup_key_t_val_ret(0, kt, False)
+        assert out.cpu().numpy().tobytes() == ORC.gather(table, keys.astype(np.int64)).tobytes()
+        if impl != "DIRECT":
+            n_local = int((nid[keys] == 0).sum())
+            assert _basics.last_group_offset(0) == [0, n_local, n]
+    if impl != "DIRECT":
+        step = _basics.info(0)["lookups"] - 1
+        assert _basics.step_value(step, kLogL1MissBytes) == (n - n_local) * dim * 4
+
+
+def test_fp16_table_and_small_rows():
+    rng = np.random.default_rng(9)
+    n_item, dim, pct = 30_000, 64, 0.2
+    co.config(make_config(n_item, pct))
+    co.coll_cache_record_init(0)
+    keys = rng.integers(0, n_item, size=100_000)
+    co.coll_torch_record(0, torch.from_numpy(keys).to(torch.int32))
+    emb = co.coll_torch_create_emb_shm(0, n_item, dim, torch.float16)
+    table = fill_table(emb, rng)
+    assert table.dtype == np.float16 and table.strides[0] == 128
+    co.coll_torch_init_t(0, 0, emb, pct)
+    q = rng.integers(0, n_item, size=10_001)
+    out = co.coll_torch_lookup_key_t_val_ret(0, torch.from_numpy(q).to(torch.int32).cuda(), True)
+    assert out.dtype == torch.float16 and out.shape == ((10_001 + 7) // 8 * 8, dim)
+    assert out[:10_001].cpu().numpy().tobytes() == ORC.gather(table, q.astype(np.int64)).tobytes()
+
+
+def test_create_emb_from_file(tmp_path):
+    rng = np.random.default_rng(2)
+    arr = rng.standard_normal((1000, 32)).astype(np.float32)
+    f = tmp_path / "feat.bin"
+    arr.tofile(f)
+    co.config(make_config(1000, 1.0))
+    emb = co.coll_torch_create_emb_shm(0, 1000, 32, torch.float32, str(f))
+    assert emb.numpy().tobytes() == arr.tobytes()
+    co.coll_torch_init_t(0, 0, emb, 1.0)
+    q = torch.arange(999, -1, -1, dtype=torch.int32, device="cuda")
+    assert co.coll_torch_lookup_key_t_val_ret(0, q, False).cpu().numpy().tobytes() == arr[::-1].tobytes()
+
+
+@pytest.mark.parametrize("table_kind", ["FLAT", "HASH"])
+@pytest.mark.parametrize("foreground", [True, False])
+def test_refresh_evicts_and_inserts_like_the_oracle(table_kind, foreground, monkeypatch):
+    monkeypatch.setenv("COLL_HASH_TABLE", table_kind)
+    monkeypatch.setenv("COLL_REFRESH_SLEEP_US", "100")
+    monkeypatch.setenv("COLL_REFRESH_BATCH_ROWS", "512")
+    rng = np.random.default_rng(11)
+    n_item, dim, pct = 40_000, 128, 0.25
+    co.config(make_config(n_item, pct))
+    co.coll_cache_record_init(0)
+    perm1 = rng.permutation(n_item)
+    s1 = perm1[zipf_ranks(rng, 200_000, n_item, 1.05)]
+    co.coll_torch_record(0, torch.from_numpy(s1).to(torch.int32))
+    emb = co.coll_torch_create_emb_shm(0, n_item, dim, torch.float32)
+    table = fill_table(emb, rng)
+    co.coll_torch_init_t(0, 0, emb, pct)
+    old_cached, old_nid = expected_cached_set(s1.astype(np.uint32), n_item, pct)
+    cap = _basics.info(0)["capacity_rows"]
+
+    def check_lookup(nid, seed):
+        r = np.random.default_rng(seed)
+        keys = r.integers(0, n_item, size=20_000)
+        out = co.coll_torch_lookup_key_t_val_ret(0, torch.from_numpy(keys).to(torch.int32).cuda(), False)
+        assert out.cpu().numpy().tobytes() == ORC.gather(table, keys.astype(np.int64)).tobytes()
+        if nid is not None:
+            assert _basics.last_group_offset(0)[1] == int((nid[keys] == 0).sum())
+
+    check_lookup(old_nid, 1)
+    # hotness moves: a new permutation for the next interval
+    for rnd in range(2):
+        perm2 = rng.permutation(n_item)
+        s2 = perm2[zipf_ranks(rng, 200_000, n_item, 1.05)]
+        co.coll_torch_record(0, torch.from_numpy(s2).to(torch.int32))
+        new_cached, new_nid = expected_cached_set(s2.astype(np.uint32), n_item, pct)
+        if foreground:
+            co.coll_torch_refresh(0, True)
+        else:
+            # background refresh on its own thread while the caller keeps looking keys up
+            t = threading.Thread(target=co.coll_torch_refresh, args=(0, False))
+            t.start()
+            i = 0
+            while t.is_alive():
+                check_lookup(None, 100 + i)
+                i += 1
+            t.join()
+            assert i >= 1
+        info = _basics.info(0)
+        got = np.zeros(len(new_cached), np.uint32)
+        assert _basics.C_LIB_CTYPES.coll_cache_get_cached_keys(0, got.ctypes.data, len(got)) == len(new_cached)
+        assert np.array_equal(got, new_cached)
+        assert info["cached_rows"] == len(new_cached) and info["free_slots"] + info["cached_rows"] == cap
+        assert len(np.setdiff1d(old_cached, new_cached)) > 1000  # the refresh really moved rows
+        check_lookup(new_nid, 2 + rnd)
+        old_cached = new_cached
+
+
+def test_reference_cpu_runnable_config_full_size():
+    """1M x 128 fp32 host table, 65536 int64 keys Zipf(1.1) over a seeded permutation, hottest 10 % cached."""
+    rng = np.random.default_rng(1)
+    n_item, dim, pct, n = 1_000_000, 128, 0.10, 65_536
+    co.config(make_config(n_item, pct))
+    co.coll_cache_record_init(0)
+    emb = co.coll_torch_create_emb_shm(0, n_item, dim, torch.float32)
+    emb.normal_(generator=torch.Generator().manual_seed(1))
+    table = emb.numpy()
+    perm = np.random.default_rng(2).permutation(n_item)
+    r3 = np.random.default_rng(3)
+    batches = [perm[zipf_ranks(r3, n, n_item, 1.1)] for _ in range(4)]
+    for b in batches[:3]:
+        co.coll_torch_record(0, torch.from_numpy(b))
+    co.coll_torch_init_t(0, 0, emb, pct)
+    _, nid = expected_cached_set(np.concatenate(batches[:3]).astype(np.uint32), n_item, pct)
+    assert _basics.info(0)["cached_rows"] == 100_000
+    for b in batches:
+        out = co.coll_torch_lookup_key_t_val_ret(0, torch.from_numpy(b).cuda(), False)
+        assert out.shape == (n, dim)
+        assert out.cpu().numpy().tobytes() == ORC.gather(table, b.astype(np.int64), omp=True).tobytes()
+        assert _basics.last_group_offset(0) == [0, int((nid[b] == 0).sum()), n]

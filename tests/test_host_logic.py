@@ -1,0 +1,142 @@
+"""CPU tests of the host logic behind the C-ABI (no GPU call): config marshalling, hotness recording and ranking,
+frequency-ranked placement — each against the oracle / closed forms."""
+import ctypes
+import os
+import subprocess
+import sys
+import textwrap
+
+import numpy as np
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+sys.path.insert(0, os.path.join(ROOT, "ugache_amd"))
+
+import collcache.common as cc  # noqa: E402
+from oracle_lib import Oracle  # noqa: E402
+
+ORC = Oracle()
+C = cc._basics.C_LIB_CTYPES
+
+
+def _config(num_total_item, pct=0.1, threads=4):
+    cc._basics.shutdown()
+    cc._basics.config({"cache_percentage": pct, "_cache_policy": cc.kCollCacheAsymmLink, "num_device": 1,
+                       "num_global_step_per_epoch": 10, "num_epoch": 2, "num_total_item": num_total_item,
+                       "omp_thread_num": threads})
+
+
+@pytest.fixture(autouse=True)
+def _teardown():
+    yield
+    cc._basics.shutdown()
+
+
+def _zipf_keys(rng, n, space, s):
+    u = rng.random(n)
+    h = float(space)
+    r = np.floor(((h ** (1 - s) - 1) * u + 1) ** (1 / (1 - s))).astype(np.int64)
+    return np.clip(r - 1, 0, space - 1)
+
+
+@pytest.mark.parametrize("kdtype", [np.uint32, np.int64])
+def test_record_and_rank_match_oracle(kdtype):
+    rng = np.random.default_rng(3)
+    n_item = 50_000
+    _config(n_item)
+    cc._basics.coll_cache_record_init(0)
+    perm = rng.permutation(n_item)
+    stream = []
+    for _ in range(5):
+        keys = perm[_zipf_keys(rng, 70_000, n_item, 1.1)].astype(kdtype)
+        stream.append(keys)
+        if kdtype == np.int64:
+            C.coll_cache_record_i64(0, keys.ctypes.data, len(keys))
+        else:
+            C.coll_cache_record(0, keys.ctypes.data, len(keys))
+    assert C.coll_cache_max_num_keys() == 70_000
+    allk = np.concatenate(stream).astype(np.uint32)
+    want_k, want_c = ORC.freq_rank(allk)
+    got_k = np.zeros(n_item, np.uint32)
+    got_c = np.zeros(n_item, np.uint32)
+    m = C.coll_cache_rank_hotness(0, got_k.ctypes.data, got_c.ctypes.data, n_item)
+    assert m == len(want_k)
+    assert np.array_equal(got_k[:m], want_k) and np.array_equal(got_c[:m], want_c)
+    # the counts were consumed: ranking again sees nothing new
+    assert C.coll_cache_rank_hotness(0, None, None, 0) == 0
+
+
+@pytest.mark.parametrize("pct", [0.0, 0.1, 0.25, 0.333, 0.999])
+def test_placement_matches_oracle_rep_solve(pct):
+    rng = np.random.default_rng(5)
+    n_item = 20_011
+    stream = (rng.zipf(1.2, size=100_000) % n_item).astype(np.uint32)
+    rank_k, rank_c = ORC.full_rank(stream, n_item)
+    want, want_n = ORC.rep_solve(rank_k, n_item, pct * 100)
+    got = np.zeros(n_item, np.uint32)
+    n_cached = C.coll_cache_place_ranked(rank_k.ctypes.data, rank_c.ctypes.data, n_item, pct, got.ctypes.data)
+    assert n_cached == want_n == int(n_item * (pct * 100 / 100.0))
+    assert np.array_equal(got, want)
+    # closed form: the cached set is the n_cached keys with the largest (count, key)
+    cached = np.nonzero(got == 0)[0]
+    assert set(cached.tolist()) == set(rank_k[:n_cached].tolist())
+
+
+def test_config_is_once_per_process_and_requires_keys():
+    # violations abort() like the reference's CHECKs, so they are observed in a child process
+    code = textwrap.dedent("""
+        import sys
+        sys.path.insert(0, %r)
+        import collcache.common as cc
+        cfg = {"cache_percentage": 0.1, "_cache_policy": 13, "num_device": 1, "num_global_step_per_epoch": 1,
+               "num_epoch": 1, "num_total_item": 10, "omp_thread_num": 1}
+        mode = sys.argv[1]
+        if mode == "twice":
+            cc._basics.config(cfg); cc._basics.config(cfg)
+        elif mode == "missing":
+            del cfg["num_total_item"]; cc._basics.config(cfg)
+        elif mode == "two_gpus":
+            cfg["num_device"] = 2; cc._basics.config(cfg)
+        elif mode == "ok":
+            cc._basics.config(cfg); cc._basics.coll_cache_record_init(0)
+        print("survived")
+    """ % os.path.join(ROOT, "ugache_amd"))
+    for mode, ok in [("ok", True), ("twice", False), ("missing", False), ("two_gpus", False)]:
+        p = subprocess.run([sys.executable, "-c", code, mode], stdout=subprocess.PIPE, stderr=subprocess.PIPE, text=True)
+        if ok:
+            assert p.returncode == 0 and "survived" in p.stdout, p.stderr
+        else:
+            assert p.returncode == -6 and "survived" not in p.stdout  # SIGABRT
+            assert "Check failed" in p.stderr
+
+
+def test_wait_one_child_reports_failed_children():
+    """coll_cache_wait_one_child (operation.cc:219-230): 1 for a child that exits non-zero or dies by signal."""
+    code = textwrap.dedent("""
+        import os, sys
+        sys.path.insert(0, %r)
+        import collcache.common as cc
+        res = []
+        for how in ("ok", "fail", "abort"):
+            pid = os.fork()
+            if pid == 0:
+                if how == "ok": os._exit(0)
+                if how == "fail": os._exit(3)
+                os.abort()
+            res.append(cc._basics.wait_one_child())
+        print(res)
+    """ % os.path.join(ROOT, "ugache_amd"))
+    p = subprocess.run([sys.executable, "-c", code], stdout=subprocess.PIPE, stderr=subprocess.PIPE, text=True)
+    assert p.returncode == 0, p.stderr
+    assert "[0, 1, 1]" in p.stdout
+
+
+def test_profiler_hooks_store_and_report(capfd):
+    _config(100)
+    cc._basics.log_step_by_key(3, cc.kLogL1FeatureBytes, 4096.0)
+    cc._basics.log_step_by_key(3, cc.kLogL2CacheCopyTime, 0.5)
+    assert cc._basics.step_value(3, cc.kLogL1FeatureBytes) == 4096.0
+    assert cc._basics.step_value(4, cc.kLogL1FeatureBytes) == 0.0
+    cc._basics.report_step(3)
+    out = capfd.readouterr().out
+    assert "cache feat copy 0.500000" in out and "feature nbytes" in out

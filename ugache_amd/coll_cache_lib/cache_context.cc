@@ -1,0 +1,553 @@
+#include "cache_context.h"
+
+#include <unistd.h>
+
+#include <algorithm>
+#include <cstring>
+#include <iostream>
+
+#include "facade.h"
+#include "logging.h"
+#include "timer.h"
+
+namespace coll_cache_lib {
+
+namespace {
+
+// location ids with one GPU: the GPU is 0, the host is num_device == 1 (cache_context.cu:2421-2422)
+constexpr int kLocalLoc = UGK_LOC_LOCAL;
+constexpr int kCpuLoc = UGK_LOC_HOST;
+
+int PointerKind(const void *p) {
+  int kind = 0;
+  UGK_CALL(ugk_pointer_kind(p, &kind));
+  return kind;
+}
+
+void RequireDeviceAccessible(const void *cpu_data) {
+  CHECK(PointerKind(cpu_data) != 0)
+      << "the host embedding table must be pinned, GPU-mapped memory (ugk_host_malloc / coll_cache_alloc_host_table / "
+         "a torch tensor created with pin_memory=True): this platform does not page-lock an existing allocation the "
+         "way the reference does with cudaHostRegister";
+}
+
+}  // namespace
+
+CacheContext::~CacheContext() { delete _new_hash_table; }
+
+// cache_context.cu:1887-1904 — 0 % cache: every row is read from the host table
+void CacheContext::build_no_cache(int location_id, std::shared_ptr<CollCache> coll_cache_ptr, void *cpu_src_data,
+                                  DataType dtype, size_t dim, Context gpu_ctx, StreamHandle stream) {
+  RequireDeviceAccessible(cpu_src_data);
+  _cpu_location_id = 0;
+  _local_location_id = location_id;
+  _num_location = 1;
+  _cache_nbytes = 0;
+  _device_cache_data.assign(1, cpu_src_data);
+  _cache_nodes = 0;
+  _cache_space_capacity = 0;
+  LOG(INFO) << "Collaborative GPU cache (policy: no cache)";
+  std::cout << "test_result:init:cache_nbytes=" << _cache_nbytes << "\n";
+}
+
+// cache_context.cu:1906-1938 — 100 % cache: the whole table is copied into HBM, keys index it directly
+void CacheContext::build_full_cache(int location_id, std::shared_ptr<CollCache> coll_cache_ptr, void *cpu_src_data,
+                                    DataType dtype, size_t dim, Context gpu_ctx, size_t num_total_nodes,
+                                    StreamHandle stream) {
+  _cpu_location_id = -1;
+  _local_location_id = location_id;
+  _num_location = 1;
+  Timer t;
+  _cache_nbytes = num_total_nodes * _row_bytes;
+  _cache_space_capacity = num_total_nodes;
+  _cache_nodes = num_total_nodes;
+  _device_cache_data_local_handle = _eager_gpu_mem_allocator(_cache_nbytes);
+  void *local_cache = _device_cache_data_local_handle->ptr();
+  UGK_CALL(ugk_memcpy_async(local_cache, cpu_src_data, _cache_nbytes, stream));
+  UGK_CALL(ugk_stream_sync(stream));
+  _device_cache_data.assign(1, local_cache);
+  LOG(INFO) << "Collaborative GPU cache (policy: full cache) " << num_total_nodes << " nodes ( "
+            << ToReadableSize(_cache_nbytes) << " | " << t.Passed() << " secs )";
+  std::cout << "test_result:init:cache_nbytes=" << _cache_nbytes << "\n";
+}
+
+// cache_context.cu:2414-2599 — partial cache: frequency-ranked fill + lookup table
+void CacheContext::build_with_advise_new_hash(int location_id, std::shared_ptr<CollCache> coll_cache_ptr,
+                                              void *cpu_data, DataType dtype, size_t dim, Context gpu_ctx,
+                                              double cache_percentage, StreamHandle stream) {
+  RequireDeviceAccessible(cpu_data);
+  CHECK_EQ(RunConfig::num_device, (size_t)1) << "this build serves one GPU and its host";
+  _num_location = (int)RunConfig::num_device + 1;
+  _cpu_location_id = (int)RunConfig::num_device;
+  CHECK_EQ(_cpu_location_id, kCpuLoc);
+  CHECK_EQ(location_id, kLocalLoc);
+  _local_location_id = location_id;
+  CHECK_NOTNULL(coll_cache_ptr->_nid_to_block);
+  CHECK_NOTNULL(coll_cache_ptr->_block_access_advise);
+  CHECK_NOTNULL(coll_cache_ptr->_block_density);
+  const size_t num_total_nodes = coll_cache_ptr->_nid_to_block->Shape()[0];
+  _num_total_nodes = num_total_nodes;
+  Timer t;
+
+  _device_cache_data.assign(_num_location, nullptr);
+  _device_cache_data[_cpu_location_id] = cpu_data;
+
+  // 1. keys this GPU caches (ascending key order), from the placement
+  _new_hash_table = new CacheEntryManager;
+  _new_hash_table->_device_id = gpu_ctx.device_id;
+  TensorPtr *keys_for_each_source = _new_hash_table->_keys_for_each_src;
+  const size_t num_block = coll_cache_ptr->_block_access_advise->Shape()[1];
+  TensorPtr advise_line = Tensor::FromBlob(
+      coll_cache_ptr->_block_access_advise->Ptr<uint8_t>() + (size_t)location_id * num_block, kU8, {num_block},
+      CPU_CLIB(), "advise_line");
+  CacheEntryManager::DetectKeysForAllSource(coll_cache_ptr->_nid_to_block, advise_line, location_id,
+                                            coll_cache_ptr->_block_density, num_total_nodes, keys_for_each_source,
+                                            (int)RunConfig::num_device);
+  const size_t num_cached_nodes = keys_for_each_source[location_id]->NumItem();
+  _new_hash_table->_remote_keys = Tensor::Empty(kI32, {0}, CPU_CLIB(), "");
+  const size_t num_cpu_nodes = num_total_nodes - num_cached_nodes;
+
+  // 2. cache space: capacity leaves 0.1 % of the key space as slack for refresh (cache_context.cu:2473)
+  _cache_space_capacity = (size_t)(num_total_nodes * (cache_percentage + 0.001));
+  CHECK_LE(num_cached_nodes, _cache_space_capacity);
+  _cache_nbytes = _cache_space_capacity * _row_bytes;
+  _cache_nodes = num_cached_nodes;
+  _device_cache_data_local_handle = _eager_gpu_mem_allocator(_cache_nbytes);
+  _device_cache_data[_local_location_id] = _device_cache_data_local_handle->ptr();
+
+  // 3. lookup table: flat (4 bytes per key of the key space) when that is small or when the reference would pick
+  //    it (cache_context.cu:2489-2497), open addressing otherwise
+  bool use_flat = TableSize(std::max<size_t>(num_cached_nodes, 2)) > num_total_nodes / 2 ||
+                  num_total_nodes * sizeof(IdType) <= ((size_t)256 << 20);
+  if (RunConfig::force_table_kind == 1) use_flat = true;
+  if (RunConfig::force_table_kind == 2) use_flat = false;
+  if (use_flat) {
+    _new_hash_table->CreateFlat(_eager_gpu_mem_allocator, num_total_nodes, stream);
+  } else {
+    _new_hash_table->CreateHash(_eager_gpu_mem_allocator, std::max<size_t>(_cache_space_capacity, 1), stream);
+  }
+
+  // 4. fill: rows of the cached keys host -> HBM in list order, slot = position in the list
+  if (num_cached_nodes > 0) {
+    auto cache_node_list = Tensor::CopyToExternal(keys_for_each_source[location_id], _eager_gpu_mem_allocator,
+                                                  _trainer_ctx, stream);
+    MemHandle st = _eager_gpu_mem_allocator(256);
+    UGK_CALL(ugk_fill_u32(st->ptr<uint32_t>(), 0, 1, stream));
+    UGK_CALL(ugk_gather_direct_u32(cpu_data, num_total_nodes, cache_node_list->CPtr<uint32_t>(), num_cached_nodes,
+                                   _device_cache_data[_local_location_id], _row_bytes, 0, st->ptr<uint32_t>(),
+                                   stream));
+    _new_hash_table->InsertSeqOffWithLoc(cache_node_list, location_id, stream);
+    uint32_t fill_status = 0;
+    UGK_CALL(ugk_memcpy_async(&fill_status, st->ptr(), sizeof(fill_status), stream));
+    UGK_CALL(ugk_stream_sync(stream));
+    CHECK_EQ(fill_status, 0u) << "cache fill gathered a key outside the host table";
+    _new_hash_table->CheckStatus(stream, "cache fill");
+  }
+  UGK_CALL(ugk_stream_sync(stream));
+
+  // 5. bookkeeping for refresh: cached key list and free slots [n_cached, capacity) (cache_context.cu:2577-2585)
+  _new_hash_table->_cached_keys = keys_for_each_source[location_id];
+  _new_hash_table->_cache_space_capacity = (IdType)_cache_space_capacity;
+  _new_hash_table->cpu_location_id = _cpu_location_id;
+  _new_hash_table->num_total_key = num_total_nodes;
+  _new_hash_table->_free_offsets = Tensor::Empty(kI32, {_cache_space_capacity}, CPU_CLIB(), "free_offsets");
+  _new_hash_table->_free_offsets->ForceScale(kI32, {_cache_space_capacity - num_cached_nodes}, CPU_CLIB(), "");
+  for (size_t i = 0; i < _cache_space_capacity - num_cached_nodes; i++)
+    _new_hash_table->_free_offsets->Ptr<IdType>()[i] = (IdType)(num_cached_nodes + i);
+
+  LOG(INFO) << "Asymm Coll cache (policy: " << (int)RunConfig::cache_policy << ") | local " << num_cached_nodes
+            << " / " << num_total_nodes << " nodes ( " << ToPercentage(num_cached_nodes / (double)num_total_nodes)
+            << "~" << ToPercentage(cache_percentage) << ") | cpu " << num_cpu_nodes << " / " << num_total_nodes
+            << " | " << ToReadableSize(_cache_nbytes) << " | " << t.Passed() << " secs";
+  std::cout << "test_result:init:feat_nbytes=" << num_total_nodes * _row_bytes << "\n";
+  std::cout << "test_result:init:cache_nbytes=" << _cache_nbytes << "\n";
+}
+
+// cache_context.cu:2601-2647
+void CacheContext::build(std::function<MemHandle(size_t)> gpu_mem_allocator, int location_id,
+                         std::shared_ptr<CollCache> coll_cache_ptr, void *cpu_data, DataType dtype, size_t dim,
+                         Context gpu_ctx, double cache_percentage, StreamHandle stream) {
+  _coll_cache = coll_cache_ptr;
+  _gpu_mem_allocator = gpu_mem_allocator;
+  _trainer_ctx = gpu_ctx;
+  _dtype = dtype;
+  _dim = dim;
+  _row_bytes = GetDataTypeBytes(dtype) * dim;
+  _num_total_nodes = RunConfig::num_total_item;
+  CHECK_NOTNULL(cpu_data);
+  CHECK_GT(_row_bytes, (size_t)0);
+  UGK_CALL(ugk_set_device(gpu_ctx.device_id));
+  const int dev = gpu_ctx.device_id;
+  _eager_gpu_mem_allocator = [dev](size_t nbytes) -> MemHandle { return EagerGPUAlloc(dev, nbytes); };
+
+  if (cache_percentage == 0) {
+    return build_no_cache(location_id, coll_cache_ptr, cpu_data, dtype, dim, gpu_ctx, stream);
+  } else if (cache_percentage == 1) {
+    return build_full_cache(location_id, coll_cache_ptr, cpu_data, dtype, dim, gpu_ctx, RunConfig::num_total_item,
+                            stream);
+  } else if (_coll_cache->_block_access_advise) {
+    build_with_advise_new_hash(location_id, coll_cache_ptr, cpu_data, dtype, dim, gpu_ctx, cache_percentage, stream);
+  } else {
+    LOG(FATAL) << "a partial cache needs a placement: call build_v2, which solves before it builds";
+  }
+}
+
+// ---------------------------------------------------------------------------------------------------------
+// ExtractSession
+// ---------------------------------------------------------------------------------------------------------
+ExtractSession::ExtractSession(std::shared_ptr<CacheContext> cache_ctx) : _cache_ctx(cache_ctx) {
+  const int dev = _cache_ctx->_trainer_ctx.device_id;
+  UGK_CALL(ugk_set_device(dev));
+  UGK_CALL(ugk_stream_create(&_local_ext_stream));
+  UGK_CALL(ugk_stream_create(&_cpu_ext_stream));
+  UGK_CALL(ugk_event_create(&_ev_classified));
+  UGK_CALL(ugk_event_create(&_ev_local_done));
+  UGK_CALL(ugk_event_create(&_ev_cpu_done));
+  for (auto &e : _ev_t) UGK_CALL(ugk_event_create(&e));
+  _state_handle = EagerGPUAlloc(dev, 256);
+  uint32_t *state = _state_handle->ptr<uint32_t>();
+  UGK_CALL(ugk_fill_u32(state, 0, 64, nullptr));
+  UGK_CALL(ugk_stream_sync(nullptr));
+  _counts[0] = state;
+  _counts[1] = state + 2;
+  _status = state + 4;
+  _host_mirror_handle = PinnedHostAlloc(256);
+  _host_mirror = _host_mirror_handle->ptr<uint32_t>();
+  memset(_host_mirror, 0, 256);
+  const auto &desc = RunConfig::coll_cache_link_desc;
+  if (!desc.cpu_sm.empty()) _cpu_blocks = (unsigned)desc.cpu_sm[0];
+}
+
+ExtractSession::~ExtractSession() {
+  ugk_stream_destroy(_local_ext_stream);
+  ugk_stream_destroy(_cpu_ext_stream);
+  ugk_event_destroy(_ev_classified);
+  ugk_event_destroy(_ev_local_done);
+  ugk_event_destroy(_ev_cpu_done);
+  for (auto &e : _ev_t) ugk_event_destroy(e);
+}
+
+void ExtractSession::EnsureIdx(size_t num_nodes) {
+  const size_t need = num_nodes * sizeof(ugk_idx_t);
+  if (_idx_handle == nullptr || _idx_handle->nbytes() < need) {
+    _idx_handle = nullptr;
+    _idx_handle = _cache_ctx->_gpu_mem_allocator(need + need / 4 + 256);
+    CHECK_NOTNULL(_idx_handle);
+  }
+}
+
+void ExtractSession::CheckStatusWord(uint32_t st) const {
+  CHECK_EQ(st, 0u) << "extraction kernels reported status 0x" << std::hex << st
+                   << ": a key is outside the table it has to be read from (num_total_item="
+                   << std::dec << _cache_ctx->_num_total_nodes << ")";
+}
+
+template <typename KeyT>
+static int GatherDirect(const void *src, uint64_t rows, const KeyT *keys, size_t n, void *out, size_t rb,
+                        unsigned max_blocks, uint32_t *status, StreamHandle s);
+template <>
+int GatherDirect<IdType>(const void *src, uint64_t rows, const IdType *keys, size_t n, void *out, size_t rb,
+                         unsigned max_blocks, uint32_t *status, StreamHandle s) {
+  return ugk_gather_direct_u32(src, rows, keys, n, out, rb, max_blocks, status, s);
+}
+template <>
+int GatherDirect<Id64Type>(const void *src, uint64_t rows, const Id64Type *keys, size_t n, void *out, size_t rb,
+                           unsigned max_blocks, uint32_t *status, StreamHandle s) {
+  return ugk_gather_direct_i64(src, rows, keys, n, out, rb, max_blocks, status, s);
+}
+static int Classify(ugk_table_t t, const IdType *keys, size_t n, uint64_t host_rows, ugk_idx_t *idx, uint32_t *c,
+                    uint32_t *next, uint32_t *st, StreamHandle s) {
+  return ugk_classify_u32(t, keys, n, host_rows, idx, c, next, st, s);
+}
+static int Classify(ugk_table_t t, const Id64Type *keys, size_t n, uint64_t host_rows, ugk_idx_t *idx, uint32_t *c,
+                    uint32_t *next, uint32_t *st, StreamHandle s) {
+  return ugk_classify_i64(t, keys, n, host_rows, idx, c, next, st, s);
+}
+static int ExtractMix(ugk_table_t t, const IdType *keys, size_t n, const void *cache, uint64_t cache_rows,
+                      const void *host, uint64_t host_rows, void *out, size_t rb, uint32_t *st, StreamHandle s) {
+  return ugk_extract_mix_u32(t, keys, n, cache, cache_rows, host, host_rows, out, rb, st, s);
+}
+static int ExtractMix(ugk_table_t t, const Id64Type *keys, size_t n, const void *cache, uint64_t cache_rows,
+                      const void *host, uint64_t host_rows, void *out, size_t rb, uint32_t *st, StreamHandle s) {
+  return ugk_extract_mix_i64(t, keys, n, cache, cache_rows, host, host_rows, out, rb, st, s);
+}
+
+// cache_context.cu:1199-1794
+template <typename KeyT>
+void ExtractSession::ExtractFeatImpl(const KeyT *nodes, size_t num_nodes, void *output, StreamHandle stream,
+                                     uint64_t task_key) {
+  CacheContext *ctx = _cache_ctx.get();
+  auto profiler = ctx->_coll_cache ? ctx->_coll_cache->_profiler : nullptr;
+  const size_t rb = ctx->_row_bytes;
+  const size_t nbytes = num_nodes * rb;
+  _group_offset[0] = 0;
+  if (num_nodes == 0) {
+    _group_offset[1] = _group_offset[2] = 0;
+    ctx->progress.fetch_add(1);
+    return;
+  }
+  CHECK_NOTNULL(nodes);
+  CHECK_NOTNULL(output);
+
+  if (ctx->IsDirectMapping()) {
+    // fast path: no table, one gather.  Full cache reads HBM with the whole chip; no cache reads the host table
+    // with the host-link budget.
+    CHECK_EQ(ctx->_num_location, 1);
+    const bool from_host = ctx->_cpu_location_id != -1;
+    Timer t0;
+    UGK_CALL(GatherDirect<KeyT>(ctx->_device_cache_data[0], ctx->_num_total_nodes, nodes, num_nodes, output, rb,
+                                from_host ? _cpu_blocks : 0, _status, stream));
+    UGK_CALL(ugk_memcpy_async(_host_mirror + 4, _status, sizeof(uint32_t), stream));
+    UGK_CALL(ugk_stream_sync(stream));
+    CheckStatusWord(_host_mirror[4]);
+    const double combine_time = t0.Passed();
+    _group_offset[1] = from_host ? 0 : (uint32_t)num_nodes;
+    _group_offset[2] = (uint32_t)num_nodes;
+    if (profiler && task_key != 0xffffffffffffffffull) {
+      profiler->LogStep(task_key, kLogL1FeatureBytes, nbytes);
+      if (!from_host) {
+        profiler->LogStep(task_key, kLogL3CacheCombineCacheTime, combine_time);
+      } else {
+        profiler->LogStep(task_key, kLogL1MissBytes, nbytes);
+        profiler->LogStep(task_key, kLogL3CacheCombineMissTime, combine_time);
+        profiler->LogEpochAdd(task_key, kLogEpochMissBytes, nbytes);
+      }
+      profiler->LogEpochAdd(task_key, kLogEpochFeatureBytes, nbytes);
+    }
+    ctx->progress.fetch_add(1);
+    return;
+  }
+
+  const ugk_table_t table = ctx->_new_hash_table->_table;
+  const void *cache = ctx->_device_cache_data[ctx->_local_location_id];
+  const void *host = ctx->_device_cache_data[ctx->_cpu_location_id];
+  const uint64_t cache_rows = ctx->_cache_space_capacity;
+  const uint64_t host_rows = ctx->_num_total_nodes;
+
+  if (RunConfig::concurrent_link_impl == kDirectNoGroup) {
+    // one fused lookup + gather kernel, source chosen per row (cache_context.cu:1295-1329)
+    Timer t0;
+    UGK_CALL(ExtractMix(table, nodes, num_nodes, cache, cache_rows, host, host_rows, output, rb, _status, stream));
+    UGK_CALL(ugk_memcpy_async(_host_mirror + 4, _status, sizeof(uint32_t), stream));
+    UGK_CALL(ugk_stream_sync(stream));
+    CheckStatusWord(_host_mirror[4]);
+    _group_offset[1] = _group_offset[2] = (uint32_t)num_nodes;  // group sizes are not produced on this path
+    if (profiler && task_key != 0xffffffffffffffffull) {
+      profiler->LogStep(task_key, kLogL1FeatureBytes, nbytes);
+      profiler->LogStep(task_key, kLogL3CacheCombineCacheTime, t0.Passed());
+      profiler->LogEpochAdd(task_key, kLogEpochFeatureBytes, nbytes);
+    }
+    ctx->progress.fetch_add(1);
+    return;
+  }
+
+  // classify + partition on the caller's stream, then one gather per source
+  EnsureIdx(num_nodes);
+  ugk_idx_t *idx = _idx_handle->ptr<ugk_idx_t>();
+  uint32_t *cur = _counts[_cur], *next = _counts[_cur ^ 1];
+  UGK_CALL(ugk_event_record(_ev_t[0], stream));
+  UGK_CALL(Classify(table, nodes, num_nodes, host_rows, idx, cur, next, _status, stream));
+  UGK_CALL(ugk_event_record(_ev_classified, stream));
+  if (RunConfig::concurrent_link_impl == kSMMaskPhase) {
+    // factored extraction: the host-link gather gets a few workgroups on its own stream, the HBM gather
+    // the rest of the chip on another; both read their group bounds from the device-side counters
+    UGK_CALL(ugk_stream_wait_event(_cpu_ext_stream, _ev_classified));
+    UGK_CALL(ugk_gather_group(host, host_rows, idx, cur, UGK_LOC_HOST, num_nodes, output, rb, _cpu_blocks, _status,
+                              _cpu_ext_stream));
+    UGK_CALL(ugk_event_record(_ev_cpu_done, _cpu_ext_stream));
+    UGK_CALL(ugk_stream_wait_event(_local_ext_stream, _ev_classified));
+    UGK_CALL(ugk_gather_group(cache, cache_rows, idx, cur, UGK_LOC_LOCAL, num_nodes, output, rb, 0, _status,
+                              _local_ext_stream));
+    UGK_CALL(ugk_event_record(_ev_local_done, _local_ext_stream));
+    UGK_CALL(ugk_stream_wait_event(stream, _ev_cpu_done));
+    UGK_CALL(ugk_stream_wait_event(stream, _ev_local_done));
+  } else {
+    // sequential: host group, then local group (cache_context.cu:1719-1792)
+    UGK_CALL(ugk_gather_group(host, host_rows, idx, cur, UGK_LOC_HOST, num_nodes, output, rb, 0, _status, stream));
+    UGK_CALL(ugk_event_record(_ev_cpu_done, stream));
+    UGK_CALL(ugk_gather_group(cache, cache_rows, idx, cur, UGK_LOC_LOCAL, num_nodes, output, rb, 0, _status,
+                              stream));
+    UGK_CALL(ugk_event_record(_ev_local_done, stream));
+  }
+  // counters + status of this lookup -> pinned host, then the single blocking wait of the call
+  UGK_CALL(ugk_memcpy_async(_host_mirror, _state_handle->ptr(), 5 * sizeof(uint32_t), stream));
+  UGK_CALL(ugk_stream_sync(stream));
+  const uint32_t n_local = _host_mirror[_cur * 2], n_miss = _host_mirror[_cur * 2 + 1];
+  _cur ^= 1;
+  CheckStatusWord(_host_mirror[4]);
+  CHECK_EQ((size_t)n_local + n_miss, num_nodes);
+  _group_offset[1] = n_local;
+  _group_offset[2] = (uint32_t)num_nodes;
+
+  if (profiler && task_key != 0xffffffffffffffffull) {
+    float ms_idx = 0, ms_miss = 0, ms_local = 0;
+    UGK_CALL(ugk_event_elapsed_ms(_ev_t[0], _ev_classified, &ms_idx));
+    UGK_CALL(ugk_event_elapsed_ms(_ev_classified, _ev_cpu_done, &ms_miss));
+    if (RunConfig::concurrent_link_impl == kSMMaskPhase)
+      UGK_CALL(ugk_event_elapsed_ms(_ev_classified, _ev_local_done, &ms_local));
+    else
+      UGK_CALL(ugk_event_elapsed_ms(_ev_cpu_done, _ev_local_done, &ms_local));
+    profiler->LogStep(task_key, kLogL1FeatureBytes, nbytes);
+    profiler->LogStep(task_key, kLogL1MissBytes, (double)n_miss * rb);
+    profiler->LogStep(task_key, kLogL1RemoteBytes, 0);
+    profiler->LogStep(task_key, kLogL3CacheGetIndexTime, ms_idx * 1e-3);
+    profiler->LogStep(task_key, kLogL3CacheCombineMissTime, ms_miss * 1e-3);
+    profiler->LogStep(task_key, kLogL3CacheCombineRemoteTime, 0);
+    profiler->LogStep(task_key, kLogL3CacheCombineCacheTime, ms_local * 1e-3);
+  }
+  ctx->progress.fetch_add(1);
+}
+
+void ExtractSession::ExtractFeat(const IdType *nodes, const size_t num_nodes, void *output, StreamHandle stream,
+                                 uint64_t task_key) {
+  ExtractFeatImpl<IdType>(nodes, num_nodes, output, stream, task_key);
+}
+
+void ExtractSession::ExtractFeat64(const Id64Type *nodes, const size_t num_nodes, void *output, StreamHandle stream,
+                                   uint64_t task_key) {
+  ExtractFeatImpl<Id64Type>(nodes, num_nodes, output, stream, task_key);
+}
+
+// ---------------------------------------------------------------------------------------------------------
+// RefreshSession
+// ---------------------------------------------------------------------------------------------------------
+RefreshSession::~RefreshSession() {
+  if (low_pri_stream) ugk_stream_destroy(low_pri_stream);
+}
+
+TensorPtr RefreshSession::Empty1DReuse(TensorPtr &preserved_buffer, DataType dtype, std::vector<size_t> shape,
+                                       Context ctx) {
+  CHECK_EQ(shape.size(), (size_t)1);
+  if (preserved_buffer && preserved_buffer->CanForceScale(dtype, shape)) {
+    preserved_buffer->ForceScale(dtype, shape, ctx, "");
+    return preserved_buffer;
+  }
+  preserved_buffer = Tensor::EmptyExternal(dtype, shape, _cache_ctx->_eager_gpu_mem_allocator, ctx, "");
+  return preserved_buffer;
+}
+
+TensorPtr RefreshSession::CopyTo1DReuse(TensorPtr &preserved_buffer, TensorPtr src, Context ctx,
+                                        StreamHandle stream) {
+  auto ret = Empty1DReuse(preserved_buffer, src->Type(), src->Shape(), ctx);
+  UGK_CALL(ugk_memcpy_async(ret->MutableData(), src->Data(), src->NumBytes(), stream));
+  UGK_CALL(ugk_stream_sync(stream));  // src is pageable host memory owned by the caller
+  return ret;
+}
+
+// cache_context.cu:3944-4107, the one-GPU part: steps 1-3, 5 and 6
+void RefreshSession::refresh_after_solve_new(bool foreground) {
+  CacheContext *ctx = _cache_ctx.get();
+  auto table = ctx->_new_hash_table;
+  CHECK_NOTNULL(table) << "refresh needs a partial cache (0 < cache_percentage < 1)";
+  const Context gpu_ctx = ctx->_trainer_ctx;
+  const int local = ctx->_local_location_id;
+  auto coll_cache = ctx->_coll_cache;
+  UGK_CALL(ugk_set_device(gpu_ctx.device_id));
+  if (low_pri_stream == nullptr) UGK_CALL(ugk_stream_create(&low_pri_stream));
+  if (!_status_handle) {
+    _status_handle = EagerGPUAlloc(gpu_ctx.device_id, 256);
+    UGK_CALL(ugk_fill_u32(_status_handle->ptr<uint32_t>(), 0, 64, stream));
+  }
+
+  // Step 1: key list of the new placement
+  TensorPtr key_list_of_each_src[9] = {nullptr};
+  const size_t num_block = coll_cache->_block_access_advise->Shape()[1];
+  TensorPtr advise_line = Tensor::FromBlob(coll_cache->_block_access_advise->Ptr<uint8_t>() + (size_t)local * num_block,
+                                           kU8, {num_block}, CPU_CLIB(), "advise_line");
+  CacheEntryManager::DetectKeysForAllSource(coll_cache->_nid_to_block, advise_line, local, coll_cache->_block_density,
+                                            RunConfig::num_total_item, key_list_of_each_src,
+                                            (int)RunConfig::num_device);
+  const size_t num_new_local_key = key_list_of_each_src[local]->NumItem();
+  CHECK(num_new_local_key <= ctx->_cache_space_capacity) << "cache space can not hold refreshed new cache";
+
+  // Step 2: keys to insert = new local and not old local
+  TensorPtr new_insert_keys;
+  {
+    const IdType *old_n2b = coll_cache->_old_nid_to_block->CPtr<IdType>();
+    const uint8_t *old_place = coll_cache->_old_block_placement->CPtr<uint8_t>();
+    new_insert_keys = table->DetectKeysWithCond(
+        key_list_of_each_src[local]->CPtr<IdType>(), num_new_local_key,
+        [old_n2b, old_place, local](const IdType &key) { return (old_place[old_n2b[key]] & (1 << local)) == 0; },
+        num_new_local_key);
+  }
+  const size_t num_preserved_key = num_new_local_key - new_insert_keys->NumItem();
+
+  // Step 3: keys to evict = old cached and not new local; their slots go back to the free list, then evict
+  TensorPtr new_evict_keys;
+  {
+    const IdType *n2b = coll_cache->_nid_to_block->CPtr<IdType>();
+    const uint8_t *place = coll_cache->_block_placement->CPtr<uint8_t>();
+    new_evict_keys = table->DetectKeysWithCond(
+        table->_cached_keys->CPtr<IdType>(), table->_cached_keys->NumItem(),
+        [n2b, place, local](const IdType &key) { return (place[n2b[key]] & (1 << local)) == 0; },
+        table->_cached_keys->NumItem() - num_preserved_key);
+  }
+  const size_t num_evicted = new_evict_keys->NumItem();
+  CHECK_EQ(num_evicted + num_preserved_key, table->_cached_keys->NumItem());
+  if (num_evicted > 0) {
+    auto evict_keys_gpu = CopyTo1DReuse(__keys_buffer, new_evict_keys, gpu_ctx, stream);
+    auto evict_offs_gpu = Empty1DReuse(__offs_buffer, kI32, {num_evicted}, gpu_ctx);
+    table->LookupOffset(evict_keys_gpu, evict_offs_gpu, stream);
+    TensorPtr evict_offs_cpu = Tensor::Empty(kI32, {num_evicted}, CPU_CLIB(), "");
+    UGK_CALL(ugk_memcpy_async(evict_offs_cpu->MutableData(), evict_offs_gpu->Data(), evict_offs_gpu->NumBytes(),
+                              stream));
+    UGK_CALL(ugk_stream_sync(stream));
+    table->ReturnOffset(evict_offs_cpu);
+    CHECK(num_evicted <= table->_free_offsets->NumItem());
+    table->Evict(evict_keys_gpu, stream);
+    table->CheckStatus(stream, "refresh evict");
+  }
+  LOG(INFO) << "refresh: preserved " << num_preserved_key << ", evict " << num_evicted << ", insert "
+            << new_insert_keys->NumItem() << ", free slots " << table->_free_offsets->NumItem();
+
+  // Step 5: let one more lookup finish, so that no gather in flight still reads a slot about to be reused
+  const size_t current_progress = ctx->progress.load();
+  AnonymousBarrier::_refresh_instance->Wait();
+  {
+    Timer t0;
+    while (!foreground && ctx->progress.load() < current_progress + 1) {
+      if (t0.PassedSec() >= 20) break;
+      usleep(50);
+    }
+  }
+
+  // Step 6: copy the new rows host -> HBM into slots taken from the front of the free list, then publish them
+  const size_t num_insert = new_insert_keys->NumItem();
+  if (num_insert > 0) {
+    auto insert_keys_gpu = CopyTo1DReuse(__keys_buffer, new_insert_keys, gpu_ctx, low_pri_stream);
+    auto reserved_offset =
+        CopyTo1DReuse(__offs_buffer, table->ReserveOffsetFront((IdType)num_insert), gpu_ctx, low_pri_stream);
+    const void *host = ctx->_device_cache_data[ctx->_cpu_location_id];
+    void *cache = ctx->_device_cache_data[ctx->_local_location_id];
+    uint32_t *status = _status_handle->ptr<uint32_t>();
+    // background refresh copies in small throttled batches so that foreground lookups keep the host link
+    const size_t batch = foreground ? num_insert : std::max<size_t>(RunConfig::refresh_batch_rows, 1);
+    const unsigned limit_block = foreground ? 0 : RunConfig::refresh_limit_block;
+    for (size_t begin = 0; begin < num_insert; begin += batch) {
+      const size_t cur = std::min(batch, num_insert - begin);
+      UGK_CALL(ugk_gather_scatter_u32(host, ctx->_num_total_nodes, insert_keys_gpu->CPtr<uint32_t>() + begin,
+                                      reserved_offset->CPtr<uint32_t>() + begin, cur, cache,
+                                      ctx->_cache_space_capacity, ctx->_row_bytes, limit_block, status,
+                                      low_pri_stream));
+      if (!foreground && begin + batch < num_insert) {
+        UGK_CALL(ugk_stream_sync(low_pri_stream));
+        usleep(RunConfig::refresh_sleep_us);
+      }
+    }
+    uint32_t st = 0;
+    UGK_CALL(ugk_memcpy_async(&st, status, sizeof(st), low_pri_stream));
+    UGK_CALL(ugk_stream_sync(low_pri_stream));
+    CHECK_EQ(st, 0u) << "refresh row copy touched a row outside its table";
+    table->InsertWithLoc(insert_keys_gpu, reserved_offset, local, stream);
+    table->CheckStatus(stream, "refresh insert");
+  }
+  AnonymousBarrier::_refresh_instance->Wait();
+
+  table->_cached_keys = key_list_of_each_src[local];
+  ctx->_cache_nodes = num_new_local_key;
+  CHECK_EQ(table->_free_offsets->NumItem() + num_new_local_key, ctx->_cache_space_capacity);
+}
+
+void RefreshSession::refresh_after_solve_main(bool foreground) { refresh_after_solve_new(foreground); }
+
+}  // namespace coll_cache_lib

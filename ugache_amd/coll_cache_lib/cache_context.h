@@ -1,0 +1,134 @@
+// Per-GPU cache state and the sessions that work on it.  Class names, public members and method signatures
+// follow coll_cache_lib/cache_context.h of the reference (CacheContext :256-339, ExtractSession :420-512,
+// RefreshSession :514-532) so that the facade and its callers are source compatible; the bodies are a
+// single-GPU, HIP-stream design:
+//   * no per-source worker threads and job syncers: the calling thread enqueues the classify kernel on the
+//     caller's stream and the two per-source gathers on two library-owned streams, ordered by events;
+//   * no host round trip between lookup and gather: group sizes stay in device memory, the gathers read them;
+//   * one blocking synchronisation per lookup (the API stays synchronous: output is complete on return).
+#pragma once
+
+#include <atomic>
+#include <functional>
+#include <memory>
+#include <vector>
+
+#include "cache_hashtable.h"
+#include "common.h"
+#include "profiler.h"
+#include "run_config.h"
+#include "ugache_hip.h"
+
+namespace coll_cache_lib {
+
+using namespace common;
+
+class CollCache;
+class ExtractSession;
+class RefreshSession;
+
+class CacheContext {
+ public:
+  std::atomic<size_t> progress{0};  // completed lookups; refresh waits on it (cache_context.h:258)
+
+ private:
+  BarHandle _barrier;
+  Context _trainer_ctx;
+  DataType _dtype = kF32;
+  size_t _dim = 0;
+  size_t _row_bytes = 0;
+  int _num_location = -1;
+  int _cpu_location_id = -1;
+  int _local_location_id = -1;
+  size_t _cache_nbytes = 0;
+  size_t _cache_nodes = 0;
+  size_t _cache_space_capacity = 0;  // rows
+  size_t _num_total_nodes = 0;
+  std::shared_ptr<CollCache> _coll_cache;
+  CacheEntryManager *_new_hash_table = nullptr;
+  // per location: [local] = cache in HBM, [cpu] = host table (cache_context.h:285)
+  std::vector<void *> _device_cache_data;
+  MemHandle _device_cache_data_local_handle;
+  std::function<MemHandle(size_t)> _gpu_mem_allocator;
+  std::function<MemHandle(size_t)> _eager_gpu_mem_allocator;
+
+  friend class ExtractSession;
+  friend class RefreshSession;
+  friend class CollCache;
+
+  inline bool IsDirectMapping() { return _new_hash_table == nullptr; }
+
+  void build_no_cache(int location_id, std::shared_ptr<CollCache> coll_cache_ptr, void *cpu_data, DataType dtype,
+                      size_t dim, Context gpu_ctx, StreamHandle stream = nullptr);
+  void build_full_cache(int location_id, std::shared_ptr<CollCache> coll_cache_ptr, void *cpu_data, DataType dtype,
+                        size_t dim, Context gpu_ctx, size_t num_total_nodes, StreamHandle stream = nullptr);
+  void build_with_advise_new_hash(int location_id, std::shared_ptr<CollCache> coll_cache_ptr, void *cpu_data,
+                                  DataType dtype, size_t dim, Context gpu_ctx, double cache_percentage,
+                                  StreamHandle stream = nullptr);
+
+ public:
+  CacheContext(BarHandle barrier) : _barrier(barrier) {}
+  ~CacheContext();
+  void build(std::function<MemHandle(size_t)> gpu_mem_allocator, int location_id,
+             std::shared_ptr<CollCache> coll_cache_ptr, void *cpu_data, DataType dtype, size_t dim, Context gpu_ctx,
+             double cache_percentage, StreamHandle stream = nullptr);
+  // introspection used by tests and reports
+  size_t CacheCapacityRows() const { return _cache_space_capacity; }
+  size_t CachedRows() const { return _cache_nodes; }
+  size_t RowBytes() const { return _row_bytes; }
+  int TableKind() const { return _new_hash_table ? _new_hash_table->_table.kind : 0; }
+  const CacheEntryManager *EntryManager() const { return _new_hash_table; }
+};
+
+class ExtractSession {
+  std::shared_ptr<CacheContext> _cache_ctx;
+  MemHandle _idx_handle;          // ugk_idx_t[n], from the caller's allocator, regrown on demand
+  MemHandle _state_handle;        // device: two counter pairs + status word
+  MemHandle _host_mirror_handle;  // pinned host: counters + status of the last lookup
+  uint32_t *_counts[2] = {nullptr, nullptr};
+  uint32_t *_status = nullptr;
+  uint32_t *_host_mirror = nullptr;
+  int _cur = 0;
+  StreamHandle _local_ext_stream = nullptr;
+  StreamHandle _cpu_ext_stream = nullptr;
+  void *_ev_classified = nullptr, *_ev_local_done = nullptr, *_ev_cpu_done = nullptr;
+  void *_ev_t[4] = {nullptr, nullptr, nullptr, nullptr};
+  unsigned _cpu_blocks = 32;
+  uint32_t _group_offset[3] = {0, 0, 0};
+
+  template <typename KeyT>
+  void ExtractFeatImpl(const KeyT *nodes, size_t num_nodes, void *output, StreamHandle stream, uint64_t task_key);
+  void EnsureIdx(size_t num_nodes);
+  void CheckStatusWord(uint32_t st) const;
+
+ public:
+  ExtractSession(std::shared_ptr<CacheContext> cache_ctx);
+  ~ExtractSession();
+  // cache_context.h:510.  nodes: device pointer to num_nodes keys; output: device [num_nodes, dim]; blocking.
+  void ExtractFeat(const IdType *nodes, const size_t num_nodes, void *output, StreamHandle stream,
+                   uint64_t task_key);
+  // same for 64-bit keys (dense ids below num_total_item); an extension over the reference
+  void ExtractFeat64(const Id64Type *nodes, const size_t num_nodes, void *output, StreamHandle stream,
+                     uint64_t task_key);
+  // {0, #local, n} of the last lookup — the reference's group_offset (cache_context.cu:825-847)
+  const uint32_t *LastGroupOffset() const { return _group_offset; }
+};
+
+class RefreshSession {
+ public:
+  StreamHandle stream = nullptr;
+  StreamHandle low_pri_stream = nullptr;  // a second default-priority stream: row copies of the refresh
+  std::shared_ptr<CacheContext> _cache_ctx;
+  void refresh_after_solve_main(bool foreground);
+  ~RefreshSession();
+
+ private:
+  void refresh_after_solve_new(bool foreground);
+  TensorPtr Empty1DReuse(TensorPtr &preserved_buffer, DataType dtype, std::vector<size_t> shape, Context ctx);
+  TensorPtr CopyTo1DReuse(TensorPtr &preserved_buffer, TensorPtr src, Context ctx, StreamHandle stream);
+  TensorPtr __keys_buffer;
+  TensorPtr __offs_buffer;
+  MemHandle _status_handle;
+};
+
+}  // namespace coll_cache_lib

@@ -1,0 +1,103 @@
+// Host-side owner of the GPU lookup table and of the cache-slot bookkeeping.  Same role and method names as
+// CacheEntryManager in the reference (coll_cache_lib/cuda/cache_hashtable.cuh:529-849); the table itself
+// lives behind the C-ABI of ugache_hip.h (flat table for dense ids, open addressing otherwise).
+#pragma once
+
+#include <cmath>
+#include <cstring>
+#include <functional>
+#include <vector>
+
+#include "common.h"
+#include "logging.h"
+#include "run_config.h"
+#include "ugache_hip.h"
+
+namespace coll_cache_lib {
+namespace common {
+
+constexpr IdType kEmptyPos = 0xffffffff;  // cache_hashtable.h:17
+
+// packed (location, offset) value of the flat table, identical to cache_hashtable.h:20-28
+struct EmbCacheOff {
+  IdType data;
+  EmbCacheOff(IdType loc, IdType off) { data = (loc << 28) + off; }
+  IdType loc() const { return (data >> 28) & 0x0f; }
+  IdType off() const { return data & 0x0fffffff; }
+};
+
+// cache_hashtable.cu:222-225; kept for the flat-vs-open-addressing decision rule
+inline size_t TableSize(const size_t num, const size_t scale = 2) {
+  const size_t next_pow2 = (size_t)1 << static_cast<size_t>(1 + std::log2((double)(num >> 1)));
+  return next_pow2 << scale;
+}
+
+class CacheEntryManager {
+ public:
+  TensorPtr _cached_keys;   // host, u32: keys currently cached on this GPU
+  TensorPtr _remote_keys;   // always empty with one GPU
+  TensorPtr _free_offsets;  // host, u32: free cache slots, allocation sized for the whole capacity
+  ugk_table_t _table = {0, 0, nullptr, 0};
+  MemHandle _table_handle;
+  MemHandle _status_handle;  // device status word for maintenance kernels
+  IdType _cache_space_capacity = 0;
+  size_t num_total_key = 0;
+  int cpu_location_id = 1;
+  int _device_id = 0;
+  TensorPtr _keys_for_each_src[9];
+
+  // allocate and clear the table (FlatHashTable / SimpleHashTable ctors, cache_hashtable.cu:432-457, 588-607)
+  void CreateFlat(const std::function<MemHandle(size_t)> &allocator, size_t num_keys, StreamHandle stream);
+  void CreateHash(const std::function<MemHandle(size_t)> &allocator, size_t num_entries, StreamHandle stream);
+
+  // cuh:574-582 — off[i] = slot of keys[i] (the key itself when absent); tensors are device memory
+  void LookupOffset(TensorPtr keys, TensorPtr off, StreamHandle stream);
+  // cuh:601-608
+  void InsertWithLoc(TensorPtr keys, TensorPtr off, int loc, StreamHandle stream);
+  void InsertSeqOffWithLoc(TensorPtr keys, int loc, StreamHandle stream);
+  // cuh:622-625
+  void Evict(TensorPtr keys_to_evict, StreamHandle stream);
+  // cuh:635-655 — free-list: returned offsets go to the back, reservations come from the front
+  void ReturnOffset(TensorPtr new_offsets);
+  TensorPtr ReserveOffsetFront(IdType num_new_insert_keys);
+  // aborts if a maintenance kernel flagged an error (duplicate insert, absent evict, full table ...)
+  void CheckStatus(StreamHandle stream, const char *what);
+
+  // cuh:693-740 — keys of `inputs` satisfying cond, in input order (deterministic, unlike the reference's
+  // thread-interleaved order)
+  template <typename InputIterator, typename CondT>
+  TensorPtr DetectKeysWithCond(InputIterator inputs, size_t num_input, CondT cond, size_t max_result_storage = 0) {
+    const int nthr = std::max(1, RunConfig::solver_omp_thread_num_per_gpu);
+    std::vector<size_t> counts(nthr + 1, 0);
+    const size_t chunk = (num_input + nthr - 1) / nthr;
+#pragma omp parallel for num_threads(nthr) schedule(static, 1)
+    for (int t = 0; t < nthr; t++) {
+      size_t c = 0;
+      const size_t lo = std::min(num_input, chunk * t), hi = std::min(num_input, chunk * (t + 1));
+      for (size_t i = lo; i < hi; i++) c += cond(inputs[i]) ? 1 : 0;
+      counts[t + 1] = c;
+    }
+    for (int t = 0; t < nthr; t++) counts[t + 1] += counts[t];
+    const size_t total = counts[nthr];
+    if (max_result_storage != 0) CHECK_LE(total, max_result_storage);
+    TensorPtr out = Tensor::Empty(kI32, {total}, CPU_CLIB(), "");
+    IdType *dst = out->Ptr<IdType>();
+#pragma omp parallel for num_threads(nthr) schedule(static, 1)
+    for (int t = 0; t < nthr; t++) {
+      size_t pos = counts[t];
+      const size_t lo = std::min(num_input, chunk * t), hi = std::min(num_input, chunk * (t + 1));
+      for (size_t i = lo; i < hi; i++)
+        if (cond(inputs[i])) dst[pos++] = inputs[i];
+    }
+    return out;
+  }
+
+  // cuh:741-835 — per-source key lists from nid_to_block + this GPU's line of the access advise.
+  // node_list_of_src[dev] is filled for dev in [0, num_gpu); keys whose source is the host are not listed.
+  static void DetectKeysForAllSource(TensorPtr nid_to_block, TensorPtr block_access_advise, int local_location_id,
+                                     TensorPtr block_density, size_t num_total_item, TensorPtr *node_list_of_src,
+                                     int num_gpu = 1);
+};
+
+}  // namespace common
+}  // namespace coll_cache_lib

@@ -1,0 +1,198 @@
+#include "facade.h"
+
+#include <iostream>
+
+#include "logging.h"
+#include "placement.h"
+#include "run_config.h"
+#include "timer.h"
+
+namespace coll_cache_lib {
+
+// facade.cc:74-88
+void CollCache::lookup(int replica_id, const IdType *nodes, const size_t num_nodes, void *output,
+                       StreamHandle stream, uint64_t step_key) {
+  Timer t;
+  CHECK_LT((size_t)replica_id, _session_list.size());
+  _session_list[replica_id]->ExtractFeat(nodes, num_nodes, output, stream, step_key);
+  _profiler->LogStep(step_key, common::kLogL2CacheCopyTime, t.Passed());
+}
+
+void CollCache::lookup64(int replica_id, const Id64Type *nodes, const size_t num_nodes, void *output,
+                         StreamHandle stream, uint64_t step_key) {
+  Timer t;
+  CHECK_LT((size_t)replica_id, _session_list.size());
+  _session_list[replica_id]->ExtractFeat64(nodes, num_nodes, output, stream, step_key);
+  _profiler->LogStep(step_key, common::kLogL2CacheCopyTime, t.Passed());
+}
+
+namespace {
+// every policy of the reference that runs a solver (facade.cc:110-152) reduces to the frequency-ranked
+// placement when there is one GPU
+void CheckPolicy() {
+  switch (RunConfig::cache_policy) {
+    case kRepCache:
+    case kPartRepCache:
+    case kPartitionCache:
+    case kCollCacheIntuitive:
+    case kCollCache:
+    case kCollCacheAsymmLink:
+    case kCollFineGrain:
+    case kCliquePart:
+      return;
+    default:
+      LOG(FATAL) << "cache policy " << (int)RunConfig::cache_policy << " has no solver";
+  }
+}
+}  // namespace
+
+// facade.cc:93-160
+void CollCache::solve_impl_master(IdType *ranking_nodes_list_ptr, IdType *ranking_nodes_freq_list_ptr,
+                                  IdType num_node) {
+  CheckPolicy();
+  std::vector<int> trainer_to_stream(RunConfig::num_device, 0);
+  std::vector<coll_cache::PerT> trainer_cache_percent(RunConfig::num_device, RunConfig::cache_percentage * 100);
+  auto ranking_nodes_list =
+      Tensor::FromBlob(ranking_nodes_list_ptr, kI32, {1, (size_t)num_node}, CPU(CPU_FOREIGN), "ranking_nodes_list");
+  auto ranking_nodes_freq_list = Tensor::FromBlob(ranking_nodes_freq_list_ptr, kI32, {1, (size_t)num_node},
+                                                  CPU(CPU_FOREIGN), "ranking_nodes_freq_list");
+  coll_cache::FreqRankSolver solver;
+  _nid_to_block = Tensor::Empty(kI32, {(size_t)num_node}, CPU_CLIB(), "nid_to_block");
+  solver.Build(ranking_nodes_list, ranking_nodes_freq_list, trainer_to_stream, num_node, _nid_to_block);
+  solver.Solve(trainer_to_stream, trainer_cache_percent, "BIN", RunConfig::coll_cache_hyperparam_T_local,
+               RunConfig::coll_cache_hyperparam_T_cpu);
+  _block_placement = solver.block_placement;
+  _block_access_advise = solver.block_access_from;
+  _block_density = solver.block_density_tensor;
+}
+
+// facade.cc:161-236
+void CollCache::solve_impl_master(ContFreqBuf *freq_rank, IdType num_node) {
+  CheckPolicy();
+  std::vector<int> trainer_to_stream(RunConfig::num_device, 0);
+  std::vector<coll_cache::PerT> trainer_cache_percent(RunConfig::num_device, RunConfig::cache_percentage * 100);
+  coll_cache::FreqRankSolver solver;
+  _nid_to_block = Tensor::Empty(kI32, {(size_t)num_node}, CPU_CLIB(), "nid_to_block");
+  solver.BuildSingleStream(freq_rank, trainer_to_stream, num_node, _nid_to_block);
+  solver.Solve(trainer_to_stream, trainer_cache_percent, "BIN", RunConfig::coll_cache_hyperparam_T_local,
+               RunConfig::coll_cache_hyperparam_T_cpu);
+  _block_placement = solver.block_placement;
+  _block_access_advise = solver.block_access_from;
+  _block_density = solver.block_density_tensor;
+}
+
+void CollCache::build_common(int replica_id, std::function<void()> solve, IdType num_node,
+                             std::function<MemHandle(size_t)> gpu_mem_allocator, void *cpu_data, DataType dtype,
+                             size_t dim, double cache_percentage, StreamHandle stream) {
+  CHECK_EQ(replica_id, 0) << "this build serves one replica on one GPU";
+  CHECK_EQ(RunConfig::num_device, (size_t)1) << "num_device must be 1";
+  if (RunConfig::device_id_list.empty()) RunConfig::device_id_list = {0};
+  const int device_id = RunConfig::device_id_list[replica_id];
+  RunConfig::LoadConfigFromEnv();
+  RunConfig::num_total_item = num_node;
+  RunConfig::cache_percentage = cache_percentage;
+  // rows are handled as opaque bytes; keep the reference's re-expression in 16-byte units for its logs
+  // (facade.cc:457-465)
+  if (RunConfig::coll_cache_scale_nb != 0) {
+    const size_t emb_vec_nb = GetDataTypeBytes(dtype) * dim;
+    if (emb_vec_nb >= RunConfig::coll_cache_scale_nb && emb_vec_nb % RunConfig::coll_cache_scale_nb == 0) {
+      dim = emb_vec_nb / RunConfig::coll_cache_scale_nb;
+      dtype = nb_to_dt(RunConfig::coll_cache_scale_nb);
+    }
+  }
+  RunConfig::coll_cache_link_desc = coll_cache::AsymmLinkDesc::AutoBuild(GPU(device_id));
+  this->_cache_ctx_list.resize(RunConfig::num_device);
+  this->_session_list.resize(RunConfig::num_device);
+  this->_refresh_session_list.resize(RunConfig::num_device);
+  RunConfig::solver_omp_thread_num = RunConfig::omp_thread_num;
+  RunConfig::solver_omp_thread_num_per_gpu = std::max<int>(1, RunConfig::omp_thread_num / (int)RunConfig::num_device);
+
+  const bool need_solver = (cache_percentage != 0 && cache_percentage != 1);
+  if (need_solver) solve();
+  this->_replica_barrier->Wait();
+
+  auto cache_ctx = std::make_shared<CacheContext>(_replica_barrier);
+  Context gpu_ctx = GPU(device_id);
+  cache_ctx->build(gpu_mem_allocator, replica_id, this->shared_from_this(), cpu_data, dtype, dim, gpu_ctx,
+                   cache_percentage, stream);
+  UGK_CALL(ugk_stream_sync(stream));
+  this->_cache_ctx_list[replica_id] = cache_ctx;
+  this->_session_list[replica_id] = std::make_shared<ExtractSession>(cache_ctx);
+  this->_refresh_session_list[replica_id] = std::make_shared<RefreshSession>();
+  this->_refresh_session_list[replica_id]->_cache_ctx = cache_ctx;
+  this->_refresh_session_list[replica_id]->stream = stream;
+  this->_replica_barrier->Wait();
+  RunConfig::solver_omp_thread_num = RunConfig::refresher_omp_thread_num;
+  RunConfig::solver_omp_thread_num_per_gpu = RunConfig::refresher_omp_thread_num_per_gpu;
+}
+
+// facade.cc:283-381
+void CollCache::build_v2(int replica_id, IdType *ranking_nodes_list_ptr, IdType *ranking_nodes_freq_list_ptr,
+                         IdType num_node, std::function<MemHandle(size_t)> gpu_mem_allocator, void *cpu_data,
+                         DataType dtype, size_t dim, double cache_percentage, StreamHandle stream) {
+  build_common(
+      replica_id,
+      [&]() { solve_impl_master(ranking_nodes_list_ptr, ranking_nodes_freq_list_ptr, num_node); }, num_node,
+      gpu_mem_allocator, cpu_data, dtype, dim, cache_percentage, stream);
+}
+
+// facade.cc:430-511
+void CollCache::build_v2(int replica_id, ContFreqBuf *freq_rank, IdType num_node,
+                         std::function<MemHandle(size_t)> gpu_mem_allocator, void *cpu_data, DataType dtype,
+                         size_t dim, double cache_percentage, StreamHandle stream) {
+  build_common(
+      replica_id, [&]() { solve_impl_master(freq_rank, num_node); }, num_node, gpu_mem_allocator, cpu_data, dtype,
+      dim, cache_percentage, stream);
+}
+
+void CollCache::preserve_old_solution() {
+  this->_old_block_access_advise = this->_block_access_advise;
+  this->_old_block_density = this->_block_density;
+  this->_old_block_placement = this->_block_placement;
+  this->_old_nid_to_block = this->_nid_to_block;
+  this->_block_access_advise = nullptr;
+  this->_block_density = nullptr;
+  this->_block_placement = nullptr;
+  this->_nid_to_block = nullptr;
+}
+
+// facade.cc:383-428
+void CollCache::refresh(int replica_id, IdType *ranking_nodes_list_ptr, IdType *ranking_nodes_freq_list_ptr,
+                        StreamHandle stream, bool foreground) {
+  CHECK_EQ(replica_id, 0);
+  CHECK_NOTNULL(_nid_to_block) << "refresh needs a cache built with 0 < cache_percentage < 1";
+  AnonymousBarrier::_refresh_instance->Wait();
+  preserve_old_solution();
+  solve_impl_master(ranking_nodes_list_ptr, ranking_nodes_freq_list_ptr, (IdType)RunConfig::num_total_item);
+  AnonymousBarrier::_refresh_instance->Wait();
+  this->_refresh_session_list[replica_id]->stream = stream;
+  this->_refresh_session_list[replica_id]->refresh_after_solve_main(foreground);
+  AnonymousBarrier::_refresh_instance->Wait();
+}
+
+// facade.cc:513-557
+void CollCache::refresh(int replica_id, ContFreqBuf *freq_rank, StreamHandle stream, bool foreground) {
+  CHECK_EQ(replica_id, 0);
+  CHECK_NOTNULL(_nid_to_block) << "refresh needs a cache built with 0 < cache_percentage < 1";
+  AnonymousBarrier::_refresh_instance->Wait();
+  preserve_old_solution();
+  solve_impl_master(freq_rank, (IdType)RunConfig::num_total_item);
+  AnonymousBarrier::_refresh_instance->Wait();
+  this->_refresh_session_list[replica_id]->stream = stream;
+  this->_refresh_session_list[replica_id]->refresh_after_solve_main(foreground);
+  AnonymousBarrier::_refresh_instance->Wait();
+}
+
+void CollCache::report_last_epoch(uint64_t epoch) { _profiler->ReportStepAverageLastEpoch(epoch + 1, 0); }
+
+void CollCache::report_avg() {
+  _profiler->ReportStepAverage(RunConfig::num_epoch - 1, RunConfig::num_global_step_per_epoch - 1);
+  std::cout.flush();
+}
+
+void CollCache::report(uint64_t key) {
+  _profiler->ReportStep(RunConfig::GetEpochFromKey(key), RunConfig::GetStepFromKey(key));
+  std::cout.flush();
+}
+
+}  // namespace coll_cache_lib

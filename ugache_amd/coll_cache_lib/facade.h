@@ -1,0 +1,89 @@
+// The process-wide cache manager: same class, methods and argument meaning as coll_cache_lib/facade.h:17-82 of
+// the reference.  One CollCache per process, one replica per GPU (this build: one replica).
+#pragma once
+
+#include <functional>
+#include <memory>
+#include <vector>
+
+#include "cache_context.h"
+#include "common.h"
+#include "freq_recorder.h"
+#include "profiler.h"
+
+namespace coll_cache_lib {
+
+using namespace common;
+
+class CollCache : public std::enable_shared_from_this<CollCache> {
+ private:
+  TensorPtr _nid_to_block;
+  TensorPtr _block_density;
+  TensorPtr _block_placement;
+  TensorPtr _block_access_advise;
+  TensorPtr _old_nid_to_block;
+  TensorPtr _old_block_density;
+  TensorPtr _old_block_placement;
+  TensorPtr _old_block_access_advise;
+  BarHandle _process_barrier;
+  BarHandle _replica_barrier;
+  friend class CacheContext;
+  friend class RefreshSession;
+  friend class ExtractSession;
+  std::vector<std::shared_ptr<CacheContext>> _cache_ctx_list;
+  std::vector<std::shared_ptr<ExtractSession>> _session_list;
+  std::vector<std::shared_ptr<RefreshSession>> _refresh_session_list;
+  void solve_impl_master(IdType *ranking_nodes_list_ptr, IdType *ranking_nodes_freq_list_ptr, IdType num_node);
+  void solve_impl_master(ContFreqBuf *freq_rank, IdType num_node);
+  void preserve_old_solution();
+  void build_common(int replica_id, std::function<void()> solve, IdType num_node,
+                    std::function<MemHandle(size_t)> gpu_mem_allocator, void *cpu_data, DataType dtype, size_t dim,
+                    double cache_percentage, StreamHandle stream);
+
+ public:
+  CollCache(BarHandle process_barrier, BarHandle replica_barrier)
+      : _process_barrier(process_barrier), _replica_barrier(replica_barrier), _profiler(std::make_shared<Profiler>()) {}
+
+  // nodes / output are device pointers; blocking: output is complete on return (facade.cc:74-88)
+  void lookup(int replica_id, const IdType *nodes, const size_t num_nodes, void *output, StreamHandle stream,
+              uint64_t step_key);
+  // 64-bit keys, dense ids (extension)
+  void lookup64(int replica_id, const Id64Type *nodes, const size_t num_nodes, void *output, StreamHandle stream,
+                uint64_t step_key);
+
+  // rank list + frequency list over all num_node keys (facade.cc:283-381)
+  void build_v2(int replica_id, IdType *ranking_nodes_list_ptr, IdType *ranking_nodes_freq_list_ptr, IdType num_node,
+                std::function<MemHandle(size_t)> gpu_mem_allocator, void *cpu_data, DataType dtype, size_t dim,
+                double cache_percentage, StreamHandle stream = nullptr);
+  // observed keys only, in rank order (facade.cc:430-511)
+  void build_v2(int replica_id, ContFreqBuf *freq_rank, IdType num_node,
+                std::function<MemHandle(size_t)> gpu_mem_allocator, void *cpu_data, DataType dtype, size_t dim,
+                double cache_percentage, StreamHandle stream = nullptr);
+  // re-place by new hotness, evict + insert (facade.cc:383-428, 513-557)
+  void refresh(int replica_id, IdType *ranking_nodes_list_ptr, IdType *ranking_nodes_freq_list_ptr,
+               StreamHandle stream = nullptr, bool foreground = false);
+  void refresh(int replica_id, ContFreqBuf *freq_rank, StreamHandle stream = nullptr, bool foreground = false);
+
+  void report_avg();
+  void report_last_epoch(uint64_t epoch);
+  void report(uint64_t key);
+  std::shared_ptr<Profiler> _profiler;
+
+  inline void set_step_profile_value(uint64_t key, LogStepItem item, double val) { _profiler->LogStep(key, item, val); }
+  inline void add_epoch_profile_value(uint64_t key, LogEpochItem item, double val) {
+    _profiler->LogEpochAdd(key, item, val);
+  }
+
+  // drops the per-replica objects (they hold a reference back to this object)
+  void release_replicas() {
+    _refresh_session_list.clear();
+    _session_list.clear();
+    _cache_ctx_list.clear();
+  }
+  // introspection (tests, reports)
+  std::shared_ptr<CacheContext> cache_ctx(int replica_id) { return _cache_ctx_list.at(replica_id); }
+  std::shared_ptr<ExtractSession> session(int replica_id) { return _session_list.at(replica_id); }
+  TensorPtr nid_to_block() { return _nid_to_block; }
+};
+
+}  // namespace coll_cache_lib

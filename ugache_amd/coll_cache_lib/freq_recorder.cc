@@ -1,0 +1,115 @@
+#include "freq_recorder.h"
+
+#include <algorithm>
+#include <cstring>
+#include <limits>
+#include <parallel/algorithm>
+
+#include "logging.h"
+#include "run_config.h"
+
+namespace coll_cache_lib {
+namespace common {
+
+void ContFreqBuf::add(const IdType &key, const CntT &cnt) {
+  for (auto &e : entries) {
+    if (e.key == key) {
+      e.cnt += cnt;
+      return;
+    }
+  }
+  entries.push_back({key, cnt});
+  buf = entries.data();
+}
+
+CntT ContFreqBuf::get(const IdType &key) const {
+  for (auto &e : entries)
+    if (e.key == key) return e.cnt;
+  return 0;
+}
+
+void ContFreqBuf::sort_desc() {
+  uint64_t *w = reinterpret_cast<uint64_t *>(entries.data());
+  __gnu_parallel::sort(w, w + entries.size(), std::greater<uint64_t>());
+  buf = entries.data();
+}
+
+void ContFreqBuf::GetLegacyFreqRank(LegacyFreqBuf *output, size_t total_num_node) const {
+  output->rank_vec.resize(total_num_node);
+  output->freq_vec.assign(total_num_node, 0);
+  std::vector<uint8_t> seen(total_num_node, 0);
+  const size_t m = entries.size();
+  CHECK_LE(m, total_num_node);
+  for (size_t r = 0; r < m; r++) {
+    CHECK_LT(entries[r].key, total_num_node);
+    output->rank_vec[r] = entries[r].key;
+    output->freq_vec[r] = entries[r].cnt;
+    seen[entries[r].key] = 1;
+  }
+  size_t pos = m;
+  for (size_t k = 0; k < total_num_node; k++)
+    if (!seen[k]) output->rank_vec[pos++] = (uint32_t)k;
+  CHECK_EQ(pos, total_num_node);
+}
+
+FreqRecorder::FreqRecorder(size_t num_nodes, int local_id) : _num_nodes(num_nodes), _local_id(local_id) {
+  CHECK(num_nodes < std::numeric_limits<IdType>::max() / 2);
+  _live.assign(num_nodes, 0);
+  global_cont_freq_buf = new ContFreqBuf;
+}
+
+FreqRecorder::~FreqRecorder() { delete global_cont_freq_buf; }
+
+template <typename KeyT>
+void FreqRecorder::Record(const KeyT *input, size_t num_inputs) {
+  std::lock_guard<std::mutex> g(_mu);
+  CntT *cnt = _live.data();
+  const size_t n_nodes = _num_nodes;
+  bool bad = false;
+#pragma omp parallel for num_threads(RunConfig::solver_omp_thread_num_per_gpu) reduction(|| : bad) if (num_inputs > 65536)
+  for (size_t i = 0; i < num_inputs; i++) {
+    const uint64_t k = (uint64_t)input[i];
+    if (k >= n_nodes) {
+      bad = true;
+      continue;
+    }
+    __atomic_fetch_add(&cnt[k], 1u, __ATOMIC_RELAXED);
+  }
+  CHECK(!bad) << "FreqRecorder::Record: a key is not below num_total_item=" << n_nodes;
+}
+template void FreqRecorder::Record<Id64Type>(const Id64Type *input, size_t num_inputs);
+template void FreqRecorder::Record<IdType>(const IdType *input, size_t num_inputs);
+
+void FreqRecorder::LocalCombineToShared() {
+  std::lock_guard<std::mutex> g(_mu);
+  if (_shared.empty()) {
+    _shared.swap(_live);
+    _live.assign(_num_nodes, 0);
+  } else {
+    for (size_t i = 0; i < _num_nodes; i++) _shared[i] += _live[i];
+    std::fill(_live.begin(), _live.end(), 0);
+  }
+}
+
+void FreqRecorder::GlobalCombine() {
+  std::lock_guard<std::mutex> g(_mu);
+  auto &e = global_cont_freq_buf->entries;
+  e.clear();
+  for (size_t k = 0; k < _shared.size(); k++)
+    if (_shared[k]) e.push_back({(IdType)k, _shared[k]});
+  global_cont_freq_buf->buf = e.data();
+  LOG(INFO) << "freq recorder global combine: " << e.size() << " distinct keys";
+  _shared.clear();
+  _shared.shrink_to_fit();
+}
+
+void FreqRecorder::Sort() {
+  global_cont_freq_buf->sort_desc();
+  auto &e = global_cont_freq_buf->entries;
+  if (e.size() >= 5)
+    LOG(INFO) << "top 5 freq is " << e[0].cnt << "," << e[1].cnt << "," << e[2].cnt << "," << e[3].cnt << ","
+              << e[4].cnt;
+}
+
+}  // namespace common
+}  // namespace coll_cache_lib

@@ -1,0 +1,65 @@
+// Hotness counting on the host: the input of the frequency-ranked cache fill and of refresh.
+// Same role and call sequence as coll_cache_lib/freq_recorder.{h,cc} of the reference
+// (Record -> LocalCombineToShared -> GlobalCombine -> Sort, freq_recorder.cc:227-293) and the same rank order:
+// entries {key, cnt} compared as the 64-bit word (cnt << 32 | key), descending, i.e. higher count first and,
+// among equal counts, the larger key first.  Keys are dense ids below num_nodes, so counts live in one flat
+// array updated with atomic adds instead of per-thread hash maps.
+#pragma once
+
+#include <cstdint>
+#include <mutex>
+#include <vector>
+
+#include "common.h"
+
+namespace coll_cache_lib {
+namespace common {
+
+using CntT = IdType;
+using OffT = uint32_t;
+
+struct FreqEntry {
+  IdType key;
+  CntT cnt;
+};
+static_assert(sizeof(FreqEntry) == 8, "FreqEntry is sorted as one 64-bit word");
+
+struct LegacyFreqBuf {
+  std::vector<uint32_t> rank_vec, freq_vec;
+};
+
+// Distinct observed keys with their counts; after FreqRecorder::Sort() in rank order.
+struct ContFreqBuf {
+  std::vector<FreqEntry> entries;
+  FreqEntry *buf = nullptr;  // == entries.data()
+  size_t size() const { return entries.size(); }
+  void add(const IdType &key, const CntT &cnt);  // linear probe over `entries`; for small hand-built buffers
+  CntT get(const IdType &key) const;
+  // all num_node keys in rank order: observed keys first, then the never-seen ones in ascending key order
+  // (the reference appends them in a thread-dependent order, freq_recorder.cc:305-333)
+  void GetLegacyFreqRank(LegacyFreqBuf *output, size_t total_num_node) const;
+  void sort_desc();
+};
+
+class FreqRecorder {
+ public:
+  FreqRecorder(size_t num_nodes, int local_id);
+  ~FreqRecorder();
+  template <typename KeyT>
+  void Record(const KeyT *inputs, size_t num_input);
+  void LocalCombineToShared();
+  void GlobalCombine();
+  void Sort();
+  inline size_t NumNodes() const { return _num_nodes; }
+  ContFreqBuf *global_cont_freq_buf;
+
+ private:
+  size_t _num_nodes;
+  int _local_id;
+  std::vector<CntT> _live;    // counts being recorded
+  std::vector<CntT> _shared;  // counts handed over by LocalCombineToShared
+  std::mutex _mu;
+};
+
+}  // namespace common
+}  // namespace coll_cache_lib

@@ -1,0 +1,336 @@
+// The extern "C" shim over the facade: the counterpart of python/collcache/common/operation.cc.
+#include "operation.h"
+
+#include <sys/wait.h>
+
+#include <cstring>
+#include <iostream>
+#include <string>
+#include <unordered_map>
+
+#include "facade.h"
+#include "freq_recorder.h"
+#include "logging.h"
+#include "placement.h"
+#include "profiler.h"
+#include "run_config.h"
+#include "ugache_hip.h"
+
+namespace coll_cache_lib {
+namespace common {
+
+namespace {
+std::shared_ptr<CollCache> _coll_cache = nullptr;
+std::shared_ptr<Profiler> _profiler = nullptr;
+std::vector<std::shared_ptr<FreqRecorder>> _freq_recorder;
+size_t steps[9] = {0};
+size_t internal_feat_dim = 0;
+size_t outside_feat_dim = 0;
+
+class CallbackMemHandle : public ExternelGPUMemoryHandler {
+ public:
+  void *ptr_ = nullptr;
+  size_t nbytes_ = 0;
+  coll_cache_release_fn release_ = nullptr;
+  void *user_ = nullptr;
+  ~CallbackMemHandle() override {
+    if (release_ && ptr_) release_(ptr_, user_);
+  }
+  void *ptr() override { return ptr_; }
+  size_t nbytes() override { return nbytes_; }
+};
+
+std::function<MemHandle(size_t)> MakeAllocator(coll_cache_alloc_fn alloc, coll_cache_release_fn release, void *user,
+                                               int replica_id) {
+  if (alloc == nullptr) {
+    const int dev = RunConfig::device_id_list.empty() ? 0 : RunConfig::device_id_list[replica_id];
+    return [dev](size_t nbytes) -> MemHandle { return EagerGPUAlloc(dev, nbytes); };
+  }
+  return [alloc, release, user](size_t nbytes) -> MemHandle {
+    auto h = std::make_shared<CallbackMemHandle>();
+    h->ptr_ = alloc(nbytes, user);
+    CHECK(h->ptr_ != nullptr || nbytes == 0) << "allocator callback returned NULL for " << nbytes << " bytes";
+    h->nbytes_ = nbytes;
+    h->release_ = release;
+    h->user_ = user;
+    return h;
+  };
+}
+
+void coll_cache_config_from_map(std::unordered_map<std::string, std::string> &configs) {
+  using CRC = RunConfig;
+  CHECK(!CRC::is_configured);
+  CHECK(configs.count("cache_percentage"));
+  CHECK(configs.count("_cache_policy"));
+  CHECK(configs.count("num_device"));
+  CHECK(configs.count("num_global_step_per_epoch"));
+  CHECK(configs.count("num_epoch"));
+  CHECK(configs.count("num_total_item"));
+  CHECK(configs.count("omp_thread_num"));
+
+  CRC::cache_percentage = std::stod(configs["cache_percentage"]);
+  CRC::cache_policy = static_cast<CachePolicy>(std::stoi(configs["_cache_policy"]));
+  CRC::cross_process = true;
+  CRC::num_device = std::stoull(configs["num_device"]);
+  CHECK_EQ(CRC::num_device, (size_t)1) << "this build serves one GPU: num_device must be 1";
+  CRC::device_id_list.resize(CRC::num_device);
+  for (size_t i = 0; i < CRC::num_device; i++) CRC::device_id_list[i] = (int)i;
+  CRC::num_global_step_per_epoch = std::stoull(configs["num_global_step_per_epoch"]);
+  CRC::num_epoch = std::stoull(configs["num_epoch"]);
+  CRC::num_total_item = std::stoull(configs["num_total_item"]);
+  CRC::omp_thread_num = std::stoi(configs["omp_thread_num"]);
+  CHECK_GT(CRC::omp_thread_num, 0);
+  CRC::solver_omp_thread_num = CRC::omp_thread_num;
+  CRC::solver_omp_thread_num_per_gpu = std::max<int>(1, CRC::omp_thread_num / (int)CRC::num_device);
+  CRC::is_configured = true;
+
+  _profiler = std::make_shared<Profiler>();
+  AnonymousBarrier::_global_instance->SetWorker((int)CRC::num_device);
+  AnonymousBarrier::_refresh_instance->SetWorker((int)CRC::num_device);
+  _coll_cache = std::make_shared<CollCache>(nullptr, AnonymousBarrier::_global_instance);
+  _coll_cache->_profiler = _profiler;
+}
+
+ContFreqBuf *CombineAndRank(int replica_id) {
+  CHECK_LT((size_t)replica_id, _freq_recorder.size()) << "coll_cache_record_init was not called";
+  CHECK_NOTNULL(_freq_recorder[replica_id]);
+  _freq_recorder[replica_id]->LocalCombineToShared();
+  AnonymousBarrier::_global_instance->Wait();
+  ContFreqBuf *freq_rank = nullptr;
+  if (replica_id == 0) {
+    _freq_recorder[0]->GlobalCombine();
+    _freq_recorder[0]->Sort();
+    freq_rank = _freq_recorder[0]->global_cont_freq_buf;
+  }
+  return freq_rank;
+}
+
+void NormalizeHalf(DataType &dtype, size_t &dim) {
+  outside_feat_dim = dim;
+  if (dtype == kF16) {  // operation.cc:132-136: the library moves bytes, fp16 rows travel as dim/2 fp32 words
+    CHECK(dim % 2 == 0);
+    dtype = kF32;
+    dim /= 2;
+  }
+  internal_feat_dim = dim;
+}
+
+}  // namespace
+
+size_t max_num_keys = 0;
+
+void coll_cache_init(int replica_id, size_t key_space_size, std::function<MemHandle(size_t)> allocator,
+                     void *cpu_data, DataType dtype, size_t dim, double cache_percentage, StreamHandle stream) {
+  CHECK(RunConfig::is_configured);
+  NormalizeHalf(dtype, dim);
+  ContFreqBuf *freq_rank = nullptr;
+  const bool need_rank = cache_percentage != 0 && cache_percentage != 1;
+  if (need_rank) freq_rank = CombineAndRank(replica_id);
+  _coll_cache->build_v2(replica_id, freq_rank, (IdType)key_space_size, allocator, cpu_data, dtype, dim,
+                        cache_percentage, stream);
+  LOG(INFO) << "coll cache has been initialized successfully";
+}
+
+extern "C" {
+
+void coll_cache_config(const char **config_keys, const char **config_values, const size_t num_config_items) {
+  CHECK(!RunConfig::is_configured);
+  std::unordered_map<std::string, std::string> configs;
+  for (size_t i = 0; i < num_config_items; i++) configs[std::string(config_keys[i])] = std::string(config_values[i]);
+  coll_cache_config_from_map(configs);
+}
+
+void coll_cache_log_step_by_key(uint64_t key, int item, double val) {
+  CHECK_NOTNULL(_profiler);
+  CHECK_LT(item, (int)kNumLogStepItems);
+  CHECK_GE(item, 0);
+  _profiler->LogStep(key, static_cast<LogStepItem>(item), val);
+}
+
+void coll_cache_report_step_by_key(uint64_t key) {
+  CHECK_NOTNULL(_profiler);
+  _profiler->ReportStep(RunConfig::GetEpochFromKey(key), RunConfig::GetStepFromKey(key));
+  std::cout.flush();
+}
+
+void coll_cache_report_step_average_by_key(uint64_t key) {
+  CHECK_NOTNULL(_profiler);
+  _profiler->ReportStepAverage(RunConfig::num_epoch - 1, RunConfig::num_global_step_per_epoch - 1);
+  _profiler->ReportStepItemPercentiles(RunConfig::num_epoch - 1, RunConfig::num_global_step_per_epoch - 1,
+                                       kLogL2CacheCopyTime, {50, 90, 95, 99, 99.9}, "tail_logl2featcopy");
+  std::cout.flush();
+}
+
+void coll_cache_record_init(int replica_id) {
+  CHECK(RunConfig::is_configured);
+  _freq_recorder.resize(RunConfig::num_device);
+  CHECK_LT((size_t)replica_id, _freq_recorder.size());
+  _freq_recorder[replica_id] = std::make_shared<FreqRecorder>(RunConfig::num_total_item, replica_id);
+}
+
+void coll_cache_train_barrier(void) { AnonymousBarrier::_global_instance->Wait(); }
+
+int coll_cache_wait_one_child(void) {
+  int child_stat = 0;
+  pid_t pid = waitpid(-1, &child_stat, 0);
+  if (pid < 0) return 0;
+  if (WIFSIGNALED(child_stat)) {
+    LOG(ERROR) << "detect an abnormal terminated child, signal is " << strsignal(WTERMSIG(child_stat));
+    return 1;
+  }
+  if (WEXITSTATUS(child_stat) != 0) {
+    LOG(ERROR) << "detect a terminated child " << pid << ", status is " << WEXITSTATUS(child_stat);
+    return 1;
+  }
+  return 0;
+}
+
+void coll_cache_print_memory_usage(void) {
+  size_t free_b = 0, total_b = 0;
+  UGK_CALL(ugk_mem_info(&free_b, &total_b));
+  std::cout << "[HIP] gpu: usage: " << ToReadableSize(total_b - free_b) << "\n";
+  std::cout.flush();
+}
+
+void coll_cache_lookup(int replica_id, uint32_t *key, size_t num_keys, void *output, StreamHandle stream) {
+  CHECK_NOTNULL(_coll_cache);
+  const uint64_t step_key = steps[replica_id] * RunConfig::num_device + replica_id;
+  steps[replica_id]++;
+  _coll_cache->lookup(replica_id, key, num_keys, output, stream, step_key);
+}
+
+void coll_cache_lookup_i64(int replica_id, const int64_t *key, size_t num_keys, void *output, StreamHandle stream) {
+  CHECK_NOTNULL(_coll_cache);
+  const uint64_t step_key = steps[replica_id] * RunConfig::num_device + replica_id;
+  steps[replica_id]++;
+  _coll_cache->lookup64(replica_id, key, num_keys, output, stream, step_key);
+}
+
+void coll_cache_record(int replica_id, uint32_t *key, size_t num_keys) {
+  CHECK_LT((size_t)replica_id, _freq_recorder.size()) << "coll_cache_record_init was not called";
+  _freq_recorder[replica_id]->Record(key, num_keys);
+  max_num_keys = std::max(max_num_keys, num_keys);
+}
+
+void coll_cache_record_i64(int replica_id, const int64_t *key, size_t num_keys) {
+  CHECK_LT((size_t)replica_id, _freq_recorder.size()) << "coll_cache_record_init was not called";
+  _freq_recorder[replica_id]->Record(key, num_keys);
+  max_num_keys = std::max(max_num_keys, num_keys);
+}
+
+void coll_cache_init_c(int replica_id, size_t key_space_size, coll_cache_alloc_fn alloc, coll_cache_release_fn release,
+                       void *user, void *cpu_data, int dtype, size_t dim, double cache_percentage,
+                       StreamHandle stream) {
+  CHECK(RunConfig::is_configured);
+  coll_cache_init(replica_id, key_space_size, MakeAllocator(alloc, release, user, replica_id), cpu_data,
+                  static_cast<DataType>(dtype), dim, cache_percentage, stream);
+}
+
+void coll_cache_init_ranked_c(int replica_id, size_t key_space_size, const uint32_t *rank_keys,
+                              const uint32_t *rank_freq, coll_cache_alloc_fn alloc, coll_cache_release_fn release,
+                              void *user, void *cpu_data, int dtype, size_t dim, double cache_percentage,
+                              StreamHandle stream) {
+  CHECK(RunConfig::is_configured);
+  DataType dt = static_cast<DataType>(dtype);
+  NormalizeHalf(dt, dim);
+  _coll_cache->build_v2(replica_id, const_cast<IdType *>(rank_keys), const_cast<IdType *>(rank_freq),
+                        (IdType)key_space_size, MakeAllocator(alloc, release, user, replica_id), cpu_data, dt, dim,
+                        cache_percentage, stream);
+}
+
+void coll_cache_refresh(int replica_id, StreamHandle stream, int foreground) {
+  CHECK_NOTNULL(_coll_cache);
+  ContFreqBuf *freq_rank = CombineAndRank(replica_id);
+  _coll_cache->refresh(replica_id, freq_rank, stream, foreground != 0);
+}
+
+void *coll_cache_alloc_host_table(size_t nbytes) {
+  void *p = nullptr;
+  UGK_CALL(ugk_host_malloc(&p, nbytes));
+  return p;
+}
+
+void coll_cache_free_host_table(void *ptr) { UGK_CALL(ugk_host_free(ptr)); }
+
+size_t coll_cache_max_num_keys(void) { return max_num_keys; }
+void coll_cache_set_max_num_keys(size_t n) { max_num_keys = n; }
+
+void coll_cache_last_group_offset(int replica_id, uint32_t out[3]) {
+  CHECK_NOTNULL(_coll_cache);
+  const uint32_t *g = _coll_cache->session(replica_id)->LastGroupOffset();
+  out[0] = g[0];
+  out[1] = g[1];
+  out[2] = g[2];
+}
+
+void coll_cache_get_info(int replica_id, uint64_t out[8]) {
+  CHECK_NOTNULL(_coll_cache);
+  auto ctx = _coll_cache->cache_ctx(replica_id);
+  memset(out, 0, 8 * sizeof(uint64_t));
+  out[0] = ctx->CacheCapacityRows();
+  out[1] = ctx->CachedRows();
+  out[2] = (uint64_t)ctx->TableKind();
+  out[3] = ctx->RowBytes();
+  out[4] = RunConfig::num_total_item;
+  out[5] = ctx->progress.load();
+  out[6] = ctx->EntryManager() ? ctx->EntryManager()->_free_offsets->NumItem() : 0;
+}
+
+size_t coll_cache_get_cached_keys(int replica_id, uint32_t *out, size_t capacity) {
+  CHECK_NOTNULL(_coll_cache);
+  auto mgr = _coll_cache->cache_ctx(replica_id)->EntryManager();
+  if (!mgr || !mgr->_cached_keys) return 0;
+  const size_t n = mgr->_cached_keys->NumItem();
+  if (out) memcpy(out, mgr->_cached_keys->Data(), std::min(n, capacity) * sizeof(uint32_t));
+  return n;
+}
+
+double coll_cache_get_step_value(uint64_t key, int item) {
+  CHECK_NOTNULL(_profiler);
+  CHECK(item >= 0 && item < (int)kNumLogStepItems);
+  return _profiler->GetStep(key, static_cast<LogStepItem>(item));
+}
+
+size_t coll_cache_rank_hotness(int replica_id, uint32_t *keys_out, uint32_t *cnts_out, size_t capacity) {
+  CHECK(RunConfig::is_configured);
+  ContFreqBuf *rank = CombineAndRank(replica_id);
+  CHECK_NOTNULL(rank);
+  const size_t n = rank->size();
+  for (size_t i = 0; i < std::min(n, capacity); i++) {
+    if (keys_out) keys_out[i] = rank->buf[i].key;
+    if (cnts_out) cnts_out[i] = rank->buf[i].cnt;
+  }
+  return n;
+}
+
+uint32_t coll_cache_place_ranked(const uint32_t *rank_keys, const uint32_t *rank_freq, uint32_t num_node,
+                                 double cache_percentage, uint32_t *nid_to_block_out) {
+  CHECK_NOTNULL(rank_keys);
+  CHECK_NOTNULL(rank_freq);
+  CHECK_NOTNULL(nid_to_block_out);
+  coll_cache::FreqRankSolver solver;
+  auto keys = Tensor::FromBlob(const_cast<uint32_t *>(rank_keys), kI32, {1, (size_t)num_node}, CPU(CPU_FOREIGN), "");
+  auto freq = Tensor::FromBlob(const_cast<uint32_t *>(rank_freq), kI32, {1, (size_t)num_node}, CPU(CPU_FOREIGN), "");
+  auto n2b = Tensor::FromBlob(nid_to_block_out, kI32, {(size_t)num_node}, CPU(CPU_FOREIGN), "");
+  solver.Build(keys, freq, {0}, num_node, n2b);
+  solver.Solve({0}, {cache_percentage * 100}, "BIN", RunConfig::coll_cache_hyperparam_T_local,
+               RunConfig::coll_cache_hyperparam_T_cpu);
+  uint32_t cached = 0;
+  for (uint32_t k = 0; k < num_node; k++) cached += nid_to_block_out[k] == 0;
+  return cached;
+}
+
+void coll_cache_shutdown(void) {
+  if (_coll_cache) _coll_cache->release_replicas();
+  _coll_cache = nullptr;
+  _profiler = nullptr;
+  _freq_recorder.clear();
+  memset(steps, 0, sizeof(steps));
+  max_num_keys = 0;
+  RunConfig::is_configured = false;
+}
+
+}  // extern "C"
+
+}  // namespace common
+}  // namespace coll_cache_lib

@@ -1,0 +1,99 @@
+#include "run_config.h"
+
+#include <cstdlib>
+
+#include "logging.h"
+#include "ugache_hip.h"
+
+namespace coll_cache_lib {
+namespace common {
+
+bool RunConfig::is_configured = false;
+CachePolicy RunConfig::cache_policy = kCollCacheAsymmLink;
+double RunConfig::cache_percentage = 0;
+size_t RunConfig::num_device = 1;
+std::vector<int> RunConfig::device_id_list = {0};
+bool RunConfig::cross_process = false;
+int RunConfig::worker_id = 0;
+uint64_t RunConfig::num_global_step_per_epoch = 0;
+uint64_t RunConfig::num_epoch = 0;
+uint64_t RunConfig::num_total_item = 0;
+int RunConfig::omp_thread_num = 40;
+int RunConfig::solver_omp_thread_num = 40;
+int RunConfig::solver_omp_thread_num_per_gpu = 5;
+int RunConfig::refresher_omp_thread_num = 8;
+int RunConfig::refresher_omp_thread_num_per_gpu = 1;
+size_t RunConfig::option_empty_feat = 0;
+ConcurrentLinkImpl RunConfig::concurrent_link_impl = kSMMaskPhase;
+size_t RunConfig::coll_cache_scale_nb = 16;
+bool RunConfig::use_flat_hashtable = true;
+double RunConfig::coll_cache_hyperparam_T_local = 1;
+double RunConfig::coll_cache_hyperparam_T_cpu = 8000.0 / 50.0;
+coll_cache::AsymmLinkDesc RunConfig::coll_cache_link_desc;
+double RunConfig::hash_load_factor = 0.7;
+int RunConfig::force_table_kind = 0;
+size_t RunConfig::refresh_batch_rows = 4092;
+unsigned RunConfig::refresh_sleep_us = 3000;
+unsigned RunConfig::refresh_limit_block = 20;
+
+void RunConfig::LoadConfigFromEnv() {
+  // every knob goes back to its default first, so a process that builds a second cache sees only its current
+  // environment
+  concurrent_link_impl = kSMMaskPhase;
+  coll_cache_scale_nb = 16;
+  hash_load_factor = 0.7;
+  force_table_kind = 0;
+  refresh_batch_rows = 4092;
+  refresh_sleep_us = 3000;
+  refresh_limit_block = 20;
+  if (GetEnv("SAMGRAPH_EMPTY_FEAT") != "" && GetEnv("SAMGRAPH_EMPTY_FEAT") != "0") {
+    LOG(FATAL) << "SAMGRAPH_EMPTY_FEAT (mock host table) is not supported by this build: every key must have a "
+                  "real row in the host table";
+  }
+  const std::string no_group = GetEnv("SAMGRAPH_COLL_CACHE_NO_GROUP");
+  const std::string impl = GetEnv("SAMGRAPH_COLL_CACHE_CONCURRENT_LINK_IMPL");
+  if (no_group == "DIRECT" || impl == "DIRECT") {
+    concurrent_link_impl = kDirectNoGroup;
+  } else if (impl == "" || impl == "SMMaskPhase" || impl == "MPSPhase") {
+    concurrent_link_impl = kSMMaskPhase;
+  } else if (impl == "NONE" || impl == "NoConcurrent") {
+    concurrent_link_impl = kNoConcurrentLink;
+  } else {
+    LOG(FATAL) << "concurrent link impl '" << impl << "' has no counterpart on one GPU (use SMMaskPhase, DIRECT or NONE)";
+  }
+  if (GetEnv("COLL_CACHE_SCALE") != "") coll_cache_scale_nb = std::stoul(GetEnv("COLL_CACHE_SCALE"));
+  if (GetEnv("COLL_HASH_LOAD_FACTOR") != "") hash_load_factor = std::stod(GetEnv("COLL_HASH_LOAD_FACTOR"));
+  const std::string tbl = GetEnv("COLL_HASH_TABLE");
+  if (tbl == "FLAT") force_table_kind = 1;
+  else if (tbl == "HASH") force_table_kind = 2;
+  else if (tbl != "") LOG(FATAL) << "COLL_HASH_TABLE must be FLAT or HASH, got " << tbl;
+  if (GetEnv("COLL_REFRESH_BATCH_ROWS") != "") refresh_batch_rows = std::stoul(GetEnv("COLL_REFRESH_BATCH_ROWS"));
+  if (GetEnv("COLL_REFRESH_SLEEP_US") != "") refresh_sleep_us = std::stoul(GetEnv("COLL_REFRESH_SLEEP_US"));
+  if (GetEnv("COLL_REFRESH_LIMIT_BLOCK") != "") refresh_limit_block = std::stoul(GetEnv("COLL_REFRESH_LIMIT_BLOCK"));
+  LOG(INFO) << "using concurrent impl " << concurrent_link_impl;
+}
+
+namespace coll_cache {
+
+AsymmLinkDesc AsymmLinkDesc::AutoBuild(Context ctx) {
+  // The reference aborts on anything that is not an A100/V100 (asymm_link_desc.cc:247-292).  Here any device
+  // the HIP layer can open is accepted; the numbers are MI355X's (HBM3E ~8 TB/s, PCIe Gen5 x16 host link).
+  AsymmLinkDesc desc;
+  ugk_device_info_t info;
+  UGK_CALL(ugk_get_device_info(ctx.device_id, &info));
+  desc.gpu_model = info.name;
+  desc.link_src.assign(RunConfig::num_device, {});
+  int cpu_blocks = 32;
+  if (GetEnv("COLL_CPU_SM_NUM_OVERRIDE") != "") cpu_blocks = std::stoi(GetEnv("COLL_CPU_SM_NUM_OVERRIDE"));
+  CHECK_GT(cpu_blocks, 0);
+  desc.cpu_sm.assign(RunConfig::num_device, cpu_blocks);
+  desc.local_sm.assign(RunConfig::num_device, 0);
+  desc.local_bw_GBps = 8000;
+  desc.cpu_bw_GBps = 50;
+  if (GetEnv("COLL_CPU_TIME_OVERRIDE") != "") RunConfig::coll_cache_hyperparam_T_cpu = std::stod(GetEnv("COLL_CPU_TIME_OVERRIDE"));
+  return desc;
+}
+
+}  // namespace coll_cache
+}  // namespace common
+}  // namespace coll_cache_lib

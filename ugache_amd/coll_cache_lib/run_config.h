@@ -1,0 +1,74 @@
+// Process-wide configuration, mirroring coll_cache_lib/run_config.{h,cc} of the reference for the fields the
+// extraction path reads (run_config.h:30-111; LoadConfigFromEnv run_config.cc:84-172).
+#pragma once
+
+#include <cstdint>
+#include <string>
+#include <vector>
+
+#include "common.h"
+
+namespace coll_cache_lib {
+namespace common {
+
+// How ExtractFeat combines the two sources (run_config.h ConcurrentLinkImpl; only the variants that make
+// sense with one GPU and its host are kept).
+enum ConcurrentLinkImpl {
+  kNoConcurrentLink = 0,  // host group, then local group, on the caller's stream
+  kSMMaskPhase,           // default: the two groups as concurrent kernels on their own streams
+  kDirectNoGroup,         // one fused lookup+gather kernel, no partition (SAMGRAPH_COLL_CACHE_NO_GROUP=DIRECT)
+};
+
+namespace coll_cache {
+// Single-GPU slice of AsymmLinkDesc (coll_cache/asymm_link_desc.{h,cc}): no peer links, a compute budget for
+// the host-miss gather and one for the local gather, and the bandwidth figures the placement model assumes.
+struct AsymmLinkDesc {
+  std::vector<std::vector<std::vector<int>>> link_src;  // [dst gpu][link][src gpus]; empty lists with one GPU
+  std::vector<int> cpu_sm;     // workgroups given to the host-miss gather (the reference counts SMs)
+  std::vector<int> local_sm;   // 0 = fill the chip
+  double local_bw_GBps = 0;    // HBM
+  double cpu_bw_GBps = 0;      // host link
+  std::string gpu_model;
+  static AsymmLinkDesc AutoBuild(Context ctx);
+};
+}  // namespace coll_cache
+
+struct RunConfig {
+  static bool is_configured;
+  static CachePolicy cache_policy;
+  static double cache_percentage;
+  static size_t num_device;
+  static std::vector<int> device_id_list;
+  static bool cross_process;
+  static int worker_id;
+  static uint64_t num_global_step_per_epoch;
+  static uint64_t num_epoch;
+  static uint64_t num_total_item;
+  static int omp_thread_num;
+  static int solver_omp_thread_num;
+  static int solver_omp_thread_num_per_gpu;
+  static int refresher_omp_thread_num;
+  static int refresher_omp_thread_num_per_gpu;
+  static size_t option_empty_feat;  // SAMGRAPH_EMPTY_FEAT mock tables are not supported: must stay 0
+  static ConcurrentLinkImpl concurrent_link_impl;
+  static size_t coll_cache_scale_nb;
+  static bool use_flat_hashtable;
+  static double coll_cache_hyperparam_T_local;
+  static double coll_cache_hyperparam_T_cpu;
+  static coll_cache::AsymmLinkDesc coll_cache_link_desc;
+  // knobs of this implementation
+  static double hash_load_factor;      // COLL_HASH_LOAD_FACTOR, default 0.7
+  static int force_table_kind;         // COLL_HASH_TABLE=FLAT|HASH -> 1|2, 0 = decide by size
+  static size_t refresh_batch_rows;    // COLL_REFRESH_BATCH_ROWS, default 4092 (cache_context.cu:4057)
+  static unsigned refresh_sleep_us;    // COLL_REFRESH_SLEEP_US, default 3000 (cache_context.cu:4069)
+  static unsigned refresh_limit_block; // COLL_REFRESH_LIMIT_BLOCK, default 20 (cache_context.cu:4068)
+
+  static void LoadConfigFromEnv();
+  static inline uint64_t GetBatchKey(uint64_t epoch, uint64_t step) { return epoch * num_global_step_per_epoch + step; }
+  static inline uint64_t GetEpochFromKey(uint64_t key) { return num_global_step_per_epoch ? key / num_global_step_per_epoch : 0; }
+  static inline uint64_t GetStepFromKey(uint64_t key) { return num_global_step_per_epoch ? key % num_global_step_per_epoch : key; }
+  static inline bool UseGPUCache() { return cache_percentage > 0; }
+};
+
+}  // namespace common
+}  // namespace coll_cache_lib

@@ -1,0 +1,183 @@
+"""Counterpart of python/collcache/torch/adapter.{py,cc} of the reference: the PyTorch front of the cache.
+
+The reference binds these entry points with pybind11; here they are plain Python over the extern "C" shim, with
+torch used only for what the C++ adapter used it for: device memory (the allocator handle and the reused output
+buffer, adapter.cc:126-149, 204-237) and the stream.  Same names, argument meaning and return shapes.
+"""
+import ctypes
+import os
+import sys
+
+import torch
+
+from ..common import *  # noqa: F401,F403
+from ..common import ALLOC_FN, RELEASE_FN, _basics, kF16, kF32
+
+config = _basics.config
+log_step_by_key = _basics.log_step_by_key
+report_step = _basics.report_step
+report_step_average = _basics.report_step_average
+wait_one_child = _basics.wait_one_child
+print_memory_usage = _basics.print_memory_usage
+coll_cache_record_init = _basics.coll_cache_record_init
+
+_C = _basics.C_LIB_CTYPES
+
+
+class _State:
+    dev_id = {}            # replica -> device index
+    external_dtype = torch.float32
+    external_feat_dim = 0
+    internal_feat_dim = 0
+    batch_emb_reuse = None  # int8 tensor backing the reused output buffer
+    held = {}              # device pointer -> tensor handed to the library by the allocator callback
+    host_tables = []       # keeps pinned tables alive
+    host_ptrs = []         # pinned allocations made by coll_torch_create_emb_shm
+    alloc_cb = None
+    release_cb = None
+
+
+def _make_allocator(dev_id):
+    """TorchMemHandle (adapter.h:37-46): library memory is an int8 torch tensor kept alive until released."""
+    def _alloc(nbytes, _user):
+        t = torch.empty((max(int(nbytes), 1),), dtype=torch.int8, device="cuda:%d" % dev_id)
+        _State.held[t.data_ptr()] = t
+        return t.data_ptr()
+
+    def _release(ptr, _user):
+        _State.held.pop(ptr, None)
+
+    _State.alloc_cb = ALLOC_FN(_alloc)
+    _State.release_cb = RELEASE_FN(_release)
+    return _State.alloc_cb, _State.release_cb
+
+
+def _stream_handle(dev_id):
+    # lookups run on torch's current stream, so they are ordered after whatever produced the keys
+    return ctypes.c_void_p(torch.cuda.current_stream(dev_id).cuda_stream)
+
+
+def _setup_dims(dim, use_fp16):
+    _State.external_feat_dim = dim
+    if use_fp16:
+        if dim % 2 != 0:
+            sys.stderr.write("dimension must be even\n")
+            os.abort()
+        _State.external_dtype = torch.float16
+        _State.internal_feat_dim = dim // 2
+    else:
+        _State.external_dtype = torch.float32
+        _State.internal_feat_dim = dim
+
+
+def coll_torch_init_t(replica_id, dev_id, emb, cache_percentage):
+    """adapter.cc:151-190: build the cache of `replica_id` on GPU `dev_id` from the host table `emb`."""
+    torch.cuda.set_device(dev_id)
+    _State.dev_id[replica_id] = dev_id
+    alloc, release = _make_allocator(dev_id)
+    use_fp16 = emb.dtype == torch.float16
+    if not use_fp16 and emb.dtype != torch.float32:
+        raise TypeError("embedding table must be float32 or float16, got %s" % emb.dtype)
+    dim = emb.size(1)
+    _setup_dims(dim, use_fp16)
+    info_keys = emb.size(0)
+    _C.coll_cache_init_c(replica_id, info_keys, alloc, release, None, emb.data_ptr(), kF16 if use_fp16 else kF32, dim,
+                         float(cache_percentage), _stream_handle(dev_id))
+    _State.host_tables.append(emb)
+
+
+def coll_torch_init(replica_id, key_space_size, dev_id, cpu_data, dim, cache_percentage, use_fp16):
+    """adapter.cc:126-149: same with a raw host pointer (integer address)."""
+    torch.cuda.set_device(dev_id)
+    _State.dev_id[replica_id] = dev_id
+    alloc, release = _make_allocator(dev_id)
+    _setup_dims(dim, use_fp16)
+    _C.coll_cache_init_c(replica_id, key_space_size, alloc, release, None, cpu_data, kF16 if use_fp16 else kF32, dim,
+                         float(cache_percentage), _stream_handle(dev_id))
+
+
+def coll_torch_test(local_id, keys):
+    """adapter.cc:192-203: an uninitialised tensor of the output's shape."""
+    dev = _State.dev_id.get(local_id, 0)
+    return torch.empty((keys.size(0), _State.external_feat_dim), dtype=torch.float32, device="cuda:%d" % dev)
+
+
+def coll_torch_lookup_key_t_val_ret(local_id, keys, pad_to_8=True):
+    """adapter.cc:204-237: look the keys (GPU int32/uint32 tensor, or int64) up; returns a [ceil8(N), dim] view of one
+    reused output buffer — the next lookup overwrites it."""
+    dev = _State.dev_id.get(local_id, 0)
+    n = keys.size(0)
+    padded_len = (n + 7) // 8 * 8 if pad_to_8 else n
+    max_num_keys = _C.coll_cache_max_num_keys()
+    if padded_len > max_num_keys:
+        sys.stderr.write("Warning, found a larger batch, re allocating emb output now %d %d\n" % (padded_len, max_num_keys))
+        max_num_keys = max(max_num_keys, padded_len)
+        _State.batch_emb_reuse = None
+    if _State.batch_emb_reuse is None:
+        max_num_keys = int(max_num_keys * 1.05)
+        _C.coll_cache_set_max_num_keys(max_num_keys)
+        _State.batch_emb_reuse = torch.empty((max(max_num_keys, 1) * _State.internal_feat_dim * 4,), dtype=torch.int8,
+                                             device="cuda:%d" % dev)
+    elem = 2 if _State.external_dtype == torch.float16 else 4
+    tensor = _State.batch_emb_reuse[: padded_len * _State.external_feat_dim * elem].view(_State.external_dtype).view(
+        padded_len, _State.external_feat_dim)
+    if keys.dtype == torch.int64:
+        _C.coll_cache_lookup_i64(local_id, keys.data_ptr(), n, tensor.data_ptr(), _stream_handle(dev))
+    else:
+        _C.coll_cache_lookup(local_id, keys.data_ptr(), n, tensor.data_ptr(), _stream_handle(dev))
+    return tensor
+
+
+def coll_torch_record(local_id, keys):
+    """adapter.cc:270-272: count the hotness of a batch of keys (CPU tensor)."""
+    if keys.is_cuda:
+        keys = keys.cpu()
+    keys = keys.contiguous()
+    if keys.dtype == torch.int64:
+        _C.coll_cache_record_i64(local_id, keys.data_ptr(), keys.numel())
+    else:
+        _C.coll_cache_record(local_id, keys.data_ptr(), keys.numel())
+
+
+_ELEM = {torch.float32: 4, torch.float16: 2, torch.float64: 8, torch.int32: 4, torch.int64: 8, torch.uint8: 1,
+         torch.int8: 1}
+
+
+def coll_torch_create_emb_shm(replica_id, n_keys, dim, dtype, fname=""):
+    """adapter.cc:239-268: the host embedding table as a CPU tensor [n_keys, dim].  The reference places it in POSIX
+    shared memory and page-locks it later; here it is allocated pinned and GPU-mapped from the start.  If `fname` is
+    given the file must hold exactly n_keys * dim elements and is read into the table."""
+    nbytes = int(n_keys) * int(dim) * _ELEM[dtype]
+    ptr = _C.coll_cache_alloc_host_table(max(nbytes, 64))
+    _State.host_ptrs.append(ptr)
+    buf = (ctypes.c_uint8 * max(nbytes, 64)).from_address(ptr)
+    tensor = torch.frombuffer(buf, dtype=dtype, count=int(n_keys) * int(dim)).view(int(n_keys), int(dim))
+    if fname != "":
+        size = os.stat(fname).st_size
+        if size != nbytes:
+            sys.stderr.write("feat file on disk not equal with claimed shape %d != %dx%dx%d\n"
+                             % (size, _ELEM[dtype], n_keys, dim))
+            os.abort()
+        with open(fname, "rb") as f:
+            f.readinto(buf)
+    return tensor
+
+
+def coll_torch_refresh(replica_id, foreground=False):
+    """re-place by the hotness recorded since the last build/refresh (the TF binding's LookupManager::refresh)."""
+    dev = _State.dev_id.get(replica_id, 0)
+    _basics.refresh(replica_id, _stream_handle(dev), foreground)
+
+
+def coll_torch_shutdown():
+    """drop the cache and every buffer it holds, including the tables made by coll_torch_create_emb_shm, which
+    must not be used afterwards (the reference has no teardown)."""
+    torch.cuda.synchronize()
+    _basics.shutdown()
+    for p in _State.host_ptrs:
+        _C.coll_cache_free_host_table(p)
+    _State.host_ptrs.clear()
+    _State.batch_emb_reuse = None
+    _State.held.clear()
+    _State.host_tables.clear()
+    _State.dev_id.clear()
