@@ -294,13 +294,17 @@ void ExtractSession::ExtractFeatImpl(const KeyT *nodes, size_t num_nodes, void *
     // with the host-link budget.
     CHECK_EQ(ctx->_num_location, 1);
     const bool from_host = ctx->_cpu_location_id != -1;
-    Timer t0;
+    // the gather is bracketed by events on its own stream: the logged combine time is the kernel's duration
+    UGK_CALL(ugk_event_record(_ev_t[0], stream));
     UGK_CALL(GatherDirect<KeyT>(ctx->_device_cache_data[0], ctx->_num_total_nodes, nodes, num_nodes, output, rb,
                                 from_host ? _cpu_blocks : 0, _status, stream));
+    UGK_CALL(ugk_event_record(_ev_t[1], stream));
     UGK_CALL(ugk_memcpy_async(_host_mirror + 4, _status, sizeof(uint32_t), stream));
     UGK_CALL(ugk_stream_sync(stream));
     CheckStatusWord(_host_mirror[4]);
-    const double combine_time = t0.Passed();
+    float combine_ms = 0;
+    UGK_CALL(ugk_event_elapsed_ms(_ev_t[0], _ev_t[1], &combine_ms));
+    const double combine_time = combine_ms * 1e-3;
     _group_offset[1] = from_host ? 0 : (uint32_t)num_nodes;
     _group_offset[2] = (uint32_t)num_nodes;
     if (profiler && task_key != 0xffffffffffffffffull) {
@@ -326,15 +330,18 @@ void ExtractSession::ExtractFeatImpl(const KeyT *nodes, size_t num_nodes, void *
 
   if (RunConfig::concurrent_link_impl == kDirectNoGroup) {
     // one fused lookup + gather kernel, source chosen per row (cache_context.cu:1295-1329)
-    Timer t0;
+    UGK_CALL(ugk_event_record(_ev_t[0], stream));
     UGK_CALL(ExtractMix(table, nodes, num_nodes, cache, cache_rows, host, host_rows, output, rb, _status, stream));
+    UGK_CALL(ugk_event_record(_ev_t[1], stream));
     UGK_CALL(ugk_memcpy_async(_host_mirror + 4, _status, sizeof(uint32_t), stream));
     UGK_CALL(ugk_stream_sync(stream));
     CheckStatusWord(_host_mirror[4]);
+    float mix_ms = 0;
+    UGK_CALL(ugk_event_elapsed_ms(_ev_t[0], _ev_t[1], &mix_ms));
     _group_offset[1] = _group_offset[2] = (uint32_t)num_nodes;  // group sizes are not produced on this path
     if (profiler && task_key != 0xffffffffffffffffull) {
       profiler->LogStep(task_key, kLogL1FeatureBytes, nbytes);
-      profiler->LogStep(task_key, kLogL3CacheCombineCacheTime, t0.Passed());
+      profiler->LogStep(task_key, kLogL3CacheCombineCacheTime, mix_ms * 1e-3);
       profiler->LogEpochAdd(task_key, kLogEpochFeatureBytes, nbytes);
     }
     ctx->progress.fetch_add(1);

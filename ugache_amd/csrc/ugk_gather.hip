@@ -4,12 +4,18 @@
 // flight rather than around arithmetic:
 //   * a row of V 16-byte vectors is copied by LPR = min(64, pow2ceil(V)) adjacent lanes, so one wavefront
 //     instruction moves 64/LPR whole rows as fully coalesced segments (512-B rows: 2 rows, 128-B rows: 8);
-//   * every lane keeps UNROLL independent rows in flight (all loads issued before the first store);
-//   * loads and stores carry the non-temporal hint: rows are touched once, the output is write-only;
+//   * every lane keeps UNROLL = 2 independent rows in flight (both loads issued before the first store) and
+//     the launch uses many small workgroups (one or two passes each): measured on MI355X this beats deeper
+//     unrolling with fewer, longer-lived workgroups by ~15 %;
+//   * loads carry the non-temporal hint (table rows are touched once); stores are ordinary write-back stores
+//     while the output fits the 256 MB memory-side cache, so the consumer finds it there, and non-temporal
+//     beyond that;
 //   * the grid is a grid-stride launch sized from the CU count, or capped by the caller so a host-link
 //     gather occupies only a few CUs while the HBM gather runs next to it;
 //   * keys / index records are range-checked against the source's row count: a bad key sets a status bit
 //     and its row is skipped instead of faulting.
+#include <cstdlib>
+
 #include "ugk_internal.h"
 
 namespace ugk {
@@ -70,7 +76,7 @@ template <typename V, int LPR, int UNROLL, typename Idx>
 __global__ __launch_bounds__(kBlock) void gather_kernel(Idx ix, const V *__restrict__ src, uint64_t src_rows,
                                                         V *__restrict__ out, uint64_t out_rows, uint32_t vpr,
                                                         const uint32_t *__restrict__ counts, uint32_t group, size_t n,
-                                                        uint32_t *status) {
+                                                        uint32_t *status, bool nt_store) {
   size_t begin = 0, count = n;
   if (counts) {
     const uint32_t c = counts[group];
@@ -108,22 +114,36 @@ __global__ __launch_bounds__(kBlock) void gather_kernel(Idx ix, const V *__restr
           if (ok[u]) v[u] = ld_stream(src + s[u] * vpr + col);
 #pragma unroll
         for (int u = 0; u < UNROLL; ++u)
-          if (ok[u]) st_stream(out + d[u] * vpr + col, v[u]);
+          if (ok[u]) {
+            if (nt_store) st_stream(out + d[u] * vpr + col, v[u]);
+            else out[d[u] * vpr + col] = v[u];
+          }
       }
     }
   }
+}
+
+// Non-temporal stores only when the output cannot stay in the memory-side cache anyway.
+// UGK_GATHER_NT_STORE=0/1 forces the choice.
+bool nt_store_for(size_t out_bytes) {
+  static int forced = [] {
+    const char *e = getenv("UGK_GATHER_NT_STORE");
+    return e ? atoi(e) : -1;
+  }();
+  if (forced >= 0) return forced != 0;
+  return out_bytes > ((size_t)192 << 20);
 }
 
 template <typename V, int LPR, typename Idx>
 int launch_one(Idx ix, const void *src, uint64_t src_rows, void *out, uint64_t out_rows, uint32_t vpr,
                const uint32_t *counts, uint32_t group, size_t n, unsigned max_blocks, uint32_t *status,
                hipStream_t stream) {
-  constexpr int UNROLL = 4;
+  constexpr int UNROLL = 2;
   constexpr size_t kPerIter = (size_t)(kBlock / LPR) * UNROLL;
   const unsigned grid = clamp_grid((n + kPerIter - 1) / kPerIter, max_blocks);
   hipLaunchKernelGGL((gather_kernel<V, LPR, UNROLL, Idx>), dim3(grid), dim3(kBlock), 0, stream, ix,
                      reinterpret_cast<const V *>(src), src_rows, reinterpret_cast<V *>(out), out_rows, vpr, counts,
-                     group, n, status);
+                     group, n, status, nt_store_for(n * (size_t)vpr * sizeof(V)));
   UGK_HIP(hipGetLastError());
   return 0;
 }

@@ -33,7 +33,8 @@ typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
 // Number of compute units of the current device (cached per device).
 int cu_count();
 
-// Blocks per CU used to size grid-stride launches that should fill the chip; UGK_BLOCKS_PER_CU overrides.
+// Upper bound, in workgroups per CU, of grid-stride launches that should fill the chip (default 64: many short
+// workgroups balance better than few long ones on this part); UGK_BLOCKS_PER_CU overrides.
 int blocks_per_cu();
 
 static inline hipStream_t as_stream(void *s) { return reinterpret_cast<hipStream_t>(s); }

@@ -33,7 +33,7 @@ int blocks_per_cu() {
   if (v == 0) {
     const char *e = getenv("UGK_BLOCKS_PER_CU");
     v = e ? atoi(e) : 0;
-    if (v <= 0) v = 16;
+    if (v <= 0) v = 64;
   }
   return v;
 }
