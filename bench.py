@@ -38,6 +38,9 @@ def main():
     ap.add_argument("--workload", default="c2_all_hit_10Mx128xfp32_262144_u32_uniform", choices=sorted(WORKLOADS))
     ap.add_argument("--cpu-seconds", type=float, default=10.0, help="CPU baseline budget")
     ap.add_argument("--pool", type=int, default=64, help="distinct key batches cycled through the steps")
+    ap.add_argument("--calibrate", action="store_true",
+                    help="also run 5 plain device copies of 1 GiB (ugk_copy_rows) so a counter run has a kernel of "
+                         "known traffic next to the gather")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs the extraction path of ONE GPU (no collectives, no peer source); "
@@ -96,6 +99,15 @@ def main():
     ms_per_step = elapsed / K * 1e3
     keys_per_s = n_keys * K / elapsed
 
+    if args.calibrate:
+        cal_src = torch.empty(1 << 30, dtype=torch.uint8, device=dev)
+        cal_dst = torch.empty(1 << 30, dtype=torch.uint8, device=dev)
+        torch.cuda.synchronize()
+        for _ in range(5):
+            hip.call("ugk_copy_rows", cal_dst.data_ptr(), cal_src.data_ptr(), 1 << 30, stream)
+        torch.cuda.synchronize()
+        del cal_src, cal_dst
+
     # ---- parity of the last timed batch, byte for byte against the oracle -------------------------------------
     orc = Oracle()
     table_np = emb.numpy()
@@ -128,7 +140,7 @@ def main():
     while True:
         cpu_step(n_cpu)
         n_cpu += 1
-        if time.perf_counter() - t0 >= args.cpu_seconds or n_cpu >= 2000:
+        if time.perf_counter() - t0 >= args.cpu_seconds or n_cpu >= 100000:
             break
     cpu_elapsed = time.perf_counter() - t0
     cpu_keys_per_s = n_keys * n_cpu / cpu_elapsed
@@ -154,7 +166,7 @@ def main():
         "parity": "bit-exact vs CPU oracle (last timed batch)",
         "device": info["name"] + " " + info["arch"],
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-                     "frac": achieved / HBM_PEAK_GBPS, "traffic": None, "kernel": "gather_kernel<u32x4,32,4,DirectU32>",
+                     "frac": achieved / HBM_PEAK_GBPS, "traffic": None, "kernel": "gather_kernel<u32x4,32,2,DirectU32>",
                      "algorithmic_bytes_per_launch": alg_bytes, "avg_kernel_us": kernel_avg_s * 1e6,
                      "keys_per_s_kernel_only": n_keys / kernel_avg_s},
         "cpu_baseline": {"value": cpu_keys_per_s, "unit": "keys/s", "cores": cores, "kind": "port",

@@ -10,8 +10,11 @@
  *   - every function returns 0 on success, non-zero on failure; ugk_last_error() then describes it
  *     (thread-local, valid until the next failing call on the same thread);
  *   - all launches are asynchronous on `stream` (NULL = the null stream) unless stated otherwise;
- *   - `status` is a device word the kernels OR error bits into instead of faulting
- *     (UGK_ST_*); the host reads it after synchronising;
+ *   - `status_dev` is a device word the kernels OR error bits into instead of faulting (UGK_ST_*);
+ *   - `host_mirror` (per-batch entry points only, may be NULL) points at 4 words of pinned host memory that
+ *     the kernels write with ordinary stores so the caller needs no device-to-host copy after its one
+ *     synchronisation: [0] = non-zero if any error bit was raised (details are in status_dev),
+ *     [1] / [2] = size of the local / host group as seen by ugk_gather_group; the caller clears [0];
  *   - pointers named *_dev must be device-accessible (HBM, or pinned host memory from ugk_host_malloc).
  */
 #ifndef UGACHE_HIP_H_
@@ -116,9 +119,11 @@ int ugk_copy_rows(void *dst_dev, const void *src_dev, size_t nbytes, void *strea
  * chip; a non-zero value caps the grid (the reference's limit_block / per-source SM budget). */
 /* IdxStoreDirect (cache_context.h:341-354): srcrow = keys[i], dst = i */
 int ugk_gather_direct_u32(const void *src_dev, uint64_t src_rows, const uint32_t *keys_dev, size_t n, void *out_dev,
-                          size_t row_bytes, unsigned max_blocks, uint32_t *status_dev, void *stream);
+                          size_t row_bytes, unsigned max_blocks, uint32_t *status_dev, uint32_t *host_mirror,
+                          void *stream);
 int ugk_gather_direct_i64(const void *src_dev, uint64_t src_rows, const int64_t *keys_dev, size_t n, void *out_dev,
-                          size_t row_bytes, unsigned max_blocks, uint32_t *status_dev, void *stream);
+                          size_t row_bytes, unsigned max_blocks, uint32_t *status_dev, uint32_t *host_mirror,
+                          void *stream);
 /* IdxStoreDst (cache_context.h:356-361): srcrow = keys[i], dst = dst_off[i] (cache fill / refresh insert) */
 int ugk_gather_scatter_u32(const void *src_dev, uint64_t src_rows, const uint32_t *keys_dev,
                            const uint32_t *dst_off_dev, size_t n, void *out_dev, uint64_t out_rows, size_t row_bytes,
@@ -133,7 +138,7 @@ int ugk_gather_scatter_i64(const void *src_dev, uint64_t src_rows, const int64_t
  * so no host round trip is needed between classify and gather.  n is the batch size (grid upper bound). */
 int ugk_gather_group(const void *src_dev, uint64_t src_rows, const ugk_idx_t *idx_dev, const uint32_t *counts_dev,
                      uint32_t group, size_t n, void *out_dev, size_t row_bytes, unsigned max_blocks,
-                     uint32_t *status_dev, void *stream);
+                     uint32_t *status_dev, uint32_t *host_mirror, void *stream);
 /* same with an explicit list (count known on the host) */
 int ugk_gather_idx(const void *src_dev, uint64_t src_rows, const ugk_idx_t *idx_dev, size_t count, void *out_dev,
                    size_t row_bytes, unsigned max_blocks, uint32_t *status_dev, void *stream);
@@ -172,18 +177,20 @@ int ugk_hash_census(const ugk_bucket_t *table_dev, size_t nbuckets, uint64_t *ce
  * caller can rotate two counter pairs and never launch a memset.  host_rows bounds the miss offsets.
  * A key found with a location other than local/host sets UGK_ST_KEY_OUT_OF_RANGE (one GPU has two sources). */
 int ugk_classify_u32(ugk_table_t t, const uint32_t *keys_dev, size_t n, uint64_t host_rows, ugk_idx_t *idx_dev,
-                     uint32_t *counts_dev, uint32_t *next_counts_dev, uint32_t *status_dev, void *stream);
+                     uint32_t *counts_dev, uint32_t *next_counts_dev, uint32_t *status_dev, uint32_t *host_mirror,
+                     void *stream);
 int ugk_classify_i64(ugk_table_t t, const int64_t *keys_dev, size_t n, uint64_t host_rows, ugk_idx_t *idx_dev,
-                     uint32_t *counts_dev, uint32_t *next_counts_dev, uint32_t *status_dev, void *stream);
+                     uint32_t *counts_dev, uint32_t *next_counts_dev, uint32_t *status_dev, uint32_t *host_mirror,
+                     void *stream);
 
 /* ---- single-kernel mixed-source extraction: kDirectNoGroup with DataIterMixLoc
  *      (cache_context.cu:137-159, 1295-1329): lookup and gather fused, source picked per row ---------- */
 int ugk_extract_mix_u32(ugk_table_t t, const uint32_t *keys_dev, size_t n, const void *cache_dev, uint64_t cache_rows,
                         const void *host_dev, uint64_t host_rows, void *out_dev, size_t row_bytes,
-                        uint32_t *status_dev, void *stream);
+                        uint32_t *status_dev, uint32_t *host_mirror, void *stream);
 int ugk_extract_mix_i64(ugk_table_t t, const int64_t *keys_dev, size_t n, const void *cache_dev, uint64_t cache_rows,
                         const void *host_dev, uint64_t host_rows, void *out_dev, size_t row_bytes,
-                        uint32_t *status_dev, void *stream);
+                        uint32_t *status_dev, uint32_t *host_mirror, void *stream);
 
 /* ---- key dedup (the caller-side array_ops.unique of
  *      python_tf2/collcache_tf2/collcache_tf2/core/sparse_lookup_layer.py:197) ------------------------

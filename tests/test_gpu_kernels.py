@@ -30,7 +30,7 @@ def _gather_direct(table_np, keys_np, max_blocks=0):
     out = dev_bytes(len(keys_np) * rb, fill=0xEE)
     st = dev_zeros_u32(1)
     fn = "ugk_gather_direct_i64" if keys_np.dtype == np.int64 else "ugk_gather_direct_u32"
-    hip.call(fn, ptr(tbl), rows, ptr(keys), len(keys_np), ptr(out), rb, max_blocks, ptr(st), None)
+    hip.call(fn, ptr(tbl), rows, ptr(keys), len(keys_np), ptr(out), rb, max_blocks, ptr(st), None, None)
     return to_np(out)[: len(keys_np) * rb].reshape(len(keys_np), rb), status_value(st)
 
 
@@ -106,7 +106,7 @@ def test_gather_from_pinned_host_memory():
         out = dev_bytes(5000 * 512)
         st = dev_zeros_u32(1)
         d_keys = to_dev(keys)
-        hip.call("ugk_gather_direct_u32", pin.ptr, 2000, ptr(d_keys), 5000, ptr(out), 512, 8, ptr(st), None)
+        hip.call("ugk_gather_direct_u32", pin.ptr, 2000, ptr(d_keys), 5000, ptr(out), 512, 8, ptr(st), None, None)
         assert status_value(st) == 0
         assert to_np(out).reshape(5000, 512).tobytes() == table[keys].tobytes()
         kind = C.c_int(-1)
@@ -135,7 +135,7 @@ def test_gather_full_size_all_hit_closed_form():
     out = torch.empty((n, dim), dtype=torch.int32, device="cuda")
     st = dev_zeros_u32(1)
     hip.call("ugk_gather_direct_u32", table.data_ptr(), rows, keys.data_ptr(), n, out.data_ptr(), dim * 4, 0, ptr(st),
-             None)
+             None, None)
     assert status_value(st) == 0
     k = keys.unsqueeze(1)
     want = (k * 131 + c * 7919) ^ (k >> 3)
@@ -300,7 +300,7 @@ def _classify(tb, keys_np, host_rows):
     st = dev_zeros_u32(1)
     fn = "ugk_classify_i64" if keys_np.dtype == np.int64 else "ugk_classify_u32"
     keys = to_dev(keys_np)
-    hip.call(fn, tb, ptr(keys), n, host_rows, ptr(idx), ptr(counts), ptr(counts) + 8, ptr(st), None)
+    hip.call(fn, tb, ptr(keys), n, host_rows, ptr(idx), ptr(counts), ptr(counts) + 8, ptr(st), None, None)
     sync()
     c = to_np(counts, np.uint32)
     return idx, counts, c, status_value(st), keys
@@ -344,15 +344,18 @@ def test_classify_partition_and_factored_gather(mode, kdtype, n):
 
     # factored extraction: host group and local group as two launches reading the device-side counts
     pin = pinned_from(host)
+    mirror = pinned_from(np.array([0, 0xFFFFFFFF, 0xFFFFFFFF, 0xFFFFFFFF], np.uint32))
     try:
         out = dev_bytes(n * rb, fill=0xCD)
         st2 = dev_zeros_u32(1)
         cache_dev = to_dev(cache)
         hip.call("ugk_gather_group", pin.ptr, nkeys, ptr(idx), ptr(counts), hip.LOC_HOST, n, ptr(out), rb, 4, ptr(st2),
-                 None)
+                 mirror.ptr, None)
         hip.call("ugk_gather_group", ptr(cache_dev), cap, ptr(idx), ptr(counts), hip.LOC_LOCAL, n, ptr(out), rb, 0,
-                 ptr(st2), None)
+                 ptr(st2), mirror.ptr, None)
         assert status_value(st2) == 0
+        if n:  # the gathers publish their group sizes in pinned host memory
+            assert mirror.array.tolist() == [0, int(c[0]), int(c[1]), 0xFFFFFFFF]
         want_out, _ = ORC.extract_feat(keys.astype(np.uint32), cache, host, flat=oflat)
         assert to_np(out)[: n * rb].tobytes() == want_out.tobytes()
         assert want_out.tobytes() == host[keys.astype(np.int64)].tobytes()
@@ -360,12 +363,13 @@ def test_classify_partition_and_factored_gather(mode, kdtype, n):
         # fused single-kernel variant gives the same bytes
         out2 = dev_bytes(n * rb, fill=0x11)
         fn = "ugk_extract_mix_i64" if kdtype == np.int64 else "ugk_extract_mix_u32"
-        hip.call(fn, tb, ptr(keys_dev), n, ptr(cache_dev), cap, pin.ptr, nkeys, ptr(out2), rb, ptr(st2), None)
+        hip.call(fn, tb, ptr(keys_dev), n, ptr(cache_dev), cap, pin.ptr, nkeys, ptr(out2), rb, ptr(st2), None, None)
         assert status_value(st2) == 0
         assert to_np(out2)[: n * rb].tobytes() == want_out.tobytes()
     finally:
         sync()
         pin.free()
+        mirror.free()
 
 
 def test_classify_rejects_keys_beyond_the_host_table():
@@ -394,7 +398,7 @@ def test_extract_mix_other_row_sizes(row_bytes):
         st = dev_zeros_u32(1)
         d_keys, d_cache = to_dev(keys), to_dev(cache)
         hip.call("ugk_extract_mix_u32", tb, ptr(d_keys), len(keys), ptr(d_cache), len(cached), pin.ptr,
-                 nkeys, ptr(out), row_bytes, ptr(st), None)
+                 nkeys, ptr(out), row_bytes, ptr(st), None, None)
         assert status_value(st) == 0
         assert to_np(out)[: len(keys) * row_bytes].tobytes() == host[keys].tobytes()
     finally:

@@ -135,7 +135,7 @@ void CacheContext::build_with_advise_new_hash(int location_id, std::shared_ptr<C
     UGK_CALL(ugk_fill_u32(st->ptr<uint32_t>(), 0, 1, stream));
     UGK_CALL(ugk_gather_direct_u32(cpu_data, num_total_nodes, cache_node_list->CPtr<uint32_t>(), num_cached_nodes,
                                    _device_cache_data[_local_location_id], _row_bytes, 0, st->ptr<uint32_t>(),
-                                   stream));
+                                   nullptr, stream));
     _new_hash_table->InsertSeqOffWithLoc(cache_node_list, location_id, stream);
     uint32_t fill_status = 0;
     UGK_CALL(ugk_memcpy_async(&fill_status, st->ptr(), sizeof(fill_status), stream));
@@ -236,40 +236,41 @@ void ExtractSession::EnsureIdx(size_t num_nodes) {
   }
 }
 
-void ExtractSession::CheckStatusWord(uint32_t st) const {
+void ExtractSession::CheckStatusWord(StreamHandle stream) const {
+  if (_host_mirror[0] == 0) return;  // common case: nothing to fetch from the device
+  uint32_t st = 0;
+  UGK_CALL(ugk_memcpy_async(&st, _status, sizeof(st), stream));
+  UGK_CALL(ugk_stream_sync(stream));
   CHECK_EQ(st, 0u) << "extraction kernels reported status 0x" << std::hex << st
                    << ": a key is outside the table it has to be read from (num_total_item="
                    << std::dec << _cache_ctx->_num_total_nodes << ")";
 }
 
-template <typename KeyT>
-static int GatherDirect(const void *src, uint64_t rows, const KeyT *keys, size_t n, void *out, size_t rb,
-                        unsigned max_blocks, uint32_t *status, StreamHandle s);
-template <>
-int GatherDirect<IdType>(const void *src, uint64_t rows, const IdType *keys, size_t n, void *out, size_t rb,
-                         unsigned max_blocks, uint32_t *status, StreamHandle s) {
-  return ugk_gather_direct_u32(src, rows, keys, n, out, rb, max_blocks, status, s);
+static int GatherDirect(const void *src, uint64_t rows, const IdType *keys, size_t n, void *out, size_t rb,
+                        unsigned max_blocks, uint32_t *status, uint32_t *mirror, StreamHandle s) {
+  return ugk_gather_direct_u32(src, rows, keys, n, out, rb, max_blocks, status, mirror, s);
 }
-template <>
-int GatherDirect<Id64Type>(const void *src, uint64_t rows, const Id64Type *keys, size_t n, void *out, size_t rb,
-                           unsigned max_blocks, uint32_t *status, StreamHandle s) {
-  return ugk_gather_direct_i64(src, rows, keys, n, out, rb, max_blocks, status, s);
+static int GatherDirect(const void *src, uint64_t rows, const Id64Type *keys, size_t n, void *out, size_t rb,
+                        unsigned max_blocks, uint32_t *status, uint32_t *mirror, StreamHandle s) {
+  return ugk_gather_direct_i64(src, rows, keys, n, out, rb, max_blocks, status, mirror, s);
 }
 static int Classify(ugk_table_t t, const IdType *keys, size_t n, uint64_t host_rows, ugk_idx_t *idx, uint32_t *c,
-                    uint32_t *next, uint32_t *st, StreamHandle s) {
-  return ugk_classify_u32(t, keys, n, host_rows, idx, c, next, st, s);
+                    uint32_t *next, uint32_t *st, uint32_t *mirror, StreamHandle s) {
+  return ugk_classify_u32(t, keys, n, host_rows, idx, c, next, st, mirror, s);
 }
 static int Classify(ugk_table_t t, const Id64Type *keys, size_t n, uint64_t host_rows, ugk_idx_t *idx, uint32_t *c,
-                    uint32_t *next, uint32_t *st, StreamHandle s) {
-  return ugk_classify_i64(t, keys, n, host_rows, idx, c, next, st, s);
+                    uint32_t *next, uint32_t *st, uint32_t *mirror, StreamHandle s) {
+  return ugk_classify_i64(t, keys, n, host_rows, idx, c, next, st, mirror, s);
 }
 static int ExtractMix(ugk_table_t t, const IdType *keys, size_t n, const void *cache, uint64_t cache_rows,
-                      const void *host, uint64_t host_rows, void *out, size_t rb, uint32_t *st, StreamHandle s) {
-  return ugk_extract_mix_u32(t, keys, n, cache, cache_rows, host, host_rows, out, rb, st, s);
+                      const void *host, uint64_t host_rows, void *out, size_t rb, uint32_t *st, uint32_t *mirror,
+                      StreamHandle s) {
+  return ugk_extract_mix_u32(t, keys, n, cache, cache_rows, host, host_rows, out, rb, st, mirror, s);
 }
 static int ExtractMix(ugk_table_t t, const Id64Type *keys, size_t n, const void *cache, uint64_t cache_rows,
-                      const void *host, uint64_t host_rows, void *out, size_t rb, uint32_t *st, StreamHandle s) {
-  return ugk_extract_mix_i64(t, keys, n, cache, cache_rows, host, host_rows, out, rb, st, s);
+                      const void *host, uint64_t host_rows, void *out, size_t rb, uint32_t *st, uint32_t *mirror,
+                      StreamHandle s) {
+  return ugk_extract_mix_i64(t, keys, n, cache, cache_rows, host, host_rows, out, rb, st, mirror, s);
 }
 
 // cache_context.cu:1199-1794
@@ -296,12 +297,11 @@ void ExtractSession::ExtractFeatImpl(const KeyT *nodes, size_t num_nodes, void *
     const bool from_host = ctx->_cpu_location_id != -1;
     // the gather is bracketed by events on its own stream: the logged combine time is the kernel's duration
     UGK_CALL(ugk_event_record(_ev_t[0], stream));
-    UGK_CALL(GatherDirect<KeyT>(ctx->_device_cache_data[0], ctx->_num_total_nodes, nodes, num_nodes, output, rb,
-                                from_host ? _cpu_blocks : 0, _status, stream));
+    UGK_CALL(GatherDirect(ctx->_device_cache_data[0], ctx->_num_total_nodes, nodes, num_nodes, output, rb,
+                          from_host ? _cpu_blocks : 0, _status, _host_mirror, stream));
     UGK_CALL(ugk_event_record(_ev_t[1], stream));
-    UGK_CALL(ugk_memcpy_async(_host_mirror + 4, _status, sizeof(uint32_t), stream));
     UGK_CALL(ugk_stream_sync(stream));
-    CheckStatusWord(_host_mirror[4]);
+    CheckStatusWord(stream);
     float combine_ms = 0;
     UGK_CALL(ugk_event_elapsed_ms(_ev_t[0], _ev_t[1], &combine_ms));
     const double combine_time = combine_ms * 1e-3;
@@ -331,11 +331,11 @@ void ExtractSession::ExtractFeatImpl(const KeyT *nodes, size_t num_nodes, void *
   if (RunConfig::concurrent_link_impl == kDirectNoGroup) {
     // one fused lookup + gather kernel, source chosen per row (cache_context.cu:1295-1329)
     UGK_CALL(ugk_event_record(_ev_t[0], stream));
-    UGK_CALL(ExtractMix(table, nodes, num_nodes, cache, cache_rows, host, host_rows, output, rb, _status, stream));
+    UGK_CALL(ExtractMix(table, nodes, num_nodes, cache, cache_rows, host, host_rows, output, rb, _status,
+                        _host_mirror, stream));
     UGK_CALL(ugk_event_record(_ev_t[1], stream));
-    UGK_CALL(ugk_memcpy_async(_host_mirror + 4, _status, sizeof(uint32_t), stream));
     UGK_CALL(ugk_stream_sync(stream));
-    CheckStatusWord(_host_mirror[4]);
+    CheckStatusWord(stream);
     float mix_ms = 0;
     UGK_CALL(ugk_event_elapsed_ms(_ev_t[0], _ev_t[1], &mix_ms));
     _group_offset[1] = _group_offset[2] = (uint32_t)num_nodes;  // group sizes are not produced on this path
@@ -353,35 +353,36 @@ void ExtractSession::ExtractFeatImpl(const KeyT *nodes, size_t num_nodes, void *
   ugk_idx_t *idx = _idx_handle->ptr<ugk_idx_t>();
   uint32_t *cur = _counts[_cur], *next = _counts[_cur ^ 1];
   UGK_CALL(ugk_event_record(_ev_t[0], stream));
-  UGK_CALL(Classify(table, nodes, num_nodes, host_rows, idx, cur, next, _status, stream));
+  UGK_CALL(Classify(table, nodes, num_nodes, host_rows, idx, cur, next, _status, _host_mirror, stream));
   UGK_CALL(ugk_event_record(_ev_classified, stream));
   if (RunConfig::concurrent_link_impl == kSMMaskPhase) {
     // factored extraction: the host-link gather gets a few workgroups on its own stream, the HBM gather
     // the rest of the chip on another; both read their group bounds from the device-side counters
     UGK_CALL(ugk_stream_wait_event(_cpu_ext_stream, _ev_classified));
     UGK_CALL(ugk_gather_group(host, host_rows, idx, cur, UGK_LOC_HOST, num_nodes, output, rb, _cpu_blocks, _status,
-                              _cpu_ext_stream));
+                              _host_mirror, _cpu_ext_stream));
     UGK_CALL(ugk_event_record(_ev_cpu_done, _cpu_ext_stream));
     UGK_CALL(ugk_stream_wait_event(_local_ext_stream, _ev_classified));
     UGK_CALL(ugk_gather_group(cache, cache_rows, idx, cur, UGK_LOC_LOCAL, num_nodes, output, rb, 0, _status,
-                              _local_ext_stream));
+                              _host_mirror, _local_ext_stream));
     UGK_CALL(ugk_event_record(_ev_local_done, _local_ext_stream));
     UGK_CALL(ugk_stream_wait_event(stream, _ev_cpu_done));
     UGK_CALL(ugk_stream_wait_event(stream, _ev_local_done));
   } else {
     // sequential: host group, then local group (cache_context.cu:1719-1792)
-    UGK_CALL(ugk_gather_group(host, host_rows, idx, cur, UGK_LOC_HOST, num_nodes, output, rb, 0, _status, stream));
+    UGK_CALL(ugk_gather_group(host, host_rows, idx, cur, UGK_LOC_HOST, num_nodes, output, rb, 0, _status,
+                              _host_mirror, stream));
     UGK_CALL(ugk_event_record(_ev_cpu_done, stream));
     UGK_CALL(ugk_gather_group(cache, cache_rows, idx, cur, UGK_LOC_LOCAL, num_nodes, output, rb, 0, _status,
-                              stream));
+                              _host_mirror, stream));
     UGK_CALL(ugk_event_record(_ev_local_done, stream));
   }
-  // counters + status of this lookup -> pinned host, then the single blocking wait of the call
-  UGK_CALL(ugk_memcpy_async(_host_mirror, _state_handle->ptr(), 5 * sizeof(uint32_t), stream));
+  // the single blocking wait of the call; the gathers have written their group sizes (and the kernels any error
+  // flag) into the pinned mirror, so no device-to-host copy is needed
   UGK_CALL(ugk_stream_sync(stream));
-  const uint32_t n_local = _host_mirror[_cur * 2], n_miss = _host_mirror[_cur * 2 + 1];
+  const uint32_t n_local = _host_mirror[1 + UGK_LOC_LOCAL], n_miss = _host_mirror[1 + UGK_LOC_HOST];
   _cur ^= 1;
-  CheckStatusWord(_host_mirror[4]);
+  CheckStatusWord(stream);
   CHECK_EQ((size_t)n_local + n_miss, num_nodes);
   _group_offset[1] = n_local;
   _group_offset[2] = (uint32_t)num_nodes;

@@ -84,7 +84,7 @@ class ExtractSession {
   std::shared_ptr<CacheContext> _cache_ctx;
   MemHandle _idx_handle;          // ugk_idx_t[n], from the caller's allocator, regrown on demand
   MemHandle _state_handle;        // device: two counter pairs + status word
-  MemHandle _host_mirror_handle;  // pinned host: counters + status of the last lookup
+  MemHandle _host_mirror_handle;  // pinned host, written by the kernels: [0] error flag, [1] #local, [2] #host
   uint32_t *_counts[2] = {nullptr, nullptr};
   uint32_t *_status = nullptr;
   uint32_t *_host_mirror = nullptr;
@@ -99,7 +99,7 @@ class ExtractSession {
   template <typename KeyT>
   void ExtractFeatImpl(const KeyT *nodes, size_t num_nodes, void *output, StreamHandle stream, uint64_t task_key);
   void EnsureIdx(size_t num_nodes);
-  void CheckStatusWord(uint32_t st) const;
+  void CheckStatusWord(StreamHandle stream) const;
 
  public:
   ExtractSession(std::shared_ptr<CacheContext> cache_ctx);

@@ -76,12 +76,13 @@ template <typename V, int LPR, int UNROLL, typename Idx>
 __global__ __launch_bounds__(kBlock) void gather_kernel(Idx ix, const V *__restrict__ src, uint64_t src_rows,
                                                         V *__restrict__ out, uint64_t out_rows, uint32_t vpr,
                                                         const uint32_t *__restrict__ counts, uint32_t group, size_t n,
-                                                        uint32_t *status, bool nt_store) {
+                                                        uint32_t *status, uint32_t *host_mirror, bool nt_store) {
   size_t begin = 0, count = n;
   if (counts) {
     const uint32_t c = counts[group];
     count = c;
     begin = (group == UGK_LOC_LOCAL) ? 0 : n - c;
+    if (host_mirror && blockIdx.x == 0 && threadIdx.x == 0) host_mirror[1 + group] = c;
   }
   constexpr int RPB = kBlock / LPR;  // rows copied by one block instruction
   const uint32_t lane = threadIdx.x % LPR;
@@ -101,7 +102,10 @@ __global__ __launch_bounds__(kBlock) void gather_kernel(Idx ix, const V *__restr
         ix.get(begin + r, s[u], d[u]);
         if (s[u] >= src_rows || d[u] >= out_rows) {
           ok[u] = false;
-          if (lane == 0) atomicOr(status, UGK_ST_KEY_OUT_OF_RANGE);
+          if (lane == 0) {
+            atomicOr(status, UGK_ST_KEY_OUT_OF_RANGE);
+            if (host_mirror) host_mirror[0] = UGK_ST_KEY_OUT_OF_RANGE;
+          }
         }
       }
     }
@@ -137,13 +141,13 @@ bool nt_store_for(size_t out_bytes) {
 template <typename V, int LPR, typename Idx>
 int launch_one(Idx ix, const void *src, uint64_t src_rows, void *out, uint64_t out_rows, uint32_t vpr,
                const uint32_t *counts, uint32_t group, size_t n, unsigned max_blocks, uint32_t *status,
-               hipStream_t stream) {
+               uint32_t *host_mirror, hipStream_t stream) {
   constexpr int UNROLL = 2;
   constexpr size_t kPerIter = (size_t)(kBlock / LPR) * UNROLL;
   const unsigned grid = clamp_grid((n + kPerIter - 1) / kPerIter, max_blocks);
   hipLaunchKernelGGL((gather_kernel<V, LPR, UNROLL, Idx>), dim3(grid), dim3(kBlock), 0, stream, ix,
                      reinterpret_cast<const V *>(src), src_rows, reinterpret_cast<V *>(out), out_rows, vpr, counts,
-                     group, n, status, nt_store_for(n * (size_t)vpr * sizeof(V)));
+                     group, n, status, host_mirror, nt_store_for(n * (size_t)vpr * sizeof(V)));
   UGK_HIP(hipGetLastError());
   return 0;
 }
@@ -151,10 +155,11 @@ int launch_one(Idx ix, const void *src, uint64_t src_rows, void *out, uint64_t o
 template <typename V, typename Idx, bool ALL_LPR>
 int launch_vec(Idx ix, const void *src, uint64_t src_rows, void *out, uint64_t out_rows, size_t row_bytes,
                const uint32_t *counts, uint32_t group, size_t n, unsigned max_blocks, uint32_t *status,
-               hipStream_t stream) {
+               uint32_t *host_mirror, hipStream_t stream) {
   const uint32_t vpr = (uint32_t)(row_bytes / sizeof(V));
 #define UGK_GO(L) \
-  return launch_one<V, L, Idx>(ix, src, src_rows, out, out_rows, vpr, counts, group, n, max_blocks, status, stream)
+  return launch_one<V, L, Idx>(ix, src, src_rows, out, out_rows, vpr, counts, group, n, max_blocks, status, host_mirror, \
+                               stream)
   if (ALL_LPR) {
     if (vpr <= 1) UGK_GO(1);
     if (vpr <= 2) UGK_GO(2);
@@ -174,7 +179,7 @@ int launch_vec(Idx ix, const void *src, uint64_t src_rows, void *out, uint64_t o
 template <typename Idx>
 int launch_gather(Idx ix, const void *src, uint64_t src_rows, void *out, uint64_t out_rows, size_t row_bytes,
                   const uint32_t *counts, uint32_t group, size_t n, unsigned max_blocks, uint32_t *status,
-                  void *stream) {
+                  uint32_t *host_mirror, void *stream) {
   if (n == 0) return 0;
   UGK_REQUIRE(src && out, "gather: null source or output");
   UGK_REQUIRE(status, "gather: null status word");
@@ -184,18 +189,21 @@ int launch_gather(Idx ix, const void *src, uint64_t src_rows, void *out, uint64_
   hipStream_t st = as_stream(stream);
   if (align % 16 == 0)
     return launch_vec<u32x4, Idx, true>(ix, src, src_rows, out, out_rows, row_bytes, counts, group, n, max_blocks,
-                                        status, st);
+                                            status, host_mirror, st);
   if (align % 8 == 0)
     return launch_vec<unsigned long long, Idx, false>(ix, src, src_rows, out, out_rows, row_bytes, counts, group, n,
-                                                      max_blocks, status, st);
+                                                      max_blocks,
+                                            status, host_mirror, st);
   if (align % 4 == 0)
     return launch_vec<uint32_t, Idx, false>(ix, src, src_rows, out, out_rows, row_bytes, counts, group, n,
-                                            max_blocks, status, st);
+                                            max_blocks,
+                                            status, host_mirror, st);
   if (align % 2 == 0)
     return launch_vec<uint16_t, Idx, false>(ix, src, src_rows, out, out_rows, row_bytes, counts, group, n,
-                                            max_blocks, status, st);
+                                            max_blocks,
+                                            status, host_mirror, st);
   return launch_vec<uint8_t, Idx, false>(ix, src, src_rows, out, out_rows, row_bytes, counts, group, n, max_blocks,
-                                         status, st);
+                                            status, host_mirror, st);
 }
 
 }  // namespace
@@ -206,17 +214,19 @@ using namespace ugk;
 extern "C" {
 
 int ugk_gather_direct_u32(const void *src_dev, uint64_t src_rows, const uint32_t *keys_dev, size_t n, void *out_dev,
-                          size_t row_bytes, unsigned max_blocks, uint32_t *status_dev, void *stream) {
+                          size_t row_bytes, unsigned max_blocks, uint32_t *status_dev, uint32_t *host_mirror,
+                          void *stream) {
   UGK_REQUIRE(n == 0 || keys_dev, "ugk_gather_direct_u32: null keys");
   return launch_gather(DirectU32{keys_dev}, src_dev, src_rows, out_dev, kNoLimit, row_bytes, nullptr, 0, n,
-                       max_blocks, status_dev, stream);
+                       max_blocks, status_dev, host_mirror, stream);
 }
 
 int ugk_gather_direct_i64(const void *src_dev, uint64_t src_rows, const int64_t *keys_dev, size_t n, void *out_dev,
-                          size_t row_bytes, unsigned max_blocks, uint32_t *status_dev, void *stream) {
+                          size_t row_bytes, unsigned max_blocks, uint32_t *status_dev, uint32_t *host_mirror,
+                          void *stream) {
   UGK_REQUIRE(n == 0 || keys_dev, "ugk_gather_direct_i64: null keys");
   return launch_gather(DirectI64{keys_dev}, src_dev, src_rows, out_dev, kNoLimit, row_bytes, nullptr, 0, n,
-                       max_blocks, status_dev, stream);
+                       max_blocks, status_dev, host_mirror, stream);
 }
 
 int ugk_gather_scatter_u32(const void *src_dev, uint64_t src_rows, const uint32_t *keys_dev,
@@ -224,7 +234,7 @@ int ugk_gather_scatter_u32(const void *src_dev, uint64_t src_rows, const uint32_
                            unsigned max_blocks, uint32_t *status_dev, void *stream) {
   UGK_REQUIRE(n == 0 || (keys_dev && dst_off_dev), "ugk_gather_scatter_u32: null keys or destinations");
   return launch_gather(ScatterU32{keys_dev, dst_off_dev}, src_dev, src_rows, out_dev, out_rows, row_bytes, nullptr, 0,
-                       n, max_blocks, status_dev, stream);
+                       n, max_blocks, status_dev, nullptr, stream);
 }
 
 int ugk_gather_scatter_i64(const void *src_dev, uint64_t src_rows, const int64_t *keys_dev,
@@ -232,23 +242,23 @@ int ugk_gather_scatter_i64(const void *src_dev, uint64_t src_rows, const int64_t
                            unsigned max_blocks, uint32_t *status_dev, void *stream) {
   UGK_REQUIRE(n == 0 || (keys_dev && dst_off_dev), "ugk_gather_scatter_i64: null keys or destinations");
   return launch_gather(ScatterI64{keys_dev, dst_off_dev}, src_dev, src_rows, out_dev, out_rows, row_bytes, nullptr, 0,
-                       n, max_blocks, status_dev, stream);
+                       n, max_blocks, status_dev, nullptr, stream);
 }
 
 int ugk_gather_group(const void *src_dev, uint64_t src_rows, const ugk_idx_t *idx_dev, const uint32_t *counts_dev,
                      uint32_t group, size_t n, void *out_dev, size_t row_bytes, unsigned max_blocks,
-                     uint32_t *status_dev, void *stream) {
+                     uint32_t *status_dev, uint32_t *host_mirror, void *stream) {
   UGK_REQUIRE(n == 0 || (idx_dev && counts_dev), "ugk_gather_group: null index list or counts");
   UGK_REQUIRE(group == UGK_LOC_LOCAL || group == UGK_LOC_HOST, "ugk_gather_group: group %u is not local/host", group);
   return launch_gather(IdxList{idx_dev}, src_dev, src_rows, out_dev, n, row_bytes, counts_dev, group, n, max_blocks,
-                       status_dev, stream);
+                       status_dev, host_mirror, stream);
 }
 
 int ugk_gather_idx(const void *src_dev, uint64_t src_rows, const ugk_idx_t *idx_dev, size_t count, void *out_dev,
                    size_t row_bytes, unsigned max_blocks, uint32_t *status_dev, void *stream) {
   UGK_REQUIRE(count == 0 || idx_dev, "ugk_gather_idx: null index list");
   return launch_gather(IdxList{idx_dev}, src_dev, src_rows, out_dev, kNoLimit, row_bytes, nullptr, 0, count,
-                       max_blocks, status_dev, stream);
+                       max_blocks, status_dev, nullptr, stream);
 }
 
 }  // extern "C"

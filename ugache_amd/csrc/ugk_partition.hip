@@ -20,7 +20,8 @@ constexpr int kWavesPerBlock = kBlock / kWave;
 template <typename K, int KIND>
 __global__ __launch_bounds__(kBlock) void classify_kernel(ugk_table_t t, const K *__restrict__ keys, size_t n,
                                                           uint64_t host_rows, ugk_idx_t *__restrict__ idx,
-                                                          uint32_t *counts, uint32_t *next_counts, uint32_t *status) {
+                                                          uint32_t *counts, uint32_t *next_counts, uint32_t *status,
+                                                          uint32_t *host_mirror) {
   __shared__ uint2 stage[kTile];
   __shared__ uint32_t wave_tot[kItems][kWavesPerBlock][2];
   __shared__ uint32_t base[2];
@@ -54,6 +55,7 @@ __global__ __launch_bounds__(kBlock) void classify_kernel(ugk_table_t t, const K
           o = (uint32_t)key;
         } else {
           atomicOr(status, UGK_ST_KEY_OUT_OF_RANGE);
+          if (host_mirror) host_mirror[0] = UGK_ST_KEY_OUT_OF_RANGE;
         }
       }
       const uint64_t hb = __ballot(c == 1), mb = __ballot(c == 2);
@@ -105,7 +107,7 @@ __global__ __launch_bounds__(kBlock) void extract_mix_kernel(ugk_table_t t, cons
                                                              const u32x4 *__restrict__ cache, uint64_t cache_rows,
                                                              const u32x4 *__restrict__ host, uint64_t host_rows,
                                                              u32x4 *__restrict__ out, uint32_t vpr,
-                                                             uint32_t *status) {
+                                                             uint32_t *status, uint32_t *host_mirror) {
   constexpr int RPW = kWave / LPR;  // rows per wavefront instruction
   constexpr int UNROLL = (RPW * 4 <= kWave) ? 4 : (kWave / RPW);
   const int lane = (int)lane_id();
@@ -122,7 +124,10 @@ __global__ __launch_bounds__(kBlock) void extract_mix_kernel(ugk_table_t t, cons
       if (f.hit && f.loc == UGK_LOC_LOCAL && f.off < cache_rows) rowp = cache + (uint64_t)f.off * vpr;
       else if (f.hit && f.loc == UGK_LOC_HOST && f.off < host_rows) rowp = host + (uint64_t)f.off * vpr;
       else if (!f.hit && key < host_rows) rowp = host + key * vpr;
-      else atomicOr(status, UGK_ST_KEY_OUT_OF_RANGE);
+      else {
+        atomicOr(status, UGK_ST_KEY_OUT_OF_RANGE);
+        if (host_mirror) host_mirror[0] = UGK_ST_KEY_OUT_OF_RANGE;
+      }
     }
     const uint64_t rowbits = reinterpret_cast<uint64_t>(rowp);
     for (int r0 = 0; r0 < kWave; r0 += RPW * UNROLL) {
@@ -225,7 +230,7 @@ size_t dedup_capacity(size_t n) {
 
 template <typename K>
 int classify(ugk_table_t t, const K *keys, size_t n, uint64_t host_rows, ugk_idx_t *idx, uint32_t *counts,
-             uint32_t *next_counts, uint32_t *status, void *stream) {
+             uint32_t *next_counts, uint32_t *status, uint32_t *host_mirror, void *stream) {
   UGK_REQUIRE(counts && status, "ugk_classify: null counters or status");
   UGK_REQUIRE(n <= 0xffffffffull, "ugk_classify: batch of %zu keys exceeds 2^32", n);
   UGK_REQUIRE(t.kind == 1 || t.kind == 2, "ugk_classify: table kind %d is not flat(1) or hash(2)", t.kind);
@@ -238,21 +243,23 @@ int classify(ugk_table_t t, const K *keys, size_t n, uint64_t host_rows, ugk_idx
   const unsigned grid = clamp_grid((n + kTile - 1) / kTile, 0);
   if (t.kind == 1)
     hipLaunchKernelGGL((classify_kernel<K, 1>), dim3(grid), dim3(kBlock), 0, as_stream(stream), t, keys, n, host_rows,
-                       idx, counts, next_counts, status);
+                       idx, counts, next_counts, status, host_mirror);
   else
     hipLaunchKernelGGL((classify_kernel<K, 2>), dim3(grid), dim3(kBlock), 0, as_stream(stream), t, keys, n, host_rows,
-                       idx, counts, next_counts, status);
+                       idx, counts, next_counts, status, host_mirror);
   UGK_HIP(hipGetLastError());
   return 0;
 }
 
 template <typename K, int KIND>
 int extract_mix_lpr(ugk_table_t t, const K *keys, size_t n, const void *cache, uint64_t cache_rows, const void *host,
-                    uint64_t host_rows, void *out, uint32_t vpr, uint32_t *status, hipStream_t st) {
+                    uint64_t host_rows, void *out, uint32_t vpr, uint32_t *status, uint32_t *host_mirror,
+                    hipStream_t st) {
   const unsigned grid = clamp_grid((n + kBlock - 1) / kBlock, 0);
 #define UGK_GO(L)                                                                                                 \
   hipLaunchKernelGGL((extract_mix_kernel<K, KIND, L>), dim3(grid), dim3(kBlock), 0, st, t, keys, n,               \
-                     (const u32x4 *)cache, cache_rows, (const u32x4 *)host, host_rows, (u32x4 *)out, vpr, status)
+                     (const u32x4 *)cache, cache_rows, (const u32x4 *)host, host_rows, (u32x4 *)out, vpr, status, \
+                     host_mirror)
   if (vpr <= 1) UGK_GO(1);
   else if (vpr <= 2) UGK_GO(2);
   else if (vpr <= 4) UGK_GO(4);
@@ -267,7 +274,8 @@ int extract_mix_lpr(ugk_table_t t, const K *keys, size_t n, const void *cache, u
 
 template <typename K>
 int extract_mix(ugk_table_t t, const K *keys, size_t n, const void *cache, uint64_t cache_rows, const void *host,
-                uint64_t host_rows, void *out, size_t row_bytes, uint32_t *status, void *stream) {
+                uint64_t host_rows, void *out, size_t row_bytes, uint32_t *status, uint32_t *host_mirror,
+                void *stream) {
   if (n == 0) return 0;
   UGK_REQUIRE(keys && out && status, "ugk_extract_mix: null keys, output or status");
   UGK_REQUIRE(t.kind == 1 || t.kind == 2, "ugk_extract_mix: table kind %d is not flat(1) or hash(2)", t.kind);
@@ -283,8 +291,10 @@ int extract_mix(ugk_table_t t, const K *keys, size_t n, const void *cache, uint6
               "ugk_extract_mix: rows and buffers must be multiples of 16 bytes (row_bytes=%zu)", row_bytes);
   const uint32_t vpr = (uint32_t)(row_bytes / 16);
   if (t.kind == 1)
-    return extract_mix_lpr<K, 1>(t, keys, n, cache, cache_rows, host, host_rows, out, vpr, status, as_stream(stream));
-  return extract_mix_lpr<K, 2>(t, keys, n, cache, cache_rows, host, host_rows, out, vpr, status, as_stream(stream));
+    return extract_mix_lpr<K, 1>(t, keys, n, cache, cache_rows, host, host_rows, out, vpr, status, host_mirror,
+                                 as_stream(stream));
+  return extract_mix_lpr<K, 2>(t, keys, n, cache, cache_rows, host, host_rows, out, vpr, status, host_mirror,
+                               as_stream(stream));
 }
 
 template <typename K>
@@ -315,25 +325,29 @@ using namespace ugk;
 extern "C" {
 
 int ugk_classify_u32(ugk_table_t t, const uint32_t *keys_dev, size_t n, uint64_t host_rows, ugk_idx_t *idx_dev,
-                     uint32_t *counts_dev, uint32_t *next_counts_dev, uint32_t *status_dev, void *stream) {
-  return classify<uint32_t>(t, keys_dev, n, host_rows, idx_dev, counts_dev, next_counts_dev, status_dev, stream);
+                     uint32_t *counts_dev, uint32_t *next_counts_dev, uint32_t *status_dev, uint32_t *host_mirror,
+                     void *stream) {
+  return classify<uint32_t>(t, keys_dev, n, host_rows, idx_dev, counts_dev, next_counts_dev, status_dev, host_mirror,
+                            stream);
 }
 int ugk_classify_i64(ugk_table_t t, const int64_t *keys_dev, size_t n, uint64_t host_rows, ugk_idx_t *idx_dev,
-                     uint32_t *counts_dev, uint32_t *next_counts_dev, uint32_t *status_dev, void *stream) {
-  return classify<int64_t>(t, keys_dev, n, host_rows, idx_dev, counts_dev, next_counts_dev, status_dev, stream);
+                     uint32_t *counts_dev, uint32_t *next_counts_dev, uint32_t *status_dev, uint32_t *host_mirror,
+                     void *stream) {
+  return classify<int64_t>(t, keys_dev, n, host_rows, idx_dev, counts_dev, next_counts_dev, status_dev, host_mirror,
+                           stream);
 }
 
 int ugk_extract_mix_u32(ugk_table_t t, const uint32_t *keys_dev, size_t n, const void *cache_dev, uint64_t cache_rows,
                         const void *host_dev, uint64_t host_rows, void *out_dev, size_t row_bytes,
-                        uint32_t *status_dev, void *stream) {
+                        uint32_t *status_dev, uint32_t *host_mirror, void *stream) {
   return extract_mix<uint32_t>(t, keys_dev, n, cache_dev, cache_rows, host_dev, host_rows, out_dev, row_bytes,
-                               status_dev, stream);
+                               status_dev, host_mirror, stream);
 }
 int ugk_extract_mix_i64(ugk_table_t t, const int64_t *keys_dev, size_t n, const void *cache_dev, uint64_t cache_rows,
                         const void *host_dev, uint64_t host_rows, void *out_dev, size_t row_bytes,
-                        uint32_t *status_dev, void *stream) {
+                        uint32_t *status_dev, uint32_t *host_mirror, void *stream) {
   return extract_mix<int64_t>(t, keys_dev, n, cache_dev, cache_rows, host_dev, host_rows, out_dev, row_bytes,
-                              status_dev, stream);
+                              status_dev, host_mirror, stream);
 }
 
 size_t ugk_dedup_workspace_bytes(size_t n) { return dedup_capacity(n) * 8 + ((n + 1) / 2 * 2) * 4 + 64; }
