@@ -23,6 +23,10 @@ for p in (ROOT, os.path.join(ROOT, "ugache_amd"), os.path.join(ROOT, "tests")):
 
 HBM_PEAK_GBPS = 8000.0  # MI355X published HBM3E bandwidth
 
+# HBM-side bytes per launch of the dominant kernel, from the FETCH_SIZE / WRITE_SIZE counter runs summarised in
+# profiles/gather_kernel_c2_all_hit.md (each counter scaled by its reading for a 1 GiB copy kernel)
+MEASURED_TRAFFIC_BYTES = {"c2_all_hit_10Mx128xfp32_262144_u32_uniform": 270_550_000}
+
 WORKLOADS = {
     # name: (rows, dim, keys per batch, key dtype)
     "c2_all_hit_10Mx128xfp32_262144_u32_uniform": (10_000_000, 128, 262_144, "u32"),
@@ -166,7 +170,7 @@ def main():
         "parity": "bit-exact vs CPU oracle (last timed batch)",
         "device": info["name"] + " " + info["arch"],
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-                     "frac": achieved / HBM_PEAK_GBPS, "traffic": None, "kernel": "gather_kernel<u32x4,32,2,DirectU32>",
+                     "frac": achieved / HBM_PEAK_GBPS, "traffic": MEASURED_TRAFFIC_BYTES.get(args.workload), "kernel": "gather_kernel<u32x4,32,2,DirectU32>",
                      "algorithmic_bytes_per_launch": alg_bytes, "avg_kernel_us": kernel_avg_s * 1e6,
                      "keys_per_s_kernel_only": n_keys / kernel_avg_s},
         "cpu_baseline": {"value": cpu_keys_per_s, "unit": "keys/s", "cores": cores, "kind": "port",
