@@ -96,6 +96,9 @@ int ugk_host_free(void *ptr);
 /* kind: 0 = ordinary host memory (kernels cannot read it), 1 = pinned host, 2 = device */
 int ugk_pointer_kind(const void *ptr, int *kind);
 int ugk_stream_create(void **stream);
+/* stream whose kernels run on `num_cus` compute units only (the counterpart of the reference's SM-masked contexts
+ * for the host source, mps_util.h:36-49 / cache_context.cu:4208-4218); default priority */
+int ugk_stream_create_cu_masked(void **stream, int num_cus);
 int ugk_stream_destroy(void *stream);
 int ugk_stream_sync(void *stream);
 int ugk_device_sync(void);

@@ -199,7 +199,13 @@ ExtractSession::ExtractSession(std::shared_ptr<CacheContext> cache_ctx) : _cache
   const int dev = _cache_ctx->_trainer_ctx.device_id;
   UGK_CALL(ugk_set_device(dev));
   UGK_CALL(ugk_stream_create(&_local_ext_stream));
-  UGK_CALL(ugk_stream_create(&_cpu_ext_stream));
+  const auto &link_desc = RunConfig::coll_cache_link_desc;
+  const int cpu_cus = link_desc.cpu_cu.empty() ? 0 : link_desc.cpu_cu[0];
+  if (cpu_cus > 0) {
+    UGK_CALL(ugk_stream_create_cu_masked(&_cpu_ext_stream, cpu_cus));
+  } else {
+    UGK_CALL(ugk_stream_create(&_cpu_ext_stream));
+  }
   UGK_CALL(ugk_event_create(&_ev_classified));
   UGK_CALL(ugk_event_create(&_ev_local_done));
   UGK_CALL(ugk_event_create(&_ev_cpu_done));
@@ -356,17 +362,29 @@ void ExtractSession::ExtractFeatImpl(const KeyT *nodes, size_t num_nodes, void *
   UGK_CALL(Classify(table, nodes, num_nodes, host_rows, idx, cur, next, _status, _host_mirror, stream));
   UGK_CALL(ugk_event_record(_ev_classified, stream));
   if (RunConfig::concurrent_link_impl == kSMMaskPhase) {
-    // factored extraction: the host-link gather gets a few workgroups on its own stream, the HBM gather
-    // the rest of the chip on another; both read their group bounds from the device-side counters
-    UGK_CALL(ugk_stream_wait_event(_cpu_ext_stream, _ev_classified));
-    UGK_CALL(ugk_gather_group(host, host_rows, idx, cur, UGK_LOC_HOST, num_nodes, output, rb, _cpu_blocks, _status,
-                              _host_mirror, _cpu_ext_stream));
-    UGK_CALL(ugk_event_record(_ev_cpu_done, _cpu_ext_stream));
+    // factored extraction: two concurrent kernels that read their group bounds from the device-side counters.
+    // A long host-link gather runs on the stream confined to a few CUs, so its slow loads do not clog the memory
+    // pipelines the HBM gather needs; the HBM gather then stays on the caller's stream.  A short host-link gather
+    // (decided from the previous batch) stays on the caller's stream right behind the classify kernel instead, which
+    // saves the cross-stream hand-off on the critical path.
+    // The HBM gather always runs on a library stream created non-blocking: the confined stream cannot be created
+    // that way, so a caller passing the legacy null stream would otherwise see its HBM gather serialised behind
+    // the host-link gather by the null stream's implicit synchronisation.
+    if (_host_on_main) {
+      UGK_CALL(ugk_gather_group(host, host_rows, idx, cur, UGK_LOC_HOST, num_nodes, output, rb, _cpu_blocks_inline,
+                                _status, _host_mirror, stream));
+      UGK_CALL(ugk_event_record(_ev_cpu_done, stream));
+    } else {
+      UGK_CALL(ugk_stream_wait_event(_cpu_ext_stream, _ev_classified));
+      UGK_CALL(ugk_gather_group(host, host_rows, idx, cur, UGK_LOC_HOST, num_nodes, output, rb, _cpu_blocks, _status,
+                                _host_mirror, _cpu_ext_stream));
+      UGK_CALL(ugk_event_record(_ev_cpu_done, _cpu_ext_stream));
+    }
     UGK_CALL(ugk_stream_wait_event(_local_ext_stream, _ev_classified));
     UGK_CALL(ugk_gather_group(cache, cache_rows, idx, cur, UGK_LOC_LOCAL, num_nodes, output, rb, 0, _status,
                               _host_mirror, _local_ext_stream));
     UGK_CALL(ugk_event_record(_ev_local_done, _local_ext_stream));
-    UGK_CALL(ugk_stream_wait_event(stream, _ev_cpu_done));
+    if (!_host_on_main) UGK_CALL(ugk_stream_wait_event(stream, _ev_cpu_done));
     UGK_CALL(ugk_stream_wait_event(stream, _ev_local_done));
   } else {
     // sequential: host group, then local group (cache_context.cu:1719-1792)
@@ -387,14 +405,16 @@ void ExtractSession::ExtractFeatImpl(const KeyT *nodes, size_t num_nodes, void *
   _group_offset[1] = n_local;
   _group_offset[2] = (uint32_t)num_nodes;
 
+  float ms_idx = 0, ms_miss = 0, ms_local = 0;
+  UGK_CALL(ugk_event_elapsed_ms(_ev_t[0], _ev_classified, &ms_idx));
+  UGK_CALL(ugk_event_elapsed_ms(_ev_classified, _ev_cpu_done, &ms_miss));
+  if (RunConfig::concurrent_link_impl == kSMMaskPhase) {
+    UGK_CALL(ugk_event_elapsed_ms(_ev_classified, _ev_local_done, &ms_local));
+    _host_on_main = ms_miss < 0.25f;  // placement of the next batch's host-link gather
+  } else {
+    UGK_CALL(ugk_event_elapsed_ms(_ev_cpu_done, _ev_local_done, &ms_local));
+  }
   if (profiler && task_key != 0xffffffffffffffffull) {
-    float ms_idx = 0, ms_miss = 0, ms_local = 0;
-    UGK_CALL(ugk_event_elapsed_ms(_ev_t[0], _ev_classified, &ms_idx));
-    UGK_CALL(ugk_event_elapsed_ms(_ev_classified, _ev_cpu_done, &ms_miss));
-    if (RunConfig::concurrent_link_impl == kSMMaskPhase)
-      UGK_CALL(ugk_event_elapsed_ms(_ev_classified, _ev_local_done, &ms_local));
-    else
-      UGK_CALL(ugk_event_elapsed_ms(_ev_cpu_done, _ev_local_done, &ms_local));
     profiler->LogStep(task_key, kLogL1FeatureBytes, nbytes);
     profiler->LogStep(task_key, kLogL1MissBytes, (double)n_miss * rb);
     profiler->LogStep(task_key, kLogL1RemoteBytes, 0);

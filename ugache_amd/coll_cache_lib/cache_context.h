@@ -93,7 +93,9 @@ class ExtractSession {
   StreamHandle _cpu_ext_stream = nullptr;
   void *_ev_classified = nullptr, *_ev_local_done = nullptr, *_ev_cpu_done = nullptr;
   void *_ev_t[4] = {nullptr, nullptr, nullptr, nullptr};
-  unsigned _cpu_blocks = 32;
+  unsigned _cpu_blocks = 32;        // workgroups of the host-link gather on its own (CU-confined) stream
+  unsigned _cpu_blocks_inline = 32; // ... when it runs on the caller's stream instead
+  bool _host_on_main = false;  // host-link gather on the caller's stream (short miss groups) or on the confined stream
   uint32_t _group_offset[3] = {0, 0, 0};
 
   template <typename KeyT>

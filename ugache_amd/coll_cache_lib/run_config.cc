@@ -83,10 +83,19 @@ AsymmLinkDesc AsymmLinkDesc::AutoBuild(Context ctx) {
   UGK_CALL(ugk_get_device_info(ctx.device_id, &info));
   desc.gpu_model = info.name;
   desc.link_src.assign(RunConfig::num_device, {});
-  int cpu_blocks = 32;
+  // The host-link gather runs on a stream confined to a few CUs (COLL_CPU_CU_NUM, default 8, 0 = unconfined) and
+  // is launched with COLL_CPU_SM_NUM_OVERRIDE workgroups (default 128 when confined, 32 otherwise).  Measured on
+  // MI355X: 64-256 workgroups packed on 8 CUs read the host table at 95 % of the link while the HBM gather next to
+  // it keeps its speed; the same workgroups spread over the chip slow the HBM gather down 5-10x.
+  int cpu_cus = 8;
+  if (GetEnv("COLL_CPU_CU_NUM") != "") cpu_cus = std::stoi(GetEnv("COLL_CPU_CU_NUM"));
+  CHECK_GE(cpu_cus, 0);
+  CHECK_LE(cpu_cus, info.compute_units);
+  int cpu_blocks = cpu_cus > 0 ? 128 : 32;
   if (GetEnv("COLL_CPU_SM_NUM_OVERRIDE") != "") cpu_blocks = std::stoi(GetEnv("COLL_CPU_SM_NUM_OVERRIDE"));
   CHECK_GT(cpu_blocks, 0);
   desc.cpu_sm.assign(RunConfig::num_device, cpu_blocks);
+  desc.cpu_cu.assign(RunConfig::num_device, cpu_cus);
   desc.local_sm.assign(RunConfig::num_device, 0);
   desc.local_bw_GBps = 8000;
   desc.cpu_bw_GBps = 50;

@@ -25,6 +25,7 @@ namespace coll_cache {
 struct AsymmLinkDesc {
   std::vector<std::vector<std::vector<int>>> link_src;  // [dst gpu][link][src gpus]; empty lists with one GPU
   std::vector<int> cpu_sm;     // workgroups given to the host-miss gather (the reference counts SMs)
+  std::vector<int> cpu_cu;     // compute units the host-miss gather is confined to (0 = no confinement)
   std::vector<int> local_sm;   // 0 = fill the chip
   double local_bw_GBps = 0;    // HBM
   double cpu_bw_GBps = 0;      // host link

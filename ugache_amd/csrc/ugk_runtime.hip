@@ -167,6 +167,20 @@ int ugk_stream_create(void **stream) {
   return 0;
 }
 
+int ugk_stream_create_cu_masked(void **stream, int num_cus) {
+  UGK_REQUIRE(stream, "ugk_stream_create_cu_masked: null output");
+  const int total = cu_count();
+  UGK_REQUIRE(num_cus > 0 && num_cus <= total, "ugk_stream_create_cu_masked: %d CUs requested, device has %d", num_cus,
+              total);
+  uint32_t mask[32] = {0};
+  UGK_REQUIRE(total <= 32 * 32, "ugk_stream_create_cu_masked: device reports %d CUs", total);
+  for (int i = 0; i < num_cus; ++i) mask[i / 32] |= 1u << (i % 32);
+  hipStream_t s;
+  UGK_HIP(hipExtStreamCreateWithCUMask(&s, (uint32_t)((total + 31) / 32), mask));
+  *stream = s;
+  return 0;
+}
+
 int ugk_stream_destroy(void *stream) {
   if (stream) UGK_HIP(hipStreamDestroy(as_stream(stream)));
   return 0;

@@ -53,6 +53,7 @@ SIGNATURES = {
     "ugk_host_free": [_vp],
     "ugk_pointer_kind": [_vp, C.POINTER(_i)],
     "ugk_stream_create": [C.POINTER(_vp)],
+    "ugk_stream_create_cu_masked": [C.POINTER(_vp), _i],
     "ugk_stream_destroy": [_vp],
     "ugk_stream_sync": [_vp],
     "ugk_device_sync": [],
