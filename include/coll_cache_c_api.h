@@ -75,6 +75,11 @@ void coll_cache_init_ranked_c(int replica_id, size_t key_space_size, const uint3
  * (coll_cache_lib/constant.h:28). */
 void coll_cache_lookup_i64(int replica_id, const int64_t *key, size_t num_keys, void *output, StreamHandle stream);
 void coll_cache_record_i64(int replica_id, const int64_t *key, size_t num_keys);
+/* Sparse-id mode (extension; call after coll_cache_config and before recording or building): the caller's id of
+ * host row r is (r * mul) mod 2^bits with mul odd, so 64-bit hashed ids from a 2^bits space address a dense host table
+ * of num_total_item rows.  Cached ids live in the open-addressing GPU table; a missed id is turned back into its row
+ * with the modular inverse.  mul == 0 restores plain row-number keys.  Lookups and records then take int64 ids. */
+void coll_cache_set_key_map(uint64_t mul, int bits);
 /* LookupManager::refresh (python_tf2/collcache_tf2/collcache_tf2/core/lookup_manager.cc:317-333) ->
  * CollCache::refresh (coll_cache_lib/facade.cc:513-557): re-rank by the hotness recorded since the last
  * build/refresh, evict and insert.  foreground != 0 skips the wait for an in-flight lookup and the throttling. */
@@ -90,7 +95,7 @@ void coll_cache_set_max_num_keys(size_t n);
  * (coll_cache_lib/cache_context.cu:825-847) */
 void coll_cache_last_group_offset(int replica_id, uint32_t out[3]);
 /* out[0] cache capacity in rows, [1] cached rows, [2] lookup table kind (0 none/direct, 1 flat, 2 open addressing),
- * [3] row bytes, [4] key space, [5] completed lookups, [6] free cache slots, [7] reserved */
+ * [3] row bytes, [4] key space, [5] completed lookups, [6] free cache slots, [7] lookup-table rebuilds so far */
 void coll_cache_get_info(int replica_id, uint64_t out[8]);
 /* cached keys of replica_id (ascending): copies up to `capacity` keys, returns the number cached */
 size_t coll_cache_get_cached_keys(int replica_id, uint32_t *out, size_t capacity);

@@ -66,6 +66,11 @@ typedef struct {
   int32_t reserved;
   void *table;
   uint64_t size; /* flat: number of keys; hash: number of buckets */
+  /* host row of a key the table does not hold: key itself when fb_mul == 0 (the reference's CPUFallback,
+   * cache_hashtable.cuh:388-395), else (key * fb_mul) & fb_mask — the inverse of an odd-multiplier bijection on
+   * 2^k ids, which lets sparse hashed ids address a dense host table without a second table */
+  uint64_t fb_mul;
+  uint64_t fb_mask;
 } ugk_table_t;
 
 typedef struct {

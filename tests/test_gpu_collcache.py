@@ -249,3 +249,63 @@ def test_reference_cpu_runnable_config_full_size():
         assert out.shape == (n, dim)
         assert out.cpu().numpy().tobytes() == ORC.gather(table, b.astype(np.int64), omp=True).tobytes()
         assert _basics.last_group_offset(0) == [0, int((nid[b] == 0).sum()), n]
+
+
+def test_sparse_ids_hash_table_with_refresh_each_step(monkeypatch):
+    """The hashtable-mode configuration, scaled down: ids are 64-bit values from a 2^40 space (id = row * odd mod 2^40),
+    rows are 64 fp16 (128 B), the cached ids sit in the open-addressing table at 0.7 load, every step is followed by a
+    refresh that evicts / inserts by the newly recorded hotness; tombstones trigger table rebuilds on the way."""
+    monkeypatch.setenv("COLL_HASH_REBUILD_FRAC", "0.05")
+    MUL, BITS = 0x9E3779B97F4A7C15, 40
+    mask = np.uint64((1 << BITS) - 1)
+    rng = np.random.default_rng(5)
+    n_item, dim, pct, n = 400_000, 64, 0.10, 100_000
+
+    def ids_of(rows):
+        return ((rows.astype(np.uint64) * np.uint64(MUL)) & mask).astype(np.int64)
+
+    co.config(make_config(n_item, pct))
+    _basics.set_key_map(MUL, BITS)
+    co.coll_cache_record_init(0)
+    perm = rng.permutation(n_item)
+
+    def stream(k):
+        return [perm[zipf_ranks(rng, n, n_item, 1.05)] for _ in range(k)]
+
+    s0 = stream(4)
+    for b in s0:
+        co.coll_torch_record(0, torch.from_numpy(ids_of(b)))
+    emb = co.coll_torch_create_emb_shm(0, n_item, dim, torch.float16)
+    table = fill_table(emb, rng)
+    co.coll_torch_init_t(0, 0, emb, pct)
+    info = _basics.info(0)
+    assert info["table_kind"] == 2 and info["row_bytes"] == 128
+    cached, nid = expected_cached_set(np.concatenate(s0).astype(np.uint32), n_item, pct)
+    cap = info["capacity_rows"]
+    assert info["cached_rows"] == len(cached)
+
+    rebuilds = 0
+    for step in range(6):
+        rows_b = perm[zipf_ranks(rng, n, n_item, 1.05)]
+        keys = torch.from_numpy(ids_of(rows_b)).cuda()
+        assert int(keys.max()) > (1 << 32)  # genuinely wide ids
+        out = co.coll_torch_lookup_key_t_val_ret(0, keys, False)
+        assert out.dtype == torch.float16 and out.shape == (n, dim)
+        assert out.cpu().numpy().tobytes() == ORC.gather(table, rows_b.astype(np.int64)).tobytes()
+        assert _basics.last_group_offset(0) == [0, int((nid[rows_b] == 0).sum()), n]
+        # hotness drifts: part of the permutation is reshuffled, then re-ranked from what was recorded since
+        swap = rng.choice(n_item, n_item // 50, replace=False)
+        perm[swap] = perm[rng.permutation(swap)]
+        s = stream(3)
+        for b in s:
+            co.coll_torch_record(0, torch.from_numpy(ids_of(b)))
+        co.coll_torch_refresh(0, True)
+        new_cached, nid = expected_cached_set(np.concatenate(s).astype(np.uint32), n_item, pct)
+        info = _basics.info(0)
+        got = np.zeros(len(new_cached), np.uint32)
+        assert _basics.C_LIB_CTYPES.coll_cache_get_cached_keys(0, got.ctypes.data, len(got)) == len(new_cached)
+        assert np.array_equal(got, new_cached)  # reported as row numbers
+        assert info["free_slots"] + info["cached_rows"] == cap
+        rebuilds = info["table_rebuilds"]
+        cached = new_cached
+    assert rebuilds >= 1

@@ -121,6 +121,10 @@ void CacheContext::build_with_advise_new_hash(int location_id, std::shared_ptr<C
                   num_total_nodes * sizeof(IdType) <= ((size_t)256 << 20);
   if (RunConfig::force_table_kind == 1) use_flat = true;
   if (RunConfig::force_table_kind == 2) use_flat = false;
+  if (RunConfig::key_map_mul != 0) {
+    CHECK(RunConfig::force_table_kind != 1) << "sparse ids cannot index a flat table";
+    use_flat = false;
+  }
   if (use_flat) {
     _new_hash_table->CreateFlat(_eager_gpu_mem_allocator, num_total_nodes, stream);
   } else {
@@ -136,7 +140,11 @@ void CacheContext::build_with_advise_new_hash(int location_id, std::shared_ptr<C
     UGK_CALL(ugk_gather_direct_u32(cpu_data, num_total_nodes, cache_node_list->CPtr<uint32_t>(), num_cached_nodes,
                                    _device_cache_data[_local_location_id], _row_bytes, 0, st->ptr<uint32_t>(),
                                    nullptr, stream));
-    _new_hash_table->InsertSeqOffWithLoc(cache_node_list, location_id, stream);
+    auto table_keys = RunConfig::key_map_mul == 0
+                          ? cache_node_list
+                          : _new_hash_table->TableKeysToDevice(keys_for_each_source[location_id],
+                                                               _eager_gpu_mem_allocator, _trainer_ctx, stream);
+    _new_hash_table->InsertSeqOffWithLoc(table_keys, location_id, stream);
     uint32_t fill_status = 0;
     UGK_CALL(ugk_memcpy_async(&fill_status, st->ptr(), sizeof(fill_status), stream));
     UGK_CALL(ugk_stream_sync(stream));
@@ -180,6 +188,8 @@ void CacheContext::build(std::function<MemHandle(size_t)> gpu_mem_allocator, int
   const int dev = gpu_ctx.device_id;
   _eager_gpu_mem_allocator = [dev](size_t nbytes) -> MemHandle { return EagerGPUAlloc(dev, nbytes); };
 
+  CHECK(RunConfig::key_map_mul == 0 || (cache_percentage != 0 && cache_percentage != 1))
+      << "sparse-id mode needs a partial cache (the direct-mapping paths index the table by key)";
   if (cache_percentage == 0) {
     return build_no_cache(location_id, coll_cache_ptr, cpu_data, dtype, dim, gpu_ctx, stream);
   } else if (cache_percentage == 1) {
@@ -428,6 +438,8 @@ void ExtractSession::ExtractFeatImpl(const KeyT *nodes, size_t num_nodes, void *
 
 void ExtractSession::ExtractFeat(const IdType *nodes, const size_t num_nodes, void *output, StreamHandle stream,
                                  uint64_t task_key) {
+  CHECK(RunConfig::key_map_mul == 0 || RunConfig::key_map_mask <= 0xffffffffull)
+      << "sparse ids wider than 32 bits need the 64-bit lookup";
   ExtractFeatImpl<IdType>(nodes, num_nodes, output, stream, task_key);
 }
 
@@ -513,7 +525,9 @@ void RefreshSession::refresh_after_solve_new(bool foreground) {
   const size_t num_evicted = new_evict_keys->NumItem();
   CHECK_EQ(num_evicted + num_preserved_key, table->_cached_keys->NumItem());
   if (num_evicted > 0) {
-    auto evict_keys_gpu = CopyTo1DReuse(__keys_buffer, new_evict_keys, gpu_ctx, stream);
+    auto evict_keys_gpu = RunConfig::key_map_mul == 0
+                              ? CopyTo1DReuse(__keys_buffer, new_evict_keys, gpu_ctx, stream)
+                              : table->TableKeysToDevice(new_evict_keys, ctx->_eager_gpu_mem_allocator, gpu_ctx, stream);
     auto evict_offs_gpu = Empty1DReuse(__offs_buffer, kI32, {num_evicted}, gpu_ctx);
     table->LookupOffset(evict_keys_gpu, evict_offs_gpu, stream);
     TensorPtr evict_offs_cpu = Tensor::Empty(kI32, {num_evicted}, CPU_CLIB(), "");
@@ -566,13 +580,18 @@ void RefreshSession::refresh_after_solve_new(bool foreground) {
     UGK_CALL(ugk_memcpy_async(&st, status, sizeof(st), low_pri_stream));
     UGK_CALL(ugk_stream_sync(low_pri_stream));
     CHECK_EQ(st, 0u) << "refresh row copy touched a row outside its table";
-    table->InsertWithLoc(insert_keys_gpu, reserved_offset, local, stream);
+    auto insert_table_keys =
+        RunConfig::key_map_mul == 0
+            ? insert_keys_gpu
+            : table->TableKeysToDevice(new_insert_keys, ctx->_eager_gpu_mem_allocator, gpu_ctx, stream);
+    table->InsertWithLoc(insert_table_keys, reserved_offset, local, stream);
     table->CheckStatus(stream, "refresh insert");
   }
   AnonymousBarrier::_refresh_instance->Wait();
 
   table->_cached_keys = key_list_of_each_src[local];
   ctx->_cache_nodes = num_new_local_key;
+  table->MaybeRebuild(ctx->_eager_gpu_mem_allocator, gpu_ctx, local, stream);
   CHECK_EQ(table->_free_offsets->NumItem() + num_new_local_key, ctx->_cache_space_capacity);
 }
 

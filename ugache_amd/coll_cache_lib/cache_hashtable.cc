@@ -20,7 +20,7 @@ void CacheEntryManager::CreateFlat(const std::function<MemHandle(size_t)> &alloc
   LOG(INFO) << "flat lookup table over " << num_keys << " keys, " << ToReadableSize(num_keys * sizeof(IdType));
   _table_handle = allocator(num_keys * sizeof(IdType));
   CHECK_NOTNULL(_table_handle);
-  _table = {1, 0, _table_handle->ptr(), num_keys};
+  _table = {1, 0, _table_handle->ptr(), num_keys, 0, 0};
   UGK_CALL(ugk_fill_u32(_table_handle->ptr<uint32_t>(), kEmptyPos, num_keys, stream));
   RunConfig::use_flat_hashtable = true;
 }
@@ -33,31 +33,78 @@ void CacheEntryManager::CreateHash(const std::function<MemHandle(size_t)> &alloc
   _table_handle = allocator(nb * sizeof(ugk_bucket_t) + 128);
   CHECK_NOTNULL(_table_handle);
   void *base = Align128(_table_handle->ptr());
-  _table = {2, 0, base, nb};
+  _table = {2, 0, base, nb, RunConfig::key_map_inv, RunConfig::key_map_mask};
   UGK_CALL(ugk_hash_init(static_cast<ugk_bucket_t *>(base), nb, stream));
   RunConfig::use_flat_hashtable = false;
 }
 
+TensorPtr CacheEntryManager::TableKeysToDevice(TensorPtr host_rows, const std::function<MemHandle(size_t)> &allocator,
+                                               Context ctx, StreamHandle stream) {
+  if (RunConfig::key_map_mul == 0) return Tensor::CopyToExternal(host_rows, allocator, ctx, stream);
+  const size_t n = host_rows->NumItem();
+  TensorPtr ids = Tensor::Empty(kI64, {n}, CPU_CLIB(), "");
+  const IdType *rows = host_rows->CPtr<IdType>();
+  int64_t *out = ids->Ptr<int64_t>();
+#pragma omp parallel for num_threads(std::max(1, RunConfig::solver_omp_thread_num_per_gpu)) if (n > 65536)
+  for (size_t i = 0; i < n; i++) out[i] = (int64_t)RunConfig::KeyOfRow(rows[i]);
+  return Tensor::CopyToExternal(ids, allocator, ctx, stream);
+}
+
 void CacheEntryManager::LookupOffset(TensorPtr keys, TensorPtr off, StreamHandle stream) {
   CHECK_EQ(keys->NumItem(), off->NumItem());
-  UGK_CALL(ugk_table_lookup_u32(_table, keys->CPtr<uint32_t>(), keys->NumItem(), (uint32_t)cpu_location_id, nullptr,
-                                off->Ptr<uint32_t>(), stream));
+  if (keys->Type() == kI64)
+    UGK_CALL(ugk_table_lookup_i64(_table, keys->CPtr<int64_t>(), keys->NumItem(), (uint32_t)cpu_location_id, nullptr,
+                                  off->Ptr<uint32_t>(), stream));
+  else
+    UGK_CALL(ugk_table_lookup_u32(_table, keys->CPtr<uint32_t>(), keys->NumItem(), (uint32_t)cpu_location_id, nullptr,
+                                  off->Ptr<uint32_t>(), stream));
 }
 
 void CacheEntryManager::InsertWithLoc(TensorPtr keys, TensorPtr off, int loc, StreamHandle stream) {
   CHECK_EQ(keys->NumItem(), off->NumItem());
-  UGK_CALL(ugk_table_insert_u32(_table, keys->CPtr<uint32_t>(), off->CPtr<uint32_t>(), 0, (uint32_t)loc,
-                                keys->NumItem(), StatusPtr(this, stream), stream));
+  if (keys->Type() == kI64)
+    UGK_CALL(ugk_table_insert_i64(_table, keys->CPtr<int64_t>(), off->CPtr<uint32_t>(), 0, (uint32_t)loc,
+                                  keys->NumItem(), StatusPtr(this, stream), stream));
+  else
+    UGK_CALL(ugk_table_insert_u32(_table, keys->CPtr<uint32_t>(), off->CPtr<uint32_t>(), 0, (uint32_t)loc,
+                                  keys->NumItem(), StatusPtr(this, stream), stream));
 }
 
 void CacheEntryManager::InsertSeqOffWithLoc(TensorPtr keys, int loc, StreamHandle stream) {
-  UGK_CALL(ugk_table_insert_u32(_table, keys->CPtr<uint32_t>(), nullptr, 0, (uint32_t)loc, keys->NumItem(),
-                                StatusPtr(this, stream), stream));
+  if (keys->Type() == kI64)
+    UGK_CALL(ugk_table_insert_i64(_table, keys->CPtr<int64_t>(), nullptr, 0, (uint32_t)loc, keys->NumItem(),
+                                  StatusPtr(this, stream), stream));
+  else
+    UGK_CALL(ugk_table_insert_u32(_table, keys->CPtr<uint32_t>(), nullptr, 0, (uint32_t)loc, keys->NumItem(),
+                                  StatusPtr(this, stream), stream));
 }
 
 void CacheEntryManager::Evict(TensorPtr keys_to_evict, StreamHandle stream) {
-  UGK_CALL(ugk_table_evict_u32(_table, keys_to_evict->CPtr<uint32_t>(), keys_to_evict->NumItem(),
-                               StatusPtr(this, stream), stream));
+  if (keys_to_evict->Type() == kI64)
+    UGK_CALL(ugk_table_evict_i64(_table, keys_to_evict->CPtr<int64_t>(), keys_to_evict->NumItem(),
+                                 StatusPtr(this, stream), stream));
+  else
+    UGK_CALL(ugk_table_evict_u32(_table, keys_to_evict->CPtr<uint32_t>(), keys_to_evict->NumItem(),
+                                 StatusPtr(this, stream), stream));
+  if (_table.kind == 2) _num_tombstones += keys_to_evict->NumItem();
+}
+
+bool CacheEntryManager::MaybeRebuild(const std::function<MemHandle(size_t)> &allocator, Context ctx, int loc,
+                                     StreamHandle stream) {
+  if (_table.kind != 2) return false;
+  if ((double)_num_tombstones <= RunConfig::hash_rebuild_tombstone_frac * (double)_table.size) return false;
+  const size_t n = _cached_keys->NumItem();
+  LOG(INFO) << "rebuilding the lookup table: " << _num_tombstones << " tombstones in " << _table.size << " buckets, "
+            << n << " live keys";
+  TensorPtr keys = TableKeysToDevice(_cached_keys, allocator, ctx, stream);
+  TensorPtr offs = Tensor::EmptyExternal(kI32, {n}, allocator, ctx, "");
+  if (n > 0) LookupOffset(keys, offs, stream);
+  UGK_CALL(ugk_hash_init(static_cast<ugk_bucket_t *>(_table.table), _table.size, stream));
+  if (n > 0) InsertWithLoc(keys, offs, loc, stream);
+  CheckStatus(stream, "table rebuild");
+  _num_tombstones = 0;
+  _num_rebuilds++;
+  return true;
 }
 
 void CacheEntryManager::CheckStatus(StreamHandle stream, const char *what) {

@@ -37,7 +37,7 @@ class CacheEntryManager {
   TensorPtr _cached_keys;   // host, u32: keys currently cached on this GPU
   TensorPtr _remote_keys;   // always empty with one GPU
   TensorPtr _free_offsets;  // host, u32: free cache slots, allocation sized for the whole capacity
-  ugk_table_t _table = {0, 0, nullptr, 0};
+  ugk_table_t _table = {0, 0, nullptr, 0, 0, 0};
   MemHandle _table_handle;
   MemHandle _status_handle;  // device status word for maintenance kernels
   IdType _cache_space_capacity = 0;
@@ -50,7 +50,12 @@ class CacheEntryManager {
   void CreateFlat(const std::function<MemHandle(size_t)> &allocator, size_t num_keys, StreamHandle stream);
   void CreateHash(const std::function<MemHandle(size_t)> &allocator, size_t num_entries, StreamHandle stream);
 
-  // cuh:574-582 — off[i] = slot of keys[i] (the key itself when absent); tensors are device memory
+  // Device copy of a host list of row numbers in the form the table is keyed by: the uint32 row numbers
+  // themselves, or — in sparse-id mode — the int64 caller-side ids of those rows.
+  TensorPtr TableKeysToDevice(TensorPtr host_rows, const std::function<MemHandle(size_t)> &allocator, Context ctx,
+                              StreamHandle stream);
+  // The methods below take device tensors of table keys (kI32 row numbers or kI64 ids, see above).
+  // cuh:574-582 — off[i] = slot of keys[i] (the key's host row when absent)
   void LookupOffset(TensorPtr keys, TensorPtr off, StreamHandle stream);
   // cuh:601-608
   void InsertWithLoc(TensorPtr keys, TensorPtr off, int loc, StreamHandle stream);
@@ -62,6 +67,12 @@ class CacheEntryManager {
   TensorPtr ReserveOffsetFront(IdType num_new_insert_keys);
   // aborts if a maintenance kernel flagged an error (duplicate insert, absent evict, full table ...)
   void CheckStatus(StreamHandle stream, const char *what);
+  // Evictions leave tombstones in the open-addressing table.  Once they exceed
+  // RunConfig::hash_rebuild_tombstone_frac of the buckets the table is cleared and the cached keys re-inserted
+  // with their current slots.  Lookups racing with the rebuild see misses, which the host table serves correctly.
+  bool MaybeRebuild(const std::function<MemHandle(size_t)> &allocator, Context ctx, int loc, StreamHandle stream);
+  size_t _num_tombstones = 0;
+  size_t _num_rebuilds = 0;
 
   // cuh:693-740 — keys of `inputs` satisfying cond, in input order (deterministic, unlike the reference's
   // thread-interleaved order)

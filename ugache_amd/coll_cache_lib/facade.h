@@ -81,6 +81,11 @@ class CollCache : public std::enable_shared_from_this<CollCache> {
     _cache_ctx_list.clear();
   }
   // introspection (tests, reports)
+  size_t num_replicas_built() const {
+    size_t n = 0;
+    for (auto &c : _cache_ctx_list) n += c != nullptr;
+    return n;
+  }
   std::shared_ptr<CacheContext> cache_ctx(int replica_id) { return _cache_ctx_list.at(replica_id); }
   std::shared_ptr<ExtractSession> session(int replica_id) { return _session_list.at(replica_id); }
   TensorPtr nid_to_block() { return _nid_to_block; }

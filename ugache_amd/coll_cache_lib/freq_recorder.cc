@@ -68,14 +68,14 @@ void FreqRecorder::Record(const KeyT *input, size_t num_inputs) {
   bool bad = false;
 #pragma omp parallel for num_threads(RunConfig::solver_omp_thread_num_per_gpu) reduction(|| : bad) if (num_inputs > 65536)
   for (size_t i = 0; i < num_inputs; i++) {
-    const uint64_t k = (uint64_t)input[i];
-    if (k >= n_nodes) {
+    const uint64_t k = RunConfig::RowOfKey((uint64_t)input[i]);
+    if (k >= n_nodes || (RunConfig::key_map_mul && (uint64_t)input[i] > RunConfig::key_map_mask)) {
       bad = true;
       continue;
     }
     __atomic_fetch_add(&cnt[k], 1u, __ATOMIC_RELAXED);
   }
-  CHECK(!bad) << "FreqRecorder::Record: a key is not below num_total_item=" << n_nodes;
+  CHECK(!bad) << "FreqRecorder::Record: a key has no row among num_total_item=" << n_nodes;
 }
 template void FreqRecorder::Record<Id64Type>(const Id64Type *input, size_t num_inputs);
 template void FreqRecorder::Record<IdType>(const IdType *input, size_t num_inputs);

@@ -238,6 +238,12 @@ void coll_cache_init_ranked_c(int replica_id, size_t key_space_size, const uint3
                         cache_percentage, stream);
 }
 
+void coll_cache_set_key_map(uint64_t mul, int bits) {
+  CHECK(RunConfig::is_configured) << "coll_cache_config comes first";
+  CHECK(_coll_cache == nullptr || _coll_cache->num_replicas_built() == 0) << "the key map cannot change after the build";
+  RunConfig::SetKeyMap(mul, bits);
+}
+
 void coll_cache_refresh(int replica_id, StreamHandle stream, int foreground) {
   CHECK_NOTNULL(_coll_cache);
   ContFreqBuf *freq_rank = CombineAndRank(replica_id);
@@ -274,6 +280,7 @@ void coll_cache_get_info(int replica_id, uint64_t out[8]) {
   out[4] = RunConfig::num_total_item;
   out[5] = ctx->progress.load();
   out[6] = ctx->EntryManager() ? ctx->EntryManager()->_free_offsets->NumItem() : 0;
+  out[7] = ctx->EntryManager() ? ctx->EntryManager()->_num_rebuilds : 0;
 }
 
 size_t coll_cache_get_cached_keys(int replica_id, uint32_t *out, size_t capacity) {
@@ -328,6 +335,7 @@ void coll_cache_shutdown(void) {
   memset(steps, 0, sizeof(steps));
   max_num_keys = 0;
   RunConfig::is_configured = false;
+  RunConfig::SetKeyMap(0, 0);
 }
 
 }  // extern "C"

@@ -35,6 +35,26 @@ int RunConfig::force_table_kind = 0;
 size_t RunConfig::refresh_batch_rows = 4092;
 unsigned RunConfig::refresh_sleep_us = 3000;
 unsigned RunConfig::refresh_limit_block = 20;
+double RunConfig::hash_rebuild_tombstone_frac = 0.15;
+uint64_t RunConfig::key_map_mul = 0;
+uint64_t RunConfig::key_map_inv = 0;
+uint64_t RunConfig::key_map_mask = 0;
+
+void RunConfig::SetKeyMap(uint64_t mul, int bits) {
+  if (mul == 0) {
+    key_map_mul = key_map_inv = key_map_mask = 0;
+    return;
+  }
+  CHECK(mul & 1) << "the key-map multiplier must be odd to be invertible modulo a power of two";
+  CHECK(bits >= 1 && bits <= 62) << "key space of 2^" << bits << " ids is not supported";
+  // inverse of an odd number modulo 2^64 by Newton's iteration (each step doubles the number of correct bits)
+  uint64_t inv = mul;
+  for (int i = 0; i < 6; i++) inv *= 2 - mul * inv;
+  CHECK_EQ(mul * inv, (uint64_t)1);
+  key_map_mul = mul;
+  key_map_inv = inv;
+  key_map_mask = (bits == 64) ? ~0ull : ((1ull << bits) - 1);
+}
 
 void RunConfig::LoadConfigFromEnv() {
   // every knob goes back to its default first, so a process that builds a second cache sees only its current
@@ -46,6 +66,7 @@ void RunConfig::LoadConfigFromEnv() {
   refresh_batch_rows = 4092;
   refresh_sleep_us = 3000;
   refresh_limit_block = 20;
+  hash_rebuild_tombstone_frac = 0.15;
   if (GetEnv("SAMGRAPH_EMPTY_FEAT") != "" && GetEnv("SAMGRAPH_EMPTY_FEAT") != "0") {
     LOG(FATAL) << "SAMGRAPH_EMPTY_FEAT (mock host table) is not supported by this build: every key must have a "
                   "real row in the host table";
@@ -70,6 +91,7 @@ void RunConfig::LoadConfigFromEnv() {
   if (GetEnv("COLL_REFRESH_BATCH_ROWS") != "") refresh_batch_rows = std::stoul(GetEnv("COLL_REFRESH_BATCH_ROWS"));
   if (GetEnv("COLL_REFRESH_SLEEP_US") != "") refresh_sleep_us = std::stoul(GetEnv("COLL_REFRESH_SLEEP_US"));
   if (GetEnv("COLL_REFRESH_LIMIT_BLOCK") != "") refresh_limit_block = std::stoul(GetEnv("COLL_REFRESH_LIMIT_BLOCK"));
+  if (GetEnv("COLL_HASH_REBUILD_FRAC") != "") hash_rebuild_tombstone_frac = std::stod(GetEnv("COLL_HASH_REBUILD_FRAC"));
   LOG(INFO) << "using concurrent impl " << concurrent_link_impl;
 }
 

@@ -63,6 +63,17 @@ struct RunConfig {
   static size_t refresh_batch_rows;    // COLL_REFRESH_BATCH_ROWS, default 4092 (cache_context.cu:4057)
   static unsigned refresh_sleep_us;    // COLL_REFRESH_SLEEP_US, default 3000 (cache_context.cu:4069)
   static unsigned refresh_limit_block; // COLL_REFRESH_LIMIT_BLOCK, default 20 (cache_context.cu:4068)
+  static double hash_rebuild_tombstone_frac;  // COLL_HASH_REBUILD_FRAC, default 0.15: rebuild the table after refresh
+                                              // once this share of its buckets are tombstones
+  // Sparse-id mode (an extension; the reference's keys are dense uint32 row numbers): the caller's key of host row
+  // r is (r * key_map_mul) mod 2^bits with key_map_mul odd, a bijection on the id space, so the library can turn
+  // a key back into its row with key_map_inv.  key_map_mul == 0: keys are row numbers.
+  static uint64_t key_map_mul;
+  static uint64_t key_map_inv;
+  static uint64_t key_map_mask;
+  static void SetKeyMap(uint64_t mul, int bits);
+  static inline uint64_t KeyOfRow(uint64_t row) { return key_map_mul ? ((row * key_map_mul) & key_map_mask) : row; }
+  static inline uint64_t RowOfKey(uint64_t key) { return key_map_mul ? ((key * key_map_inv) & key_map_mask) : key; }
 
   static void LoadConfigFromEnv();
   static inline uint64_t GetBatchKey(uint64_t epoch, uint64_t step) { return epoch * num_global_step_per_epoch + step; }

@@ -109,6 +109,7 @@ C_API = {
     "coll_cache_lookup_i64": (None, [ctypes.c_int, ctypes.c_void_p, ctypes.c_size_t, ctypes.c_void_p,
                                      ctypes.c_void_p]),
     "coll_cache_record_i64": (None, [ctypes.c_int, ctypes.c_void_p, ctypes.c_size_t]),
+    "coll_cache_set_key_map": (None, [ctypes.c_uint64, ctypes.c_int]),
     "coll_cache_refresh": (None, [ctypes.c_int, ctypes.c_void_p, ctypes.c_int]),
     "coll_cache_alloc_host_table": (ctypes.c_void_p, [ctypes.c_size_t]),
     "coll_cache_free_host_table": (None, [ctypes.c_void_p]),
@@ -185,11 +186,15 @@ class CollCacheBasics(object):
     def info(self, replica_id=0):
         out = (ctypes.c_uint64 * 8)()
         self.C_LIB_CTYPES.coll_cache_get_info(replica_id, ctypes.byref(out))
-        names = ["capacity_rows", "cached_rows", "table_kind", "row_bytes", "key_space", "lookups", "free_slots"]
+        names = ["capacity_rows", "cached_rows", "table_kind", "row_bytes", "key_space", "lookups", "free_slots",
+                 "table_rebuilds"]
         return dict(zip(names, list(out)))
 
     def step_value(self, key, item):
         return self.C_LIB_CTYPES.coll_cache_get_step_value(key, item)
+
+    def set_key_map(self, mul, bits):
+        self.C_LIB_CTYPES.coll_cache_set_key_map(mul, bits)
 
     def shutdown(self):
         self.C_LIB_CTYPES.coll_cache_shutdown()

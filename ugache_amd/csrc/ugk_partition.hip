@@ -50,9 +50,9 @@ __global__ __launch_bounds__(kBlock) void classify_kernel(ugk_table_t t, const K
         } else if (f.hit && f.loc == UGK_LOC_HOST && f.off < host_rows) {
           c = 2;
           o = f.off;
-        } else if (!f.hit && key < host_rows && key <= 0xffffffffull) {
+        } else if (!f.hit && fallback_row(t, key) < host_rows && fallback_row(t, key) <= 0xffffffffull) {
           c = 2;
-          o = (uint32_t)key;
+          o = (uint32_t)fallback_row(t, key);
         } else {
           atomicOr(status, UGK_ST_KEY_OUT_OF_RANGE);
           if (host_mirror) host_mirror[0] = UGK_ST_KEY_OUT_OF_RANGE;
@@ -123,7 +123,7 @@ __global__ __launch_bounds__(kBlock) void extract_mix_kernel(ugk_table_t t, cons
     if (active) {
       if (f.hit && f.loc == UGK_LOC_LOCAL && f.off < cache_rows) rowp = cache + (uint64_t)f.off * vpr;
       else if (f.hit && f.loc == UGK_LOC_HOST && f.off < host_rows) rowp = host + (uint64_t)f.off * vpr;
-      else if (!f.hit && key < host_rows) rowp = host + key * vpr;
+      else if (!f.hit && fallback_row(t, key) < host_rows) rowp = host + fallback_row(t, key) * vpr;
       else {
         atomicOr(status, UGK_ST_KEY_OUT_OF_RANGE);
         if (host_mirror) host_mirror[0] = UGK_ST_KEY_OUT_OF_RANGE;

@@ -173,6 +173,12 @@ __device__ __forceinline__ uint64_t key_to_u64<int64_t>(int64_t k) {
   return (uint64_t)k;
 }
 
+// host row of a key that is not in the table
+__device__ __forceinline__ uint64_t fallback_row(const ugk_table_t &t, uint64_t key) {
+  if (t.fb_mul == 0) return key;
+  return key <= t.fb_mask ? ((key * t.fb_mul) & t.fb_mask) : ~0ull;  // ids beyond the id space have no row
+}
+
 // keys that collide with the two reserved bucket states cannot live in the hash table
 __device__ __forceinline__ bool key_is_reserved(uint64_t k) { return k >= UGK_HASH_TOMB; }
 

@@ -126,7 +126,7 @@ __global__ __launch_bounds__(kBlock) void lookup_kernel(ugk_table_t t, const K *
     const Found f = table_lookup<KIND>(t, key, active);
     if (active) {
       if (loc_out) loc_out[i] = f.hit ? f.loc : fallback_loc;
-      if (off_out) off_out[i] = f.hit ? f.off : (uint32_t)key;
+      if (off_out) off_out[i] = f.hit ? f.off : (uint32_t)fallback_row(t, key);
     }
   }
 }

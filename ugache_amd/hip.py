@@ -29,7 +29,8 @@ class UgkError(RuntimeError):
 
 class Table(C.Structure):
     """ugk_table_t"""
-    _fields_ = [("kind", C.c_int32), ("reserved", C.c_int32), ("table", C.c_void_p), ("size", C.c_uint64)]
+    _fields_ = [("kind", C.c_int32), ("reserved", C.c_int32), ("table", C.c_void_p), ("size", C.c_uint64),
+                ("fb_mul", C.c_uint64), ("fb_mask", C.c_uint64)]
 
 
 class DeviceInfo(C.Structure):
@@ -123,8 +124,8 @@ def call(name, *args):
     return 0
 
 
-def table(kind, ptr, size):
-    return Table(kind, 0, ptr, size)
+def table(kind, ptr, size, fb_mul=0, fb_mask=0):
+    return Table(kind, 0, ptr, size, fb_mul, fb_mask)
 
 
 def device_info(dev=0):
