@@ -50,6 +50,13 @@ MIXED = {
                                                                     n_keys=8192 * 26, zipf=1.2,
                                                                     pct=(20e9 / 512) / (26 * 4_194_304), fields=26,
                                                                     presample=100),
+    # hashtable mode: ids are (row * odd) mod 2^40, rows are 64 fp16 = 128 B, 10 % of the rows cached in the
+    # open-addressing table at 0.7 load; a foreground refresh is timed after the lookups
+    "c5_hash_500Mx64xfp16_1M_i64_zipf1.05_cache50M": dict(rows=500_000_000, dim=64, dtype="float16", n_keys=1 << 20,
+                                                          zipf=1.05, pct=0.1, fields=1, presample=50, sparse=True),
+    "c5_hash_quarter_125Mx64xfp16_1M_i64_zipf1.05_cache12.5M": dict(rows=125_000_000, dim=64, dtype="float16",
+                                                                    n_keys=1 << 20, zipf=1.05, pct=0.1, fields=1,
+                                                                    presample=50, sparse=True),
     "c1_cpu_ref_1Mx128xfp32_65536_i64_zipf1.1_cache10pct": dict(rows=1_000_000, dim=128, dtype="float32",
                                                                 n_keys=65_536, zipf=1.1, pct=0.10, fields=1,
                                                                 presample=20),
@@ -240,6 +247,10 @@ def run_mixed(args):
 
     co.config({"cache_percentage": pct, "_cache_policy": co.kCollCacheAsymmLink, "num_device": 1,
                "num_global_step_per_epoch": K + W, "num_epoch": 1, "num_total_item": rows, "omp_thread_num": 16})
+    sparse = bool(spec.get("sparse"))
+    KEY_MUL, KEY_BITS = 0x9E3779B97F4A7C15, 40
+    if sparse:
+        _basics.set_key_map(KEY_MUL, KEY_BITS)
     co.coll_cache_record_init(0)
     note = lambda msg: print("[bench %6.1fs] %s" % (time.perf_counter() - t_setup, msg), file=sys.stderr, flush=True)
     emb = co.coll_torch_create_emb_shm(0, rows, dim, tdtype)
@@ -253,7 +264,15 @@ def run_mixed(args):
     perms = [torch.randperm(per_field, generator=gp, device=dev, dtype=torch.int64) for _ in range(fields)]
     gz = torch.Generator(device=dev).manual_seed(3)
 
+    def ids_of(rows_t):
+        """caller-side ids of rows: identity, or (row * odd) mod 2^40 in sparse-id mode (int64 multiply wraps)"""
+        if not sparse:
+            return rows_t
+        mul = torch.tensor(KEY_MUL - (1 << 64), dtype=torch.int64, device=rows_t.device)
+        return (rows_t * mul) & ((1 << KEY_BITS) - 1)
+
     def make_batch():
+        """one batch of ROW numbers"""
         if fields == 1:
             return perms[0][zipf_ranks_gpu(torch, n_keys, per_field, spec["zipf"], gz, dev)]
         per = n_keys // fields  # [samples, fields] laid out row-major: key = f * per_field + perm_f[rank]
@@ -262,13 +281,14 @@ def run_mixed(args):
         return torch.stack(cols, dim=1).reshape(-1)
 
     for _ in range(spec["presample"]):
-        co.coll_torch_record(0, make_batch().cpu())
+        co.coll_torch_record(0, ids_of(make_batch()).cpu())
     note("hotness of %d presample batches recorded" % spec["presample"])
     co.coll_torch_init_t(0, 0, emb, pct)
     info_cache = _basics.info(0)
     note("cache built: %d rows cached" % info_cache["cached_rows"])
 
-    keys_pool = torch.stack([make_batch() for _ in range(pool)])
+    rows_pool = torch.stack([make_batch() for _ in range(pool)])
+    keys_pool = ids_of(rows_pool)
     out = torch.empty((n_keys, row_bytes), dtype=torch.uint8, device=dev)
     C = _basics.C_LIB_CTYPES
     stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
@@ -302,8 +322,8 @@ def run_mixed(args):
 
     orc = Oracle()
     table_np = emb.numpy().view(np.uint8).reshape(rows, row_bytes)
-    last_keys = keys_pool[(W + K - 1) % pool].cpu().numpy()
-    if out.cpu().numpy().tobytes() != orc.gather(table_np, last_keys, omp=True).tobytes():
+    last_rows = rows_pool[(W + K - 1) % pool].cpu().numpy()
+    if out.cpu().numpy().tobytes() != orc.gather(table_np, last_rows, omp=True).tobytes():
         sys.exit("bench.py: GPU output differs from the CPU oracle — no numbers reported")
 
     steps = range(W, W + K)
@@ -316,9 +336,35 @@ def run_mixed(args):
     hit_alg = n_hit * (2 * row_bytes + 8)  # row read + row written + 8-byte index record
     achieved = hit_alg / t_hit / 1e9 if t_hit > 0 else 0.0
 
-    keys_host = keys_pool.cpu().numpy()
+    # the CPU baseline gathers by row number (it is spared the id -> row translation of sparse-id mode)
+    keys_host = rows_pool.cpu().numpy()
     cpu_kps, n_cpu, cpu_el, cores = cpu_baseline(orc, table_np, keys_host, n_keys, row_bytes, args.cpu_seconds)
     uniq = float(np.mean([len(np.unique(keys_host[i])) for i in range(min(pool, 4))]))
+
+    refresh = None
+    if sparse:
+        # one foreground refresh: the same hotness again, plus 1 % of the cache size worth of so-far uncached rows
+        # pushed to the top, so that about 1 % of the cached rows are evicted and replaced
+        before = _basics.info(0)
+        n_new = before["cached_rows"] // 100
+        for _ in range(spec["presample"]):
+            co.coll_torch_record(0, ids_of(make_batch()).cpu())
+        cold = perms[0][per_field - n_new:]  # the coldest ranks of the permutation
+        boost = ids_of(cold).cpu()
+        for _ in range(64):
+            co.coll_torch_record(0, boost)
+        note("hotness for the refresh recorded")
+        t0 = time.perf_counter()
+        co.coll_torch_refresh(0, True)
+        refresh_s = time.perf_counter() - t0
+        after = _basics.info(0)
+        note("refresh done in %.2f s" % refresh_s)
+        step(0)
+        torch.cuda.synchronize()
+        if out.cpu().numpy().tobytes() != orc.gather(table_np, rows_pool[0].cpu().numpy(), omp=True).tobytes():
+            sys.exit("bench.py: GPU output differs from the CPU oracle after the refresh")
+        refresh = {"seconds": refresh_s, "boosted_rows": n_new, "table_rebuilds": after["table_rebuilds"],
+                   "cached_rows_after": after["cached_rows"], "free_slots_after": after["free_slots"]}
 
     info = hip.device_info(0)
     keys_per_s = n_keys * K / elapsed
@@ -327,8 +373,9 @@ def run_mixed(args):
         "value": keys_per_s, "unit": "keys/s", "n_gpus": 1, "steps": K, "warmup": W,
         "ms_per_step": elapsed / K * 1e3, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "u8", "data": "synthetic",
+        "refresh": refresh,
         "config": {"workload": args.workload, "table_rows": rows, "row_bytes": row_bytes, "keys_per_batch": n_keys,
-                   "key_dtype": "int64", "cache_percentage": pct, "cached_rows": info_cache["cached_rows"],
+                   "key_dtype": "int64", "sparse_ids": sparse, "cache_percentage": pct, "cached_rows": info_cache["cached_rows"],
                    "cache_capacity_rows": info_cache["capacity_rows"], "table_kind": info_cache["table_kind"],
                    "zipf_s": spec["zipf"], "fields": fields, "presample_batches": spec["presample"],
                    "entry_point": "coll_cache_lookup_i64", "distinct_key_batches": pool,
