@@ -1,0 +1,87 @@
+"""Error behaviour at the boundary on a GPU box: the reference's convention is CHECK -> message -> abort(), and a bad
+key must never fault the GPU.  Each case runs in a child process (the parent never touches the GPU here)."""
+import os
+import subprocess
+import sys
+import textwrap
+
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+PRELUDE = textwrap.dedent("""
+    import sys
+    sys.path.insert(0, %r)
+    import numpy as np, torch
+    import collcache.torch as co
+    cfg = lambda n, pct: {"cache_percentage": pct, "_cache_policy": co.kCollCacheAsymmLink, "num_device": 1,
+                          "num_global_step_per_epoch": 10, "num_epoch": 1, "num_total_item": n, "omp_thread_num": 4}
+""" % os.path.join(ROOT, "ugache_amd"))
+
+
+def run(body, env=None):
+    e = dict(os.environ)
+    e.update(env or {})
+    return subprocess.run([sys.executable, "-c", PRELUDE + textwrap.dedent(body)], stdout=subprocess.PIPE,
+                          stderr=subprocess.PIPE, text=True, env=e, timeout=170)
+
+
+@pytest.mark.parametrize("pct", [1.0, 0.0, 0.3])
+def test_key_out_of_range_aborts_with_a_message_instead_of_faulting(pct):
+    p = run("""
+        n = 5000
+        co.config(cfg(n, %r)); co.coll_cache_record_init(0)
+        co.coll_torch_record(0, torch.arange(0, n, 3, dtype=torch.int32))
+        emb = co.coll_torch_create_emb_shm(0, n, 32, torch.float32); emb.normal_()
+        co.coll_torch_init_t(0, 0, emb, %r)
+        good = co.coll_torch_lookup_key_t_val_ret(0, torch.arange(100, dtype=torch.int32, device="cuda"), False)
+        assert torch.equal(good.cpu(), emb[:100])
+        print("good lookup ok", flush=True)
+        bad = torch.tensor([1, 2, n, 3], dtype=torch.int32, device="cuda")
+        co.coll_torch_lookup_key_t_val_ret(0, bad, False)
+        print("survived")
+    """ % (pct, pct))
+    assert "good lookup ok" in p.stdout and "survived" not in p.stdout
+    assert p.returncode == -6, p.stderr[-2000:]
+    assert "extraction kernels reported status" in p.stderr and "outside the table" in p.stderr
+
+
+def test_ordinary_host_memory_is_refused_for_a_partial_cache():
+    p = run("""
+        n = 1000
+        co.config(cfg(n, 0.5)); co.coll_cache_record_init(0)
+        co.coll_torch_record(0, torch.arange(0, n, dtype=torch.int32))
+        emb = torch.randn(n, 16)            # pageable host memory, not from coll_torch_create_emb_shm
+        co.coll_torch_init_t(0, 0, emb, 0.5)
+        print("survived")
+    """)
+    assert p.returncode == -6 and "survived" not in p.stdout
+    assert "must be pinned" in p.stderr
+
+
+def test_ordinary_host_memory_is_fine_for_a_full_cache():
+    p = run("""
+        n = 1000
+        co.config(cfg(n, 1.0))
+        emb = torch.randn(n, 16)
+        co.coll_torch_init_t(0, 0, emb, 1.0)
+        q = torch.randint(0, n, (333,), dtype=torch.int32)
+        out = co.coll_torch_lookup_key_t_val_ret(0, q.cuda(), False)
+        assert torch.equal(out.cpu(), emb[q.long()])
+        print("survived")
+    """)
+    assert p.returncode == 0 and "survived" in p.stdout, p.stderr[-2000:]
+
+
+def test_mock_table_env_is_rejected():
+    p = run("""
+        n = 1000
+        co.config(cfg(n, 1.0))
+        emb = torch.randn(n, 16)
+        co.coll_torch_init_t(0, 0, emb, 1.0)
+        print("survived")
+    """, env={"SAMGRAPH_EMPTY_FEAT": "10"})
+    assert p.returncode == -6 and "survived" not in p.stdout
+    assert "SAMGRAPH_EMPTY_FEAT" in p.stderr
