@@ -75,6 +75,8 @@ def parse_args():
                     choices=sorted(ALL_HIT) + sorted(MIXED))
     ap.add_argument("--cpu-seconds", type=float, default=10.0, help="CPU baseline budget")
     ap.add_argument("--pool", type=int, default=None, help="distinct key batches cycled through the steps")
+    ap.add_argument("--dedup", action="store_true",
+                    help="mixed workloads: COLL_DEDUP_KEYS=1, every distinct key of a batch is extracted once")
     ap.add_argument("--calibrate", action="store_true",
                     help="also run 5 plain device copies of 1 GiB (ugk_copy_rows) so a counter run has a kernel of "
                          "known traffic next to the gather")
@@ -245,6 +247,8 @@ def run_mixed(args):
     dev = torch.device("cuda:0")
     t_setup = time.perf_counter()
 
+    if args.dedup:
+        os.environ["COLL_DEDUP_KEYS"] = "1"
     co.config({"cache_percentage": pct, "_cache_policy": co.kCollCacheAsymmLink, "num_device": 1,
                "num_global_step_per_epoch": K + W, "num_epoch": 1, "num_total_item": rows, "omp_thread_num": 16})
     sparse = bool(spec.get("sparse"))
@@ -333,6 +337,10 @@ def run_mixed(args):
     miss_bytes = float(np.mean([_basics.step_value(s, kLogL1MissBytes) for s in steps]))
     n_miss = miss_bytes / row_bytes
     n_hit = n_keys - n_miss
+    if args.dedup:  # the gathers ran over the distinct keys: take their group sizes from the last timed batch
+        g = _basics.last_group_offset(0)
+        n_hit, n_miss = float(g[1]), float(g[2] - g[1])
+        miss_bytes = n_miss * row_bytes
     hit_alg = n_hit * (2 * row_bytes + 8)  # row read + row written + 8-byte index record
     achieved = hit_alg / t_hit / 1e9 if t_hit > 0 else 0.0
 
@@ -378,7 +386,7 @@ def run_mixed(args):
                    "key_dtype": "int64", "sparse_ids": sparse, "cache_percentage": pct, "cached_rows": info_cache["cached_rows"],
                    "cache_capacity_rows": info_cache["capacity_rows"], "table_kind": info_cache["table_kind"],
                    "zipf_s": spec["zipf"], "fields": fields, "presample_batches": spec["presample"],
-                   "entry_point": "coll_cache_lookup_i64", "distinct_key_batches": pool,
+                   "entry_point": "coll_cache_lookup_i64", "distinct_key_batches": pool, "dedup": bool(args.dedup),
                    "unique_keys_per_batch": uniq, "seeds": {"table": 1, "perm": 2, "keys": 3}},
         "effective_extraction_GBps": n_keys * row_bytes / (elapsed / K) / 1e9,
         "parity": "bit-exact vs CPU oracle (last timed batch)",

@@ -135,18 +135,23 @@ int ugk_gather_direct_i64(const void *src_dev, uint64_t src_rows, const int64_t 
 /* IdxStoreDst (cache_context.h:356-361): srcrow = keys[i], dst = dst_off[i] (cache fill / refresh insert) */
 int ugk_gather_scatter_u32(const void *src_dev, uint64_t src_rows, const uint32_t *keys_dev,
                            const uint32_t *dst_off_dev, size_t n, void *out_dev, uint64_t out_rows, size_t row_bytes,
-                           unsigned max_blocks, uint32_t *status_dev, void *stream);
+                           unsigned max_blocks, uint32_t *status_dev, uint32_t *host_mirror, void *stream);
 int ugk_gather_scatter_i64(const void *src_dev, uint64_t src_rows, const int64_t *keys_dev,
                            const uint32_t *dst_off_dev, size_t n, void *out_dev, uint64_t out_rows, size_t row_bytes,
-                           unsigned max_blocks, uint32_t *status_dev, void *stream);
+                           unsigned max_blocks, uint32_t *status_dev, uint32_t *host_mirror, void *stream);
+/* re-expansion after a deduplicated extraction: for every i whose representative r = rep_dev[inverse_dev[i]] differs
+ * from i, out[i, :] = out[r, :] (rows r were written by the gathers, rows i are their duplicates) */
+int ugk_replicate_rows(void *out_dev, size_t row_bytes, const uint32_t *inverse_dev, const uint32_t *rep_dev, size_t n,
+                       void *stream);
 /* CombineOneGroup with DataIterPerLoc<IdxStoreCompact> (cache_context.cu:195-212, 855-859).
  * The group is idx[begin, begin+count) where, with c = counts_dev (written by ugk_classify_*):
  *   group UGK_LOC_LOCAL: begin = 0,            count = c[0]
  *   group UGK_LOC_HOST : begin = n - c[1],     count = c[1]
- * so no host round trip is needed between classify and gather.  n is the batch size (grid upper bound). */
+ * so no host round trip is needed between classify and gather.  n is the number of classified keys (grid upper
+ * bound), out_rows the rows of the output (n, or more when classify ran with a destination map). */
 int ugk_gather_group(const void *src_dev, uint64_t src_rows, const ugk_idx_t *idx_dev, const uint32_t *counts_dev,
-                     uint32_t group, size_t n, void *out_dev, size_t row_bytes, unsigned max_blocks,
-                     uint32_t *status_dev, uint32_t *host_mirror, void *stream);
+                     uint32_t group, size_t n, void *out_dev, uint64_t out_rows, size_t row_bytes,
+                     unsigned max_blocks, uint32_t *status_dev, uint32_t *host_mirror, void *stream);
 /* same with an explicit list (count known on the host) */
 int ugk_gather_idx(const void *src_dev, uint64_t src_rows, const ugk_idx_t *idx_dev, size_t count, void *out_dev,
                    size_t row_bytes, unsigned max_blocks, uint32_t *status_dev, void *stream);
@@ -183,13 +188,15 @@ int ugk_hash_census(const ugk_bucket_t *table_dev, size_t nbuckets, uint64_t *ce
  *   host misses fill idx[n - c[1], n)      as {dst_off = i, src_off = host row = key}
  * counts_dev[0..1] must be zero on entry; the kernel also zeroes next_counts_dev[0..1] (may be NULL) so a
  * caller can rotate two counter pairs and never launch a memset.  host_rows bounds the miss offsets.
- * A key found with a location other than local/host sets UGK_ST_KEY_OUT_OF_RANGE (one GPU has two sources). */
-int ugk_classify_u32(ugk_table_t t, const uint32_t *keys_dev, size_t n, uint64_t host_rows, ugk_idx_t *idx_dev,
-                     uint32_t *counts_dev, uint32_t *next_counts_dev, uint32_t *status_dev, uint32_t *host_mirror,
-                     void *stream);
-int ugk_classify_i64(ugk_table_t t, const int64_t *keys_dev, size_t n, uint64_t host_rows, ugk_idx_t *idx_dev,
-                     uint32_t *counts_dev, uint32_t *next_counts_dev, uint32_t *status_dev, uint32_t *host_mirror,
-                     void *stream);
+ * A key found with a location other than local/host sets UGK_ST_KEY_OUT_OF_RANGE (one GPU has two sources).
+ * dst_map_dev (may be NULL): output row of key i is dst_map_dev[i] instead of i (deduplicated extraction: the keys
+ * are the distinct ones, their output rows the first occurrences). */
+int ugk_classify_u32(ugk_table_t t, const uint32_t *keys_dev, size_t n, uint64_t host_rows, const uint32_t *dst_map_dev,
+                     ugk_idx_t *idx_dev, uint32_t *counts_dev, uint32_t *next_counts_dev, uint32_t *status_dev,
+                     uint32_t *host_mirror, void *stream);
+int ugk_classify_i64(ugk_table_t t, const int64_t *keys_dev, size_t n, uint64_t host_rows, const uint32_t *dst_map_dev,
+                     ugk_idx_t *idx_dev, uint32_t *counts_dev, uint32_t *next_counts_dev, uint32_t *status_dev,
+                     uint32_t *host_mirror, void *stream);
 
 /* ---- single-kernel mixed-source extraction: kDirectNoGroup with DataIterMixLoc
  *      (cache_context.cu:137-159, 1295-1329): lookup and gather fused, source picked per row ---------- */
@@ -205,12 +212,16 @@ int ugk_extract_mix_i64(ugk_table_t t, const int64_t *keys_dev, size_t n, const 
  * unique_out[0..*n_unique) = distinct keys (order unspecified), inverse_out[i] = position of keys[i] in it.
  * workspace_dev: ugk_dedup_workspace_bytes(n) bytes, zero-filled once at allocation and then reused as is
  * (slots are epoch-tagged, so no per-call clearing); epoch must be non-zero and different on every call
- * that shares the workspace.  n_unique_dev must be zero on entry. */
+ * that shares the workspace.  n_unique_dev must be zero on entry.
+ * rep_out_dev (may be NULL): rep_out_dev[u] = index of the first occurrence that introduced unique key u.
+ * n_unique_host (may be NULL): pinned host word that receives *n_unique_dev when the second kernel runs. */
 size_t ugk_dedup_workspace_bytes(size_t n);
 int ugk_dedup_u32(const uint32_t *keys_dev, size_t n, void *workspace_dev, uint32_t epoch, uint32_t *unique_out_dev,
-                  uint32_t *inverse_out_dev, uint32_t *n_unique_dev, void *stream);
+                  uint32_t *inverse_out_dev, uint32_t *rep_out_dev, uint32_t *n_unique_dev, uint32_t *n_unique_host,
+                  void *stream);
 int ugk_dedup_i64(const int64_t *keys_dev, size_t n, void *workspace_dev, uint32_t epoch, int64_t *unique_out_dev,
-                  uint32_t *inverse_out_dev, uint32_t *n_unique_dev, void *stream);
+                  uint32_t *inverse_out_dev, uint32_t *rep_out_dev, uint32_t *n_unique_dev, uint32_t *n_unique_host,
+                  void *stream);
 
 #ifdef __cplusplus
 }

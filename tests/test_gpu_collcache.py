@@ -40,7 +40,8 @@ def make_config(num_total_item, pct, threads=8):
 
 @pytest.fixture(autouse=True)
 def _fresh_cache(monkeypatch):
-    for v in ("COLL_HASH_TABLE", "SAMGRAPH_COLL_CACHE_CONCURRENT_LINK_IMPL", "SAMGRAPH_COLL_CACHE_NO_GROUP"):
+    for v in ("COLL_HASH_TABLE", "SAMGRAPH_COLL_CACHE_CONCURRENT_LINK_IMPL", "SAMGRAPH_COLL_CACHE_NO_GROUP",
+              "COLL_DEDUP_KEYS", "COLL_DEDUP_MIN_KEYS"):
         monkeypatch.delenv(v, raising=False)
     yield
     if torch.cuda.is_available():
@@ -139,6 +140,46 @@ def test_partial_cache_matches_oracle(table_kind, impl, kdtype, monkeypatch):
     if impl != "DIRECT":
         step = _basics.info(0)["lookups"] - 1
         assert _basics.step_value(step, kLogL1MissBytes) == (n - n_local) * dim * 4
+
+
+@pytest.mark.parametrize("pct", [0.0, 0.1, 1.0])
+@pytest.mark.parametrize("table_kind", ["FLAT", "HASH"])
+@pytest.mark.parametrize("kdtype", [torch.int32, torch.int64])
+def test_dedup_in_front_of_the_extraction(pct, table_kind, kdtype, monkeypatch):
+    """COLL_DEDUP_KEYS=1: each distinct key is extracted once and the duplicates are copied inside the output; the
+    output must stay identical to the plain gather, the group sizes count distinct keys."""
+    if pct in (0.0, 1.0) and table_kind == "HASH":
+        pytest.skip("direct mapping has no table")
+    monkeypatch.setenv("COLL_HASH_TABLE", table_kind)
+    monkeypatch.setenv("COLL_DEDUP_KEYS", "1")
+    monkeypatch.setenv("COLL_DEDUP_MIN_KEYS", "64")
+    rng = np.random.default_rng(21)
+    n_item, dim = 30_000, 96
+    co.config(make_config(n_item, pct))
+    co.coll_cache_record_init(0)
+    perm = rng.permutation(n_item)
+    rec = perm[zipf_ranks(rng, 60_000, n_item, 1.2)]
+    co.coll_torch_record(0, torch.from_numpy(rec).to(kdtype))
+    emb = co.coll_torch_create_emb_shm(0, n_item, dim, torch.float32)
+    table = fill_table(emb, rng)
+    co.coll_torch_init_t(0, 0, emb, pct)
+    _, nid = expected_cached_set(rec.astype(np.uint32), n_item, pct)
+    # 50_000 after 1000 regrows the buffers; 8 is below the threshold (no dedup); the repeat reuses the set (epochs)
+    for n in (8, 1000, 50_000, 50_000, 777):
+        keys = perm[zipf_ranks(rng, n, n_item, 1.3)]
+        if n == 777:
+            keys[:] = keys[0]  # one distinct key
+        kt = torch.from_numpy(keys).to(kdtype).cuda()
+        out = co.coll_torch_lookup_key_t_val_ret(0, kt, False)
+        assert out.cpu().numpy().tobytes() == ORC.gather(table, keys.astype(np.int64)).tobytes(), n
+        uniq = np.unique(keys) if n >= 64 else keys
+        if pct == 1.0:
+            want = [0, len(uniq), len(uniq)]
+        elif pct == 0.0:
+            want = [0, 0, len(uniq)]
+        else:
+            want = [0, int((nid[uniq] == 0).sum()), len(uniq)]
+        assert _basics.last_group_offset(0) == want
 
 
 def test_fp16_table_and_small_rows():

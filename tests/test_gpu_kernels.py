@@ -85,7 +85,7 @@ def test_gather_scatter(kdtype):
     st = dev_zeros_u32(1)
     fn = "ugk_gather_scatter_i64" if kdtype == np.int64 else "ugk_gather_scatter_u32"
     d_table, d_keys, d_dst = to_dev(table), to_dev(keys), to_dev(dst)
-    hip.call(fn, ptr(d_table), 500, ptr(d_keys), ptr(d_dst), n, ptr(out), 400, 512, 0, ptr(st), None)
+    hip.call(fn, ptr(d_table), 500, ptr(d_keys), ptr(d_dst), n, ptr(out), 400, 512, 0, ptr(st), None, None)
     want = np.zeros((400, 512), np.uint8)
     want[dst] = table[keys.astype(np.int64)]
     assert status_value(st) == 0 and to_np(out).reshape(400, 512).tobytes() == want.tobytes()
@@ -93,7 +93,7 @@ def test_gather_scatter(kdtype):
     bad = dst.copy()
     bad[0] = 400
     d_bad = to_dev(bad)
-    hip.call(fn, ptr(d_table), 500, ptr(d_keys), ptr(d_bad), n, ptr(out), 400, 512, 0, ptr(st), None)
+    hip.call(fn, ptr(d_table), 500, ptr(d_keys), ptr(d_bad), n, ptr(out), 400, 512, 0, ptr(st), None, None)
     assert status_value(st) & hip.ST_KEY_OUT_OF_RANGE
 
 
@@ -300,7 +300,7 @@ def _classify(tb, keys_np, host_rows):
     st = dev_zeros_u32(1)
     fn = "ugk_classify_i64" if keys_np.dtype == np.int64 else "ugk_classify_u32"
     keys = to_dev(keys_np)
-    hip.call(fn, tb, ptr(keys), n, host_rows, ptr(idx), ptr(counts), ptr(counts) + 8, ptr(st), None, None)
+    hip.call(fn, tb, ptr(keys), n, host_rows, None, ptr(idx), ptr(counts), ptr(counts) + 8, ptr(st), None, None)
     sync()
     c = to_np(counts, np.uint32)
     return idx, counts, c, status_value(st), keys
@@ -349,9 +349,9 @@ def test_classify_partition_and_factored_gather(mode, kdtype, n):
         out = dev_bytes(n * rb, fill=0xCD)
         st2 = dev_zeros_u32(1)
         cache_dev = to_dev(cache)
-        hip.call("ugk_gather_group", pin.ptr, nkeys, ptr(idx), ptr(counts), hip.LOC_HOST, n, ptr(out), rb, 4, ptr(st2),
+        hip.call("ugk_gather_group", pin.ptr, nkeys, ptr(idx), ptr(counts), hip.LOC_HOST, n, ptr(out), n, rb, 4, ptr(st2),
                  mirror.ptr, None)
-        hip.call("ugk_gather_group", ptr(cache_dev), cap, ptr(idx), ptr(counts), hip.LOC_LOCAL, n, ptr(out), rb, 0,
+        hip.call("ugk_gather_group", ptr(cache_dev), cap, ptr(idx), ptr(counts), hip.LOC_LOCAL, n, ptr(out), n, rb, 0,
                  ptr(st2), mirror.ptr, None)
         assert status_value(st2) == 0
         if n:  # the gathers publish their group sizes in pinned host memory
@@ -422,9 +422,10 @@ def test_dedup_matches_numpy_unique(kdtype, n):
         uniq = dev_bytes(n * np.dtype(kdtype).itemsize)
         inv = dev_zeros_u32(n)
         nu = dev_zeros_u32(1)
+        rep = dev_zeros_u32(n)
         fn = "ugk_dedup_i64" if kdtype == np.int64 else "ugk_dedup_u32"
         d_keys = to_dev(keys)
-        hip.call(fn, ptr(d_keys), n, ptr(ws), epoch, ptr(uniq), ptr(inv), ptr(nu), None)
+        hip.call(fn, ptr(d_keys), n, ptr(ws), epoch, ptr(uniq), ptr(inv), ptr(rep), ptr(nu), None, None)
         sync()
         k = int(to_np(nu, np.uint32)[0])
         u = to_np(uniq, kdtype)[:k]
@@ -433,3 +434,52 @@ def test_dedup_matches_numpy_unique(kdtype, n):
         assert k == len(want_u) == len(np.unique(keys))
         assert np.array_equal(np.sort(u.astype(np.int64)), np.sort(want_u))
         assert i.max() < k and np.array_equal(u[i], keys)
+        r = to_np(rep, np.uint32)[:k]
+        assert np.array_equal(keys[r], u) and np.array_equal(i[r], np.arange(k))  # representatives
+
+
+def test_classify_with_destination_map():
+    """dst_map redirects the output row of key i; sources and group sizes are unchanged"""
+    rng = np.random.default_rng(31)
+    nkeys = 5000
+    cached = rng.choice(nkeys, 1500, replace=False).astype(np.uint32)
+    mem, tb = _make_flat(nkeys)
+    assert _insert(tb, cached) == 0
+    n = 3333
+    keys = rng.integers(0, nkeys, size=n).astype(np.uint32)
+    dmap = rng.permutation(10 * n)[:n].astype(np.uint32)
+    idx0, _, c0, st0, _ = _classify(tb, keys, nkeys)
+    idx = dev_bytes(n * 8, fill=0xAB)
+    counts = dev_zeros_u32(4)
+    st = dev_zeros_u32(1)
+    d_keys, d_map = to_dev(keys), to_dev(dmap)
+    hip.call("ugk_classify_u32", tb, ptr(d_keys), n, nkeys, ptr(d_map), ptr(idx), ptr(counts), ptr(counts) + 8,
+             ptr(st), None, None)
+    sync()
+    c = to_np(counts, np.uint32)
+    assert st0 == 0 and status_value(st) == 0 and c[0] == c0[0] and c[1] == c0[1]
+    plain = to_np(idx0, IDX_DTYPE)[:n].copy()
+    plain["dst_off"] = dmap[plain["dst_off"]]
+    got = to_np(idx, IDX_DTYPE)[:n]
+
+    def canon(a):
+        return np.sort(a["dst_off"].astype(np.uint64) << 32 | a["src"].astype(np.uint64))
+    assert np.array_equal(canon(got[: c[0]]), canon(plain[: c[0]]))
+    assert np.array_equal(canon(got[c[0]:]), canon(plain[c[0]:]))
+
+
+@pytest.mark.parametrize("row_bytes", [512, 64, 2048, 12, 100])
+def test_replicate_rows_fills_duplicates_from_their_representative(row_bytes):
+    rng = np.random.default_rng(row_bytes)
+    n = 20_011
+    keys = rng.integers(0, 3000, size=n)
+    uniq, first, inv = np.unique(keys, return_index=True, return_inverse=True)
+    table = _rand_table(rng, 3000, row_bytes)
+    out = np.full((n, row_bytes), 0xEE, np.uint8)
+    out[first] = table[uniq]  # what the gathers leave behind: representatives only
+    d_out = to_dev(out)
+    d_inv, d_rep = to_dev(inv.astype(np.uint32)), to_dev(first.astype(np.uint32))
+    hip.call("ugk_replicate_rows", ptr(d_out), row_bytes, ptr(d_inv), ptr(d_rep), n, None)
+    sync()
+    assert to_np(d_out)[: n * row_bytes].tobytes() == table[keys].tobytes()
+    assert hip.call("ugk_replicate_rows", ptr(d_out), row_bytes, None, None, 0, None) == 0

@@ -270,13 +270,66 @@ static int GatherDirect(const void *src, uint64_t rows, const Id64Type *keys, si
                         unsigned max_blocks, uint32_t *status, uint32_t *mirror, StreamHandle s) {
   return ugk_gather_direct_i64(src, rows, keys, n, out, rb, max_blocks, status, mirror, s);
 }
-static int Classify(ugk_table_t t, const IdType *keys, size_t n, uint64_t host_rows, ugk_idx_t *idx, uint32_t *c,
-                    uint32_t *next, uint32_t *st, uint32_t *mirror, StreamHandle s) {
-  return ugk_classify_u32(t, keys, n, host_rows, idx, c, next, st, mirror, s);
+static int GatherScatter(const void *src, uint64_t rows, const IdType *keys, const uint32_t *dst, size_t n, void *out,
+                         uint64_t out_rows, size_t rb, unsigned max_blocks, uint32_t *status, uint32_t *mirror,
+                         StreamHandle s) {
+  return ugk_gather_scatter_u32(src, rows, keys, dst, n, out, out_rows, rb, max_blocks, status, mirror, s);
 }
-static int Classify(ugk_table_t t, const Id64Type *keys, size_t n, uint64_t host_rows, ugk_idx_t *idx, uint32_t *c,
-                    uint32_t *next, uint32_t *st, uint32_t *mirror, StreamHandle s) {
-  return ugk_classify_i64(t, keys, n, host_rows, idx, c, next, st, mirror, s);
+static int GatherScatter(const void *src, uint64_t rows, const Id64Type *keys, const uint32_t *dst, size_t n, void *out,
+                         uint64_t out_rows, size_t rb, unsigned max_blocks, uint32_t *status, uint32_t *mirror,
+                         StreamHandle s) {
+  return ugk_gather_scatter_i64(src, rows, keys, dst, n, out, out_rows, rb, max_blocks, status, mirror, s);
+}
+static int Classify(ugk_table_t t, const IdType *keys, size_t n, uint64_t host_rows, const uint32_t *dst_map,
+                    ugk_idx_t *idx, uint32_t *c, uint32_t *next, uint32_t *st, uint32_t *mirror, StreamHandle s) {
+  return ugk_classify_u32(t, keys, n, host_rows, dst_map, idx, c, next, st, mirror, s);
+}
+static int Classify(ugk_table_t t, const Id64Type *keys, size_t n, uint64_t host_rows, const uint32_t *dst_map,
+                    ugk_idx_t *idx, uint32_t *c, uint32_t *next, uint32_t *st, uint32_t *mirror, StreamHandle s) {
+  return ugk_classify_i64(t, keys, n, host_rows, dst_map, idx, c, next, st, mirror, s);
+}
+static int Dedup(const IdType *keys, size_t n, void *ws, uint32_t epoch, IdType *uniq, uint32_t *inv, uint32_t *rep,
+                 uint32_t *nu, uint32_t *nu_host, StreamHandle s) {
+  return ugk_dedup_u32(keys, n, ws, epoch, uniq, inv, rep, nu, nu_host, s);
+}
+static int Dedup(const Id64Type *keys, size_t n, void *ws, uint32_t epoch, Id64Type *uniq, uint32_t *inv, uint32_t *rep,
+                 uint32_t *nu, uint32_t *nu_host, StreamHandle s) {
+  return ugk_dedup_i64(keys, n, ws, epoch, uniq, inv, rep, nu, nu_host, s);
+}
+
+// Deduplication in front of the extraction: the distinct keys of the batch, the index of the first occurrence of
+// each (where its row is gathered to) and, per input position, which distinct key it is.  One blocking wait: the
+// host needs the number of distinct keys to size the launches that follow.
+template <typename KeyT>
+size_t ExtractSession::DedupKeys(const KeyT *nodes, size_t num_nodes, StreamHandle stream) {
+  const size_t ws_bytes = ugk_dedup_workspace_bytes(num_nodes);
+  auto alloc = _cache_ctx->_gpu_mem_allocator;
+  if (_dedup_ws == nullptr || _dedup_ws->nbytes() < ws_bytes) {
+    _dedup_ws = nullptr;
+    const size_t grown = ugk_dedup_workspace_bytes(num_nodes + num_nodes / 4);
+    _dedup_ws = alloc(grown);
+    CHECK_NOTNULL(_dedup_ws);
+    UGK_CALL(ugk_fill_u32(_dedup_ws->ptr<uint32_t>(), 0, grown / 4, stream));
+    _dedup_epoch = 0;
+  }
+  if (_dedup_out == nullptr || _dedup_cap < num_nodes) {
+    _dedup_out = nullptr;
+    _dedup_cap = (num_nodes + num_nodes / 4 + 63) / 64 * 64;
+    _dedup_out = alloc(_dedup_cap * 16);
+    CHECK_NOTNULL(_dedup_out);
+  }
+  if (++_dedup_epoch == 0) {  // the tag wrapped: stale entries of 2^32 batches ago must not read as current
+    UGK_CALL(ugk_fill_u32(_dedup_ws->ptr<uint32_t>(), 0, _dedup_ws->nbytes() / 4, stream));
+    _dedup_epoch = 1;
+  }
+  uint32_t *n_unique = _status + 1;
+  UGK_CALL(ugk_fill_u32(n_unique, 0, 1, stream));
+  UGK_CALL(Dedup(nodes, num_nodes, _dedup_ws->ptr<void>(), _dedup_epoch, DedupUnique<KeyT>(),
+                 DedupInverse(), DedupRep(), n_unique, _host_mirror + 3, stream));
+  UGK_CALL(ugk_stream_sync(stream));
+  const size_t nu = _host_mirror[3];
+  CHECK(nu >= 1 && nu <= num_nodes) << "deduplication produced " << nu << " keys from " << num_nodes;
+  return nu;
 }
 static int ExtractMix(ugk_table_t t, const IdType *keys, size_t n, const void *cache, uint64_t cache_rows,
                       const void *host, uint64_t host_rows, void *out, size_t rb, uint32_t *st, uint32_t *mirror,
@@ -306,6 +359,21 @@ void ExtractSession::ExtractFeatImpl(const KeyT *nodes, size_t num_nodes, void *
   CHECK_NOTNULL(nodes);
   CHECK_NOTNULL(output);
 
+  // with deduplication the extraction proper runs over the distinct keys and writes each row where the key first
+  // occurs; the duplicates are filled in from there at the end
+  const size_t num_input = num_nodes;
+  const uint32_t *dst_map = nullptr, *inverse = nullptr;
+  float ms_dedup = 0;
+  if (RunConfig::dedup_keys && num_nodes >= RunConfig::dedup_min_keys) {
+    UGK_CALL(ugk_event_record(_ev_t[2], stream));
+    const size_t nu = DedupKeys(nodes, num_nodes, stream);
+    UGK_CALL(ugk_event_record(_ev_t[3], stream));
+    nodes = DedupUnique<KeyT>();
+    dst_map = DedupRep();
+    inverse = DedupInverse();
+    num_nodes = nu;
+  }
+
   if (ctx->IsDirectMapping()) {
     // fast path: no table, one gather.  Full cache reads HBM with the whole chip; no cache reads the host table
     // with the host-link budget.
@@ -313,9 +381,15 @@ void ExtractSession::ExtractFeatImpl(const KeyT *nodes, size_t num_nodes, void *
     const bool from_host = ctx->_cpu_location_id != -1;
     // the gather is bracketed by events on its own stream: the logged combine time is the kernel's duration
     UGK_CALL(ugk_event_record(_ev_t[0], stream));
-    UGK_CALL(GatherDirect(ctx->_device_cache_data[0], ctx->_num_total_nodes, nodes, num_nodes, output, rb,
-                          from_host ? _cpu_blocks : 0, _status, _host_mirror, stream));
+    if (dst_map == nullptr) {
+      UGK_CALL(GatherDirect(ctx->_device_cache_data[0], ctx->_num_total_nodes, nodes, num_nodes, output, rb,
+                            from_host ? _cpu_blocks : 0, _status, _host_mirror, stream));
+    } else {
+      UGK_CALL(GatherScatter(ctx->_device_cache_data[0], ctx->_num_total_nodes, nodes, dst_map, num_nodes, output,
+                             num_input, rb, from_host ? _cpu_blocks : 0, _status, _host_mirror, stream));
+    }
     UGK_CALL(ugk_event_record(_ev_t[1], stream));
+    if (dst_map) UGK_CALL(ugk_replicate_rows(output, rb, inverse, dst_map, num_input, stream));
     UGK_CALL(ugk_stream_sync(stream));
     CheckStatusWord(stream);
     float combine_ms = 0;
@@ -344,7 +418,7 @@ void ExtractSession::ExtractFeatImpl(const KeyT *nodes, size_t num_nodes, void *
   const uint64_t cache_rows = ctx->_cache_space_capacity;
   const uint64_t host_rows = ctx->_num_total_nodes;
 
-  if (RunConfig::concurrent_link_impl == kDirectNoGroup) {
+  if (RunConfig::concurrent_link_impl == kDirectNoGroup && dst_map == nullptr) {
     // one fused lookup + gather kernel, source chosen per row (cache_context.cu:1295-1329)
     UGK_CALL(ugk_event_record(_ev_t[0], stream));
     UGK_CALL(ExtractMix(table, nodes, num_nodes, cache, cache_rows, host, host_rows, output, rb, _status,
@@ -369,7 +443,7 @@ void ExtractSession::ExtractFeatImpl(const KeyT *nodes, size_t num_nodes, void *
   ugk_idx_t *idx = _idx_handle->ptr<ugk_idx_t>();
   uint32_t *cur = _counts[_cur], *next = _counts[_cur ^ 1];
   UGK_CALL(ugk_event_record(_ev_t[0], stream));
-  UGK_CALL(Classify(table, nodes, num_nodes, host_rows, idx, cur, next, _status, _host_mirror, stream));
+  UGK_CALL(Classify(table, nodes, num_nodes, host_rows, dst_map, idx, cur, next, _status, _host_mirror, stream));
   UGK_CALL(ugk_event_record(_ev_classified, stream));
   if (RunConfig::concurrent_link_impl == kSMMaskPhase) {
     // factored extraction: two concurrent kernels that read their group bounds from the device-side counters.
@@ -381,30 +455,31 @@ void ExtractSession::ExtractFeatImpl(const KeyT *nodes, size_t num_nodes, void *
     // that way, so a caller passing the legacy null stream would otherwise see its HBM gather serialised behind
     // the host-link gather by the null stream's implicit synchronisation.
     if (_host_on_main) {
-      UGK_CALL(ugk_gather_group(host, host_rows, idx, cur, UGK_LOC_HOST, num_nodes, output, rb, _cpu_blocks_inline,
-                                _status, _host_mirror, stream));
+      UGK_CALL(ugk_gather_group(host, host_rows, idx, cur, UGK_LOC_HOST, num_nodes, output, num_input, rb,
+                                _cpu_blocks_inline, _status, _host_mirror, stream));
       UGK_CALL(ugk_event_record(_ev_cpu_done, stream));
     } else {
       UGK_CALL(ugk_stream_wait_event(_cpu_ext_stream, _ev_classified));
-      UGK_CALL(ugk_gather_group(host, host_rows, idx, cur, UGK_LOC_HOST, num_nodes, output, rb, _cpu_blocks, _status,
-                                _host_mirror, _cpu_ext_stream));
+      UGK_CALL(ugk_gather_group(host, host_rows, idx, cur, UGK_LOC_HOST, num_nodes, output, num_input, rb, _cpu_blocks,
+                                _status, _host_mirror, _cpu_ext_stream));
       UGK_CALL(ugk_event_record(_ev_cpu_done, _cpu_ext_stream));
     }
     UGK_CALL(ugk_stream_wait_event(_local_ext_stream, _ev_classified));
-    UGK_CALL(ugk_gather_group(cache, cache_rows, idx, cur, UGK_LOC_LOCAL, num_nodes, output, rb, 0, _status,
-                              _host_mirror, _local_ext_stream));
+    UGK_CALL(ugk_gather_group(cache, cache_rows, idx, cur, UGK_LOC_LOCAL, num_nodes, output, num_input, rb, 0,
+                              _status, _host_mirror, _local_ext_stream));
     UGK_CALL(ugk_event_record(_ev_local_done, _local_ext_stream));
     if (!_host_on_main) UGK_CALL(ugk_stream_wait_event(stream, _ev_cpu_done));
     UGK_CALL(ugk_stream_wait_event(stream, _ev_local_done));
   } else {
     // sequential: host group, then local group (cache_context.cu:1719-1792)
-    UGK_CALL(ugk_gather_group(host, host_rows, idx, cur, UGK_LOC_HOST, num_nodes, output, rb, 0, _status,
-                              _host_mirror, stream));
+    UGK_CALL(ugk_gather_group(host, host_rows, idx, cur, UGK_LOC_HOST, num_nodes, output, num_input, rb, 0,
+                              _status, _host_mirror, stream));
     UGK_CALL(ugk_event_record(_ev_cpu_done, stream));
-    UGK_CALL(ugk_gather_group(cache, cache_rows, idx, cur, UGK_LOC_LOCAL, num_nodes, output, rb, 0, _status,
-                              _host_mirror, stream));
+    UGK_CALL(ugk_gather_group(cache, cache_rows, idx, cur, UGK_LOC_LOCAL, num_nodes, output, num_input, rb, 0,
+                              _status, _host_mirror, stream));
     UGK_CALL(ugk_event_record(_ev_local_done, stream));
   }
+  if (dst_map) UGK_CALL(ugk_replicate_rows(output, rb, inverse, dst_map, num_input, stream));
   // the single blocking wait of the call; the gathers have written their group sizes (and the kernels any error
   // flag) into the pinned mirror, so no device-to-host copy is needed
   UGK_CALL(ugk_stream_sync(stream));
@@ -424,6 +499,8 @@ void ExtractSession::ExtractFeatImpl(const KeyT *nodes, size_t num_nodes, void *
   } else {
     UGK_CALL(ugk_event_elapsed_ms(_ev_cpu_done, _ev_local_done, &ms_local));
   }
+  if (dst_map) UGK_CALL(ugk_event_elapsed_ms(_ev_t[2], _ev_t[3], &ms_dedup));
+  ms_idx += ms_dedup;
   if (profiler && task_key != 0xffffffffffffffffull) {
     profiler->LogStep(task_key, kLogL1FeatureBytes, nbytes);
     profiler->LogStep(task_key, kLogL1MissBytes, (double)n_miss * rb);
@@ -570,7 +647,7 @@ void RefreshSession::refresh_after_solve_new(bool foreground) {
       UGK_CALL(ugk_gather_scatter_u32(host, ctx->_num_total_nodes, insert_keys_gpu->CPtr<uint32_t>() + begin,
                                       reserved_offset->CPtr<uint32_t>() + begin, cur, cache,
                                       ctx->_cache_space_capacity, ctx->_row_bytes, limit_block, status,
-                                      low_pri_stream));
+                                      nullptr, low_pri_stream));
       if (!foreground && begin + batch < num_insert) {
         UGK_CALL(ugk_stream_sync(low_pri_stream));
         usleep(RunConfig::refresh_sleep_us);

@@ -97,6 +97,17 @@ class ExtractSession {
   unsigned _cpu_blocks_inline = 32; // ... when it runs on the caller's stream instead
   bool _host_on_main = false;  // host-link gather on the caller's stream (short miss groups) or on the confined stream
   uint32_t _group_offset[3] = {0, 0, 0};
+  // deduplication in front of the extraction (RunConfig::dedup_keys)
+  MemHandle _dedup_ws;   // epoch-tagged set, zero-filled when allocated
+  MemHandle _dedup_out;  // [n] distinct keys | [n] inverse | [n] first occurrence
+  uint32_t _dedup_epoch = 0;
+  size_t _dedup_cap = 0;  // keys the three arrays are sized for (distinct keys take 8 bytes each whatever the type)
+  template <typename KeyT>
+  KeyT *DedupUnique() const { return _dedup_out->ptr<KeyT>(); }
+  uint32_t *DedupInverse() const { return reinterpret_cast<uint32_t *>(_dedup_out->ptr<char>() + _dedup_cap * 8); }
+  uint32_t *DedupRep() const { return DedupInverse() + _dedup_cap; }
+  template <typename KeyT>
+  size_t DedupKeys(const KeyT *nodes, size_t num_nodes, StreamHandle stream);
 
   template <typename KeyT>
   void ExtractFeatImpl(const KeyT *nodes, size_t num_nodes, void *output, StreamHandle stream, uint64_t task_key);

@@ -127,6 +127,22 @@ __global__ __launch_bounds__(kBlock) void gather_kernel(Idx ix, const V *__restr
   }
 }
 
+// Re-expansion of duplicates inside one buffer: row i takes the bytes of its representative row.  Source and
+// destination are the same allocation but never the same row, so the pointers are deliberately not __restrict__.
+template <typename V, int LPR>
+__global__ __launch_bounds__(kBlock) void replicate_kernel(V *out, uint32_t vpr, const uint32_t *__restrict__ inverse,
+                                                           const uint32_t *__restrict__ rep, size_t n) {
+  constexpr int RPB = kBlock / LPR;
+  const uint32_t lane = threadIdx.x % LPR, rib = threadIdx.x / LPR;
+  for (size_t base = (size_t)blockIdx.x * RPB; base < n; base += (size_t)gridDim.x * RPB) {
+    const size_t i = base + rib;
+    if (i >= n) continue;
+    const size_t r = rep[inverse[i]];
+    if (r == i) continue;
+    for (uint32_t col = lane; col < vpr; col += LPR) out[i * vpr + col] = out[r * vpr + col];
+  }
+}
+
 // Non-temporal stores only when the output cannot stay in the memory-side cache anyway.
 // UGK_GATHER_NT_STORE=0/1 forces the choice.
 bool nt_store_for(size_t out_bytes) {
@@ -231,27 +247,53 @@ int ugk_gather_direct_i64(const void *src_dev, uint64_t src_rows, const int64_t 
 
 int ugk_gather_scatter_u32(const void *src_dev, uint64_t src_rows, const uint32_t *keys_dev,
                            const uint32_t *dst_off_dev, size_t n, void *out_dev, uint64_t out_rows, size_t row_bytes,
-                           unsigned max_blocks, uint32_t *status_dev, void *stream) {
+                           unsigned max_blocks, uint32_t *status_dev, uint32_t *host_mirror, void *stream) {
   UGK_REQUIRE(n == 0 || (keys_dev && dst_off_dev), "ugk_gather_scatter_u32: null keys or destinations");
   return launch_gather(ScatterU32{keys_dev, dst_off_dev}, src_dev, src_rows, out_dev, out_rows, row_bytes, nullptr, 0,
-                       n, max_blocks, status_dev, nullptr, stream);
+                       n, max_blocks, status_dev, host_mirror, stream);
 }
 
 int ugk_gather_scatter_i64(const void *src_dev, uint64_t src_rows, const int64_t *keys_dev,
                            const uint32_t *dst_off_dev, size_t n, void *out_dev, uint64_t out_rows, size_t row_bytes,
-                           unsigned max_blocks, uint32_t *status_dev, void *stream) {
+                           unsigned max_blocks, uint32_t *status_dev, uint32_t *host_mirror, void *stream) {
   UGK_REQUIRE(n == 0 || (keys_dev && dst_off_dev), "ugk_gather_scatter_i64: null keys or destinations");
   return launch_gather(ScatterI64{keys_dev, dst_off_dev}, src_dev, src_rows, out_dev, out_rows, row_bytes, nullptr, 0,
-                       n, max_blocks, status_dev, nullptr, stream);
+                       n, max_blocks, status_dev, host_mirror, stream);
 }
 
 int ugk_gather_group(const void *src_dev, uint64_t src_rows, const ugk_idx_t *idx_dev, const uint32_t *counts_dev,
-                     uint32_t group, size_t n, void *out_dev, size_t row_bytes, unsigned max_blocks,
-                     uint32_t *status_dev, uint32_t *host_mirror, void *stream) {
+                     uint32_t group, size_t n, void *out_dev, uint64_t out_rows, size_t row_bytes,
+                     unsigned max_blocks, uint32_t *status_dev, uint32_t *host_mirror, void *stream) {
   UGK_REQUIRE(n == 0 || (idx_dev && counts_dev), "ugk_gather_group: null index list or counts");
   UGK_REQUIRE(group == UGK_LOC_LOCAL || group == UGK_LOC_HOST, "ugk_gather_group: group %u is not local/host", group);
-  return launch_gather(IdxList{idx_dev}, src_dev, src_rows, out_dev, n, row_bytes, counts_dev, group, n, max_blocks,
+  return launch_gather(IdxList{idx_dev}, src_dev, src_rows, out_dev, out_rows, row_bytes, counts_dev, group, n, max_blocks,
                        status_dev, host_mirror, stream);
+}
+
+int ugk_replicate_rows(void *out_dev, size_t row_bytes, const uint32_t *inverse_dev, const uint32_t *rep_dev, size_t n,
+                       void *stream) {
+  if (n == 0) return 0;
+  UGK_REQUIRE(out_dev && inverse_dev && rep_dev, "ugk_replicate_rows: null pointer");
+  UGK_REQUIRE(row_bytes > 0, "ugk_replicate_rows: empty rows");
+  hipStream_t st = as_stream(stream);
+  if (((uintptr_t)out_dev | row_bytes) % 16 == 0) {
+    const uint32_t vpr = (uint32_t)(row_bytes / 16);
+    if (vpr <= 8) {
+      const unsigned grid = clamp_grid((n + kBlock / 8 - 1) / (kBlock / 8), 0);
+      hipLaunchKernelGGL((replicate_kernel<u32x4, 8>), dim3(grid), dim3(kBlock), 0, st, (u32x4 *)out_dev, vpr,
+                         inverse_dev, rep_dev, n);
+    } else {
+      const unsigned grid = clamp_grid((n + kBlock / 32 - 1) / (kBlock / 32), 0);
+      hipLaunchKernelGGL((replicate_kernel<u32x4, 32>), dim3(grid), dim3(kBlock), 0, st, (u32x4 *)out_dev, vpr,
+                         inverse_dev, rep_dev, n);
+    }
+  } else {
+    const unsigned grid = clamp_grid((n + kBlock / 32 - 1) / (kBlock / 32), 0);
+    hipLaunchKernelGGL((replicate_kernel<uint8_t, 32>), dim3(grid), dim3(kBlock), 0, st, (uint8_t *)out_dev,
+                       (uint32_t)row_bytes, inverse_dev, rep_dev, n);
+  }
+  UGK_HIP(hipGetLastError());
+  return 0;
 }
 
 int ugk_gather_idx(const void *src_dev, uint64_t src_rows, const ugk_idx_t *idx_dev, size_t count, void *out_dev,

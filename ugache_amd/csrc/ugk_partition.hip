@@ -19,7 +19,8 @@ constexpr int kWavesPerBlock = kBlock / kWave;
 
 template <typename K, int KIND>
 __global__ __launch_bounds__(kBlock) void classify_kernel(ugk_table_t t, const K *__restrict__ keys, size_t n,
-                                                          uint64_t host_rows, ugk_idx_t *__restrict__ idx,
+                                                          uint64_t host_rows, const uint32_t *__restrict__ dst_map,
+                                                          ugk_idx_t *__restrict__ idx,
                                                           uint32_t *counts, uint32_t *next_counts, uint32_t *status,
                                                           uint32_t *host_mirror) {
   __shared__ uint2 stage[kTile];
@@ -87,7 +88,8 @@ __global__ __launch_bounds__(kBlock) void classify_kernel(ugk_table_t t, const K
     }
 #pragma unroll
     for (int j = 0; j < kItems; ++j) {
-      const uint32_t i32 = (uint32_t)(tile0 + (size_t)j * kBlock + tid);
+      uint32_t i32 = (uint32_t)(tile0 + (size_t)j * kBlock + tid);
+      if (dst_map && cls[j] != 0) i32 = dst_map[i32];
       if (cls[j] == 1) stage[hoff[j] + pre[j]] = make_uint2(i32, off[j]);
       if (cls[j] == 2) stage[kTile - M + moff[j] + pre[j]] = make_uint2(i32, off[j]);
     }
@@ -157,7 +159,8 @@ template <typename K>
 __global__ __launch_bounds__(kBlock) void dedup_claim_kernel(const K *__restrict__ keys, size_t n,
                                                              unsigned long long *slots, size_t cap_mask,
                                                              uint32_t epoch, uint32_t *uid_of, K *unique_out,
-                                                             uint32_t *inverse, uint32_t *n_unique) {
+                                                             uint32_t *inverse, uint32_t *rep_of,
+                                                             uint32_t *n_unique) {
   __shared__ uint32_t wave_tot[kWavesPerBlock];
   __shared__ uint32_t base;
   __shared__ K stage[kBlock];
@@ -210,14 +213,19 @@ __global__ __launch_bounds__(kBlock) void dedup_claim_kernel(const K *__restrict
     if (tid == 0) base = total ? atomicAdd(n_unique, total) : 0u;
     if (winner) stage[before + pre] = key;
     __syncthreads();
-    if (winner) uid_of[i] = base + before + pre;
+    if (winner) {
+      uid_of[i] = base + before + pre;
+      if (rep_of) rep_of[base + before + pre] = (uint32_t)i;
+    }
     if ((uint32_t)tid < total) unique_out[base + tid] = stage[tid];
     __syncthreads();
   }
 }
 
 __global__ __launch_bounds__(kBlock) void dedup_resolve_kernel(size_t n, const uint32_t *__restrict__ uid_of,
-                                                               uint32_t *inverse) {
+                                                               uint32_t *inverse, const uint32_t *n_unique,
+                                                               uint32_t *n_unique_host) {
+  if (n_unique_host && blockIdx.x == 0 && threadIdx.x == 0) *n_unique_host = *n_unique;
   for (size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x; i < n; i += (size_t)gridDim.x * kBlock)
     inverse[i] = uid_of[inverse[i]];
 }
@@ -229,8 +237,8 @@ size_t dedup_capacity(size_t n) {
 }
 
 template <typename K>
-int classify(ugk_table_t t, const K *keys, size_t n, uint64_t host_rows, ugk_idx_t *idx, uint32_t *counts,
-             uint32_t *next_counts, uint32_t *status, uint32_t *host_mirror, void *stream) {
+int classify(ugk_table_t t, const K *keys, size_t n, uint64_t host_rows, const uint32_t *dst_map, ugk_idx_t *idx,
+             uint32_t *counts, uint32_t *next_counts, uint32_t *status, uint32_t *host_mirror, void *stream) {
   UGK_REQUIRE(counts && status, "ugk_classify: null counters or status");
   UGK_REQUIRE(n <= 0xffffffffull, "ugk_classify: batch of %zu keys exceeds 2^32", n);
   UGK_REQUIRE(t.kind == 1 || t.kind == 2, "ugk_classify: table kind %d is not flat(1) or hash(2)", t.kind);
@@ -243,10 +251,10 @@ int classify(ugk_table_t t, const K *keys, size_t n, uint64_t host_rows, ugk_idx
   const unsigned grid = clamp_grid((n + kTile - 1) / kTile, 0);
   if (t.kind == 1)
     hipLaunchKernelGGL((classify_kernel<K, 1>), dim3(grid), dim3(kBlock), 0, as_stream(stream), t, keys, n, host_rows,
-                       idx, counts, next_counts, status, host_mirror);
+                       dst_map, idx, counts, next_counts, status, host_mirror);
   else
     hipLaunchKernelGGL((classify_kernel<K, 2>), dim3(grid), dim3(kBlock), 0, as_stream(stream), t, keys, n, host_rows,
-                       idx, counts, next_counts, status, host_mirror);
+                       dst_map, idx, counts, next_counts, status, host_mirror);
   UGK_HIP(hipGetLastError());
   return 0;
 }
@@ -298,8 +306,8 @@ int extract_mix(ugk_table_t t, const K *keys, size_t n, const void *cache, uint6
 }
 
 template <typename K>
-int dedup(const K *keys, size_t n, void *workspace, uint32_t epoch, K *unique_out, uint32_t *inverse,
-          uint32_t *n_unique, void *stream) {
+int dedup(const K *keys, size_t n, void *workspace, uint32_t epoch, K *unique_out, uint32_t *inverse, uint32_t *rep_of,
+          uint32_t *n_unique, uint32_t *n_unique_host, void *stream) {
   if (n == 0) return 0;
   UGK_REQUIRE(keys && workspace && unique_out && inverse && n_unique, "ugk_dedup: null pointer");
   UGK_REQUIRE(epoch != 0, "ugk_dedup: epoch must be non-zero");
@@ -310,9 +318,10 @@ int dedup(const K *keys, size_t n, void *workspace, uint32_t epoch, K *unique_ou
   uint32_t *uid_of = reinterpret_cast<uint32_t *>(slots + cap);
   const unsigned grid = clamp_grid((n + kBlock - 1) / kBlock, 0);
   hipLaunchKernelGGL(dedup_claim_kernel<K>, dim3(grid), dim3(kBlock), 0, as_stream(stream), keys, n, slots, cap - 1,
-                     epoch, uid_of, unique_out, inverse, n_unique);
+                     epoch, uid_of, unique_out, inverse, rep_of, n_unique);
   UGK_HIP(hipGetLastError());
-  hipLaunchKernelGGL(dedup_resolve_kernel, dim3(grid), dim3(kBlock), 0, as_stream(stream), n, uid_of, inverse);
+  hipLaunchKernelGGL(dedup_resolve_kernel, dim3(grid), dim3(kBlock), 0, as_stream(stream), n, uid_of, inverse,
+                     n_unique, n_unique_host);
   UGK_HIP(hipGetLastError());
   return 0;
 }
@@ -324,17 +333,17 @@ using namespace ugk;
 
 extern "C" {
 
-int ugk_classify_u32(ugk_table_t t, const uint32_t *keys_dev, size_t n, uint64_t host_rows, ugk_idx_t *idx_dev,
-                     uint32_t *counts_dev, uint32_t *next_counts_dev, uint32_t *status_dev, uint32_t *host_mirror,
-                     void *stream) {
-  return classify<uint32_t>(t, keys_dev, n, host_rows, idx_dev, counts_dev, next_counts_dev, status_dev, host_mirror,
-                            stream);
+int ugk_classify_u32(ugk_table_t t, const uint32_t *keys_dev, size_t n, uint64_t host_rows, const uint32_t *dst_map_dev,
+                     ugk_idx_t *idx_dev, uint32_t *counts_dev, uint32_t *next_counts_dev, uint32_t *status_dev,
+                     uint32_t *host_mirror, void *stream) {
+  return classify<uint32_t>(t, keys_dev, n, host_rows, dst_map_dev, idx_dev, counts_dev, next_counts_dev, status_dev,
+                            host_mirror, stream);
 }
-int ugk_classify_i64(ugk_table_t t, const int64_t *keys_dev, size_t n, uint64_t host_rows, ugk_idx_t *idx_dev,
-                     uint32_t *counts_dev, uint32_t *next_counts_dev, uint32_t *status_dev, uint32_t *host_mirror,
-                     void *stream) {
-  return classify<int64_t>(t, keys_dev, n, host_rows, idx_dev, counts_dev, next_counts_dev, status_dev, host_mirror,
-                           stream);
+int ugk_classify_i64(ugk_table_t t, const int64_t *keys_dev, size_t n, uint64_t host_rows, const uint32_t *dst_map_dev,
+                     ugk_idx_t *idx_dev, uint32_t *counts_dev, uint32_t *next_counts_dev, uint32_t *status_dev,
+                     uint32_t *host_mirror, void *stream) {
+  return classify<int64_t>(t, keys_dev, n, host_rows, dst_map_dev, idx_dev, counts_dev, next_counts_dev, status_dev,
+                           host_mirror, stream);
 }
 
 int ugk_extract_mix_u32(ugk_table_t t, const uint32_t *keys_dev, size_t n, const void *cache_dev, uint64_t cache_rows,
@@ -353,12 +362,16 @@ int ugk_extract_mix_i64(ugk_table_t t, const int64_t *keys_dev, size_t n, const 
 size_t ugk_dedup_workspace_bytes(size_t n) { return dedup_capacity(n) * 8 + ((n + 1) / 2 * 2) * 4 + 64; }
 
 int ugk_dedup_u32(const uint32_t *keys_dev, size_t n, void *workspace_dev, uint32_t epoch, uint32_t *unique_out_dev,
-                  uint32_t *inverse_out_dev, uint32_t *n_unique_dev, void *stream) {
-  return dedup<uint32_t>(keys_dev, n, workspace_dev, epoch, unique_out_dev, inverse_out_dev, n_unique_dev, stream);
+                  uint32_t *inverse_out_dev, uint32_t *rep_out_dev, uint32_t *n_unique_dev, uint32_t *n_unique_host,
+                  void *stream) {
+  return dedup<uint32_t>(keys_dev, n, workspace_dev, epoch, unique_out_dev, inverse_out_dev, rep_out_dev, n_unique_dev,
+                         n_unique_host, stream);
 }
 int ugk_dedup_i64(const int64_t *keys_dev, size_t n, void *workspace_dev, uint32_t epoch, int64_t *unique_out_dev,
-                  uint32_t *inverse_out_dev, uint32_t *n_unique_dev, void *stream) {
-  return dedup<int64_t>(keys_dev, n, workspace_dev, epoch, unique_out_dev, inverse_out_dev, n_unique_dev, stream);
+                  uint32_t *inverse_out_dev, uint32_t *rep_out_dev, uint32_t *n_unique_dev, uint32_t *n_unique_host,
+                  void *stream) {
+  return dedup<int64_t>(keys_dev, n, workspace_dev, epoch, unique_out_dev, inverse_out_dev, rep_out_dev, n_unique_dev,
+                        n_unique_host, stream);
 }
 
 }  // extern "C"

@@ -70,9 +70,10 @@ SIGNATURES = {
     "ugk_copy_rows": [_vp, _vp, _sz, _vp],
     "ugk_gather_direct_u32": [_vp, _u64, _vp, _sz, _vp, _sz, C.c_uint, _vp, _vp, _vp],
     "ugk_gather_direct_i64": [_vp, _u64, _vp, _sz, _vp, _sz, C.c_uint, _vp, _vp, _vp],
-    "ugk_gather_scatter_u32": [_vp, _u64, _vp, _vp, _sz, _vp, _u64, _sz, C.c_uint, _vp, _vp],
-    "ugk_gather_scatter_i64": [_vp, _u64, _vp, _vp, _sz, _vp, _u64, _sz, C.c_uint, _vp, _vp],
-    "ugk_gather_group": [_vp, _u64, _vp, _vp, _u32, _sz, _vp, _sz, C.c_uint, _vp, _vp, _vp],
+    "ugk_gather_scatter_u32": [_vp, _u64, _vp, _vp, _sz, _vp, _u64, _sz, C.c_uint, _vp, _vp, _vp],
+    "ugk_gather_scatter_i64": [_vp, _u64, _vp, _vp, _sz, _vp, _u64, _sz, C.c_uint, _vp, _vp, _vp],
+    "ugk_replicate_rows": [_vp, _sz, _vp, _vp, _sz, _vp],
+    "ugk_gather_group": [_vp, _u64, _vp, _vp, _u32, _sz, _vp, _u64, _sz, C.c_uint, _vp, _vp, _vp],
     "ugk_gather_idx": [_vp, _u64, _vp, _sz, _vp, _sz, C.c_uint, _vp, _vp],
     "ugk_hash_buckets_for": [_sz, C.c_double],
     "ugk_hash_init": [_vp, _sz, _vp],
@@ -83,13 +84,13 @@ SIGNATURES = {
     "ugk_table_lookup_u32": [Table, _vp, _sz, _u32, _vp, _vp, _vp],
     "ugk_table_lookup_i64": [Table, _vp, _sz, _u32, _vp, _vp, _vp],
     "ugk_hash_census": [_vp, _sz, _vp, _vp],
-    "ugk_classify_u32": [Table, _vp, _sz, _u64, _vp, _vp, _vp, _vp, _vp, _vp],
-    "ugk_classify_i64": [Table, _vp, _sz, _u64, _vp, _vp, _vp, _vp, _vp, _vp],
+    "ugk_classify_u32": [Table, _vp, _sz, _u64, _vp, _vp, _vp, _vp, _vp, _vp, _vp],
+    "ugk_classify_i64": [Table, _vp, _sz, _u64, _vp, _vp, _vp, _vp, _vp, _vp, _vp],
     "ugk_extract_mix_u32": [Table, _vp, _sz, _vp, _u64, _vp, _u64, _vp, _sz, _vp, _vp, _vp],
     "ugk_extract_mix_i64": [Table, _vp, _sz, _vp, _u64, _vp, _u64, _vp, _sz, _vp, _vp, _vp],
     "ugk_dedup_workspace_bytes": [_sz],
-    "ugk_dedup_u32": [_vp, _sz, _vp, _u32, _vp, _vp, _vp, _vp],
-    "ugk_dedup_i64": [_vp, _sz, _vp, _u32, _vp, _vp, _vp, _vp],
+    "ugk_dedup_u32": [_vp, _sz, _vp, _u32, _vp, _vp, _vp, _vp, _vp, _vp],
+    "ugk_dedup_i64": [_vp, _sz, _vp, _u32, _vp, _vp, _vp, _vp, _vp, _vp],
     "ugk_last_error": [],
 }
 _RESTYPES = {"ugk_hash_buckets_for": _sz, "ugk_dedup_workspace_bytes": _sz, "ugk_last_error": C.c_char_p}
