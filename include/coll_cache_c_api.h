@@ -110,6 +110,11 @@ size_t coll_cache_rank_hotness(int replica_id, uint32_t *keys_out, uint32_t *cnt
  * (cached) or 1 (host); returns the number of cached keys */
 uint32_t coll_cache_place_ranked(const uint32_t *rank_keys, const uint32_t *rank_freq, uint32_t num_node,
                                  double cache_percentage, uint32_t *nid_to_block_out);
+/* the two steps above in one, as coll_cache_init_c and coll_cache_refresh run them (ranking consumed from the
+ * recorder, solver fed with the observed keys only: solve_impl_master(ContFreqBuf*), facade.cc:161-236); keys never
+ * recorded rank behind all recorded ones in ascending order.  num_node must equal num_total_item. */
+uint32_t coll_cache_place_recorded(int replica_id, uint32_t num_node, double cache_percentage,
+                                   uint32_t *nid_to_block_out);
 /* drop every global object so that coll_cache_config may be called again (the reference has no teardown) */
 void coll_cache_shutdown(void);
 

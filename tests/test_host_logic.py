@@ -82,6 +82,26 @@ def test_placement_matches_oracle_rep_solve(pct):
     assert set(cached.tolist()) == set(rank_k[:n_cached].tolist())
 
 
+@pytest.mark.parametrize("pct,n_stream", [(0.05, 100_000), (0.4, 100_000), (0.9, 3_000), (0.0, 10), (0.999, 1)])
+def test_placement_from_the_recorder_matches_the_full_rank_list(pct, n_stream):
+    """the solver fed with the observed keys only (what init and refresh run) gives the placement of the full rank
+    list, also when the cache is larger than the observed set and never-recorded keys fill it in ascending order"""
+    rng = np.random.default_rng(n_stream)
+    n_item = 70_000
+    _config(n_item, pct)
+    cc._basics.coll_cache_record_init(0)
+    stream = (rng.zipf(1.2, size=n_stream) % n_item).astype(np.uint32)
+    C.coll_cache_record(0, stream.ctypes.data, len(stream))
+    rank_k, _ = ORC.full_rank(stream, n_item)
+    want, want_n = ORC.rep_solve(rank_k, n_item, pct * 100)
+    got = np.full(n_item, 7, np.uint32)
+    n_cached = C.coll_cache_place_recorded(0, n_item, pct, got.ctypes.data)
+    assert n_cached == want_n
+    assert np.array_equal(got, want)
+    if pct == 0.9:
+        assert want_n > len(np.unique(stream))  # this case did reach into the never-recorded keys
+
+
 def test_config_is_once_per_process_and_requires_keys():
     # violations abort() like the reference's CHECKs, so they are observed in a child process
     code = textwrap.dedent("""

@@ -567,6 +567,8 @@ void RefreshSession::refresh_after_solve_new(bool foreground) {
   }
 
   // Step 1: key list of the new placement
+  Timer t_phase;
+  double detect_s = 0, evict_s = 0, wait_s = 0, insert_s = 0;
   TensorPtr key_list_of_each_src[9] = {nullptr};
   const size_t num_block = coll_cache->_block_access_advise->Shape()[1];
   TensorPtr advise_line = Tensor::FromBlob(coll_cache->_block_access_advise->Ptr<uint8_t>() + (size_t)local * num_block,
@@ -601,6 +603,8 @@ void RefreshSession::refresh_after_solve_new(bool foreground) {
   }
   const size_t num_evicted = new_evict_keys->NumItem();
   CHECK_EQ(num_evicted + num_preserved_key, table->_cached_keys->NumItem());
+  detect_s = t_phase.Passed();
+  t_phase.Reset();
   if (num_evicted > 0) {
     auto evict_keys_gpu = RunConfig::key_map_mul == 0
                               ? CopyTo1DReuse(__keys_buffer, new_evict_keys, gpu_ctx, stream)
@@ -619,6 +623,8 @@ void RefreshSession::refresh_after_solve_new(bool foreground) {
   LOG(INFO) << "refresh: preserved " << num_preserved_key << ", evict " << num_evicted << ", insert "
             << new_insert_keys->NumItem() << ", free slots " << table->_free_offsets->NumItem();
 
+  evict_s = t_phase.Passed();
+  t_phase.Reset();
   // Step 5: let one more lookup finish, so that no gather in flight still reads a slot about to be reused
   const size_t current_progress = ctx->progress.load();
   AnonymousBarrier::_refresh_instance->Wait();
@@ -630,6 +636,8 @@ void RefreshSession::refresh_after_solve_new(bool foreground) {
     }
   }
 
+  wait_s = t_phase.Passed();
+  t_phase.Reset();
   // Step 6: copy the new rows host -> HBM into slots taken from the front of the free list, then publish them
   const size_t num_insert = new_insert_keys->NumItem();
   if (num_insert > 0) {
@@ -666,9 +674,14 @@ void RefreshSession::refresh_after_solve_new(bool foreground) {
   }
   AnonymousBarrier::_refresh_instance->Wait();
 
+  insert_s = t_phase.Passed();
+  t_phase.Reset();
   table->_cached_keys = key_list_of_each_src[local];
   ctx->_cache_nodes = num_new_local_key;
-  table->MaybeRebuild(ctx->_eager_gpu_mem_allocator, gpu_ctx, local, stream);
+  const bool rebuilt = table->MaybeRebuild(ctx->_eager_gpu_mem_allocator, gpu_ctx, local, stream);
+  LOG(INFO) << "refresh: key lists " << detect_s << " s, evict " << evict_s << " s, wait for a lookup " << wait_s
+            << " s, row copy + insert " << insert_s << " s, table rebuild " << (rebuilt ? t_phase.Passed() : 0.0)
+            << " s";
   CHECK_EQ(table->_free_offsets->NumItem() + num_new_local_key, ctx->_cache_space_capacity);
 }
 

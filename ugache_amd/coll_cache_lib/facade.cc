@@ -122,8 +122,12 @@ void CollCache::build_common(int replica_id, std::function<void()> solve, IdType
   this->_refresh_session_list[replica_id]->_cache_ctx = cache_ctx;
   this->_refresh_session_list[replica_id]->stream = stream;
   this->_replica_barrier->Wait();
+  // after the build the host scans belong to the refresher.  The reference's defaults (8 threads, 1 per GPU of an
+  // 8-GPU node: run_config.cc:53-54) give the one GPU here all of them.
   RunConfig::solver_omp_thread_num = RunConfig::refresher_omp_thread_num;
-  RunConfig::solver_omp_thread_num_per_gpu = RunConfig::refresher_omp_thread_num_per_gpu;
+  RunConfig::solver_omp_thread_num_per_gpu =
+      std::max<int>(RunConfig::refresher_omp_thread_num_per_gpu,
+                    RunConfig::refresher_omp_thread_num / (int)RunConfig::num_device);
 }
 
 // facade.cc:283-381
@@ -175,12 +179,16 @@ void CollCache::refresh(int replica_id, ContFreqBuf *freq_rank, StreamHandle str
   CHECK_EQ(replica_id, 0);
   CHECK_NOTNULL(_nid_to_block) << "refresh needs a cache built with 0 < cache_percentage < 1";
   AnonymousBarrier::_refresh_instance->Wait();
+  Timer t_solve;
   preserve_old_solution();
   solve_impl_master(freq_rank, (IdType)RunConfig::num_total_item);
+  const double solve_s = t_solve.Passed();
   AnonymousBarrier::_refresh_instance->Wait();
+  Timer t_apply;
   this->_refresh_session_list[replica_id]->stream = stream;
   this->_refresh_session_list[replica_id]->refresh_after_solve_main(foreground);
   AnonymousBarrier::_refresh_instance->Wait();
+  LOG(INFO) << "refresh: placement " << solve_s << " s, evict + insert " << t_apply.Passed() << " s";
 }
 
 void CollCache::report_last_epoch(uint64_t epoch) { _profiler->ReportStepAverageLastEpoch(epoch + 1, 0); }

@@ -1,6 +1,7 @@
 #include "freq_recorder.h"
 
 #include <algorithm>
+#include <cstdlib>
 #include <cstring>
 #include <limits>
 #include <parallel/algorithm>
@@ -52,18 +53,28 @@ void ContFreqBuf::GetLegacyFreqRank(LegacyFreqBuf *output, size_t total_num_node
   CHECK_EQ(pos, total_num_node);
 }
 
+namespace {
+int ScanThreads() { return std::max(1, RunConfig::solver_omp_thread_num_per_gpu); }
+}  // namespace
+
 FreqRecorder::FreqRecorder(size_t num_nodes, int local_id) : _num_nodes(num_nodes), _local_id(local_id) {
   CHECK(num_nodes < std::numeric_limits<IdType>::max() / 2);
-  _live.assign(num_nodes, 0);
+  _live = static_cast<CntT *>(calloc(std::max<size_t>(num_nodes, 1), sizeof(CntT)));
+  _shared = static_cast<CntT *>(calloc(std::max<size_t>(num_nodes, 1), sizeof(CntT)));
+  CHECK(_live != nullptr && _shared != nullptr) << "no memory for the counters of " << num_nodes << " keys";
   global_cont_freq_buf = new ContFreqBuf;
 }
 
-FreqRecorder::~FreqRecorder() { delete global_cont_freq_buf; }
+FreqRecorder::~FreqRecorder() {
+  delete global_cont_freq_buf;
+  free(_live);
+  free(_shared);
+}
 
 template <typename KeyT>
 void FreqRecorder::Record(const KeyT *input, size_t num_inputs) {
   std::lock_guard<std::mutex> g(_mu);
-  CntT *cnt = _live.data();
+  CntT *cnt = _live;
   const size_t n_nodes = _num_nodes;
   bool bad = false;
 #pragma omp parallel for num_threads(RunConfig::solver_omp_thread_num_per_gpu) reduction(|| : bad) if (num_inputs > 65536)
@@ -82,12 +93,14 @@ template void FreqRecorder::Record<IdType>(const IdType *input, size_t num_input
 
 void FreqRecorder::LocalCombineToShared() {
   std::lock_guard<std::mutex> g(_mu);
-  if (_shared.empty()) {
-    _shared.swap(_live);
-    _live.assign(_num_nodes, 0);
-  } else {
-    for (size_t i = 0; i < _num_nodes; i++) _shared[i] += _live[i];
-    std::fill(_live.begin(), _live.end(), 0);
+  CntT *shared = _shared, *live = _live;
+  const size_t n = _num_nodes;
+#pragma omp parallel for num_threads(ScanThreads())
+  for (size_t i = 0; i < n; i++) {
+    if (live[i]) {  // the recorded keys are a small part of the key space: write only where something was counted
+      shared[i] += live[i];
+      live[i] = 0;
+    }
   }
 }
 
@@ -95,12 +108,32 @@ void FreqRecorder::GlobalCombine() {
   std::lock_guard<std::mutex> g(_mu);
   auto &e = global_cont_freq_buf->entries;
   e.clear();
-  for (size_t k = 0; k < _shared.size(); k++)
-    if (_shared[k]) e.push_back({(IdType)k, _shared[k]});
+  // count, scan, fill: the entries come out in ascending key order whatever the thread count
+  const int nthr = ScanThreads();
+  const size_t n = _num_nodes, chunk = (n + nthr - 1) / nthr;
+  CntT *shared = _shared;
+  std::vector<size_t> first(nthr + 1, 0);
+#pragma omp parallel for num_threads(nthr) schedule(static, 1)
+  for (int t = 0; t < nthr; t++) {
+    const size_t lo = std::min(n, chunk * t), hi = std::min(n, chunk * (t + 1));
+    size_t c = 0;
+    for (size_t k = lo; k < hi; k++) c += shared[k] != 0;
+    first[t + 1] = c;
+  }
+  for (int t = 0; t < nthr; t++) first[t + 1] += first[t];
+  e.resize(first[nthr]);
+#pragma omp parallel for num_threads(nthr) schedule(static, 1)
+  for (int t = 0; t < nthr; t++) {
+    const size_t lo = std::min(n, chunk * t), hi = std::min(n, chunk * (t + 1));
+    size_t pos = first[t];
+    for (size_t k = lo; k < hi; k++)
+      if (shared[k]) {
+        e[pos++] = {(IdType)k, shared[k]};
+        shared[k] = 0;  // the next round of counts starts from zero
+      }
+  }
   global_cont_freq_buf->buf = e.data();
   LOG(INFO) << "freq recorder global combine: " << e.size() << " distinct keys";
-  _shared.clear();
-  _shared.shrink_to_fit();
 }
 
 void FreqRecorder::Sort() {

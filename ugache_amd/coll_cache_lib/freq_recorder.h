@@ -56,8 +56,9 @@ class FreqRecorder {
  private:
   size_t _num_nodes;
   int _local_id;
-  std::vector<CntT> _live;    // counts being recorded
-  std::vector<CntT> _shared;  // counts handed over by LocalCombineToShared
+  // one counter per key of the key space, calloc-backed so that pages nobody counted in are never touched
+  CntT *_live = nullptr;    // counts being recorded
+  CntT *_shared = nullptr;  // counts handed over by LocalCombineToShared
   std::mutex _mu;
 };
 

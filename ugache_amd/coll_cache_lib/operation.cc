@@ -14,6 +14,7 @@
 #include "placement.h"
 #include "profiler.h"
 #include "run_config.h"
+#include "timer.h"
 #include "ugache_hip.h"
 
 namespace coll_cache_lib {
@@ -246,7 +247,9 @@ void coll_cache_set_key_map(uint64_t mul, int bits) {
 
 void coll_cache_refresh(int replica_id, StreamHandle stream, int foreground) {
   CHECK_NOTNULL(_coll_cache);
+  Timer t_rank;
   ContFreqBuf *freq_rank = CombineAndRank(replica_id);
+  LOG(INFO) << "refresh: ranking " << t_rank.Passed() << " s";
   _coll_cache->refresh(replica_id, freq_rank, stream, foreground != 0);
 }
 
@@ -320,6 +323,23 @@ uint32_t coll_cache_place_ranked(const uint32_t *rank_keys, const uint32_t *rank
   auto freq = Tensor::FromBlob(const_cast<uint32_t *>(rank_freq), kI32, {1, (size_t)num_node}, CPU(CPU_FOREIGN), "");
   auto n2b = Tensor::FromBlob(nid_to_block_out, kI32, {(size_t)num_node}, CPU(CPU_FOREIGN), "");
   solver.Build(keys, freq, {0}, num_node, n2b);
+  solver.Solve({0}, {cache_percentage * 100}, "BIN", RunConfig::coll_cache_hyperparam_T_local,
+               RunConfig::coll_cache_hyperparam_T_cpu);
+  uint32_t cached = 0;
+  for (uint32_t k = 0; k < num_node; k++) cached += nid_to_block_out[k] == 0;
+  return cached;
+}
+
+uint32_t coll_cache_place_recorded(int replica_id, uint32_t num_node, double cache_percentage,
+                                   uint32_t *nid_to_block_out) {
+  CHECK(RunConfig::is_configured);
+  CHECK_NOTNULL(nid_to_block_out);
+  CHECK_EQ((size_t)num_node, RunConfig::num_total_item);
+  ContFreqBuf *rank = CombineAndRank(replica_id);
+  CHECK_NOTNULL(rank);
+  coll_cache::FreqRankSolver solver;
+  auto n2b = Tensor::FromBlob(nid_to_block_out, kI32, {(size_t)num_node}, CPU(CPU_FOREIGN), "");
+  solver.BuildSingleStream(rank, {0}, num_node, n2b);
   solver.Solve({0}, {cache_percentage * 100}, "BIN", RunConfig::coll_cache_hyperparam_T_local,
                RunConfig::coll_cache_hyperparam_T_cpu);
   uint32_t cached = 0;

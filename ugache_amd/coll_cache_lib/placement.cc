@@ -1,5 +1,6 @@
 #include "placement.h"
 
+#include <algorithm>
 #include <cstring>
 #include <iostream>
 
@@ -18,6 +19,7 @@ void FreqRankSolver::Build(TensorPtr stream_id_list, TensorPtr stream_freq_list,
   CHECK_EQ(stream_freq_list->NumItem(), (size_t)num_node);
   _rank_keys = stream_id_list;
   _rank_freq = stream_freq_list;
+  _cont = nullptr;
   _nid_to_block = nid_to_block_tensor;
   _num_node = num_node;
 }
@@ -25,14 +27,66 @@ void FreqRankSolver::Build(TensorPtr stream_id_list, TensorPtr stream_freq_list,
 void FreqRankSolver::BuildSingleStream(ContFreqBuf *freq_rank, std::vector<int> device_to_stream,
                                        const IdType num_node, const TensorPtr nid_to_block_tensor) {
   CHECK_NOTNULL(freq_rank);
-  LegacyFreqBuf legacy;
-  freq_rank->GetLegacyFreqRank(&legacy, num_node);
-  _rank_keys = Tensor::Empty(kI32, {(size_t)num_node}, CPU_CLIB(), "rank_keys");
-  _rank_freq = Tensor::Empty(kI32, {(size_t)num_node}, CPU_CLIB(), "rank_freq");
-  memcpy(_rank_keys->MutableData(), legacy.rank_vec.data(), (size_t)num_node * sizeof(IdType));
-  memcpy(_rank_freq->MutableData(), legacy.freq_vec.data(), (size_t)num_node * sizeof(IdType));
+  CHECK_LE(freq_rank->size(), (size_t)num_node);
+  _cont = freq_rank;
+  _rank_keys = nullptr;
+  _rank_freq = nullptr;
   _nid_to_block = nid_to_block_tensor;
   _num_node = num_node;
+}
+
+// Same result as walking the full rank list (observed keys in rank order, then the never-observed keys in
+// ascending order), without materialising it: the key space can be hundreds of millions of keys of which a refresh
+// has observed a small part.
+void FreqRankSolver::SolveFromObserved(IdType num_cached_nodes, double *rep_w_out, double *cpu_w_out) {
+  const size_t num_node = _num_node, m = _cont->size(), k_cached = num_cached_nodes;
+  const auto *e = _cont->buf;
+  IdType *nid_to_block = _nid_to_block->Ptr<IdType>();
+  const int nthr = std::max(1, RunConfig::omp_thread_num);
+#pragma omp parallel for num_threads(nthr)
+  for (size_t k = 0; k < num_node; k++) nid_to_block[k] = 1;
+  double rep_w = 0, cpu_w = 0;
+  bool bad = false;
+  const size_t top = std::min(m, k_cached);
+#pragma omp parallel for num_threads(nthr) reduction(+ : rep_w, cpu_w) reduction(|| : bad)
+  for (size_t r = 0; r < m; r++) {
+    if (e[r].key >= num_node) {
+      bad = true;
+    } else if (r < top) {
+      nid_to_block[e[r].key] = 0;
+      rep_w += e[r].cnt;
+    } else {
+      cpu_w += e[r].cnt;
+    }
+  }
+  CHECK(!bad) << "a ranked key is outside the key space of " << num_node;
+  if (k_cached > m) {
+    // the cache is larger than the observed set: fill it up with the smallest never-observed keys.  All m observed
+    // keys are block 0 by now, so "never observed" reads as "still block 1".
+    const size_t extra = k_cached - m;
+    const size_t chunk = (num_node + nthr - 1) / nthr;
+    std::vector<size_t> before(nthr + 1, 0);
+#pragma omp parallel for num_threads(nthr) schedule(static, 1)
+    for (int t = 0; t < nthr; t++) {
+      const size_t lo = std::min(num_node, chunk * t), hi = std::min(num_node, chunk * (t + 1));
+      size_t c = 0;
+      for (size_t k = lo; k < hi; k++) c += nid_to_block[k] == 1;
+      before[t + 1] = c;
+    }
+    for (int t = 0; t < nthr; t++) before[t + 1] += before[t];
+#pragma omp parallel for num_threads(nthr) schedule(static, 1)
+    for (int t = 0; t < nthr; t++) {
+      const size_t lo = std::min(num_node, chunk * t), hi = std::min(num_node, chunk * (t + 1));
+      size_t seen = before[t];
+      for (size_t k = lo; k < hi && seen < extra; k++)
+        if (nid_to_block[k] == 1) {
+          nid_to_block[k] = 0;
+          seen++;
+        }
+    }
+  }
+  *rep_w_out = rep_w;
+  *cpu_w_out = cpu_w;
 }
 
 void FreqRankSolver::Solve(std::vector<int> device_to_stream, std::vector<PerT> device_to_cache_percent,
@@ -43,19 +97,23 @@ void FreqRankSolver::Solve(std::vector<int> device_to_stream, std::vector<PerT> 
   const int num_block = 2;
   const IdType num_node = _num_node;
   const IdType num_cached_nodes = (IdType)(num_node * (device_to_cache_percent[0] / (double)100));
-  const IdType *rank = _rank_keys->CPtr<IdType>();
-  const IdType *freq = _rank_freq->CPtr<IdType>();
   IdType *nid_to_block = _nid_to_block->Ptr<IdType>();
   double rep_w = 0, cpu_w = 0;
+  if (_cont != nullptr) {
+    SolveFromObserved(num_cached_nodes, &rep_w, &cpu_w);
+  } else {
+    const IdType *rank = _rank_keys->CPtr<IdType>();
+    const IdType *freq = _rank_freq->CPtr<IdType>();
 #pragma omp parallel for num_threads(RunConfig::omp_thread_num) reduction(+ : rep_w, cpu_w)
-  for (IdType r = 0; r < num_node; r++) {
-    const IdType key = rank[r];
-    if (r < num_cached_nodes) {
-      nid_to_block[key] = 0;
-      rep_w += freq[r];
-    } else {
-      nid_to_block[key] = 1;
-      cpu_w += freq[r];
+    for (IdType r = 0; r < num_node; r++) {
+      const IdType key = rank[r];
+      if (r < num_cached_nodes) {
+        nid_to_block[key] = 0;
+        rep_w += freq[r];
+      } else {
+        nid_to_block[key] = 1;
+        cpu_w += freq[r];
+      }
     }
   }
   const double total_w = rep_w + cpu_w;

@@ -46,8 +46,12 @@ class FreqRankSolver : public CollCacheSolver {
              double T_local, double T_cpu) override;
 
  private:
-  TensorPtr _rank_keys;  // u32 [num_node]
-  TensorPtr _rank_freq;  // u32 [num_node]
+  TensorPtr _rank_keys;  // u32 [num_node]   (Build)
+  TensorPtr _rank_freq;  // u32 [num_node]   (Build)
+  // BuildSingleStream: the observed keys in rank order; the never-observed keys follow in ascending order
+  // (ContFreqBuf::GetLegacyFreqRank) without being written out
+  const ContFreqBuf *_cont = nullptr;
+  void SolveFromObserved(IdType num_cached_nodes, double *rep_w, double *cpu_w);
   TensorPtr _nid_to_block;
   IdType _num_node = 0;
 };

@@ -68,6 +68,7 @@ void RunConfig::LoadConfigFromEnv() {
   refresh_batch_rows = 4092;
   refresh_sleep_us = 3000;
   refresh_limit_block = 20;
+  refresher_omp_thread_num = 8;
   hash_rebuild_tombstone_frac = 0.15;
   dedup_keys = false;
   dedup_min_keys = 4096;
@@ -92,6 +93,7 @@ void RunConfig::LoadConfigFromEnv() {
   if (tbl == "FLAT") force_table_kind = 1;
   else if (tbl == "HASH") force_table_kind = 2;
   else if (tbl != "") LOG(FATAL) << "COLL_HASH_TABLE must be FLAT or HASH, got " << tbl;
+  if (GetEnv("COLL_REFRESH_THREADS") != "") refresher_omp_thread_num = std::max(1, std::stoi(GetEnv("COLL_REFRESH_THREADS")));
   if (GetEnv("COLL_REFRESH_BATCH_ROWS") != "") refresh_batch_rows = std::stoul(GetEnv("COLL_REFRESH_BATCH_ROWS"));
   if (GetEnv("COLL_REFRESH_SLEEP_US") != "") refresh_sleep_us = std::stoul(GetEnv("COLL_REFRESH_SLEEP_US"));
   if (GetEnv("COLL_REFRESH_LIMIT_BLOCK") != "") refresh_limit_block = std::stoul(GetEnv("COLL_REFRESH_LIMIT_BLOCK"));

@@ -122,6 +122,7 @@ C_API = {
     "coll_cache_rank_hotness": (ctypes.c_size_t, [ctypes.c_int, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_size_t]),
     "coll_cache_place_ranked": (ctypes.c_uint32, [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_uint32, ctypes.c_double,
                                                  ctypes.c_void_p]),
+    "coll_cache_place_recorded": (ctypes.c_uint32, [ctypes.c_int, ctypes.c_uint32, ctypes.c_double, ctypes.c_void_p]),
     "coll_cache_shutdown": (None, []),
 }
 
