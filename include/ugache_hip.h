@@ -223,6 +223,25 @@ int ugk_dedup_i64(const int64_t *keys_dev, size_t n, void *workspace_dev, uint32
                   uint32_t *inverse_out_dev, uint32_t *rep_out_dev, uint32_t *n_unique_dev, uint32_t *n_unique_host,
                   void *stream);
 
+/* ---- hotness counters on the device: FreqRecorder::Record (freq_recorder.cc:227-253) without the copy of the keys
+ *      to the host, the record thread of python_tf2/collcache_tf2/collcache_tf2/core/lookup_manager.cc:291-312 ----
+ * counts_dev: one uint32 per row of the host table, zero-filled once.  ugk_record_*: counts_dev[row(key)] += 1 for
+ * every key of the batch; row(key) = key for dense ids (key_inv = 0), else (key * key_inv) & key_mask, the inverse of
+ * the sparse-id map (the fb_mul / fb_mask of ugk_table_t).  A key without a row sets UGK_ST_KEY_OUT_OF_RANGE and is
+ * not counted. */
+int ugk_record_u32(const uint32_t *keys_dev, size_t n, uint64_t key_inv, uint64_t key_mask, uint32_t *counts_dev,
+                   uint64_t num_rows, uint32_t *status_dev, uint32_t *host_mirror, void *stream);
+int ugk_record_i64(const int64_t *keys_dev, size_t n, uint64_t key_inv, uint64_t key_mask, uint32_t *counts_dev,
+                   uint64_t num_rows, uint32_t *status_dev, uint32_t *host_mirror, void *stream);
+/* hands rows [first_row, first_row + num_rows) to the host: every non-zero counter becomes one word
+ * (count << 32) | row in entries_dev (order unspecified; the layout of the reference's FreqEntry {key, cnt},
+ * freq_recorder.h:32-40) and is reset to zero in the same atomic step, so a ugk_record_* running concurrently loses
+ * nothing.  At most `capacity` entries are written; counters that did not fit stay as they are.
+ * n_entries_dev: device word, zero on first use, left zero.  host_out: two pinned host words,
+ * [0] = entries written, [1] = 1 when rows were left over (call again). */
+int ugk_record_drain(uint32_t *counts_dev, uint64_t first_row, uint64_t num_rows, uint64_t *entries_dev,
+                     uint32_t capacity, uint32_t *n_entries_dev, uint32_t *host_out, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

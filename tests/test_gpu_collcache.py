@@ -41,7 +41,7 @@ def make_config(num_total_item, pct, threads=8):
 @pytest.fixture(autouse=True)
 def _fresh_cache(monkeypatch):
     for v in ("COLL_HASH_TABLE", "SAMGRAPH_COLL_CACHE_CONCURRENT_LINK_IMPL", "SAMGRAPH_COLL_CACHE_NO_GROUP",
-              "COLL_DEDUP_KEYS", "COLL_DEDUP_MIN_KEYS"):
+              "COLL_DEDUP_KEYS", "COLL_DEDUP_MIN_KEYS", "COLL_GPU_RECORD", "COLL_GPU_RECORD_EVERY"):
         monkeypatch.delenv(v, raising=False)
     yield
     if torch.cuda.is_available():
@@ -268,6 +268,65 @@ def test_refresh_evicts_and_inserts_like_the_oracle(table_kind, foreground, monk
         old_cached = new_cached
 
 
+@pytest.mark.parametrize("pct,impl,dedup", [(0.25, "", False), (0.25, "NONE", True), (0.25, "DIRECT", False),
+                                            (1.0, "", False), (0.0, "", True)])
+@pytest.mark.parametrize("kdtype", [torch.int32, torch.int64])
+def test_hotness_counted_on_the_device_ranks_like_the_host_recorder(pct, impl, dedup, kdtype, monkeypatch):
+    """COLL_GPU_RECORD=1: the lookups count their keys in device-side counters; the ranking taken from them equals
+    the oracle's ranking of the concatenated key stream (what coll_torch_record of the same keys gives), and a
+    refresh driven by them caches the oracle's top set."""
+    monkeypatch.setenv("COLL_GPU_RECORD", "1")
+    if impl:
+        monkeypatch.setenv("SAMGRAPH_COLL_CACHE_CONCURRENT_LINK_IMPL", impl)
+    if dedup:
+        monkeypatch.setenv("COLL_DEDUP_KEYS", "1")
+        monkeypatch.setenv("COLL_DEDUP_MIN_KEYS", "64")
+    rng = np.random.default_rng(33)
+    n_item, dim = 30_000, 64
+    co.config(make_config(n_item, pct))
+    co.coll_cache_record_init(0)
+    perm1 = rng.permutation(n_item)
+    s1 = perm1[zipf_ranks(rng, 100_000, n_item, 1.1)]
+    if 0.0 < pct < 1.0:  # the build consumes this ranking; without a partial cache nothing would
+        co.coll_torch_record(0, torch.from_numpy(s1).to(kdtype))
+    emb = co.coll_torch_create_emb_shm(0, n_item, dim, torch.float32)
+    table = fill_table(emb, rng)
+    co.coll_torch_init_t(0, 0, emb, pct)
+
+    perm2 = rng.permutation(n_item)
+    stream = []
+    for n in (1, 50_000, 3_000, 50_000):
+        keys = perm2[zipf_ranks(rng, n, n_item, 1.1)]
+        stream.append(keys)
+        out = co.coll_torch_lookup_key_t_val_ret(0, torch.from_numpy(keys).to(kdtype).cuda(), False)
+        assert out.cpu().numpy().tobytes() == ORC.gather(table, keys.astype(np.int64)).tobytes()
+    allk = np.concatenate(stream).astype(np.uint32)
+    if 0.0 < pct < 1.0:
+        # a host-side record joins the device-side counts
+        extra = perm2[zipf_ranks(rng, 10_000, n_item, 1.1)]
+        co.coll_torch_record(0, torch.from_numpy(extra).to(kdtype))
+        allk = np.concatenate([allk, extra.astype(np.uint32)])
+        new_cached, new_nid = expected_cached_set(allk, n_item, pct)
+        co.coll_torch_refresh(0, True)
+        got = np.zeros(len(new_cached), np.uint32)
+        assert _basics.C_LIB_CTYPES.coll_cache_get_cached_keys(0, got.ctypes.data, len(got)) == len(new_cached)
+        assert np.array_equal(got, new_cached)
+        keys = rng.integers(0, n_item, size=20_000)
+        out = co.coll_torch_lookup_key_t_val_ret(0, torch.from_numpy(keys).to(kdtype).cuda(), False)
+        assert out.cpu().numpy().tobytes() == ORC.gather(table, keys.astype(np.int64)).tobytes()
+        if impl != "DIRECT":  # the fused kernel produces no group sizes
+            assert _basics.last_group_offset(0)[1] == (int((new_nid[keys] == 0).sum()) if not dedup else
+                                                       int((new_nid[np.unique(keys)] == 0).sum()))
+        allk = keys.astype(np.uint32)  # the refresh consumed the counts; only this last lookup is left
+    want_k, want_c = ORC.freq_rank(allk)
+    got_k = np.zeros(n_item, np.uint32)
+    got_c = np.zeros(n_item, np.uint32)
+    m = _basics.C_LIB_CTYPES.coll_cache_rank_hotness(0, got_k.ctypes.data, got_c.ctypes.data, n_item)
+    assert m == len(want_k)
+    assert np.array_equal(got_k[:m], want_k) and np.array_equal(got_c[:m], want_c)
+    assert _basics.C_LIB_CTYPES.coll_cache_rank_hotness(0, None, None, 0) == 0  # drained
+
+
 def test_reference_cpu_runnable_config_full_size():
     """1M x 128 fp32 host table, 65536 int64 keys Zipf(1.1) over a seeded permutation, hottest 10 % cached."""
     rng = np.random.default_rng(1)
@@ -292,11 +351,14 @@ def test_reference_cpu_runnable_config_full_size():
         assert _basics.last_group_offset(0) == [0, int((nid[b] == 0).sum()), n]
 
 
-def test_sparse_ids_hash_table_with_refresh_each_step(monkeypatch):
+@pytest.mark.parametrize("gpu_record", [False, True])
+def test_sparse_ids_hash_table_with_refresh_each_step(gpu_record, monkeypatch):
     """The hashtable-mode configuration, scaled down: ids are 64-bit values from a 2^40 space (id = row * odd mod 2^40),
     rows are 64 fp16 (128 B), the cached ids sit in the open-addressing table at 0.7 load, every step is followed by a
     refresh that evicts / inserts by the newly recorded hotness; tombstones trigger table rebuilds on the way."""
     monkeypatch.setenv("COLL_HASH_REBUILD_FRAC", "0.05")
+    if gpu_record:  # the hotness of a refresh comes from the lookups themselves, counted per row on the device
+        monkeypatch.setenv("COLL_GPU_RECORD", "1")
     MUL, BITS = 0x9E3779B97F4A7C15, 40
     mask = np.uint64((1 << BITS) - 1)
     rng = np.random.default_rng(5)
@@ -339,9 +401,13 @@ def test_sparse_ids_hash_table_with_refresh_each_step(monkeypatch):
         perm[swap] = perm[rng.permutation(swap)]
         s = stream(3)
         for b in s:
-            co.coll_torch_record(0, torch.from_numpy(ids_of(b)))
+            if gpu_record:
+                co.coll_torch_lookup_key_t_val_ret(0, torch.from_numpy(ids_of(b)).cuda(), False)
+            else:
+                co.coll_torch_record(0, torch.from_numpy(ids_of(b)))
         co.coll_torch_refresh(0, True)
-        new_cached, nid = expected_cached_set(np.concatenate(s).astype(np.uint32), n_item, pct)
+        seen = ([rows_b] + s) if gpu_record else s
+        new_cached, nid = expected_cached_set(np.concatenate(seen).astype(np.uint32), n_item, pct)
         info = _basics.info(0)
         got = np.zeros(len(new_cached), np.uint32)
         assert _basics.C_LIB_CTYPES.coll_cache_get_cached_keys(0, got.ctypes.data, len(got)) == len(new_cached)

@@ -483,3 +483,68 @@ def test_replicate_rows_fills_duplicates_from_their_representative(row_bytes):
     sync()
     assert to_np(d_out)[: n * row_bytes].tobytes() == table[keys].tobytes()
     assert hip.call("ugk_replicate_rows", ptr(d_out), row_bytes, None, None, 0, None) == 0
+
+
+@pytest.mark.parametrize("kdtype", [np.uint32, np.int64])
+@pytest.mark.parametrize("sparse", [False, True])
+def test_record_and_drain_match_bincount(kdtype, sparse):
+    """device-side hotness counters: record == numpy.bincount of the rows; drain hands out every non-zero counter
+    exactly once as (count << 32 | row) and leaves the counters at zero"""
+    rng = np.random.default_rng(17 + sparse)
+    num_rows = 100_003
+    bits = 31 if kdtype == np.uint32 else 40
+    mul = (0x9E3779B97F4A7C15 | 1) & ((1 << bits) - 1) if sparse else 0
+    mask = (1 << bits) - 1 if sparse else 0
+    inv = pow(mul, -1, 1 << bits) if sparse else 0
+    counts = dev_zeros_u32(num_rows)
+    st = dev_zeros_u32(1)
+    want = np.zeros(num_rows, np.int64)
+    for n in (1, 5000, 200_001):
+        rows = (rng.zipf(1.2, size=n) % num_rows).astype(np.uint64)
+        keys = ((rows * np.uint64(mul)) & np.uint64(mask)) if sparse else rows
+        d_keys = to_dev(keys.astype(kdtype))
+        fn = "ugk_record_i64" if kdtype == np.int64 else "ugk_record_u32"
+        hip.call(fn, ptr(d_keys), n, inv, mask, ptr(counts), num_rows, ptr(st), None, None)
+        want += np.bincount(rows.astype(np.int64), minlength=num_rows)
+    sync()
+    assert status_value(st) == 0
+    assert np.array_equal(to_np(counts, np.uint32)[:num_rows].astype(np.int64), want)
+
+    # drain in two row ranges, the second with a list too short for it (left-over rows come with the next call)
+    cap = 30_000
+    entries = dev_bytes(cap * 8)
+    n_entries = dev_zeros_u32(1)
+    out = PinnedArray((2,), np.uint32)
+    try:
+        got = np.zeros(num_rows, np.int64)
+        calls = 0
+        for first, cnt in ((0, 50_000), (50_000, num_rows - 50_000)):
+            while True:
+                hip.call("ugk_record_drain", ptr(counts), first, cnt, ptr(entries), cap, ptr(n_entries), out.ptr, None)
+                sync()
+                calls += 1
+                k, more = int(out.array[0]), int(out.array[1])
+                e = to_np(entries, np.uint64)[:k]
+                r, c = (e & np.uint64(0xFFFFFFFF)).astype(np.int64), (e >> np.uint64(32)).astype(np.int64)
+                assert len(np.unique(r)) == k and (c > 0).all() and ((r >= first) & (r < first + cnt)).all()
+                assert (got[r] == 0).all()
+                got[r] = c
+                if not more:
+                    break
+                assert k == cap
+                assert calls < 20
+        assert np.array_equal(got, want)
+        assert not to_np(counts, np.uint32)[:num_rows].any()
+        assert int(to_np(n_entries, np.uint32)[0]) == 0
+    finally:
+        out.free()
+
+
+def test_record_rejects_keys_without_a_row():
+    counts = dev_zeros_u32(10)
+    st = dev_zeros_u32(1)
+    d_keys = to_dev(np.array([3, 10, -1, 3], np.int64))
+    hip.call("ugk_record_i64", ptr(d_keys), 4, 0, 0, ptr(counts), 10, ptr(st), None, None)
+    sync()
+    assert status_value(st) & hip.ST_KEY_OUT_OF_RANGE
+    assert to_np(counts, np.uint32)[:10].tolist() == [0, 0, 0, 2, 0, 0, 0, 0, 0, 0]

@@ -20,7 +20,7 @@ INCLUDE = os.path.join(ROOT, "include")
 HIP_LIB = os.path.join(PKG, "libugache_hip.so")
 HOST_LIB = os.path.join(PKG, "libcoll_cache.so")
 
-HIP_SOURCES = ["ugk_runtime.hip", "ugk_gather.hip", "ugk_table.hip", "ugk_partition.hip"]
+HIP_SOURCES = ["ugk_runtime.hip", "ugk_gather.hip", "ugk_table.hip", "ugk_partition.hip", "ugk_hotness.hip"]
 
 HIPCC_FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-shared",

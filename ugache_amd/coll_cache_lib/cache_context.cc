@@ -232,9 +232,20 @@ ExtractSession::ExtractSession(std::shared_ptr<CacheContext> cache_ctx) : _cache
   memset(_host_mirror, 0, 256);
   const auto &desc = RunConfig::coll_cache_link_desc;
   if (!desc.cpu_sm.empty()) _cpu_blocks = (unsigned)desc.cpu_sm[0];
+  if (RunConfig::gpu_record) {
+    const size_t rows = _cache_ctx->_num_total_nodes;
+    _hot_counts = EagerGPUAlloc(dev, std::max<size_t>(rows, 1) * sizeof(uint32_t));
+    UGK_CALL(ugk_fill_u32(_hot_counts->ptr<uint32_t>(), 0, rows, nullptr));
+    const size_t cap = std::min<size_t>(std::max<size_t>(rows, 1), kHotDrainRows);
+    _hot_entries = EagerGPUAlloc(dev, cap * sizeof(uint64_t));
+    _hot_entries_host = PinnedHostAlloc(cap * sizeof(uint64_t));
+    UGK_CALL(ugk_stream_create(&_record_stream));
+    UGK_CALL(ugk_stream_sync(nullptr));
+  }
 }
 
 ExtractSession::~ExtractSession() {
+  if (_record_stream) ugk_stream_destroy(_record_stream);
   ugk_stream_destroy(_local_ext_stream);
   ugk_stream_destroy(_cpu_ext_stream);
   ugk_event_destroy(_ev_classified);
@@ -295,6 +306,52 @@ static int Dedup(const IdType *keys, size_t n, void *ws, uint32_t epoch, IdType 
 static int Dedup(const Id64Type *keys, size_t n, void *ws, uint32_t epoch, Id64Type *uniq, uint32_t *inv, uint32_t *rep,
                  uint32_t *nu, uint32_t *nu_host, StreamHandle s) {
   return ugk_dedup_i64(keys, n, ws, epoch, uniq, inv, rep, nu, nu_host, s);
+}
+
+static int Record(const IdType *keys, size_t n, uint64_t mul, uint64_t mask, uint32_t *counts, uint64_t rows,
+                  uint32_t *st, uint32_t *mirror, StreamHandle s) {
+  return ugk_record_u32(keys, n, mul, mask, counts, rows, st, mirror, s);
+}
+static int Record(const Id64Type *keys, size_t n, uint64_t mul, uint64_t mask, uint32_t *counts, uint64_t rows,
+                  uint32_t *st, uint32_t *mirror, StreamHandle s) {
+  return ugk_record_i64(keys, n, mul, mask, counts, rows, st, mirror, s);
+}
+
+// FreqRecorder::Record of this batch on the device (freq_recorder.cc:227-253): enqueued behind the kernels of the
+// lookup that are on the caller's stream, so it overlaps the gathers on the library's streams.
+template <typename KeyT>
+void ExtractSession::RecordKeys(const KeyT *nodes, size_t num_nodes, StreamHandle stream) {
+  if (!_hot_counts || (_num_lookups++ % RunConfig::gpu_record_every) != 0) return;
+  UGK_CALL(Record(nodes, num_nodes, RunConfig::key_map_inv, RunConfig::key_map_mask, _hot_counts->ptr<uint32_t>(),
+                  _cache_ctx->_num_total_nodes, _status, _host_mirror, stream));
+}
+
+size_t ExtractSession::DrainHotness(FreqRecorder *recorder) {
+  CHECK_NOTNULL(recorder);
+  if (!_hot_counts) return 0;
+  UGK_CALL(ugk_set_device(_cache_ctx->_trainer_ctx.device_id));
+  const size_t rows = _cache_ctx->_num_total_nodes;
+  const size_t cap = _hot_entries->nbytes() / sizeof(uint64_t);
+  uint32_t *n_entries = _status + 2;       // device word, kept at zero between drains
+  uint32_t *host_out = _host_mirror + 4;   // [4] entries written, [5] rows left over
+  uint64_t *dev_list = _hot_entries->ptr<uint64_t>();
+  auto *host_list = _hot_entries_host->ptr<FreqEntry>();
+  static_assert(sizeof(FreqEntry) == sizeof(uint64_t), "an entry is one (count << 32 | row) word");
+  size_t moved = 0;
+  for (size_t first = 0; first < rows; first += cap) {
+    const size_t cur = std::min(cap, rows - first);  // as many rows as the list has room for: nothing is left over
+    UGK_CALL(ugk_record_drain(_hot_counts->ptr<uint32_t>(), first, cur, dev_list, (uint32_t)cap, n_entries, host_out,
+                              _record_stream));
+    UGK_CALL(ugk_stream_sync(_record_stream));
+    const size_t got = host_out[0];
+    CHECK_EQ(host_out[1], 0u);
+    if (got == 0) continue;
+    UGK_CALL(ugk_memcpy_async(host_list, dev_list, got * sizeof(uint64_t), _record_stream));
+    UGK_CALL(ugk_stream_sync(_record_stream));
+    recorder->AddEntries(host_list, got);
+    moved += got;
+  }
+  return moved;
 }
 
 // Deduplication in front of the extraction: the distinct keys of the batch, the index of the first occurrence of
@@ -362,6 +419,7 @@ void ExtractSession::ExtractFeatImpl(const KeyT *nodes, size_t num_nodes, void *
   // with deduplication the extraction proper runs over the distinct keys and writes each row where the key first
   // occurs; the duplicates are filled in from there at the end
   const size_t num_input = num_nodes;
+  const KeyT *input_nodes = nodes;
   const uint32_t *dst_map = nullptr, *inverse = nullptr;
   float ms_dedup = 0;
   if (RunConfig::dedup_keys && num_nodes >= RunConfig::dedup_min_keys) {
@@ -390,6 +448,7 @@ void ExtractSession::ExtractFeatImpl(const KeyT *nodes, size_t num_nodes, void *
     }
     UGK_CALL(ugk_event_record(_ev_t[1], stream));
     if (dst_map) UGK_CALL(ugk_replicate_rows(output, rb, inverse, dst_map, num_input, stream));
+    RecordKeys(input_nodes, num_input, stream);
     UGK_CALL(ugk_stream_sync(stream));
     CheckStatusWord(stream);
     float combine_ms = 0;
@@ -424,6 +483,7 @@ void ExtractSession::ExtractFeatImpl(const KeyT *nodes, size_t num_nodes, void *
     UGK_CALL(ExtractMix(table, nodes, num_nodes, cache, cache_rows, host, host_rows, output, rb, _status,
                         _host_mirror, stream));
     UGK_CALL(ugk_event_record(_ev_t[1], stream));
+    RecordKeys(input_nodes, num_input, stream);
     UGK_CALL(ugk_stream_sync(stream));
     CheckStatusWord(stream);
     float mix_ms = 0;
@@ -468,6 +528,7 @@ void ExtractSession::ExtractFeatImpl(const KeyT *nodes, size_t num_nodes, void *
     UGK_CALL(ugk_gather_group(cache, cache_rows, idx, cur, UGK_LOC_LOCAL, num_nodes, output, num_input, rb, 0,
                               _status, _host_mirror, _local_ext_stream));
     UGK_CALL(ugk_event_record(_ev_local_done, _local_ext_stream));
+    RecordKeys(input_nodes, num_input, stream);  // on the caller's stream, beside the gathers of the other streams
     if (!_host_on_main) UGK_CALL(ugk_stream_wait_event(stream, _ev_cpu_done));
     UGK_CALL(ugk_stream_wait_event(stream, _ev_local_done));
   } else {
@@ -478,6 +539,7 @@ void ExtractSession::ExtractFeatImpl(const KeyT *nodes, size_t num_nodes, void *
     UGK_CALL(ugk_gather_group(cache, cache_rows, idx, cur, UGK_LOC_LOCAL, num_nodes, output, num_input, rb, 0,
                               _status, _host_mirror, stream));
     UGK_CALL(ugk_event_record(_ev_local_done, stream));
+    RecordKeys(input_nodes, num_input, stream);
   }
   if (dst_map) UGK_CALL(ugk_replicate_rows(output, rb, inverse, dst_map, num_input, stream));
   // the single blocking wait of the call; the gathers have written their group sizes (and the kernels any error

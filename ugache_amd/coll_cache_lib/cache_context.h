@@ -15,6 +15,7 @@
 
 #include "cache_hashtable.h"
 #include "common.h"
+#include "freq_recorder.h"
 #include "profiler.h"
 #include "run_config.h"
 #include "ugache_hip.h"
@@ -109,6 +110,16 @@ class ExtractSession {
   template <typename KeyT>
   size_t DedupKeys(const KeyT *nodes, size_t num_nodes, StreamHandle stream);
 
+  // hotness counters on the device (RunConfig::gpu_record)
+  MemHandle _hot_counts;         // uint32 per row of the host table
+  MemHandle _hot_entries;        // compact (count << 32 | row) list of one drain step
+  MemHandle _hot_entries_host;   // pinned copy of it
+  StreamHandle _record_stream = nullptr;  // drains run here, beside the lookups
+  size_t _num_lookups = 0;
+  static constexpr size_t kHotDrainRows = 32u << 20;  // rows per drain step = capacity of the entry list
+  template <typename KeyT>
+  void RecordKeys(const KeyT *nodes, size_t num_nodes, StreamHandle stream);
+
   template <typename KeyT>
   void ExtractFeatImpl(const KeyT *nodes, size_t num_nodes, void *output, StreamHandle stream, uint64_t task_key);
   void EnsureIdx(size_t num_nodes);
@@ -125,6 +136,9 @@ class ExtractSession {
                      uint64_t task_key);
   // {0, #local, n} of the last lookup — the reference's group_offset (cache_context.cu:825-847)
   const uint32_t *LastGroupOffset() const { return _group_offset; }
+  // moves what the lookups have counted on the device since the last call into `recorder` (FreqRecorder::Record's
+  // result for the same keys); safe to call from another thread while lookups run.  Returns the rows moved.
+  size_t DrainHotness(FreqRecorder *recorder);
 };
 
 class RefreshSession {

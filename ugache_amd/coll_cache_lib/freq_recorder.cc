@@ -91,6 +91,21 @@ void FreqRecorder::Record(const KeyT *input, size_t num_inputs) {
 template void FreqRecorder::Record<Id64Type>(const Id64Type *input, size_t num_inputs);
 template void FreqRecorder::Record<IdType>(const IdType *input, size_t num_inputs);
 
+void FreqRecorder::AddEntries(const FreqEntry *entries, size_t num_entries) {
+  std::lock_guard<std::mutex> g(_mu);
+  CntT *cnt = _live;
+  const size_t n_nodes = _num_nodes;
+  bool bad = false;
+#pragma omp parallel for num_threads(ScanThreads()) reduction(|| : bad) if (num_entries > 65536)
+  for (size_t i = 0; i < num_entries; i++) {
+    if (entries[i].key >= n_nodes)
+      bad = true;
+    else
+      __atomic_fetch_add(&cnt[entries[i].key], entries[i].cnt, __ATOMIC_RELAXED);
+  }
+  CHECK(!bad) << "FreqRecorder::AddEntries: a row is outside num_total_item=" << n_nodes;
+}
+
 void FreqRecorder::LocalCombineToShared() {
   std::lock_guard<std::mutex> g(_mu);
   CntT *shared = _shared, *live = _live;

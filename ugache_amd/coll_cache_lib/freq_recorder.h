@@ -47,6 +47,8 @@ class FreqRecorder {
   ~FreqRecorder();
   template <typename KeyT>
   void Record(const KeyT *inputs, size_t num_input);
+  // counts gathered elsewhere (the device-side counters): entries with distinct keys, added to the live counts
+  void AddEntries(const FreqEntry *entries, size_t num_entries);
   void LocalCombineToShared();
   void GlobalCombine();
   void Sort();

@@ -95,6 +95,11 @@ void coll_cache_config_from_map(std::unordered_map<std::string, std::string> &co
 ContFreqBuf *CombineAndRank(int replica_id) {
   CHECK_LT((size_t)replica_id, _freq_recorder.size()) << "coll_cache_record_init was not called";
   CHECK_NOTNULL(_freq_recorder[replica_id]);
+  // what the lookups counted on the device joins what coll_cache_record counted on the host
+  if (_coll_cache && _coll_cache->num_replicas_built() > (size_t)replica_id && _coll_cache->session(replica_id)) {
+    const size_t rows = _coll_cache->session(replica_id)->DrainHotness(_freq_recorder[replica_id].get());
+    if (rows) LOG(INFO) << "hotness of " << rows << " rows taken from the device counters";
+  }
   _freq_recorder[replica_id]->LocalCombineToShared();
   AnonymousBarrier::_global_instance->Wait();
   ContFreqBuf *freq_rank = nullptr;

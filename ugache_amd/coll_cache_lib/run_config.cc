@@ -36,6 +36,8 @@ size_t RunConfig::refresh_batch_rows = 4092;
 unsigned RunConfig::refresh_sleep_us = 3000;
 unsigned RunConfig::refresh_limit_block = 20;
 double RunConfig::hash_rebuild_tombstone_frac = 0.15;
+bool RunConfig::gpu_record = false;
+size_t RunConfig::gpu_record_every = 1;
 bool RunConfig::dedup_keys = false;
 size_t RunConfig::dedup_min_keys = 4096;
 uint64_t RunConfig::key_map_mul = 0;
@@ -72,6 +74,8 @@ void RunConfig::LoadConfigFromEnv() {
   hash_rebuild_tombstone_frac = 0.15;
   dedup_keys = false;
   dedup_min_keys = 4096;
+  gpu_record = false;
+  gpu_record_every = 1;
   if (GetEnv("SAMGRAPH_EMPTY_FEAT") != "" && GetEnv("SAMGRAPH_EMPTY_FEAT") != "0") {
     LOG(FATAL) << "SAMGRAPH_EMPTY_FEAT (mock host table) is not supported by this build: every key must have a "
                   "real row in the host table";
@@ -97,6 +101,9 @@ void RunConfig::LoadConfigFromEnv() {
   if (GetEnv("COLL_REFRESH_BATCH_ROWS") != "") refresh_batch_rows = std::stoul(GetEnv("COLL_REFRESH_BATCH_ROWS"));
   if (GetEnv("COLL_REFRESH_SLEEP_US") != "") refresh_sleep_us = std::stoul(GetEnv("COLL_REFRESH_SLEEP_US"));
   if (GetEnv("COLL_REFRESH_LIMIT_BLOCK") != "") refresh_limit_block = std::stoul(GetEnv("COLL_REFRESH_LIMIT_BLOCK"));
+  if (GetEnv("COLL_GPU_RECORD") != "") gpu_record = GetEnv("COLL_GPU_RECORD") != "0";
+  if (GetEnv("COLL_GPU_RECORD_EVERY") != "")
+    gpu_record_every = std::max<size_t>(1, std::stoull(GetEnv("COLL_GPU_RECORD_EVERY")));
   if (GetEnv("COLL_DEDUP_KEYS") != "") dedup_keys = GetEnv("COLL_DEDUP_KEYS") != "0";
   if (GetEnv("COLL_DEDUP_MIN_KEYS") != "") dedup_min_keys = std::stoull(GetEnv("COLL_DEDUP_MIN_KEYS"));
   if (GetEnv("COLL_HASH_REBUILD_FRAC") != "") hash_rebuild_tombstone_frac = std::stod(GetEnv("COLL_HASH_REBUILD_FRAC"));

@@ -63,6 +63,8 @@ struct RunConfig {
   static size_t refresh_batch_rows;    // COLL_REFRESH_BATCH_ROWS, default 4092 (cache_context.cu:4057)
   static unsigned refresh_sleep_us;    // COLL_REFRESH_SLEEP_US, default 3000 (cache_context.cu:4069)
   static unsigned refresh_limit_block; // COLL_REFRESH_LIMIT_BLOCK, default 20 (cache_context.cu:4068)
+  static bool gpu_record;          // COLL_GPU_RECORD=1: every lookup counts its keys in device-side hotness counters
+  static size_t gpu_record_every;  // COLL_GPU_RECORD_EVERY, default 1: ... only every n-th lookup
   static bool dedup_keys;        // COLL_DEDUP_KEYS=1: extract each distinct key of a batch once, then copy the duplicates
   static size_t dedup_min_keys;  // COLL_DEDUP_MIN_KEYS, default 4096: shorter batches skip the deduplication
   static double hash_rebuild_tombstone_frac;  // COLL_HASH_REBUILD_FRAC, default 0.15: rebuild the table after refresh

@@ -1,0 +1,127 @@
+// Hotness counters on the device: one uint32 per row of the host table, bumped by the keys of a batch, and
+// handed to the host as a compact (row, count) list.
+//
+// record : counts[row(key)] += 1, one atomic per key.  HBM-bound by the key read plus one 64-byte line touched
+//          per distinct row; runs beside the gathers on the caller's stream.
+// drain  : scans the counters, turns every non-zero one into a (count << 32 | row) word in a compact list and
+//          resets it to zero.  Reading and resetting is one atomic exchange, so a record kernel that runs at
+//          the same time loses nothing: its increment lands either before the exchange (drained now) or after
+//          it (drained next time).
+#include "ugk_internal.h"
+#include "ugk_table.cuh"
+
+namespace ugk {
+namespace {
+
+constexpr int kWavesPerBlock = kBlock / kWave;
+
+template <typename K>
+__global__ __launch_bounds__(kBlock) void record_kernel(const K *__restrict__ keys, size_t n, ugk_table_t map,
+                                                        uint32_t *counts, uint64_t num_rows, uint32_t *status,
+                                                        uint32_t *host_mirror) {
+  bool bad = false;
+  for (size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x; i < n; i += (size_t)gridDim.x * kBlock) {
+    const uint64_t row = fallback_row(map, key_to_u64<K>(keys[i]));
+    if (row < num_rows)
+      atomicAdd(counts + row, 1u);
+    else
+      bad = true;
+  }
+  if (__ballot(bad) && lane_id() == 0) {
+    atomicOr(status, (uint32_t)UGK_ST_KEY_OUT_OF_RANGE);
+    if (host_mirror) host_mirror[0] = 1;
+  }
+}
+
+__global__ __launch_bounds__(kBlock) void drain_kernel(uint32_t *counts, uint64_t num_rows, uint64_t first_row,
+                                                       unsigned long long *entries, uint32_t capacity,
+                                                       uint32_t *n_entries) {
+  __shared__ uint32_t wave_tot[kWavesPerBlock];
+  __shared__ uint32_t base;
+  const int tid = threadIdx.x;
+  const int lane = tid & (kWave - 1), wave = tid / kWave;
+  const uint64_t n_round = (num_rows + kBlock - 1) / kBlock * kBlock;
+  for (uint64_t i = (uint64_t)blockIdx.x * kBlock + tid; i < n_round; i += (uint64_t)gridDim.x * kBlock) {
+    // a plain read first: most counters are zero and need no atomic
+    const bool hot = i < num_rows && __builtin_nontemporal_load(counts + i) != 0;
+    const uint64_t wb = __ballot(hot);
+    const uint32_t pre = __popcll(wb & ((1ull << lane) - 1ull));
+    if (lane == 0) wave_tot[wave] = __popcll(wb);
+    __syncthreads();
+    uint32_t before = 0, total = 0;
+#pragma unroll
+    for (int w = 0; w < kWavesPerBlock; ++w) {
+      if (w == wave) before = total;
+      total += wave_tot[w];
+    }
+    if (tid == 0) base = total ? atomicAdd(n_entries, total) : 0u;
+    __syncthreads();
+    if (hot) {
+      const uint32_t slot = base + before + pre;
+      if (slot < capacity) {  // a full list leaves the counter alone: the next call picks it up
+        const uint32_t c = atomicExch(counts + i, 0u);
+        entries[slot] = ((unsigned long long)c << 32) | (uint32_t)(first_row + i);
+      }
+    }
+    __syncthreads();
+  }
+}
+
+__global__ void drain_finish_kernel(uint32_t *n_entries, uint32_t capacity, uint32_t *host_out) {
+  // entries claimed beyond the capacity were not written; report what the list holds and whether rows are left
+  const uint32_t claimed = *n_entries;
+  host_out[0] = claimed < capacity ? claimed : capacity;
+  host_out[1] = claimed > capacity ? 1u : 0u;
+  *n_entries = 0;
+}
+
+template <typename K>
+int record(const K *keys, size_t n, uint64_t key_inv, uint64_t key_mask, uint32_t *counts, uint64_t num_rows,
+           uint32_t *status, uint32_t *host_mirror, void *stream) {
+  if (n == 0) return 0;
+  UGK_REQUIRE(keys && counts && status, "ugk_record: null pointer");
+  UGK_REQUIRE(key_inv == 0 || (key_inv & 1ull), "ugk_record: the inverse key multiplier must be odd");
+  ugk_table_t map{};
+  map.fb_mul = key_inv;
+  map.fb_mask = key_mask;
+  const unsigned grid = clamp_grid((n + kBlock - 1) / kBlock, 0);
+  hipLaunchKernelGGL(record_kernel<K>, dim3(grid), dim3(kBlock), 0, as_stream(stream), keys, n, map, counts, num_rows,
+                     status, host_mirror);
+  UGK_HIP(hipGetLastError());
+  return 0;
+}
+
+}  // namespace
+}  // namespace ugk
+
+using namespace ugk;
+
+extern "C" {
+
+int ugk_record_u32(const uint32_t *keys_dev, size_t n, uint64_t key_inv, uint64_t key_mask, uint32_t *counts_dev,
+                   uint64_t num_rows, uint32_t *status_dev, uint32_t *host_mirror, void *stream) {
+  return record<uint32_t>(keys_dev, n, key_inv, key_mask, counts_dev, num_rows, status_dev, host_mirror, stream);
+}
+
+int ugk_record_i64(const int64_t *keys_dev, size_t n, uint64_t key_inv, uint64_t key_mask, uint32_t *counts_dev,
+                   uint64_t num_rows, uint32_t *status_dev, uint32_t *host_mirror, void *stream) {
+  return record<int64_t>(keys_dev, n, key_inv, key_mask, counts_dev, num_rows, status_dev, host_mirror, stream);
+}
+
+int ugk_record_drain(uint32_t *counts_dev, uint64_t first_row, uint64_t num_rows, uint64_t *entries_dev,
+                     uint32_t capacity, uint32_t *n_entries_dev, uint32_t *host_out, void *stream) {
+  UGK_REQUIRE(counts_dev && entries_dev && n_entries_dev && host_out, "ugk_record_drain: null pointer");
+  UGK_REQUIRE(capacity > 0, "ugk_record_drain: empty entry list");
+  UGK_REQUIRE(first_row + num_rows <= 0xffffffffull, "ugk_record_drain: rows must fit 32 bits");
+  if (num_rows) {
+    const unsigned grid = clamp_grid((num_rows + kBlock - 1) / kBlock, 0);
+    hipLaunchKernelGGL(drain_kernel, dim3(grid), dim3(kBlock), 0, as_stream(stream), counts_dev + first_row, num_rows,
+                       first_row, reinterpret_cast<unsigned long long *>(entries_dev), capacity, n_entries_dev);
+    UGK_HIP(hipGetLastError());
+  }
+  hipLaunchKernelGGL(drain_finish_kernel, dim3(1), dim3(1), 0, as_stream(stream), n_entries_dev, capacity, host_out);
+  UGK_HIP(hipGetLastError());
+  return 0;
+}
+
+}  // extern "C"

@@ -91,6 +91,9 @@ SIGNATURES = {
     "ugk_dedup_workspace_bytes": [_sz],
     "ugk_dedup_u32": [_vp, _sz, _vp, _u32, _vp, _vp, _vp, _vp, _vp, _vp],
     "ugk_dedup_i64": [_vp, _sz, _vp, _u32, _vp, _vp, _vp, _vp, _vp, _vp],
+    "ugk_record_u32": [_vp, _sz, _u64, _u64, _vp, _u64, _vp, _vp, _vp],
+    "ugk_record_i64": [_vp, _sz, _u64, _u64, _vp, _u64, _vp, _vp, _vp],
+    "ugk_record_drain": [_vp, _u64, _u64, _vp, _u32, _vp, _vp, _vp],
     "ugk_last_error": [],
 }
 _RESTYPES = {"ugk_hash_buckets_for": _sz, "ugk_dedup_workspace_bytes": _sz, "ugk_last_error": C.c_char_p}
