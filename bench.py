@@ -77,6 +77,9 @@ def parse_args():
     ap.add_argument("--pool", type=int, default=None, help="distinct key batches cycled through the steps")
     ap.add_argument("--dedup", action="store_true",
                     help="mixed workloads: COLL_DEDUP_KEYS=1, every distinct key of a batch is extracted once")
+    ap.add_argument("--gpu-record", action="store_true",
+                    help="mixed workloads: COLL_GPU_RECORD=1, every lookup counts its keys in device-side hotness "
+                         "counters (drained by the refresh)")
     ap.add_argument("--calibrate", action="store_true",
                     help="also run 5 plain device copies of 1 GiB (ugk_copy_rows) so a counter run has a kernel of "
                          "known traffic next to the gather")
@@ -249,6 +252,8 @@ def run_mixed(args):
 
     if args.dedup:
         os.environ["COLL_DEDUP_KEYS"] = "1"
+    if args.gpu_record:
+        os.environ["COLL_GPU_RECORD"] = "1"
     co.config({"cache_percentage": pct, "_cache_policy": co.kCollCacheAsymmLink, "num_device": 1,
                "num_global_step_per_epoch": K + W, "num_epoch": 1, "num_total_item": rows, "omp_thread_num": 16})
     sparse = bool(spec.get("sparse"))
@@ -386,7 +391,7 @@ def run_mixed(args):
                    "key_dtype": "int64", "sparse_ids": sparse, "cache_percentage": pct, "cached_rows": info_cache["cached_rows"],
                    "cache_capacity_rows": info_cache["capacity_rows"], "table_kind": info_cache["table_kind"],
                    "zipf_s": spec["zipf"], "fields": fields, "presample_batches": spec["presample"],
-                   "entry_point": "coll_cache_lookup_i64", "distinct_key_batches": pool, "dedup": bool(args.dedup),
+                   "entry_point": "coll_cache_lookup_i64", "distinct_key_batches": pool, "dedup": bool(args.dedup), "gpu_record": bool(args.gpu_record),
                    "unique_keys_per_batch": uniq, "seeds": {"table": 1, "perm": 2, "keys": 3}},
         "effective_extraction_GBps": n_keys * row_bytes / (elapsed / K) / 1e9,
         "parity": "bit-exact vs CPU oracle (last timed batch)",

@@ -240,12 +240,16 @@ ExtractSession::ExtractSession(std::shared_ptr<CacheContext> cache_ctx) : _cache
     _hot_entries = EagerGPUAlloc(dev, cap * sizeof(uint64_t));
     _hot_entries_host = PinnedHostAlloc(cap * sizeof(uint64_t));
     UGK_CALL(ugk_stream_create(&_record_stream));
+    UGK_CALL(ugk_event_create(&_ev_rec_begin));
+    UGK_CALL(ugk_event_create(&_ev_rec_done));
     UGK_CALL(ugk_stream_sync(nullptr));
   }
 }
 
 ExtractSession::~ExtractSession() {
   if (_record_stream) ugk_stream_destroy(_record_stream);
+  if (_ev_rec_begin) ugk_event_destroy(_ev_rec_begin);
+  if (_ev_rec_done) ugk_event_destroy(_ev_rec_done);
   ugk_stream_destroy(_local_ext_stream);
   ugk_stream_destroy(_cpu_ext_stream);
   ugk_event_destroy(_ev_classified);
@@ -317,13 +321,29 @@ static int Record(const Id64Type *keys, size_t n, uint64_t mul, uint64_t mask, u
   return ugk_record_i64(keys, n, mul, mask, counts, rows, st, mirror, s);
 }
 
-// FreqRecorder::Record of this batch on the device (freq_recorder.cc:227-253): enqueued behind the kernels of the
-// lookup that are on the caller's stream, so it overlaps the gathers on the library's streams.
+// FreqRecorder::Record of this batch on the device (freq_recorder.cc:227-253).  It runs on a stream of its own behind
+// `after` (an event already recorded on the caller's stream; none: the point the caller's stream has reached now), so
+// it overlaps the gathers; JoinRecord makes the caller's stream wait for it before the lookup returns (the keys
+// belong to the caller again after that).
 template <typename KeyT>
-void ExtractSession::RecordKeys(const KeyT *nodes, size_t num_nodes, StreamHandle stream) {
+void ExtractSession::RecordKeys(const KeyT *nodes, size_t num_nodes, StreamHandle stream, void *after) {
+  _record_pending = false;
   if (!_hot_counts || (_num_lookups++ % RunConfig::gpu_record_every) != 0) return;
+  if (after == nullptr) {
+    UGK_CALL(ugk_event_record(_ev_rec_begin, stream));
+    after = _ev_rec_begin;
+  }
+  UGK_CALL(ugk_stream_wait_event(_record_stream, after));
   UGK_CALL(Record(nodes, num_nodes, RunConfig::key_map_inv, RunConfig::key_map_mask, _hot_counts->ptr<uint32_t>(),
-                  _cache_ctx->_num_total_nodes, _status, _host_mirror, stream));
+                  _cache_ctx->_num_total_nodes, _status, _host_mirror, _record_stream));
+  UGK_CALL(ugk_event_record(_ev_rec_done, _record_stream));
+  _record_pending = true;
+}
+
+void ExtractSession::JoinRecord(StreamHandle stream) {
+  if (!_record_pending) return;
+  UGK_CALL(ugk_stream_wait_event(stream, _ev_rec_done));
+  _record_pending = false;
 }
 
 size_t ExtractSession::DrainHotness(FreqRecorder *recorder) {
@@ -438,6 +458,7 @@ void ExtractSession::ExtractFeatImpl(const KeyT *nodes, size_t num_nodes, void *
     CHECK_EQ(ctx->_num_location, 1);
     const bool from_host = ctx->_cpu_location_id != -1;
     // the gather is bracketed by events on its own stream: the logged combine time is the kernel's duration
+    RecordKeys(input_nodes, num_input, stream, nullptr);
     UGK_CALL(ugk_event_record(_ev_t[0], stream));
     if (dst_map == nullptr) {
       UGK_CALL(GatherDirect(ctx->_device_cache_data[0], ctx->_num_total_nodes, nodes, num_nodes, output, rb,
@@ -448,7 +469,7 @@ void ExtractSession::ExtractFeatImpl(const KeyT *nodes, size_t num_nodes, void *
     }
     UGK_CALL(ugk_event_record(_ev_t[1], stream));
     if (dst_map) UGK_CALL(ugk_replicate_rows(output, rb, inverse, dst_map, num_input, stream));
-    RecordKeys(input_nodes, num_input, stream);
+    JoinRecord(stream);
     UGK_CALL(ugk_stream_sync(stream));
     CheckStatusWord(stream);
     float combine_ms = 0;
@@ -479,11 +500,12 @@ void ExtractSession::ExtractFeatImpl(const KeyT *nodes, size_t num_nodes, void *
 
   if (RunConfig::concurrent_link_impl == kDirectNoGroup && dst_map == nullptr) {
     // one fused lookup + gather kernel, source chosen per row (cache_context.cu:1295-1329)
+    RecordKeys(input_nodes, num_input, stream, nullptr);
     UGK_CALL(ugk_event_record(_ev_t[0], stream));
     UGK_CALL(ExtractMix(table, nodes, num_nodes, cache, cache_rows, host, host_rows, output, rb, _status,
                         _host_mirror, stream));
     UGK_CALL(ugk_event_record(_ev_t[1], stream));
-    RecordKeys(input_nodes, num_input, stream);
+    JoinRecord(stream);
     UGK_CALL(ugk_stream_sync(stream));
     CheckStatusWord(stream);
     float mix_ms = 0;
@@ -505,6 +527,8 @@ void ExtractSession::ExtractFeatImpl(const KeyT *nodes, size_t num_nodes, void *
   UGK_CALL(ugk_event_record(_ev_t[0], stream));
   UGK_CALL(Classify(table, nodes, num_nodes, host_rows, dst_map, idx, cur, next, _status, _host_mirror, stream));
   UGK_CALL(ugk_event_record(_ev_classified, stream));
+  // the classify kernel is short and latency-bound: the counting starts behind it, beside the gathers
+  RecordKeys(input_nodes, num_input, stream, _ev_classified);
   if (RunConfig::concurrent_link_impl == kSMMaskPhase) {
     // factored extraction: two concurrent kernels that read their group bounds from the device-side counters.
     // A long host-link gather runs on the stream confined to a few CUs, so its slow loads do not clog the memory
@@ -528,7 +552,6 @@ void ExtractSession::ExtractFeatImpl(const KeyT *nodes, size_t num_nodes, void *
     UGK_CALL(ugk_gather_group(cache, cache_rows, idx, cur, UGK_LOC_LOCAL, num_nodes, output, num_input, rb, 0,
                               _status, _host_mirror, _local_ext_stream));
     UGK_CALL(ugk_event_record(_ev_local_done, _local_ext_stream));
-    RecordKeys(input_nodes, num_input, stream);  // on the caller's stream, beside the gathers of the other streams
     if (!_host_on_main) UGK_CALL(ugk_stream_wait_event(stream, _ev_cpu_done));
     UGK_CALL(ugk_stream_wait_event(stream, _ev_local_done));
   } else {
@@ -539,9 +562,9 @@ void ExtractSession::ExtractFeatImpl(const KeyT *nodes, size_t num_nodes, void *
     UGK_CALL(ugk_gather_group(cache, cache_rows, idx, cur, UGK_LOC_LOCAL, num_nodes, output, num_input, rb, 0,
                               _status, _host_mirror, stream));
     UGK_CALL(ugk_event_record(_ev_local_done, stream));
-    RecordKeys(input_nodes, num_input, stream);
   }
   if (dst_map) UGK_CALL(ugk_replicate_rows(output, rb, inverse, dst_map, num_input, stream));
+  JoinRecord(stream);
   // the single blocking wait of the call; the gathers have written their group sizes (and the kernels any error
   // flag) into the pinned mirror, so no device-to-host copy is needed
   UGK_CALL(ugk_stream_sync(stream));

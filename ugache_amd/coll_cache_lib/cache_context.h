@@ -114,11 +114,14 @@ class ExtractSession {
   MemHandle _hot_counts;         // uint32 per row of the host table
   MemHandle _hot_entries;        // compact (count << 32 | row) list of one drain step
   MemHandle _hot_entries_host;   // pinned copy of it
-  StreamHandle _record_stream = nullptr;  // drains run here, beside the lookups
+  StreamHandle _record_stream = nullptr;  // record kernels and drains run here, beside the extraction
+  void *_ev_rec_begin = nullptr, *_ev_rec_done = nullptr;
+  bool _record_pending = false;
+  void JoinRecord(StreamHandle stream);
   size_t _num_lookups = 0;
   static constexpr size_t kHotDrainRows = 32u << 20;  // rows per drain step = capacity of the entry list
   template <typename KeyT>
-  void RecordKeys(const KeyT *nodes, size_t num_nodes, StreamHandle stream);
+  void RecordKeys(const KeyT *nodes, size_t num_nodes, StreamHandle stream, void *after);
 
   template <typename KeyT>
   void ExtractFeatImpl(const KeyT *nodes, size_t num_nodes, void *output, StreamHandle stream, uint64_t task_key);

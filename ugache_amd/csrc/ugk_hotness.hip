@@ -1,8 +1,8 @@
 // Hotness counters on the device: one uint32 per row of the host table, bumped by the keys of a batch, and
 // handed to the host as a compact (row, count) list.
 //
-// record : counts[row(key)] += 1, one atomic per key.  HBM-bound by the key read plus one 64-byte line touched
-//          per distinct row; runs beside the gathers on the caller's stream.
+// record : counts[row(key)] += 1.  HBM-bound by the key read plus one 64-byte line touched per distinct row; runs
+//          beside the gathers on the caller's stream.
 // drain  : scans the counters, turns every non-zero one into a (count << 32 | row) word in a compact list and
 //          resets it to zero.  Reading and resetting is one atomic exchange, so a record kernel that runs at
 //          the same time loses nothing: its increment lands either before the exchange (drained now) or after
@@ -15,17 +15,61 @@ namespace {
 
 constexpr int kWavesPerBlock = kBlock / kWave;
 
+// Hot rows are hot: with a skewed key distribution a few counters would take most of the atomics of a batch and
+// serialise them in the memory-side atomic units.  Each workgroup therefore first counts its tile of keys in a small
+// LDS table (row -> count, open addressing, at most half full) and then adds every distinct row of the tile to the
+// global counters once.
+constexpr int kRecKeysPerThread = 8;
+constexpr int kRecTile = kBlock * kRecKeysPerThread;  // 2048 keys per tile
+constexpr int kRecSlots = 2 * kRecTile;               // 4096 slots, 32 KB of LDS
+constexpr uint32_t kRecEmpty = 0xffffffffu;           // rows are below 2^32 - 1
+
 template <typename K>
 __global__ __launch_bounds__(kBlock) void record_kernel(const K *__restrict__ keys, size_t n, ugk_table_t map,
                                                         uint32_t *counts, uint64_t num_rows, uint32_t *status,
                                                         uint32_t *host_mirror) {
+  __shared__ uint32_t slot_row[kRecSlots];
+  __shared__ uint32_t slot_cnt[kRecSlots];
+  const int tid = threadIdx.x;
+  for (int s = tid; s < kRecSlots; s += kBlock) {
+    slot_row[s] = kRecEmpty;
+    slot_cnt[s] = 0;
+  }
+  __syncthreads();
   bool bad = false;
-  for (size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x; i < n; i += (size_t)gridDim.x * kBlock) {
-    const uint64_t row = fallback_row(map, key_to_u64<K>(keys[i]));
-    if (row < num_rows)
-      atomicAdd(counts + row, 1u);
-    else
-      bad = true;
+  const size_t n_tiles = (n + kRecTile - 1) / kRecTile;
+  for (size_t tile = blockIdx.x; tile < n_tiles; tile += gridDim.x) {
+    const size_t base = tile * kRecTile;
+#pragma unroll
+    for (int j = 0; j < kRecKeysPerThread; ++j) {
+      const size_t i = base + (size_t)j * kBlock + tid;
+      if (i >= n) continue;
+      const uint64_t row64 = fallback_row(map, key_to_u64<K>(keys[i]));
+      if (row64 >= num_rows) {
+        bad = true;
+        continue;
+      }
+      const uint32_t row = (uint32_t)row64;
+      uint32_t h = (uint32_t)(fmix64(row) >> 40) & (kRecSlots - 1);
+      for (;;) {
+        const uint32_t seen = atomicCAS(&slot_row[h], kRecEmpty, row);
+        if (seen == kRecEmpty || seen == row) {
+          atomicAdd(&slot_cnt[h], 1u);
+          break;
+        }
+        h = (h + 1) & (kRecSlots - 1);
+      }
+    }
+    __syncthreads();
+    for (int s = tid; s < kRecSlots; s += kBlock) {
+      const uint32_t c = slot_cnt[s];
+      if (c) {
+        atomicAdd(counts + slot_row[s], c);
+        slot_row[s] = kRecEmpty;
+        slot_cnt[s] = 0;
+      }
+    }
+    __syncthreads();
   }
   if (__ballot(bad) && lane_id() == 0) {
     atomicOr(status, (uint32_t)UGK_ST_KEY_OUT_OF_RANGE);
@@ -81,10 +125,11 @@ int record(const K *keys, size_t n, uint64_t key_inv, uint64_t key_mask, uint32_
   if (n == 0) return 0;
   UGK_REQUIRE(keys && counts && status, "ugk_record: null pointer");
   UGK_REQUIRE(key_inv == 0 || (key_inv & 1ull), "ugk_record: the inverse key multiplier must be odd");
+  UGK_REQUIRE(num_rows < 0xffffffffull, "ugk_record: rows must fit 32 bits");
   ugk_table_t map{};
   map.fb_mul = key_inv;
   map.fb_mask = key_mask;
-  const unsigned grid = clamp_grid((n + kBlock - 1) / kBlock, 0);
+  const unsigned grid = clamp_grid((n + kRecTile - 1) / kRecTile, 0);
   hipLaunchKernelGGL(record_kernel<K>, dim3(grid), dim3(kBlock), 0, as_stream(stream), keys, n, map, counts, num_rows,
                      status, host_mirror);
   UGK_HIP(hipGetLastError());
