@@ -37,11 +37,17 @@ __global__ __launch_bounds__(kBlock) void classify_kernel(ugk_table_t t, const K
 
   for (size_t tile0 = (size_t)blockIdx.x * kTile; tile0 < n; tile0 += (size_t)gridDim.x * kTile) {
     uint32_t cls[kItems], off[kItems], pre[kItems];
+    uint64_t key_of[kItems];
+#pragma unroll
+    for (int j = 0; j < kItems; ++j) {
+      const size_t i = tile0 + (size_t)j * kBlock + tid;
+      key_of[j] = i < n ? key_to_u64<K>(keys[i]) : 0;
+    }
 #pragma unroll
     for (int j = 0; j < kItems; ++j) {
       const size_t i = tile0 + (size_t)j * kBlock + tid;
       const bool active = i < n;
-      const uint64_t key = active ? key_to_u64<K>(keys[i]) : 0;
+      const uint64_t key = key_of[j];
       const Found f = table_lookup<KIND>(t, key, active);
       uint32_t c = 0, o = 0;
       if (active) {

@@ -2,17 +2,19 @@
 //
 // flat table  : one uint32 per key of the key space, (loc << 28) + off, 0xffffffff = absent.
 // hash table  : ugk_bucket_t[nbuckets] (16 bytes each, nbuckets a multiple of 8, base 128-byte aligned),
-//               linear probing from home(key) = mulhi64(fmix64(key), nbuckets).
+//               linear probing from home(key) = 8 * mulhi64(fmix64(key), nbuckets / 8): a probe sequence
+//               starts at the first bucket of a 128-byte line, so at load 0.7 nine keys in ten are found
+//               (or ruled out) inside the one line their lookup reads first.
 //               A search stops at a never-used bucket, walks over tombstones and other keys.
 //               A matching key only counts when its VALID bit is set; a key that is half-way through an
 //               insert or an evict therefore reads as a miss, which is always correct because the host
 //               table holds every row.
 //
-// Lookup is wavefront-cooperative.  Phase 1: every lane probes the home bucket of its own key with one
-// 16-byte load.  Phase 2: lanes that hit a foreign key are served eight at a time: eight 8-lane groups
-// each take one pending key and read one 128-byte line (eight adjacent buckets) per step, a wavefront
-// ballot decides match / never-used / continue.  A collision therefore costs one line per step, not
-// one dependent 16-byte load per bucket.
+// Lookup is wavefront-cooperative: an 8-lane group reads one 128-byte line (eight adjacent buckets) of one key's
+// probe sequence per step and a wavefront ballot decides match / never-used / continue.  Step 1 reads the
+// home line of all 64 keys of the wavefront in eight rounds whose loads are independent of each other (all in
+// flight together); step 2 follows the few keys whose home line was full without a match, eight at a time.
+// A lookup therefore costs one line in the common case and never a chain of dependent 16-byte loads.
 #pragma once
 
 #include "ugk_internal.h"
@@ -29,7 +31,7 @@ __device__ __forceinline__ uint64_t fmix64(uint64_t x) {
 }
 
 __device__ __forceinline__ uint64_t hash_home(uint64_t key, uint64_t nbuckets) {
-  return __umul64hi(fmix64(key), nbuckets);
+  return __umul64hi(fmix64(key), nbuckets >> 3) << 3;
 }
 
 struct Found {
@@ -67,32 +69,79 @@ __device__ __forceinline__ Found flat_lookup(const uint32_t *table, uint64_t nke
   return f;
 }
 
-// Wavefront-cooperative hash lookup.  Must be called by all 64 lanes of the wavefront (inactive lanes pass
+// Wavefront-cooperative hash lookup in two steps.  All 64 lanes of the wavefront must call both (inactive lanes pass
 // active = false).
-__device__ __forceinline__ Found hash_lookup_wave(const ugk_bucket_t *table, uint64_t nb, uint64_t key, bool active) {
-  Found f{false, 0, 0};
-  uint64_t home = 0;
-  bool pending = false;
-  if (active) {
-    home = hash_home(key, nb);
-    const ugk_bucket_t b = load_bucket(table + home);
-    if (b.key == key) {
-      if (b.meta & UGK_META_VALID) {
-        f.hit = true;
-        f.loc = b.meta & 0xfu;
-        f.off = b.off;
+struct HashProbe {
+  Found f;
+  uint64_t next_win;  // first bucket of the line step 2 has to read next
+  bool pending;       // the home line was full and did not hold the key
+};
+
+// step 1: the home line of every lane's key.  In round r the eight 8-lane groups serve lanes 8r .. 8r+7.
+__device__ __forceinline__ HashProbe hash_probe_home(const ugk_bucket_t *table, uint64_t nb, uint64_t key,
+                                                     bool active) {
+  HashProbe p{Found{false, 0, 0}, 0, false};
+  const int lane = (int)lane_id();
+  const int grp = lane >> 3, sub = lane & 7;
+  const uint64_t home = active ? hash_home(key, nb) : 0;
+  u32x4 raw[8];
+  uint64_t kk[8];
+  bool act[8];
+#pragma unroll
+  for (int r = 0; r < 8; ++r) {
+    const int owner = r * 8 + grp;
+    kk[r] = shfl64(key, owner);
+    const uint64_t hb = shfl64(home, owner);
+    act[r] = __shfl((int)active, owner) != 0;
+    raw[r] = u32x4{0xffffffffu, 0xffffffffu, 0u, 0u};  // reads as a never-used bucket
+    if (act[r]) raw[r] = *reinterpret_cast<const u32x4 *>(table + hb + sub);
+  }
+#pragma unroll
+  for (int r = 0; r < 8; ++r) {
+    const uint64_t bkey = ((uint64_t)raw[r].y << 32) | raw[r].x;
+    const bool is_match = act[r] && bkey == kk[r];
+    const bool is_empty = act[r] && bkey == UGK_HASH_EMPTY;
+    const uint32_t mb = (uint32_t)((__ballot(is_match) >> (grp * 8)) & 0xffull);
+    const uint32_t eb = (uint32_t)((__ballot(is_empty) >> (grp * 8)) & 0xffull);
+    const int fm = mb ? (__ffs(mb) - 1) : 8;
+    const int fe = eb ? (__ffs(eb) - 1) : 8;
+    const bool g_found = fm < fe;  // a key sits in front of the first never-used bucket of its probe sequence
+    const bool g_done = g_found || fe < 8;
+    const int hit_lane = grp * 8 + (g_found ? fm : 0);
+    const uint32_t h_off = __shfl(raw[r].z, hit_lane);
+    const uint32_t h_meta = __shfl(raw[r].w, hit_lane);
+    const uint32_t g_flags = (g_done ? 1u : 0u) | (g_found ? 2u : 0u);
+    // the owner of this round's key served by group g is lane 8r + g: it reads its group's result
+    const int from = (lane & 7) * 8;
+    const uint32_t r_flags = __shfl(g_flags, from);
+    const uint32_t r_off = __shfl(h_off, from);
+    const uint32_t r_meta = __shfl(h_meta, from);
+    if ((lane >> 3) == r && active) {
+      if (r_flags & 1u) {
+        if ((r_flags & 2u) && (r_meta & UGK_META_VALID)) {
+          p.f.hit = true;
+          p.f.loc = r_meta & 0xfu;
+          p.f.off = r_off;
+        }
+      } else {
+        p.pending = true;
       }
-    } else if (b.key != UGK_HASH_EMPTY) {
-      pending = true;
     }
   }
+  p.next_win = home + 8 >= nb ? 0 : home + 8;
+  return p;
+}
+
+// step 2: the pending lanes are served eight at a time, one 128-byte line per 8-lane group and step
+__device__ __forceinline__ Found hash_probe_rest(const ugk_bucket_t *table, uint64_t nb, uint64_t key, HashProbe p) {
+  Found f = p.f;
+  bool pending = p.pending;
   uint64_t pend = __ballot(pending);
   if (pend == 0) return f;
 
   const int lane = (int)lane_id();
   const int grp = lane >> 3, sub = lane & 7;
-  uint64_t win = home & ~7ull;              // next 8-bucket window this lane's key has to examine
-  int min_sub = (int)(home & 7);            // in the home window only buckets after the home bucket count
+  uint64_t win = p.next_win;  // next 8-bucket window this lane's key has to examine
   uint64_t steps = 0;
   const uint64_t max_steps = nb / 8 + 1;    // a full lap: give up (table without a never-used bucket)
 
@@ -106,11 +155,10 @@ __device__ __forceinline__ Found hash_lookup_wave(const ugk_bucket_t *table, uin
     const int from = gactive ? src : lane;
     const uint64_t k = shfl64(key, from);
     const uint64_t w = shfl64(win, from);
-    const int ms = __shfl(min_sub, from);
 
     bool is_match = false, is_empty = false;
     ugk_bucket_t bb{0, 0, 0};
-    if (gactive && sub > ms) {
+    if (gactive) {
       bb = load_bucket(table + w + sub);
       is_match = bb.key == k;
       is_empty = bb.key == UGK_HASH_EMPTY;
@@ -145,13 +193,16 @@ __device__ __forceinline__ Found hash_lookup_wave(const ugk_bucket_t *table, uin
       } else {
         win += 8;
         if (win >= nb) win = 0;
-        min_sub = -1;
         if (++steps > max_steps) pending = false;
       }
     }
     pend = __ballot(pending);
   }
   return f;
+}
+
+__device__ __forceinline__ Found hash_lookup_wave(const ugk_bucket_t *table, uint64_t nb, uint64_t key, bool active) {
+  return hash_probe_rest(table, nb, key, hash_probe_home(table, nb, key, active));
 }
 
 // Table lookup dispatch.  KIND is ugk_table_t::kind.  All lanes of the wavefront must call it.
