@@ -115,6 +115,22 @@ uint32_t coll_cache_place_ranked(const uint32_t *rank_keys, const uint32_t *rank
  * recorded rank behind all recorded ones in ascending order.  num_node must equal num_total_item. */
 uint32_t coll_cache_place_recorded(int replica_id, uint32_t num_node, double cache_percentage,
                                    uint32_t *nid_to_block_out);
+/* ---- serving loop: LookupManager::forward (python_tf2/collcache_tf2/collcache_tf2_cc/collcache_tf2_cc_infra/src/
+ *      lookup_manager.cc:158-213, record thread :291-312, refresh :317-333) without TensorFlow -------------------
+ * coll_cache_forward_config: enable_refresh and refresh_iter are ps_config's coll_cache_enable_refresh and
+ * coll_cache_refresh_iter (inference_utils.cpp:62-140); record_fraction is the share of each batch whose hotness is
+ * recorded, a prefix of the batch (the reference records the first 5 %: 0.05); periodic != 0 starts a refresh every
+ * refresh_iter steps instead of once at step refresh_iter.
+ * coll_cache_forward_*: one step = record the prefix (on the device when COLL_GPU_RECORD=1, else a copy of the prefix
+ * to the host and coll_cache_record), blocking lookup, and at the configured step a refresh started on a background
+ * thread (skipped with a log line while the previous one still runs).  output as in coll_cache_lookup. */
+void coll_cache_forward_config(int enable_refresh, uint64_t refresh_iter, double record_fraction, int periodic);
+void coll_cache_forward(int replica_id, uint32_t *key, size_t num_keys, void *output, StreamHandle stream);
+void coll_cache_forward_i64(int replica_id, const int64_t *key, size_t num_keys, void *output, StreamHandle stream);
+/* 1 while a background refresh started by coll_cache_forward runs */
+int coll_cache_forward_refresh_ongoing(void);
+/* waits for it; returns the number of refreshes coll_cache_forward has completed so far */
+uint64_t coll_cache_forward_join(void);
 /* drop every global object so that coll_cache_config may be called again (the reference has no teardown) */
 void coll_cache_shutdown(void);
 

@@ -4,6 +4,7 @@ example/gnn/dgl_sample.py:238-259 of the reference) and checked bit-for-bit agai
 import os
 import sys
 import threading
+import time
 
 import numpy as np
 import pytest
@@ -212,6 +213,29 @@ def test_create_emb_from_file(tmp_path):
     assert co.coll_torch_lookup_key_t_val_ret(0, q, False).cpu().numpy().tobytes() == arr[::-1].tobytes()
 
 
+def test_raw_model_directory_and_mock_table(tmp_path):
+    """the serving stack's table formats (modelloader.cpp:52-107): a directory with `key` + `emb_vector`, or
+    mock_<rows>_<dim>"""
+    rng = np.random.default_rng(2)
+    n_item, dim = 5_000, 24
+    rows = rng.standard_normal((n_item, dim)).astype(np.float32)
+    d = tmp_path / "model" / "sparse_embedding0"
+    d.mkdir(parents=True)
+    np.arange(n_item, dtype=np.int64).tofile(d / "key")
+    rows.tofile(d / "emb_vector")
+    co.config(make_config(n_item, 0.0))
+    co.coll_cache_record_init(0)
+    emb = co.coll_torch_load_raw_model(0, str(d))
+    assert tuple(emb.shape) == (n_item, dim) and emb.dtype == torch.float32
+    assert emb.numpy().tobytes() == rows.tobytes()
+    co.coll_torch_init_t(0, 0, emb, 0.0)
+    keys = rng.integers(0, n_item, size=777)
+    out = co.coll_torch_lookup_key_t_val_ret(0, torch.from_numpy(keys).cuda(), False)
+    assert out.cpu().numpy().tobytes() == rows[keys].tobytes()
+    mock = co.coll_torch_load_raw_model(0, "mock_1000_16")
+    assert tuple(mock.shape) == (1000, 16) and not mock.any()
+
+
 @pytest.mark.parametrize("table_kind", ["FLAT", "HASH"])
 @pytest.mark.parametrize("foreground", [True, False])
 def test_refresh_evicts_and_inserts_like_the_oracle(table_kind, foreground, monkeypatch):
@@ -325,6 +349,54 @@ def test_hotness_counted_on_the_device_ranks_like_the_host_recorder(pct, impl, d
     assert m == len(want_k)
     assert np.array_equal(got_k[:m], want_k) and np.array_equal(got_c[:m], want_c)
     assert _basics.C_LIB_CTYPES.coll_cache_rank_hotness(0, None, None, 0) == 0  # drained
+
+
+@pytest.mark.parametrize("gpu_record", [False, True])
+@pytest.mark.parametrize("kdtype", [torch.int32, torch.int64])
+def test_serving_loop_records_a_prefix_and_refreshes_in_the_background(gpu_record, kdtype, monkeypatch):
+    """LookupManager::forward re-expressed (lookup_manager.cc:158-213): every step records the first share of its
+    batch, looks the batch up, and at step refresh_iter starts a background refresh from what was recorded."""
+    if gpu_record:
+        monkeypatch.setenv("COLL_GPU_RECORD", "1")
+    monkeypatch.setenv("COLL_REFRESH_SLEEP_US", "100")
+    rng = np.random.default_rng(44)
+    n_item, dim, pct, frac = 30_000, 32, 0.2, 0.5
+    co.config(make_config(n_item, pct))
+    co.coll_cache_record_init(0)
+    perm1 = rng.permutation(n_item)
+    co.coll_torch_record(0, torch.from_numpy(perm1[zipf_ranks(rng, 100_000, n_item, 1.1)]).to(kdtype))
+    emb = co.coll_torch_create_emb_shm(0, n_item, dim, torch.float32)
+    table = fill_table(emb, rng)
+    co.coll_torch_init_t(0, 0, emb, pct)
+    co.coll_torch_forward_config(True, 3, frac, False)
+
+    perm2 = rng.permutation(n_item)
+    recorded = []
+    for step in range(7):
+        n = 40_000 + 1000 * step
+        keys = perm2[zipf_ranks(rng, n, n_item, 1.1)]
+        out = co.coll_torch_forward(0, torch.from_numpy(keys).to(kdtype).cuda(), False)
+        assert out.cpu().numpy().tobytes() == ORC.gather(table, keys.astype(np.int64)).tobytes()
+        recorded.append(keys[: int(n * frac)])
+        if step < 3:
+            assert co.coll_torch_forward_join() == 0
+        if step == 3:
+            # the refresh started at the end of this step; it waits for one more lookup to pass before it reuses
+            # cache slots (an empty one will do, and records nothing)
+            empty = torch.zeros(0, dtype=kdtype, device="cuda")
+            while _basics.C_LIB_CTYPES.coll_cache_forward_refresh_ongoing():
+                co.coll_torch_lookup_key_t_val_ret(0, empty, False)
+                time.sleep(0.001)
+            assert co.coll_torch_forward_join() == 1
+            new_cached, new_nid = expected_cached_set(np.concatenate(recorded).astype(np.uint32), n_item, pct)
+            got = np.zeros(len(new_cached), np.uint32)
+            assert _basics.C_LIB_CTYPES.coll_cache_get_cached_keys(0, got.ctypes.data, len(got)) == len(new_cached)
+            assert np.array_equal(got, new_cached)
+        if step > 3:
+            assert _basics.last_group_offset(0)[1] == int((new_nid[keys] == 0).sum())
+    assert co.coll_torch_forward_join() == 1  # not periodic: one refresh only
+    # plain lookups count whole batches again
+    co.coll_torch_forward_config(False, 0, frac, False)
 
 
 def test_reference_cpu_runnable_config_full_size():

@@ -329,6 +329,8 @@ template <typename KeyT>
 void ExtractSession::RecordKeys(const KeyT *nodes, size_t num_nodes, StreamHandle stream, void *after) {
   _record_pending = false;
   if (!_hot_counts || (_num_lookups++ % RunConfig::gpu_record_every) != 0) return;
+  num_nodes = std::min(num_nodes, _record_limit);
+  if (num_nodes == 0) return;
   if (after == nullptr) {
     UGK_CALL(ugk_event_record(_ev_rec_begin, stream));
     after = _ev_rec_begin;

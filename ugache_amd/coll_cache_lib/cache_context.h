@@ -9,6 +9,7 @@
 #pragma once
 
 #include <atomic>
+#include <cstdint>
 #include <functional>
 #include <memory>
 #include <vector>
@@ -117,6 +118,7 @@ class ExtractSession {
   StreamHandle _record_stream = nullptr;  // record kernels and drains run here, beside the extraction
   void *_ev_rec_begin = nullptr, *_ev_rec_done = nullptr;
   bool _record_pending = false;
+  size_t _record_limit = SIZE_MAX;
   void JoinRecord(StreamHandle stream);
   size_t _num_lookups = 0;
   static constexpr size_t kHotDrainRows = 32u << 20;  // rows per drain step = capacity of the entry list
@@ -142,6 +144,9 @@ class ExtractSession {
   // moves what the lookups have counted on the device since the last call into `recorder` (FreqRecorder::Record's
   // result for the same keys); safe to call from another thread while lookups run.  Returns the rows moved.
   size_t DrainHotness(FreqRecorder *recorder);
+  // the device-side counting of the following lookups covers only the first `num_keys` keys of a batch
+  // (the recorded prefix of LookupManager's record thread); SIZE_MAX, the default: the whole batch
+  void SetRecordLimit(size_t num_keys) { _record_limit = num_keys; }
 };
 
 class RefreshSession {

@@ -5,7 +5,10 @@
 
 #include <cstring>
 #include <iostream>
+#include <atomic>
 #include <string>
+#include <thread>
+#include <vector>
 #include <unordered_map>
 
 #include "facade.h"
@@ -258,6 +261,96 @@ void coll_cache_refresh(int replica_id, StreamHandle stream, int foreground) {
   _coll_cache->refresh(replica_id, freq_rank, stream, foreground != 0);
 }
 
+}  // extern "C"
+
+// ---- serving loop ------------------------------------------------------------------------------------------
+namespace {
+struct ForwardState {
+  bool enable_refresh = false;
+  bool periodic = false;
+  uint64_t refresh_iter = 0;
+  double record_fraction = 0.05;
+  uint64_t step = 0;
+  std::thread refresh_thread;
+  std::atomic<bool> refresh_ongoing{false};
+  std::atomic<uint64_t> refreshes_done{0};
+  std::vector<char> host_keys;  // staging of the recorded prefix on the host-record path
+};
+ForwardState _forward;
+
+void ForwardJoin() {
+  if (_forward.refresh_thread.joinable()) _forward.refresh_thread.join();
+}
+
+template <typename KeyT>
+void ForwardStep(int replica_id, const KeyT *key, size_t num_keys, void *output, StreamHandle stream) {
+  CHECK_NOTNULL(_coll_cache);
+  CHECK_EQ(replica_id, 0);
+  ForwardState &fw = _forward;
+  auto session = _coll_cache->session(replica_id);
+  const size_t num_record = fw.enable_refresh ? (size_t)(num_keys * fw.record_fraction) : 0;
+  if (RunConfig::gpu_record) {
+    session->SetRecordLimit(num_record);  // counted by the lookup itself
+  } else if (num_record > 0) {
+    // lookup_manager.cc:295-306: copy the prefix to the host and count it there
+    fw.host_keys.resize(num_record * sizeof(KeyT));
+    UGK_CALL(ugk_memcpy_async(fw.host_keys.data(), key, num_record * sizeof(KeyT), stream));
+    UGK_CALL(ugk_stream_sync(stream));
+    _freq_recorder[replica_id]->Record(reinterpret_cast<const KeyT *>(fw.host_keys.data()), num_record);
+  }
+  const uint64_t step_key = steps[replica_id] * RunConfig::num_device + replica_id;
+  steps[replica_id]++;
+  if (sizeof(KeyT) == 8)
+    _coll_cache->lookup64(replica_id, reinterpret_cast<const Id64Type *>(key), num_keys, output, stream, step_key);
+  else
+    _coll_cache->lookup(replica_id, reinterpret_cast<const IdType *>(key), num_keys, output, stream, step_key);
+  if (RunConfig::gpu_record) session->SetRecordLimit(SIZE_MAX);
+  const bool due = fw.enable_refresh && fw.refresh_iter > 0 &&
+                   (fw.periodic ? (fw.step > 0 && fw.step % fw.refresh_iter == 0) : fw.step == fw.refresh_iter);
+  if (due) {
+    if (!fw.refresh_ongoing.load()) {
+      fw.refresh_ongoing.store(true);
+      ForwardJoin();
+      fw.refresh_thread = std::thread([replica_id, stream]() {
+        coll_cache_refresh(replica_id, stream, /*foreground=*/0);
+        _forward.refreshes_done.fetch_add(1);
+        _forward.refresh_ongoing.store(false);
+      });
+    } else {
+      LOG(ERROR) << "skip refresh due to refresh already ongoing";
+    }
+  }
+  fw.step++;
+}
+}  // namespace
+
+extern "C" {
+
+void coll_cache_forward_config(int enable_refresh, uint64_t refresh_iter, double record_fraction, int periodic) {
+  CHECK(record_fraction >= 0 && record_fraction <= 1) << "record_fraction is a share of the batch";
+  ForwardJoin();
+  _forward.enable_refresh = enable_refresh != 0;
+  _forward.refresh_iter = refresh_iter;
+  _forward.record_fraction = record_fraction;
+  _forward.periodic = periodic != 0;
+  _forward.step = 0;
+}
+
+void coll_cache_forward(int replica_id, uint32_t *key, size_t num_keys, void *output, StreamHandle stream) {
+  ForwardStep<IdType>(replica_id, key, num_keys, output, stream);
+}
+
+void coll_cache_forward_i64(int replica_id, const int64_t *key, size_t num_keys, void *output, StreamHandle stream) {
+  ForwardStep<Id64Type>(replica_id, key, num_keys, output, stream);
+}
+
+int coll_cache_forward_refresh_ongoing(void) { return _forward.refresh_ongoing.load() ? 1 : 0; }
+
+uint64_t coll_cache_forward_join(void) {
+  ForwardJoin();
+  return _forward.refreshes_done.load();
+}
+
 void *coll_cache_alloc_host_table(size_t nbytes) {
   void *p = nullptr;
   UGK_CALL(ugk_host_malloc(&p, nbytes));
@@ -353,6 +446,10 @@ uint32_t coll_cache_place_recorded(int replica_id, uint32_t num_node, double cac
 }
 
 void coll_cache_shutdown(void) {
+  ForwardJoin();
+  _forward.enable_refresh = false;
+  _forward.step = 0;
+  _forward.refreshes_done.store(0);
   if (_coll_cache) _coll_cache->release_replicas();
   _coll_cache = nullptr;
   _profiler = nullptr;

@@ -102,9 +102,7 @@ def coll_torch_test(local_id, keys):
     return torch.empty((keys.size(0), _State.external_feat_dim), dtype=torch.float32, device="cuda:%d" % dev)
 
 
-def coll_torch_lookup_key_t_val_ret(local_id, keys, pad_to_8=True):
-    """adapter.cc:204-237: look the keys (GPU int32/uint32 tensor, or int64) up; returns a [ceil8(N), dim] view of one
-    reused output buffer — the next lookup overwrites it."""
+def _lookup_into_reused_buffer(local_id, keys, pad_to_8, fn32, fn64):
     dev = _State.dev_id.get(local_id, 0)
     n = keys.size(0)
     padded_len = (n + 7) // 8 * 8 if pad_to_8 else n
@@ -122,10 +120,35 @@ def coll_torch_lookup_key_t_val_ret(local_id, keys, pad_to_8=True):
     tensor = _State.batch_emb_reuse[: padded_len * _State.external_feat_dim * elem].view(_State.external_dtype).view(
         padded_len, _State.external_feat_dim)
     if keys.dtype == torch.int64:
-        _C.coll_cache_lookup_i64(local_id, keys.data_ptr(), n, tensor.data_ptr(), _stream_handle(dev))
+        fn64(local_id, keys.data_ptr(), n, tensor.data_ptr(), _stream_handle(dev))
     else:
-        _C.coll_cache_lookup(local_id, keys.data_ptr(), n, tensor.data_ptr(), _stream_handle(dev))
+        fn32(local_id, keys.data_ptr(), n, tensor.data_ptr(), _stream_handle(dev))
     return tensor
+
+
+def coll_torch_lookup_key_t_val_ret(local_id, keys, pad_to_8=True):
+    """adapter.cc:204-237: look the keys (GPU int32/uint32 tensor, or int64) up; returns a [ceil8(N), dim] view of one
+    reused output buffer — the next lookup overwrites it."""
+    return _lookup_into_reused_buffer(local_id, keys, pad_to_8, _C.coll_cache_lookup, _C.coll_cache_lookup_i64)
+
+
+def coll_torch_forward_config(enable_refresh, refresh_iter, record_fraction=0.05, periodic=False):
+    """the serving loop's settings (ps_config's coll_cache_enable_refresh / coll_cache_refresh_iter,
+    python_tf2/collcache_tf2/collcache_tf2_cc/collcache_tf2_cc_infra/src/inference_utils.cpp:62-140)"""
+    _C.coll_cache_forward_config(int(bool(enable_refresh)), int(refresh_iter), float(record_fraction),
+                                 int(bool(periodic)))
+
+
+def coll_torch_forward(local_id, keys, pad_to_8=True):
+    """one serving step (LookupManager::forward, lookup_manager.cc:158-213): the hotness of a prefix of the batch is
+    recorded, the keys are looked up, and at the configured step a refresh starts on a background thread.  Returns
+    the same reused buffer view as coll_torch_lookup_key_t_val_ret."""
+    return _lookup_into_reused_buffer(local_id, keys, pad_to_8, _C.coll_cache_forward, _C.coll_cache_forward_i64)
+
+
+def coll_torch_forward_join():
+    """wait for a background refresh started by coll_torch_forward; returns how many have completed"""
+    return int(_C.coll_cache_forward_join())
 
 
 def coll_torch_record(local_id, keys):
@@ -161,6 +184,33 @@ def coll_torch_create_emb_shm(replica_id, n_keys, dim, dtype, fname=""):
         with open(fname, "rb") as f:
             f.readinto(buf)
     return tensor
+
+
+def coll_torch_load_raw_model(replica_id, path, dim=None, dtype=torch.float32):
+    """the host table from the serving stack's model directory (RawModelLoader::master_load,
+    python_tf2/collcache_tf2/collcache_tf2_cc/collcache_tf2_cc_infra/src/modelloader.cpp:52-107):
+      `path`/key         int64 per row — only its length is used, the number of rows; row i belongs to key i
+      `path`/emb_vector  the rows, `dtype` elements, read into the table as they are
+    or `mock_<rows>_<dim>`: a table of that shape whose contents nobody defines (the reference leaves the mapped
+    memory as it is; here it is zero-filled, so every key still has a row).  `dim` is only needed for a directory
+    whose key file is empty.  Returns the pinned CPU tensor [rows, dim] for coll_torch_init_t."""
+    name = os.path.basename(os.path.normpath(path))
+    if name.startswith("mock_"):
+        parts = name.split("_")
+        n_keys, mdim = int(parts[1]), int(parts[-1])
+        t = coll_torch_create_emb_shm(replica_id, n_keys, mdim, dtype)
+        t.zero_()
+        return t
+    n_keys = os.stat(os.path.join(path, "key")).st_size // 8
+    vec = os.path.join(path, "emb_vector")
+    vec_bytes = os.stat(vec).st_size
+    if dim is None:
+        if n_keys == 0 or vec_bytes % (n_keys * _ELEM[dtype]) != 0:
+            sys.stderr.write("emb_vector of %d bytes does not hold %d rows of whole %d-byte elements\n"
+                             % (vec_bytes, n_keys, _ELEM[dtype]))
+            os.abort()
+        dim = vec_bytes // (n_keys * _ELEM[dtype])
+    return coll_torch_create_emb_shm(replica_id, n_keys, dim, dtype, vec)
 
 
 def coll_torch_refresh(replica_id, foreground=False):
