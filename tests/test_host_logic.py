@@ -160,3 +160,53 @@ def test_profiler_hooks_store_and_report(capfd):
     cc._basics.report_step(3)
     out = capfd.readouterr().out
     assert "cache feat copy 0.500000" in out and "feature nbytes" in out
+
+
+def _scrape_profiler_block(text):
+    """what the reference's eval scripts do with a profiler block (eval/gnn/common/common_parser.py:311-336): the
+    first word inside '[' of a header line prefixes the keys, every other line is 'L<n>' + cells split on '|', a cell
+    is 'name value [unit]'"""
+    import re
+    unit = {"Bytes": 1, "KB": 1024, "MB": 1024 ** 2, "GB": 1024 ** 3}
+    vals, prefix = {}, None
+    for line in text.splitlines():
+        if line.startswith("    ["):
+            prefix = re.match(r"    \[([^ ]+) .*", line).group(1)
+            continue
+        if prefix is None or not line.startswith("        L"):
+            continue
+        line = line.strip()
+        level, rest = line[:2], line[2:]
+        for cell in rest.split("|"):
+            item = prefix + " " + level + " " + cell.strip()
+            m = re.match(r"([^\.]*) +([0-9\.]*)( (MB|Bytes|KB|GB))?", item)
+            key, val = m.group(1).strip(), float(m.group(2))
+            if m.group(3):
+                val *= unit[m.group(4)]
+            assert key not in vals, key
+            vals[key] = val
+    return vals
+
+
+def test_step_report_has_the_layout_the_eval_scripts_scrape(capfd):
+    _config(100)
+    logged = {cc.kLogL1FeatureBytes: 3.0 * 1024 ** 2, cc.kLogL1MissBytes: 512.0 * 1024, cc.kLogL1RemoteBytes: 0.0,
+              cc.kLogL2CacheCopyTime: 0.25, cc.kLogL3CacheGetIndexTime: 0.001, cc.kLogL3CacheCombineMissTime: 0.002,
+              cc.kLogL3CacheCombineCacheTime: 0.003, cc.kLogL3CacheCombineRemoteTime: 0.0}
+    for step, scale in ((0, 1.0), (1, 3.0)):
+        for item, v in logged.items():
+            cc._basics.log_step_by_key(step, item, v * scale)
+    cc._basics.report_step_average(1)
+    out = capfd.readouterr().out
+    vals = _scrape_profiler_block(out)
+    want = {"Step(average) L1 feature nbytes": 6.0 * 1024 ** 2, "Step(average) L1 miss nbytes": 1024.0 ** 2,
+            "Step(average) L1 remote nbytes": 0.0, "Step(average) L2 cache feat copy": 0.5,
+            "Step(average) L3 cache get_index": 0.002, "Step(average) L3 cache combine_miss": 0.004,
+            "Step(average) L3 cache combine cache": 0.006, "Step(average) L3 cache combine remote": 0.0,
+            "Step(average) L1 convert time": 0.0, "Step(average) L1 train": 0.0, "Step(average) L1 sample": 0.0}
+    for k, v in want.items():
+        assert k in vals, (k, sorted(vals))
+        assert abs(vals[k] - v) <= 1e-6 * max(1.0, v), (k, vals[k], v)
+    # the three header lines and every level's line count (7 + 3 + 8)
+    assert out.count("Profiler Level") == 3 and out.count("\n        L1  ") == 7
+    assert out.count("\n        L2  ") == 3 and out.count("\n        L3  ") == 8

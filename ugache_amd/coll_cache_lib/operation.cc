@@ -259,6 +259,7 @@ void coll_cache_refresh(int replica_id, StreamHandle stream, int foreground) {
   ContFreqBuf *freq_rank = CombineAndRank(replica_id);
   LOG(INFO) << "refresh: ranking " << t_rank.Passed() << " s";
   _coll_cache->refresh(replica_id, freq_rank, stream, foreground != 0);
+  if (_profiler) _profiler->SetRefreshDuration(t_rank.Passed());
 }
 
 }  // extern "C"

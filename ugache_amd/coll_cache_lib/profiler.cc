@@ -2,6 +2,8 @@
 
 #include <algorithm>
 #include <cstdio>
+#include <cstdlib>
+#include <string>
 #include <iostream>
 
 #include "common.h"
@@ -40,23 +42,103 @@ double Profiler::GetStep(uint64_t key, LogStepItem item) {
   return it == _steps.end() ? 0.0 : it->second.v[item];
 }
 
+namespace {
+
+// One cell of the step report: "<label><pad><value>".  The layout (labels, column padding, value formats, cells
+// per line) is the text the reference prints (profiler.cc:559-760) and its eval scripts split on '|'
+// (eval/gnn/common/common_parser.py:311-336); the table below states it, the loop in Output() prints it.
+enum CellFmt { kSec10, kSec, kSize10, kCount10 };  // %10.6lf, %.6lf, %10s of a readable size, %10.0lf
+struct Cell {
+  const char *label;  // with its trailing padding
+  int item;           // LogStepItem, or one of the two pseudo items below
+  CellFmt fmt;
+};
+constexpr int kItemSeqDuration = -1, kItemRefreshDuration = -2, kEndOfLine = -3;
+#define EOL {nullptr, kEndOfLine, kSec}
+
+const Cell kLevel1[] = {
+    {"sample         ", kLogL1SampleTime, kSec10}, {"send         ", kLogL1SendTime, kSec10}, EOL,
+    {"recv           ", kLogL1RecvTime, kSec10}, {"copy         ", kLogL1CopyTime, kSec10},
+    {"convert time ", kLogL1ConvertTime, kSec}, {"train  ", kLogL1TrainTime, kSec}, EOL,
+    {"feature nbytes ", kLogL1FeatureBytes, kSize10}, {"label nbytes ", kLogL1LabelBytes, kSize10}, EOL,
+    {"id nbytes      ", kLogL1IdBytes, kSize10}, {"graph nbytes ", kLogL1GraphBytes, kSize10}, EOL,
+    {"miss nbytes    ", kLogL1MissBytes, kSize10}, {"remote nbytes ", kLogL1RemoteBytes, kSize10}, EOL,
+    {"num nodes      ", kLogL1NumNode, kCount10}, {"num samples  ", kLogL1NumSample, kCount10}, EOL,
+    {"seq duration   ", kItemSeqDuration, kSec10}, {"refresh duration ", kItemRefreshDuration, kSec10}, EOL,
+};
+const Cell kLevel2[] = {
+    {"shuffle     ", kLogL2ShuffleTime, kSec}, {"core sample  ", kLogL2CoreSampleTime, kSec},
+    {"id remap        ", kLogL2IdRemapTime, kSec}, EOL,
+    {"graph copy  ", kLogL2GraphCopyTime, kSec}, {"id copy      ", kLogL2IdCopyTime, kSec},
+    {"cache feat copy ", kLogL2CacheCopyTime, kSec}, EOL,
+    {"last layer sample time ", kLogL2LastLayerTime, kSec}, {"size ", kLogL2LastLayerSize, kSec}, EOL,
+};
+const Cell kLevel3[] = {
+    {"khop sample coo  ", kLogL3KHopSampleCooTime, kSec}, {"khop sort coo      ", kLogL3KHopSampleSortCooTime, kSec},
+    {"khop count edge     ", kLogL3KHopSampleCountEdgeTime, kSec},
+    {"khop compact edge ", kLogL3KHopSampleCompactEdgesTime, kSec}, EOL,
+    {"walk sample coo  ", kLogL3RandomWalkSampleCooTime, kSec}, {"walk topk total    ", kLogL3RandomWalkTopKTime, kSec},
+    {"walk topk step1     ", kLogL3RandomWalkTopKStep1Time, kSec},
+    {"walk topk step2   ", kLogL3RandomWalkTopKStep2Time, kSec}, EOL,
+    {"walk topk step3  ", kLogL3RandomWalkTopKStep3Time, kSec}, {"walk topk step4    ", kLogL3RandomWalkTopKStep4Time, kSec},
+    {"walk topk step5     ", kLogL3RandomWalkTopKStep5Time, kSec}, EOL,
+    {"walk topk step6  ", kLogL3RandomWalkTopKStep6Time, kSec}, {"walk topk step7    ", kLogL3RandomWalkTopKStep7Time, kSec},
+    EOL,
+    {"remap unique     ", kLogL3RemapFillUniqueTime, kSec}, {"remap populate     ", kLogL3RemapPopulateTime, kSec},
+    {"remap mapnode       ", kLogL3RemapMapNodeTime, kSec}, {"remap mapedge     ", kLogL3RemapMapEdgeTime, kSec}, EOL,
+    {"cache get_index  ", kLogL3CacheGetIndexTime, kSec}, {"cache copy_index   ", KLogL3CacheCopyIndexTime, kSec},
+    {"cache extract_miss  ", kLogL3CacheExtractMissTime, kSec}, EOL,
+    {"cache copy_miss  ", kLogL3CacheCopyMissTime, kSec}, {"cache combine_miss ", kLogL3CacheCombineMissTime, kSec},
+    {"cache combine cache ", kLogL3CacheCombineCacheTime, kSec},
+    {"cache combine remote ", kLogL3CacheCombineRemoteTime, kSec}, EOL,
+    {"label extract  ", kLogL3LabelExtractTime, kSec}, EOL,
+};
+#undef EOL
+
+template <size_t N>
+void PrintLevel(std::ostream &out, int level, const Cell (&cells)[N], const std::string &type, uint64_t epoch,
+                uint64_t step, const double *v, double seq_duration, double refresh_duration) {
+  char buf[96];
+  snprintf(buf, sizeof(buf), "    [%s Profiler Level %d E%u S%u]\n", type.c_str(), level, (unsigned)epoch,
+           (unsigned)step);
+  out << buf;
+  bool first = true;
+  for (const Cell &c : cells) {
+    if (c.item == kEndOfLine) {
+      out << "\n";
+      first = true;
+      continue;
+    }
+    out << (first ? "        L" + std::to_string(level) + "  " : std::string(" | ")) << c.label;
+    first = false;
+    const double val = c.item == kItemSeqDuration ? seq_duration
+                       : c.item == kItemRefreshDuration ? refresh_duration
+                                                        : v[c.item];
+    switch (c.fmt) {
+      case kSec10: snprintf(buf, sizeof(buf), "%10.6lf", val); break;
+      case kSec: snprintf(buf, sizeof(buf), "%.6lf", val); break;
+      case kCount10: snprintf(buf, sizeof(buf), "%10.0lf", val); break;
+      case kSize10: snprintf(buf, sizeof(buf), "%10s", ToReadableSize((size_t)val).c_str()); break;
+    }
+    out << buf;
+  }
+}
+
+int ProfileLevel() {
+  const char *e = getenv("SAMGRAPH_PROFILE_LEVEL");  // constant.cc:64; anything but 1 or 2 means all three levels
+  if (e && std::string(e) == "1") return 1;
+  if (e && std::string(e) == "2") return 2;
+  return 3;
+}
+
+}  // namespace
+
 void Profiler::Output(const std::string &type, uint64_t epoch, uint64_t step, const double *v) {
-  char buf[1024];
-  snprintf(buf, sizeof(buf),
-           "    [%s Profiler Level 1 E%llu S%llu]\n"
-           "        L1  feature nbytes %10s | miss nbytes  %10s | remote nbytes %10s\n"
-           "    [%s Profiler Level 2 E%llu S%llu]\n"
-           "        L2  cache feat copy %.6lf\n"
-           "    [%s Profiler Level 3 E%llu S%llu]\n"
-           "        L3  cache get_index  %.6lf | cache combine_miss %.6lf | cache combine cache %.6lf | "
-           "cache combine remote %.6lf\n",
-           type.c_str(), (unsigned long long)epoch, (unsigned long long)step,
-           ToReadableSize((size_t)v[kLogL1FeatureBytes]).c_str(), ToReadableSize((size_t)v[kLogL1MissBytes]).c_str(),
-           ToReadableSize((size_t)v[kLogL1RemoteBytes]).c_str(), type.c_str(), (unsigned long long)epoch,
-           (unsigned long long)step, v[kLogL2CacheCopyTime], type.c_str(), (unsigned long long)epoch,
-           (unsigned long long)step, v[kLogL3CacheGetIndexTime], v[kLogL3CacheCombineMissTime],
-           v[kLogL3CacheCombineCacheTime], v[kLogL3CacheCombineRemoteTime]);
-  std::cout << buf;
+  const int level = ProfileLevel();
+  const double seq = 0, refresh = _refresh_duration;
+  PrintLevel(std::cout, 1, kLevel1, type, epoch, step, v, seq, refresh);
+  if (level >= 2) PrintLevel(std::cout, 2, kLevel2, type, epoch, step, v, seq, refresh);
+  if (level >= 3) PrintLevel(std::cout, 3, kLevel3, type, epoch, step, v, seq, refresh);
 }
 
 void Profiler::ReportStep(uint64_t epoch, uint64_t step) {

@@ -51,10 +51,13 @@ class Profiler {
   void ReportStepItemPercentiles(uint64_t epoch, uint64_t step, LogStepItem item, std::vector<double> percentiles,
                                  const std::string &name);
   void ReportStepAverageLastEpoch(uint64_t epoch, uint64_t step);
+  // duration of the last refresh, printed in the level-1 block (profiler.h: _refresh_duration)
+  void SetRefreshDuration(double seconds) { _refresh_duration = seconds; }
 
  private:
   void Output(const std::string &type, uint64_t epoch, uint64_t step, const double *vals);
   std::mutex _mu;
+  double _refresh_duration = 0;
   struct Row {
     double v[kNumLogStepItems] = {0};
     uint64_t set_mask[(kNumLogStepItems + 63) / 64] = {0};
