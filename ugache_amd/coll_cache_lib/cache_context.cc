@@ -224,9 +224,10 @@ ExtractSession::ExtractSession(std::shared_ptr<CacheContext> cache_ctx) : _cache
   uint32_t *state = _state_handle->ptr<uint32_t>();
   UGK_CALL(ugk_fill_u32(state, 0, 64, nullptr));
   UGK_CALL(ugk_stream_sync(nullptr));
-  _counts[0] = state;
-  _counts[1] = state + 2;
-  _status = state + 4;
+  _state = state;
+  _counts[0] = state + kStCounts0;
+  _counts[1] = state + kStCounts1;
+  _status = state + kStStatus;
   _host_mirror_handle = PinnedHostAlloc(256);
   _host_mirror = _host_mirror_handle->ptr<uint32_t>();
   memset(_host_mirror, 0, 256);
@@ -268,7 +269,7 @@ void ExtractSession::EnsureIdx(size_t num_nodes) {
 }
 
 void ExtractSession::CheckStatusWord(StreamHandle stream) const {
-  if (_host_mirror[0] == 0) return;  // common case: nothing to fetch from the device
+  if (_host_mirror[kMirError] == 0) return;  // common case: nothing to fetch from the device
   uint32_t st = 0;
   UGK_CALL(ugk_memcpy_async(&st, _status, sizeof(st), stream));
   UGK_CALL(ugk_stream_sync(stream));
@@ -354,8 +355,9 @@ size_t ExtractSession::DrainHotness(FreqRecorder *recorder) {
   UGK_CALL(ugk_set_device(_cache_ctx->_trainer_ctx.device_id));
   const size_t rows = _cache_ctx->_num_total_nodes;
   const size_t cap = _hot_entries->nbytes() / sizeof(uint64_t);
-  uint32_t *n_entries = _status + 2;       // device word, kept at zero between drains
-  uint32_t *host_out = _host_mirror + 4;   // [4] entries written, [5] rows left over
+  std::lock_guard<std::mutex> guard(_drain_mu);
+  uint32_t *n_entries = _state + kStDrainEntries;       // device word, kept at zero between drains
+  uint32_t *host_out = _host_mirror + kMirDrainCount;   // entries written, then "rows left over"
   uint64_t *dev_list = _hot_entries->ptr<uint64_t>();
   auto *host_list = _hot_entries_host->ptr<FreqEntry>();
   static_assert(sizeof(FreqEntry) == sizeof(uint64_t), "an entry is one (count << 32 | row) word");
@@ -366,7 +368,7 @@ size_t ExtractSession::DrainHotness(FreqRecorder *recorder) {
                               _record_stream));
     UGK_CALL(ugk_stream_sync(_record_stream));
     const size_t got = host_out[0];
-    CHECK_EQ(host_out[1], 0u);
+    CHECK_EQ(host_out[kMirDrainMore - kMirDrainCount], 0u);
     if (got == 0) continue;
     UGK_CALL(ugk_memcpy_async(host_list, dev_list, got * sizeof(uint64_t), _record_stream));
     UGK_CALL(ugk_stream_sync(_record_stream));
@@ -401,12 +403,12 @@ size_t ExtractSession::DedupKeys(const KeyT *nodes, size_t num_nodes, StreamHand
     UGK_CALL(ugk_fill_u32(_dedup_ws->ptr<uint32_t>(), 0, _dedup_ws->nbytes() / 4, stream));
     _dedup_epoch = 1;
   }
-  uint32_t *n_unique = _status + 1;
+  uint32_t *n_unique = _state + kStNumUnique;
   UGK_CALL(ugk_fill_u32(n_unique, 0, 1, stream));
   UGK_CALL(Dedup(nodes, num_nodes, _dedup_ws->ptr<void>(), _dedup_epoch, DedupUnique<KeyT>(),
-                 DedupInverse(), DedupRep(), n_unique, _host_mirror + 3, stream));
+                 DedupInverse(), DedupRep(), n_unique, _host_mirror + kMirNumUnique, stream));
   UGK_CALL(ugk_stream_sync(stream));
-  const size_t nu = _host_mirror[3];
+  const size_t nu = _host_mirror[kMirNumUnique];
   CHECK(nu >= 1 && nu <= num_nodes) << "deduplication produced " << nu << " keys from " << num_nodes;
   return nu;
 }
@@ -570,7 +572,8 @@ void ExtractSession::ExtractFeatImpl(const KeyT *nodes, size_t num_nodes, void *
   // the single blocking wait of the call; the gathers have written their group sizes (and the kernels any error
   // flag) into the pinned mirror, so no device-to-host copy is needed
   UGK_CALL(ugk_stream_sync(stream));
-  const uint32_t n_local = _host_mirror[1 + UGK_LOC_LOCAL], n_miss = _host_mirror[1 + UGK_LOC_HOST];
+  const uint32_t n_local = _host_mirror[kMirGroupSizes + UGK_LOC_LOCAL],
+                 n_miss = _host_mirror[kMirGroupSizes + UGK_LOC_HOST];
   _cur ^= 1;
   CheckStatusWord(stream);
   CHECK_EQ((size_t)n_local + n_miss, num_nodes);

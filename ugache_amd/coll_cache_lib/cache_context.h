@@ -12,6 +12,7 @@
 #include <cstdint>
 #include <functional>
 #include <memory>
+#include <mutex>
 #include <vector>
 
 #include "cache_hashtable.h"
@@ -83,6 +84,10 @@ class CacheContext {
 };
 
 class ExtractSession {
+  // words of the device-side state block (64 zero-filled uint32)
+  enum StateWord { kStCounts0 = 0, kStCounts1 = 2, kStStatus = 4, kStNumUnique = 5, kStDrainEntries = 6 };
+  // words of the pinned host mirror the kernels write; [1] and [2] are indexed 1 + location
+  enum MirrorWord { kMirError = 0, kMirGroupSizes = 1, kMirNumUnique = 3, kMirDrainCount = 4, kMirDrainMore = 5 };
   std::shared_ptr<CacheContext> _cache_ctx;
   MemHandle _idx_handle;          // ugk_idx_t[n], from the caller's allocator, regrown on demand
   MemHandle _state_handle;        // device: two counter pairs + status word
@@ -119,6 +124,8 @@ class ExtractSession {
   void *_ev_rec_begin = nullptr, *_ev_rec_done = nullptr;
   bool _record_pending = false;
   size_t _record_limit = SIZE_MAX;
+  std::mutex _drain_mu;  // one drain at a time: they share the entry list and its pinned copy
+  uint32_t *_state = nullptr;
   void JoinRecord(StreamHandle stream);
   size_t _num_lookups = 0;
   static constexpr size_t kHotDrainRows = 32u << 20;  // rows per drain step = capacity of the entry list
