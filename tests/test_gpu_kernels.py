@@ -518,7 +518,7 @@ def test_record_and_drain_match_bincount(kdtype, sparse):
     try:
         got = np.zeros(num_rows, np.int64)
         calls = 0
-        for first, cnt in ((0, 50_000), (50_000, num_rows - 50_000)):
+        for first, cnt in ((0, 50_001), (50_001, num_rows - 50_001)):
             while True:
                 hip.call("ugk_record_drain", ptr(counts), first, cnt, ptr(entries), cap, ptr(n_entries), out.ptr, None)
                 sync()
@@ -548,3 +548,27 @@ def test_record_rejects_keys_without_a_row():
     sync()
     assert status_value(st) & hip.ST_KEY_OUT_OF_RANGE
     assert to_np(counts, np.uint32)[:10].tolist() == [0, 0, 0, 2, 0, 0, 0, 0, 0, 0]
+
+
+@pytest.mark.parametrize("first,cnt", [(0, 1), (1, 1), (3, 2), (1, 3), (2, 7), (5, 64), (7, 257), (0, 0)])
+def test_drain_of_short_and_unaligned_row_ranges(first, cnt):
+    total = 300
+    host = np.arange(1, total + 1, dtype=np.uint32)  # every counter non-zero
+    counts = to_dev(host)
+    entries = dev_bytes(512 * 8)
+    n_entries = dev_zeros_u32(1)
+    out = PinnedArray((2,), np.uint32)
+    try:
+        hip.call("ugk_record_drain", ptr(counts), first, cnt, ptr(entries), 512, ptr(n_entries), out.ptr, None)
+        sync()
+        k = int(out.array[0])
+        assert k == cnt and int(out.array[1]) == 0
+        e = np.sort(to_np(entries, np.uint64)[:k])
+        rows = np.arange(first, first + cnt, dtype=np.uint64)
+        assert np.array_equal(e, np.sort(((rows + np.uint64(1)) << np.uint64(32)) | rows))
+        left = to_np(counts, np.uint32)[:total]
+        want = host.copy()
+        want[first:first + cnt] = 0
+        assert np.array_equal(left, want)  # nothing outside the range was touched
+    finally:
+        out.free()

@@ -77,37 +77,64 @@ __global__ __launch_bounds__(kBlock) void record_kernel(const K *__restrict__ ke
   }
 }
 
+// Most counters are zero, so the scan is wavefront-granular and branch-free until something is found: a wavefront
+// reads 64 x 4 counters (one 16-byte load per lane), and only if any of them is non-zero does it reserve list slots
+// (one atomic per wavefront) and exchange those counters for zero.
 __global__ __launch_bounds__(kBlock) void drain_kernel(uint32_t *counts, uint64_t num_rows, uint64_t first_row,
                                                        unsigned long long *entries, uint32_t capacity,
                                                        uint32_t *n_entries) {
-  __shared__ uint32_t wave_tot[kWavesPerBlock];
-  __shared__ uint32_t base;
-  const int tid = threadIdx.x;
-  const int lane = tid & (kWave - 1), wave = tid / kWave;
-  const uint64_t n_round = (num_rows + kBlock - 1) / kBlock * kBlock;
-  for (uint64_t i = (uint64_t)blockIdx.x * kBlock + tid; i < n_round; i += (uint64_t)gridDim.x * kBlock) {
-    // a plain read first: most counters are zero and need no atomic
-    const bool hot = i < num_rows && __builtin_nontemporal_load(counts + i) != 0;
-    const uint64_t wb = __ballot(hot);
-    const uint32_t pre = __popcll(wb & ((1ull << lane) - 1ull));
-    if (lane == 0) wave_tot[wave] = __popcll(wb);
-    __syncthreads();
-    uint32_t before = 0, total = 0;
-#pragma unroll
-    for (int w = 0; w < kWavesPerBlock; ++w) {
-      if (w == wave) before = total;
-      total += wave_tot[w];
+  const int lane = (int)lane_id();
+  const uint64_t wave = ((uint64_t)blockIdx.x * kBlock + threadIdx.x) / kWave;
+  const uint64_t n_waves = (uint64_t)gridDim.x * (kBlock / kWave);
+  // counts is 4-byte aligned only as far as this function knows: peel to a 16-byte boundary with scalar reads
+  const uint64_t head = min<uint64_t>(num_rows, (4 - (((uintptr_t)counts / 4) & 3)) & 3);
+  const uint64_t n_vec = (num_rows - head) / 4;
+  const u32x4 *vec = reinterpret_cast<const u32x4 *>(counts + head);
+  for (uint64_t v0 = wave * kWave; v0 < n_vec + kWave; v0 += n_waves * kWave) {
+    // the last trip of wavefront 0's successor range also covers the scalar head and tail (at most 6 rows)
+    const uint64_t v = v0 + lane;
+    u32x4 c{0, 0, 0, 0};
+    uint64_t row0 = 0;
+    if (v < n_vec) {
+      c = __builtin_nontemporal_load(vec + v);
+      row0 = head + v * 4;
+    } else if (v == n_vec) {  // one lane picks up the unaligned head rows
+      row0 = 0;
+      if (head > 0) c.x = counts[0];
+      if (head > 1) c.y = counts[1];
+      if (head > 2) c.z = counts[2];
+    } else if (v == n_vec + 1) {  // and one the tail rows behind the last full vector
+      row0 = head + n_vec * 4;
+      const uint64_t left = num_rows - row0;
+      if (left > 0) c.x = counts[row0];
+      if (left > 1) c.y = counts[row0 + 1];
+      if (left > 2) c.z = counts[row0 + 2];
     }
-    if (tid == 0) base = total ? atomicAdd(n_entries, total) : 0u;
-    __syncthreads();
-    if (hot) {
-      const uint32_t slot = base + before + pre;
-      if (slot < capacity) {  // a full list leaves the counter alone: the next call picks it up
-        const uint32_t c = atomicExch(counts + i, 0u);
-        entries[slot] = ((unsigned long long)c << 32) | (uint32_t)(first_row + i);
+    const uint32_t mine = (c.x != 0) + (c.y != 0) + (c.z != 0) + (c.w != 0);
+    if (__ballot(mine != 0) == 0) continue;
+    // inclusive prefix of `mine` over the wavefront
+    uint32_t incl = mine;
+#pragma unroll
+    for (int d = 1; d < kWave; d <<= 1) {
+      const uint32_t up = __shfl_up(incl, d);
+      if (lane >= d) incl += up;
+    }
+    const uint32_t total = __shfl(incl, kWave - 1);
+    uint32_t base = 0;
+    if (lane == 0) base = atomicAdd(n_entries, total);
+    base = __shfl(base, 0);
+    uint32_t slot = base + incl - mine;
+    const uint32_t cc[4] = {c.x, c.y, c.z, c.w};
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      if (cc[k] != 0) {
+        if (slot < capacity) {  // a full list leaves the counter alone: the next call picks it up
+          const uint32_t got = atomicExch(counts + row0 + k, 0u);
+          entries[slot] = ((unsigned long long)got << 32) | (uint32_t)(first_row + row0 + k);
+        }
+        ++slot;
       }
     }
-    __syncthreads();
   }
 }
 
@@ -159,7 +186,7 @@ int ugk_record_drain(uint32_t *counts_dev, uint64_t first_row, uint64_t num_rows
   UGK_REQUIRE(capacity > 0, "ugk_record_drain: empty entry list");
   UGK_REQUIRE(first_row + num_rows <= 0xffffffffull, "ugk_record_drain: rows must fit 32 bits");
   if (num_rows) {
-    const unsigned grid = clamp_grid((num_rows + kBlock - 1) / kBlock, 0);
+    const unsigned grid = clamp_grid((num_rows / 4 + 2 * kWave + kBlock - 1) / kBlock, 0);
     hipLaunchKernelGGL(drain_kernel, dim3(grid), dim3(kBlock), 0, as_stream(stream), counts_dev + first_row, num_rows,
                        first_row, reinterpret_cast<unsigned long long *>(entries_dev), capacity, n_entries_dev);
     UGK_HIP(hipGetLastError());
