@@ -77,64 +77,93 @@ __global__ __launch_bounds__(kBlock) void record_kernel(const K *__restrict__ ke
   }
 }
 
-// Most counters are zero, so the scan is wavefront-granular and branch-free until something is found: a wavefront
-// reads 64 x 4 counters (one 16-byte load per lane), and only if any of them is non-zero does it reserve list slots
-// (one atomic per wavefront) and exchange those counters for zero.
+// A wavefront owns a contiguous run of counters and goes over it twice: first it counts the non-zero ones, reserves
+// that many list slots with ONE atomic (a reservation per 256 counters would serialise on the list's single counter:
+// with 1 % of the rows hot nearly every group of 256 holds one), then it reads the run again, exchanges the non-zero
+// counters for zero and writes their entries.  Counters only grow between the two passes, so the second pass finds at
+// least what the first one counted; what it finds beyond the reservation stays for the next drain.
+struct DrainVec {
+  u32x4 c;
+  uint64_t row0;
+};
+
+// vector v of the run: 4 adjacent counters from a 16-byte load; two pseudo vectors behind the last one carry the
+// (at most 3 + 3) counters in front of the first and behind the last aligned vector
+__device__ __forceinline__ DrainVec drain_load(const uint32_t *counts, uint64_t num_rows, uint64_t head, uint64_t n_vec,
+                                               uint64_t v) {
+  DrainVec d{u32x4{0, 0, 0, 0}, 0};
+  if (v < n_vec) {
+    d.c = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(counts + head) + v);
+    d.row0 = head + v * 4;
+  } else if (v == n_vec) {
+    if (head > 0) d.c.x = counts[0];
+    if (head > 1) d.c.y = counts[1];
+    if (head > 2) d.c.z = counts[2];
+  } else if (v == n_vec + 1) {
+    d.row0 = head + n_vec * 4;
+    const uint64_t left = num_rows - d.row0;
+    if (left > 0) d.c.x = counts[d.row0];
+    if (left > 1) d.c.y = counts[d.row0 + 1];
+    if (left > 2) d.c.z = counts[d.row0 + 2];
+  }
+  return d;
+}
+
+__device__ __forceinline__ uint32_t nonzeros(const u32x4 &c) {
+  return (c.x != 0) + (c.y != 0) + (c.z != 0) + (c.w != 0);
+}
+
 __global__ __launch_bounds__(kBlock) void drain_kernel(uint32_t *counts, uint64_t num_rows, uint64_t first_row,
                                                        unsigned long long *entries, uint32_t capacity,
                                                        uint32_t *n_entries) {
   const int lane = (int)lane_id();
   const uint64_t wave = ((uint64_t)blockIdx.x * kBlock + threadIdx.x) / kWave;
   const uint64_t n_waves = (uint64_t)gridDim.x * (kBlock / kWave);
-  // counts is 4-byte aligned only as far as this function knows: peel to a 16-byte boundary with scalar reads
-  const uint64_t head = min<uint64_t>(num_rows, (4 - (((uintptr_t)counts / 4) & 3)) & 3);
+  const uint64_t head = min((uint64_t)num_rows, (uint64_t)((4 - (((uintptr_t)counts / 4) & 3)) & 3));
   const uint64_t n_vec = (num_rows - head) / 4;
-  const u32x4 *vec = reinterpret_cast<const u32x4 *>(counts + head);
-  for (uint64_t v0 = wave * kWave; v0 < n_vec + kWave; v0 += n_waves * kWave) {
-    // the last trip of wavefront 0's successor range also covers the scalar head and tail (at most 6 rows)
+  const uint64_t n_all = n_vec + 2;
+  const uint64_t per_wave = ((n_all + n_waves - 1) / n_waves + kWave - 1) / kWave * kWave;
+  const uint64_t begin = wave * per_wave, end = min(n_all, begin + per_wave);
+  if (begin >= end) return;
+
+  uint32_t found = 0;
+  for (uint64_t v0 = begin; v0 < end; v0 += kWave) {
     const uint64_t v = v0 + lane;
-    u32x4 c{0, 0, 0, 0};
-    uint64_t row0 = 0;
-    if (v < n_vec) {
-      c = __builtin_nontemporal_load(vec + v);
-      row0 = head + v * 4;
-    } else if (v == n_vec) {  // one lane picks up the unaligned head rows
-      row0 = 0;
-      if (head > 0) c.x = counts[0];
-      if (head > 1) c.y = counts[1];
-      if (head > 2) c.z = counts[2];
-    } else if (v == n_vec + 1) {  // and one the tail rows behind the last full vector
-      row0 = head + n_vec * 4;
-      const uint64_t left = num_rows - row0;
-      if (left > 0) c.x = counts[row0];
-      if (left > 1) c.y = counts[row0 + 1];
-      if (left > 2) c.z = counts[row0 + 2];
-    }
-    const uint32_t mine = (c.x != 0) + (c.y != 0) + (c.z != 0) + (c.w != 0);
-    if (__ballot(mine != 0) == 0) continue;
-    // inclusive prefix of `mine` over the wavefront
+    if (v < end) found += nonzeros(drain_load(counts, num_rows, head, n_vec, v).c);
+  }
+#pragma unroll
+  for (int d = kWave / 2; d > 0; d >>= 1) found += __shfl_xor(found, d);
+  if (found == 0) return;  // wavefront-uniform
+  uint32_t base = 0;
+  if (lane == 0) base = atomicAdd(n_entries, found);
+  base = __shfl(base, 0);
+
+  uint32_t used = 0;  // slots of the reservation handed out so far (wavefront-uniform)
+  for (uint64_t v0 = begin; v0 < end && used < found; v0 += kWave) {
+    const uint64_t v = v0 + lane;
+    DrainVec d{u32x4{0, 0, 0, 0}, 0};
+    if (v < end) d = drain_load(counts, num_rows, head, n_vec, v);
+    const uint32_t mine = nonzeros(d.c);
     uint32_t incl = mine;
 #pragma unroll
-    for (int d = 1; d < kWave; d <<= 1) {
-      const uint32_t up = __shfl_up(incl, d);
-      if (lane >= d) incl += up;
+    for (int s = 1; s < kWave; s <<= 1) {
+      const uint32_t up = __shfl_up(incl, s);
+      if (lane >= s) incl += up;
     }
-    const uint32_t total = __shfl(incl, kWave - 1);
-    uint32_t base = 0;
-    if (lane == 0) base = atomicAdd(n_entries, total);
-    base = __shfl(base, 0);
-    uint32_t slot = base + incl - mine;
-    const uint32_t cc[4] = {c.x, c.y, c.z, c.w};
+    uint32_t idx = used + incl - mine;
+    const uint32_t cc[4] = {d.c.x, d.c.y, d.c.z, d.c.w};
 #pragma unroll
     for (int k = 0; k < 4; ++k) {
       if (cc[k] != 0) {
-        if (slot < capacity) {  // a full list leaves the counter alone: the next call picks it up
-          const uint32_t got = atomicExch(counts + row0 + k, 0u);
-          entries[slot] = ((unsigned long long)got << 32) | (uint32_t)(first_row + row0 + k);
+        // beyond the reservation or beyond the list: the counter stays as it is for the next drain
+        if (idx < found && base + idx < capacity) {
+          const uint32_t got = atomicExch(counts + d.row0 + k, 0u);
+          entries[base + idx] = ((unsigned long long)got << 32) | (uint32_t)(first_row + d.row0 + k);
         }
-        ++slot;
+        ++idx;
       }
     }
+    used += __shfl(incl, kWave - 1);
   }
 }
 
@@ -186,7 +215,8 @@ int ugk_record_drain(uint32_t *counts_dev, uint64_t first_row, uint64_t num_rows
   UGK_REQUIRE(capacity > 0, "ugk_record_drain: empty entry list");
   UGK_REQUIRE(first_row + num_rows <= 0xffffffffull, "ugk_record_drain: rows must fit 32 bits");
   if (num_rows) {
-    const unsigned grid = clamp_grid((num_rows / 4 + 2 * kWave + kBlock - 1) / kBlock, 0);
+    // few, long wavefronts: one reservation each (8 workgroups per CU)
+    const unsigned grid = clamp_grid((num_rows / 4 + 2 + kBlock - 1) / kBlock, (unsigned)cu_count() * 8u);
     hipLaunchKernelGGL(drain_kernel, dim3(grid), dim3(kBlock), 0, as_stream(stream), counts_dev + first_row, num_rows,
                        first_row, reinterpret_cast<unsigned long long *>(entries_dev), capacity, n_entries_dev);
     UGK_HIP(hipGetLastError());

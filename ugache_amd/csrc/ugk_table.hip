@@ -2,6 +2,7 @@
 // Insert and evict run at cache-fill / refresh time only, so they use a simple per-lane probe loop; the
 // per-batch lookup is the wavefront-cooperative one in ugk_table.cuh.
 #include <cmath>
+#include <cstddef>
 
 #include "ugk_internal.h"
 #include "ugk_table.cuh"
@@ -49,6 +50,13 @@ __device__ __forceinline__ uint64_t load_key_relaxed(const ugk_bucket_t *b) {
   return __atomic_load_n(&b->key, __ATOMIC_RELAXED);
 }
 
+// off and meta are the second 8 bytes of a bucket: one aligned 8-byte store changes both at once
+__device__ __forceinline__ void store_off_meta(ugk_bucket_t *b, uint32_t off, uint32_t meta) {
+  static_assert(offsetof(ugk_bucket_t, off) == 8 && offsetof(ugk_bucket_t, meta) == 12 && sizeof(ugk_bucket_t) == 16,
+                "bucket layout");
+  __atomic_store_n(reinterpret_cast<uint64_t *>(&b->off), ((uint64_t)meta << 32) | off, __ATOMIC_RELAXED);
+}
+
 template <typename K>
 __global__ __launch_bounds__(kBlock) void hash_insert_kernel(ugk_bucket_t *table, uint64_t nb, const K *keys,
                                                              const uint32_t *offs, uint32_t seq_base, uint32_t loc,
@@ -68,10 +76,9 @@ __global__ __launch_bounds__(kBlock) void hash_insert_kernel(ugk_bucket_t *table
         const uint64_t seen = atomicCAS(reinterpret_cast<unsigned long long *>(&table[pos].key),
                                         (unsigned long long)cur, (unsigned long long)key);
         if (seen == cur) {
-          // the bucket is ours: publish the value, then the valid bit
-          table[pos].off = off;
-          __threadfence();
-          __atomic_store_n(&table[pos].meta, UGK_META_VALID | (loc & 0xfu), __ATOMIC_RELEASE);
+          // the bucket is ours: slot and valid bit appear together, in one 8-byte store.  Until then the bucket reads
+          // as "key present, not valid", i.e. as a miss.
+          store_off_meta(table + pos, off, UGK_META_VALID | (loc & 0xfu));
           placed = true;
           break;
         }
@@ -100,9 +107,10 @@ __global__ __launch_bounds__(kBlock) void hash_evict_kernel(ugk_bucket_t *table,
     for (uint64_t step = 0; step < nb && !done; ++step) {
       const uint64_t cur = load_key_relaxed(table + pos);
       if (cur == key) {
-        __atomic_store_n(&table[pos].meta, 0u, __ATOMIC_RELEASE);
-        __threadfence();
-        __atomic_store_n(&table[pos].key, UGK_HASH_TOMB, __ATOMIC_RELEASE);
+        // either order of these two stores is safe for a concurrent lookup: it sees the key still valid (its slot
+        // keeps the row until a later lookup has passed), not valid, or gone
+        store_off_meta(table + pos, 0u, 0u);
+        __atomic_store_n(&table[pos].key, UGK_HASH_TOMB, __ATOMIC_RELAXED);
         done = true;
       } else if (cur == UGK_HASH_EMPTY) {
         atomicOr(status, UGK_ST_EVICT_ABSENT);
