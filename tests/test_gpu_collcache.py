@@ -100,7 +100,7 @@ def test_direct_mapping_full_and_no_cache(kdtype, pct):
 
 
 @pytest.mark.parametrize("table_kind", ["FLAT", "HASH"])
-@pytest.mark.parametrize("impl", ["", "DIRECT", "NONE"])
+@pytest.mark.parametrize("impl", ["", "SMMaskPhase", "DIRECT", "NONE"])
 @pytest.mark.parametrize("kdtype", [torch.int32, torch.int64])
 def test_partial_cache_matches_oracle(table_kind, impl, kdtype, monkeypatch):
     monkeypatch.setenv("COLL_HASH_TABLE", table_kind)
@@ -135,12 +135,10 @@ def test_partial_cache_matches_oracle(table_kind, impl, kdtype, monkeypatch):
         kt = torch.from_numpy(keys).to(kdtype).cuda()
         out = co.coll_torch_lookup_key_t_val_ret(0, kt, False)
         assert out.cpu().numpy().tobytes() == ORC.gather(table, keys.astype(np.int64)).tobytes()
-        if impl != "DIRECT":
-            n_local = int((nid[keys] == 0).sum())
-            assert _basics.last_group_offset(0) == [0, n_local, n]
-    if impl != "DIRECT":
-        step = _basics.info(0)["lookups"] - 1
-        assert _basics.step_value(step, kLogL1MissBytes) == (n - n_local) * dim * 4
+        n_local = int((nid[keys] == 0).sum())
+        assert _basics.last_group_offset(0) == [0, n_local, n]
+    step = _basics.info(0)["lookups"] - 1
+    assert _basics.step_value(step, kLogL1MissBytes) == (n - n_local) * dim * 4
 
 
 @pytest.mark.parametrize("pct", [0.0, 0.1, 1.0])
@@ -238,8 +236,11 @@ def test_raw_model_directory_and_mock_table(tmp_path):
 
 @pytest.mark.parametrize("table_kind", ["FLAT", "HASH"])
 @pytest.mark.parametrize("foreground", [True, False])
-def test_refresh_evicts_and_inserts_like_the_oracle(table_kind, foreground, monkeypatch):
+@pytest.mark.parametrize("impl", ["", "SMMaskPhase"])
+def test_refresh_evicts_and_inserts_like_the_oracle(table_kind, foreground, impl, monkeypatch):
     monkeypatch.setenv("COLL_HASH_TABLE", table_kind)
+    if impl:
+        monkeypatch.setenv("SAMGRAPH_COLL_CACHE_CONCURRENT_LINK_IMPL", impl)
     monkeypatch.setenv("COLL_REFRESH_SLEEP_US", "100")
     monkeypatch.setenv("COLL_REFRESH_BATCH_ROWS", "512")
     rng = np.random.default_rng(11)
@@ -292,7 +293,7 @@ def test_refresh_evicts_and_inserts_like_the_oracle(table_kind, foreground, monk
         old_cached = new_cached
 
 
-@pytest.mark.parametrize("pct,impl,dedup", [(0.25, "", False), (0.25, "NONE", True), (0.25, "DIRECT", False),
+@pytest.mark.parametrize("pct,impl,dedup", [(0.25, "", False), (0.25, "NONE", True), (0.25, "SMMaskPhase", False),
                                             (1.0, "", False), (0.0, "", True)])
 @pytest.mark.parametrize("kdtype", [torch.int32, torch.int64])
 def test_hotness_counted_on_the_device_ranks_like_the_host_recorder(pct, impl, dedup, kdtype, monkeypatch):
@@ -338,9 +339,8 @@ def test_hotness_counted_on_the_device_ranks_like_the_host_recorder(pct, impl, d
         keys = rng.integers(0, n_item, size=20_000)
         out = co.coll_torch_lookup_key_t_val_ret(0, torch.from_numpy(keys).to(kdtype).cuda(), False)
         assert out.cpu().numpy().tobytes() == ORC.gather(table, keys.astype(np.int64)).tobytes()
-        if impl != "DIRECT":  # the fused kernel produces no group sizes
-            assert _basics.last_group_offset(0)[1] == (int((new_nid[keys] == 0).sum()) if not dedup else
-                                                       int((new_nid[np.unique(keys)] == 0).sum()))
+        assert _basics.last_group_offset(0)[1] == (int((new_nid[keys] == 0).sum()) if not dedup else
+                                                   int((new_nid[np.unique(keys)] == 0).sum()))
         allk = keys.astype(np.uint32)  # the refresh consumed the counts; only this last lookup is left
     want_k, want_c = ORC.freq_rank(allk)
     got_k = np.zeros(n_item, np.uint32)

@@ -363,9 +363,17 @@ def test_classify_partition_and_factored_gather(mode, kdtype, n):
         # fused single-kernel variant gives the same bytes
         out2 = dev_bytes(n * rb, fill=0x11)
         fn = "ugk_extract_mix_i64" if kdtype == np.int64 else "ugk_extract_mix_u32"
-        hip.call(fn, tb, ptr(keys_dev), n, ptr(cache_dev), cap, pin.ptr, nkeys, ptr(out2), rb, ptr(st2), None, None)
-        assert status_value(st2) == 0
-        assert to_np(out2)[: n * rb].tobytes() == want_out.tobytes()
+        mix_counts = dev_zeros_u32(3)
+        for _ in range(2):  # the second launch finds the counters left at zero by the first
+            mirror.array[...] = 0xFFFFFFFF
+            hip.call(fn, tb, ptr(keys_dev), n, ptr(cache_dev), cap, pin.ptr, nkeys, ptr(out2), rb, ptr(st2), mirror.ptr,
+                     ptr(mix_counts), None)
+            sync()
+            assert status_value(st2) == 0
+            assert to_np(out2)[: n * rb].tobytes() == want_out.tobytes()
+            if n:  # same group sizes as classify found
+                assert mirror.array.tolist()[1:3] == [int(c[0]), int(c[1])]
+            assert not to_np(mix_counts, np.uint32)[:3].any()
     finally:
         sync()
         pin.free()
@@ -398,7 +406,7 @@ def test_extract_mix_other_row_sizes(row_bytes):
         st = dev_zeros_u32(1)
         d_keys, d_cache = to_dev(keys), to_dev(cache)
         hip.call("ugk_extract_mix_u32", tb, ptr(d_keys), len(keys), ptr(d_cache), len(cached), pin.ptr,
-                 nkeys, ptr(out), row_bytes, ptr(st), None, None)
+                 nkeys, ptr(out), row_bytes, ptr(st), None, None, None)
         assert status_value(st) == 0
         assert to_np(out)[: len(keys) * row_bytes].tobytes() == host[keys].tobytes()
     finally:

@@ -412,15 +412,16 @@ size_t ExtractSession::DedupKeys(const KeyT *nodes, size_t num_nodes, StreamHand
   CHECK(nu >= 1 && nu <= num_nodes) << "deduplication produced " << nu << " keys from " << num_nodes;
   return nu;
 }
+
 static int ExtractMix(ugk_table_t t, const IdType *keys, size_t n, const void *cache, uint64_t cache_rows,
                       const void *host, uint64_t host_rows, void *out, size_t rb, uint32_t *st, uint32_t *mirror,
-                      StreamHandle s) {
-  return ugk_extract_mix_u32(t, keys, n, cache, cache_rows, host, host_rows, out, rb, st, mirror, s);
+                      uint32_t *counts, StreamHandle s) {
+  return ugk_extract_mix_u32(t, keys, n, cache, cache_rows, host, host_rows, out, rb, st, mirror, counts, s);
 }
 static int ExtractMix(ugk_table_t t, const Id64Type *keys, size_t n, const void *cache, uint64_t cache_rows,
                       const void *host, uint64_t host_rows, void *out, size_t rb, uint32_t *st, uint32_t *mirror,
-                      StreamHandle s) {
-  return ugk_extract_mix_i64(t, keys, n, cache, cache_rows, host, host_rows, out, rb, st, mirror, s);
+                      uint32_t *counts, StreamHandle s) {
+  return ugk_extract_mix_i64(t, keys, n, cache, cache_rows, host, host_rows, out, rb, st, mirror, counts, s);
 }
 
 // cache_context.cu:1199-1794
@@ -503,22 +504,31 @@ void ExtractSession::ExtractFeatImpl(const KeyT *nodes, size_t num_nodes, void *
   const uint64_t host_rows = ctx->_num_total_nodes;
 
   if (RunConfig::concurrent_link_impl == kDirectNoGroup && dst_map == nullptr) {
-    // one fused lookup + gather kernel, source chosen per row (cache_context.cu:1295-1329)
+    // one fused lookup + gather kernel, source chosen per row (cache_context.cu:1295-1329).  The default here: the
+    // host link is busy from the first wavefront on, with no classify pass and no cross-stream hand-off in front of
+    // it, and since the link bounds a mixed batch it does not matter that host loads spread over the chip slow the
+    // HBM loads next to them.
     RecordKeys(input_nodes, num_input, stream, nullptr);
     UGK_CALL(ugk_event_record(_ev_t[0], stream));
     UGK_CALL(ExtractMix(table, nodes, num_nodes, cache, cache_rows, host, host_rows, output, rb, _status,
-                        _host_mirror, stream));
+                        _host_mirror, _state + kStMixCounts, stream));
     UGK_CALL(ugk_event_record(_ev_t[1], stream));
     JoinRecord(stream);
     UGK_CALL(ugk_stream_sync(stream));
     CheckStatusWord(stream);
+    const uint32_t n_local = _host_mirror[kMirGroupSizes + UGK_LOC_LOCAL],
+                   n_miss = _host_mirror[kMirGroupSizes + UGK_LOC_HOST];
+    CHECK_EQ((size_t)n_local + n_miss, num_nodes);
     float mix_ms = 0;
     UGK_CALL(ugk_event_elapsed_ms(_ev_t[0], _ev_t[1], &mix_ms));
-    _group_offset[1] = _group_offset[2] = (uint32_t)num_nodes;  // group sizes are not produced on this path
+    _group_offset[1] = n_local;
+    _group_offset[2] = (uint32_t)num_nodes;
     if (profiler && task_key != 0xffffffffffffffffull) {
       profiler->LogStep(task_key, kLogL1FeatureBytes, nbytes);
+      profiler->LogStep(task_key, kLogL1MissBytes, (double)n_miss * rb);
       profiler->LogStep(task_key, kLogL3CacheCombineCacheTime, mix_ms * 1e-3);
       profiler->LogEpochAdd(task_key, kLogEpochFeatureBytes, nbytes);
+      profiler->LogEpochAdd(task_key, kLogEpochMissBytes, (double)n_miss * rb);
     }
     ctx->progress.fetch_add(1);
     return;

@@ -85,7 +85,8 @@ class CacheContext {
 
 class ExtractSession {
   // words of the device-side state block (64 zero-filled uint32)
-  enum StateWord { kStCounts0 = 0, kStCounts1 = 2, kStStatus = 4, kStNumUnique = 5, kStDrainEntries = 6 };
+  enum StateWord { kStCounts0 = 0, kStCounts1 = 2, kStStatus = 4, kStNumUnique = 5, kStDrainEntries = 6,
+                   kStMixCounts = 8 /* 3 words */ };
   // words of the pinned host mirror the kernels write; [1] and [2] are indexed 1 + location
   enum MirrorWord { kMirError = 0, kMirGroupSizes = 1, kMirNumUnique = 3, kMirDrainCount = 4, kMirDrainMore = 5 };
   std::shared_ptr<CacheContext> _cache_ctx;

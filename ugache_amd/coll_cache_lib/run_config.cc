@@ -24,7 +24,7 @@ int RunConfig::solver_omp_thread_num_per_gpu = 5;
 int RunConfig::refresher_omp_thread_num = 8;
 int RunConfig::refresher_omp_thread_num_per_gpu = 1;
 size_t RunConfig::option_empty_feat = 0;
-ConcurrentLinkImpl RunConfig::concurrent_link_impl = kSMMaskPhase;
+ConcurrentLinkImpl RunConfig::concurrent_link_impl = kDirectNoGroup;
 size_t RunConfig::coll_cache_scale_nb = 16;
 bool RunConfig::use_flat_hashtable = true;
 double RunConfig::coll_cache_hyperparam_T_local = 1;
@@ -63,7 +63,7 @@ void RunConfig::SetKeyMap(uint64_t mul, int bits) {
 void RunConfig::LoadConfigFromEnv() {
   // every knob goes back to its default first, so a process that builds a second cache sees only its current
   // environment
-  concurrent_link_impl = kSMMaskPhase;
+  concurrent_link_impl = kDirectNoGroup;
   coll_cache_scale_nb = 16;
   hash_load_factor = 0.7;
   force_table_kind = 0;
@@ -82,9 +82,12 @@ void RunConfig::LoadConfigFromEnv() {
   }
   const std::string no_group = GetEnv("SAMGRAPH_COLL_CACHE_NO_GROUP");
   const std::string impl = GetEnv("SAMGRAPH_COLL_CACHE_CONCURRENT_LINK_IMPL");
-  if (no_group == "DIRECT" || impl == "DIRECT") {
+  // The reference defaults to its factored extraction (MPSPhase on its platforms).  With one GPU and its host as the
+  // only two sources the fused kernel is the faster one on this hardware, so it is what an unset variable selects;
+  // the reference's names still select the reference's structure.
+  if (no_group == "DIRECT" || impl == "DIRECT" || impl == "") {
     concurrent_link_impl = kDirectNoGroup;
-  } else if (impl == "" || impl == "SMMaskPhase" || impl == "MPSPhase") {
+  } else if (impl == "SMMaskPhase" || impl == "MPSPhase") {
     concurrent_link_impl = kSMMaskPhase;
   } else if (impl == "NONE" || impl == "NoConcurrent") {
     concurrent_link_impl = kNoConcurrentLink;

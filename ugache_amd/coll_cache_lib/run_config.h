@@ -15,8 +15,8 @@ namespace common {
 // sense with one GPU and its host are kept).
 enum ConcurrentLinkImpl {
   kNoConcurrentLink = 0,  // host group, then local group, on the caller's stream
-  kSMMaskPhase,           // default: the two groups as concurrent kernels on their own streams
-  kDirectNoGroup,         // one fused lookup+gather kernel, no partition (SAMGRAPH_COLL_CACHE_NO_GROUP=DIRECT)
+  kSMMaskPhase,           // the two groups as concurrent kernels on their own streams (SMMaskPhase / MPSPhase)
+  kDirectNoGroup,         // default: one fused lookup+gather kernel, no partition (also SAMGRAPH_COLL_CACHE_NO_GROUP=DIRECT)
 };
 
 namespace coll_cache {

@@ -13,8 +13,6 @@
 namespace ugk {
 namespace {
 
-constexpr int kWavesPerBlock = kBlock / kWave;
-
 // Hot rows are hot: with a skewed key distribution a few counters would take most of the atomics of a batch and
 // serialise them in the memory-side atomic units.  Each workgroup therefore first counts its tile of keys in a small
 // LDS table (row -> count, open addressing, at most half full) and then adds every distinct row of the tile to the

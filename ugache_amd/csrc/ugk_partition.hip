@@ -115,8 +115,13 @@ __global__ __launch_bounds__(kBlock) void extract_mix_kernel(ugk_table_t t, cons
                                                              const u32x4 *__restrict__ cache, uint64_t cache_rows,
                                                              const u32x4 *__restrict__ host, uint64_t host_rows,
                                                              u32x4 *__restrict__ out, uint32_t vpr,
-                                                             uint32_t *status, uint32_t *host_mirror) {
+                                                             uint32_t *status, uint32_t *host_mirror,
+                                                             uint32_t *counts) {
   constexpr int RPW = kWave / LPR;  // rows per wavefront instruction
+  __shared__ uint32_t block_tot[2];
+  if (threadIdx.x < 2) block_tot[threadIdx.x] = 0;
+  __syncthreads();
+  uint32_t wave_local = 0, wave_host = 0;  // rows this wavefront took from each source (wavefront-uniform)
   constexpr int UNROLL = (RPW * 4 <= kWave) ? 4 : (kWave / RPW);
   const int lane = (int)lane_id();
   const int sub = lane % LPR, rg = lane / LPR;
@@ -138,6 +143,11 @@ __global__ __launch_bounds__(kBlock) void extract_mix_kernel(ugk_table_t t, cons
       }
     }
     const uint64_t rowbits = reinterpret_cast<uint64_t>(rowp);
+    if (counts) {
+      const bool from_cache = rowp != nullptr && f.hit && f.loc == UGK_LOC_LOCAL;
+      wave_local += __popcll(__ballot(from_cache));
+      wave_host += __popcll(__ballot(rowp != nullptr && !from_cache));
+    }
     for (int r0 = 0; r0 < kWave; r0 += RPW * UNROLL) {
       const u32x4 *p[UNROLL];
 #pragma unroll
@@ -153,6 +163,28 @@ __global__ __launch_bounds__(kBlock) void extract_mix_kernel(ugk_table_t t, cons
           for (int u = 0; u < UNROLL; ++u)
             if (p[u]) __builtin_nontemporal_store(v[u], out + (b0 + r0 + u * RPW + rg) * vpr + col);
         }
+      }
+    }
+  }
+  if (counts == nullptr) return;
+  // group sizes for the host: per workgroup one atomic per source, and the workgroup that finishes last (ticket
+  // counter) hands the totals to the pinned mirror and leaves the three device words at zero for the next launch
+  if (lane == 0) {
+    if (wave_local) atomicAdd(&block_tot[0], wave_local);
+    if (wave_host) atomicAdd(&block_tot[1], wave_host);
+  }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    if (block_tot[0]) atomicAdd(counts + 0, block_tot[0]);
+    if (block_tot[1]) atomicAdd(counts + 1, block_tot[1]);
+    __threadfence();
+    if (atomicAdd(counts + 2, 1u) == gridDim.x - 1) {
+      __threadfence();
+      const uint32_t n_local = atomicExch(counts + 0, 0u), n_host = atomicExch(counts + 1, 0u);
+      atomicExch(counts + 2, 0u);
+      if (host_mirror) {
+        host_mirror[1 + UGK_LOC_LOCAL] = n_local;
+        host_mirror[1 + UGK_LOC_HOST] = n_host;
       }
     }
   }
@@ -268,12 +300,12 @@ int classify(ugk_table_t t, const K *keys, size_t n, uint64_t host_rows, const u
 template <typename K, int KIND>
 int extract_mix_lpr(ugk_table_t t, const K *keys, size_t n, const void *cache, uint64_t cache_rows, const void *host,
                     uint64_t host_rows, void *out, uint32_t vpr, uint32_t *status, uint32_t *host_mirror,
-                    hipStream_t st) {
+                    uint32_t *counts, hipStream_t st) {
   const unsigned grid = clamp_grid((n + kBlock - 1) / kBlock, 0);
 #define UGK_GO(L)                                                                                                 \
   hipLaunchKernelGGL((extract_mix_kernel<K, KIND, L>), dim3(grid), dim3(kBlock), 0, st, t, keys, n,               \
                      (const u32x4 *)cache, cache_rows, (const u32x4 *)host, host_rows, (u32x4 *)out, vpr, status, \
-                     host_mirror)
+                     host_mirror, counts)
   if (vpr <= 1) UGK_GO(1);
   else if (vpr <= 2) UGK_GO(2);
   else if (vpr <= 4) UGK_GO(4);
@@ -289,7 +321,7 @@ int extract_mix_lpr(ugk_table_t t, const K *keys, size_t n, const void *cache, u
 template <typename K>
 int extract_mix(ugk_table_t t, const K *keys, size_t n, const void *cache, uint64_t cache_rows, const void *host,
                 uint64_t host_rows, void *out, size_t row_bytes, uint32_t *status, uint32_t *host_mirror,
-                void *stream) {
+                uint32_t *counts, void *stream) {
   if (n == 0) return 0;
   UGK_REQUIRE(keys && out && status, "ugk_extract_mix: null keys, output or status");
   UGK_REQUIRE(t.kind == 1 || t.kind == 2, "ugk_extract_mix: table kind %d is not flat(1) or hash(2)", t.kind);
@@ -306,9 +338,9 @@ int extract_mix(ugk_table_t t, const K *keys, size_t n, const void *cache, uint6
   const uint32_t vpr = (uint32_t)(row_bytes / 16);
   if (t.kind == 1)
     return extract_mix_lpr<K, 1>(t, keys, n, cache, cache_rows, host, host_rows, out, vpr, status, host_mirror,
-                                 as_stream(stream));
+                                 counts, as_stream(stream));
   return extract_mix_lpr<K, 2>(t, keys, n, cache, cache_rows, host, host_rows, out, vpr, status, host_mirror,
-                               as_stream(stream));
+                               counts, as_stream(stream));
 }
 
 template <typename K>
@@ -354,15 +386,15 @@ int ugk_classify_i64(ugk_table_t t, const int64_t *keys_dev, size_t n, uint64_t 
 
 int ugk_extract_mix_u32(ugk_table_t t, const uint32_t *keys_dev, size_t n, const void *cache_dev, uint64_t cache_rows,
                         const void *host_dev, uint64_t host_rows, void *out_dev, size_t row_bytes,
-                        uint32_t *status_dev, uint32_t *host_mirror, void *stream) {
+                        uint32_t *status_dev, uint32_t *host_mirror, uint32_t *counts_dev, void *stream) {
   return extract_mix<uint32_t>(t, keys_dev, n, cache_dev, cache_rows, host_dev, host_rows, out_dev, row_bytes,
-                               status_dev, host_mirror, stream);
+                               status_dev, host_mirror, counts_dev, stream);
 }
 int ugk_extract_mix_i64(ugk_table_t t, const int64_t *keys_dev, size_t n, const void *cache_dev, uint64_t cache_rows,
                         const void *host_dev, uint64_t host_rows, void *out_dev, size_t row_bytes,
-                        uint32_t *status_dev, uint32_t *host_mirror, void *stream) {
+                        uint32_t *status_dev, uint32_t *host_mirror, uint32_t *counts_dev, void *stream) {
   return extract_mix<int64_t>(t, keys_dev, n, cache_dev, cache_rows, host_dev, host_rows, out_dev, row_bytes,
-                              status_dev, host_mirror, stream);
+                              status_dev, host_mirror, counts_dev, stream);
 }
 
 size_t ugk_dedup_workspace_bytes(size_t n) { return dedup_capacity(n) * 8 + ((n + 1) / 2 * 2) * 4 + 64; }

@@ -86,8 +86,8 @@ SIGNATURES = {
     "ugk_hash_census": [_vp, _sz, _vp, _vp],
     "ugk_classify_u32": [Table, _vp, _sz, _u64, _vp, _vp, _vp, _vp, _vp, _vp, _vp],
     "ugk_classify_i64": [Table, _vp, _sz, _u64, _vp, _vp, _vp, _vp, _vp, _vp, _vp],
-    "ugk_extract_mix_u32": [Table, _vp, _sz, _vp, _u64, _vp, _u64, _vp, _sz, _vp, _vp, _vp],
-    "ugk_extract_mix_i64": [Table, _vp, _sz, _vp, _u64, _vp, _u64, _vp, _sz, _vp, _vp, _vp],
+    "ugk_extract_mix_u32": [Table, _vp, _sz, _vp, _u64, _vp, _u64, _vp, _sz, _vp, _vp, _vp, _vp],
+    "ugk_extract_mix_i64": [Table, _vp, _sz, _vp, _u64, _vp, _u64, _vp, _sz, _vp, _vp, _vp, _vp],
     "ugk_dedup_workspace_bytes": [_sz],
     "ugk_dedup_u32": [_vp, _sz, _vp, _u32, _vp, _vp, _vp, _vp, _vp, _vp],
     "ugk_dedup_i64": [_vp, _sz, _vp, _u32, _vp, _vp, _vp, _vp, _vp, _vp],
