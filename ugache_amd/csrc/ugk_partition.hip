@@ -167,24 +167,28 @@ __global__ __launch_bounds__(kBlock) void extract_mix_kernel(ugk_table_t t, cons
     }
   }
   if (counts == nullptr) return;
-  // group sizes for the host: per workgroup one atomic per source, and the workgroup that finishes last (ticket
-  // counter) hands the totals to the pinned mirror and leaves the three device words at zero for the next launch
+  // Group sizes for the host.  Every workgroup adds its two sums with ONE 64-bit atomic and then takes a ticket; the
+  // workgroup that draws the last ticket hands the totals to the pinned mirror and leaves the words at zero for the
+  // next launch.  No memory fence anywhere: a device-scope fence per workgroup would write back and invalidate the
+  // L2 of its XCD thousands of times per launch.  Atomics are performed at the point of coherence, and the ticket is
+  // made to depend on the value the first atomic returned, so it cannot be issued before that atomic has been
+  // performed.
   if (lane == 0) {
     if (wave_local) atomicAdd(&block_tot[0], wave_local);
     if (wave_host) atomicAdd(&block_tot[1], wave_host);
   }
   __syncthreads();
   if (threadIdx.x == 0) {
-    if (block_tot[0]) atomicAdd(counts + 0, block_tot[0]);
-    if (block_tot[1]) atomicAdd(counts + 1, block_tot[1]);
-    __threadfence();
-    if (atomicAdd(counts + 2, 1u) == gridDim.x - 1) {
-      __threadfence();
-      const uint32_t n_local = atomicExch(counts + 0, 0u), n_host = atomicExch(counts + 1, 0u);
+    unsigned long long *pair = reinterpret_cast<unsigned long long *>(counts);  // low word local, high word host
+    const unsigned long long mine = ((unsigned long long)block_tot[1] << 32) | block_tot[0];
+    const unsigned long long before = atomicAdd(pair, mine);
+    const uint32_t never = before == ~0ull ? 1u : 0u;  // always 0 (the sums stay below 2^32); carries the dependency
+    if (atomicAdd(counts + 2, 1u + never) == gridDim.x - 1) {
+      const unsigned long long total = atomicExch(pair, 0ull);
       atomicExch(counts + 2, 0u);
       if (host_mirror) {
-        host_mirror[1 + UGK_LOC_LOCAL] = n_local;
-        host_mirror[1 + UGK_LOC_HOST] = n_host;
+        host_mirror[1 + UGK_LOC_LOCAL] = (uint32_t)total;
+        host_mirror[1 + UGK_LOC_HOST] = (uint32_t)(total >> 32);
       }
     }
   }
@@ -324,6 +328,7 @@ int extract_mix(ugk_table_t t, const K *keys, size_t n, const void *cache, uint6
                 uint32_t *counts, void *stream) {
   if (n == 0) return 0;
   UGK_REQUIRE(keys && out && status, "ugk_extract_mix: null keys, output or status");
+  UGK_REQUIRE((uintptr_t)counts % 8 == 0, "ugk_extract_mix: the count words must be 8-byte aligned");
   UGK_REQUIRE(t.kind == 1 || t.kind == 2, "ugk_extract_mix: table kind %d is not flat(1) or hash(2)", t.kind);
   UGK_REQUIRE(t.table && t.size, "ugk_extract_mix: empty table");
   if (t.kind == 2)
