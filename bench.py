@@ -63,6 +63,10 @@ MIXED = {
     "small_mixed_4Mx128xfp32_262144_i64_zipf0.9_cache25pct": dict(rows=4_000_000, dim=128, dtype="float32",
                                                                   n_keys=262_144, zipf=0.9, pct=0.25, fields=1,
                                                                   presample=20),
+    # nearly every key hits, through the table: the HBM side of the mixed-source kernels on its own
+    "c2_table_10Mx128xfp32_262144_i64_zipf0.5_cache99pct": dict(rows=10_000_000, dim=128, dtype="float32",
+                                                                n_keys=262_144, zipf=0.5, pct=0.99, fields=1,
+                                                                presample=60),
 }
 
 
