@@ -226,7 +226,7 @@ def run_all_hit(args):
         "gpu_over_cpu": keys_per_s / cpu_kps,
     }
     co.coll_torch_shutdown()
-    print(json.dumps(result))
+    emit(result)
 
 
 def zipf_ranks_gpu(torch, n, space, s, gen, dev):
@@ -435,11 +435,26 @@ def run_mixed(args):
         "setup_seconds": setup_s,
     }
     co.coll_torch_shutdown()
-    print(json.dumps(result))
+    emit(result)
+
+
+_REAL_STDOUT = None
+
+
+def emit(result):
+    """the one JSON line, on the real stdout"""
+    sys.stdout.flush()
+    os.write(_REAL_STDOUT if _REAL_STDOUT is not None else 1, (json.dumps(result) + "\n").encode())
 
 
 def main():
+    global _REAL_STDOUT
     args = parse_args()
+    # the library prints the reference's progress lines ("test_result:init:...", solver summary) on stdout; they go
+    # to stderr here so that stdout carries the result line only
+    sys.stdout.flush()
+    _REAL_STDOUT = os.dup(1)
+    os.dup2(2, 1)
     import torch
 
     if not torch.cuda.is_available():
