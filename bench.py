@@ -63,6 +63,9 @@ MIXED = {
     "small_mixed_4Mx128xfp32_262144_i64_zipf0.9_cache25pct": dict(rows=4_000_000, dim=128, dtype="float32",
                                                                   n_keys=262_144, zipf=0.9, pct=0.25, fields=1,
                                                                   presample=20),
+    # no cache at all: every row crosses the host link (where deduplication of a skewed batch pays)
+    "c1_nocache_1Mx128xfp32_65536_i64_zipf1.1": dict(rows=1_000_000, dim=128, dtype="float32", n_keys=65_536,
+                                                     zipf=1.1, pct=0.0, fields=1, presample=1),
     # nearly every key hits, through the table: the HBM side of the mixed-source kernels on its own
     "c2_table_10Mx128xfp32_262144_i64_zipf0.5_cache99pct": dict(rows=10_000_000, dim=128, dtype="float32",
                                                                 n_keys=262_144, zipf=0.5, pct=0.99, fields=1,
