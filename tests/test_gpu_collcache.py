@@ -181,6 +181,35 @@ def test_dedup_in_front_of_the_extraction(pct, table_kind, kdtype, monkeypatch):
         assert _basics.last_group_offset(0) == want
 
 
+@pytest.mark.parametrize("impl", ["", "SMMaskPhase", "NONE"])
+@pytest.mark.parametrize("table_kind", ["FLAT", "HASH"])
+def test_committed_golden_case_end_to_end(impl, table_kind, monkeypatch):
+    """tests/golden/extract_small.json (written by brute-force Python, tests/golden/make_fixtures.py): record the
+    stream, build, look the keys up — cached set, capacity, group sizes and every output byte as in the file"""
+    import json
+    monkeypatch.setenv("COLL_HASH_TABLE", table_kind)
+    if impl:
+        monkeypatch.setenv("SAMGRAPH_COLL_CACHE_CONCURRENT_LINK_IMPL", impl)
+    with open(os.path.join(ROOT, "tests", "golden", "extract_small.json")) as f:
+        g = json.load(f)
+    n_item, rb, pct = g["n_item"], g["row_bytes"], g["cache_percentage"]
+    co.config(make_config(n_item, pct))
+    co.coll_cache_record_init(0)
+    co.coll_torch_record(0, torch.tensor(g["record_stream"], dtype=torch.int32))
+    emb = co.coll_torch_create_emb_shm(0, n_item, rb // 4, torch.float32)
+    emb.numpy().view(np.uint8)[...] = np.array(g["table"], np.uint8)
+    co.coll_torch_init_t(0, 0, emb, pct)
+    info = _basics.info(0)
+    assert info["capacity_rows"] == g["capacity_rows"] and info["cached_rows"] == len(g["cached_keys"])
+    got = np.zeros(len(g["cached_keys"]), np.uint32)
+    assert _basics.C_LIB_CTYPES.coll_cache_get_cached_keys(0, got.ctypes.data, len(got)) == len(got)
+    assert got.tolist() == g["cached_keys"]
+    for kdtype in (torch.int32, torch.int64):
+        out = co.coll_torch_lookup_key_t_val_ret(0, torch.tensor(g["lookup_keys"], dtype=kdtype).cuda(), False)
+        assert out.cpu().numpy().view(np.uint8).tolist() == g["expected_output"]
+        assert _basics.last_group_offset(0) == g["expected_group_offset"]
+
+
 def test_fp16_table_and_small_rows():
     rng = np.random.default_rng(9)
     n_item, dim, pct = 30_000, 64, 0.2

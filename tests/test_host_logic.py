@@ -210,3 +210,22 @@ def test_step_report_has_the_layout_the_eval_scripts_scrape(capfd):
     # the three header lines and every level's line count (7 + 3 + 8)
     assert out.count("Profiler Level") == 3 and out.count("\n        L1  ") == 7
     assert out.count("\n        L2  ") == 3 and out.count("\n        L3  ") == 8
+
+
+def test_recorder_and_placement_reproduce_the_committed_golden_case():
+    import json
+    with open(os.path.join(ROOT, "tests", "golden", "extract_small.json")) as f:
+        g = json.load(f)
+    n_item, pct = g["n_item"], g["cache_percentage"]
+    _config(n_item, pct)
+    cc._basics.coll_cache_record_init(0)
+    stream = np.array(g["record_stream"], np.uint32)
+    C.coll_cache_record(0, stream.ctypes.data, len(stream))
+    got = np.full(n_item, 9, np.uint32)
+    assert C.coll_cache_place_recorded(0, n_item, pct, got.ctypes.data) == len(g["cached_keys"])
+    assert np.nonzero(got == 0)[0].tolist() == g["cached_keys"]
+    C.coll_cache_record(0, stream.ctypes.data, len(stream))
+    k = np.zeros(n_item, np.uint32)
+    c = np.zeros(n_item, np.uint32)
+    m = C.coll_cache_rank_hotness(0, k.ctypes.data, c.ctypes.data, n_item)
+    assert k[:m].tolist() == g["rank_keys_observed"] and c[:m].tolist() == g["rank_counts_observed"]

@@ -398,3 +398,24 @@ def test_dedup_matches_numpy_unique():
         nu, first = np.unique(keys, return_index=True)
         assert np.array_equal(np.sort(uniq), nu)
         assert np.array_equal(uniq, keys[np.sort(first)])  # first-occurrence order
+
+
+def test_oracle_reproduces_the_committed_golden_case():
+    """tests/golden/extract_small.json was written by brute-force Python loops (tests/golden/make_fixtures.py), not
+    by the oracle: ranking, placement, capacity and the gather must all land on it"""
+    import json
+    import os
+    with open(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "extract_small.json")) as f:
+        g = json.load(f)
+    n_item, pct = g["n_item"], g["cache_percentage"]
+    stream = np.array(g["record_stream"], np.uint32)
+    rk, rc = ORC.freq_rank(stream)
+    assert rk.tolist() == g["rank_keys_observed"] and rc.tolist() == g["rank_counts_observed"]
+    full_k, _ = ORC.full_rank(stream, n_item)
+    nid, n_cached = ORC.rep_solve(full_k, n_item, pct * 100)
+    assert np.nonzero(nid == 0)[0].tolist() == g["cached_keys"] and n_cached == len(g["cached_keys"])
+    assert ORC.lib.orc_cache_capacity(n_item, pct) == g["capacity_rows"]
+    table = np.array(g["table"], np.uint8)
+    keys = np.array(g["lookup_keys"], np.int64)
+    assert ORC.gather(table, keys).tolist() == g["expected_output"]
+    assert [0, int((nid[keys] == 0).sum()), len(keys)] == g["expected_group_offset"]
