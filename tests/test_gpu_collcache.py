@@ -227,6 +227,27 @@ def test_fp16_table_and_small_rows():
     assert out[:10_001].cpu().numpy().tobytes() == ORC.gather(table, q.astype(np.int64)).tobytes()
 
 
+@pytest.mark.parametrize("dim,dtype", [(3, torch.float32), (5, torch.float16), (1, torch.float32), (7, torch.float32)])
+@pytest.mark.parametrize("pct", [0.2, 1.0, 0.0])
+def test_rows_that_are_not_multiples_of_16_bytes(dim, dtype, pct):
+    """12-, 10-, 4- and 28-byte rows: the 16-byte-lane kernels do not apply, narrower lanes take over"""
+    rng = np.random.default_rng(dim)
+    n_item = 9_000
+    if dtype == torch.float16 and dim % 2:
+        pytest.skip("fp16 rows travel as dim/2 fp32 words (operation.cc:132-136): the dimension must be even")
+    co.config(make_config(n_item, pct))
+    co.coll_cache_record_init(0)
+    co.coll_torch_record(0, torch.from_numpy(rng.integers(0, n_item, size=40_000)).to(torch.int32))
+    emb = co.coll_torch_create_emb_shm(0, n_item, dim, dtype)
+    table = fill_table(emb, rng)
+    co.coll_torch_init_t(0, 0, emb, pct)
+    for n in (1, 4097):
+        q = rng.integers(0, n_item, size=n)
+        out = co.coll_torch_lookup_key_t_val_ret(0, torch.from_numpy(q).cuda(), False)
+        assert out.shape == (n, dim)
+        assert out.cpu().numpy().tobytes() == ORC.gather(table, q.astype(np.int64)).tobytes()
+
+
 def test_create_emb_from_file(tmp_path):
     rng = np.random.default_rng(2)
     arr = rng.standard_normal((1000, 32)).astype(np.float32)

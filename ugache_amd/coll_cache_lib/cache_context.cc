@@ -503,7 +503,10 @@ void ExtractSession::ExtractFeatImpl(const KeyT *nodes, size_t num_nodes, void *
   const uint64_t cache_rows = ctx->_cache_space_capacity;
   const uint64_t host_rows = ctx->_num_total_nodes;
 
-  if (RunConfig::concurrent_link_impl == kDirectNoGroup && dst_map == nullptr) {
+  // the fused kernel moves 16-byte vectors; rows or buffers that are not multiples of 16 bytes take the factored
+  // path, whose gathers fall back to narrower lanes
+  const bool vec16 = (((uintptr_t)cache | (uintptr_t)host | (uintptr_t)output | (uintptr_t)rb) & 15u) == 0;
+  if (RunConfig::concurrent_link_impl == kDirectNoGroup && dst_map == nullptr && vec16) {
     // one fused lookup + gather kernel, source chosen per row (cache_context.cu:1295-1329).  The default here: the
     // host link is busy from the first wavefront on, with no classify pass and no cross-stream hand-off in front of
     // it, and since the link bounds a mixed batch it does not matter that host loads spread over the chip slow the
@@ -543,7 +546,7 @@ void ExtractSession::ExtractFeatImpl(const KeyT *nodes, size_t num_nodes, void *
   UGK_CALL(ugk_event_record(_ev_classified, stream));
   // the classify kernel is short and latency-bound: the counting starts behind it, beside the gathers
   RecordKeys(input_nodes, num_input, stream, _ev_classified);
-  if (RunConfig::concurrent_link_impl == kSMMaskPhase) {
+  if (RunConfig::concurrent_link_impl != kNoConcurrentLink) {
     // factored extraction: two concurrent kernels that read their group bounds from the device-side counters.
     // A long host-link gather runs on the stream confined to a few CUs, so its slow loads do not clog the memory
     // pipelines the HBM gather needs; the HBM gather then stays on the caller's stream.  A short host-link gather
@@ -593,7 +596,7 @@ void ExtractSession::ExtractFeatImpl(const KeyT *nodes, size_t num_nodes, void *
   float ms_idx = 0, ms_miss = 0, ms_local = 0;
   UGK_CALL(ugk_event_elapsed_ms(_ev_t[0], _ev_classified, &ms_idx));
   UGK_CALL(ugk_event_elapsed_ms(_ev_classified, _ev_cpu_done, &ms_miss));
-  if (RunConfig::concurrent_link_impl == kSMMaskPhase) {
+  if (RunConfig::concurrent_link_impl != kNoConcurrentLink) {
     UGK_CALL(ugk_event_elapsed_ms(_ev_classified, _ev_local_done, &ms_local));
     _host_on_main = ms_miss < 0.25f;  // placement of the next batch's host-link gather
   } else {
