@@ -75,6 +75,19 @@ void coll_cache_init_ranked_c(int replica_id, size_t key_space_size, const uint3
  * (coll_cache_lib/constant.h:28). */
 void coll_cache_lookup_i64(int replica_id, const int64_t *key, size_t num_keys, void *output, StreamHandle stream);
 void coll_cache_record_i64(int replica_id, const int64_t *key, size_t num_keys);
+/* Stream-ordered lookups (extension; the reference's lookup always blocks, facade.cc:74-88 and the synchronisations
+ * of cache_context.cu:1199-1794).  coll_cache_lookup_async* enqueue the batch on `stream` and return: `output` is
+ * complete for anything enqueued on the same stream afterwards, which is all a framework op needs; about 10 us of
+ * blocking round trip per batch disappear.  `key` and `output` must stay valid until the work has run.  All
+ * stream-ordered lookups of a replica, and its refreshes, must use one stream.  coll_cache_lookup_wait blocks until
+ * everything enqueued so far has finished, aborts if a key was outside its table, and makes
+ * coll_cache_last_group_offset describe the last batch; any blocking lookup does the same first.  No per-step profiler
+ * values are logged for stream-ordered batches.  Batches the one-kernel paths cannot take (COLL_DEDUP_KEYS, a factored
+ * SAMGRAPH_COLL_CACHE_CONCURRENT_LINK_IMPL, rows not multiples of 16 bytes with a partial cache) block as usual. */
+void coll_cache_lookup_async(int replica_id, const uint32_t *key, size_t num_keys, void *output, StreamHandle stream);
+void coll_cache_lookup_async_i64(int replica_id, const int64_t *key, size_t num_keys, void *output,
+                                 StreamHandle stream);
+void coll_cache_lookup_wait(int replica_id, StreamHandle stream);
 /* Sparse-id mode (extension; call after coll_cache_config and before recording or building): the caller's id of
  * host row r is (r * mul) mod 2^bits with mul odd, so 64-bit hashed ids from a 2^bits space address a dense host table
  * of num_total_item rows.  Cached ids live in the open-addressing GPU table; a missed id is turned back into its row

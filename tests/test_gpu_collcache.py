@@ -449,6 +449,68 @@ def test_serving_loop_records_a_prefix_and_refreshes_in_the_background(gpu_recor
     co.coll_torch_forward_config(False, 0, frac, False)
 
 
+@pytest.mark.parametrize("pct,table_kind", [(1.0, "FLAT"), (0.0, "FLAT"), (0.25, "FLAT"), (0.25, "HASH")])
+@pytest.mark.parametrize("kdtype", [torch.int32, torch.int64])
+def test_stream_ordered_lookups(pct, table_kind, kdtype, monkeypatch):
+    """coll_cache_lookup_async: batches are enqueued without waiting; what is enqueued behind them on the same stream
+    (here: a clone of the reused output buffer) sees their rows; wait() collects status and group sizes; a refresh in
+    between keeps everything exact."""
+    monkeypatch.setenv("COLL_HASH_TABLE", table_kind)
+    monkeypatch.setenv("COLL_REFRESH_SLEEP_US", "100")
+    rng = np.random.default_rng(77)
+    n_item, dim = 40_000, 128
+    co.config(make_config(n_item, pct))
+    co.coll_cache_record_init(0)
+    perm = rng.permutation(n_item)
+    s1 = perm[zipf_ranks(rng, 100_000, n_item, 1.1)]
+    partial = 0.0 < pct < 1.0
+    if partial:
+        co.coll_torch_record(0, torch.from_numpy(s1).to(kdtype))
+    emb = co.coll_torch_create_emb_shm(0, n_item, dim, torch.float32)
+    table = fill_table(emb, rng)
+    co.coll_torch_init_t(0, 0, emb, pct)
+    _, nid = expected_cached_set(s1.astype(np.uint32), n_item, pct) if partial else (None, None)
+
+    def burst(nid):
+        keep, clones, batches = [], [], []
+        for n in (30_000, 1, 4096, 30_000, 12_345):
+            keys = perm[zipf_ranks(rng, n, n_item, 1.1)]
+            kt = torch.from_numpy(keys).to(kdtype).cuda()
+            keep.append(kt)  # the keys must outlive the enqueued work
+            out = co.coll_torch_lookup_async(0, kt, False)
+            clones.append(out.clone())  # enqueued behind the lookup on the same stream
+            batches.append(keys)
+        co.coll_torch_lookup_wait(0)
+        for keys, c in zip(batches, clones):
+            assert c.cpu().numpy().tobytes() == ORC.gather(table, keys.astype(np.int64)).tobytes()
+        n = len(batches[-1])
+        n_local = n if pct == 1.0 else 0 if pct == 0.0 else int((nid[batches[-1]] == 0).sum())
+        assert _basics.last_group_offset(0) == [0, n_local, n]
+
+    burst(nid)
+    assert _basics.info(0)["lookups"] == 5
+    if partial:
+        perm2 = rng.permutation(n_item)
+        s2 = perm2[zipf_ranks(rng, 100_000, n_item, 1.1)]
+        co.coll_torch_record(0, torch.from_numpy(s2).to(kdtype))
+        # enqueue a batch, then refresh in the background without waiting for it first
+        keys = perm[zipf_ranks(rng, 20_000, n_item, 1.1)]
+        kt = torch.from_numpy(keys).to(kdtype).cuda()
+        pre = co.coll_torch_lookup_async(0, kt, False).clone()
+        t = threading.Thread(target=co.coll_torch_refresh, args=(0, False))
+        t.start()
+        t.join()
+        assert pre.cpu().numpy().tobytes() == ORC.gather(table, keys.astype(np.int64)).tobytes()
+        _, nid2 = expected_cached_set(s2.astype(np.uint32), n_item, pct)
+        burst(nid2)
+    # a blocking lookup settles what is in flight first
+    keys = rng.integers(0, n_item, size=1000)
+    kt = torch.from_numpy(keys).to(kdtype).cuda()
+    a = co.coll_torch_lookup_async(0, kt, False).clone()
+    b = co.coll_torch_lookup_key_t_val_ret(0, kt, False)
+    assert a.cpu().numpy().tobytes() == b.cpu().numpy().tobytes() == ORC.gather(table, keys.astype(np.int64)).tobytes()
+
+
 def test_reference_cpu_runnable_config_full_size():
     """1M x 128 fp32 host table, 65536 int64 keys Zipf(1.1) over a seeded permutation, hottest 10 % cached."""
     rng = np.random.default_rng(1)

@@ -48,6 +48,26 @@ def test_key_out_of_range_aborts_with_a_message_instead_of_faulting(pct):
     assert "extraction kernels reported status" in p.stderr and "outside the table" in p.stderr
 
 
+@pytest.mark.parametrize("pct", [1.0, 0.3])
+def test_stream_ordered_lookup_reports_a_bad_key_at_the_wait(pct):
+    p = run("""
+        n = 5000
+        co.config(cfg(n, %r)); co.coll_cache_record_init(0)
+        co.coll_torch_record(0, torch.arange(0, n, 3, dtype=torch.int32))
+        emb = co.coll_torch_create_emb_shm(0, n, 32, torch.float32); emb.normal_()
+        co.coll_torch_init_t(0, 0, emb, %r)
+        bad = torch.tensor([1, 2, n + 7, 3], dtype=torch.int64, device="cuda")
+        co.coll_torch_lookup_async(0, bad, False)
+        torch.cuda.synchronize()
+        print("enqueue returned", flush=True)
+        co.coll_torch_lookup_wait(0)
+        print("survived")
+    """ % (pct, pct))
+    assert "enqueue returned" in p.stdout and "survived" not in p.stdout
+    assert p.returncode == -6, p.stderr[-2000:]
+    assert "extraction kernels reported status" in p.stderr
+
+
 def test_ordinary_host_memory_is_refused_for_a_partial_cache():
     p = run("""
         n = 1000

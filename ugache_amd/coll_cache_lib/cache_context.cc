@@ -432,6 +432,7 @@ void ExtractSession::ExtractFeatImpl(const KeyT *nodes, size_t num_nodes, void *
   auto profiler = ctx->_coll_cache ? ctx->_coll_cache->_profiler : nullptr;
   const size_t rb = ctx->_row_bytes;
   const size_t nbytes = num_nodes * rb;
+  Wait(stream);  // stream-ordered lookups still in flight share the mirror words this call reads
   _group_offset[0] = 0;
   if (num_nodes == 0) {
     _group_offset[1] = _group_offset[2] = 0;
@@ -616,6 +617,69 @@ void ExtractSession::ExtractFeatImpl(const KeyT *nodes, size_t num_nodes, void *
   ctx->progress.fetch_add(1);
 }
 
+template <typename KeyT>
+void ExtractSession::ExtractFeatAsyncImpl(const KeyT *nodes, size_t num_nodes, void *output, StreamHandle stream) {
+  CacheContext *ctx = _cache_ctx.get();
+  const size_t rb = ctx->_row_bytes;
+  if (num_nodes == 0) return;
+  CHECK_NOTNULL(nodes);
+  CHECK_NOTNULL(output);
+  const bool dedup = RunConfig::dedup_keys && num_nodes >= RunConfig::dedup_min_keys;
+  if (ctx->IsDirectMapping() && !dedup) {
+    const bool from_host = ctx->_cpu_location_id != -1;
+    RecordKeys(nodes, num_nodes, stream, nullptr);
+    UGK_CALL(GatherDirect(ctx->_device_cache_data[0], ctx->_num_total_nodes, nodes, num_nodes, output, rb,
+                          from_host ? _cpu_blocks : 0, _status, _host_mirror, stream));
+    JoinRecord(stream);
+    // what a blocking lookup would have read from the mirror
+    _host_mirror[kMirGroupSizes + UGK_LOC_LOCAL] = from_host ? 0 : (uint32_t)num_nodes;
+    _host_mirror[kMirGroupSizes + UGK_LOC_HOST] = from_host ? (uint32_t)num_nodes : 0;
+  } else if (!ctx->IsDirectMapping() && !dedup && RunConfig::concurrent_link_impl == kDirectNoGroup &&
+             (((uintptr_t)ctx->_device_cache_data[ctx->_local_location_id] |
+               (uintptr_t)ctx->_device_cache_data[ctx->_cpu_location_id] | (uintptr_t)output | (uintptr_t)rb) &
+              15u) == 0) {
+    RecordKeys(nodes, num_nodes, stream, nullptr);
+    UGK_CALL(ExtractMix(ctx->_new_hash_table->_table, nodes, num_nodes,
+                        ctx->_device_cache_data[ctx->_local_location_id], ctx->_cache_space_capacity,
+                        ctx->_device_cache_data[ctx->_cpu_location_id], ctx->_num_total_nodes, output, rb, _status,
+                        _host_mirror, _state + kStMixCounts, stream));
+    JoinRecord(stream);
+  } else {
+    Wait(stream);
+    ExtractFeatImpl<KeyT>(nodes, num_nodes, output, stream, 0xffffffffffffffffull);
+    return;
+  }
+  _async_used.store(true);
+  _async_pending++;
+  _async_last_nodes = num_nodes;
+}
+
+void ExtractSession::ExtractFeatAsync(const IdType *nodes, const size_t num_nodes, void *output,
+                                      StreamHandle stream) {
+  CHECK(RunConfig::key_map_mul == 0 || RunConfig::key_map_mask <= 0xffffffffull)
+      << "sparse ids wider than 32 bits need the 64-bit lookup";
+  ExtractFeatAsyncImpl<IdType>(nodes, num_nodes, output, stream);
+}
+
+void ExtractSession::ExtractFeatAsync64(const Id64Type *nodes, const size_t num_nodes, void *output,
+                                        StreamHandle stream) {
+  ExtractFeatAsyncImpl<Id64Type>(nodes, num_nodes, output, stream);
+}
+
+void ExtractSession::Wait(StreamHandle stream) {
+  if (_async_pending == 0) return;
+  UGK_CALL(ugk_stream_sync(stream));
+  CheckStatusWord(stream);
+  const uint32_t n_local = _host_mirror[kMirGroupSizes + UGK_LOC_LOCAL],
+                 n_miss = _host_mirror[kMirGroupSizes + UGK_LOC_HOST];
+  CHECK_EQ((size_t)n_local + n_miss, _async_last_nodes);
+  _group_offset[0] = 0;
+  _group_offset[1] = n_local;
+  _group_offset[2] = (uint32_t)_async_last_nodes;
+  _cache_ctx->progress.fetch_add(_async_pending);
+  _async_pending = 0;
+}
+
 void ExtractSession::ExtractFeat(const IdType *nodes, const size_t num_nodes, void *output, StreamHandle stream,
                                  uint64_t task_key) {
   CHECK(RunConfig::key_map_mul == 0 || RunConfig::key_map_mask <= 0xffffffffull)
@@ -728,12 +792,17 @@ void RefreshSession::refresh_after_solve_new(bool foreground) {
 
   evict_s = t_phase.Passed();
   t_phase.Reset();
-  // Step 5: let one more lookup finish, so that no gather in flight still reads a slot about to be reused
+  // Step 5: let one more lookup finish, so that no gather in flight still reads a slot about to be reused.  With
+  // stream-ordered lookups "finished" is a matter of the stream: everything enqueued before this point still saw
+  // the old table, everything after it sees the evicted keys as misses.
   const size_t current_progress = ctx->progress.load();
+  auto session = coll_cache->session(ctx->_local_location_id);
+  const bool stream_ordered = session && session->UsesStreamOrder();
+  if (stream_ordered) UGK_CALL(ugk_stream_sync(stream));
   AnonymousBarrier::_refresh_instance->Wait();
   {
     Timer t0;
-    while (!foreground && ctx->progress.load() < current_progress + 1) {
+    while (!foreground && !stream_ordered && ctx->progress.load() < current_progress + 1) {
       if (t0.PassedSec() >= 20) break;
       usleep(50);
     }

@@ -133,6 +133,12 @@ class ExtractSession {
   template <typename KeyT>
   void RecordKeys(const KeyT *nodes, size_t num_nodes, StreamHandle stream, void *after);
 
+  size_t _async_pending = 0;       // stream-ordered lookups enqueued since the last Wait()
+  size_t _async_last_nodes = 0;    // size of the last of them
+  std::atomic<bool> _async_used{false};
+  template <typename KeyT>
+  void ExtractFeatAsyncImpl(const KeyT *nodes, size_t num_nodes, void *output, StreamHandle stream);
+
   template <typename KeyT>
   void ExtractFeatImpl(const KeyT *nodes, size_t num_nodes, void *output, StreamHandle stream, uint64_t task_key);
   void EnsureIdx(size_t num_nodes);
@@ -147,6 +153,18 @@ class ExtractSession {
   // same for 64-bit keys (dense ids below num_total_item); an extension over the reference
   void ExtractFeat64(const Id64Type *nodes, const size_t num_nodes, void *output, StreamHandle stream,
                      uint64_t task_key);
+  // Stream-ordered variants (an extension; the reference's lookup always blocks): the kernels of the batch are
+  // enqueued on `stream` and the call returns without waiting; `output` is complete for whatever is enqueued on the
+  // same stream afterwards.  All stream-ordered lookups of a session must use one stream.  Error flags, group sizes
+  // and profiler values are collected by Wait().  Batches the fused / direct kernels cannot take (deduplication on,
+  // rows not multiples of 16 bytes, a factored mode selected) run through the blocking path instead.
+  void ExtractFeatAsync(const IdType *nodes, const size_t num_nodes, void *output, StreamHandle stream);
+  void ExtractFeatAsync64(const Id64Type *nodes, const size_t num_nodes, void *output, StreamHandle stream);
+  // blocks until every stream-ordered lookup enqueued so far has finished, aborts if one of them met a key outside
+  // its table, and makes LastGroupOffset() describe the last of them
+  void Wait(StreamHandle stream);
+  // true once a stream-ordered lookup was enqueued: a refresh then waits for the stream instead of for `progress`
+  bool UsesStreamOrder() const { return _async_used.load(); }
   // {0, #local, n} of the last lookup — the reference's group_offset (cache_context.cu:825-847)
   const uint32_t *LastGroupOffset() const { return _group_offset; }
   // moves what the lookups have counted on the device since the last call into `recorder` (FreqRecorder::Record's

@@ -87,6 +87,14 @@ class CollCache : public std::enable_shared_from_this<CollCache> {
     return n;
   }
   std::shared_ptr<CacheContext> cache_ctx(int replica_id) { return _cache_ctx_list.at(replica_id); }
+  // stream-ordered lookups (ExtractSession::ExtractFeatAsync / Wait); an extension over the reference
+  void lookup_async(int replica_id, const IdType *nodes, size_t num_nodes, void *output, StreamHandle stream) {
+    _session_list.at(replica_id)->ExtractFeatAsync(nodes, num_nodes, output, stream);
+  }
+  void lookup_async64(int replica_id, const Id64Type *nodes, size_t num_nodes, void *output, StreamHandle stream) {
+    _session_list.at(replica_id)->ExtractFeatAsync64(nodes, num_nodes, output, stream);
+  }
+  void lookup_wait(int replica_id, StreamHandle stream) { _session_list.at(replica_id)->Wait(stream); }
   std::shared_ptr<ExtractSession> session(int replica_id) { return _session_list.at(replica_id); }
   TensorPtr nid_to_block() { return _nid_to_block; }
 };

@@ -215,6 +215,25 @@ void coll_cache_lookup_i64(int replica_id, const int64_t *key, size_t num_keys, 
   _coll_cache->lookup64(replica_id, key, num_keys, output, stream, step_key);
 }
 
+void coll_cache_lookup_async(int replica_id, const uint32_t *key, size_t num_keys, void *output,
+                             StreamHandle stream) {
+  CHECK_NOTNULL(_coll_cache);
+  steps[replica_id]++;
+  _coll_cache->lookup_async(replica_id, key, num_keys, output, stream);
+}
+
+void coll_cache_lookup_async_i64(int replica_id, const int64_t *key, size_t num_keys, void *output,
+                                 StreamHandle stream) {
+  CHECK_NOTNULL(_coll_cache);
+  steps[replica_id]++;
+  _coll_cache->lookup_async64(replica_id, key, num_keys, output, stream);
+}
+
+void coll_cache_lookup_wait(int replica_id, StreamHandle stream) {
+  CHECK_NOTNULL(_coll_cache);
+  _coll_cache->lookup_wait(replica_id, stream);
+}
+
 void coll_cache_record(int replica_id, uint32_t *key, size_t num_keys) {
   CHECK_LT((size_t)replica_id, _freq_recorder.size()) << "coll_cache_record_init was not called";
   _freq_recorder[replica_id]->Record(key, num_keys);

@@ -132,6 +132,20 @@ def coll_torch_lookup_key_t_val_ret(local_id, keys, pad_to_8=True):
     return _lookup_into_reused_buffer(local_id, keys, pad_to_8, _C.coll_cache_lookup, _C.coll_cache_lookup_i64)
 
 
+def coll_torch_lookup_async(local_id, keys, pad_to_8=True):
+    """stream-ordered form of coll_torch_lookup_key_t_val_ret: the batch is enqueued on torch's current stream and
+    the call returns without waiting, like any torch op; the returned view of the reused buffer is valid for work
+    enqueued on that stream afterwards.  `keys` must stay alive until the work has run (keep a reference, or call
+    coll_torch_lookup_wait)."""
+    return _lookup_into_reused_buffer(local_id, keys, pad_to_8, _C.coll_cache_lookup_async,
+                                      _C.coll_cache_lookup_async_i64)
+
+
+def coll_torch_lookup_wait(local_id):
+    """wait for the stream-ordered lookups enqueued so far; aborts if one of them met a key outside its table"""
+    _C.coll_cache_lookup_wait(local_id, _stream_handle(_State.dev_id.get(local_id, 0)))
+
+
 def coll_torch_forward_config(enable_refresh, refresh_iter, record_fraction=0.05, periodic=False):
     """the serving loop's settings (ps_config's coll_cache_enable_refresh / coll_cache_refresh_iter,
     python_tf2/collcache_tf2/collcache_tf2_cc/collcache_tf2_cc_infra/src/inference_utils.cpp:62-140)"""
