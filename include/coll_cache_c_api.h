@@ -82,7 +82,9 @@ void coll_cache_record_i64(int replica_id, const int64_t *key, size_t num_keys);
  * stream-ordered lookups of a replica, and its refreshes, must use one stream.  coll_cache_lookup_wait blocks until
  * everything enqueued so far has finished, aborts if a key was outside its table, and makes
  * coll_cache_last_group_offset describe the last batch; any blocking lookup does the same first.  No per-step profiler
- * values are logged for stream-ordered batches.  Batches the one-kernel paths cannot take (COLL_DEDUP_KEYS, a factored
+ * values are logged for stream-ordered batches.  Such a call is kernel launches only (no synchronisation, no
+ * allocation, no memset), so it may be recorded into a HIP graph by a caller that captures its stream.  Batches the
+ * one-kernel paths cannot take (COLL_DEDUP_KEYS, a factored
  * SAMGRAPH_COLL_CACHE_CONCURRENT_LINK_IMPL, rows not multiples of 16 bytes with a partial cache) block as usual. */
 void coll_cache_lookup_async(int replica_id, const uint32_t *key, size_t num_keys, void *output, StreamHandle stream);
 void coll_cache_lookup_async_i64(int replica_id, const int64_t *key, size_t num_keys, void *output,

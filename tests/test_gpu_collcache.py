@@ -511,6 +511,40 @@ def test_stream_ordered_lookups(pct, table_kind, kdtype, monkeypatch):
     assert a.cpu().numpy().tobytes() == b.cpu().numpy().tobytes() == ORC.gather(table, keys.astype(np.int64)).tobytes()
 
 
+@pytest.mark.parametrize("pct", [1.0, 0.25])
+def test_stream_ordered_lookup_inside_a_captured_graph(pct):
+    """a stream-ordered lookup is launches only (no synchronisation, no allocation, no memset node), so a caller can
+    capture it; every replay, with eager work and synchronisations in between, must give the eager result"""
+    rng = np.random.default_rng(5)
+    n_item, dim, n = 20_000, 64, 8_192
+    co.config(make_config(n_item, pct))
+    co.coll_cache_record_init(0)
+    if pct < 1.0:
+        co.coll_torch_record(0, torch.from_numpy(rng.integers(0, n_item, size=60_000)).to(torch.int32))
+    emb = co.coll_torch_create_emb_shm(0, n_item, dim, torch.float32)
+    table = fill_table(emb, rng)
+    co.coll_torch_init_t(0, 0, emb, pct)
+    keys = torch.zeros(n, dtype=torch.int64, device="cuda")
+    result = torch.zeros((n, dim), dtype=torch.float32, device="cuda")
+    # warm-up outside the capture: the reused output buffer gets allocated here
+    keys.copy_(torch.from_numpy(rng.integers(0, n_item, size=n)))
+    co.coll_torch_lookup_async(0, keys, False)
+    co.coll_torch_lookup_wait(0)
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g):
+        out = co.coll_torch_lookup_async(0, keys, False)
+        result.copy_(out)
+    for it in range(4):
+        q = rng.integers(0, n_item, size=n)
+        keys.copy_(torch.from_numpy(q))
+        g.replay()
+        torch.cuda.synchronize()
+        assert result.cpu().numpy().tobytes() == ORC.gather(table, q.astype(np.int64)).tobytes(), it
+        # eager work between the replays
+        eager = co.coll_torch_lookup_key_t_val_ret(0, keys, False)
+        assert eager.cpu().numpy().tobytes() == result.cpu().numpy().tobytes()
+
+
 def test_reference_cpu_runnable_config_full_size():
     """1M x 128 fp32 host table, 65536 int64 keys Zipf(1.1) over a seeded permutation, hottest 10 % cached."""
     rng = np.random.default_rng(1)
