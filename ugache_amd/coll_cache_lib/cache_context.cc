@@ -362,6 +362,7 @@ size_t ExtractSession::DrainHotness(FreqRecorder *recorder) {
   auto *host_list = _hot_entries_host->ptr<FreqEntry>();
   static_assert(sizeof(FreqEntry) == sizeof(uint64_t), "an entry is one (count << 32 | row) word");
   size_t moved = 0;
+  recorder->BeginEntries();
   for (size_t first = 0; first < rows; first += cap) {
     const size_t cur = std::min(cap, rows - first);  // as many rows as the list has room for: nothing is left over
     UGK_CALL(ugk_record_drain(_hot_counts->ptr<uint32_t>(), first, cur, dev_list, (uint32_t)cap, n_entries, host_out,

@@ -86,30 +86,47 @@ void FreqRecorder::Record(const KeyT *input, size_t num_inputs) {
     }
     __atomic_fetch_add(&cnt[k], 1u, __ATOMIC_RELAXED);
   }
+  if (num_inputs) _live_dirty = true;
   CHECK(!bad) << "FreqRecorder::Record: a key has no row among num_total_item=" << n_nodes;
 }
 template void FreqRecorder::Record<Id64Type>(const Id64Type *input, size_t num_inputs);
 template void FreqRecorder::Record<IdType>(const IdType *input, size_t num_inputs);
 
-void FreqRecorder::AddEntries(const FreqEntry *entries, size_t num_entries) {
-  std::lock_guard<std::mutex> g(_mu);
-  CntT *cnt = _live;
-  const size_t n_nodes = _num_nodes;
+void FreqRecorder::ScatterHandedOver(CntT *into) {
+  const size_t n = _handed_over.size(), n_nodes = _num_nodes;
+  const FreqEntry *e = _handed_over.data();
   bool bad = false;
-#pragma omp parallel for num_threads(ScanThreads()) reduction(|| : bad) if (num_entries > 65536)
-  for (size_t i = 0; i < num_entries; i++) {
-    if (entries[i].key >= n_nodes)
+#pragma omp parallel for num_threads(ScanThreads()) reduction(|| : bad) if (n > 65536)
+  for (size_t i = 0; i < n; i++) {
+    if (e[i].key >= n_nodes)
       bad = true;
     else
-      __atomic_fetch_add(&cnt[entries[i].key], entries[i].cnt, __ATOMIC_RELAXED);
+      __atomic_fetch_add(&into[e[i].key], e[i].cnt, __ATOMIC_RELAXED);
   }
-  CHECK(!bad) << "FreqRecorder::AddEntries: a row is outside num_total_item=" << n_nodes;
+  CHECK(!bad) << "FreqRecorder: a handed-over row is outside num_total_item=" << n_nodes;
+  _handed_over.clear();
+}
+
+void FreqRecorder::BeginEntries() {
+  std::lock_guard<std::mutex> g(_mu);
+  if (_handed_over.empty()) return;
+  // an earlier hand-over is still pending: its keys may come again, so it goes into the array now
+  ScatterHandedOver(_live);
+  _live_dirty = true;
+}
+
+void FreqRecorder::AddEntries(const FreqEntry *entries, size_t num_entries) {
+  std::lock_guard<std::mutex> g(_mu);
+  _handed_over.insert(_handed_over.end(), entries, entries + num_entries);
 }
 
 void FreqRecorder::LocalCombineToShared() {
   std::lock_guard<std::mutex> g(_mu);
+  if (!_live_dirty) return;  // nothing was counted on the host: no scan
   CntT *shared = _shared, *live = _live;
   const size_t n = _num_nodes;
+  _live_dirty = false;
+  _shared_dirty = true;
 #pragma omp parallel for num_threads(ScanThreads())
   for (size_t i = 0; i < n; i++) {
     if (live[i]) {  // the recorded keys are a small part of the key space: write only where something was counted
@@ -123,6 +140,18 @@ void FreqRecorder::GlobalCombine() {
   std::lock_guard<std::mutex> g(_mu);
   auto &e = global_cont_freq_buf->entries;
   e.clear();
+  if (!_shared_dirty) {
+    // only handed-over entries (distinct keys): they are the list, whatever their order — Sort() follows
+    const size_t n_nodes = _num_nodes;
+    for (const auto &x : _handed_over) CHECK_LT((size_t)x.key, n_nodes);
+    e.swap(_handed_over);
+    _handed_over.clear();
+    global_cont_freq_buf->buf = e.data();
+    LOG(INFO) << "freq recorder global combine: " << e.size() << " distinct keys (handed over)";
+    return;
+  }
+  if (!_handed_over.empty()) ScatterHandedOver(_shared);
+  _shared_dirty = false;
   // count, scan, fill: the entries come out in ascending key order whatever the thread count
   const int nthr = ScanThreads();
   const size_t n = _num_nodes, chunk = (n + nthr - 1) / nthr;

@@ -47,7 +47,11 @@ class FreqRecorder {
   ~FreqRecorder();
   template <typename KeyT>
   void Record(const KeyT *inputs, size_t num_input);
-  // counts gathered elsewhere (the device-side counters): entries with distinct keys, added to the live counts
+  // Counts gathered elsewhere (the device-side counters).  BeginEntries opens one hand-over; the AddEntries calls that
+  // follow bring entries whose keys are distinct within the hand-over.  As long as nothing was recorded on the host
+  // the entries are kept as a list and become the ranking input directly, so a refresh driven by the device-side
+  // counters never scans the per-key arrays of the whole key space.
+  void BeginEntries();
   void AddEntries(const FreqEntry *entries, size_t num_entries);
   void LocalCombineToShared();
   void GlobalCombine();
@@ -61,6 +65,9 @@ class FreqRecorder {
   // one counter per key of the key space, calloc-backed so that pages nobody counted in are never touched
   CntT *_live = nullptr;    // counts being recorded
   CntT *_shared = nullptr;  // counts handed over by LocalCombineToShared
+  bool _live_dirty = false, _shared_dirty = false;  // the array holds a non-zero counter
+  std::vector<FreqEntry> _handed_over;              // entries of the open hand-over, not in the arrays
+  void ScatterHandedOver(CntT *into);
   std::mutex _mu;
 };
 
