@@ -747,28 +747,15 @@ void RefreshSession::refresh_after_solve_new(bool foreground) {
   const size_t num_new_local_key = key_list_of_each_src[local]->NumItem();
   CHECK(num_new_local_key <= ctx->_cache_space_capacity) << "cache space can not hold refreshed new cache";
 
-  // Step 2: keys to insert = new local and not old local
-  TensorPtr new_insert_keys;
-  {
-    const IdType *old_n2b = coll_cache->_old_nid_to_block->CPtr<IdType>();
-    const uint8_t *old_place = coll_cache->_old_block_placement->CPtr<uint8_t>();
-    new_insert_keys = table->DetectKeysWithCond(
-        key_list_of_each_src[local]->CPtr<IdType>(), num_new_local_key,
-        [old_n2b, old_place, local](const IdType &key) { return (old_place[old_n2b[key]] & (1 << local)) == 0; },
-        num_new_local_key);
-  }
+  // Steps 2 and 3: keys to insert = new local and not old local; keys to evict = old local and not new local
+  // (DetectKeysWithCond over the other placement's nid_to_block in the reference, cache_context.cu:3975-4003).
+  // Both lists are ascending (DetectKeysForAllSource), so the two differences are merges.
+  const IdType *new_keys = key_list_of_each_src[local]->CPtr<IdType>();
+  const IdType *old_keys = table->_cached_keys->CPtr<IdType>();
+  const size_t num_old_local_key = table->_cached_keys->NumItem();
+  TensorPtr new_insert_keys = CacheEntryManager::SortedDifference(new_keys, num_new_local_key, old_keys, num_old_local_key);
   const size_t num_preserved_key = num_new_local_key - new_insert_keys->NumItem();
-
-  // Step 3: keys to evict = old cached and not new local; their slots go back to the free list, then evict
-  TensorPtr new_evict_keys;
-  {
-    const IdType *n2b = coll_cache->_nid_to_block->CPtr<IdType>();
-    const uint8_t *place = coll_cache->_block_placement->CPtr<uint8_t>();
-    new_evict_keys = table->DetectKeysWithCond(
-        table->_cached_keys->CPtr<IdType>(), table->_cached_keys->NumItem(),
-        [n2b, place, local](const IdType &key) { return (place[n2b[key]] & (1 << local)) == 0; },
-        table->_cached_keys->NumItem() - num_preserved_key);
-  }
+  TensorPtr new_evict_keys = CacheEntryManager::SortedDifference(old_keys, num_old_local_key, new_keys, num_new_local_key);
   const size_t num_evicted = new_evict_keys->NumItem();
   CHECK_EQ(num_evicted + num_preserved_key, table->_cached_keys->NumItem());
   detect_s = t_phase.Passed();

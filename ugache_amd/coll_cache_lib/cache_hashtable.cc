@@ -1,5 +1,7 @@
 #include "cache_hashtable.h"
 
+#include <algorithm>
+
 namespace coll_cache_lib {
 namespace common {
 
@@ -131,6 +133,34 @@ TensorPtr CacheEntryManager::ReserveOffsetFront(IdType n) {
   return ret;
 }
 
+TensorPtr CacheEntryManager::SortedDifference(const IdType *a, size_t na, const IdType *b, size_t nb) {
+  const int nthr = std::max(1, RunConfig::solver_omp_thread_num_per_gpu);
+  const size_t chunk = (na + nthr - 1) / nthr;
+  std::vector<size_t> counts(nthr + 1, 0);
+  // thread t owns a[lo, hi) and walks b from the first element not below a[lo]
+  auto walk = [&](int t, IdType *dst) -> size_t {
+    const size_t lo = std::min(na, chunk * t), hi = std::min(na, chunk * (t + 1));
+    if (lo >= hi) return 0;
+    size_t j = std::lower_bound(b, b + nb, a[lo]) - b;
+    size_t out = 0;
+    for (size_t i = lo; i < hi; i++) {
+      while (j < nb && b[j] < a[i]) j++;
+      if (j < nb && b[j] == a[i]) continue;
+      if (dst) dst[out] = a[i];
+      out++;
+    }
+    return out;
+  };
+#pragma omp parallel for num_threads(nthr) schedule(static, 1)
+  for (int t = 0; t < nthr; t++) counts[t + 1] = walk(t, nullptr);
+  for (int t = 0; t < nthr; t++) counts[t + 1] += counts[t];
+  TensorPtr out = Tensor::Empty(kI32, {counts[nthr]}, CPU_CLIB(), "");
+  IdType *dst = out->Ptr<IdType>();
+#pragma omp parallel for num_threads(nthr) schedule(static, 1)
+  for (int t = 0; t < nthr; t++) walk(t, dst + counts[t]);
+  return out;
+}
+
 void CacheEntryManager::DetectKeysForAllSource(TensorPtr nid_to_block, TensorPtr block_access_advise,
                                                int local_location_id, TensorPtr block_density, size_t num_total_item,
                                                TensorPtr *node_list_of_src, int num_gpu) {
@@ -138,19 +168,40 @@ void CacheEntryManager::DetectKeysForAllSource(TensorPtr nid_to_block, TensorPtr
   CHECK_LE(num_gpu, 8);
   const IdType *n2b = nid_to_block->CPtr<IdType>();
   const uint8_t *advise = block_access_advise->CPtr<uint8_t>();
+  const size_t num_block = block_access_advise->Shape()[0];
   const int nthr = std::max(1, RunConfig::solver_omp_thread_num_per_gpu);
   const size_t chunk = (num_total_item + nthr - 1) / nthr;
+  // One GPU is one list: with the usual two blocks "key k is read from the GPU" is the comparison n2b[k] == b for the
+  // one block b the GPU serves, which the compiler turns into a vector compare over the whole key space; other
+  // shapes go through the block -> source table.
+  int only_block = -1;
+  if (num_gpu == 1) {
+    int served = 0;
+    for (size_t blk = 0; blk < num_block; blk++)
+      if (advise[blk] == 0) {
+        served++;
+        only_block = (int)blk;
+      }
+    if (served != 1) only_block = -1;
+  }
   // two passes (count, then fill) so every list comes out in ascending key order
   std::vector<std::vector<size_t>> counts(num_gpu, std::vector<size_t>(nthr + 1, 0));
 #pragma omp parallel for num_threads(nthr) schedule(static, 1)
   for (int t = 0; t < nthr; t++) {
-    std::vector<size_t> c(num_gpu, 0);
     const size_t lo = std::min(num_total_item, chunk * t), hi = std::min(num_total_item, chunk * (t + 1));
-    for (size_t k = lo; k < hi; k++) {
-      const int src = advise[n2b[k]];
-      if (src < num_gpu) c[src]++;
+    if (only_block >= 0) {
+      const IdType want = (IdType)only_block;
+      size_t c = 0;
+      for (size_t k = lo; k < hi; k++) c += n2b[k] == want;
+      counts[0][t + 1] = c;
+    } else {
+      size_t c[8] = {0};
+      for (size_t k = lo; k < hi; k++) {
+        const int src = advise[n2b[k]];
+        if (src < num_gpu) c[src]++;
+      }
+      for (int d = 0; d < num_gpu; d++) counts[d][t + 1] = c[d];
     }
-    for (int d = 0; d < num_gpu; d++) counts[d][t + 1] = c[d];
   }
   for (int d = 0; d < num_gpu; d++) {
     for (int t = 0; t < nthr; t++) counts[d][t + 1] += counts[d][t];
@@ -158,12 +209,19 @@ void CacheEntryManager::DetectKeysForAllSource(TensorPtr nid_to_block, TensorPtr
   }
 #pragma omp parallel for num_threads(nthr) schedule(static, 1)
   for (int t = 0; t < nthr; t++) {
-    std::vector<size_t> pos(num_gpu);
-    for (int d = 0; d < num_gpu; d++) pos[d] = counts[d][t];
     const size_t lo = std::min(num_total_item, chunk * t), hi = std::min(num_total_item, chunk * (t + 1));
-    for (size_t k = lo; k < hi; k++) {
-      const int src = advise[n2b[k]];
-      if (src < num_gpu) node_list_of_src[src]->Ptr<IdType>()[pos[src]++] = (IdType)k;
+    if (only_block >= 0) {
+      const IdType want = (IdType)only_block;
+      IdType *dst = node_list_of_src[0]->Ptr<IdType>() + counts[0][t];
+      for (size_t k = lo; k < hi; k++)
+        if (n2b[k] == want) *dst++ = (IdType)k;
+    } else {
+      size_t pos[8];
+      for (int d = 0; d < num_gpu; d++) pos[d] = counts[d][t];
+      for (size_t k = lo; k < hi; k++) {
+        const int src = advise[n2b[k]];
+        if (src < num_gpu) node_list_of_src[src]->Ptr<IdType>()[pos[src]++] = (IdType)k;
+      }
     }
   }
   (void)local_location_id;

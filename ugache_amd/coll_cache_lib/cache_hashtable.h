@@ -103,6 +103,11 @@ class CacheEntryManager {
     return out;
   }
 
+  // a \ b for two ascending key lists, ascending again: what DetectKeysWithCond computes when the condition is "not in
+  // the other placement", as a parallel merge over the two lists instead of one random read per key into a per-key
+  // array of the whole key space
+  static TensorPtr SortedDifference(const IdType *a, size_t na, const IdType *b, size_t nb);
+
   // cuh:741-835 — per-source key lists from nid_to_block + this GPU's line of the access advise.
   // node_list_of_src[dev] is filled for dev in [0, num_gpu); keys whose source is the host are not listed.
   static void DetectKeysForAllSource(TensorPtr nid_to_block, TensorPtr block_access_advise, int local_location_id,
