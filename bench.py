@@ -29,7 +29,7 @@ HBM_PEAK_GBPS = 8000.0  # MI355X published HBM3E bandwidth
 
 # HBM-side bytes per launch of the dominant kernel, from the FETCH_SIZE / WRITE_SIZE counter runs summarised in
 # profiles/gather_kernel_c2_all_hit.md (each counter scaled by its reading for a 1 GiB copy kernel)
-MEASURED_TRAFFIC_BYTES = {"c2_all_hit_10Mx128xfp32_262144_u32_uniform": 270_550_000}
+MEASURED_TRAFFIC_BYTES = {"c2_all_hit_10Mx128xfp32_262144_u32_uniform": 270_530_000}
 
 ALL_HIT = {
     # name: (rows, dim, keys per batch)
