@@ -29,7 +29,9 @@ HBM_PEAK_GBPS = 8000.0  # MI355X published HBM3E bandwidth
 
 # HBM-side bytes per launch of the dominant kernel, from the FETCH_SIZE / WRITE_SIZE counter runs summarised in
 # profiles/gather_kernel_c2_all_hit.md (each counter scaled by its reading for a 1 GiB copy kernel)
-MEASURED_TRAFFIC_BYTES = {"c2_all_hit_10Mx128xfp32_262144_u32_uniform": 270_530_000}
+MEASURED_TRAFFIC_BYTES = {"c2_all_hit_10Mx128xfp32_262144_u32_uniform": 270_530_000,
+                          # fused kernel; includes the 126 MB of rows that reach the L2 over the host link
+                          "c3_gnn_100Mx128xfp32_1M_i64_zipf0.9_cache25pct": 1_137_700_000}
 
 ALL_HIT = {
     # name: (rows, dim, keys per batch)
@@ -494,7 +496,8 @@ def run_mixed(args):
         "stages_us": stages,
         "hit_rate": n_hit / n_keys,
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-                     "frac": achieved / HBM_PEAK_GBPS, "traffic": None,
+                     "frac": achieved / HBM_PEAK_GBPS,
+                     "traffic": MEASURED_TRAFFIC_BYTES.get(args.workload) if fused else None,
                      "kernel": kernel_name,
                      "algorithmic_bytes_per_launch": hit_alg, "avg_kernel_us": t_hit * 1e6},
         "host_link": {"achieved": miss_bytes / t_link / 1e9 if t_link > 0 else 0.0, "measured_peak": link_gbps,
