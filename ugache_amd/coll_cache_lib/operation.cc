@@ -470,7 +470,11 @@ void coll_cache_shutdown(void) {
   _forward.enable_refresh = false;
   _forward.step = 0;
   _forward.refreshes_done.store(0);
-  if (_coll_cache) _coll_cache->release_replicas();
+  if (_coll_cache && _coll_cache->num_replicas_built() > 0) {
+    // stream-ordered lookups may still be in flight; their buffers and streams go away below
+    UGK_CALL(ugk_device_sync());
+    _coll_cache->release_replicas();
+  }
   _coll_cache = nullptr;
   _profiler = nullptr;
   _freq_recorder.clear();
