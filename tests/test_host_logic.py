@@ -229,3 +229,10 @@ def test_recorder_and_placement_reproduce_the_committed_golden_case():
     c = np.zeros(n_item, np.uint32)
     m = C.coll_cache_rank_hotness(0, k.ctypes.data, c.ctypes.data, n_item)
     assert k[:m].tolist() == g["rank_keys_observed"] and c[:m].tolist() == g["rank_counts_observed"]
+
+
+def test_bench_refuses_more_than_one_gpu():
+    p = subprocess.run([sys.executable, os.path.join(ROOT, "bench.py"), "--gpus", "2"], stdout=subprocess.PIPE,
+                       stderr=subprocess.PIPE, text=True, timeout=120)
+    assert p.returncode != 0 and p.stdout == ""
+    assert "ONE GPU" in p.stderr and "--gpus 1" in p.stderr
