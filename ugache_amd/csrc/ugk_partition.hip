@@ -203,63 +203,80 @@ __global__ __launch_bounds__(kBlock) void dedup_claim_kernel(const K *__restrict
                                                              uint32_t epoch, uint32_t *uid_of, K *unique_out,
                                                              uint32_t *inverse, uint32_t *rep_of,
                                                              uint32_t *n_unique) {
-  __shared__ uint32_t wave_tot[kWavesPerBlock];
+  // a tile of kTile keys per pass (kItems per lane): one reservation of unique ids per tile, so the single counter
+  // they come from sees a quarter of the atomics a 256-key tile would send it
+  __shared__ uint32_t wave_tot[kItems][kWavesPerBlock];
   __shared__ uint32_t base;
-  __shared__ K stage[kBlock];
+  __shared__ K stage[kTile];
   const int tid = threadIdx.x;
   const int lane = tid & (kWave - 1), wave = tid / kWave;
-  const size_t n_round = (n + kBlock - 1) / kBlock * kBlock;
-  for (size_t i = (size_t)blockIdx.x * kBlock + tid; i < n_round; i += (size_t)gridDim.x * kBlock) {
-    const bool active = i < n;
-    bool winner = false;
-    K key = 0;
-    if (active) {
-      key = keys[i];
-      size_t h = fmix64(key_to_u64<K>(key)) & cap_mask;
-      uint32_t rep = (uint32_t)i;
-      for (;;) {
-        unsigned long long s = __atomic_load_n(slots + h, __ATOMIC_RELAXED);
-        bool claimed = false;
-        while ((uint32_t)(s >> 32) != epoch) {
-          const unsigned long long want = ((unsigned long long)epoch << 32) | (uint32_t)i;
-          const unsigned long long seen = atomicCAS(slots + h, s, want);
-          if (seen == s) {
-            claimed = true;
+  for (size_t tile0 = (size_t)blockIdx.x * kTile; tile0 < n; tile0 += (size_t)gridDim.x * kTile) {
+    bool winner[kItems];
+    K key[kItems];
+    uint32_t pre[kItems];
+#pragma unroll
+    for (int j = 0; j < kItems; ++j) {
+      const size_t i = tile0 + (size_t)j * kBlock + tid;
+      winner[j] = false;
+      key[j] = 0;
+      if (i < n) {
+        key[j] = keys[i];
+        size_t h = fmix64(key_to_u64<K>(key[j])) & cap_mask;
+        uint32_t rep = (uint32_t)i;
+        for (;;) {
+          unsigned long long s = __atomic_load_n(slots + h, __ATOMIC_RELAXED);
+          bool claimed = false;
+          while ((uint32_t)(s >> 32) != epoch) {
+            const unsigned long long want = ((unsigned long long)epoch << 32) | (uint32_t)i;
+            const unsigned long long seen = atomicCAS(slots + h, s, want);
+            if (seen == s) {
+              claimed = true;
+              break;
+            }
+            s = seen;
+          }
+          if (claimed) {
+            winner[j] = true;
             break;
           }
-          s = seen;
+          const uint32_t other = (uint32_t)s;
+          if (keys[other] == key[j]) {
+            rep = other;
+            break;
+          }
+          h = (h + 1) & cap_mask;
         }
-        if (claimed) {
-          winner = true;
-          break;
-        }
-        const uint32_t j = (uint32_t)s;
-        if (keys[j] == key) {
-          rep = j;
-          break;
-        }
-        h = (h + 1) & cap_mask;
+        inverse[i] = rep;  // index of the representative; replaced by its unique id in the second kernel
       }
-      inverse[i] = rep;  // index of the representative; replaced by its unique id in the second kernel
+      const uint64_t wb = __ballot(winner[j]);
+      pre[j] = __popcll(wb & ((1ull << lane) - 1ull));
+      if (lane == 0) wave_tot[j][wave] = __popcll(wb);
     }
-    const uint64_t wb = __ballot(winner);
-    const uint32_t pre = __popcll(wb & ((1ull << lane) - 1ull));
-    if (lane == 0) wave_tot[wave] = __popcll(wb);
     __syncthreads();
-    uint32_t before = 0, total = 0;
+    uint32_t total = 0, before[kItems];
 #pragma unroll
-    for (int w = 0; w < kWavesPerBlock; ++w) {
-      if (w == wave) before = total;
-      total += wave_tot[w];
+    for (int j = 0; j < kItems; ++j) {
+#pragma unroll
+      for (int w = 0; w < kWavesPerBlock; ++w) {
+        if (w == wave) before[j] = total;
+        total += wave_tot[j][w];
+      }
     }
     if (tid == 0) base = total ? atomicAdd(n_unique, total) : 0u;
-    if (winner) stage[before + pre] = key;
+#pragma unroll
+    for (int j = 0; j < kItems; ++j)
+      if (winner[j]) stage[before[j] + pre[j]] = key[j];
     __syncthreads();
-    if (winner) {
-      uid_of[i] = base + before + pre;
-      if (rep_of) rep_of[base + before + pre] = (uint32_t)i;
+#pragma unroll
+    for (int j = 0; j < kItems; ++j) {
+      if (winner[j]) {
+        const size_t i = tile0 + (size_t)j * kBlock + tid;
+        const uint32_t uid = base + before[j] + pre[j];
+        uid_of[i] = uid;
+        if (rep_of) rep_of[uid] = (uint32_t)i;
+      }
     }
-    if ((uint32_t)tid < total) unique_out[base + tid] = stage[tid];
+    for (uint32_t p = tid; p < total; p += kBlock) unique_out[base + p] = stage[p];
     __syncthreads();
   }
 }
@@ -359,10 +376,11 @@ int dedup(const K *keys, size_t n, void *workspace, uint32_t epoch, K *unique_ou
   const size_t cap = dedup_capacity(n);
   unsigned long long *slots = reinterpret_cast<unsigned long long *>(workspace);
   uint32_t *uid_of = reinterpret_cast<uint32_t *>(slots + cap);
-  const unsigned grid = clamp_grid((n + kBlock - 1) / kBlock, 0);
-  hipLaunchKernelGGL(dedup_claim_kernel<K>, dim3(grid), dim3(kBlock), 0, as_stream(stream), keys, n, slots, cap - 1,
-                     epoch, uid_of, unique_out, inverse, rep_of, n_unique);
+  const unsigned claim_grid = clamp_grid((n + kTile - 1) / kTile, 0);
+  hipLaunchKernelGGL(dedup_claim_kernel<K>, dim3(claim_grid), dim3(kBlock), 0, as_stream(stream), keys, n, slots,
+                     cap - 1, epoch, uid_of, unique_out, inverse, rep_of, n_unique);
   UGK_HIP(hipGetLastError());
+  const unsigned grid = clamp_grid((n + kBlock - 1) / kBlock, 0);
   hipLaunchKernelGGL(dedup_resolve_kernel, dim3(grid), dim3(kBlock), 0, as_stream(stream), n, uid_of, inverse,
                      n_unique, n_unique_host);
   UGK_HIP(hipGetLastError());
