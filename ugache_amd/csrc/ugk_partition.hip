@@ -7,6 +7,8 @@
 // ONE atomic per source, stages the compacted records in LDS and writes them out as contiguous, coalesced
 // runs: hits grow from the front of idx[], misses from the back, so idx[] and the two counters describe the
 // same (location-grouped) array the reference obtains by sorting.
+#include <cstdlib>
+
 #include "ugk_internal.h"
 #include "ugk_table.cuh"
 
@@ -116,7 +118,7 @@ __global__ __launch_bounds__(kBlock) void extract_mix_kernel(ugk_table_t t, cons
                                                              const u32x4 *__restrict__ host, uint64_t host_rows,
                                                              u32x4 *__restrict__ out, uint32_t vpr,
                                                              uint32_t *status, uint32_t *host_mirror,
-                                                             uint32_t *counts) {
+                                                             uint32_t *counts, bool nt_store) {
   constexpr int RPW = kWave / LPR;  // rows per wavefront instruction
   __shared__ uint32_t block_tot[2];
   if (threadIdx.x < 2) block_tot[threadIdx.x] = 0;
@@ -161,7 +163,11 @@ __global__ __launch_bounds__(kBlock) void extract_mix_kernel(ugk_table_t t, cons
             if (p[u]) v[u] = __builtin_nontemporal_load(p[u] + col);
 #pragma unroll
           for (int u = 0; u < UNROLL; ++u)
-            if (p[u]) __builtin_nontemporal_store(v[u], out + (b0 + r0 + u * RPW + rg) * vpr + col);
+            if (p[u]) {
+              u32x4 *dst = out + (b0 + r0 + u * RPW + rg) * vpr + col;
+              if (nt_store) __builtin_nontemporal_store(v[u], dst);
+              else *dst = v[u];
+            }
         }
       }
     }
@@ -323,10 +329,17 @@ int extract_mix_lpr(ugk_table_t t, const K *keys, size_t n, const void *cache, u
                     uint64_t host_rows, void *out, uint32_t vpr, uint32_t *status, uint32_t *host_mirror,
                     uint32_t *counts, hipStream_t st) {
   const unsigned grid = clamp_grid((n + kBlock - 1) / kBlock, 0);
+  // ordinary write-back stores while the output fits the memory-side cache (the consumer finds it there),
+  // non-temporal beyond; UGK_GATHER_NT_STORE=0/1 forces the choice
+  static const int forced_nt = [] {
+    const char *e = getenv("UGK_GATHER_NT_STORE");
+    return e ? atoi(e) : -1;
+  }();
+  const bool nt = forced_nt >= 0 ? forced_nt != 0 : n * (size_t)vpr * 16 > ((size_t)192 << 20);
 #define UGK_GO(L)                                                                                                 \
   hipLaunchKernelGGL((extract_mix_kernel<K, KIND, L>), dim3(grid), dim3(kBlock), 0, st, t, keys, n,               \
                      (const u32x4 *)cache, cache_rows, (const u32x4 *)host, host_rows, (u32x4 *)out, vpr, status, \
-                     host_mirror, counts)
+                     host_mirror, counts, nt)
   if (vpr <= 1) UGK_GO(1);
   else if (vpr <= 2) UGK_GO(2);
   else if (vpr <= 4) UGK_GO(4);

@@ -84,47 +84,53 @@ __device__ __forceinline__ HashProbe hash_probe_home(const ugk_bucket_t *table, 
   const int lane = (int)lane_id();
   const int grp = lane >> 3, sub = lane & 7;
   const uint64_t home = active ? hash_home(key, nb) : 0;
-  u32x4 raw[8];
-  uint64_t kk[8];
-  bool act[8];
+  // two passes of four rounds: the four line loads of a pass are in flight together; holding all eight rounds at
+  // once costs 50 more vector registers and halves the occupancy of the kernels built on this
 #pragma unroll
-  for (int r = 0; r < 8; ++r) {
-    const int owner = r * 8 + grp;
-    kk[r] = shfl64(key, owner);
-    const uint64_t hb = shfl64(home, owner);
-    act[r] = __shfl((int)active, owner) != 0;
-    raw[r] = u32x4{0xffffffffu, 0xffffffffu, 0u, 0u};  // reads as a never-used bucket
-    if (act[r]) raw[r] = *reinterpret_cast<const u32x4 *>(table + hb + sub);
-  }
+  for (int half = 0; half < 2; ++half) {
+    u32x4 raw[4];
+    uint64_t kk[4];
+    bool act[4];
 #pragma unroll
-  for (int r = 0; r < 8; ++r) {
-    const uint64_t bkey = ((uint64_t)raw[r].y << 32) | raw[r].x;
-    const bool is_match = act[r] && bkey == kk[r];
-    const bool is_empty = act[r] && bkey == UGK_HASH_EMPTY;
-    const uint32_t mb = (uint32_t)((__ballot(is_match) >> (grp * 8)) & 0xffull);
-    const uint32_t eb = (uint32_t)((__ballot(is_empty) >> (grp * 8)) & 0xffull);
-    const int fm = mb ? (__ffs(mb) - 1) : 8;
-    const int fe = eb ? (__ffs(eb) - 1) : 8;
-    const bool g_found = fm < fe;  // a key sits in front of the first never-used bucket of its probe sequence
-    const bool g_done = g_found || fe < 8;
-    const int hit_lane = grp * 8 + (g_found ? fm : 0);
-    const uint32_t h_off = __shfl(raw[r].z, hit_lane);
-    const uint32_t h_meta = __shfl(raw[r].w, hit_lane);
-    const uint32_t g_flags = (g_done ? 1u : 0u) | (g_found ? 2u : 0u);
-    // the owner of this round's key served by group g is lane 8r + g: it reads its group's result
-    const int from = (lane & 7) * 8;
-    const uint32_t r_flags = __shfl(g_flags, from);
-    const uint32_t r_off = __shfl(h_off, from);
-    const uint32_t r_meta = __shfl(h_meta, from);
-    if ((lane >> 3) == r && active) {
-      if (r_flags & 1u) {
-        if ((r_flags & 2u) && (r_meta & UGK_META_VALID)) {
-          p.f.hit = true;
-          p.f.loc = r_meta & 0xfu;
-          p.f.off = r_off;
+    for (int q = 0; q < 4; ++q) {
+      const int owner = (half * 4 + q) * 8 + grp;
+      kk[q] = shfl64(key, owner);
+      const uint64_t hb = shfl64(home, owner);
+      act[q] = __shfl((int)active, owner) != 0;
+      raw[q] = u32x4{0xffffffffu, 0xffffffffu, 0u, 0u};  // reads as a never-used bucket
+      if (act[q]) raw[q] = *reinterpret_cast<const u32x4 *>(table + hb + sub);
+    }
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      const int r = half * 4 + q;
+      const uint64_t bkey = ((uint64_t)raw[q].y << 32) | raw[q].x;
+      const bool is_match = act[q] && bkey == kk[q];
+      const bool is_empty = act[q] && bkey == UGK_HASH_EMPTY;
+      const uint32_t mb = (uint32_t)((__ballot(is_match) >> (grp * 8)) & 0xffull);
+      const uint32_t eb = (uint32_t)((__ballot(is_empty) >> (grp * 8)) & 0xffull);
+      const int fm = mb ? (__ffs(mb) - 1) : 8;
+      const int fe = eb ? (__ffs(eb) - 1) : 8;
+      const bool g_found = fm < fe;  // a key sits in front of the first never-used bucket of its probe sequence
+      const bool g_done = g_found || fe < 8;
+      const int hit_lane = grp * 8 + (g_found ? fm : 0);
+      const uint32_t h_off = __shfl(raw[q].z, hit_lane);
+      const uint32_t h_meta = __shfl(raw[q].w, hit_lane);
+      const uint32_t g_flags = (g_done ? 1u : 0u) | (g_found ? 2u : 0u);
+      // the owner of this round's key served by group g is lane 8r + g: it reads its group's result
+      const int from = (lane & 7) * 8;
+      const uint32_t r_flags = __shfl(g_flags, from);
+      const uint32_t r_off = __shfl(h_off, from);
+      const uint32_t r_meta = __shfl(h_meta, from);
+      if ((lane >> 3) == r && active) {
+        if (r_flags & 1u) {
+          if ((r_flags & 2u) && (r_meta & UGK_META_VALID)) {
+            p.f.hit = true;
+            p.f.loc = r_meta & 0xfu;
+            p.f.off = r_off;
+          }
+        } else {
+          p.pending = true;
         }
-      } else {
-        p.pending = true;
       }
     }
   }
