@@ -248,6 +248,24 @@ def test_rows_that_are_not_multiples_of_16_bytes(dim, dtype, pct):
         assert out.cpu().numpy().tobytes() == ORC.gather(table, q.astype(np.int64)).tobytes()
 
 
+def test_key_tensors_are_checked_and_strided_ones_accepted():
+    rng = np.random.default_rng(3)
+    n_item, dim = 5_000, 32
+    co.config(make_config(n_item, 1.0))
+    emb = co.coll_torch_create_emb_shm(0, n_item, dim, torch.float32)
+    table = fill_table(emb, rng)
+    co.coll_torch_init_t(0, 0, emb, 1.0)
+    q = rng.integers(0, n_item, size=(2000, 2))
+    strided = torch.from_numpy(q).cuda()[:, 1]  # every second element: not contiguous
+    assert not strided.is_contiguous()
+    out = co.coll_torch_lookup_key_t_val_ret(0, strided, False)
+    assert out.cpu().numpy().tobytes() == ORC.gather(table, q[:, 1].astype(np.int64)).tobytes()
+    with pytest.raises(TypeError):
+        co.coll_torch_lookup_key_t_val_ret(0, strided.to(torch.float32), False)
+    with pytest.raises(ValueError):
+        co.coll_torch_lookup_key_t_val_ret(0, strided.cpu(), False)
+
+
 def test_create_emb_from_file(tmp_path):
     rng = np.random.default_rng(2)
     arr = rng.standard_normal((1000, 32)).astype(np.float32)

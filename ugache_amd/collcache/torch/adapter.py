@@ -30,6 +30,7 @@ class _State:
     external_feat_dim = 0
     internal_feat_dim = 0
     batch_emb_reuse = None  # int8 tensor backing the reused output buffer
+    last_keys = None        # key tensor of the most recent lookup
     held = {}              # device pointer -> tensor handed to the library by the allocator callback
     host_tables = []       # keeps pinned tables alive
     host_ptrs = []         # pinned allocations made by coll_torch_create_emb_shm
@@ -104,6 +105,13 @@ def coll_torch_test(local_id, keys):
 
 def _lookup_into_reused_buffer(local_id, keys, pad_to_8, fn32, fn64):
     dev = _State.dev_id.get(local_id, 0)
+    if keys.dtype not in (torch.int32, torch.int64, torch.uint32):
+        raise TypeError("keys must be int32 / uint32 or int64, got %s" % keys.dtype)
+    if not keys.is_cuda:
+        raise ValueError("keys must live on the GPU (the reference reads key.data_ptr() from device code too)")
+    if not keys.is_contiguous():
+        keys = keys.contiguous()
+    _State.last_keys = keys  # a stream-ordered lookup reads them after this call has returned
     n = keys.size(0)
     padded_len = (n + 7) // 8 * 8 if pad_to_8 else n
     max_num_keys = _C.coll_cache_max_num_keys()
@@ -237,6 +245,7 @@ def coll_torch_shutdown():
     """drop the cache and every buffer it holds, including the tables made by coll_torch_create_emb_shm, which
     must not be used afterwards (the reference has no teardown)."""
     torch.cuda.synchronize()
+    _State.last_keys = None
     _basics.shutdown()
     for p in _State.host_ptrs:
         _C.coll_cache_free_host_table(p)
