@@ -563,6 +563,63 @@ def test_stream_ordered_lookup_inside_a_captured_graph(pct):
         assert eager.cpu().numpy().tobytes() == result.cpu().numpy().tobytes()
 
 
+def _random_case(seed):
+    r = np.random.default_rng(1000 + seed)
+    dims = [1, 2, 3, 4, 8, 12, 16, 31, 32, 64, 100, 128, 256, 300]
+    return dict(seed=seed, n_item=int(r.integers(1, 60_000)), dim=int(r.choice(dims)),
+                pct=float(r.choice([0.0, 0.01, 0.1, 0.37, 0.9, 0.999, 1.0])),
+                table_kind=str(r.choice(["FLAT", "HASH"])), impl=str(r.choice(["", "SMMaskPhase", "NONE"])),
+                i64=bool(r.integers(0, 2)), dedup=bool(r.integers(0, 4) == 0), gpu_record=bool(r.integers(0, 4) == 0),
+                zipf=float(r.choice([0.6, 1.05, 1.4])), half=bool(r.integers(0, 3) == 0))
+
+
+@pytest.mark.parametrize("case", [_random_case(i) for i in range(96)], ids=lambda c: "seed%d" % c["seed"])
+def test_random_configurations_are_exact(case, monkeypatch):
+    """seeded random sweep over table size, row width, cache share, table kind, extraction mode, key width and the
+    optional stages: blocking and stream-ordered lookups of ragged batch sizes (0, 1, odd, larger than the table)
+    must reproduce table[keys] byte for byte"""
+    monkeypatch.setenv("COLL_HASH_TABLE", case["table_kind"])
+    if case["impl"]:
+        monkeypatch.setenv("SAMGRAPH_COLL_CACHE_CONCURRENT_LINK_IMPL", case["impl"])
+    if case["dedup"]:
+        monkeypatch.setenv("COLL_DEDUP_KEYS", "1")
+        monkeypatch.setenv("COLL_DEDUP_MIN_KEYS", "16")
+    if case["gpu_record"]:
+        monkeypatch.setenv("COLL_GPU_RECORD", "1")
+    rng = np.random.default_rng(case["seed"])
+    n_item, dim, pct = case["n_item"], case["dim"], case["pct"]
+    kdtype = torch.int64 if case["i64"] else torch.int32
+    co.config(make_config(n_item, pct))
+    co.coll_cache_record_init(0)
+    perm = rng.permutation(n_item)
+    co.coll_torch_record(0, torch.from_numpy(perm[zipf_ranks(rng, 5 * n_item + 10, n_item, case["zipf"])]).to(kdtype))
+    fdtype = torch.float16 if case["half"] and dim % 2 == 0 else torch.float32
+    emb = co.coll_torch_create_emb_shm(0, n_item, dim, fdtype)
+    table = fill_table(emb, rng)
+    co.coll_torch_init_t(0, 0, emb, pct)
+    info = _basics.info(0)
+    assert info["capacity_rows"] == ORC.lib.orc_cache_capacity(n_item, pct) or pct in (0.0, 1.0)
+    for n in (0, 1, 7, 63, 64, 65, 1023, int(rng.integers(2_000, 70_000))):
+        keys = perm[zipf_ranks(rng, n, n_item, case["zipf"])] if n else np.zeros(0, np.int64)
+        kt = torch.from_numpy(keys).to(kdtype).cuda()
+        want = ORC.gather(table, keys.astype(np.int64)).tobytes()
+        out = co.coll_torch_lookup_key_t_val_ret(0, kt, False)
+        assert out.shape == (n, dim) and out.cpu().numpy().tobytes() == want, ("blocking", n)
+        g = _basics.last_group_offset(0)
+        assert g[0] == 0 and g[1] <= g[2] <= n
+        a = co.coll_torch_lookup_async(0, kt, False).clone()
+        co.coll_torch_lookup_wait(0)
+        assert a.cpu().numpy().tobytes() == want, ("stream-ordered", n)
+    if 0.0 < pct < 1.0 and n_item > 100:
+        co.coll_torch_record(0, torch.from_numpy(perm[::-1][zipf_ranks(rng, 3 * n_item, n_item, 1.1)].copy()).to(kdtype))
+        co.coll_torch_refresh(0, True)
+        info = _basics.info(0)
+        assert info["free_slots"] + info["cached_rows"] == info["capacity_rows"]
+        keys = rng.integers(0, n_item, size=5_000)
+        out = co.coll_torch_lookup_key_t_val_ret(0, torch.from_numpy(keys).to(kdtype).cuda(), False)
+        assert out.cpu().numpy().tobytes() == ORC.gather(table, keys.astype(np.int64)).tobytes()
+
+
 def test_reference_cpu_runnable_config_full_size():
     """1M x 128 fp32 host table, 65536 int64 keys Zipf(1.1) over a seeded permutation, hottest 10 % cached."""
     rng = np.random.default_rng(1)
