@@ -267,6 +267,49 @@ def test_hash_table_against_dict_and_oracle_table(kdtype, space, n):
     assert occ == n and occ + tomb + empty == nb
 
 
+@pytest.mark.parametrize("load", [0.5, 0.7, 0.9])
+def test_hash_table_under_churn_follows_a_dict(load):
+    """refresh-like churn: rounds of evicting a tenth of the keys and inserting as many new ones, tombstones piling
+    up in between; after every round each present key returns its latest value, every evicted or never-inserted key
+    misses, and occupied + tombstoned + never used == buckets"""
+    rng = np.random.default_rng(int(load * 10))
+    n = 40_000
+    mem, tb, nb = _make_hash(n, load=load)
+    model = {}
+    keys = np.unique(rng.integers(0, 1 << 40, size=2 * n))[:n].astype(np.int64)
+    offs = rng.integers(0, 1 << 31, size=n).astype(np.uint32)
+    assert _insert(tb, keys, offs) == 0
+    model.update(zip(keys.tolist(), offs.tolist()))
+    gone = set()
+    cen = torch.zeros(3, dtype=torch.int64, device="cuda")
+    for rnd in range(12):
+        present = np.fromiter(model.keys(), np.int64, len(model))
+        ev = rng.choice(present, n // 10, replace=False)
+        assert _evict(tb, ev) == 0
+        for k in ev.tolist():
+            del model[k]
+            gone.add(k)
+        fresh = np.setdiff1d(np.unique(rng.integers(0, 1 << 40, size=n // 5)).astype(np.int64), present)[: n // 10]
+        back = np.array(list(gone)[: n // 50], np.int64)  # some evicted keys come back
+        ins = np.unique(np.concatenate([back, fresh]))
+        ins = rng.permutation(ins)[: n // 10]  # as many in as out: the table keeps its load
+        ins_off = rng.integers(0, 1 << 31, size=len(ins)).astype(np.uint32)
+        st = _insert(tb, ins, ins_off)
+        assert st == 0, (rnd, st)
+        for k, o in zip(ins.tolist(), ins_off.tolist()):
+            model[k] = o
+            gone.discard(k)
+        present = np.fromiter(model.keys(), np.int64, len(model))
+        absent = np.array(list(gone)[:5000] + rng.integers(1 << 41, 1 << 42, size=1000).tolist(), np.int64)
+        loc, off = _lookup(tb, np.concatenate([present, absent]), fallback=1)
+        assert (loc[: len(present)] == 0).all() and (loc[len(present):] == 1).all(), rnd
+        assert np.array_equal(off[: len(present)], np.array([model[k] for k in present.tolist()], np.uint32)), rnd
+        hip.call("ugk_hash_census", tb.table, nb, cen.data_ptr(), None)
+        sync()
+        occ, tomb, empty = cen.cpu().tolist()
+        assert occ == len(model) and occ + tomb + empty == nb, rnd
+
+
 def test_hash_table_dense_collisions_and_host_entries():
     """Load factor 0.9 with sequential keys forces long probe runs; host-located entries carry explicit rows."""
     n = 50_000
