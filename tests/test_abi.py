@@ -72,3 +72,36 @@ def test_python_surface_matches_reference_names():
     assert cc.kLogL3LabelExtractTime == 53
     assert cc.kLogEpochFeatureBytes == 13 and cc.kLogEpochMissBytes == 14
     assert cc.gpu(1) == "cuda:1" and cc.cpu() == "cpu:0"
+
+
+def test_torch_surface_has_the_reference_entry_points():
+    """python/collcache/torch/adapter.py:29-54 and the module-level helpers of python/collcache/common/__init__.py
+    (:47-171, 173-262), by name and by parameter list"""
+    import inspect
+    import sys
+    torch = pytest.importorskip("torch")
+    del torch
+    sys.path.insert(0, os.path.join(ROOT, "ugache_amd"))
+    import collcache.torch as co
+    want = {
+        "config": ["run_config"],
+        "coll_cache_record_init": ["replica_id"],
+        "coll_torch_record": ["local_id", "keys"],
+        "coll_torch_create_emb_shm": ["replica_id", "n_keys", "dim", "dtype", "fname"],
+        "coll_torch_init_t": ["replica_id", "dev_id", "emb", "cache_percentage"],
+        "coll_torch_lookup_key_t_val_ret": ["local_id", "keys", "pad_to_8"],
+        "coll_torch_test": ["local_id", "keys"],
+        "log_step_by_key": ["key", "item", "val"],
+        "report_step": ["key"],
+        "report_step_average": ["key"],
+        "wait_one_child": [],
+        "print_memory_usage": [],
+    }
+    for name, params in want.items():
+        fn = getattr(co, name, None)
+        assert callable(fn), name
+        got = [p for p in inspect.signature(fn).parameters]
+        assert got[: len(params)] == params, (name, got)
+    assert inspect.signature(co.coll_torch_lookup_key_t_val_ret).parameters["pad_to_8"].default is True
+    assert inspect.signature(co.coll_torch_create_emb_shm).parameters["fname"].default == ""
+    assert co.kCollCacheAsymmLink == 13
