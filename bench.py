@@ -106,17 +106,29 @@ def parse_args():
 
 def stream_ordered_leg(C, fn, key_ptr_of, n_keys, out, stream, torch, W, K):
     """the same K steps through the stream-ordered entry point: batches are enqueued back to back, one wait at the
-    end.  Returns seconds per step."""
+    end.  Returns (wall seconds per step, seconds per launch between two HIP events recorded on the same stream right
+    before the first and right after the last of the K launches)."""
+    from ugache_amd import hip
+    ev = [ctypes.c_void_p(), ctypes.c_void_p()]
+    for e in ev:
+        hip.call("ugk_event_create", ctypes.byref(e))
     for i in range(W):
         fn(0, key_ptr_of(i), n_keys, out.data_ptr(), stream)
     C.coll_cache_lookup_wait(0, stream)
     torch.cuda.synchronize()
     t0 = time.perf_counter()
+    hip.call("ugk_event_record", ev[0], stream)
     for i in range(W, W + K):
         fn(0, key_ptr_of(i), n_keys, out.data_ptr(), stream)
+    hip.call("ugk_event_record", ev[1], stream)
     C.coll_cache_lookup_wait(0, stream)
     torch.cuda.synchronize()
-    return (time.perf_counter() - t0) / K
+    wall = (time.perf_counter() - t0) / K
+    ms = ctypes.c_float()
+    hip.call("ugk_event_elapsed_ms", ev[0], ev[1], ctypes.byref(ms))
+    for e in ev:
+        hip.call("ugk_event_destroy", e)
+    return wall, ms.value * 1e-3 / K
 
 
 def cpu_baseline(orc, table_np, keys_host, n_keys, row_bytes, seconds):
@@ -200,8 +212,8 @@ def run_all_hit(args):
     elapsed = time.perf_counter() - t0
 
     key_ptrs = [keys_pool[i].data_ptr() for i in range(pool)]
-    so_step_s = stream_ordered_leg(C, C.coll_cache_lookup_async, lambda i: key_ptrs[i % pool], n_keys, out, stream,
-                                   torch, W, K)
+    so_step_s, so_launch_s = stream_ordered_leg(C, C.coll_cache_lookup_async, lambda i: key_ptrs[i % pool], n_keys, out,
+                                                stream, torch, W, K)
 
     if args.calibrate:
         cal_src = torch.empty(1 << 30, dtype=torch.uint8, device=dev)
@@ -219,9 +231,13 @@ def run_all_hit(args):
     if out.cpu().numpy().tobytes() != orc.gather(table_np, last_keys, omp=True).tobytes():
         sys.exit("bench.py: GPU output differs from the CPU oracle — no numbers reported")
 
-    # dominant kernel: per-launch duration from the HIP events the library records around the gather on its stream
-    # (logged per step as kLogL3CacheCombineCacheTime), averaged over the K timed steps
-    kernel_avg_s = float(np.mean([_basics.step_value(s, kLogL3CacheCombineCacheTime) for s in range(W, W + K)]))
+    # dominant kernel: average launch duration over a timed region of K launches, from two HIP events on the kernel's
+    # stream around the K back-to-back launches of the stream-ordered leg (nothing else runs on that stream between
+    # them).  The library also brackets every blocking launch with an event pair of its own (logged per step as
+    # kLogL3CacheCombineCacheTime); that figure carries about 2.4 us of marker latency per launch and is reported
+    # beside it.
+    kernel_avg_s = so_launch_s
+    per_launch_pair_s = float(np.mean([_basics.step_value(s, kLogL3CacheCombineCacheTime) for s in range(W, W + K)]))
     alg_bytes = n_keys * (2 * row_bytes + 4)  # row read + row written + key read, per key
     achieved = alg_bytes / kernel_avg_s / 1e9
 
@@ -245,7 +261,9 @@ def run_all_hit(args):
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                      "frac": achieved / HBM_PEAK_GBPS, "traffic": MEASURED_TRAFFIC_BYTES.get(args.workload),
                      "kernel": "gather_kernel<u32x4,32,2,DirectU32>", "algorithmic_bytes_per_launch": alg_bytes,
-                     "avg_kernel_us": kernel_avg_s * 1e6, "keys_per_s_kernel_only": n_keys / kernel_avg_s},
+                     "avg_kernel_us": kernel_avg_s * 1e6, "keys_per_s_kernel_only": n_keys / kernel_avg_s,
+                     "timing": "2 HIP events around %d back-to-back launches on the kernel's stream" % K,
+                     "avg_kernel_us_event_pair_per_blocking_launch": per_launch_pair_s * 1e6},
         "cpu_baseline": {"value": cpu_kps, "unit": "keys/s", "cores": cores, "kind": "port",
                          "sample": "%d batches of %d keys from the same pool, %.1f s, OpenMP gather over keys"
                                    % (n_cpu, n_keys, cpu_el),
@@ -368,8 +386,8 @@ def run_mixed(args):
     note("timed region done: %.3f ms/step" % (elapsed / K * 1e3))
     g_blocking = _basics.last_group_offset(0)
     key_ptrs = [keys_pool[i].data_ptr() for i in range(pool)]
-    so_step_s = stream_ordered_leg(C, C.coll_cache_lookup_async_i64, lambda i: key_ptrs[i % pool], n_keys, out, stream,
-                                   torch, W, K)
+    so_step_s, so_launch_s = stream_ordered_leg(C, C.coll_cache_lookup_async_i64, lambda i: key_ptrs[i % pool], n_keys,
+                                                out, stream, torch, W, K)
     note("stream-ordered leg done: %.3f ms/step" % (so_step_s * 1e3))
 
     orc = Oracle()
@@ -391,6 +409,12 @@ def run_mixed(args):
         miss_bytes = n_miss * row_bytes
     fused = t_miss == 0.0 and t_idx == 0.0  # one kernel did lookup and both gathers: its time is logged as t_hit
     entry = 128 if info_cache["table_kind"] == 2 else 4  # bytes of table read per key: a bucket line / a flat word
+    per_launch_pair_us = t_hit * 1e6
+    if fused and not args.dedup:
+        # one kernel per step: its average duration over the K back-to-back launches of the stream-ordered leg (two
+        # HIP events on its stream) replaces the per-launch event pair of the blocking calls, which carries about
+        # 2.4 us of marker latency
+        t_hit = so_launch_s
     if fused:
         # HBM side of the fused kernel: key + table entry per key, hit rows read and written, missed rows written
         hit_alg = n_keys * (8 + entry) + n_hit * 2 * row_bytes + n_miss * row_bytes
@@ -499,7 +523,8 @@ def run_mixed(args):
                      "frac": achieved / HBM_PEAK_GBPS,
                      "traffic": MEASURED_TRAFFIC_BYTES.get(args.workload) if fused else None,
                      "kernel": kernel_name,
-                     "algorithmic_bytes_per_launch": hit_alg, "avg_kernel_us": t_hit * 1e6},
+                     "algorithmic_bytes_per_launch": hit_alg, "avg_kernel_us": t_hit * 1e6,
+                     "avg_kernel_us_event_pair_per_blocking_launch": per_launch_pair_us},
         "host_link": {"achieved": miss_bytes / t_link / 1e9 if t_link > 0 else 0.0, "measured_peak": link_gbps,
                       "unit": "GB/s", "frac": (miss_bytes / t_link / 1e9) / link_gbps if t_link > 0 else 0.0,
                       "miss_rows_per_batch": n_miss, "peak_probe": "pinned host -> HBM hipMemcpyAsync, best of 3"},
