@@ -433,6 +433,51 @@ def test_classify_rejects_keys_beyond_the_host_table():
     assert sorted(got[2:]["dst_off"].tolist()) == [0, 2] and sorted(got[2:]["src"].tolist()) == [5, 7]
 
 
+def test_extract_mix_skips_keys_without_a_row_and_still_hands_over_its_counts():
+    """a key beyond the host table flags the launch and leaves its output row alone; the skipped rows are counted with
+    the host rows, the count words are left at zero, and the next (clean) launch reports exact group sizes"""
+    rng = np.random.default_rng(11)
+    nkeys, rb, n = 3000, 64, 2000
+    host = _rand_table(rng, nkeys, rb)
+    mem, tb = _make_flat(nkeys)
+    cached = np.arange(0, nkeys, 3, dtype=np.uint32)
+    assert _insert(tb, cached) == 0
+    cache = host[cached].copy()
+    keys = rng.integers(0, nkeys, size=n).astype(np.int64)
+    bad = rng.choice(n, 37, replace=False)
+    dirty = keys.copy()
+    dirty[bad] = nkeys + rng.integers(0, 1 << 35, size=len(bad))
+    pin = pinned_from(host)
+    mirror = pinned_from(np.zeros(4, np.uint32))
+    try:
+        st = dev_zeros_u32(1)
+        mix_counts = dev_zeros_u32(4)
+        d_cache = to_dev(cache)
+        for batch in (dirty, keys):
+            out = dev_bytes(n * rb, fill=0x5A)
+            d_keys = to_dev(batch)
+            mirror.array[...] = 0
+            st.zero_()
+            hip.call("ugk_extract_mix_i64", tb, ptr(d_keys), n, ptr(d_cache), len(cached), pin.ptr, nkeys, ptr(out), rb,
+                     ptr(st), mirror.ptr, ptr(mix_counts), None)
+            flagged = status_value(st)
+            got = to_np(out)[: n * rb].reshape(n, rb)
+            ok = batch < nkeys
+            assert got[ok].tobytes() == host[batch[ok]].tobytes()
+            assert (got[~ok] == 0x5A).all()
+            local = int((batch[ok] % 3 == 0).sum())
+            assert mirror.array.tolist()[1:3] == [local, n - local]
+            assert not to_np(mix_counts, np.uint32)[:3].any()
+            if ok.all():
+                assert flagged == 0 and mirror.array[0] == 0
+            else:
+                assert flagged & hip.ST_KEY_OUT_OF_RANGE and mirror.array[0] == hip.ST_KEY_OUT_OF_RANGE
+    finally:
+        sync()
+        pin.free()
+        mirror.free()
+
+
 @pytest.mark.parametrize("row_bytes", [128, 64, 1024])
 def test_extract_mix_other_row_sizes(row_bytes):
     rng = np.random.default_rng(row_bytes)

@@ -146,9 +146,11 @@ __global__ __launch_bounds__(kBlock) void extract_mix_kernel(ugk_table_t t, cons
     }
     const uint64_t rowbits = reinterpret_cast<uint64_t>(rowp);
     if (counts) {
+      // rows from the cache, and all others (host rows, and rows skipped for a key without a row: the launch is
+      // flagged then and its group sizes mean nothing, but the two sums still add up to n)
       const bool from_cache = rowp != nullptr && f.hit && f.loc == UGK_LOC_LOCAL;
       wave_local += __popcll(__ballot(from_cache));
-      wave_host += __popcll(__ballot(rowp != nullptr && !from_cache));
+      wave_host += __popcll(__ballot(active && !from_cache));
     }
     for (int r0 = 0; r0 < kWave; r0 += RPW * UNROLL) {
       const u32x4 *p[UNROLL];
@@ -173,28 +175,26 @@ __global__ __launch_bounds__(kBlock) void extract_mix_kernel(ugk_table_t t, cons
     }
   }
   if (counts == nullptr) return;
-  // Group sizes for the host.  Every workgroup adds its two sums with ONE 64-bit atomic and then takes a ticket; the
-  // workgroup that draws the last ticket hands the totals to the pinned mirror and leaves the words at zero for the
-  // next launch.  No memory fence anywhere: a device-scope fence per workgroup would write back and invalidate the
-  // L2 of its XCD thousands of times per launch.  Atomics are performed at the point of coherence, and the ticket is
-  // made to depend on the value the first atomic returned, so it cannot be issued before that atomic has been
-  // performed.
+  // Group sizes for the host.  Every workgroup adds its two sums with ONE 64-bit atomic; every key is counted in
+  // exactly one of them, so the workgroup whose add brings their total to n is the last one: it hands the totals to
+  // the pinned mirror and leaves the words at zero for the next launch.  No memory fence and no second atomic: a
+  // device-scope fence per workgroup would write back and invalidate the L2 of its XCD thousands of times per launch,
+  // and atomics on one address are performed one after the other at the memory side (about 8 ns each), which a
+  // thousand workgroups finishing together feel.
   if (lane == 0) {
     if (wave_local) atomicAdd(&block_tot[0], wave_local);
     if (wave_host) atomicAdd(&block_tot[1], wave_host);
   }
   __syncthreads();
-  if (threadIdx.x == 0) {
-    unsigned long long *pair = reinterpret_cast<unsigned long long *>(counts);  // low word local, high word host
+  if (threadIdx.x == 0 && (block_tot[0] | block_tot[1])) {
+    unsigned long long *pair = reinterpret_cast<unsigned long long *>(counts);  // low word local, high word others
     const unsigned long long mine = ((unsigned long long)block_tot[1] << 32) | block_tot[0];
-    const unsigned long long before = atomicAdd(pair, mine);
-    const uint32_t never = before == ~0ull ? 1u : 0u;  // always 0 (the sums stay below 2^32); carries the dependency
-    if (atomicAdd(counts + 2, 1u + never) == gridDim.x - 1) {
-      const unsigned long long total = atomicExch(pair, 0ull);
-      atomicExch(counts + 2, 0u);
+    const unsigned long long after = atomicAdd(pair, mine) + mine;
+    if ((after & 0xffffffffull) + (after >> 32) == (unsigned long long)n) {
+      atomicExch(pair, 0ull);
       if (host_mirror) {
-        host_mirror[1 + UGK_LOC_LOCAL] = (uint32_t)total;
-        host_mirror[1 + UGK_LOC_HOST] = (uint32_t)(total >> 32);
+        host_mirror[1 + UGK_LOC_LOCAL] = (uint32_t)after;
+        host_mirror[1 + UGK_LOC_HOST] = (uint32_t)(after >> 32);
       }
     }
   }
@@ -359,6 +359,7 @@ int extract_mix(ugk_table_t t, const K *keys, size_t n, const void *cache, uint6
   if (n == 0) return 0;
   UGK_REQUIRE(keys && out && status, "ugk_extract_mix: null keys, output or status");
   UGK_REQUIRE((uintptr_t)counts % 8 == 0, "ugk_extract_mix: the count words must be 8-byte aligned");
+  UGK_REQUIRE(n <= 0xffffffffull, "ugk_extract_mix: batch of %zu keys exceeds 2^32", n);
   UGK_REQUIRE(t.kind == 1 || t.kind == 2, "ugk_extract_mix: table kind %d is not flat(1) or hash(2)", t.kind);
   UGK_REQUIRE(t.table && t.size, "ugk_extract_mix: empty table");
   if (t.kind == 2)
