@@ -94,6 +94,10 @@ def parse_args():
     ap.add_argument("--concurrent-refresh", action="store_true",
                     help="sparse-id workloads, with --gpu-record: after the timed steps, time the lookups again while "
                          "a second thread refreshes the cache back to back from the device-side hotness counters")
+    ap.add_argument("--device-refresh", action="store_true",
+                    help="sparse-id workloads: COLL_GPU_RECORD=1 COLL_GPU_REFRESH=1 COLL_GPU_REFRESH_KEEP=1; after the "
+                         "timed steps, time steps that each end with a refresh computed on the device from the "
+                         "accumulated hotness, with 1 %% of the cache replaced per step")
     ap.add_argument("--calibrate", action="store_true",
                     help="also run 5 plain device copies of 1 GiB (ugk_copy_rows) so a counter run has a kernel of "
                          "known traffic next to the gather")
@@ -308,6 +312,10 @@ def run_mixed(args):
         os.environ["SAMGRAPH_COLL_CACHE_CONCURRENT_LINK_IMPL"] = args.impl
     if args.dedup:
         os.environ["COLL_DEDUP_KEYS"] = "1"
+    if args.device_refresh:
+        args.gpu_record = True
+        os.environ["COLL_GPU_REFRESH"] = "1"
+        os.environ["COLL_GPU_REFRESH_KEEP"] = "1"
     if args.gpu_record:
         os.environ["COLL_GPU_RECORD"] = "1"
     co.config({"cache_percentage": pct, "_cache_policy": co.kCollCacheAsymmLink, "num_device": 1,
@@ -436,7 +444,50 @@ def run_mixed(args):
     uniq = float(np.mean([len(np.unique(keys_host[i])) for i in range(min(pool, 4))]))
 
     refresh = None
-    if sparse:
+    each_step = None
+    if sparse and args.device_refresh:
+        # Every step ends with a refresh computed on the device from the hotness accumulated so far.  Hotness drifts by
+        # 1 % of the cache per step: a slice of so-far never-looked-up rows is looked up once between the steps
+        # (untimed), which ranks them above the never-observed rows the cache is filled up with, so each refresh evicts
+        # and inserts at least that many rows.
+        before = _basics.info(0)
+        n_new = before["cached_rows"] // 100
+        t0 = time.perf_counter()
+        co.coll_torch_refresh(0, True)  # settles the cache on what the timed steps counted
+        settle_s = time.perf_counter() - t0
+        note("first refresh on the device (settling): %.4f s" % settle_s)
+        n_steps = min(K, 20)
+        t_lookup = t_refresh = 0.0
+        cold_end = per_field
+        for i in range(n_steps):
+            cold = perms[0][cold_end - n_new:cold_end]
+            cold_end -= n_new
+            drift = ids_of(cold).contiguous()
+            C.coll_cache_lookup_i64(0, drift.data_ptr(), n_new, out.data_ptr(), stream)
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            step(i)
+            torch.cuda.synchronize()
+            t1 = time.perf_counter()
+            co.coll_torch_refresh(0, True)
+            t2 = time.perf_counter()
+            t_lookup += t1 - t0
+            t_refresh += t2 - t1
+        after = _basics.info(0)
+        step(0)
+        torch.cuda.synchronize()
+        if out.cpu().numpy().tobytes() != orc.gather(table_np, rows_pool[0].cpu().numpy(), omp=True).tobytes():
+            sys.exit("bench.py: GPU output differs from the CPU oracle after the per-step refreshes")
+        each_step = {"steps": n_steps, "lookup_ms": t_lookup / n_steps * 1e3, "refresh_ms": t_refresh / n_steps * 1e3,
+                     "ms_per_step": (t_lookup + t_refresh) / n_steps * 1e3,
+                     "keys_per_s": n_keys * n_steps / (t_lookup + t_refresh),
+                     "drift_rows_looked_up_per_step": n_new, "first_refresh_s": settle_s,
+                     "table_rebuilds": after["table_rebuilds"], "cached_rows_after": after["cached_rows"],
+                     "free_slots_after": after["free_slots"],
+                     "note": "refresh = rank + place + evict/insert lists on the device (COLL_GPU_REFRESH=1, hotness "
+                             "accumulating), row copy over the host link, table update; foreground, after each lookup"}
+        note("refresh each step: lookup %.3f ms + refresh %.3f ms" % (each_step["lookup_ms"], each_step["refresh_ms"]))
+    elif sparse:
         # one foreground refresh: the same hotness again, plus 1 % of the cache size worth of so-far uncached rows
         # pushed to the top, so that about 1 % of the cached rows are evicted and replaced
         before = _basics.info(0)
@@ -507,12 +558,12 @@ def run_mixed(args):
         "value": keys_per_s, "unit": "keys/s", "n_gpus": 1, "steps": K, "warmup": W,
         "ms_per_step": elapsed / K * 1e3, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "u8", "data": "synthetic",
-        "refresh": refresh, "under_concurrent_refresh": under_refresh,
+        "refresh": refresh, "refresh_each_step": each_step, "under_concurrent_refresh": under_refresh,
         "config": {"workload": args.workload, "table_rows": rows, "row_bytes": row_bytes, "keys_per_batch": n_keys,
                    "key_dtype": "int64", "sparse_ids": sparse, "cache_percentage": pct, "cached_rows": info_cache["cached_rows"],
                    "cache_capacity_rows": info_cache["capacity_rows"], "table_kind": info_cache["table_kind"],
                    "zipf_s": spec["zipf"], "fields": fields, "presample_batches": spec["presample"],
-                   "entry_point": "coll_cache_lookup_i64", "distinct_key_batches": pool, "impl": args.impl or "fused (default)", "dedup": bool(args.dedup), "gpu_record": bool(args.gpu_record),
+                   "entry_point": "coll_cache_lookup_i64", "distinct_key_batches": pool, "impl": args.impl or "fused (default)", "dedup": bool(args.dedup), "gpu_record": bool(args.gpu_record), "device_refresh": bool(args.device_refresh),
                    "unique_keys_per_batch": uniq, "seeds": {"table": 1, "perm": 2, "keys": 3}},
         "effective_extraction_GBps": n_keys * row_bytes / (elapsed / K) / 1e9,
         "parity": "bit-exact vs CPU oracle (last timed batch)",

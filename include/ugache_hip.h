@@ -246,6 +246,43 @@ int ugk_record_i64(const int64_t *keys_dev, size_t n, uint64_t key_inv, uint64_t
 int ugk_record_drain(uint32_t *counts_dev, uint64_t first_row, uint64_t num_rows, uint64_t *entries_dev,
                      uint32_t capacity, uint32_t *n_entries_dev, uint32_t *host_out, void *stream);
 
+/* ---- re-placement on the device, from the counters of ugk_record_* ---------------------------------------------
+ * Stands, for hotness counted on the device, for the host passes of a refresh: FreqRecorder::Sort
+ * (freq_recorder.cc:275-281), RepSolver::Solve (optimal_solver_class.cc:1869-1924) and the key-list scans
+ * DetectKeysForAllSource / DetectKeysWithCond (cache_hashtable.cuh:693-835) behind
+ * RefreshSession::refresh_after_solve_new (cache_context.cu:3944-4107).
+ * Rank of row r with counter c: c > 0: (c << 32) | r;  c == 0: 0xffffffff - r  (never-counted rows rank behind all
+ * counted ones, in ascending row order).  All ranks are distinct.
+ * ugk_rank_select: leaves in ws_dev (ugk_rank_workspace_bytes() bytes, 8-byte aligned) the k-th largest rank of
+ * rows [0, num_rows) as a threshold (k == 0: nothing reaches it; k >= num_rows: every row does).  counts_dev
+ * must be 16-byte aligned; num_rows < 2^32 - 1.  Six streaming passes over the counters; no host round trip.
+ * ugk_rank_threshold: copies the threshold to the host (blocking; for tests and logs).
+ * ugk_rank_mark: bit r of bitmap_dev (ceil(num_rows / 64) words, every word written) = rank(r) >= threshold;
+ * with reset_counts != 0 the counters are zeroed in the same pass. */
+size_t ugk_rank_workspace_bytes(void);
+int ugk_rank_select(const uint32_t *counts_dev, uint64_t num_rows, uint64_t k, void *ws_dev, void *stream);
+int ugk_rank_threshold(const void *ws_dev, uint64_t *threshold_host, void *stream);
+int ugk_rank_mark(uint32_t *counts_dev, uint64_t num_rows, const void *ws_dev, uint64_t *bitmap_dev, int reset_counts,
+                  void *stream);
+/* Ordered compaction over bitmaps.  The set S = { p < nbits : bit p of m is set }, m = (invert_a ? ~a : a) & ~b
+ * (b_dev may be NULL).  ugk_bitmap_count writes |S| to *total_host (pinned host word, may be NULL) and leaves the
+ * per-chunk offsets in ws_dev (ugk_bitmap_workspace_bytes() bytes); ugk_bitmap_emit, called with the same a, b,
+ * invert_a and nbits while the bitmaps are unchanged, writes the first max_out elements of S in ascending order.
+ * With these, evict = cached & ~new, insert = new & ~cached and free slots = ~used are the same three launches
+ * (the set algebra of cache_context.cu:3975-4003).  nbits <= 2^32 - 1. */
+size_t ugk_bitmap_workspace_bytes(void);
+int ugk_bitmap_count(const uint64_t *a_dev, const uint64_t *b_dev, int invert_a, uint64_t nbits, void *ws_dev,
+                     uint32_t *total_host, void *stream);
+int ugk_bitmap_emit(const uint64_t *a_dev, const uint64_t *b_dev, int invert_a, uint64_t nbits, const void *ws_dev,
+                    uint32_t *out_dev, uint64_t max_out, void *stream);
+/* sets (set != 0) or clears the bits listed in idx_dev; a position >= nbits flags UGK_ST_KEY_OUT_OF_RANGE */
+int ugk_bitmap_update(uint64_t *bitmap_dev, uint64_t nbits, const uint32_t *idx_dev, size_t n, int set,
+                      uint32_t *status_dev, void *stream);
+/* sparse-id mode: caller-side id of each listed host row, (row * mul) & mask (the inverse of the map ugk_table_t
+ * carries in fb_mul / fb_mask) */
+int ugk_rows_to_keys(const uint32_t *rows_dev, size_t n, uint64_t mul, uint64_t mask, int64_t *keys_out_dev,
+                     void *stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -42,7 +42,8 @@ def make_config(num_total_item, pct, threads=8):
 @pytest.fixture(autouse=True)
 def _fresh_cache(monkeypatch):
     for v in ("COLL_HASH_TABLE", "SAMGRAPH_COLL_CACHE_CONCURRENT_LINK_IMPL", "SAMGRAPH_COLL_CACHE_NO_GROUP",
-              "COLL_DEDUP_KEYS", "COLL_DEDUP_MIN_KEYS", "COLL_GPU_RECORD", "COLL_GPU_RECORD_EVERY"):
+              "COLL_DEDUP_KEYS", "COLL_DEDUP_MIN_KEYS", "COLL_GPU_RECORD", "COLL_GPU_RECORD_EVERY", "COLL_GPU_REFRESH",
+              "COLL_GPU_REFRESH_KEEP"):
         monkeypatch.delenv(v, raising=False)
     yield
     if torch.cuda.is_available():
@@ -361,6 +362,93 @@ def test_refresh_evicts_and_inserts_like_the_oracle(table_kind, foreground, impl
         old_cached = new_cached
 
 
+@pytest.mark.parametrize("table_kind", ["FLAT", "HASH"])
+@pytest.mark.parametrize("foreground", [True, False])
+@pytest.mark.parametrize("keep", [False, True])
+def test_refresh_on_the_device_places_like_the_oracle(table_kind, foreground, keep, monkeypatch):
+    """COLL_GPU_RECORD=1 + COLL_GPU_REFRESH=1: ranking, placement and the evict / insert lists of a refresh are computed
+    on the device from the hotness the lookups counted there.  The cached set afterwards is the oracle's top set of the
+    counted key stream (of the last interval, or of everything so far with COLL_GPU_REFRESH_KEEP=1), exactly as after
+    a refresh on the host; the two kinds of refresh can alternate."""
+    monkeypatch.setenv("COLL_HASH_TABLE", table_kind)
+    monkeypatch.setenv("COLL_GPU_RECORD", "1")
+    monkeypatch.setenv("COLL_GPU_REFRESH", "1")
+    if keep:
+        monkeypatch.setenv("COLL_GPU_REFRESH_KEEP", "1")
+    monkeypatch.setenv("COLL_REFRESH_SLEEP_US", "100")
+    monkeypatch.setenv("COLL_REFRESH_BATCH_ROWS", "512")
+    rng = np.random.default_rng(21)
+    n_item, dim, pct = 50_001, 64, 0.2
+    co.config(make_config(n_item, pct))
+    co.coll_cache_record_init(0)
+    perm = rng.permutation(n_item)
+    s0 = perm[zipf_ranks(rng, 150_000, n_item, 1.05)]
+    co.coll_torch_record(0, torch.from_numpy(s0).to(torch.int32))
+    emb = co.coll_torch_create_emb_shm(0, n_item, dim, torch.float32)
+    table = fill_table(emb, rng)
+    co.coll_torch_init_t(0, 0, emb, pct)
+    cached, nid = expected_cached_set(s0.astype(np.uint32), n_item, pct)
+    cap = _basics.info(0)["capacity_rows"]
+    counted = []  # what the device-side counters hold
+
+    def lookup(keys, want_nid):
+        out = co.coll_torch_lookup_key_t_val_ret(0, torch.from_numpy(keys).to(torch.int32).cuda(), False)
+        counted.append(keys.astype(np.uint32))
+        assert out.cpu().numpy().tobytes() == ORC.gather(table, keys.astype(np.int64)).tobytes()
+        if want_nid is not None:
+            assert _basics.last_group_offset(0)[1] == int((want_nid[keys] == 0).sum())
+
+    def refresh():
+        if foreground:
+            co.coll_torch_refresh(0, True)
+            return
+        t = threading.Thread(target=co.coll_torch_refresh, args=(0, False))
+        t.start()
+        while t.is_alive():  # a background refresh waits for one more lookup to pass; these are not counted
+            out = co.coll_torch_lookup_key_t_val_ret(0, torch.zeros(0, dtype=torch.int32).cuda(), False)
+            assert out.shape[0] == 0
+            time.sleep(0.001)
+        t.join()
+
+    def check_cached(want):
+        info = _basics.info(0)
+        assert info["cached_rows"] == len(want) and info["free_slots"] + info["cached_rows"] == cap
+        got = np.zeros(len(want), np.uint32)
+        assert _basics.C_LIB_CTYPES.coll_cache_get_cached_keys(0, got.ctypes.data, len(got)) == len(want)
+        assert np.array_equal(got, want)
+        info = _basics.info(0)  # the same from the host-side lists, now up to date
+        assert info["cached_rows"] == len(want) and info["free_slots"] + info["cached_rows"] == cap
+
+    for rnd in range(3):
+        swap = rng.choice(n_item, n_item // 10, replace=False)
+        perm[swap] = perm[rng.permutation(swap)]
+        for n in (30_000, 1, 40_000):
+            lookup(perm[zipf_ranks(rng, n, n_item, 1.05)], nid)
+        refresh()
+        new_cached, nid = expected_cached_set(np.concatenate(counted), n_item, pct)
+        assert len(np.setdiff1d(cached, new_cached)) > 200  # the refresh really moved rows
+        if not keep:
+            counted.clear()
+        check_cached(new_cached)
+        cached = new_cached
+        lookup(rng.integers(0, n_item, size=20_000), nid)
+
+    # a refresh on the host in between (hotness recorded on the host joins the device-side counts) ...
+    extra = perm[zipf_ranks(rng, 60_000, n_item, 1.3)]
+    co.coll_torch_record(0, torch.from_numpy(extra).to(torch.int32))
+    co.coll_torch_refresh(0, True)
+    cached, nid = expected_cached_set(np.concatenate(counted + [extra.astype(np.uint32)]), n_item, pct)
+    counted.clear()  # the host refresh drained the counters
+    check_cached(cached)
+    lookup(rng.integers(0, n_item, size=20_000), nid)
+    # ... and the device takes over again from the host-side lists
+    lookup(perm[zipf_ranks(rng, 50_000, n_item, 0.9)], nid)
+    refresh()
+    cached, nid = expected_cached_set(np.concatenate(counted), n_item, pct)
+    check_cached(cached)
+    lookup(rng.integers(0, n_item, size=20_000), nid)
+
+
 @pytest.mark.parametrize("pct,impl,dedup", [(0.25, "", False), (0.25, "NONE", True), (0.25, "SMMaskPhase", False),
                                             (1.0, "", False), (0.0, "", True)])
 @pytest.mark.parametrize("kdtype", [torch.int32, torch.int64])
@@ -644,7 +732,7 @@ def test_reference_cpu_runnable_config_full_size():
         assert _basics.last_group_offset(0) == [0, int((nid[b] == 0).sum()), n]
 
 
-@pytest.mark.parametrize("gpu_record", [False, True])
+@pytest.mark.parametrize("gpu_record", [False, True, "and_refresh"])
 def test_sparse_ids_hash_table_with_refresh_each_step(gpu_record, monkeypatch):
     """The hashtable-mode configuration, scaled down: ids are 64-bit values from a 2^40 space (id = row * odd mod 2^40),
     rows are 64 fp16 (128 B), the cached ids sit in the open-addressing table at 0.7 load, every step is followed by a
@@ -652,6 +740,8 @@ def test_sparse_ids_hash_table_with_refresh_each_step(gpu_record, monkeypatch):
     monkeypatch.setenv("COLL_HASH_REBUILD_FRAC", "0.05")
     if gpu_record:  # the hotness of a refresh comes from the lookups themselves, counted per row on the device
         monkeypatch.setenv("COLL_GPU_RECORD", "1")
+    if gpu_record == "and_refresh":  # ... and is ranked, placed and turned into evict / insert lists there too
+        monkeypatch.setenv("COLL_GPU_REFRESH", "1")
     MUL, BITS = 0x9E3779B97F4A7C15, 40
     mask = np.uint64((1 << BITS) - 1)
     rng = np.random.default_rng(5)

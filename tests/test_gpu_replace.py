@@ -1,0 +1,185 @@
+"""GPU parity of the device-side re-placement kernels (rank select, membership bitmap, ordered bitmap compaction)
+against numpy: a full sort for the rank threshold, flatnonzero for the compactions."""
+import ctypes as C
+
+import numpy as np
+import pytest
+
+from gpu_util import PinnedArray, dev_bytes, dev_zeros_u32, ptr, status_value, sync, to_dev, to_np
+from ugache_amd import hip
+
+pytestmark = pytest.mark.gpu
+
+
+def ranks_of(counts):
+    """observed rows by (count << 32 | row), never-observed rows behind them in ascending row order
+    (freq_recorder.cc:275-281 for the observed ones)"""
+    rows = np.arange(len(counts), dtype=np.uint64)
+    c = counts.astype(np.uint64)
+    return np.where(c > 0, (c << np.uint64(32)) | rows, np.uint64(0xFFFFFFFF) - rows)
+
+
+def _counts(rng, n, kind):
+    if kind == "zipf":  # most rows never observed, a few hot
+        c = np.zeros(n, np.uint32)
+        hit = rng.zipf(1.2, size=max(n // 2, 1)) % n
+        np.add.at(c, hit, 1)
+        return c
+    if kind == "ties":  # few distinct values: the row number decides
+        return rng.integers(0, 3, size=n).astype(np.uint32)
+    if kind == "huge":  # counts in every digit of the 32 bits
+        return (rng.integers(0, 1 << 32, size=n, dtype=np.uint64) * (rng.random(n) < 0.7)).astype(np.uint32)
+    if kind == "zero":
+        return np.zeros(n, np.uint32)
+    raise AssertionError(kind)
+
+
+def _select(counts, k):
+    n = len(counts)
+    d_counts = to_dev(counts)
+    ws = dev_bytes(hip.lib().ugk_rank_workspace_bytes())
+    hip.call("ugk_rank_select", ptr(d_counts), n, k, ptr(ws), None)
+    th = C.c_uint64(0)
+    hip.call("ugk_rank_threshold", ptr(ws), C.byref(th), None)
+    return d_counts, ws, th.value
+
+
+@pytest.mark.parametrize("kind", ["zipf", "ties", "huge", "zero"])
+@pytest.mark.parametrize("n", [1, 3, 63, 64, 65, 1000, 100_003, 2_000_001])
+def test_rank_select_and_mark_match_a_full_sort(kind, n):
+    rng = np.random.default_rng(n * 7 + len(kind))
+    counts = _counts(rng, n, kind)
+    ranks = ranks_of(counts)
+    order = np.sort(ranks)[::-1]
+    observed = int((counts > 0).sum())
+    ks = sorted({0, 1, n // 3, max(observed - 1, 0), observed, min(observed + 1, n), n - 1, n, n + 5})
+    for k in ks:
+        d_counts, ws, th = _select(counts, k)
+        if k == 0:
+            want = np.zeros(n, bool)
+        elif k >= n:
+            want = np.ones(n, bool)
+        else:
+            assert th == int(order[k - 1]), (kind, n, k)
+            want = ranks >= order[k - 1]
+        assert int(want.sum()) == min(k, n)
+        words = (n + 63) // 64
+        for reset in (0, 1):
+            bitmap = dev_bytes(words * 8, fill=0xA5)
+            hip.call("ugk_rank_mark", ptr(d_counts), n, ptr(ws), ptr(bitmap), reset, None)
+            sync()
+            got = np.unpackbits(to_np(bitmap)[: words * 8], bitorder="little")
+            assert np.array_equal(got[:n].astype(bool), want), (kind, n, k, reset)
+            assert not got[n:].any()  # the tail of the last word is clear
+            left = to_np(d_counts, np.uint32)[:n]
+            assert np.array_equal(left, counts if reset == 0 else np.zeros(n, np.uint32))
+
+
+def test_rank_select_picks_the_hotter_rows_and_breaks_ties_towards_larger_rows():
+    # hand-worked: counts 0 5 5 0 9 1 0 -> order 4, 2, 1, 5, then the never-observed rows 0, 3, 6
+    counts = np.array([0, 5, 5, 0, 9, 1, 0], np.uint32)
+    for k, want_rows in [(1, [4]), (2, [4, 2]), (3, [4, 2, 1]), (4, [4, 2, 1, 5]), (5, [4, 2, 1, 5, 0]),
+                         (6, [4, 2, 1, 5, 0, 3])]:
+        d_counts, ws, _ = _select(counts, k)
+        bitmap = dev_bytes(8)
+        hip.call("ugk_rank_mark", ptr(d_counts), len(counts), ptr(ws), ptr(bitmap), 0, None)
+        sync()
+        got = np.flatnonzero(np.unpackbits(to_np(bitmap)[:8], bitorder="little"))
+        assert sorted(got.tolist()) == sorted(want_rows)
+
+
+def _bits(rng, nbits, density):
+    words = (nbits + 63) // 64
+    b = rng.random(words * 64) < density
+    return np.packbits(b, bitorder="little").view(np.uint64), b
+
+
+@pytest.mark.parametrize("nbits", [1, 64, 65, 4097, 1_000_003, 40_000_000])
+@pytest.mark.parametrize("mode", ["a", "not_a", "a_and_not_b", "not_a_and_not_b"])
+def test_bitmap_compaction_matches_flatnonzero(nbits, mode):
+    rng = np.random.default_rng(nbits % 1000 + len(mode))
+    a_w, a = _bits(rng, nbits, 0.02 if nbits > 10_000_000 else 0.3)
+    b_w, b = _bits(rng, nbits, 0.5)
+    m = a.copy()
+    if mode.startswith("not_a"):
+        m = ~m
+    use_b = mode.endswith("not_b")
+    if use_b:
+        m &= ~b
+    m[nbits:] = False
+    want = np.flatnonzero(m).astype(np.uint32)
+    d_a, d_b = to_dev(a_w), to_dev(b_w)
+    ws = dev_bytes(hip.lib().ugk_bitmap_workspace_bytes())
+    total = PinnedArray((4,), np.uint32)
+    try:
+        total.array[...] = 0xFFFFFFFF
+        inv = 1 if mode.startswith("not_a") else 0
+        hip.call("ugk_bitmap_count", ptr(d_a), ptr(d_b) if use_b else None, inv, nbits, ptr(ws), total.ptr, None)
+        sync()
+        assert int(total.array[0]) == len(want)
+        for max_out in sorted({len(want), len(want) // 2, 1}):
+            out = dev_zeros_u32(max(len(want), 1) + 8)
+            out.fill_(-1)
+            hip.call("ugk_bitmap_emit", ptr(d_a), ptr(d_b) if use_b else None, inv, nbits, ptr(ws), ptr(out), max_out,
+                     None)
+            sync()
+            got = to_np(out, np.uint32)
+            lim = min(max_out, len(want))
+            assert np.array_equal(got[:lim], want[:lim])
+            assert (got[lim: lim + 8] == 0xFFFFFFFF).all()  # nothing written beyond the limit
+    finally:
+        sync()
+        total.free()
+
+
+def test_bitmap_compaction_of_an_empty_and_a_full_set():
+    nbits = 70_000
+    ws = dev_bytes(hip.lib().ugk_bitmap_workspace_bytes())
+    total = PinnedArray((4,), np.uint32)
+    try:
+        zero = to_dev(np.zeros((nbits + 63) // 64, np.uint64))
+        hip.call("ugk_bitmap_count", ptr(zero), None, 0, nbits, ptr(ws), total.ptr, None)
+        sync()
+        assert total.array[0] == 0
+        hip.call("ugk_bitmap_count", ptr(zero), None, 1, nbits, ptr(ws), total.ptr, None)
+        out = dev_zeros_u32(nbits)
+        hip.call("ugk_bitmap_emit", ptr(zero), None, 1, nbits, ptr(ws), ptr(out), nbits, None)
+        sync()
+        assert total.array[0] == nbits
+        assert np.array_equal(to_np(out, np.uint32)[:nbits], np.arange(nbits, dtype=np.uint32))
+    finally:
+        sync()
+        total.free()
+
+
+def test_bitmap_update_sets_and_clears_listed_bits():
+    rng = np.random.default_rng(5)
+    nbits = 123_457
+    w, b = _bits(rng, nbits, 0.4)
+    d = to_dev(w)
+    st = dev_zeros_u32(1)
+    on = rng.choice(nbits, 5000, replace=False).astype(np.uint32)
+    off = rng.choice(nbits, 7000, replace=False).astype(np.uint32)
+    d_on, d_off = to_dev(on), to_dev(off)
+    hip.call("ugk_bitmap_update", ptr(d), nbits, ptr(d_on), len(on), 1, ptr(st), None)
+    hip.call("ugk_bitmap_update", ptr(d), nbits, ptr(d_off), len(off), 0, ptr(st), None)
+    assert status_value(st) == 0
+    b[on] = True
+    b[off] = False
+    got = np.unpackbits(to_np(d, np.uint8)[: len(w) * 8], bitorder="little").astype(bool)
+    assert np.array_equal(got, b)
+    bad = to_dev(np.array([3, nbits], np.uint32))
+    hip.call("ugk_bitmap_update", ptr(d), nbits, ptr(bad), 2, 1, ptr(st), None)
+    assert status_value(st) & hip.ST_KEY_OUT_OF_RANGE
+
+
+def test_rows_to_keys_is_the_forward_id_map():
+    rng = np.random.default_rng(9)
+    bits, mul = 40, 0x9E3779B97F4A7C15 | 1
+    rows = rng.integers(0, 1 << 31, size=10_001).astype(np.uint32)
+    d_rows = to_dev(rows)
+    out = dev_bytes(len(rows) * 8)
+    hip.call("ugk_rows_to_keys", ptr(d_rows), len(rows), mul, (1 << bits) - 1, ptr(out), None)
+    sync()
+    want = np.array([(int(r) * mul) & ((1 << bits) - 1) for r in rows], np.int64)
+    assert np.array_equal(to_np(out, np.int64)[: len(rows)], want)

@@ -20,7 +20,8 @@ INCLUDE = os.path.join(ROOT, "include")
 HIP_LIB = os.path.join(PKG, "libugache_hip.so")
 HOST_LIB = os.path.join(PKG, "libcoll_cache.so")
 
-HIP_SOURCES = ["ugk_runtime.hip", "ugk_gather.hip", "ugk_table.hip", "ugk_partition.hip", "ugk_hotness.hip"]
+HIP_SOURCES = ["ugk_runtime.hip", "ugk_gather.hip", "ugk_table.hip", "ugk_partition.hip", "ugk_hotness.hip",
+               "ugk_refresh.hip"]
 
 HIPCC_FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-shared",

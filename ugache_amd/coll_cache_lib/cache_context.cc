@@ -243,6 +243,7 @@ ExtractSession::ExtractSession(std::shared_ptr<CacheContext> cache_ctx) : _cache
     UGK_CALL(ugk_stream_create(&_record_stream));
     UGK_CALL(ugk_event_create(&_ev_rec_begin));
     UGK_CALL(ugk_event_create(&_ev_rec_done));
+    UGK_CALL(ugk_event_create(&_ev_placed));
     UGK_CALL(ugk_stream_sync(nullptr));
   }
 }
@@ -251,6 +252,7 @@ ExtractSession::~ExtractSession() {
   if (_record_stream) ugk_stream_destroy(_record_stream);
   if (_ev_rec_begin) ugk_event_destroy(_ev_rec_begin);
   if (_ev_rec_done) ugk_event_destroy(_ev_rec_done);
+  if (_ev_placed) ugk_event_destroy(_ev_placed);
   ugk_stream_destroy(_local_ext_stream);
   ugk_stream_destroy(_cpu_ext_stream);
   ugk_event_destroy(_ev_classified);
@@ -332,6 +334,7 @@ void ExtractSession::RecordKeys(const KeyT *nodes, size_t num_nodes, StreamHandl
   if (!_hot_counts || (_num_lookups++ % RunConfig::gpu_record_every) != 0) return;
   num_nodes = std::min(num_nodes, _record_limit);
   if (num_nodes == 0) return;
+  std::lock_guard<std::mutex> guard(_drain_mu);  // not in the middle of a placement's passes
   if (after == nullptr) {
     UGK_CALL(ugk_event_record(_ev_rec_begin, stream));
     after = _ev_rec_begin;
@@ -347,6 +350,18 @@ void ExtractSession::JoinRecord(StreamHandle stream) {
   if (!_record_pending) return;
   UGK_CALL(ugk_stream_wait_event(stream, _ev_rec_done));
   _record_pending = false;
+}
+
+void ExtractSession::PlaceOnDevice(size_t num_cached, uint64_t *in_new_bits, void *rank_ws, bool reset_counts,
+                                   StreamHandle stream) {
+  CHECK_NOTNULL(_hot_counts) << "placement on the device needs the device-side hotness counters (COLL_GPU_RECORD=1)";
+  const size_t rows = _cache_ctx->_num_total_nodes;
+  std::lock_guard<std::mutex> guard(_drain_mu);
+  UGK_CALL(ugk_rank_select(_hot_counts->ptr<uint32_t>(), rows, num_cached, rank_ws, _record_stream));
+  UGK_CALL(ugk_rank_mark(_hot_counts->ptr<uint32_t>(), rows, rank_ws, in_new_bits, reset_counts ? 1 : 0,
+                         _record_stream));
+  UGK_CALL(ugk_event_record(_ev_placed, _record_stream));
+  UGK_CALL(ugk_stream_wait_event(stream, _ev_placed));
 }
 
 size_t ExtractSession::DrainHotness(FreqRecorder *recorder) {
@@ -719,6 +734,31 @@ TensorPtr RefreshSession::CopyTo1DReuse(TensorPtr &preserved_buffer, TensorPtr s
   return ret;
 }
 
+void RefreshSession::CopyRowsIntoSlots(const uint32_t *rows_dev, const uint32_t *slots_dev, size_t num_rows,
+                                       bool foreground) {
+  CacheContext *ctx = _cache_ctx.get();
+  const void *host = ctx->_device_cache_data[ctx->_cpu_location_id];
+  void *cache = ctx->_device_cache_data[ctx->_local_location_id];
+  uint32_t *status = _status_handle->ptr<uint32_t>();
+  // background refresh copies in small throttled batches so that foreground lookups keep the host link
+  const size_t batch = foreground ? num_rows : std::max<size_t>(RunConfig::refresh_batch_rows, 1);
+  const unsigned limit_block = foreground ? 0 : RunConfig::refresh_limit_block;
+  for (size_t begin = 0; begin < num_rows; begin += batch) {
+    const size_t cur = std::min(batch, num_rows - begin);
+    UGK_CALL(ugk_gather_scatter_u32(host, ctx->_num_total_nodes, rows_dev + begin, slots_dev + begin, cur, cache,
+                                    ctx->_cache_space_capacity, ctx->_row_bytes, limit_block, status, nullptr,
+                                    low_pri_stream));
+    if (!foreground && begin + batch < num_rows) {
+      UGK_CALL(ugk_stream_sync(low_pri_stream));
+      usleep(RunConfig::refresh_sleep_us);
+    }
+  }
+  uint32_t st = 0;
+  UGK_CALL(ugk_memcpy_async(&st, status, sizeof(st), low_pri_stream));
+  UGK_CALL(ugk_stream_sync(low_pri_stream));
+  CHECK_EQ(st, 0u) << "refresh row copy touched a row outside its table";
+}
+
 // cache_context.cu:3944-4107, the one-GPU part: steps 1-3, 5 and 6
 void RefreshSession::refresh_after_solve_new(bool foreground) {
   CacheContext *ctx = _cache_ctx.get();
@@ -734,6 +774,7 @@ void RefreshSession::refresh_after_solve_new(bool foreground) {
     UGK_CALL(ugk_fill_u32(_status_handle->ptr<uint32_t>(), 0, 64, stream));
   }
 
+  table->EnsureHostLists(ctx->_eager_gpu_mem_allocator, gpu_ctx, stream);  // after a refresh on the device
   // Step 1: key list of the new placement
   Timer t_phase;
   double detect_s = 0, evict_s = 0, wait_s = 0, insert_s = 0;
@@ -804,27 +845,7 @@ void RefreshSession::refresh_after_solve_new(bool foreground) {
     auto insert_keys_gpu = CopyTo1DReuse(__keys_buffer, new_insert_keys, gpu_ctx, low_pri_stream);
     auto reserved_offset =
         CopyTo1DReuse(__offs_buffer, table->ReserveOffsetFront((IdType)num_insert), gpu_ctx, low_pri_stream);
-    const void *host = ctx->_device_cache_data[ctx->_cpu_location_id];
-    void *cache = ctx->_device_cache_data[ctx->_local_location_id];
-    uint32_t *status = _status_handle->ptr<uint32_t>();
-    // background refresh copies in small throttled batches so that foreground lookups keep the host link
-    const size_t batch = foreground ? num_insert : std::max<size_t>(RunConfig::refresh_batch_rows, 1);
-    const unsigned limit_block = foreground ? 0 : RunConfig::refresh_limit_block;
-    for (size_t begin = 0; begin < num_insert; begin += batch) {
-      const size_t cur = std::min(batch, num_insert - begin);
-      UGK_CALL(ugk_gather_scatter_u32(host, ctx->_num_total_nodes, insert_keys_gpu->CPtr<uint32_t>() + begin,
-                                      reserved_offset->CPtr<uint32_t>() + begin, cur, cache,
-                                      ctx->_cache_space_capacity, ctx->_row_bytes, limit_block, status,
-                                      nullptr, low_pri_stream));
-      if (!foreground && begin + batch < num_insert) {
-        UGK_CALL(ugk_stream_sync(low_pri_stream));
-        usleep(RunConfig::refresh_sleep_us);
-      }
-    }
-    uint32_t st = 0;
-    UGK_CALL(ugk_memcpy_async(&st, status, sizeof(st), low_pri_stream));
-    UGK_CALL(ugk_stream_sync(low_pri_stream));
-    CHECK_EQ(st, 0u) << "refresh row copy touched a row outside its table";
+    CopyRowsIntoSlots(insert_keys_gpu->CPtr<uint32_t>(), reserved_offset->CPtr<uint32_t>(), num_insert, foreground);
     auto insert_table_keys =
         RunConfig::key_map_mul == 0
             ? insert_keys_gpu
@@ -837,6 +858,7 @@ void RefreshSession::refresh_after_solve_new(bool foreground) {
   insert_s = t_phase.Passed();
   t_phase.Reset();
   table->_cached_keys = key_list_of_each_src[local];
+  table->_dev_lists_valid = false;  // the host lists hold the truth now
   ctx->_cache_nodes = num_new_local_key;
   const bool rebuilt = table->MaybeRebuild(ctx->_eager_gpu_mem_allocator, gpu_ctx, local, stream);
   LOG(INFO) << "refresh: key lists " << detect_s << " s, evict " << evict_s << " s, wait for a lookup " << wait_s
@@ -846,5 +868,107 @@ void RefreshSession::refresh_after_solve_new(bool foreground) {
 }
 
 void RefreshSession::refresh_after_solve_main(bool foreground) { refresh_after_solve_new(foreground); }
+
+void RefreshSession::refresh_on_device(ExtractSession *session, size_t num_cached, bool foreground) {
+  CacheContext *ctx = _cache_ctx.get();
+  auto table = ctx->_new_hash_table;
+  CHECK_NOTNULL(table) << "refresh needs a partial cache (0 < cache_percentage < 1)";
+  CHECK_NOTNULL(session);
+  CHECK(session->CountsOnDevice()) << "refresh on the device needs the device-side hotness counters";
+  CHECK_LE(num_cached, (size_t)ctx->_cache_space_capacity) << "cache space can not hold refreshed new cache";
+  const Context gpu_ctx = ctx->_trainer_ctx;
+  const int local = ctx->_local_location_id;
+  const auto &alloc = ctx->_eager_gpu_mem_allocator;
+  const size_t num_rows = ctx->_num_total_nodes, capacity = ctx->_cache_space_capacity;
+  UGK_CALL(ugk_set_device(gpu_ctx.device_id));
+  if (low_pri_stream == nullptr) UGK_CALL(ugk_stream_create(&low_pri_stream));
+  if (!_status_handle) {
+    _status_handle = EagerGPUAlloc(gpu_ctx.device_id, 256);
+    UGK_CALL(ugk_fill_u32(_status_handle->ptr<uint32_t>(), 0, 64, stream));
+  }
+  Timer t_phase;
+  table->EnsureDeviceLists(alloc, gpu_ctx, stream);
+  const double sync_s = t_phase.Passed();
+  t_phase.Reset();
+
+  // Steps 1-3: the new placement as a bitmap, then evict = cached & ~new and insert = new & ~cached, ascending
+  session->PlaceOnDevice(num_cached, table->InNewBits(), table->_dev_rank_ws->ptr(), !RunConfig::gpu_refresh_keep,
+                         stream);
+  size_t num_evicted = 0, num_insert = 0;
+  TensorPtr evict_rows = table->CompactBits(table->InCacheBits(), table->InNewBits(), false, num_rows, SIZE_MAX,
+                                            __evict_rows, alloc, gpu_ctx, stream, &num_evicted);
+  TensorPtr insert_rows = table->CompactBits(table->InNewBits(), table->InCacheBits(), false, num_rows, SIZE_MAX,
+                                             __insert_rows, alloc, gpu_ctx, stream, &num_insert);
+  const size_t num_old = table->_num_cached;
+  CHECK_LE(num_evicted, num_old);
+  const size_t num_preserved_key = num_old - num_evicted;
+  CHECK_EQ(num_preserved_key + num_insert, std::min(num_cached, num_rows));
+  const double place_s = t_phase.Passed();
+  t_phase.Reset();
+
+  // Step 4: the evicted keys leave the table, their slots become free
+  if (num_evicted > 0) {
+    TensorPtr evict_keys = table->RowsToTableKeys(evict_rows, __evict_ids, alloc, gpu_ctx, stream);
+    TensorPtr evict_slots = Empty1DReuse(__evict_slots, kI32, {num_evicted}, gpu_ctx);
+    table->LookupOffset(evict_keys, evict_slots, stream);
+    UGK_CALL(ugk_bitmap_update(table->SlotUsedBits(), capacity, evict_slots->CPtr<uint32_t>(), num_evicted, 0,
+                               _status_handle->ptr<uint32_t>(), stream));
+    table->Evict(evict_keys, stream);
+    table->CheckStatus(stream, "refresh evict");
+  }
+  LOG(INFO) << "refresh on the device: preserved " << num_preserved_key << ", evict " << num_evicted << ", insert "
+            << num_insert << ", free slots " << table->_num_free + num_evicted;
+  const double evict_s = t_phase.Passed();
+  t_phase.Reset();
+
+  // Step 5: let one more lookup finish, so that no gather in flight still reads a slot about to be reused
+  const size_t current_progress = ctx->progress.load();
+  const bool stream_ordered = session->UsesStreamOrder();
+  if (stream_ordered) UGK_CALL(ugk_stream_sync(stream));
+  AnonymousBarrier::_refresh_instance->Wait();
+  {
+    Timer t0;
+    while (!foreground && !stream_ordered && ctx->progress.load() < current_progress + 1) {
+      if (t0.PassedSec() >= 20) break;
+      usleep(50);
+    }
+  }
+  const double wait_s = t_phase.Passed();
+  t_phase.Reset();
+
+  // Step 6: the first free slots, ascending, take the new rows, ascending; then the keys are published
+  if (num_insert > 0) {
+    size_t num_free = 0;
+    TensorPtr slots = table->CompactBits(table->SlotUsedBits(), nullptr, true, capacity, num_insert, __free_slots,
+                                         alloc, gpu_ctx, stream, &num_free);
+    CHECK_EQ(num_free, table->_num_free + num_evicted);
+    CHECK_LE(num_insert, num_free) << "free cache slots exhausted";
+    UGK_CALL(ugk_stream_sync(stream));  // the lists are read on the copy stream next
+    CopyRowsIntoSlots(insert_rows->CPtr<uint32_t>(), slots->CPtr<uint32_t>(), num_insert, foreground);
+    UGK_CALL(ugk_bitmap_update(table->SlotUsedBits(), capacity, slots->CPtr<uint32_t>(), num_insert, 1,
+                               _status_handle->ptr<uint32_t>(), stream));
+    TensorPtr insert_keys = table->RowsToTableKeys(insert_rows, __insert_ids, alloc, gpu_ctx, stream);
+    table->InsertWithLoc(insert_keys, slots, local, stream);
+    table->CheckStatus(stream, "refresh insert");
+  }
+  uint32_t st = 0;
+  UGK_CALL(ugk_memcpy_async(&st, _status_handle->ptr<uint32_t>(), sizeof(st), stream));
+  UGK_CALL(ugk_stream_sync(stream));
+  CHECK_EQ(st, 0u) << "refresh on the device: a listed row or slot is outside its bitmap";
+  AnonymousBarrier::_refresh_instance->Wait();
+  const double insert_s = t_phase.Passed();
+  t_phase.Reset();
+
+  std::swap(table->_dev_in_cache, table->_dev_in_new);
+  table->_num_cached = num_preserved_key + num_insert;
+  table->_num_free = capacity - table->_num_cached;
+  table->_host_lists_valid = false;  // the bitmaps hold the truth now
+  ctx->_cache_nodes = table->_num_cached;
+  const bool rebuilt = table->MaybeRebuild(alloc, gpu_ctx, local, stream);
+  LOG(INFO) << "refresh on the device: bitmaps " << sync_s << " s, placement + key lists " << place_s << " s, evict "
+            << evict_s << " s, wait for a lookup " << wait_s << " s, row copy + insert " << insert_s
+            << " s, table rebuild " << (rebuilt ? t_phase.Passed() : 0.0) << " s";
+}
+
 
 }  // namespace coll_cache_lib

@@ -81,6 +81,10 @@ class CacheContext {
   size_t RowBytes() const { return _row_bytes; }
   int TableKind() const { return _new_hash_table ? _new_hash_table->_table.kind : 0; }
   const CacheEntryManager *EntryManager() const { return _new_hash_table; }
+  // brings the host-side key and slot lists up to date after a refresh on the device (not while a refresh runs)
+  void SyncHostLists() {
+    if (_new_hash_table) _new_hash_table->EnsureHostLists(_eager_gpu_mem_allocator, _trainer_ctx, nullptr);
+  }
 };
 
 class ExtractSession {
@@ -122,10 +126,12 @@ class ExtractSession {
   MemHandle _hot_entries;        // compact (count << 32 | row) list of one drain step
   MemHandle _hot_entries_host;   // pinned copy of it
   StreamHandle _record_stream = nullptr;  // record kernels and drains run here, beside the extraction
-  void *_ev_rec_begin = nullptr, *_ev_rec_done = nullptr;
+  void *_ev_rec_begin = nullptr, *_ev_rec_done = nullptr, *_ev_placed = nullptr;
   bool _record_pending = false;
   size_t _record_limit = SIZE_MAX;
-  std::mutex _drain_mu;  // one drain at a time: they share the entry list and its pinned copy
+  // one drain at a time (they share the entry list and its pinned copy); also held while a record kernel or the
+  // passes of a placement are enqueued on the record stream, so that the passes see one state of the counters
+  std::mutex _drain_mu;
   uint32_t *_state = nullptr;
   void JoinRecord(StreamHandle stream);
   size_t _num_lookups = 0;
@@ -170,6 +176,12 @@ class ExtractSession {
   // moves what the lookups have counted on the device since the last call into `recorder` (FreqRecorder::Record's
   // result for the same keys); safe to call from another thread while lookups run.  Returns the rows moved.
   size_t DrainHotness(FreqRecorder *recorder);
+  // Ranks the rows by what the lookups have counted on the device (same order as FreqRecorder::Sort, never-counted
+  // rows behind the counted ones in ascending order) and sets bit r of in_new_bits for the num_cached best rows.
+  // Runs on the record stream, ordered against the counting of every lookup; `stream` waits for the result.
+  // reset_counts: the next interval starts from zero, as after DrainHotness.
+  bool CountsOnDevice() const { return _hot_counts != nullptr; }
+  void PlaceOnDevice(size_t num_cached, uint64_t *in_new_bits, void *rank_ws, bool reset_counts, StreamHandle stream);
   // the device-side counting of the following lookups covers only the first `num_keys` keys of a batch
   // (the recorded prefix of LookupManager's record thread); SIZE_MAX, the default: the whole batch
   void SetRecordLimit(size_t num_keys) { _record_limit = num_keys; }
@@ -181,14 +193,22 @@ class RefreshSession {
   StreamHandle low_pri_stream = nullptr;  // a second default-priority stream: row copies of the refresh
   std::shared_ptr<CacheContext> _cache_ctx;
   void refresh_after_solve_main(bool foreground);
+  // The whole refresh on the device (RunConfig::gpu_refresh): placement from the device-side hotness counters of
+  // `session`, evict = cached & ~new and insert = new & ~cached as bitmap compactions, free slots from the slot bitmap;
+  // then the same evict / wait / copy / insert steps as refresh_after_solve_new (cache_context.cu:3944-4107).
+  void refresh_on_device(ExtractSession *session, size_t num_cached, bool foreground);
   ~RefreshSession();
 
  private:
   void refresh_after_solve_new(bool foreground);
   TensorPtr Empty1DReuse(TensorPtr &preserved_buffer, DataType dtype, std::vector<size_t> shape, Context ctx);
   TensorPtr CopyTo1DReuse(TensorPtr &preserved_buffer, TensorPtr src, Context ctx, StreamHandle stream);
+  // copies the listed host rows into the listed cache slots (step 6): in one launch when in the foreground, in
+  // small throttled batches behind running lookups otherwise
+  void CopyRowsIntoSlots(const uint32_t *rows_dev, const uint32_t *slots_dev, size_t num_rows, bool foreground);
   TensorPtr __keys_buffer;
   TensorPtr __offs_buffer;
+  TensorPtr __evict_rows, __insert_rows, __free_slots, __evict_ids, __insert_ids, __evict_slots;
   MemHandle _status_handle;
 };
 

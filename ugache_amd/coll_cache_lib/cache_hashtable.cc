@@ -94,12 +94,29 @@ void CacheEntryManager::Evict(TensorPtr keys_to_evict, StreamHandle stream) {
 bool CacheEntryManager::MaybeRebuild(const std::function<MemHandle(size_t)> &allocator, Context ctx, int loc,
                                      StreamHandle stream) {
   if (_table.kind != 2) return false;
-  if ((double)_num_tombstones <= RunConfig::hash_rebuild_tombstone_frac * (double)_table.size) return false;
-  const size_t n = _cached_keys->NumItem();
+  const double limit = RunConfig::hash_rebuild_tombstone_frac * (double)_table.size;
+  if ((double)_num_tombstones <= limit) return false;
+  // _num_tombstones counts evictions; inserts reuse tombstones they pass, so look before rebuilding
+  uint64_t *census_dev = reinterpret_cast<uint64_t *>(StatusPtr(this, stream) + 16);
+  uint64_t census[3] = {0, 0, 0};
+  UGK_CALL(ugk_hash_census(static_cast<const ugk_bucket_t *>(_table.table), _table.size, census_dev, stream));
+  UGK_CALL(ugk_memcpy_async(census, census_dev, sizeof(census), stream));
+  UGK_CALL(ugk_stream_sync(stream));
+  _num_tombstones = census[1];
+  if ((double)_num_tombstones <= limit) return false;
+  TensorPtr keys, offs, key_buffer;
+  size_t n = 0;
+  if (_dev_lists_valid) {  // the cached rows are known on the device: the key list never leaves it
+    TensorPtr rows = CompactBits(InCacheBits(), nullptr, false, num_total_key, SIZE_MAX, _dev_list_buffer, allocator,
+                                 ctx, stream, &n);
+    keys = RowsToTableKeys(rows, key_buffer, allocator, ctx, stream);
+  } else {
+    n = _cached_keys->NumItem();
+    keys = TableKeysToDevice(_cached_keys, allocator, ctx, stream);
+  }
   LOG(INFO) << "rebuilding the lookup table: " << _num_tombstones << " tombstones in " << _table.size << " buckets, "
             << n << " live keys";
-  TensorPtr keys = TableKeysToDevice(_cached_keys, allocator, ctx, stream);
-  TensorPtr offs = Tensor::EmptyExternal(kI32, {n}, allocator, ctx, "");
+  offs = Tensor::EmptyExternal(kI32, {n}, allocator, ctx, "");
   if (n > 0) LookupOffset(keys, offs, stream);
   UGK_CALL(ugk_hash_init(static_cast<ugk_bucket_t *>(_table.table), _table.size, stream));
   if (n > 0) InsertWithLoc(keys, offs, loc, stream);
@@ -107,6 +124,108 @@ bool CacheEntryManager::MaybeRebuild(const std::function<MemHandle(size_t)> &all
   _num_tombstones = 0;
   _num_rebuilds++;
   return true;
+}
+
+namespace {
+TensorPtr ReuseList(TensorPtr &buffer, DataType dtype, size_t n, const std::function<MemHandle(size_t)> &allocator,
+                    Context ctx) {
+  const std::vector<size_t> shape = {n};
+  if (buffer && buffer->CanForceScale(dtype, shape)) {
+    buffer->ForceScale(dtype, shape, ctx, "");
+    return buffer;
+  }
+  // room to grow: these lists change size from refresh to refresh
+  const size_t elem = dtype == kI64 ? 8 : 4;
+  buffer = Tensor::EmptyExternal(kU8, {std::max<size_t>(n + n / 4, 1024) * elem}, allocator, ctx, "");
+  buffer->ForceScale(dtype, shape, ctx, "");
+  return buffer;
+}
+}  // namespace
+
+TensorPtr CacheEntryManager::CompactBits(const uint64_t *a, const uint64_t *b, bool invert_a, uint64_t nbits,
+                                         size_t limit, TensorPtr &buffer,
+                                         const std::function<MemHandle(size_t)> &allocator, Context ctx,
+                                         StreamHandle stream, size_t *total_out) {
+  uint32_t *total = DevWords();
+  UGK_CALL(ugk_bitmap_count(a, b, invert_a ? 1 : 0, nbits, _dev_bm_ws->ptr(), total, stream));
+  UGK_CALL(ugk_stream_sync(stream));
+  const size_t found = *total;
+  if (total_out) *total_out = found;
+  const size_t n = std::min(found, limit);
+  TensorPtr list = ReuseList(buffer, kI32, n, allocator, ctx);
+  if (n) UGK_CALL(ugk_bitmap_emit(a, b, invert_a ? 1 : 0, nbits, _dev_bm_ws->ptr(), list->Ptr<uint32_t>(), n, stream));
+  return list;
+}
+
+TensorPtr CacheEntryManager::RowsToTableKeys(TensorPtr rows_dev, TensorPtr &buffer,
+                                             const std::function<MemHandle(size_t)> &allocator, Context ctx,
+                                             StreamHandle stream) {
+  if (RunConfig::key_map_mul == 0) return rows_dev;
+  const size_t n = rows_dev->NumItem();
+  TensorPtr ids = ReuseList(buffer, kI64, n, allocator, ctx);
+  UGK_CALL(ugk_rows_to_keys(rows_dev->CPtr<uint32_t>(), n, RunConfig::key_map_mul, RunConfig::key_map_mask,
+                            ids->Ptr<int64_t>(), stream));
+  return ids;
+}
+
+void CacheEntryManager::EnsureDeviceLists(const std::function<MemHandle(size_t)> &allocator, Context ctx,
+                                          StreamHandle stream) {
+  const size_t row_words = (num_total_key + 63) / 64, slot_words = ((size_t)_cache_space_capacity + 63) / 64;
+  if (!_dev_in_cache) {
+    _dev_in_cache = EagerGPUAlloc(_device_id, row_words * 8);
+    _dev_in_new = EagerGPUAlloc(_device_id, row_words * 8);
+    _dev_slot_used = EagerGPUAlloc(_device_id, std::max<size_t>(slot_words, 1) * 8);
+    _dev_rank_ws = EagerGPUAlloc(_device_id, ugk_rank_workspace_bytes());
+    _dev_bm_ws = EagerGPUAlloc(_device_id, ugk_bitmap_workspace_bytes());
+    _dev_words = PinnedHostAlloc(256);
+    memset(_dev_words->ptr(), 0, 256);
+  }
+  if (_dev_lists_valid) return;
+  CHECK(_host_lists_valid);
+  UGK_CALL(ugk_fill_u32(_dev_in_cache->ptr<uint32_t>(), 0, row_words * 2, stream));
+  UGK_CALL(ugk_fill_u32(_dev_slot_used->ptr<uint32_t>(), 0, std::max<size_t>(slot_words, 1) * 2, stream));
+  const size_t n = _cached_keys->NumItem();
+  if (n > 0) {
+    TensorPtr rows = ReuseList(_dev_list_buffer, kI32, n, allocator, ctx);
+    UGK_CALL(ugk_memcpy_async(rows->MutableData(), _cached_keys->Data(), n * sizeof(IdType), stream));
+    UGK_CALL(ugk_stream_sync(stream));  // the source is pageable host memory
+    uint32_t *status = StatusPtr(this, stream);
+    UGK_CALL(ugk_bitmap_update(InCacheBits(), num_total_key, rows->CPtr<uint32_t>(), n, 1, status, stream));
+    TensorPtr key_buffer;
+    TensorPtr keys = RowsToTableKeys(rows, key_buffer, allocator, ctx, stream);
+    TensorPtr slots = Tensor::EmptyExternal(kI32, {n}, allocator, ctx, "");
+    LookupOffset(keys, slots, stream);
+    UGK_CALL(ugk_bitmap_update(SlotUsedBits(), _cache_space_capacity, slots->CPtr<uint32_t>(), n, 1, status, stream));
+    CheckStatus(stream, "placement bitmaps");
+  }
+  _num_cached = n;
+  _num_free = _free_offsets->NumItem();
+  CHECK_EQ(_num_cached + _num_free, (size_t)_cache_space_capacity);
+  _dev_lists_valid = true;
+}
+
+void CacheEntryManager::EnsureHostLists(const std::function<MemHandle(size_t)> &allocator, Context ctx,
+                                        StreamHandle stream) {
+  if (_host_lists_valid) return;
+  CHECK(_dev_lists_valid);
+  UGK_CALL(ugk_set_device(_device_id));
+  size_t n_cached = 0, n_free = 0;
+  TensorPtr rows =
+      CompactBits(InCacheBits(), nullptr, false, num_total_key, SIZE_MAX, _dev_list_buffer, allocator, ctx, stream,
+                  &n_cached);
+  _cached_keys = Tensor::Empty(kI32, {n_cached}, CPU_CLIB(), "cached_keys");
+  if (n_cached) UGK_CALL(ugk_memcpy_async(_cached_keys->MutableData(), rows->Data(), n_cached * sizeof(IdType), stream));
+  UGK_CALL(ugk_stream_sync(stream));
+  TensorPtr slots = CompactBits(SlotUsedBits(), nullptr, true, _cache_space_capacity, SIZE_MAX, _dev_list_buffer,
+                                allocator, ctx, stream, &n_free);
+  _free_offsets = Tensor::Empty(kI32, {(size_t)_cache_space_capacity}, CPU_CLIB(), "free_offsets");
+  _free_offsets->ForceScale(kI32, {n_free}, CPU_CLIB(), "");
+  if (n_free) UGK_CALL(ugk_memcpy_async(_free_offsets->MutableData(), slots->Data(), n_free * sizeof(IdType), stream));
+  UGK_CALL(ugk_stream_sync(stream));
+  CHECK_EQ(n_cached, _num_cached);
+  CHECK_EQ(n_free, _num_free);
+  CHECK_EQ(n_cached + n_free, (size_t)_cache_space_capacity);
+  _host_lists_valid = true;
 }
 
 void CacheEntryManager::CheckStatus(StreamHandle stream, const char *what) {

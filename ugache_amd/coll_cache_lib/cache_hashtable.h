@@ -74,6 +74,37 @@ class CacheEntryManager {
   size_t _num_tombstones = 0;
   size_t _num_rebuilds = 0;
 
+  // ---- the same bookkeeping on the device, for refreshes that never leave it -----------------------------------
+  // Membership of the cache as one bit per row of the host table, occupancy of the cache as one bit per slot.  A
+  // refresh on the device reads and updates these; a refresh on the host reads and updates _cached_keys and
+  // _free_offsets.  Whichever ran last holds the truth, the other side is brought up to date when it is next needed.
+  MemHandle _dev_in_cache, _dev_in_new;  // ceil(num_total_key / 64) words each
+  MemHandle _dev_slot_used;              // ceil(capacity / 64) words
+  MemHandle _dev_rank_ws, _dev_bm_ws;    // workspaces of ugk_rank_* / ugk_bitmap_*
+  MemHandle _dev_words;                  // pinned host words the kernels report counts in
+  TensorPtr _dev_list_buffer;            // scratch list for bringing either side up to date
+  bool _dev_lists_valid = false;
+  bool _host_lists_valid = true;
+  size_t _num_cached = 0, _num_free = 0;  // valid when the host lists are not
+  size_t NumCached() const { return _host_lists_valid ? (_cached_keys ? _cached_keys->NumItem() : 0) : _num_cached; }
+  size_t NumFree() const { return _host_lists_valid ? (_free_offsets ? _free_offsets->NumItem() : 0) : _num_free; }
+  uint64_t *InCacheBits() const { return _dev_in_cache->ptr<uint64_t>(); }
+  uint64_t *InNewBits() const { return _dev_in_new->ptr<uint64_t>(); }
+  uint64_t *SlotUsedBits() const { return _dev_slot_used->ptr<uint64_t>(); }
+  uint32_t *DevWords() const { return _dev_words->ptr<uint32_t>(); }
+  // bitmaps from the host lists (allocates them on first use)
+  void EnsureDeviceLists(const std::function<MemHandle(size_t)> &allocator, Context ctx, StreamHandle stream);
+  // host lists from the bitmaps: cached rows ascending, free slots ascending
+  void EnsureHostLists(const std::function<MemHandle(size_t)> &allocator, Context ctx, StreamHandle stream);
+  // |S| and the first `limit` elements of S = set bits of (invert_a ? ~a : a) & ~b below nbits, ascending, in a device
+  // list taken from `buffer` (grown when too small); blocks once, for the count
+  TensorPtr CompactBits(const uint64_t *a, const uint64_t *b, bool invert_a, uint64_t nbits, size_t limit,
+                        TensorPtr &buffer, const std::function<MemHandle(size_t)> &allocator, Context ctx,
+                        StreamHandle stream, size_t *total_out);
+  // device list of host rows -> device list of table keys (the rows themselves, or their ids in sparse-id mode)
+  TensorPtr RowsToTableKeys(TensorPtr rows_dev, TensorPtr &buffer, const std::function<MemHandle(size_t)> &allocator,
+                            Context ctx, StreamHandle stream);
+
   // cuh:693-740 — keys of `inputs` satisfying cond, in input order (deterministic, unlike the reference's
   // thread-interleaved order)
   template <typename InputIterator, typename CondT>

@@ -191,6 +191,20 @@ void CollCache::refresh(int replica_id, ContFreqBuf *freq_rank, StreamHandle str
   LOG(INFO) << "refresh: placement " << solve_s << " s, evict + insert " << t_apply.Passed() << " s";
 }
 
+void CollCache::refresh_on_device(int replica_id, StreamHandle stream, bool foreground) {
+  CHECK_EQ(replica_id, 0);
+  CHECK_NOTNULL(_nid_to_block) << "refresh needs a cache built with 0 < cache_percentage < 1";
+  CheckPolicy();
+  AnonymousBarrier::_refresh_instance->Wait();
+  Timer t_apply;
+  const size_t num_cached = coll_cache::FreqRankSolver::NumCachedNodes((IdType)RunConfig::num_total_item,
+                                                                       RunConfig::cache_percentage * 100);
+  this->_refresh_session_list[replica_id]->stream = stream;
+  this->_refresh_session_list[replica_id]->refresh_on_device(_session_list[replica_id].get(), num_cached, foreground);
+  AnonymousBarrier::_refresh_instance->Wait();
+  LOG(INFO) << "refresh on the device: " << t_apply.Passed() << " s";
+}
+
 void CollCache::report_last_epoch(uint64_t epoch) { _profiler->ReportStepAverageLastEpoch(epoch + 1, 0); }
 
 void CollCache::report_avg() {

@@ -63,6 +63,9 @@ class CollCache : public std::enable_shared_from_this<CollCache> {
   void refresh(int replica_id, IdType *ranking_nodes_list_ptr, IdType *ranking_nodes_freq_list_ptr,
                StreamHandle stream = nullptr, bool foreground = false);
   void refresh(int replica_id, ContFreqBuf *freq_rank, StreamHandle stream = nullptr, bool foreground = false);
+  // the same refresh with ranking, placement and key lists computed on the device from the hotness the lookups
+  // counted there (RunConfig::gpu_refresh); _nid_to_block is not updated by it
+  void refresh_on_device(int replica_id, StreamHandle stream = nullptr, bool foreground = false);
 
   void report_avg();
   void report_last_epoch(uint64_t epoch);

@@ -57,6 +57,11 @@ class FreqRecorder {
   void GlobalCombine();
   void Sort();
   inline size_t NumNodes() const { return _num_nodes; }
+  // true when counts wait here for the next ranking (recorded on the host, or handed over from the device)
+  bool HasCounts() {
+    std::lock_guard<std::mutex> g(_mu);
+    return _live_dirty || _shared_dirty || !_handed_over.empty();
+  }
   ContFreqBuf *global_cont_freq_buf;
 
  private:

@@ -275,6 +275,14 @@ void coll_cache_set_key_map(uint64_t mul, int bits) {
 void coll_cache_refresh(int replica_id, StreamHandle stream, int foreground) {
   CHECK_NOTNULL(_coll_cache);
   Timer t_rank;
+  // hotness counted on the device only, and asked to stay there: rank, place and diff on the device
+  if (RunConfig::gpu_refresh && RunConfig::gpu_record && (size_t)replica_id < _freq_recorder.size() &&
+      _freq_recorder[replica_id] && !_freq_recorder[replica_id]->HasCounts() && _coll_cache->session(replica_id) &&
+      _coll_cache->session(replica_id)->CountsOnDevice()) {
+    _coll_cache->refresh_on_device(replica_id, stream, foreground != 0);
+    if (_profiler) _profiler->SetRefreshDuration(t_rank.Passed());
+    return;
+  }
   ContFreqBuf *freq_rank = CombineAndRank(replica_id);
   LOG(INFO) << "refresh: ranking " << t_rank.Passed() << " s";
   _coll_cache->refresh(replica_id, freq_rank, stream, foreground != 0);
@@ -400,12 +408,13 @@ void coll_cache_get_info(int replica_id, uint64_t out[8]) {
   out[3] = ctx->RowBytes();
   out[4] = RunConfig::num_total_item;
   out[5] = ctx->progress.load();
-  out[6] = ctx->EntryManager() ? ctx->EntryManager()->_free_offsets->NumItem() : 0;
+  out[6] = ctx->EntryManager() ? ctx->EntryManager()->NumFree() : 0;
   out[7] = ctx->EntryManager() ? ctx->EntryManager()->_num_rebuilds : 0;
 }
 
 size_t coll_cache_get_cached_keys(int replica_id, uint32_t *out, size_t capacity) {
   CHECK_NOTNULL(_coll_cache);
+  _coll_cache->cache_ctx(replica_id)->SyncHostLists();
   auto mgr = _coll_cache->cache_ctx(replica_id)->EntryManager();
   if (!mgr || !mgr->_cached_keys) return 0;
   const size_t n = mgr->_cached_keys->NumItem();

@@ -96,7 +96,7 @@ void FreqRankSolver::Solve(std::vector<int> device_to_stream, std::vector<PerT> 
   CHECK_EQ(num_device, 1) << "this build places keys for one GPU and its host";
   const int num_block = 2;
   const IdType num_node = _num_node;
-  const IdType num_cached_nodes = (IdType)(num_node * (device_to_cache_percent[0] / (double)100));
+  const IdType num_cached_nodes = NumCachedNodes(num_node, device_to_cache_percent[0]);
   IdType *nid_to_block = _nid_to_block->Ptr<IdType>();
   double rep_w = 0, cpu_w = 0;
   if (_cont != nullptr) {

@@ -44,6 +44,8 @@ class FreqRankSolver : public CollCacheSolver {
                          const TensorPtr nid_to_block_tensor) override;
   void Solve(std::vector<int> device_to_stream, std::vector<PerT> device_to_cache_percent, std::string mode,
              double T_local, double T_cpu) override;
+  // how many of num_node keys a cache of `percent` % holds (optimal_solver_class.cc:1878)
+  static IdType NumCachedNodes(IdType num_node, PerT percent) { return (IdType)(num_node * (percent / (double)100)); }
 
  private:
   TensorPtr _rank_keys;  // u32 [num_node]   (Build)

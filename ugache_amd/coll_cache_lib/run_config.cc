@@ -38,6 +38,8 @@ unsigned RunConfig::refresh_limit_block = 20;
 double RunConfig::hash_rebuild_tombstone_frac = 0.15;
 bool RunConfig::gpu_record = false;
 size_t RunConfig::gpu_record_every = 1;
+bool RunConfig::gpu_refresh = false;
+bool RunConfig::gpu_refresh_keep = false;
 bool RunConfig::dedup_keys = false;
 size_t RunConfig::dedup_min_keys = 4096;
 uint64_t RunConfig::key_map_mul = 0;
@@ -76,6 +78,8 @@ void RunConfig::LoadConfigFromEnv() {
   dedup_min_keys = 4096;
   gpu_record = false;
   gpu_record_every = 1;
+  gpu_refresh = false;
+  gpu_refresh_keep = false;
   if (GetEnv("SAMGRAPH_EMPTY_FEAT") != "" && GetEnv("SAMGRAPH_EMPTY_FEAT") != "0") {
     LOG(FATAL) << "SAMGRAPH_EMPTY_FEAT (mock host table) is not supported by this build: every key must have a "
                   "real row in the host table";
@@ -105,6 +109,8 @@ void RunConfig::LoadConfigFromEnv() {
   if (GetEnv("COLL_REFRESH_SLEEP_US") != "") refresh_sleep_us = std::stoul(GetEnv("COLL_REFRESH_SLEEP_US"));
   if (GetEnv("COLL_REFRESH_LIMIT_BLOCK") != "") refresh_limit_block = std::stoul(GetEnv("COLL_REFRESH_LIMIT_BLOCK"));
   if (GetEnv("COLL_GPU_RECORD") != "") gpu_record = GetEnv("COLL_GPU_RECORD") != "0";
+  if (GetEnv("COLL_GPU_REFRESH") != "") gpu_refresh = GetEnv("COLL_GPU_REFRESH") != "0";
+  if (GetEnv("COLL_GPU_REFRESH_KEEP") != "") gpu_refresh_keep = GetEnv("COLL_GPU_REFRESH_KEEP") != "0";
   if (GetEnv("COLL_GPU_RECORD_EVERY") != "")
     gpu_record_every = std::max<size_t>(1, std::stoull(GetEnv("COLL_GPU_RECORD_EVERY")));
   if (GetEnv("COLL_DEDUP_KEYS") != "") dedup_keys = GetEnv("COLL_DEDUP_KEYS") != "0";

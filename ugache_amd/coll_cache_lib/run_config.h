@@ -65,6 +65,12 @@ struct RunConfig {
   static unsigned refresh_limit_block; // COLL_REFRESH_LIMIT_BLOCK, default 20 (cache_context.cu:4068)
   static bool gpu_record;          // COLL_GPU_RECORD=1: every lookup counts its keys in device-side hotness counters
   static size_t gpu_record_every;  // COLL_GPU_RECORD_EVERY, default 1: ... only every n-th lookup
+  // COLL_GPU_REFRESH=1 (with COLL_GPU_RECORD=1): a refresh whose hotness was all counted on the device ranks, places
+  // and diffs on the device too; the host sees two short key lists instead of per-key arrays of the key space
+  static bool gpu_refresh;
+  // COLL_GPU_REFRESH_KEEP=1: such a refresh leaves the counters as they are (hotness accumulates over refreshes)
+  // instead of starting the next interval from zero
+  static bool gpu_refresh_keep;
   static bool dedup_keys;        // COLL_DEDUP_KEYS=1: extract each distinct key of a batch once, then copy the duplicates
   static size_t dedup_min_keys;  // COLL_DEDUP_MIN_KEYS, default 4096: shorter batches skip the deduplication
   static double hash_rebuild_tombstone_frac;  // COLL_HASH_REBUILD_FRAC, default 0.15: rebuild the table after refresh

@@ -1,0 +1,392 @@
+// Re-placement of the cache on the device, from the hotness counters the lookups keep there: which rows belong to
+// the K best-ranked ones, which cached rows fell out, which rows come in, which cache slots are free.  The rank order
+// is the one FreqRecorder::Sort + RepSolver::Solve use on the host (freq_recorder.cc:275-281,
+// optimal_solver_class.cc:1869-1924): observed rows by (count << 32 | row) descending, never-observed rows behind
+// them in ascending row order.
+//
+// select : exact K-th largest rank by a most-significant-digit radix select over all counters (six histogram passes
+//          of 10-11 bits over 64-bit ranks; every pass is one streaming read of the counters, HBM-bound).
+// mark   : one more pass turns "rank >= threshold" into a bitmap with one bit per row (and may reset the counters).
+// bitmap : ordered compaction of the set bits of a, ~a, a & ~b into an ascending index list (count, scan, emit), and
+//          setting / clearing listed bits.  Membership of the cache and occupancy of its slots live in such bitmaps,
+//          so evict = cached & ~new, insert = new & ~cached, free slots = ~used are all the same three launches.
+#include "ugk_internal.h"
+
+namespace ugk {
+namespace {
+
+constexpr int kHistBins = 2048;          // 11-bit digits at most
+constexpr int kBmChunks = 8192;          // fixed partition of a bitmap, independent of the launch grid
+constexpr int kSelectPasses = 6;
+constexpr int kPassShift[kSelectPasses] = {53, 42, 32, 21, 10, 0};
+constexpr int kPassBits[kSelectPasses] = {11, 11, 10, 11, 11, 10};
+
+// workspace of select/mark: [0] threshold so far (digits picked from the top), [1] how many ranks at or above the
+// final threshold are still to be found inside the current prefix, then the histogram
+struct RankWs {
+  unsigned long long prefix;
+  unsigned long long remaining;
+  uint32_t hist[kHistBins];
+};
+
+__device__ __forceinline__ unsigned long long rank_of(uint32_t cnt, uint32_t row) {
+  return cnt ? ((unsigned long long)cnt << 32) | row : (unsigned long long)(0xffffffffu - row);
+}
+
+__global__ __launch_bounds__(kBlock) void rank_hist_kernel(const uint32_t *__restrict__ counts, uint64_t n,
+                                                           RankWs *ws, int shift, int bits) {
+  __shared__ uint32_t lh[kHistBins];
+  const int tid = threadIdx.x;
+  for (int b = tid; b < kHistBins; b += kBlock) lh[b] = 0;
+  __syncthreads();
+  const unsigned long long prefix = ws->prefix;
+  const unsigned long long hi_mask = shift + bits >= 64 ? 0ull : ~0ull << (shift + bits);
+  const unsigned long long want = prefix & hi_mask;
+  const uint32_t digit_mask = (1u << bits) - 1u;
+  // consecutive rows mostly share a digit (all cold rows in the count passes, neighbours in the high row passes):
+  // a lane keeps a run and touches the LDS histogram only when the digit changes
+  uint32_t last = 0, run = 0;
+  const uint64_t n_vec = n / 4;
+  const u32x4 *cv = reinterpret_cast<const u32x4 *>(counts);
+  for (uint64_t v = (uint64_t)blockIdx.x * kBlock + tid; v < n_vec; v += (uint64_t)gridDim.x * kBlock) {
+    const u32x4 c = __builtin_nontemporal_load(cv + v);
+    const uint32_t cc[4] = {c.x, c.y, c.z, c.w};
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      const unsigned long long r = rank_of(cc[k], (uint32_t)(v * 4 + k));
+      if ((r & hi_mask) == want) {
+        const uint32_t d = (uint32_t)(r >> shift) & digit_mask;
+        if (d == last) {
+          ++run;
+        } else {
+          if (run) atomicAdd(&lh[last], run);
+          last = d;
+          run = 1;
+        }
+      }
+    }
+  }
+  if (blockIdx.x == 0 && tid < (int)(n - n_vec * 4)) {  // the last n % 4 rows
+    const uint64_t row = n_vec * 4 + tid;
+    const unsigned long long r = rank_of(counts[row], (uint32_t)row);
+    if ((r & hi_mask) == want) atomicAdd(&lh[(uint32_t)(r >> shift) & digit_mask], 1u);
+  }
+  if (run) atomicAdd(&lh[last], run);
+  __syncthreads();
+  for (int b = tid; b < kHistBins; b += kBlock)
+    if (lh[b]) atomicAdd(&ws->hist[b], lh[b]);
+}
+
+// one workgroup: the digit d with  #(bins above d) < remaining <= #(bins at or above d)
+__global__ __launch_bounds__(kBlock) void rank_pick_kernel(RankWs *ws, int shift) {
+  constexpr int kPer = kHistBins / kBlock;  // 8 bins per thread
+  __shared__ unsigned long long suffix[kBlock + 1];
+  const int tid = threadIdx.x;
+  uint32_t h[kPer];
+  unsigned long long mine = 0;
+#pragma unroll
+  for (int j = 0; j < kPer; ++j) {
+    h[j] = ws->hist[tid * kPer + j];
+    mine += h[j];
+  }
+  suffix[tid] = mine;
+  if (tid == 0) suffix[kBlock] = 0;
+  __syncthreads();
+  for (int s = 1; s < kBlock; s <<= 1) {  // inclusive suffix sums
+    const unsigned long long add = tid + s < kBlock ? suffix[tid + s] : 0;
+    __syncthreads();
+    suffix[tid] += add;
+    __syncthreads();
+  }
+  const unsigned long long need = ws->remaining;
+  __syncthreads();
+  if (suffix[tid] >= need && suffix[tid + 1] < need) {
+    unsigned long long above = suffix[tid + 1];
+#pragma unroll
+    for (int j = kPer - 1; j >= 0; --j) {
+      if (above + h[j] >= need) {
+        ws->prefix |= (unsigned long long)(tid * kPer + j) << shift;
+        ws->remaining = need - above;
+        break;
+      }
+      above += h[j];
+    }
+  }
+#pragma unroll
+  for (int j = 0; j < kPer; ++j) ws->hist[tid * kPer + j] = 0;
+}
+
+__global__ void rank_init_kernel(RankWs *ws, unsigned long long prefix, unsigned long long remaining) {
+  const int tid = threadIdx.x;
+  if (tid == 0) {
+    ws->prefix = prefix;
+    ws->remaining = remaining;
+  }
+  for (int b = tid; b < kHistBins; b += blockDim.x) ws->hist[b] = 0;
+}
+
+// bit r of the bitmap = rank(r) >= threshold.  A wavefront takes 64 consecutive rows per load, so a ballot is a word.
+constexpr int kMarkWords = 8;  // words (loads in flight) per wavefront and round
+__global__ __launch_bounds__(kBlock) void rank_mark_kernel(uint32_t *counts, uint64_t n, const RankWs *ws,
+                                                           unsigned long long *bitmap, int reset_counts) {
+  const unsigned long long threshold = ws->prefix;
+  const int lane = (int)lane_id();
+  const uint64_t n_words = (n + 63) / 64;
+  const uint64_t wave = ((uint64_t)blockIdx.x * kBlock + threadIdx.x) / kWave;
+  const uint64_t n_waves = (uint64_t)gridDim.x * (kBlock / kWave);
+  for (uint64_t w0 = wave * kMarkWords; w0 < n_words; w0 += n_waves * kMarkWords) {
+    uint32_t c[kMarkWords];
+#pragma unroll
+    for (int k = 0; k < kMarkWords; ++k) {
+      const uint64_t row = (w0 + k) * 64 + lane;
+      c[k] = row < n ? counts[row] : 0u;
+    }
+#pragma unroll
+    for (int k = 0; k < kMarkWords; ++k) {
+      const uint64_t row = (w0 + k) * 64 + lane;
+      const bool in = row < n && rank_of(c[k], (uint32_t)row) >= threshold;
+      const unsigned long long word = __ballot(in);
+      if (lane == k && w0 + k < n_words) bitmap[w0 + k] = word;
+      if (reset_counts && row < n && c[k] != 0) counts[row] = 0;
+    }
+  }
+}
+
+// ---- bitmaps ----------------------------------------------------------------------------------------------
+struct BmWs {
+  uint32_t total;
+  uint32_t pad[3];
+  uint32_t base[kBmChunks];  // per chunk: first the count, after the scan the exclusive prefix
+};
+
+__device__ __forceinline__ unsigned long long bm_word(const unsigned long long *a, const unsigned long long *b,
+                                                      bool invert_a, uint64_t nbits, uint64_t w) {
+  unsigned long long m = a[w];
+  if (invert_a) m = ~m;
+  if (b) m &= ~b[w];
+  const uint64_t first = w * 64;
+  if (nbits - first < 64) m &= (1ull << (nbits - first)) - 1ull;  // the last, partial word
+  return m;
+}
+
+static inline uint64_t bm_words_per_chunk(uint64_t n_words) {
+  return ((n_words + kBmChunks - 1) / kBmChunks + kWave - 1) / kWave * kWave;
+}
+
+__global__ __launch_bounds__(kBlock) void bitmap_count_kernel(const unsigned long long *a, const unsigned long long *b,
+                                                              int invert_a, uint64_t nbits, uint64_t per_chunk,
+                                                              BmWs *ws) {
+  const int lane = (int)lane_id();
+  const uint64_t n_words = (nbits + 63) / 64;
+  const uint64_t wave = ((uint64_t)blockIdx.x * kBlock + threadIdx.x) / kWave;
+  const uint64_t n_waves = (uint64_t)gridDim.x * (kBlock / kWave);
+  for (uint64_t chunk = wave; chunk < (uint64_t)kBmChunks; chunk += n_waves) {
+    const uint64_t begin = chunk * per_chunk, end = min(n_words, begin + per_chunk);
+    uint32_t found = 0;
+    for (uint64_t w0 = begin; w0 < end; w0 += kWave) {
+      const uint64_t w = w0 + lane;
+      if (w < end) found += __popcll(bm_word(a, b, invert_a != 0, nbits, w));
+    }
+#pragma unroll
+    for (int d = kWave / 2; d > 0; d >>= 1) found += __shfl_xor(found, d);
+    if (lane == 0) ws->base[chunk] = found;
+  }
+}
+
+__global__ __launch_bounds__(kBlock) void bitmap_scan_kernel(BmWs *ws, uint32_t *total_host) {
+  constexpr int kPer = kBmChunks / kBlock;  // 32 chunks per thread
+  __shared__ uint32_t part[kBlock];
+  const int tid = threadIdx.x;
+  uint32_t sum = 0;
+  for (int j = 0; j < kPer; ++j) sum += ws->base[tid * kPer + j];
+  part[tid] = sum;
+  __syncthreads();
+  for (int s = 1; s < kBlock; s <<= 1) {  // inclusive prefix sums
+    const uint32_t add = tid >= s ? part[tid - s] : 0;
+    __syncthreads();
+    part[tid] += add;
+    __syncthreads();
+  }
+  uint32_t run = part[tid] - sum;
+  for (int j = 0; j < kPer; ++j) {
+    const uint32_t c = ws->base[tid * kPer + j];
+    ws->base[tid * kPer + j] = run;
+    run += c;
+  }
+  if (tid == kBlock - 1) {
+    ws->total = part[tid];
+    if (total_host) *total_host = part[tid];
+  }
+}
+
+__global__ __launch_bounds__(kBlock) void bitmap_emit_kernel(const unsigned long long *a, const unsigned long long *b,
+                                                             int invert_a, uint64_t nbits, uint64_t per_chunk,
+                                                             const BmWs *ws, uint32_t *out, uint64_t max_out) {
+  const int lane = (int)lane_id();
+  const uint64_t n_words = (nbits + 63) / 64;
+  const uint64_t wave = ((uint64_t)blockIdx.x * kBlock + threadIdx.x) / kWave;
+  const uint64_t n_waves = (uint64_t)gridDim.x * (kBlock / kWave);
+  for (uint64_t chunk = wave; chunk < (uint64_t)kBmChunks; chunk += n_waves) {
+    const uint64_t begin = chunk * per_chunk, end = min(n_words, begin + per_chunk);
+    uint64_t pos0 = ws->base[chunk];
+    for (uint64_t w0 = begin; w0 < end && pos0 < max_out; w0 += kWave) {
+      const uint64_t w = w0 + lane;
+      unsigned long long m = w < end ? bm_word(a, b, invert_a != 0, nbits, w) : 0ull;
+      const uint32_t mine = __popcll(m);
+      uint32_t incl = mine;
+#pragma unroll
+      for (int s = 1; s < kWave; s <<= 1) {
+        const uint32_t up = __shfl_up(incl, s);
+        if (lane >= s) incl += up;
+      }
+      uint64_t pos = pos0 + incl - mine;
+      while (m) {
+        const int bit = __builtin_ctzll(m);
+        m &= m - 1;
+        if (pos < max_out) out[pos] = (uint32_t)(w * 64 + bit);
+        ++pos;
+      }
+      pos0 += __shfl(incl, kWave - 1);
+    }
+  }
+}
+
+__global__ __launch_bounds__(kBlock) void bitmap_update_kernel(unsigned long long *bitmap, uint64_t nbits,
+                                                               const uint32_t *idx, size_t n, int set,
+                                                               uint32_t *status) {
+  for (size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x; i < n; i += (size_t)gridDim.x * kBlock) {
+    const uint32_t p = idx[i];
+    if (p >= nbits) {
+      atomicOr(status, UGK_ST_KEY_OUT_OF_RANGE);
+      continue;
+    }
+    const unsigned long long bit = 1ull << (p & 63);
+    if (set) atomicOr(bitmap + (p >> 6), bit);
+    else atomicAnd(bitmap + (p >> 6), ~bit);
+  }
+}
+
+__global__ __launch_bounds__(kBlock) void rows_to_keys_kernel(const uint32_t *rows, size_t n, uint64_t mul,
+                                                              uint64_t mask, long long *keys) {
+  for (size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x; i < n; i += (size_t)gridDim.x * kBlock)
+    keys[i] = (long long)(((uint64_t)rows[i] * mul) & mask);
+}
+
+}  // namespace
+}  // namespace ugk
+
+using namespace ugk;
+
+extern "C" {
+
+size_t ugk_rank_workspace_bytes(void) { return sizeof(RankWs); }
+
+int ugk_rank_select(const uint32_t *counts_dev, uint64_t num_rows, uint64_t k, void *ws_dev, void *stream) {
+  UGK_REQUIRE(counts_dev && ws_dev, "ugk_rank_select: null pointer");
+  UGK_REQUIRE(num_rows > 0 && num_rows < 0xffffffffull, "ugk_rank_select: %llu rows do not fit 32 bits",
+              (unsigned long long)num_rows);
+  UGK_REQUIRE((uintptr_t)counts_dev % 16 == 0 && (uintptr_t)ws_dev % 8 == 0, "ugk_rank_select: misaligned buffer");
+  RankWs *ws = static_cast<RankWs *>(ws_dev);
+  hipStream_t st = as_stream(stream);
+  if (k == 0 || k >= num_rows) {  // nothing, or everything, ranks at or above the threshold
+    hipLaunchKernelGGL(rank_init_kernel, dim3(1), dim3(kBlock), 0, st, ws, k == 0 ? ~0ull : 0ull, 0ull);
+    UGK_HIP(hipGetLastError());
+    return 0;
+  }
+  hipLaunchKernelGGL(rank_init_kernel, dim3(1), dim3(kBlock), 0, st, ws, 0ull, (unsigned long long)k);
+  // a few long workgroups: every workgroup ends with a flush of its histogram into the shared one
+  const unsigned grid = clamp_grid((num_rows / 4 + kBlock - 1) / kBlock, (unsigned)cu_count() * 8u);
+  for (int p = 0; p < kSelectPasses; ++p) {
+    hipLaunchKernelGGL(rank_hist_kernel, dim3(grid), dim3(kBlock), 0, st, counts_dev, num_rows, ws, kPassShift[p],
+                       kPassBits[p]);
+    hipLaunchKernelGGL(rank_pick_kernel, dim3(1), dim3(kBlock), 0, st, ws, kPassShift[p]);
+  }
+  UGK_HIP(hipGetLastError());
+  return 0;
+}
+
+int ugk_rank_threshold(const void *ws_dev, uint64_t *threshold_host, void *stream) {
+  UGK_REQUIRE(ws_dev && threshold_host, "ugk_rank_threshold: null pointer");
+  UGK_HIP(hipMemcpyAsync(threshold_host, ws_dev, sizeof(uint64_t), hipMemcpyDeviceToHost, as_stream(stream)));
+  UGK_HIP(hipStreamSynchronize(as_stream(stream)));
+  return 0;
+}
+
+int ugk_rank_mark(uint32_t *counts_dev, uint64_t num_rows, const void *ws_dev, uint64_t *bitmap_dev, int reset_counts,
+                  void *stream) {
+  UGK_REQUIRE(counts_dev && ws_dev && bitmap_dev, "ugk_rank_mark: null pointer");
+  UGK_REQUIRE(num_rows > 0 && num_rows < 0xffffffffull, "ugk_rank_mark: %llu rows do not fit 32 bits",
+              (unsigned long long)num_rows);
+  const uint64_t n_words = (num_rows + 63) / 64;
+  const unsigned grid =
+      clamp_grid((n_words + kMarkWords * (kBlock / kWave) - 1) / (kMarkWords * (kBlock / kWave)), 0);
+  hipLaunchKernelGGL(rank_mark_kernel, dim3(grid), dim3(kBlock), 0, as_stream(stream), counts_dev, num_rows,
+                     static_cast<const RankWs *>(ws_dev), reinterpret_cast<unsigned long long *>(bitmap_dev),
+                     reset_counts);
+  UGK_HIP(hipGetLastError());
+  return 0;
+}
+
+size_t ugk_bitmap_workspace_bytes(void) { return sizeof(BmWs); }
+
+int ugk_bitmap_count(const uint64_t *a_dev, const uint64_t *b_dev, int invert_a, uint64_t nbits, void *ws_dev,
+                     uint32_t *total_host, void *stream) {
+  UGK_REQUIRE(a_dev && ws_dev, "ugk_bitmap_count: null pointer");
+  UGK_REQUIRE(nbits > 0 && nbits <= 0xffffffffull, "ugk_bitmap_count: %llu bits do not fit 32-bit positions",
+              (unsigned long long)nbits);
+  const uint64_t n_words = (nbits + 63) / 64;
+  const uint64_t per_chunk = bm_words_per_chunk(n_words);
+  // every chunk slot is written (the empty ones with zero), so the scan needs no clearing in front of it
+  const unsigned grid = clamp_grid((kBmChunks + (kBlock / kWave) - 1) / (kBlock / kWave), (unsigned)cu_count() * 8u);
+  hipLaunchKernelGGL(bitmap_count_kernel, dim3(grid), dim3(kBlock), 0, as_stream(stream),
+                     reinterpret_cast<const unsigned long long *>(a_dev),
+                     reinterpret_cast<const unsigned long long *>(b_dev), invert_a, nbits, per_chunk,
+                     static_cast<BmWs *>(ws_dev));
+  hipLaunchKernelGGL(bitmap_scan_kernel, dim3(1), dim3(kBlock), 0, as_stream(stream), static_cast<BmWs *>(ws_dev),
+                     total_host);
+  UGK_HIP(hipGetLastError());
+  return 0;
+}
+
+int ugk_bitmap_emit(const uint64_t *a_dev, const uint64_t *b_dev, int invert_a, uint64_t nbits, const void *ws_dev,
+                    uint32_t *out_dev, uint64_t max_out, void *stream) {
+  UGK_REQUIRE(a_dev && ws_dev, "ugk_bitmap_emit: null pointer");
+  UGK_REQUIRE(nbits > 0 && nbits <= 0xffffffffull, "ugk_bitmap_emit: %llu bits do not fit 32-bit positions",
+              (unsigned long long)nbits);
+  if (max_out == 0) return 0;
+  UGK_REQUIRE(out_dev, "ugk_bitmap_emit: null output list");
+  const uint64_t n_words = (nbits + 63) / 64;
+  const uint64_t per_chunk = bm_words_per_chunk(n_words);
+  const unsigned grid = clamp_grid((kBmChunks + (kBlock / kWave) - 1) / (kBlock / kWave), (unsigned)cu_count() * 8u);
+  hipLaunchKernelGGL(bitmap_emit_kernel, dim3(grid), dim3(kBlock), 0, as_stream(stream),
+                     reinterpret_cast<const unsigned long long *>(a_dev),
+                     reinterpret_cast<const unsigned long long *>(b_dev), invert_a, nbits, per_chunk,
+                     static_cast<const BmWs *>(ws_dev), out_dev, max_out);
+  UGK_HIP(hipGetLastError());
+  return 0;
+}
+
+int ugk_bitmap_update(uint64_t *bitmap_dev, uint64_t nbits, const uint32_t *idx_dev, size_t n, int set,
+                      uint32_t *status_dev, void *stream) {
+  if (n == 0) return 0;
+  UGK_REQUIRE(bitmap_dev && idx_dev && status_dev, "ugk_bitmap_update: null pointer");
+  const unsigned grid = clamp_grid((n + kBlock - 1) / kBlock, 0);
+  hipLaunchKernelGGL(bitmap_update_kernel, dim3(grid), dim3(kBlock), 0, as_stream(stream),
+                     reinterpret_cast<unsigned long long *>(bitmap_dev), nbits, idx_dev, n, set, status_dev);
+  UGK_HIP(hipGetLastError());
+  return 0;
+}
+
+int ugk_rows_to_keys(const uint32_t *rows_dev, size_t n, uint64_t mul, uint64_t mask, int64_t *keys_out_dev,
+                     void *stream) {
+  if (n == 0) return 0;
+  UGK_REQUIRE(rows_dev && keys_out_dev, "ugk_rows_to_keys: null pointer");
+  UGK_REQUIRE(mul & 1ull, "ugk_rows_to_keys: the key multiplier must be odd");
+  const unsigned grid = clamp_grid((n + kBlock - 1) / kBlock, 0);
+  hipLaunchKernelGGL(rows_to_keys_kernel, dim3(grid), dim3(kBlock), 0, as_stream(stream), rows_dev, n, mul, mask,
+                     reinterpret_cast<long long *>(keys_out_dev));
+  UGK_HIP(hipGetLastError());
+  return 0;
+}
+
+}  // extern "C"

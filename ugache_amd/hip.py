@@ -94,9 +94,19 @@ SIGNATURES = {
     "ugk_record_u32": [_vp, _sz, _u64, _u64, _vp, _u64, _vp, _vp, _vp],
     "ugk_record_i64": [_vp, _sz, _u64, _u64, _vp, _u64, _vp, _vp, _vp],
     "ugk_record_drain": [_vp, _u64, _u64, _vp, _u32, _vp, _vp, _vp],
+    "ugk_rank_workspace_bytes": [],
+    "ugk_rank_select": [_vp, _u64, _u64, _vp, _vp],
+    "ugk_rank_threshold": [_vp, _vp, _vp],
+    "ugk_rank_mark": [_vp, _u64, _vp, _vp, C.c_int, _vp],
+    "ugk_bitmap_workspace_bytes": [],
+    "ugk_bitmap_count": [_vp, _vp, C.c_int, _u64, _vp, _vp, _vp],
+    "ugk_bitmap_emit": [_vp, _vp, C.c_int, _u64, _vp, _vp, _u64, _vp],
+    "ugk_bitmap_update": [_vp, _u64, _vp, _sz, C.c_int, _vp, _vp],
+    "ugk_rows_to_keys": [_vp, _sz, _u64, _u64, _vp, _vp],
     "ugk_last_error": [],
 }
-_RESTYPES = {"ugk_hash_buckets_for": _sz, "ugk_dedup_workspace_bytes": _sz, "ugk_last_error": C.c_char_p}
+_RESTYPES = {"ugk_hash_buckets_for": _sz, "ugk_dedup_workspace_bytes": _sz, "ugk_rank_workspace_bytes": _sz,
+             "ugk_bitmap_workspace_bytes": _sz, "ugk_last_error": C.c_char_p}
 _NO_CHECK = set(_RESTYPES) | {"ugk_abi_version"}
 
 _lib = None
