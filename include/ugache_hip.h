@@ -253,17 +253,18 @@ int ugk_record_drain(uint32_t *counts_dev, uint64_t first_row, uint64_t num_rows
  * RefreshSession::refresh_after_solve_new (cache_context.cu:3944-4107).
  * Rank of row r with counter c: c > 0: (c << 32) | r;  c == 0: 0xffffffff - r  (never-counted rows rank behind all
  * counted ones, in ascending row order).  All ranks are distinct.
- * ugk_rank_select: leaves in ws_dev (ugk_rank_workspace_bytes() bytes, 8-byte aligned) the k-th largest rank of
- * rows [0, num_rows) as a threshold (k == 0: nothing reaches it; k >= num_rows: every row does).  counts_dev
- * must be 16-byte aligned; num_rows < 2^32 - 1.  Six streaming passes over the counters; no host round trip.
- * ugk_rank_threshold: copies the threshold to the host (blocking; for tests and logs).
- * ugk_rank_mark: bit r of bitmap_dev (ceil(num_rows / 64) words, every word written) = rank(r) >= threshold;
- * with reset_counts != 0 the counters are zeroed in the same pass. */
+ * ugk_rank_place: bit r of in_new_dev (ceil(num_rows / 64) words, every word written) = row r is one of the k
+ * best-ranked rows of [0, num_rows) (k == 0: no row; k >= num_rows: every row).  Two streaming passes over the
+ * counters (five when the k-th best count is 2047 or more) and a few launches over bitmaps; no host round trip.
+ * counts_dev must be 16-byte aligned; num_rows < 2^32 - 1; ws_dev: ugk_rank_workspace_bytes() bytes, 8-byte aligned;
+ * scratch_bitmap_dev: as large as in_new_dev, overwritten.  With reset_counts != 0 the counters are zeroed in the
+ * second pass.
+ * ugk_rank_threshold: copies the rank of the k-th best row of the last ugk_rank_place to the host (blocking; for tests
+ * and logs; all ones for k == 0, zero for k >= num_rows). */
 size_t ugk_rank_workspace_bytes(void);
-int ugk_rank_select(const uint32_t *counts_dev, uint64_t num_rows, uint64_t k, void *ws_dev, void *stream);
+int ugk_rank_place(uint32_t *counts_dev, uint64_t num_rows, uint64_t k, void *ws_dev, uint64_t *in_new_dev,
+                   uint64_t *scratch_bitmap_dev, int reset_counts, void *stream);
 int ugk_rank_threshold(const void *ws_dev, uint64_t *threshold_host, void *stream);
-int ugk_rank_mark(uint32_t *counts_dev, uint64_t num_rows, const void *ws_dev, uint64_t *bitmap_dev, int reset_counts,
-                  void *stream);
 /* Ordered compaction over bitmaps.  The set S = { p < nbits : bit p of m is set }, m = (invert_a ? ~a : a) & ~b
  * (b_dev may be NULL).  ugk_bitmap_count writes |S| to *total_host (pinned host word, may be NULL) and leaves the
  * per-chunk offsets in ws_dev (ugk_bitmap_workspace_bytes() bytes); ugk_bitmap_emit, called with the same a, b,

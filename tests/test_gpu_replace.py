@@ -31,22 +31,30 @@ def _counts(rng, n, kind):
         return (rng.integers(0, 1 << 32, size=n, dtype=np.uint64) * (rng.random(n) < 0.7)).astype(np.uint32)
     if kind == "zero":
         return np.zeros(n, np.uint32)
+    if kind == "saturated":  # the k-th best count lies at or beyond the 2047 the first histogram pass tells apart
+        return rng.integers(2040, 2060, size=n).astype(np.uint32) * (rng.random(n) < 0.9)
     raise AssertionError(kind)
 
 
-def _select(counts, k):
+def _place(counts, k, reset):
+    """-> membership bits of the k best rows, the rank threshold, the counters afterwards"""
     n = len(counts)
+    words = (n + 63) // 64
     d_counts = to_dev(counts)
     ws = dev_bytes(hip.lib().ugk_rank_workspace_bytes())
-    hip.call("ugk_rank_select", ptr(d_counts), n, k, ptr(ws), None)
+    bitmap = dev_bytes(words * 8, fill=0xA5)
+    scratch = dev_bytes(words * 8, fill=0x5A)
+    hip.call("ugk_rank_place", ptr(d_counts), n, k, ptr(ws), ptr(bitmap), ptr(scratch), reset, None)
     th = C.c_uint64(0)
     hip.call("ugk_rank_threshold", ptr(ws), C.byref(th), None)
-    return d_counts, ws, th.value
+    bits = np.unpackbits(to_np(bitmap)[: words * 8], bitorder="little")
+    assert not bits[n:].any()  # the tail of the last word is clear
+    return bits[:n].astype(bool), th.value, to_np(d_counts, np.uint32)[:n]
 
 
-@pytest.mark.parametrize("kind", ["zipf", "ties", "huge", "zero"])
+@pytest.mark.parametrize("kind", ["zipf", "ties", "huge", "zero", "saturated"])
 @pytest.mark.parametrize("n", [1, 3, 63, 64, 65, 1000, 100_003, 2_000_001])
-def test_rank_select_and_mark_match_a_full_sort(kind, n):
+def test_rank_place_matches_a_full_sort(kind, n):
     rng = np.random.default_rng(n * 7 + len(kind))
     counts = _counts(rng, n, kind)
     ranks = ranks_of(counts)
@@ -54,38 +62,28 @@ def test_rank_select_and_mark_match_a_full_sort(kind, n):
     observed = int((counts > 0).sum())
     ks = sorted({0, 1, n // 3, max(observed - 1, 0), observed, min(observed + 1, n), n - 1, n, n + 5})
     for k in ks:
-        d_counts, ws, th = _select(counts, k)
         if k == 0:
             want = np.zeros(n, bool)
         elif k >= n:
             want = np.ones(n, bool)
         else:
-            assert th == int(order[k - 1]), (kind, n, k)
             want = ranks >= order[k - 1]
         assert int(want.sum()) == min(k, n)
-        words = (n + 63) // 64
         for reset in (0, 1):
-            bitmap = dev_bytes(words * 8, fill=0xA5)
-            hip.call("ugk_rank_mark", ptr(d_counts), n, ptr(ws), ptr(bitmap), reset, None)
-            sync()
-            got = np.unpackbits(to_np(bitmap)[: words * 8], bitorder="little")
-            assert np.array_equal(got[:n].astype(bool), want), (kind, n, k, reset)
-            assert not got[n:].any()  # the tail of the last word is clear
-            left = to_np(d_counts, np.uint32)[:n]
+            got, th, left = _place(counts, k, reset)
+            if 0 < k < n:
+                assert th == int(order[k - 1]), (kind, n, k)
+            assert np.array_equal(got, want), (kind, n, k, reset)
             assert np.array_equal(left, counts if reset == 0 else np.zeros(n, np.uint32))
 
 
-def test_rank_select_picks_the_hotter_rows_and_breaks_ties_towards_larger_rows():
+def test_rank_place_picks_the_hotter_rows_and_breaks_ties_towards_larger_rows():
     # hand-worked: counts 0 5 5 0 9 1 0 -> order 4, 2, 1, 5, then the never-observed rows 0, 3, 6
     counts = np.array([0, 5, 5, 0, 9, 1, 0], np.uint32)
     for k, want_rows in [(1, [4]), (2, [4, 2]), (3, [4, 2, 1]), (4, [4, 2, 1, 5]), (5, [4, 2, 1, 5, 0]),
                          (6, [4, 2, 1, 5, 0, 3])]:
-        d_counts, ws, _ = _select(counts, k)
-        bitmap = dev_bytes(8)
-        hip.call("ugk_rank_mark", ptr(d_counts), len(counts), ptr(ws), ptr(bitmap), 0, None)
-        sync()
-        got = np.flatnonzero(np.unpackbits(to_np(bitmap)[:8], bitorder="little"))
-        assert sorted(got.tolist()) == sorted(want_rows)
+        got, _, _ = _place(counts, k, 0)
+        assert sorted(np.flatnonzero(got).tolist()) == sorted(want_rows)
 
 
 def _bits(rng, nbits, density):

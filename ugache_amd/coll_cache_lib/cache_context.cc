@@ -352,14 +352,13 @@ void ExtractSession::JoinRecord(StreamHandle stream) {
   _record_pending = false;
 }
 
-void ExtractSession::PlaceOnDevice(size_t num_cached, uint64_t *in_new_bits, void *rank_ws, bool reset_counts,
-                                   StreamHandle stream) {
+void ExtractSession::PlaceOnDevice(size_t num_cached, uint64_t *in_new_bits, uint64_t *scratch_bits, void *rank_ws,
+                                   bool reset_counts, StreamHandle stream) {
   CHECK_NOTNULL(_hot_counts) << "placement on the device needs the device-side hotness counters (COLL_GPU_RECORD=1)";
   const size_t rows = _cache_ctx->_num_total_nodes;
   std::lock_guard<std::mutex> guard(_drain_mu);
-  UGK_CALL(ugk_rank_select(_hot_counts->ptr<uint32_t>(), rows, num_cached, rank_ws, _record_stream));
-  UGK_CALL(ugk_rank_mark(_hot_counts->ptr<uint32_t>(), rows, rank_ws, in_new_bits, reset_counts ? 1 : 0,
-                         _record_stream));
+  UGK_CALL(ugk_rank_place(_hot_counts->ptr<uint32_t>(), rows, num_cached, rank_ws, in_new_bits, scratch_bits,
+                          reset_counts ? 1 : 0, _record_stream));
   UGK_CALL(ugk_event_record(_ev_placed, _record_stream));
   UGK_CALL(ugk_stream_wait_event(stream, _ev_placed));
 }
@@ -892,8 +891,8 @@ void RefreshSession::refresh_on_device(ExtractSession *session, size_t num_cache
   t_phase.Reset();
 
   // Steps 1-3: the new placement as a bitmap, then evict = cached & ~new and insert = new & ~cached, ascending
-  session->PlaceOnDevice(num_cached, table->InNewBits(), table->_dev_rank_ws->ptr(), !RunConfig::gpu_refresh_keep,
-                         stream);
+  session->PlaceOnDevice(num_cached, table->InNewBits(), table->_dev_scratch_bits->ptr<uint64_t>(),
+                         table->_dev_rank_ws->ptr(), !RunConfig::gpu_refresh_keep, stream);
   size_t num_evicted = 0, num_insert = 0;
   TensorPtr evict_rows = table->CompactBits(table->InCacheBits(), table->InNewBits(), false, num_rows, SIZE_MAX,
                                             __evict_rows, alloc, gpu_ctx, stream, &num_evicted);

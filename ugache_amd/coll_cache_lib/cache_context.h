@@ -181,7 +181,8 @@ class ExtractSession {
   // Runs on the record stream, ordered against the counting of every lookup; `stream` waits for the result.
   // reset_counts: the next interval starts from zero, as after DrainHotness.
   bool CountsOnDevice() const { return _hot_counts != nullptr; }
-  void PlaceOnDevice(size_t num_cached, uint64_t *in_new_bits, void *rank_ws, bool reset_counts, StreamHandle stream);
+  void PlaceOnDevice(size_t num_cached, uint64_t *in_new_bits, uint64_t *scratch_bits, void *rank_ws,
+                     bool reset_counts, StreamHandle stream);
   // the device-side counting of the following lookups covers only the first `num_keys` keys of a batch
   // (the recorded prefix of LookupManager's record thread); SIZE_MAX, the default: the whole batch
   void SetRecordLimit(size_t num_keys) { _record_limit = num_keys; }

@@ -174,6 +174,7 @@ void CacheEntryManager::EnsureDeviceLists(const std::function<MemHandle(size_t)>
   if (!_dev_in_cache) {
     _dev_in_cache = EagerGPUAlloc(_device_id, row_words * 8);
     _dev_in_new = EagerGPUAlloc(_device_id, row_words * 8);
+    _dev_scratch_bits = EagerGPUAlloc(_device_id, row_words * 8);
     _dev_slot_used = EagerGPUAlloc(_device_id, std::max<size_t>(slot_words, 1) * 8);
     _dev_rank_ws = EagerGPUAlloc(_device_id, ugk_rank_workspace_bytes());
     _dev_bm_ws = EagerGPUAlloc(_device_id, ugk_bitmap_workspace_bytes());

@@ -79,6 +79,7 @@ class CacheEntryManager {
   // refresh on the device reads and updates these; a refresh on the host reads and updates _cached_keys and
   // _free_offsets.  Whichever ran last holds the truth, the other side is brought up to date when it is next needed.
   MemHandle _dev_in_cache, _dev_in_new;  // ceil(num_total_key / 64) words each
+  MemHandle _dev_scratch_bits;           // as large, scratch of the placement
   MemHandle _dev_slot_used;              // ceil(capacity / 64) words
   MemHandle _dev_rank_ws, _dev_bm_ws;    // workspaces of ugk_rank_* / ugk_bitmap_*
   MemHandle _dev_words;                  // pinned host words the kernels report counts in

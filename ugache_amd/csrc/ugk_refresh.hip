@@ -4,9 +4,16 @@
 // optimal_solver_class.cc:1869-1924): observed rows by (count << 32 | row) descending, never-observed rows behind
 // them in ascending row order.
 //
-// select : exact K-th largest rank by a most-significant-digit radix select over all counters (six histogram passes
-//          of 10-11 bits over 64-bit ranks; every pass is one streaming read of the counters, HBM-bound).
-// mark   : one more pass turns "rank >= threshold" into a bitmap with one bit per row (and may reset the counters).
+// place  : the K best-ranked rows as a bitmap, in two streaming passes over the counters (HBM-bound) and a few
+//          launches over bitmaps:
+//            1. histogram of min(count, 2047) -> the count T of the K-th best row and how many rows with count T are
+//               still needed (counts of 2047 and more are rare: then three more histogram passes over the digits of
+//               the count settle T exactly);
+//            2. split: bit r of `gt` = count[r] > T, bit r of `eq` = count[r] == T (and the counters are reset if the
+//               caller wants the next interval to start from zero);
+//            3. the needed rows among `eq` are its topmost set bits (T > 0: larger row first) or its lowest ones
+//               (T == 0: never-observed rows in ascending order): the position of the last needed bit is found with the
+//               chunk offsets of the ordered compaction below; result = gt | (eq restricted to that side of it).
 // bitmap : ordered compaction of the set bits of a, ~a, a & ~b into an ascending index list (count, scan, emit), and
 //          setting / clearing listed bits.  Membership of the cache and occupancy of its slots live in such bitmaps,
 //          so evict = cached & ~new, insert = new & ~cached, free slots = ~used are all the same three launches.
@@ -15,62 +22,76 @@
 namespace ugk {
 namespace {
 
-constexpr int kHistBins = 2048;          // 11-bit digits at most
-constexpr int kBmChunks = 8192;          // fixed partition of a bitmap, independent of the launch grid
-constexpr int kSelectPasses = 6;
-constexpr int kPassShift[kSelectPasses] = {53, 42, 32, 21, 10, 0};
-constexpr int kPassBits[kSelectPasses] = {11, 11, 10, 11, 11, 10};
+constexpr int kHistBins = 2048;        // 11-bit digits at most
+constexpr uint32_t kSatCount = kHistBins - 1;
+constexpr int kBmChunks = 8192;        // fixed partition of a bitmap, independent of the launch grid
+constexpr int kCountPasses = 3;        // digits of a 32-bit count, most significant first
+constexpr int kPassShift[kCountPasses] = {21, 10, 0};
+constexpr int kPassBits[kCountPasses] = {11, 11, 10};
 
-// workspace of select/mark: [0] threshold so far (digits picked from the top), [1] how many ranks at or above the
-// final threshold are still to be found inside the current prefix, then the histogram
+struct BmWs {
+  uint32_t total;
+  uint32_t pad[3];
+  uint32_t base[kBmChunks];  // per chunk: first the count, after the scan the exclusive prefix
+};
+
+// workspace of a placement
 struct RankWs {
-  unsigned long long prefix;
-  unsigned long long remaining;
+  unsigned long long threshold;  // rank of the K-th best row (for reports)
+  unsigned long long remaining;  // rows still to be found: first among all rows, in the end among those with count T
+  uint32_t count_t;              // T (digits picked so far)
+  uint32_t settled;              // the saturating first pass found T
+  uint32_t last_row;             // the last needed row among those with count T
+  uint32_t pad;
   uint32_t hist[kHistBins];
+  BmWs bm;                       // chunk offsets of `eq`
 };
 
 __device__ __forceinline__ unsigned long long rank_of(uint32_t cnt, uint32_t row) {
   return cnt ? ((unsigned long long)cnt << 32) | row : (unsigned long long)(0xffffffffu - row);
 }
 
+// mode 0: digit = min(count, 2047) of every row.  mode 1: digit (shift, bits) of the counts that match the digits
+// picked so far; skipped when the first pass settled T.
 __global__ __launch_bounds__(kBlock) void rank_hist_kernel(const uint32_t *__restrict__ counts, uint64_t n,
-                                                           RankWs *ws, int shift, int bits) {
+                                                           RankWs *ws, int mode, int shift, int bits) {
+  if (mode == 1 && ws->settled) return;
   __shared__ uint32_t lh[kHistBins];
   const int tid = threadIdx.x;
   for (int b = tid; b < kHistBins; b += kBlock) lh[b] = 0;
   __syncthreads();
-  const unsigned long long prefix = ws->prefix;
-  const unsigned long long hi_mask = shift + bits >= 64 ? 0ull : ~0ull << (shift + bits);
-  const unsigned long long want = prefix & hi_mask;
+  const uint32_t hi_mask = (mode == 0 || shift + bits >= 32) ? 0u : ~0u << (shift + bits);
+  const uint32_t want = ws->count_t & hi_mask;
   const uint32_t digit_mask = (1u << bits) - 1u;
-  // consecutive rows mostly share a digit (all cold rows in the count passes, neighbours in the high row passes):
-  // a lane keeps a run and touches the LDS histogram only when the digit changes
+  // consecutive rows mostly share a digit (the cold ones all do): a lane keeps a run and touches the LDS histogram
+  // only when the digit changes
   uint32_t last = 0, run = 0;
+  auto take = [&](uint32_t c) {
+    uint32_t d;
+    if (mode == 0) {
+      d = c < kSatCount ? c : kSatCount;
+    } else {
+      if ((c & hi_mask) != want) return;
+      d = (c >> shift) & digit_mask;
+    }
+    if (d == last) {
+      ++run;
+    } else {
+      if (run) atomicAdd(&lh[last], run);
+      last = d;
+      run = 1;
+    }
+  };
   const uint64_t n_vec = n / 4;
   const u32x4 *cv = reinterpret_cast<const u32x4 *>(counts);
   for (uint64_t v = (uint64_t)blockIdx.x * kBlock + tid; v < n_vec; v += (uint64_t)gridDim.x * kBlock) {
     const u32x4 c = __builtin_nontemporal_load(cv + v);
-    const uint32_t cc[4] = {c.x, c.y, c.z, c.w};
-#pragma unroll
-    for (int k = 0; k < 4; ++k) {
-      const unsigned long long r = rank_of(cc[k], (uint32_t)(v * 4 + k));
-      if ((r & hi_mask) == want) {
-        const uint32_t d = (uint32_t)(r >> shift) & digit_mask;
-        if (d == last) {
-          ++run;
-        } else {
-          if (run) atomicAdd(&lh[last], run);
-          last = d;
-          run = 1;
-        }
-      }
-    }
+    take(c.x);
+    take(c.y);
+    take(c.z);
+    take(c.w);
   }
-  if (blockIdx.x == 0 && tid < (int)(n - n_vec * 4)) {  // the last n % 4 rows
-    const uint64_t row = n_vec * 4 + tid;
-    const unsigned long long r = rank_of(counts[row], (uint32_t)row);
-    if ((r & hi_mask) == want) atomicAdd(&lh[(uint32_t)(r >> shift) & digit_mask], 1u);
-  }
+  if (blockIdx.x == 0 && tid < (int)(n - n_vec * 4)) take(counts[n_vec * 4 + tid]);  // the last n % 4 rows
   if (run) atomicAdd(&lh[last], run);
   __syncthreads();
   for (int b = tid; b < kHistBins; b += kBlock)
@@ -78,10 +99,11 @@ __global__ __launch_bounds__(kBlock) void rank_hist_kernel(const uint32_t *__res
 }
 
 // one workgroup: the digit d with  #(bins above d) < remaining <= #(bins at or above d)
-__global__ __launch_bounds__(kBlock) void rank_pick_kernel(RankWs *ws, int shift) {
+__global__ __launch_bounds__(kBlock) void rank_pick_kernel(RankWs *ws, int mode, int shift) {
   constexpr int kPer = kHistBins / kBlock;  // 8 bins per thread
   __shared__ unsigned long long suffix[kBlock + 1];
   const int tid = threadIdx.x;
+  if (mode == 1 && ws->settled) return;  // uniform: nothing was counted either
   uint32_t h[kPer];
   unsigned long long mine = 0;
 #pragma unroll
@@ -105,8 +127,17 @@ __global__ __launch_bounds__(kBlock) void rank_pick_kernel(RankWs *ws, int shift
 #pragma unroll
     for (int j = kPer - 1; j >= 0; --j) {
       if (above + h[j] >= need) {
-        ws->prefix |= (unsigned long long)(tid * kPer + j) << shift;
-        ws->remaining = need - above;
+        const uint32_t d = (uint32_t)(tid * kPer + j);
+        if (mode == 0) {
+          if (d < kSatCount) {  // counts below the saturation value are exact: T is known
+            ws->count_t = d;
+            ws->remaining = need - above;
+            ws->settled = 1;
+          }
+        } else {
+          ws->count_t |= d << shift;
+          ws->remaining = need - above;
+        }
         break;
       }
       above += h[j];
@@ -116,20 +147,25 @@ __global__ __launch_bounds__(kBlock) void rank_pick_kernel(RankWs *ws, int shift
   for (int j = 0; j < kPer; ++j) ws->hist[tid * kPer + j] = 0;
 }
 
-__global__ void rank_init_kernel(RankWs *ws, unsigned long long prefix, unsigned long long remaining) {
+__global__ void rank_init_kernel(RankWs *ws, unsigned long long remaining) {
   const int tid = threadIdx.x;
   if (tid == 0) {
-    ws->prefix = prefix;
+    ws->threshold = 0;
     ws->remaining = remaining;
+    ws->count_t = 0;
+    ws->settled = 0;
+    ws->last_row = 0;
   }
   for (int b = tid; b < kHistBins; b += blockDim.x) ws->hist[b] = 0;
 }
 
-// bit r of the bitmap = rank(r) >= threshold.  A wavefront takes 64 consecutive rows per load, so a ballot is a word.
+// bit r of gt = count[r] > T, of eq = count[r] == T.  A wavefront takes 64 consecutive rows per load, so a ballot is
+// a word.
 constexpr int kMarkWords = 8;  // words (loads in flight) per wavefront and round
-__global__ __launch_bounds__(kBlock) void rank_mark_kernel(uint32_t *counts, uint64_t n, const RankWs *ws,
-                                                           unsigned long long *bitmap, int reset_counts) {
-  const unsigned long long threshold = ws->prefix;
+__global__ __launch_bounds__(kBlock) void rank_split_kernel(uint32_t *counts, uint64_t n, const RankWs *ws,
+                                                            unsigned long long *gt, unsigned long long *eq,
+                                                            int reset_counts) {
+  const uint32_t t = ws->count_t;
   const int lane = (int)lane_id();
   const uint64_t n_words = (n + 63) / 64;
   const uint64_t wave = ((uint64_t)blockIdx.x * kBlock + threadIdx.x) / kWave;
@@ -144,21 +180,93 @@ __global__ __launch_bounds__(kBlock) void rank_mark_kernel(uint32_t *counts, uin
 #pragma unroll
     for (int k = 0; k < kMarkWords; ++k) {
       const uint64_t row = (w0 + k) * 64 + lane;
-      const bool in = row < n && rank_of(c[k], (uint32_t)row) >= threshold;
-      const unsigned long long word = __ballot(in);
-      if (lane == k && w0 + k < n_words) bitmap[w0 + k] = word;
+      const unsigned long long above = __ballot(row < n && c[k] > t);
+      const unsigned long long equal = __ballot(row < n && c[k] == t);
+      if (lane == k && w0 + k < n_words) {
+        gt[w0 + k] = above;
+        eq[w0 + k] = equal;
+      }
       if (reset_counts && row < n && c[k] != 0) counts[row] = 0;
     }
   }
 }
 
-// ---- bitmaps ----------------------------------------------------------------------------------------------
-struct BmWs {
-  uint32_t total;
-  uint32_t pad[3];
-  uint32_t base[kBmChunks];  // per chunk: first the count, after the scan the exclusive prefix
-};
+// one workgroup: the row of the last needed bit of eq.  With T > 0 the needed rows are the `remaining` topmost set
+// bits, the last of them is bit number total - remaining (counted from the bottom, from 0); with T == 0 they are the
+// lowest ones, the last is number remaining - 1.
+__global__ __launch_bounds__(kBlock) void rank_locate_kernel(RankWs *ws, const unsigned long long *eq, uint64_t nbits,
+                                                             uint64_t per_chunk) {
+  __shared__ uint32_t chunk_of;
+  const int tid = threadIdx.x;
+  const uint32_t total = ws->bm.total;
+  const uint32_t index = ws->count_t ? total - (uint32_t)ws->remaining : (uint32_t)ws->remaining - 1u;
+  constexpr int kPer = kBmChunks / kBlock;
+  for (int j = 0; j < kPer; ++j) {
+    const int c = tid * kPer + j;
+    const uint32_t lo = ws->bm.base[c], hi = c + 1 < kBmChunks ? ws->bm.base[c + 1] : total;
+    if (lo <= index && index < hi) chunk_of = (uint32_t)c;  // exactly one chunk holds it
+  }
+  __syncthreads();
+  if (tid >= kWave) return;
+  const uint32_t c = chunk_of;
+  const uint64_t n_words = (nbits + 63) / 64;
+  const uint64_t begin = (uint64_t)c * per_chunk, end = min(n_words, begin + per_chunk);
+  uint32_t skip = index - ws->bm.base[c];  // set bits of the chunk below the wanted one
+  for (uint64_t w0 = begin; w0 < end; w0 += kWave) {
+    const uint64_t w = w0 + tid;
+    unsigned long long m = w < end ? eq[w] : 0ull;
+    const uint32_t mine = __popcll(m);
+    uint32_t incl = mine;
+#pragma unroll
+    for (int s = 1; s < kWave; s <<= 1) {
+      const uint32_t up = __shfl_up(incl, s);
+      if (tid >= s) incl += up;
+    }
+    const uint32_t all = __shfl(incl, kWave - 1);
+    if (skip < all) {  // in this group of words; wavefront-uniform
+      if (incl - mine <= skip && skip < incl) {
+        uint32_t drop = skip - (incl - mine);
+        while (drop--) m &= m - 1;
+        const uint32_t row = (uint32_t)(w * 64 + __builtin_ctzll(m));
+        ws->last_row = row;
+        ws->threshold = rank_of(ws->count_t, row);
+      }
+      return;
+    }
+    skip -= all;
+  }
+}
 
+// in_new = gt | (eq on the needed side of last_row); gt is in_new itself
+__global__ __launch_bounds__(kBlock) void rank_combine_kernel(const RankWs *ws, unsigned long long *in_new,
+                                                              const unsigned long long *eq, uint64_t n_words) {
+  const uint64_t wl = ws->last_row >> 6;
+  const unsigned bl = ws->last_row & 63u;
+  const bool upward = ws->count_t != 0;  // rows at and above last_row, or at and below it
+  for (uint64_t w = (uint64_t)blockIdx.x * kBlock + threadIdx.x; w < n_words; w += (uint64_t)gridDim.x * kBlock) {
+    unsigned long long mask;
+    if (upward) mask = w > wl ? ~0ull : (w == wl ? ~0ull << bl : 0ull);
+    else mask = w < wl ? ~0ull : (w == wl ? (bl == 63 ? ~0ull : (1ull << (bl + 1)) - 1ull) : 0ull);
+    in_new[w] |= eq[w] & mask;
+  }
+}
+
+// every row, or none: bitmap of n set (or clear) bits, counters reset on request
+__global__ __launch_bounds__(kBlock) void rank_fill_kernel(uint32_t *counts, uint64_t n, unsigned long long *bitmap,
+                                                           int all, int reset_counts, RankWs *ws) {
+  const uint64_t n_words = (n + 63) / 64;
+  const uint64_t stride = (uint64_t)gridDim.x * kBlock;
+  for (uint64_t w = (uint64_t)blockIdx.x * kBlock + threadIdx.x; w < n_words; w += stride) {
+    unsigned long long m = all ? ~0ull : 0ull;
+    if (all && n - w * 64 < 64) m = (1ull << (n - w * 64)) - 1ull;
+    bitmap[w] = m;
+  }
+  if (reset_counts)
+    for (uint64_t r = (uint64_t)blockIdx.x * kBlock + threadIdx.x; r < n; r += stride) counts[r] = 0;
+  if (blockIdx.x == 0 && threadIdx.x == 0) ws->threshold = all ? 0ull : ~0ull;
+}
+
+// ---- bitmaps ----------------------------------------------------------------------------------------------
 __device__ __forceinline__ unsigned long long bm_word(const unsigned long long *a, const unsigned long long *b,
                                                       bool invert_a, uint64_t nbits, uint64_t w) {
   unsigned long long m = a[w];
@@ -281,26 +389,46 @@ extern "C" {
 
 size_t ugk_rank_workspace_bytes(void) { return sizeof(RankWs); }
 
-int ugk_rank_select(const uint32_t *counts_dev, uint64_t num_rows, uint64_t k, void *ws_dev, void *stream) {
-  UGK_REQUIRE(counts_dev && ws_dev, "ugk_rank_select: null pointer");
-  UGK_REQUIRE(num_rows > 0 && num_rows < 0xffffffffull, "ugk_rank_select: %llu rows do not fit 32 bits",
+int ugk_rank_place(uint32_t *counts_dev, uint64_t num_rows, uint64_t k, void *ws_dev, uint64_t *in_new_dev,
+                   uint64_t *scratch_bitmap_dev, int reset_counts, void *stream) {
+  UGK_REQUIRE(counts_dev && ws_dev && in_new_dev && scratch_bitmap_dev, "ugk_rank_place: null pointer");
+  UGK_REQUIRE(num_rows > 0 && num_rows < 0xffffffffull, "ugk_rank_place: %llu rows do not fit 32 bits",
               (unsigned long long)num_rows);
-  UGK_REQUIRE((uintptr_t)counts_dev % 16 == 0 && (uintptr_t)ws_dev % 8 == 0, "ugk_rank_select: misaligned buffer");
+  UGK_REQUIRE((uintptr_t)counts_dev % 16 == 0 && (uintptr_t)ws_dev % 8 == 0, "ugk_rank_place: misaligned buffer");
   RankWs *ws = static_cast<RankWs *>(ws_dev);
   hipStream_t st = as_stream(stream);
-  if (k == 0 || k >= num_rows) {  // nothing, or everything, ranks at or above the threshold
-    hipLaunchKernelGGL(rank_init_kernel, dim3(1), dim3(kBlock), 0, st, ws, k == 0 ? ~0ull : 0ull, 0ull);
+  unsigned long long *in_new = reinterpret_cast<unsigned long long *>(in_new_dev);
+  unsigned long long *eq = reinterpret_cast<unsigned long long *>(scratch_bitmap_dev);
+  const uint64_t n_words = (num_rows + 63) / 64;
+  if (k == 0 || k >= num_rows) {  // no row, or every row
+    const unsigned grid = clamp_grid(((reset_counts ? num_rows : n_words) + kBlock - 1) / kBlock, 0);
+    hipLaunchKernelGGL(rank_fill_kernel, dim3(grid), dim3(kBlock), 0, st, counts_dev, num_rows, in_new,
+                       k == 0 ? 0 : 1, reset_counts, ws);
     UGK_HIP(hipGetLastError());
     return 0;
   }
-  hipLaunchKernelGGL(rank_init_kernel, dim3(1), dim3(kBlock), 0, st, ws, 0ull, (unsigned long long)k);
+  hipLaunchKernelGGL(rank_init_kernel, dim3(1), dim3(kBlock), 0, st, ws, (unsigned long long)k);
   // a few long workgroups: every workgroup ends with a flush of its histogram into the shared one
-  const unsigned grid = clamp_grid((num_rows / 4 + kBlock - 1) / kBlock, (unsigned)cu_count() * 8u);
-  for (int p = 0; p < kSelectPasses; ++p) {
-    hipLaunchKernelGGL(rank_hist_kernel, dim3(grid), dim3(kBlock), 0, st, counts_dev, num_rows, ws, kPassShift[p],
-                       kPassBits[p]);
-    hipLaunchKernelGGL(rank_pick_kernel, dim3(1), dim3(kBlock), 0, st, ws, kPassShift[p]);
+  const unsigned hist_grid = clamp_grid((num_rows / 4 + kBlock - 1) / kBlock, (unsigned)cu_count() * 8u);
+  hipLaunchKernelGGL(rank_hist_kernel, dim3(hist_grid), dim3(kBlock), 0, st, counts_dev, num_rows, ws, 0, 0, 11);
+  hipLaunchKernelGGL(rank_pick_kernel, dim3(1), dim3(kBlock), 0, st, ws, 0, 0);
+  for (int p = 0; p < kCountPasses; ++p) {  // leave at once when the first pass settled T
+    hipLaunchKernelGGL(rank_hist_kernel, dim3(hist_grid), dim3(kBlock), 0, st, counts_dev, num_rows, ws, 1,
+                       kPassShift[p], kPassBits[p]);
+    hipLaunchKernelGGL(rank_pick_kernel, dim3(1), dim3(kBlock), 0, st, ws, 1, kPassShift[p]);
   }
+  const unsigned split_grid =
+      clamp_grid((n_words + kMarkWords * (kBlock / kWave) - 1) / (kMarkWords * (kBlock / kWave)), 0);
+  hipLaunchKernelGGL(rank_split_kernel, dim3(split_grid), dim3(kBlock), 0, st, counts_dev, num_rows, ws, in_new, eq,
+                     reset_counts);
+  const uint64_t per_chunk = bm_words_per_chunk(n_words);
+  const unsigned bm_grid = clamp_grid((kBmChunks + (kBlock / kWave) - 1) / (kBlock / kWave), (unsigned)cu_count() * 8u);
+  hipLaunchKernelGGL(bitmap_count_kernel, dim3(bm_grid), dim3(kBlock), 0, st, eq, (const unsigned long long *)nullptr, 0,
+                     num_rows, per_chunk, &ws->bm);
+  hipLaunchKernelGGL(bitmap_scan_kernel, dim3(1), dim3(kBlock), 0, st, &ws->bm, (uint32_t *)nullptr);
+  hipLaunchKernelGGL(rank_locate_kernel, dim3(1), dim3(kBlock), 0, st, ws, eq, num_rows, per_chunk);
+  const unsigned comb_grid = clamp_grid((n_words + kBlock - 1) / kBlock, 0);
+  hipLaunchKernelGGL(rank_combine_kernel, dim3(comb_grid), dim3(kBlock), 0, st, ws, in_new, eq, n_words);
   UGK_HIP(hipGetLastError());
   return 0;
 }
@@ -309,21 +437,6 @@ int ugk_rank_threshold(const void *ws_dev, uint64_t *threshold_host, void *strea
   UGK_REQUIRE(ws_dev && threshold_host, "ugk_rank_threshold: null pointer");
   UGK_HIP(hipMemcpyAsync(threshold_host, ws_dev, sizeof(uint64_t), hipMemcpyDeviceToHost, as_stream(stream)));
   UGK_HIP(hipStreamSynchronize(as_stream(stream)));
-  return 0;
-}
-
-int ugk_rank_mark(uint32_t *counts_dev, uint64_t num_rows, const void *ws_dev, uint64_t *bitmap_dev, int reset_counts,
-                  void *stream) {
-  UGK_REQUIRE(counts_dev && ws_dev && bitmap_dev, "ugk_rank_mark: null pointer");
-  UGK_REQUIRE(num_rows > 0 && num_rows < 0xffffffffull, "ugk_rank_mark: %llu rows do not fit 32 bits",
-              (unsigned long long)num_rows);
-  const uint64_t n_words = (num_rows + 63) / 64;
-  const unsigned grid =
-      clamp_grid((n_words + kMarkWords * (kBlock / kWave) - 1) / (kMarkWords * (kBlock / kWave)), 0);
-  hipLaunchKernelGGL(rank_mark_kernel, dim3(grid), dim3(kBlock), 0, as_stream(stream), counts_dev, num_rows,
-                     static_cast<const RankWs *>(ws_dev), reinterpret_cast<unsigned long long *>(bitmap_dev),
-                     reset_counts);
-  UGK_HIP(hipGetLastError());
   return 0;
 }
 
