@@ -507,13 +507,15 @@ def test_hotness_counted_on_the_device_ranks_like_the_host_recorder(pct, impl, d
     assert _basics.C_LIB_CTYPES.coll_cache_rank_hotness(0, None, None, 0) == 0  # drained
 
 
-@pytest.mark.parametrize("gpu_record", [False, True])
+@pytest.mark.parametrize("gpu_record", [False, True, "and_refresh"])
 @pytest.mark.parametrize("kdtype", [torch.int32, torch.int64])
 def test_serving_loop_records_a_prefix_and_refreshes_in_the_background(gpu_record, kdtype, monkeypatch):
     """LookupManager::forward re-expressed (lookup_manager.cc:158-213): every step records the first share of its
     batch, looks the batch up, and at step refresh_iter starts a background refresh from what was recorded."""
     if gpu_record:
         monkeypatch.setenv("COLL_GPU_RECORD", "1")
+    if gpu_record == "and_refresh":  # the background refresh is computed on the device as well
+        monkeypatch.setenv("COLL_GPU_REFRESH", "1")
     monkeypatch.setenv("COLL_REFRESH_SLEEP_US", "100")
     rng = np.random.default_rng(44)
     n_item, dim, pct, frac = 30_000, 32, 0.2, 0.5
