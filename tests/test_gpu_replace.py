@@ -86,6 +86,21 @@ def test_rank_place_picks_the_hotter_rows_and_breaks_ties_towards_larger_rows():
         assert sorted(np.flatnonzero(got).tolist()) == sorted(want_rows)
 
 
+def test_rank_place_on_the_committed_golden_case():
+    """tests/golden/extract_small.json: the record stream counted per row, the 16 best rows placed on the device are
+    the fixture's cached set (written by brute-force loops, not by the oracle)"""
+    import json
+    import os
+    with open(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "extract_small.json")) as f:
+        fx = json.load(f)
+    counts = np.bincount(np.array(fx["record_stream"]), minlength=fx["n_item"]).astype(np.uint32)
+    k = int(fx["n_item"] * fx["cache_percentage"])
+    got, th, _ = _place(counts, k, 0)
+    assert np.flatnonzero(got).tolist() == fx["cached_keys"]
+    last = fx["rank_keys_observed"][k - 1]
+    assert th == (fx["rank_counts_observed"][k - 1] << 32) | last
+
+
 def _bits(rng, nbits, density):
     words = (nbits + 63) // 64
     b = rng.random(words * 64) < density

@@ -334,7 +334,7 @@ void ExtractSession::RecordKeys(const KeyT *nodes, size_t num_nodes, StreamHandl
   if (!_hot_counts || (_num_lookups++ % RunConfig::gpu_record_every) != 0) return;
   num_nodes = std::min(num_nodes, _record_limit);
   if (num_nodes == 0) return;
-  std::lock_guard<std::mutex> guard(_drain_mu);  // not in the middle of a placement's passes
+  std::lock_guard<std::mutex> guard(_enqueue_mu);  // not in the middle of a placement's passes
   if (after == nullptr) {
     UGK_CALL(ugk_event_record(_ev_rec_begin, stream));
     after = _ev_rec_begin;
@@ -356,7 +356,8 @@ void ExtractSession::PlaceOnDevice(size_t num_cached, uint64_t *in_new_bits, uin
                                    bool reset_counts, StreamHandle stream) {
   CHECK_NOTNULL(_hot_counts) << "placement on the device needs the device-side hotness counters (COLL_GPU_RECORD=1)";
   const size_t rows = _cache_ctx->_num_total_nodes;
-  std::lock_guard<std::mutex> guard(_drain_mu);
+  std::lock_guard<std::mutex> no_drain(_drain_mu);
+  std::lock_guard<std::mutex> guard(_enqueue_mu);
   UGK_CALL(ugk_rank_place(_hot_counts->ptr<uint32_t>(), rows, num_cached, rank_ws, in_new_bits, scratch_bits,
                           reset_counts ? 1 : 0, _record_stream));
   UGK_CALL(ugk_event_record(_ev_placed, _record_stream));

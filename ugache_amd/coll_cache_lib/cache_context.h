@@ -129,9 +129,10 @@ class ExtractSession {
   void *_ev_rec_begin = nullptr, *_ev_rec_done = nullptr, *_ev_placed = nullptr;
   bool _record_pending = false;
   size_t _record_limit = SIZE_MAX;
-  // one drain at a time (they share the entry list and its pinned copy); also held while a record kernel or the
-  // passes of a placement are enqueued on the record stream, so that the passes see one state of the counters
-  std::mutex _drain_mu;
+  std::mutex _drain_mu;  // one drain at a time: they share the entry list and its pinned copy
+  // held while a record kernel, or the passes of a placement, are enqueued on the record stream, so that no record
+  // kernel lands between two passes and all of them see one state of the counters (a placement holds both)
+  std::mutex _enqueue_mu;
   uint32_t *_state = nullptr;
   void JoinRecord(StreamHandle stream);
   size_t _num_lookups = 0;
