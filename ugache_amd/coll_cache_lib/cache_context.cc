@@ -734,6 +734,21 @@ TensorPtr RefreshSession::CopyTo1DReuse(TensorPtr &preserved_buffer, TensorPtr s
   return ret;
 }
 
+// cache_context.cu:4045-4052.  With stream-ordered lookups "finished" is a matter of the stream: everything enqueued
+// before this point still saw the old table, everything after it sees the evicted keys as misses.
+void RefreshSession::WaitForOneLookup(ExtractSession *session, bool foreground) {
+  CacheContext *ctx = _cache_ctx.get();
+  const size_t current_progress = ctx->progress.load();
+  const bool stream_ordered = session && session->UsesStreamOrder();
+  if (stream_ordered) UGK_CALL(ugk_stream_sync(stream));
+  AnonymousBarrier::_refresh_instance->Wait();
+  Timer t0;
+  while (!foreground && !stream_ordered && ctx->progress.load() < current_progress + 1) {
+    if (t0.PassedSec() >= 20) break;
+    usleep(50);
+  }
+}
+
 void RefreshSession::CopyRowsIntoSlots(const uint32_t *rows_dev, const uint32_t *slots_dev, size_t num_rows,
                                        bool foreground) {
   CacheContext *ctx = _cache_ctx.get();
@@ -824,18 +839,8 @@ void RefreshSession::refresh_after_solve_new(bool foreground) {
   // Step 5: let one more lookup finish, so that no gather in flight still reads a slot about to be reused.  With
   // stream-ordered lookups "finished" is a matter of the stream: everything enqueued before this point still saw
   // the old table, everything after it sees the evicted keys as misses.
-  const size_t current_progress = ctx->progress.load();
   auto session = coll_cache->session(ctx->_local_location_id);
-  const bool stream_ordered = session && session->UsesStreamOrder();
-  if (stream_ordered) UGK_CALL(ugk_stream_sync(stream));
-  AnonymousBarrier::_refresh_instance->Wait();
-  {
-    Timer t0;
-    while (!foreground && !stream_ordered && ctx->progress.load() < current_progress + 1) {
-      if (t0.PassedSec() >= 20) break;
-      usleep(50);
-    }
-  }
+  WaitForOneLookup(session.get(), foreground);
 
   wait_s = t_phase.Passed();
   t_phase.Reset();
@@ -922,17 +927,7 @@ void RefreshSession::refresh_on_device(ExtractSession *session, size_t num_cache
   t_phase.Reset();
 
   // Step 5: let one more lookup finish, so that no gather in flight still reads a slot about to be reused
-  const size_t current_progress = ctx->progress.load();
-  const bool stream_ordered = session->UsesStreamOrder();
-  if (stream_ordered) UGK_CALL(ugk_stream_sync(stream));
-  AnonymousBarrier::_refresh_instance->Wait();
-  {
-    Timer t0;
-    while (!foreground && !stream_ordered && ctx->progress.load() < current_progress + 1) {
-      if (t0.PassedSec() >= 20) break;
-      usleep(50);
-    }
-  }
+  WaitForOneLookup(session, foreground);
   const double wait_s = t_phase.Passed();
   t_phase.Reset();
 

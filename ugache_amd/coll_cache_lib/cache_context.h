@@ -205,6 +205,8 @@ class RefreshSession {
   void refresh_after_solve_new(bool foreground);
   TensorPtr Empty1DReuse(TensorPtr &preserved_buffer, DataType dtype, std::vector<size_t> shape, Context ctx);
   TensorPtr CopyTo1DReuse(TensorPtr &preserved_buffer, TensorPtr src, Context ctx, StreamHandle stream);
+  // step 5: lets one more lookup finish, so that no gather in flight still reads a slot about to be reused
+  void WaitForOneLookup(ExtractSession *session, bool foreground);
   // copies the listed host rows into the listed cache slots (step 6): in one launch when in the foreground, in
   // small throttled batches behind running lookups otherwise
   void CopyRowsIntoSlots(const uint32_t *rows_dev, const uint32_t *slots_dev, size_t num_rows, bool foreground);
