@@ -710,6 +710,73 @@ def test_random_configurations_are_exact(case, monkeypatch):
         assert out.cpu().numpy().tobytes() == ORC.gather(table, keys.astype(np.int64)).tobytes()
 
 
+def _random_refresh_case(seed):
+    r = np.random.default_rng(5000 + seed)
+    return dict(seed=seed, n_item=int(r.integers(130, 90_000)), dim=int(r.choice([4, 16, 32, 64, 100])),
+                pct=float(r.choice([0.01, 0.1, 0.37, 0.9, 0.99])), table_kind=str(r.choice(["FLAT", "HASH"])),
+                keep=bool(r.integers(0, 2)), sparse=bool(r.integers(0, 3) == 0), zipf=float(r.choice([0.6, 1.05, 1.4])),
+                rounds=int(r.integers(2, 5)), stream_ordered=bool(r.integers(0, 3) == 0))
+
+
+@pytest.mark.parametrize("case", [_random_refresh_case(i) for i in range(24)], ids=lambda c: "seed%d" % c["seed"])
+def test_random_sequences_of_refreshes_on_the_device(case, monkeypatch):
+    """seeded random sweep over table size, cache share (from nearly nothing cached to nearly everything), table kind,
+    sparse ids, accumulating or per-interval hotness: after every refresh computed on the device the cached rows are
+    the oracle's top set of the counted key stream, slots are conserved and lookups reproduce table[keys]"""
+    monkeypatch.setenv("COLL_HASH_TABLE", "HASH" if case["sparse"] else case["table_kind"])
+    monkeypatch.setenv("COLL_GPU_RECORD", "1")
+    monkeypatch.setenv("COLL_GPU_REFRESH", "1")
+    monkeypatch.setenv("COLL_HASH_REBUILD_FRAC", "0.02")
+    if case["keep"]:
+        monkeypatch.setenv("COLL_GPU_REFRESH_KEEP", "1")
+    rng = np.random.default_rng(case["seed"])
+    n_item, dim, pct = case["n_item"], case["dim"], case["pct"]
+    MUL, BITS = 0x9E3779B97F4A7C15, 40
+
+    def ids_of(rows):
+        if not case["sparse"]:
+            return torch.from_numpy(rows.astype(np.int64))
+        return torch.from_numpy(((rows.astype(np.uint64) * np.uint64(MUL)) & np.uint64((1 << BITS) - 1)).astype(np.int64))
+
+    co.config(make_config(n_item, pct))
+    if case["sparse"]:
+        _basics.set_key_map(MUL, BITS)
+    co.coll_cache_record_init(0)
+    perm = rng.permutation(n_item)
+    s0 = perm[zipf_ranks(rng, 3 * n_item, n_item, case["zipf"])]
+    co.coll_torch_record(0, ids_of(s0))
+    emb = co.coll_torch_create_emb_shm(0, n_item, dim, torch.float32)
+    table = fill_table(emb, rng)
+    co.coll_torch_init_t(0, 0, emb, pct)
+    cap = _basics.info(0)["capacity_rows"]
+    _, nid = expected_cached_set(s0.astype(np.uint32), n_item, pct)
+    counted = []
+    for rnd in range(case["rounds"]):
+        swap = rng.choice(n_item, max(n_item // 8, 2), replace=False)
+        perm[swap] = perm[rng.permutation(swap)]
+        for n in (int(rng.integers(1, 2 * n_item + 2)), 1, int(rng.integers(1, 5_000))):
+            rows = perm[zipf_ranks(rng, n, n_item, case["zipf"])]
+            kt = ids_of(rows).cuda()
+            if case["stream_ordered"]:
+                out = co.coll_torch_lookup_async(0, kt, False).clone()
+                co.coll_torch_lookup_wait(0)
+            else:
+                out = co.coll_torch_lookup_key_t_val_ret(0, kt, False)
+            counted.append(rows.astype(np.uint32))
+            assert out.cpu().numpy().tobytes() == ORC.gather(table, rows.astype(np.int64)).tobytes()
+            assert _basics.last_group_offset(0)[1] == int((nid[rows] == 0).sum())
+        co.coll_torch_refresh(0, True)
+        want, nid = expected_cached_set(np.concatenate(counted), n_item, pct)
+        if not case["keep"]:
+            counted.clear()
+        info = _basics.info(0)
+        assert info["cached_rows"] == len(want) and info["free_slots"] + info["cached_rows"] == cap
+        if rnd % 2 == 1 or rnd == case["rounds"] - 1:  # the key list by way of the host-side lists, not every time
+            got = np.zeros(len(want), np.uint32)
+            assert _basics.C_LIB_CTYPES.coll_cache_get_cached_keys(0, got.ctypes.data, len(got)) == len(want)
+            assert np.array_equal(got, want)
+
+
 def test_reference_cpu_runnable_config_full_size():
     """1M x 128 fp32 host table, 65536 int64 keys Zipf(1.1) over a seeded permutation, hottest 10 % cached."""
     rng = np.random.default_rng(1)
