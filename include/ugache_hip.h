@@ -233,18 +233,24 @@ int ugk_dedup_i64(const int64_t *keys_dev, size_t n, void *workspace_dev, uint32
  * every key of the batch; row(key) = key for dense ids (key_inv = 0), else (key * key_inv) & key_mask, the inverse of
  * the sparse-id map (the fb_mul / fb_mask of ugk_table_t).  A key without a row sets UGK_ST_KEY_OUT_OF_RANGE and is
  * not counted. */
+/* observed_dev (may be NULL): one bit per row, ceil(num_rows / 64) words, zero-filled once; the bit of a row is set
+ * when its counter leaves zero, so the bitmap is "counter above zero" at every launch boundary.  ugk_record_drain
+ * clears the bits of the counters it resets; ugk_rank_place reads it to skip its passes over the counters. */
 int ugk_record_u32(const uint32_t *keys_dev, size_t n, uint64_t key_inv, uint64_t key_mask, uint32_t *counts_dev,
-                   uint64_t num_rows, uint32_t *status_dev, uint32_t *host_mirror, void *stream);
+                   uint64_t num_rows, uint64_t *observed_dev, uint32_t *status_dev, uint32_t *host_mirror,
+                   void *stream);
 int ugk_record_i64(const int64_t *keys_dev, size_t n, uint64_t key_inv, uint64_t key_mask, uint32_t *counts_dev,
-                   uint64_t num_rows, uint32_t *status_dev, uint32_t *host_mirror, void *stream);
+                   uint64_t num_rows, uint64_t *observed_dev, uint32_t *status_dev, uint32_t *host_mirror,
+                   void *stream);
 /* hands rows [first_row, first_row + num_rows) to the host: every non-zero counter becomes one word
  * (count << 32) | row in entries_dev (order unspecified; the layout of the reference's FreqEntry {key, cnt},
  * freq_recorder.h:32-40) and is reset to zero in the same atomic step, so a ugk_record_* running concurrently loses
  * nothing.  At most `capacity` entries are written; counters that did not fit stay as they are.
  * n_entries_dev: device word, zero on first use, left zero.  host_out: two pinned host words,
  * [0] = entries written, [1] = 1 when rows were left over (call again). */
-int ugk_record_drain(uint32_t *counts_dev, uint64_t first_row, uint64_t num_rows, uint64_t *entries_dev,
-                     uint32_t capacity, uint32_t *n_entries_dev, uint32_t *host_out, void *stream);
+int ugk_record_drain(uint32_t *counts_dev, uint64_t first_row, uint64_t num_rows, uint64_t *observed_dev,
+                     uint64_t *entries_dev, uint32_t capacity, uint32_t *n_entries_dev, uint32_t *host_out,
+                     void *stream);
 
 /* ---- re-placement on the device, from the counters of ugk_record_* ---------------------------------------------
  * Stands, for hotness counted on the device, for the host passes of a refresh: FreqRecorder::Sort
@@ -257,13 +263,14 @@ int ugk_record_drain(uint32_t *counts_dev, uint64_t first_row, uint64_t num_rows
  * best-ranked rows of [0, num_rows) (k == 0: no row; k >= num_rows: every row).  Two streaming passes over the
  * counters (five when the k-th best count is 2047 or more) and a few launches over bitmaps; no host round trip.
  * counts_dev must be 16-byte aligned; num_rows < 2^32 - 1; ws_dev: ugk_rank_workspace_bytes() bytes, 8-byte aligned;
- * scratch_bitmap_dev: as large as in_new_dev, overwritten.  With reset_counts != 0 the counters are zeroed in the
- * second pass.
+ * scratch_bitmap_dev: as large as in_new_dev, overwritten.  With reset_counts != 0 the counters (and observed_dev)
+ * are zeroed on the way.  observed_dev (may be NULL): the bitmap ugk_record_* keeps; when fewer rows were observed
+ * than k asks for, the k-th best count is 0 without looking and no pass over the counters is made at all.
  * ugk_rank_threshold: copies the rank of the k-th best row of the last ugk_rank_place to the host (blocking; for tests
  * and logs; all ones for k == 0, zero for k >= num_rows). */
 size_t ugk_rank_workspace_bytes(void);
 int ugk_rank_place(uint32_t *counts_dev, uint64_t num_rows, uint64_t k, void *ws_dev, uint64_t *in_new_dev,
-                   uint64_t *scratch_bitmap_dev, int reset_counts, void *stream);
+                   uint64_t *scratch_bitmap_dev, uint64_t *observed_dev, int reset_counts, void *stream);
 int ugk_rank_threshold(const void *ws_dev, uint64_t *threshold_host, void *stream);
 /* Ordered compaction over bitmaps.  The set S = { p < nbits : bit p of m is set }, m = (invert_a ? ~a : a) & ~b
  * (b_dev may be NULL).  ugk_bitmap_count writes |S| to *total_host (pinned host word, may be NULL) and leaves the

@@ -583,9 +583,11 @@ def test_replicate_rows_fills_duplicates_from_their_representative(row_bytes):
 
 @pytest.mark.parametrize("kdtype", [np.uint32, np.int64])
 @pytest.mark.parametrize("sparse", [False, True])
-def test_record_and_drain_match_bincount(kdtype, sparse):
+@pytest.mark.parametrize("with_bitmap", [False, True])
+def test_record_and_drain_match_bincount(kdtype, sparse, with_bitmap):
     """device-side hotness counters: record == numpy.bincount of the rows; drain hands out every non-zero counter
-    exactly once as (count << 32 | row) and leaves the counters at zero"""
+    exactly once as (count << 32 | row) and leaves the counters at zero; the optional bitmap of observed rows is
+    "counter above zero" after every launch"""
     rng = np.random.default_rng(17 + sparse)
     num_rows = 100_003
     bits = 31 if kdtype == np.uint32 else 40
@@ -593,6 +595,11 @@ def test_record_and_drain_match_bincount(kdtype, sparse):
     mask = (1 << bits) - 1 if sparse else 0
     inv = pow(mul, -1, 1 << bits) if sparse else 0
     counts = dev_zeros_u32(num_rows)
+    observed = to_dev(np.zeros((num_rows + 63) // 64, np.uint64)) if with_bitmap else None
+
+    def observed_rows():
+        return np.flatnonzero(np.unpackbits(to_np(observed, np.uint8), bitorder="little"))
+
     st = dev_zeros_u32(1)
     want = np.zeros(num_rows, np.int64)
     for n in (1, 5000, 200_001):
@@ -600,8 +607,11 @@ def test_record_and_drain_match_bincount(kdtype, sparse):
         keys = ((rows * np.uint64(mul)) & np.uint64(mask)) if sparse else rows
         d_keys = to_dev(keys.astype(kdtype))
         fn = "ugk_record_i64" if kdtype == np.int64 else "ugk_record_u32"
-        hip.call(fn, ptr(d_keys), n, inv, mask, ptr(counts), num_rows, ptr(st), None, None)
+        hip.call(fn, ptr(d_keys), n, inv, mask, ptr(counts), num_rows, ptr(observed), ptr(st), None, None)
         want += np.bincount(rows.astype(np.int64), minlength=num_rows)
+        if with_bitmap:
+            sync()
+            assert np.array_equal(observed_rows(), np.flatnonzero(want))
     sync()
     assert status_value(st) == 0
     assert np.array_equal(to_np(counts, np.uint32)[:num_rows].astype(np.int64), want)
@@ -616,9 +626,12 @@ def test_record_and_drain_match_bincount(kdtype, sparse):
         calls = 0
         for first, cnt in ((0, 50_001), (50_001, num_rows - 50_001)):
             while True:
-                hip.call("ugk_record_drain", ptr(counts), first, cnt, ptr(entries), cap, ptr(n_entries), out.ptr, None)
+                hip.call("ugk_record_drain", ptr(counts), first, cnt, ptr(observed), ptr(entries), cap, ptr(n_entries),
+                         out.ptr, None)
                 sync()
                 calls += 1
+                if with_bitmap:  # also half-way through: a bit is clear exactly where the counter was reset
+                    assert np.array_equal(observed_rows(), np.flatnonzero(to_np(counts, np.uint32)[:num_rows]))
                 k, more = int(out.array[0]), int(out.array[1])
                 e = to_np(entries, np.uint64)[:k]
                 r, c = (e & np.uint64(0xFFFFFFFF)).astype(np.int64), (e >> np.uint64(32)).astype(np.int64)
@@ -640,7 +653,7 @@ def test_record_rejects_keys_without_a_row():
     counts = dev_zeros_u32(10)
     st = dev_zeros_u32(1)
     d_keys = to_dev(np.array([3, 10, -1, 3], np.int64))
-    hip.call("ugk_record_i64", ptr(d_keys), 4, 0, 0, ptr(counts), 10, ptr(st), None, None)
+    hip.call("ugk_record_i64", ptr(d_keys), 4, 0, 0, ptr(counts), 10, None, ptr(st), None, None)
     sync()
     assert status_value(st) & hip.ST_KEY_OUT_OF_RANGE
     assert to_np(counts, np.uint32)[:10].tolist() == [0, 0, 0, 2, 0, 0, 0, 0, 0, 0]
@@ -655,7 +668,7 @@ def test_drain_of_short_and_unaligned_row_ranges(first, cnt):
     n_entries = dev_zeros_u32(1)
     out = PinnedArray((2,), np.uint32)
     try:
-        hip.call("ugk_record_drain", ptr(counts), first, cnt, ptr(entries), 512, ptr(n_entries), out.ptr, None)
+        hip.call("ugk_record_drain", ptr(counts), first, cnt, None, ptr(entries), 512, ptr(n_entries), out.ptr, None)
         sync()
         k = int(out.array[0])
         assert k == cnt and int(out.array[1]) == 0

@@ -36,7 +36,7 @@ def _counts(rng, n, kind):
     raise AssertionError(kind)
 
 
-def _place(counts, k, reset):
+def _place(counts, k, reset, with_observed=False):
     """-> membership bits of the k best rows, the rank threshold, the counters afterwards"""
     n = len(counts)
     words = (n + 63) // 64
@@ -44,11 +44,19 @@ def _place(counts, k, reset):
     ws = dev_bytes(hip.lib().ugk_rank_workspace_bytes())
     bitmap = dev_bytes(words * 8, fill=0xA5)
     scratch = dev_bytes(words * 8, fill=0x5A)
-    hip.call("ugk_rank_place", ptr(d_counts), n, k, ptr(ws), ptr(bitmap), ptr(scratch), reset, None)
+    observed = None
+    if with_observed:  # the bitmap ugk_record_* would have kept: counter above zero
+        pad = np.zeros(words * 64, bool)
+        pad[:n] = counts > 0
+        observed = to_dev(np.packbits(pad, bitorder="little").view(np.uint64))
+    hip.call("ugk_rank_place", ptr(d_counts), n, k, ptr(ws), ptr(bitmap), ptr(scratch), ptr(observed), reset, None)
     th = C.c_uint64(0)
     hip.call("ugk_rank_threshold", ptr(ws), C.byref(th), None)
     bits = np.unpackbits(to_np(bitmap)[: words * 8], bitorder="little")
     assert not bits[n:].any()  # the tail of the last word is clear
+    if with_observed:
+        left = np.unpackbits(to_np(observed, np.uint8)[: words * 8], bitorder="little")[:n].astype(bool)
+        assert np.array_equal(left, (counts > 0) & (reset == 0))  # cleared together with the counters
     return bits[:n].astype(bool), th.value, to_np(d_counts, np.uint32)[:n]
 
 
@@ -69,11 +77,11 @@ def test_rank_place_matches_a_full_sort(kind, n):
         else:
             want = ranks >= order[k - 1]
         assert int(want.sum()) == min(k, n)
-        for reset in (0, 1):
-            got, th, left = _place(counts, k, reset)
+        for reset, with_observed in ((0, False), (1, False), (0, True), (1, True)):
+            got, th, left = _place(counts, k, reset, with_observed)
             if 0 < k < n:
-                assert th == int(order[k - 1]), (kind, n, k)
-            assert np.array_equal(got, want), (kind, n, k, reset)
+                assert th == int(order[k - 1]), (kind, n, k, with_observed)
+            assert np.array_equal(got, want), (kind, n, k, reset, with_observed)
             assert np.array_equal(left, counts if reset == 0 else np.zeros(n, np.uint32))
 
 

@@ -237,6 +237,11 @@ ExtractSession::ExtractSession(std::shared_ptr<CacheContext> cache_ctx) : _cache
     const size_t rows = _cache_ctx->_num_total_nodes;
     _hot_counts = EagerGPUAlloc(dev, std::max<size_t>(rows, 1) * sizeof(uint32_t));
     UGK_CALL(ugk_fill_u32(_hot_counts->ptr<uint32_t>(), 0, rows, nullptr));
+    if (RunConfig::gpu_refresh) {  // which rows have been counted at all: lets a placement skip the cold ones
+      const size_t words = (std::max<size_t>(rows, 1) + 63) / 64;
+      _hot_observed = EagerGPUAlloc(dev, words * 8);
+      UGK_CALL(ugk_fill_u32(_hot_observed->ptr<uint32_t>(), 0, words * 2, nullptr));
+    }
     const size_t cap = std::min<size_t>(std::max<size_t>(rows, 1), kHotDrainRows);
     _hot_entries = EagerGPUAlloc(dev, cap * sizeof(uint64_t));
     _hot_entries_host = PinnedHostAlloc(cap * sizeof(uint64_t));
@@ -316,39 +321,60 @@ static int Dedup(const Id64Type *keys, size_t n, void *ws, uint32_t epoch, Id64T
 }
 
 static int Record(const IdType *keys, size_t n, uint64_t mul, uint64_t mask, uint32_t *counts, uint64_t rows,
-                  uint32_t *st, uint32_t *mirror, StreamHandle s) {
-  return ugk_record_u32(keys, n, mul, mask, counts, rows, st, mirror, s);
+                  uint64_t *observed, uint32_t *st, uint32_t *mirror, StreamHandle s) {
+  return ugk_record_u32(keys, n, mul, mask, counts, rows, observed, st, mirror, s);
 }
 static int Record(const Id64Type *keys, size_t n, uint64_t mul, uint64_t mask, uint32_t *counts, uint64_t rows,
-                  uint32_t *st, uint32_t *mirror, StreamHandle s) {
-  return ugk_record_i64(keys, n, mul, mask, counts, rows, st, mirror, s);
+                  uint64_t *observed, uint32_t *st, uint32_t *mirror, StreamHandle s) {
+  return ugk_record_i64(keys, n, mul, mask, counts, rows, observed, st, mirror, s);
 }
 
 // FreqRecorder::Record of this batch on the device (freq_recorder.cc:227-253).  It runs on a stream of its own behind
-// `after` (an event already recorded on the caller's stream; none: the point the caller's stream has reached now), so
-// it overlaps the gathers; JoinRecord makes the caller's stream wait for it before the lookup returns (the keys
-// belong to the caller again after that).
+// an event on the caller's stream (the point where the keys are ready), so it overlaps the gathers; JoinRecord makes
+// the caller's stream wait for it before the lookup returns (the keys belong to the caller again after that).
+// RecordBegin marks that point and says whether this lookup is counted at all; the extraction kernels are launched
+// next, and only then RecordLaunch enqueues the counting: its handful of API calls then run while the GPU already
+// works on the batch instead of in front of it.
+void *ExtractSession::RecordBegin(StreamHandle stream) {
+  _record_pending = false;
+  if (!_hot_counts || (_num_lookups++ % RunConfig::gpu_record_every) != 0) return nullptr;
+  UGK_CALL(ugk_event_record(_ev_rec_begin, stream));
+  return _ev_rec_begin;
+}
+
+template <typename KeyT>
+void ExtractSession::RecordLaunch(const KeyT *nodes, size_t num_nodes, void *after) {
+  if (after == nullptr) return;
+  num_nodes = std::min(num_nodes, _record_limit);
+  if (num_nodes == 0) return;
+  std::lock_guard<std::mutex> guard(_enqueue_mu);  // not in the middle of a placement's passes
+  UGK_CALL(ugk_stream_wait_event(_record_stream, after));
+  UGK_CALL(Record(nodes, num_nodes, RunConfig::key_map_inv, RunConfig::key_map_mask, _hot_counts->ptr<uint32_t>(),
+                  _cache_ctx->_num_total_nodes, ObservedBits(), _status, _host_mirror, _record_stream));
+  UGK_CALL(ugk_event_record(_ev_rec_done, _record_stream));
+  _record_pending = true;
+}
+
+// the counting behind an event the caller has already recorded on its stream (the classify kernel's)
 template <typename KeyT>
 void ExtractSession::RecordKeys(const KeyT *nodes, size_t num_nodes, StreamHandle stream, void *after) {
   _record_pending = false;
   if (!_hot_counts || (_num_lookups++ % RunConfig::gpu_record_every) != 0) return;
-  num_nodes = std::min(num_nodes, _record_limit);
-  if (num_nodes == 0) return;
-  std::lock_guard<std::mutex> guard(_enqueue_mu);  // not in the middle of a placement's passes
-  if (after == nullptr) {
-    UGK_CALL(ugk_event_record(_ev_rec_begin, stream));
-    after = _ev_rec_begin;
-  }
-  UGK_CALL(ugk_stream_wait_event(_record_stream, after));
-  UGK_CALL(Record(nodes, num_nodes, RunConfig::key_map_inv, RunConfig::key_map_mask, _hot_counts->ptr<uint32_t>(),
-                  _cache_ctx->_num_total_nodes, _status, _host_mirror, _record_stream));
-  UGK_CALL(ugk_event_record(_ev_rec_done, _record_stream));
-  _record_pending = true;
+  (void)stream;
+  RecordLaunch(nodes, num_nodes, after);
 }
 
 void ExtractSession::JoinRecord(StreamHandle stream) {
   if (!_record_pending) return;
   UGK_CALL(ugk_stream_wait_event(stream, _ev_rec_done));
+  _record_pending = false;
+}
+
+// the same for a blocking lookup, after its own wait: the counting has normally finished by then, and waiting for
+// its event on the host keeps a cross-stream dependency out of the caller's stream
+void ExtractSession::JoinRecordOnHost() {
+  if (!_record_pending) return;
+  UGK_CALL(ugk_event_sync(_ev_rec_done));
   _record_pending = false;
 }
 
@@ -359,7 +385,7 @@ void ExtractSession::PlaceOnDevice(size_t num_cached, uint64_t *in_new_bits, uin
   std::lock_guard<std::mutex> no_drain(_drain_mu);
   std::lock_guard<std::mutex> guard(_enqueue_mu);
   UGK_CALL(ugk_rank_place(_hot_counts->ptr<uint32_t>(), rows, num_cached, rank_ws, in_new_bits, scratch_bits,
-                          reset_counts ? 1 : 0, _record_stream));
+                          ObservedBits(), reset_counts ? 1 : 0, _record_stream));
   UGK_CALL(ugk_event_record(_ev_placed, _record_stream));
   UGK_CALL(ugk_stream_wait_event(stream, _ev_placed));
 }
@@ -380,8 +406,8 @@ size_t ExtractSession::DrainHotness(FreqRecorder *recorder) {
   recorder->BeginEntries();
   for (size_t first = 0; first < rows; first += cap) {
     const size_t cur = std::min(cap, rows - first);  // as many rows as the list has room for: nothing is left over
-    UGK_CALL(ugk_record_drain(_hot_counts->ptr<uint32_t>(), first, cur, dev_list, (uint32_t)cap, n_entries, host_out,
-                              _record_stream));
+    UGK_CALL(ugk_record_drain(_hot_counts->ptr<uint32_t>(), first, cur, ObservedBits(), dev_list, (uint32_t)cap,
+                              n_entries, host_out, _record_stream));
     UGK_CALL(ugk_stream_sync(_record_stream));
     const size_t got = host_out[0];
     CHECK_EQ(host_out[kMirDrainMore - kMirDrainCount], 0u);
@@ -480,7 +506,7 @@ void ExtractSession::ExtractFeatImpl(const KeyT *nodes, size_t num_nodes, void *
     CHECK_EQ(ctx->_num_location, 1);
     const bool from_host = ctx->_cpu_location_id != -1;
     // the gather is bracketed by events on its own stream: the logged combine time is the kernel's duration
-    RecordKeys(input_nodes, num_input, stream, nullptr);
+    void *keys_ready = RecordBegin(stream);
     UGK_CALL(ugk_event_record(_ev_t[0], stream));
     if (dst_map == nullptr) {
       UGK_CALL(GatherDirect(ctx->_device_cache_data[0], ctx->_num_total_nodes, nodes, num_nodes, output, rb,
@@ -490,9 +516,10 @@ void ExtractSession::ExtractFeatImpl(const KeyT *nodes, size_t num_nodes, void *
                              num_input, rb, from_host ? _cpu_blocks : 0, _status, _host_mirror, stream));
     }
     UGK_CALL(ugk_event_record(_ev_t[1], stream));
+    RecordLaunch(input_nodes, num_input, keys_ready);
     if (dst_map) UGK_CALL(ugk_replicate_rows(output, rb, inverse, dst_map, num_input, stream));
-    JoinRecord(stream);
     UGK_CALL(ugk_stream_sync(stream));
+    JoinRecordOnHost();
     CheckStatusWord(stream);
     float combine_ms = 0;
     UGK_CALL(ugk_event_elapsed_ms(_ev_t[0], _ev_t[1], &combine_ms));
@@ -528,13 +555,14 @@ void ExtractSession::ExtractFeatImpl(const KeyT *nodes, size_t num_nodes, void *
     // host link is busy from the first wavefront on, with no classify pass and no cross-stream hand-off in front of
     // it, and since the link bounds a mixed batch it does not matter that host loads spread over the chip slow the
     // HBM loads next to them.
-    RecordKeys(input_nodes, num_input, stream, nullptr);
+    void *keys_ready = RecordBegin(stream);
     UGK_CALL(ugk_event_record(_ev_t[0], stream));
     UGK_CALL(ExtractMix(table, nodes, num_nodes, cache, cache_rows, host, host_rows, output, rb, _status,
                         _host_mirror, _state + kStMixCounts, stream));
     UGK_CALL(ugk_event_record(_ev_t[1], stream));
-    JoinRecord(stream);
+    RecordLaunch(input_nodes, num_input, keys_ready);
     UGK_CALL(ugk_stream_sync(stream));
+    JoinRecordOnHost();
     CheckStatusWord(stream);
     const uint32_t n_local = _host_mirror[kMirGroupSizes + UGK_LOC_LOCAL],
                    n_miss = _host_mirror[kMirGroupSizes + UGK_LOC_HOST];
@@ -598,10 +626,10 @@ void ExtractSession::ExtractFeatImpl(const KeyT *nodes, size_t num_nodes, void *
     UGK_CALL(ugk_event_record(_ev_local_done, stream));
   }
   if (dst_map) UGK_CALL(ugk_replicate_rows(output, rb, inverse, dst_map, num_input, stream));
-  JoinRecord(stream);
   // the single blocking wait of the call; the gathers have written their group sizes (and the kernels any error
   // flag) into the pinned mirror, so no device-to-host copy is needed
   UGK_CALL(ugk_stream_sync(stream));
+  JoinRecordOnHost();
   const uint32_t n_local = _host_mirror[kMirGroupSizes + UGK_LOC_LOCAL],
                  n_miss = _host_mirror[kMirGroupSizes + UGK_LOC_HOST];
   _cur ^= 1;
@@ -643,9 +671,10 @@ void ExtractSession::ExtractFeatAsyncImpl(const KeyT *nodes, size_t num_nodes, v
   const bool dedup = RunConfig::dedup_keys && num_nodes >= RunConfig::dedup_min_keys;
   if (ctx->IsDirectMapping() && !dedup) {
     const bool from_host = ctx->_cpu_location_id != -1;
-    RecordKeys(nodes, num_nodes, stream, nullptr);
+    void *keys_ready = RecordBegin(stream);
     UGK_CALL(GatherDirect(ctx->_device_cache_data[0], ctx->_num_total_nodes, nodes, num_nodes, output, rb,
                           from_host ? _cpu_blocks : 0, _status, _host_mirror, stream));
+    RecordLaunch(nodes, num_nodes, keys_ready);
     JoinRecord(stream);
     // what a blocking lookup would have read from the mirror
     _host_mirror[kMirGroupSizes + UGK_LOC_LOCAL] = from_host ? 0 : (uint32_t)num_nodes;
@@ -654,11 +683,12 @@ void ExtractSession::ExtractFeatAsyncImpl(const KeyT *nodes, size_t num_nodes, v
              (((uintptr_t)ctx->_device_cache_data[ctx->_local_location_id] |
                (uintptr_t)ctx->_device_cache_data[ctx->_cpu_location_id] | (uintptr_t)output | (uintptr_t)rb) &
               15u) == 0) {
-    RecordKeys(nodes, num_nodes, stream, nullptr);
+    void *keys_ready = RecordBegin(stream);
     UGK_CALL(ExtractMix(ctx->_new_hash_table->_table, nodes, num_nodes,
                         ctx->_device_cache_data[ctx->_local_location_id], ctx->_cache_space_capacity,
                         ctx->_device_cache_data[ctx->_cpu_location_id], ctx->_num_total_nodes, output, rb, _status,
                         _host_mirror, _state + kStMixCounts, stream));
+    RecordLaunch(nodes, num_nodes, keys_ready);
     JoinRecord(stream);
   } else {
     Wait(stream);

@@ -123,6 +123,8 @@ class ExtractSession {
 
   // hotness counters on the device (RunConfig::gpu_record)
   MemHandle _hot_counts;         // uint32 per row of the host table
+  MemHandle _hot_observed;       // one bit per row: its counter is above zero (kept when refreshes run on the device)
+  uint64_t *ObservedBits() const { return _hot_observed ? _hot_observed->ptr<uint64_t>() : nullptr; }
   MemHandle _hot_entries;        // compact (count << 32 | row) list of one drain step
   MemHandle _hot_entries_host;   // pinned copy of it
   StreamHandle _record_stream = nullptr;  // record kernels and drains run here, beside the extraction
@@ -135,10 +137,14 @@ class ExtractSession {
   std::mutex _enqueue_mu;
   uint32_t *_state = nullptr;
   void JoinRecord(StreamHandle stream);
+  void JoinRecordOnHost();
   size_t _num_lookups = 0;
   static constexpr size_t kHotDrainRows = 32u << 20;  // rows per drain step = capacity of the entry list
   template <typename KeyT>
   void RecordKeys(const KeyT *nodes, size_t num_nodes, StreamHandle stream, void *after);
+  void *RecordBegin(StreamHandle stream);
+  template <typename KeyT>
+  void RecordLaunch(const KeyT *nodes, size_t num_nodes, void *after);
 
   size_t _async_pending = 0;       // stream-ordered lookups enqueued since the last Wait()
   size_t _async_last_nodes = 0;    // size of the last of them

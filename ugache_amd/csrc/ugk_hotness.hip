@@ -24,7 +24,8 @@ constexpr uint32_t kRecEmpty = 0xffffffffu;           // rows are below 2^32 - 1
 
 template <typename K>
 __global__ __launch_bounds__(kBlock) void record_kernel(const K *__restrict__ keys, size_t n, ugk_table_t map,
-                                                        uint32_t *counts, uint64_t num_rows, uint32_t *status,
+                                                        uint32_t *counts, uint64_t num_rows,
+                                                        unsigned long long *observed, uint32_t *status,
                                                         uint32_t *host_mirror) {
   __shared__ uint32_t slot_row[kRecSlots];
   __shared__ uint32_t slot_cnt[kRecSlots];
@@ -59,13 +60,35 @@ __global__ __launch_bounds__(kBlock) void record_kernel(const K *__restrict__ ke
       }
     }
     __syncthreads();
-    for (int s = tid; s < kRecSlots; s += kBlock) {
-      const uint32_t c = slot_cnt[s];
-      if (c) {
-        atomicAdd(counts + slot_row[s], c);
-        slot_row[s] = kRecEmpty;
-        slot_cnt[s] = 0;
+    if (observed == nullptr) {
+      for (int s = tid; s < kRecSlots; s += kBlock) {
+        const uint32_t c = slot_cnt[s];
+        if (c) {
+          atomicAdd(counts + slot_row[s], c);
+          slot_row[s] = kRecEmpty;
+          slot_cnt[s] = 0;
+        }
       }
+    } else {
+      // a counter that leaves zero sets its row's bit: all adds of the thread go out first, their returned values are
+      // looked at afterwards, so the round trips overlap
+      constexpr int kPer = kRecSlots / kBlock;
+      uint32_t rows[kPer], before[kPer];
+#pragma unroll
+      for (int j = 0; j < kPer; ++j) {
+        const int s = j * kBlock + tid;
+        const uint32_t c = slot_cnt[s];
+        rows[j] = slot_row[s];
+        before[j] = 1;
+        if (c) {
+          before[j] = atomicAdd(counts + rows[j], c);
+          slot_row[s] = kRecEmpty;
+          slot_cnt[s] = 0;
+        }
+      }
+#pragma unroll
+      for (int j = 0; j < kPer; ++j)
+        if (before[j] == 0) atomicOr(observed + (rows[j] >> 6), 1ull << (rows[j] & 63));
     }
     __syncthreads();
   }
@@ -112,8 +135,8 @@ __device__ __forceinline__ uint32_t nonzeros(const u32x4 &c) {
 }
 
 __global__ __launch_bounds__(kBlock) void drain_kernel(uint32_t *counts, uint64_t num_rows, uint64_t first_row,
-                                                       unsigned long long *entries, uint32_t capacity,
-                                                       uint32_t *n_entries) {
+                                                       unsigned long long *observed, unsigned long long *entries,
+                                                       uint32_t capacity, uint32_t *n_entries) {
   const int lane = (int)lane_id();
   const uint64_t wave = ((uint64_t)blockIdx.x * kBlock + threadIdx.x) / kWave;
   const uint64_t n_waves = (uint64_t)gridDim.x * (kBlock / kWave);
@@ -155,8 +178,12 @@ __global__ __launch_bounds__(kBlock) void drain_kernel(uint32_t *counts, uint64_
       if (cc[k] != 0) {
         // beyond the reservation or beyond the list: the counter stays as it is for the next drain
         if (idx < found && base + idx < capacity) {
+          // the bit first: an increment that lands between the two steps is part of `got`, one that lands after
+          // them finds the counter at zero and sets the bit again
+          const uint64_t row = first_row + d.row0 + k;
+          if (observed) atomicAnd(observed + (row >> 6), ~(1ull << (row & 63)));
           const uint32_t got = atomicExch(counts + d.row0 + k, 0u);
-          entries[base + idx] = ((unsigned long long)got << 32) | (uint32_t)(first_row + d.row0 + k);
+          entries[base + idx] = ((unsigned long long)got << 32) | (uint32_t)row;
         }
         ++idx;
       }
@@ -175,7 +202,7 @@ __global__ void drain_finish_kernel(uint32_t *n_entries, uint32_t capacity, uint
 
 template <typename K>
 int record(const K *keys, size_t n, uint64_t key_inv, uint64_t key_mask, uint32_t *counts, uint64_t num_rows,
-           uint32_t *status, uint32_t *host_mirror, void *stream) {
+           uint64_t *observed, uint32_t *status, uint32_t *host_mirror, void *stream) {
   if (n == 0) return 0;
   UGK_REQUIRE(keys && counts && status, "ugk_record: null pointer");
   UGK_REQUIRE(key_inv == 0 || (key_inv & 1ull), "ugk_record: the inverse key multiplier must be odd");
@@ -185,7 +212,7 @@ int record(const K *keys, size_t n, uint64_t key_inv, uint64_t key_mask, uint32_
   map.fb_mask = key_mask;
   const unsigned grid = clamp_grid((n + kRecTile - 1) / kRecTile, 0);
   hipLaunchKernelGGL(record_kernel<K>, dim3(grid), dim3(kBlock), 0, as_stream(stream), keys, n, map, counts, num_rows,
-                     status, host_mirror);
+                     reinterpret_cast<unsigned long long *>(observed), status, host_mirror);
   UGK_HIP(hipGetLastError());
   return 0;
 }
@@ -198,17 +225,22 @@ using namespace ugk;
 extern "C" {
 
 int ugk_record_u32(const uint32_t *keys_dev, size_t n, uint64_t key_inv, uint64_t key_mask, uint32_t *counts_dev,
-                   uint64_t num_rows, uint32_t *status_dev, uint32_t *host_mirror, void *stream) {
-  return record<uint32_t>(keys_dev, n, key_inv, key_mask, counts_dev, num_rows, status_dev, host_mirror, stream);
+                   uint64_t num_rows, uint64_t *observed_dev, uint32_t *status_dev, uint32_t *host_mirror,
+                   void *stream) {
+  return record<uint32_t>(keys_dev, n, key_inv, key_mask, counts_dev, num_rows, observed_dev, status_dev, host_mirror,
+                          stream);
 }
 
 int ugk_record_i64(const int64_t *keys_dev, size_t n, uint64_t key_inv, uint64_t key_mask, uint32_t *counts_dev,
-                   uint64_t num_rows, uint32_t *status_dev, uint32_t *host_mirror, void *stream) {
-  return record<int64_t>(keys_dev, n, key_inv, key_mask, counts_dev, num_rows, status_dev, host_mirror, stream);
+                   uint64_t num_rows, uint64_t *observed_dev, uint32_t *status_dev, uint32_t *host_mirror,
+                   void *stream) {
+  return record<int64_t>(keys_dev, n, key_inv, key_mask, counts_dev, num_rows, observed_dev, status_dev, host_mirror,
+                         stream);
 }
 
-int ugk_record_drain(uint32_t *counts_dev, uint64_t first_row, uint64_t num_rows, uint64_t *entries_dev,
-                     uint32_t capacity, uint32_t *n_entries_dev, uint32_t *host_out, void *stream) {
+int ugk_record_drain(uint32_t *counts_dev, uint64_t first_row, uint64_t num_rows, uint64_t *observed_dev,
+                     uint64_t *entries_dev, uint32_t capacity, uint32_t *n_entries_dev, uint32_t *host_out,
+                     void *stream) {
   UGK_REQUIRE(counts_dev && entries_dev && n_entries_dev && host_out, "ugk_record_drain: null pointer");
   UGK_REQUIRE(capacity > 0, "ugk_record_drain: empty entry list");
   UGK_REQUIRE(first_row + num_rows <= 0xffffffffull, "ugk_record_drain: rows must fit 32 bits");
@@ -216,7 +248,8 @@ int ugk_record_drain(uint32_t *counts_dev, uint64_t first_row, uint64_t num_rows
     // few, long wavefronts: one reservation each (8 workgroups per CU)
     const unsigned grid = clamp_grid((num_rows / 4 + 2 + kBlock - 1) / kBlock, (unsigned)cu_count() * 8u);
     hipLaunchKernelGGL(drain_kernel, dim3(grid), dim3(kBlock), 0, as_stream(stream), counts_dev + first_row, num_rows,
-                       first_row, reinterpret_cast<unsigned long long *>(entries_dev), capacity, n_entries_dev);
+                       first_row, reinterpret_cast<unsigned long long *>(observed_dev),
+                       reinterpret_cast<unsigned long long *>(entries_dev), capacity, n_entries_dev);
     UGK_HIP(hipGetLastError());
   }
   hipLaunchKernelGGL(drain_finish_kernel, dim3(1), dim3(1), 0, as_stream(stream), n_entries_dev, capacity, host_out);

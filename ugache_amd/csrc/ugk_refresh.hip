@@ -11,6 +11,8 @@
 //               the count settle T exactly);
 //            2. split: bit r of `gt` = count[r] > T, bit r of `eq` = count[r] == T (and the counters are reset if the
 //               caller wants the next interval to start from zero);
+//          When the caller keeps a bitmap of the observed rows (counter above zero) and fewer rows were observed than
+//          are wanted, T is 0 without looking: gt = observed, eq = ~observed, and steps 1 and 2 are bitmap launches.
 //            3. the needed rows among `eq` are its topmost set bits (T > 0: larger row first) or its lowest ones
 //               (T == 0: never-observed rows in ascending order): the position of the last needed bit is found with the
 //               chunk offsets of the ordered compaction below; result = gt | (eq restricted to that side of it).
@@ -42,7 +44,8 @@ struct RankWs {
   uint32_t count_t;              // T (digits picked so far)
   uint32_t settled;              // the saturating first pass found T
   uint32_t last_row;             // the last needed row among those with count T
-  uint32_t pad;
+  uint32_t from_bitmap;          // fewer rows were observed than are wanted: T = 0, no pass over the counters
+
   uint32_t hist[kHistBins];
   BmWs bm;                       // chunk offsets of `eq`
 };
@@ -55,7 +58,7 @@ __device__ __forceinline__ unsigned long long rank_of(uint32_t cnt, uint32_t row
 // picked so far; skipped when the first pass settled T.
 __global__ __launch_bounds__(kBlock) void rank_hist_kernel(const uint32_t *__restrict__ counts, uint64_t n,
                                                            RankWs *ws, int mode, int shift, int bits) {
-  if (mode == 1 && ws->settled) return;
+  if (ws->from_bitmap || (mode == 1 && ws->settled)) return;
   __shared__ uint32_t lh[kHistBins];
   const int tid = threadIdx.x;
   for (int b = tid; b < kHistBins; b += kBlock) lh[b] = 0;
@@ -103,7 +106,7 @@ __global__ __launch_bounds__(kBlock) void rank_pick_kernel(RankWs *ws, int mode,
   constexpr int kPer = kHistBins / kBlock;  // 8 bins per thread
   __shared__ unsigned long long suffix[kBlock + 1];
   const int tid = threadIdx.x;
-  if (mode == 1 && ws->settled) return;  // uniform: nothing was counted either
+  if (ws->from_bitmap || (mode == 1 && ws->settled)) return;  // uniform: nothing was counted either
   uint32_t h[kPer];
   unsigned long long mine = 0;
 #pragma unroll
@@ -155,6 +158,7 @@ __global__ void rank_init_kernel(RankWs *ws, unsigned long long remaining) {
     ws->count_t = 0;
     ws->settled = 0;
     ws->last_row = 0;
+    ws->from_bitmap = 0;
   }
   for (int b = tid; b < kHistBins; b += blockDim.x) ws->hist[b] = 0;
 }
@@ -165,6 +169,7 @@ constexpr int kMarkWords = 8;  // words (loads in flight) per wavefront and roun
 __global__ __launch_bounds__(kBlock) void rank_split_kernel(uint32_t *counts, uint64_t n, const RankWs *ws,
                                                             unsigned long long *gt, unsigned long long *eq,
                                                             int reset_counts) {
+  if (ws->from_bitmap) return;
   const uint32_t t = ws->count_t;
   const int lane = (int)lane_id();
   const uint64_t n_words = (n + 63) / 64;
@@ -188,6 +193,38 @@ __global__ __launch_bounds__(kBlock) void rank_split_kernel(uint32_t *counts, ui
       }
       if (reset_counts && row < n && c[k] != 0) counts[row] = 0;
     }
+  }
+}
+
+// after the observed rows were counted (ws->bm.total): fewer than wanted means every observed row is in and the rest
+// comes from the never-observed ones, lowest row first
+__global__ void rank_decide_kernel(RankWs *ws) {
+  if (ws->bm.total < ws->remaining) {
+    ws->from_bitmap = 1;
+    ws->settled = 1;
+    ws->count_t = 0;
+    ws->remaining -= ws->bm.total;
+  }
+}
+
+// the split of that case: gt = observed, eq = ~observed; counters of observed rows reset on request
+__global__ __launch_bounds__(kBlock) void rank_split_bitmap_kernel(uint32_t *counts, uint64_t n, const RankWs *ws,
+                                                                   const unsigned long long *observed,
+                                                                   unsigned long long *gt, unsigned long long *eq,
+                                                                   int reset_counts) {
+  if (!ws->from_bitmap) return;
+  const uint64_t n_words = (n + 63) / 64;
+  for (uint64_t w = (uint64_t)blockIdx.x * kBlock + threadIdx.x; w < n_words; w += (uint64_t)gridDim.x * kBlock) {
+    unsigned long long m = observed[w];
+    unsigned long long rest = ~m;
+    if (n - w * 64 < 64) rest &= (1ull << (n - w * 64)) - 1ull;
+    gt[w] = m;
+    eq[w] = rest;
+    if (reset_counts)
+      while (m) {
+        counts[w * 64 + __builtin_ctzll(m)] = 0;
+        m &= m - 1;
+      }
   }
 }
 
@@ -239,7 +276,8 @@ __global__ __launch_bounds__(kBlock) void rank_locate_kernel(RankWs *ws, const u
 
 // in_new = gt | (eq on the needed side of last_row); gt is in_new itself
 __global__ __launch_bounds__(kBlock) void rank_combine_kernel(const RankWs *ws, unsigned long long *in_new,
-                                                              const unsigned long long *eq, uint64_t n_words) {
+                                                              const unsigned long long *eq, uint64_t n_words,
+                                                              unsigned long long *observed_to_clear) {
   const uint64_t wl = ws->last_row >> 6;
   const unsigned bl = ws->last_row & 63u;
   const bool upward = ws->count_t != 0;  // rows at and above last_row, or at and below it
@@ -248,18 +286,21 @@ __global__ __launch_bounds__(kBlock) void rank_combine_kernel(const RankWs *ws, 
     if (upward) mask = w > wl ? ~0ull : (w == wl ? ~0ull << bl : 0ull);
     else mask = w < wl ? ~0ull : (w == wl ? (bl == 63 ? ~0ull : (1ull << (bl + 1)) - 1ull) : 0ull);
     in_new[w] |= eq[w] & mask;
+    if (observed_to_clear) observed_to_clear[w] = 0;  // the counters were reset: no row is observed any more
   }
 }
 
 // every row, or none: bitmap of n set (or clear) bits, counters reset on request
 __global__ __launch_bounds__(kBlock) void rank_fill_kernel(uint32_t *counts, uint64_t n, unsigned long long *bitmap,
-                                                           int all, int reset_counts, RankWs *ws) {
+                                                           int all, int reset_counts, RankWs *ws,
+                                                           unsigned long long *observed) {
   const uint64_t n_words = (n + 63) / 64;
   const uint64_t stride = (uint64_t)gridDim.x * kBlock;
   for (uint64_t w = (uint64_t)blockIdx.x * kBlock + threadIdx.x; w < n_words; w += stride) {
     unsigned long long m = all ? ~0ull : 0ull;
     if (all && n - w * 64 < 64) m = (1ull << (n - w * 64)) - 1ull;
     bitmap[w] = m;
+    if (reset_counts && observed) observed[w] = 0;
   }
   if (reset_counts)
     for (uint64_t r = (uint64_t)blockIdx.x * kBlock + threadIdx.x; r < n; r += stride) counts[r] = 0;
@@ -390,7 +431,7 @@ extern "C" {
 size_t ugk_rank_workspace_bytes(void) { return sizeof(RankWs); }
 
 int ugk_rank_place(uint32_t *counts_dev, uint64_t num_rows, uint64_t k, void *ws_dev, uint64_t *in_new_dev,
-                   uint64_t *scratch_bitmap_dev, int reset_counts, void *stream) {
+                   uint64_t *scratch_bitmap_dev, uint64_t *observed_dev, int reset_counts, void *stream) {
   UGK_REQUIRE(counts_dev && ws_dev && in_new_dev && scratch_bitmap_dev, "ugk_rank_place: null pointer");
   UGK_REQUIRE(num_rows > 0 && num_rows < 0xffffffffull, "ugk_rank_place: %llu rows do not fit 32 bits",
               (unsigned long long)num_rows);
@@ -399,15 +440,27 @@ int ugk_rank_place(uint32_t *counts_dev, uint64_t num_rows, uint64_t k, void *ws
   hipStream_t st = as_stream(stream);
   unsigned long long *in_new = reinterpret_cast<unsigned long long *>(in_new_dev);
   unsigned long long *eq = reinterpret_cast<unsigned long long *>(scratch_bitmap_dev);
+  unsigned long long *observed = reinterpret_cast<unsigned long long *>(observed_dev);
   const uint64_t n_words = (num_rows + 63) / 64;
   if (k == 0 || k >= num_rows) {  // no row, or every row
     const unsigned grid = clamp_grid(((reset_counts ? num_rows : n_words) + kBlock - 1) / kBlock, 0);
     hipLaunchKernelGGL(rank_fill_kernel, dim3(grid), dim3(kBlock), 0, st, counts_dev, num_rows, in_new,
-                       k == 0 ? 0 : 1, reset_counts, ws);
+                       k == 0 ? 0 : 1, reset_counts, ws, observed);
     UGK_HIP(hipGetLastError());
     return 0;
   }
   hipLaunchKernelGGL(rank_init_kernel, dim3(1), dim3(kBlock), 0, st, ws, (unsigned long long)k);
+  const uint64_t per_chunk = bm_words_per_chunk(n_words);
+  const unsigned bm_grid = clamp_grid((kBmChunks + (kBlock / kWave) - 1) / (kBlock / kWave), (unsigned)cu_count() * 8u);
+  const unsigned word_grid = clamp_grid((n_words + kBlock - 1) / kBlock, 0);
+  if (observed) {
+    hipLaunchKernelGGL(bitmap_count_kernel, dim3(bm_grid), dim3(kBlock), 0, st, observed,
+                       (const unsigned long long *)nullptr, 0, num_rows, per_chunk, &ws->bm);
+    hipLaunchKernelGGL(bitmap_scan_kernel, dim3(1), dim3(kBlock), 0, st, &ws->bm, (uint32_t *)nullptr);
+    hipLaunchKernelGGL(rank_decide_kernel, dim3(1), dim3(1), 0, st, ws);
+    hipLaunchKernelGGL(rank_split_bitmap_kernel, dim3(word_grid), dim3(kBlock), 0, st, counts_dev, num_rows, ws,
+                       observed, in_new, eq, reset_counts);
+  }
   // a few long workgroups: every workgroup ends with a flush of its histogram into the shared one
   const unsigned hist_grid = clamp_grid((num_rows / 4 + kBlock - 1) / kBlock, (unsigned)cu_count() * 8u);
   hipLaunchKernelGGL(rank_hist_kernel, dim3(hist_grid), dim3(kBlock), 0, st, counts_dev, num_rows, ws, 0, 0, 11);
@@ -421,14 +474,12 @@ int ugk_rank_place(uint32_t *counts_dev, uint64_t num_rows, uint64_t k, void *ws
       clamp_grid((n_words + kMarkWords * (kBlock / kWave) - 1) / (kMarkWords * (kBlock / kWave)), 0);
   hipLaunchKernelGGL(rank_split_kernel, dim3(split_grid), dim3(kBlock), 0, st, counts_dev, num_rows, ws, in_new, eq,
                      reset_counts);
-  const uint64_t per_chunk = bm_words_per_chunk(n_words);
-  const unsigned bm_grid = clamp_grid((kBmChunks + (kBlock / kWave) - 1) / (kBlock / kWave), (unsigned)cu_count() * 8u);
   hipLaunchKernelGGL(bitmap_count_kernel, dim3(bm_grid), dim3(kBlock), 0, st, eq, (const unsigned long long *)nullptr, 0,
                      num_rows, per_chunk, &ws->bm);
   hipLaunchKernelGGL(bitmap_scan_kernel, dim3(1), dim3(kBlock), 0, st, &ws->bm, (uint32_t *)nullptr);
   hipLaunchKernelGGL(rank_locate_kernel, dim3(1), dim3(kBlock), 0, st, ws, eq, num_rows, per_chunk);
-  const unsigned comb_grid = clamp_grid((n_words + kBlock - 1) / kBlock, 0);
-  hipLaunchKernelGGL(rank_combine_kernel, dim3(comb_grid), dim3(kBlock), 0, st, ws, in_new, eq, n_words);
+  hipLaunchKernelGGL(rank_combine_kernel, dim3(word_grid), dim3(kBlock), 0, st, ws, in_new, eq, n_words,
+                     reset_counts ? observed : (unsigned long long *)nullptr);
   UGK_HIP(hipGetLastError());
   return 0;
 }
