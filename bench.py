@@ -95,7 +95,7 @@ def parse_args():
                     help="sparse-id workloads, with --gpu-record: after the timed steps, time the lookups again while "
                          "a second thread refreshes the cache back to back from the device-side hotness counters")
     ap.add_argument("--device-refresh", action="store_true",
-                    help="sparse-id workloads: COLL_GPU_RECORD=1 COLL_GPU_REFRESH=1 COLL_GPU_REFRESH_KEEP=1; after the "
+                    help="mixed workloads: COLL_GPU_RECORD=1 COLL_GPU_REFRESH=1 COLL_GPU_REFRESH_KEEP=1; after the "
                          "timed steps, time steps that each end with a refresh computed on the device from the "
                          "accumulated hotness, with 1 %% of the cache replaced per step")
     ap.add_argument("--calibrate", action="store_true",
@@ -445,7 +445,7 @@ def run_mixed(args):
 
     refresh = None
     each_step = None
-    if sparse and args.device_refresh:
+    if args.device_refresh:
         # Every step ends with a refresh computed on the device from the hotness accumulated so far.  Hotness drifts by
         # 1 % of the cache per step: a slice of so-far never-looked-up rows is looked up once between the steps
         # (untimed), which ranks them above the never-observed rows the cache is filled up with, so each refresh evicts
