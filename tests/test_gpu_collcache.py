@@ -868,3 +868,55 @@ def test_sparse_ids_hash_table_with_refresh_each_step(gpu_record, monkeypatch):
         rebuilds = info["table_rebuilds"]
         cached = new_cached
     assert rebuilds >= 1
+
+
+def test_serving_stack_from_a_ps_config_file(tmp_path):
+    """The TF2 binding's serving stack for PyTorch (collcache.torch.serving): a ps_config JSON with the keys
+    inference_utils.cpp:55-160 reads, a model directory of `key` + `emb_vector` files, Config -> record_hotness ->
+    Init -> LookupLayer.  Every lookup reproduces table[keys]; the refresh armed by the configuration runs in the
+    background at step coll_cache_refresh_iter and re-places by the recorded 5 % prefixes."""
+    import json
+    import collcache.torch.serving as hps
+    rng = np.random.default_rng(77)
+    n_item, dim = 20_000, 16
+    rows = rng.standard_normal((n_item, dim)).astype(np.float32)
+    model = tmp_path / "dlrm_sparse.model"
+    model.mkdir()
+    np.arange(n_item, dtype=np.int64).tofile(model / "key")
+    rows.tofile(model / "emb_vector")
+    cfg = {"iteration_per_epoch": 50, "epoch": 1, "coll_cache_enable_refresh": True, "coll_cache_refresh_iter": 4,
+           "models": [{"model": "dlrm", "sparse_files": [str(model)], "gpucacheper": 0.3, "max_batch_size": 4096,
+                       "deployed_device_list": [0], "maxnum_catfeature_query_per_table_per_sample": [26],
+                       "embedding_vecsize_per_table": [dim], "max_vocabulary_size": [n_item]}]}
+    path = tmp_path / "ps_config.json"
+    path.write_text(json.dumps(cfg))
+    try:
+        assert hps.Config(ps_config_file=str(path)) == "OK"
+        perm = rng.permutation(n_item)
+        warm = [perm[zipf_ranks(rng, 30_000, n_item, 1.1)] for _ in range(3)]
+        for b in warm:
+            hps.record_hotness(torch.from_numpy(b).cuda())
+        assert hps.Init(ps_config_file=str(path), global_batch_size=1024) == "OK"
+        want_cached, nid = expected_cached_set(np.concatenate(warm).astype(np.uint32), n_item, 0.3)
+        layer = hps.LookupLayer(model_name="dlrm", table_id=0, emb_vec_size=dim, emb_vec_dtype=torch.float32)
+        perm2 = rng.permutation(n_item)
+        recorded = []
+        for step in range(8):
+            keys = perm2[zipf_ranks(rng, 1024 * 26, n_item, 1.1)].reshape(1024, 26)
+            emb = layer(torch.from_numpy(keys).cuda())
+            assert tuple(emb.shape) == (1024, 26, dim) and emb.dtype == torch.float32
+            assert emb.cpu().numpy().tobytes() == rows[keys].tobytes()
+            assert _basics.last_group_offset(0)[1] == int((nid[keys.reshape(-1)] == 0).sum())
+            recorded.append(keys.reshape(-1)[: int(keys.size * hps.RECORD_FRACTION)])
+            if step == 4:  # the refresh started behind this step; let it finish (it waits for one more lookup)
+                empty = torch.zeros(0, dtype=torch.int64, device="cuda")
+                while _basics.C_LIB_CTYPES.coll_cache_forward_refresh_ongoing():
+                    co.coll_torch_lookup_key_t_val_ret(0, empty, False)
+                    time.sleep(0.001)
+                assert co.coll_torch_forward_join() == 1
+                _, nid = expected_cached_set(np.concatenate(recorded).astype(np.uint32), n_item, 0.3)
+        hps.SetStepProfileValue(profile_type=kLogL1FeatureBytes, value=123.0)
+        assert _basics.step_value(hps._last_step_key(), kLogL1FeatureBytes) == 123.0
+        hps.Report()
+    finally:
+        hps.Shutdown()

@@ -236,3 +236,63 @@ def test_bench_refuses_more_than_one_gpu():
                        stderr=subprocess.PIPE, text=True, timeout=120)
     assert p.returncode != 0 and p.stdout == ""
     assert "ONE GPU" in p.stderr and "--gpus 1" in p.stderr
+
+
+def _ps_config(tmp_path, edit=None):
+    import json
+    cfg = {"iteration_per_epoch": 100, "epoch": 2, "coll_cache_refresh_iter": 7,
+           "models": [{"model": "dlrm", "sparse_files": ["/models/dlrm_sparse.model"], "gpucacheper": 0.15,
+                       "deployed_device_list": [0], "maxnum_catfeature_query_per_table_per_sample": [26],
+                       "embedding_vecsize_per_table": [128], "max_vocabulary_size": [1000]}]}
+    if edit:
+        edit(cfg)
+    p = tmp_path / "ps_config.json"
+    p.write_text(json.dumps(cfg))
+    return str(p)
+
+
+def test_ps_config_is_read_like_the_serving_stack_reads_it(tmp_path):
+    """keys, defaults and insisted-on keys of parameter_server_config (inference_utils.cpp:55-160)"""
+    from collcache.torch.serving import PsConfig
+    c = PsConfig(_ps_config(tmp_path))
+    assert (c.iteration_per_epoch, c.epoch, c.coll_cache_refresh_iter) == (100, 2, 7)
+    assert c.coll_cache_enable_refresh is False and c.use_multi_worker is False  # soft defaults
+    assert c.coll_cache_policy == 13 and c.max_batch_size == 64 and c.i64_input_key is True
+    assert c.model_name == "dlrm" and c.sparse_files == ["/models/dlrm_sparse.model"]
+    assert abs(c.cache_size_percentage - 0.15) < 1e-12
+    assert c.embedding_vecsize_per_table == [128] and c.max_vocabulary_size == [1000]
+    assert c.maxnum_catfeature_query_per_table_per_sample == [26] and c.deployed_devices == [0]
+
+    def no_gpucacheper(cfg):
+        del cfg["models"][0]["gpucacheper"]
+        del cfg["coll_cache_refresh_iter"]
+        cfg["coll_cache_enable_refresh"] = True
+        cfg["models"][0]["i64_input_key"] = False
+    c = PsConfig(_ps_config(tmp_path, no_gpucacheper))
+    assert abs(c.cache_size_percentage - 0.2) < 1e-12 and c.coll_cache_refresh_iter is None
+    assert c.coll_cache_enable_refresh is True and c.i64_input_key is False
+
+
+@pytest.mark.parametrize("broken", ["iteration_per_epoch", "epoch", "models", "sparse_files", "deployed_device_list",
+                                    "embedding_vecsize_per_table", "two_models", "two_devices"])
+def test_ps_config_without_a_required_key_aborts_with_a_message(tmp_path, broken):
+    def edit(cfg):
+        if broken in ("iteration_per_epoch", "epoch", "models"):
+            del cfg[broken]
+        elif broken == "two_models":
+            cfg["models"].append(dict(cfg["models"][0]))
+        elif broken == "two_devices":
+            cfg["models"][0]["deployed_device_list"] = [0, 1]
+        else:
+            del cfg["models"][0][broken]
+    path = _ps_config(tmp_path, edit)
+    code = textwrap.dedent("""
+        import sys
+        sys.path.insert(0, %r)
+        from collcache.torch.serving import PsConfig
+        PsConfig(%r)
+        print("not reached")
+    """) % (os.path.join(ROOT, "ugache_amd"), path)
+    r = subprocess.run([sys.executable, "-c", code], capture_output=True, text=True)
+    assert r.returncode == -6 and "not reached" not in r.stdout  # abort(), like COLL_CHECK
+    assert "ps_config:" in r.stderr
