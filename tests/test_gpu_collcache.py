@@ -915,6 +915,33 @@ def test_serving_stack_from_a_ps_config_file(tmp_path):
                     time.sleep(0.001)
                 assert co.coll_torch_forward_join() == 1
                 _, nid = expected_cached_set(np.concatenate(recorded).astype(np.uint32), n_item, 0.3)
+        # embedding_lookup_sparse over the cache: ragged rows of ids with weights, the three combiners, against float64
+        sparse = hps.SparseLookupLayer(model_name="dlrm", table_id=0, emb_vec_size=dim, emb_vec_dtype=torch.float32)
+        n_rows = 500
+        lens = rng.integers(1, 9, size=n_rows)
+        seg = np.repeat(np.arange(n_rows), lens)
+        col = np.concatenate([np.arange(k) for k in lens])
+        ids = perm2[zipf_ranks(rng, len(seg), n_item, 1.1)]
+        w = rng.uniform(0.1, 2.0, size=len(seg)).astype(np.float32)
+        ind = torch.from_numpy(np.stack([seg, col])).cuda()
+        sp_ids = torch.sparse_coo_tensor(ind, torch.from_numpy(ids).cuda(), (n_rows, 8))
+        sp_w = torch.sparse_coo_tensor(ind, torch.from_numpy(w).cuda(), (n_rows, 8))
+        e64, w64 = rows[ids].astype(np.float64), w.astype(np.float64)
+        for combiner in ("sum", "mean", "sqrtn", None):
+            for weights in (sp_w, None):
+                ww = w64 if weights is not None else np.ones_like(w64)
+                want = np.zeros((n_rows, dim))
+                np.add.at(want, seg, e64 * ww[:, None])
+                if combiner in ("mean", None):
+                    want /= np.bincount(seg, weights=ww, minlength=n_rows)[:, None]
+                elif combiner == "sqrtn":
+                    want /= np.sqrt(np.bincount(seg, weights=ww * ww, minlength=n_rows))[:, None]
+                got = sparse(sp_ids, weights, combiner=combiner).cpu().numpy()
+                assert got.shape == (n_rows, dim)
+                # fp32 sums of at most 8 terms against float64: tolerance 1e-5 relative to the row's magnitude
+                assert np.allclose(got, want, rtol=1e-5, atol=1e-5 * np.abs(want).max())
+        with pytest.raises(ValueError):
+            sparse(sp_ids, None, combiner="max")
         hps.SetStepProfileValue(profile_type=kLogL1FeatureBytes, value=123.0)
         assert _basics.step_value(hps._last_step_key(), kLogL1FeatureBytes) == 123.0
         hps.Report()

@@ -5,7 +5,8 @@ background.
 Mirrors, call for call,
   collcache_tf2.Config / Init / Report / wait_one_child / SetStepProfileValue
       (python_tf2/collcache_tf2/collcache_tf2/core/initialize.py:33-39, 79-127, 129-290, 292-295)
-  collcache_tf2.LookupLayer (core/lookup_layer.py:22-110)
+  collcache_tf2.LookupLayer (core/lookup_layer.py:22-110), collcache_tf2.SparseLookupLayer
+      (core/sparse_lookup_layer.py:27-265)
 over LookupManager::{config, record_hotness, init, forward} (python_tf2/collcache_tf2/collcache_tf2_cc/
 collcache_tf2_cc_infra/src/lookup_manager.cc:49-212) and the ps_config parser
 (collcache_tf2_cc_infra/src/inference_utils.cpp:55-160).  One process, one replica, one GPU.
@@ -175,6 +176,62 @@ class LookupLayer(torch.nn.Module):
             _abort("%d keys exceed max_batch_size x maxnum_catfeature_query_per_table_per_sample" % flat.numel())
         emb = _adapter.coll_torch_forward(0, flat, False)
         return emb.reshape(tuple(inputs.shape) + (self.emb_vec_size,))
+
+
+class SparseLookupLayer(torch.nn.Module):
+    """collcache_tf2.SparseLookupLayer (core/sparse_lookup_layer.py:27-265), i.e. embedding_lookup_sparse over the
+    cache: `sp_ids` is an N x M sparse COO tensor of int64 ids in row-major order with at least one id per row,
+    `sp_weights` a sparse tensor of the same indices or None; the distinct ids are looked up once
+    (unique -> lookup -> gather, sparse_lookup_layer.py:196-209), multiplied by their weights and combined per row:
+    "sum", "mean" (weighted sum / sum of weights) or "sqrtn" (weighted sum / sqrt of the sum of squared weights);
+    `max_norm` clips every embedding's l2 norm before combining.  Returns [N, emb_vec_size]."""
+
+    def __init__(self, model_name, table_id, emb_vec_size, emb_vec_dtype=torch.float32, **kwargs):
+        super().__init__()
+        self.lookup = LookupLayer(model_name, table_id, emb_vec_size, emb_vec_dtype)
+        self.emb_vec_size = emb_vec_size
+
+    def forward(self, sp_ids, sp_weights=None, name=None, combiner=None, max_norm=None):
+        if combiner is None:
+            combiner = "mean"
+        if combiner not in ("mean", "sqrtn", "sum"):
+            raise ValueError("combiner must be one of 'mean', 'sqrtn' or 'sum', got %s" % combiner)
+        if not (isinstance(sp_ids, torch.Tensor) and sp_ids.is_sparse):
+            raise TypeError("sp_ids must be a sparse COO tensor, got %s" % type(sp_ids))
+        if sp_weights is not None and not (isinstance(sp_weights, torch.Tensor) and sp_weights.is_sparse):
+            raise TypeError("sp_weights must be either None or a sparse COO tensor, got %s" % type(sp_weights))
+        # entries as given (row-major order is the caller's contract); coalesce() would merge duplicate positions
+        segment_ids = sp_ids._indices()[0]
+        ids, idx = torch.unique(sp_ids._values(), return_inverse=True)
+        embeddings = self.lookup(ids).index_select(0, idx)
+        original_dtype = embeddings.dtype
+        if embeddings.dtype in (torch.float16, torch.bfloat16):
+            embeddings = embeddings.float()  # low-precision rows are combined in fp32
+        if max_norm is not None:
+            norms = embeddings.norm(dim=1, keepdim=True)
+            embeddings = embeddings * torch.clamp(max_norm / norms.clamp_min(1e-30), max=1.0)
+        num_rows = int(sp_ids.shape[0])
+        if sp_weights is None:
+            weights = torch.ones(embeddings.shape[0], dtype=embeddings.dtype, device=embeddings.device)
+        else:
+            weights = sp_weights._values().to(embeddings.dtype)
+            embeddings = embeddings * weights.unsqueeze(1)
+
+        def segment_sum(x):
+            out = torch.zeros((num_rows,) + tuple(x.shape[1:]), dtype=x.dtype, device=x.device)
+            return out.index_add_(0, segment_ids, x)
+
+        combined = segment_sum(embeddings)
+        if combiner == "mean":
+            denom = segment_sum(weights).unsqueeze(1)
+        elif combiner == "sqrtn":
+            denom = segment_sum(weights * weights).sqrt().unsqueeze(1)
+        else:
+            denom = None
+        if denom is not None:  # div_no_nan: a zero denominator gives zero
+            combined = torch.where(denom != 0, combined / torch.where(denom != 0, denom, torch.ones_like(denom)),
+                                   torch.zeros_like(combined))
+        return combined.to(original_dtype)
 
 
 def _last_step_key():
