@@ -947,3 +947,34 @@ def test_serving_stack_from_a_ps_config_file(tmp_path):
         hps.Report()
     finally:
         hps.Shutdown()
+
+
+@pytest.mark.parametrize("impl", ["", "SMMaskPhase"])
+def test_counting_every_third_lookup_on_the_device(impl, monkeypatch):
+    """COLL_GPU_RECORD_EVERY=3: lookups 0, 3, 6, ... are counted, the others are not; the ranking drained from the
+    device equals the oracle's ranking of exactly those batches"""
+    monkeypatch.setenv("COLL_GPU_RECORD", "1")
+    monkeypatch.setenv("COLL_GPU_RECORD_EVERY", "3")
+    if impl:
+        monkeypatch.setenv("SAMGRAPH_COLL_CACHE_CONCURRENT_LINK_IMPL", impl)
+    rng = np.random.default_rng(3)
+    n_item, dim, pct = 10_000, 32, 0.2
+    co.config(make_config(n_item, pct))
+    co.coll_cache_record_init(0)
+    co.coll_torch_record(0, torch.from_numpy(rng.integers(0, n_item, size=50_000)).to(torch.int32))
+    emb = co.coll_torch_create_emb_shm(0, n_item, dim, torch.float32)
+    table = fill_table(emb, rng)
+    co.coll_torch_init_t(0, 0, emb, pct)
+    counted = []
+    for i in range(8):
+        keys = rng.integers(0, n_item, size=5_000 + i)
+        out = co.coll_torch_lookup_key_t_val_ret(0, torch.from_numpy(keys).to(torch.int32).cuda(), False)
+        assert out.cpu().numpy().tobytes() == ORC.gather(table, keys.astype(np.int64)).tobytes()
+        if i % 3 == 0:
+            counted.append(keys.astype(np.uint32))
+    want_k, want_c = ORC.freq_rank(np.concatenate(counted))
+    got_k = np.zeros(n_item, np.uint32)
+    got_c = np.zeros(n_item, np.uint32)
+    m = _basics.C_LIB_CTYPES.coll_cache_rank_hotness(0, got_k.ctypes.data, got_c.ctypes.data, n_item)
+    assert m == len(want_k)
+    assert np.array_equal(got_k[:m], want_k) and np.array_equal(got_c[:m], want_c)
