@@ -586,6 +586,7 @@ void ExtractSession::ExtractFeatImpl(const KeyT *nodes, size_t num_nodes, void *
   EnsureIdx(num_nodes);
   ugk_idx_t *idx = _idx_handle->ptr<ugk_idx_t>();
   uint32_t *cur = _counts[_cur], *next = _counts[_cur ^ 1];
+  bool joined_on_host = false;
   UGK_CALL(ugk_event_record(_ev_t[0], stream));
   UGK_CALL(Classify(table, nodes, num_nodes, host_rows, dst_map, idx, cur, next, _status, _host_mirror, stream));
   UGK_CALL(ugk_event_record(_ev_classified, stream));
@@ -614,8 +615,13 @@ void ExtractSession::ExtractFeatImpl(const KeyT *nodes, size_t num_nodes, void *
     UGK_CALL(ugk_gather_group(cache, cache_rows, idx, cur, UGK_LOC_LOCAL, num_nodes, output, num_input, rb, 0,
                               _status, _host_mirror, _local_ext_stream));
     UGK_CALL(ugk_event_record(_ev_local_done, _local_ext_stream));
-    if (!_host_on_main) UGK_CALL(ugk_stream_wait_event(stream, _ev_cpu_done));
-    UGK_CALL(ugk_stream_wait_event(stream, _ev_local_done));
+    // with nothing left to enqueue behind the gathers the host waits for their two events itself (below); only the
+    // re-expansion of a deduplicated batch needs both groups complete inside the caller's stream
+    joined_on_host = dst_map == nullptr;
+    if (!joined_on_host) {
+      if (!_host_on_main) UGK_CALL(ugk_stream_wait_event(stream, _ev_cpu_done));
+      UGK_CALL(ugk_stream_wait_event(stream, _ev_local_done));
+    }
   } else {
     // sequential: host group, then local group (cache_context.cu:1719-1792)
     UGK_CALL(ugk_gather_group(host, host_rows, idx, cur, UGK_LOC_HOST, num_nodes, output, num_input, rb, 0,
@@ -626,9 +632,15 @@ void ExtractSession::ExtractFeatImpl(const KeyT *nodes, size_t num_nodes, void *
     UGK_CALL(ugk_event_record(_ev_local_done, stream));
   }
   if (dst_map) UGK_CALL(ugk_replicate_rows(output, rb, inverse, dst_map, num_input, stream));
-  // the single blocking wait of the call; the gathers have written their group sizes (and the kernels any error
-  // flag) into the pinned mirror, so no device-to-host copy is needed
-  UGK_CALL(ugk_stream_sync(stream));
+  // the blocking wait of the call; the gathers have written their group sizes (and the kernels any error flag) into
+  // the pinned mirror, so no device-to-host copy is needed.  Waiting for the events of the two gather streams on the
+  // host keeps two cross-stream dependencies out of the caller's stream, which cost more than the wait itself.
+  if (joined_on_host) {
+    UGK_CALL(ugk_event_sync(_ev_cpu_done));
+    UGK_CALL(ugk_event_sync(_ev_local_done));
+  } else {
+    UGK_CALL(ugk_stream_sync(stream));
+  }
   JoinRecordOnHost();
   const uint32_t n_local = _host_mirror[kMirGroupSizes + UGK_LOC_LOCAL],
                  n_miss = _host_mirror[kMirGroupSizes + UGK_LOC_HOST];
