@@ -663,7 +663,11 @@ def _random_case(seed):
                 zipf=float(r.choice([0.6, 1.05, 1.4])), half=bool(r.integers(0, 3) == 0))
 
 
-@pytest.mark.parametrize("case", [_random_case(i) for i in range(96)], ids=lambda c: "seed%d" % c["seed"])
+# UGACHE_TEST_SEEDS widens the two seeded sweeps of this file for an occasional longer run
+_SEEDS = int(os.environ.get("UGACHE_TEST_SEEDS", "0"))
+
+
+@pytest.mark.parametrize("case", [_random_case(i) for i in range(max(96, _SEEDS))], ids=lambda c: "seed%d" % c["seed"])
 def test_random_configurations_are_exact(case, monkeypatch):
     """seeded random sweep over table size, row width, cache share, table kind, extraction mode, key width and the
     optional stages: blocking and stream-ordered lookups of ragged batch sizes (0, 1, odd, larger than the table)
@@ -710,6 +714,46 @@ def test_random_configurations_are_exact(case, monkeypatch):
         assert out.cpu().numpy().tobytes() == ORC.gather(table, keys.astype(np.int64)).tobytes()
 
 
+@pytest.mark.parametrize("device", [False, True])
+def test_refresh_of_a_table_too_small_for_spare_slots(device, monkeypatch):
+    """400 rows, 10 % cached: the capacity (size_t)(400 * 0.101) = 40 equals the number of cached rows, so a refresh has
+    exactly as many free slots (the evicted ones) as rows to insert.  The reference's strict check
+    (cache_hashtable.cuh:648) would abort there; here the refresh goes through, on the host and on the device."""
+    if device:
+        monkeypatch.setenv("COLL_GPU_RECORD", "1")
+        monkeypatch.setenv("COLL_GPU_REFRESH", "1")
+    rng = np.random.default_rng(258)
+    n_item, dim, pct = 400, 100, 0.1
+    co.config(make_config(n_item, pct))
+    co.coll_cache_record_init(0)
+    perm = rng.permutation(n_item)
+    s0 = perm[zipf_ranks(rng, 2010, n_item, 1.4)]
+    co.coll_torch_record(0, torch.from_numpy(s0))
+    emb = co.coll_torch_create_emb_shm(0, n_item, dim, torch.float32)
+    table = fill_table(emb, rng)
+    co.coll_torch_init_t(0, 0, emb, pct)
+    info = _basics.info(0)
+    assert info["capacity_rows"] == 40 and info["cached_rows"] == 40 and info["free_slots"] == 0
+    old, _ = expected_cached_set(s0.astype(np.uint32), n_item, pct)
+    s1 = perm[::-1][zipf_ranks(rng, 1200, n_item, 1.1)].copy()
+    if device:
+        co.coll_torch_lookup_key_t_val_ret(0, torch.from_numpy(s1).cuda(), False)
+    else:
+        co.coll_torch_record(0, torch.from_numpy(s1))
+    co.coll_torch_refresh(0, True)
+    want, nid = expected_cached_set(s1.astype(np.uint32), n_item, pct)
+    assert len(np.setdiff1d(old, want)) > 10
+    got = np.zeros(len(want), np.uint32)
+    assert _basics.C_LIB_CTYPES.coll_cache_get_cached_keys(0, got.ctypes.data, len(got)) == len(want)
+    assert np.array_equal(got, want)
+    info = _basics.info(0)
+    assert info["cached_rows"] == 40 and info["free_slots"] == 0
+    keys = rng.integers(0, n_item, size=5_000)
+    out = co.coll_torch_lookup_key_t_val_ret(0, torch.from_numpy(keys).cuda(), False)
+    assert out.cpu().numpy().tobytes() == ORC.gather(table, keys).tobytes()
+    assert _basics.last_group_offset(0)[1] == int((nid[keys] == 0).sum())
+
+
 def _random_refresh_case(seed):
     r = np.random.default_rng(5000 + seed)
     return dict(seed=seed, n_item=int(r.integers(130, 90_000)), dim=int(r.choice([4, 16, 32, 64, 100])),
@@ -718,7 +762,8 @@ def _random_refresh_case(seed):
                 rounds=int(r.integers(2, 5)), stream_ordered=bool(r.integers(0, 3) == 0))
 
 
-@pytest.mark.parametrize("case", [_random_refresh_case(i) for i in range(24)], ids=lambda c: "seed%d" % c["seed"])
+@pytest.mark.parametrize("case", [_random_refresh_case(i) for i in range(max(24, _SEEDS // 2))],
+                         ids=lambda c: "seed%d" % c["seed"])
 def test_random_sequences_of_refreshes_on_the_device(case, monkeypatch):
     """seeded random sweep over table size, cache share (from nearly nothing cached to nearly everything), table kind,
     sparse ids, accumulating or per-interval hotness: after every refresh computed on the device the cached rows are

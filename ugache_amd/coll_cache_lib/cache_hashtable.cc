@@ -245,7 +245,10 @@ void CacheEntryManager::ReturnOffset(TensorPtr new_offsets) {
 }
 
 TensorPtr CacheEntryManager::ReserveOffsetFront(IdType n) {
-  CHECK(_free_offsets->Shape()[0] > n) << "free cache slots exhausted: " << _free_offsets->Shape()[0] << " <= " << n;
+  // the reference insists on one slot more than it takes (cache_hashtable.cuh:648), which a table so small that the
+  // 0.1 % of spare capacity rounds to no slot at all (capacity == cached rows) can never offer; taking every free
+  // slot is fine
+  CHECK(_free_offsets->Shape()[0] >= n) << "free cache slots exhausted: " << _free_offsets->Shape()[0] << " < " << n;
   TensorPtr ret = Tensor::CopyBlob(_free_offsets->CPtr<IdType>(), kI32, {(size_t)n}, CPU_CLIB(), CPU_CLIB(), "");
   const size_t rest = _free_offsets->NumItem() - n;
   memmove(_free_offsets->Ptr<IdType>(), _free_offsets->Ptr<IdType>() + n, rest * sizeof(IdType));
