@@ -1023,3 +1023,59 @@ def test_counting_every_third_lookup_on_the_device(impl, monkeypatch):
     m = _basics.C_LIB_CTYPES.coll_cache_rank_hotness(0, got_k.ctypes.data, got_c.ctypes.data, n_item)
     assert m == len(want_k)
     assert np.array_equal(got_k[:m], want_k) and np.array_equal(got_c[:m], want_c)
+
+
+@pytest.mark.parametrize("table_kind", ["FLAT", "HASH"])
+def test_lookups_stay_exact_while_the_device_refreshes_under_them(table_kind, monkeypatch):
+    """a thread refreshes back to back on the device (background mode, hotness accumulating from the very lookups that
+    run beside it) while the caller looks keys up: every output is table[keys], and when the dust settles the cache
+    holds exactly its share of rows in exactly that many slots"""
+    monkeypatch.setenv("COLL_HASH_TABLE", table_kind)
+    monkeypatch.setenv("COLL_GPU_RECORD", "1")
+    monkeypatch.setenv("COLL_GPU_REFRESH", "1")
+    monkeypatch.setenv("COLL_GPU_REFRESH_KEEP", "1")
+    monkeypatch.setenv("COLL_REFRESH_SLEEP_US", "50")
+    monkeypatch.setenv("COLL_REFRESH_BATCH_ROWS", "256")
+    monkeypatch.setenv("COLL_HASH_REBUILD_FRAC", "0.05")
+    rng = np.random.default_rng(91)
+    n_item, dim, pct = 60_000, 32, 0.15
+    co.config(make_config(n_item, pct))
+    co.coll_cache_record_init(0)
+    perm = rng.permutation(n_item)
+    co.coll_torch_record(0, torch.from_numpy(perm[zipf_ranks(rng, 100_000, n_item, 1.05)]))
+    emb = co.coll_torch_create_emb_shm(0, n_item, dim, torch.float32)
+    table = fill_table(emb, rng)
+    co.coll_torch_init_t(0, 0, emb, pct)
+    cap = _basics.info(0)["capacity_rows"]
+    stop, done = [False], [0]
+
+    def refresher():
+        while not stop[0]:
+            co.coll_torch_refresh(0, False)
+            done[0] += 1
+
+    t = threading.Thread(target=refresher)
+    t.start()
+    try:
+        for step in range(150):
+            if step % 10 == 0:  # hotness keeps moving
+                swap = rng.choice(n_item, n_item // 20, replace=False)
+                perm[swap] = perm[rng.permutation(swap)]
+            keys = perm[zipf_ranks(rng, int(rng.integers(1, 30_000)), n_item, 1.05)]
+            out = co.coll_torch_lookup_key_t_val_ret(0, torch.from_numpy(keys).cuda(), False)
+            assert out.cpu().numpy().tobytes() == ORC.gather(table, keys).tobytes(), step
+    finally:
+        stop[0] = True
+        while t.is_alive():  # a refresh in flight waits for one more lookup to pass
+            co.coll_torch_lookup_key_t_val_ret(0, torch.zeros(0, dtype=torch.int64).cuda(), False)
+            t.join(timeout=0.005)
+    assert done[0] >= 3
+    info = _basics.info(0)
+    assert info["cached_rows"] == int(n_item * pct) and info["cached_rows"] + info["free_slots"] == cap
+    got = np.zeros(info["cached_rows"], np.uint32)
+    assert _basics.C_LIB_CTYPES.coll_cache_get_cached_keys(0, got.ctypes.data, len(got)) == len(got)
+    assert len(np.unique(got)) == len(got)
+    keys = rng.integers(0, n_item, size=40_000)
+    out = co.coll_torch_lookup_key_t_val_ret(0, torch.from_numpy(keys).cuda(), False)
+    assert out.cpu().numpy().tobytes() == ORC.gather(table, keys).tobytes()
+    assert _basics.last_group_offset(0)[1] == int(np.isin(keys, got).sum())
