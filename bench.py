@@ -203,8 +203,13 @@ def run_all_hit(args):
     C = _basics.C_LIB_CTYPES
     stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
 
+    # device addresses taken once: slicing a tensor and asking for its pointer costs several microseconds of Python per
+    # step, which is the caller's time, not the path's
+    key_ptrs = [keys_pool[i].data_ptr() for i in range(pool)]
+    out_ptr = out.data_ptr()
+
     def step(i):
-        C.coll_cache_lookup(0, keys_pool[i % pool].data_ptr(), n_keys, out.data_ptr(), stream)
+        C.coll_cache_lookup(0, key_ptrs[i % pool], n_keys, out_ptr, stream)
 
     for i in range(W):
         step(i)
@@ -215,7 +220,6 @@ def run_all_hit(args):
     torch.cuda.synchronize()
     elapsed = time.perf_counter() - t0
 
-    key_ptrs = [keys_pool[i].data_ptr() for i in range(pool)]
     so_step_s, so_launch_s = stream_ordered_leg(C, C.coll_cache_lookup_async, lambda i: key_ptrs[i % pool], n_keys, out,
                                                 stream, torch, W, K)
 
@@ -380,8 +384,11 @@ def run_mixed(args):
     link_gbps = max(link)
     del probe
 
+    key_ptrs = [keys_pool[i].data_ptr() for i in range(pool)]  # taken once, outside the timed steps
+    out_ptr = out.data_ptr()
+
     def step(i):
-        C.coll_cache_lookup_i64(0, keys_pool[i % pool].data_ptr(), n_keys, out.data_ptr(), stream)
+        C.coll_cache_lookup_i64(0, key_ptrs[i % pool], n_keys, out_ptr, stream)
 
     for i in range(W):
         step(i)
@@ -393,7 +400,6 @@ def run_mixed(args):
     elapsed = time.perf_counter() - t0
     note("timed region done: %.3f ms/step" % (elapsed / K * 1e3))
     g_blocking = _basics.last_group_offset(0)
-    key_ptrs = [keys_pool[i].data_ptr() for i in range(pool)]
     so_step_s, so_launch_s = stream_ordered_leg(C, C.coll_cache_lookup_async_i64, lambda i: key_ptrs[i % pool], n_keys,
                                                 out, stream, torch, W, K)
     note("stream-ordered leg done: %.3f ms/step" % (so_step_s * 1e3))
