@@ -200,16 +200,21 @@ int ugk_classify_i64(ugk_table_t t, const int64_t *keys_dev, size_t n, uint64_t 
 
 /* ---- single-kernel mixed-source extraction: kDirectNoGroup with DataIterMixLoc
  *      (cache_context.cu:137-159, 1295-1329): lookup and gather fused, source picked per row ----------
- * counts_dev (may be NULL): three device words (8-byte aligned; the third is reserved), zero on first use and left
- * zero, through which the kernel adds up how many rows came from each source; the totals land in host_mirror[1]
- * (local) and host_mirror[2] (host), the group sizes ugk_gather_group reports on the factored path.  Rows skipped
- * for a key without a row (status_dev flagged) are counted with the host rows.  n must stay below 2^32. */
+ * group_counts_host (may be NULL): pinned, GPU-mapped host memory (ugk_host_malloc) of ugk_extract_mix_max_groups()
+ * 8-byte words.  Workgroup b leaves in word b, for the keys it handled, (rows not taken from the cache << 32) | rows
+ * taken from the cache — a posted write nobody waits for.  *num_groups_host (ordinary host memory, written by the call
+ * itself before it returns, may be NULL) = the number of workgroups launched: once the stream has been waited for,
+ * the sum of that many words gives the group sizes ugk_gather_group reports on the factored path.  Rows skipped for
+ * a key without a row (status_dev flagged) are counted with the host rows.  n must stay below 2^32. */
+unsigned ugk_extract_mix_max_groups(void);
 int ugk_extract_mix_u32(ugk_table_t t, const uint32_t *keys_dev, size_t n, const void *cache_dev, uint64_t cache_rows,
                         const void *host_dev, uint64_t host_rows, void *out_dev, size_t row_bytes,
-                        uint32_t *status_dev, uint32_t *host_mirror, uint32_t *counts_dev, void *stream);
+                        uint32_t *status_dev, uint32_t *host_mirror, uint64_t *group_counts_host,
+                        uint32_t *num_groups_host, void *stream);
 int ugk_extract_mix_i64(ugk_table_t t, const int64_t *keys_dev, size_t n, const void *cache_dev, uint64_t cache_rows,
                         const void *host_dev, uint64_t host_rows, void *out_dev, size_t row_bytes,
-                        uint32_t *status_dev, uint32_t *host_mirror, uint32_t *counts_dev, void *stream);
+                        uint32_t *status_dev, uint32_t *host_mirror, uint64_t *group_counts_host,
+                        uint32_t *num_groups_host, void *stream);
 
 /* ---- key dedup (the caller-side array_ops.unique of
  *      python_tf2/collcache_tf2/collcache_tf2/core/sparse_lookup_layer.py:197) ------------------------

@@ -406,21 +406,34 @@ def test_classify_partition_and_factored_gather(mode, kdtype, n):
         # fused single-kernel variant gives the same bytes
         out2 = dev_bytes(n * rb, fill=0x11)
         fn = "ugk_extract_mix_i64" if kdtype == np.int64 else "ugk_extract_mix_u32"
-        mix_counts = dev_zeros_u32(3)
-        for _ in range(2):  # the second launch finds the counters left at zero by the first
-            mirror.array[...] = 0xFFFFFFFF
-            hip.call(fn, tb, ptr(keys_dev), n, ptr(cache_dev), cap, pin.ptr, nkeys, ptr(out2), rb, ptr(st2), mirror.ptr,
-                     ptr(mix_counts), None)
-            sync()
+        for _ in range(2):
+            got_sizes = _extract_mix(fn, tb, keys_dev, n, cache_dev, cap, pin, nkeys, out2, rb, st2, mirror)
             assert status_value(st2) == 0
             assert to_np(out2)[: n * rb].tobytes() == want_out.tobytes()
-            if n:  # same group sizes as classify found
-                assert mirror.array.tolist()[1:3] == [int(c[0]), int(c[1])]
-            assert not to_np(mix_counts, np.uint32)[:3].any()
+            assert got_sizes == [int(c[0]), int(c[1])]  # same group sizes as classify found
     finally:
         sync()
         pin.free()
         mirror.free()
+
+
+def _extract_mix(fn, tb, keys_dev, n, cache_dev, cache_rows, pin, host_rows, out, rb, st, mirror):
+    """one fused launch; -> [rows from the cache, other rows], the sum of the words its workgroups leave in pinned
+    host memory"""
+    words = PinnedArray((hip.lib().ugk_extract_mix_max_groups(),), np.uint64)
+    try:
+        words.array[...] = np.uint64(0xDEADBEEFDEADBEEF)
+        groups = C.c_uint32(12345)
+        hip.call(fn, tb, ptr(keys_dev), n, ptr(cache_dev), cache_rows, pin.ptr, host_rows, ptr(out), rb, ptr(st),
+                 mirror.ptr if mirror is not None else None, words.ptr, C.byref(groups), None)
+        sync()
+        g = groups.value
+        assert g == (0 if n == 0 else min((n + 255) // 256, len(words.array)))
+        w = words.array[:g]
+        assert (words.array[g:] == np.uint64(0xDEADBEEFDEADBEEF)).all()  # nothing written beyond the launched groups
+        return [int((w & np.uint64(0xFFFFFFFF)).sum()), int((w >> np.uint64(32)).sum())]
+    finally:
+        words.free()
 
 
 def test_classify_rejects_keys_beyond_the_host_table():
@@ -451,23 +464,21 @@ def test_extract_mix_skips_keys_without_a_row_and_still_hands_over_its_counts():
     mirror = pinned_from(np.zeros(4, np.uint32))
     try:
         st = dev_zeros_u32(1)
-        mix_counts = dev_zeros_u32(4)
         d_cache = to_dev(cache)
         for batch in (dirty, keys):
             out = dev_bytes(n * rb, fill=0x5A)
             d_keys = to_dev(batch)
             mirror.array[...] = 0
             st.zero_()
-            hip.call("ugk_extract_mix_i64", tb, ptr(d_keys), n, ptr(d_cache), len(cached), pin.ptr, nkeys, ptr(out), rb,
-                     ptr(st), mirror.ptr, ptr(mix_counts), None)
+            sizes = _extract_mix("ugk_extract_mix_i64", tb, d_keys, n, d_cache, len(cached), pin, nkeys, out, rb, st,
+                                 mirror)
             flagged = status_value(st)
             got = to_np(out)[: n * rb].reshape(n, rb)
             ok = batch < nkeys
             assert got[ok].tobytes() == host[batch[ok]].tobytes()
             assert (got[~ok] == 0x5A).all()
             local = int((batch[ok] % 3 == 0).sum())
-            assert mirror.array.tolist()[1:3] == [local, n - local]
-            assert not to_np(mix_counts, np.uint32)[:3].any()
+            assert sizes == [local, n - local]
             if ok.all():
                 assert flagged == 0 and mirror.array[0] == 0
             else:
@@ -494,7 +505,7 @@ def test_extract_mix_other_row_sizes(row_bytes):
         st = dev_zeros_u32(1)
         d_keys, d_cache = to_dev(keys), to_dev(cache)
         hip.call("ugk_extract_mix_u32", tb, ptr(d_keys), len(keys), ptr(d_cache), len(cached), pin.ptr,
-                 nkeys, ptr(out), row_bytes, ptr(st), None, None, None)
+                 nkeys, ptr(out), row_bytes, ptr(st), None, None, None, None)
         assert status_value(st) == 0
         assert to_np(out)[: len(keys) * row_bytes].tobytes() == host[keys].tobytes()
     finally:

@@ -228,6 +228,7 @@ ExtractSession::ExtractSession(std::shared_ptr<CacheContext> cache_ctx) : _cache
   _counts[0] = state + kStCounts0;
   _counts[1] = state + kStCounts1;
   _status = state + kStStatus;
+  _mix_counts = PinnedHostAlloc((size_t)ugk_extract_mix_max_groups() * sizeof(uint64_t));
   _host_mirror_handle = PinnedHostAlloc(256);
   _host_mirror = _host_mirror_handle->ptr<uint32_t>();
   memset(_host_mirror, 0, 256);
@@ -457,13 +458,25 @@ size_t ExtractSession::DedupKeys(const KeyT *nodes, size_t num_nodes, StreamHand
 
 static int ExtractMix(ugk_table_t t, const IdType *keys, size_t n, const void *cache, uint64_t cache_rows,
                       const void *host, uint64_t host_rows, void *out, size_t rb, uint32_t *st, uint32_t *mirror,
-                      uint32_t *counts, StreamHandle s) {
-  return ugk_extract_mix_u32(t, keys, n, cache, cache_rows, host, host_rows, out, rb, st, mirror, counts, s);
+                      uint64_t *counts, uint32_t *groups, StreamHandle s) {
+  return ugk_extract_mix_u32(t, keys, n, cache, cache_rows, host, host_rows, out, rb, st, mirror, counts, groups, s);
 }
 static int ExtractMix(ugk_table_t t, const Id64Type *keys, size_t n, const void *cache, uint64_t cache_rows,
                       const void *host, uint64_t host_rows, void *out, size_t rb, uint32_t *st, uint32_t *mirror,
-                      uint32_t *counts, StreamHandle s) {
-  return ugk_extract_mix_i64(t, keys, n, cache, cache_rows, host, host_rows, out, rb, st, mirror, counts, s);
+                      uint64_t *counts, uint32_t *groups, StreamHandle s) {
+  return ugk_extract_mix_i64(t, keys, n, cache, cache_rows, host, host_rows, out, rb, st, mirror, counts, groups, s);
+}
+
+// group sizes of the last fused launch: the sum of the words its workgroups left in pinned host memory
+void ExtractSession::SumMixCounts() {
+  const uint64_t *w = _mix_counts->ptr<uint64_t>();
+  uint64_t local = 0, others = 0;
+  for (uint32_t g = 0; g < _mix_groups; g++) {
+    local += (uint32_t)w[g];
+    others += w[g] >> 32;
+  }
+  _host_mirror[kMirGroupSizes + UGK_LOC_LOCAL] = (uint32_t)local;
+  _host_mirror[kMirGroupSizes + UGK_LOC_HOST] = (uint32_t)others;
 }
 
 // cache_context.cu:1199-1794
@@ -558,12 +571,13 @@ void ExtractSession::ExtractFeatImpl(const KeyT *nodes, size_t num_nodes, void *
     void *keys_ready = RecordBegin(stream);
     UGK_CALL(ugk_event_record(_ev_t[0], stream));
     UGK_CALL(ExtractMix(table, nodes, num_nodes, cache, cache_rows, host, host_rows, output, rb, _status,
-                        _host_mirror, _state + kStMixCounts, stream));
+                        _host_mirror, _mix_counts->ptr<uint64_t>(), &_mix_groups, stream));
     UGK_CALL(ugk_event_record(_ev_t[1], stream));
     RecordLaunch(input_nodes, num_input, keys_ready);
     UGK_CALL(ugk_stream_sync(stream));
     JoinRecordOnHost();
     CheckStatusWord(stream);
+    SumMixCounts();
     const uint32_t n_local = _host_mirror[kMirGroupSizes + UGK_LOC_LOCAL],
                    n_miss = _host_mirror[kMirGroupSizes + UGK_LOC_HOST];
     CHECK_EQ((size_t)n_local + n_miss, num_nodes);
@@ -688,6 +702,7 @@ void ExtractSession::ExtractFeatAsyncImpl(const KeyT *nodes, size_t num_nodes, v
                           from_host ? _cpu_blocks : 0, _status, _host_mirror, stream));
     RecordLaunch(nodes, num_nodes, keys_ready);
     JoinRecord(stream);
+    _async_last_fused = false;
     // what a blocking lookup would have read from the mirror
     _host_mirror[kMirGroupSizes + UGK_LOC_LOCAL] = from_host ? 0 : (uint32_t)num_nodes;
     _host_mirror[kMirGroupSizes + UGK_LOC_HOST] = from_host ? (uint32_t)num_nodes : 0;
@@ -699,9 +714,10 @@ void ExtractSession::ExtractFeatAsyncImpl(const KeyT *nodes, size_t num_nodes, v
     UGK_CALL(ExtractMix(ctx->_new_hash_table->_table, nodes, num_nodes,
                         ctx->_device_cache_data[ctx->_local_location_id], ctx->_cache_space_capacity,
                         ctx->_device_cache_data[ctx->_cpu_location_id], ctx->_num_total_nodes, output, rb, _status,
-                        _host_mirror, _state + kStMixCounts, stream));
+                        _host_mirror, _mix_counts->ptr<uint64_t>(), &_mix_groups, stream));
     RecordLaunch(nodes, num_nodes, keys_ready);
     JoinRecord(stream);
+    _async_last_fused = true;
   } else {
     Wait(stream);
     ExtractFeatImpl<KeyT>(nodes, num_nodes, output, stream, 0xffffffffffffffffull);
@@ -728,6 +744,7 @@ void ExtractSession::Wait(StreamHandle stream) {
   if (_async_pending == 0) return;
   UGK_CALL(ugk_stream_sync(stream));
   CheckStatusWord(stream);
+  if (_async_last_fused) SumMixCounts();
   const uint32_t n_local = _host_mirror[kMirGroupSizes + UGK_LOC_LOCAL],
                  n_miss = _host_mirror[kMirGroupSizes + UGK_LOC_HOST];
   CHECK_EQ((size_t)n_local + n_miss, _async_last_nodes);

@@ -89,8 +89,7 @@ class CacheContext {
 
 class ExtractSession {
   // words of the device-side state block (64 zero-filled uint32)
-  enum StateWord { kStCounts0 = 0, kStCounts1 = 2, kStStatus = 4, kStNumUnique = 5, kStDrainEntries = 6,
-                   kStMixCounts = 8 /* 3 words */ };
+  enum StateWord { kStCounts0 = 0, kStCounts1 = 2, kStStatus = 4, kStNumUnique = 5, kStDrainEntries = 6 };
   // words of the pinned host mirror the kernels write; [1] and [2] are indexed 1 + location
   enum MirrorWord { kMirError = 0, kMirGroupSizes = 1, kMirNumUnique = 3, kMirDrainCount = 4, kMirDrainMore = 5 };
   std::shared_ptr<CacheContext> _cache_ctx;
@@ -146,6 +145,10 @@ class ExtractSession {
   template <typename KeyT>
   void RecordLaunch(const KeyT *nodes, size_t num_nodes, void *after);
 
+  MemHandle _mix_counts;           // pinned: one word per workgroup of the fused kernel, its two row counts
+  uint32_t _mix_groups = 0;        // workgroups of the last fused launch
+  bool _async_last_fused = false;  // the last stream-ordered lookup was a fused launch (its counts wait to be summed)
+  void SumMixCounts();
   size_t _async_pending = 0;       // stream-ordered lookups enqueued since the last Wait()
   size_t _async_last_nodes = 0;    // size of the last of them
   std::atomic<bool> _async_used{false};

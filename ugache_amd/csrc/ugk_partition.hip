@@ -118,7 +118,7 @@ __global__ __launch_bounds__(kBlock) void extract_mix_kernel(ugk_table_t t, cons
                                                              const u32x4 *__restrict__ host, uint64_t host_rows,
                                                              u32x4 *__restrict__ out, uint32_t vpr,
                                                              uint32_t *status, uint32_t *host_mirror,
-                                                             uint32_t *counts, bool nt_store) {
+                                                             unsigned long long *counts, bool nt_store) {
   constexpr int RPW = kWave / LPR;  // rows per wavefront instruction
   __shared__ uint32_t block_tot[2];
   if (threadIdx.x < 2) block_tot[threadIdx.x] = 0;
@@ -175,29 +175,18 @@ __global__ __launch_bounds__(kBlock) void extract_mix_kernel(ugk_table_t t, cons
     }
   }
   if (counts == nullptr) return;
-  // Group sizes for the host.  Every workgroup adds its two sums with ONE 64-bit atomic; every key is counted in
-  // exactly one of them, so the workgroup whose add brings their total to n is the last one: it hands the totals to
-  // the pinned mirror and leaves the words at zero for the next launch.  No memory fence and no second atomic: a
-  // device-scope fence per workgroup would write back and invalidate the L2 of its XCD thousands of times per launch,
-  // and atomics on one address are performed one after the other at the memory side (about 8 ns each), which a
-  // thousand workgroups finishing together feel.
+  // Group sizes for the host: every workgroup leaves its two sums in a word of its own in pinned host memory, a posted
+  // write nobody waits for; the host adds the words up after it has waited for the stream.  Handing them over through
+  // device-side atomics cost more than it looks: a 64-bit add and a dependent ticket per workgroup 16 us of a 69 us
+  // launch at 99 % hits (same-address atomics are performed one after the other at the memory side), one add whose
+  // result tells the last workgroup still 5 us (every workgroup ends by waiting for the round trip), and a device-scope
+  // fence per workgroup 13-49 % of a whole step (each writes back and invalidates the L2 of its XCD).
   if (lane == 0) {
     if (wave_local) atomicAdd(&block_tot[0], wave_local);
     if (wave_host) atomicAdd(&block_tot[1], wave_host);
   }
   __syncthreads();
-  if (threadIdx.x == 0 && (block_tot[0] | block_tot[1])) {
-    unsigned long long *pair = reinterpret_cast<unsigned long long *>(counts);  // low word local, high word others
-    const unsigned long long mine = ((unsigned long long)block_tot[1] << 32) | block_tot[0];
-    const unsigned long long after = atomicAdd(pair, mine) + mine;
-    if ((after & 0xffffffffull) + (after >> 32) == (unsigned long long)n) {
-      atomicExch(pair, 0ull);
-      if (host_mirror) {
-        host_mirror[1 + UGK_LOC_LOCAL] = (uint32_t)after;
-        host_mirror[1 + UGK_LOC_HOST] = (uint32_t)(after >> 32);
-      }
-    }
-  }
+  if (threadIdx.x == 0) counts[blockIdx.x] = ((unsigned long long)block_tot[1] << 32) | block_tot[0];
 }
 
 // ---- dedup -----------------------------------------------------------------------------------------------
@@ -327,8 +316,9 @@ int classify(ugk_table_t t, const K *keys, size_t n, uint64_t host_rows, const u
 template <typename K, int KIND>
 int extract_mix_lpr(ugk_table_t t, const K *keys, size_t n, const void *cache, uint64_t cache_rows, const void *host,
                     uint64_t host_rows, void *out, uint32_t vpr, uint32_t *status, uint32_t *host_mirror,
-                    uint32_t *counts, hipStream_t st) {
+                    uint64_t *counts, uint32_t *num_groups, hipStream_t st) {
   const unsigned grid = clamp_grid((n + kBlock - 1) / kBlock, 0);
+  if (num_groups) *num_groups = grid;
   // ordinary write-back stores while the output fits the memory-side cache (the consumer finds it there),
   // non-temporal beyond; UGK_GATHER_NT_STORE=0/1 forces the choice
   static const int forced_nt = [] {
@@ -339,7 +329,7 @@ int extract_mix_lpr(ugk_table_t t, const K *keys, size_t n, const void *cache, u
 #define UGK_GO(L)                                                                                                 \
   hipLaunchKernelGGL((extract_mix_kernel<K, KIND, L>), dim3(grid), dim3(kBlock), 0, st, t, keys, n,               \
                      (const u32x4 *)cache, cache_rows, (const u32x4 *)host, host_rows, (u32x4 *)out, vpr, status, \
-                     host_mirror, counts, nt)
+                     host_mirror, reinterpret_cast<unsigned long long *>(counts), nt)
   if (vpr <= 1) UGK_GO(1);
   else if (vpr <= 2) UGK_GO(2);
   else if (vpr <= 4) UGK_GO(4);
@@ -355,7 +345,8 @@ int extract_mix_lpr(ugk_table_t t, const K *keys, size_t n, const void *cache, u
 template <typename K>
 int extract_mix(ugk_table_t t, const K *keys, size_t n, const void *cache, uint64_t cache_rows, const void *host,
                 uint64_t host_rows, void *out, size_t row_bytes, uint32_t *status, uint32_t *host_mirror,
-                uint32_t *counts, void *stream) {
+                uint64_t *counts, uint32_t *num_groups, void *stream) {
+  if (num_groups) *num_groups = 0;
   if (n == 0) return 0;
   UGK_REQUIRE(keys && out && status, "ugk_extract_mix: null keys, output or status");
   UGK_REQUIRE((uintptr_t)counts % 8 == 0, "ugk_extract_mix: the count words must be 8-byte aligned");
@@ -374,9 +365,9 @@ int extract_mix(ugk_table_t t, const K *keys, size_t n, const void *cache, uint6
   const uint32_t vpr = (uint32_t)(row_bytes / 16);
   if (t.kind == 1)
     return extract_mix_lpr<K, 1>(t, keys, n, cache, cache_rows, host, host_rows, out, vpr, status, host_mirror,
-                                 counts, as_stream(stream));
+                                 counts, num_groups, as_stream(stream));
   return extract_mix_lpr<K, 2>(t, keys, n, cache, cache_rows, host, host_rows, out, vpr, status, host_mirror,
-                               counts, as_stream(stream));
+                               counts, num_groups, as_stream(stream));
 }
 
 template <typename K>
@@ -421,17 +412,21 @@ int ugk_classify_i64(ugk_table_t t, const int64_t *keys_dev, size_t n, uint64_t 
                            host_mirror, stream);
 }
 
+unsigned ugk_extract_mix_max_groups(void) { return clamp_grid(~(size_t)0, 0); }
+
 int ugk_extract_mix_u32(ugk_table_t t, const uint32_t *keys_dev, size_t n, const void *cache_dev, uint64_t cache_rows,
                         const void *host_dev, uint64_t host_rows, void *out_dev, size_t row_bytes,
-                        uint32_t *status_dev, uint32_t *host_mirror, uint32_t *counts_dev, void *stream) {
+                        uint32_t *status_dev, uint32_t *host_mirror, uint64_t *group_counts_host,
+                        uint32_t *num_groups_host, void *stream) {
   return extract_mix<uint32_t>(t, keys_dev, n, cache_dev, cache_rows, host_dev, host_rows, out_dev, row_bytes,
-                               status_dev, host_mirror, counts_dev, stream);
+                               status_dev, host_mirror, group_counts_host, num_groups_host, stream);
 }
 int ugk_extract_mix_i64(ugk_table_t t, const int64_t *keys_dev, size_t n, const void *cache_dev, uint64_t cache_rows,
                         const void *host_dev, uint64_t host_rows, void *out_dev, size_t row_bytes,
-                        uint32_t *status_dev, uint32_t *host_mirror, uint32_t *counts_dev, void *stream) {
+                        uint32_t *status_dev, uint32_t *host_mirror, uint64_t *group_counts_host,
+                        uint32_t *num_groups_host, void *stream) {
   return extract_mix<int64_t>(t, keys_dev, n, cache_dev, cache_rows, host_dev, host_rows, out_dev, row_bytes,
-                              status_dev, host_mirror, counts_dev, stream);
+                              status_dev, host_mirror, group_counts_host, num_groups_host, stream);
 }
 
 size_t ugk_dedup_workspace_bytes(size_t n) { return dedup_capacity(n) * 8 + ((n + 1) / 2 * 2) * 4 + 64; }

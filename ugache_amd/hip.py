@@ -86,8 +86,9 @@ SIGNATURES = {
     "ugk_hash_census": [_vp, _sz, _vp, _vp],
     "ugk_classify_u32": [Table, _vp, _sz, _u64, _vp, _vp, _vp, _vp, _vp, _vp, _vp],
     "ugk_classify_i64": [Table, _vp, _sz, _u64, _vp, _vp, _vp, _vp, _vp, _vp, _vp],
-    "ugk_extract_mix_u32": [Table, _vp, _sz, _vp, _u64, _vp, _u64, _vp, _sz, _vp, _vp, _vp, _vp],
-    "ugk_extract_mix_i64": [Table, _vp, _sz, _vp, _u64, _vp, _u64, _vp, _sz, _vp, _vp, _vp, _vp],
+    "ugk_extract_mix_max_groups": [],
+    "ugk_extract_mix_u32": [Table, _vp, _sz, _vp, _u64, _vp, _u64, _vp, _sz, _vp, _vp, _vp, _vp, _vp],
+    "ugk_extract_mix_i64": [Table, _vp, _sz, _vp, _u64, _vp, _u64, _vp, _sz, _vp, _vp, _vp, _vp, _vp],
     "ugk_dedup_workspace_bytes": [_sz],
     "ugk_dedup_u32": [_vp, _sz, _vp, _u32, _vp, _vp, _vp, _vp, _vp, _vp],
     "ugk_dedup_i64": [_vp, _sz, _vp, _u32, _vp, _vp, _vp, _vp, _vp, _vp],
@@ -104,7 +105,7 @@ SIGNATURES = {
     "ugk_rows_to_keys": [_vp, _sz, _u64, _u64, _vp, _vp],
     "ugk_last_error": [],
 }
-_RESTYPES = {"ugk_hash_buckets_for": _sz, "ugk_dedup_workspace_bytes": _sz, "ugk_rank_workspace_bytes": _sz,
+_RESTYPES = {"ugk_extract_mix_max_groups": C.c_uint, "ugk_hash_buckets_for": _sz, "ugk_dedup_workspace_bytes": _sz, "ugk_rank_workspace_bytes": _sz,
              "ugk_bitmap_workspace_bytes": _sz, "ugk_last_error": C.c_char_p}
 _NO_CHECK = set(_RESTYPES) | {"ugk_abi_version"}
 
