@@ -75,6 +75,16 @@ void coll_cache_init_ranked_c(int replica_id, size_t key_space_size, const uint3
  * (coll_cache_lib/constant.h:28). */
 void coll_cache_lookup_i64(int replica_id, const int64_t *key, size_t num_keys, void *output, StreamHandle stream);
 void coll_cache_record_i64(int replica_id, const int64_t *key, size_t num_keys);
+/* The distinct keys of a batch looked up once (extension; the "unique -> lookup -> gather(idx)" of the TF2 binding's
+ * sparse layer, python_tf2/collcache_tf2/collcache_tf2/core/sparse_lookup_layer.py:196-209, with the unique done on the
+ * GPU inside the call): output[u, :] = row of the u-th distinct key (in order of first claim, not sorted),
+ * inverse_out[i] = which distinct key position i holds, so output[inverse_out[i], :] is the row of key[i].  output
+ * (device) needs room for num_keys rows, inverse_out (device) for num_keys words.  Blocking.  Returns the number of
+ * distinct keys. */
+size_t coll_cache_lookup_unique(int replica_id, const uint32_t *key, size_t num_keys, void *output,
+                                uint32_t *inverse_out, StreamHandle stream);
+size_t coll_cache_lookup_unique_i64(int replica_id, const int64_t *key, size_t num_keys, void *output,
+                                    uint32_t *inverse_out, StreamHandle stream);
 /* Stream-ordered lookups (extension; the reference's lookup always blocks, facade.cc:74-88 and the synchronisations
  * of cache_context.cu:1199-1794).  coll_cache_lookup_async* enqueue the batch on `stream` and return: `output` is
  * complete for anything enqueued on the same stream afterwards, which is all a framework op needs; about 10 us of

@@ -985,6 +985,11 @@ def test_serving_stack_from_a_ps_config_file(tmp_path):
                 assert got.shape == (n_rows, dim)
                 # fp32 sums of at most 8 terms against float64: tolerance 1e-5 relative to the row's magnitude
                 assert np.allclose(got, want, rtol=1e-5, atol=1e-5 * np.abs(want).max())
+                # the same with the unique done by the library's GPU hash set inside the lookup
+                fused = hps.SparseLookupLayer(model_name="dlrm", table_id=0, emb_vec_size=dim,
+                                              emb_vec_dtype=torch.float32, unique_in_library=True)
+                got2 = fused(sp_ids, weights, combiner=combiner).cpu().numpy()
+                assert np.allclose(got2, want, rtol=1e-5, atol=1e-5 * np.abs(want).max())
         with pytest.raises(ValueError):
             sparse(sp_ids, None, combiner="max")
         hps.SetStepProfileValue(profile_type=kLogL1FeatureBytes, value=123.0)
@@ -1079,3 +1084,45 @@ def test_lookups_stay_exact_while_the_device_refreshes_under_them(table_kind, mo
     out = co.coll_torch_lookup_key_t_val_ret(0, torch.from_numpy(keys).cuda(), False)
     assert out.cpu().numpy().tobytes() == ORC.gather(table, keys).tobytes()
     assert _basics.last_group_offset(0)[1] == int(np.isin(keys, got).sum())
+
+
+@pytest.mark.parametrize("pct,table_kind", [(1.0, "FLAT"), (0.0, "FLAT"), (0.25, "FLAT"), (0.25, "HASH")])
+@pytest.mark.parametrize("kdtype", [torch.int32, torch.int64])
+def test_lookup_of_the_distinct_keys_with_inverse(pct, table_kind, kdtype, monkeypatch):
+    """coll_cache_lookup_unique: every distinct key of the batch is extracted once; emb[inverse[i]] is the row of
+    keys[i], the number of rows is numpy.unique's, and the group sizes are those of the distinct keys"""
+    monkeypatch.setenv("COLL_HASH_TABLE", table_kind)
+    rng = np.random.default_rng(int(pct * 100) + (kdtype == torch.int64))
+    n_item, dim = 30_000, 48
+    co.config(make_config(n_item, pct))
+    co.coll_cache_record_init(0)
+    perm = rng.permutation(n_item)
+    s0 = perm[zipf_ranks(rng, 100_000, n_item, 1.2)]
+    if 0.0 < pct < 1.0:
+        co.coll_torch_record(0, torch.from_numpy(s0).to(kdtype))
+    emb = co.coll_torch_create_emb_shm(0, n_item, dim, torch.float32)
+    table = fill_table(emb, rng)
+    co.coll_torch_init_t(0, 0, emb, pct)
+    nid = expected_cached_set(s0.astype(np.uint32), n_item, pct)[1] if 0.0 < pct < 1.0 else None
+    for n in (1, 2, 63, 64, 65, 5_000, 120_000):
+        keys = perm[zipf_ranks(rng, n, n_item, 1.2)]
+        if n == 2:
+            keys[1] = keys[0]
+        rows, inverse = co.coll_torch_lookup_unique(0, torch.from_numpy(keys).to(kdtype).cuda())
+        uniq = np.unique(keys)
+        assert rows.shape == (len(uniq), dim) and inverse.shape == (n,) and inverse.dtype == torch.int32
+        inv = inverse.cpu().numpy()
+        assert inv.min() >= 0 and inv.max() == len(uniq) - 1
+        got = rows.cpu().numpy()[inv]
+        assert got.tobytes() == ORC.gather(table, keys.astype(np.int64)).tobytes()
+        g = _basics.last_group_offset(0)
+        assert g[2] == len(uniq)
+        if nid is not None:
+            assert g[1] == int((nid[uniq] == 0).sum())
+    rows, inverse = co.coll_torch_lookup_unique(0, torch.zeros(0, dtype=kdtype).cuda())
+    assert rows.shape[0] == 0 and inverse.numel() == 0
+    # an ordinary lookup afterwards is not deduplicated
+    keys = rng.integers(0, n_item, size=10_000)
+    out = co.coll_torch_lookup_key_t_val_ret(0, torch.from_numpy(keys).to(kdtype).cuda(), False)
+    assert out.cpu().numpy().tobytes() == ORC.gather(table, keys).tobytes()
+    assert _basics.last_group_offset(0)[2] == len(keys)

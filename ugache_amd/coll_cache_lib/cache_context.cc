@@ -503,7 +503,7 @@ void ExtractSession::ExtractFeatImpl(const KeyT *nodes, size_t num_nodes, void *
   const KeyT *input_nodes = nodes;
   const uint32_t *dst_map = nullptr, *inverse = nullptr;
   float ms_dedup = 0;
-  if (RunConfig::dedup_keys && num_nodes >= RunConfig::dedup_min_keys) {
+  if (RunConfig::dedup_keys && num_nodes >= RunConfig::dedup_min_keys && !_skip_dedup) {
     UGK_CALL(ugk_event_record(_ev_t[2], stream));
     const size_t nu = DedupKeys(nodes, num_nodes, stream);
     UGK_CALL(ugk_event_record(_ev_t[3], stream));
@@ -726,6 +726,37 @@ void ExtractSession::ExtractFeatAsyncImpl(const KeyT *nodes, size_t num_nodes, v
   _async_used.store(true);
   _async_pending++;
   _async_last_nodes = num_nodes;
+}
+
+template <typename KeyT>
+size_t ExtractSession::ExtractUniqueImpl(const KeyT *nodes, size_t num_nodes, void *output, uint32_t *inverse_out,
+                                         StreamHandle stream, uint64_t task_key) {
+  Wait(stream);
+  if (num_nodes == 0) {
+    ExtractFeatImpl<KeyT>(nodes, 0, output, stream, task_key);
+    return 0;
+  }
+  CHECK_NOTNULL(nodes);
+  CHECK_NOTNULL(output);
+  CHECK_NOTNULL(inverse_out);
+  const size_t nu = DedupKeys(nodes, num_nodes, stream);
+  UGK_CALL(ugk_memcpy_async(inverse_out, DedupInverse(), num_nodes * sizeof(uint32_t), stream));
+  _skip_dedup = true;
+  ExtractFeatImpl<KeyT>(DedupUnique<KeyT>(), nu, output, stream, task_key);  // blocks: the copy above is done too
+  _skip_dedup = false;
+  return nu;
+}
+
+size_t ExtractSession::ExtractUnique(const IdType *nodes, size_t num_nodes, void *output, uint32_t *inverse_out,
+                                     StreamHandle stream, uint64_t task_key) {
+  CHECK(RunConfig::key_map_mul == 0 || RunConfig::key_map_mask <= 0xffffffffull)
+      << "sparse ids wider than 32 bits need the 64-bit lookup";
+  return ExtractUniqueImpl<IdType>(nodes, num_nodes, output, inverse_out, stream, task_key);
+}
+
+size_t ExtractSession::ExtractUnique64(const Id64Type *nodes, size_t num_nodes, void *output, uint32_t *inverse_out,
+                                       StreamHandle stream, uint64_t task_key) {
+  return ExtractUniqueImpl<Id64Type>(nodes, num_nodes, output, inverse_out, stream, task_key);
 }
 
 void ExtractSession::ExtractFeatAsync(const IdType *nodes, const size_t num_nodes, void *output,

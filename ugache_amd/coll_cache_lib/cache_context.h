@@ -157,6 +157,10 @@ class ExtractSession {
 
   template <typename KeyT>
   void ExtractFeatImpl(const KeyT *nodes, size_t num_nodes, void *output, StreamHandle stream, uint64_t task_key);
+  template <typename KeyT>
+  size_t ExtractUniqueImpl(const KeyT *nodes, size_t num_nodes, void *output, uint32_t *inverse_out,
+                           StreamHandle stream, uint64_t task_key);
+  bool _skip_dedup = false;  // the keys handed to ExtractFeatImpl are distinct already
   void EnsureIdx(size_t num_nodes);
   void CheckStatusWord(StreamHandle stream) const;
 
@@ -169,6 +173,15 @@ class ExtractSession {
   // same for 64-bit keys (dense ids below num_total_item); an extension over the reference
   void ExtractFeat64(const Id64Type *nodes, const size_t num_nodes, void *output, StreamHandle stream,
                      uint64_t task_key);
+  // The distinct keys of the batch looked up once (an extension; the "unique -> lookup -> gather(idx)" of the TF2
+  // layer, sparse_lookup_layer.py:196-209, with the unique inside): output[u, :] = row of the u-th distinct key
+  // (in order of first claim, not sorted), inverse_out[i] = which distinct key position i holds, so that
+  // output[inverse_out[i], :] is the row of nodes[i].  output needs room for num_nodes rows, inverse_out (device) for
+  // num_nodes words.  Blocking.  Returns the number of distinct keys.
+  size_t ExtractUnique(const IdType *nodes, size_t num_nodes, void *output, uint32_t *inverse_out,
+                       StreamHandle stream, uint64_t task_key);
+  size_t ExtractUnique64(const Id64Type *nodes, size_t num_nodes, void *output, uint32_t *inverse_out,
+                         StreamHandle stream, uint64_t task_key);
   // Stream-ordered variants (an extension; the reference's lookup always blocks): the kernels of the batch are
   // enqueued on `stream` and the call returns without waiting; `output` is complete for whatever is enqueued on the
   // same stream afterwards.  All stream-ordered lookups of a session must use one stream.  Error flags, group sizes

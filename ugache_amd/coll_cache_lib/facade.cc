@@ -26,6 +26,25 @@ void CollCache::lookup64(int replica_id, const Id64Type *nodes, const size_t num
   _profiler->LogStep(step_key, common::kLogL2CacheCopyTime, t.Passed());
 }
 
+size_t CollCache::lookup_unique(int replica_id, const IdType *nodes, size_t num_nodes, void *output,
+                                uint32_t *inverse_out, StreamHandle stream, uint64_t step_key) {
+  Timer t;
+  CHECK_LT((size_t)replica_id, _session_list.size());
+  const size_t nu = _session_list[replica_id]->ExtractUnique(nodes, num_nodes, output, inverse_out, stream, step_key);
+  _profiler->LogStep(step_key, common::kLogL2CacheCopyTime, t.Passed());
+  return nu;
+}
+
+size_t CollCache::lookup_unique64(int replica_id, const Id64Type *nodes, size_t num_nodes, void *output,
+                                  uint32_t *inverse_out, StreamHandle stream, uint64_t step_key) {
+  Timer t;
+  CHECK_LT((size_t)replica_id, _session_list.size());
+  const size_t nu =
+      _session_list[replica_id]->ExtractUnique64(nodes, num_nodes, output, inverse_out, stream, step_key);
+  _profiler->LogStep(step_key, common::kLogL2CacheCopyTime, t.Passed());
+  return nu;
+}
+
 namespace {
 // every policy of the reference that runs a solver (facade.cc:110-152) reduces to the frequency-ranked
 // placement when there is one GPU

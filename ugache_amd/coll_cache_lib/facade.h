@@ -50,6 +50,11 @@ class CollCache : public std::enable_shared_from_this<CollCache> {
   // 64-bit keys, dense ids (extension)
   void lookup64(int replica_id, const Id64Type *nodes, const size_t num_nodes, void *output, StreamHandle stream,
                 uint64_t step_key);
+  // distinct keys looked up once: rows of the distinct keys + which of them every position holds (extension)
+  size_t lookup_unique(int replica_id, const IdType *nodes, size_t num_nodes, void *output, uint32_t *inverse_out,
+                       StreamHandle stream, uint64_t step_key);
+  size_t lookup_unique64(int replica_id, const Id64Type *nodes, size_t num_nodes, void *output, uint32_t *inverse_out,
+                         StreamHandle stream, uint64_t step_key);
 
   // rank list + frequency list over all num_node keys (facade.cc:283-381)
   void build_v2(int replica_id, IdType *ranking_nodes_list_ptr, IdType *ranking_nodes_freq_list_ptr, IdType num_node,

@@ -215,6 +215,22 @@ void coll_cache_lookup_i64(int replica_id, const int64_t *key, size_t num_keys, 
   _coll_cache->lookup64(replica_id, key, num_keys, output, stream, step_key);
 }
 
+size_t coll_cache_lookup_unique(int replica_id, const uint32_t *key, size_t num_keys, void *output,
+                                uint32_t *inverse_out, StreamHandle stream) {
+  CHECK_NOTNULL(_coll_cache);
+  const uint64_t step_key = steps[replica_id] * RunConfig::num_device + replica_id;
+  steps[replica_id]++;
+  return _coll_cache->lookup_unique(replica_id, key, num_keys, output, inverse_out, stream, step_key);
+}
+
+size_t coll_cache_lookup_unique_i64(int replica_id, const int64_t *key, size_t num_keys, void *output,
+                                    uint32_t *inverse_out, StreamHandle stream) {
+  CHECK_NOTNULL(_coll_cache);
+  const uint64_t step_key = steps[replica_id] * RunConfig::num_device + replica_id;
+  steps[replica_id]++;
+  return _coll_cache->lookup_unique64(replica_id, key, num_keys, output, inverse_out, stream, step_key);
+}
+
 void coll_cache_lookup_async(int replica_id, const uint32_t *key, size_t num_keys, void *output,
                              StreamHandle stream) {
   CHECK_NOTNULL(_coll_cache);

@@ -123,6 +123,10 @@ C_API = {
     "coll_cache_place_ranked": (ctypes.c_uint32, [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_uint32, ctypes.c_double,
                                                  ctypes.c_void_p]),
     "coll_cache_place_recorded": (ctypes.c_uint32, [ctypes.c_int, ctypes.c_uint32, ctypes.c_double, ctypes.c_void_p]),
+    "coll_cache_lookup_unique": (ctypes.c_size_t, [ctypes.c_int, ctypes.c_void_p, ctypes.c_size_t, ctypes.c_void_p,
+                                                   ctypes.c_void_p, ctypes.c_void_p]),
+    "coll_cache_lookup_unique_i64": (ctypes.c_size_t, [ctypes.c_int, ctypes.c_void_p, ctypes.c_size_t,
+                                                       ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p]),
     "coll_cache_lookup_async": (None, [ctypes.c_int, ctypes.c_void_p, ctypes.c_size_t, ctypes.c_void_p,
                                        ctypes.c_void_p]),
     "coll_cache_lookup_async_i64": (None, [ctypes.c_int, ctypes.c_void_p, ctypes.c_size_t, ctypes.c_void_p,

@@ -153,6 +153,24 @@ def coll_torch_lookup_key_t_val_ret(local_id, keys, pad_to_8=True):
     return _lookup_into_reused_buffer(local_id, keys, pad_to_8, _C.coll_cache_lookup, _C.coll_cache_lookup_i64)
 
 
+def coll_torch_lookup_unique(local_id, keys):
+    """the distinct keys of the batch looked up once (extension): returns (emb, inverse) with emb [num_distinct, dim] a
+    view of the reused output buffer and inverse an int32 tensor [len(keys)] such that emb[inverse[i]] is the row of
+    keys[i] — the `ids, idx = unique(ids); emb = lookup(ids)` of the TF2 sparse layer in one call, with the unique done
+    by the library's GPU hash set (distinct keys come in order of first claim, not sorted)."""
+    inverse = torch.empty((keys.numel(),), dtype=torch.int32, device=keys.device)
+    found = [0]
+
+    def fn32(replica, key_ptr, n, out_ptr, stream):
+        found[0] = _C.coll_cache_lookup_unique(replica, key_ptr, n, out_ptr, inverse.data_ptr(), stream)
+
+    def fn64(replica, key_ptr, n, out_ptr, stream):
+        found[0] = _C.coll_cache_lookup_unique_i64(replica, key_ptr, n, out_ptr, inverse.data_ptr(), stream)
+
+    out = _lookup_into_reused_buffer(local_id, keys.reshape(-1), False, fn32, fn64)
+    return out[: found[0]], inverse
+
+
 def coll_torch_lookup_async(local_id, keys, pad_to_8=True):
     """stream-ordered form of coll_torch_lookup_key_t_val_ret: the batch is enqueued on torch's current stream and
     the call returns without waiting, like any torch op; the returned view of the reused buffer is valid for work

@@ -159,7 +159,8 @@ class LookupLayer(torch.nn.Module):
         self.emb_vec_size = emb_vec_size
         self.emb_vec_dtype = emb_vec_dtype
 
-    def forward(self, inputs):
+    def check(self, inputs):
+        """the configuration's say on a batch of keys (model, table, width, key type, size)"""
         cfg = _Manager.cfg
         if cfg is None or not _Manager.initialized:
             _abort("Init() has not been called")
@@ -171,10 +172,12 @@ class LookupLayer(torch.nn.Module):
         want = torch.int64 if cfg.i64_input_key else torch.int32
         if inputs.dtype != want:
             _abort("keys must be %s (i64_input_key = %s)" % (want, cfg.i64_input_key))
-        flat = inputs.reshape(-1)
-        if flat.numel() > cfg.max_batch_size * cfg.maxnum_catfeature_query_per_table_per_sample[0]:
-            _abort("%d keys exceed max_batch_size x maxnum_catfeature_query_per_table_per_sample" % flat.numel())
-        emb = _adapter.coll_torch_forward(0, flat, False)
+        if inputs.numel() > cfg.max_batch_size * cfg.maxnum_catfeature_query_per_table_per_sample[0]:
+            _abort("%d keys exceed max_batch_size x maxnum_catfeature_query_per_table_per_sample" % inputs.numel())
+
+    def forward(self, inputs):
+        self.check(inputs)
+        emb = _adapter.coll_torch_forward(0, inputs.reshape(-1), False)
         return emb.reshape(tuple(inputs.shape) + (self.emb_vec_size,))
 
 
@@ -190,6 +193,7 @@ class SparseLookupLayer(torch.nn.Module):
         super().__init__()
         self.lookup = LookupLayer(model_name, table_id, emb_vec_size, emb_vec_dtype)
         self.emb_vec_size = emb_vec_size
+        self.unique_in_library = bool(kwargs.get("unique_in_library", False))
 
     def forward(self, sp_ids, sp_weights=None, name=None, combiner=None, max_norm=None):
         if combiner is None:
@@ -202,8 +206,14 @@ class SparseLookupLayer(torch.nn.Module):
             raise TypeError("sp_weights must be either None or a sparse COO tensor, got %s" % type(sp_weights))
         # entries as given (row-major order is the caller's contract); coalesce() would merge duplicate positions
         segment_ids = sp_ids._indices()[0]
-        ids, idx = torch.unique(sp_ids._values(), return_inverse=True)
-        embeddings = self.lookup(ids).index_select(0, idx)
+        ids = sp_ids._values()
+        if self.unique_in_library:  # unique + lookup in one call, the unique by the library's GPU hash set
+            self.lookup.check(ids)
+            emb_unique, idx = _adapter.coll_torch_lookup_unique(0, ids)
+            embeddings = emb_unique.index_select(0, idx.long())
+        else:
+            ids, idx = torch.unique(ids, return_inverse=True)
+            embeddings = self.lookup(ids).index_select(0, idx)
         original_dtype = embeddings.dtype
         if embeddings.dtype in (torch.float16, torch.bfloat16):
             embeddings = embeddings.float()  # low-precision rows are combined in fp32
