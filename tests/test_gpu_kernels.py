@@ -428,7 +428,7 @@ def _extract_mix(fn, tb, keys_dev, n, cache_dev, cache_rows, pin, host_rows, out
                  mirror.ptr if mirror is not None else None, words.ptr, C.byref(groups), None)
         sync()
         g = groups.value
-        assert g == (0 if n == 0 else min((n + 255) // 256, len(words.array)))
+        assert (g == 0) if n == 0 else (1 <= g <= len(words.array))
         w = words.array[:g]
         assert (words.array[g:] == np.uint64(0xDEADBEEFDEADBEEF)).all()  # nothing written beyond the launched groups
         return [int((w & np.uint64(0xFFFFFFFF)).sum()), int((w >> np.uint64(32)).sum())]
