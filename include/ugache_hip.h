@@ -186,7 +186,7 @@ int ugk_hash_census(const ugk_bucket_t *table_dev, size_t nbuckets, uint64_t *ce
  * wavefront-ballot prefix scan and LDS-staged compaction into idx_dev[0..n):
  *   local hits  fill idx[0, c[0])          as {dst_off = i, src_off = cache slot}
  *   host misses fill idx[n - c[1], n)      as {dst_off = i, src_off = host row = key}
- * counts_dev[0..1] must be zero on entry; the kernel also zeroes next_counts_dev[0..1] (may be NULL) so a
+ * counts_dev[0..1] (one 8-byte aligned word) must be zero on entry; the kernel also zeroes next_counts_dev[0..1] (may be NULL) so a
  * caller can rotate two counter pairs and never launch a memset.  host_rows bounds the miss offsets.
  * A key found with a location other than local/host sets UGK_ST_KEY_OUT_OF_RANGE (one GPU has two sources).
  * dst_map_dev (may be NULL): output row of key i is dst_map_dev[i] instead of i (deduplicated extraction: the keys

@@ -91,8 +91,13 @@ __global__ __launch_bounds__(kBlock) void classify_kernel(ugk_table_t t, const K
       }
     }
     if (tid == 0) {
-      base[0] = H ? atomicAdd(counts + 0, H) : 0u;
-      base[1] = M ? atomicAdd(counts + 1, M) : 0u;
+      // both reservations with one 64-bit add (the two counters share an aligned word, neither can carry: their sum
+      // stays below 2^32): atomics on one address are performed one after the other, so half as many is half the queue
+      const unsigned long long add = ((unsigned long long)M << 32) | H;
+      const unsigned long long before =
+          add ? atomicAdd(reinterpret_cast<unsigned long long *>(counts), add) : 0ull;
+      base[0] = (uint32_t)before;
+      base[1] = (uint32_t)(before >> 32);
     }
 #pragma unroll
     for (int j = 0; j < kItems; ++j) {
@@ -295,6 +300,7 @@ int classify(ugk_table_t t, const K *keys, size_t n, uint64_t host_rows, const u
              uint32_t *counts, uint32_t *next_counts, uint32_t *status, uint32_t *host_mirror, void *stream) {
   UGK_REQUIRE(counts && status, "ugk_classify: null counters or status");
   UGK_REQUIRE(n <= 0xffffffffull, "ugk_classify: batch of %zu keys exceeds 2^32", n);
+  UGK_REQUIRE((uintptr_t)counts % 8 == 0, "ugk_classify: the two counters must share an 8-byte aligned word");
   UGK_REQUIRE(t.kind == 1 || t.kind == 2, "ugk_classify: table kind %d is not flat(1) or hash(2)", t.kind);
   UGK_REQUIRE(t.table && t.size, "ugk_classify: empty table");
   if (t.kind == 2)
