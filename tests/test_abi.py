@@ -3,6 +3,7 @@
 import ctypes
 import os
 import re
+import sys
 
 import pytest
 
@@ -105,3 +106,22 @@ def test_torch_surface_has_the_reference_entry_points():
     assert inspect.signature(co.coll_torch_lookup_key_t_val_ret).parameters["pad_to_8"].default is True
     assert inspect.signature(co.coll_torch_create_emb_shm).parameters["fname"].default == ""
     assert co.kCollCacheAsymmLink == 13
+
+
+def test_serving_module_has_the_tf2_bindings_entry_points():
+    """collcache.torch.serving carries the names the reference's inference scripts call on collcache_tf2
+    (python_tf2/collcache_tf2/collcache_tf2/core/initialize.py:33-39, 79, 129, 292; core/lookup_layer.py:22;
+    core/sparse_lookup_layer.py:27),"""
+    torch = pytest.importorskip("torch")
+    sys.path.insert(0, os.path.join(ROOT, "ugache_amd"))
+    import inspect
+    import collcache.torch.serving as hps
+    want = ["Config", "Init", "Report", "NopDep", "wait_one_child", "SetStepProfileValue", "LookupLayer",
+            "SparseLookupLayer"]
+    for name in want:
+        assert hasattr(hps, name), name
+    assert list(inspect.signature(hps.LookupLayer.__init__).parameters)[1:5] == [
+        "model_name", "table_id", "emb_vec_size", "emb_vec_dtype"]
+    assert list(inspect.signature(hps.SparseLookupLayer.forward).parameters)[1:6] == [
+        "sp_ids", "sp_weights", "name", "combiner", "max_norm"]
+    assert issubclass(hps.LookupLayer, torch.nn.Module) and issubclass(hps.SparseLookupLayer, torch.nn.Module)

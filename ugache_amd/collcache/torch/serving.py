@@ -264,6 +264,12 @@ def wait_one_child():
     return _adapter.wait_one_child()
 
 
+def NopDep(dense, emb):
+    """collcache_tf2.NopDep: `dense`, made to depend on `emb` having been computed.  A TensorFlow graph needs the
+    dependency spelled out; here lookups are blocking or stream-ordered, so `dense` comes back as it is."""
+    return dense
+
+
 def Shutdown():
     """drop everything so that Config() may be called again (the reference has no teardown)"""
     _adapter.coll_torch_forward_join()
