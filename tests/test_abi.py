@@ -111,7 +111,7 @@ def test_torch_surface_has_the_reference_entry_points():
 def test_serving_module_has_the_tf2_bindings_entry_points():
     """collcache.torch.serving carries the names the reference's inference scripts call on collcache_tf2
     (python_tf2/collcache_tf2/collcache_tf2/core/initialize.py:33-39, 79, 129, 292; core/lookup_layer.py:22;
-    core/sparse_lookup_layer.py:27),"""
+    core/sparse_lookup_layer.py:27)"""
     torch = pytest.importorskip("torch")
     sys.path.insert(0, os.path.join(ROOT, "ugache_amd"))
     import inspect
