@@ -135,6 +135,13 @@ def stream_ordered_leg(C, fn, key_ptr_of, n_keys, out, stream, torch, W, K):
     return wall, ms.value * 1e-3 / K
 
 
+def step_spread(t0, stamps):
+    """median and 95th percentile of the wall time of the blocking calls of a timed region, in milliseconds"""
+    import numpy as np
+    d = np.diff(np.concatenate(([t0], np.asarray(stamps)))) * 1e3
+    return {"median": float(np.median(d)), "p95": float(np.percentile(d, 95)), "max": float(d.max())}
+
+
 def cpu_baseline(orc, table_np, keys_host, n_keys, row_bytes, seconds):
     """the oracle's OpenMP gather over the same key batches; returns (keys/s, batches, elapsed, threads)"""
     import numpy as np
@@ -214,11 +221,14 @@ def run_all_hit(args):
     for i in range(W):
         step(i)
     torch.cuda.synchronize()
+    stamps = [0.0] * K  # the call blocks until the rows are in place, so a clock read after it bounds that step
     t0 = time.perf_counter()
     for i in range(W, W + K):
         step(i)
+        stamps[i - W] = time.perf_counter()
     torch.cuda.synchronize()
     elapsed = time.perf_counter() - t0
+    spread = step_spread(t0, stamps)
 
     so_step_s, so_launch_s = stream_ordered_leg(C, C.coll_cache_lookup_async, lambda i: key_ptrs[i % pool], n_keys, out,
                                                 stream, torch, W, K)
@@ -258,7 +268,8 @@ def run_all_hit(args):
     result = {
         "metric": "embedding keys/sec + effective extraction GB/s (% HBM / host-link roofline), 1 GPU",
         "value": keys_per_s, "unit": "keys/s", "n_gpus": 1, "steps": K, "warmup": W,
-        "ms_per_step": elapsed / K * 1e3, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "ms_per_step": elapsed / K * 1e3, "ms_per_step_spread": spread,
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "u8", "data": "synthetic",
         "config": {"workload": args.workload, "table_rows": rows, "row_bytes": row_bytes, "keys_per_batch": n_keys,
                    "key_dtype": "uint32", "cache_percentage": 1.0, "entry_point": "coll_cache_lookup",
@@ -393,11 +404,14 @@ def run_mixed(args):
     for i in range(W):
         step(i)
     torch.cuda.synchronize()
+    stamps = [0.0] * K  # the call blocks until the rows are in place, so a clock read after it bounds that step
     t0 = time.perf_counter()
     for i in range(W, W + K):
         step(i)
+        stamps[i - W] = time.perf_counter()
     torch.cuda.synchronize()
     elapsed = time.perf_counter() - t0
+    spread = step_spread(t0, stamps)
     note("timed region done: %.3f ms/step" % (elapsed / K * 1e3))
     g_blocking = _basics.last_group_offset(0)
     so_step_s, so_launch_s = stream_ordered_leg(C, C.coll_cache_lookup_async_i64, lambda i: key_ptrs[i % pool], n_keys,
@@ -562,7 +576,8 @@ def run_mixed(args):
     result = {
         "metric": "embedding keys/sec + effective extraction GB/s (% HBM / host-link roofline), 1 GPU",
         "value": keys_per_s, "unit": "keys/s", "n_gpus": 1, "steps": K, "warmup": W,
-        "ms_per_step": elapsed / K * 1e3, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "ms_per_step": elapsed / K * 1e3, "ms_per_step_spread": spread,
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "u8", "data": "synthetic",
         "refresh": refresh, "refresh_each_step": each_step, "under_concurrent_refresh": under_refresh,
         "config": {"workload": args.workload, "table_rows": rows, "row_bytes": row_bytes, "keys_per_batch": n_keys,
