@@ -436,6 +436,68 @@ def _extract_mix(fn, tb, keys_dev, n, cache_dev, cache_rows, pin, host_rows, out
         words.free()
 
 
+def test_outputs_beyond_4_GiB():
+    """9M keys of 512-byte rows: the output (4.6 GB) passes 2^32 bytes, so every byte offset the kernels form must be a
+    64-bit one.  table[r, c] is a closed form of (r, c); all three extraction paths are checked against it on the
+    device, slice by slice."""
+    rows, dim, n = 300_000, 128, 9_000_000
+    rb = dim * 4
+    assert n * rb > 1 << 32
+    r = torch.arange(rows, device="cuda", dtype=torch.int32).unsqueeze(1)
+    c = torch.arange(dim, device="cuda", dtype=torch.int32).unsqueeze(0)
+    table = (r * 131 + c * 7919) ^ (r >> 3)
+    g = torch.Generator(device="cuda").manual_seed(9)
+    keys = torch.randint(0, rows, (n,), generator=g, device="cuda", dtype=torch.int32)
+    keys[-1] = rows - 1
+    keys[0] = 0
+
+    def check(out):
+        for lo in range(0, n, 1_000_000):
+            k = keys[lo : lo + 1_000_000].unsqueeze(1)
+            assert torch.equal(out[lo : lo + 1_000_000], (k * 131 + c * 7919) ^ (k >> 3)), lo
+
+    st = dev_zeros_u32(1)
+    out = torch.full((n, dim), 0x55555555, dtype=torch.int32, device="cuda")
+    hip.call("ugk_gather_direct_u32", table.data_ptr(), rows, keys.data_ptr(), n, out.data_ptr(), rb, 0, ptr(st), None,
+             None)
+    assert status_value(st) == 0
+    check(out)
+
+    # every third row cached, in shuffled slots; the others are read from pinned host memory
+    cached = np.arange(0, rows, 3, dtype=np.uint32)
+    slots = np.random.default_rng(9).permutation(len(cached)).astype(np.uint32)
+    mem, tb = _make_flat(rows)
+    assert _insert(tb, cached, slots) == 0
+    cache = torch.empty((len(cached), dim), dtype=torch.int32, device="cuda")
+    cache[torch.from_numpy(slots.astype(np.int64)).cuda()] = table[torch.from_numpy(cached.astype(np.int64)).cuda()]
+    pin = PinnedArray((rows, dim), np.int32)
+    mirror = pinned_from(np.zeros(4, np.uint32))
+    try:
+        pin.array[...] = table.cpu().numpy()
+        n_local = int((keys % 3 == 0).sum())
+        out.fill_(0x55555555)
+        sizes = _extract_mix("ugk_extract_mix_u32", tb, keys, n, cache, len(cached), pin, rows, out, rb, st, mirror)
+        assert status_value(st) == 0 and sizes == [n_local, n - n_local]
+        check(out)
+
+        out.fill_(0x55555555)
+        idx = dev_bytes(n * 8)
+        counts = dev_zeros_u32(4)
+        hip.call("ugk_classify_u32", tb, keys.data_ptr(), n, rows, None, ptr(idx), ptr(counts), ptr(counts) + 8, ptr(st),
+                 None, None)
+        hip.call("ugk_gather_group", pin.ptr, rows, ptr(idx), ptr(counts), hip.LOC_HOST, n, out.data_ptr(), n, rb, 0,
+                 ptr(st), None, None)
+        hip.call("ugk_gather_group", cache.data_ptr(), len(cached), ptr(idx), ptr(counts), hip.LOC_LOCAL, n,
+                 out.data_ptr(), n, rb, 0, ptr(st), None, None)
+        assert status_value(st) == 0
+        assert to_np(counts, np.uint32)[:2].tolist() == [n_local, n - n_local]
+        check(out)
+    finally:
+        sync()
+        pin.free()
+        mirror.free()
+
+
 def test_classify_rejects_keys_beyond_the_host_table():
     mem, tb = _make_flat(100)
     keys = np.array([5, 100, 7, 1 << 33], np.int64)
