@@ -877,6 +877,32 @@ def test_batch_whose_output_passes_4_GiB(impl, dedup, monkeypatch):
         assert _basics.last_group_offset(0) == [0, int((nid[keys] == 0).sum()), n]
 
 
+def test_cache_of_more_than_2_pow_28_slots():
+    """290M rows of 16 bytes, 95 % cached: 275M cache slots, more than the 28 bits of a flat entry hold, so the table is
+    the open-addressing one with its 32-bit slot field.  Nothing is recorded, so rows [0, K) are the cached ones;
+    table[r, c] = 4 r + c as int32 bits."""
+    n_item, dim, pct, n = 290_000_000, 4, 0.95, 2_000_000
+    co.config(make_config(n_item, pct))
+    co.coll_cache_record_init(0)
+    emb = co.coll_torch_create_emb_shm(0, n_item, dim, torch.float32)
+    flat = emb.view(torch.int32).view(-1)
+    for lo in range(0, flat.numel(), 1 << 28):
+        hi = min(lo + (1 << 28), flat.numel())
+        torch.arange(lo, hi, dtype=torch.int32, out=flat[lo:hi])
+    co.coll_torch_init_t(0, 0, emb, pct)
+    info = _basics.info(0)
+    k = int(n_item * pct)
+    assert info["table_kind"] == 2 and info["cached_rows"] == k
+    assert info["capacity_rows"] == ORC.lib.orc_cache_capacity(n_item, pct) > 1 << 28
+    g = torch.Generator(device="cuda").manual_seed(12)
+    keys = torch.randint(0, n_item, (n,), generator=g, device="cuda", dtype=torch.int64)
+    keys[:4] = torch.tensor([0, k - 1, k, n_item - 1], device="cuda")
+    out = co.coll_torch_lookup_key_t_val_ret(0, keys, False)
+    want = (keys * 4).unsqueeze(1) + torch.arange(dim, device="cuda")
+    assert torch.equal(out.view(torch.int32), want.to(torch.int32))
+    assert _basics.last_group_offset(0) == [0, int((keys < k).sum()), n]
+
+
 @pytest.mark.parametrize("gpu_record", [False, True, "and_refresh"])
 def test_sparse_ids_hash_table_with_refresh_each_step(gpu_record, monkeypatch):
     """The hashtable-mode configuration, scaled down: ids are 64-bit values from a 2^40 space (id = row * odd mod 2^40),

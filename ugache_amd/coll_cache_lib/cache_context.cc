@@ -125,6 +125,13 @@ void CacheContext::build_with_advise_new_hash(int location_id, std::shared_ptr<C
     CHECK(RunConfig::force_table_kind != 1) << "sparse ids cannot index a flat table";
     use_flat = false;
   }
+  // a flat entry packs (location << 28) + slot (cache_hashtable.h:20-28): beyond 2^28 slots only a bucket's 32-bit
+  // slot field can name them all
+  if (_cache_space_capacity > ((size_t)1 << 28)) {
+    CHECK(RunConfig::force_table_kind != 1)
+        << "a flat table addresses 2^28 cache slots, this cache has " << _cache_space_capacity;
+    use_flat = false;
+  }
   if (use_flat) {
     _new_hash_table->CreateFlat(_eager_gpu_mem_allocator, num_total_nodes, stream);
   } else {
