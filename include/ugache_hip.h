@@ -205,16 +205,20 @@ int ugk_classify_i64(ugk_table_t t, const int64_t *keys_dev, size_t n, uint64_t 
  * taken from the cache — a posted write nobody waits for.  *num_groups_host (ordinary host memory, written by the call
  * itself before it returns, may be NULL) = the number of workgroups launched: once the stream has been waited for,
  * the sum of that many words gives the group sizes ugk_gather_group reports on the factored path.  Rows skipped for
- * a key without a row (status_dev flagged) are counted with the host rows.  n must stay below 2^32. */
+ * a key without a row (status_dev flagged) are counted with the host rows.  n must stay below 2^32.
+ * others_hint: the caller's estimate of how many of the n rows will NOT come from the cache (the previous batch's
+ * count scaled to n, say), UGK_HINT_UNKNOWN if it has none.  Only the launch shape depends on it (a small batch that
+ * nearly all hits a flat table is given 32 instead of 64 keys per wavefront), never a byte of the result. */
+#define UGK_HINT_UNKNOWN 0xffffffffu
 unsigned ugk_extract_mix_max_groups(void);
 int ugk_extract_mix_u32(ugk_table_t t, const uint32_t *keys_dev, size_t n, const void *cache_dev, uint64_t cache_rows,
                         const void *host_dev, uint64_t host_rows, void *out_dev, size_t row_bytes,
                         uint32_t *status_dev, uint32_t *host_mirror, uint64_t *group_counts_host,
-                        uint32_t *num_groups_host, void *stream);
+                        uint32_t *num_groups_host, uint32_t others_hint, void *stream);
 int ugk_extract_mix_i64(ugk_table_t t, const int64_t *keys_dev, size_t n, const void *cache_dev, uint64_t cache_rows,
                         const void *host_dev, uint64_t host_rows, void *out_dev, size_t row_bytes,
                         uint32_t *status_dev, uint32_t *host_mirror, uint64_t *group_counts_host,
-                        uint32_t *num_groups_host, void *stream);
+                        uint32_t *num_groups_host, uint32_t others_hint, void *stream);
 
 /* ---- key dedup (the caller-side array_ops.unique of
  *      python_tf2/collcache_tf2/collcache_tf2/core/sparse_lookup_layer.py:197) ------------------------

@@ -406,8 +406,9 @@ def test_classify_partition_and_factored_gather(mode, kdtype, n):
         # fused single-kernel variant gives the same bytes
         out2 = dev_bytes(n * rb, fill=0x11)
         fn = "ugk_extract_mix_i64" if kdtype == np.int64 else "ugk_extract_mix_u32"
-        for _ in range(2):
-            got_sizes = _extract_mix(fn, tb, keys_dev, n, cache_dev, cap, pin, nkeys, out2, rb, st2, mirror)
+        for hint in (hip.HINT_UNKNOWN, 0, n):  # no guess; "all from the cache" (32 keys per wavefront); "none"
+            out2.fill_(0x11)
+            got_sizes = _extract_mix(fn, tb, keys_dev, n, cache_dev, cap, pin, nkeys, out2, rb, st2, mirror, hint)
             assert status_value(st2) == 0
             assert to_np(out2)[: n * rb].tobytes() == want_out.tobytes()
             assert got_sizes == [int(c[0]), int(c[1])]  # same group sizes as classify found
@@ -417,15 +418,16 @@ def test_classify_partition_and_factored_gather(mode, kdtype, n):
         mirror.free()
 
 
-def _extract_mix(fn, tb, keys_dev, n, cache_dev, cache_rows, pin, host_rows, out, rb, st, mirror):
+def _extract_mix(fn, tb, keys_dev, n, cache_dev, cache_rows, pin, host_rows, out, rb, st, mirror,
+                 hint=hip.HINT_UNKNOWN):
     """one fused launch; -> [rows from the cache, other rows], the sum of the words its workgroups leave in pinned
-    host memory"""
+    host memory.  hint: the caller's guess of the second number, which may change the launch shape only."""
     words = PinnedArray((hip.lib().ugk_extract_mix_max_groups(),), np.uint64)
     try:
         words.array[...] = np.uint64(0xDEADBEEFDEADBEEF)
         groups = C.c_uint32(12345)
         hip.call(fn, tb, ptr(keys_dev), n, ptr(cache_dev), cache_rows, pin.ptr, host_rows, ptr(out), rb, ptr(st),
-                 mirror.ptr if mirror is not None else None, words.ptr, C.byref(groups), None)
+                 mirror.ptr if mirror is not None else None, words.ptr, C.byref(groups), hint, None)
         sync()
         g = groups.value
         assert (g == 0) if n == 0 else (1 <= g <= len(words.array))
@@ -567,7 +569,7 @@ def test_extract_mix_other_row_sizes(row_bytes):
         st = dev_zeros_u32(1)
         d_keys, d_cache = to_dev(keys), to_dev(cache)
         hip.call("ugk_extract_mix_u32", tb, ptr(d_keys), len(keys), ptr(d_cache), len(cached), pin.ptr,
-                 nkeys, ptr(out), row_bytes, ptr(st), None, None, None, None)
+                 nkeys, ptr(out), row_bytes, ptr(st), None, None, None, hip.HINT_UNKNOWN, None)
         assert status_value(st) == 0
         assert to_np(out)[: len(keys) * row_bytes].tobytes() == host[keys].tobytes()
     finally:

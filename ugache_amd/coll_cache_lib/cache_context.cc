@@ -465,13 +465,15 @@ size_t ExtractSession::DedupKeys(const KeyT *nodes, size_t num_nodes, StreamHand
 
 static int ExtractMix(ugk_table_t t, const IdType *keys, size_t n, const void *cache, uint64_t cache_rows,
                       const void *host, uint64_t host_rows, void *out, size_t rb, uint32_t *st, uint32_t *mirror,
-                      uint64_t *counts, uint32_t *groups, StreamHandle s) {
-  return ugk_extract_mix_u32(t, keys, n, cache, cache_rows, host, host_rows, out, rb, st, mirror, counts, groups, s);
+                      uint64_t *counts, uint32_t *groups, uint32_t hint, StreamHandle s) {
+  return ugk_extract_mix_u32(t, keys, n, cache, cache_rows, host, host_rows, out, rb, st, mirror, counts, groups, hint,
+                             s);
 }
 static int ExtractMix(ugk_table_t t, const Id64Type *keys, size_t n, const void *cache, uint64_t cache_rows,
                       const void *host, uint64_t host_rows, void *out, size_t rb, uint32_t *st, uint32_t *mirror,
-                      uint64_t *counts, uint32_t *groups, StreamHandle s) {
-  return ugk_extract_mix_i64(t, keys, n, cache, cache_rows, host, host_rows, out, rb, st, mirror, counts, groups, s);
+                      uint64_t *counts, uint32_t *groups, uint32_t hint, StreamHandle s) {
+  return ugk_extract_mix_i64(t, keys, n, cache, cache_rows, host, host_rows, out, rb, st, mirror, counts, groups, hint,
+                             s);
 }
 
 // group sizes of the last fused launch: the sum of the words its workgroups left in pinned host memory
@@ -484,6 +486,14 @@ void ExtractSession::SumMixCounts() {
   }
   _host_mirror[kMirGroupSizes + UGK_LOC_LOCAL] = (uint32_t)local;
   _host_mirror[kMirGroupSizes + UGK_LOC_HOST] = (uint32_t)others;
+  _mix_seen_rows = local + others;
+  _mix_seen_others = others;
+}
+
+// what the next fused launch is told to expect: the share of rows the last one took from outside the cache
+uint32_t ExtractSession::MixOthersHint(size_t num_nodes) const {
+  if (_mix_seen_rows == 0) return UGK_HINT_UNKNOWN;
+  return (uint32_t)((double)_mix_seen_others / (double)_mix_seen_rows * (double)num_nodes);
 }
 
 // cache_context.cu:1199-1794
@@ -578,7 +588,8 @@ void ExtractSession::ExtractFeatImpl(const KeyT *nodes, size_t num_nodes, void *
     void *keys_ready = RecordBegin(stream);
     UGK_CALL(ugk_event_record(_ev_t[0], stream));
     UGK_CALL(ExtractMix(table, nodes, num_nodes, cache, cache_rows, host, host_rows, output, rb, _status,
-                        _host_mirror, _mix_counts->ptr<uint64_t>(), &_mix_groups, stream));
+                        _host_mirror, _mix_counts->ptr<uint64_t>(), &_mix_groups, MixOthersHint(num_nodes),
+                        stream));
     UGK_CALL(ugk_event_record(_ev_t[1], stream));
     RecordLaunch(input_nodes, num_input, keys_ready);
     UGK_CALL(ugk_stream_sync(stream));
@@ -721,7 +732,8 @@ void ExtractSession::ExtractFeatAsyncImpl(const KeyT *nodes, size_t num_nodes, v
     UGK_CALL(ExtractMix(ctx->_new_hash_table->_table, nodes, num_nodes,
                         ctx->_device_cache_data[ctx->_local_location_id], ctx->_cache_space_capacity,
                         ctx->_device_cache_data[ctx->_cpu_location_id], ctx->_num_total_nodes, output, rb, _status,
-                        _host_mirror, _mix_counts->ptr<uint64_t>(), &_mix_groups, stream));
+                        _host_mirror, _mix_counts->ptr<uint64_t>(), &_mix_groups, MixOthersHint(num_nodes),
+                        stream));
     RecordLaunch(nodes, num_nodes, keys_ready);
     JoinRecord(stream);
     _async_last_fused = true;

@@ -149,6 +149,8 @@ class ExtractSession {
   uint32_t _mix_groups = 0;        // workgroups of the last fused launch
   bool _async_last_fused = false;  // the last stream-ordered lookup was a fused launch (its counts wait to be summed)
   void SumMixCounts();
+  uint64_t _mix_seen_rows = 0, _mix_seen_others = 0;  // what the last summed fused launch found
+  uint32_t MixOthersHint(size_t num_nodes) const;
   size_t _async_pending = 0;       // stream-ordered lookups enqueued since the last Wait()
   size_t _async_last_nodes = 0;    // size of the last of them
   std::atomic<bool> _async_used{false};

@@ -117,7 +117,7 @@ __global__ __launch_bounds__(kBlock) void classify_kernel(ugk_table_t t, const K
 }
 
 // ---- fused lookup + gather: every wavefront resolves 64 keys, then copies their 64 rows ------------------
-template <typename K, int KIND, int LPR>
+template <typename K, int KIND, int LPR, int KPW>
 __global__ __launch_bounds__(kBlock) void extract_mix_kernel(ugk_table_t t, const K *__restrict__ keys, size_t n,
                                                              const u32x4 *__restrict__ cache, uint64_t cache_rows,
                                                              const u32x4 *__restrict__ host, uint64_t host_rows,
@@ -129,14 +129,15 @@ __global__ __launch_bounds__(kBlock) void extract_mix_kernel(ugk_table_t t, cons
   if (threadIdx.x < 2) block_tot[threadIdx.x] = 0;
   __syncthreads();
   uint32_t wave_local = 0, wave_host = 0;  // rows this wavefront took from each source (wavefront-uniform)
-  constexpr int UNROLL = (RPW * 4 <= kWave) ? 4 : (kWave / RPW);
+  constexpr int UNROLL = (RPW * 4 <= KPW) ? 4 : (KPW / RPW);
+  static_assert(KPW <= kWave && KPW % (RPW * UNROLL) == 0, "keys per wavefront must be whole rounds of rows");
   const int lane = (int)lane_id();
   const int sub = lane % LPR, rg = lane / LPR;
   const size_t wave_global = (size_t)blockIdx.x * kWavesPerBlock + threadIdx.x / kWave;
   const size_t n_waves = (size_t)gridDim.x * kWavesPerBlock;
-  for (size_t b0 = wave_global * kWave; b0 < n; b0 += n_waves * kWave) {
+  for (size_t b0 = wave_global * KPW; b0 < n; b0 += n_waves * KPW) {
     const size_t i = b0 + lane;
-    const bool active = i < n;
+    const bool active = lane < KPW && i < n;
     const uint64_t key = active ? key_to_u64<K>(keys[i]) : 0;
     const Found f = table_lookup<KIND>(t, key, active);
     const u32x4 *rowp = nullptr;
@@ -157,7 +158,7 @@ __global__ __launch_bounds__(kBlock) void extract_mix_kernel(ugk_table_t t, cons
       wave_local += __popcll(__ballot(from_cache));
       wave_host += __popcll(__ballot(active && !from_cache));
     }
-    for (int r0 = 0; r0 < kWave; r0 += RPW * UNROLL) {
+    for (int r0 = 0; r0 < KPW; r0 += RPW * UNROLL) {
       const u32x4 *p[UNROLL];
 #pragma unroll
       for (int u = 0; u < UNROLL; ++u) p[u] = reinterpret_cast<const u32x4 *>(shfl64(rowbits, r0 + u * RPW + rg));
@@ -322,9 +323,7 @@ int classify(ugk_table_t t, const K *keys, size_t n, uint64_t host_rows, const u
 template <typename K, int KIND>
 int extract_mix_lpr(ugk_table_t t, const K *keys, size_t n, const void *cache, uint64_t cache_rows, const void *host,
                     uint64_t host_rows, void *out, uint32_t vpr, uint32_t *status, uint32_t *host_mirror,
-                    uint64_t *counts, uint32_t *num_groups, hipStream_t st) {
-  const unsigned grid = clamp_grid((n + kBlock - 1) / kBlock, 0);
-  if (num_groups) *num_groups = grid;
+                    uint64_t *counts, uint32_t *num_groups, uint32_t others_hint, hipStream_t st) {
   // ordinary write-back stores while the output fits the memory-side cache (the consumer finds it there),
   // non-temporal beyond; UGK_GATHER_NT_STORE=0/1 forces the choice
   static const int forced_nt = [] {
@@ -332,11 +331,28 @@ int extract_mix_lpr(ugk_table_t t, const K *keys, size_t n, const void *cache, u
     return e ? atoi(e) : -1;
   }();
   const bool nt = forced_nt >= 0 ? forced_nt != 0 : n * (size_t)vpr * 16 > ((size_t)192 << 20);
-#define UGK_GO(L)                                                                                                 \
-  hipLaunchKernelGGL((extract_mix_kernel<K, KIND, L>), dim3(grid), dim3(kBlock), 0, st, t, keys, n,               \
+  // Keys per wavefront.  64 fill every lane of the lookup.  A batch that nearly all comes from the cache is bound by
+  // HBM, and a small one then leaves half the wavefront slots of the chip empty: 32 keys per wavefront double the
+  // wavefronts with rows in flight (262,144 keys, 99 % hits, flat table: 55 -> 51 us).  Batches bound by the host link
+  // run 1-2 % slower that way, and the hash table's probe wants all 64 lanes (68 -> 74 us), so both keep 64.
+  const size_t slots = (size_t)cu_count() * 4 * 8;  // wavefronts resident at 8 per SIMD
+  const bool half = KIND == 1 && vpr > 1 && others_hint != UGK_HINT_UNKNOWN && (size_t)others_hint * 50 <= n &&
+                    (n + 31) / 32 <= slots;
+  const size_t keys_per_group = half ? kBlock / 2 : kBlock;
+  const unsigned grid = clamp_grid((n + keys_per_group - 1) / keys_per_group, 0);
+  if (num_groups) *num_groups = grid;
+#define UGK_GO2(L, W)                                                                                              \
+  hipLaunchKernelGGL((extract_mix_kernel<K, KIND, L, W>), dim3(grid), dim3(kBlock), 0, st, t, keys, n,            \
                      (const u32x4 *)cache, cache_rows, (const u32x4 *)host, host_rows, (u32x4 *)out, vpr, status, \
                      host_mirror, reinterpret_cast<unsigned long long *>(counts), nt)
-  if (vpr <= 1) UGK_GO(1);
+#define UGK_GO(L)        \
+  do {                   \
+    if (half)            \
+      UGK_GO2(L, 32);    \
+    else                 \
+      UGK_GO2(L, kWave); \
+  } while (0)
+  if (vpr <= 1) UGK_GO2(1, kWave);
   else if (vpr <= 2) UGK_GO(2);
   else if (vpr <= 4) UGK_GO(4);
   else if (vpr <= 8) UGK_GO(8);
@@ -344,6 +360,7 @@ int extract_mix_lpr(ugk_table_t t, const K *keys, size_t n, const void *cache, u
   else if (vpr <= 32) UGK_GO(32);
   else UGK_GO(64);
 #undef UGK_GO
+#undef UGK_GO2
   UGK_HIP(hipGetLastError());
   return 0;
 }
@@ -351,7 +368,7 @@ int extract_mix_lpr(ugk_table_t t, const K *keys, size_t n, const void *cache, u
 template <typename K>
 int extract_mix(ugk_table_t t, const K *keys, size_t n, const void *cache, uint64_t cache_rows, const void *host,
                 uint64_t host_rows, void *out, size_t row_bytes, uint32_t *status, uint32_t *host_mirror,
-                uint64_t *counts, uint32_t *num_groups, void *stream) {
+                uint64_t *counts, uint32_t *num_groups, uint32_t others_hint, void *stream) {
   if (num_groups) *num_groups = 0;
   if (n == 0) return 0;
   UGK_REQUIRE(keys && out && status, "ugk_extract_mix: null keys, output or status");
@@ -371,9 +388,9 @@ int extract_mix(ugk_table_t t, const K *keys, size_t n, const void *cache, uint6
   const uint32_t vpr = (uint32_t)(row_bytes / 16);
   if (t.kind == 1)
     return extract_mix_lpr<K, 1>(t, keys, n, cache, cache_rows, host, host_rows, out, vpr, status, host_mirror,
-                                 counts, num_groups, as_stream(stream));
+                                 counts, num_groups, others_hint, as_stream(stream));
   return extract_mix_lpr<K, 2>(t, keys, n, cache, cache_rows, host, host_rows, out, vpr, status, host_mirror,
-                               counts, num_groups, as_stream(stream));
+                               counts, num_groups, others_hint, as_stream(stream));
 }
 
 template <typename K>
@@ -423,16 +440,16 @@ unsigned ugk_extract_mix_max_groups(void) { return clamp_grid(~(size_t)0, 0); }
 int ugk_extract_mix_u32(ugk_table_t t, const uint32_t *keys_dev, size_t n, const void *cache_dev, uint64_t cache_rows,
                         const void *host_dev, uint64_t host_rows, void *out_dev, size_t row_bytes,
                         uint32_t *status_dev, uint32_t *host_mirror, uint64_t *group_counts_host,
-                        uint32_t *num_groups_host, void *stream) {
+                        uint32_t *num_groups_host, uint32_t others_hint, void *stream) {
   return extract_mix<uint32_t>(t, keys_dev, n, cache_dev, cache_rows, host_dev, host_rows, out_dev, row_bytes,
-                               status_dev, host_mirror, group_counts_host, num_groups_host, stream);
+                               status_dev, host_mirror, group_counts_host, num_groups_host, others_hint, stream);
 }
 int ugk_extract_mix_i64(ugk_table_t t, const int64_t *keys_dev, size_t n, const void *cache_dev, uint64_t cache_rows,
                         const void *host_dev, uint64_t host_rows, void *out_dev, size_t row_bytes,
                         uint32_t *status_dev, uint32_t *host_mirror, uint64_t *group_counts_host,
-                        uint32_t *num_groups_host, void *stream) {
+                        uint32_t *num_groups_host, uint32_t others_hint, void *stream) {
   return extract_mix<int64_t>(t, keys_dev, n, cache_dev, cache_rows, host_dev, host_rows, out_dev, row_bytes,
-                              status_dev, host_mirror, group_counts_host, num_groups_host, stream);
+                              status_dev, host_mirror, group_counts_host, num_groups_host, others_hint, stream);
 }
 
 size_t ugk_dedup_workspace_bytes(size_t n) { return dedup_capacity(n) * 8 + ((n + 1) / 2 * 2) * 4 + 64; }

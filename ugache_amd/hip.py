@@ -17,6 +17,7 @@ ST_EVICT_ABSENT = 0x8
 LOC_LOCAL = 0
 LOC_HOST = 1
 EMPTY_U32 = 0xFFFFFFFF
+HINT_UNKNOWN = 0xFFFFFFFF
 
 TABLE_NONE = 0
 TABLE_FLAT = 1
@@ -87,8 +88,8 @@ SIGNATURES = {
     "ugk_classify_u32": [Table, _vp, _sz, _u64, _vp, _vp, _vp, _vp, _vp, _vp, _vp],
     "ugk_classify_i64": [Table, _vp, _sz, _u64, _vp, _vp, _vp, _vp, _vp, _vp, _vp],
     "ugk_extract_mix_max_groups": [],
-    "ugk_extract_mix_u32": [Table, _vp, _sz, _vp, _u64, _vp, _u64, _vp, _sz, _vp, _vp, _vp, _vp, _vp],
-    "ugk_extract_mix_i64": [Table, _vp, _sz, _vp, _u64, _vp, _u64, _vp, _sz, _vp, _vp, _vp, _vp, _vp],
+    "ugk_extract_mix_u32": [Table, _vp, _sz, _vp, _u64, _vp, _u64, _vp, _sz, _vp, _vp, _vp, _vp, _u32, _vp],
+    "ugk_extract_mix_i64": [Table, _vp, _sz, _vp, _u64, _vp, _u64, _vp, _sz, _vp, _vp, _vp, _vp, _u32, _vp],
     "ugk_dedup_workspace_bytes": [_sz],
     "ugk_dedup_u32": [_vp, _sz, _vp, _u32, _vp, _vp, _vp, _vp, _vp, _vp],
     "ugk_dedup_i64": [_vp, _sz, _vp, _u32, _vp, _vp, _vp, _vp, _vp, _vp],
