@@ -447,12 +447,18 @@ def run_mixed(args):
         # HBM side of the fused kernel: key + table entry per key, hit rows read and written, missed rows written
         hit_alg = n_keys * (8 + entry) + n_hit * 2 * row_bytes + n_miss * row_bytes
         t_link = t_hit
-        # 32 keys per wavefront for a small batch that nearly all hits a flat table, 64 otherwise (the library passes
-        # the last batch's share of rows from outside the cache on as a hint)
-        slots = hip.device_info(0)["compute_units"] * 4 * 8  # wavefronts resident at 8 per SIMD
-        kpw = 32 if info_cache["table_kind"] == 1 and n_miss * 50 <= n_keys and n_keys <= 32 * slots else 64
+        # keys per wavefront, by the launcher's rule: the fewest whose wavefronts are all resident at once (the hash
+        # probe wants one notch more; the top band of the flat table needs the library's hint of <= 2 % misses)
+        slots = hip.device_info(0)["compute_units"] * 4 * 8
+        lpr = min(64, max(1, 1 << (max(1, row_bytes // 16) - 1).bit_length()))
+        if info_cache["table_kind"] == 1:
+            kpw = 8 if n_keys <= slots * 8 else 16 if n_keys <= slots * 16 else \
+                32 if n_keys <= slots * 32 and n_miss * 50 <= n_keys else 64
+        else:
+            kpw = 16 if n_keys <= slots * 8 else 32 if n_keys <= slots * 16 else 64
+        kpw = max(kpw, 64 // lpr)
         kernel_name = ("extract_mix_kernel<long,%d,%d,%d> (lookup + both gathers; bound by the host link, see "
-                       "host_link)" % (info_cache["table_kind"], min(64, max(1, row_bytes // 16)), kpw))
+                       "host_link)" % (info_cache["table_kind"], lpr, kpw))
         stages = {"extract_mix": t_hit * 1e6}
     else:
         hit_alg = n_hit * (2 * row_bytes + 8)  # row read + row written + 8-byte index record

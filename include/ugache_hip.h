@@ -208,7 +208,7 @@ int ugk_classify_i64(ugk_table_t t, const int64_t *keys_dev, size_t n, uint64_t 
  * a key without a row (status_dev flagged) are counted with the host rows.  n must stay below 2^32.
  * others_hint: the caller's estimate of how many of the n rows will NOT come from the cache (the previous batch's
  * count scaled to n, say), UGK_HINT_UNKNOWN if it has none.  Only the launch shape depends on it (a small batch that
- * nearly all hits a flat table is given 32 instead of 64 keys per wavefront), never a byte of the result. */
+ * nearly all hits a flat table is cut into shorter wavefronts than one bound by the host link), never a byte of the result. */
 #define UGK_HINT_UNKNOWN 0xffffffffu
 unsigned ugk_extract_mix_max_groups(void);
 int ugk_extract_mix_u32(ugk_table_t t, const uint32_t *keys_dev, size_t n, const void *cache_dev, uint64_t cache_rows,

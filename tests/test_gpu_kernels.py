@@ -500,6 +500,48 @@ def test_outputs_beyond_4_GiB():
         mirror.free()
 
 
+@pytest.mark.parametrize("kind", ["flat", "hash"])
+@pytest.mark.parametrize("rb", [32, 128, 512, 2048])
+def test_extract_mix_at_every_launch_shape(kind, rb):
+    """the fused kernel cuts a batch into wavefronts of 8, 16, 32 or 64 keys by the batch size, the table kind, the row
+    size and the caller's hint; the bytes and the group sizes are the same at every shape"""
+    rng = np.random.default_rng(rb)
+    nkeys = 40_000
+    host = _rand_table(rng, nkeys, rb)
+    cached = rng.choice(nkeys, nkeys * 3 // 4, replace=False).astype(np.int64)
+    slots = rng.permutation(len(cached)).astype(np.uint32)
+    cache = np.zeros((len(cached), rb), np.uint8)
+    cache[slots] = host[cached]
+    if kind == "flat":
+        mem, tb = _make_flat(nkeys)
+    else:
+        mem, tb, _ = _make_hash(len(cached))
+    assert _insert(tb, cached, slots) == 0
+    is_cached = np.zeros(nkeys, bool)
+    is_cached[cached] = True
+    pin = pinned_from(host)
+    mirror = pinned_from(np.zeros(4, np.uint32))
+    try:
+        st = dev_zeros_u32(1)
+        d_cache = to_dev(cache)
+        for n in (1, 63, 5_000, 70_000, 140_000, 270_000):
+            keys = rng.integers(0, nkeys, size=n).astype(np.int64)
+            d_keys = to_dev(keys)
+            want = host[keys].tobytes()
+            n_local = int(is_cached[keys].sum())
+            for hint in (hip.HINT_UNKNOWN, 0):
+                out = dev_bytes(n * rb, fill=0x3C)
+                sizes = _extract_mix("ugk_extract_mix_i64", tb, d_keys, n, d_cache, len(cached), pin, nkeys, out, rb, st,
+                                     mirror, hint)
+                assert status_value(st) == 0
+                assert sizes == [n_local, n - n_local], (n, hint)
+                assert to_np(out)[: n * rb].tobytes() == want, (n, hint)
+    finally:
+        sync()
+        pin.free()
+        mirror.free()
+
+
 def test_classify_rejects_keys_beyond_the_host_table():
     mem, tb = _make_flat(100)
     keys = np.array([5, 100, 7, 1 << 33], np.int64)

@@ -331,26 +331,56 @@ int extract_mix_lpr(ugk_table_t t, const K *keys, size_t n, const void *cache, u
     return e ? atoi(e) : -1;
   }();
   const bool nt = forced_nt >= 0 ? forced_nt != 0 : n * (size_t)vpr * 16 > ((size_t)192 << 20);
-  // Keys per wavefront.  64 fill every lane of the lookup.  A batch that nearly all comes from the cache is bound by
-  // HBM, and a small one then leaves half the wavefront slots of the chip empty: 32 keys per wavefront double the
-  // wavefronts with rows in flight (262,144 keys, 99 % hits, flat table: 55 -> 51 us).  Batches bound by the host link
-  // run 1-2 % slower that way, and the hash table's probe wants all 64 lanes (68 -> 74 us), so both keep 64.
-  const size_t slots = (size_t)cu_count() * 4 * 8;  // wavefronts resident at 8 per SIMD
-  const bool half = KIND == 1 && vpr > 1 && others_hint != UGK_HINT_UNKNOWN && (size_t)others_hint * 50 <= n &&
-                    (n + 31) / 32 <= slots;
-  const size_t keys_per_group = half ? kBlock / 2 : kBlock;
+  // Keys per wavefront.  A wavefront copies its rows a few at a time, one round trip to memory per round, so a batch
+  // that leaves wavefront slots of the chip empty finishes sooner when it is cut into more, shorter wavefronts: the
+  // fewest keys per wavefront whose wavefronts are all resident at once (8 per SIMD).  Measured on 512-byte rows at
+  // 1 % misses, flat table, 64 / 32 / 16 / 8 keys per wavefront: 8,192 keys 16.0 / 11.6 / 7.1 / 6.3 us, 65,536 keys
+  // 31.6 / 21.4 / 17.0 / 16.1 us, 131,072 keys 37.6 / 29.9 / 29.6 / 30.2 us, 262,144 keys 54.2 / 49.6 / 51.1 / 51.7 us,
+  // 524,288 keys 90.5 / 93.1 / 94.4 / 95.5 us.  The hash table's probe works on all 64 lanes at once and wants one
+  // notch more (65,536 keys 44.8 / 33.0 / 26.7 / 30.5 us, 262,144 keys 66.7 / 71.5 / 75.6 / 80.1 us).  In the top band
+  // of the flat table a batch bound by the host link runs 1-2 % slower with 32 than with 64, so 32 is taken there only
+  // when the caller expects at most 2 % of the rows from outside the cache.
+  const size_t slots = (size_t)cu_count() * 4 * 8;
+  const bool few_others = others_hint != UGK_HINT_UNKNOWN && (size_t)others_hint * 50 <= n;
+  int kpw = kWave;
+  if (KIND == 1) {
+    if (n <= slots * 8) kpw = 8;
+    else if (n <= slots * 16) kpw = 16;
+    else if (n <= slots * 32 && few_others) kpw = 32;
+  } else {
+    if (n <= slots * 8) kpw = 16;
+    else if (n <= slots * 16) kpw = 32;
+  }
+  const int lpr = vpr <= 1 ? 1 : vpr <= 2 ? 2 : vpr <= 4 ? 4 : vpr <= 8 ? 8 : vpr <= 16 ? 16 : vpr <= 32 ? 32 : 64;
+  if (kpw < kWave / lpr) kpw = kWave / lpr;  // one wavefront instruction copies 64 / lpr rows
+  const size_t keys_per_group = (size_t)kpw * kWavesPerBlock;
   const unsigned grid = clamp_grid((n + keys_per_group - 1) / keys_per_group, 0);
   if (num_groups) *num_groups = grid;
 #define UGK_GO2(L, W)                                                                                              \
   hipLaunchKernelGGL((extract_mix_kernel<K, KIND, L, W>), dim3(grid), dim3(kBlock), 0, st, t, keys, n,            \
                      (const u32x4 *)cache, cache_rows, (const u32x4 *)host, host_rows, (u32x4 *)out, vpr, status, \
                      host_mirror, reinterpret_cast<unsigned long long *>(counts), nt)
-#define UGK_GO(L)        \
-  do {                   \
-    if (half)            \
-      UGK_GO2(L, 32);    \
-    else                 \
-      UGK_GO2(L, kWave); \
+#define UGK_GO(L)                                   \
+  do {                                              \
+    if constexpr (kWave / L <= 8) {                 \
+      if (kpw == 8) {                               \
+        UGK_GO2(L, 8);                              \
+        break;                                      \
+      }                                             \
+    }                                               \
+    if constexpr (kWave / L <= 16) {                \
+      if (kpw == 16) {                              \
+        UGK_GO2(L, 16);                             \
+        break;                                      \
+      }                                             \
+    }                                               \
+    if constexpr (kWave / L <= 32) {                \
+      if (kpw == 32) {                              \
+        UGK_GO2(L, 32);                             \
+        break;                                      \
+      }                                             \
+    }                                               \
+    UGK_GO2(L, kWave);                              \
   } while (0)
   if (vpr <= 1) UGK_GO2(1, kWave);
   else if (vpr <= 2) UGK_GO(2);
