@@ -83,7 +83,9 @@ typedef struct {
 } ugk_device_info_t;
 
 const char *ugk_last_error(void);
-/* version of this ABI; bumped on any signature change */
+/* version of this ABI; bumped on any signature change.  ugk_abi_version() is what the loaded library was built with:
+ * a caller compiled against another UGK_ABI_VERSION must not go on. */
+#define UGK_ABI_VERSION 3
 int ugk_abi_version(void);
 
 /* ---- runtime plumbing: Device::{AllocDataSpace,FreeDataSpace,CopyDataFromTo,StreamSync,CreateStream}

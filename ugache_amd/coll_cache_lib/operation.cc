@@ -64,6 +64,7 @@ std::function<MemHandle(size_t)> MakeAllocator(coll_cache_alloc_fn alloc, coll_c
 void coll_cache_config_from_map(std::unordered_map<std::string, std::string> &configs) {
   using CRC = RunConfig;
   CHECK(!CRC::is_configured);
+  CHECK_EQ(ugk_abi_version(), UGK_ABI_VERSION) << "libugache_hip.so and libcoll_cache.so come from different builds";
   CHECK(configs.count("cache_percentage"));
   CHECK(configs.count("_cache_policy"));
   CHECK(configs.count("num_device"));

@@ -79,7 +79,7 @@ using namespace ugk;
 extern "C" {
 
 const char *ugk_last_error(void) { return g_err; }
-int ugk_abi_version(void) { return 3; }
+int ugk_abi_version(void) { return UGK_ABI_VERSION; }
 
 int ugk_device_count(int *count) {
   UGK_REQUIRE(count, "ugk_device_count: null output");
