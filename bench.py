@@ -135,6 +135,12 @@ def stream_ordered_leg(C, fn, key_ptr_of, n_keys, out, stream, torch, W, K):
     return wall, ms.value * 1e-3 / K
 
 
+# what the library's own per-step time is: a device event pair around the launch (COLL_KERNEL_EVENTS=1), or a host
+# timer around launch and wait (default, as in the reference)
+PER_CALL_KEY = {True: "avg_kernel_us_event_pair_per_blocking_launch",
+                False: "launch_to_completion_us_host_timer_per_blocking_call"}
+
+
 def step_spread(t0, stamps):
     """median and 95th percentile of the wall time of the blocking calls of a timed region, in milliseconds"""
     import numpy as np
@@ -251,9 +257,9 @@ def run_all_hit(args):
 
     # dominant kernel: average launch duration over a timed region of K launches, from two HIP events on the kernel's
     # stream around the K back-to-back launches of the stream-ordered leg (nothing else runs on that stream between
-    # them).  The library also brackets every blocking launch with an event pair of its own (logged per step as
-    # kLogL3CacheCombineCacheTime); that figure carries about 2.4 us of marker latency per launch and is reported
-    # beside it.
+    # them).  The library logs a time of its own for every blocking call (kLogL3CacheCombineCacheTime), reported
+    # beside it: from a host timer around launch and wait, like the reference's, or with COLL_KERNEL_EVENTS=1 from a
+    # device event pair around the launch (about 2.4 us of marker latency in the figure, 1.9 us added to the step).
     kernel_avg_s = so_launch_s
     per_launch_pair_s = float(np.mean([_basics.step_value(s, kLogL3CacheCombineCacheTime) for s in range(W, W + K)]))
     alg_bytes = n_keys * (2 * row_bytes + 4)  # row read + row written + key read, per key
@@ -282,7 +288,7 @@ def run_all_hit(args):
                      "kernel": "gather_kernel<u32x4,32,2,DirectU32>", "algorithmic_bytes_per_launch": alg_bytes,
                      "avg_kernel_us": kernel_avg_s * 1e6, "keys_per_s_kernel_only": n_keys / kernel_avg_s,
                      "timing": "2 HIP events around %d back-to-back launches on the kernel's stream" % K,
-                     "avg_kernel_us_event_pair_per_blocking_launch": per_launch_pair_s * 1e6},
+                     PER_CALL_KEY[os.environ.get("COLL_KERNEL_EVENTS", "0") != "0"]: per_launch_pair_s * 1e6},
         "cpu_baseline": {"value": cpu_kps, "unit": "keys/s", "cores": cores, "kind": "port",
                          "sample": "%d batches of %d keys from the same pool, %.1f s, OpenMP gather over keys"
                                    % (n_cpu, n_keys, cpu_el),
@@ -327,6 +333,7 @@ def run_mixed(args):
         os.environ["SAMGRAPH_COLL_CACHE_CONCURRENT_LINK_IMPL"] = args.impl
     if args.dedup:
         os.environ["COLL_DEDUP_KEYS"] = "1"
+        os.environ.setdefault("COLL_KERNEL_EVENTS", "1")  # the extraction after the dedup timed on the device
     if args.device_refresh:
         args.gpu_record = True
         os.environ["COLL_GPU_REFRESH"] = "1"
@@ -606,7 +613,7 @@ def run_mixed(args):
                      "traffic": MEASURED_TRAFFIC_BYTES.get(args.workload) if fused else None,
                      "kernel": kernel_name,
                      "algorithmic_bytes_per_launch": hit_alg, "avg_kernel_us": t_hit * 1e6,
-                     "avg_kernel_us_event_pair_per_blocking_launch": per_launch_pair_us},
+                     PER_CALL_KEY[os.environ.get("COLL_KERNEL_EVENTS", "0") != "0"]: per_launch_pair_us},
         "host_link": {"achieved": miss_bytes / t_link / 1e9 if t_link > 0 else 0.0, "measured_peak": link_gbps,
                       "unit": "GB/s", "frac": (miss_bytes / t_link / 1e9) / link_gbps if t_link > 0 else 0.0,
                       "miss_rows_per_batch": n_miss, "peak_probe": "pinned host -> HBM hipMemcpyAsync, best of 3"},

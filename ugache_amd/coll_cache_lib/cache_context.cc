@@ -535,9 +535,13 @@ void ExtractSession::ExtractFeatImpl(const KeyT *nodes, size_t num_nodes, void *
     // with the host-link budget.
     CHECK_EQ(ctx->_num_location, 1);
     const bool from_host = ctx->_cpu_location_id != -1;
-    // the gather is bracketed by events on its own stream: the logged combine time is the kernel's duration
+    // the logged combine time: a host timer around launch and wait, as in the reference (Timer around Combine + StreamSync,
+    // cache_context.cu:1206-1216, 1312-1315), or with COLL_KERNEL_EVENTS=1 the kernel's duration from an event pair on its
+    // stream, which costs 1.9 us per step
     void *keys_ready = RecordBegin(stream);
-    UGK_CALL(ugk_event_record(_ev_t[0], stream));
+    const bool events = RunConfig::kernel_events;
+    Timer t_host;
+    if (events) UGK_CALL(ugk_event_record(_ev_t[0], stream));
     if (dst_map == nullptr) {
       UGK_CALL(GatherDirect(ctx->_device_cache_data[0], ctx->_num_total_nodes, nodes, num_nodes, output, rb,
                             from_host ? _cpu_blocks : 0, _status, _host_mirror, stream));
@@ -545,15 +549,16 @@ void ExtractSession::ExtractFeatImpl(const KeyT *nodes, size_t num_nodes, void *
       UGK_CALL(GatherScatter(ctx->_device_cache_data[0], ctx->_num_total_nodes, nodes, dst_map, num_nodes, output,
                              num_input, rb, from_host ? _cpu_blocks : 0, _status, _host_mirror, stream));
     }
-    UGK_CALL(ugk_event_record(_ev_t[1], stream));
+    if (events) UGK_CALL(ugk_event_record(_ev_t[1], stream));
     RecordLaunch(input_nodes, num_input, keys_ready);
     if (dst_map) UGK_CALL(ugk_replicate_rows(output, rb, inverse, dst_map, num_input, stream));
     UGK_CALL(ugk_stream_sync(stream));
+    const double host_time = t_host.Passed();
     JoinRecordOnHost();
     CheckStatusWord(stream);
     float combine_ms = 0;
-    UGK_CALL(ugk_event_elapsed_ms(_ev_t[0], _ev_t[1], &combine_ms));
-    const double combine_time = combine_ms * 1e-3;
+    if (events) UGK_CALL(ugk_event_elapsed_ms(_ev_t[0], _ev_t[1], &combine_ms));
+    const double combine_time = events ? combine_ms * 1e-3 : host_time;
     _group_offset[1] = from_host ? 0 : (uint32_t)num_nodes;
     _group_offset[2] = (uint32_t)num_nodes;
     if (profiler && task_key != 0xffffffffffffffffull) {
@@ -586,21 +591,24 @@ void ExtractSession::ExtractFeatImpl(const KeyT *nodes, size_t num_nodes, void *
     // it, and since the link bounds a mixed batch it does not matter that host loads spread over the chip slow the
     // HBM loads next to them.
     void *keys_ready = RecordBegin(stream);
-    UGK_CALL(ugk_event_record(_ev_t[0], stream));
+    const bool events = RunConfig::kernel_events;
+    Timer t_host;
+    if (events) UGK_CALL(ugk_event_record(_ev_t[0], stream));
     UGK_CALL(ExtractMix(table, nodes, num_nodes, cache, cache_rows, host, host_rows, output, rb, _status,
                         _host_mirror, _mix_counts->ptr<uint64_t>(), &_mix_groups, MixOthersHint(num_nodes),
                         stream));
-    UGK_CALL(ugk_event_record(_ev_t[1], stream));
+    if (events) UGK_CALL(ugk_event_record(_ev_t[1], stream));
     RecordLaunch(input_nodes, num_input, keys_ready);
     UGK_CALL(ugk_stream_sync(stream));
+    const double host_time = t_host.Passed();
     JoinRecordOnHost();
     CheckStatusWord(stream);
     SumMixCounts();
     const uint32_t n_local = _host_mirror[kMirGroupSizes + UGK_LOC_LOCAL],
                    n_miss = _host_mirror[kMirGroupSizes + UGK_LOC_HOST];
     CHECK_EQ((size_t)n_local + n_miss, num_nodes);
-    float mix_ms = 0;
-    UGK_CALL(ugk_event_elapsed_ms(_ev_t[0], _ev_t[1], &mix_ms));
+    float mix_ms = (float)(host_time * 1e3);
+    if (events) UGK_CALL(ugk_event_elapsed_ms(_ev_t[0], _ev_t[1], &mix_ms));
     _group_offset[1] = n_local;
     _group_offset[2] = (uint32_t)num_nodes;
     if (profiler && task_key != 0xffffffffffffffffull) {

@@ -71,6 +71,7 @@ struct RunConfig {
   // COLL_GPU_REFRESH_KEEP=1: such a refresh leaves the counters as they are (hotness accumulates over refreshes)
   // instead of starting the next interval from zero
   static bool gpu_refresh_keep;
+  static bool kernel_events;  // COLL_KERNEL_EVENTS: per-step kernel times from device events (1) or a host timer (0)
   static bool dedup_keys;        // COLL_DEDUP_KEYS=1: extract each distinct key of a batch once, then copy the duplicates
   static size_t dedup_min_keys;  // COLL_DEDUP_MIN_KEYS, default 4096: shorter batches skip the deduplication
   static double hash_rebuild_tombstone_frac;  // COLL_HASH_REBUILD_FRAC, default 0.15: rebuild the table after refresh
