@@ -651,6 +651,42 @@ def test_dedup_matches_numpy_unique(kdtype, n):
         assert np.array_equal(keys[r], u) and np.array_equal(i[r], np.arange(k))  # representatives
 
 
+@pytest.mark.parametrize("kdtype", [np.uint32, np.int64])
+@pytest.mark.parametrize("n", [1000, 70_000, 300_000])
+@pytest.mark.parametrize("shape", ["one_key", "two_keys", "geometric", "hot_and_cold"])
+def test_dedup_of_skewed_keys(kdtype, n, shape):
+    """batches whose duplicates meet inside a tile: the occurrences of a key elect one leader in LDS, and only leaders
+    reach the device-wide set"""
+    rng = np.random.default_rng(n + len(shape))
+    space = (1 << 31) if kdtype == np.uint32 else (1 << 40)
+    if shape == "one_key":
+        keys = np.full(n, 12345 % space)
+    elif shape == "two_keys":
+        keys = np.where(rng.random(n) < 0.5, 7, space - 1)
+    elif shape == "geometric":
+        keys = (rng.geometric(0.01, size=n) * 2654435761) % space
+    else:  # a tenth of the batch is one hot key, the rest are distinct
+        keys = rng.choice(space, size=n, replace=False) if space > 10 * n else rng.integers(0, space, size=n)
+        keys[rng.random(n) < 0.1] = 99
+    keys = keys.astype(kdtype)
+    ws = dev_bytes(hip.lib().ugk_dedup_workspace_bytes(n), fill=0)
+    d_keys = to_dev(keys)
+    for epoch in (1, 2):
+        uniq = dev_bytes(n * np.dtype(kdtype).itemsize)
+        inv, nu, rep = dev_zeros_u32(n), dev_zeros_u32(1), dev_zeros_u32(n)
+        fn = "ugk_dedup_i64" if kdtype == np.int64 else "ugk_dedup_u32"
+        hip.call(fn, ptr(d_keys), n, ptr(ws), epoch, ptr(uniq), ptr(inv), ptr(rep), ptr(nu), None, None)
+        sync()
+        k = int(to_np(nu, np.uint32)[0])
+        u = to_np(uniq, kdtype)[:k]
+        i = to_np(inv, np.uint32)[:n]
+        assert k == len(np.unique(keys))
+        assert np.array_equal(np.sort(u), np.unique(keys))
+        assert i.max() < k and np.array_equal(u[i], keys)
+        r = to_np(rep, np.uint32)[:k]
+        assert np.array_equal(keys[r], u) and np.array_equal(i[r], np.arange(k))
+
+
 def test_classify_with_destination_map():
     """dst_map redirects the output row of key i; sources and group sizes are unchanged"""
     rng = np.random.default_rng(31)
