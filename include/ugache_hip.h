@@ -85,7 +85,7 @@ typedef struct {
 const char *ugk_last_error(void);
 /* version of this ABI; bumped on any signature change.  ugk_abi_version() is what the loaded library was built with:
  * a caller compiled against another UGK_ABI_VERSION must not go on. */
-#define UGK_ABI_VERSION 3
+#define UGK_ABI_VERSION 4
 int ugk_abi_version(void);
 
 /* ---- runtime plumbing: Device::{AllocDataSpace,FreeDataSpace,CopyDataFromTo,StreamSync,CreateStream}
@@ -225,18 +225,19 @@ int ugk_extract_mix_i64(ugk_table_t t, const int64_t *keys_dev, size_t n, const 
 /* ---- key dedup (the caller-side array_ops.unique of
  *      python_tf2/collcache_tf2/collcache_tf2/core/sparse_lookup_layer.py:197) ------------------------
  * unique_out[0..*n_unique) = distinct keys (order unspecified), inverse_out[i] = position of keys[i] in it.
- * workspace_dev: ugk_dedup_workspace_bytes(n) bytes, zero-filled once at allocation and then reused as is
- * (slots are epoch-tagged, so no per-call clearing); epoch must be non-zero and different on every call
- * that shares the workspace.  n_unique_dev must be zero on entry.
+ * workspace_dev: workspace_bytes >= ugk_dedup_workspace_bytes(n) bytes, zero-filled once at allocation and then
+ * reused as is by batches of any size up to the one it was sized for (slots are epoch-tagged, so no per-call
+ * clearing; the layout inside depends on workspace_bytes only, which must therefore be the same on every call that
+ * shares the workspace); epoch must be non-zero and different on every such call.  n_unique_dev must be zero on entry.
  * rep_out_dev (may be NULL): rep_out_dev[u] = index of the first occurrence that introduced unique key u.
  * n_unique_host (may be NULL): pinned host word that receives *n_unique_dev when the second kernel runs. */
 size_t ugk_dedup_workspace_bytes(size_t n);
-int ugk_dedup_u32(const uint32_t *keys_dev, size_t n, void *workspace_dev, uint32_t epoch, uint32_t *unique_out_dev,
-                  uint32_t *inverse_out_dev, uint32_t *rep_out_dev, uint32_t *n_unique_dev, uint32_t *n_unique_host,
-                  void *stream);
-int ugk_dedup_i64(const int64_t *keys_dev, size_t n, void *workspace_dev, uint32_t epoch, int64_t *unique_out_dev,
-                  uint32_t *inverse_out_dev, uint32_t *rep_out_dev, uint32_t *n_unique_dev, uint32_t *n_unique_host,
-                  void *stream);
+int ugk_dedup_u32(const uint32_t *keys_dev, size_t n, void *workspace_dev, size_t workspace_bytes, uint32_t epoch,
+                  uint32_t *unique_out_dev, uint32_t *inverse_out_dev, uint32_t *rep_out_dev, uint32_t *n_unique_dev,
+                  uint32_t *n_unique_host, void *stream);
+int ugk_dedup_i64(const int64_t *keys_dev, size_t n, void *workspace_dev, size_t workspace_bytes, uint32_t epoch,
+                  int64_t *unique_out_dev, uint32_t *inverse_out_dev, uint32_t *rep_out_dev, uint32_t *n_unique_dev,
+                  uint32_t *n_unique_host, void *stream);
 
 /* ---- hotness counters on the device: FreqRecorder::Record (freq_recorder.cc:227-253) without the copy of the keys
  *      to the host, the record thread of python_tf2/collcache_tf2/collcache_tf2/core/lookup_manager.cc:291-312 ----

@@ -1183,3 +1183,253 @@ def test_lookup_of_the_distinct_keys_with_inverse(pct, table_kind, kdtype, monke
     out = co.coll_torch_lookup_key_t_val_ret(0, torch.from_numpy(keys).to(kdtype).cuda(), False)
     assert out.cpu().numpy().tobytes() == ORC.gather(table, keys).tobytes()
     assert _basics.last_group_offset(0)[2] == len(keys)
+
+
+# ---- the GNN-shaped and the DLR-shaped configuration ---------------------------------------------------------------
+def zipf_ranks_dev(n, space, s, gen):
+    """zipf_ranks on the device (same inverse CDF), for batches of a million keys and more"""
+    u = torch.rand(n, generator=gen, device="cuda", dtype=torch.float64)
+    h = float(space)
+    r = torch.floor(((h ** (1.0 - s) - 1.0) * u + 1.0) ** (1.0 / (1.0 - s))).to(torch.int64) - 1
+    return r.clamp_(0, space - 1)
+
+
+_GNN_CASES = {}
+
+
+def _gnn_case(n_item, n_keys, presample):
+    """seeded GNN-shaped key stream: Zipf(0.9) ranks over a seeded permutation of the row ids; the presampled batches,
+    the oracle's placement for them and a few lookup batches (the oracle's ranking of a 100M-row key space takes half a
+    minute, so a case is computed once per size)"""
+    key = (n_item, n_keys, presample)
+    if key not in _GNN_CASES:
+        _GNN_CASES.clear()  # one case at a time: the full-size one holds gigabytes
+        gp = torch.Generator(device="cuda").manual_seed(2)
+        perm = torch.randperm(n_item, generator=gp, device="cuda", dtype=torch.int64)
+        gz = torch.Generator(device="cuda").manual_seed(3)
+        pre = [perm[zipf_ranks_dev(n_keys, n_item, 0.9, gz)].cpu() for _ in range(presample)]
+        sizes = (n_keys, n_keys, n_keys // 3 + 5, 65_536, n_keys)
+        batches = [perm[zipf_ranks_dev(n, n_item, 0.9, gz)] for n in sizes]
+        stream = torch.cat(pre).numpy().astype(np.uint32)
+        _, nid = expected_cached_set(stream, n_item, 0.25)
+        del stream, perm
+        _GNN_CASES[key] = (pre, batches, nid)
+    return _GNN_CASES[key]
+
+
+@pytest.mark.parametrize("impl", ["", "SMMaskPhase"])
+@pytest.mark.parametrize("dedup", [False, True])
+def test_config3_gnn_quarter_cached_zipf_keys_with_dedup(impl, dedup, monkeypatch):
+    """The GNN-feature-shaped configuration at 16M rows (the oracle covers that in seconds): 128 fp32 per row in pinned
+    host memory, the top 25 % of the rows by the hotness of 50 presampled batches cached, batches of 2^20 int64 keys
+    Zipf(0.9) of which nearly half are duplicates; fused and factored extraction, with and without COLL_DEDUP_KEYS.
+    Output bytes, cached set and group sizes against the oracle, for batches of several sizes."""
+    if impl:
+        monkeypatch.setenv("SAMGRAPH_COLL_CACHE_CONCURRENT_LINK_IMPL", impl)
+    if dedup:
+        monkeypatch.setenv("COLL_DEDUP_KEYS", "1")
+    n_item, dim, pct, n_keys = 16_000_000, 128, 0.25, 1 << 20
+    pre, batches, nid = _gnn_case(n_item, n_keys, 50)
+    co.config(make_config(n_item, pct))
+    co.coll_cache_record_init(0)
+    for b in pre:
+        co.coll_torch_record(0, b)
+    emb = co.coll_torch_create_emb_shm(0, n_item, dim, torch.float32)
+    g = torch.Generator(device="cuda").manual_seed(1)
+    for r0 in range(0, n_item, 2_000_000):
+        emb[r0 : r0 + 2_000_000].copy_(torch.randn((2_000_000, dim), generator=g, device="cuda"))
+    table = emb.numpy()
+    co.coll_torch_init_t(0, 0, emb, pct)
+    info = _basics.info(0)
+    assert info["table_kind"] == 1 and info["cached_rows"] == n_item // 4 == int((nid == 0).sum())
+    assert info["capacity_rows"] == ORC.lib.orc_cache_capacity(n_item, pct)
+    got_cached = np.zeros(info["cached_rows"], np.uint32)
+    assert _basics.C_LIB_CTYPES.coll_cache_get_cached_keys(0, got_cached.ctypes.data, len(got_cached)) == len(got_cached)
+    assert np.array_equal(got_cached, np.nonzero(nid == 0)[0])
+    for kt in batches:
+        keys = kt.cpu().numpy()
+        n = len(keys)
+        uniq = np.unique(keys)
+        if n == n_keys:
+            assert 0.35 < 1 - len(uniq) / n < 0.55  # the configuration's "about 40 % duplicates"
+        out = co.coll_torch_lookup_key_t_val_ret(0, kt, False)
+        assert out.shape == (n, dim)
+        assert out.cpu().numpy().tobytes() == ORC.gather(table, keys, omp=True).tobytes()
+        counted = uniq if dedup else keys
+        assert _basics.last_group_offset(0) == [0, int((nid[counted] == 0).sum()), len(counted)]
+    # the distinct keys and their inverse instead of the re-expanded rows
+    rows, inverse = co.coll_torch_lookup_unique(0, batches[0])
+    keys = batches[0].cpu().numpy()
+    assert rows.shape[0] == len(np.unique(keys))
+    assert torch.equal(rows[inverse.long()].view(torch.int32), emb.cuda()[batches[0]].view(torch.int32))
+
+
+@pytest.mark.parametrize("impl,dedup", [("", False), ("SMMaskPhase", True)])
+def test_config3_gnn_full_size_closed_form(impl, dedup, monkeypatch):
+    """The same configuration at its full size: 100M rows x 128 fp32 = 51.2 GB pinned, 25M rows (12.8 GB) cached, 2^20
+    int64 keys per batch.  table[r, c] = (128 r + c) mod 2^32 as int32 bits, so every output word is checked on the
+    device without a second copy of the rows; cached set and group sizes against the oracle's placement."""
+    if impl:
+        monkeypatch.setenv("SAMGRAPH_COLL_CACHE_CONCURRENT_LINK_IMPL", impl)
+    if dedup:
+        monkeypatch.setenv("COLL_DEDUP_KEYS", "1")
+    n_item, dim, pct, n_keys = 100_000_000, 128, 0.25, 1 << 20
+    pre, batches, nid = _gnn_case(n_item, n_keys, 50)
+    co.config(make_config(n_item, pct, threads=16))
+    co.coll_cache_record_init(0)
+    for b in pre:
+        co.coll_torch_record(0, b)
+    emb = co.coll_torch_create_emb_shm(0, n_item, dim, torch.float32)
+    words = emb.view(torch.int32)
+    col = torch.arange(dim, device="cuda", dtype=torch.int64)
+    for r0 in range(0, n_item, 4_000_000):
+        r = torch.arange(r0, min(n_item, r0 + 4_000_000), device="cuda", dtype=torch.int64)
+        words[r0 : r0 + len(r)].copy_(((r.unsqueeze(1) * dim + col) & 0xffffffff).to(torch.int32))
+    co.coll_torch_init_t(0, 0, emb, pct)
+    info = _basics.info(0)
+    assert info["table_kind"] == 1 and info["cached_rows"] == 25_000_000 == int((nid == 0).sum())
+    assert info["capacity_rows"] == ORC.lib.orc_cache_capacity(n_item, pct)
+    got_cached = np.zeros(info["cached_rows"], np.uint32)
+    assert _basics.C_LIB_CTYPES.coll_cache_get_cached_keys(0, got_cached.ctypes.data, len(got_cached)) == len(got_cached)
+    assert np.array_equal(got_cached, np.nonzero(nid == 0)[0])
+    for kt in batches:
+        n = len(kt)
+        out = co.coll_torch_lookup_key_t_val_ret(0, kt, False)
+        assert out.shape == (n, dim)
+        want = ((kt.unsqueeze(1) * dim + col) & 0xffffffff).to(torch.int32)
+        assert torch.equal(out.view(torch.int32), want)
+        keys = kt.cpu().numpy()
+        counted = np.unique(keys) if dedup else keys
+        if n == n_keys:
+            assert 0.3 < 1 - len(np.unique(keys)) / n < 0.45
+        assert _basics.last_group_offset(0) == [0, int((nid[counted] == 0).sum()), len(counted)]
+
+
+@pytest.mark.parametrize("impl", ["", "SMMaskPhase"])
+def test_config4_dlr_26_fields_through_the_lookup_layer(impl, tmp_path, monkeypatch):
+    """The DLR-shaped configuration with 262,144 rows per field (26 x 8M rows = 106 GB cannot be pinned on one box):
+    26 tables of 128 fp32 concatenated into one id space, key = f * rows_per_field + perm_f[rank] with an independent
+    seeded permutation and Zipf(1.2) ranks per field, the hottest 35.8 % of the id space cached (the configuration's 40 GB of
+    106 GB), batches of 8192 samples x 26 fields as an int64 [8192, 26] tensor through the serving stack's LookupLayer,
+    which returns [8192, 26, 128]."""
+    import json
+    import collcache.torch.serving as hps
+    if impl:
+        monkeypatch.setenv("SAMGRAPH_COLL_CACHE_CONCURRENT_LINK_IMPL", impl)
+    fields, per_field, dim, samples = 26, 262_144, 128, 8192
+    n_item = fields * per_field
+    pct = (40e9 / 512) / (26 * 8_388_608)
+    cfg = {"iteration_per_epoch": 200, "epoch": 1, "coll_cache_enable_refresh": False,
+           "models": [{"model": "dlrm", "sparse_files": ["mock_%d_%d" % (n_item, dim)], "gpucacheper": pct,
+                       "max_batch_size": samples, "deployed_device_list": [0],
+                       "maxnum_catfeature_query_per_table_per_sample": [fields], "embedding_vecsize_per_table": [dim],
+                       "max_vocabulary_size": [n_item]}]}
+    path = tmp_path / "ps_config.json"
+    path.write_text(json.dumps(cfg))
+    gp = torch.Generator(device="cuda").manual_seed(2)
+    perms = [torch.randperm(per_field, generator=gp, device="cuda", dtype=torch.int64) for _ in range(fields)]
+    gz = torch.Generator(device="cuda").manual_seed(3)
+
+    def make_batch(n_samples):
+        cols = [perms[f][zipf_ranks_dev(n_samples, per_field, 1.2, gz)] + f * per_field for f in range(fields)]
+        return torch.stack(cols, dim=1)  # [samples, fields]
+
+    try:
+        assert hps.Config(ps_config_file=str(path)) == "OK"
+        pre = [make_batch(samples) for _ in range(100)]
+        for b in pre:
+            hps.record_hotness(b)
+        emb = co.coll_torch_create_emb_shm(0, n_item, dim, torch.float32)
+        g = torch.Generator(device="cuda").manual_seed(1)
+        for r0 in range(0, n_item, per_field * 2):
+            emb[r0 : r0 + per_field * 2].copy_(torch.randn((per_field * 2, dim), generator=g, device="cuda"))
+        table = emb.numpy()
+        assert hps.Init(ps_config_file=str(path), global_batch_size=samples, emb_table=emb) == "OK"
+        stream = torch.cat([b.reshape(-1) for b in pre]).cpu().numpy().astype(np.uint32)
+        want_cached, nid = expected_cached_set(stream, n_item, pct)
+        info = _basics.info(0)
+        assert info["cached_rows"] == len(want_cached) == int(n_item * (pct * 100 / 100.0))
+        got_cached = np.zeros(len(want_cached), np.uint32)
+        assert _basics.C_LIB_CTYPES.coll_cache_get_cached_keys(0, got_cached.ctypes.data, len(got_cached)) == len(want_cached)
+        assert np.array_equal(got_cached, want_cached)
+        layer = hps.LookupLayer(model_name="dlrm", table_id=0, emb_vec_size=dim, emb_vec_dtype=torch.float32)
+        for n_samples in (samples, samples, 1000, 1, samples):
+            keys = make_batch(n_samples)
+            assert keys.shape == (n_samples, fields) and keys.dtype == torch.int64
+            out = layer(keys)
+            assert tuple(out.shape) == (n_samples, fields, dim) and out.dtype == torch.float32
+            flat = keys.reshape(-1).cpu().numpy()
+            # every field's keys stay inside that field's table
+            assert np.array_equal(flat.reshape(n_samples, fields) // per_field, np.tile(np.arange(fields), (n_samples, 1)))
+            assert out.cpu().numpy().tobytes() == ORC.gather(table, flat, omp=True).tobytes()
+            assert _basics.last_group_offset(0) == [0, int((nid[flat] == 0).sum()), len(flat)]
+    finally:
+        hps.Shutdown()
+
+
+@pytest.mark.parametrize("table_kind", ["FLAT", "HASH"])
+@pytest.mark.parametrize("impl", ["", "SMMaskPhase"])
+def test_refresh_on_one_stream_while_lookups_run_on_another(table_kind, impl, monkeypatch):
+    """Stream-ordered lookups are enqueued on a stream of the caller's while a second thread refreshes the cache, in
+    background mode, on the default stream: the refresh must wait for the lookups in flight on the OTHER stream (and,
+    in the factored mode, for the gathers on the library's own streams) before it overwrites the slots of the rows it
+    evicted.  Every output is table[keys]; at the end the cache holds what the oracle places for the last hotness."""
+    monkeypatch.setenv("COLL_HASH_TABLE", table_kind)
+    monkeypatch.setenv("COLL_REFRESH_SLEEP_US", "50")
+    monkeypatch.setenv("COLL_REFRESH_BATCH_ROWS", "512")
+    monkeypatch.setenv("COLL_HASH_REBUILD_FRAC", "0.02")
+    if impl:
+        monkeypatch.setenv("SAMGRAPH_COLL_CACHE_CONCURRENT_LINK_IMPL", impl)
+    rng = np.random.default_rng(123)
+    n_item, dim, pct = 80_000, 64, 0.2
+    co.config(make_config(n_item, pct))
+    co.coll_cache_record_init(0)
+    perm = rng.permutation(n_item)
+    co.coll_torch_record(0, torch.from_numpy(perm[zipf_ranks(rng, 150_000, n_item, 1.05)]))
+    emb = co.coll_torch_create_emb_shm(0, n_item, dim, torch.float32)
+    table = fill_table(emb, rng)
+    co.coll_torch_init_t(0, 0, emb, pct)
+    stop, done, last_stream = [False], [0], [None]
+    r2 = np.random.default_rng(5)
+
+    def refresher():  # torch's current stream of this thread is the default stream
+        while not stop[0] or done[0] < 3:
+            p2 = r2.permutation(n_item)
+            s = p2[zipf_ranks(r2, 150_000, n_item, 1.05)]
+            co.coll_torch_record(0, torch.from_numpy(s))
+            co.coll_torch_refresh(0, False)
+            last_stream[0] = s
+            done[0] += 1
+
+    side = torch.cuda.Stream()
+    t = threading.Thread(target=refresher)
+    t.start()
+    try:
+        with torch.cuda.stream(side):
+            for step in range(60):
+                keep, clones, batches = [], [], []
+                for _ in range(4):
+                    keys = perm[zipf_ranks(rng, int(rng.integers(1, 40_000)), n_item, 1.05)]
+                    kt = torch.from_numpy(keys).cuda()
+                    keep.append(kt)
+                    clones.append(co.coll_torch_lookup_async(0, kt, False).clone())
+                    batches.append(keys)
+                if step % 3 == 0:  # a blocking lookup in between settles the stream-ordered ones first
+                    keys = perm[zipf_ranks(rng, 20_000, n_item, 1.05)]
+                    out = co.coll_torch_lookup_key_t_val_ret(0, torch.from_numpy(keys).cuda(), False)
+                    assert out.cpu().numpy().tobytes() == ORC.gather(table, keys).tobytes(), step
+                co.coll_torch_lookup_wait(0)
+                for keys, c in zip(batches, clones):
+                    assert c.cpu().numpy().tobytes() == ORC.gather(table, keys).tobytes(), step
+    finally:
+        stop[0] = True
+        t.join()
+    assert done[0] >= 3
+    want_cached, nid = expected_cached_set(last_stream[0].astype(np.uint32), n_item, pct)
+    got = np.zeros(len(want_cached), np.uint32)
+    assert _basics.C_LIB_CTYPES.coll_cache_get_cached_keys(0, got.ctypes.data, len(got)) == len(want_cached)
+    assert np.array_equal(got, want_cached)
+    keys = rng.integers(0, n_item, size=30_000)
+    out = co.coll_torch_lookup_key_t_val_ret(0, torch.from_numpy(keys).cuda(), False)
+    assert out.cpu().numpy().tobytes() == ORC.gather(table, keys).tobytes()
+    assert _basics.last_group_offset(0) == [0, int((nid[keys] == 0).sum()), len(keys)]

@@ -638,7 +638,7 @@ def test_dedup_matches_numpy_unique(kdtype, n):
         rep = dev_zeros_u32(n)
         fn = "ugk_dedup_i64" if kdtype == np.int64 else "ugk_dedup_u32"
         d_keys = to_dev(keys)
-        hip.call(fn, ptr(d_keys), n, ptr(ws), epoch, ptr(uniq), ptr(inv), ptr(rep), ptr(nu), None, None)
+        hip.call(fn, ptr(d_keys), n, ptr(ws), ws_bytes, epoch, ptr(uniq), ptr(inv), ptr(rep), ptr(nu), None, None)
         sync()
         k = int(to_np(nu, np.uint32)[0])
         u = to_np(uniq, kdtype)[:k]
@@ -669,13 +669,14 @@ def test_dedup_of_skewed_keys(kdtype, n, shape):
         keys = rng.choice(space, size=n, replace=False) if space > 10 * n else rng.integers(0, space, size=n)
         keys[rng.random(n) < 0.1] = 99
     keys = keys.astype(kdtype)
-    ws = dev_bytes(hip.lib().ugk_dedup_workspace_bytes(n), fill=0)
+    ws_bytes = hip.lib().ugk_dedup_workspace_bytes(n)
+    ws = dev_bytes(ws_bytes, fill=0)
     d_keys = to_dev(keys)
     for epoch in (1, 2):
         uniq = dev_bytes(n * np.dtype(kdtype).itemsize)
         inv, nu, rep = dev_zeros_u32(n), dev_zeros_u32(1), dev_zeros_u32(n)
         fn = "ugk_dedup_i64" if kdtype == np.int64 else "ugk_dedup_u32"
-        hip.call(fn, ptr(d_keys), n, ptr(ws), epoch, ptr(uniq), ptr(inv), ptr(rep), ptr(nu), None, None)
+        hip.call(fn, ptr(d_keys), n, ptr(ws), ws_bytes, epoch, ptr(uniq), ptr(inv), ptr(rep), ptr(nu), None, None)
         sync()
         k = int(to_np(nu, np.uint32)[0])
         u = to_np(uniq, kdtype)[:k]
@@ -685,6 +686,40 @@ def test_dedup_of_skewed_keys(kdtype, n, shape):
         assert i.max() < k and np.array_equal(u[i], keys)
         r = to_np(rep, np.uint32)[:k]
         assert np.array_equal(keys[r], u) and np.array_equal(i[r], np.arange(k))
+
+
+@pytest.mark.parametrize("kdtype", [np.uint32, np.int64])
+def test_dedup_of_small_and_large_batches_sharing_one_workspace(kdtype):
+    """One workspace, sized for the largest batch, serves batches of every smaller size in any order: the slot set and
+    the per-occurrence ids sit where the workspace's own size puts them, so nothing a small batch writes can read as a
+    claim of the current epoch to a larger one.  Few distinct keys and small epochs make stale words look plausible."""
+    rng = np.random.default_rng(99)
+    n_max = 40_000
+    ws_bytes = hip.lib().ugk_dedup_workspace_bytes(n_max)
+    ws = dev_bytes(ws_bytes, fill=0)
+    fn = "ugk_dedup_i64" if kdtype == np.int64 else "ugk_dedup_u32"
+    pool = rng.integers(0, 3000, size=600)
+    epoch = 0
+    for n in (700, 40_000, 1100, 33_000, 5, 40_000, 2050, 2049, 40_000, 1024, 39_999):
+        epoch += 1
+        keys = pool[rng.integers(0, len(pool), size=n)].astype(kdtype)
+        uniq = dev_bytes(n * np.dtype(kdtype).itemsize)
+        inv, nu, rep = dev_zeros_u32(n), dev_zeros_u32(1), dev_zeros_u32(n)
+        hip.call(fn, ptr(to_dev(keys)), n, ptr(ws), ws_bytes, epoch, ptr(uniq), ptr(inv), ptr(rep), ptr(nu), None, None)
+        sync()
+        k = int(to_np(nu, np.uint32)[0])
+        u = to_np(uniq, kdtype)[:k]
+        i = to_np(inv, np.uint32)[:n]
+        assert k == len(np.unique(keys)), (n, epoch)
+        assert np.array_equal(np.sort(u), np.unique(keys))
+        assert i.max() < k and np.array_equal(u[i], keys)
+        r = to_np(rep, np.uint32)[:k]
+        assert np.array_equal(keys[r], u) and np.array_equal(i[r], np.arange(k))
+    # a batch the workspace was not sized for is refused, not squeezed in
+    with pytest.raises(hip.UgkError):
+        n = 4 * n_max
+        hip.call(fn, ptr(to_dev(np.zeros(n, kdtype))), n, ptr(ws), ws_bytes, epoch + 1, ptr(dev_bytes(n * 8)),
+                 ptr(dev_zeros_u32(n)), None, ptr(dev_zeros_u32(1)), None, None)
 
 
 def test_classify_with_destination_map():

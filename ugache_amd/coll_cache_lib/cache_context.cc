@@ -319,13 +319,13 @@ static int Classify(ugk_table_t t, const Id64Type *keys, size_t n, uint64_t host
                     ugk_idx_t *idx, uint32_t *c, uint32_t *next, uint32_t *st, uint32_t *mirror, StreamHandle s) {
   return ugk_classify_i64(t, keys, n, host_rows, dst_map, idx, c, next, st, mirror, s);
 }
-static int Dedup(const IdType *keys, size_t n, void *ws, uint32_t epoch, IdType *uniq, uint32_t *inv, uint32_t *rep,
-                 uint32_t *nu, uint32_t *nu_host, StreamHandle s) {
-  return ugk_dedup_u32(keys, n, ws, epoch, uniq, inv, rep, nu, nu_host, s);
+static int Dedup(const IdType *keys, size_t n, void *ws, size_t ws_bytes, uint32_t epoch, IdType *uniq, uint32_t *inv,
+                 uint32_t *rep, uint32_t *nu, uint32_t *nu_host, StreamHandle s) {
+  return ugk_dedup_u32(keys, n, ws, ws_bytes, epoch, uniq, inv, rep, nu, nu_host, s);
 }
-static int Dedup(const Id64Type *keys, size_t n, void *ws, uint32_t epoch, Id64Type *uniq, uint32_t *inv, uint32_t *rep,
-                 uint32_t *nu, uint32_t *nu_host, StreamHandle s) {
-  return ugk_dedup_i64(keys, n, ws, epoch, uniq, inv, rep, nu, nu_host, s);
+static int Dedup(const Id64Type *keys, size_t n, void *ws, size_t ws_bytes, uint32_t epoch, Id64Type *uniq,
+                 uint32_t *inv, uint32_t *rep, uint32_t *nu, uint32_t *nu_host, StreamHandle s) {
+  return ugk_dedup_i64(keys, n, ws, ws_bytes, epoch, uniq, inv, rep, nu, nu_host, s);
 }
 
 static int Record(const IdType *keys, size_t n, uint64_t mul, uint64_t mask, uint32_t *counts, uint64_t rows,
@@ -435,11 +435,12 @@ template <typename KeyT>
 size_t ExtractSession::DedupKeys(const KeyT *nodes, size_t num_nodes, StreamHandle stream) {
   const size_t ws_bytes = ugk_dedup_workspace_bytes(num_nodes);
   auto alloc = _cache_ctx->_gpu_mem_allocator;
-  if (_dedup_ws == nullptr || _dedup_ws->nbytes() < ws_bytes) {
+  if (_dedup_ws == nullptr || _dedup_ws_bytes < ws_bytes) {
     _dedup_ws = nullptr;
     const size_t grown = ugk_dedup_workspace_bytes(num_nodes + num_nodes / 4);
     _dedup_ws = alloc(grown);
     CHECK_NOTNULL(_dedup_ws);
+    _dedup_ws_bytes = grown;  // the allocator may hand out more; the layout follows what was asked for and zero-filled
     UGK_CALL(ugk_fill_u32(_dedup_ws->ptr<uint32_t>(), 0, grown / 4, stream));
     _dedup_epoch = 0;
   }
@@ -450,12 +451,12 @@ size_t ExtractSession::DedupKeys(const KeyT *nodes, size_t num_nodes, StreamHand
     CHECK_NOTNULL(_dedup_out);
   }
   if (++_dedup_epoch == 0) {  // the tag wrapped: stale entries of 2^32 batches ago must not read as current
-    UGK_CALL(ugk_fill_u32(_dedup_ws->ptr<uint32_t>(), 0, _dedup_ws->nbytes() / 4, stream));
+    UGK_CALL(ugk_fill_u32(_dedup_ws->ptr<uint32_t>(), 0, _dedup_ws_bytes / 4, stream));
     _dedup_epoch = 1;
   }
   uint32_t *n_unique = _state + kStNumUnique;
   UGK_CALL(ugk_fill_u32(n_unique, 0, 1, stream));
-  UGK_CALL(Dedup(nodes, num_nodes, _dedup_ws->ptr<void>(), _dedup_epoch, DedupUnique<KeyT>(),
+  UGK_CALL(Dedup(nodes, num_nodes, _dedup_ws->ptr<void>(), _dedup_ws_bytes, _dedup_epoch, DedupUnique<KeyT>(),
                  DedupInverse(), DedupRep(), n_unique, _host_mirror + kMirNumUnique, stream));
   UGK_CALL(ugk_stream_sync(stream));
   const size_t nu = _host_mirror[kMirNumUnique];
@@ -504,6 +505,11 @@ void ExtractSession::ExtractFeatImpl(const KeyT *nodes, size_t num_nodes, void *
   auto profiler = ctx->_coll_cache ? ctx->_coll_cache->_profiler : nullptr;
   const size_t rb = ctx->_row_bytes;
   const size_t nbytes = num_nodes * rb;
+  struct InFlight {  // counted from before the first kernel reads the table until the output is complete
+    ExtractSession *s;
+    explicit InFlight(ExtractSession *session) : s(session) { s->_blocking_started.fetch_add(1); }
+    ~InFlight() { s->_blocking_finished.fetch_add(1); }
+  } in_flight(this);
   Wait(stream);  // stream-ordered lookups still in flight share the mirror words this call reads
   _group_offset[0] = 0;
   if (num_nodes == 0) {
@@ -576,7 +582,7 @@ void ExtractSession::ExtractFeatImpl(const KeyT *nodes, size_t num_nodes, void *
     return;
   }
 
-  const ugk_table_t table = ctx->_new_hash_table->_table;
+  const ugk_table_t table = ctx->_new_hash_table->Table();
   const void *cache = ctx->_device_cache_data[ctx->_local_location_id];
   const void *host = ctx->_device_cache_data[ctx->_cpu_location_id];
   const uint64_t cache_rows = ctx->_cache_space_capacity;
@@ -721,6 +727,8 @@ void ExtractSession::ExtractFeatAsyncImpl(const KeyT *nodes, size_t num_nodes, v
   CHECK_NOTNULL(nodes);
   CHECK_NOTNULL(output);
   const bool dedup = RunConfig::dedup_keys && num_nodes >= RunConfig::dedup_min_keys;
+  NoteAsyncStream(stream);  // before the first kernel is enqueued: a refresh that does not see the stream yet has
+                            // finished its evictions before that kernel can start
   if (ctx->IsDirectMapping() && !dedup) {
     const bool from_host = ctx->_cpu_location_id != -1;
     void *keys_ready = RecordBegin(stream);
@@ -737,7 +745,7 @@ void ExtractSession::ExtractFeatAsyncImpl(const KeyT *nodes, size_t num_nodes, v
                (uintptr_t)ctx->_device_cache_data[ctx->_cpu_location_id] | (uintptr_t)output | (uintptr_t)rb) &
               15u) == 0) {
     void *keys_ready = RecordBegin(stream);
-    UGK_CALL(ExtractMix(ctx->_new_hash_table->_table, nodes, num_nodes,
+    UGK_CALL(ExtractMix(ctx->_new_hash_table->Table(), nodes, num_nodes,
                         ctx->_device_cache_data[ctx->_local_location_id], ctx->_cache_space_capacity,
                         ctx->_device_cache_data[ctx->_cpu_location_id], ctx->_num_total_nodes, output, rb, _status,
                         _host_mirror, _mix_counts->ptr<uint64_t>(), &_mix_groups, MixOthersHint(num_nodes),
@@ -750,7 +758,6 @@ void ExtractSession::ExtractFeatAsyncImpl(const KeyT *nodes, size_t num_nodes, v
     ExtractFeatImpl<KeyT>(nodes, num_nodes, output, stream, 0xffffffffffffffffull);
     return;
   }
-  _async_used.store(true);
   _async_pending++;
   _async_last_nodes = num_nodes;
 }
@@ -796,6 +803,37 @@ void ExtractSession::ExtractFeatAsync(const IdType *nodes, const size_t num_node
 void ExtractSession::ExtractFeatAsync64(const Id64Type *nodes, const size_t num_nodes, void *output,
                                         StreamHandle stream) {
   ExtractFeatAsyncImpl<Id64Type>(nodes, num_nodes, output, stream);
+}
+
+void ExtractSession::NoteAsyncStream(StreamHandle stream) {
+  if (_async_any && stream == _async_stream_last) return;  // the common case costs a compare
+  std::lock_guard<std::mutex> guard(_async_mu);
+  if (std::find(_async_streams.begin(), _async_streams.end(), stream) == _async_streams.end())
+    _async_streams.push_back(stream);
+  _async_stream_last = stream;
+  _async_any = true;
+}
+
+void ExtractSession::WaitForLookupsInFlight(bool foreground, double timeout_s) {
+  std::vector<StreamHandle> streams;
+  {
+    std::lock_guard<std::mutex> guard(_async_mu);
+    streams = _async_streams;
+  }
+  for (StreamHandle s : streams) UGK_CALL(ugk_stream_sync(s));
+  if (foreground) return;
+  // a blocking lookup counts itself before its first kernel is enqueued: one that is not counted yet starts after the
+  // evictions have completed
+  const size_t started = _blocking_started.load();
+  Timer t0;
+  while (_blocking_finished.load() < started) {
+    if (t0.PassedSec() >= timeout_s) {
+      LOG(ERROR) << "refresh: a lookup that started before the eviction has not returned after " << timeout_s
+                 << " s; going on";
+      break;
+    }
+    usleep(20);
+  }
 }
 
 void ExtractSession::Wait(StreamHandle stream) {
@@ -851,19 +889,12 @@ TensorPtr RefreshSession::CopyTo1DReuse(TensorPtr &preserved_buffer, TensorPtr s
   return ret;
 }
 
-// cache_context.cu:4045-4052.  With stream-ordered lookups "finished" is a matter of the stream: everything enqueued
-// before this point still saw the old table, everything after it sees the evicted keys as misses.
+// cache_context.cu:4045-4052.  The reference waits until `progress` has moved by one (or 20 s have passed); here the
+// session knows which lookups are in flight, on whichever stream, so the wait is for exactly those and an idle cache
+// is not waited for at all.
 void RefreshSession::WaitForOneLookup(ExtractSession *session, bool foreground) {
-  CacheContext *ctx = _cache_ctx.get();
-  const size_t current_progress = ctx->progress.load();
-  const bool stream_ordered = session && session->UsesStreamOrder();
-  if (stream_ordered) UGK_CALL(ugk_stream_sync(stream));
   AnonymousBarrier::_refresh_instance->Wait();
-  Timer t0;
-  while (!foreground && !stream_ordered && ctx->progress.load() < current_progress + 1) {
-    if (t0.PassedSec() >= 20) break;
-    usleep(50);
-  }
+  if (session) session->WaitForLookupsInFlight(foreground, 20.0);
 }
 
 void RefreshSession::CopyRowsIntoSlots(const uint32_t *rows_dev, const uint32_t *slots_dev, size_t num_rows,
@@ -982,7 +1013,9 @@ void RefreshSession::refresh_after_solve_new(bool foreground) {
   table->_cached_keys = key_list_of_each_src[local];
   table->_dev_lists_valid = false;  // the host lists hold the truth now
   ctx->_cache_nodes = num_new_local_key;
-  const bool rebuilt = table->MaybeRebuild(ctx->_eager_gpu_mem_allocator, gpu_ctx, local, stream);
+  const bool rebuilt = table->MaybeRebuild(ctx->_eager_gpu_mem_allocator, gpu_ctx, local, stream, [&]() {
+    if (session) session->WaitForLookupsInFlight(foreground, 20.0);
+  });
   LOG(INFO) << "refresh: key lists " << detect_s << " s, evict " << evict_s << " s, wait for a lookup " << wait_s
             << " s, row copy + insert " << insert_s << " s, table rebuild " << (rebuilt ? t_phase.Passed() : 0.0)
             << " s";
@@ -1076,7 +1109,9 @@ void RefreshSession::refresh_on_device(ExtractSession *session, size_t num_cache
   table->_num_free = capacity - table->_num_cached;
   table->_host_lists_valid = false;  // the bitmaps hold the truth now
   ctx->_cache_nodes = table->_num_cached;
-  const bool rebuilt = table->MaybeRebuild(alloc, gpu_ctx, local, stream);
+  const bool rebuilt = table->MaybeRebuild(alloc, gpu_ctx, local, stream, [&]() {
+    session->WaitForLookupsInFlight(foreground, 20.0);
+  });
   LOG(INFO) << "refresh on the device: bitmaps " << sync_s << " s, placement + key lists " << place_s << " s, evict "
             << evict_s << " s, wait for a lookup " << wait_s << " s, row copy + insert " << insert_s
             << " s, table rebuild " << (rebuilt ? t_phase.Passed() : 0.0) << " s";

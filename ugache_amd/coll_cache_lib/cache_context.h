@@ -111,6 +111,7 @@ class ExtractSession {
   // deduplication in front of the extraction (RunConfig::dedup_keys)
   MemHandle _dedup_ws;   // epoch-tagged set, zero-filled when allocated
   MemHandle _dedup_out;  // [n] distinct keys | [n] inverse | [n] first occurrence
+  size_t _dedup_ws_bytes = 0;  // size the set was laid out and zero-filled for
   uint32_t _dedup_epoch = 0;
   size_t _dedup_cap = 0;  // keys the three arrays are sized for (distinct keys take 8 bytes each whatever the type)
   template <typename KeyT>
@@ -153,7 +154,14 @@ class ExtractSession {
   uint32_t MixOthersHint(size_t num_nodes) const;
   size_t _async_pending = 0;       // stream-ordered lookups enqueued since the last Wait()
   size_t _async_last_nodes = 0;    // size of the last of them
-  std::atomic<bool> _async_used{false};
+  // What a refresh has to see finished before it reuses the slots of evicted rows: blocking lookups are counted when
+  // they start and when they end, the streams stream-ordered lookups were enqueued on are remembered (normally one).
+  std::atomic<size_t> _blocking_started{0}, _blocking_finished{0};
+  std::mutex _async_mu;
+  std::vector<StreamHandle> _async_streams;  // guarded by _async_mu
+  bool _async_any = false;                   // the lookup thread's own: _async_stream_last is valid
+  StreamHandle _async_stream_last = nullptr;
+  void NoteAsyncStream(StreamHandle stream);
   template <typename KeyT>
   void ExtractFeatAsyncImpl(const KeyT *nodes, size_t num_nodes, void *output, StreamHandle stream);
 
@@ -194,8 +202,12 @@ class ExtractSession {
   // blocks until every stream-ordered lookup enqueued so far has finished, aborts if one of them met a key outside
   // its table, and makes LastGroupOffset() describe the last of them
   void Wait(StreamHandle stream);
-  // true once a stream-ordered lookup was enqueued: a refresh then waits for the stream instead of for `progress`
-  bool UsesStreamOrder() const { return _async_used.load(); }
+  // For a refresh, between evicting rows and overwriting their slots: returns once every lookup that may have
+  // resolved a key to one of those slots has finished reading — the stream-ordered ones enqueued so far (a wait for
+  // each stream they went to; the streams must still exist, so call Wait() before destroying one) and, unless
+  // `foreground` says that no lookup runs beside the refresh, the blocking ones that had started (bounded by
+  // `timeout_s`).  Lookups that start later see the evicted keys as misses and read the host table.
+  void WaitForLookupsInFlight(bool foreground, double timeout_s);
   // {0, #local, n} of the last lookup — the reference's group_offset (cache_context.cu:825-847)
   const uint32_t *LastGroupOffset() const { return _group_offset; }
   // moves what the lookups have counted on the device since the last call into `recorder` (FreqRecorder::Record's

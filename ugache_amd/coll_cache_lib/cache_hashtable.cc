@@ -92,7 +92,7 @@ void CacheEntryManager::Evict(TensorPtr keys_to_evict, StreamHandle stream) {
 }
 
 bool CacheEntryManager::MaybeRebuild(const std::function<MemHandle(size_t)> &allocator, Context ctx, int loc,
-                                     StreamHandle stream) {
+                                     StreamHandle stream, const std::function<void()> &wait_for_lookups) {
   if (_table.kind != 2) return false;
   const double limit = RunConfig::hash_rebuild_tombstone_frac * (double)_table.size;
   if ((double)_num_tombstones <= limit) return false;
@@ -118,9 +118,28 @@ bool CacheEntryManager::MaybeRebuild(const std::function<MemHandle(size_t)> &all
             << n << " live keys";
   offs = Tensor::EmptyExternal(kI32, {n}, allocator, ctx, "");
   if (n > 0) LookupOffset(keys, offs, stream);
-  UGK_CALL(ugk_hash_init(static_cast<ugk_bucket_t *>(_table.table), _table.size, stream));
-  if (n > 0) InsertWithLoc(keys, offs, loc, stream);
-  CheckStatus(stream, "table rebuild");
+  // the keys go into a second table; the one in use keeps serving lookups until the swap
+  MemHandle fresh_handle = allocator(_table.size * sizeof(ugk_bucket_t) + 128);
+  CHECK_NOTNULL(fresh_handle);
+  ugk_table_t fresh = _table;
+  fresh.table = Align128(fresh_handle->ptr());
+  UGK_CALL(ugk_hash_init(static_cast<ugk_bucket_t *>(fresh.table), fresh.size, stream));
+  if (n > 0) {
+    if (keys->Type() == kI64)
+      UGK_CALL(ugk_table_insert_i64(fresh, keys->CPtr<int64_t>(), offs->CPtr<uint32_t>(), 0, (uint32_t)loc, n,
+                                    StatusPtr(this, stream), stream));
+    else
+      UGK_CALL(ugk_table_insert_u32(fresh, keys->CPtr<uint32_t>(), offs->CPtr<uint32_t>(), 0, (uint32_t)loc, n,
+                                    StatusPtr(this, stream), stream));
+  }
+  CheckStatus(stream, "table rebuild");  // waits for the stream: the new table is complete
+  {
+    std::lock_guard<std::mutex> guard(_table_mu);
+    _table = fresh;
+    std::swap(_table_handle, fresh_handle);
+  }
+  if (wait_for_lookups) wait_for_lookups();
+  fresh_handle = nullptr;  // the old buckets
   _num_tombstones = 0;
   _num_rebuilds++;
   return true;

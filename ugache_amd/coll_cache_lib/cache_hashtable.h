@@ -6,6 +6,7 @@
 #include <cmath>
 #include <cstring>
 #include <functional>
+#include <mutex>
 #include <vector>
 
 #include "common.h"
@@ -39,6 +40,14 @@ class CacheEntryManager {
   TensorPtr _free_offsets;  // host, u32: free cache slots, allocation sized for the whole capacity
   ugk_table_t _table = {0, 0, nullptr, 0, 0, 0};
   MemHandle _table_handle;
+  // A rebuild publishes a new table while lookups run on another thread: they take their copy of the handle through
+  // Table(), the rebuild swaps it under the same lock and frees the old buckets only once the lookups that may still
+  // hold them have finished.
+  mutable std::mutex _table_mu;
+  ugk_table_t Table() const {
+    std::lock_guard<std::mutex> guard(_table_mu);
+    return _table;
+  }
   MemHandle _status_handle;  // device status word for maintenance kernels
   IdType _cache_space_capacity = 0;
   size_t num_total_key = 0;
@@ -68,9 +77,12 @@ class CacheEntryManager {
   // aborts if a maintenance kernel flagged an error (duplicate insert, absent evict, full table ...)
   void CheckStatus(StreamHandle stream, const char *what);
   // Evictions leave tombstones in the open-addressing table.  Once they exceed
-  // RunConfig::hash_rebuild_tombstone_frac of the buckets the table is cleared and the cached keys re-inserted
-  // with their current slots.  Lookups racing with the rebuild see misses, which the host table serves correctly.
-  bool MaybeRebuild(const std::function<MemHandle(size_t)> &allocator, Context ctx, int loc, StreamHandle stream);
+  // RunConfig::hash_rebuild_tombstone_frac of the buckets the cached keys are inserted, with their current slots, into
+  // a second table of the same size, which then takes the place of the first.  Lookups racing with the rebuild keep
+  // hitting in the old table until the swap; `wait_for_lookups` (may be empty) is called after the swap and must return
+  // only when no lookup that took the old handle is still running, after which the old buckets are released.
+  bool MaybeRebuild(const std::function<MemHandle(size_t)> &allocator, Context ctx, int loc, StreamHandle stream,
+                    const std::function<void()> &wait_for_lookups);
   size_t _num_tombstones = 0;
   size_t _num_rebuilds = 0;
 

@@ -135,7 +135,11 @@ def Init(ps_config_file=None, global_batch_size=1, **kwargs):
     if global_batch_size > cfg.max_batch_size:
         _abort("global_batch_size / num_replicas_in_sync must be <= max_batchsize configured in ps_config.json.")
     dim = cfg.embedding_vecsize_per_table[0]
-    table = _adapter.coll_torch_load_raw_model(0, cfg.sparse_files[0], dim=dim, dtype=torch.float32)
+    # `emb_table` (an extension): a table that is in memory already, as coll_torch_create_emb_shm returns it, instead of
+    # the model directory named by the configuration
+    table = kwargs.get("emb_table")
+    if table is None:
+        table = _adapter.coll_torch_load_raw_model(0, cfg.sparse_files[0], dim=dim, dtype=torch.float32)
     if table.shape[0] != cfg.max_vocabulary_size[0] or table.shape[1] != dim:
         _abort("the model holds %d rows of %d values, the configuration says %d rows of %d"
                % (table.shape[0], table.shape[1], cfg.max_vocabulary_size[0], dim))

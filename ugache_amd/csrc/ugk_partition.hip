@@ -478,15 +478,26 @@ int extract_mix(ugk_table_t t, const K *keys, size_t n, const void *cache, uint6
                                counts, num_groups, others_hint, as_stream(stream));
 }
 
+// The workspace is laid out by its own size, not by the batch's: `cap` slot words, then cap / 2 words of unique ids by
+// first occurrence (a batch may bring at most cap / 2 keys).  Batches of any size that share a workspace therefore agree
+// on what is a slot and what is not, which the epoch tags rely on.
+size_t dedup_capacity_of_workspace(size_t bytes) {
+  size_t cap = 0;
+  for (size_t c = 1024; c * 10 + 64 <= bytes; c <<= 1) cap = c;
+  return cap;
+}
+
 template <typename K>
-int dedup(const K *keys, size_t n, void *workspace, uint32_t epoch, K *unique_out, uint32_t *inverse, uint32_t *rep_of,
-          uint32_t *n_unique, uint32_t *n_unique_host, void *stream) {
+int dedup(const K *keys, size_t n, void *workspace, size_t workspace_bytes, uint32_t epoch, K *unique_out,
+          uint32_t *inverse, uint32_t *rep_of, uint32_t *n_unique, uint32_t *n_unique_host, void *stream) {
   if (n == 0) return 0;
   UGK_REQUIRE(keys && workspace && unique_out && inverse && n_unique, "ugk_dedup: null pointer");
   UGK_REQUIRE(epoch != 0, "ugk_dedup: epoch must be non-zero");
   UGK_REQUIRE(n <= 0x7fffffffull, "ugk_dedup: batch of %zu keys exceeds 2^31", n);
   UGK_REQUIRE((uintptr_t)workspace % 8 == 0, "ugk_dedup: workspace must be 8-byte aligned");
-  const size_t cap = dedup_capacity(n);
+  const size_t cap = dedup_capacity_of_workspace(workspace_bytes);
+  UGK_REQUIRE(cap >= 2 * n, "ugk_dedup: a workspace of %zu bytes holds batches of up to %zu keys, this one has %zu",
+              workspace_bytes, cap / 2, n);
   unsigned long long *slots = reinterpret_cast<unsigned long long *>(workspace);
   uint32_t *uid_of = reinterpret_cast<uint32_t *>(slots + cap);
   // 256-key tiles while 1024-key ones would leave compute units idle; beyond that the larger tile wins, because more
@@ -545,19 +556,19 @@ int ugk_extract_mix_i64(ugk_table_t t, const int64_t *keys_dev, size_t n, const 
                               status_dev, host_mirror, group_counts_host, num_groups_host, others_hint, stream);
 }
 
-size_t ugk_dedup_workspace_bytes(size_t n) { return dedup_capacity(n) * 8 + ((n + 1) / 2 * 2) * 4 + 64; }
+size_t ugk_dedup_workspace_bytes(size_t n) { return dedup_capacity(n) * 10 + 64; }
 
-int ugk_dedup_u32(const uint32_t *keys_dev, size_t n, void *workspace_dev, uint32_t epoch, uint32_t *unique_out_dev,
-                  uint32_t *inverse_out_dev, uint32_t *rep_out_dev, uint32_t *n_unique_dev, uint32_t *n_unique_host,
-                  void *stream) {
-  return dedup<uint32_t>(keys_dev, n, workspace_dev, epoch, unique_out_dev, inverse_out_dev, rep_out_dev, n_unique_dev,
-                         n_unique_host, stream);
+int ugk_dedup_u32(const uint32_t *keys_dev, size_t n, void *workspace_dev, size_t workspace_bytes, uint32_t epoch,
+                  uint32_t *unique_out_dev, uint32_t *inverse_out_dev, uint32_t *rep_out_dev, uint32_t *n_unique_dev,
+                  uint32_t *n_unique_host, void *stream) {
+  return dedup<uint32_t>(keys_dev, n, workspace_dev, workspace_bytes, epoch, unique_out_dev, inverse_out_dev,
+                         rep_out_dev, n_unique_dev, n_unique_host, stream);
 }
-int ugk_dedup_i64(const int64_t *keys_dev, size_t n, void *workspace_dev, uint32_t epoch, int64_t *unique_out_dev,
-                  uint32_t *inverse_out_dev, uint32_t *rep_out_dev, uint32_t *n_unique_dev, uint32_t *n_unique_host,
-                  void *stream) {
-  return dedup<int64_t>(keys_dev, n, workspace_dev, epoch, unique_out_dev, inverse_out_dev, rep_out_dev, n_unique_dev,
-                        n_unique_host, stream);
+int ugk_dedup_i64(const int64_t *keys_dev, size_t n, void *workspace_dev, size_t workspace_bytes, uint32_t epoch,
+                  int64_t *unique_out_dev, uint32_t *inverse_out_dev, uint32_t *rep_out_dev, uint32_t *n_unique_dev,
+                  uint32_t *n_unique_host, void *stream) {
+  return dedup<int64_t>(keys_dev, n, workspace_dev, workspace_bytes, epoch, unique_out_dev, inverse_out_dev,
+                        rep_out_dev, n_unique_dev, n_unique_host, stream);
 }
 
 }  // extern "C"

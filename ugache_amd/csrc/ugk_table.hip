@@ -68,28 +68,41 @@ __global__ __launch_bounds__(kBlock) void hash_insert_kernel(ugk_bucket_t *table
       atomicOr(status, UGK_ST_KEY_OUT_OF_RANGE);
       continue;
     }
+    // The key goes into the first reusable bucket of its probe sequence, but only once the whole sequence up to its
+    // first never-used bucket has been seen not to hold the key already: a tombstone in front of a live copy of the
+    // key must not hide it.  Keys of one launch are distinct, so the only contest is for buckets, and a lost bucket
+    // sends the search back to where it was lost.
+    constexpr uint64_t kNone = ~0ull;
     uint64_t pos = hash_home(key, nb);
+    uint64_t first_tomb = kNone;
     bool placed = false;
-    for (uint64_t step = 0; step < nb && !placed; ++step) {
-      uint64_t cur = load_key_relaxed(table + pos);
-      while (cur == UGK_HASH_EMPTY || cur == UGK_HASH_TOMB) {
-        const uint64_t seen = atomicCAS(reinterpret_cast<unsigned long long *>(&table[pos].key),
-                                        (unsigned long long)cur, (unsigned long long)key);
-        if (seen == cur) {
-          // the bucket is ours: slot and valid bit appear together, in one 8-byte store.  Until then the bucket reads
-          // as "key present, not valid", i.e. as a miss.
-          store_off_meta(table + pos, off, UGK_META_VALID | (loc & 0xfu));
-          placed = true;
-          break;
-        }
-        cur = seen;  // somebody else took it; re-examine what is there now
-      }
-      if (placed) break;
+    for (uint64_t step = 0; step < 2 * nb + 2 && !placed; ++step) {
+      const uint64_t cur = load_key_relaxed(table + pos);
       if (cur == key) {
         atomicOr(status, UGK_ST_DUP_KEY);
         placed = true;
         break;
       }
+      const bool lap_done = step >= nb && first_tomb != kNone;  // no never-used bucket at all: take the tombstone
+      if (cur == UGK_HASH_EMPTY || lap_done) {
+        const uint64_t target = first_tomb != kNone ? first_tomb : pos;
+        const uint64_t expect = first_tomb != kNone ? UGK_HASH_TOMB : UGK_HASH_EMPTY;
+        const uint64_t seen = atomicCAS(reinterpret_cast<unsigned long long *>(&table[target].key),
+                                        (unsigned long long)expect, (unsigned long long)key);
+        if (seen == expect) {
+          // the bucket is ours: slot and valid bit appear together, in one 8-byte store.  Until then the bucket reads
+          // as "key present, not valid", i.e. as a miss.
+          store_off_meta(table + target, off, UGK_META_VALID | (loc & 0xfu));
+          placed = true;
+          break;
+        }
+        // somebody else took it: go on from there (what lies between there and here has been examined, but walking it
+        // again is simpler than remembering it, and rare)
+        pos = target;
+        first_tomb = kNone;
+        continue;
+      }
+      if (cur == UGK_HASH_TOMB && first_tomb == kNone) first_tomb = pos;
       if (++pos == nb) pos = 0;
     }
     if (!placed) atomicOr(status, UGK_ST_TABLE_FULL);

@@ -91,8 +91,8 @@ SIGNATURES = {
     "ugk_extract_mix_u32": [Table, _vp, _sz, _vp, _u64, _vp, _u64, _vp, _sz, _vp, _vp, _vp, _vp, _u32, _vp],
     "ugk_extract_mix_i64": [Table, _vp, _sz, _vp, _u64, _vp, _u64, _vp, _sz, _vp, _vp, _vp, _vp, _u32, _vp],
     "ugk_dedup_workspace_bytes": [_sz],
-    "ugk_dedup_u32": [_vp, _sz, _vp, _u32, _vp, _vp, _vp, _vp, _vp, _vp],
-    "ugk_dedup_i64": [_vp, _sz, _vp, _u32, _vp, _vp, _vp, _vp, _vp, _vp],
+    "ugk_dedup_u32": [_vp, _sz, _vp, _sz, _u32, _vp, _vp, _vp, _vp, _vp, _vp],
+    "ugk_dedup_i64": [_vp, _sz, _vp, _sz, _u32, _vp, _vp, _vp, _vp, _vp, _vp],
     "ugk_record_u32": [_vp, _sz, _u64, _u64, _vp, _u64, _vp, _vp, _vp, _vp],
     "ugk_record_i64": [_vp, _sz, _u64, _u64, _vp, _u64, _vp, _vp, _vp, _vp],
     "ugk_record_drain": [_vp, _u64, _u64, _vp, _vp, _u32, _vp, _vp, _vp],
