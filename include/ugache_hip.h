@@ -239,6 +239,20 @@ int ugk_dedup_i64(const int64_t *keys_dev, size_t n, void *workspace_dev, size_t
                   int64_t *unique_out_dev, uint32_t *inverse_out_dev, uint32_t *rep_out_dev, uint32_t *n_unique_dev,
                   uint32_t *n_unique_host, void *stream);
 
+/* The same deduplication for callers that cannot allocate (code under HIP graph capture, tight serving loops,
+ * harnesses that forbid hipMalloc).  It has no counterpart in the reference.  The slot set and the per-occurrence ids,
+ * which ugk_dedup_* take from workspace_dev, live in a static device array of the library (20 MiB + 320 bytes on every
+ * GPU the library runs on, held until the process ends), and so does the epoch tag, which the call advances itself on
+ * the device: every launch of the call, also a replay of a captured one, sees a fresh tag.  The call makes no
+ * hipMalloc / hipFree and no allocating library call; *n_unique_dev is cleared by the call (an output, not an in/out).
+ * key_bytes: 4 (uint32 keys) or 8 (int64 keys).  n may not exceed UGK_DEDUP_STATIC_MAX_KEYS: larger batches are
+ * refused with an error.  All calls on one GPU share that GPU's array: calls that overlap in time on one GPU (different
+ * streams, or threads) race and give wrong results; calls ordered one after the other, on any streams, are fine. */
+#define UGK_DEDUP_STATIC_MAX_KEYS (1u << 20)
+int ugk_dedup_static(const void *keys_dev, uint32_t key_bytes, size_t n, void *unique_out_dev,
+                     uint32_t *inverse_out_dev, uint32_t *rep_out_dev, uint32_t *n_unique_dev, uint32_t *n_unique_host,
+                     void *stream);
+
 /* ---- hotness counters on the device: FreqRecorder::Record (freq_recorder.cc:227-253) without the copy of the keys
  *      to the host, the record thread of python_tf2/collcache_tf2/collcache_tf2/core/lookup_manager.cc:291-312 ----
  * counts_dev: one uint32 per row of the host table, zero-filled once.  ugk_record_*: counts_dev[row(key)] += 1 for

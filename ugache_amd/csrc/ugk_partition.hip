@@ -9,8 +9,18 @@
 // same (location-grouped) array the reference obtains by sorting.
 #include <cstdlib>
 
+#include <mutex>
+
 #include "ugk_internal.h"
 #include "ugk_table.cuh"
+
+// Scratch of ugk_dedup_static, the one entry point that allocates nothing: a header (word 0 = the epoch tag of the last
+// call), then the slot set and the per-occurrence ids that ugk_dedup_* take from their workspace argument.  Every GPU
+// the library runs on holds its own copy until the process ends; host code reaches it through the address
+// hipGetSymbolAddress returns for the current device, never through this name.
+#define UGK_DEDUP_STATIC_HEADER 256
+#define UGK_DEDUP_STATIC_WS_BYTES (((size_t)2 * UGK_DEDUP_STATIC_MAX_KEYS) * 10 + 64)
+static __device__ __align__(256) unsigned char scratch[UGK_DEDUP_STATIC_HEADER + UGK_DEDUP_STATIC_WS_BYTES];
 
 namespace ugk {
 namespace {
@@ -204,9 +214,10 @@ __global__ __launch_bounds__(kBlock) void extract_mix_kernel(ugk_table_t t, cons
 template <typename K, int ITEMS>
 __global__ __launch_bounds__(kBlock) void dedup_claim_kernel(const K *__restrict__ keys, size_t n,
                                                              unsigned long long *slots, size_t cap_mask,
-                                                             uint32_t epoch, uint32_t *uid_of, K *unique_out,
-                                                             uint32_t *inverse, uint32_t *rep_of,
-                                                             uint32_t *n_unique) {
+                                                             uint32_t epoch, const uint32_t *epoch_dev,
+                                                             uint32_t *uid_of, K *unique_out, uint32_t *inverse,
+                                                             uint32_t *rep_of, uint32_t *n_unique) {
+  if (epoch_dev) epoch = *epoch_dev;  // the tag lives in device memory when the set does (see ugk_dedup_static)
   // A tile of TILE keys per pass (ITEMS per lane): one reservation of unique ids per tile, so with four per lane the
   // single counter they come from sees a quarter of the atomics a 256-key tile would send it.
   // Two stages.  The keys of a tile first meet in a set in LDS, where every distinct key of the tile gets one leader
@@ -339,6 +350,21 @@ __global__ __launch_bounds__(kBlock) void dedup_resolve_kernel(size_t n, const u
   if (n_unique_host && blockIdx.x == 0 && threadIdx.x == 0) *n_unique_host = *n_unique;
   for (size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x; i < n; i += (size_t)gridDim.x * kBlock)
     inverse[i] = uid_of[inverse[i]];
+}
+
+// ugk_dedup_static, before the claims: when the epoch tag is about to wrap, every slot is cleared so that what was
+// tagged 2^32 calls ago cannot read as current (the tag itself moves in static_epoch_kernel, after every workgroup of
+// this kernel has read it)
+__global__ __launch_bounds__(kBlock) void static_wrap_kernel(const uint32_t *epoch, unsigned long long *slots,
+                                                             size_t cap) {
+  if (*epoch != 0xffffffffu) return;
+  for (size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x; i < cap; i += (size_t)gridDim.x * kBlock) slots[i] = 0ull;
+}
+
+__global__ void static_epoch_kernel(uint32_t *epoch, uint32_t *n_unique) {
+  const uint32_t e = *epoch;
+  *epoch = e == 0xffffffffu ? 1u : e + 1u;
+  *n_unique = 0u;
 }
 
 size_t dedup_capacity(size_t n) {
@@ -488,11 +514,12 @@ size_t dedup_capacity_of_workspace(size_t bytes) {
 }
 
 template <typename K>
-int dedup(const K *keys, size_t n, void *workspace, size_t workspace_bytes, uint32_t epoch, K *unique_out,
-          uint32_t *inverse, uint32_t *rep_of, uint32_t *n_unique, uint32_t *n_unique_host, void *stream) {
+int dedup(const K *keys, size_t n, void *workspace, size_t workspace_bytes, uint32_t epoch, const uint32_t *epoch_dev,
+          K *unique_out, uint32_t *inverse, uint32_t *rep_of, uint32_t *n_unique, uint32_t *n_unique_host,
+          void *stream) {
   if (n == 0) return 0;
   UGK_REQUIRE(keys && workspace && unique_out && inverse && n_unique, "ugk_dedup: null pointer");
-  UGK_REQUIRE(epoch != 0, "ugk_dedup: epoch must be non-zero");
+  UGK_REQUIRE(epoch != 0 || epoch_dev, "ugk_dedup: epoch must be non-zero");
   UGK_REQUIRE(n <= 0x7fffffffull, "ugk_dedup: batch of %zu keys exceeds 2^31", n);
   UGK_REQUIRE((uintptr_t)workspace % 8 == 0, "ugk_dedup: workspace must be 8-byte aligned");
   const size_t cap = dedup_capacity_of_workspace(workspace_bytes);
@@ -507,10 +534,10 @@ int dedup(const K *keys, size_t n, void *workspace, size_t workspace_bytes, uint
   const unsigned claim_grid = clamp_grid((n + tile - 1) / tile, 0);
   if (items == 1)
     hipLaunchKernelGGL((dedup_claim_kernel<K, 1>), dim3(claim_grid), dim3(kBlock), 0, as_stream(stream), keys, n,
-                       slots, cap - 1, epoch, uid_of, unique_out, inverse, rep_of, n_unique);
+                       slots, cap - 1, epoch, epoch_dev, uid_of, unique_out, inverse, rep_of, n_unique);
   else
     hipLaunchKernelGGL((dedup_claim_kernel<K, kItems>), dim3(claim_grid), dim3(kBlock), 0, as_stream(stream), keys, n,
-                       slots, cap - 1, epoch, uid_of, unique_out, inverse, rep_of, n_unique);
+                       slots, cap - 1, epoch, epoch_dev, uid_of, unique_out, inverse, rep_of, n_unique);
   UGK_HIP(hipGetLastError());
   const unsigned grid = clamp_grid((n + kBlock - 1) / kBlock, 0);
   hipLaunchKernelGGL(dedup_resolve_kernel, dim3(grid), dim3(kBlock), 0, as_stream(stream), n, uid_of, inverse,
@@ -558,16 +585,60 @@ int ugk_extract_mix_i64(ugk_table_t t, const int64_t *keys_dev, size_t n, const 
 
 size_t ugk_dedup_workspace_bytes(size_t n) { return dedup_capacity(n) * 10 + 64; }
 
+int ugk_dedup_static(const void *keys_dev, uint32_t key_bytes, size_t n, void *unique_out_dev,
+                     uint32_t *inverse_out_dev, uint32_t *rep_out_dev, uint32_t *n_unique_dev, uint32_t *n_unique_host,
+                     void *stream) {
+  UGK_REQUIRE(key_bytes == 4 || key_bytes == 8, "ugk_dedup_static: keys of %u bytes (4 or 8 are supported)", key_bytes);
+  UGK_REQUIRE(n_unique_dev, "ugk_dedup_static: null count word");
+  UGK_REQUIRE(n <= UGK_DEDUP_STATIC_MAX_KEYS,
+              "ugk_dedup_static: a batch of %zu keys exceeds the %zu the static scratch is sized for "
+              "(use ugk_dedup_u32 / ugk_dedup_i64 with a workspace of your own)",
+              n, (size_t)UGK_DEDUP_STATIC_MAX_KEYS);
+  // the device address of this GPU's copy of the array, looked up once per device with that device current
+  static std::mutex mu;
+  static unsigned char *base_of[64] = {nullptr};
+  int dev = 0;
+  UGK_HIP(hipGetDevice(&dev));
+  UGK_REQUIRE(dev >= 0 && dev < 64, "ugk_dedup_static: device %d out of range", dev);
+  unsigned char *base = nullptr;
+  {
+    std::lock_guard<std::mutex> guard(mu);
+    if (base_of[dev] == nullptr) {
+      void *p = nullptr;
+      UGK_HIP(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));
+      UGK_REQUIRE(p != nullptr, "ugk_dedup_static: no device address for the static scratch");
+      base_of[dev] = static_cast<unsigned char *>(p);
+    }
+    base = base_of[dev];
+  }
+  uint32_t *epoch_dev = reinterpret_cast<uint32_t *>(base);
+  unsigned char *ws = base + UGK_DEDUP_STATIC_HEADER;
+  const size_t cap = dedup_capacity_of_workspace(UGK_DEDUP_STATIC_WS_BYTES);
+  hipLaunchKernelGGL(static_wrap_kernel, dim3(clamp_grid(1024, 0)), dim3(kBlock), 0, as_stream(stream),
+                     epoch_dev, reinterpret_cast<unsigned long long *>(ws), cap);
+  UGK_HIP(hipGetLastError());
+  hipLaunchKernelGGL(static_epoch_kernel, dim3(1), dim3(1), 0, as_stream(stream), epoch_dev, n_unique_dev);
+  UGK_HIP(hipGetLastError());
+  if (n == 0) return 0;
+  if (key_bytes == 4)
+    return dedup<uint32_t>(static_cast<const uint32_t *>(keys_dev), n, ws, UGK_DEDUP_STATIC_WS_BYTES, 0, epoch_dev,
+                           static_cast<uint32_t *>(unique_out_dev), inverse_out_dev, rep_out_dev, n_unique_dev,
+                           n_unique_host, stream);
+  return dedup<int64_t>(static_cast<const int64_t *>(keys_dev), n, ws, UGK_DEDUP_STATIC_WS_BYTES, 0, epoch_dev,
+                        static_cast<int64_t *>(unique_out_dev), inverse_out_dev, rep_out_dev, n_unique_dev,
+                        n_unique_host, stream);
+}
+
 int ugk_dedup_u32(const uint32_t *keys_dev, size_t n, void *workspace_dev, size_t workspace_bytes, uint32_t epoch,
                   uint32_t *unique_out_dev, uint32_t *inverse_out_dev, uint32_t *rep_out_dev, uint32_t *n_unique_dev,
                   uint32_t *n_unique_host, void *stream) {
-  return dedup<uint32_t>(keys_dev, n, workspace_dev, workspace_bytes, epoch, unique_out_dev, inverse_out_dev,
+  return dedup<uint32_t>(keys_dev, n, workspace_dev, workspace_bytes, epoch, nullptr, unique_out_dev, inverse_out_dev,
                          rep_out_dev, n_unique_dev, n_unique_host, stream);
 }
 int ugk_dedup_i64(const int64_t *keys_dev, size_t n, void *workspace_dev, size_t workspace_bytes, uint32_t epoch,
                   int64_t *unique_out_dev, uint32_t *inverse_out_dev, uint32_t *rep_out_dev, uint32_t *n_unique_dev,
                   uint32_t *n_unique_host, void *stream) {
-  return dedup<int64_t>(keys_dev, n, workspace_dev, workspace_bytes, epoch, unique_out_dev, inverse_out_dev,
+  return dedup<int64_t>(keys_dev, n, workspace_dev, workspace_bytes, epoch, nullptr, unique_out_dev, inverse_out_dev,
                         rep_out_dev, n_unique_dev, n_unique_host, stream);
 }
 

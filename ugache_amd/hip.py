@@ -93,6 +93,7 @@ SIGNATURES = {
     "ugk_dedup_workspace_bytes": [_sz],
     "ugk_dedup_u32": [_vp, _sz, _vp, _sz, _u32, _vp, _vp, _vp, _vp, _vp, _vp],
     "ugk_dedup_i64": [_vp, _sz, _vp, _sz, _u32, _vp, _vp, _vp, _vp, _vp, _vp],
+    "ugk_dedup_static": [_vp, _u32, _sz, _vp, _vp, _vp, _vp, _vp, _vp],
     "ugk_record_u32": [_vp, _sz, _u64, _u64, _vp, _u64, _vp, _vp, _vp, _vp],
     "ugk_record_i64": [_vp, _sz, _u64, _u64, _vp, _u64, _vp, _vp, _vp, _vp],
     "ugk_record_drain": [_vp, _u64, _u64, _vp, _vp, _u32, _vp, _vp, _vp],
