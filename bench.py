@@ -9,6 +9,12 @@ cached, 262,144 uniform uint32 keys per batch, duplicates allowed.  `--workload`
 configurations (pinned host table + frequency-ranked HBM cache); those print the same JSON shape plus a `host_link`
 object and per-stage times.
 
+Without `--workload` the line carries both halves of the metric: the all-hit configuration is the top level (with two
+more all-hit legs whose output cannot stay in the 256 MB memory-side cache), and the GNN-shaped and the hashtable-mode
+configuration run at full size, one after the other, each in a child process of its own (this process never touches
+the GPU), and appear under `legs` with their host-link rates.  Every pooled key batch of every leg is compared with the
+CPU oracle after its timed region; a difference ends the run without a number.
+
 Prints ONE JSON line with keys/s (whole job), the roofline of the dominant HBM kernel (algorithmic bytes per launch /
 its average duration, measured live with HIP events on the kernel's stream inside the timed region) and the CPU
 baseline (the oracle's OpenMP gather on the host cores, bounded sample of the same batches).
@@ -80,8 +86,10 @@ def parse_args():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=None)
     ap.add_argument("--warmup", type=int, default=None)
-    ap.add_argument("--workload", default="c2_all_hit_10Mx128xfp32_262144_u32_uniform",
-                    choices=sorted(ALL_HIT) + sorted(MIXED))
+    ap.add_argument("--workload", default=None, choices=sorted(ALL_HIT) + sorted(MIXED),
+                    help="run this one workload in this process (default: the all-hit configuration at the top level "
+                         "plus the mixed-source legs, each in a child process)")
+    ap.add_argument("--no-legs", action="store_true", help="default run without the mixed-source legs")
     ap.add_argument("--cpu-seconds", type=float, default=10.0, help="CPU baseline budget")
     ap.add_argument("--pool", type=int, default=None, help="distinct key batches cycled through the steps")
     ap.add_argument("--impl", default="", choices=["", "DIRECT", "SMMaskPhase", "NONE"],
@@ -108,22 +116,26 @@ def parse_args():
     return args
 
 
-def stream_ordered_leg(C, fn, key_ptr_of, n_keys, out, stream, torch, W, K):
+def stream_ordered_leg(C, fn, key_ptr_of, n_keys, out, stream, torch, W, K, out_ptr_of=None):
     """the same K steps through the stream-ordered entry point: batches are enqueued back to back, one wait at the
     end.  Returns (wall seconds per step, seconds per launch between two HIP events recorded on the same stream right
-    before the first and right after the last of the K launches)."""
+    before the first and right after the last of the K launches).  out_ptr_of(i): where step i writes (default: the
+    one buffer `out`)."""
     from ugache_amd import hip
+    if out_ptr_of is None:
+        one = out.data_ptr()
+        out_ptr_of = lambda i: one
     ev = [ctypes.c_void_p(), ctypes.c_void_p()]
     for e in ev:
         hip.call("ugk_event_create", ctypes.byref(e))
     for i in range(W):
-        fn(0, key_ptr_of(i), n_keys, out.data_ptr(), stream)
+        fn(0, key_ptr_of(i), n_keys, out_ptr_of(i), stream)
     C.coll_cache_lookup_wait(0, stream)
     torch.cuda.synchronize()
     t0 = time.perf_counter()
     hip.call("ugk_event_record", ev[0], stream)
     for i in range(W, W + K):
-        fn(0, key_ptr_of(i), n_keys, out.data_ptr(), stream)
+        fn(0, key_ptr_of(i), n_keys, out_ptr_of(i), stream)
     hip.call("ugk_event_record", ev[1], stream)
     C.coll_cache_lookup_wait(0, stream)
     torch.cuda.synchronize()
@@ -146,6 +158,20 @@ def step_spread(t0, stamps):
     import numpy as np
     d = np.diff(np.concatenate(([t0], np.asarray(stamps)))) * 1e3
     return {"median": float(np.median(d)), "p95": float(np.percentile(d, 95)), "max": float(d.max())}
+
+
+def check_every_batch(orc, table_np, rows_host, lookup_into, out, what):
+    """one more pass over the pool after the timed region: every pooled batch is looked up again (blocking) and its
+    output compared byte for byte with the oracle's gather of the same rows.  Ends the run on the first difference.
+    rows_host[i]: the host-table row of every key of batch i; lookup_into(i): looks batch i up into `out`."""
+    import torch
+
+    for i in range(len(rows_host)):
+        lookup_into(i)
+        torch.cuda.synchronize()
+        if out.cpu().numpy().tobytes() != orc.gather(table_np, rows_host[i], omp=True).tobytes():
+            sys.exit("bench.py: GPU output of %s batch %d differs from the CPU oracle — no numbers reported" % (what, i))
+    return len(rows_host)
 
 
 def cpu_baseline(orc, table_np, keys_host, n_keys, row_bytes, seconds):
@@ -248,12 +274,19 @@ def run_all_hit(args):
         torch.cuda.synchronize()
         del cal_src, cal_dst
 
-    # parity of the last timed batch, byte for byte against the oracle
+    # parity, byte for byte against the oracle: the last batch of the stream-ordered leg as it left it, then every
+    # pooled batch through the blocking entry point
     orc = Oracle()
     table_np = emb.numpy()
-    last_keys = keys_pool[(W + K - 1) % pool].cpu().numpy().view(np.uint32)
-    if out.cpu().numpy().tobytes() != orc.gather(table_np, last_keys, omp=True).tobytes():
+    keys_host = keys_pool.cpu().numpy().view(np.uint32)
+    if out.cpu().numpy().tobytes() != orc.gather(table_np, keys_host[(W + K - 1) % pool], omp=True).tobytes():
         sys.exit("bench.py: GPU output differs from the CPU oracle — no numbers reported")
+    n_checked = check_every_batch(orc, table_np, keys_host, step, out, "all-hit")
+
+    large = None
+    if rows >= 1_000_000:
+        large = all_hit_large_output_legs(C, orc, table_np, keys_pool, key_ptrs, keys_host, rows, dim, row_bytes,
+                                          n_keys, stream, dev, W, K)
 
     # dominant kernel: average launch duration over a timed region of K launches, from two HIP events on the kernel's
     # stream around the K back-to-back launches of the stream-ordered leg (nothing else runs on that stream between
@@ -265,7 +298,6 @@ def run_all_hit(args):
     alg_bytes = n_keys * (2 * row_bytes + 4)  # row read + row written + key read, per key
     achieved = alg_bytes / kernel_avg_s / 1e9
 
-    keys_host = keys_pool.cpu().numpy().view(np.uint32)
     table_bytes = table_np.view(np.uint8).reshape(rows, row_bytes)
     cpu_kps, n_cpu, cpu_el, cores = cpu_baseline(orc, table_bytes, keys_host, n_keys, row_bytes, args.cpu_seconds)
 
@@ -281,10 +313,12 @@ def run_all_hit(args):
                    "key_dtype": "uint32", "cache_percentage": 1.0, "entry_point": "coll_cache_lookup",
                    "distinct_key_batches": pool, "seeds": {"table": 1, "keys": 4}},
         "effective_extraction_GBps": n_keys * row_bytes / (elapsed / K) / 1e9,
-        "parity": "bit-exact vs CPU oracle (last timed batch)",
+        "parity": "bit-exact vs CPU oracle: every one of the %d pooled batches, after the timed region" % n_checked,
         "device": info["name"] + " " + info["arch"],
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                      "frac": achieved / HBM_PEAK_GBPS, "traffic": MEASURED_TRAFFIC_BYTES.get(args.workload),
+                     "traffic_source": "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs summarised in "
+                                       "profiles/gather_kernel_c2_all_hit.md (not read in this run)",
                      "kernel": "gather_kernel<u32x4,32,2,DirectU32>", "algorithmic_bytes_per_launch": alg_bytes,
                      "avg_kernel_us": kernel_avg_s * 1e6, "keys_per_s_kernel_only": n_keys / kernel_avg_s,
                      "timing": "2 HIP events around %d back-to-back launches on the kernel's stream" % K,
@@ -298,8 +332,58 @@ def run_all_hit(args):
                            "entry_point": "coll_cache_lookup_async (extension: enqueue only, one wait after the K "
                                           "steps; same batches, last one checked against the oracle as well)"},
     }
+    if large is not None:
+        result["all_hit_large_output"] = large
     co.coll_torch_shutdown()
-    emit(result)
+    return result
+
+
+def all_hit_large_output_legs(C, orc, table_np, keys_pool, key_ptrs, keys_host, rows, dim, row_bytes, n_keys, stream,
+                              dev, W, K):
+    """The same gather where the output cannot live in the 256 MB memory-side cache from one launch to the next:
+    (a) batches of 2^20 keys, 537 MB of output per launch; (b) the configuration's own 262,144-key batches with the
+    output rotated over 8 buffers of 134 MB.  Kernel time = two HIP events on the stream around K back-to-back
+    stream-ordered launches; every batch timed in (a) and the last 8 of (b) are compared with the oracle."""
+    import torch
+
+    pool = len(key_ptrs)
+    res = {}
+    # (a) one million keys per launch
+    n_big = 1 << 20
+    big_pool = 4
+    g = torch.Generator(device=dev).manual_seed(5)
+    big_keys = torch.randint(0, rows, (big_pool, n_big), generator=g, device=dev, dtype=torch.int32)
+    big_ptrs = [big_keys[i].data_ptr() for i in range(big_pool)]
+    big_out = torch.empty((n_big, dim), dtype=torch.float32, device=dev)
+    _, t_big = stream_ordered_leg(C, C.coll_cache_lookup_async, lambda i: big_ptrs[i % big_pool], n_big, big_out,
+                                  stream, torch, W, K)
+    big_host = big_keys.cpu().numpy().view("uint32")
+    check_every_batch(orc, table_np, big_host,
+                      lambda i: C.coll_cache_lookup(0, big_ptrs[i], n_big, big_out.data_ptr(), stream), big_out,
+                      "1M-key all-hit")
+    alg = n_big * (2 * row_bytes + 4)
+    res["keys_1M"] = {"keys_per_batch": n_big, "output_bytes_per_launch": n_big * row_bytes,
+                      "avg_kernel_us": t_big * 1e6, "algorithmic_bytes_per_launch": alg,
+                      "achieved_GBps": alg / t_big / 1e9, "frac_of_hbm_peak": alg / t_big / 1e9 / HBM_PEAK_GBPS,
+                      "keys_per_s_kernel_only": n_big / t_big, "batches_checked": big_pool}
+    del big_out, big_keys
+    # (b) the configuration's batches, outputs rotated
+    R = 8
+    outs = [torch.empty((n_keys, dim), dtype=torch.float32, device=dev) for _ in range(R)]
+    out_ptrs = [o.data_ptr() for o in outs]
+    _, t_rot = stream_ordered_leg(C, C.coll_cache_lookup_async, lambda i: key_ptrs[i % pool], n_keys, outs[0], stream,
+                                  torch, W, K, out_ptr_of=lambda i: out_ptrs[i % R])
+    for i in range(max(W, W + K - R), W + K):  # the last launches' outputs are still in their buffers
+        if outs[i % R].cpu().numpy().tobytes() != orc.gather(table_np, keys_host[i % pool], omp=True).tobytes():
+            sys.exit("bench.py: GPU output of rotated all-hit launch %d differs from the CPU oracle" % i)
+    alg = n_keys * (2 * row_bytes + 4)
+    res["outputs_rotated"] = {"keys_per_batch": n_keys, "output_buffers": R,
+                              "output_bytes_in_rotation": R * n_keys * row_bytes, "avg_kernel_us": t_rot * 1e6,
+                              "algorithmic_bytes_per_launch": alg, "achieved_GBps": alg / t_rot / 1e9,
+                              "frac_of_hbm_peak": alg / t_rot / 1e9 / HBM_PEAK_GBPS,
+                              "launches_checked": min(K, R)}
+    res["timing"] = "2 HIP events around %d back-to-back stream-ordered launches on the kernel's stream" % K
+    return res
 
 
 def zipf_ranks_gpu(torch, n, space, s, gen, dev):
@@ -427,11 +511,13 @@ def run_mixed(args):
 
     orc = Oracle()
     table_np = emb.numpy().view(np.uint8).reshape(rows, row_bytes)
-    last_rows = rows_pool[(W + K - 1) % pool].cpu().numpy()
-    if out.cpu().numpy().tobytes() != orc.gather(table_np, last_rows, omp=True).tobytes():
+    rows_host = rows_pool.cpu().numpy()
+    if out.cpu().numpy().tobytes() != orc.gather(table_np, rows_host[(W + K - 1) % pool], omp=True).tobytes():
         sys.exit("bench.py: GPU output differs from the CPU oracle — no numbers reported")
+    n_checked = check_every_batch(orc, table_np, rows_host, step, out, args.workload)
+    note("all %d pooled batches equal the oracle's gather" % n_checked)
 
-    steps = range(W, W + K)
+    steps = range(W, W + K)  # (the parity pass above ran later steps; these are the timed ones)
     t_idx = float(np.mean([_basics.step_value(s, kLogL3CacheGetIndexTime) for s in steps]))
     t_miss = float(np.mean([_basics.step_value(s, kLogL3CacheCombineMissTime) for s in steps]))
     t_hit = float(np.mean([_basics.step_value(s, kLogL3CacheCombineCacheTime) for s in steps]))
@@ -475,8 +561,13 @@ def run_mixed(args):
         stages = {"classify_partition": t_idx * 1e6, "host_gather": t_miss * 1e6, "hbm_gather": t_hit * 1e6}
     achieved = hit_alg / t_hit / 1e9 if t_hit > 0 else 0.0
 
+    miss_alone = miss_stream_alone(C, _basics, step, stream, torch, W, K, pool, rows_host, table_np, orc, out,
+                                   row_bytes, link_gbps, kLogL1MissBytes, kLogL3CacheCombineCacheTime,
+                                   kLogL3CacheCombineMissTime, args.workload, note)
+    ceiling = random_row_ceiling(hip, torch, emb, rows, row_bytes, dev, stream, note)
+
     # the CPU baseline gathers by row number (it is spared the id -> row translation of sparse-id mode)
-    keys_host = rows_pool.cpu().numpy()
+    keys_host = rows_host
     cpu_kps, n_cpu, cpu_el, cores = cpu_baseline(orc, table_np, keys_host, n_keys, row_bytes, args.cpu_seconds)
     uniq = float(np.mean([len(np.unique(keys_host[i])) for i in range(min(pool, 4))]))
 
@@ -604,7 +695,7 @@ def run_mixed(args):
                    "entry_point": "coll_cache_lookup_i64", "distinct_key_batches": pool, "impl": args.impl or "fused (default)", "dedup": bool(args.dedup), "gpu_record": bool(args.gpu_record), "device_refresh": bool(args.device_refresh),
                    "unique_keys_per_batch": uniq, "seeds": {"table": 1, "perm": 2, "keys": 3}},
         "effective_extraction_GBps": n_keys * row_bytes / (elapsed / K) / 1e9,
-        "parity": "bit-exact vs CPU oracle (last timed batch)",
+        "parity": "bit-exact vs CPU oracle: every one of the %d pooled batches, after the timed region" % n_checked,
         "device": info["name"] + " " + info["arch"],
         "stages_us": stages,
         "hit_rate": n_hit / n_keys,
@@ -616,10 +707,15 @@ def run_mixed(args):
                      PER_CALL_KEY[os.environ.get("COLL_KERNEL_EVENTS", "0") != "0"]: per_launch_pair_us},
         "host_link": {"achieved": miss_bytes / t_link / 1e9 if t_link > 0 else 0.0, "measured_peak": link_gbps,
                       "unit": "GB/s", "frac": (miss_bytes / t_link / 1e9) / link_gbps if t_link > 0 else 0.0,
-                      "miss_rows_per_batch": n_miss, "peak_probe": "pinned host -> HBM hipMemcpyAsync, best of 3"},
+                      "miss_rows_per_batch": n_miss, "peak_probe": "pinned host -> HBM hipMemcpyAsync, best of 3",
+                      "random_row_ceiling": ceiling,
+                      "frac_of_row_ceiling": ((miss_bytes / t_link / 1e9) / ceiling["best_GBps"]
+                                              if t_link > 0 and ceiling["best_GBps"] > 0 else None),
+                      "miss_stream_alone": miss_alone},
         "cpu_baseline": {"value": cpu_kps, "unit": "keys/s", "cores": cores, "kind": "port",
-                         "sample": "%d batches of %d keys from the same pool, %.1f s, OpenMP gather over keys"
-                                   % (n_cpu, n_keys, cpu_el),
+                         "sample": "%d batches of %d keys from the same pool, %.1f s, OpenMP gather over keys by row "
+                                   "number out of the whole host table (no lookup or classify step: the fastest the "
+                                   "CPU path can be)" % (n_cpu, n_keys, cpu_el),
                          "effective_GBps": n_keys * row_bytes * n_cpu / cpu_el / 1e9},
         "gpu_over_cpu": keys_per_s / cpu_kps,
         "setup_seconds": setup_s,
@@ -628,6 +724,137 @@ def run_mixed(args):
                                           "steps; same batches, last one checked against the oracle as well)"},
     }
     co.coll_torch_shutdown()
+    return result
+
+
+def miss_stream_alone(C, _basics, step, stream, torch, W, K, pool, rows_host, table_np, orc, out, row_bytes, link_gbps,
+                      kLogL1MissBytes, kLogL3CacheCombineCacheTime, kLogL3CacheCombineMissTime, workload, note):
+    """The host-link half on its own, through the library: COLL_SKIP_LOCAL=1 (the reference's aid for exactly this,
+    cache_context.cu:728-741) drops the keys the cache serves in front of the extraction, so the extraction kernel
+    moves the missed rows only.  Its time is what the library logs for the step: a host timer around the kernel's
+    launch and the wait for it (about 10 us more than the kernel itself)."""
+    import numpy as np
+
+    os.environ["COLL_SKIP_LOCAL"] = "1"
+    try:
+        first = _basics.info(0)["lookups"]
+        for i in range(W + K):
+            step(i)
+        torch.cuda.synchronize()
+        steps = range(first + W, first + W + K)
+        t = np.array([max(_basics.step_value(s, kLogL3CacheCombineCacheTime),
+                          _basics.step_value(s, kLogL3CacheCombineMissTime)) for s in steps])
+        b = np.array([_basics.step_value(s, kLogL1MissBytes) for s in steps])
+        # parity of the compacted output: the rows of the keys the cache does not hold, in their order
+        last = (W + K - 1) % pool
+        g = _basics.last_group_offset(0)
+        m = int(g[2])
+        got = out[:m].cpu().numpy().tobytes()
+    finally:
+        del os.environ["COLL_SKIP_LOCAL"]
+    step(last)  # the same batch in full tells which keys were missed: group sizes [0, hits, n]
+    torch.cuda.synchronize()
+    full = out.cpu().numpy()
+    want_full = orc.gather(table_np, rows_host[last], omp=True)
+    if full.tobytes() != want_full.tobytes() or m != int(_basics.last_group_offset(0)[2] - _basics.last_group_offset(0)[1]):
+        sys.exit("bench.py: %s: the skip-local run and the full run disagree on the missed keys" % workload)
+    # every row of the compacted output must be a row of the batch, in batch order: match them greedily
+    want = want_full.reshape(len(rows_host[last]), row_bytes)
+    comp = np.frombuffer(got, np.uint8).reshape(m, row_bytes)
+    j = 0
+    for i in range(len(want)):
+        if j < m and want[i].tobytes() == comp[j].tobytes():
+            j += 1
+    if j != m:
+        sys.exit("bench.py: %s: the skip-local output is not the missed rows in batch order" % workload)
+    gbps = float(b.sum() / t.sum() / 1e9)
+    note("miss stream alone: %.1f GB/s over %.0f rows per batch" % (gbps, b.mean() / row_bytes))
+    return {"achieved_GBps": gbps, "frac_of_measured_peak": gbps / link_gbps, "rows_per_batch": float(b.mean() / row_bytes),
+            "us_per_batch": float(t.mean() * 1e6), "how": "COLL_SKIP_LOCAL=1 through coll_cache_lookup_i64; time = the "
+            "library's per-step log (host timer around launch and wait of the extraction kernel)"}
+
+
+def random_row_ceiling(hip, torch, emb, rows, row_bytes, dev, stream, note):
+    """What rows of this size reach over the host link at all: a stand-alone gather (ugk_gather_direct_i64, no table) of
+    uniformly random rows out of the whole pinned table, timed with two HIP events around 5 launches, for several grid
+    caps; the best is the ceiling a miss stream of such rows can be measured against."""
+    n = max(1 << 16, min(1 << 20, (256 << 20) // row_bytes))
+    g = torch.Generator(device=dev).manual_seed(11)
+    keys = torch.randint(0, rows, (n,), generator=g, device=dev, dtype=torch.int64)
+    dst = torch.empty((n, row_bytes), dtype=torch.uint8, device=dev)
+    st = torch.zeros(4, dtype=torch.int32, device=dev)
+    ev = [ctypes.c_void_p(), ctypes.c_void_p()]
+    for e in ev:
+        hip.call("ugk_event_create", ctypes.byref(e))
+    res = {}
+    for blocks in (0, 2048, 512, 128):
+        def go():
+            hip.call("ugk_gather_direct_i64", emb.data_ptr(), rows, keys.data_ptr(), n, dst.data_ptr(), row_bytes,
+                     blocks, st.data_ptr(), None, stream)
+        go()
+        torch.cuda.synchronize()
+        hip.call("ugk_event_record", ev[0], stream)
+        for _ in range(5):
+            go()
+        hip.call("ugk_event_record", ev[1], stream)
+        torch.cuda.synchronize()
+        ms = ctypes.c_float()
+        hip.call("ugk_event_elapsed_ms", ev[0], ev[1], ctypes.byref(ms))
+        res["workgroups_%s" % (blocks or "unlimited")] = n * row_bytes * 5 / (ms.value * 1e-3) / 1e9
+    for e in ev:
+        hip.call("ugk_event_destroy", e)
+    if int(st[0].item()) != 0:
+        sys.exit("bench.py: the random-row probe read outside the table")
+    best = max(res.values())
+    note("random %d-byte rows over the link: best %.1f GB/s" % (row_bytes, best))
+    return {"best_GBps": best, "by_grid_cap_GBps": res, "rows_per_launch": n, "row_bytes": row_bytes,
+            "span_bytes": rows * row_bytes, "how": "ugk_gather_direct_i64 of uniformly random rows of the pinned table, "
+            "2 HIP events around 5 launches"}
+
+
+# what a leg contributes to the default line: enough to recompute both halves of the metric
+LEG_KEYS = ("value", "unit", "ms_per_step", "ms_per_step_spread", "steps", "warmup", "config", "hit_rate",
+            "effective_extraction_GBps", "parity", "stages_us", "roofline", "host_link", "cpu_baseline", "gpu_over_cpu",
+            "refresh", "setup_seconds", "stream_ordered")
+DEFAULT_LEGS = ("c3_gnn_100Mx128xfp32_1M_i64_zipf0.9_cache25pct", "c5_hash_500Mx64xfp16_1M_i64_zipf1.05_cache50M")
+
+
+def run_child(workload, args, cpu_seconds):
+    """one workload in a child process (this process has not touched the GPU); returns its JSON line as a dict"""
+    import subprocess
+
+    cmd = [sys.executable, os.path.abspath(__file__), "--workload", workload, "--cpu-seconds", str(cpu_seconds)]
+    if args.steps is not None:
+        cmd += ["--steps", str(args.steps)]
+    if args.warmup is not None:
+        cmd += ["--warmup", str(args.warmup)]
+    if args.pool is not None:
+        cmd += ["--pool", str(args.pool)]
+    t0 = time.perf_counter()
+    proc = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=None, text=True)
+    lines = [l for l in proc.stdout.splitlines() if l.startswith("{")]
+    if proc.returncode != 0 or not lines:
+        return None, "exit status %d after %.0f s" % (proc.returncode, time.perf_counter() - t0)
+    return json.loads(lines[-1]), None
+
+
+def run_default(args):
+    main_name = "c2_all_hit_10Mx128xfp32_262144_u32_uniform"
+    result, err = run_child(main_name, args, args.cpu_seconds)
+    if result is None:
+        sys.exit("bench.py: the all-hit configuration failed: %s" % err)
+    legs = {}
+    if not args.no_legs:
+        for name in DEFAULT_LEGS:
+            leg, err = run_child(name, args, min(args.cpu_seconds, 5.0))
+            if leg is None:
+                # a leg that cannot report (a parity failure ends it without a number) takes the whole line with it
+                sys.exit("bench.py: leg %s failed: %s" % (name, err))
+            legs[name] = {k: leg[k] for k in LEG_KEYS if k in leg}
+    result["legs"] = legs
+    result["legs_note"] = ("each leg is the same bench.py with --workload <name>, run after the top-level workload in "
+                           "a process of its own, same --steps and --warmup; value / roofline / cpu_baseline at the top "
+                           "level are the all-hit configuration's alone")
     emit(result)
 
 
@@ -643,6 +870,8 @@ def emit(result):
 def main():
     global _REAL_STDOUT
     args = parse_args()
+    if args.workload is None:
+        return run_default(args)
     # the library prints the reference's progress lines ("test_result:init:...", solver summary) on stdout; they go
     # to stderr here so that stdout carries the result line only
     sys.stdout.flush()
@@ -656,10 +885,7 @@ def main():
 
     hip.lib()  # the HIP library must be there: no fallback path exists
     torch.cuda.set_device(0)
-    if args.workload in ALL_HIT:
-        run_all_hit(args)
-    else:
-        run_mixed(args)
+    emit(run_all_hit(args) if args.workload in ALL_HIT else run_mixed(args))
 
 
 if __name__ == "__main__":

@@ -200,6 +200,17 @@ int ugk_classify_i64(ugk_table_t t, const int64_t *keys_dev, size_t n, uint64_t 
                      ugk_idx_t *idx_dev, uint32_t *counts_dev, uint32_t *next_counts_dev, uint32_t *status_dev,
                      uint32_t *host_mirror, void *stream);
 
+/* ---- the keys the cache does not serve: the COLL_SKIP_LOCAL pre-filter of GetMissCacheIndex
+ *      (cache_context.cu:728-741: CubSelectIndex with CubSelectOpLocIsNot, then SelectArrayByIdx) ---------------------
+ * ugk_nonlocal_flags_*: bit i of flags_dev (ceil(n / 64) words, every word written) = key i is not found in the table
+ * with the local location (it is found with the host's, or not at all).  The ascending positions of the set bits come
+ * from ugk_bitmap_count + ugk_bitmap_emit (below), which is the reference's stable select; ugk_select_keys_*:
+ * out_dev[j] = keys_dev[sel_dev[j]] for j < m. */
+int ugk_nonlocal_flags_u32(ugk_table_t t, const uint32_t *keys_dev, size_t n, uint64_t *flags_dev, void *stream);
+int ugk_nonlocal_flags_i64(ugk_table_t t, const int64_t *keys_dev, size_t n, uint64_t *flags_dev, void *stream);
+int ugk_select_keys_u32(const uint32_t *keys_dev, const uint32_t *sel_dev, size_t m, uint32_t *out_dev, void *stream);
+int ugk_select_keys_i64(const int64_t *keys_dev, const uint32_t *sel_dev, size_t m, int64_t *out_dev, void *stream);
+
 /* ---- single-kernel mixed-source extraction: kDirectNoGroup with DataIterMixLoc
  *      (cache_context.cu:137-159, 1295-1329): lookup and gather fused, source picked per row ----------
  * group_counts_host (may be NULL): pinned, GPU-mapped host memory (ugk_host_malloc) of ugk_extract_mix_max_groups()

@@ -1185,6 +1185,52 @@ def test_lookup_of_the_distinct_keys_with_inverse(pct, table_kind, kdtype, monke
     assert _basics.last_group_offset(0)[2] == len(keys)
 
 
+@pytest.mark.parametrize("table_kind", ["FLAT", "HASH"])
+@pytest.mark.parametrize("impl", ["", "SMMaskPhase", "NONE"])
+@pytest.mark.parametrize("kdtype", [torch.int32, torch.int64])
+def test_skip_local_extracts_only_what_the_cache_does_not_hold(table_kind, impl, kdtype, monkeypatch):
+    """COLL_SKIP_LOCAL=1, the reference's aid for timing the other sources alone (cache_context.cu:728-741): the keys the
+    cache serves are dropped in front of the extraction, the rest keep their order and their rows fill the first rows
+    of the output (the reference numbers the destinations by position in the compacted key list); what lies behind
+    them is not touched.  The variable is read by every lookup, so it can be switched on and off on a built cache."""
+    monkeypatch.setenv("COLL_HASH_TABLE", table_kind)
+    if impl:
+        monkeypatch.setenv("SAMGRAPH_COLL_CACHE_CONCURRENT_LINK_IMPL", impl)
+    rng = np.random.default_rng(17)
+    n_item, dim, pct = 60_000, 32, 0.2
+    co.config(make_config(n_item, pct))
+    co.coll_cache_record_init(0)
+    perm = rng.permutation(n_item)
+    s0 = perm[zipf_ranks(rng, 100_000, n_item, 1.1)]
+    co.coll_torch_record(0, torch.from_numpy(s0).to(kdtype))
+    emb = co.coll_torch_create_emb_shm(0, n_item, dim, torch.float32)
+    table = fill_table(emb, rng)
+    co.coll_torch_init_t(0, 0, emb, pct)
+    _, nid = expected_cached_set(s0.astype(np.uint32), n_item, pct)
+    for n in (1, 64, 5000, 70_001):
+        keys = perm[zipf_ranks(rng, n, n_item, 1.1)]
+        kt = torch.from_numpy(keys).to(kdtype).cuda()
+        full = co.coll_torch_lookup_key_t_val_ret(0, kt, False).clone()
+        assert full.cpu().numpy().tobytes() == ORC.gather(table, keys.astype(np.int64)).tobytes()
+        miss = keys[nid[keys] != 0]
+        monkeypatch.setenv("COLL_SKIP_LOCAL", "1")
+        # the reused output buffer still holds the rows of the full lookup: the untouched tail is recognisable
+        out = co.coll_torch_lookup_key_t_val_ret(0, kt, False)
+        monkeypatch.delenv("COLL_SKIP_LOCAL")
+        got = out.cpu().numpy()
+        m = len(miss)
+        assert _basics.last_group_offset(0) == [0, 0, m]
+        assert got[:m].tobytes() == ORC.gather(table, miss.astype(np.int64)).tobytes()
+        assert got[m:].tobytes() == full.cpu().numpy()[m:].tobytes()
+        step = _basics.info(0)["lookups"] - 1
+        assert _basics.step_value(step, kLogL1FeatureBytes) == _basics.step_value(step, kLogL1MissBytes) == m * dim * 4
+    # every key cached: nothing is extracted
+    hot = np.nonzero(nid == 0)[0][:1000]
+    monkeypatch.setenv("COLL_SKIP_LOCAL", "1")
+    co.coll_torch_lookup_key_t_val_ret(0, torch.from_numpy(hot).to(kdtype).cuda(), False)
+    assert _basics.last_group_offset(0) == [0, 0, 0]
+
+
 # ---- the GNN-shaped and the DLR-shaped configuration ---------------------------------------------------------------
 def zipf_ranks_dev(n, space, s, gen):
     """zipf_ranks on the device (same inverse CDF), for batches of a million keys and more"""

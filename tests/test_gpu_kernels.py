@@ -722,6 +722,54 @@ def test_dedup_of_small_and_large_batches_sharing_one_workspace(kdtype):
                  ptr(dev_zeros_u32(n)), None, ptr(dev_zeros_u32(1)), None, None)
 
 
+@pytest.mark.parametrize("mode", ["flat", "hash"])
+@pytest.mark.parametrize("kdtype", [np.uint32, np.int64])
+@pytest.mark.parametrize("n", [1, 63, 64, 65, 4097, 200_000])
+def test_nonlocal_flags_and_stable_selection(mode, kdtype, n):
+    """the pre-filter in front of an extraction that skips the cache's rows: bit i = key i is not served by the cache
+    (found with the host's location, or absent), the set bits compacted in ascending order, the keys picked by them —
+    numpy's boolean mask, order kept"""
+    rng = np.random.default_rng(n * 3 + (mode == "hash"))
+    nkeys = 50_000
+    local = rng.choice(nkeys, 15_000, replace=False).astype(kdtype)
+    rest = np.setdiff1d(np.arange(nkeys), local)
+    on_host = rng.choice(rest, 5_000, replace=False).astype(kdtype)  # present, with the host's location
+    if mode == "flat":
+        mem, tb = _make_flat(nkeys)
+    else:
+        mem, tb, _ = _make_hash(20_000)
+    assert _insert(tb, local) == 0
+    assert _insert(tb, on_host, offs_np=on_host.astype(np.uint32), loc=1) == 0
+    keys = rng.integers(0, nkeys, size=n).astype(kdtype)
+    words = (n + 63) // 64
+    flags = dev_bytes(words * 8 + 8, fill=0xAB)
+    d_keys = to_dev(keys)
+    sfx = "i64" if kdtype == np.int64 else "u32"
+    hip.call("ugk_nonlocal_flags_" + sfx, tb, ptr(d_keys), n, ptr(flags), None)
+    sync()
+    want_mask = ~np.isin(keys, local)
+    got_words = to_np(flags, np.uint64)[:words]
+    got_mask = np.unpackbits(got_words.view(np.uint8), bitorder="little")[:n].astype(bool)
+    assert np.array_equal(got_mask, want_mask)
+    assert not np.unpackbits(got_words.view(np.uint8), bitorder="little")[n:].any()  # bits past the batch are clear
+    assert to_np(flags, np.uint64)[words] == 0xABABABABABABABAB  # nothing written past the bitmap
+    ws = dev_bytes(hip.lib().ugk_bitmap_workspace_bytes())
+    total = PinnedArray((2,), np.uint32)
+    hip.call("ugk_bitmap_count", ptr(flags), None, 0, n, ptr(ws), total.ptr, None)
+    sync()
+    m = int(total.array[0])
+    assert m == int(want_mask.sum())
+    if m:
+        sel = dev_zeros_u32(m)
+        out = dev_bytes(m * np.dtype(kdtype).itemsize)
+        hip.call("ugk_bitmap_emit", ptr(flags), None, 0, n, ptr(ws), ptr(sel), m, None)
+        hip.call("ugk_select_keys_" + sfx, ptr(d_keys), ptr(sel), m, ptr(out), None)
+        sync()
+        assert np.array_equal(to_np(sel, np.uint32)[:m], np.nonzero(want_mask)[0])
+        assert np.array_equal(to_np(out, kdtype)[:m], keys[want_mask])
+    total.free()
+
+
 def test_classify_with_destination_map():
     """dst_map redirects the output row of key i; sources and group sizes are unchanged"""
     rng = np.random.default_rng(31)

@@ -477,6 +477,50 @@ static int ExtractMix(ugk_table_t t, const Id64Type *keys, size_t n, const void 
                              s);
 }
 
+static int NonLocalFlags(ugk_table_t t, const IdType *keys, size_t n, uint64_t *flags, StreamHandle s) {
+  return ugk_nonlocal_flags_u32(t, keys, n, flags, s);
+}
+static int NonLocalFlags(ugk_table_t t, const Id64Type *keys, size_t n, uint64_t *flags, StreamHandle s) {
+  return ugk_nonlocal_flags_i64(t, keys, n, flags, s);
+}
+static int SelectKeys(const IdType *keys, const uint32_t *sel, size_t m, IdType *out, StreamHandle s) {
+  return ugk_select_keys_u32(keys, sel, m, out, s);
+}
+static int SelectKeys(const Id64Type *keys, const uint32_t *sel, size_t m, Id64Type *out, StreamHandle s) {
+  return ugk_select_keys_i64(keys, sel, m, out, s);
+}
+
+// COLL_SKIP_LOCAL=1 (cache_context.cu:728-741), a measurement aid of the reference: the keys the local cache serves
+// are dropped in front of the extraction, the others keep their order and are extracted into the first rows of the
+// output, so that the traffic of the other sources can be timed on its own.  Returns how many keys are left; they are
+// in SkipKeys().  One blocking wait, for that count (the reference waits there as well).
+template <typename KeyT>
+size_t ExtractSession::SelectNonLocal(const ugk_table_t &table, const KeyT *nodes, size_t num_nodes,
+                                      StreamHandle stream) {
+  const size_t words = (num_nodes + 63) / 64;
+  const size_t need = words * 8 + num_nodes * 4 + num_nodes * sizeof(KeyT) + ugk_bitmap_workspace_bytes() + 64;
+  if (_skip_handle == nullptr || _skip_handle->nbytes() < need) {
+    _skip_handle = nullptr;
+    _skip_handle = _cache_ctx->_gpu_mem_allocator(need + need / 4);
+    CHECK_NOTNULL(_skip_handle);
+  }
+  // [bitmap | bitmap workspace | compacted keys | selected positions], each 8-byte aligned
+  char *base = _skip_handle->ptr<char>();
+  uint64_t *flags = reinterpret_cast<uint64_t *>(base);
+  void *bm_ws = base + words * 8;
+  _skip_keys = base + words * 8 + (ugk_bitmap_workspace_bytes() + 7) / 8 * 8;
+  uint32_t *sel = reinterpret_cast<uint32_t *>(static_cast<char *>(_skip_keys) + num_nodes * sizeof(KeyT));
+  UGK_CALL(NonLocalFlags(table, nodes, num_nodes, flags, stream));
+  UGK_CALL(ugk_bitmap_count(flags, nullptr, 0, num_nodes, bm_ws, _host_mirror + kMirSkipCount, stream));
+  UGK_CALL(ugk_stream_sync(stream));
+  const size_t m = _host_mirror[kMirSkipCount];
+  CHECK_LE(m, num_nodes);
+  if (m == 0) return 0;
+  UGK_CALL(ugk_bitmap_emit(flags, nullptr, 0, num_nodes, bm_ws, sel, m, stream));
+  UGK_CALL(SelectKeys(nodes, sel, m, static_cast<KeyT *>(_skip_keys), stream));
+  return m;
+}
+
 // group sizes of the last fused launch: the sum of the words its workgroups left in pinned host memory
 void ExtractSession::SumMixCounts() {
   const uint64_t *w = _mix_counts->ptr<uint64_t>();
@@ -526,7 +570,8 @@ void ExtractSession::ExtractFeatImpl(const KeyT *nodes, size_t num_nodes, void *
   const KeyT *input_nodes = nodes;
   const uint32_t *dst_map = nullptr, *inverse = nullptr;
   float ms_dedup = 0;
-  if (RunConfig::dedup_keys && num_nodes >= RunConfig::dedup_min_keys && !_skip_dedup) {
+  const bool skip_local = !ctx->IsDirectMapping() && GetEnv("COLL_SKIP_LOCAL") == "1";
+  if (RunConfig::dedup_keys && num_nodes >= RunConfig::dedup_min_keys && !_skip_dedup && !skip_local) {
     UGK_CALL(ugk_event_record(_ev_t[2], stream));
     const size_t nu = DedupKeys(nodes, num_nodes, stream);
     UGK_CALL(ugk_event_record(_ev_t[3], stream));
@@ -588,6 +633,17 @@ void ExtractSession::ExtractFeatImpl(const KeyT *nodes, size_t num_nodes, void *
   const uint64_t cache_rows = ctx->_cache_space_capacity;
   const uint64_t host_rows = ctx->_num_total_nodes;
 
+  if (skip_local) {
+    num_nodes = SelectNonLocal(table, nodes, num_nodes, stream);
+    nodes = static_cast<const KeyT *>(_skip_keys);
+    if (num_nodes == 0) {
+      _group_offset[1] = _group_offset[2] = 0;
+      ctx->progress.fetch_add(1);
+      return;
+    }
+  }
+  const size_t nbytes_extracted = skip_local ? num_nodes * rb : nbytes;
+
   // the fused kernel moves 16-byte vectors; rows or buffers that are not multiples of 16 bytes take the factored
   // path, whose gathers fall back to narrower lanes
   const bool vec16 = (((uintptr_t)cache | (uintptr_t)host | (uintptr_t)output | (uintptr_t)rb) & 15u) == 0;
@@ -618,10 +674,10 @@ void ExtractSession::ExtractFeatImpl(const KeyT *nodes, size_t num_nodes, void *
     _group_offset[1] = n_local;
     _group_offset[2] = (uint32_t)num_nodes;
     if (profiler && task_key != 0xffffffffffffffffull) {
-      profiler->LogStep(task_key, kLogL1FeatureBytes, nbytes);
+      profiler->LogStep(task_key, kLogL1FeatureBytes, nbytes_extracted);
       profiler->LogStep(task_key, kLogL1MissBytes, (double)n_miss * rb);
       profiler->LogStep(task_key, kLogL3CacheCombineCacheTime, mix_ms * 1e-3);
-      profiler->LogEpochAdd(task_key, kLogEpochFeatureBytes, nbytes);
+      profiler->LogEpochAdd(task_key, kLogEpochFeatureBytes, nbytes_extracted);
       profiler->LogEpochAdd(task_key, kLogEpochMissBytes, (double)n_miss * rb);
     }
     ctx->progress.fetch_add(1);
@@ -708,7 +764,7 @@ void ExtractSession::ExtractFeatImpl(const KeyT *nodes, size_t num_nodes, void *
   if (dst_map) UGK_CALL(ugk_event_elapsed_ms(_ev_t[2], _ev_t[3], &ms_dedup));
   ms_idx += ms_dedup;
   if (profiler && task_key != 0xffffffffffffffffull) {
-    profiler->LogStep(task_key, kLogL1FeatureBytes, nbytes);
+    profiler->LogStep(task_key, kLogL1FeatureBytes, nbytes_extracted);
     profiler->LogStep(task_key, kLogL1MissBytes, (double)n_miss * rb);
     profiler->LogStep(task_key, kLogL1RemoteBytes, 0);
     profiler->LogStep(task_key, kLogL3CacheGetIndexTime, ms_idx * 1e-3);

@@ -91,7 +91,8 @@ class ExtractSession {
   // words of the device-side state block (64 zero-filled uint32)
   enum StateWord { kStCounts0 = 0, kStCounts1 = 2, kStStatus = 4, kStNumUnique = 5, kStDrainEntries = 6 };
   // words of the pinned host mirror the kernels write; [1] and [2] are indexed 1 + location
-  enum MirrorWord { kMirError = 0, kMirGroupSizes = 1, kMirNumUnique = 3, kMirDrainCount = 4, kMirDrainMore = 5 };
+  enum MirrorWord { kMirError = 0, kMirGroupSizes = 1, kMirNumUnique = 3, kMirDrainCount = 4, kMirDrainMore = 5,
+                    kMirSkipCount = 6 };
   std::shared_ptr<CacheContext> _cache_ctx;
   MemHandle _idx_handle;          // ugk_idx_t[n], from the caller's allocator, regrown on demand
   MemHandle _state_handle;        // device: two counter pairs + status word
@@ -171,6 +172,11 @@ class ExtractSession {
   size_t ExtractUniqueImpl(const KeyT *nodes, size_t num_nodes, void *output, uint32_t *inverse_out,
                            StreamHandle stream, uint64_t task_key);
   bool _skip_dedup = false;  // the keys handed to ExtractFeatImpl are distinct already
+  // COLL_SKIP_LOCAL=1: the keys the cache does not serve, compacted in their order, and the scratch around them
+  MemHandle _skip_handle;
+  void *_skip_keys = nullptr;
+  template <typename KeyT>
+  size_t SelectNonLocal(const ugk_table_t &table, const KeyT *nodes, size_t num_nodes, StreamHandle stream);
   void EnsureIdx(size_t num_nodes);
   void CheckStatusWord(StreamHandle stream) const;
 

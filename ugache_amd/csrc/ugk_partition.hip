@@ -129,6 +129,30 @@ __global__ __launch_bounds__(kBlock) void classify_kernel(ugk_table_t t, const K
   }
 }
 
+// ---- which keys are NOT served by the cache: one bit per key, a wavefront's ballot is one bitmap word ---------
+template <typename K, int KIND>
+__global__ __launch_bounds__(kBlock) void nonlocal_flags_kernel(ugk_table_t t, const K *__restrict__ keys, size_t n,
+                                                                unsigned long long *__restrict__ flags) {
+  const size_t n_words = (n + kWave - 1) / kWave;
+  const int lane = (int)lane_id();
+  for (size_t w = (size_t)blockIdx.x * kWavesPerBlock + threadIdx.x / kWave; w < n_words;
+       w += (size_t)gridDim.x * kWavesPerBlock) {
+    const size_t i = w * kWave + lane;
+    const bool active = i < n;
+    const uint64_t key = active ? key_to_u64<K>(keys[i]) : 0;
+    const Found f = table_lookup<KIND>(t, key, active);
+    const uint64_t bits = __ballot(active && !(f.hit && f.loc == UGK_LOC_LOCAL));
+    if (lane == 0) flags[w] = bits;
+  }
+}
+
+template <typename K>
+__global__ __launch_bounds__(kBlock) void select_keys_kernel(const K *__restrict__ keys, const uint32_t *__restrict__ sel,
+                                                             size_t m, K *__restrict__ out) {
+  for (size_t j = (size_t)blockIdx.x * kBlock + threadIdx.x; j < m; j += (size_t)gridDim.x * kBlock)
+    out[j] = keys[sel[j]];
+}
+
 // ---- fused lookup + gather: every wavefront resolves 64 keys, then copies their 64 rows ------------------
 template <typename K, int KIND, int LPR, int KPW>
 __global__ __launch_bounds__(kBlock) void extract_mix_kernel(ugk_table_t t, const K *__restrict__ keys, size_t n,
@@ -401,6 +425,37 @@ int classify(ugk_table_t t, const K *keys, size_t n, uint64_t host_rows, const u
   return 0;
 }
 
+template <typename K>
+int nonlocal_flags(ugk_table_t t, const K *keys, size_t n, uint64_t *flags, void *stream) {
+  if (n == 0) return 0;
+  UGK_REQUIRE(keys && flags, "ugk_nonlocal_flags: null keys or bitmap");
+  UGK_REQUIRE((uintptr_t)flags % 8 == 0, "ugk_nonlocal_flags: the bitmap must be 8-byte aligned");
+  UGK_REQUIRE(t.kind == 1 || t.kind == 2, "ugk_nonlocal_flags: table kind %d is not flat(1) or hash(2)", t.kind);
+  UGK_REQUIRE(t.table && t.size, "ugk_nonlocal_flags: empty table");
+  if (t.kind == 2)
+    UGK_REQUIRE(t.size % 8 == 0 && (uintptr_t)t.table % 128 == 0,
+                "ugk_nonlocal_flags: hash table must be 128-byte aligned with a multiple of 8 buckets");
+  const unsigned grid = clamp_grid((n + kBlock - 1) / kBlock, 0);
+  if (t.kind == 1)
+    hipLaunchKernelGGL((nonlocal_flags_kernel<K, 1>), dim3(grid), dim3(kBlock), 0, as_stream(stream), t, keys, n,
+                       reinterpret_cast<unsigned long long *>(flags));
+  else
+    hipLaunchKernelGGL((nonlocal_flags_kernel<K, 2>), dim3(grid), dim3(kBlock), 0, as_stream(stream), t, keys, n,
+                       reinterpret_cast<unsigned long long *>(flags));
+  UGK_HIP(hipGetLastError());
+  return 0;
+}
+
+template <typename K>
+int select_keys(const K *keys, const uint32_t *sel, size_t m, K *out, void *stream) {
+  if (m == 0) return 0;
+  UGK_REQUIRE(keys && sel && out, "ugk_select_keys: null pointer");
+  const unsigned grid = clamp_grid((m + kBlock - 1) / kBlock, 0);
+  hipLaunchKernelGGL(select_keys_kernel<K>, dim3(grid), dim3(kBlock), 0, as_stream(stream), keys, sel, m, out);
+  UGK_HIP(hipGetLastError());
+  return 0;
+}
+
 template <typename K, int KIND>
 int extract_mix_lpr(ugk_table_t t, const K *keys, size_t n, const void *cache, uint64_t cache_rows, const void *host,
                     uint64_t host_rows, void *out, uint32_t vpr, uint32_t *status, uint32_t *host_mirror,
@@ -564,6 +619,19 @@ int ugk_classify_i64(ugk_table_t t, const int64_t *keys_dev, size_t n, uint64_t 
                      uint32_t *host_mirror, void *stream) {
   return classify<int64_t>(t, keys_dev, n, host_rows, dst_map_dev, idx_dev, counts_dev, next_counts_dev, status_dev,
                            host_mirror, stream);
+}
+
+int ugk_nonlocal_flags_u32(ugk_table_t t, const uint32_t *keys_dev, size_t n, uint64_t *flags_dev, void *stream) {
+  return nonlocal_flags<uint32_t>(t, keys_dev, n, flags_dev, stream);
+}
+int ugk_nonlocal_flags_i64(ugk_table_t t, const int64_t *keys_dev, size_t n, uint64_t *flags_dev, void *stream) {
+  return nonlocal_flags<int64_t>(t, keys_dev, n, flags_dev, stream);
+}
+int ugk_select_keys_u32(const uint32_t *keys_dev, const uint32_t *sel_dev, size_t m, uint32_t *out_dev, void *stream) {
+  return select_keys<uint32_t>(keys_dev, sel_dev, m, out_dev, stream);
+}
+int ugk_select_keys_i64(const int64_t *keys_dev, const uint32_t *sel_dev, size_t m, int64_t *out_dev, void *stream) {
+  return select_keys<int64_t>(keys_dev, sel_dev, m, out_dev, stream);
 }
 
 unsigned ugk_extract_mix_max_groups(void) { return clamp_grid(~(size_t)0, 0); }

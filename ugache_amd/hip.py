@@ -87,6 +87,10 @@ SIGNATURES = {
     "ugk_hash_census": [_vp, _sz, _vp, _vp],
     "ugk_classify_u32": [Table, _vp, _sz, _u64, _vp, _vp, _vp, _vp, _vp, _vp, _vp],
     "ugk_classify_i64": [Table, _vp, _sz, _u64, _vp, _vp, _vp, _vp, _vp, _vp, _vp],
+    "ugk_nonlocal_flags_u32": [Table, _vp, _sz, _vp, _vp],
+    "ugk_nonlocal_flags_i64": [Table, _vp, _sz, _vp, _vp],
+    "ugk_select_keys_u32": [_vp, _vp, _sz, _vp, _vp],
+    "ugk_select_keys_i64": [_vp, _vp, _sz, _vp, _vp],
     "ugk_extract_mix_max_groups": [],
     "ugk_extract_mix_u32": [Table, _vp, _sz, _vp, _u64, _vp, _u64, _vp, _sz, _vp, _vp, _vp, _vp, _u32, _vp],
     "ugk_extract_mix_i64": [Table, _vp, _sz, _vp, _u64, _vp, _u64, _vp, _sz, _vp, _vp, _vp, _vp, _u32, _vp],
