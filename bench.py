@@ -540,15 +540,19 @@ def run_mixed(args):
         # HBM side of the fused kernel: key + table entry per key, hit rows read and written, missed rows written
         hit_alg = n_keys * (8 + entry) + n_hit * 2 * row_bytes + n_miss * row_bytes
         t_link = t_hit
-        # keys per wavefront, by the launcher's rule: the fewest whose wavefronts are all resident at once (the hash
-        # probe wants one notch more; the top band of the flat table needs the library's hint of <= 2 % misses)
+        # keys per wavefront, by the launcher's rule (ugk_partition.hip): short wavefronts except where the lookups
+        # weigh more (small rows, the hash probe)
         slots = hip.device_info(0)["compute_units"] * 4 * 8
         lpr = min(64, max(1, 1 << (max(1, row_bytes // 16) - 1).bit_length()))
+        small_rows = lpr <= 8
         if info_cache["table_kind"] == 1:
-            kpw = 8 if n_keys <= slots * 8 else 16 if n_keys <= slots * 16 else \
-                32 if n_keys <= slots * 32 and n_miss * 50 <= n_keys else 64
+            kpw = 32 if small_rows else 8
+        elif n_keys <= slots:
+            kpw = 8
+        elif small_rows:
+            kpw = 32 if n_keys <= slots * 16 else 64
         else:
-            kpw = 16 if n_keys <= slots * 8 else 32 if n_keys <= slots * 16 else 64
+            kpw = 16 if n_keys <= slots * 8 else 32 if n_keys <= slots * 16 else 64 if n_keys <= slots * 32 else 16
         kpw = max(kpw, 64 // lpr)
         kernel_name = ("extract_mix_kernel<long,%d,%d,%d> (lookup + both gathers; bound by the host link, see "
                        "host_link)" % (info_cache["table_kind"], lpr, kpw))

@@ -71,6 +71,11 @@ void coll_cache_init_ranked_c(int replica_id, size_t key_space_size, const uint3
                               const uint32_t *rank_freq, coll_cache_alloc_fn alloc, coll_cache_release_fn release,
                               void *user, void *cpu_data, int dtype, size_t dim, double cache_percentage,
                               StreamHandle stream);
+/* CollCache::build (coll_cache_lib/facade.h:52-54, facade.cc:38-72) for C callers: builds every replica from the
+ * placement the library already holds, with an allocator made per replica from the callback pair.  A cache of 0 % or
+ * 100 % needs no placement; a partial one needs an earlier coll_cache_init* to have solved (build places nothing). */
+void coll_cache_build_all_c(coll_cache_alloc_fn alloc, coll_cache_release_fn release, void *user, void *cpu_data,
+                            int dtype, size_t dim, double cache_percentage, StreamHandle stream);
 /* 64-bit (dense) keys: siblings of coll_cache_lookup / coll_cache_record.  The reference is uint32 end to end
  * (coll_cache_lib/constant.h:28). */
 void coll_cache_lookup_i64(int replica_id, const int64_t *key, size_t num_keys, void *output, StreamHandle stream);

@@ -39,7 +39,11 @@ extern "C" {
 #define UGK_EMPTY_U32 0xffffffffu /* cache_hashtable.h:17 kEmptyPos */
 
 /* One gather work item.  Takes the place of SrcKeyDstVal (cache_context.h:47-52); the location is not
- * stored because every group holds one location only. */
+ * stored because every group holds one location only.
+ * Both fields are 32 bits, as in the reference: an index list addresses outputs of up to 2^32 rows and sources of up
+ * to 2^32 rows.  ugk_classify_* therefore flags (UGK_ST_KEY_OUT_OF_RANGE) a key whose host row does not fit 32 bits
+ * instead of listing it, so the factored extraction (ugk_classify_* + ugk_gather_group) serves host tables of up to
+ * 2^32 rows; ugk_extract_mix_* and ugk_gather_direct_i64 carry 64-bit rows and have no such limit. */
 typedef struct {
   uint32_t dst_off; /* output row */
   uint32_t src_off; /* row inside the group's source (cache slot, or host row) */
@@ -85,7 +89,7 @@ typedef struct {
 const char *ugk_last_error(void);
 /* version of this ABI; bumped on any signature change.  ugk_abi_version() is what the loaded library was built with:
  * a caller compiled against another UGK_ABI_VERSION must not go on. */
-#define UGK_ABI_VERSION 4
+#define UGK_ABI_VERSION 5
 int ugk_abi_version(void);
 
 /* ---- runtime plumbing: Device::{AllocDataSpace,FreeDataSpace,CopyDataFromTo,StreamSync,CreateStream}
@@ -127,6 +131,17 @@ int ugk_copy_rows(void *dst_dev, const void *src_dev, size_t nbytes, void *strea
 /* ---- gather: extract_data + Combine (cache_context.cu:214-231, 1076-1100) -----------------------
  * out[dst(i), :] = src[srcrow(i), :] for row_bytes bytes.  max_blocks = 0 lets the kernel fill the
  * chip; a non-zero value caps the grid (the reference's limit_block / per-source SM budget). */
+/* Where the rows an extraction writes go next, for the launches the calling thread makes from now on (the gathers and
+ * ugk_extract_mix_*).  UGK_OUTPUT_AUTO: decided by size — an output of up to 192 MB is written with ordinary stores and
+ * stays in the 256 MB memory-side cache for its consumer, a larger one with non-temporal stores.  UGK_OUTPUT_STREAMS:
+ * non-temporal stores whatever the size (a caller that rotates its outputs over more buffers than the cache holds: the
+ * rows of one launch are evicted by the next anyway, and evicting them costs more than streaming them, 51.4 us against
+ * 47.5 us for 262,144 rows of 512 bytes).  UGK_OUTPUT_STAYS: ordinary stores whatever the size.  Never a byte of the
+ * result depends on it.  The environment variable UGK_GATHER_NT_STORE=0/1 overrides both. */
+#define UGK_OUTPUT_AUTO 0
+#define UGK_OUTPUT_STREAMS 1
+#define UGK_OUTPUT_STAYS 2
+int ugk_set_output_hint(int hint);
 /* IdxStoreDirect (cache_context.h:341-354): srcrow = keys[i], dst = i */
 int ugk_gather_direct_u32(const void *src_dev, uint64_t src_rows, const uint32_t *keys_dev, size_t n, void *out_dev,
                           size_t row_bytes, unsigned max_blocks, uint32_t *status_dev, uint32_t *host_mirror,

@@ -110,6 +110,31 @@ def test_torch_surface_has_the_reference_entry_points():
     assert co.kCollCacheAsymmLink == 13
 
 
+def test_c_lib_module_of_the_torch_binding():
+    """`from collcache.torch import c_lib` (python/collcache/torch/adapter.py:25) gives a module with the six entry
+    points PYBIND11_MODULE(c_lib, m) defines (adapter.cc:274-281), with the C++ functions' parameter order"""
+    import inspect
+    pytest.importorskip("torch")
+    sys.path.insert(0, os.path.join(ROOT, "ugache_amd"))
+    from collcache.torch import c_lib
+    import collcache.torch as co
+    want = {
+        "coll_torch_init": ["replica_id", "key_space_size", "dev_id", "cpu_data", "dim", "cache_percentage",
+                            "use_fp16"],                                       # adapter.cc:126-128
+        "coll_torch_init_t": ["replica_id", "dev_id", "emb", "cache_percentage"],  # adapter.cc:151
+        "coll_torch_test": ["local_id", "keys"],                                # adapter.cc:192
+        "coll_torch_record": ["local_id", "keys"],                              # adapter.cc:270
+        "coll_torch_lookup_key_t_val_ret": ["local_id", "keys", "pad_to_8"],    # adapter.cc:204
+        "coll_torch_create_emb_shm": ["replica_id", "n_keys", "dim", "dtype", "fname"],  # adapter.cc:239
+    }
+    for name, params in want.items():
+        fn = getattr(c_lib, name, None)
+        assert callable(fn), name
+        assert [p for p in inspect.signature(fn).parameters][: len(params)] == params, name
+        # the adapter's function of the same name forwards to it
+        assert callable(getattr(co, name)) and getattr(co, name) is not fn
+
+
 def test_serving_module_has_the_tf2_bindings_entry_points():
     """collcache.torch.serving carries the names the reference's inference scripts call on collcache_tf2
     (python_tf2/collcache_tf2/collcache_tf2/core/initialize.py:33-39, 79, 129, 292; core/lookup_layer.py:22;

@@ -100,6 +100,51 @@ def test_direct_mapping_full_and_no_cache(kdtype, pct):
     assert _basics.info(0)["lookups"] == 8
 
 
+@pytest.mark.parametrize("pct", [1.0, 0.0, 0.3])
+def test_build_of_every_replica_with_an_allocator_builder(pct):
+    """CollCache::build(allocator_builder, ...) (facade.h:52-54, facade.cc:38-72) through its C hook: every replica
+    (the one) is built with the allocator the builder makes for it, from the placement the object holds.  A partial
+    cache is first built by coll_cache_init, then rebuilt the reference's way from the same placement."""
+    import ctypes
+    from collcache.torch import c_lib
+    rng = np.random.default_rng(3)
+    n_item, dim = 30_000, 64
+    co.config(make_config(n_item, pct))
+    co.coll_cache_record_init(0)
+    perm = rng.permutation(n_item)
+    s0 = perm[zipf_ranks(rng, 60_000, n_item, 1.1)]
+    emb = co.coll_torch_create_emb_shm(0, n_item, dim, torch.float32)
+    table = fill_table(emb, rng)
+    nid = None
+    if 0.0 < pct < 1.0:
+        co.coll_torch_record(0, torch.from_numpy(s0))
+        co.coll_torch_init_t(0, 0, emb, pct)  # solves the placement
+        _, nid = expected_cached_set(s0.astype(np.uint32), n_item, pct)
+    else:
+        c_lib._State.dev_id[0] = 0
+        c_lib._setup_dims(dim, False)
+    handed_out = []
+    alloc, release = c_lib._make_allocator(0)
+
+    def counting_alloc(nbytes, user):
+        handed_out.append(nbytes)
+        return alloc(nbytes, user)
+
+    cb = c_lib.ALLOC_FN(counting_alloc)
+    stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    _basics.C_LIB_CTYPES.coll_cache_build_all_c(cb, release, None, emb.data_ptr(), co.kF32, dim, pct, stream)
+    info = _basics.info(0)
+    assert info["cached_rows"] == (n_item if pct == 1.0 else 0 if pct == 0.0 else int((nid == 0).sum()))
+    for n in (1, 5000, 40_000):
+        keys = perm[zipf_ranks(rng, n, n_item, 1.1)]
+        out = co.coll_torch_lookup_key_t_val_ret(0, torch.from_numpy(keys).cuda(), False)
+        assert out.cpu().numpy().tobytes() == ORC.gather(table, keys).tobytes()
+        want_local = n if pct == 1.0 else 0 if pct == 0.0 else int((nid[keys] == 0).sum())
+        assert _basics.last_group_offset(0) == [0, want_local, n]
+    if 0.0 < pct < 1.0:
+        assert handed_out  # the factored / dedup scratch of a partial cache comes from the builder's allocator
+
+
 @pytest.mark.parametrize("table_kind", ["FLAT", "HASH"])
 @pytest.mark.parametrize("impl", ["", "SMMaskPhase", "DIRECT", "NONE"])
 @pytest.mark.parametrize("kdtype", [torch.int32, torch.int64])

@@ -521,6 +521,28 @@ size_t ExtractSession::SelectNonLocal(const ugk_table_t &table, const KeyT *node
   return m;
 }
 
+void ExtractSession::NoteOutput(const void *output, size_t nbytes) {
+  int hint = _out_hint;
+  if (_out_ptr[(_out_next + kOutRing - 1) % kOutRing] != output || _out_bytes[(_out_next + kOutRing - 1) % kOutRing] != nbytes) {
+    _out_ptr[_out_next] = output;
+    _out_bytes[_out_next] = nbytes;
+    _out_next = (_out_next + 1) % kOutRing;
+    // bytes of the distinct buffers among the last few outputs (the ring only grows on a change of buffer, so one
+    // reused buffer occupies one entry)
+    size_t distinct = 0;
+    for (int i = 0; i < kOutRing; i++) {
+      bool seen = _out_ptr[i] == nullptr;
+      for (int j = 0; j < i && !seen; j++) seen = _out_ptr[j] == _out_ptr[i];
+      if (!seen) distinct += _out_bytes[i];
+    }
+    hint = distinct > ((size_t)192 << 20) ? UGK_OUTPUT_STREAMS : UGK_OUTPUT_AUTO;
+  }
+  // the hint is a thread's own in the kernel library: set it on every call that may come from another thread than
+  // the last one did, which costs a store
+  UGK_CALL(ugk_set_output_hint(hint));
+  _out_hint = hint;
+}
+
 // group sizes of the last fused launch: the sum of the words its workgroups left in pinned host memory
 void ExtractSession::SumMixCounts() {
   const uint64_t *w = _mix_counts->ptr<uint64_t>();
@@ -563,6 +585,7 @@ void ExtractSession::ExtractFeatImpl(const KeyT *nodes, size_t num_nodes, void *
   }
   CHECK_NOTNULL(nodes);
   CHECK_NOTNULL(output);
+  NoteOutput(output, nbytes);
 
   // with deduplication the extraction proper runs over the distinct keys and writes each row where the key first
   // occurs; the duplicates are filled in from there at the end
@@ -783,6 +806,7 @@ void ExtractSession::ExtractFeatAsyncImpl(const KeyT *nodes, size_t num_nodes, v
   CHECK_NOTNULL(nodes);
   CHECK_NOTNULL(output);
   const bool dedup = RunConfig::dedup_keys && num_nodes >= RunConfig::dedup_min_keys;
+  NoteOutput(output, num_nodes * rb);
   NoteAsyncStream(stream);  // before the first kernel is enqueued: a refresh that does not see the stream yet has
                             // finished its evictions before that kernel can start
   if (ctx->IsDirectMapping() && !dedup) {

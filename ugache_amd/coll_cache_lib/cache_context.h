@@ -171,6 +171,15 @@ class ExtractSession {
   template <typename KeyT>
   size_t ExtractUniqueImpl(const KeyT *nodes, size_t num_nodes, void *output, uint32_t *inverse_out,
                            StreamHandle stream, uint64_t task_key);
+  // Where the outputs of the last lookups went.  A caller that hands the same buffer over every time (the reference's
+  // adapter does, adapter.cc:204-237) finds its rows in the memory-side cache; one that rotates over more buffers than
+  // that cache holds is better served by streaming stores, and the kernels are told so (ugk_set_output_hint).
+  static constexpr int kOutRing = 8;
+  const void *_out_ptr[kOutRing] = {nullptr};
+  size_t _out_bytes[kOutRing] = {0};
+  int _out_next = 0;
+  int _out_hint = UGK_OUTPUT_AUTO;
+  void NoteOutput(const void *output, size_t nbytes);
   bool _skip_dedup = false;  // the keys handed to ExtractFeatImpl are distinct already
   // COLL_SKIP_LOCAL=1: the keys the cache does not serve, compacted in their order, and the scratch around them
   MemHandle _skip_handle;

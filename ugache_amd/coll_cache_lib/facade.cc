@@ -149,6 +149,18 @@ void CollCache::build_common(int replica_id, std::function<void()> solve, IdType
                     RunConfig::refresher_omp_thread_num / (int)RunConfig::num_device);
 }
 
+// facade.cc:38-72
+void CollCache::build(std::function<std::function<MemHandle(size_t)>(int)> allocator_builder, void *cpu_data,
+                      DataType dtype, size_t dim, double cache_percentage, StreamHandle stream) {
+  const bool partial = cache_percentage != 0 && cache_percentage != 1;
+  CHECK(!partial || (_nid_to_block != nullptr && _block_access_advise != nullptr))
+      << "CollCache::build places nothing itself: a partial cache needs the placement of an earlier build_v2 / refresh";
+  const IdType num_node = partial ? (IdType)_nid_to_block->Shape()[0] : (IdType)RunConfig::num_total_item;
+  for (size_t replica_id = 0; replica_id < RunConfig::num_device; replica_id++)
+    build_common((int)replica_id, []() {}, num_node, allocator_builder((int)replica_id), cpu_data, dtype, dim,
+                 cache_percentage, stream);
+}
+
 // facade.cc:283-381
 void CollCache::build_v2(int replica_id, IdType *ranking_nodes_list_ptr, IdType *ranking_nodes_freq_list_ptr,
                          IdType num_node, std::function<MemHandle(size_t)> gpu_mem_allocator, void *cpu_data,

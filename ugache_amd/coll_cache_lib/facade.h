@@ -44,6 +44,11 @@ class CollCache : public std::enable_shared_from_this<CollCache> {
   CollCache(BarHandle process_barrier, BarHandle replica_barrier)
       : _process_barrier(process_barrier), _replica_barrier(replica_barrier), _profiler(std::make_shared<Profiler>()) {}
 
+  // facade.h:52-54, facade.cc:38-72: builds every replica (here: the one) with the allocator `allocator_builder` makes
+  // for it, from the placement the object already holds; a partial cache therefore needs a build_v2 or refresh to have
+  // solved before (the reference's own solve() in front of it is dead code), 0 % and 100 % need nothing
+  void build(std::function<std::function<MemHandle(size_t)>(int)> allocator_builder, void *cpu_data, DataType dtype,
+             size_t dim, double cache_percentage, StreamHandle stream = nullptr);
   // nodes / output are device pointers; blocking: output is complete on return (facade.cc:74-88)
   void lookup(int replica_id, const IdType *nodes, const size_t num_nodes, void *output, StreamHandle stream,
               uint64_t step_key);

@@ -283,6 +283,16 @@ void coll_cache_init_ranked_c(int replica_id, size_t key_space_size, const uint3
                         cache_percentage, stream);
 }
 
+void coll_cache_build_all_c(coll_cache_alloc_fn alloc, coll_cache_release_fn release, void *user, void *cpu_data,
+                            int dtype, size_t dim, double cache_percentage, StreamHandle stream) {
+  CHECK(RunConfig::is_configured);
+  CHECK_NOTNULL(_coll_cache);
+  DataType dt = static_cast<DataType>(dtype);
+  NormalizeHalf(dt, dim);
+  _coll_cache->build([=](int replica_id) { return MakeAllocator(alloc, release, user, replica_id); }, cpu_data, dt, dim,
+                     cache_percentage, stream);
+}
+
 void coll_cache_set_key_map(uint64_t mul, int bits) {
   CHECK(RunConfig::is_configured) << "coll_cache_config comes first";
   CHECK(_coll_cache == nullptr || _coll_cache->num_replicas_built() == 0) << "the key map cannot change after the build";

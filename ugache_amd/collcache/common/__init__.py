@@ -106,6 +106,8 @@ C_API = {
     "coll_cache_init_ranked_c": (None, [ctypes.c_int, ctypes.c_size_t, ctypes.c_void_p, ctypes.c_void_p, ALLOC_FN,
                                         RELEASE_FN, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int, ctypes.c_size_t,
                                         ctypes.c_double, ctypes.c_void_p]),
+    "coll_cache_build_all_c": (None, [ALLOC_FN, RELEASE_FN, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int,
+                                      ctypes.c_size_t, ctypes.c_double, ctypes.c_void_p]),
     "coll_cache_lookup_i64": (None, [ctypes.c_int, ctypes.c_void_p, ctypes.c_size_t, ctypes.c_void_p,
                                      ctypes.c_void_p]),
     "coll_cache_record_i64": (None, [ctypes.c_int, ctypes.c_void_p, ctypes.c_size_t]),

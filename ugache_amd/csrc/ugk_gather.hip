@@ -4,14 +4,14 @@
 // flight rather than around arithmetic:
 //   * a row of V 16-byte vectors is copied by LPR = min(64, pow2ceil(V)) adjacent lanes, so one wavefront
 //     instruction moves 64/LPR whole rows as fully coalesced segments (512-B rows: 2 rows, 128-B rows: 8);
-//   * every lane keeps UNROLL = 2 independent rows in flight (both loads issued before the first store) and
-//     the launch uses many small workgroups (one or two passes each): measured on MI355X this beats deeper
-//     unrolling with fewer, longer-lived workgroups by ~15 %;
+//   * every lane keeps UNROLL = 2 independent rows in flight (both loads issued before the first store) and the
+//     launch uses many small workgroups of one pass each:
+//     measured on MI355X this beats deeper unrolling with fewer, longer-lived workgroups by ~15 %;
 //   * loads carry the non-temporal hint (table rows are touched once); stores are ordinary write-back stores
 //     while the output fits the 256 MB memory-side cache, so the consumer finds it there, and non-temporal
-//     beyond that;
-//   * the grid is a grid-stride launch sized from the CU count, or capped by the caller so a host-link
-//     gather occupies only a few CUs while the HBM gather runs next to it;
+//     beyond that or when the caller says its outputs do not stay there (ugk_set_output_hint);
+//   * the grid has one workgroup per pass of rows, or is capped by the caller so a host-link gather occupies
+//     only a few CUs while the HBM gather runs next to it (then the workgroups stride over the batch);
 //   * keys / index records are range-checked against the source's row count: a bad key sets a status bit
 //     and its row is skipped instead of faulting.
 #include <cstdlib>
@@ -72,11 +72,13 @@ __device__ __forceinline__ void st_stream(V *p, V v) {
   __builtin_nontemporal_store(v, p);
 }
 
-template <typename V, int LPR, int UNROLL, typename Idx>
+// NT_STORE is a template parameter, not a launch argument: with a run-time flag the optimiser merges the two stores
+// of `if (nt) stream(p, v); else *p = v;` into one and the non-temporal hint is lost (seen with UNROLL = 1).
+template <typename V, int LPR, int UNROLL, bool NT_STORE, typename Idx>
 __global__ __launch_bounds__(kBlock) void gather_kernel(Idx ix, const V *__restrict__ src, uint64_t src_rows,
                                                         V *__restrict__ out, uint64_t out_rows, uint32_t vpr,
                                                         const uint32_t *__restrict__ counts, uint32_t group, size_t n,
-                                                        uint32_t *status, uint32_t *host_mirror, bool nt_store) {
+                                                        uint32_t *status, uint32_t *host_mirror) {
   size_t begin = 0, count = n;
   if (counts) {
     const uint32_t c = counts[group];
@@ -90,22 +92,23 @@ __global__ __launch_bounds__(kBlock) void gather_kernel(Idx ix, const V *__restr
   constexpr size_t kPerIter = (size_t)RPB * UNROLL;
 
   for (size_t base = (size_t)blockIdx.x * kPerIter; base < count; base += (size_t)gridDim.x * kPerIter) {
+    // the index words of all rows of the pass first, in flight together (a row past the end takes the last one's),
+    // then the checks: a check between two of them would make the second wait for the first
     uint64_t s[UNROLL], d[UNROLL];
     bool ok[UNROLL];
 #pragma unroll
     for (int u = 0; u < UNROLL; ++u) {
       const size_t r = base + (size_t)u * RPB + rib;
       ok[u] = r < count;
-      s[u] = 0;
-      d[u] = 0;
-      if (ok[u]) {
-        ix.get(begin + r, s[u], d[u]);
-        if (s[u] >= src_rows || d[u] >= out_rows) {
-          ok[u] = false;
-          if (lane == 0) {
-            atomicOr(status, UGK_ST_KEY_OUT_OF_RANGE);
-            if (host_mirror) host_mirror[0] = UGK_ST_KEY_OUT_OF_RANGE;
-          }
+      ix.get(begin + (ok[u] ? r : count - 1), s[u], d[u]);
+    }
+#pragma unroll
+    for (int u = 0; u < UNROLL; ++u) {
+      if (ok[u] && (s[u] >= src_rows || d[u] >= out_rows)) {
+        ok[u] = false;
+        if (lane == 0) {
+          atomicOr(status, UGK_ST_KEY_OUT_OF_RANGE);
+          if (host_mirror) host_mirror[0] = UGK_ST_KEY_OUT_OF_RANGE;
         }
       }
     }
@@ -119,7 +122,7 @@ __global__ __launch_bounds__(kBlock) void gather_kernel(Idx ix, const V *__restr
 #pragma unroll
         for (int u = 0; u < UNROLL; ++u)
           if (ok[u]) {
-            if (nt_store) st_stream(out + d[u] * vpr + col, v[u]);
+            if constexpr (NT_STORE) st_stream(out + d[u] * vpr + col, v[u]);
             else out[d[u] * vpr + col] = v[u];
           }
       }
@@ -143,29 +146,42 @@ __global__ __launch_bounds__(kBlock) void replicate_kernel(V *out, uint32_t vpr,
   }
 }
 
-// Non-temporal stores only when the output cannot stay in the memory-side cache anyway.
-// UGK_GATHER_NT_STORE=0/1 forces the choice.
-bool nt_store_for(size_t out_bytes) {
-  static int forced = [] {
-    const char *e = getenv("UGK_GATHER_NT_STORE");
-    return e ? atoi(e) : -1;
-  }();
-  if (forced >= 0) return forced != 0;
-  return out_bytes > ((size_t)192 << 20);
+// A launch that may fill the chip (max_blocks == 0) gets one workgroup per pass of rows, however many that makes:
+// workgroups start in order, so the rows being written at any moment form one window that moves through the output,
+// which the memory side turns into far better write bursts than the same workgroups striding over the whole output
+// (2 M keys of 512 bytes: 360 us against 377 us with 16,384 grid-striding workgroups; 1 M keys: 181 against 187 us).
+unsigned gather_grid(size_t passes, unsigned max_blocks) {
+  if (max_blocks) return clamp_grid(passes, max_blocks);
+  if (passes == 0) passes = 1;
+  return (unsigned)(passes > 0x7fffffffull ? 0x7fffffffull : passes);
+}
+
+template <typename V, int LPR, int UNROLL, typename Idx>
+int launch_unrolled(Idx ix, const void *src, uint64_t src_rows, void *out, uint64_t out_rows, uint32_t vpr,
+                    const uint32_t *counts, uint32_t group, size_t n, unsigned max_blocks, uint32_t *status,
+                    uint32_t *host_mirror, bool nt, hipStream_t stream) {
+  constexpr size_t kPerIter = (size_t)(kBlock / LPR) * UNROLL;
+  const unsigned grid = gather_grid((n + kPerIter - 1) / kPerIter, max_blocks);
+  if (nt)
+    hipLaunchKernelGGL((gather_kernel<V, LPR, UNROLL, true, Idx>), dim3(grid), dim3(kBlock), 0, stream, ix,
+                       reinterpret_cast<const V *>(src), src_rows, reinterpret_cast<V *>(out), out_rows, vpr, counts,
+                       group, n, status, host_mirror);
+  else
+    hipLaunchKernelGGL((gather_kernel<V, LPR, UNROLL, false, Idx>), dim3(grid), dim3(kBlock), 0, stream, ix,
+                       reinterpret_cast<const V *>(src), src_rows, reinterpret_cast<V *>(out), out_rows, vpr, counts,
+                       group, n, status, host_mirror);
+  UGK_HIP(hipGetLastError());
+  return 0;
 }
 
 template <typename V, int LPR, typename Idx>
 int launch_one(Idx ix, const void *src, uint64_t src_rows, void *out, uint64_t out_rows, uint32_t vpr,
                const uint32_t *counts, uint32_t group, size_t n, unsigned max_blocks, uint32_t *status,
                uint32_t *host_mirror, hipStream_t stream) {
-  constexpr int UNROLL = 2;
-  constexpr size_t kPerIter = (size_t)(kBlock / LPR) * UNROLL;
-  const unsigned grid = clamp_grid((n + kPerIter - 1) / kPerIter, max_blocks);
-  hipLaunchKernelGGL((gather_kernel<V, LPR, UNROLL, Idx>), dim3(grid), dim3(kBlock), 0, stream, ix,
-                     reinterpret_cast<const V *>(src), src_rows, reinterpret_cast<V *>(out), out_rows, vpr, counts,
-                     group, n, status, host_mirror, nt_store_for(n * (size_t)vpr * sizeof(V)));
-  UGK_HIP(hipGetLastError());
-  return 0;
+  // two rows in flight per lane; one was measured with streaming stores and is no better (262,144 keys of 512 bytes
+  // into rotating outputs 49.3 us against 47.9 us, 1 M keys 184 against 180 us)
+  return launch_unrolled<V, LPR, 2, Idx>(ix, src, src_rows, out, out_rows, vpr, counts, group, n, max_blocks, status,
+                                         host_mirror, nt_store_for(n * (size_t)vpr * sizeof(V)), stream);
 }
 
 template <typename V, typename Idx, bool ALL_LPR>
@@ -223,11 +239,32 @@ int launch_gather(Idx ix, const void *src, uint64_t src_rows, void *out, uint64_
 }
 
 }  // namespace
+
+namespace {
+thread_local int g_output_hint = 0;
+}
+bool nt_store_for(size_t out_bytes) {
+  static int forced = [] {
+    const char *e = getenv("UGK_GATHER_NT_STORE");
+    return e ? atoi(e) : -1;
+  }();
+  if (forced >= 0) return forced != 0;
+  if (g_output_hint == UGK_OUTPUT_STREAMS) return true;
+  if (g_output_hint == UGK_OUTPUT_STAYS) return false;
+  return out_bytes > ((size_t)192 << 20);
+}
 }  // namespace ugk
 
 using namespace ugk;
 
 extern "C" {
+
+int ugk_set_output_hint(int hint) {
+  UGK_REQUIRE(hint == UGK_OUTPUT_AUTO || hint == UGK_OUTPUT_STREAMS || hint == UGK_OUTPUT_STAYS,
+              "ugk_set_output_hint: unknown hint %d", hint);
+  g_output_hint = hint;
+  return 0;
+}
 
 int ugk_gather_direct_u32(const void *src_dev, uint64_t src_rows, const uint32_t *keys_dev, size_t n, void *out_dev,
                           size_t row_bytes, unsigned max_blocks, uint32_t *status_dev, uint32_t *host_mirror,

@@ -46,6 +46,11 @@ static inline unsigned clamp_grid(size_t want, unsigned max_blocks) {
   return (unsigned)want;
 }
 
+// Non-temporal stores for an extraction whose output of `out_bytes` will not stay in the 256 MB memory-side cache
+// anyway; ordinary write-back stores otherwise, so that the consumer finds the rows there.  The caller's hint
+// (ugk_set_output_hint) and UGK_GATHER_NT_STORE=0/1 override the size rule.
+bool nt_store_for(size_t out_bytes);
+
 __device__ __forceinline__ unsigned lane_id() { return __lane_id(); }
 
 }  // namespace ugk

@@ -154,13 +154,16 @@ __global__ __launch_bounds__(kBlock) void select_keys_kernel(const K *__restrict
 }
 
 // ---- fused lookup + gather: every wavefront resolves 64 keys, then copies their 64 rows ------------------
-template <typename K, int KIND, int LPR, int KPW>
+typedef const __attribute__((address_space(1))) u32x4 *grow_t;  // a row in global memory (HBM, or mapped host memory)
+typedef __attribute__((address_space(1))) u32x4 *gout_t;
+
+template <typename K, int KIND, int LPR, int KPW, bool NT_STORE>
 __global__ __launch_bounds__(kBlock) void extract_mix_kernel(ugk_table_t t, const K *__restrict__ keys, size_t n,
                                                              const u32x4 *__restrict__ cache, uint64_t cache_rows,
                                                              const u32x4 *__restrict__ host, uint64_t host_rows,
                                                              u32x4 *__restrict__ out, uint32_t vpr,
                                                              uint32_t *status, uint32_t *host_mirror,
-                                                             unsigned long long *counts, bool nt_store) {
+                                                             unsigned long long *counts) {
   constexpr int RPW = kWave / LPR;  // rows per wavefront instruction
   __shared__ uint32_t block_tot[2];
   if (threadIdx.x < 2) block_tot[threadIdx.x] = 0;
@@ -176,7 +179,8 @@ __global__ __launch_bounds__(kBlock) void extract_mix_kernel(ugk_table_t t, cons
     const size_t i = b0 + lane;
     const bool active = lane < KPW && i < n;
     const uint64_t key = active ? key_to_u64<K>(keys[i]) : 0;
-    const Found f = table_lookup<KIND>(t, key, active);
+    // a full wavefront of keys probes its eight home lines in one go (see hash_probe_home)
+    const Found f = table_lookup<KIND, KPW == kWave ? 1 : 2>(t, key, active);
     const u32x4 *rowp = nullptr;
     if (active) {
       if (f.hit && f.loc == UGK_LOC_LOCAL && f.off < cache_rows) rowp = cache + (uint64_t)f.off * vpr;
@@ -187,30 +191,39 @@ __global__ __launch_bounds__(kBlock) void extract_mix_kernel(ugk_table_t t, cons
         if (host_mirror) host_mirror[0] = UGK_ST_KEY_OUT_OF_RANGE;
       }
     }
-    const uint64_t rowbits = reinterpret_cast<uint64_t>(rowp);
+    // A key without a row copies nothing; its lanes read the head of the output instead (mapped whatever the key), so
+    // that the loads below carry no branch: behind a branch each of them waits for the one before.
+    const bool has_row = rowp != nullptr;
+    const uint64_t rowbits = has_row ? reinterpret_cast<uint64_t>(rowp) : reinterpret_cast<uint64_t>(out);
     if (counts) {
       // rows from the cache, and all others (host rows, and rows skipped for a key without a row: the launch is
       // flagged then and its group sizes mean nothing, but the two sums still add up to n)
-      const bool from_cache = rowp != nullptr && f.hit && f.loc == UGK_LOC_LOCAL;
+      const bool from_cache = has_row && f.hit && f.loc == UGK_LOC_LOCAL;
       wave_local += __popcll(__ballot(from_cache));
       wave_host += __popcll(__ballot(active && !from_cache));
     }
     for (int r0 = 0; r0 < KPW; r0 += RPW * UNROLL) {
-      const u32x4 *p[UNROLL];
+      // the row addresses travel between lanes as integers; turned back into pointers they must be told to be global
+      // memory again, or the loads become generic ones, which the hardware cannot keep several of in flight in order
+      grow_t p[UNROLL];
+      bool ok[UNROLL];
 #pragma unroll
-      for (int u = 0; u < UNROLL; ++u) p[u] = reinterpret_cast<const u32x4 *>(shfl64(rowbits, r0 + u * RPW + rg));
+      for (int u = 0; u < UNROLL; ++u) {
+        p[u] = reinterpret_cast<grow_t>(shfl64(rowbits, r0 + u * RPW + rg));
+        ok[u] = __shfl((int)has_row, r0 + u * RPW + rg) != 0;
+      }
       for (uint32_t c0 = 0; c0 < vpr; c0 += LPR) {
         const uint32_t col = c0 + sub;
         if (col < vpr) {
           u32x4 v[UNROLL];
 #pragma unroll
-          for (int u = 0; u < UNROLL; ++u)
-            if (p[u]) v[u] = __builtin_nontemporal_load(p[u] + col);
+          for (int u = 0; u < UNROLL; ++u) v[u] = __builtin_nontemporal_load(p[u] + col);
 #pragma unroll
           for (int u = 0; u < UNROLL; ++u)
-            if (p[u]) {
-              u32x4 *dst = out + (b0 + r0 + u * RPW + rg) * vpr + col;
-              if (nt_store) __builtin_nontemporal_store(v[u], dst);
+            if (ok[u]) {
+              gout_t dst = (gout_t)out + (b0 + r0 + u * RPW + rg) * vpr + col;
+              // a template parameter: the two stores of a run-time choice get merged and lose the hint
+              if constexpr (NT_STORE) __builtin_nontemporal_store(v[u], dst);
               else *dst = v[u];
             }
         }
@@ -461,41 +474,54 @@ int extract_mix_lpr(ugk_table_t t, const K *keys, size_t n, const void *cache, u
                     uint64_t host_rows, void *out, uint32_t vpr, uint32_t *status, uint32_t *host_mirror,
                     uint64_t *counts, uint32_t *num_groups, uint32_t others_hint, hipStream_t st) {
   // ordinary write-back stores while the output fits the memory-side cache (the consumer finds it there),
-  // non-temporal beyond; UGK_GATHER_NT_STORE=0/1 forces the choice
-  static const int forced_nt = [] {
-    const char *e = getenv("UGK_GATHER_NT_STORE");
-    return e ? atoi(e) : -1;
-  }();
-  const bool nt = forced_nt >= 0 ? forced_nt != 0 : n * (size_t)vpr * 16 > ((size_t)192 << 20);
-  // Keys per wavefront.  A wavefront copies its rows a few at a time, one round trip to memory per round, so a batch
-  // that leaves wavefront slots of the chip empty finishes sooner when it is cut into more, shorter wavefronts: the
-  // fewest keys per wavefront whose wavefronts are all resident at once (8 per SIMD).  Measured on 512-byte rows at
-  // 1 % misses, flat table, 64 / 32 / 16 / 8 keys per wavefront: 8,192 keys 16.0 / 11.6 / 7.1 / 6.3 us, 65,536 keys
-  // 31.6 / 21.4 / 17.0 / 16.1 us, 131,072 keys 37.6 / 29.9 / 29.6 / 30.2 us, 262,144 keys 54.2 / 49.6 / 51.1 / 51.7 us,
-  // 524,288 keys 90.5 / 93.1 / 94.4 / 95.5 us.  The hash table's probe works on all 64 lanes at once and wants one
-  // notch more (65,536 keys 44.8 / 33.0 / 26.7 / 30.5 us, 262,144 keys 66.7 / 71.5 / 75.6 / 80.1 us).  In the top band
-  // of the flat table a batch bound by the host link runs 1-2 % slower with 32 than with 64, so 32 is taken there only
-  // when the caller expects at most 2 % of the rows from outside the cache.
+  // non-temporal beyond, or as the caller's hint says
+  const bool nt = nt_store_for(n * (size_t)vpr * 16);
+  // Keys per wavefront.  A wavefront resolves its keys together and then copies their rows a few at a time; once its
+  // first stores are out, every later load of the wavefront returns behind them, so wavefronts of one round of rows
+  // (8 keys of 512 bytes) keep memory busier than long ones, and short ones also fill a chip that a small batch
+  // would leave half empty.  What speaks for longer wavefronts is the lookup: a hash probe works on all 64 lanes at
+  // once, and with small rows the lookups are a larger share of the work.  Measured on MI355X, 1 % misses, 8 / 16 / 32 /
+  // 64 keys per wavefront, us per launch:
+  //   flat, 512-byte rows:  8,192 keys 5.7 / 6.9 / 10.2 / 16.2;  65,536 keys 15.9 / 16.0 / 16.1 / 19.9;  262,144 keys
+  //                         48.6 / 49.5 / 50.8 / 47.7;  1 M keys 189.7 / 191.4 / 202.7 / 203.7
+  //   flat, 128-byte rows:  65,536 keys 8.2 / 7.7 / 7.6 / 8.5;  262,144 keys 21.0 / 21.8 / 19.5 / 20.1;  1 M keys 64.8 /
+  //                         65.5 / 64.0 / 64.2
+  //   hash, 512-byte rows:  8,192 keys 12.4 / 13.8 / 17.5 / 23.3;  65,536 keys 25.9 / 24.5 / 26.3 / 30.8;  131,072 keys
+  //                         38.2 / 37.8 / 32.7 / 35.1;  262,144 keys 63.0 / 58.7 / 61.3 / 53.1;  1 M keys 215.3 / 211.4 /
+  //                         219.3 / 226.4
+  //   hash, 128-byte rows:  65,536 keys 22.0 / 18.9 / 18.7 / 19.9;  262,144 keys 49.0 / 37.0 / 31.2 / 28.9;  1 M keys
+  //                         150.7 / 112.3 / 82.1 / 79.5
+  // and the same order at 10 % misses, where the host link bounds the launch and the spread is 1-3 %.  The batch sizes
+  // above are multiples of the chip's wavefront slots (256 CUs x 32 = 8,192), which is how the rule below states them.
+  // others_hint is not consulted any more: since the row loads of a wavefront are in flight together, the mix of
+  // sources no longer changes which shape wins.
+  (void)others_hint;
   const size_t slots = (size_t)cu_count() * 4 * 8;
-  const bool few_others = others_hint != UGK_HINT_UNKNOWN && (size_t)others_hint * 50 <= n;
-  int kpw = kWave;
-  if (KIND == 1) {
-    if (n <= slots * 8) kpw = 8;
-    else if (n <= slots * 16) kpw = 16;
-    else if (n <= slots * 32 && few_others) kpw = 32;
-  } else {
-    if (n <= slots * 8) kpw = 16;
-    else if (n <= slots * 16) kpw = 32;
-  }
   const int lpr = vpr <= 1 ? 1 : vpr <= 2 ? 2 : vpr <= 4 ? 4 : vpr <= 8 ? 8 : vpr <= 16 ? 16 : vpr <= 32 ? 32 : 64;
+  const bool small_rows = lpr <= 8;  // rows of up to 128 bytes
+  int kpw;
+  if (KIND == 1) {
+    kpw = small_rows ? 32 : 8;
+  } else if (n <= slots) {
+    kpw = 8;
+  } else if (small_rows) {
+    kpw = n <= slots * 16 ? 32 : 64;
+  } else {
+    kpw = n <= slots * 8 ? 16 : n <= slots * 16 ? 32 : n <= slots * 32 ? 64 : 16;
+  }
   if (kpw < kWave / lpr) kpw = kWave / lpr;  // one wavefront instruction copies 64 / lpr rows
   const size_t keys_per_group = (size_t)kpw * kWavesPerBlock;
   const unsigned grid = clamp_grid((n + keys_per_group - 1) / keys_per_group, 0);
   if (num_groups) *num_groups = grid;
-#define UGK_GO2(L, W)                                                                                              \
-  hipLaunchKernelGGL((extract_mix_kernel<K, KIND, L, W>), dim3(grid), dim3(kBlock), 0, st, t, keys, n,            \
+#define UGK_GO3(L, W, NT)                                                                                          \
+  hipLaunchKernelGGL((extract_mix_kernel<K, KIND, L, W, NT>), dim3(grid), dim3(kBlock), 0, st, t, keys, n,        \
                      (const u32x4 *)cache, cache_rows, (const u32x4 *)host, host_rows, (u32x4 *)out, vpr, status, \
-                     host_mirror, reinterpret_cast<unsigned long long *>(counts), nt)
+                     host_mirror, reinterpret_cast<unsigned long long *>(counts))
+#define UGK_GO2(L, W)         \
+  do {                        \
+    if (nt) UGK_GO3(L, W, true); \
+    else UGK_GO3(L, W, false);   \
+  } while (0)
 #define UGK_GO(L)                                   \
   do {                                              \
     if constexpr (kWave / L <= 8) {                 \
@@ -527,6 +553,7 @@ int extract_mix_lpr(ugk_table_t t, const K *keys, size_t n, const void *cache, u
   else UGK_GO(64);
 #undef UGK_GO
 #undef UGK_GO2
+#undef UGK_GO3
   UGK_HIP(hipGetLastError());
   return 0;
 }

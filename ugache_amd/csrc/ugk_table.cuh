@@ -78,22 +78,25 @@ struct HashProbe {
 };
 
 // step 1: the home line of every lane's key.  In round r the eight 8-lane groups serve lanes 8r .. 8r+7.
+// PASSES = 2: two passes of four rounds, the four line loads of a pass in flight together; PASSES = 1: all eight
+// rounds in flight at once, which saves a round trip to memory per wavefront and costs about 30 more vector
+// registers (fewer wavefronts per SIMD: taken where the launch does not fill them all anyway).
+template <int PASSES>
 __device__ __forceinline__ HashProbe hash_probe_home(const ugk_bucket_t *table, uint64_t nb, uint64_t key,
                                                      bool active) {
+  constexpr int PER = 8 / PASSES;  // rounds whose loads are in flight together
   HashProbe p{Found{false, 0, 0}, 0, false};
   const int lane = (int)lane_id();
   const int grp = lane >> 3, sub = lane & 7;
   const uint64_t home = active ? hash_home(key, nb) : 0;
-  // two passes of four rounds: the four line loads of a pass are in flight together; holding all eight rounds at
-  // once costs 50 more vector registers and halves the occupancy of the kernels built on this
 #pragma unroll
-  for (int half = 0; half < 2; ++half) {
-    u32x4 raw[4];
-    uint64_t kk[4];
-    bool act[4];
+  for (int pass = 0; pass < PASSES; ++pass) {
+    u32x4 raw[PER];
+    uint64_t kk[PER];
+    bool act[PER];
 #pragma unroll
-    for (int q = 0; q < 4; ++q) {
-      const int owner = (half * 4 + q) * 8 + grp;
+    for (int q = 0; q < PER; ++q) {
+      const int owner = (pass * PER + q) * 8 + grp;
       kk[q] = shfl64(key, owner);
       const uint64_t hb = shfl64(home, owner);
       act[q] = __shfl((int)active, owner) != 0;
@@ -101,8 +104,8 @@ __device__ __forceinline__ HashProbe hash_probe_home(const ugk_bucket_t *table, 
       if (act[q]) raw[q] = *reinterpret_cast<const u32x4 *>(table + hb + sub);
     }
 #pragma unroll
-    for (int q = 0; q < 4; ++q) {
-      const int r = half * 4 + q;
+    for (int q = 0; q < PER; ++q) {
+      const int r = pass * PER + q;
       const uint64_t bkey = ((uint64_t)raw[q].y << 32) | raw[q].x;
       const bool is_match = act[q] && bkey == kk[q];
       const bool is_empty = act[q] && bkey == UGK_HASH_EMPTY;
@@ -207,15 +210,17 @@ __device__ __forceinline__ Found hash_probe_rest(const ugk_bucket_t *table, uint
   return f;
 }
 
+template <int PASSES = 2>
 __device__ __forceinline__ Found hash_lookup_wave(const ugk_bucket_t *table, uint64_t nb, uint64_t key, bool active) {
-  return hash_probe_rest(table, nb, key, hash_probe_home(table, nb, key, active));
+  return hash_probe_rest(table, nb, key, hash_probe_home<PASSES>(table, nb, key, active));
 }
 
 // Table lookup dispatch.  KIND is ugk_table_t::kind.  All lanes of the wavefront must call it.
-template <int KIND>
+template <int KIND, int PASSES = 2>
 __device__ __forceinline__ Found table_lookup(const ugk_table_t &t, uint64_t key, bool active) {
   if (KIND == 1) return flat_lookup(reinterpret_cast<const uint32_t *>(t.table), t.size, key, active);
-  if (KIND == 2) return hash_lookup_wave(reinterpret_cast<const ugk_bucket_t *>(t.table), t.size, key, active);
+  if (KIND == 2)
+    return hash_lookup_wave<PASSES>(reinterpret_cast<const ugk_bucket_t *>(t.table), t.size, key, active);
   return Found{false, 0, 0};
 }
 

@@ -69,6 +69,7 @@ SIGNATURES = {
     "ugk_fill_u32": [_vp, _u32, _sz, _vp],
     "ugk_arange_u32": [_vp, _u32, _sz, _vp],
     "ugk_copy_rows": [_vp, _vp, _sz, _vp],
+    "ugk_set_output_hint": [C.c_int],
     "ugk_gather_direct_u32": [_vp, _u64, _vp, _sz, _vp, _sz, C.c_uint, _vp, _vp, _vp],
     "ugk_gather_direct_i64": [_vp, _u64, _vp, _sz, _vp, _sz, C.c_uint, _vp, _vp, _vp],
     "ugk_gather_scatter_u32": [_vp, _u64, _vp, _vp, _sz, _vp, _u64, _sz, C.c_uint, _vp, _vp, _vp],
