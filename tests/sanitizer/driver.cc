@@ -1,0 +1,156 @@
+// TEST INFRASTRUCTURE ONLY: drives the host library through its C boundary (include/coll_cache_c_api.h) on the CPU,
+// linked against the CPU model of the kernel layer next to this file, so that the library's threads can run under
+// AddressSanitizer / UBSan and ThreadSanitizer:
+//   build -> blocking lookups on one thread  ||  hotness records + background refreshes on another
+//         -> stream-ordered lookups on one stream  ||  a refresh on another stream
+//         -> the serving loop (coll_cache_forward) with its own background refresh thread -> shutdown,
+// once per table kind and per refresh kind (host lists / device bitmaps).  Every looked-up row is compared with the
+// host table, so a refresh that reused a slot too early is also seen as a wrong row.
+//
+// usage: driver <FLAT|HASH> <host|device> [lookup steps per phase, default 150]
+#include <algorithm>
+#include <atomic>
+#include <cstdint>
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+#include <random>
+#include <thread>
+#include <vector>
+
+#include "coll_cache_c_api.h"
+
+namespace {
+
+constexpr size_t kRows = 20000, kDim = 32;  // 128-byte rows
+float cell(size_t row, size_t col) { return (float)(row * 131 + col * 7) * 0.5f; }
+
+std::vector<uint32_t> skewed_keys(std::mt19937_64 &g, size_t n, uint64_t shift) {
+  // a hot set that moves with `shift`, so that every refresh has rows to evict and to insert
+  std::vector<uint32_t> k(n);
+  for (auto &x : k) {
+    const uint64_t r = g();
+    x = (r & 3) ? (uint32_t)((shift + (r >> 8) % (kRows / 5)) % kRows) : (uint32_t)((r >> 8) % kRows);
+  }
+  return k;
+}
+
+long check_rows(const float *table, const float *out, const uint32_t *keys, size_t n) {
+  long bad = 0;
+  for (size_t i = 0; i < n; ++i)
+    if (memcmp(out + i * kDim, table + (size_t)keys[i] * kDim, kDim * sizeof(float)) != 0) ++bad;
+  return bad;
+}
+
+}  // namespace
+
+int main(int argc, char **argv) {
+  if (argc != 3 && argc != 4) {
+    fprintf(stderr, "usage: %s <FLAT|HASH> <host|device> [steps]\n", argv[0]);
+    return 2;
+  }
+  const int steps = argc == 4 ? atoi(argv[3]) : 150;
+  const bool on_device = strcmp(argv[2], "device") == 0;
+  setenv("COLL_HASH_TABLE", argv[1], 1);
+  setenv("COLL_GPU_RECORD", on_device ? "1" : "0", 1);
+  setenv("COLL_GPU_REFRESH", on_device ? "1" : "0", 1);
+  setenv("SAMGRAPH_LOG_LEVEL", "warn", 0);
+
+  const char *keys[] = {"cache_percentage", "_cache_policy", "num_device", "num_global_step_per_epoch", "num_epoch",
+                        "num_total_item",   "omp_thread_num"};
+  const char *vals[] = {"0.25", "13", "1", "10", "1", "20000", "4"};
+  long bad_rows = 0;
+  for (int round = 0; round < 2; ++round) {
+    coll_cache_config(keys, vals, 7);
+    float *table = static_cast<float *>(coll_cache_alloc_host_table(kRows * kDim * sizeof(float)));
+    for (size_t r = 0; r < kRows; ++r)
+      for (size_t c = 0; c < kDim; ++c) table[r * kDim + c] = cell(r, c);
+    std::mt19937_64 g(17 + round);
+    coll_cache_record_init(0);
+    for (int b = 0; b < 20; ++b) {
+      auto k = skewed_keys(g, 4096, 0);
+      coll_cache_record(0, k.data(), k.size());
+    }
+    coll_cache_init_c(0, kRows, nullptr, nullptr, nullptr, table, /*kF32*/ 0, kDim, 0.25, nullptr);
+
+    // 1. blocking lookups and records on this thread, background refreshes on another
+    std::atomic<bool> stop{false};
+    std::atomic<int> refreshes{0};
+    std::thread refresher([&] {
+      while (!stop.load()) {
+        coll_cache_refresh(0, nullptr, /*foreground=*/0);
+        refreshes.fetch_add(1);
+        std::this_thread::sleep_for(std::chrono::milliseconds(2));
+      }
+    });
+    std::vector<float> out(4096 * kDim);
+    for (int step = 0; step < steps || refreshes.load() < 3; ++step) {
+      auto k = skewed_keys(g, 1 + g() % 4096, (uint64_t)step * 97);
+      if (!on_device) coll_cache_record(0, k.data(), k.size());
+      coll_cache_lookup(0, k.data(), k.size(), out.data(), nullptr);
+      bad_rows += check_rows(table, out.data(), k.data(), k.size());
+      if (step > 100 * steps) break;
+    }
+    stop.store(true);
+    refresher.join();
+
+    // 2. stream-ordered lookups on the null stream while a refresh runs on a stream of its own
+    {
+      std::thread one_refresh([&] { coll_cache_refresh(0, nullptr, /*foreground=*/0); });
+      std::vector<std::vector<uint32_t>> batches;
+      std::vector<std::vector<float>> outs;
+      for (int b = 0; b < 8; ++b) {
+        batches.push_back(skewed_keys(g, 2048, 5000 + b));
+        outs.emplace_back(2048 * kDim);
+      }
+      for (int b = 0; b < 8; ++b)
+        coll_cache_lookup_async(0, batches[b].data(), batches[b].size(), outs[b].data(), nullptr);
+      coll_cache_lookup_wait(0, nullptr);
+      one_refresh.join();
+      for (int b = 0; b < 8; ++b) bad_rows += check_rows(table, outs[b].data(), batches[b].data(), batches[b].size());
+    }
+
+    // 3. wide keys, the distinct-keys lookup, a foreground refresh
+    {
+      std::vector<int64_t> k64(3000);
+      std::vector<uint32_t> k32(3000), inverse(3000);
+      for (size_t i = 0; i < k64.size(); ++i) k32[i] = (uint32_t)(k64[i] = (int64_t)(g() % (kRows / 50)));
+      if (!on_device) coll_cache_record_i64(0, k64.data(), k64.size());
+      coll_cache_lookup_i64(0, k64.data(), k64.size(), out.data(), nullptr);
+      bad_rows += check_rows(table, out.data(), k32.data(), k32.size());
+      coll_cache_refresh(0, nullptr, /*foreground=*/1);
+      const size_t nu = coll_cache_lookup_unique(0, k32.data(), k32.size(), out.data(), inverse.data(), nullptr);
+      for (size_t i = 0; i < k32.size(); ++i)
+        if (inverse[i] >= nu ||
+            memcmp(out.data() + (size_t)inverse[i] * kDim, table + (size_t)k32[i] * kDim, kDim * sizeof(float)) != 0)
+          ++bad_rows;
+    }
+
+    // 4. the serving loop with its own background refresh thread
+    coll_cache_forward_config(1, 7, 0.25, 1);
+    for (int step = 0; step < std::max(steps / 2, 24); ++step) {
+      auto k = skewed_keys(g, 3000, 9000 + (uint64_t)step * 53);
+      coll_cache_forward(0, k.data(), k.size(), out.data(), nullptr);
+      bad_rows += check_rows(table, out.data(), k.data(), k.size());
+    }
+    const uint64_t done = coll_cache_forward_join();
+    uint64_t info[8];
+    coll_cache_get_info(0, info);
+    printf("round %d: %d background refreshes, %llu from the serving loop, %llu table rebuilds, %llu rows cached of "
+           "%llu slots, %ld bad rows\n",
+           round, refreshes.load(), (unsigned long long)done, (unsigned long long)info[7],
+           (unsigned long long)info[1], (unsigned long long)info[0], bad_rows);
+    if (done == 0 || refreshes.load() < 3) {
+      fprintf(stderr, "the refreshes this run is about did not happen\n");
+      return 1;
+    }
+    coll_cache_shutdown();
+    coll_cache_free_host_table(table);
+  }
+  if (bad_rows) {
+    fprintf(stderr, "%ld looked-up rows differ from the host table\n", bad_rows);
+    return 1;
+  }
+  printf("OK\n");
+  return 0;
+}

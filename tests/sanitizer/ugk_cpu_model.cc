@@ -1,0 +1,756 @@
+// TEST INFRASTRUCTURE ONLY: a plain CPU model of the ugk_* C-ABI of include/ugache_hip.h.
+//
+// It exists so that the host library (ugache_amd/coll_cache_lib/*.cc) can be linked into one executable without a GPU
+// and run under AddressSanitizer / UBSan and, separately, ThreadSanitizer: the library's own threads (lookups, the
+// record stream, foreground and background refreshes, the serving loop) then run against "device memory" that is
+// ordinary host memory.  It is never built into the package, never loaded by it and is no fallback: the product's
+// libcoll_cache.so links libugache_hip.so only.
+//
+// Model: every call runs to completion inside the calling thread (a stream is a token, waiting for one is a no-op), so
+// the order the library enqueues work in is the order it runs in.  Words that kernels touch with atomics on the GPU
+// (table entries, buckets, counters, bitmap words, status words) are touched with atomics here; rows are
+// copied with memcpy.  A refresh that overwrote a cache slot a lookup on another thread might still read would
+// therefore show up as a data race under ThreadSanitizer, which is what the hand-shake between the two is there to
+// prevent.  Layouts follow the header where it fixes them (flat entries, ugk_bucket_t, index records, bitmaps); the
+// probe sequence of the hash table and the order of lists the header calls unspecified are this model's own.
+#include <algorithm>
+#include <atomic>
+#include <chrono>
+#include <cmath>
+#include <cstdarg>
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+#include <map>
+#include <mutex>
+#include <unordered_map>
+#include <vector>
+
+#include "ugache_hip.h"
+
+namespace {
+
+thread_local char g_err[512];
+int fail(const char *fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_err, sizeof(g_err), fmt, ap);
+  va_end(ap);
+  return 1;
+}
+#define REQUIRE(c, ...) \
+  do {                  \
+    if (!(c)) return fail(__VA_ARGS__); \
+  } while (0)
+
+std::mutex g_mem_mu;
+std::map<uintptr_t, std::pair<size_t, int>> g_blocks;  // base -> (bytes, kind)
+
+int alloc_block(void **ptr, size_t nbytes, int kind) {
+  void *p = nullptr;
+  const size_t bytes = (std::max<size_t>(nbytes, 1) + 255) / 256 * 256;
+  if (posix_memalign(&p, 256, bytes) != 0) return fail("out of memory (%zu bytes)", nbytes);
+  memset(p, 0xA5, bytes);  // fresh device memory holds no particular value
+  std::lock_guard<std::mutex> g(g_mem_mu);
+  g_blocks[(uintptr_t)p] = {bytes, kind};
+  *ptr = p;
+  return 0;
+}
+int free_block(void *ptr, int kind) {
+  if (!ptr) return 0;
+  {
+    std::lock_guard<std::mutex> g(g_mem_mu);
+    auto it = g_blocks.find((uintptr_t)ptr);
+    if (it == g_blocks.end() || it->second.second != kind) return fail("free of a pointer that was not allocated here");
+    g_blocks.erase(it);
+  }
+  free(ptr);
+  return 0;
+}
+
+// Loads acquire and stores release: what a kernel wrote before it published a word (a row copied into a slot before
+// its key went into the table, by an earlier launch on the GPU) is visible to whoever reads that word.
+template <typename T>
+T ld(const T *p) {
+  return __atomic_load_n(p, __ATOMIC_ACQUIRE);
+}
+template <typename T>
+void st(T *p, T v) {
+  __atomic_store_n(p, v, __ATOMIC_RELEASE);
+}
+void or_status(uint32_t *status, uint32_t bits, uint32_t *mirror = nullptr) {
+  __atomic_fetch_or(status, bits, __ATOMIC_RELAXED);
+  if (mirror) st(mirror, bits);
+}
+
+uint64_t fmix64(uint64_t x) {
+  x ^= x >> 33;
+  x *= 0xff51afd7ed558ccdull;
+  x ^= x >> 33;
+  x *= 0xc4ceb9fe1a85ec53ull;
+  x ^= x >> 33;
+  return x;
+}
+uint64_t k64(uint32_t k) { return k; }
+uint64_t k64(int64_t k) { return (uint64_t)k; }
+uint64_t fallback_row(const ugk_table_t &t, uint64_t key) {
+  if (t.fb_mul == 0) return key;
+  return key <= t.fb_mask ? ((key * t.fb_mul) & t.fb_mask) : ~0ull;
+}
+
+struct Found {
+  bool hit;
+  uint32_t loc, off;
+};
+Found lookup(const ugk_table_t &t, uint64_t key) {
+  Found f{false, 0, 0};
+  if (t.kind == 1) {
+    if (key < t.size) {
+      const uint32_t v = ld(reinterpret_cast<const uint32_t *>(t.table) + key);
+      if (v != UGK_EMPTY_U32) f = Found{true, (v >> 28) & 0xfu, v & 0x0fffffffu};
+    }
+  } else if (t.kind == 2) {
+    const ugk_bucket_t *b = reinterpret_cast<const ugk_bucket_t *>(t.table);
+    uint64_t pos = fmix64(key) % t.size;
+    for (uint64_t step = 0; step < t.size; ++step) {
+      const uint64_t cur = ld(&b[pos].key);
+      if (cur == key) {
+        const uint64_t om = ld(reinterpret_cast<const uint64_t *>(&b[pos].off));
+        const uint32_t meta = (uint32_t)(om >> 32);
+        if (meta & UGK_META_VALID) f = Found{true, meta & 0xfu, (uint32_t)om};
+        return f;
+      }
+      if (cur == UGK_HASH_EMPTY) return f;
+      if (++pos == t.size) pos = 0;
+    }
+  }
+  return f;
+}
+int check_table(const ugk_table_t &t, const char *who) {
+  REQUIRE(t.kind == 1 || t.kind == 2, "%s: table kind %d is not flat(1) or hash(2)", who, t.kind);
+  REQUIRE(t.table && t.size, "%s: empty table", who);
+  return 0;
+}
+
+void copy_row(void *dst, const void *src, size_t bytes) { memcpy(dst, src, bytes); }
+
+template <typename K>
+int gather_direct(const void *src, uint64_t src_rows, const K *keys, const uint32_t *dst, size_t n, void *out,
+                  uint64_t out_rows, size_t rb, uint32_t *status, uint32_t *mirror) {
+  if (n == 0) return 0;
+  REQUIRE(src && out && keys && status, "gather: null pointer");
+  for (size_t i = 0; i < n; ++i) {
+    const uint64_t s = k64(keys[i]), d = dst ? dst[i] : i;
+    if (s >= src_rows || d >= out_rows) {
+      or_status(status, UGK_ST_KEY_OUT_OF_RANGE, mirror);
+      continue;
+    }
+    copy_row((char *)out + d * rb, (const char *)src + s * rb, rb);
+  }
+  return 0;
+}
+
+int gather_list(const void *src, uint64_t src_rows, const ugk_idx_t *idx, size_t count, void *out, uint64_t out_rows,
+                size_t rb, uint32_t *status, uint32_t *mirror) {
+  for (size_t i = 0; i < count; ++i) {
+    if (idx[i].src_off >= src_rows || idx[i].dst_off >= out_rows) {
+      or_status(status, UGK_ST_KEY_OUT_OF_RANGE, mirror);
+      continue;
+    }
+    copy_row((char *)out + (size_t)idx[i].dst_off * rb, (const char *)src + (size_t)idx[i].src_off * rb, rb);
+  }
+  return 0;
+}
+
+template <typename K>
+int table_insert(ugk_table_t t, const K *keys, const uint32_t *offs, uint32_t seq_base, uint32_t loc, size_t n,
+                 uint32_t *status) {
+  if (n == 0) return 0;
+  if (check_table(t, "ugk_table_insert")) return 1;
+  REQUIRE(keys && status && loc < 16, "ugk_table_insert: bad argument");
+  for (size_t i = 0; i < n; ++i) {
+    const uint64_t key = k64(keys[i]);
+    const uint32_t off = offs ? offs[i] : seq_base + (uint32_t)i;
+    if (t.kind == 1) {
+      if (key >= t.size || off > 0x0fffffffu) {
+        or_status(status, UGK_ST_KEY_OUT_OF_RANGE);
+        continue;
+      }
+      const uint32_t old = __atomic_exchange_n(reinterpret_cast<uint32_t *>(t.table) + key, (loc << 28) + off,
+                                               __ATOMIC_ACQ_REL);
+      if (old != UGK_EMPTY_U32) or_status(status, UGK_ST_DUP_KEY);
+      continue;
+    }
+    if (key >= UGK_HASH_TOMB) {
+      or_status(status, UGK_ST_KEY_OUT_OF_RANGE);
+      continue;
+    }
+    ugk_bucket_t *b = reinterpret_cast<ugk_bucket_t *>(t.table);
+    uint64_t pos = fmix64(key) % t.size, first_tomb = ~0ull;
+    bool placed = false;
+    for (uint64_t step = 0; step < t.size && !placed; ++step) {
+      const uint64_t cur = ld(&b[pos].key);
+      if (cur == key) {
+        or_status(status, UGK_ST_DUP_KEY);
+        placed = true;
+      } else if (cur == UGK_HASH_EMPTY) {
+        break;
+      } else {
+        if (cur == UGK_HASH_TOMB && first_tomb == ~0ull) first_tomb = pos;
+        if (++pos == t.size) pos = 0;
+      }
+    }
+    if (placed) continue;
+    const uint64_t target = first_tomb != ~0ull ? first_tomb : pos;
+    const uint64_t cur = ld(&b[target].key);
+    if (cur != UGK_HASH_EMPTY && cur != UGK_HASH_TOMB) {
+      or_status(status, UGK_ST_TABLE_FULL);
+      continue;
+    }
+    st(&b[target].key, key);  // "present, not valid" until the next store: reads as a miss
+    st(reinterpret_cast<uint64_t *>(&b[target].off), ((uint64_t)(UGK_META_VALID | loc) << 32) | off);
+  }
+  return 0;
+}
+
+template <typename K>
+int table_evict(ugk_table_t t, const K *keys, size_t n, uint32_t *status) {
+  if (n == 0) return 0;
+  if (check_table(t, "ugk_table_evict")) return 1;
+  REQUIRE(keys && status, "ugk_table_evict: null pointer");
+  for (size_t i = 0; i < n; ++i) {
+    const uint64_t key = k64(keys[i]);
+    if (t.kind == 1) {
+      if (key >= t.size) {
+        or_status(status, UGK_ST_KEY_OUT_OF_RANGE);
+        continue;
+      }
+      const uint32_t old =
+          __atomic_exchange_n(reinterpret_cast<uint32_t *>(t.table) + key, UGK_EMPTY_U32, __ATOMIC_ACQ_REL);
+      if (old == UGK_EMPTY_U32) or_status(status, UGK_ST_EVICT_ABSENT);
+      continue;
+    }
+    ugk_bucket_t *b = reinterpret_cast<ugk_bucket_t *>(t.table);
+    uint64_t pos = fmix64(key) % t.size;
+    bool done = false;
+    for (uint64_t step = 0; step < t.size && !done && key < UGK_HASH_TOMB; ++step) {
+      const uint64_t cur = ld(&b[pos].key);
+      if (cur == key) {
+        st(reinterpret_cast<uint64_t *>(&b[pos].off), (uint64_t)0);
+        st(&b[pos].key, (uint64_t)UGK_HASH_TOMB);
+        done = true;
+      } else if (cur == UGK_HASH_EMPTY) {
+        break;
+      } else if (++pos == t.size) {
+        pos = 0;
+      }
+    }
+    if (!done) or_status(status, UGK_ST_EVICT_ABSENT);
+  }
+  return 0;
+}
+
+template <typename K>
+int table_lookup(ugk_table_t t, const K *keys, size_t n, uint32_t fallback_loc, uint32_t *loc_out, uint32_t *off_out) {
+  if (n == 0) return 0;
+  if (check_table(t, "ugk_table_lookup")) return 1;
+  for (size_t i = 0; i < n; ++i) {
+    const uint64_t key = k64(keys[i]);
+    const Found f = lookup(t, key);
+    if (loc_out) loc_out[i] = f.hit ? f.loc : fallback_loc;
+    if (off_out) off_out[i] = f.hit ? f.off : (uint32_t)fallback_row(t, key);
+  }
+  return 0;
+}
+
+template <typename K>
+int classify(ugk_table_t t, const K *keys, size_t n, uint64_t host_rows, const uint32_t *dst_map, ugk_idx_t *idx,
+             uint32_t *counts, uint32_t *next_counts, uint32_t *status, uint32_t *mirror) {
+  REQUIRE(counts && status, "ugk_classify: null counters or status");
+  if (check_table(t, "ugk_classify")) return 1;
+  if (next_counts) next_counts[0] = next_counts[1] = 0;
+  uint32_t h = counts[0], m = counts[1];
+  for (size_t i = 0; i < n; ++i) {
+    const uint64_t key = k64(keys[i]);
+    const Found f = lookup(t, key);
+    const uint32_t d = dst_map ? dst_map[i] : (uint32_t)i;
+    if (f.hit && f.loc == UGK_LOC_LOCAL) idx[h++] = ugk_idx_t{d, f.off};
+    else if (f.hit && f.loc == UGK_LOC_HOST && f.off < host_rows) idx[n - ++m] = ugk_idx_t{d, f.off};
+    else if (!f.hit && fallback_row(t, key) < host_rows && fallback_row(t, key) <= 0xffffffffull)
+      idx[n - ++m] = ugk_idx_t{d, (uint32_t)fallback_row(t, key)};
+    else or_status(status, UGK_ST_KEY_OUT_OF_RANGE, mirror);
+  }
+  counts[0] = h;
+  counts[1] = m;
+  return 0;
+}
+
+template <typename K>
+int nonlocal_flags(ugk_table_t t, const K *keys, size_t n, uint64_t *flags) {
+  if (n == 0) return 0;
+  if (check_table(t, "ugk_nonlocal_flags")) return 1;
+  for (size_t w = 0; w < (n + 63) / 64; ++w) {
+    uint64_t bits = 0;
+    for (size_t i = w * 64; i < std::min(n, w * 64 + 64); ++i) {
+      const Found f = lookup(t, k64(keys[i]));
+      if (!(f.hit && f.loc == UGK_LOC_LOCAL)) bits |= 1ull << (i & 63);
+    }
+    flags[w] = bits;
+  }
+  return 0;
+}
+
+template <typename K>
+int extract_mix(ugk_table_t t, const K *keys, size_t n, const void *cache, uint64_t cache_rows, const void *host,
+                uint64_t host_rows, void *out, size_t rb, uint32_t *status, uint32_t *mirror, uint64_t *counts,
+                uint32_t *num_groups) {
+  if (num_groups) *num_groups = 0;
+  if (n == 0) return 0;
+  REQUIRE(keys && out && status, "ugk_extract_mix: null keys, output or status");
+  if (check_table(t, "ugk_extract_mix")) return 1;
+  REQUIRE(rb > 0 && rb % 16 == 0, "ugk_extract_mix: rows must be multiples of 16 bytes (row_bytes=%zu)", rb);
+  uint64_t local = 0, others = 0;
+  for (size_t i = 0; i < n; ++i) {
+    const uint64_t key = k64(keys[i]);
+    const Found f = lookup(t, key);
+    const char *row = nullptr;
+    bool from_cache = false;
+    if (f.hit && f.loc == UGK_LOC_LOCAL && f.off < cache_rows) {
+      row = (const char *)cache + (size_t)f.off * rb;
+      from_cache = true;
+    } else if (f.hit && f.loc == UGK_LOC_HOST && f.off < host_rows) {
+      row = (const char *)host + (size_t)f.off * rb;
+    } else if (!f.hit && fallback_row(t, key) < host_rows) {
+      row = (const char *)host + fallback_row(t, key) * rb;
+    } else {
+      or_status(status, UGK_ST_KEY_OUT_OF_RANGE, mirror);
+    }
+    if (row) copy_row((char *)out + i * rb, row, rb);
+    if (from_cache) ++local;
+    else ++others;
+  }
+  if (counts) counts[0] = (others << 32) | local;
+  if (num_groups) *num_groups = 1;
+  return 0;
+}
+
+template <typename K>
+int dedup(const K *keys, size_t n, K *unique_out, uint32_t *inverse, uint32_t *rep, uint32_t *n_unique,
+          uint32_t *n_unique_host) {
+  if (n == 0) return 0;
+  REQUIRE(keys && unique_out && inverse && n_unique, "ugk_dedup: null pointer");
+  std::unordered_map<uint64_t, uint32_t> seen;
+  uint32_t nu = *n_unique;
+  for (size_t i = 0; i < n; ++i) {
+    auto it = seen.find(k64(keys[i]));
+    if (it == seen.end()) {
+      seen.emplace(k64(keys[i]), nu);
+      unique_out[nu] = keys[i];
+      if (rep) rep[nu] = (uint32_t)i;
+      inverse[i] = nu++;
+    } else {
+      inverse[i] = it->second;
+    }
+  }
+  *n_unique = nu;
+  if (n_unique_host) *n_unique_host = nu;
+  return 0;
+}
+
+template <typename K>
+int record(const K *keys, size_t n, uint64_t key_inv, uint64_t key_mask, uint32_t *counts, uint64_t num_rows,
+           uint64_t *observed, uint32_t *status, uint32_t *mirror) {
+  if (n == 0) return 0;
+  REQUIRE(keys && counts && status, "ugk_record: null pointer");
+  ugk_table_t map{};
+  map.fb_mul = key_inv;
+  map.fb_mask = key_mask;
+  for (size_t i = 0; i < n; ++i) {
+    const uint64_t row = fallback_row(map, k64(keys[i]));
+    if (row >= num_rows) {
+      or_status(status, UGK_ST_KEY_OUT_OF_RANGE, mirror);
+      continue;
+    }
+    const uint32_t before = __atomic_fetch_add(counts + row, 1u, __ATOMIC_RELAXED);
+    if (before == 0 && observed) __atomic_fetch_or(observed + (row >> 6), 1ull << (row & 63), __ATOMIC_RELAXED);
+  }
+  return 0;
+}
+
+uint64_t bm_word(const uint64_t *a, const uint64_t *b, int invert_a, uint64_t nbits, uint64_t w) {
+  uint64_t m = ld(a + w);
+  if (invert_a) m = ~m;
+  if (b) m &= ~ld(b + w);
+  if (nbits - w * 64 < 64) m &= (1ull << (nbits - w * 64)) - 1ull;
+  return m;
+}
+
+struct Event {
+  std::chrono::steady_clock::time_point at;
+};
+
+}  // namespace
+
+extern "C" {
+
+const char *ugk_last_error(void) { return g_err; }
+int ugk_abi_version(void) { return UGK_ABI_VERSION; }
+
+int ugk_device_count(int *count) {
+  *count = 1;
+  return 0;
+}
+int ugk_set_device(int dev) {
+  REQUIRE(dev == 0, "no device %d", dev);
+  return 0;
+}
+int ugk_get_device_info(int dev, ugk_device_info_t *info) {
+  REQUIRE(dev == 0 && info, "no device %d", dev);
+  memset(info, 0, sizeof(*info));
+  snprintf(info->name, sizeof(info->name), "cpu model of the ugk C-ABI (tests only)");
+  snprintf(info->arch, sizeof(info->arch), "none");
+  info->compute_units = 256;
+  info->wavefront_size = 64;
+  info->total_mem = 64ull << 30;
+  info->lds_per_block = 65536;
+  return 0;
+}
+int ugk_mem_info(size_t *free_bytes, size_t *total_bytes) {
+  if (free_bytes) *free_bytes = 32ull << 30;
+  if (total_bytes) *total_bytes = 64ull << 30;
+  return 0;
+}
+int ugk_malloc(void **ptr, size_t nbytes) { return alloc_block(ptr, nbytes, 2); }
+int ugk_free(void *ptr) { return free_block(ptr, 2); }
+int ugk_host_malloc(void **ptr, size_t nbytes) { return alloc_block(ptr, nbytes, 1); }
+int ugk_host_free(void *ptr) { return free_block(ptr, 1); }
+int ugk_pointer_kind(const void *ptr, int *kind) {
+  std::lock_guard<std::mutex> g(g_mem_mu);
+  *kind = 0;
+  auto it = g_blocks.upper_bound((uintptr_t)ptr);
+  if (it != g_blocks.begin()) {
+    --it;
+    if ((uintptr_t)ptr < it->first + it->second.first) *kind = it->second.second;
+  }
+  return 0;
+}
+int ugk_stream_create(void **stream) {
+  *stream = malloc(8);
+  return *stream ? 0 : fail("out of memory");
+}
+int ugk_stream_create_cu_masked(void **stream, int num_cus) {
+  REQUIRE(num_cus > 0, "ugk_stream_create_cu_masked: %d compute units", num_cus);
+  return ugk_stream_create(stream);
+}
+int ugk_stream_destroy(void *stream) {
+  free(stream);
+  return 0;
+}
+int ugk_stream_sync(void *) { return 0; }
+int ugk_device_sync(void) { return 0; }
+int ugk_event_create(void **event) {
+  *event = new Event{std::chrono::steady_clock::now()};
+  return 0;
+}
+int ugk_event_destroy(void *event) {
+  delete static_cast<Event *>(event);
+  return 0;
+}
+int ugk_event_record(void *event, void *) {
+  REQUIRE(event, "null event");
+  static_cast<Event *>(event)->at = std::chrono::steady_clock::now();
+  return 0;
+}
+int ugk_event_sync(void *) { return 0; }
+int ugk_stream_wait_event(void *, void *) { return 0; }
+int ugk_event_elapsed_ms(void *start, void *stop, float *ms) {
+  REQUIRE(start && stop && ms, "null event");
+  *ms = std::chrono::duration<float, std::milli>(static_cast<Event *>(stop)->at - static_cast<Event *>(start)->at)
+            .count();
+  return 0;
+}
+int ugk_memcpy_async(void *dst, const void *src, size_t nbytes, void *) {
+  if (nbytes) memmove(dst, src, nbytes);
+  return 0;
+}
+int ugk_fill_u32(uint32_t *dst, uint32_t value, size_t nwords, void *) {
+  for (size_t i = 0; i < nwords; ++i) st(dst + i, value);
+  return 0;
+}
+int ugk_arange_u32(uint32_t *dst, uint32_t start, size_t n, void *) {
+  for (size_t i = 0; i < n; ++i) dst[i] = start + (uint32_t)i;
+  return 0;
+}
+int ugk_copy_rows(void *dst, const void *src, size_t nbytes, void *) {
+  memcpy(dst, src, nbytes);
+  return 0;
+}
+
+int ugk_set_output_hint(int hint) {
+  REQUIRE(hint >= 0 && hint <= 2, "ugk_set_output_hint: unknown hint %d", hint);
+  return 0;
+}
+int ugk_gather_direct_u32(const void *src, uint64_t src_rows, const uint32_t *keys, size_t n, void *out, size_t rb,
+                          unsigned, uint32_t *status, uint32_t *mirror, void *) {
+  return gather_direct(src, src_rows, keys, nullptr, n, out, ~0ull, rb, status, mirror);
+}
+int ugk_gather_direct_i64(const void *src, uint64_t src_rows, const int64_t *keys, size_t n, void *out, size_t rb,
+                          unsigned, uint32_t *status, uint32_t *mirror, void *) {
+  return gather_direct(src, src_rows, keys, nullptr, n, out, ~0ull, rb, status, mirror);
+}
+int ugk_gather_scatter_u32(const void *src, uint64_t src_rows, const uint32_t *keys, const uint32_t *dst, size_t n,
+                           void *out, uint64_t out_rows, size_t rb, unsigned, uint32_t *status, uint32_t *mirror,
+                           void *) {
+  REQUIRE(n == 0 || dst, "ugk_gather_scatter_u32: null destinations");
+  return gather_direct(src, src_rows, keys, dst, n, out, out_rows, rb, status, mirror);
+}
+int ugk_gather_scatter_i64(const void *src, uint64_t src_rows, const int64_t *keys, const uint32_t *dst, size_t n,
+                           void *out, uint64_t out_rows, size_t rb, unsigned, uint32_t *status, uint32_t *mirror,
+                           void *) {
+  REQUIRE(n == 0 || dst, "ugk_gather_scatter_i64: null destinations");
+  return gather_direct(src, src_rows, keys, dst, n, out, out_rows, rb, status, mirror);
+}
+int ugk_replicate_rows(void *out, size_t rb, const uint32_t *inverse, const uint32_t *rep, size_t n, void *) {
+  for (size_t i = 0; i < n; ++i) {
+    const size_t r = rep[inverse[i]];
+    if (r != i) memcpy((char *)out + i * rb, (char *)out + r * rb, rb);
+  }
+  return 0;
+}
+int ugk_gather_group(const void *src, uint64_t src_rows, const ugk_idx_t *idx, const uint32_t *counts, uint32_t group,
+                     size_t n, void *out, uint64_t out_rows, size_t rb, unsigned, uint32_t *status, uint32_t *mirror,
+                     void *) {
+  if (n == 0) return 0;
+  REQUIRE(idx && counts && (group == UGK_LOC_LOCAL || group == UGK_LOC_HOST), "ugk_gather_group: bad argument");
+  const uint32_t c = counts[group];
+  if (mirror) mirror[1 + group] = c;
+  const size_t begin = group == UGK_LOC_LOCAL ? 0 : n - c;
+  return gather_list(src, src_rows, idx + begin, c, out, out_rows, rb, status, mirror);
+}
+int ugk_gather_idx(const void *src, uint64_t src_rows, const ugk_idx_t *idx, size_t count, void *out, size_t rb,
+                   unsigned, uint32_t *status, void *) {
+  return gather_list(src, src_rows, idx, count, out, ~0ull, rb, status, nullptr);
+}
+
+size_t ugk_hash_buckets_for(size_t n_entries, double load_factor) {
+  if (!(load_factor > 0.0) || load_factor > 0.95) load_factor = 0.7;
+  size_t nb = (size_t)std::ceil((double)n_entries / load_factor) + 1;
+  if (nb < 64) nb = 64;
+  return (nb + 7) / 8 * 8;
+}
+int ugk_hash_init(ugk_bucket_t *table, size_t nbuckets, void *) {
+  REQUIRE(table && nbuckets && nbuckets % 8 == 0, "ugk_hash_init: bad table");
+  for (size_t i = 0; i < nbuckets; ++i) {
+    st(&table[i].key, (uint64_t)UGK_HASH_EMPTY);
+    st(reinterpret_cast<uint64_t *>(&table[i].off), (uint64_t)0);
+  }
+  return 0;
+}
+int ugk_table_insert_u32(ugk_table_t t, const uint32_t *keys, const uint32_t *offs, uint32_t seq_base, uint32_t loc,
+                         size_t n, uint32_t *status, void *) {
+  return table_insert(t, keys, offs, seq_base, loc, n, status);
+}
+int ugk_table_insert_i64(ugk_table_t t, const int64_t *keys, const uint32_t *offs, uint32_t seq_base, uint32_t loc,
+                         size_t n, uint32_t *status, void *) {
+  return table_insert(t, keys, offs, seq_base, loc, n, status);
+}
+int ugk_table_evict_u32(ugk_table_t t, const uint32_t *keys, size_t n, uint32_t *status, void *) {
+  return table_evict(t, keys, n, status);
+}
+int ugk_table_evict_i64(ugk_table_t t, const int64_t *keys, size_t n, uint32_t *status, void *) {
+  return table_evict(t, keys, n, status);
+}
+int ugk_table_lookup_u32(ugk_table_t t, const uint32_t *keys, size_t n, uint32_t fallback_loc, uint32_t *loc_out,
+                         uint32_t *off_out, void *) {
+  return table_lookup(t, keys, n, fallback_loc, loc_out, off_out);
+}
+int ugk_table_lookup_i64(ugk_table_t t, const int64_t *keys, size_t n, uint32_t fallback_loc, uint32_t *loc_out,
+                         uint32_t *off_out, void *) {
+  return table_lookup(t, keys, n, fallback_loc, loc_out, off_out);
+}
+int ugk_hash_census(const ugk_bucket_t *table, size_t nbuckets, uint64_t *census, void *) {
+  REQUIRE(table && census, "ugk_hash_census: null pointer");
+  uint64_t occ = 0, tomb = 0, empty = 0;
+  for (size_t i = 0; i < nbuckets; ++i) {
+    const uint64_t k = ld(&table[i].key);
+    if (k == UGK_HASH_EMPTY) ++empty;
+    else if (k == UGK_HASH_TOMB) ++tomb;
+    else ++occ;
+  }
+  census[0] = occ;
+  census[1] = tomb;
+  census[2] = empty;
+  return 0;
+}
+
+int ugk_classify_u32(ugk_table_t t, const uint32_t *keys, size_t n, uint64_t host_rows, const uint32_t *dst_map,
+                     ugk_idx_t *idx, uint32_t *counts, uint32_t *next_counts, uint32_t *status, uint32_t *mirror,
+                     void *) {
+  return classify(t, keys, n, host_rows, dst_map, idx, counts, next_counts, status, mirror);
+}
+int ugk_classify_i64(ugk_table_t t, const int64_t *keys, size_t n, uint64_t host_rows, const uint32_t *dst_map,
+                     ugk_idx_t *idx, uint32_t *counts, uint32_t *next_counts, uint32_t *status, uint32_t *mirror,
+                     void *) {
+  return classify(t, keys, n, host_rows, dst_map, idx, counts, next_counts, status, mirror);
+}
+int ugk_nonlocal_flags_u32(ugk_table_t t, const uint32_t *keys, size_t n, uint64_t *flags, void *) {
+  return nonlocal_flags(t, keys, n, flags);
+}
+int ugk_nonlocal_flags_i64(ugk_table_t t, const int64_t *keys, size_t n, uint64_t *flags, void *) {
+  return nonlocal_flags(t, keys, n, flags);
+}
+int ugk_select_keys_u32(const uint32_t *keys, const uint32_t *sel, size_t m, uint32_t *out, void *) {
+  for (size_t j = 0; j < m; ++j) out[j] = keys[sel[j]];
+  return 0;
+}
+int ugk_select_keys_i64(const int64_t *keys, const uint32_t *sel, size_t m, int64_t *out, void *) {
+  for (size_t j = 0; j < m; ++j) out[j] = keys[sel[j]];
+  return 0;
+}
+
+unsigned ugk_extract_mix_max_groups(void) { return 16; }
+int ugk_extract_mix_u32(ugk_table_t t, const uint32_t *keys, size_t n, const void *cache, uint64_t cache_rows,
+                        const void *host, uint64_t host_rows, void *out, size_t rb, uint32_t *status, uint32_t *mirror,
+                        uint64_t *counts, uint32_t *num_groups, uint32_t, void *) {
+  return extract_mix(t, keys, n, cache, cache_rows, host, host_rows, out, rb, status, mirror, counts, num_groups);
+}
+int ugk_extract_mix_i64(ugk_table_t t, const int64_t *keys, size_t n, const void *cache, uint64_t cache_rows,
+                        const void *host, uint64_t host_rows, void *out, size_t rb, uint32_t *status, uint32_t *mirror,
+                        uint64_t *counts, uint32_t *num_groups, uint32_t, void *) {
+  return extract_mix(t, keys, n, cache, cache_rows, host, host_rows, out, rb, status, mirror, counts, num_groups);
+}
+
+size_t ugk_dedup_workspace_bytes(size_t) { return 64; }
+int ugk_dedup_u32(const uint32_t *keys, size_t n, void *, size_t, uint32_t epoch, uint32_t *unique_out,
+                  uint32_t *inverse, uint32_t *rep, uint32_t *n_unique, uint32_t *n_unique_host, void *) {
+  REQUIRE(epoch != 0, "ugk_dedup: epoch must be non-zero");
+  return dedup(keys, n, unique_out, inverse, rep, n_unique, n_unique_host);
+}
+int ugk_dedup_i64(const int64_t *keys, size_t n, void *, size_t, uint32_t epoch, int64_t *unique_out,
+                  uint32_t *inverse, uint32_t *rep, uint32_t *n_unique, uint32_t *n_unique_host, void *) {
+  REQUIRE(epoch != 0, "ugk_dedup: epoch must be non-zero");
+  return dedup(keys, n, unique_out, inverse, rep, n_unique, n_unique_host);
+}
+int ugk_dedup_static(const void *keys, uint32_t key_bytes, size_t n, void *unique_out, uint32_t *inverse,
+                     uint32_t *rep, uint32_t *n_unique, uint32_t *n_unique_host, void *) {
+  REQUIRE(key_bytes == 4 || key_bytes == 8, "ugk_dedup_static: keys of %u bytes", key_bytes);
+  REQUIRE(n <= UGK_DEDUP_STATIC_MAX_KEYS, "ugk_dedup_static: batch too large");
+  *n_unique = 0;
+  if (key_bytes == 4)
+    return dedup((const uint32_t *)keys, n, (uint32_t *)unique_out, inverse, rep, n_unique, n_unique_host);
+  return dedup((const int64_t *)keys, n, (int64_t *)unique_out, inverse, rep, n_unique, n_unique_host);
+}
+
+int ugk_record_u32(const uint32_t *keys, size_t n, uint64_t key_inv, uint64_t key_mask, uint32_t *counts,
+                   uint64_t num_rows, uint64_t *observed, uint32_t *status, uint32_t *mirror, void *) {
+  return record(keys, n, key_inv, key_mask, counts, num_rows, observed, status, mirror);
+}
+int ugk_record_i64(const int64_t *keys, size_t n, uint64_t key_inv, uint64_t key_mask, uint32_t *counts,
+                   uint64_t num_rows, uint64_t *observed, uint32_t *status, uint32_t *mirror, void *) {
+  return record(keys, n, key_inv, key_mask, counts, num_rows, observed, status, mirror);
+}
+int ugk_record_drain(uint32_t *counts, uint64_t first_row, uint64_t num_rows, uint64_t *observed, uint64_t *entries,
+                     uint32_t capacity, uint32_t *n_entries, uint32_t *host_out, void *) {
+  REQUIRE(counts && entries && n_entries && host_out && capacity, "ugk_record_drain: bad argument");
+  uint32_t written = 0, more = 0;
+  for (uint64_t r = first_row; r < first_row + num_rows; ++r) {
+    if (ld(counts + r) == 0) continue;
+    if (written == capacity) {
+      more = 1;
+      break;
+    }
+    if (observed) __atomic_fetch_and(observed + (r >> 6), ~(1ull << (r & 63)), __ATOMIC_RELAXED);
+    const uint32_t got = __atomic_exchange_n(counts + r, 0u, __ATOMIC_RELAXED);
+    entries[written++] = ((uint64_t)got << 32) | (uint32_t)r;
+  }
+  host_out[0] = written;
+  host_out[1] = more;
+  *n_entries = 0;
+  return 0;
+}
+
+size_t ugk_rank_workspace_bytes(void) { return 64; }
+int ugk_rank_place(uint32_t *counts, uint64_t num_rows, uint64_t k, void *ws, uint64_t *in_new, uint64_t *scratch,
+                   uint64_t *observed, int reset_counts, void *) {
+  REQUIRE(counts && ws && in_new && scratch, "ugk_rank_place: null pointer");
+  REQUIRE(num_rows > 0 && num_rows < 0xffffffffull, "ugk_rank_place: rows do not fit 32 bits");
+  const uint64_t n_words = (num_rows + 63) / 64;
+  std::vector<uint64_t> rank(num_rows);
+  for (uint64_t r = 0; r < num_rows; ++r) {
+    const uint32_t c = ld(counts + r);
+    rank[r] = c ? ((uint64_t)c << 32) | r : (uint64_t)(0xffffffffu - r);
+  }
+  uint64_t threshold;
+  if (k == 0) threshold = ~0ull;
+  else if (k >= num_rows) threshold = 0;
+  else {
+    std::vector<uint64_t> tmp(rank);
+    std::nth_element(tmp.begin(), tmp.begin() + (k - 1), tmp.end(), std::greater<uint64_t>());
+    threshold = tmp[k - 1];
+  }
+  for (uint64_t w = 0; w < n_words; ++w) {
+    uint64_t m = 0;
+    for (uint64_t r = w * 64; r < std::min(num_rows, w * 64 + 64); ++r)
+      if (k != 0 && rank[r] >= threshold) m |= 1ull << (r & 63);
+    in_new[w] = m;
+    scratch[w] = 0;
+  }
+  if (reset_counts) {
+    for (uint64_t r = 0; r < num_rows; ++r) st(counts + r, 0u);
+    if (observed)
+      for (uint64_t w = 0; w < n_words; ++w) st(observed + w, (uint64_t)0);
+  }
+  *static_cast<uint64_t *>(ws) = threshold;
+  return 0;
+}
+int ugk_rank_threshold(const void *ws, uint64_t *threshold_host, void *) {
+  *threshold_host = *static_cast<const uint64_t *>(ws);
+  return 0;
+}
+size_t ugk_bitmap_workspace_bytes(void) { return 64; }
+int ugk_bitmap_count(const uint64_t *a, const uint64_t *b, int invert_a, uint64_t nbits, void *ws,
+                     uint32_t *total_host, void *) {
+  REQUIRE(a && ws && nbits > 0 && nbits <= 0xffffffffull, "ugk_bitmap_count: bad argument");
+  uint32_t total = 0;
+  for (uint64_t w = 0; w < (nbits + 63) / 64; ++w) total += __builtin_popcountll(bm_word(a, b, invert_a, nbits, w));
+  *static_cast<uint32_t *>(ws) = total;
+  if (total_host) *total_host = total;
+  return 0;
+}
+int ugk_bitmap_emit(const uint64_t *a, const uint64_t *b, int invert_a, uint64_t nbits, const void *ws, uint32_t *out,
+                    uint64_t max_out, void *) {
+  REQUIRE(a && ws && nbits > 0 && nbits <= 0xffffffffull, "ugk_bitmap_emit: bad argument");
+  if (max_out == 0) return 0;
+  REQUIRE(out, "ugk_bitmap_emit: null output list");
+  uint64_t pos = 0;
+  for (uint64_t w = 0; w < (nbits + 63) / 64 && pos < max_out; ++w) {
+    uint64_t m = bm_word(a, b, invert_a, nbits, w);
+    while (m && pos < max_out) {
+      out[pos++] = (uint32_t)(w * 64 + __builtin_ctzll(m));
+      m &= m - 1;
+    }
+  }
+  return 0;
+}
+int ugk_bitmap_update(uint64_t *bitmap, uint64_t nbits, const uint32_t *idx, size_t n, int set, uint32_t *status,
+                      void *) {
+  if (n == 0) return 0;
+  REQUIRE(bitmap && idx && status, "ugk_bitmap_update: null pointer");
+  for (size_t i = 0; i < n; ++i) {
+    const uint32_t p = idx[i];
+    if (p >= nbits) {
+      or_status(status, UGK_ST_KEY_OUT_OF_RANGE);
+      continue;
+    }
+    if (set) __atomic_fetch_or(bitmap + (p >> 6), 1ull << (p & 63), __ATOMIC_RELAXED);
+    else __atomic_fetch_and(bitmap + (p >> 6), ~(1ull << (p & 63)), __ATOMIC_RELAXED);
+  }
+  return 0;
+}
+int ugk_rows_to_keys(const uint32_t *rows, size_t n, uint64_t mul, uint64_t mask, int64_t *keys_out, void *) {
+  REQUIRE(n == 0 || (rows && keys_out && (mul & 1ull)), "ugk_rows_to_keys: bad argument");
+  for (size_t i = 0; i < n; ++i) keys_out[i] = (int64_t)(((uint64_t)rows[i] * mul) & mask);
+  return 0;
+}
+
+}  // extern "C"

@@ -563,6 +563,15 @@ uint32_t ExtractSession::MixOthersHint(size_t num_nodes) const {
   return (uint32_t)((double)_mix_seen_others / (double)_mix_seen_rows * (double)num_nodes);
 }
 
+// A lookup the refresh thread must wait for: counted from before it reads the table handle until its output is complete
+// (blocking lookups) or until its kernels are enqueued on their stream (stream-ordered ones, which the refresh then
+// finds by waiting for that stream).
+struct ExtractSession::InFlight {
+  ExtractSession *s;
+  explicit InFlight(ExtractSession *session) : s(session) { s->_blocking_started.fetch_add(1); }
+  ~InFlight() { s->_blocking_finished.fetch_add(1); }
+};
+
 // cache_context.cu:1199-1794
 template <typename KeyT>
 void ExtractSession::ExtractFeatImpl(const KeyT *nodes, size_t num_nodes, void *output, StreamHandle stream,
@@ -571,11 +580,7 @@ void ExtractSession::ExtractFeatImpl(const KeyT *nodes, size_t num_nodes, void *
   auto profiler = ctx->_coll_cache ? ctx->_coll_cache->_profiler : nullptr;
   const size_t rb = ctx->_row_bytes;
   const size_t nbytes = num_nodes * rb;
-  struct InFlight {  // counted from before the first kernel reads the table until the output is complete
-    ExtractSession *s;
-    explicit InFlight(ExtractSession *session) : s(session) { s->_blocking_started.fetch_add(1); }
-    ~InFlight() { s->_blocking_finished.fetch_add(1); }
-  } in_flight(this);
+  InFlight in_flight(this);  // from before the first kernel reads the table until the output is complete
   Wait(stream);  // stream-ordered lookups still in flight share the mirror words this call reads
   _group_offset[0] = 0;
   if (num_nodes == 0) {
@@ -809,6 +814,10 @@ void ExtractSession::ExtractFeatAsyncImpl(const KeyT *nodes, size_t num_nodes, v
   NoteOutput(output, num_nodes * rb);
   NoteAsyncStream(stream);  // before the first kernel is enqueued: a refresh that does not see the stream yet has
                             // finished its evictions before that kernel can start
+  // Between reading the table handle and enqueueing the kernel that uses it this call is "in flight" on the host: a
+  // refresh that swaps the table for a rebuilt one waits for the count before it waits for the stream and frees the old
+  // buckets, so the kernel below never reads freed memory.
+  InFlight enqueueing(this);
   if (ctx->IsDirectMapping() && !dedup) {
     const bool from_host = ctx->_cpu_location_id != -1;
     void *keys_ready = RecordBegin(stream);
@@ -895,25 +904,27 @@ void ExtractSession::NoteAsyncStream(StreamHandle stream) {
 }
 
 void ExtractSession::WaitForLookupsInFlight(bool foreground, double timeout_s) {
+  if (!foreground) {
+    // A lookup counts itself before it reads the table: one that is not counted yet starts after the evictions (or the
+    // table swap) have completed.  Blocking lookups stay counted until their output is complete, stream-ordered ones
+    // until their kernels are enqueued, which is why the streams are waited for after the count, not before.
+    const size_t started = _blocking_started.load();
+    Timer t0;
+    while (_blocking_finished.load() < started) {
+      if (t0.PassedSec() >= timeout_s) {
+        LOG(ERROR) << "refresh: a lookup that started before the eviction has not returned after " << timeout_s
+                   << " s; going on";
+        break;
+      }
+      usleep(20);
+    }
+  }
   std::vector<StreamHandle> streams;
   {
     std::lock_guard<std::mutex> guard(_async_mu);
     streams = _async_streams;
   }
   for (StreamHandle s : streams) UGK_CALL(ugk_stream_sync(s));
-  if (foreground) return;
-  // a blocking lookup counts itself before its first kernel is enqueued: one that is not counted yet starts after the
-  // evictions have completed
-  const size_t started = _blocking_started.load();
-  Timer t0;
-  while (_blocking_finished.load() < started) {
-    if (t0.PassedSec() >= timeout_s) {
-      LOG(ERROR) << "refresh: a lookup that started before the eviction has not returned after " << timeout_s
-                 << " s; going on";
-      break;
-    }
-    usleep(20);
-  }
 }
 
 void ExtractSession::Wait(StreamHandle stream) {

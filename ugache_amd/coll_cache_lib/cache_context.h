@@ -157,6 +157,7 @@ class ExtractSession {
   size_t _async_last_nodes = 0;    // size of the last of them
   // What a refresh has to see finished before it reuses the slots of evicted rows: blocking lookups are counted when
   // they start and when they end, the streams stream-ordered lookups were enqueued on are remembered (normally one).
+  struct InFlight;
   std::atomic<size_t> _blocking_started{0}, _blocking_finished{0};
   std::mutex _async_mu;
   std::vector<StreamHandle> _async_streams;  // guarded by _async_mu
