@@ -109,6 +109,11 @@ def parse_args():
     ap.add_argument("--calibrate", action="store_true",
                     help="also run 5 plain device copies of 1 GiB (ugk_copy_rows) so a counter run has a kernel of "
                          "known traffic next to the gather")
+    ap.add_argument("--probe", default=None, choices=["kpw", "row_span", "cu_mask"],
+                    help="instead of a workload, run one of the stand-alone measurements behind the launch rules "
+                         "(ugache_amd/probes.py): keys per wavefront of the fused kernel, random rows over the host "
+                         "link by span, host-link gather confined to a few compute units; prints one JSON line")
+    ap.add_argument("--quick", action="store_true", help="with --probe: a reduced sweep")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs the extraction path of ONE GPU (no collectives, no peer source); "
@@ -874,6 +879,11 @@ def emit(result):
 def main():
     global _REAL_STDOUT
     args = parse_args()
+    if args.probe:
+        from ugache_amd import probes
+
+        probes.run(args.probe, args.quick)
+        return
     if args.workload is None:
         return run_default(args)
     # the library prints the reference's progress lines ("test_result:init:...", solver summary) on stdout; they go

@@ -142,7 +142,12 @@ def test_build_of_every_replica_with_an_allocator_builder(pct):
         want_local = n if pct == 1.0 else 0 if pct == 0.0 else int((nid[keys] == 0).sum())
         assert _basics.last_group_offset(0) == [0, want_local, n]
     if 0.0 < pct < 1.0:
-        assert handed_out  # the factored / dedup scratch of a partial cache comes from the builder's allocator
+        # the fused extraction needs no scratch; the set of a distinct-keys lookup comes from the builder's allocator
+        assert not handed_out
+        keys = perm[zipf_ranks(rng, 5000, n_item, 1.1)]
+        rows, inverse = co.coll_torch_lookup_unique(0, torch.from_numpy(keys).cuda())
+        assert rows[inverse.long()].cpu().numpy().tobytes() == ORC.gather(table, keys).tobytes()
+        assert handed_out
 
 
 @pytest.mark.parametrize("table_kind", ["FLAT", "HASH"])

@@ -509,6 +509,12 @@ int extract_mix_lpr(ugk_table_t t, const K *keys, size_t n, const void *cache, u
   } else {
     kpw = n <= slots * 8 ? 16 : n <= slots * 16 ? 32 : n <= slots * 32 ? 64 : 16;
   }
+  // UGK_MIX_KPW=8|16|32|64 forces the shape (read on every launch: the sweep that measures the rule above changes it
+  // between launches); never a byte of the result depends on it
+  if (const char *forced = getenv("UGK_MIX_KPW")) {
+    const int v = atoi(forced);
+    if (v == 8 || v == 16 || v == 32 || v == 64) kpw = v;
+  }
   if (kpw < kWave / lpr) kpw = kWave / lpr;  // one wavefront instruction copies 64 / lpr rows
   const size_t keys_per_group = (size_t)kpw * kWavesPerBlock;
   const unsigned grid = clamp_grid((n + keys_per_group - 1) / keys_per_group, 0);

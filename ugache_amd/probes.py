@@ -1,0 +1,243 @@
+"""Stand-alone measurements behind the launch rules of the extraction kernels, callable as `bench.py --probe NAME`.
+
+Each probe drives the kernels through the C-ABI of include/ugache_hip.h on synthetic inputs and times them with two
+HIP events around back-to-back launches on the launch stream.  They measure and print; they check only that no launch
+flagged an error (the parity tests check results).
+
+  kpw       keys per wavefront of the fused lookup + gather kernel (ugk_extract_mix_i64), every shape forced in turn
+            with UGK_MIX_KPW, by table kind, row size, miss rate and batch size
+  row_span  uniformly random rows of 128 and 512 bytes gathered out of one large pinned host allocation, the rows drawn
+            from its first S GiB: what small rows reach over the host link, and how that depends on the span
+  cu_mask   a host-link gather on a side stream next to an HBM gather on the main stream: side stream plain or
+            confined to 8 / 16 / 32 compute units (ugk_stream_create_cu_masked), grid capped to 32 - 256 workgroups
+"""
+import ctypes as C
+import json
+import os
+import sys
+import time
+
+
+def _event(hip):
+    e = C.c_void_p()
+    hip.call("ugk_event_create", C.byref(e))
+    return e
+
+
+def _elapsed_us(hip, a, b):
+    ms = C.c_float()
+    hip.call("ugk_event_elapsed_ms", a, b, C.byref(ms))
+    return ms.value * 1e3
+
+
+def _timed(hip, stream, fn, reps, warm=3):
+    """average microseconds per call of fn(i), reps calls back to back between two events on `stream`"""
+    for i in range(warm):
+        fn(i)
+    hip.call("ugk_stream_sync", stream)
+    a, b = _event(hip), _event(hip)
+    hip.call("ugk_event_record", a, stream)
+    for i in range(reps):
+        fn(i)
+    hip.call("ugk_event_record", b, stream)
+    hip.call("ugk_event_sync", b)
+    us = _elapsed_us(hip, a, b) / reps
+    hip.call("ugk_event_destroy", a)
+    hip.call("ugk_event_destroy", b)
+    return us
+
+
+def _pinned(hip, nbytes):
+    p = C.c_void_p()
+    hip.call("ugk_host_malloc", C.byref(p), nbytes)
+    return p
+
+
+def _check_status(torch, st, what):
+    if int(st[0].item()) != 0:
+        sys.exit("probe %s: a launch flagged status %d" % (what, int(st[0].item())))
+
+
+def probe_kpw(hip, torch, note, quick=False):
+    rows = 2_000_000
+    stream = C.c_void_p()
+    hip.call("ugk_stream_create", C.byref(stream))
+    words = _pinned(hip, hip.lib().ugk_extract_mix_max_groups() * 8)
+    groups = C.c_uint32(0)
+    st = torch.zeros(4, dtype=torch.int32, device="cuda")
+    sizes = (8192, 65536, 262144) if quick else (8192, 32768, 65536, 131072, 212992, 262144, 524288, 1048576)
+    cases = ((512, 1),) if quick else ((512, 1), (512, 10), (128, 1), (128, 10))
+    out_rows = []
+    saved = os.environ.get("UGK_MIX_KPW")
+    for kind in ("flat", "hash"):
+        for rb, miss_pct in cases:
+            ncache = int(rows * (1 - miss_pct / 100))
+            if kind == "flat":
+                mem = torch.empty(rows, dtype=torch.int32, device="cuda")
+                hip.call("ugk_fill_u32", mem.data_ptr(), hip.EMPTY_U32, rows, stream)
+                tb = hip.table(hip.TABLE_FLAT, mem.data_ptr(), rows)
+            else:
+                nb = hip.lib().ugk_hash_buckets_for(ncache, 0.7)
+                mem = torch.empty(nb * 16 + 128, dtype=torch.uint8, device="cuda")
+                base = (mem.data_ptr() + 127) // 128 * 128
+                hip.call("ugk_hash_init", base, nb, stream)
+                tb = hip.table(hip.TABLE_HASH, base, nb)
+            cached = torch.arange(ncache, dtype=torch.int64, device="cuda")
+            hip.call("ugk_table_insert_i64", tb, cached.data_ptr(), None, 0, hip.LOC_LOCAL, ncache, st.data_ptr(), stream)
+            cache = torch.randint(0, 2 ** 31 - 1, (ncache, rb // 4), dtype=torch.int32, device="cuda")
+            host = _pinned(hip, rows * rb)
+            C.memset(host, 7, rows * rb)
+            pool = 8
+            for n in sizes:
+                keys = torch.randint(0, rows, (pool, n), device="cuda", dtype=torch.int64)
+                out = torch.empty((n, rb // 4), dtype=torch.int32, device="cuda")
+                torch.cuda.synchronize()
+                row = {"table": kind, "row_bytes": rb, "miss_pct": miss_pct, "keys": n, "us_by_keys_per_wavefront": {}}
+                for kpw in ("rule", 8, 16, 32, 64):
+                    if kpw == "rule":
+                        os.environ.pop("UGK_MIX_KPW", None)
+                    else:
+                        os.environ["UGK_MIX_KPW"] = str(kpw)
+
+                    def go(i):
+                        hip.call("ugk_extract_mix_i64", tb, keys[i % pool].data_ptr(), n, cache.data_ptr(), ncache,
+                                 host, rows, out.data_ptr(), rb, st.data_ptr(), None, words, C.byref(groups),
+                                 hip.HINT_UNKNOWN, stream)
+                    row["us_by_keys_per_wavefront"][str(kpw)] = round(_timed(hip, stream, go, 50), 2)
+                out_rows.append(row)
+                note("kpw %s %d B %d %% misses, %d keys: %s" % (kind, rb, miss_pct, n, row["us_by_keys_per_wavefront"]))
+                del keys, out
+            _check_status(torch, st, "kpw")
+            hip.call("ugk_host_free", host)
+            del cache, mem, cached
+    if saved is None:
+        os.environ.pop("UGK_MIX_KPW", None)
+    else:
+        os.environ["UGK_MIX_KPW"] = saved
+    hip.call("ugk_host_free", words)
+    return {"probe": "kpw", "table_rows": rows, "launches_timed": 50,
+            "how": "ugk_extract_mix_i64 over a table of which 99 % / 90 % is cached (uniform keys); 'rule' = the "
+                   "launcher's own choice, the others forced with UGK_MIX_KPW; 2 HIP events around 50 launches",
+            "rows": out_rows}
+
+
+def probe_row_span(hip, torch, note, quick=False):
+    GiB = 1 << 30
+    total = (8 if quick else 60) * GiB
+    stream = C.c_void_p()
+    hip.call("ugk_stream_create", C.byref(stream))
+    t0 = time.perf_counter()
+    host = _pinned(hip, total)
+    note("pinned %d GiB in %.1f s" % (total // GiB, time.perf_counter() - t0))
+    st = torch.zeros(4, dtype=torch.int32, device="cuda")
+    g = torch.Generator(device="cuda").manual_seed(1)
+    res = []
+    spans = (1, 4, 8) if quick else (1, 4, 16, 32, 60)
+    for rb in (128, 512):
+        for span in spans:
+            rows = span * GiB // rb
+            for n in (159_000, 262_144):
+                keys = torch.randint(0, rows, (8, n), generator=g, device="cuda", dtype=torch.int64)
+                out = torch.empty(n * rb, dtype=torch.uint8, device="cuda")
+                torch.cuda.synchronize()
+                by_cap = {}
+                for cap in (128, 512, 0):
+                    def go(i):
+                        hip.call("ugk_gather_direct_i64", host, rows, keys[i % 8].data_ptr(), n, out.data_ptr(), rb,
+                                 cap, st.data_ptr(), None, stream)
+                    us = _timed(hip, stream, go, 8, warm=2)
+                    by_cap[str(cap or "unlimited")] = round(n * rb / us / 1e3, 2)
+                res.append({"row_bytes": rb, "span_GiB": span, "rows_per_launch": n, "GBps_by_workgroup_cap": by_cap})
+                note("rows of %d B over the first %d GiB, n = %d: %s GB/s" % (rb, span, n, by_cap))
+                del keys, out
+    _check_status(torch, st, "row_span")
+    hip.call("ugk_host_free", host)
+    return {"probe": "row_span", "allocation_GiB": total // GiB,
+            "how": "ugk_gather_direct_i64 of uniformly random rows of one pinned allocation (which the probe "
+                   "does not fill), 2 HIP events around 8 launches", "rows": res}
+
+
+def probe_cu_mask(hip, torch, note, quick=False):
+    rows, rb = (4_194_304 if quick else 16_777_216), 512
+    nbytes = rows * rb
+    main, plain = C.c_void_p(), C.c_void_p()
+    hip.call("ugk_stream_create", C.byref(main))
+    hip.call("ugk_stream_create", C.byref(plain))
+    host = _pinned(hip, nbytes)
+    drows = 10_000_000
+    dtable = torch.empty((drows, rb // 4), dtype=torch.float32, device="cuda").normal_()
+    g = torch.Generator(device="cuda").manual_seed(4)
+    n_miss, n_hit = 250_000, 800_000
+    mk = torch.randint(0, rows, (n_miss,), generator=g, device="cuda", dtype=torch.int32)
+    hk = torch.randint(0, drows, (n_hit,), generator=g, device="cuda", dtype=torch.int32)
+    mout = torch.empty((n_miss, rb // 4), dtype=torch.float32, device="cuda")
+    hout = torch.empty((n_hit, rb // 4), dtype=torch.float32, device="cuda")
+    st = torch.zeros(4, dtype=torch.int32, device="cuda")
+    torch.cuda.synchronize()
+    ev = [_event(hip) for _ in range(4)]
+    res = []
+
+    def trial(side, blocks, label):
+        last = None
+        for _ in range(4):
+            hip.call("ugk_event_record", ev[0], side)
+            hip.call("ugk_gather_direct_u32", host, rows, mk.data_ptr(), n_miss, mout.data_ptr(), rb, blocks,
+                     st.data_ptr(), None, side)
+            hip.call("ugk_event_record", ev[1], side)
+            hip.call("ugk_event_record", ev[2], main)
+            hip.call("ugk_gather_direct_u32", dtable.data_ptr(), drows, hk.data_ptr(), n_hit, hout.data_ptr(), rb, 0,
+                     st.data_ptr(), None, main)
+            hip.call("ugk_event_record", ev[3], main)
+            hip.call("ugk_stream_sync", side)
+            hip.call("ugk_stream_sync", main)
+            last = (_elapsed_us(hip, ev[0], ev[1]), _elapsed_us(hip, ev[2], ev[3]))
+        res.append({"side_stream": label, "workgroup_cap": blocks, "host_gather_us": round(last[0], 1),
+                    "host_gather_GBps": round(n_miss * rb / last[0] / 1e3, 2),
+                    "concurrent_hbm_gather_us": round(last[1], 1)})
+        note("%s, %d workgroups: host gather %.1f us (%.1f GB/s), HBM gather next to it %.1f us"
+             % (label, blocks, last[0], n_miss * rb / last[0] / 1e3, last[1]))
+
+    def alone():
+        def go(i):
+            hip.call("ugk_gather_direct_u32", dtable.data_ptr(), drows, hk.data_ptr(), n_hit, hout.data_ptr(), rb, 0,
+                     st.data_ptr(), None, main)
+        return _timed(hip, main, go, 8)
+
+    hbm_alone = alone()
+    note("HBM gather alone: %.1f us" % hbm_alone)
+    for blocks in (32, 64, 128, 256):
+        trial(plain, blocks, "plain")
+    for ncu in (8, 16, 32):
+        masked = C.c_void_p()
+        hip.call("ugk_stream_create_cu_masked", C.byref(masked), ncu)
+        for blocks in (32, 64, 128, 256):
+            trial(masked, blocks, "confined to %d CUs" % ncu)
+        hip.call("ugk_stream_destroy", masked)
+    _check_status(torch, st, "cu_mask")
+    hip.call("ugk_host_free", host)
+    return {"probe": "cu_mask", "host_rows": rows, "row_bytes": rb, "host_gather_rows": n_miss, "hbm_gather_rows": n_hit,
+            "hbm_gather_alone_us": round(hbm_alone, 1),
+            "how": "ugk_gather_direct_u32 from pinned host memory on a side stream and from HBM on the main stream, "
+                   "launched together, one event pair around each; the last of 4 rounds", "rows": res}
+
+
+PROBES = {"kpw": probe_kpw, "row_span": probe_row_span, "cu_mask": probe_cu_mask}
+
+
+def run(name, quick=False):
+    import torch
+
+    from . import hip
+
+    if not torch.cuda.is_available():
+        sys.exit("probes need a GPU")
+    t0 = time.perf_counter()
+
+    def note(msg):
+        print("[probe %6.1fs] %s" % (time.perf_counter() - t0, msg), file=sys.stderr, flush=True)
+
+    res = PROBES[name](hip, torch, note, quick)
+    info = hip.device_info(0)
+    res["device"] = "%s %s" % (info["name"], info["arch"])
+    print(json.dumps(res), flush=True)
+    return res
