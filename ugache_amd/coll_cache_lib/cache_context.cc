@@ -989,27 +989,30 @@ void RefreshSession::WaitForOneLookup(ExtractSession *session, bool foreground) 
 }
 
 void RefreshSession::CopyRowsIntoSlots(const uint32_t *rows_dev, const uint32_t *slots_dev, size_t num_rows,
-                                       bool foreground) {
+                                       bool foreground, StreamHandle copy_stream) {
   CacheContext *ctx = _cache_ctx.get();
   const void *host = ctx->_device_cache_data[ctx->_cpu_location_id];
   void *cache = ctx->_device_cache_data[ctx->_local_location_id];
   uint32_t *status = _status_handle->ptr<uint32_t>();
   // background refresh copies in small throttled batches so that foreground lookups keep the host link
   const size_t batch = foreground ? num_rows : std::max<size_t>(RunConfig::refresh_batch_rows, 1);
-  const unsigned limit_block = foreground ? 0 : RunConfig::refresh_limit_block;
+  // alone on the chip the copy still takes a capped grid: rows of 512 bytes and more cross the link faster from 128
+  // workgroups than from as many as the rows would fill (56.9 against 52.7 GB/s)
+  const unsigned limit_block = foreground ? 128 : RunConfig::refresh_limit_block;
   for (size_t begin = 0; begin < num_rows; begin += batch) {
     const size_t cur = std::min(batch, num_rows - begin);
     UGK_CALL(ugk_gather_scatter_u32(host, ctx->_num_total_nodes, rows_dev + begin, slots_dev + begin, cur, cache,
                                     ctx->_cache_space_capacity, ctx->_row_bytes, limit_block, status, nullptr,
-                                    low_pri_stream));
+                                    copy_stream));
     if (!foreground && begin + batch < num_rows) {
-      UGK_CALL(ugk_stream_sync(low_pri_stream));
+      UGK_CALL(ugk_stream_sync(copy_stream));
       usleep(RunConfig::refresh_sleep_us);
     }
   }
+  if (copy_stream == stream) return;  // the caller looks at the status word when it waits for its stream
   uint32_t st = 0;
-  UGK_CALL(ugk_memcpy_async(&st, status, sizeof(st), low_pri_stream));
-  UGK_CALL(ugk_stream_sync(low_pri_stream));
+  UGK_CALL(ugk_memcpy_async(&st, status, sizeof(st), copy_stream));
+  UGK_CALL(ugk_stream_sync(copy_stream));
   CHECK_EQ(st, 0u) << "refresh row copy touched a row outside its table";
 }
 
@@ -1089,7 +1092,8 @@ void RefreshSession::refresh_after_solve_new(bool foreground) {
     auto insert_keys_gpu = CopyTo1DReuse(__keys_buffer, new_insert_keys, gpu_ctx, low_pri_stream);
     auto reserved_offset =
         CopyTo1DReuse(__offs_buffer, table->ReserveOffsetFront((IdType)num_insert), gpu_ctx, low_pri_stream);
-    CopyRowsIntoSlots(insert_keys_gpu->CPtr<uint32_t>(), reserved_offset->CPtr<uint32_t>(), num_insert, foreground);
+    CopyRowsIntoSlots(insert_keys_gpu->CPtr<uint32_t>(), reserved_offset->CPtr<uint32_t>(), num_insert, foreground,
+                      low_pri_stream);
     auto insert_table_keys =
         RunConfig::key_map_mul == 0
             ? insert_keys_gpu
@@ -1137,14 +1141,18 @@ void RefreshSession::refresh_on_device(ExtractSession *session, size_t num_cache
   const double sync_s = t_phase.Passed();
   t_phase.Reset();
 
-  // Steps 1-3: the new placement as a bitmap, then evict = cached & ~new and insert = new & ~cached, ascending
+  // Steps 1-3: the new placement as a bitmap, then evict = cached & ~new and insert = new & ~cached, ascending.  Both
+  // sets are counted before the one wait that tells the host their sizes.
   session->PlaceOnDevice(num_cached, table->InNewBits(), table->_dev_scratch_bits->ptr<uint64_t>(),
                          table->_dev_rank_ws->ptr(), !RunConfig::gpu_refresh_keep, stream);
-  size_t num_evicted = 0, num_insert = 0;
-  TensorPtr evict_rows = table->CompactBits(table->InCacheBits(), table->InNewBits(), false, num_rows, SIZE_MAX,
-                                            __evict_rows, alloc, gpu_ctx, stream, &num_evicted);
-  TensorPtr insert_rows = table->CompactBits(table->InNewBits(), table->InCacheBits(), false, num_rows, SIZE_MAX,
-                                             __insert_rows, alloc, gpu_ctx, stream, &num_insert);
+  volatile uint32_t *n_evict_word = table->CountBits(table->InCacheBits(), table->InNewBits(), false, num_rows, 0, stream);
+  volatile uint32_t *n_insert_word = table->CountBits(table->InNewBits(), table->InCacheBits(), false, num_rows, 1, stream);
+  UGK_CALL(ugk_stream_sync(stream));
+  const size_t num_evicted = *n_evict_word, num_insert = *n_insert_word;
+  TensorPtr evict_rows = table->EmitBits(table->InCacheBits(), table->InNewBits(), false, num_rows, 0, num_evicted,
+                                         __evict_rows, alloc, gpu_ctx, stream);
+  TensorPtr insert_rows = table->EmitBits(table->InNewBits(), table->InCacheBits(), false, num_rows, 1, num_insert,
+                                          __insert_rows, alloc, gpu_ctx, stream);
   const size_t num_old = table->_num_cached;
   CHECK_LE(num_evicted, num_old);
   const size_t num_preserved_key = num_old - num_evicted;
@@ -1152,7 +1160,8 @@ void RefreshSession::refresh_on_device(ExtractSession *session, size_t num_cache
   const double place_s = t_phase.Passed();
   t_phase.Reset();
 
-  // Step 4: the evicted keys leave the table, their slots become free
+  // Step 4: the evicted keys leave the table, their slots become free.  A foreground refresh looks at the status words
+  // of its kernels once, at the end; a background one, which lookups run beside, after every step.
   if (num_evicted > 0) {
     TensorPtr evict_keys = table->RowsToTableKeys(evict_rows, __evict_ids, alloc, gpu_ctx, stream);
     TensorPtr evict_slots = Empty1DReuse(__evict_slots, kI32, {num_evicted}, gpu_ctx);
@@ -1160,7 +1169,7 @@ void RefreshSession::refresh_on_device(ExtractSession *session, size_t num_cache
     UGK_CALL(ugk_bitmap_update(table->SlotUsedBits(), capacity, evict_slots->CPtr<uint32_t>(), num_evicted, 0,
                                _status_handle->ptr<uint32_t>(), stream));
     table->Evict(evict_keys, stream);
-    table->CheckStatus(stream, "refresh evict");
+    if (!foreground) table->CheckStatus(stream, "refresh evict");
   }
   LOG(INFO) << "refresh on the device: preserved " << num_preserved_key << ", evict " << num_evicted << ", insert "
             << num_insert << ", free slots " << table->_num_free + num_evicted;
@@ -1173,24 +1182,32 @@ void RefreshSession::refresh_on_device(ExtractSession *session, size_t num_cache
   t_phase.Reset();
 
   // Step 6: the first free slots, ascending, take the new rows, ascending; then the keys are published
+  const size_t num_free_expected = table->_num_free + num_evicted;
+  volatile uint32_t *n_free_word = nullptr;
   if (num_insert > 0) {
-    size_t num_free = 0;
-    TensorPtr slots = table->CompactBits(table->SlotUsedBits(), nullptr, true, capacity, num_insert, __free_slots,
-                                         alloc, gpu_ctx, stream, &num_free);
-    CHECK_EQ(num_free, table->_num_free + num_evicted);
-    CHECK_LE(num_insert, num_free) << "free cache slots exhausted";
-    UGK_CALL(ugk_stream_sync(stream));  // the lists are read on the copy stream next
-    CopyRowsIntoSlots(insert_rows->CPtr<uint32_t>(), slots->CPtr<uint32_t>(), num_insert, foreground);
+    CHECK_LE(num_insert, num_free_expected) << "free cache slots exhausted";
+    // how many slots are free is known without looking (what was free plus what was evicted); the count the compaction
+    // makes on its way is compared with that once the refresh has been waited for
+    n_free_word = table->CountBits(table->SlotUsedBits(), nullptr, true, capacity, 0, stream);
+    TensorPtr slots =
+        table->EmitBits(table->SlotUsedBits(), nullptr, true, capacity, 0, num_insert, __free_slots, alloc, gpu_ctx, stream);
+    if (foreground) {
+      // nothing runs beside a foreground refresh: the copy goes on the refresh's own stream, behind the lists it reads
+      CopyRowsIntoSlots(insert_rows->CPtr<uint32_t>(), slots->CPtr<uint32_t>(), num_insert, true, stream);
+    } else {
+      UGK_CALL(ugk_stream_sync(stream));  // the lists are read on the copy stream next
+      CopyRowsIntoSlots(insert_rows->CPtr<uint32_t>(), slots->CPtr<uint32_t>(), num_insert, false, low_pri_stream);
+    }
     UGK_CALL(ugk_bitmap_update(table->SlotUsedBits(), capacity, slots->CPtr<uint32_t>(), num_insert, 1,
                                _status_handle->ptr<uint32_t>(), stream));
     TensorPtr insert_keys = table->RowsToTableKeys(insert_rows, __insert_ids, alloc, gpu_ctx, stream);
     table->InsertWithLoc(insert_keys, slots, local, stream);
-    table->CheckStatus(stream, "refresh insert");
   }
   uint32_t st = 0;
   UGK_CALL(ugk_memcpy_async(&st, _status_handle->ptr<uint32_t>(), sizeof(st), stream));
-  UGK_CALL(ugk_stream_sync(stream));
-  CHECK_EQ(st, 0u) << "refresh on the device: a listed row or slot is outside its bitmap";
+  table->CheckStatus(stream, "refresh on the device");  // waits for the stream
+  CHECK_EQ(st, 0u) << "refresh on the device: a listed row or slot is outside its table or bitmap";
+  if (n_free_word) CHECK_EQ((size_t)*n_free_word, num_free_expected);
   AnonymousBarrier::_refresh_instance->Wait();
   const double insert_s = t_phase.Passed();
   t_phase.Reset();

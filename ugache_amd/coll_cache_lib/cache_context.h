@@ -261,7 +261,8 @@ class RefreshSession {
   void WaitForOneLookup(ExtractSession *session, bool foreground);
   // copies the listed host rows into the listed cache slots (step 6): in one launch when in the foreground, in
   // small throttled batches behind running lookups otherwise
-  void CopyRowsIntoSlots(const uint32_t *rows_dev, const uint32_t *slots_dev, size_t num_rows, bool foreground);
+  void CopyRowsIntoSlots(const uint32_t *rows_dev, const uint32_t *slots_dev, size_t num_rows, bool foreground,
+                         StreamHandle copy_stream);
   TensorPtr __keys_buffer;
   TensorPtr __offs_buffer;
   TensorPtr __evict_rows, __insert_rows, __free_slots, __evict_ids, __insert_ids, __evict_slots;

@@ -176,6 +176,24 @@ TensorPtr CacheEntryManager::CompactBits(const uint64_t *a, const uint64_t *b, b
   return list;
 }
 
+volatile uint32_t *CacheEntryManager::CountBits(const uint64_t *a, const uint64_t *b, bool invert_a, uint64_t nbits,
+                                                int which, StreamHandle stream) {
+  CHECK(which == 0 || which == 1);
+  uint32_t *total = DevWords() + 8 + which;
+  void *ws = which == 0 ? _dev_bm_ws->ptr() : _dev_bm_ws2->ptr();
+  UGK_CALL(ugk_bitmap_count(a, b, invert_a ? 1 : 0, nbits, ws, total, stream));
+  return total;
+}
+
+TensorPtr CacheEntryManager::EmitBits(const uint64_t *a, const uint64_t *b, bool invert_a, uint64_t nbits, int which,
+                                      size_t n, TensorPtr &buffer, const std::function<MemHandle(size_t)> &allocator,
+                                      Context ctx, StreamHandle stream) {
+  TensorPtr list = ReuseList(buffer, kI32, n, allocator, ctx);
+  const void *ws = which == 0 ? _dev_bm_ws->ptr() : _dev_bm_ws2->ptr();
+  if (n) UGK_CALL(ugk_bitmap_emit(a, b, invert_a ? 1 : 0, nbits, ws, list->Ptr<uint32_t>(), n, stream));
+  return list;
+}
+
 TensorPtr CacheEntryManager::RowsToTableKeys(TensorPtr rows_dev, TensorPtr &buffer,
                                              const std::function<MemHandle(size_t)> &allocator, Context ctx,
                                              StreamHandle stream) {
@@ -197,6 +215,7 @@ void CacheEntryManager::EnsureDeviceLists(const std::function<MemHandle(size_t)>
     _dev_slot_used = EagerGPUAlloc(_device_id, std::max<size_t>(slot_words, 1) * 8);
     _dev_rank_ws = EagerGPUAlloc(_device_id, ugk_rank_workspace_bytes());
     _dev_bm_ws = EagerGPUAlloc(_device_id, ugk_bitmap_workspace_bytes());
+    _dev_bm_ws2 = EagerGPUAlloc(_device_id, ugk_bitmap_workspace_bytes());
     _dev_words = PinnedHostAlloc(256);
     memset(_dev_words->ptr(), 0, 256);
   }

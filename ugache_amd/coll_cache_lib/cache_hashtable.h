@@ -94,6 +94,7 @@ class CacheEntryManager {
   MemHandle _dev_scratch_bits;           // as large, scratch of the placement
   MemHandle _dev_slot_used;              // ceil(capacity / 64) words
   MemHandle _dev_rank_ws, _dev_bm_ws;    // workspaces of ugk_rank_* / ugk_bitmap_*
+  MemHandle _dev_bm_ws2;                 // a second one, so that two compactions can be counted before one wait
   MemHandle _dev_words;                  // pinned host words the kernels report counts in
   TensorPtr _dev_list_buffer;            // scratch list for bringing either side up to date
   bool _dev_lists_valid = false;
@@ -114,6 +115,15 @@ class CacheEntryManager {
   TensorPtr CompactBits(const uint64_t *a, const uint64_t *b, bool invert_a, uint64_t nbits, size_t limit,
                         TensorPtr &buffer, const std::function<MemHandle(size_t)> &allocator, Context ctx,
                         StreamHandle stream, size_t *total_out);
+  // The two halves of CompactBits for callers that count several sets before they wait once: CountBits enqueues the
+  // count of set `which` (0 or 1, each with a workspace of its own) and returns the pinned word it will land in;
+  // EmitBits, after the bitmaps' count is known (waited for, or known by other means), enqueues the list of the first n
+  // elements.
+  volatile uint32_t *CountBits(const uint64_t *a, const uint64_t *b, bool invert_a, uint64_t nbits, int which,
+                               StreamHandle stream);
+  TensorPtr EmitBits(const uint64_t *a, const uint64_t *b, bool invert_a, uint64_t nbits, int which, size_t n,
+                     TensorPtr &buffer, const std::function<MemHandle(size_t)> &allocator, Context ctx,
+                     StreamHandle stream);
   // device list of host rows -> device list of table keys (the rows themselves, or their ids in sparse-id mode)
   TensorPtr RowsToTableKeys(TensorPtr rows_dev, TensorPtr &buffer, const std::function<MemHandle(size_t)> &allocator,
                             Context ctx, StreamHandle stream);

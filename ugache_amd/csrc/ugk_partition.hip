@@ -153,9 +153,97 @@ __global__ __launch_bounds__(kBlock) void select_keys_kernel(const K *__restrict
     out[j] = keys[sel[j]];
 }
 
-// ---- fused lookup + gather: every wavefront resolves 64 keys, then copies their 64 rows ------------------
+// ---- fused lookup + gather: every wavefront resolves its keys, then copies their rows -----------------------
+// Measured and dropped: persistent wavefronts over a flat table that work two batches ahead (while the rows of batch i
+// are copied, the table words of batch i + 1 and the keys of batch i + 2 are on their way), on 2 - 16 workgroups per
+// compute unit: bit-exact, and 1 - 8 % slower at every size (262,144 keys of 512 bytes, 1 % misses: 49.8 - 52.4 us
+// against 48.5 us).  With eight short wavefronts per SIMD the chip already overlaps one wavefront's table round trip
+// with the others' row copies, and wavefronts that stride over the batch give up the moving window of output rows
+// that workgroups started in order write.
 typedef const __attribute__((address_space(1))) u32x4 *grow_t;  // a row in global memory (HBM, or mapped host memory)
 typedef __attribute__((address_space(1))) u32x4 *gout_t;
+
+// where a key's row lives, as an integer address (the head of the output for a key without a row, see below)
+struct MixRow {
+  uint64_t bits;
+  bool has_row, from_cache;
+};
+
+__device__ __forceinline__ MixRow mix_resolve(const ugk_table_t &t, uint64_t key, bool active, const Found &f,
+                                              const u32x4 *cache, uint64_t cache_rows, const u32x4 *host,
+                                              uint64_t host_rows, const u32x4 *out, uint32_t vpr, uint32_t *status,
+                                              uint32_t *host_mirror) {
+  const u32x4 *rowp = nullptr;
+  if (active) {
+    if (f.hit && f.loc == UGK_LOC_LOCAL && f.off < cache_rows) rowp = cache + (uint64_t)f.off * vpr;
+    else if (f.hit && f.loc == UGK_LOC_HOST && f.off < host_rows) rowp = host + (uint64_t)f.off * vpr;
+    else if (!f.hit && fallback_row(t, key) < host_rows) rowp = host + fallback_row(t, key) * vpr;
+    else {
+      atomicOr(status, UGK_ST_KEY_OUT_OF_RANGE);
+      if (host_mirror) host_mirror[0] = UGK_ST_KEY_OUT_OF_RANGE;
+    }
+  }
+  // A key without a row copies nothing; its lanes read the head of the output instead (mapped whatever the key), so
+  // that the loads of the copy carry no branch: behind a branch each of them waits for the one before.
+  MixRow r;
+  r.has_row = rowp != nullptr;
+  r.bits = r.has_row ? reinterpret_cast<uint64_t>(rowp) : reinterpret_cast<uint64_t>(out);
+  r.from_cache = r.has_row && f.hit && f.loc == UGK_LOC_LOCAL;
+  return r;
+}
+
+// the rows of one wavefront's KPW keys, lane l holding the address of key b0 + l's row
+template <int LPR, int KPW, bool NT_STORE>
+__device__ __forceinline__ void mix_copy(const MixRow &row, u32x4 *out, size_t b0, uint32_t vpr) {
+  constexpr int RPW = kWave / LPR;  // rows per wavefront instruction
+  constexpr int UNROLL = (RPW * 4 <= KPW) ? 4 : (KPW / RPW);
+  static_assert(KPW <= kWave && KPW % (RPW * UNROLL) == 0, "keys per wavefront must be whole rounds of rows");
+  const int lane = (int)lane_id();
+  const int sub = lane % LPR, rg = lane / LPR;
+  for (int r0 = 0; r0 < KPW; r0 += RPW * UNROLL) {
+    // the row addresses travel between lanes as integers; turned back into pointers they must be told to be global
+    // memory again, or the loads become generic ones, which the hardware cannot keep several of in flight in order
+    grow_t p[UNROLL];
+    bool ok[UNROLL];
+#pragma unroll
+    for (int u = 0; u < UNROLL; ++u) {
+      p[u] = reinterpret_cast<grow_t>(shfl64(row.bits, r0 + u * RPW + rg));
+      ok[u] = __shfl((int)row.has_row, r0 + u * RPW + rg) != 0;
+    }
+    for (uint32_t c0 = 0; c0 < vpr; c0 += LPR) {
+      const uint32_t col = c0 + sub;
+      if (col < vpr) {
+        u32x4 v[UNROLL];
+#pragma unroll
+        for (int u = 0; u < UNROLL; ++u) v[u] = __builtin_nontemporal_load(p[u] + col);
+#pragma unroll
+        for (int u = 0; u < UNROLL; ++u)
+          if (ok[u]) {
+            gout_t dst = (gout_t)out + (b0 + r0 + u * RPW + rg) * vpr + col;
+            // a template parameter: the two stores of a run-time choice get merged and lose the hint
+            if constexpr (NT_STORE) __builtin_nontemporal_store(v[u], dst);
+            else *dst = v[u];
+          }
+      }
+    }
+  }
+}
+
+// Group sizes for the host: every workgroup leaves its two sums in a word of its own in pinned host memory, a posted
+// write nobody waits for; the host adds the words up after it has waited for the stream.  Handing them over through
+// device-side atomics cost more than it looks: a 64-bit add and a dependent ticket per workgroup 16 us of a 69 us
+// launch at 99 % hits (same-address atomics are performed one after the other at the memory side), one add whose
+// result tells the last workgroup still 5 us (every workgroup ends by waiting for the round trip), and a device-scope
+// fence per workgroup 13-49 % of a whole step (each writes back and invalidates the L2 of its XCD).
+__device__ __forceinline__ void mix_leave_counts(uint32_t *block_tot, uint32_t wave_local, uint32_t wave_host,
+                                                 unsigned long long *counts) {
+  if (lane_id() == 0) {
+    if (wave_local) atomicAdd(&block_tot[0], wave_local);
+    if (wave_host) atomicAdd(&block_tot[1], wave_host);
+  }
+  __syncthreads();
+  if (threadIdx.x == 0) counts[blockIdx.x] = ((unsigned long long)block_tot[1] << 32) | block_tot[0];
+}
 
 template <typename K, int KIND, int LPR, int KPW, bool NT_STORE>
 __global__ __launch_bounds__(kBlock) void extract_mix_kernel(ugk_table_t t, const K *__restrict__ keys, size_t n,
@@ -164,15 +252,11 @@ __global__ __launch_bounds__(kBlock) void extract_mix_kernel(ugk_table_t t, cons
                                                              u32x4 *__restrict__ out, uint32_t vpr,
                                                              uint32_t *status, uint32_t *host_mirror,
                                                              unsigned long long *counts) {
-  constexpr int RPW = kWave / LPR;  // rows per wavefront instruction
   __shared__ uint32_t block_tot[2];
   if (threadIdx.x < 2) block_tot[threadIdx.x] = 0;
   __syncthreads();
   uint32_t wave_local = 0, wave_host = 0;  // rows this wavefront took from each source (wavefront-uniform)
-  constexpr int UNROLL = (RPW * 4 <= KPW) ? 4 : (KPW / RPW);
-  static_assert(KPW <= kWave && KPW % (RPW * UNROLL) == 0, "keys per wavefront must be whole rounds of rows");
   const int lane = (int)lane_id();
-  const int sub = lane % LPR, rg = lane / LPR;
   const size_t wave_global = (size_t)blockIdx.x * kWavesPerBlock + threadIdx.x / kWave;
   const size_t n_waves = (size_t)gridDim.x * kWavesPerBlock;
   for (size_t b0 = wave_global * KPW; b0 < n; b0 += n_waves * KPW) {
@@ -181,68 +265,16 @@ __global__ __launch_bounds__(kBlock) void extract_mix_kernel(ugk_table_t t, cons
     const uint64_t key = active ? key_to_u64<K>(keys[i]) : 0;
     // a full wavefront of keys probes its eight home lines in one go (see hash_probe_home)
     const Found f = table_lookup<KIND, KPW == kWave ? 1 : 2>(t, key, active);
-    const u32x4 *rowp = nullptr;
-    if (active) {
-      if (f.hit && f.loc == UGK_LOC_LOCAL && f.off < cache_rows) rowp = cache + (uint64_t)f.off * vpr;
-      else if (f.hit && f.loc == UGK_LOC_HOST && f.off < host_rows) rowp = host + (uint64_t)f.off * vpr;
-      else if (!f.hit && fallback_row(t, key) < host_rows) rowp = host + fallback_row(t, key) * vpr;
-      else {
-        atomicOr(status, UGK_ST_KEY_OUT_OF_RANGE);
-        if (host_mirror) host_mirror[0] = UGK_ST_KEY_OUT_OF_RANGE;
-      }
-    }
-    // A key without a row copies nothing; its lanes read the head of the output instead (mapped whatever the key), so
-    // that the loads below carry no branch: behind a branch each of them waits for the one before.
-    const bool has_row = rowp != nullptr;
-    const uint64_t rowbits = has_row ? reinterpret_cast<uint64_t>(rowp) : reinterpret_cast<uint64_t>(out);
+    const MixRow row = mix_resolve(t, key, active, f, cache, cache_rows, host, host_rows, out, vpr, status, host_mirror);
     if (counts) {
       // rows from the cache, and all others (host rows, and rows skipped for a key without a row: the launch is
       // flagged then and its group sizes mean nothing, but the two sums still add up to n)
-      const bool from_cache = has_row && f.hit && f.loc == UGK_LOC_LOCAL;
-      wave_local += __popcll(__ballot(from_cache));
-      wave_host += __popcll(__ballot(active && !from_cache));
+      wave_local += __popcll(__ballot(row.from_cache));
+      wave_host += __popcll(__ballot(active && !row.from_cache));
     }
-    for (int r0 = 0; r0 < KPW; r0 += RPW * UNROLL) {
-      // the row addresses travel between lanes as integers; turned back into pointers they must be told to be global
-      // memory again, or the loads become generic ones, which the hardware cannot keep several of in flight in order
-      grow_t p[UNROLL];
-      bool ok[UNROLL];
-#pragma unroll
-      for (int u = 0; u < UNROLL; ++u) {
-        p[u] = reinterpret_cast<grow_t>(shfl64(rowbits, r0 + u * RPW + rg));
-        ok[u] = __shfl((int)has_row, r0 + u * RPW + rg) != 0;
-      }
-      for (uint32_t c0 = 0; c0 < vpr; c0 += LPR) {
-        const uint32_t col = c0 + sub;
-        if (col < vpr) {
-          u32x4 v[UNROLL];
-#pragma unroll
-          for (int u = 0; u < UNROLL; ++u) v[u] = __builtin_nontemporal_load(p[u] + col);
-#pragma unroll
-          for (int u = 0; u < UNROLL; ++u)
-            if (ok[u]) {
-              gout_t dst = (gout_t)out + (b0 + r0 + u * RPW + rg) * vpr + col;
-              // a template parameter: the two stores of a run-time choice get merged and lose the hint
-              if constexpr (NT_STORE) __builtin_nontemporal_store(v[u], dst);
-              else *dst = v[u];
-            }
-        }
-      }
-    }
+    mix_copy<LPR, KPW, NT_STORE>(row, out, b0, vpr);
   }
-  if (counts == nullptr) return;
-  // Group sizes for the host: every workgroup leaves its two sums in a word of its own in pinned host memory, a posted
-  // write nobody waits for; the host adds the words up after it has waited for the stream.  Handing them over through
-  // device-side atomics cost more than it looks: a 64-bit add and a dependent ticket per workgroup 16 us of a 69 us
-  // launch at 99 % hits (same-address atomics are performed one after the other at the memory side), one add whose
-  // result tells the last workgroup still 5 us (every workgroup ends by waiting for the round trip), and a device-scope
-  // fence per workgroup 13-49 % of a whole step (each writes back and invalidates the L2 of its XCD).
-  if (lane == 0) {
-    if (wave_local) atomicAdd(&block_tot[0], wave_local);
-    if (wave_host) atomicAdd(&block_tot[1], wave_host);
-  }
-  __syncthreads();
-  if (threadIdx.x == 0) counts[blockIdx.x] = ((unsigned long long)block_tot[1] << 32) | block_tot[0];
+  if (counts) mix_leave_counts(block_tot, wave_local, wave_host, counts);
 }
 
 // ---- dedup -----------------------------------------------------------------------------------------------

@@ -31,10 +31,16 @@ constexpr int kCountPasses = 3;        // digits of a 32-bit count, most signifi
 constexpr int kPassShift[kCountPasses] = {21, 10, 0};
 constexpr int kPassBits[kCountPasses] = {11, 11, 10};
 
+// A bitmap is cut twice: into kBmChunks chunks of whole 64-word blocks (what the one-workgroup scan works on), and
+// into those blocks, each one wavefront load wide.  The emit pass runs one wavefront per block, so set bits that all
+// sit in a few chunks (the rows a refresh evicts are often one contiguous run) are still spread over the chip.
+constexpr uint64_t kBmMaxBits = 1ull << 32;
+constexpr uint32_t kBmMaxBlocks = (uint32_t)(kBmMaxBits / 64 / kWave);  // 2^20
 struct BmWs {
   uint32_t total;
   uint32_t pad[3];
-  uint32_t base[kBmChunks];  // per chunk: first the count, after the scan the exclusive prefix
+  uint32_t base[kBmChunks];      // per chunk: first the count, after the scan the exclusive prefix
+  uint32_t block[kBmMaxBlocks];  // per 64-word block: its count
 };
 
 // workspace of a placement
@@ -334,10 +340,12 @@ __global__ __launch_bounds__(kBlock) void bitmap_count_kernel(const unsigned lon
     uint32_t found = 0;
     for (uint64_t w0 = begin; w0 < end; w0 += kWave) {
       const uint64_t w = w0 + lane;
-      if (w < end) found += __popcll(bm_word(a, b, invert_a != 0, nbits, w));
-    }
+      uint32_t mine = w < end ? __popcll(bm_word(a, b, invert_a != 0, nbits, w)) : 0u;
 #pragma unroll
-    for (int d = kWave / 2; d > 0; d >>= 1) found += __shfl_xor(found, d);
+      for (int d = kWave / 2; d > 0; d >>= 1) mine += __shfl_xor(mine, d);
+      if (lane == 0) ws->block[w0 / kWave] = mine;  // chunks begin on block boundaries
+      found += mine;
+    }
     if (lane == 0) ws->base[chunk] = found;
   }
 }
@@ -373,29 +381,35 @@ __global__ __launch_bounds__(kBlock) void bitmap_emit_kernel(const unsigned long
                                                              const BmWs *ws, uint32_t *out, uint64_t max_out) {
   const int lane = (int)lane_id();
   const uint64_t n_words = (nbits + 63) / 64;
+  const uint64_t n_blocks = (n_words + kWave - 1) / kWave;
   const uint64_t wave = ((uint64_t)blockIdx.x * kBlock + threadIdx.x) / kWave;
   const uint64_t n_waves = (uint64_t)gridDim.x * (kBlock / kWave);
-  for (uint64_t chunk = wave; chunk < (uint64_t)kBmChunks; chunk += n_waves) {
-    const uint64_t begin = chunk * per_chunk, end = min(n_words, begin + per_chunk);
-    uint64_t pos0 = ws->base[chunk];
-    for (uint64_t w0 = begin; w0 < end && pos0 < max_out; w0 += kWave) {
-      const uint64_t w = w0 + lane;
-      unsigned long long m = w < end ? bm_word(a, b, invert_a != 0, nbits, w) : 0ull;
-      const uint32_t mine = __popcll(m);
-      uint32_t incl = mine;
+  const uint64_t blocks_per_chunk = per_chunk / kWave;
+  for (uint64_t blk = wave; blk < n_blocks; blk += n_waves) {
+    if (ws->block[blk] == 0) continue;  // wavefront-uniform
+    // where the block's elements go: its chunk's offset plus the counts of the chunk's earlier blocks
+    const uint64_t chunk = blk / blocks_per_chunk, first = chunk * blocks_per_chunk;
+    uint32_t before = 0;
+    for (uint64_t q = first + lane; q < blk; q += kWave) before += ws->block[q];
 #pragma unroll
-      for (int s = 1; s < kWave; s <<= 1) {
-        const uint32_t up = __shfl_up(incl, s);
-        if (lane >= s) incl += up;
-      }
-      uint64_t pos = pos0 + incl - mine;
-      while (m) {
-        const int bit = __builtin_ctzll(m);
-        m &= m - 1;
-        if (pos < max_out) out[pos] = (uint32_t)(w * 64 + bit);
-        ++pos;
-      }
-      pos0 += __shfl(incl, kWave - 1);
+    for (int d = kWave / 2; d > 0; d >>= 1) before += __shfl_xor(before, d);
+    const uint64_t pos0 = (uint64_t)ws->base[chunk] + before;
+    if (pos0 >= max_out) continue;
+    const uint64_t w = blk * kWave + lane;
+    unsigned long long m = w < n_words ? bm_word(a, b, invert_a != 0, nbits, w) : 0ull;
+    const uint32_t mine = __popcll(m);
+    uint32_t incl = mine;
+#pragma unroll
+    for (int s = 1; s < kWave; s <<= 1) {
+      const uint32_t up = __shfl_up(incl, s);
+      if (lane >= s) incl += up;
+    }
+    uint64_t pos = pos0 + incl - mine;
+    while (m) {
+      const int bit = __builtin_ctzll(m);
+      m &= m - 1;
+      if (pos < max_out) out[pos] = (uint32_t)(w * 64 + bit);
+      ++pos;
     }
   }
 }
@@ -521,7 +535,8 @@ int ugk_bitmap_emit(const uint64_t *a_dev, const uint64_t *b_dev, int invert_a, 
   UGK_REQUIRE(out_dev, "ugk_bitmap_emit: null output list");
   const uint64_t n_words = (nbits + 63) / 64;
   const uint64_t per_chunk = bm_words_per_chunk(n_words);
-  const unsigned grid = clamp_grid((kBmChunks + (kBlock / kWave) - 1) / (kBlock / kWave), (unsigned)cu_count() * 8u);
+  const uint64_t n_blocks = (n_words + kWave - 1) / kWave;
+  const unsigned grid = clamp_grid((n_blocks + (kBlock / kWave) - 1) / (kBlock / kWave), 0);
   hipLaunchKernelGGL(bitmap_emit_kernel, dim3(grid), dim3(kBlock), 0, as_stream(stream),
                      reinterpret_cast<const unsigned long long *>(a_dev),
                      reinterpret_cast<const unsigned long long *>(b_dev), invert_a, nbits, per_chunk,

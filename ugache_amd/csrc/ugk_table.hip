@@ -57,55 +57,87 @@ __device__ __forceinline__ void store_off_meta(ugk_bucket_t *b, uint32_t off, ui
   __atomic_store_n(reinterpret_cast<uint64_t *>(&b->off), ((uint64_t)meta << 32) | off, __ATOMIC_RELAXED);
 }
 
+// Insert, eight keys per wavefront: an 8-lane group walks one key's probe sequence a 128-byte line (eight buckets) at a
+// time, as the lookup does.  The key goes into the first reusable bucket of its probe sequence (a tombstone, else the
+// first never-used bucket), but only once the whole sequence up to that never-used bucket has been seen not to hold the
+// key already: a tombstone in front of a live copy of the key must not hide it.  With tombstones piling up between
+// rebuilds that walk is tens of buckets long, which one lane per key did as a chain of dependent 16-byte loads (462 k
+// keys into a 71 M-bucket table with 13 % tombstones: 207 us).  Keys of one launch are distinct, so the only contest is
+// for buckets; a group that loses one starts its walk again.
 template <typename K>
 __global__ __launch_bounds__(kBlock) void hash_insert_kernel(ugk_bucket_t *table, uint64_t nb, const K *keys,
                                                              const uint32_t *offs, uint32_t seq_base, uint32_t loc,
                                                              size_t n, uint32_t *status) {
-  for (size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x; i < n; i += (size_t)gridDim.x * kBlock) {
-    const uint64_t key = key_to_u64<K>(keys[i]);
-    const uint32_t off = offs ? offs[i] : seq_base + (uint32_t)i;
-    if (key_is_reserved(key)) {
-      atomicOr(status, UGK_ST_KEY_OUT_OF_RANGE);
-      continue;
+  constexpr uint64_t kNone = ~0ull;
+  const int lane = (int)lane_id();
+  const int grp = lane >> 3, sub = lane & 7;
+  const size_t wave = ((size_t)blockIdx.x * kBlock + threadIdx.x) / kWave;
+  const size_t n_waves = (size_t)gridDim.x * (kBlock / kWave);
+  const uint64_t lines = nb >> 3;
+  for (size_t i0 = wave * 8; i0 < n; i0 += n_waves * 8) {  // wavefront-uniform: every ballot below sees all 64 lanes
+    const size_t i = i0 + grp;
+    const bool active = i < n;
+    const uint64_t key = active ? key_to_u64<K>(keys[i]) : 0;
+    const uint32_t off = active ? (offs ? offs[i] : seq_base + (uint32_t)i) : 0;
+    bool done = !active;
+    if (active && key_is_reserved(key)) {
+      if (sub == 0) atomicOr(status, UGK_ST_KEY_OUT_OF_RANGE);
+      done = true;
     }
-    // The key goes into the first reusable bucket of its probe sequence, but only once the whole sequence up to its
-    // first never-used bucket has been seen not to hold the key already: a tombstone in front of a live copy of the
-    // key must not hide it.  Keys of one launch are distinct, so the only contest is for buckets, and a lost bucket
-    // sends the search back to where it was lost.
-    constexpr uint64_t kNone = ~0ull;
-    uint64_t pos = hash_home(key, nb);
-    uint64_t first_tomb = kNone;
-    bool placed = false;
-    for (uint64_t step = 0; step < 2 * nb + 2 && !placed; ++step) {
-      const uint64_t cur = load_key_relaxed(table + pos);
-      if (cur == key) {
-        atomicOr(status, UGK_ST_DUP_KEY);
-        placed = true;
-        break;
+    const uint64_t home = done ? 0 : hash_home(key, nb);
+    uint64_t win = home, first_tomb = kNone, steps = 0;
+    while (__ballot(!done)) {
+      uint64_t cur = 0;  // reads as some other key
+      if (!done) cur = load_key_relaxed(table + win + sub);
+      const uint32_t mb = (uint32_t)((__ballot(!done && cur == key) >> (grp * 8)) & 0xffull);
+      const uint32_t eb = (uint32_t)((__ballot(!done && cur == UGK_HASH_EMPTY) >> (grp * 8)) & 0xffull);
+      const uint32_t tb = (uint32_t)((__ballot(!done && cur == UGK_HASH_TOMB) >> (grp * 8)) & 0xffull);
+      // what the group does with this line: 0 walk on, 1 the key is there already, 2 claim `target`
+      int action = 0;
+      uint64_t target = 0, expect = 0;
+      if (!done) {
+        const int fe = eb ? (__ffs(eb) - 1) : 8;
+        const uint32_t in_front = fe < 8 ? ((1u << fe) - 1u) : 0xffu;  // buckets in front of the first never-used one
+        if (mb & in_front) {
+          action = 1;
+        } else {
+          if (first_tomb == kNone && (tb & in_front)) first_tomb = win + (uint64_t)(__ffs(tb & in_front) - 1);
+          const bool lap_done = steps >= lines && first_tomb != kNone;  // no never-used bucket at all: take the tombstone
+          if (fe < 8 || lap_done) {
+            action = 2;
+            target = first_tomb != kNone ? first_tomb : win + (uint64_t)fe;
+            expect = first_tomb != kNone ? UGK_HASH_TOMB : UGK_HASH_EMPTY;
+          }
+        }
       }
-      const bool lap_done = step >= nb && first_tomb != kNone;  // no never-used bucket at all: take the tombstone
-      if (cur == UGK_HASH_EMPTY || lap_done) {
-        const uint64_t target = first_tomb != kNone ? first_tomb : pos;
-        const uint64_t expect = first_tomb != kNone ? UGK_HASH_TOMB : UGK_HASH_EMPTY;
-        const uint64_t seen = atomicCAS(reinterpret_cast<unsigned long long *>(&table[target].key),
-                                        (unsigned long long)expect, (unsigned long long)key);
+      uint64_t seen = 0;
+      if (action == 2 && sub == 0)
+        seen = atomicCAS(reinterpret_cast<unsigned long long *>(&table[target].key), (unsigned long long)expect,
+                         (unsigned long long)key);
+      seen = shfl64(seen, grp * 8);
+      if (action == 1) {
+        if (sub == 0) atomicOr(status, UGK_ST_DUP_KEY);
+        done = true;
+      } else if (action == 2) {
         if (seen == expect) {
           // the bucket is ours: slot and valid bit appear together, in one 8-byte store.  Until then the bucket reads
           // as "key present, not valid", i.e. as a miss.
-          store_off_meta(table + target, off, UGK_META_VALID | (loc & 0xfu));
-          placed = true;
-          break;
+          if (sub == 0) store_off_meta(table + target, off, UGK_META_VALID | (loc & 0xfu));
+          done = true;
+        } else {  // another key of this launch took it: walk again from the start (rare)
+          win = home;
+          first_tomb = kNone;
+          steps = 0;
         }
-        // somebody else took it: go on from there (what lies between there and here has been examined, but walking it
-        // again is simpler than remembering it, and rare)
-        pos = target;
-        first_tomb = kNone;
-        continue;
+      } else if (!done) {
+        win += 8;
+        if (win >= nb) win = 0;
+        if (++steps > 2 * lines + 2) {
+          if (sub == 0) atomicOr(status, UGK_ST_TABLE_FULL);
+          done = true;
+        }
       }
-      if (cur == UGK_HASH_TOMB && first_tomb == kNone) first_tomb = pos;
-      if (++pos == nb) pos = 0;
     }
-    if (!placed) atomicOr(status, UGK_ST_TABLE_FULL);
   }
 }
 
@@ -194,7 +226,7 @@ int table_insert(ugk_table_t t, const K *keys, const uint32_t *offs, uint32_t se
     hipLaunchKernelGGL(flat_insert_kernel<K>, dim3(grid), dim3(kBlock), 0, as_stream(stream), (uint32_t *)t.table,
                        t.size, keys, offs, seq_base, loc, n, status);
   else
-    hipLaunchKernelGGL(hash_insert_kernel<K>, dim3(grid), dim3(kBlock), 0, as_stream(stream),
+    hipLaunchKernelGGL(hash_insert_kernel<K>, dim3(clamp_grid((n + 31) / 32, 0)), dim3(kBlock), 0, as_stream(stream),
                        (ugk_bucket_t *)t.table, t.size, keys, offs, seq_base, loc, n, status);
   UGK_HIP(hipGetLastError());
   return 0;
