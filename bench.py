@@ -619,6 +619,11 @@ def run_mixed(args):
                      "ms_per_step": (t_lookup + t_refresh) / n_steps * 1e3,
                      "keys_per_s": n_keys * n_steps / (t_lookup + t_refresh),
                      "drift_rows_looked_up_per_step": n_new, "first_refresh_s": settle_s,
+                     "row_copy_floor_ms": n_new * row_bytes / (ceiling["best_GBps"] * 1e9) * 1e3,
+                     "row_copy_floor_note": "at most drift_rows rows cross the host link per refresh (fewer when some "
+                                            "of them were cached as filler); the floor is that many rows of this size "
+                                            "at host_link.random_row_ceiling, the rate uniformly random rows of this "
+                                            "size reach out of this table",
                      "table_rebuilds": after["table_rebuilds"], "cached_rows_after": after["cached_rows"],
                      "free_slots_after": after["free_slots"],
                      "note": "refresh = rank + place + evict/insert lists on the device (COLL_GPU_REFRESH=1, hotness "
@@ -824,15 +829,16 @@ def random_row_ceiling(hip, torch, emb, rows, row_bytes, dev, stream, note):
 # what a leg contributes to the default line: enough to recompute both halves of the metric
 LEG_KEYS = ("value", "unit", "ms_per_step", "ms_per_step_spread", "steps", "warmup", "config", "hit_rate",
             "effective_extraction_GBps", "parity", "stages_us", "roofline", "host_link", "cpu_baseline", "gpu_over_cpu",
-            "refresh", "setup_seconds", "stream_ordered")
+            "refresh", "refresh_each_step", "setup_seconds", "stream_ordered")
 DEFAULT_LEGS = ("c3_gnn_100Mx128xfp32_1M_i64_zipf0.9_cache25pct", "c5_hash_500Mx64xfp16_1M_i64_zipf1.05_cache50M")
 
 
-def run_child(workload, args, cpu_seconds):
+def run_child(workload, args, cpu_seconds, extra=()):
     """one workload in a child process (this process has not touched the GPU); returns its JSON line as a dict"""
     import subprocess
 
     cmd = [sys.executable, os.path.abspath(__file__), "--workload", workload, "--cpu-seconds", str(cpu_seconds)]
+    cmd += list(extra)
     if args.steps is not None:
         cmd += ["--steps", str(args.steps)]
     if args.warmup is not None:
@@ -860,6 +866,13 @@ def run_default(args):
                 # a leg that cannot report (a parity failure ends it without a number) takes the whole line with it
                 sys.exit("bench.py: leg %s failed: %s" % (name, err))
             legs[name] = {k: leg[k] for k in LEG_KEYS if k in leg}
+        # config 5's "a refresh with every step": the same workload with the hotness counted and the cache re-placed on
+        # the device (COLL_GPU_RECORD=1 COLL_GPU_REFRESH=1), 1 % of the cache replaced per step
+        name = DEFAULT_LEGS[-1]
+        leg, err = run_child(name, args, 0.5, extra=("--device-refresh",))
+        if leg is None:
+            sys.exit("bench.py: leg %s --device-refresh failed: %s" % (name, err))
+        legs[name + "+device_refresh"] = {k: leg[k] for k in LEG_KEYS if k in leg and k != "cpu_baseline"}
     result["legs"] = legs
     result["legs_note"] = ("each leg is the same bench.py with --workload <name>, run after the top-level workload in "
                            "a process of its own, same --steps and --warmup; value / roofline / cpu_baseline at the top "

@@ -525,9 +525,11 @@ int extract_mix_lpr(ugk_table_t t, const K *keys, size_t n, const void *cache, u
   //                         150.7 / 112.3 / 82.1 / 79.5
   // and the same order at 10 % misses, where the host link bounds the launch and the spread is 1-3 %.  The batch sizes
   // above are multiples of the chip's wavefront slots (256 CUs x 32 = 8,192), which is how the rule below states them.
-  // others_hint is not consulted any more: since the row loads of a wavefront are in flight together, the mix of
-  // sources no longer changes which shape wins.
-  (void)others_hint;
+  // others_hint does not enter the shape any more: since the row loads of a wavefront are in flight together, the mix
+  // of sources no longer changes which shape wins.  It caps the grid instead when most rows come over the host link:
+  // rows of 512 bytes and more cross it faster from 128 workgroups than from as many as the batch would fill (56.9
+  // against 52.7 GB/s for uniformly random rows), and the few rows the cache serves do not miss the other workgroups.
+  const bool mostly_host = others_hint != UGK_HINT_UNKNOWN && (size_t)others_hint * 2 >= n && vpr >= 32;
   const size_t slots = (size_t)cu_count() * 4 * 8;
   const int lpr = vpr <= 1 ? 1 : vpr <= 2 ? 2 : vpr <= 4 ? 4 : vpr <= 8 ? 8 : vpr <= 16 ? 16 : vpr <= 32 ? 32 : 64;
   const bool small_rows = lpr <= 8;  // rows of up to 128 bytes
@@ -549,7 +551,7 @@ int extract_mix_lpr(ugk_table_t t, const K *keys, size_t n, const void *cache, u
   }
   if (kpw < kWave / lpr) kpw = kWave / lpr;  // one wavefront instruction copies 64 / lpr rows
   const size_t keys_per_group = (size_t)kpw * kWavesPerBlock;
-  const unsigned grid = clamp_grid((n + keys_per_group - 1) / keys_per_group, 0);
+  const unsigned grid = clamp_grid((n + keys_per_group - 1) / keys_per_group, mostly_host ? 128u : 0u);
   if (num_groups) *num_groups = grid;
 #define UGK_GO3(L, W, NT)                                                                                          \
   hipLaunchKernelGGL((extract_mix_kernel<K, KIND, L, W, NT>), dim3(grid), dim3(kBlock), 0, st, t, keys, n,        \
