@@ -106,6 +106,9 @@ def parse_args():
                     help="mixed workloads: COLL_GPU_RECORD=1 COLL_GPU_REFRESH=1 COLL_GPU_REFRESH_KEEP=1; after the "
                          "timed steps, time steps that each end with a refresh computed on the device from the "
                          "accumulated hotness, with 1 %% of the cache replaced per step")
+    ap.add_argument("--stage-rows", type=int, default=1 << 22,
+                    help="with --device-refresh: entries of the set of recently missed rows kept in HBM "
+                         "(COLL_MISS_STAGE_ROWS; 0 = none, every inserted row crosses the host link again)")
     ap.add_argument("--calibrate", action="store_true",
                     help="also run 5 plain device copies of 1 GiB (ugk_copy_rows) so a counter run has a kernel of "
                          "known traffic next to the gather")
@@ -427,6 +430,9 @@ def run_mixed(args):
         args.gpu_record = True
         os.environ["COLL_GPU_REFRESH"] = "1"
         os.environ["COLL_GPU_REFRESH_KEEP"] = "1"
+        # rows the lookups fetch from the host table are filed in HBM (4 Mi entries), where the refresh finds most of
+        # the rows it inserts; COLL_MISS_STAGE_ROWS=0 in the environment turns that off for a comparison
+        os.environ.setdefault("COLL_MISS_STAGE_ROWS", str(args.stage_rows))
     if args.gpu_record:
         os.environ["COLL_GPU_RECORD"] = "1"
     co.config({"cache_percentage": pct, "_cache_policy": co.kCollCacheAsymmLink, "num_device": 1,
@@ -594,6 +600,7 @@ def run_mixed(args):
         settle_s = time.perf_counter() - t0
         note("first refresh on the device (settling): %.4f s" % settle_s)
         n_steps = min(K, 20)
+        staged_before = _basics.C_LIB_CTYPES.coll_cache_rows_from_stage(0)
         t_lookup = t_refresh = 0.0
         cold_end = per_field
         for i in range(n_steps):
@@ -611,6 +618,7 @@ def run_mixed(args):
             t_lookup += t1 - t0
             t_refresh += t2 - t1
         after = _basics.info(0)
+        staged_rows = _basics.C_LIB_CTYPES.coll_cache_rows_from_stage(0) - staged_before
         step(0)
         torch.cuda.synchronize()
         if out.cpu().numpy().tobytes() != orc.gather(table_np, rows_pool[0].cpu().numpy(), omp=True).tobytes():
@@ -626,6 +634,8 @@ def run_mixed(args):
                                             "size reach out of this table",
                      "table_rebuilds": after["table_rebuilds"], "cached_rows_after": after["cached_rows"],
                      "free_slots_after": after["free_slots"],
+                     "stage_rows": int(os.environ.get("COLL_MISS_STAGE_ROWS", "0")),
+                     "rows_taken_from_the_stage_per_refresh": staged_rows / n_steps,
                      "note": "refresh = rank + place + evict/insert lists on the device (COLL_GPU_REFRESH=1, hotness "
                              "accumulating), row copy over the host link, table update; foreground, after each lookup"}
         note("refresh each step: lookup %.3f ms + refresh %.3f ms" % (each_step["lookup_ms"], each_step["refresh_ms"]))

@@ -89,7 +89,7 @@ typedef struct {
 const char *ugk_last_error(void);
 /* version of this ABI; bumped on any signature change.  ugk_abi_version() is what the loaded library was built with:
  * a caller compiled against another UGK_ABI_VERSION must not go on. */
-#define UGK_ABI_VERSION 5
+#define UGK_ABI_VERSION 6
 int ugk_abi_version(void);
 
 /* ---- runtime plumbing: Device::{AllocDataSpace,FreeDataSpace,CopyDataFromTo,StreamSync,CreateStream}
@@ -234,9 +234,11 @@ int ugk_select_keys_i64(const int64_t *keys_dev, const uint32_t *sel_dev, size_t
  * itself before it returns, may be NULL) = the number of workgroups launched: once the stream has been waited for,
  * the sum of that many words gives the group sizes ugk_gather_group reports on the factored path.  Rows skipped for
  * a key without a row (status_dev flagged) are counted with the host rows.  n must stay below 2^32.
- * others_hint: the caller's estimate of how many of the n rows will NOT come from the cache (the previous batch's
- * count scaled to n, say), UGK_HINT_UNKNOWN if it has none.  Only the launch shape depends on it (a small batch that
- * nearly all hits a flat table is cut into shorter wavefronts than one bound by the host link), never a byte of the result. */
+ * others_hint: how many of the n rows will NOT come from the cache, where the caller knows (a batch of keys selected
+ * for being non-local, say), UGK_HINT_UNKNOWN where it does not.  Only the launch shape depends on it (at half the rows
+ * or more, and rows of 512 bytes or more, the grid is capped to 128 workgroups: the host link takes rows faster from a
+ * few workgroups than from a chip full of them, and a batch that mostly hits would be three times slower on so few, so
+ * a guess is worse than no hint), never a byte of the result. */
 #define UGK_HINT_UNKNOWN 0xffffffffu
 unsigned ugk_extract_mix_max_groups(void);
 int ugk_extract_mix_u32(ugk_table_t t, const uint32_t *keys_dev, size_t n, const void *cache_dev, uint64_t cache_rows,
@@ -247,6 +249,40 @@ int ugk_extract_mix_i64(ugk_table_t t, const int64_t *keys_dev, size_t n, const 
                         const void *host_dev, uint64_t host_rows, void *out_dev, size_t row_bytes,
                         uint32_t *status_dev, uint32_t *host_mirror, uint64_t *group_counts_host,
                         uint32_t *num_groups_host, uint32_t others_hint, void *stream);
+
+/* ---- rows that crossed the host link once, kept where a refresh finds them ---------------------------------------
+ * The rows a refresh inserts (RefreshSession::refresh_after_solve_new, cache_context.cu:4054-4090: rows copied host ->
+ * HBM in throttled batches) are rows recent lookups missed, i.e. rows that have just crossed the host link into some
+ * lookup's output.  A stage is a direct-mapped set of such rows in HBM: entry h = fmix64(row) & mask holds the bytes of
+ * the host row named by the low 32 bits of owner[h] whenever the high 32 bits (the tag of the launch that wrote it) are
+ * non-zero.  ugk_extract_mix_staged_* is ugk_extract_mix_* that also files every row it takes from the host table in the
+ * stage (first writer of a launch wins an entry; `epoch` must be non-zero and differ from launch to launch);
+ * ugk_gather_scatter_staged_u32 is ugk_gather_scatter_u32 out of the host table that takes a row from the stage when it
+ * is there, and adds the number of such rows to *staged_dev (device word, may be NULL).  Results are the same
+ * bytes with and without a stage: the host table does not change under a cache.  An entry is only consistent at launch
+ * boundaries, so the staged gather must not run while a staging extraction runs (a foreground refresh qualifies).
+ * rows_dev: (mask + 1) x row_bytes bytes; owner_dev: mask + 1 words, zero-filled once; host rows must fit 32 bits. */
+typedef struct {
+  void *rows_dev;
+  uint64_t *owner_dev;
+  uint64_t mask;  /* entries - 1, entries a power of two */
+  uint32_t epoch; /* launch tag, non-zero (ignored by the gather) */
+  uint32_t reserved;
+} ugk_stage_t;
+int ugk_extract_mix_staged_u32(ugk_table_t t, const uint32_t *keys_dev, size_t n, const void *cache_dev,
+                               uint64_t cache_rows, const void *host_dev, uint64_t host_rows, void *out_dev,
+                               size_t row_bytes, uint32_t *status_dev, uint32_t *host_mirror,
+                               uint64_t *group_counts_host, uint32_t *num_groups_host, uint32_t others_hint,
+                               ugk_stage_t stage, void *stream);
+int ugk_extract_mix_staged_i64(ugk_table_t t, const int64_t *keys_dev, size_t n, const void *cache_dev,
+                               uint64_t cache_rows, const void *host_dev, uint64_t host_rows, void *out_dev,
+                               size_t row_bytes, uint32_t *status_dev, uint32_t *host_mirror,
+                               uint64_t *group_counts_host, uint32_t *num_groups_host, uint32_t others_hint,
+                               ugk_stage_t stage, void *stream);
+int ugk_gather_scatter_staged_u32(const void *host_dev, uint64_t host_rows, const uint32_t *rows_dev,
+                                  const uint32_t *dst_off_dev, size_t n, void *out_dev, uint64_t out_rows,
+                                  size_t row_bytes, ugk_stage_t stage, unsigned max_blocks, uint32_t *status_dev,
+                                  uint32_t *staged_dev, void *stream);
 
 /* ---- key dedup (the caller-side array_ops.unique of
  *      python_tf2/collcache_tf2/collcache_tf2/core/sparse_lookup_layer.py:197) ------------------------

@@ -303,7 +303,7 @@ int nonlocal_flags(ugk_table_t t, const K *keys, size_t n, uint64_t *flags) {
 template <typename K>
 int extract_mix(ugk_table_t t, const K *keys, size_t n, const void *cache, uint64_t cache_rows, const void *host,
                 uint64_t host_rows, void *out, size_t rb, uint32_t *status, uint32_t *mirror, uint64_t *counts,
-                uint32_t *num_groups) {
+                uint32_t *num_groups, const ugk_stage_t *stage = nullptr) {
   if (num_groups) *num_groups = 0;
   if (n == 0) return 0;
   REQUIRE(keys && out && status, "ugk_extract_mix: null keys, output or status");
@@ -326,6 +326,16 @@ int extract_mix(ugk_table_t t, const K *keys, size_t n, const void *cache, uint6
       or_status(status, UGK_ST_KEY_OUT_OF_RANGE, mirror);
     }
     if (row) copy_row((char *)out + i * rb, row, rb);
+    if (row && !from_cache && stage) {
+      const uint64_t r = (uint64_t)(row - (const char *)host) / rb;
+      const uint64_t h = fmix64(r) & stage->mask;
+      const uint64_t cur = stage->owner_dev[h];
+      const uint32_t tag = (uint32_t)(cur >> 32);
+      if (r <= 0xffffffffull && tag != stage->epoch && !(tag != 0 && (uint32_t)cur == (uint32_t)r)) {
+        stage->owner_dev[h] = ((uint64_t)stage->epoch << 32) | (uint32_t)r;
+        copy_row((char *)stage->rows_dev + h * rb, row, rb);
+      }
+    }
     if (from_cache) ++local;
     else ++others;
   }
@@ -618,6 +628,43 @@ int ugk_extract_mix_i64(ugk_table_t t, const int64_t *keys, size_t n, const void
                         const void *host, uint64_t host_rows, void *out, size_t rb, uint32_t *status, uint32_t *mirror,
                         uint64_t *counts, uint32_t *num_groups, uint32_t, void *) {
   return extract_mix(t, keys, n, cache, cache_rows, host, host_rows, out, rb, status, mirror, counts, num_groups);
+}
+
+int ugk_extract_mix_staged_u32(ugk_table_t t, const uint32_t *keys, size_t n, const void *cache, uint64_t cache_rows,
+                               const void *host, uint64_t host_rows, void *out, size_t rb, uint32_t *status,
+                               uint32_t *mirror, uint64_t *counts, uint32_t *num_groups, uint32_t, ugk_stage_t stage,
+                               void *) {
+  REQUIRE(stage.rows_dev && stage.owner_dev && stage.epoch, "ugk_extract_mix_staged: bad stage");
+  return extract_mix(t, keys, n, cache, cache_rows, host, host_rows, out, rb, status, mirror, counts, num_groups,
+                     &stage);
+}
+int ugk_extract_mix_staged_i64(ugk_table_t t, const int64_t *keys, size_t n, const void *cache, uint64_t cache_rows,
+                               const void *host, uint64_t host_rows, void *out, size_t rb, uint32_t *status,
+                               uint32_t *mirror, uint64_t *counts, uint32_t *num_groups, uint32_t, ugk_stage_t stage,
+                               void *) {
+  REQUIRE(stage.rows_dev && stage.owner_dev && stage.epoch, "ugk_extract_mix_staged: bad stage");
+  return extract_mix(t, keys, n, cache, cache_rows, host, host_rows, out, rb, status, mirror, counts, num_groups,
+                     &stage);
+}
+int ugk_gather_scatter_staged_u32(const void *host, uint64_t host_rows, const uint32_t *rows, const uint32_t *dst,
+                                  size_t n, void *out, uint64_t out_rows, size_t rb, ugk_stage_t stage, unsigned,
+                                  uint32_t *status, uint32_t *staged, void *) {
+  if (n == 0) return 0;
+  REQUIRE(host && rows && dst && out && status && stage.rows_dev && stage.owner_dev, "staged gather: null pointer");
+  for (size_t i = 0; i < n; ++i) {
+    const uint64_t r = rows[i];
+    if (r >= host_rows || dst[i] >= out_rows) {
+      or_status(status, UGK_ST_KEY_OUT_OF_RANGE);
+      continue;
+    }
+    const uint64_t h = fmix64(r) & stage.mask;
+    const uint64_t cur = stage.owner_dev[h];
+    const bool filed = (cur >> 32) != 0 && (uint32_t)cur == (uint32_t)r;
+    copy_row((char *)out + (size_t)dst[i] * rb, filed ? (const char *)stage.rows_dev + h * rb : (const char *)host + r * rb,
+             rb);
+    if (filed && staged) ++*staged;
+  }
+  return 0;
 }
 
 size_t ugk_dedup_workspace_bytes(size_t) { return 64; }

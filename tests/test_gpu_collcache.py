@@ -415,7 +415,8 @@ def test_refresh_evicts_and_inserts_like_the_oracle(table_kind, foreground, impl
 @pytest.mark.parametrize("table_kind", ["FLAT", "HASH"])
 @pytest.mark.parametrize("foreground", [True, False])
 @pytest.mark.parametrize("keep", [False, True])
-def test_refresh_on_the_device_places_like_the_oracle(table_kind, foreground, keep, monkeypatch):
+@pytest.mark.parametrize("stage", [0, 16384])
+def test_refresh_on_the_device_places_like_the_oracle(table_kind, foreground, keep, stage, monkeypatch):
     """COLL_GPU_RECORD=1 + COLL_GPU_REFRESH=1: ranking, placement and the evict / insert lists of a refresh are computed
     on the device from the hotness the lookups counted there.  The cached set afterwards is the oracle's top set of the
     counted key stream (of the last interval, or of everything so far with COLL_GPU_REFRESH_KEEP=1), exactly as after
@@ -427,6 +428,8 @@ def test_refresh_on_the_device_places_like_the_oracle(table_kind, foreground, ke
         monkeypatch.setenv("COLL_GPU_REFRESH_KEEP", "1")
     monkeypatch.setenv("COLL_REFRESH_SLEEP_US", "100")
     monkeypatch.setenv("COLL_REFRESH_BATCH_ROWS", "512")
+    if stage:  # lookups file the rows they fetch from the host table; foreground refreshes insert from there
+        monkeypatch.setenv("COLL_MISS_STAGE_ROWS", str(stage))
     rng = np.random.default_rng(21)
     n_item, dim, pct = 50_001, 64, 0.2
     co.config(make_config(n_item, pct))
@@ -482,6 +485,9 @@ def test_refresh_on_the_device_places_like_the_oracle(table_kind, foreground, ke
         check_cached(new_cached)
         cached = new_cached
         lookup(rng.integers(0, n_item, size=20_000), nid)
+    from_stage = _basics.C_LIB_CTYPES.coll_cache_rows_from_stage(0)
+    # rows that come in were looked up (and missed) shortly before: a foreground refresh finds most of them filed
+    assert (from_stage > 1000) if (stage and foreground) else (from_stage == 0)
 
     # a refresh on the host in between (hotness recorded on the host joins the device-side counts) ...
     extra = perm[zipf_ranks(rng, 60_000, n_item, 1.3)]

@@ -542,6 +542,101 @@ def test_extract_mix_at_every_launch_shape(kind, rb):
         mirror.free()
 
 
+def _fmix64(x):
+    x = np.asarray(x, np.uint64).copy()
+    x ^= x >> np.uint64(33)
+    x *= np.uint64(0xFF51AFD7ED558CCD)
+    x ^= x >> np.uint64(33)
+    x *= np.uint64(0xC4CEB9FE1A85EC53)
+    x ^= x >> np.uint64(33)
+    return x
+
+
+@pytest.mark.parametrize("kind", ["flat", "hash"])
+@pytest.mark.parametrize("rb", [64, 128, 512])
+def test_rows_from_the_host_are_filed_in_the_stage_and_found_there(kind, rb):
+    """ugk_extract_mix_staged_*: same output and group sizes as the plain extraction; afterwards every owner word with a
+    tag names a host row whose bytes its entry holds, entries are where fmix64(row) & mask says, and rows of the cache
+    are never filed.  ugk_gather_scatter_staged_u32: the bytes of ugk_gather_scatter_u32; the number of rows it reports
+    as taken from the stage is the number of listed rows the owner words name."""
+    rng = np.random.default_rng(rb + (kind == "hash"))
+    nkeys, entries = 30_000, 4096
+    host = _rand_table(rng, nkeys, rb)
+    cached = rng.choice(nkeys, nkeys // 2, replace=False).astype(np.int64)
+    slots = rng.permutation(len(cached)).astype(np.uint32)
+    cache = np.zeros((len(cached), rb), np.uint8)
+    cache[slots] = host[cached]
+    if kind == "flat":
+        mem, tb = _make_flat(nkeys)
+    else:
+        mem, tb, _ = _make_hash(len(cached))
+    assert _insert(tb, cached, slots) == 0
+    is_cached = np.zeros(nkeys, bool)
+    is_cached[cached] = True
+    pin = pinned_from(host)
+    mirror = pinned_from(np.zeros(4, np.uint32))
+    try:
+        st = dev_zeros_u32(1)
+        d_cache = to_dev(cache)
+        stage_rows = dev_bytes(entries * rb, fill=0xEE)
+        owner = to_dev(np.zeros(entries, np.uint64))
+        words = PinnedArray((hip.lib().ugk_extract_mix_max_groups(),), np.uint64)
+        groups = C.c_uint32(0)
+        seen_hosts = set()
+        for epoch, n in enumerate((1, 700, 9_000, 70_000), start=1):
+            keys = rng.integers(0, nkeys, size=n).astype(np.int64)
+            d_keys = to_dev(keys)
+            out = dev_bytes(n * rb, fill=0x3C)
+            stage = hip.Stage(ptr(stage_rows), ptr(owner), entries - 1, epoch, 0)
+            hip.call("ugk_extract_mix_staged_i64", tb, ptr(d_keys), n, ptr(d_cache), len(cached), pin.ptr, nkeys,
+                     ptr(out), rb, ptr(st), mirror.ptr, words.ptr, C.byref(groups), hip.HINT_UNKNOWN, stage, None)
+            sync()
+            assert status_value(st) == 0
+            w = words.array[: groups.value]
+            n_local = int(is_cached[keys].sum())
+            assert [int((w & np.uint64(0xFFFFFFFF)).sum()), int((w >> np.uint64(32)).sum())] == [n_local, n - n_local]
+            assert to_np(out)[: n * rb].tobytes() == host[keys].tobytes()
+            seen_hosts.update(keys[~is_cached[keys]].tolist())
+            own = to_np(owner, np.uint64)[:entries]
+            tags, rows = (own >> np.uint64(32)).astype(np.int64), (own & np.uint64(0xFFFFFFFF)).astype(np.int64)
+            filled = np.flatnonzero(tags != 0)
+            assert (len(filled) > 0) == bool(seen_hosts) and tags.max() <= epoch
+            assert all(int(r) in seen_hosts for r in rows[filled])  # only rows that came from the host, never cached ones
+            assert np.array_equal(_fmix64(rows[filled]) & np.uint64(entries - 1), filled.astype(np.uint64))
+            got = to_np(stage_rows)[: entries * rb].reshape(entries, rb)
+            assert np.array_equal(got[filled], host[rows[filled]])
+            # every host row of this batch whose entry was free of this launch's tag before it is there now, or lost
+            # its entry to another row of the same launch
+            missed = np.unique(keys[~is_cached[keys]])
+            h = (_fmix64(missed) & np.uint64(entries - 1)).astype(np.int64)
+            assert (tags[h] != 0).all()
+        # the staged gather: rows from everywhere, some filed, some not
+        own = to_np(owner, np.uint64)[:entries]
+        filed_rows = (own[(own >> np.uint64(32)) != 0] & np.uint64(0xFFFFFFFF)).astype(np.uint32)
+        take = np.unique(np.concatenate([filed_rows[::2], rng.integers(0, nkeys, size=5000).astype(np.uint32)]))
+        rng.shuffle(take)
+        dst = rng.permutation(len(take) + 100)[: len(take)].astype(np.uint32)
+        out_rows = len(take) + 100
+        out = dev_bytes(out_rows * rb, fill=0x11)
+        n_staged = dev_zeros_u32(1)
+        d_take, d_dst = to_dev(take), to_dev(dst)
+        stage = hip.Stage(ptr(stage_rows), ptr(owner), entries - 1, 0, 0)
+        for cap in (0, 7):
+            hip.call("ugk_gather_scatter_staged_u32", pin.ptr, nkeys, ptr(d_take), ptr(d_dst), len(take), ptr(out),
+                     out_rows, rb, stage, cap, ptr(st), ptr(n_staged), None)
+        sync()
+        assert status_value(st) == 0
+        want = np.full((out_rows, rb), 0x11, np.uint8)
+        want[dst] = host[take]
+        assert to_np(out)[: out_rows * rb].tobytes() == want.tobytes()
+        assert int(to_np(n_staged, np.uint32)[0]) == 2 * int(np.isin(take, filed_rows).sum())
+        words.free()
+    finally:
+        sync()
+        pin.free()
+        mirror.free()
+
+
 def test_classify_rejects_keys_beyond_the_host_table():
     mem, tb = _make_flat(100)
     keys = np.array([5, 100, 7, 1 << 33], np.int64)

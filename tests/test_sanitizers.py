@@ -26,6 +26,7 @@ def drivers():
 def _run(exe, table, refresh, steps):
     env = dict(os.environ)
     env["COLL_HASH_REBUILD_FRAC"] = "0.02"  # a few hundred evictions already rebuild the open-addressing table
+    env["COLL_MISS_STAGE_ROWS"] = "4096"  # lookups file the rows they fetch from the host, foreground refreshes read them
     env["ASAN_OPTIONS"] = "detect_leaks=1:abort_on_error=0"
     env["UBSAN_OPTIONS"] = "print_stacktrace=1:halt_on_error=1"
     env["TSAN_OPTIONS"] = "halt_on_error=0:second_deadlock_stack=1"

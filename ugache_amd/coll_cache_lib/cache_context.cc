@@ -241,6 +241,18 @@ ExtractSession::ExtractSession(std::shared_ptr<CacheContext> cache_ctx) : _cache
   memset(_host_mirror, 0, 256);
   const auto &desc = RunConfig::coll_cache_link_desc;
   if (!desc.cpu_sm.empty()) _cpu_blocks = (unsigned)desc.cpu_sm[0];
+  if (RunConfig::miss_stage_rows > 0 && !_cache_ctx->IsDirectMapping() && _cache_ctx->_row_bytes % 16 == 0 &&
+      _cache_ctx->_num_total_nodes <= 0x100000000ull) {
+    size_t entries = 1024;
+    while (entries < RunConfig::miss_stage_rows) entries <<= 1;
+    _stage_rows = EagerGPUAlloc(dev, entries * _cache_ctx->_row_bytes);
+    _stage_owner = EagerGPUAlloc(dev, entries * sizeof(uint64_t));
+    UGK_CALL(ugk_fill_u32(_stage_owner->ptr<uint32_t>(), 0, entries * 2, nullptr));
+    UGK_CALL(ugk_stream_sync(nullptr));
+    _stage.rows_dev = _stage_rows->ptr();
+    _stage.owner_dev = _stage_owner->ptr<uint64_t>();
+    _stage.mask = entries - 1;
+  }
   if (RunConfig::gpu_record) {
     const size_t rows = _cache_ctx->_num_total_nodes;
     _hot_counts = EagerGPUAlloc(dev, std::max<size_t>(rows, 1) * sizeof(uint32_t));
@@ -466,13 +478,19 @@ size_t ExtractSession::DedupKeys(const KeyT *nodes, size_t num_nodes, StreamHand
 
 static int ExtractMix(ugk_table_t t, const IdType *keys, size_t n, const void *cache, uint64_t cache_rows,
                       const void *host, uint64_t host_rows, void *out, size_t rb, uint32_t *st, uint32_t *mirror,
-                      uint64_t *counts, uint32_t *groups, uint32_t hint, StreamHandle s) {
+                      uint64_t *counts, uint32_t *groups, uint32_t hint, const ugk_stage_t *stage, StreamHandle s) {
+  if (stage)
+    return ugk_extract_mix_staged_u32(t, keys, n, cache, cache_rows, host, host_rows, out, rb, st, mirror, counts,
+                                      groups, hint, *stage, s);
   return ugk_extract_mix_u32(t, keys, n, cache, cache_rows, host, host_rows, out, rb, st, mirror, counts, groups, hint,
                              s);
 }
 static int ExtractMix(ugk_table_t t, const Id64Type *keys, size_t n, const void *cache, uint64_t cache_rows,
                       const void *host, uint64_t host_rows, void *out, size_t rb, uint32_t *st, uint32_t *mirror,
-                      uint64_t *counts, uint32_t *groups, uint32_t hint, StreamHandle s) {
+                      uint64_t *counts, uint32_t *groups, uint32_t hint, const ugk_stage_t *stage, StreamHandle s) {
+  if (stage)
+    return ugk_extract_mix_staged_i64(t, keys, n, cache, cache_rows, host, host_rows, out, rb, st, mirror, counts,
+                                      groups, hint, *stage, s);
   return ugk_extract_mix_i64(t, keys, n, cache, cache_rows, host, host_rows, out, rb, st, mirror, counts, groups, hint,
                              s);
 }
@@ -553,14 +571,6 @@ void ExtractSession::SumMixCounts() {
   }
   _host_mirror[kMirGroupSizes + UGK_LOC_LOCAL] = (uint32_t)local;
   _host_mirror[kMirGroupSizes + UGK_LOC_HOST] = (uint32_t)others;
-  _mix_seen_rows = local + others;
-  _mix_seen_others = others;
-}
-
-// what the next fused launch is told to expect: the share of rows the last one took from outside the cache
-uint32_t ExtractSession::MixOthersHint(size_t num_nodes) const {
-  if (_mix_seen_rows == 0) return UGK_HINT_UNKNOWN;
-  return (uint32_t)((double)_mix_seen_others / (double)_mix_seen_rows * (double)num_nodes);
 }
 
 // A lookup the refresh thread must wait for: counted from before it reads the table handle until its output is complete
@@ -684,9 +694,12 @@ void ExtractSession::ExtractFeatImpl(const KeyT *nodes, size_t num_nodes, void *
     const bool events = RunConfig::kernel_events;
     Timer t_host;
     if (events) UGK_CALL(ugk_event_record(_ev_t[0], stream));
+    // The hint caps the launch to a few workgroups, which is right for a batch of host rows only and three times too
+    // slow for one that mostly hits: it is given where the share is known (the keys COLL_SKIP_LOCAL selected all come
+    // from outside the cache), not guessed from the previous batch.
+    const uint32_t hint = skip_local ? (uint32_t)num_nodes : UGK_HINT_UNKNOWN;
     UGK_CALL(ExtractMix(table, nodes, num_nodes, cache, cache_rows, host, host_rows, output, rb, _status,
-                        _host_mirror, _mix_counts->ptr<uint64_t>(), &_mix_groups, MixOthersHint(num_nodes),
-                        stream));
+                        _host_mirror, _mix_counts->ptr<uint64_t>(), &_mix_groups, hint, NextStage(), stream));
     if (events) UGK_CALL(ugk_event_record(_ev_t[1], stream));
     RecordLaunch(input_nodes, num_input, keys_ready);
     UGK_CALL(ugk_stream_sync(stream));
@@ -837,7 +850,7 @@ void ExtractSession::ExtractFeatAsyncImpl(const KeyT *nodes, size_t num_nodes, v
     UGK_CALL(ExtractMix(ctx->_new_hash_table->Table(), nodes, num_nodes,
                         ctx->_device_cache_data[ctx->_local_location_id], ctx->_cache_space_capacity,
                         ctx->_device_cache_data[ctx->_cpu_location_id], ctx->_num_total_nodes, output, rb, _status,
-                        _host_mirror, _mix_counts->ptr<uint64_t>(), &_mix_groups, MixOthersHint(num_nodes),
+                        _host_mirror, _mix_counts->ptr<uint64_t>(), &_mix_groups, UGK_HINT_UNKNOWN, NextStage(),
                         stream));
     RecordLaunch(nodes, num_nodes, keys_ready);
     JoinRecord(stream);
@@ -989,7 +1002,7 @@ void RefreshSession::WaitForOneLookup(ExtractSession *session, bool foreground) 
 }
 
 void RefreshSession::CopyRowsIntoSlots(const uint32_t *rows_dev, const uint32_t *slots_dev, size_t num_rows,
-                                       bool foreground, StreamHandle copy_stream) {
+                                       bool foreground, StreamHandle copy_stream, const ugk_stage_t *stage) {
   CacheContext *ctx = _cache_ctx.get();
   const void *host = ctx->_device_cache_data[ctx->_cpu_location_id];
   void *cache = ctx->_device_cache_data[ctx->_local_location_id];
@@ -1001,9 +1014,17 @@ void RefreshSession::CopyRowsIntoSlots(const uint32_t *rows_dev, const uint32_t 
   const unsigned limit_block = foreground ? 128 : RunConfig::refresh_limit_block;
   for (size_t begin = 0; begin < num_rows; begin += batch) {
     const size_t cur = std::min(batch, num_rows - begin);
-    UGK_CALL(ugk_gather_scatter_u32(host, ctx->_num_total_nodes, rows_dev + begin, slots_dev + begin, cur, cache,
-                                    ctx->_cache_space_capacity, ctx->_row_bytes, limit_block, status, nullptr,
-                                    copy_stream));
+    if (stage) {
+      // most of the rows a refresh brings in were missed by the last few lookups, which filed them in HBM (status word 8
+      // counts the rows found there)
+      UGK_CALL(ugk_gather_scatter_staged_u32(host, ctx->_num_total_nodes, rows_dev + begin, slots_dev + begin, cur,
+                                             cache, ctx->_cache_space_capacity, ctx->_row_bytes, *stage, 0, status,
+                                             status + 8, copy_stream));
+    } else {
+      UGK_CALL(ugk_gather_scatter_u32(host, ctx->_num_total_nodes, rows_dev + begin, slots_dev + begin, cur, cache,
+                                      ctx->_cache_space_capacity, ctx->_row_bytes, limit_block, status, nullptr,
+                                      copy_stream));
+    }
     if (!foreground && begin + batch < num_rows) {
       UGK_CALL(ugk_stream_sync(copy_stream));
       usleep(RunConfig::refresh_sleep_us);
@@ -1014,6 +1035,14 @@ void RefreshSession::CopyRowsIntoSlots(const uint32_t *rows_dev, const uint32_t 
   UGK_CALL(ugk_memcpy_async(&st, status, sizeof(st), copy_stream));
   UGK_CALL(ugk_stream_sync(copy_stream));
   CHECK_EQ(st, 0u) << "refresh row copy touched a row outside its table";
+}
+
+uint64_t RefreshSession::RowsFromStage() {
+  if (!_status_handle) return 0;
+  uint32_t n = 0;
+  UGK_CALL(ugk_memcpy_async(&n, _status_handle->ptr<uint32_t>() + 8, sizeof(n), stream));
+  UGK_CALL(ugk_stream_sync(stream));
+  return n;
 }
 
 // cache_context.cu:3944-4107, the one-GPU part: steps 1-3, 5 and 6
@@ -1093,7 +1122,7 @@ void RefreshSession::refresh_after_solve_new(bool foreground) {
     auto reserved_offset =
         CopyTo1DReuse(__offs_buffer, table->ReserveOffsetFront((IdType)num_insert), gpu_ctx, low_pri_stream);
     CopyRowsIntoSlots(insert_keys_gpu->CPtr<uint32_t>(), reserved_offset->CPtr<uint32_t>(), num_insert, foreground,
-                      low_pri_stream);
+                      low_pri_stream, foreground && session ? session->Stage() : nullptr);
     auto insert_table_keys =
         RunConfig::key_map_mul == 0
             ? insert_keys_gpu
@@ -1193,20 +1222,24 @@ void RefreshSession::refresh_on_device(ExtractSession *session, size_t num_cache
         table->EmitBits(table->SlotUsedBits(), nullptr, true, capacity, 0, num_insert, __free_slots, alloc, gpu_ctx, stream);
     if (foreground) {
       // nothing runs beside a foreground refresh: the copy goes on the refresh's own stream, behind the lists it reads
-      CopyRowsIntoSlots(insert_rows->CPtr<uint32_t>(), slots->CPtr<uint32_t>(), num_insert, true, stream);
+      CopyRowsIntoSlots(insert_rows->CPtr<uint32_t>(), slots->CPtr<uint32_t>(), num_insert, true, stream,
+                        session->Stage());
     } else {
       UGK_CALL(ugk_stream_sync(stream));  // the lists are read on the copy stream next
-      CopyRowsIntoSlots(insert_rows->CPtr<uint32_t>(), slots->CPtr<uint32_t>(), num_insert, false, low_pri_stream);
+      CopyRowsIntoSlots(insert_rows->CPtr<uint32_t>(), slots->CPtr<uint32_t>(), num_insert, false, low_pri_stream,
+                        nullptr);
     }
     UGK_CALL(ugk_bitmap_update(table->SlotUsedBits(), capacity, slots->CPtr<uint32_t>(), num_insert, 1,
                                _status_handle->ptr<uint32_t>(), stream));
     TensorPtr insert_keys = table->RowsToTableKeys(insert_rows, __insert_ids, alloc, gpu_ctx, stream);
     table->InsertWithLoc(insert_keys, slots, local, stream);
   }
-  uint32_t st = 0;
-  UGK_CALL(ugk_memcpy_async(&st, _status_handle->ptr<uint32_t>(), sizeof(st), stream));
+  uint32_t stw[9] = {0};  // [0] status bits, [8] rows taken from the stage so far
+  UGK_CALL(ugk_memcpy_async(stw, _status_handle->ptr<uint32_t>(), sizeof(stw), stream));
   table->CheckStatus(stream, "refresh on the device");  // waits for the stream
-  CHECK_EQ(st, 0u) << "refresh on the device: a listed row or slot is outside its table or bitmap";
+  CHECK_EQ(stw[0], 0u) << "refresh on the device: a listed row or slot is outside its table or bitmap";
+  const uint32_t from_stage = stw[8] - _rows_from_stage;
+  _rows_from_stage = stw[8];
   if (n_free_word) CHECK_EQ((size_t)*n_free_word, num_free_expected);
   AnonymousBarrier::_refresh_instance->Wait();
   const double insert_s = t_phase.Passed();
@@ -1222,7 +1255,8 @@ void RefreshSession::refresh_on_device(ExtractSession *session, size_t num_cache
   });
   LOG(INFO) << "refresh on the device: bitmaps " << sync_s << " s, placement + key lists " << place_s << " s, evict "
             << evict_s << " s, wait for a lookup " << wait_s << " s, row copy + insert " << insert_s
-            << " s, table rebuild " << (rebuilt ? t_phase.Passed() : 0.0) << " s";
+            << " s (" << from_stage << " of " << num_insert << " rows from the stage), table rebuild "
+            << (rebuilt ? t_phase.Passed() : 0.0) << " s";
 }
 
 

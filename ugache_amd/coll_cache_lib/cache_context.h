@@ -151,8 +151,17 @@ class ExtractSession {
   uint32_t _mix_groups = 0;        // workgroups of the last fused launch
   bool _async_last_fused = false;  // the last stream-ordered lookup was a fused launch (its counts wait to be summed)
   void SumMixCounts();
-  uint64_t _mix_seen_rows = 0, _mix_seen_others = 0;  // what the last summed fused launch found
-  uint32_t MixOthersHint(size_t num_nodes) const;
+  // rows that crossed the host link, kept for the next refresh (COLL_MISS_STAGE_ROWS): written by the fused extraction,
+  // read by a foreground refresh, which by contract runs while no lookup does
+  MemHandle _stage_rows, _stage_owner;
+  ugk_stage_t _stage = {nullptr, nullptr, 0, 0, 0};
+  uint32_t _stage_epoch = 0;
+  const ugk_stage_t *NextStage() {  // the stage with a fresh launch tag, or null when there is none
+    if (_stage.rows_dev == nullptr) return nullptr;
+    if (++_stage_epoch == 0) _stage_epoch = 1;
+    _stage.epoch = _stage_epoch;
+    return &_stage;
+  }
   size_t _async_pending = 0;       // stream-ordered lookups enqueued since the last Wait()
   size_t _async_last_nodes = 0;    // size of the last of them
   // What a refresh has to see finished before it reuses the slots of evicted rows: blocking lookups are counted when
@@ -234,6 +243,8 @@ class ExtractSession {
   // Runs on the record stream, ordered against the counting of every lookup; `stream` waits for the result.
   // reset_counts: the next interval starts from zero, as after DrainHotness.
   bool CountsOnDevice() const { return _hot_counts != nullptr; }
+  // what a foreground refresh may read rows from besides the host table (null: nothing)
+  const ugk_stage_t *Stage() const { return _stage.rows_dev ? &_stage : nullptr; }
   void PlaceOnDevice(size_t num_cached, uint64_t *in_new_bits, uint64_t *scratch_bits, void *rank_ws,
                      bool reset_counts, StreamHandle stream);
   // the device-side counting of the following lookups covers only the first `num_keys` keys of a batch
@@ -259,10 +270,15 @@ class RefreshSession {
   TensorPtr CopyTo1DReuse(TensorPtr &preserved_buffer, TensorPtr src, Context ctx, StreamHandle stream);
   // step 5: lets one more lookup finish, so that no gather in flight still reads a slot about to be reused
   void WaitForOneLookup(ExtractSession *session, bool foreground);
+  uint32_t _rows_from_stage = 0;  // what status word 8 read after the last refresh on the device
+ public:
+  // rows the refreshes of this session have taken from the stage instead of the host table so far (blocks)
+  uint64_t RowsFromStage();
+ private:
   // copies the listed host rows into the listed cache slots (step 6): in one launch when in the foreground, in
   // small throttled batches behind running lookups otherwise
   void CopyRowsIntoSlots(const uint32_t *rows_dev, const uint32_t *slots_dev, size_t num_rows, bool foreground,
-                         StreamHandle copy_stream);
+                         StreamHandle copy_stream, const ugk_stage_t *stage);
   TensorPtr __keys_buffer;
   TensorPtr __offs_buffer;
   TensorPtr __evict_rows, __insert_rows, __free_slots, __evict_ids, __insert_ids, __evict_slots;

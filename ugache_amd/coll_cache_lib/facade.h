@@ -76,6 +76,12 @@ class CollCache : public std::enable_shared_from_this<CollCache> {
   // the same refresh with ranking, placement and key lists computed on the device from the hotness the lookups
   // counted there (RunConfig::gpu_refresh); _nid_to_block is not updated by it
   void refresh_on_device(int replica_id, StreamHandle stream = nullptr, bool foreground = false);
+  // rows the refreshes of a replica took from the stage of recently missed rows instead of the host table
+  uint64_t rows_from_stage(int replica_id) {
+    return (size_t)replica_id < _refresh_session_list.size() && _refresh_session_list[replica_id]
+               ? _refresh_session_list[replica_id]->RowsFromStage()
+               : 0;
+  }
 
   void report_avg();
   void report_last_epoch(uint64_t epoch);

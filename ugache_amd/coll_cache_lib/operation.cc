@@ -439,6 +439,11 @@ void coll_cache_get_info(int replica_id, uint64_t out[8]) {
   out[7] = ctx->EntryManager() ? ctx->EntryManager()->_num_rebuilds : 0;
 }
 
+uint64_t coll_cache_rows_from_stage(int replica_id) {
+  CHECK_NOTNULL(_coll_cache);
+  return _coll_cache->rows_from_stage(replica_id);
+}
+
 size_t coll_cache_get_cached_keys(int replica_id, uint32_t *out, size_t capacity) {
   CHECK_NOTNULL(_coll_cache);
   _coll_cache->cache_ctx(replica_id)->SyncHostLists();

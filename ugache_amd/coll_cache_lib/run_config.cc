@@ -40,6 +40,7 @@ bool RunConfig::gpu_record = false;
 size_t RunConfig::gpu_record_every = 1;
 bool RunConfig::gpu_refresh = false;
 bool RunConfig::gpu_refresh_keep = false;
+size_t RunConfig::miss_stage_rows = 0;
 bool RunConfig::kernel_events = false;
 bool RunConfig::dedup_keys = false;
 size_t RunConfig::dedup_min_keys = 4096;
@@ -81,6 +82,7 @@ void RunConfig::LoadConfigFromEnv() {
   gpu_record_every = 1;
   gpu_refresh = false;
   gpu_refresh_keep = false;
+  miss_stage_rows = 0;
   kernel_events = false;
   if (GetEnv("SAMGRAPH_EMPTY_FEAT") != "" && GetEnv("SAMGRAPH_EMPTY_FEAT") != "0") {
     LOG(FATAL) << "SAMGRAPH_EMPTY_FEAT (mock host table) is not supported by this build: every key must have a "
@@ -113,6 +115,7 @@ void RunConfig::LoadConfigFromEnv() {
   if (GetEnv("COLL_GPU_RECORD") != "") gpu_record = GetEnv("COLL_GPU_RECORD") != "0";
   if (GetEnv("COLL_GPU_REFRESH") != "") gpu_refresh = GetEnv("COLL_GPU_REFRESH") != "0";
   if (GetEnv("COLL_GPU_REFRESH_KEEP") != "") gpu_refresh_keep = GetEnv("COLL_GPU_REFRESH_KEEP") != "0";
+  if (GetEnv("COLL_MISS_STAGE_ROWS") != "") miss_stage_rows = (size_t)std::stoull(GetEnv("COLL_MISS_STAGE_ROWS"));
   if (GetEnv("COLL_KERNEL_EVENTS") != "") kernel_events = GetEnv("COLL_KERNEL_EVENTS") != "0";
   if (GetEnv("COLL_GPU_RECORD_EVERY") != "")
     gpu_record_every = std::max<size_t>(1, std::stoull(GetEnv("COLL_GPU_RECORD_EVERY")));

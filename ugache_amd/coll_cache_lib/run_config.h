@@ -71,6 +71,10 @@ struct RunConfig {
   // COLL_GPU_REFRESH_KEEP=1: such a refresh leaves the counters as they are (hotness accumulates over refreshes)
   // instead of starting the next interval from zero
   static bool gpu_refresh_keep;
+  // COLL_MISS_STAGE_ROWS=n (0 = off): the fused extraction also files the rows it takes from the host table in a
+  // direct-mapped set of n (rounded up to a power of two) rows in HBM, and a foreground refresh takes the rows it inserts
+  // from there when it finds them instead of over the host link again
+  static size_t miss_stage_rows;
   static bool kernel_events;  // COLL_KERNEL_EVENTS: per-step kernel times from device events (1) or a host timer (0)
   static bool dedup_keys;        // COLL_DEDUP_KEYS=1: extract each distinct key of a batch once, then copy the duplicates
   static size_t dedup_min_keys;  // COLL_DEDUP_MIN_KEYS, default 4096: shorter batches skip the deduplication

@@ -120,6 +120,7 @@ C_API = {
     "coll_cache_last_group_offset": (None, [ctypes.c_int, ctypes.POINTER(ctypes.c_uint32 * 3)]),
     "coll_cache_get_info": (None, [ctypes.c_int, ctypes.POINTER(ctypes.c_uint64 * 8)]),
     "coll_cache_get_cached_keys": (ctypes.c_size_t, [ctypes.c_int, ctypes.c_void_p, ctypes.c_size_t]),
+    "coll_cache_rows_from_stage": (ctypes.c_uint64, [ctypes.c_int]),
     "coll_cache_get_step_value": (ctypes.c_double, [ctypes.c_uint64, ctypes.c_int]),
     "coll_cache_rank_hotness": (ctypes.c_size_t, [ctypes.c_int, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_size_t]),
     "coll_cache_place_ranked": (ctypes.c_uint32, [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_uint32, ctypes.c_double,

@@ -17,6 +17,7 @@
 #include <cstdlib>
 
 #include "ugk_internal.h"
+#include "ugk_table.cuh"
 
 namespace ugk {
 namespace {
@@ -144,6 +145,61 @@ __global__ __launch_bounds__(kBlock) void replicate_kernel(V *out, uint32_t vpr,
     if (r == i) continue;
     for (uint32_t col = lane; col < vpr; col += LPR) out[i * vpr + col] = out[r * vpr + col];
   }
+}
+
+// Rows out of the host table, or out of the stage where it holds them (refresh inserts: most of the rows a refresh
+// brings in were missed by the last few lookups and are filed there).  Lanes per row chosen at run time: this runs at
+// refresh time, on some hundred thousand rows.
+__global__ __launch_bounds__(kBlock) void gather_staged_kernel(const u32x4 *__restrict__ host, uint64_t host_rows,
+                                                               const uint32_t *__restrict__ rows,
+                                                               const uint32_t *__restrict__ dst, size_t n,
+                                                               u32x4 *__restrict__ out, uint64_t out_rows, uint32_t vpr,
+                                                               uint32_t lpr, ugk_stage_t stage, uint32_t *status,
+                                                               uint32_t *staged) {
+  constexpr int UNROLL = 2;
+  __shared__ uint32_t block_staged;
+  if (threadIdx.x == 0) block_staged = 0;
+  __syncthreads();
+  const uint32_t lane = threadIdx.x % lpr, rib = threadIdx.x / lpr, rpb = kBlock / lpr;
+  const size_t per_iter = (size_t)rpb * UNROLL;
+  const u32x4 *stage_rows = reinterpret_cast<const u32x4 *>(stage.rows_dev);
+  uint32_t mine = 0;
+  for (size_t base = (size_t)blockIdx.x * per_iter; base < n; base += (size_t)gridDim.x * per_iter) {
+    const u32x4 *src[UNROLL];
+    uint64_t d[UNROLL];
+    bool ok[UNROLL];
+#pragma unroll
+    for (int u = 0; u < UNROLL; ++u) {
+      const size_t r = base + (size_t)u * rpb + rib;
+      ok[u] = r < n;
+      const uint64_t s = rows[ok[u] ? r : n - 1];
+      d[u] = dst[ok[u] ? r : n - 1];
+      if (ok[u] && (s >= host_rows || d[u] >= out_rows)) {
+        ok[u] = false;
+        if (lane == 0) atomicOr(status, UGK_ST_KEY_OUT_OF_RANGE);
+      }
+      const uint64_t h = fmix64(s) & stage.mask;
+      const unsigned long long cur = stage.owner_dev[h];
+      const bool filed = ok[u] && (cur >> 32) != 0 && (uint32_t)cur == (uint32_t)s;
+      src[u] = !ok[u] ? reinterpret_cast<const u32x4 *>(out) : filed ? stage_rows + h * vpr : host + s * vpr;
+      if (filed && lane == 0) ++mine;
+    }
+    for (uint32_t c0 = 0; c0 < vpr; c0 += lpr) {
+      const uint32_t col = c0 + lane;
+      if (col < vpr) {
+        u32x4 v[UNROLL];
+#pragma unroll
+        for (int u = 0; u < UNROLL; ++u) v[u] = ld_stream(src[u] + col);
+#pragma unroll
+        for (int u = 0; u < UNROLL; ++u)
+          if (ok[u]) out[d[u] * vpr + col] = v[u];
+      }
+    }
+  }
+  if (staged == nullptr) return;
+  if (mine) atomicAdd(&block_staged, mine);
+  __syncthreads();
+  if (threadIdx.x == 0 && block_staged) atomicAdd(staged, block_staged);
 }
 
 // A launch that may fill the chip (max_blocks == 0) gets one workgroup per pass of rows, however many that makes:
@@ -296,6 +352,30 @@ int ugk_gather_scatter_i64(const void *src_dev, uint64_t src_rows, const int64_t
   UGK_REQUIRE(n == 0 || (keys_dev && dst_off_dev), "ugk_gather_scatter_i64: null keys or destinations");
   return launch_gather(ScatterI64{keys_dev, dst_off_dev}, src_dev, src_rows, out_dev, out_rows, row_bytes, nullptr, 0,
                        n, max_blocks, status_dev, host_mirror, stream);
+}
+
+int ugk_gather_scatter_staged_u32(const void *host_dev, uint64_t host_rows, const uint32_t *rows_dev,
+                                  const uint32_t *dst_off_dev, size_t n, void *out_dev, uint64_t out_rows,
+                                  size_t row_bytes, ugk_stage_t stage, unsigned max_blocks, uint32_t *status_dev,
+                                  uint32_t *staged_dev, void *stream) {
+  if (n == 0) return 0;
+  UGK_REQUIRE(host_dev && rows_dev && dst_off_dev && out_dev && status_dev, "ugk_gather_scatter_staged_u32: null pointer");
+  UGK_REQUIRE(stage.rows_dev && stage.owner_dev && ((stage.mask + 1) & stage.mask) == 0,
+              "ugk_gather_scatter_staged_u32: the stage needs buffers and a power of two of entries");
+  const uintptr_t align = (uintptr_t)host_dev | (uintptr_t)out_dev | (uintptr_t)stage.rows_dev | (uintptr_t)row_bytes;
+  UGK_REQUIRE(row_bytes > 0 && align % 16 == 0,
+              "ugk_gather_scatter_staged_u32: rows and buffers must be multiples of 16 bytes (row_bytes=%zu)", row_bytes);
+  UGK_REQUIRE(host_rows <= 0x100000000ull, "ugk_gather_scatter_staged_u32: host rows must fit 32 bits");
+  const uint32_t vpr = (uint32_t)(row_bytes / 16);
+  uint32_t lpr = 1;
+  while (lpr < vpr && lpr < 64) lpr <<= 1;
+  const size_t per_iter = (size_t)(kBlock / lpr) * 2;
+  const unsigned grid = clamp_grid((n + per_iter - 1) / per_iter, max_blocks);
+  hipLaunchKernelGGL(gather_staged_kernel, dim3(grid), dim3(kBlock), 0, as_stream(stream),
+                     reinterpret_cast<const u32x4 *>(host_dev), host_rows, rows_dev, dst_off_dev, n,
+                     reinterpret_cast<u32x4 *>(out_dev), out_rows, vpr, lpr, stage, status_dev, staged_dev);
+  UGK_HIP(hipGetLastError());
+  return 0;
 }
 
 int ugk_gather_group(const void *src_dev, uint64_t src_rows, const ugk_idx_t *idx_dev, const uint32_t *counts_dev,

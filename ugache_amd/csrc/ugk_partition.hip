@@ -166,6 +166,7 @@ typedef __attribute__((address_space(1))) u32x4 *gout_t;
 // where a key's row lives, as an integer address (the head of the output for a key without a row, see below)
 struct MixRow {
   uint64_t bits;
+  uint64_t host_row;  // the row of the host table it is, ~0 for a row of the cache or no row
   bool has_row, from_cache;
 };
 
@@ -174,10 +175,11 @@ __device__ __forceinline__ MixRow mix_resolve(const ugk_table_t &t, uint64_t key
                                               uint64_t host_rows, const u32x4 *out, uint32_t vpr, uint32_t *status,
                                               uint32_t *host_mirror) {
   const u32x4 *rowp = nullptr;
+  uint64_t host_row = ~0ull;
   if (active) {
     if (f.hit && f.loc == UGK_LOC_LOCAL && f.off < cache_rows) rowp = cache + (uint64_t)f.off * vpr;
-    else if (f.hit && f.loc == UGK_LOC_HOST && f.off < host_rows) rowp = host + (uint64_t)f.off * vpr;
-    else if (!f.hit && fallback_row(t, key) < host_rows) rowp = host + fallback_row(t, key) * vpr;
+    else if (f.hit && f.loc == UGK_LOC_HOST && f.off < host_rows) host_row = f.off;
+    else if (!f.hit && fallback_row(t, key) < host_rows) host_row = fallback_row(t, key);
     else {
       atomicOr(status, UGK_ST_KEY_OUT_OF_RANGE);
       if (host_mirror) host_mirror[0] = UGK_ST_KEY_OUT_OF_RANGE;
@@ -185,7 +187,9 @@ __device__ __forceinline__ MixRow mix_resolve(const ugk_table_t &t, uint64_t key
   }
   // A key without a row copies nothing; its lanes read the head of the output instead (mapped whatever the key), so
   // that the loads of the copy carry no branch: behind a branch each of them waits for the one before.
+  if (host_row != ~0ull) rowp = host + host_row * vpr;
   MixRow r;
+  r.host_row = host_row;
   r.has_row = rowp != nullptr;
   r.bits = r.has_row ? reinterpret_cast<uint64_t>(rowp) : reinterpret_cast<uint64_t>(out);
   r.from_cache = r.has_row && f.hit && f.loc == UGK_LOC_LOCAL;
@@ -193,8 +197,9 @@ __device__ __forceinline__ MixRow mix_resolve(const ugk_table_t &t, uint64_t key
 }
 
 // the rows of one wavefront's KPW keys, lane l holding the address of key b0 + l's row
-template <int LPR, int KPW, bool NT_STORE>
-__device__ __forceinline__ void mix_copy(const MixRow &row, u32x4 *out, size_t b0, uint32_t vpr) {
+// stage_bits (STAGE only): where the lane's row is filed as well, 0 for a row that is not
+template <int LPR, int KPW, bool NT_STORE, bool STAGE>
+__device__ __forceinline__ void mix_copy(const MixRow &row, uint64_t stage_bits, u32x4 *out, size_t b0, uint32_t vpr) {
   constexpr int RPW = kWave / LPR;  // rows per wavefront instruction
   constexpr int UNROLL = (RPW * 4 <= KPW) ? 4 : (KPW / RPW);
   static_assert(KPW <= kWave && KPW % (RPW * UNROLL) == 0, "keys per wavefront must be whole rounds of rows");
@@ -204,11 +209,13 @@ __device__ __forceinline__ void mix_copy(const MixRow &row, u32x4 *out, size_t b
     // the row addresses travel between lanes as integers; turned back into pointers they must be told to be global
     // memory again, or the loads become generic ones, which the hardware cannot keep several of in flight in order
     grow_t p[UNROLL];
+    gout_t ps[UNROLL];
     bool ok[UNROLL];
 #pragma unroll
     for (int u = 0; u < UNROLL; ++u) {
       p[u] = reinterpret_cast<grow_t>(shfl64(row.bits, r0 + u * RPW + rg));
       ok[u] = __shfl((int)row.has_row, r0 + u * RPW + rg) != 0;
+      if constexpr (STAGE) ps[u] = reinterpret_cast<gout_t>(shfl64(stage_bits, r0 + u * RPW + rg));
     }
     for (uint32_t c0 = 0; c0 < vpr; c0 += LPR) {
       const uint32_t col = c0 + sub;
@@ -224,6 +231,11 @@ __device__ __forceinline__ void mix_copy(const MixRow &row, u32x4 *out, size_t b
             if constexpr (NT_STORE) __builtin_nontemporal_store(v[u], dst);
             else *dst = v[u];
           }
+        if constexpr (STAGE) {
+#pragma unroll
+          for (int u = 0; u < UNROLL; ++u)
+            if (ps[u]) ps[u][col] = v[u];
+        }
       }
     }
   }
@@ -245,13 +257,30 @@ __device__ __forceinline__ void mix_leave_counts(uint32_t *block_tot, uint32_t w
   if (threadIdx.x == 0) counts[blockIdx.x] = ((unsigned long long)block_tot[1] << 32) | block_tot[0];
 }
 
-template <typename K, int KIND, int LPR, int KPW, bool NT_STORE>
+// A row taken from the host table is also filed in the stage (ugk_stage_t): entry h = fmix64(row) & mask.  The first
+// wavefront of a launch that finds the entry not yet written by this launch, and not holding this very row already,
+// claims it with one compare-and-swap on its owner word and writes the row's bytes next to its stores into the output;
+// everybody else leaves it alone.  After the launch an owner word names the row whose bytes the entry holds.
+__device__ __forceinline__ uint64_t stage_claim(const ugk_stage_t &stage, const MixRow &row, uint32_t vpr) {
+  if (row.host_row > 0xffffffffull) return 0;
+  const uint32_t r32 = (uint32_t)row.host_row;
+  const uint64_t h = fmix64(row.host_row) & stage.mask;
+  unsigned long long *owner = reinterpret_cast<unsigned long long *>(stage.owner_dev) + h;
+  const unsigned long long cur = __atomic_load_n(owner, __ATOMIC_RELAXED);
+  const uint32_t tag = (uint32_t)(cur >> 32);
+  if (tag == stage.epoch || (tag != 0 && (uint32_t)cur == r32)) return 0;
+  const unsigned long long want = ((unsigned long long)stage.epoch << 32) | r32;
+  if (atomicCAS(owner, cur, want) != cur) return 0;
+  return reinterpret_cast<uint64_t>(reinterpret_cast<u32x4 *>(stage.rows_dev) + h * vpr);
+}
+
+template <typename K, int KIND, int LPR, int KPW, bool NT_STORE, bool STAGE>
 __global__ __launch_bounds__(kBlock) void extract_mix_kernel(ugk_table_t t, const K *__restrict__ keys, size_t n,
                                                              const u32x4 *__restrict__ cache, uint64_t cache_rows,
                                                              const u32x4 *__restrict__ host, uint64_t host_rows,
                                                              u32x4 *__restrict__ out, uint32_t vpr,
                                                              uint32_t *status, uint32_t *host_mirror,
-                                                             unsigned long long *counts) {
+                                                             unsigned long long *counts, ugk_stage_t stage) {
   __shared__ uint32_t block_tot[2];
   if (threadIdx.x < 2) block_tot[threadIdx.x] = 0;
   __syncthreads();
@@ -272,7 +301,9 @@ __global__ __launch_bounds__(kBlock) void extract_mix_kernel(ugk_table_t t, cons
       wave_local += __popcll(__ballot(row.from_cache));
       wave_host += __popcll(__ballot(active && !row.from_cache));
     }
-    mix_copy<LPR, KPW, NT_STORE>(row, out, b0, vpr);
+    uint64_t stage_bits = 0;
+    if constexpr (STAGE) stage_bits = stage_claim(stage, row, vpr);
+    mix_copy<LPR, KPW, NT_STORE, STAGE>(row, stage_bits, out, b0, vpr);
   }
   if (counts) mix_leave_counts(block_tot, wave_local, wave_host, counts);
 }
@@ -504,7 +535,8 @@ int select_keys(const K *keys, const uint32_t *sel, size_t m, K *out, void *stre
 template <typename K, int KIND>
 int extract_mix_lpr(ugk_table_t t, const K *keys, size_t n, const void *cache, uint64_t cache_rows, const void *host,
                     uint64_t host_rows, void *out, uint32_t vpr, uint32_t *status, uint32_t *host_mirror,
-                    uint64_t *counts, uint32_t *num_groups, uint32_t others_hint, hipStream_t st) {
+                    uint64_t *counts, uint32_t *num_groups, uint32_t others_hint, const ugk_stage_t *stage,
+                    hipStream_t st) {
   // ordinary write-back stores while the output fits the memory-side cache (the consumer finds it there),
   // non-temporal beyond, or as the caller's hint says
   const bool nt = nt_store_for(n * (size_t)vpr * 16);
@@ -553,10 +585,16 @@ int extract_mix_lpr(ugk_table_t t, const K *keys, size_t n, const void *cache, u
   const size_t keys_per_group = (size_t)kpw * kWavesPerBlock;
   const unsigned grid = clamp_grid((n + keys_per_group - 1) / keys_per_group, mostly_host ? 128u : 0u);
   if (num_groups) *num_groups = grid;
-#define UGK_GO3(L, W, NT)                                                                                          \
-  hipLaunchKernelGGL((extract_mix_kernel<K, KIND, L, W, NT>), dim3(grid), dim3(kBlock), 0, st, t, keys, n,        \
-                     (const u32x4 *)cache, cache_rows, (const u32x4 *)host, host_rows, (u32x4 *)out, vpr, status, \
-                     host_mirror, reinterpret_cast<unsigned long long *>(counts))
+  const ugk_stage_t no_stage{};
+#define UGK_GO4(L, W, NT, ST)                                                                                       \
+  hipLaunchKernelGGL((extract_mix_kernel<K, KIND, L, W, NT, ST>), dim3(grid), dim3(kBlock), 0, st, t, keys, n,     \
+                     (const u32x4 *)cache, cache_rows, (const u32x4 *)host, host_rows, (u32x4 *)out, vpr, status,  \
+                     host_mirror, reinterpret_cast<unsigned long long *>(counts), ST ? *stage : no_stage)
+#define UGK_GO3(L, W, NT)               \
+  do {                                  \
+    if (stage) UGK_GO4(L, W, NT, true); \
+    else UGK_GO4(L, W, NT, false);      \
+  } while (0)
 #define UGK_GO2(L, W)         \
   do {                        \
     if (nt) UGK_GO3(L, W, true); \
@@ -594,6 +632,7 @@ int extract_mix_lpr(ugk_table_t t, const K *keys, size_t n, const void *cache, u
 #undef UGK_GO
 #undef UGK_GO2
 #undef UGK_GO3
+#undef UGK_GO4
   UGK_HIP(hipGetLastError());
   return 0;
 }
@@ -601,7 +640,7 @@ int extract_mix_lpr(ugk_table_t t, const K *keys, size_t n, const void *cache, u
 template <typename K>
 int extract_mix(ugk_table_t t, const K *keys, size_t n, const void *cache, uint64_t cache_rows, const void *host,
                 uint64_t host_rows, void *out, size_t row_bytes, uint32_t *status, uint32_t *host_mirror,
-                uint64_t *counts, uint32_t *num_groups, uint32_t others_hint, void *stream) {
+                uint64_t *counts, uint32_t *num_groups, uint32_t others_hint, const ugk_stage_t *stage, void *stream) {
   if (num_groups) *num_groups = 0;
   if (n == 0) return 0;
   UGK_REQUIRE(keys && out && status, "ugk_extract_mix: null keys, output or status");
@@ -619,11 +658,18 @@ int extract_mix(ugk_table_t t, const K *keys, size_t n, const void *cache, uint6
   UGK_REQUIRE(row_bytes > 0 && align % 16 == 0,
               "ugk_extract_mix: rows and buffers must be multiples of 16 bytes (row_bytes=%zu)", row_bytes);
   const uint32_t vpr = (uint32_t)(row_bytes / 16);
+  if (stage) {
+    UGK_REQUIRE(stage->rows_dev && stage->owner_dev, "ugk_extract_mix_staged: null stage");
+    UGK_REQUIRE(((stage->mask + 1) & stage->mask) == 0, "ugk_extract_mix_staged: the stage needs a power of two of entries");
+    UGK_REQUIRE(stage->epoch != 0, "ugk_extract_mix_staged: the launch tag must be non-zero");
+    UGK_REQUIRE((uintptr_t)stage->rows_dev % 16 == 0 && (uintptr_t)stage->owner_dev % 8 == 0,
+                "ugk_extract_mix_staged: misaligned stage");
+  }
   if (t.kind == 1)
     return extract_mix_lpr<K, 1>(t, keys, n, cache, cache_rows, host, host_rows, out, vpr, status, host_mirror,
-                                 counts, num_groups, others_hint, as_stream(stream));
+                                 counts, num_groups, others_hint, stage, as_stream(stream));
   return extract_mix_lpr<K, 2>(t, keys, n, cache, cache_rows, host, host_rows, out, vpr, status, host_mirror,
-                               counts, num_groups, others_hint, as_stream(stream));
+                               counts, num_groups, others_hint, stage, as_stream(stream));
 }
 
 // The workspace is laid out by its own size, not by the batch's: `cap` slot words, then cap / 2 words of unique ids by
@@ -708,14 +754,34 @@ int ugk_extract_mix_u32(ugk_table_t t, const uint32_t *keys_dev, size_t n, const
                         uint32_t *status_dev, uint32_t *host_mirror, uint64_t *group_counts_host,
                         uint32_t *num_groups_host, uint32_t others_hint, void *stream) {
   return extract_mix<uint32_t>(t, keys_dev, n, cache_dev, cache_rows, host_dev, host_rows, out_dev, row_bytes,
-                               status_dev, host_mirror, group_counts_host, num_groups_host, others_hint, stream);
+                               status_dev, host_mirror, group_counts_host, num_groups_host, others_hint, nullptr,
+                               stream);
 }
 int ugk_extract_mix_i64(ugk_table_t t, const int64_t *keys_dev, size_t n, const void *cache_dev, uint64_t cache_rows,
                         const void *host_dev, uint64_t host_rows, void *out_dev, size_t row_bytes,
                         uint32_t *status_dev, uint32_t *host_mirror, uint64_t *group_counts_host,
                         uint32_t *num_groups_host, uint32_t others_hint, void *stream) {
   return extract_mix<int64_t>(t, keys_dev, n, cache_dev, cache_rows, host_dev, host_rows, out_dev, row_bytes,
-                              status_dev, host_mirror, group_counts_host, num_groups_host, others_hint, stream);
+                              status_dev, host_mirror, group_counts_host, num_groups_host, others_hint, nullptr,
+                              stream);
+}
+int ugk_extract_mix_staged_u32(ugk_table_t t, const uint32_t *keys_dev, size_t n, const void *cache_dev,
+                               uint64_t cache_rows, const void *host_dev, uint64_t host_rows, void *out_dev,
+                               size_t row_bytes, uint32_t *status_dev, uint32_t *host_mirror,
+                               uint64_t *group_counts_host, uint32_t *num_groups_host, uint32_t others_hint,
+                               ugk_stage_t stage, void *stream) {
+  return extract_mix<uint32_t>(t, keys_dev, n, cache_dev, cache_rows, host_dev, host_rows, out_dev, row_bytes,
+                               status_dev, host_mirror, group_counts_host, num_groups_host, others_hint, &stage,
+                               stream);
+}
+int ugk_extract_mix_staged_i64(ugk_table_t t, const int64_t *keys_dev, size_t n, const void *cache_dev,
+                               uint64_t cache_rows, const void *host_dev, uint64_t host_rows, void *out_dev,
+                               size_t row_bytes, uint32_t *status_dev, uint32_t *host_mirror,
+                               uint64_t *group_counts_host, uint32_t *num_groups_host, uint32_t others_hint,
+                               ugk_stage_t stage, void *stream) {
+  return extract_mix<int64_t>(t, keys_dev, n, cache_dev, cache_rows, host_dev, host_rows, out_dev, row_bytes,
+                              status_dev, host_mirror, group_counts_host, num_groups_host, others_hint, &stage,
+                              stream);
 }
 
 size_t ugk_dedup_workspace_bytes(size_t n) { return dedup_capacity(n) * 10 + 64; }

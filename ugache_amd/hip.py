@@ -34,6 +34,12 @@ class Table(C.Structure):
                 ("fb_mul", C.c_uint64), ("fb_mask", C.c_uint64)]
 
 
+class Stage(C.Structure):
+    """ugk_stage_t"""
+    _fields_ = [("rows_dev", C.c_void_p), ("owner_dev", C.c_void_p), ("mask", C.c_uint64), ("epoch", C.c_uint32),
+                ("reserved", C.c_uint32)]
+
+
 class DeviceInfo(C.Structure):
     """ugk_device_info_t"""
     _fields_ = [("name", C.c_char * 256), ("arch", C.c_char * 64), ("compute_units", C.c_int32),
@@ -95,6 +101,9 @@ SIGNATURES = {
     "ugk_extract_mix_max_groups": [],
     "ugk_extract_mix_u32": [Table, _vp, _sz, _vp, _u64, _vp, _u64, _vp, _sz, _vp, _vp, _vp, _vp, _u32, _vp],
     "ugk_extract_mix_i64": [Table, _vp, _sz, _vp, _u64, _vp, _u64, _vp, _sz, _vp, _vp, _vp, _vp, _u32, _vp],
+    "ugk_extract_mix_staged_u32": [Table, _vp, _sz, _vp, _u64, _vp, _u64, _vp, _sz, _vp, _vp, _vp, _vp, _u32, Stage, _vp],
+    "ugk_extract_mix_staged_i64": [Table, _vp, _sz, _vp, _u64, _vp, _u64, _vp, _sz, _vp, _vp, _vp, _vp, _u32, Stage, _vp],
+    "ugk_gather_scatter_staged_u32": [_vp, _u64, _vp, _vp, _sz, _vp, _u64, _sz, Stage, C.c_uint, _vp, _vp, _vp],
     "ugk_dedup_workspace_bytes": [_sz],
     "ugk_dedup_u32": [_vp, _sz, _vp, _sz, _u32, _vp, _vp, _vp, _vp, _vp, _vp],
     "ugk_dedup_i64": [_vp, _sz, _vp, _sz, _u32, _vp, _vp, _vp, _vp, _vp, _vp],
