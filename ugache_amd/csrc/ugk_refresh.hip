@@ -171,7 +171,7 @@ __global__ void rank_init_kernel(RankWs *ws, unsigned long long remaining) {
 
 // bit r of gt = count[r] > T, of eq = count[r] == T.  A wavefront takes 64 consecutive rows per load, so a ballot is
 // a word.
-constexpr int kMarkWords = 8;  // words (loads in flight) per wavefront and round
+constexpr int kMarkWords = 16;  // words (loads in flight) per wavefront and round
 __global__ __launch_bounds__(kBlock) void rank_split_kernel(uint32_t *counts, uint64_t n, const RankWs *ws,
                                                             unsigned long long *gt, unsigned long long *eq,
                                                             int reset_counts) {
@@ -186,18 +186,24 @@ __global__ __launch_bounds__(kBlock) void rank_split_kernel(uint32_t *counts, ui
 #pragma unroll
     for (int k = 0; k < kMarkWords; ++k) {
       const uint64_t row = (w0 + k) * 64 + lane;
-      c[k] = row < n ? counts[row] : 0u;
+      c[k] = row < n ? __builtin_nontemporal_load(counts + row) : 0u;
     }
+    // lane k keeps word k of the round; the words leave in one store per bitmap, as one run of adjacent words
+    unsigned long long my_gt = 0, my_eq = 0;
 #pragma unroll
     for (int k = 0; k < kMarkWords; ++k) {
       const uint64_t row = (w0 + k) * 64 + lane;
       const unsigned long long above = __ballot(row < n && c[k] > t);
       const unsigned long long equal = __ballot(row < n && c[k] == t);
-      if (lane == k && w0 + k < n_words) {
-        gt[w0 + k] = above;
-        eq[w0 + k] = equal;
+      if (lane == k) {
+        my_gt = above;
+        my_eq = equal;
       }
       if (reset_counts && row < n && c[k] != 0) counts[row] = 0;
+    }
+    if (lane < kMarkWords && w0 + lane < n_words) {
+      gt[w0 + lane] = my_gt;
+      eq[w0 + lane] = my_eq;
     }
   }
 }
