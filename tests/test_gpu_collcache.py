@@ -675,10 +675,14 @@ def test_stream_ordered_lookups(pct, table_kind, kdtype, monkeypatch):
     assert a.cpu().numpy().tobytes() == b.cpu().numpy().tobytes() == ORC.gather(table, keys.astype(np.int64)).tobytes()
 
 
-@pytest.mark.parametrize("pct", [1.0, 0.25])
-def test_stream_ordered_lookup_inside_a_captured_graph(pct):
+@pytest.mark.parametrize("pct,stage", [(1.0, 0), (0.25, 0), (0.25, 4096)])
+def test_stream_ordered_lookup_inside_a_captured_graph(pct, stage, monkeypatch):
     """a stream-ordered lookup is launches only (no synchronisation, no allocation, no memset node), so a caller can
-    capture it; every replay, with eager work and synchronisations in between, must give the eager result"""
+    capture it; every replay, with eager work and synchronisations in between, must give the eager result.  With a
+    stage of missed rows the captured launch carries one launch tag for all its replays (it files rows on the first
+    one only); the refresh that follows reads the stage and the lookups after it are still exact."""
+    if stage:
+        monkeypatch.setenv("COLL_MISS_STAGE_ROWS", str(stage))
     rng = np.random.default_rng(5)
     n_item, dim, n = 20_000, 64, 8_192
     co.config(make_config(n_item, pct))
@@ -707,6 +711,15 @@ def test_stream_ordered_lookup_inside_a_captured_graph(pct):
         # eager work between the replays
         eager = co.coll_torch_lookup_key_t_val_ret(0, keys, False)
         assert eager.cpu().numpy().tobytes() == result.cpu().numpy().tobytes()
+    if stage:
+        hot = rng.integers(0, n_item // 4, size=80_000)
+        co.coll_torch_record(0, torch.from_numpy(hot).to(torch.int32))
+        co.coll_torch_refresh(0, True)
+        q = rng.integers(0, n_item, size=n)
+        keys.copy_(torch.from_numpy(q))
+        g.replay()
+        torch.cuda.synchronize()
+        assert result.cpu().numpy().tobytes() == ORC.gather(table, q.astype(np.int64)).tobytes()
 
 
 def _random_case(seed):
@@ -716,7 +729,8 @@ def _random_case(seed):
                 pct=float(r.choice([0.0, 0.01, 0.1, 0.37, 0.9, 0.999, 1.0])),
                 table_kind=str(r.choice(["FLAT", "HASH"])), impl=str(r.choice(["", "SMMaskPhase", "NONE"])),
                 i64=bool(r.integers(0, 2)), dedup=bool(r.integers(0, 4) == 0), gpu_record=bool(r.integers(0, 4) == 0),
-                zipf=float(r.choice([0.6, 1.05, 1.4])), half=bool(r.integers(0, 3) == 0))
+                zipf=float(r.choice([0.6, 1.05, 1.4])), half=bool(r.integers(0, 3) == 0),
+                stage=int(r.choice([0, 0, 1024])))
 
 
 # UGACHE_TEST_SEEDS widens the two seeded sweeps of this file for an occasional longer run
@@ -736,6 +750,8 @@ def test_random_configurations_are_exact(case, monkeypatch):
         monkeypatch.setenv("COLL_DEDUP_MIN_KEYS", "16")
     if case["gpu_record"]:
         monkeypatch.setenv("COLL_GPU_RECORD", "1")
+    if case["stage"]:
+        monkeypatch.setenv("COLL_MISS_STAGE_ROWS", str(case["stage"]))
     rng = np.random.default_rng(case["seed"])
     n_item, dim, pct = case["n_item"], case["dim"], case["pct"]
     kdtype = torch.int64 if case["i64"] else torch.int32
@@ -815,7 +831,8 @@ def _random_refresh_case(seed):
     return dict(seed=seed, n_item=int(r.integers(130, 90_000)), dim=int(r.choice([4, 16, 32, 64, 100])),
                 pct=float(r.choice([0.01, 0.1, 0.37, 0.9, 0.99])), table_kind=str(r.choice(["FLAT", "HASH"])),
                 keep=bool(r.integers(0, 2)), sparse=bool(r.integers(0, 3) == 0), zipf=float(r.choice([0.6, 1.05, 1.4])),
-                rounds=int(r.integers(2, 5)), stream_ordered=bool(r.integers(0, 3) == 0))
+                rounds=int(r.integers(2, 5)), stream_ordered=bool(r.integers(0, 3) == 0),
+                stage=int(r.choice([0, 256, 65536])))
 
 
 @pytest.mark.parametrize("case", [_random_refresh_case(i) for i in range(max(24, _SEEDS // 2))],
@@ -828,6 +845,8 @@ def test_random_sequences_of_refreshes_on_the_device(case, monkeypatch):
     monkeypatch.setenv("COLL_GPU_RECORD", "1")
     monkeypatch.setenv("COLL_GPU_REFRESH", "1")
     monkeypatch.setenv("COLL_HASH_REBUILD_FRAC", "0.02")
+    if case["stage"]:  # the refreshes of this test run in the foreground: they insert from the stage what they find there
+        monkeypatch.setenv("COLL_MISS_STAGE_ROWS", str(case["stage"]))
     if case["keep"]:
         monkeypatch.setenv("COLL_GPU_REFRESH_KEEP", "1")
     rng = np.random.default_rng(case["seed"])
