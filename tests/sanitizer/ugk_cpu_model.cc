@@ -457,6 +457,11 @@ int ugk_stream_destroy(void *stream) {
   return 0;
 }
 int ugk_stream_sync(void *) { return 0; }
+int ugk_stream_sync_ticket(void *, uint32_t *ticket_host, uint32_t value, unsigned) {
+  REQUIRE(ticket_host, "ugk_stream_sync_ticket: null ticket word");
+  *ticket_host = value;
+  return 0;
+}
 int ugk_device_sync(void) { return 0; }
 int ugk_event_create(void **event) {
   *event = new Event{std::chrono::steady_clock::now()};

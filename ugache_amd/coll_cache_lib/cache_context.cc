@@ -573,6 +573,18 @@ void ExtractSession::SumMixCounts() {
   _host_mirror[kMirGroupSizes + UGK_LOC_HOST] = (uint32_t)others;
 }
 
+// The wait of a blocking lookup.  By default a ticket written by a one-lane kernel behind the batch's kernels is polled
+// in the pinned mirror: it turns up a few microseconds before a wait for the stream returns (COLL_SPIN_WAIT=0: wait for
+// the stream, as the reference does).
+void ExtractSession::WaitForBatch(StreamHandle stream) {
+  if (RunConfig::spin_wait_us == 0) {
+    UGK_CALL(ugk_stream_sync(stream));
+    return;
+  }
+  if (++_ticket == 0) _ticket = 1;
+  UGK_CALL(ugk_stream_sync_ticket(stream, _host_mirror + kMirTicket, _ticket, RunConfig::spin_wait_us));
+}
+
 // A lookup the refresh thread must wait for: counted from before it reads the table handle until its output is complete
 // (blocking lookups) or until its kernels are enqueued on their stream (stream-ordered ones, which the refresh then
 // finds by waiting for that stream).
@@ -641,7 +653,7 @@ void ExtractSession::ExtractFeatImpl(const KeyT *nodes, size_t num_nodes, void *
     if (events) UGK_CALL(ugk_event_record(_ev_t[1], stream));
     RecordLaunch(input_nodes, num_input, keys_ready);
     if (dst_map) UGK_CALL(ugk_replicate_rows(output, rb, inverse, dst_map, num_input, stream));
-    UGK_CALL(ugk_stream_sync(stream));
+    WaitForBatch(stream);
     const double host_time = t_host.Passed();
     JoinRecordOnHost();
     CheckStatusWord(stream);
@@ -702,7 +714,7 @@ void ExtractSession::ExtractFeatImpl(const KeyT *nodes, size_t num_nodes, void *
                         _host_mirror, _mix_counts->ptr<uint64_t>(), &_mix_groups, hint, NextStage(), stream));
     if (events) UGK_CALL(ugk_event_record(_ev_t[1], stream));
     RecordLaunch(input_nodes, num_input, keys_ready);
-    UGK_CALL(ugk_stream_sync(stream));
+    WaitForBatch(stream);
     const double host_time = t_host.Passed();
     JoinRecordOnHost();
     CheckStatusWord(stream);

@@ -92,7 +92,7 @@ class ExtractSession {
   enum StateWord { kStCounts0 = 0, kStCounts1 = 2, kStStatus = 4, kStNumUnique = 5, kStDrainEntries = 6 };
   // words of the pinned host mirror the kernels write; [1] and [2] are indexed 1 + location
   enum MirrorWord { kMirError = 0, kMirGroupSizes = 1, kMirNumUnique = 3, kMirDrainCount = 4, kMirDrainMore = 5,
-                    kMirSkipCount = 6 };
+                    kMirSkipCount = 6, kMirTicket = 7 };
   std::shared_ptr<CacheContext> _cache_ctx;
   MemHandle _idx_handle;          // ugk_idx_t[n], from the caller's allocator, regrown on demand
   MemHandle _state_handle;        // device: two counter pairs + status word
@@ -151,6 +151,8 @@ class ExtractSession {
   uint32_t _mix_groups = 0;        // workgroups of the last fused launch
   bool _async_last_fused = false;  // the last stream-ordered lookup was a fused launch (its counts wait to be summed)
   void SumMixCounts();
+  uint32_t _ticket = 0;  // last ticket a blocking lookup waited for (kMirTicket)
+  void WaitForBatch(StreamHandle stream);
   // rows that crossed the host link, kept for the next refresh (COLL_MISS_STAGE_ROWS): written by the fused extraction,
   // read by a foreground refresh, which by contract runs while no lookup does
   MemHandle _stage_rows, _stage_owner;

@@ -41,6 +41,7 @@ size_t RunConfig::gpu_record_every = 1;
 bool RunConfig::gpu_refresh = false;
 bool RunConfig::gpu_refresh_keep = false;
 size_t RunConfig::miss_stage_rows = 0;
+unsigned RunConfig::spin_wait_us = 5000;
 bool RunConfig::kernel_events = false;
 bool RunConfig::dedup_keys = false;
 size_t RunConfig::dedup_min_keys = 4096;
@@ -83,6 +84,7 @@ void RunConfig::LoadConfigFromEnv() {
   gpu_refresh = false;
   gpu_refresh_keep = false;
   miss_stage_rows = 0;
+  spin_wait_us = 5000;
   kernel_events = false;
   if (GetEnv("SAMGRAPH_EMPTY_FEAT") != "" && GetEnv("SAMGRAPH_EMPTY_FEAT") != "0") {
     LOG(FATAL) << "SAMGRAPH_EMPTY_FEAT (mock host table) is not supported by this build: every key must have a "
@@ -115,6 +117,7 @@ void RunConfig::LoadConfigFromEnv() {
   if (GetEnv("COLL_GPU_RECORD") != "") gpu_record = GetEnv("COLL_GPU_RECORD") != "0";
   if (GetEnv("COLL_GPU_REFRESH") != "") gpu_refresh = GetEnv("COLL_GPU_REFRESH") != "0";
   if (GetEnv("COLL_GPU_REFRESH_KEEP") != "") gpu_refresh_keep = GetEnv("COLL_GPU_REFRESH_KEEP") != "0";
+  if (GetEnv("COLL_SPIN_WAIT") != "") spin_wait_us = (unsigned)std::stoul(GetEnv("COLL_SPIN_WAIT"));
   if (GetEnv("COLL_MISS_STAGE_ROWS") != "") miss_stage_rows = (size_t)std::stoull(GetEnv("COLL_MISS_STAGE_ROWS"));
   if (GetEnv("COLL_KERNEL_EVENTS") != "") kernel_events = GetEnv("COLL_KERNEL_EVENTS") != "0";
   if (GetEnv("COLL_GPU_RECORD_EVERY") != "")

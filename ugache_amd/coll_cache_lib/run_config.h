@@ -75,6 +75,9 @@ struct RunConfig {
   // direct-mapped set of n (rounded up to a power of two) rows in HBM, and a foreground refresh takes the rows it inserts
   // from there when it finds them instead of over the host link again
   static size_t miss_stage_rows;
+  // COLL_SPIN_WAIT=us (default 5000; 0 = off): a blocking lookup polls a ticket its last kernel is followed by, for up
+  // to this long, before it falls back to waiting for the stream
+  static unsigned spin_wait_us;
   static bool kernel_events;  // COLL_KERNEL_EVENTS: per-step kernel times from device events (1) or a host timer (0)
   static bool dedup_keys;        // COLL_DEDUP_KEYS=1: extract each distinct key of a batch once, then copy the duplicates
   static size_t dedup_min_keys;  // COLL_DEDUP_MIN_KEYS, default 4096: shorter batches skip the deduplication

@@ -2,6 +2,8 @@
 #include <cstdlib>
 #include <cstring>
 
+#include <chrono>
+
 #include "ugk_internal.h"
 
 static thread_local char g_err[1024] = "";
@@ -187,6 +189,31 @@ int ugk_stream_destroy(void *stream) {
 }
 
 int ugk_stream_sync(void *stream) {
+  UGK_HIP(hipStreamSynchronize(as_stream(stream)));
+  return 0;
+}
+
+namespace {
+__global__ void ticket_kernel(volatile uint32_t *word, uint32_t value) { *word = value; }
+}  // namespace
+
+int ugk_stream_sync_ticket(void *stream, uint32_t *ticket_host, uint32_t value, unsigned spin_us) {
+  UGK_REQUIRE(ticket_host, "ugk_stream_sync_ticket: null ticket word");
+  hipLaunchKernelGGL(ticket_kernel, dim3(1), dim3(1), 0, as_stream(stream), ticket_host, value);
+  UGK_HIP(hipGetLastError());
+  volatile uint32_t *word = ticket_host;
+  const auto t0 = std::chrono::steady_clock::now();
+  unsigned polls = 0;
+  while (*word != value) {
+    // the clock is read every 64 polls: a poll is a load of a line the device writes into, the clock a system call away
+    if ((++polls & 63u) == 0 &&
+        std::chrono::duration_cast<std::chrono::microseconds>(std::chrono::steady_clock::now() - t0).count() >=
+            (long long)spin_us)
+      break;
+  }
+  // the ticket says that everything enqueued in front of it has run: asking the runtime as well would give back the
+  // microseconds the poll saved
+  if (*word == value) return 0;
   UGK_HIP(hipStreamSynchronize(as_stream(stream)));
   return 0;
 }
