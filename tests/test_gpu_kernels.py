@@ -122,6 +122,38 @@ def test_gather_from_pinned_host_memory():
         pin.free()
 
 
+@pytest.mark.parametrize("spin_us", [0, 1, 1_000_000])
+def test_wait_on_a_ticket_behind_the_launch(spin_us):
+    """ugk_stream_sync_ticket: the ticket kernel runs behind what was enqueued, so once the call returns - having seen
+    the ticket, or having fallen back to waiting for the stream when the poll budget ran out first - the gather in
+    front of it is complete and the word holds the ticket"""
+    rng = np.random.default_rng(7)
+    table = _rand_table(rng, 20_000, 512)
+    keys = rng.integers(0, 20_000, size=300_000).astype(np.uint32)
+    d_table, d_keys = to_dev(table), to_dev(keys)
+    out = dev_bytes(len(keys) * 512, fill=0)
+    st = dev_zeros_u32(1)
+    word = PinnedArray((16,), np.uint32)
+    try:
+        word.array[...] = 0
+        stream = C.c_void_p()
+        hip.call("ugk_stream_create", C.byref(stream))
+        sync()
+        for ticket in (1, 2, 0xFFFFFFFF):
+            out.zero_()
+            sync()
+            hip.call("ugk_gather_direct_u32", ptr(d_table), 20_000, ptr(d_keys), len(keys), ptr(out), 512, 4, ptr(st), None,
+                     stream)  # 4 workgroups: a launch of a few hundred microseconds
+            hip.call("ugk_stream_sync_ticket", stream, word.ptr, ticket, spin_us)
+            assert int(word.array[0]) == ticket
+            got = out.cpu().numpy()  # a copy on another stream: complete only if the gather was
+            assert got.tobytes() == table[keys].tobytes()
+        hip.call("ugk_stream_destroy", stream)
+    finally:
+        sync()
+        word.free()
+
+
 def test_gather_full_size_all_hit_closed_form():
     """10M x 128 fp32 table resident in HBM, 262144 uniform uint32 keys (the all-hit configuration).
     table[r, c] is a closed form of (r, c), so out[i, c] can be checked without a host copy of the table."""
