@@ -128,7 +128,7 @@ void coll_cache_last_group_offset(int replica_id, uint32_t out[3]);
  * [3] row bytes, [4] key space, [5] completed lookups, [6] free cache slots, [7] lookup-table rebuilds so far */
 void coll_cache_get_info(int replica_id, uint64_t out[8]);
 /* With COLL_MISS_STAGE_ROWS=n the fused extraction also files every row it takes from the host table in a
- * direct-mapped set of n rows in HBM, and a foreground refresh takes the rows it inserts from there when it finds them
+ * direct-mapped set of n rows in HBM, and a refresh takes the rows it inserts from there when it finds them
  * (the reference copies them over the host link again, cache_context.cu:4054-4090).  Returns how many rows the refreshes
  * of replica_id have taken from that set so far (blocks on the refresh stream; call while no refresh runs). */
 uint64_t coll_cache_rows_from_stage(int replica_id);

@@ -89,7 +89,7 @@ typedef struct {
 const char *ugk_last_error(void);
 /* version of this ABI; bumped on any signature change.  ugk_abi_version() is what the loaded library was built with:
  * a caller compiled against another UGK_ABI_VERSION must not go on. */
-#define UGK_ABI_VERSION 7
+#define UGK_ABI_VERSION 8
 int ugk_abi_version(void);
 
 /* ---- runtime plumbing: Device::{AllocDataSpace,FreeDataSpace,CopyDataFromTo,StreamSync,CreateStream}
@@ -265,9 +265,13 @@ int ugk_extract_mix_i64(ugk_table_t t, const int64_t *keys_dev, size_t n, const 
  * non-zero.  ugk_extract_mix_staged_* is ugk_extract_mix_* that also files every row it takes from the host table in the
  * stage (first writer of a launch wins an entry; `epoch` must be non-zero and differ from launch to launch);
  * ugk_gather_scatter_staged_u32 is ugk_gather_scatter_u32 out of the host table that takes a row from the stage when it
- * is there, and adds the number of such rows to *staged_dev (device word, may be NULL).  Results are the same
+ * is there, and adds the number of such rows to *staged_dev (device word, may be NULL).  With rest_count_dev (device
+ * word, zero on entry; NULL = off) the rows the stage does not hold are not copied but listed, in any order, as
+ * rest_rows_dev[j] / rest_dst_off_dev[j] for j < *rest_count_dev (lists of n words each): a background refresh copies
+ * those itself, throttled, over the host link.  Results are the same
  * bytes with and without a stage: the host table does not change under a cache.  An entry is only consistent at launch
- * boundaries, so the staged gather must not run while a staging extraction runs (a foreground refresh qualifies).
+ * boundaries, so the staged gather must not read a stage that an extraction in flight writes (a caller with lookups
+ * running beside its refreshes keeps two stages and reads the one the lookups have been switched away from).
  * rows_dev: (mask + 1) x row_bytes bytes; owner_dev: mask + 1 words, zero-filled once; host rows must fit 32 bits. */
 typedef struct {
   void *rows_dev;
@@ -289,7 +293,8 @@ int ugk_extract_mix_staged_i64(ugk_table_t t, const int64_t *keys_dev, size_t n,
 int ugk_gather_scatter_staged_u32(const void *host_dev, uint64_t host_rows, const uint32_t *rows_dev,
                                   const uint32_t *dst_off_dev, size_t n, void *out_dev, uint64_t out_rows,
                                   size_t row_bytes, ugk_stage_t stage, unsigned max_blocks, uint32_t *status_dev,
-                                  uint32_t *staged_dev, void *stream);
+                                  uint32_t *staged_dev, uint32_t *rest_rows_dev, uint32_t *rest_dst_off_dev,
+                                  uint32_t *rest_count_dev, void *stream);
 
 /* ---- key dedup (the caller-side array_ops.unique of
  *      python_tf2/collcache_tf2/collcache_tf2/core/sparse_lookup_layer.py:197) ------------------------

@@ -653,7 +653,8 @@ int ugk_extract_mix_staged_i64(ugk_table_t t, const int64_t *keys, size_t n, con
 }
 int ugk_gather_scatter_staged_u32(const void *host, uint64_t host_rows, const uint32_t *rows, const uint32_t *dst,
                                   size_t n, void *out, uint64_t out_rows, size_t rb, ugk_stage_t stage, unsigned,
-                                  uint32_t *status, uint32_t *staged, void *) {
+                                  uint32_t *status, uint32_t *staged, uint32_t *rest_rows, uint32_t *rest_dst,
+                                  uint32_t *rest_count, void *) {
   if (n == 0) return 0;
   REQUIRE(host && rows && dst && out && status && stage.rows_dev && stage.owner_dev, "staged gather: null pointer");
   for (size_t i = 0; i < n; ++i) {
@@ -665,6 +666,11 @@ int ugk_gather_scatter_staged_u32(const void *host, uint64_t host_rows, const ui
     const uint64_t h = fmix64(r) & stage.mask;
     const uint64_t cur = stage.owner_dev[h];
     const bool filed = (cur >> 32) != 0 && (uint32_t)cur == (uint32_t)r;
+    if (!filed && rest_count) {
+      rest_rows[*rest_count] = (uint32_t)r;
+      rest_dst[(*rest_count)++] = dst[i];
+      continue;
+    }
     copy_row((char *)out + (size_t)dst[i] * rb, filed ? (const char *)stage.rows_dev + h * rb : (const char *)host + r * rb,
              rb);
     if (filed && staged) ++*staged;

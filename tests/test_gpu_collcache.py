@@ -486,8 +486,9 @@ def test_refresh_on_the_device_places_like_the_oracle(table_kind, foreground, ke
         cached = new_cached
         lookup(rng.integers(0, n_item, size=20_000), nid)
     from_stage = _basics.C_LIB_CTYPES.coll_cache_rows_from_stage(0)
-    # rows that come in were looked up (and missed) shortly before: a foreground refresh finds most of them filed
-    assert (from_stage > 1000) if (stage and foreground) else (from_stage == 0)
+    # rows that come in were looked up (and missed) shortly before: the refresh finds most of them filed (a background
+    # one in the stage it switched the lookups away from)
+    assert (from_stage > 1000) if stage else (from_stage == 0)
 
     # a refresh on the host in between (hotness recorded on the host joins the device-side counts) ...
     extra = perm[zipf_ranks(rng, 60_000, n_item, 1.3)]
@@ -1163,7 +1164,8 @@ def test_counting_every_third_lookup_on_the_device(impl, monkeypatch):
 
 
 @pytest.mark.parametrize("table_kind", ["FLAT", "HASH"])
-def test_lookups_stay_exact_while_the_device_refreshes_under_them(table_kind, monkeypatch):
+@pytest.mark.parametrize("stage", [0, 8192])
+def test_lookups_stay_exact_while_the_device_refreshes_under_them(table_kind, stage, monkeypatch):
     """a thread refreshes back to back on the device (background mode, hotness accumulating from the very lookups that
     run beside it) while the caller looks keys up: every output is table[keys], and when the dust settles the cache
     holds exactly its share of rows in exactly that many slots"""
@@ -1174,6 +1176,8 @@ def test_lookups_stay_exact_while_the_device_refreshes_under_them(table_kind, mo
     monkeypatch.setenv("COLL_REFRESH_SLEEP_US", "50")
     monkeypatch.setenv("COLL_REFRESH_BATCH_ROWS", "256")
     monkeypatch.setenv("COLL_HASH_REBUILD_FRAC", "0.05")
+    if stage:  # the refreshes read the stage of missed rows the lookups beside them have been switched away from
+        monkeypatch.setenv("COLL_MISS_STAGE_ROWS", str(stage))
     rng = np.random.default_rng(91)
     n_item, dim, pct = 60_000, 32, 0.15
     co.config(make_config(n_item, pct))
@@ -1207,6 +1211,7 @@ def test_lookups_stay_exact_while_the_device_refreshes_under_them(table_kind, mo
             co.coll_torch_lookup_key_t_val_ret(0, torch.zeros(0, dtype=torch.int64).cuda(), False)
             t.join(timeout=0.005)
     assert done[0] >= 3
+    assert (_basics.C_LIB_CTYPES.coll_cache_rows_from_stage(0) > 0) == bool(stage)
     info = _basics.info(0)
     assert info["cached_rows"] == int(n_item * pct) and info["cached_rows"] + info["free_slots"] == cap
     got = np.zeros(info["cached_rows"], np.uint32)

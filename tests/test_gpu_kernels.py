@@ -655,13 +655,28 @@ def test_rows_from_the_host_are_filed_in_the_stage_and_found_there(kind, rb):
         stage = hip.Stage(ptr(stage_rows), ptr(owner), entries - 1, 0, 0)
         for cap in (0, 7):
             hip.call("ugk_gather_scatter_staged_u32", pin.ptr, nkeys, ptr(d_take), ptr(d_dst), len(take), ptr(out),
-                     out_rows, rb, stage, cap, ptr(st), ptr(n_staged), None)
+                     out_rows, rb, stage, cap, ptr(st), ptr(n_staged), None, None, None, None)
         sync()
         assert status_value(st) == 0
         want = np.full((out_rows, rb), 0x11, np.uint8)
         want[dst] = host[take]
         assert to_np(out)[: out_rows * rb].tobytes() == want.tobytes()
-        assert int(to_np(n_staged, np.uint32)[0]) == 2 * int(np.isin(take, filed_rows).sum())
+        in_stage = np.isin(take, filed_rows)
+        assert int(to_np(n_staged, np.uint32)[0]) == 2 * int(in_stage.sum())
+        # with a rest list: only what the stage holds is copied, the other rows are listed with their destinations
+        out2 = dev_bytes(out_rows * rb, fill=0x11)
+        rest_rows, rest_dst, rest_n = dev_zeros_u32(len(take)), dev_zeros_u32(len(take)), dev_zeros_u32(1)
+        hip.call("ugk_gather_scatter_staged_u32", pin.ptr, nkeys, ptr(d_take), ptr(d_dst), len(take), ptr(out2),
+                 out_rows, rb, stage, 3, ptr(st), None, ptr(rest_rows), ptr(rest_dst), ptr(rest_n), None)
+        sync()
+        assert status_value(st) == 0
+        m = int(to_np(rest_n, np.uint32)[0])
+        assert m == int((~in_stage).sum())
+        got_rest = sorted(zip(to_np(rest_rows, np.uint32)[:m].tolist(), to_np(rest_dst, np.uint32)[:m].tolist()))
+        assert got_rest == sorted(zip(take[~in_stage].tolist(), dst[~in_stage].tolist()))
+        want2 = np.full((out_rows, rb), 0x11, np.uint8)
+        want2[dst[in_stage]] = host[take[in_stage]]
+        assert to_np(out2)[: out_rows * rb].tobytes() == want2.tobytes()
         words.free()
     finally:
         sync()

@@ -245,13 +245,8 @@ ExtractSession::ExtractSession(std::shared_ptr<CacheContext> cache_ctx) : _cache
       _cache_ctx->_num_total_nodes <= 0x100000000ull) {
     size_t entries = 1024;
     while (entries < RunConfig::miss_stage_rows) entries <<= 1;
-    _stage_rows = EagerGPUAlloc(dev, entries * _cache_ctx->_row_bytes);
-    _stage_owner = EagerGPUAlloc(dev, entries * sizeof(uint64_t));
-    UGK_CALL(ugk_fill_u32(_stage_owner->ptr<uint32_t>(), 0, entries * 2, nullptr));
-    UGK_CALL(ugk_stream_sync(nullptr));
-    _stage.rows_dev = _stage_rows->ptr();
-    _stage.owner_dev = _stage_owner->ptr<uint64_t>();
-    _stage.mask = entries - 1;
+    _stage_entries = entries;
+    AllocStage(0, nullptr);
   }
   if (RunConfig::gpu_record) {
     const size_t rows = _cache_ctx->_num_total_nodes;
@@ -271,6 +266,27 @@ ExtractSession::ExtractSession(std::shared_ptr<CacheContext> cache_ctx) : _cache
     UGK_CALL(ugk_event_create(&_ev_placed));
     UGK_CALL(ugk_stream_sync(nullptr));
   }
+}
+
+void ExtractSession::AllocStage(int which, StreamHandle stream) {
+  const int dev = _cache_ctx->_trainer_ctx.device_id;
+  _stage_rows[which] = EagerGPUAlloc(dev, _stage_entries * _cache_ctx->_row_bytes);
+  _stage_owner[which] = EagerGPUAlloc(dev, _stage_entries * sizeof(uint64_t));
+  UGK_CALL(ugk_fill_u32(_stage_owner[which]->ptr<uint32_t>(), 0, _stage_entries * 2, stream));
+  UGK_CALL(ugk_stream_sync(stream));
+  _stages[which].rows_dev = _stage_rows[which]->ptr();
+  _stages[which].owner_dev = _stage_owner[which]->ptr<uint64_t>();
+  _stages[which].mask = _stage_entries - 1;
+}
+
+const ugk_stage_t *ExtractSession::StageForRefresh(bool foreground, StreamHandle stream) {
+  if (_stage_entries == 0) return nullptr;
+  const int cur = _stage_active.load();
+  if (foreground) return &_stages[cur];
+  const int other = 1 - cur;
+  if (_stages[other].rows_dev == nullptr) AllocStage(other, stream);
+  _stage_active.store(other);  // lookups that start from here on file their rows in the other stage
+  return &_stages[cur];        // readable once the lookups in flight at this point have finished
 }
 
 ExtractSession::~ExtractSession() {
@@ -1018,25 +1034,46 @@ void RefreshSession::CopyRowsIntoSlots(const uint32_t *rows_dev, const uint32_t 
   CacheContext *ctx = _cache_ctx.get();
   const void *host = ctx->_device_cache_data[ctx->_cpu_location_id];
   void *cache = ctx->_device_cache_data[ctx->_local_location_id];
-  uint32_t *status = _status_handle->ptr<uint32_t>();
-  // background refresh copies in small throttled batches so that foreground lookups keep the host link
+  uint32_t *status = _status_handle->ptr<uint32_t>();  // [0] error bits, [8] rows taken from the stage, [9] rows left
+  if (stage) {
+    // Most of the rows a refresh brings in were missed by the last few lookups, which filed them in HBM.  A foreground
+    // refresh takes every row in one launch, from the stage or from the host table.  A background one takes what the
+    // stage holds in one launch (HBM to HBM, nothing for the lookups to share the link with) and is left with a short
+    // list for the throttled copy below.
+    if (foreground) {
+      UGK_CALL(ugk_gather_scatter_staged_u32(host, ctx->_num_total_nodes, rows_dev, slots_dev, num_rows, cache,
+                                             ctx->_cache_space_capacity, ctx->_row_bytes, *stage, 0, status, status + 8,
+                                             nullptr, nullptr, nullptr, copy_stream));
+      num_rows = 0;
+    } else {
+      const Context gpu_ctx = ctx->_trainer_ctx;
+      TensorPtr rest_rows = Empty1DReuse(__rest_rows, kI32, {num_rows}, gpu_ctx);
+      TensorPtr rest_slots = Empty1DReuse(__rest_slots, kI32, {num_rows}, gpu_ctx);
+      UGK_CALL(ugk_fill_u32(status + 9, 0, 1, copy_stream));
+      UGK_CALL(ugk_gather_scatter_staged_u32(host, ctx->_num_total_nodes, rows_dev, slots_dev, num_rows, cache,
+                                             ctx->_cache_space_capacity, ctx->_row_bytes, *stage,
+                                             RunConfig::refresh_limit_block, status, status + 8,
+                                             rest_rows->Ptr<uint32_t>(), rest_slots->Ptr<uint32_t>(), status + 9,
+                                             copy_stream));
+      uint32_t left = 0;
+      UGK_CALL(ugk_memcpy_async(&left, status + 9, sizeof(left), copy_stream));
+      UGK_CALL(ugk_stream_sync(copy_stream));
+      CHECK_LE((size_t)left, num_rows);
+      rows_dev = rest_rows->CPtr<uint32_t>();
+      slots_dev = rest_slots->CPtr<uint32_t>();
+      num_rows = left;
+    }
+  }
+  // background refresh copies in small throttled batches so that foreground lookups keep the host link; alone on the
+  // chip the copy still takes a capped grid: rows of 512 bytes and more cross the link faster from 128 workgroups than
+  // from as many as the rows would fill (56.9 against 52.7 GB/s)
   const size_t batch = foreground ? num_rows : std::max<size_t>(RunConfig::refresh_batch_rows, 1);
-  // alone on the chip the copy still takes a capped grid: rows of 512 bytes and more cross the link faster from 128
-  // workgroups than from as many as the rows would fill (56.9 against 52.7 GB/s)
   const unsigned limit_block = foreground ? 128 : RunConfig::refresh_limit_block;
   for (size_t begin = 0; begin < num_rows; begin += batch) {
     const size_t cur = std::min(batch, num_rows - begin);
-    if (stage) {
-      // most of the rows a refresh brings in were missed by the last few lookups, which filed them in HBM (status word 8
-      // counts the rows found there)
-      UGK_CALL(ugk_gather_scatter_staged_u32(host, ctx->_num_total_nodes, rows_dev + begin, slots_dev + begin, cur,
-                                             cache, ctx->_cache_space_capacity, ctx->_row_bytes, *stage, 0, status,
-                                             status + 8, copy_stream));
-    } else {
-      UGK_CALL(ugk_gather_scatter_u32(host, ctx->_num_total_nodes, rows_dev + begin, slots_dev + begin, cur, cache,
-                                      ctx->_cache_space_capacity, ctx->_row_bytes, limit_block, status, nullptr,
-                                      copy_stream));
-    }
+    UGK_CALL(ugk_gather_scatter_u32(host, ctx->_num_total_nodes, rows_dev + begin, slots_dev + begin, cur, cache,
+                                    ctx->_cache_space_capacity, ctx->_row_bytes, limit_block, status, nullptr,
+                                    copy_stream));
     if (!foreground && begin + batch < num_rows) {
       UGK_CALL(ugk_stream_sync(copy_stream));
       usleep(RunConfig::refresh_sleep_us);
@@ -1072,6 +1109,10 @@ void RefreshSession::refresh_after_solve_new(bool foreground) {
     UGK_CALL(ugk_fill_u32(_status_handle->ptr<uint32_t>(), 0, 64, stream));
   }
 
+  // which stage of recently missed rows the row copy may read (a background refresh switches the lookups to the other
+  // one here, long before the wait for the lookups in flight that precedes the copy)
+  const ugk_stage_t *stage = nullptr;
+  if (auto s0 = coll_cache->session(ctx->_local_location_id)) stage = s0->StageForRefresh(foreground, stream);
   table->EnsureHostLists(ctx->_eager_gpu_mem_allocator, gpu_ctx, stream);  // after a refresh on the device
   // Step 1: key list of the new placement
   Timer t_phase;
@@ -1134,7 +1175,7 @@ void RefreshSession::refresh_after_solve_new(bool foreground) {
     auto reserved_offset =
         CopyTo1DReuse(__offs_buffer, table->ReserveOffsetFront((IdType)num_insert), gpu_ctx, low_pri_stream);
     CopyRowsIntoSlots(insert_keys_gpu->CPtr<uint32_t>(), reserved_offset->CPtr<uint32_t>(), num_insert, foreground,
-                      low_pri_stream, foreground && session ? session->Stage() : nullptr);
+                      low_pri_stream, stage);
     auto insert_table_keys =
         RunConfig::key_map_mul == 0
             ? insert_keys_gpu
@@ -1177,6 +1218,7 @@ void RefreshSession::refresh_on_device(ExtractSession *session, size_t num_cache
     _status_handle = EagerGPUAlloc(gpu_ctx.device_id, 256);
     UGK_CALL(ugk_fill_u32(_status_handle->ptr<uint32_t>(), 0, 64, stream));
   }
+  const ugk_stage_t *stage = session->StageForRefresh(foreground, stream);  // see refresh_after_solve_new
   Timer t_phase;
   table->EnsureDeviceLists(alloc, gpu_ctx, stream);
   const double sync_s = t_phase.Passed();
@@ -1234,12 +1276,11 @@ void RefreshSession::refresh_on_device(ExtractSession *session, size_t num_cache
         table->EmitBits(table->SlotUsedBits(), nullptr, true, capacity, 0, num_insert, __free_slots, alloc, gpu_ctx, stream);
     if (foreground) {
       // nothing runs beside a foreground refresh: the copy goes on the refresh's own stream, behind the lists it reads
-      CopyRowsIntoSlots(insert_rows->CPtr<uint32_t>(), slots->CPtr<uint32_t>(), num_insert, true, stream,
-                        session->Stage());
+      CopyRowsIntoSlots(insert_rows->CPtr<uint32_t>(), slots->CPtr<uint32_t>(), num_insert, true, stream, stage);
     } else {
       UGK_CALL(ugk_stream_sync(stream));  // the lists are read on the copy stream next
       CopyRowsIntoSlots(insert_rows->CPtr<uint32_t>(), slots->CPtr<uint32_t>(), num_insert, false, low_pri_stream,
-                        nullptr);
+                        stage);
     }
     UGK_CALL(ugk_bitmap_update(table->SlotUsedBits(), capacity, slots->CPtr<uint32_t>(), num_insert, 1,
                                _status_handle->ptr<uint32_t>(), stream));

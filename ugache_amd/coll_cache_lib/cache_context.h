@@ -153,16 +153,26 @@ class ExtractSession {
   void SumMixCounts();
   uint32_t _ticket = 0;  // last ticket a blocking lookup waited for (kMirTicket)
   void WaitForBatch(StreamHandle stream);
-  // rows that crossed the host link, kept for the next refresh (COLL_MISS_STAGE_ROWS): written by the fused extraction,
-  // read by a foreground refresh, which by contract runs while no lookup does
-  MemHandle _stage_rows, _stage_owner;
-  ugk_stage_t _stage = {nullptr, nullptr, 0, 0, 0};
+  // Rows that crossed the host link, kept for the next refresh (COLL_MISS_STAGE_ROWS): written by the fused extraction,
+  // read by the refresh's row copy.  A foreground refresh runs while no lookup does and reads the stage the lookups
+  // write.  A background refresh runs beside lookups, so there are two stages then: it switches the lookups over to
+  // the other one, waits (as it does anyway before it reuses slots) for the lookups that may still write the one it
+  // keeps, and reads that.  The second stage is allocated by the first background refresh.
+  MemHandle _stage_rows[2], _stage_owner[2];
+  ugk_stage_t _stages[2] = {{nullptr, nullptr, 0, 0, 0}, {nullptr, nullptr, 0, 0, 0}};
+  ugk_stage_t _stage_launch = {nullptr, nullptr, 0, 0, 0};  // what a launch is handed: the active stage with a fresh tag
+  std::atomic<int> _stage_active{0};
+  size_t _stage_entries = 0;  // 0: no stage
   uint32_t _stage_epoch = 0;
-  const ugk_stage_t *NextStage() {  // the stage with a fresh launch tag, or null when there is none
-    if (_stage.rows_dev == nullptr) return nullptr;
+  void AllocStage(int which, StreamHandle stream);
+  // Called after the lookup has counted itself in flight (InFlight): a refresh that switched the stages before it
+  // sampled that count then either sees this lookup in the count or this lookup sees the switch.
+  const ugk_stage_t *NextStage() {
+    if (_stage_entries == 0) return nullptr;
+    _stage_launch = _stages[_stage_active.load()];
     if (++_stage_epoch == 0) _stage_epoch = 1;
-    _stage.epoch = _stage_epoch;
-    return &_stage;
+    _stage_launch.epoch = _stage_epoch;
+    return &_stage_launch;
   }
   size_t _async_pending = 0;       // stream-ordered lookups enqueued since the last Wait()
   size_t _async_last_nodes = 0;    // size of the last of them
@@ -246,7 +256,7 @@ class ExtractSession {
   // reset_counts: the next interval starts from zero, as after DrainHotness.
   bool CountsOnDevice() const { return _hot_counts != nullptr; }
   // what a foreground refresh may read rows from besides the host table (null: nothing)
-  const ugk_stage_t *Stage() const { return _stage.rows_dev ? &_stage : nullptr; }
+  const ugk_stage_t *StageForRefresh(bool foreground, StreamHandle stream);
   void PlaceOnDevice(size_t num_cached, uint64_t *in_new_bits, uint64_t *scratch_bits, void *rank_ws,
                      bool reset_counts, StreamHandle stream);
   // the device-side counting of the following lookups covers only the first `num_keys` keys of a batch
@@ -273,6 +283,7 @@ class RefreshSession {
   // step 5: lets one more lookup finish, so that no gather in flight still reads a slot about to be reused
   void WaitForOneLookup(ExtractSession *session, bool foreground);
   uint32_t _rows_from_stage = 0;  // what status word 8 read after the last refresh on the device
+  TensorPtr __rest_rows, __rest_slots;  // rows a background refresh did not find in the stage
  public:
   // rows the refreshes of this session have taken from the stage instead of the host table so far (blocks)
   uint64_t RowsFromStage();

@@ -155,7 +155,8 @@ __global__ __launch_bounds__(kBlock) void gather_staged_kernel(const u32x4 *__re
                                                                const uint32_t *__restrict__ dst, size_t n,
                                                                u32x4 *__restrict__ out, uint64_t out_rows, uint32_t vpr,
                                                                uint32_t lpr, ugk_stage_t stage, uint32_t *status,
-                                                               uint32_t *staged) {
+                                                               uint32_t *staged, uint32_t *rest_rows,
+                                                               uint32_t *rest_dst, uint32_t *rest_count) {
   constexpr int UNROLL = 2;
   __shared__ uint32_t block_staged;
   if (threadIdx.x == 0) block_staged = 0;
@@ -181,6 +182,15 @@ __global__ __launch_bounds__(kBlock) void gather_staged_kernel(const u32x4 *__re
       const uint64_t h = fmix64(s) & stage.mask;
       const unsigned long long cur = stage.owner_dev[h];
       const bool filed = ok[u] && (cur >> 32) != 0 && (uint32_t)cur == (uint32_t)s;
+      if (rest_count && ok[u] && !filed) {
+        // left for the caller's own (throttled) copy over the host link: listed, not copied
+        if (lane == 0) {
+          const uint32_t at = atomicAdd(rest_count, 1u);
+          rest_rows[at] = (uint32_t)s;
+          rest_dst[at] = (uint32_t)d[u];
+        }
+        ok[u] = false;
+      }
       src[u] = !ok[u] ? reinterpret_cast<const u32x4 *>(out) : filed ? stage_rows + h * vpr : host + s * vpr;
       if (filed && lane == 0) ++mine;
     }
@@ -357,8 +367,11 @@ int ugk_gather_scatter_i64(const void *src_dev, uint64_t src_rows, const int64_t
 int ugk_gather_scatter_staged_u32(const void *host_dev, uint64_t host_rows, const uint32_t *rows_dev,
                                   const uint32_t *dst_off_dev, size_t n, void *out_dev, uint64_t out_rows,
                                   size_t row_bytes, ugk_stage_t stage, unsigned max_blocks, uint32_t *status_dev,
-                                  uint32_t *staged_dev, void *stream) {
+                                  uint32_t *staged_dev, uint32_t *rest_rows_dev, uint32_t *rest_dst_dev,
+                                  uint32_t *rest_count_dev, void *stream) {
   if (n == 0) return 0;
+  UGK_REQUIRE(rest_count_dev == nullptr || (rest_rows_dev && rest_dst_dev),
+              "ugk_gather_scatter_staged_u32: a rest count without the two rest lists");
   UGK_REQUIRE(host_dev && rows_dev && dst_off_dev && out_dev && status_dev, "ugk_gather_scatter_staged_u32: null pointer");
   UGK_REQUIRE(stage.rows_dev && stage.owner_dev && ((stage.mask + 1) & stage.mask) == 0,
               "ugk_gather_scatter_staged_u32: the stage needs buffers and a power of two of entries");
@@ -373,7 +386,8 @@ int ugk_gather_scatter_staged_u32(const void *host_dev, uint64_t host_rows, cons
   const unsigned grid = clamp_grid((n + per_iter - 1) / per_iter, max_blocks);
   hipLaunchKernelGGL(gather_staged_kernel, dim3(grid), dim3(kBlock), 0, as_stream(stream),
                      reinterpret_cast<const u32x4 *>(host_dev), host_rows, rows_dev, dst_off_dev, n,
-                     reinterpret_cast<u32x4 *>(out_dev), out_rows, vpr, lpr, stage, status_dev, staged_dev);
+                     reinterpret_cast<u32x4 *>(out_dev), out_rows, vpr, lpr, stage, status_dev, staged_dev,
+                     rest_rows_dev, rest_dst_dev, rest_count_dev);
   UGK_HIP(hipGetLastError());
   return 0;
 }
