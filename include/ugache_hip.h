@@ -89,7 +89,7 @@ typedef struct {
 const char *ugk_last_error(void);
 /* version of this ABI; bumped on any signature change.  ugk_abi_version() is what the loaded library was built with:
  * a caller compiled against another UGK_ABI_VERSION must not go on. */
-#define UGK_ABI_VERSION 8
+#define UGK_ABI_VERSION 9
 int ugk_abi_version(void);
 
 /* ---- runtime plumbing: Device::{AllocDataSpace,FreeDataSpace,CopyDataFromTo,StreamSync,CreateStream}
@@ -194,6 +194,13 @@ int ugk_table_insert_i64(ugk_table_t t, const int64_t *keys_dev, const uint32_t 
 /* evict_hashmap_unique (cache_hashtable.cu:269-308) */
 int ugk_table_evict_u32(ugk_table_t t, const uint32_t *keys_dev, size_t n, uint32_t *status_dev, void *stream);
 int ugk_table_evict_i64(ugk_table_t t, const int64_t *keys_dev, size_t n, uint32_t *status_dev, void *stream);
+/* the same, and the bit of the cache slot every evicted key held is cleared in slot_bits_dev (one bit per slot, nslots
+ * bits): what LookupOffset + ReturnOffset + Evict do to the free list (cache_context.cu:4005-4020), in the one kernel that
+ * has the bucket in its hands anyway */
+int ugk_table_evict_release_u32(ugk_table_t t, const uint32_t *keys_dev, size_t n, uint64_t *slot_bits_dev,
+                                uint64_t nslots, uint32_t *status_dev, void *stream);
+int ugk_table_evict_release_i64(ugk_table_t t, const int64_t *keys_dev, size_t n, uint64_t *slot_bits_dev,
+                                uint64_t nslots, uint32_t *status_dev, void *stream);
 /* LookupValCustom with SepLocOffset (cache_hashtable.cuh:420-434): loc_out/off_out per key; a miss gives
  * (fallback_loc, (uint32)key).  Either output may be NULL (OffsetOnly, cuh:396-407). */
 int ugk_table_lookup_u32(ugk_table_t t, const uint32_t *keys_dev, size_t n, uint32_t fallback_loc,
@@ -386,6 +393,11 @@ int ugk_bitmap_emit(const uint64_t *a_dev, const uint64_t *b_dev, int invert_a, 
 /* sets (set != 0) or clears the bits listed in idx_dev; a position >= nbits flags UGK_ST_KEY_OUT_OF_RANGE */
 int ugk_bitmap_update(uint64_t *bitmap_dev, uint64_t nbits, const uint32_t *idx_dev, size_t n, int set,
                       uint32_t *status_dev, void *stream);
+/* sets every bit up to and including position *last_pos_dev (device word): after the lowest free slots have been taken,
+ * the last of them being *last_pos_dev, that is what ReserveOffsetFront (cache_hashtable.cuh:647-655) did to the slot
+ * bitmap; a position >= nbits flags UGK_ST_KEY_OUT_OF_RANGE and changes nothing */
+int ugk_bitmap_set_through(uint64_t *bitmap_dev, uint64_t nbits, const uint32_t *last_pos_dev, uint32_t *status_dev,
+                           void *stream);
 /* sparse-id mode: caller-side id of each listed host row, (row * mul) & mask (the inverse of the map ugk_table_t
  * carries in fb_mul / fb_mask) */
 int ugk_rows_to_keys(const uint32_t *rows_dev, size_t n, uint64_t mul, uint64_t mask, int64_t *keys_out_dev,

@@ -214,7 +214,13 @@ int table_insert(ugk_table_t t, const K *keys, const uint32_t *offs, uint32_t se
 }
 
 template <typename K>
-int table_evict(ugk_table_t t, const K *keys, size_t n, uint32_t *status) {
+int table_evict(ugk_table_t t, const K *keys, size_t n, uint32_t *status, uint64_t *slot_bits = nullptr,
+                uint64_t nslots = 0) {
+  auto release = [&](uint32_t slot) {
+    if (!slot_bits) return;
+    if (slot >= nslots) or_status(status, UGK_ST_KEY_OUT_OF_RANGE);
+    else __atomic_fetch_and(slot_bits + (slot >> 6), ~(1ull << (slot & 63)), __ATOMIC_RELAXED);
+  };
   if (n == 0) return 0;
   if (check_table(t, "ugk_table_evict")) return 1;
   REQUIRE(keys && status, "ugk_table_evict: null pointer");
@@ -228,6 +234,7 @@ int table_evict(ugk_table_t t, const K *keys, size_t n, uint32_t *status) {
       const uint32_t old =
           __atomic_exchange_n(reinterpret_cast<uint32_t *>(t.table) + key, UGK_EMPTY_U32, __ATOMIC_ACQ_REL);
       if (old == UGK_EMPTY_U32) or_status(status, UGK_ST_EVICT_ABSENT);
+      else release(old & 0x0fffffffu);
       continue;
     }
     ugk_bucket_t *b = reinterpret_cast<ugk_bucket_t *>(t.table);
@@ -236,6 +243,7 @@ int table_evict(ugk_table_t t, const K *keys, size_t n, uint32_t *status) {
     for (uint64_t step = 0; step < t.size && !done && key < UGK_HASH_TOMB; ++step) {
       const uint64_t cur = ld(&b[pos].key);
       if (cur == key) {
+        release((uint32_t)ld(reinterpret_cast<const uint64_t *>(&b[pos].off)));
         st(reinterpret_cast<uint64_t *>(&b[pos].off), (uint64_t)0);
         st(&b[pos].key, (uint64_t)UGK_HASH_TOMB);
         done = true;
@@ -575,6 +583,16 @@ int ugk_table_evict_u32(ugk_table_t t, const uint32_t *keys, size_t n, uint32_t 
 int ugk_table_evict_i64(ugk_table_t t, const int64_t *keys, size_t n, uint32_t *status, void *) {
   return table_evict(t, keys, n, status);
 }
+int ugk_table_evict_release_u32(ugk_table_t t, const uint32_t *keys, size_t n, uint64_t *slot_bits, uint64_t nslots,
+                                uint32_t *status, void *) {
+  REQUIRE(n == 0 || slot_bits, "ugk_table_evict_release_u32: null slot bitmap");
+  return table_evict(t, keys, n, status, slot_bits, nslots);
+}
+int ugk_table_evict_release_i64(ugk_table_t t, const int64_t *keys, size_t n, uint64_t *slot_bits, uint64_t nslots,
+                                uint32_t *status, void *) {
+  REQUIRE(n == 0 || slot_bits, "ugk_table_evict_release_i64: null slot bitmap");
+  return table_evict(t, keys, n, status, slot_bits, nslots);
+}
 int ugk_table_lookup_u32(ugk_table_t t, const uint32_t *keys, size_t n, uint32_t fallback_loc, uint32_t *loc_out,
                          uint32_t *off_out, void *) {
   return table_lookup(t, keys, n, fallback_loc, loc_out, off_out);
@@ -803,6 +821,15 @@ int ugk_bitmap_update(uint64_t *bitmap, uint64_t nbits, const uint32_t *idx, siz
     if (set) __atomic_fetch_or(bitmap + (p >> 6), 1ull << (p & 63), __ATOMIC_RELAXED);
     else __atomic_fetch_and(bitmap + (p >> 6), ~(1ull << (p & 63)), __ATOMIC_RELAXED);
   }
+  return 0;
+}
+int ugk_bitmap_set_through(uint64_t *bitmap, uint64_t nbits, const uint32_t *last_pos, uint32_t *status, void *) {
+  REQUIRE(bitmap && last_pos && status && nbits, "ugk_bitmap_set_through: bad argument");
+  if (*last_pos >= nbits) {
+    or_status(status, UGK_ST_KEY_OUT_OF_RANGE);
+    return 0;
+  }
+  for (uint64_t p = 0; p <= *last_pos; ++p) __atomic_fetch_or(bitmap + (p >> 6), 1ull << (p & 63), __ATOMIC_RELAXED);
   return 0;
 }
 int ugk_rows_to_keys(const uint32_t *rows, size_t n, uint64_t mul, uint64_t mask, int64_t *keys_out, void *) {

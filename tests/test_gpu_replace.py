@@ -204,3 +204,79 @@ def test_rows_to_keys_is_the_forward_id_map():
     sync()
     want = np.array([(int(r) * mul) & ((1 << bits) - 1) for r in rows], np.int64)
     assert np.array_equal(to_np(out, np.int64)[: len(rows)], want)
+
+
+@pytest.mark.parametrize("nbits", [1, 63, 64, 65, 1000, 100_003])
+def test_bitmap_set_through_fills_the_low_bits(nbits):
+    """ugk_bitmap_set_through: every bit up to and including the position read from the device is set, bits above it
+    are left as they were; a position outside the bitmap is refused and changes nothing"""
+    rng = np.random.default_rng(nbits)
+    words = (nbits + 63) // 64
+    st = dev_zeros_u32(1)
+    for last in sorted({0, nbits // 2, nbits - 1}):
+        bits = rng.integers(0, 2, size=words * 64).astype(bool)
+        bm = to_dev(np.packbits(bits, bitorder="little").view(np.uint64))
+        pos = to_dev(np.array([7, last, 9], np.uint32))
+        hip.call("ugk_bitmap_set_through", ptr(bm), nbits, ptr(pos) + 4, ptr(st), None)
+        assert status_value(st) == 0
+        want = bits.copy()
+        want[: last + 1] = True
+        got = np.unpackbits(to_np(bm, np.uint64)[:words].view(np.uint8), bitorder="little").astype(bool)
+        assert np.array_equal(got, want), (nbits, last)
+    bm = to_dev(np.zeros(words, np.uint64))
+    pos = to_dev(np.array([nbits], np.uint32))
+    hip.call("ugk_bitmap_set_through", ptr(bm), nbits, ptr(pos), ptr(st), None)
+    assert status_value(st) & hip.ST_KEY_OUT_OF_RANGE
+    assert not to_np(bm, np.uint64)[:words].any()
+
+
+@pytest.mark.parametrize("kind", ["flat", "hash"])
+@pytest.mark.parametrize("kdtype", [np.uint32, np.int64])
+def test_evict_that_releases_the_slots(kind, kdtype):
+    """ugk_table_evict_release_*: the keys leave the table exactly as with ugk_table_evict_*, and the bit of the slot
+    each of them held is cleared in the slot bitmap; the bits of the keys that stay are untouched; an absent key is
+    flagged and releases nothing"""
+    rng = np.random.default_rng(5)
+    nkeys, n, nslots = 50_000, 20_000, 30_000
+    keys = rng.choice(nkeys, n, replace=False).astype(kdtype)
+    slots = rng.choice(nslots, n, replace=False).astype(np.uint32)
+    if kind == "flat":
+        mem = dev_zeros_u32(nkeys)
+        hip.call("ugk_fill_u32", ptr(mem), hip.EMPTY_U32, nkeys, None)
+        tb = hip.table(hip.TABLE_FLAT, ptr(mem), nkeys)
+    else:
+        nb = hip.lib().ugk_hash_buckets_for(n, 0.7)
+        mem = dev_bytes(nb * 16 + 128)
+        base = (ptr(mem) + 127) // 128 * 128
+        hip.call("ugk_hash_init", base, nb, None)
+        tb = hip.table(hip.TABLE_HASH, base, nb)
+    st = dev_zeros_u32(1)
+    ins = "ugk_table_insert_i64" if kdtype == np.int64 else "ugk_table_insert_u32"
+    d_keys, d_slots = to_dev(keys), to_dev(slots)
+    hip.call(ins, tb, ptr(d_keys), ptr(d_slots), 0, 0, n, ptr(st), None)
+    assert status_value(st) == 0
+    used = np.zeros((nslots + 63) // 64 * 64, bool)
+    used[slots] = True
+    used[rng.choice(np.flatnonzero(~used[:nslots]), 500, replace=False)] = True  # slots of nobody in particular
+    bm = to_dev(np.packbits(used, bitorder="little").view(np.uint64))
+    gone = rng.choice(n, n // 3, replace=False)
+    d_gone = to_dev(keys[gone])
+    fn = "ugk_table_evict_release_i64" if kdtype == np.int64 else "ugk_table_evict_release_u32"
+    hip.call(fn, tb, ptr(d_gone), len(gone), ptr(bm), nslots, ptr(st), None)
+    assert status_value(st) == 0
+    want = used.copy()
+    want[slots[gone]] = False
+    got = np.unpackbits(to_np(bm, np.uint64)[: len(used) // 64].view(np.uint8), bitorder="little").astype(bool)
+    assert np.array_equal(got, want)
+    loc, off = dev_zeros_u32(n), dev_zeros_u32(n)
+    lk = "ugk_table_lookup_i64" if kdtype == np.int64 else "ugk_table_lookup_u32"
+    hip.call(lk, tb, ptr(d_keys), n, 9, ptr(loc), ptr(off), None)
+    stays = np.ones(n, bool)
+    stays[gone] = False
+    got_loc, got_off = to_np(loc, np.uint32)[:n], to_np(off, np.uint32)[:n]
+    assert (got_loc[stays] == 0).all() and np.array_equal(got_off[stays], slots[stays]) and (got_loc[~stays] == 9).all()
+    # evicting them again: absent, and no bit moves
+    hip.call(fn, tb, ptr(d_gone), len(gone), ptr(bm), nslots, ptr(st), None)
+    assert status_value(st) & hip.ST_EVICT_ABSENT
+    got = np.unpackbits(to_np(bm, np.uint64)[: len(used) // 64].view(np.uint8), bitorder="little").astype(bool)
+    assert np.array_equal(got, want)

@@ -1247,11 +1247,7 @@ void RefreshSession::refresh_on_device(ExtractSession *session, size_t num_cache
   // of its kernels once, at the end; a background one, which lookups run beside, after every step.
   if (num_evicted > 0) {
     TensorPtr evict_keys = table->RowsToTableKeys(evict_rows, __evict_ids, alloc, gpu_ctx, stream);
-    TensorPtr evict_slots = Empty1DReuse(__evict_slots, kI32, {num_evicted}, gpu_ctx);
-    table->LookupOffset(evict_keys, evict_slots, stream);
-    UGK_CALL(ugk_bitmap_update(table->SlotUsedBits(), capacity, evict_slots->CPtr<uint32_t>(), num_evicted, 0,
-                               _status_handle->ptr<uint32_t>(), stream));
-    table->Evict(evict_keys, stream);
+    table->EvictRelease(evict_keys, stream);  // one launch: the key leaves the table, its slot the slot bitmap
     if (!foreground) table->CheckStatus(stream, "refresh evict");
   }
   LOG(INFO) << "refresh on the device: preserved " << num_preserved_key << ", evict " << num_evicted << ", insert "
@@ -1282,8 +1278,9 @@ void RefreshSession::refresh_on_device(ExtractSession *session, size_t num_cache
       CopyRowsIntoSlots(insert_rows->CPtr<uint32_t>(), slots->CPtr<uint32_t>(), num_insert, false, low_pri_stream,
                         stage);
     }
-    UGK_CALL(ugk_bitmap_update(table->SlotUsedBits(), capacity, slots->CPtr<uint32_t>(), num_insert, 1,
-                               _status_handle->ptr<uint32_t>(), stream));
+    // the slots taken are the lowest free ones: every bit up to the last of them is set now
+    UGK_CALL(ugk_bitmap_set_through(table->SlotUsedBits(), capacity, slots->CPtr<uint32_t>() + (num_insert - 1),
+                                    _status_handle->ptr<uint32_t>(), stream));
     TensorPtr insert_keys = table->RowsToTableKeys(insert_rows, __insert_ids, alloc, gpu_ctx, stream);
     table->InsertWithLoc(insert_keys, slots, local, stream);
   }

@@ -91,6 +91,16 @@ void CacheEntryManager::Evict(TensorPtr keys_to_evict, StreamHandle stream) {
   if (_table.kind == 2) _num_tombstones += keys_to_evict->NumItem();
 }
 
+void CacheEntryManager::EvictRelease(TensorPtr keys_to_evict, StreamHandle stream) {
+  if (keys_to_evict->Type() == kI64)
+    UGK_CALL(ugk_table_evict_release_i64(_table, keys_to_evict->CPtr<int64_t>(), keys_to_evict->NumItem(),
+                                         SlotUsedBits(), _cache_space_capacity, StatusPtr(this, stream), stream));
+  else
+    UGK_CALL(ugk_table_evict_release_u32(_table, keys_to_evict->CPtr<uint32_t>(), keys_to_evict->NumItem(),
+                                         SlotUsedBits(), _cache_space_capacity, StatusPtr(this, stream), stream));
+  if (_table.kind == 2) _num_tombstones += keys_to_evict->NumItem();
+}
+
 bool CacheEntryManager::MaybeRebuild(const std::function<MemHandle(size_t)> &allocator, Context ctx, int loc,
                                      StreamHandle stream, const std::function<void()> &wait_for_lookups) {
   if (_table.kind != 2) return false;

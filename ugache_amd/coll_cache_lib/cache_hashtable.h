@@ -71,6 +71,9 @@ class CacheEntryManager {
   void InsertSeqOffWithLoc(TensorPtr keys, int loc, StreamHandle stream);
   // cuh:622-625
   void Evict(TensorPtr keys_to_evict, StreamHandle stream);
+  // the same, and the evicted keys' slots leave the slot bitmap (SlotUsedBits) in the same launch: what LookupOffset +
+  // ReturnOffset + Evict do together when the bookkeeping lives on the device
+  void EvictRelease(TensorPtr keys_to_evict, StreamHandle stream);
   // cuh:635-655 — free-list: returned offsets go to the back, reservations come from the front
   void ReturnOffset(TensorPtr new_offsets);
   TensorPtr ReserveOffsetFront(IdType num_new_insert_keys);

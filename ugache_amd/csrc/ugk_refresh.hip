@@ -435,6 +435,22 @@ __global__ __launch_bounds__(kBlock) void bitmap_update_kernel(unsigned long lon
   }
 }
 
+// every bit up to and including position *last_pos: what taking the lowest free slots, the last of them *last_pos,
+// does to the slot bitmap, as a pass over the bitmap instead of one atomic per slot on words 64 neighbours share
+__global__ __launch_bounds__(kBlock) void bitmap_set_through_kernel(unsigned long long *bitmap, uint64_t nbits,
+                                                                    const uint32_t *last_pos, uint32_t *status) {
+  const uint64_t last = *last_pos;
+  if (last >= nbits) {
+    if (blockIdx.x == 0 && threadIdx.x == 0) atomicOr(status, UGK_ST_KEY_OUT_OF_RANGE);
+    return;
+  }
+  const uint64_t wl = last >> 6;
+  for (uint64_t w = (uint64_t)blockIdx.x * kBlock + threadIdx.x; w <= wl; w += (uint64_t)gridDim.x * kBlock) {
+    if (w < wl) bitmap[w] = ~0ull;
+    else bitmap[w] |= (last & 63) == 63 ? ~0ull : (1ull << ((last & 63) + 1)) - 1ull;
+  }
+}
+
 __global__ __launch_bounds__(kBlock) void rows_to_keys_kernel(const uint32_t *rows, size_t n, uint64_t mul,
                                                               uint64_t mask, long long *keys) {
   for (size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x; i < n; i += (size_t)gridDim.x * kBlock)
@@ -558,6 +574,17 @@ int ugk_bitmap_update(uint64_t *bitmap_dev, uint64_t nbits, const uint32_t *idx_
   const unsigned grid = clamp_grid((n + kBlock - 1) / kBlock, 0);
   hipLaunchKernelGGL(bitmap_update_kernel, dim3(grid), dim3(kBlock), 0, as_stream(stream),
                      reinterpret_cast<unsigned long long *>(bitmap_dev), nbits, idx_dev, n, set, status_dev);
+  UGK_HIP(hipGetLastError());
+  return 0;
+}
+
+int ugk_bitmap_set_through(uint64_t *bitmap_dev, uint64_t nbits, const uint32_t *last_pos_dev, uint32_t *status_dev,
+                           void *stream) {
+  UGK_REQUIRE(bitmap_dev && last_pos_dev && status_dev, "ugk_bitmap_set_through: null pointer");
+  UGK_REQUIRE(nbits > 0, "ugk_bitmap_set_through: empty bitmap");
+  const unsigned grid = clamp_grid(((nbits + 63) / 64 + kBlock - 1) / kBlock, 0);
+  hipLaunchKernelGGL(bitmap_set_through_kernel, dim3(grid), dim3(kBlock), 0, as_stream(stream),
+                     reinterpret_cast<unsigned long long *>(bitmap_dev), nbits, last_pos_dev, status_dev);
   UGK_HIP(hipGetLastError());
   return 0;
 }

@@ -32,8 +32,20 @@ __global__ __launch_bounds__(kBlock) void flat_insert_kernel(uint32_t *table, ui
   }
 }
 
+// slot_bits (may be null): one bit per cache slot; the bit of the slot an evicted key held is cleared on the way
+__device__ __forceinline__ void release_slot(unsigned long long *slot_bits, uint64_t nslots, uint32_t slot,
+                                             uint32_t *status) {
+  if (slot_bits == nullptr) return;
+  if (slot >= nslots) {
+    atomicOr(status, UGK_ST_KEY_OUT_OF_RANGE);
+    return;
+  }
+  atomicAnd(slot_bits + (slot >> 6), ~(1ull << (slot & 63u)));
+}
+
 template <typename K>
 __global__ __launch_bounds__(kBlock) void flat_evict_kernel(uint32_t *table, uint64_t nkeys, const K *keys, size_t n,
+                                                            unsigned long long *slot_bits, uint64_t nslots,
                                                             uint32_t *status) {
   for (size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x; i < n; i += (size_t)gridDim.x * kBlock) {
     const uint64_t key = key_to_u64<K>(keys[i]);
@@ -43,6 +55,7 @@ __global__ __launch_bounds__(kBlock) void flat_evict_kernel(uint32_t *table, uin
     }
     const uint32_t old = atomicExch(table + key, UGK_EMPTY_U32);
     if (old == UGK_EMPTY_U32) atomicOr(status, UGK_ST_EVICT_ABSENT);
+    else release_slot(slot_bits, nslots, old & 0x0fffffffu, status);
   }
 }
 
@@ -143,7 +156,8 @@ __global__ __launch_bounds__(kBlock) void hash_insert_kernel(ugk_bucket_t *table
 
 template <typename K>
 __global__ __launch_bounds__(kBlock) void hash_evict_kernel(ugk_bucket_t *table, uint64_t nb, const K *keys,
-                                                            size_t n, uint32_t *status) {
+                                                            size_t n, unsigned long long *slot_bits, uint64_t nslots,
+                                                            uint32_t *status) {
   for (size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x; i < n; i += (size_t)gridDim.x * kBlock) {
     const uint64_t key = key_to_u64<K>(keys[i]);
     uint64_t pos = key_is_reserved(key) ? 0 : hash_home(key, nb);
@@ -152,6 +166,7 @@ __global__ __launch_bounds__(kBlock) void hash_evict_kernel(ugk_bucket_t *table,
     for (uint64_t step = 0; step < nb && !done; ++step) {
       const uint64_t cur = load_key_relaxed(table + pos);
       if (cur == key) {
+        if (slot_bits) release_slot(slot_bits, nslots, __atomic_load_n(&table[pos].off, __ATOMIC_RELAXED), status);
         // either order of these two stores is safe for a concurrent lookup: it sees the key still valid (its slot
         // keeps the row until a later lookup has passed), not valid, or gone
         store_off_meta(table + pos, 0u, 0u);
@@ -233,17 +248,19 @@ int table_insert(ugk_table_t t, const K *keys, const uint32_t *offs, uint32_t se
 }
 
 template <typename K>
-int table_evict(ugk_table_t t, const K *keys, size_t n, uint32_t *status, void *stream) {
+int table_evict(ugk_table_t t, const K *keys, size_t n, uint64_t *slot_bits_dev, uint64_t nslots, uint32_t *status,
+                void *stream) {
   if (n == 0) return 0;
   if (check_table(t, "ugk_table_evict")) return 1;
   UGK_REQUIRE(keys && status, "ugk_table_evict: null keys or status");
+  unsigned long long *slot_bits = reinterpret_cast<unsigned long long *>(slot_bits_dev);
   const unsigned grid = clamp_grid((n + kBlock - 1) / kBlock, 0);
   if (t.kind == 1)
     hipLaunchKernelGGL(flat_evict_kernel<K>, dim3(grid), dim3(kBlock), 0, as_stream(stream), (uint32_t *)t.table,
-                       t.size, keys, n, status);
+                       t.size, keys, n, slot_bits, nslots, status);
   else
     hipLaunchKernelGGL(hash_evict_kernel<K>, dim3(grid), dim3(kBlock), 0, as_stream(stream), (ugk_bucket_t *)t.table,
-                       t.size, keys, n, status);
+                       t.size, keys, n, slot_bits, nslots, status);
   UGK_HIP(hipGetLastError());
   return 0;
 }
@@ -297,10 +314,20 @@ int ugk_table_insert_i64(ugk_table_t t, const int64_t *keys_dev, const uint32_t 
   return table_insert<int64_t>(t, keys_dev, offs_dev, seq_base, loc, n, status_dev, stream);
 }
 int ugk_table_evict_u32(ugk_table_t t, const uint32_t *keys_dev, size_t n, uint32_t *status_dev, void *stream) {
-  return table_evict<uint32_t>(t, keys_dev, n, status_dev, stream);
+  return table_evict<uint32_t>(t, keys_dev, n, nullptr, 0, status_dev, stream);
 }
 int ugk_table_evict_i64(ugk_table_t t, const int64_t *keys_dev, size_t n, uint32_t *status_dev, void *stream) {
-  return table_evict<int64_t>(t, keys_dev, n, status_dev, stream);
+  return table_evict<int64_t>(t, keys_dev, n, nullptr, 0, status_dev, stream);
+}
+int ugk_table_evict_release_u32(ugk_table_t t, const uint32_t *keys_dev, size_t n, uint64_t *slot_bits_dev,
+                                uint64_t nslots, uint32_t *status_dev, void *stream) {
+  UGK_REQUIRE(n == 0 || slot_bits_dev, "ugk_table_evict_release_u32: null slot bitmap");
+  return table_evict<uint32_t>(t, keys_dev, n, slot_bits_dev, nslots, status_dev, stream);
+}
+int ugk_table_evict_release_i64(ugk_table_t t, const int64_t *keys_dev, size_t n, uint64_t *slot_bits_dev,
+                                uint64_t nslots, uint32_t *status_dev, void *stream) {
+  UGK_REQUIRE(n == 0 || slot_bits_dev, "ugk_table_evict_release_i64: null slot bitmap");
+  return table_evict<int64_t>(t, keys_dev, n, slot_bits_dev, nslots, status_dev, stream);
 }
 int ugk_table_lookup_u32(ugk_table_t t, const uint32_t *keys_dev, size_t n, uint32_t fallback_loc,
                          uint32_t *loc_out_dev, uint32_t *off_out_dev, void *stream) {

@@ -90,6 +90,8 @@ SIGNATURES = {
     "ugk_table_insert_i64": [Table, _vp, _vp, _u32, _u32, _sz, _vp, _vp],
     "ugk_table_evict_u32": [Table, _vp, _sz, _vp, _vp],
     "ugk_table_evict_i64": [Table, _vp, _sz, _vp, _vp],
+    "ugk_table_evict_release_u32": [Table, _vp, _sz, _vp, _u64, _vp, _vp],
+    "ugk_table_evict_release_i64": [Table, _vp, _sz, _vp, _u64, _vp, _vp],
     "ugk_table_lookup_u32": [Table, _vp, _sz, _u32, _vp, _vp, _vp],
     "ugk_table_lookup_i64": [Table, _vp, _sz, _u32, _vp, _vp, _vp],
     "ugk_hash_census": [_vp, _sz, _vp, _vp],
@@ -120,6 +122,7 @@ SIGNATURES = {
     "ugk_bitmap_count": [_vp, _vp, C.c_int, _u64, _vp, _vp, _vp],
     "ugk_bitmap_emit": [_vp, _vp, C.c_int, _u64, _vp, _vp, _u64, _vp],
     "ugk_bitmap_update": [_vp, _u64, _vp, _sz, C.c_int, _vp, _vp],
+    "ugk_bitmap_set_through": [_vp, _u64, _vp, _vp, _vp],
     "ugk_rows_to_keys": [_vp, _sz, _u64, _u64, _vp, _vp],
     "ugk_last_error": [],
 }
