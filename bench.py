@@ -109,6 +109,9 @@ def parse_args():
     ap.add_argument("--stage-rows", type=int, default=1 << 22,
                     help="with --device-refresh: entries of the set of recently missed rows kept in HBM "
                          "(COLL_MISS_STAGE_ROWS; 0 = none, every inserted row crosses the host link again)")
+    ap.add_argument("--serving", action="store_true",
+                    help="mixed workloads: after the timed steps, time the same steps through the serving loop "
+                         "(coll_cache_forward_i64: 5 %% of every batch recorded, a background refresh every K/2 steps)")
     ap.add_argument("--calibrate", action="store_true",
                     help="also run 5 plain device copies of 1 GiB (ugk_copy_rows) so a counter run has a kernel of "
                          "known traffic next to the gather")
@@ -639,7 +642,7 @@ def run_mixed(args):
                      "note": "refresh = rank + place + evict/insert lists on the device (COLL_GPU_REFRESH=1, hotness "
                              "accumulating), row copy over the host link, table update; foreground, after each lookup"}
         note("refresh each step: lookup %.3f ms + refresh %.3f ms" % (each_step["lookup_ms"], each_step["refresh_ms"]))
-    elif sparse:
+    elif sparse and not args.serving:
         # one foreground refresh: the same hotness again, plus 1 % of the cache size worth of so-far uncached rows
         # pushed to the top, so that about 1 % of the cached rows are evicted and replaced
         before = _basics.info(0)
@@ -662,6 +665,54 @@ def run_mixed(args):
             sys.exit("bench.py: GPU output differs from the CPU oracle after the refresh")
         refresh = {"seconds": refresh_s, "boosted_rows": n_new, "table_rebuilds": after["table_rebuilds"],
                    "cached_rows_after": after["cached_rows"], "free_slots_after": after["free_slots"]}
+
+    serving = None
+    if args.serving:
+        # LookupManager::forward (lookup_manager.cc:158-213): every step records the first 5 % of the batch, looks the
+        # batch up (blocking) and, every K/2 steps, starts a refresh on a background thread.  Every step takes a batch
+        # of its own from the workload's distribution, so a refresh gains what the hotness it saw predicts, not the
+        # keys of a pool that comes round again.
+        srv_rows = torch.stack([make_batch() for _ in range(W + K)])
+        srv_keys = ids_of(srv_rows)
+        srv_ptrs = [srv_keys[i].data_ptr() for i in range(W + K)]
+        torch.cuda.synchronize()
+        C.coll_cache_forward_config(1, max(K // 2, 1), 0.05, 1)
+        for i in range(W):
+            C.coll_cache_forward_i64(0, srv_ptrs[i], n_keys, out.data_ptr(), stream)
+        torch.cuda.synchronize()
+        before, during, after_r = [], [], []  # per-step times: no refresh yet, one running behind the step, one done
+        t0 = time.perf_counter()
+        for i in range(W, W + K):
+            ts = time.perf_counter()
+            C.coll_cache_forward_i64(0, srv_ptrs[i], n_keys, out.data_ptr(), stream)
+            dt = time.perf_counter() - ts
+            if C.coll_cache_forward_refresh_ongoing():
+                during.append(dt)
+            else:
+                (after_r if during else before).append(dt)
+        torch.cuda.synchronize()
+        el = time.perf_counter() - t0
+        t1 = time.perf_counter()
+        done = int(C.coll_cache_forward_join())
+        join_s = time.perf_counter() - t1
+        C.coll_cache_forward_config(0, 0, 0.0, 0)
+        if out.cpu().numpy().tobytes() != orc.gather(table_np, srv_rows[W + K - 1].cpu().numpy(), omp=True).tobytes():
+            sys.exit("bench.py: GPU output differs from the CPU oracle in the serving loop")
+        med = lambda v: round(float(np.median(v)) * 1e3, 4) if v else None
+        serving = {"ms_per_step": el / K * 1e3, "keys_per_s": n_keys * K / el, "steps": K,
+                   "ms_per_step_median": {"before_the_refresh": med(before), "while_it_runs": med(during),
+                                          "after_it": med(after_r)},
+                   "steps_of_each": [len(before), len(during), len(after_r)],
+                   "ms_longest_step": max(before + during + after_r) * 1e3,
+                   "recorded_fraction": 0.05, "refresh_every_steps": max(K // 2, 1), "refreshes_completed": done,
+                   "seconds_waited_for_the_last_refresh": join_s,
+                   "hotness_recorded_on": "device" if args.gpu_record else "host",
+                   "batches": "one fresh batch per step",
+                   "entry_point": "coll_cache_forward_i64 (record a prefix + blocking lookup + background refresh)"}
+        note("serving loop: %.3f ms/step (median %s before, %s during, %s after the refresh; longest %.2f ms), "
+             "%d refreshes" % (serving["ms_per_step"], med(before), med(during), med(after_r),
+                               serving["ms_longest_step"], done))
+        del srv_rows, srv_keys
 
     under_refresh = None
     if args.concurrent_refresh:
@@ -712,6 +763,7 @@ def run_mixed(args):
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "u8", "data": "synthetic",
         "refresh": refresh, "refresh_each_step": each_step, "under_concurrent_refresh": under_refresh,
+        "serving_loop": serving,
         "config": {"workload": args.workload, "table_rows": rows, "row_bytes": row_bytes, "keys_per_batch": n_keys,
                    "key_dtype": "int64", "sparse_ids": sparse, "cache_percentage": pct, "cached_rows": info_cache["cached_rows"],
                    "cache_capacity_rows": info_cache["capacity_rows"], "table_kind": info_cache["table_kind"],

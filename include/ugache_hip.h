@@ -89,7 +89,7 @@ typedef struct {
 const char *ugk_last_error(void);
 /* version of this ABI; bumped on any signature change.  ugk_abi_version() is what the loaded library was built with:
  * a caller compiled against another UGK_ABI_VERSION must not go on. */
-#define UGK_ABI_VERSION 9
+#define UGK_ABI_VERSION 10
 int ugk_abi_version(void);
 
 /* ---- runtime plumbing: Device::{AllocDataSpace,FreeDataSpace,CopyDataFromTo,StreamSync,CreateStream}
@@ -373,11 +373,21 @@ int ugk_record_drain(uint32_t *counts_dev, uint64_t first_row, uint64_t num_rows
  * scratch_bitmap_dev: as large as in_new_dev, overwritten.  With reset_counts != 0 the counters (and observed_dev)
  * are zeroed on the way.  observed_dev (may be NULL): the bitmap ugk_record_* keeps; when fewer rows were observed
  * than k asks for, the k-th best count is 0 without looking and no pass over the counters is made at all.
+ * ugk_rank_place_keep: the same with keep_dev (may be NULL: then it is ugk_rank_place), a bitmap of rows that win
+ * ties: among the rows whose counter equals the k-th best count, those with their bit in keep_dev come first, and
+ * inside either group the order above holds.  With keep_dev = the rows cached now, a refresh moves no row whose
+ * hotness does not tell it apart from the row it would replace (a cache filled from a ranking the counters do not know,
+ * or wider than the set of rows observed so far, otherwise trades its never-counted rows for the lowest-numbered
+ * ones).  keep_dev is read only and may not be one of the two output bitmaps; ugk_rank_threshold reports the last row
+ * taken from the group that was cut.
  * ugk_rank_threshold: copies the rank of the k-th best row of the last ugk_rank_place to the host (blocking; for tests
  * and logs; all ones for k == 0, zero for k >= num_rows). */
 size_t ugk_rank_workspace_bytes(void);
 int ugk_rank_place(uint32_t *counts_dev, uint64_t num_rows, uint64_t k, void *ws_dev, uint64_t *in_new_dev,
                    uint64_t *scratch_bitmap_dev, uint64_t *observed_dev, int reset_counts, void *stream);
+int ugk_rank_place_keep(uint32_t *counts_dev, uint64_t num_rows, uint64_t k, void *ws_dev, uint64_t *in_new_dev,
+                        uint64_t *scratch_bitmap_dev, uint64_t *observed_dev, const uint64_t *keep_dev,
+                        int reset_counts, void *stream);
 int ugk_rank_threshold(const void *ws_dev, uint64_t *threshold_host, void *stream);
 /* Ordered compaction over bitmaps.  The set S = { p < nbits : bit p of m is set }, m = (invert_a ? ~a : a) & ~b
  * (b_dev may be NULL).  ugk_bitmap_count writes |S| to *total_host (pinned host word, may be NULL) and leaves the

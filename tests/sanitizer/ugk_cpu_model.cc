@@ -746,22 +746,33 @@ int ugk_record_drain(uint32_t *counts, uint64_t first_row, uint64_t num_rows, ui
 }
 
 size_t ugk_rank_workspace_bytes(void) { return 64; }
+int ugk_rank_place_keep(uint32_t *counts, uint64_t num_rows, uint64_t k, void *ws, uint64_t *in_new,
+                        uint64_t *scratch, uint64_t *observed, const uint64_t *keep, int reset_counts, void *);
 int ugk_rank_place(uint32_t *counts, uint64_t num_rows, uint64_t k, void *ws, uint64_t *in_new, uint64_t *scratch,
-                   uint64_t *observed, int reset_counts, void *) {
+                   uint64_t *observed, int reset_counts, void *stream) {
+  return ugk_rank_place_keep(counts, num_rows, k, ws, in_new, scratch, observed, nullptr, reset_counts, stream);
+}
+// rows ordered by (count, kept, tie) with tie = row for counted rows and 0xffffffff - row for the others: three
+// 32-bit fields do not fit one word, so the kept bit goes between the count and the tie of a 128-bit key
+int ugk_rank_place_keep(uint32_t *counts, uint64_t num_rows, uint64_t k, void *ws, uint64_t *in_new,
+                        uint64_t *scratch, uint64_t *observed, const uint64_t *keep, int reset_counts, void *) {
   REQUIRE(counts && ws && in_new && scratch, "ugk_rank_place: null pointer");
+  REQUIRE(keep != in_new && keep != scratch, "ugk_rank_place_keep: the keep bitmap is one of the output bitmaps");
   REQUIRE(num_rows > 0 && num_rows < 0xffffffffull, "ugk_rank_place: rows do not fit 32 bits");
   const uint64_t n_words = (num_rows + 63) / 64;
-  std::vector<uint64_t> rank(num_rows);
+  typedef unsigned __int128 Rank;
+  std::vector<Rank> rank(num_rows);
   for (uint64_t r = 0; r < num_rows; ++r) {
     const uint32_t c = ld(counts + r);
-    rank[r] = c ? ((uint64_t)c << 32) | r : (uint64_t)(0xffffffffu - r);
+    const uint64_t kept = keep ? (ld(keep + r / 64) >> (r & 63)) & 1 : 0;
+    rank[r] = ((Rank)c << 64) | ((Rank)kept << 32) | (c ? (uint32_t)r : 0xffffffffu - (uint32_t)r);
   }
-  uint64_t threshold;
-  if (k == 0) threshold = ~0ull;
+  Rank threshold;
+  if (k == 0) threshold = ~(Rank)0;
   else if (k >= num_rows) threshold = 0;
   else {
-    std::vector<uint64_t> tmp(rank);
-    std::nth_element(tmp.begin(), tmp.begin() + (k - 1), tmp.end(), std::greater<uint64_t>());
+    std::vector<Rank> tmp(rank);
+    std::nth_element(tmp.begin(), tmp.begin() + (k - 1), tmp.end(), std::greater<Rank>());
     threshold = tmp[k - 1];
   }
   for (uint64_t w = 0; w < n_words; ++w) {
@@ -776,7 +787,9 @@ int ugk_rank_place(uint32_t *counts, uint64_t num_rows, uint64_t k, void *ws, ui
     if (observed)
       for (uint64_t w = 0; w < n_words; ++w) st(observed + w, (uint64_t)0);
   }
-  *static_cast<uint64_t *>(ws) = threshold;
+  // reported without the kept bit: (count << 32) | row, or 0xffffffff - row
+  const uint32_t th_count = (uint32_t)(threshold >> 64), th_tie = (uint32_t)threshold;
+  *static_cast<uint64_t *>(ws) = k == 0 ? ~0ull : k >= num_rows ? 0ull : ((uint64_t)th_count << 32) | th_tie;
   return 0;
 }
 int ugk_rank_threshold(const void *ws, uint64_t *threshold_host, void *) {

@@ -43,7 +43,7 @@ def make_config(num_total_item, pct, threads=8):
 def _fresh_cache(monkeypatch):
     for v in ("COLL_HASH_TABLE", "SAMGRAPH_COLL_CACHE_CONCURRENT_LINK_IMPL", "SAMGRAPH_COLL_CACHE_NO_GROUP",
               "COLL_DEDUP_KEYS", "COLL_DEDUP_MIN_KEYS", "COLL_GPU_RECORD", "COLL_GPU_RECORD_EVERY", "COLL_GPU_REFRESH",
-              "COLL_GPU_REFRESH_KEEP"):
+              "COLL_GPU_REFRESH_KEEP", "COLL_GPU_REFRESH_STABLE"):
         monkeypatch.delenv(v, raising=False)
     yield
     if torch.cuda.is_available():
@@ -504,6 +504,81 @@ def test_refresh_on_the_device_places_like_the_oracle(table_kind, foreground, ke
     cached, nid = expected_cached_set(np.concatenate(counted), n_item, pct)
     check_cached(cached)
     lookup(rng.integers(0, n_item, size=20_000), nid)
+
+
+@pytest.mark.parametrize("table_kind", ["FLAT", "HASH"])
+@pytest.mark.parametrize("foreground", [True, False])
+@pytest.mark.parametrize("keep", [False, True])
+def test_stable_refresh_on_the_device_moves_only_rows_the_counters_tell_apart(table_kind, foreground, keep,
+                                                                              monkeypatch):
+    """COLL_GPU_REFRESH_STABLE=1: rows whose counts tie at the last count that gets in stay where they are.  The cache
+    is filled from a ranking the device-side counters know nothing of and is wider than the set of rows the lookups
+    touch, so a plain refresh would trade most never-counted cached rows for the lowest-numbered ones; the stable one
+    brings in the counted rows only.  The cached set after every refresh is the top set by (count, cached before,
+    row order), from a full sort."""
+    monkeypatch.setenv("COLL_HASH_TABLE", table_kind)
+    monkeypatch.setenv("COLL_GPU_RECORD", "1")
+    monkeypatch.setenv("COLL_GPU_REFRESH", "1")
+    monkeypatch.setenv("COLL_GPU_REFRESH_STABLE", "1")
+    if keep:
+        monkeypatch.setenv("COLL_GPU_REFRESH_KEEP", "1")
+    monkeypatch.setenv("COLL_REFRESH_SLEEP_US", "100")
+    monkeypatch.setenv("COLL_REFRESH_BATCH_ROWS", "512")
+    rng = np.random.default_rng(33)
+    n_item, dim, pct = 40_003, 32, 0.3
+    co.config(make_config(n_item, pct))
+    co.coll_cache_record_init(0)
+    perm = rng.permutation(n_item)
+    s0 = perm[zipf_ranks(rng, 200_000, n_item, 0.8)]
+    co.coll_torch_record(0, torch.from_numpy(s0).to(torch.int32))
+    emb = co.coll_torch_create_emb_shm(0, n_item, dim, torch.float32)
+    table = fill_table(emb, rng)
+    co.coll_torch_init_t(0, 0, emb, pct)
+    cached, _ = expected_cached_set(s0.astype(np.uint32), n_item, pct)
+    k = len(cached)
+    counts = np.zeros(n_item, np.int64)
+    rows = np.arange(n_item, dtype=np.int64)
+
+    def refresh():
+        if foreground:
+            co.coll_torch_refresh(0, True)
+            return
+        t = threading.Thread(target=co.coll_torch_refresh, args=(0, False))
+        t.start()
+        while t.is_alive():
+            co.coll_torch_lookup_key_t_val_ret(0, torch.zeros(0, dtype=torch.int32).cuda(), False)
+            time.sleep(0.001)
+        t.join()
+
+    moved = []
+    for rnd in range(3):
+        # a few thousand distinct rows per round, far fewer than the cache holds
+        keys = perm[zipf_ranks(rng, 6_000, n_item, 1.2)] if rnd != 1 else rng.integers(0, n_item, size=2_500)
+        out = co.coll_torch_lookup_key_t_val_ret(0, torch.from_numpy(keys).to(torch.int32).cuda(), False)
+        assert out.cpu().numpy().tobytes() == ORC.gather(table, keys.astype(np.int64)).tobytes()
+        np.add.at(counts, keys, 1)
+        refresh()
+        was = np.zeros(n_item, bool)
+        was[cached] = True
+        tie = np.where(counts > 0, rows, -rows)
+        order = np.lexsort((tie, was, counts))[::-1]
+        new_cached = np.sort(order[:k]).astype(np.uint32)
+        plain, _ = expected_cached_set(np.repeat(rows, counts).astype(np.uint32), n_item, pct)
+        moved.append((len(np.setdiff1d(cached, new_cached)), len(np.setdiff1d(cached, plain))))
+        got = np.zeros(k, np.uint32)
+        assert _basics.C_LIB_CTYPES.coll_cache_get_cached_keys(0, got.ctypes.data, k) == k
+        assert np.array_equal(got, new_cached), rnd
+        # every row that left was never counted, every row that came in was counted
+        assert not counts[np.setdiff1d(cached, new_cached)].any() and counts[np.setdiff1d(new_cached, cached)].all()
+        cached = new_cached
+        if not keep:
+            counts[:] = 0
+        probe = rng.integers(0, n_item, size=1_500)
+        out = co.coll_torch_lookup_key_t_val_ret(0, torch.from_numpy(probe).to(torch.int32).cuda(), False)
+        assert out.cpu().numpy().tobytes() == ORC.gather(table, probe.astype(np.int64)).tobytes()
+        np.add.at(counts, probe, 1)
+    # (rows the stable refresh moved, rows a plain one would have moved)
+    assert all(0 < stable < plain for stable, plain in moved) and moved[0][0] < moved[0][1] // 4, moved
 
 
 @pytest.mark.parametrize("pct,impl,dedup", [(0.25, "", False), (0.25, "NONE", True), (0.25, "SMMaskPhase", False),

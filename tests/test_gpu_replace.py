@@ -36,8 +36,9 @@ def _counts(rng, n, kind):
     raise AssertionError(kind)
 
 
-def _place(counts, k, reset, with_observed=False):
-    """-> membership bits of the k best rows, the rank threshold, the counters afterwards"""
+def _place(counts, k, reset, with_observed=False, keep=None):
+    """-> membership bits of the k best rows, the rank threshold, the counters afterwards.
+    keep (bool per row, optional): rows that win ties at the k-th count (ugk_rank_place_keep)"""
     n = len(counts)
     words = (n + 63) // 64
     d_counts = to_dev(counts)
@@ -49,7 +50,15 @@ def _place(counts, k, reset, with_observed=False):
         pad = np.zeros(words * 64, bool)
         pad[:n] = counts > 0
         observed = to_dev(np.packbits(pad, bitorder="little").view(np.uint64))
-    hip.call("ugk_rank_place", ptr(d_counts), n, k, ptr(ws), ptr(bitmap), ptr(scratch), ptr(observed), reset, None)
+    if keep is None:
+        hip.call("ugk_rank_place", ptr(d_counts), n, k, ptr(ws), ptr(bitmap), ptr(scratch), ptr(observed), reset, None)
+    else:
+        pad = np.zeros(words * 64, bool)
+        pad[:n] = keep
+        d_keep = to_dev(np.packbits(pad, bitorder="little").view(np.uint64))
+        hip.call("ugk_rank_place_keep", ptr(d_counts), n, k, ptr(ws), ptr(bitmap), ptr(scratch), ptr(observed),
+                 ptr(d_keep), reset, None)
+        assert np.array_equal(to_np(d_keep, np.uint8)[: words * 8], np.packbits(pad, bitorder="little"))  # read only
     th = C.c_uint64(0)
     hip.call("ugk_rank_threshold", ptr(ws), C.byref(th), None)
     bits = np.unpackbits(to_np(bitmap)[: words * 8], bitorder="little")
@@ -92,6 +101,56 @@ def test_rank_place_picks_the_hotter_rows_and_breaks_ties_towards_larger_rows():
                          (6, [4, 2, 1, 5, 0, 3])]:
         got, _, _ = _place(counts, k, 0)
         assert sorted(np.flatnonzero(got).tolist()) == sorted(want_rows)
+
+
+@pytest.mark.parametrize("kind", ["zipf", "ties", "zero", "saturated", "huge"])
+@pytest.mark.parametrize("n", [1, 64, 65, 1000, 100_003, 2_000_001])
+def test_rank_place_with_kept_rows_winning_ties(kind, n):
+    """rows ordered by (count, kept, row for counted rows / -row for the others), every key distinct: the k best by a
+    full lexicographic sort"""
+    rng = np.random.default_rng(n * 11 + len(kind))
+    counts = _counts(rng, n, kind)
+    rows = np.arange(n, dtype=np.int64)
+    tie = np.where(counts > 0, rows, -rows)
+    observed = int((counts > 0).sum())
+    for keep_share in (0.0, 0.2, 0.9, 1.0):
+        keep = rng.random(n) < keep_share
+        order = np.lexsort((tie, keep, counts))[::-1]  # best first; the last key of lexsort is the primary one
+        n_kept_zero = int((keep & (counts == 0)).sum())
+        ks = sorted({1, n // 3, observed, min(observed + max(n_kept_zero - 1, 0), n), min(observed + n_kept_zero, n),
+                     min(observed + n_kept_zero + 1, n), n - 1} - {0})
+        for k in ks:
+            if k >= n:
+                continue
+            want = np.zeros(n, bool)
+            want[order[:k]] = True
+            for reset, with_observed in ((0, False), (1, True), (0, True)):
+                got, th, left = _place(counts, k, reset, with_observed, keep=keep)
+                assert np.array_equal(got, want), (kind, n, k, keep_share, reset, with_observed)
+                last = order[k - 1]
+                want_th = (int(counts[last]) << 32) | int(last) if counts[last] else 0xFFFFFFFF - int(last)
+                assert th == want_th
+                assert np.array_equal(left, counts if reset == 0 else np.zeros(n, np.uint32))
+            if keep_share == 0.0:  # nothing kept: the plain placement
+                plain, _, _ = _place(counts, k, 0)
+                assert np.array_equal(plain, want)
+
+
+def test_rank_place_keeps_cached_rows_the_counters_do_not_tell_apart():
+    # hand-worked: counts 0 5 5 0 9 1 0 0, rows 3 and 7 kept.  Counted rows first: 4, 2, 1, 5; then the kept
+    # never-counted rows 3, 7 (ascending), then 0, 6.  With k = 2 the tie of rows 1 and 2 goes to the kept one.
+    counts = np.array([0, 5, 5, 0, 9, 1, 0, 0], np.uint32)
+    keep = np.zeros(8, bool)
+    keep[[3, 7]] = True
+    for k, want_rows in [(4, [4, 2, 1, 5]), (5, [4, 2, 1, 5, 3]), (6, [4, 2, 1, 5, 3, 7]), (7, [4, 2, 1, 5, 3, 7, 0])]:
+        got, _, _ = _place(counts, k, 0, keep=keep)
+        assert sorted(np.flatnonzero(got).tolist()) == sorted(want_rows), k
+    keep[:] = False
+    keep[1] = True
+    got, _, _ = _place(counts, 2, 0, keep=keep)
+    assert sorted(np.flatnonzero(got).tolist()) == [1, 4]
+    got, _, _ = _place(counts, 2, 0)
+    assert sorted(np.flatnonzero(got).tolist()) == [2, 4]
 
 
 def test_rank_place_on_the_committed_golden_case():

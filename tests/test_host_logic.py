@@ -66,6 +66,26 @@ def test_record_and_rank_match_oracle(kdtype):
     assert C.coll_cache_rank_hotness(0, None, None, 0) == 0
 
 
+@pytest.mark.parametrize("batch", [900, 70_000])
+def test_every_round_of_counts_starts_from_zero(batch):
+    """Ranking drains the counters into a second array and recording goes on in a third: over several rounds
+    (small batches take the one-thread loop, large ones the parallel one) each ranking holds that round's keys only"""
+    rng = np.random.default_rng(11)
+    n_item = 30_000
+    _config(n_item)
+    cc._basics.coll_cache_record_init(0)
+    for rnd in range(4):
+        keys = [(rng.zipf(1.3, size=batch) % n_item).astype(np.uint32) for _ in range(3)]
+        for k in keys:
+            C.coll_cache_record(0, k.ctypes.data, len(k))
+        want_k, want_c = ORC.freq_rank(np.concatenate(keys))
+        got_k = np.zeros(n_item, np.uint32)
+        got_c = np.zeros(n_item, np.uint32)
+        m = C.coll_cache_rank_hotness(0, got_k.ctypes.data, got_c.ctypes.data, n_item)
+        assert m == len(want_k), rnd
+        assert np.array_equal(got_k[:m], want_k) and np.array_equal(got_c[:m], want_c), rnd
+
+
 @pytest.mark.parametrize("pct", [0.0, 0.1, 0.25, 0.333, 0.999])
 def test_placement_matches_oracle_rep_solve(pct):
     rng = np.random.default_rng(5)

@@ -414,14 +414,15 @@ void ExtractSession::JoinRecordOnHost() {
   _record_pending = false;
 }
 
-void ExtractSession::PlaceOnDevice(size_t num_cached, uint64_t *in_new_bits, uint64_t *scratch_bits, void *rank_ws,
+void ExtractSession::PlaceOnDevice(size_t num_cached, uint64_t *in_new_bits, uint64_t *scratch_bits,
+                                   const uint64_t *keep_bits, void *rank_ws,
                                    bool reset_counts, StreamHandle stream) {
   CHECK_NOTNULL(_hot_counts) << "placement on the device needs the device-side hotness counters (COLL_GPU_RECORD=1)";
   const size_t rows = _cache_ctx->_num_total_nodes;
   std::lock_guard<std::mutex> no_drain(_drain_mu);
   std::lock_guard<std::mutex> guard(_enqueue_mu);
-  UGK_CALL(ugk_rank_place(_hot_counts->ptr<uint32_t>(), rows, num_cached, rank_ws, in_new_bits, scratch_bits,
-                          ObservedBits(), reset_counts ? 1 : 0, _record_stream));
+  UGK_CALL(ugk_rank_place_keep(_hot_counts->ptr<uint32_t>(), rows, num_cached, rank_ws, in_new_bits, scratch_bits,
+                               ObservedBits(), keep_bits, reset_counts ? 1 : 0, _record_stream));
   UGK_CALL(ugk_event_record(_ev_placed, _record_stream));
   UGK_CALL(ugk_stream_wait_event(stream, _ev_placed));
 }
@@ -1226,8 +1227,10 @@ void RefreshSession::refresh_on_device(ExtractSession *session, size_t num_cache
 
   // Steps 1-3: the new placement as a bitmap, then evict = cached & ~new and insert = new & ~cached, ascending.  Both
   // sets are counted before the one wait that tells the host their sizes.
+  // COLL_GPU_REFRESH_STABLE: rows that tie at the last count that gets in stay where they are (cached or not)
   session->PlaceOnDevice(num_cached, table->InNewBits(), table->_dev_scratch_bits->ptr<uint64_t>(),
-                         table->_dev_rank_ws->ptr(), !RunConfig::gpu_refresh_keep, stream);
+                         RunConfig::gpu_refresh_stable ? table->InCacheBits() : nullptr, table->_dev_rank_ws->ptr(),
+                         !RunConfig::gpu_refresh_keep, stream);
   volatile uint32_t *n_evict_word = table->CountBits(table->InCacheBits(), table->InNewBits(), false, num_rows, 0, stream);
   volatile uint32_t *n_insert_word = table->CountBits(table->InNewBits(), table->InCacheBits(), false, num_rows, 1, stream);
   UGK_CALL(ugk_stream_sync(stream));

@@ -253,12 +253,14 @@ class ExtractSession {
   // Ranks the rows by what the lookups have counted on the device (same order as FreqRecorder::Sort, never-counted
   // rows behind the counted ones in ascending order) and sets bit r of in_new_bits for the num_cached best rows.
   // Runs on the record stream, ordered against the counting of every lookup; `stream` waits for the result.
-  // reset_counts: the next interval starts from zero, as after DrainHotness.
+  // reset_counts: the next interval starts from zero, as after DrainHotness.  keep_bits (may be null): rows that
+  // win ties at the last count that gets in (ugk_rank_place_keep).
   bool CountsOnDevice() const { return _hot_counts != nullptr; }
+  int DeviceId() const { return _cache_ctx->_trainer_ctx.device_id; }
   // what a foreground refresh may read rows from besides the host table (null: nothing)
   const ugk_stage_t *StageForRefresh(bool foreground, StreamHandle stream);
-  void PlaceOnDevice(size_t num_cached, uint64_t *in_new_bits, uint64_t *scratch_bits, void *rank_ws,
-                     bool reset_counts, StreamHandle stream);
+  void PlaceOnDevice(size_t num_cached, uint64_t *in_new_bits, uint64_t *scratch_bits, const uint64_t *keep_bits,
+                     void *rank_ws, bool reset_counts, StreamHandle stream);
   // the device-side counting of the following lookups covers only the first `num_keys` keys of a batch
   // (the recorded prefix of LookupManager's record thread); SIZE_MAX, the default: the whole batch
   void SetRecordLimit(size_t num_keys) { _record_limit = num_keys; }

@@ -4,6 +4,7 @@
 #include <cstdlib>
 #include <cstring>
 #include <limits>
+#include <sys/mman.h>
 #ifdef _OPENMP
 #include <parallel/algorithm>
 #endif
@@ -63,18 +64,43 @@ namespace {
 int ScanThreads() { return std::max(1, RunConfig::solver_omp_thread_num_per_gpu); }
 }  // namespace
 
+namespace {
+constexpr size_t kHugePage = size_t(2) << 20;
+size_t CounterBytes(size_t num_nodes) {
+  return (std::max<size_t>(num_nodes, 1) * sizeof(CntT) + kHugePage - 1) / kHugePage * kHugePage;
+}
+/** Zeroed counters in an anonymous mapping: pages nobody counts in are never touched, and the mapping asks for huge
+ *  pages, so a batch of keys spread over a table of gigabytes faults in and walks a thousand pages, not a million. */
+CntT *MapCounters(size_t num_nodes) {
+  const size_t bytes = CounterBytes(num_nodes);
+  void *raw = mmap(nullptr, bytes + kHugePage, PROT_READ | PROT_WRITE, MAP_PRIVATE | MAP_ANONYMOUS | MAP_NORESERVE, -1, 0);
+  CHECK(raw != MAP_FAILED) << "no memory for the counters of " << num_nodes << " keys";
+  // keep the 2 MiB-aligned part: give the rest back
+  char *lo = static_cast<char *>(raw);
+  char *p = reinterpret_cast<char *>((reinterpret_cast<uintptr_t>(lo) + kHugePage - 1) & ~uintptr_t(kHugePage - 1));
+  if (p > lo) munmap(lo, p - lo);
+  if (p + bytes < lo + bytes + kHugePage) munmap(p + bytes, lo + bytes + kHugePage - (p + bytes));
+  madvise(p, bytes, MADV_HUGEPAGE);  // advice only: small pages serve as well, slower
+  return reinterpret_cast<CntT *>(p);
+}
+void UnmapCounters(CntT *p, size_t num_nodes) {
+  if (p) munmap(p, CounterBytes(num_nodes));
+}
+}  // namespace
+
 FreqRecorder::FreqRecorder(size_t num_nodes, int local_id) : _num_nodes(num_nodes), _local_id(local_id) {
   CHECK(num_nodes < std::numeric_limits<IdType>::max() / 2);
-  _live = static_cast<CntT *>(calloc(std::max<size_t>(num_nodes, 1), sizeof(CntT)));
-  _shared = static_cast<CntT *>(calloc(std::max<size_t>(num_nodes, 1), sizeof(CntT)));
-  CHECK(_live != nullptr && _shared != nullptr) << "no memory for the counters of " << num_nodes << " keys";
+  _live = MapCounters(num_nodes);
+  _spare = MapCounters(num_nodes);
+  _shared = MapCounters(num_nodes);
   global_cont_freq_buf = new ContFreqBuf;
 }
 
 FreqRecorder::~FreqRecorder() {
   delete global_cont_freq_buf;
-  free(_live);
-  free(_shared);
+  UnmapCounters(_live, _num_nodes);
+  UnmapCounters(_spare, _num_nodes);
+  UnmapCounters(_shared, _num_nodes);
 }
 
 template <typename KeyT>
@@ -83,14 +109,37 @@ void FreqRecorder::Record(const KeyT *input, size_t num_inputs) {
   CntT *cnt = _live;
   const size_t n_nodes = _num_nodes;
   bool bad = false;
-#pragma omp parallel for num_threads(RunConfig::solver_omp_thread_num_per_gpu) reduction(|| : bad) if (num_inputs > 65536)
-  for (size_t i = 0; i < num_inputs; i++) {
-    const uint64_t k = RunConfig::RowOfKey((uint64_t)input[i]);
-    if (k >= n_nodes || (RunConfig::key_map_mul && (uint64_t)input[i] > RunConfig::key_map_mask)) {
-      bad = true;
-      continue;
+  const auto row_of = [n_nodes](uint64_t key, bool *bad_key) -> uint64_t {
+    const uint64_t k = RunConfig::RowOfKey(key);
+    *bad_key = k >= n_nodes || (RunConfig::key_map_mul && key > RunConfig::key_map_mask);
+    return k;
+  };
+  if (num_inputs > 65536) {
+#pragma omp parallel for num_threads(RunConfig::solver_omp_thread_num_per_gpu) reduction(|| : bad)
+    for (size_t i = 0; i < num_inputs; i++) {
+      bool b;
+      const uint64_t k = row_of((uint64_t)input[i], &b);
+      if (b)
+        bad = true;
+      else
+        __atomic_fetch_add(&cnt[k], 1u, __ATOMIC_RELAXED);
     }
-    __atomic_fetch_add(&cnt[k], 1u, __ATOMIC_RELAXED);
+  } else {
+    // one thread under the recorder's lock: plain increments, which (unlike locked ones) leave the loads of later
+    // keys free to run ahead; the counters of a large table are far apart in memory, so the one needed 16 keys from
+    // now is asked for early
+    for (size_t i = 0; i < num_inputs; i++) {
+      bool b;
+      if (i + 16 < num_inputs) {
+        const uint64_t ahead = row_of((uint64_t)input[i + 16], &b);
+        if (!b) __builtin_prefetch(&cnt[ahead], 1);
+      }
+      const uint64_t k = row_of((uint64_t)input[i], &b);
+      if (b)
+        bad = true;
+      else
+        cnt[k]++;
+    }
   }
   if (num_inputs) _live_dirty = true;
   CHECK(!bad) << "FreqRecorder::Record: a key has no row among num_total_item=" << n_nodes;
@@ -98,9 +147,9 @@ void FreqRecorder::Record(const KeyT *input, size_t num_inputs) {
 template void FreqRecorder::Record<Id64Type>(const Id64Type *input, size_t num_inputs);
 template void FreqRecorder::Record<IdType>(const IdType *input, size_t num_inputs);
 
-void FreqRecorder::ScatterHandedOver(CntT *into) {
-  const size_t n = _handed_over.size(), n_nodes = _num_nodes;
-  const FreqEntry *e = _handed_over.data();
+void FreqRecorder::ScatterHandedOver(std::vector<FreqEntry> &list, CntT *into) {
+  const size_t n = list.size(), n_nodes = _num_nodes;
+  const FreqEntry *e = list.data();
   bool bad = false;
 #pragma omp parallel for num_threads(ScanThreads()) reduction(|| : bad) if (n > 65536)
   for (size_t i = 0; i < n; i++) {
@@ -110,14 +159,14 @@ void FreqRecorder::ScatterHandedOver(CntT *into) {
       __atomic_fetch_add(&into[e[i].key], e[i].cnt, __ATOMIC_RELAXED);
   }
   CHECK(!bad) << "FreqRecorder: a handed-over row is outside num_total_item=" << n_nodes;
-  _handed_over.clear();
+  list.clear();
 }
 
 void FreqRecorder::BeginEntries() {
   std::lock_guard<std::mutex> g(_mu);
   if (_handed_over.empty()) return;
   // an earlier hand-over is still pending: its keys may come again, so it goes into the array now
-  ScatterHandedOver(_live);
+  ScatterHandedOver(_handed_over, _live);
   _live_dirty = true;
 }
 
@@ -127,36 +176,48 @@ void FreqRecorder::AddEntries(const FreqEntry *entries, size_t num_entries) {
 }
 
 void FreqRecorder::LocalCombineToShared() {
-  std::lock_guard<std::mutex> g(_mu);
-  if (!_live_dirty) return;  // nothing was counted on the host: no scan
-  CntT *shared = _shared, *live = _live;
+  std::lock_guard<std::mutex> combine(_combine_mu);
+  CntT *drained;
+  {
+    // the recording side goes on in the other array at once: the scan below runs beside it
+    std::lock_guard<std::mutex> g(_mu);
+    if (!_live_dirty) return;  // nothing was counted on the host: no scan
+    drained = _live;
+    _live = _spare;
+    _spare = drained;
+    _live_dirty = false;
+  }
+  CntT *shared = _shared;
   const size_t n = _num_nodes;
-  _live_dirty = false;
   _shared_dirty = true;
 #pragma omp parallel for num_threads(ScanThreads())
   for (size_t i = 0; i < n; i++) {
-    if (live[i]) {  // the recorded keys are a small part of the key space: write only where something was counted
-      shared[i] += live[i];
-      live[i] = 0;
+    if (drained[i]) {  // the recorded keys are a small part of the key space: write only where something was counted
+      shared[i] += drained[i];
+      drained[i] = 0;
     }
   }
 }
 
 void FreqRecorder::GlobalCombine() {
-  std::lock_guard<std::mutex> g(_mu);
+  std::lock_guard<std::mutex> combine(_combine_mu);
+  std::vector<FreqEntry> handed_over;
+  {
+    std::lock_guard<std::mutex> g(_mu);
+    handed_over.swap(_handed_over);
+  }
   auto &e = global_cont_freq_buf->entries;
   e.clear();
   if (!_shared_dirty) {
     // only handed-over entries (distinct keys): they are the list, whatever their order — Sort() follows
     const size_t n_nodes = _num_nodes;
-    for (const auto &x : _handed_over) CHECK_LT((size_t)x.key, n_nodes);
-    e.swap(_handed_over);
-    _handed_over.clear();
+    for (const auto &x : handed_over) CHECK_LT((size_t)x.key, n_nodes);
+    e.swap(handed_over);
     global_cont_freq_buf->buf = e.data();
     LOG(INFO) << "freq recorder global combine: " << e.size() << " distinct keys (handed over)";
     return;
   }
-  if (!_handed_over.empty()) ScatterHandedOver(_shared);
+  if (!handed_over.empty()) ScatterHandedOver(handed_over, _shared);
   _shared_dirty = false;
   // count, scan, fill: the entries come out in ascending key order whatever the thread count
   const int nthr = ScanThreads();

@@ -59,6 +59,7 @@ class FreqRecorder {
   inline size_t NumNodes() const { return _num_nodes; }
   // true when counts wait here for the next ranking (recorded on the host, or handed over from the device)
   bool HasCounts() {
+    std::lock_guard<std::mutex> combine(_combine_mu);
     std::lock_guard<std::mutex> g(_mu);
     return _live_dirty || _shared_dirty || !_handed_over.empty();
   }
@@ -67,13 +68,17 @@ class FreqRecorder {
  private:
   size_t _num_nodes;
   int _local_id;
-  // one counter per key of the key space, calloc-backed so that pages nobody counted in are never touched
+  // one counter per key of the key space, in anonymous mappings so that pages nobody counted in are never touched
   CntT *_live = nullptr;    // counts being recorded
+  CntT *_spare = nullptr;   // all zero: takes the place of _live when LocalCombineToShared drains it
   CntT *_shared = nullptr;  // counts handed over by LocalCombineToShared
   bool _live_dirty = false, _shared_dirty = false;  // the array holds a non-zero counter
   std::vector<FreqEntry> _handed_over;              // entries of the open hand-over, not in the arrays
-  void ScatterHandedOver(CntT *into);
-  std::mutex _mu;
+  void ScatterHandedOver(std::vector<FreqEntry> &list, CntT *into);
+  // _mu guards what recording touches (_live, _live_dirty, _handed_over) and is held for one batch at most;
+  // _combine_mu guards the rest (_spare, _shared, _shared_dirty, the ranked list) for the length of a scan of the
+  // key space.  Where both are held, _combine_mu is taken first.
+  std::mutex _mu, _combine_mu;
 };
 
 }  // namespace common

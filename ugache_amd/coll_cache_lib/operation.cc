@@ -5,7 +5,10 @@
 
 #include <cstring>
 #include <iostream>
+#include <algorithm>
 #include <atomic>
+#include <condition_variable>
+#include <mutex>
 #include <string>
 #include <thread>
 #include <vector>
@@ -320,6 +323,107 @@ void coll_cache_refresh(int replica_id, StreamHandle stream, int foreground) {
 
 // ---- serving loop ------------------------------------------------------------------------------------------
 namespace {
+/** The thread that counts the recorded prefix of a batch on the host while the lookup of the same batch runs
+ *  (lookup_manager.cc:291-312 with the record thread of lookup_manager.cc:158-178: posted before the lookup, waited
+ *  for after it).  The prefix crosses into pinned memory on a stream of the recorder's own, behind an event on the
+ *  caller's stream, so keys that earlier work on that stream produces are complete when they are copied. */
+class RecordWorker {
+ public:
+  ~RecordWorker() { Stop(); }
+  /// hands the first `bytes` bytes of `key` (device memory, `key_bytes` per key) to the thread
+  void Post(int replica_id, int device, const void *key, size_t num, int key_bytes, StreamHandle stream) {
+    Start(device);
+    UGK_CALL(ugk_event_record(_keys_ready, stream));
+    std::lock_guard<std::mutex> g(_mu);
+    _replica = replica_id, _key = key, _num = num, _key_bytes = key_bytes;
+    _pending = true, _done = false;
+    _cv.notify_all();
+  }
+  /// returns when the posted prefix has been counted
+  void Wait() {
+    Timer t;
+    std::unique_lock<std::mutex> g(_mu);
+    _cv.wait(g, [this] { return _done; });
+    Sample(_waited_s, t.Passed());
+  }
+  void Stop() {
+    if (!_thread.joinable()) return;
+    {
+      std::lock_guard<std::mutex> g(_mu);
+      _exit = true;
+      _cv.notify_all();
+    }
+    _thread.join();
+    _exit = false;
+    if (!_copy_s.empty())
+      LOG(INFO) << "record thread: " << _copy_s.size() << " batches; median copy " << Median(_copy_s) * 1e3
+                << " ms, count " << Median(_count_s) * 1e3 << " ms, waited for after the lookup "
+                << Median(_waited_s) * 1e3 << " ms";
+    _copy_s.clear(), _count_s.clear(), _waited_s.clear();
+    if (_staging) UGK_CALL(ugk_host_free(_staging));
+    UGK_CALL(ugk_event_destroy(_keys_ready));
+    UGK_CALL(ugk_stream_destroy(_stream));
+    _staging = nullptr, _staging_bytes = 0, _keys_ready = nullptr, _stream = nullptr;
+  }
+
+ private:
+  void Start(int device) {
+    if (_thread.joinable()) return;
+    UGK_CALL(ugk_stream_create(&_stream));
+    UGK_CALL(ugk_event_create(&_keys_ready));
+    _thread = std::thread([this, device] {
+      UGK_CALL(ugk_set_device(device));
+      std::unique_lock<std::mutex> g(_mu);
+      for (;;) {
+        _cv.wait(g, [this] { return _pending || _exit; });
+        if (_exit) return;
+        _pending = false;
+        g.unlock();
+        const size_t bytes = _num * _key_bytes;
+        if (bytes > _staging_bytes) {
+          if (_staging) UGK_CALL(ugk_host_free(_staging));
+          _staging_bytes = std::max<size_t>(bytes, 2 * _staging_bytes);
+          UGK_CALL(ugk_host_malloc(&_staging, _staging_bytes));
+        }
+        Timer t_copy;
+        UGK_CALL(ugk_stream_wait_event(_stream, _keys_ready));
+        UGK_CALL(ugk_memcpy_async(_staging, _key, bytes, _stream));
+        UGK_CALL(ugk_stream_sync(_stream));
+        Sample(_copy_s, t_copy.Passed());
+        Timer t_count;
+        if (_key_bytes == 8)
+          _freq_recorder[_replica]->Record(static_cast<const Id64Type *>(_staging), _num);
+        else
+          _freq_recorder[_replica]->Record(static_cast<const IdType *>(_staging), _num);
+        Sample(_count_s, t_count.Passed());
+        g.lock();
+        _done = true;
+        _cv.notify_all();
+      }
+    });
+  }
+  std::thread _thread;
+  std::mutex _mu;
+  std::condition_variable _cv;
+  bool _pending = false, _done = true, _exit = false;
+  int _replica = 0, _key_bytes = 4;
+  const void *_key = nullptr;
+  size_t _num = 0;
+  StreamHandle _stream = nullptr;
+  void *_keys_ready = nullptr;
+  void *_staging = nullptr;  // pinned
+  // durations of the latest batches, for the log line at the end
+  static void Sample(std::vector<double> &v, double s) {
+    if (v.size() < 4096) v.push_back(s);
+  }
+  static double Median(std::vector<double> &v) {
+    std::nth_element(v.begin(), v.begin() + v.size() / 2, v.end());
+    return v[v.size() / 2];
+  }
+  std::vector<double> _copy_s, _count_s, _waited_s;
+  size_t _staging_bytes = 0;
+};
+
 struct ForwardState {
   bool enable_refresh = false;
   bool periodic = false;
@@ -329,7 +433,7 @@ struct ForwardState {
   std::thread refresh_thread;
   std::atomic<bool> refresh_ongoing{false};
   std::atomic<uint64_t> refreshes_done{0};
-  std::vector<char> host_keys;  // staging of the recorded prefix on the host-record path
+  RecordWorker recorder;  // the host-record path
 };
 ForwardState _forward;
 
@@ -347,11 +451,7 @@ void ForwardStep(int replica_id, const KeyT *key, size_t num_keys, void *output,
   if (RunConfig::gpu_record) {
     session->SetRecordLimit(num_record);  // counted by the lookup itself
   } else if (num_record > 0) {
-    // lookup_manager.cc:295-306: copy the prefix to the host and count it there
-    fw.host_keys.resize(num_record * sizeof(KeyT));
-    UGK_CALL(ugk_memcpy_async(fw.host_keys.data(), key, num_record * sizeof(KeyT), stream));
-    UGK_CALL(ugk_stream_sync(stream));
-    _freq_recorder[replica_id]->Record(reinterpret_cast<const KeyT *>(fw.host_keys.data()), num_record);
+    fw.recorder.Post(replica_id, session->DeviceId(), key, num_record, sizeof(KeyT), stream);  // counted while the lookup runs
   }
   const uint64_t step_key = steps[replica_id] * RunConfig::num_device + replica_id;
   steps[replica_id]++;
@@ -359,7 +459,10 @@ void ForwardStep(int replica_id, const KeyT *key, size_t num_keys, void *output,
     _coll_cache->lookup64(replica_id, reinterpret_cast<const Id64Type *>(key), num_keys, output, stream, step_key);
   else
     _coll_cache->lookup(replica_id, reinterpret_cast<const IdType *>(key), num_keys, output, stream, step_key);
-  if (RunConfig::gpu_record) session->SetRecordLimit(SIZE_MAX);
+  if (RunConfig::gpu_record)
+    session->SetRecordLimit(SIZE_MAX);
+  else if (num_record > 0)
+    fw.recorder.Wait();
   const bool due = fw.enable_refresh && fw.refresh_iter > 0 &&
                    (fw.periodic ? (fw.step > 0 && fw.step % fw.refresh_iter == 0) : fw.step == fw.refresh_iter);
   if (due) {
@@ -508,6 +611,7 @@ uint32_t coll_cache_place_recorded(int replica_id, uint32_t num_node, double cac
 
 void coll_cache_shutdown(void) {
   ForwardJoin();
+  _forward.recorder.Stop();
   _forward.enable_refresh = false;
   _forward.step = 0;
   _forward.refreshes_done.store(0);

@@ -71,6 +71,9 @@ struct RunConfig {
   // COLL_GPU_REFRESH_KEEP=1: such a refresh leaves the counters as they are (hotness accumulates over refreshes)
   // instead of starting the next interval from zero
   static bool gpu_refresh_keep;
+  // COLL_GPU_REFRESH_STABLE=1: among rows whose counts tie at the last count that gets in, such a refresh prefers the
+  // rows cached now, so it moves no row that the counters do not tell apart from the one it would replace
+  static bool gpu_refresh_stable;
   // COLL_MISS_STAGE_ROWS=n (0 = off): the fused extraction also files the rows it takes from the host table in a
   // direct-mapped set of n (rounded up to a power of two) rows in HBM, and a foreground refresh takes the rows it inserts
   // from there when it finds them instead of over the host link again

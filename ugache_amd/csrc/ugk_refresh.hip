@@ -51,6 +51,9 @@ struct RankWs {
   uint32_t settled;              // the saturating first pass found T
   uint32_t last_row;             // the last needed row among those with count T
   uint32_t from_bitmap;          // fewer rows were observed than are wanted: T = 0, no pass over the counters
+  uint32_t keep_mode;            // with a keep bitmap: 1 = the needed rows with count T all come from eq & keep,
+                                 // 2 = all of eq & keep is in and the rest comes from eq & ~keep
+  uint32_t pad;
 
   uint32_t hist[kHistBins];
   BmWs bm;                       // chunk offsets of `eq`
@@ -165,6 +168,7 @@ __global__ void rank_init_kernel(RankWs *ws, unsigned long long remaining) {
     ws->settled = 0;
     ws->last_row = 0;
     ws->from_bitmap = 0;
+    ws->keep_mode = 0;
   }
   for (int b = tid; b < kHistBins; b += blockDim.x) ws->hist[b] = 0;
 }
@@ -240,10 +244,30 @@ __global__ __launch_bounds__(kBlock) void rank_split_bitmap_kernel(uint32_t *cou
   }
 }
 
+// with a keep bitmap, after eq & keep was counted (ws->bm.total): enough of them means the needed rows are all kept
+// ones; otherwise every kept one is in and the rest is looked for among the others
+__global__ void rank_keep_decide_kernel(RankWs *ws) {
+  if (ws->bm.total >= ws->remaining) {
+    ws->keep_mode = 1;
+  } else {
+    ws->keep_mode = 2;
+    ws->remaining -= ws->bm.total;
+  }
+}
+
+// the rows with count T among which the last needed one is looked for
+__device__ __forceinline__ unsigned long long tie_word(const RankWs *ws, const unsigned long long *eq,
+                                                       const unsigned long long *keep, uint64_t w) {
+  unsigned long long m = eq[w];
+  if (keep) m &= ws->keep_mode == 1 ? keep[w] : ~keep[w];
+  return m;
+}
+
 // one workgroup: the row of the last needed bit of eq.  With T > 0 the needed rows are the `remaining` topmost set
 // bits, the last of them is bit number total - remaining (counted from the bottom, from 0); with T == 0 they are the
 // lowest ones, the last is number remaining - 1.
-__global__ __launch_bounds__(kBlock) void rank_locate_kernel(RankWs *ws, const unsigned long long *eq, uint64_t nbits,
+__global__ __launch_bounds__(kBlock) void rank_locate_kernel(RankWs *ws, const unsigned long long *eq,
+                                                             const unsigned long long *keep, uint64_t nbits,
                                                              uint64_t per_chunk) {
   __shared__ uint32_t chunk_of;
   const int tid = threadIdx.x;
@@ -263,7 +287,7 @@ __global__ __launch_bounds__(kBlock) void rank_locate_kernel(RankWs *ws, const u
   uint32_t skip = index - ws->bm.base[c];  // set bits of the chunk below the wanted one
   for (uint64_t w0 = begin; w0 < end; w0 += kWave) {
     const uint64_t w = w0 + tid;
-    unsigned long long m = w < end ? eq[w] : 0ull;
+    unsigned long long m = w < end ? tie_word(ws, eq, keep, w) : 0ull;
     const uint32_t mine = __popcll(m);
     uint32_t incl = mine;
 #pragma unroll
@@ -286,9 +310,11 @@ __global__ __launch_bounds__(kBlock) void rank_locate_kernel(RankWs *ws, const u
   }
 }
 
-// in_new = gt | (eq on the needed side of last_row); gt is in_new itself
+// in_new = gt | (eq on the needed side of last_row); gt is in_new itself.  With a keep bitmap the side is taken of
+// eq & keep (mode 1) or of eq & ~keep on top of all of eq & keep (mode 2).
 __global__ __launch_bounds__(kBlock) void rank_combine_kernel(const RankWs *ws, unsigned long long *in_new,
-                                                              const unsigned long long *eq, uint64_t n_words,
+                                                              const unsigned long long *eq,
+                                                              const unsigned long long *keep, uint64_t n_words,
                                                               unsigned long long *observed_to_clear) {
   const uint64_t wl = ws->last_row >> 6;
   const unsigned bl = ws->last_row & 63u;
@@ -297,7 +323,9 @@ __global__ __launch_bounds__(kBlock) void rank_combine_kernel(const RankWs *ws, 
     unsigned long long mask;
     if (upward) mask = w > wl ? ~0ull : (w == wl ? ~0ull << bl : 0ull);
     else mask = w < wl ? ~0ull : (w == wl ? (bl == 63 ? ~0ull : (1ull << (bl + 1)) - 1ull) : 0ull);
-    in_new[w] |= eq[w] & mask;
+    unsigned long long add = tie_word(ws, eq, keep, w) & mask;
+    if (keep && ws->keep_mode == 2) add |= eq[w] & keep[w];
+    in_new[w] |= add;
     if (observed_to_clear) observed_to_clear[w] = 0;  // the counters were reset: no row is observed any more
   }
 }
@@ -320,11 +348,12 @@ __global__ __launch_bounds__(kBlock) void rank_fill_kernel(uint32_t *counts, uin
 }
 
 // ---- bitmaps ----------------------------------------------------------------------------------------------
+constexpr int kBmInvertA = 1, kBmAndB = 2;  // flags: ~a instead of a; & b instead of & ~b
 __device__ __forceinline__ unsigned long long bm_word(const unsigned long long *a, const unsigned long long *b,
-                                                      bool invert_a, uint64_t nbits, uint64_t w) {
+                                                      int flags, uint64_t nbits, uint64_t w) {
   unsigned long long m = a[w];
-  if (invert_a) m = ~m;
-  if (b) m &= ~b[w];
+  if (flags & kBmInvertA) m = ~m;
+  if (b) m &= (flags & kBmAndB) ? b[w] : ~b[w];
   const uint64_t first = w * 64;
   if (nbits - first < 64) m &= (1ull << (nbits - first)) - 1ull;  // the last, partial word
   return m;
@@ -334,9 +363,11 @@ static inline uint64_t bm_words_per_chunk(uint64_t n_words) {
   return ((n_words + kBmChunks - 1) / kBmChunks + kWave - 1) / kWave * kWave;
 }
 
+// gate (may be NULL): the placement whose keep_mode must be 2 for the launch to do anything
 __global__ __launch_bounds__(kBlock) void bitmap_count_kernel(const unsigned long long *a, const unsigned long long *b,
-                                                              int invert_a, uint64_t nbits, uint64_t per_chunk,
-                                                              BmWs *ws) {
+                                                              int flags, uint64_t nbits, uint64_t per_chunk,
+                                                              BmWs *ws, const RankWs *gate) {
+  if (gate && gate->keep_mode != 2) return;
   const int lane = (int)lane_id();
   const uint64_t n_words = (nbits + 63) / 64;
   const uint64_t wave = ((uint64_t)blockIdx.x * kBlock + threadIdx.x) / kWave;
@@ -346,7 +377,7 @@ __global__ __launch_bounds__(kBlock) void bitmap_count_kernel(const unsigned lon
     uint32_t found = 0;
     for (uint64_t w0 = begin; w0 < end; w0 += kWave) {
       const uint64_t w = w0 + lane;
-      uint32_t mine = w < end ? __popcll(bm_word(a, b, invert_a != 0, nbits, w)) : 0u;
+      uint32_t mine = w < end ? __popcll(bm_word(a, b, flags, nbits, w)) : 0u;
 #pragma unroll
       for (int d = kWave / 2; d > 0; d >>= 1) mine += __shfl_xor(mine, d);
       if (lane == 0) ws->block[w0 / kWave] = mine;  // chunks begin on block boundaries
@@ -356,7 +387,8 @@ __global__ __launch_bounds__(kBlock) void bitmap_count_kernel(const unsigned lon
   }
 }
 
-__global__ __launch_bounds__(kBlock) void bitmap_scan_kernel(BmWs *ws, uint32_t *total_host) {
+__global__ __launch_bounds__(kBlock) void bitmap_scan_kernel(BmWs *ws, uint32_t *total_host, const RankWs *gate) {
+  if (gate && gate->keep_mode != 2) return;
   constexpr int kPer = kBmChunks / kBlock;  // 32 chunks per thread
   __shared__ uint32_t part[kBlock];
   const int tid = threadIdx.x;
@@ -383,7 +415,7 @@ __global__ __launch_bounds__(kBlock) void bitmap_scan_kernel(BmWs *ws, uint32_t 
 }
 
 __global__ __launch_bounds__(kBlock) void bitmap_emit_kernel(const unsigned long long *a, const unsigned long long *b,
-                                                             int invert_a, uint64_t nbits, uint64_t per_chunk,
+                                                             int flags, uint64_t nbits, uint64_t per_chunk,
                                                              const BmWs *ws, uint32_t *out, uint64_t max_out) {
   const int lane = (int)lane_id();
   const uint64_t n_words = (nbits + 63) / 64;
@@ -402,7 +434,7 @@ __global__ __launch_bounds__(kBlock) void bitmap_emit_kernel(const unsigned long
     const uint64_t pos0 = (uint64_t)ws->base[chunk] + before;
     if (pos0 >= max_out) continue;
     const uint64_t w = blk * kWave + lane;
-    unsigned long long m = w < n_words ? bm_word(a, b, invert_a != 0, nbits, w) : 0ull;
+    unsigned long long m = w < n_words ? bm_word(a, b, flags, nbits, w) : 0ull;
     const uint32_t mine = __popcll(m);
     uint32_t incl = mine;
 #pragma unroll
@@ -468,7 +500,16 @@ size_t ugk_rank_workspace_bytes(void) { return sizeof(RankWs); }
 
 int ugk_rank_place(uint32_t *counts_dev, uint64_t num_rows, uint64_t k, void *ws_dev, uint64_t *in_new_dev,
                    uint64_t *scratch_bitmap_dev, uint64_t *observed_dev, int reset_counts, void *stream) {
+  return ugk_rank_place_keep(counts_dev, num_rows, k, ws_dev, in_new_dev, scratch_bitmap_dev, observed_dev, nullptr,
+                             reset_counts, stream);
+}
+
+int ugk_rank_place_keep(uint32_t *counts_dev, uint64_t num_rows, uint64_t k, void *ws_dev, uint64_t *in_new_dev,
+                        uint64_t *scratch_bitmap_dev, uint64_t *observed_dev, const uint64_t *keep_dev,
+                        int reset_counts, void *stream) {
   UGK_REQUIRE(counts_dev && ws_dev && in_new_dev && scratch_bitmap_dev, "ugk_rank_place: null pointer");
+  UGK_REQUIRE(keep_dev != in_new_dev && keep_dev != scratch_bitmap_dev,
+              "ugk_rank_place_keep: the keep bitmap is one of the output bitmaps");
   UGK_REQUIRE(num_rows > 0 && num_rows < 0xffffffffull, "ugk_rank_place: %llu rows do not fit 32 bits",
               (unsigned long long)num_rows);
   UGK_REQUIRE((uintptr_t)counts_dev % 16 == 0 && (uintptr_t)ws_dev % 8 == 0, "ugk_rank_place: misaligned buffer");
@@ -477,6 +518,9 @@ int ugk_rank_place(uint32_t *counts_dev, uint64_t num_rows, uint64_t k, void *ws
   unsigned long long *in_new = reinterpret_cast<unsigned long long *>(in_new_dev);
   unsigned long long *eq = reinterpret_cast<unsigned long long *>(scratch_bitmap_dev);
   unsigned long long *observed = reinterpret_cast<unsigned long long *>(observed_dev);
+  const unsigned long long *keep = reinterpret_cast<const unsigned long long *>(keep_dev);
+  const unsigned long long *none = nullptr;
+  const RankWs *no_gate = nullptr;
   const uint64_t n_words = (num_rows + 63) / 64;
   if (k == 0 || k >= num_rows) {  // no row, or every row
     const unsigned grid = clamp_grid(((reset_counts ? num_rows : n_words) + kBlock - 1) / kBlock, 0);
@@ -490,9 +534,9 @@ int ugk_rank_place(uint32_t *counts_dev, uint64_t num_rows, uint64_t k, void *ws
   const unsigned bm_grid = clamp_grid((kBmChunks + (kBlock / kWave) - 1) / (kBlock / kWave), (unsigned)cu_count() * 8u);
   const unsigned word_grid = clamp_grid((n_words + kBlock - 1) / kBlock, 0);
   if (observed) {
-    hipLaunchKernelGGL(bitmap_count_kernel, dim3(bm_grid), dim3(kBlock), 0, st, observed,
-                       (const unsigned long long *)nullptr, 0, num_rows, per_chunk, &ws->bm);
-    hipLaunchKernelGGL(bitmap_scan_kernel, dim3(1), dim3(kBlock), 0, st, &ws->bm, (uint32_t *)nullptr);
+    hipLaunchKernelGGL(bitmap_count_kernel, dim3(bm_grid), dim3(kBlock), 0, st, observed, none, 0, num_rows, per_chunk,
+                       &ws->bm, no_gate);
+    hipLaunchKernelGGL(bitmap_scan_kernel, dim3(1), dim3(kBlock), 0, st, &ws->bm, (uint32_t *)nullptr, no_gate);
     hipLaunchKernelGGL(rank_decide_kernel, dim3(1), dim3(1), 0, st, ws);
     hipLaunchKernelGGL(rank_split_bitmap_kernel, dim3(word_grid), dim3(kBlock), 0, st, counts_dev, num_rows, ws,
                        observed, in_new, eq, reset_counts);
@@ -510,11 +554,23 @@ int ugk_rank_place(uint32_t *counts_dev, uint64_t num_rows, uint64_t k, void *ws
       clamp_grid((n_words + kMarkWords * (kBlock / kWave) - 1) / (kMarkWords * (kBlock / kWave)), 0);
   hipLaunchKernelGGL(rank_split_kernel, dim3(split_grid), dim3(kBlock), 0, st, counts_dev, num_rows, ws, in_new, eq,
                      reset_counts);
-  hipLaunchKernelGGL(bitmap_count_kernel, dim3(bm_grid), dim3(kBlock), 0, st, eq, (const unsigned long long *)nullptr, 0,
-                     num_rows, per_chunk, &ws->bm);
-  hipLaunchKernelGGL(bitmap_scan_kernel, dim3(1), dim3(kBlock), 0, st, &ws->bm, (uint32_t *)nullptr);
-  hipLaunchKernelGGL(rank_locate_kernel, dim3(1), dim3(kBlock), 0, st, ws, eq, num_rows, per_chunk);
-  hipLaunchKernelGGL(rank_combine_kernel, dim3(word_grid), dim3(kBlock), 0, st, ws, in_new, eq, n_words,
+  if (keep) {
+    // rows that tie at the K-th count: the kept ones first.  The second count runs only when they do not suffice.
+    hipLaunchKernelGGL(bitmap_count_kernel, dim3(bm_grid), dim3(kBlock), 0, st, eq, keep, kBmAndB, num_rows, per_chunk,
+                       &ws->bm, no_gate);
+    hipLaunchKernelGGL(bitmap_scan_kernel, dim3(1), dim3(kBlock), 0, st, &ws->bm, (uint32_t *)nullptr, no_gate);
+    hipLaunchKernelGGL(rank_keep_decide_kernel, dim3(1), dim3(1), 0, st, ws);
+    hipLaunchKernelGGL(bitmap_count_kernel, dim3(bm_grid), dim3(kBlock), 0, st, eq, keep, 0, num_rows, per_chunk,
+                       &ws->bm, (const RankWs *)ws);
+    hipLaunchKernelGGL(bitmap_scan_kernel, dim3(1), dim3(kBlock), 0, st, &ws->bm, (uint32_t *)nullptr,
+                       (const RankWs *)ws);
+  } else {
+    hipLaunchKernelGGL(bitmap_count_kernel, dim3(bm_grid), dim3(kBlock), 0, st, eq, none, 0, num_rows, per_chunk,
+                       &ws->bm, no_gate);
+    hipLaunchKernelGGL(bitmap_scan_kernel, dim3(1), dim3(kBlock), 0, st, &ws->bm, (uint32_t *)nullptr, no_gate);
+  }
+  hipLaunchKernelGGL(rank_locate_kernel, dim3(1), dim3(kBlock), 0, st, ws, eq, keep, num_rows, per_chunk);
+  hipLaunchKernelGGL(rank_combine_kernel, dim3(word_grid), dim3(kBlock), 0, st, ws, in_new, eq, keep, n_words,
                      reset_counts ? observed : (unsigned long long *)nullptr);
   UGK_HIP(hipGetLastError());
   return 0;
@@ -540,10 +596,10 @@ int ugk_bitmap_count(const uint64_t *a_dev, const uint64_t *b_dev, int invert_a,
   const unsigned grid = clamp_grid((kBmChunks + (kBlock / kWave) - 1) / (kBlock / kWave), (unsigned)cu_count() * 8u);
   hipLaunchKernelGGL(bitmap_count_kernel, dim3(grid), dim3(kBlock), 0, as_stream(stream),
                      reinterpret_cast<const unsigned long long *>(a_dev),
-                     reinterpret_cast<const unsigned long long *>(b_dev), invert_a, nbits, per_chunk,
-                     static_cast<BmWs *>(ws_dev));
+                     reinterpret_cast<const unsigned long long *>(b_dev), invert_a ? kBmInvertA : 0, nbits,
+                     per_chunk, static_cast<BmWs *>(ws_dev), (const RankWs *)nullptr);
   hipLaunchKernelGGL(bitmap_scan_kernel, dim3(1), dim3(kBlock), 0, as_stream(stream), static_cast<BmWs *>(ws_dev),
-                     total_host);
+                     total_host, (const RankWs *)nullptr);
   UGK_HIP(hipGetLastError());
   return 0;
 }
@@ -561,8 +617,8 @@ int ugk_bitmap_emit(const uint64_t *a_dev, const uint64_t *b_dev, int invert_a, 
   const unsigned grid = clamp_grid((n_blocks + (kBlock / kWave) - 1) / (kBlock / kWave), 0);
   hipLaunchKernelGGL(bitmap_emit_kernel, dim3(grid), dim3(kBlock), 0, as_stream(stream),
                      reinterpret_cast<const unsigned long long *>(a_dev),
-                     reinterpret_cast<const unsigned long long *>(b_dev), invert_a, nbits, per_chunk,
-                     static_cast<const BmWs *>(ws_dev), out_dev, max_out);
+                     reinterpret_cast<const unsigned long long *>(b_dev), invert_a ? kBmInvertA : 0, nbits,
+                     per_chunk, static_cast<const BmWs *>(ws_dev), out_dev, max_out);
   UGK_HIP(hipGetLastError());
   return 0;
 }

@@ -117,6 +117,7 @@ SIGNATURES = {
     "ugk_record_drain": [_vp, _u64, _u64, _vp, _vp, _u32, _vp, _vp, _vp],
     "ugk_rank_workspace_bytes": [],
     "ugk_rank_place": [_vp, _u64, _u64, _vp, _vp, _vp, _vp, C.c_int, _vp],
+    "ugk_rank_place_keep": [_vp, _u64, _u64, _vp, _vp, _vp, _vp, _vp, C.c_int, _vp],
     "ugk_rank_threshold": [_vp, _vp, _vp],
     "ugk_bitmap_workspace_bytes": [],
     "ugk_bitmap_count": [_vp, _vp, C.c_int, _u64, _vp, _vp, _vp],
