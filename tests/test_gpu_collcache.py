@@ -908,15 +908,17 @@ def _random_refresh_case(seed):
                 pct=float(r.choice([0.01, 0.1, 0.37, 0.9, 0.99])), table_kind=str(r.choice(["FLAT", "HASH"])),
                 keep=bool(r.integers(0, 2)), sparse=bool(r.integers(0, 3) == 0), zipf=float(r.choice([0.6, 1.05, 1.4])),
                 rounds=int(r.integers(2, 5)), stream_ordered=bool(r.integers(0, 3) == 0),
-                stage=int(r.choice([0, 256, 65536])))
+                stage=int(r.choice([0, 256, 65536])), stable=bool(r.integers(0, 3) == 0))
 
 
 @pytest.mark.parametrize("case", [_random_refresh_case(i) for i in range(max(24, _SEEDS // 2))],
                          ids=lambda c: "seed%d" % c["seed"])
 def test_random_sequences_of_refreshes_on_the_device(case, monkeypatch):
     """seeded random sweep over table size, cache share (from nearly nothing cached to nearly everything), table kind,
-    sparse ids, accumulating or per-interval hotness: after every refresh computed on the device the cached rows are
-    the oracle's top set of the counted key stream, slots are conserved and lookups reproduce table[keys]"""
+    sparse ids, accumulating or per-interval hotness, ties to row order or to the cached rows first: after every refresh
+    computed on the device the cached rows are the oracle's top set of the counted key stream (with
+    COLL_GPU_REFRESH_STABLE the top set of a full sort by count, cached before, row order), slots are conserved and
+    lookups reproduce table[keys]"""
     monkeypatch.setenv("COLL_HASH_TABLE", "HASH" if case["sparse"] else case["table_kind"])
     monkeypatch.setenv("COLL_GPU_RECORD", "1")
     monkeypatch.setenv("COLL_GPU_REFRESH", "1")
@@ -925,6 +927,8 @@ def test_random_sequences_of_refreshes_on_the_device(case, monkeypatch):
         monkeypatch.setenv("COLL_MISS_STAGE_ROWS", str(case["stage"]))
     if case["keep"]:
         monkeypatch.setenv("COLL_GPU_REFRESH_KEEP", "1")
+    if case["stable"]:
+        monkeypatch.setenv("COLL_GPU_REFRESH_STABLE", "1")
     rng = np.random.default_rng(case["seed"])
     n_item, dim, pct = case["n_item"], case["dim"], case["pct"]
     MUL, BITS = 0x9E3779B97F4A7C15, 40
@@ -945,7 +949,7 @@ def test_random_sequences_of_refreshes_on_the_device(case, monkeypatch):
     table = fill_table(emb, rng)
     co.coll_torch_init_t(0, 0, emb, pct)
     cap = _basics.info(0)["capacity_rows"]
-    _, nid = expected_cached_set(s0.astype(np.uint32), n_item, pct)
+    want, nid = expected_cached_set(s0.astype(np.uint32), n_item, pct)
     counted = []
     for rnd in range(case["rounds"]):
         swap = rng.choice(n_item, max(n_item // 8, 2), replace=False)
@@ -962,7 +966,17 @@ def test_random_sequences_of_refreshes_on_the_device(case, monkeypatch):
             assert out.cpu().numpy().tobytes() == ORC.gather(table, rows.astype(np.int64)).tobytes()
             assert _basics.last_group_offset(0)[1] == int((nid[rows] == 0).sum())
         co.coll_torch_refresh(0, True)
-        want, nid = expected_cached_set(np.concatenate(counted), n_item, pct)
+        if case["stable"]:
+            counts = np.bincount(np.concatenate(counted), minlength=n_item)
+            was = np.zeros(n_item, bool)
+            was[want] = True
+            all_rows = np.arange(n_item, dtype=np.int64)
+            order = np.lexsort((np.where(counts > 0, all_rows, -all_rows), was, counts))[::-1]
+            want = np.sort(order[:len(want)]).astype(np.uint32)
+            nid = np.ones(n_item, nid.dtype)
+            nid[want] = 0
+        else:
+            want, nid = expected_cached_set(np.concatenate(counted), n_item, pct)
         if not case["keep"]:
             counted.clear()
         info = _basics.info(0)
