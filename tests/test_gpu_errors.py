@@ -105,3 +105,25 @@ def test_mock_table_env_is_rejected():
     """, env={"SAMGRAPH_EMPTY_FEAT": "10"})
     assert p.returncode == -6 and "survived" not in p.stdout
     assert "SAMGRAPH_EMPTY_FEAT" in p.stderr
+
+
+@pytest.mark.parametrize("gpu_record", ["0", "1"])
+def test_a_process_that_never_calls_shutdown_still_exits_cleanly(gpu_record):
+    """the serving loop owns a record thread and a refresh thread: a process that just ends (no coll_torch_shutdown,
+    no join of the last refresh) must end with status 0, not in std::terminate or a failed call at unload"""
+    p = run("""
+        n = 60000
+        co.config(cfg(n, 0.2)); co.coll_cache_record_init(0)
+        rng = np.random.default_rng(0)
+        co.coll_torch_record(0, torch.from_numpy(rng.zipf(1.2, 200000) % n).to(torch.int32))
+        emb = co.coll_torch_create_emb_shm(0, n, 32, torch.float32); emb.normal_()
+        co.coll_torch_init_t(0, 0, emb, 0.2)
+        co.coll_torch_forward_config(True, 3, 0.5, True)
+        for step in range(8):
+            keys = torch.from_numpy((rng.zipf(1.1, 20000) + step * 1000) % n).to(torch.int64).cuda()
+            out = co.coll_torch_forward(0, keys)
+            assert torch.equal(out.cpu(), emb[keys.cpu()])
+        print("forwards ok", flush=True)
+    """, env={"COLL_GPU_RECORD": gpu_record, "COLL_REFRESH_SLEEP_US": "20000"})
+    assert "forwards ok" in p.stdout, p.stderr[-2000:]
+    assert p.returncode == 0, p.stderr[-2000:]

@@ -329,7 +329,9 @@ namespace {
  *  caller's stream, so keys that earlier work on that stream produces are complete when they are copied. */
 class RecordWorker {
  public:
-  ~RecordWorker() { Stop(); }
+  // at process exit without coll_cache_shutdown: the thread ends, the stream, event and staging memory are left to
+  // the runtime, which may be half gone by then
+  ~RecordWorker() { Stop(/*release=*/false); }
   /// hands the first `bytes` bytes of `key` (device memory, `key_bytes` per key) to the thread
   void Post(int replica_id, int device, const void *key, size_t num, int key_bytes, StreamHandle stream) {
     Start(device);
@@ -346,7 +348,7 @@ class RecordWorker {
     _cv.wait(g, [this] { return _done; });
     Sample(_waited_s, t.Passed());
   }
-  void Stop() {
+  void Stop(bool release = true) {
     if (!_thread.joinable()) return;
     {
       std::lock_guard<std::mutex> g(_mu);
@@ -360,6 +362,7 @@ class RecordWorker {
                 << " ms, count " << Median(_count_s) * 1e3 << " ms, waited for after the lookup "
                 << Median(_waited_s) * 1e3 << " ms";
     _copy_s.clear(), _count_s.clear(), _waited_s.clear();
+    if (!release) return;
     if (_staging) UGK_CALL(ugk_host_free(_staging));
     UGK_CALL(ugk_event_destroy(_keys_ready));
     UGK_CALL(ugk_stream_destroy(_stream));
@@ -434,6 +437,9 @@ struct ForwardState {
   std::atomic<bool> refresh_ongoing{false};
   std::atomic<uint64_t> refreshes_done{0};
   RecordWorker recorder;  // the host-record path
+  ~ForwardState() {
+    if (refresh_thread.joinable()) refresh_thread.join();  // a process that exits without coll_cache_shutdown
+  }
 };
 ForwardState _forward;
 
