@@ -169,6 +169,10 @@ void CacheContext::build_with_advise_new_hash(int location_id, std::shared_ptr<C
   _new_hash_table->_free_offsets->ForceScale(kI32, {_cache_space_capacity - num_cached_nodes}, CPU_CLIB(), "");
   for (size_t i = 0; i < _cache_space_capacity - num_cached_nodes; i++)
     _new_hash_table->_free_offsets->Ptr<IdType>()[i] = (IdType)(num_cached_nodes + i);
+  // a refresh on the device works on bitmaps of the cached rows and of the taken slots: built now, the first such
+  // refresh does not hold up, for the length of that build, the lookups that share its stream
+  if (RunConfig::gpu_refresh && RunConfig::gpu_record)
+    _new_hash_table->EnsureDeviceLists(_eager_gpu_mem_allocator, _trainer_ctx, stream);
 
   LOG(INFO) << "Asymm Coll cache (policy: " << (int)RunConfig::cache_policy << ") | local " << num_cached_nodes
             << " / " << num_total_nodes << " nodes ( " << ToPercentage(num_cached_nodes / (double)num_total_nodes)
