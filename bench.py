@@ -669,12 +669,13 @@ def run_mixed(args):
     serving = None
     if args.serving:
         # LookupManager::forward (lookup_manager.cc:158-213): every step records the first 5 % of the batch, looks the
-        # batch up (blocking) and, every K/2 steps, starts a refresh on a background thread.  Every step takes a batch
-        # of its own from the workload's distribution, so a refresh gains what the hotness it saw predicts, not the
-        # keys of a pool that comes round again.
-        srv_rows = torch.stack([make_batch() for _ in range(W + K)])
+        # batch up (blocking) and, every K/2 steps, starts a refresh on a background thread.  The steps take fresh
+        # batches from the workload's distribution (up to 256 of them, then round again), so a refresh gains what the
+        # hotness it saw predicts, not the keys of a small pool that comes round every few steps.
+        n_srv = min(W + K, 256)
+        srv_rows = torch.stack([make_batch() for _ in range(n_srv)])
         srv_keys = ids_of(srv_rows)
-        srv_ptrs = [srv_keys[i].data_ptr() for i in range(W + K)]
+        srv_ptrs = [srv_keys[i % n_srv].data_ptr() for i in range(W + K)]
         torch.cuda.synchronize()
         C.coll_cache_forward_config(1, max(K // 2, 1), 0.05, 1)
         for i in range(W):
@@ -696,7 +697,8 @@ def run_mixed(args):
         done = int(C.coll_cache_forward_join())
         join_s = time.perf_counter() - t1
         C.coll_cache_forward_config(0, 0, 0.0, 0)
-        if out.cpu().numpy().tobytes() != orc.gather(table_np, srv_rows[W + K - 1].cpu().numpy(), omp=True).tobytes():
+        if out.cpu().numpy().tobytes() != orc.gather(table_np, srv_rows[(W + K - 1) % n_srv].cpu().numpy(),
+                                                     omp=True).tobytes():
             sys.exit("bench.py: GPU output differs from the CPU oracle in the serving loop")
         med = lambda v: round(float(np.median(v)) * 1e3, 4) if v else None
         serving = {"ms_per_step": el / K * 1e3, "keys_per_s": n_keys * K / el, "steps": K,
@@ -707,7 +709,7 @@ def run_mixed(args):
                    "recorded_fraction": 0.05, "refresh_every_steps": max(K // 2, 1), "refreshes_completed": done,
                    "seconds_waited_for_the_last_refresh": join_s,
                    "hotness_recorded_on": "device" if args.gpu_record else "host",
-                   "batches": "one fresh batch per step",
+                   "batches": "%d fresh batches, one per step, cycled" % n_srv,
                    "entry_point": "coll_cache_forward_i64 (record a prefix + blocking lookup + background refresh)"}
         note("serving loop: %.3f ms/step (median %s before, %s during, %s after the refresh; longest %.2f ms), "
              "%d refreshes" % (serving["ms_per_step"], med(before), med(during), med(after_r),

@@ -89,7 +89,7 @@ typedef struct {
 const char *ugk_last_error(void);
 /* version of this ABI; bumped on any signature change.  ugk_abi_version() is what the loaded library was built with:
  * a caller compiled against another UGK_ABI_VERSION must not go on. */
-#define UGK_ABI_VERSION 10
+#define UGK_ABI_VERSION 11
 int ugk_abi_version(void);
 
 /* ---- runtime plumbing: Device::{AllocDataSpace,FreeDataSpace,CopyDataFromTo,StreamSync,CreateStream}
@@ -275,7 +275,10 @@ int ugk_extract_mix_i64(ugk_table_t t, const int64_t *keys_dev, size_t n, const 
  * is there, and adds the number of such rows to *staged_dev (device word, may be NULL).  With rest_count_dev (device
  * word, zero on entry; NULL = off) the rows the stage does not hold are not copied but listed, in any order, as
  * rest_rows_dev[j] / rest_dst_off_dev[j] for j < *rest_count_dev (lists of n words each): a background refresh copies
- * those itself, throttled, over the host link.  Results are the same
+ * those itself, throttled, over the host link.  With done_count_dev as well (device word, zero on entry; needs the
+ * rest lists) the rows that were copied out of the stage are listed too, from the back of the same lists:
+ * rest_rows_dev[n - 1 - j] / rest_dst_off_dev[n - 1 - j] for j < *done_count_dev, so that a caller can publish them
+ * in its table before the rest has arrived.  Results are the same
  * bytes with and without a stage: the host table does not change under a cache.  An entry is only consistent at launch
  * boundaries, so the staged gather must not read a stage that an extraction in flight writes (a caller with lookups
  * running beside its refreshes keeps two stages and reads the one the lookups have been switched away from).
@@ -301,7 +304,7 @@ int ugk_gather_scatter_staged_u32(const void *host_dev, uint64_t host_rows, cons
                                   const uint32_t *dst_off_dev, size_t n, void *out_dev, uint64_t out_rows,
                                   size_t row_bytes, ugk_stage_t stage, unsigned max_blocks, uint32_t *status_dev,
                                   uint32_t *staged_dev, uint32_t *rest_rows_dev, uint32_t *rest_dst_off_dev,
-                                  uint32_t *rest_count_dev, void *stream);
+                                  uint32_t *rest_count_dev, uint32_t *done_count_dev, void *stream);
 
 /* ---- key dedup (the caller-side array_ops.unique of
  *      python_tf2/collcache_tf2/collcache_tf2/core/sparse_lookup_layer.py:197) ------------------------

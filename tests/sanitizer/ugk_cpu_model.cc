@@ -672,9 +672,10 @@ int ugk_extract_mix_staged_i64(ugk_table_t t, const int64_t *keys, size_t n, con
 int ugk_gather_scatter_staged_u32(const void *host, uint64_t host_rows, const uint32_t *rows, const uint32_t *dst,
                                   size_t n, void *out, uint64_t out_rows, size_t rb, ugk_stage_t stage, unsigned,
                                   uint32_t *status, uint32_t *staged, uint32_t *rest_rows, uint32_t *rest_dst,
-                                  uint32_t *rest_count, void *) {
+                                  uint32_t *rest_count, uint32_t *done_count, void *) {
   if (n == 0) return 0;
   REQUIRE(host && rows && dst && out && status && stage.rows_dev && stage.owner_dev, "staged gather: null pointer");
+  REQUIRE(done_count == nullptr || rest_count, "staged gather: a done count without rest lists");
   for (size_t i = 0; i < n; ++i) {
     const uint64_t r = rows[i];
     if (r >= host_rows || dst[i] >= out_rows) {
@@ -692,6 +693,11 @@ int ugk_gather_scatter_staged_u32(const void *host, uint64_t host_rows, const ui
     copy_row((char *)out + (size_t)dst[i] * rb, filed ? (const char *)stage.rows_dev + h * rb : (const char *)host + r * rb,
              rb);
     if (filed && staged) ++*staged;
+    if (filed && done_count) {
+      const size_t at = n - 1 - (*done_count)++;
+      rest_rows[at] = (uint32_t)r;
+      rest_dst[at] = dst[i];
+    }
   }
   return 0;
 }

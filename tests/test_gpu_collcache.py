@@ -507,6 +507,63 @@ def test_refresh_on_the_device_places_like_the_oracle(table_kind, foreground, ke
 
 
 @pytest.mark.parametrize("table_kind", ["FLAT", "HASH"])
+@pytest.mark.parametrize("kind", ["host", "device", "device_staged"])
+def test_rows_of_a_background_refresh_hit_as_they_arrive(table_kind, kind, monkeypatch):
+    """a background refresh copies its rows in throttled batches and publishes every batch behind its copy: lookups of
+    the rows that come in, run beside the refresh, find more and more of them in the cache (never fewer), some of them
+    long before the refresh ends, and always return table[keys]"""
+    monkeypatch.setenv("COLL_HASH_TABLE", table_kind)
+    monkeypatch.setenv("COLL_REFRESH_SLEEP_US", "4000")
+    monkeypatch.setenv("COLL_REFRESH_BATCH_ROWS", "200")
+    if kind != "host":
+        monkeypatch.setenv("COLL_GPU_RECORD", "1")
+        monkeypatch.setenv("COLL_GPU_REFRESH", "1")
+    if kind == "device_staged":
+        monkeypatch.setenv("COLL_MISS_STAGE_ROWS", "2048")
+    rng = np.random.default_rng(77)
+    n_item, dim, pct = 50_000, 32, 0.2
+    co.config(make_config(n_item, pct))
+    co.coll_cache_record_init(0)
+    perm = rng.permutation(n_item)
+    s0 = perm[zipf_ranks(rng, 150_000, n_item, 1.05)]
+    co.coll_torch_record(0, torch.from_numpy(s0).to(torch.int32))
+    emb = co.coll_torch_create_emb_shm(0, n_item, dim, torch.float32)
+    table = fill_table(emb, rng)
+    co.coll_torch_init_t(0, 0, emb, pct)
+    old, _ = expected_cached_set(s0.astype(np.uint32), n_item, pct)
+    # the hot set moves to the other end of the permutation
+    s1 = perm[::-1][zipf_ranks(rng, 150_000, n_item, 1.05)].copy()
+    if kind == "host":
+        co.coll_torch_record(0, torch.from_numpy(s1).to(torch.int32))
+    else:
+        for part in np.array_split(s1, 3):
+            out = co.coll_torch_lookup_key_t_val_ret(0, torch.from_numpy(part).to(torch.int32).cuda(), False)
+            assert out.cpu().numpy().tobytes() == ORC.gather(table, part.astype(np.int64)).tobytes()
+    new, _ = expected_cached_set(s1.astype(np.uint32), n_item, pct)
+    coming = np.setdiff1d(new, old)
+    assert len(coming) > 5_000
+    probe = torch.from_numpy(coming.astype(np.int32)).cuda()
+    want = ORC.gather(table, coming.astype(np.int64)).tobytes()
+    t = threading.Thread(target=co.coll_torch_refresh, args=(0, False))
+    t.start()
+    hits = []
+    while t.is_alive():
+        out = co.coll_torch_lookup_key_t_val_ret(0, probe, False)
+        assert out.cpu().numpy().tobytes() == want
+        hits.append(_basics.last_group_offset(0)[1])
+        time.sleep(0.002)
+    t.join()
+    out = co.coll_torch_lookup_key_t_val_ret(0, probe, False)
+    assert out.cpu().numpy().tobytes() == want
+    assert _basics.last_group_offset(0)[1] == len(coming)  # all of them cached in the end
+    assert hits == sorted(hits), hits
+    assert hits[0] < len(coming) // 4 and any(len(coming) // 4 < h < len(coming) for h in hits), hits[::5]
+    got = np.zeros(len(new), np.uint32)
+    assert _basics.C_LIB_CTYPES.coll_cache_get_cached_keys(0, got.ctypes.data, len(got)) == len(new)
+    assert np.array_equal(got, new)
+
+
+@pytest.mark.parametrize("table_kind", ["FLAT", "HASH"])
 @pytest.mark.parametrize("foreground", [True, False])
 @pytest.mark.parametrize("keep", [False, True])
 def test_stable_refresh_on_the_device_moves_only_rows_the_counters_tell_apart(table_kind, foreground, keep,

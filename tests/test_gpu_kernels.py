@@ -655,7 +655,7 @@ def test_rows_from_the_host_are_filed_in_the_stage_and_found_there(kind, rb):
         stage = hip.Stage(ptr(stage_rows), ptr(owner), entries - 1, 0, 0)
         for cap in (0, 7):
             hip.call("ugk_gather_scatter_staged_u32", pin.ptr, nkeys, ptr(d_take), ptr(d_dst), len(take), ptr(out),
-                     out_rows, rb, stage, cap, ptr(st), ptr(n_staged), None, None, None, None)
+                     out_rows, rb, stage, cap, ptr(st), ptr(n_staged), None, None, None, None, None)
         sync()
         assert status_value(st) == 0
         want = np.full((out_rows, rb), 0x11, np.uint8)
@@ -666,14 +666,21 @@ def test_rows_from_the_host_are_filed_in_the_stage_and_found_there(kind, rb):
         # with a rest list: only what the stage holds is copied, the other rows are listed with their destinations
         out2 = dev_bytes(out_rows * rb, fill=0x11)
         rest_rows, rest_dst, rest_n = dev_zeros_u32(len(take)), dev_zeros_u32(len(take)), dev_zeros_u32(1)
+        done_n = dev_zeros_u32(1)
         hip.call("ugk_gather_scatter_staged_u32", pin.ptr, nkeys, ptr(d_take), ptr(d_dst), len(take), ptr(out2),
-                 out_rows, rb, stage, 3, ptr(st), None, ptr(rest_rows), ptr(rest_dst), ptr(rest_n), None)
+                 out_rows, rb, stage, 3, ptr(st), None, ptr(rest_rows), ptr(rest_dst), ptr(rest_n), ptr(done_n), None)
         sync()
         assert status_value(st) == 0
         m = int(to_np(rest_n, np.uint32)[0])
         assert m == int((~in_stage).sum())
         got_rest = sorted(zip(to_np(rest_rows, np.uint32)[:m].tolist(), to_np(rest_dst, np.uint32)[:m].tolist()))
         assert got_rest == sorted(zip(take[~in_stage].tolist(), dst[~in_stage].tolist()))
+        # ... and the rows that were copied, from the back of the same lists
+        k = int(to_np(done_n, np.uint32)[0])
+        assert k == int(in_stage.sum()) and k + m == len(take)
+        got_done = sorted(zip(to_np(rest_rows, np.uint32)[m:len(take)].tolist(),
+                              to_np(rest_dst, np.uint32)[m:len(take)].tolist()))
+        assert got_done == sorted(zip(take[in_stage].tolist(), dst[in_stage].tolist()))
         want2 = np.full((out_rows, rb), 0x11, np.uint8)
         want2[dst[in_stage]] = host[take[in_stage]]
         assert to_np(out2)[: out_rows * rb].tobytes() == want2.tobytes()

@@ -1037,51 +1037,64 @@ void RefreshSession::WaitForOneLookup(ExtractSession *session, bool foreground) 
 void RefreshSession::CopyRowsIntoSlots(const uint32_t *rows_dev, const uint32_t *slots_dev, size_t num_rows,
                                        bool foreground, StreamHandle copy_stream, const ugk_stage_t *stage) {
   CacheContext *ctx = _cache_ctx.get();
+  auto table = ctx->_new_hash_table;
+  const Context gpu_ctx = ctx->_trainer_ctx;
+  const int local = ctx->_local_location_id;
   const void *host = ctx->_device_cache_data[ctx->_cpu_location_id];
   void *cache = ctx->_device_cache_data[ctx->_local_location_id];
-  uint32_t *status = _status_handle->ptr<uint32_t>();  // [0] error bits, [8] rows taken from the stage, [9] rows left
-  if (stage) {
-    // Most of the rows a refresh brings in were missed by the last few lookups, which filed them in HBM.  A foreground
-    // refresh takes every row in one launch, from the stage or from the host table.  A background one takes what the
-    // stage holds in one launch (HBM to HBM, nothing for the lookups to share the link with) and is left with a short
-    // list for the throttled copy below.
-    if (foreground) {
+  // [0] error bits, [8] rows taken from the stage so far, [9] rows left for the link, [10] rows taken this time
+  uint32_t *status = _status_handle->ptr<uint32_t>();
+  // the rows of a list, or of a part of one, become visible to lookups: behind their copy on the same stream
+  auto publish = [&](const uint32_t *rows, const uint32_t *slots, size_t n) {
+    table->PublishRows(rows, slots, n, local, __publish_ids, ctx->_eager_gpu_mem_allocator, gpu_ctx, copy_stream);
+  };
+  if (foreground) {
+    // Nothing runs beside a foreground refresh: one launch copies every row, from the stage where it holds it (most of
+    // the rows a refresh brings in were missed by the last few lookups, which filed them in HBM) or from the host
+    // table, on a capped grid: rows of 512 bytes and more cross the link faster from 128 workgroups than from as many
+    // as the rows would fill (56.9 against 52.7 GB/s).  One more launch publishes them.
+    if (stage)
       UGK_CALL(ugk_gather_scatter_staged_u32(host, ctx->_num_total_nodes, rows_dev, slots_dev, num_rows, cache,
                                              ctx->_cache_space_capacity, ctx->_row_bytes, *stage, 0, status, status + 8,
-                                             nullptr, nullptr, nullptr, copy_stream));
-      num_rows = 0;
-    } else {
-      const Context gpu_ctx = ctx->_trainer_ctx;
+                                             nullptr, nullptr, nullptr, nullptr, copy_stream));
+    else
+      UGK_CALL(ugk_gather_scatter_u32(host, ctx->_num_total_nodes, rows_dev, slots_dev, num_rows, cache,
+                                      ctx->_cache_space_capacity, ctx->_row_bytes, 128, status, nullptr, copy_stream));
+    publish(rows_dev, slots_dev, num_rows);
+  } else {
+    if (stage) {
+      // A background refresh takes what the stage holds in one launch (HBM to HBM, nothing for the lookups to share the
+      // link with), publishes those rows at once and is left with a short list for the throttled copy below.
       TensorPtr rest_rows = Empty1DReuse(__rest_rows, kI32, {num_rows}, gpu_ctx);
       TensorPtr rest_slots = Empty1DReuse(__rest_slots, kI32, {num_rows}, gpu_ctx);
-      UGK_CALL(ugk_fill_u32(status + 9, 0, 1, copy_stream));
+      UGK_CALL(ugk_fill_u32(status + 9, 0, 2, copy_stream));
       UGK_CALL(ugk_gather_scatter_staged_u32(host, ctx->_num_total_nodes, rows_dev, slots_dev, num_rows, cache,
                                              ctx->_cache_space_capacity, ctx->_row_bytes, *stage,
                                              RunConfig::refresh_limit_block, status, status + 8,
                                              rest_rows->Ptr<uint32_t>(), rest_slots->Ptr<uint32_t>(), status + 9,
-                                             copy_stream));
-      uint32_t left = 0;
-      UGK_CALL(ugk_memcpy_async(&left, status + 9, sizeof(left), copy_stream));
+                                             status + 10, copy_stream));
+      uint32_t left_done[2] = {0, 0};
+      UGK_CALL(ugk_memcpy_async(left_done, status + 9, sizeof(left_done), copy_stream));
       UGK_CALL(ugk_stream_sync(copy_stream));
-      CHECK_LE((size_t)left, num_rows);
+      CHECK_LE((size_t)left_done[0] + left_done[1], num_rows);
       rows_dev = rest_rows->CPtr<uint32_t>();
       slots_dev = rest_slots->CPtr<uint32_t>();
-      num_rows = left;
+      publish(rows_dev + (num_rows - left_done[1]), slots_dev + (num_rows - left_done[1]), left_done[1]);
+      num_rows = left_done[0];
     }
-  }
-  // background refresh copies in small throttled batches so that foreground lookups keep the host link; alone on the
-  // chip the copy still takes a capped grid: rows of 512 bytes and more cross the link faster from 128 workgroups than
-  // from as many as the rows would fill (56.9 against 52.7 GB/s)
-  const size_t batch = foreground ? num_rows : std::max<size_t>(RunConfig::refresh_batch_rows, 1);
-  const unsigned limit_block = foreground ? 128 : RunConfig::refresh_limit_block;
-  for (size_t begin = 0; begin < num_rows; begin += batch) {
-    const size_t cur = std::min(batch, num_rows - begin);
-    UGK_CALL(ugk_gather_scatter_u32(host, ctx->_num_total_nodes, rows_dev + begin, slots_dev + begin, cur, cache,
-                                    ctx->_cache_space_capacity, ctx->_row_bytes, limit_block, status, nullptr,
-                                    copy_stream));
-    if (!foreground && begin + batch < num_rows) {
-      UGK_CALL(ugk_stream_sync(copy_stream));
-      usleep(RunConfig::refresh_sleep_us);
+    // the rest crosses the link in small throttled batches so that the lookups keep it (cache_context.cu:4054-4090);
+    // every batch is published behind its copy, so its rows hit from then on
+    const size_t batch = std::max<size_t>(RunConfig::refresh_batch_rows, 1);
+    for (size_t begin = 0; begin < num_rows; begin += batch) {
+      const size_t cur = std::min(batch, num_rows - begin);
+      UGK_CALL(ugk_gather_scatter_u32(host, ctx->_num_total_nodes, rows_dev + begin, slots_dev + begin, cur, cache,
+                                      ctx->_cache_space_capacity, ctx->_row_bytes, RunConfig::refresh_limit_block,
+                                      status, nullptr, copy_stream));
+      publish(rows_dev + begin, slots_dev + begin, cur);
+      if (begin + batch < num_rows) {
+        UGK_CALL(ugk_stream_sync(copy_stream));
+        usleep(RunConfig::refresh_sleep_us);
+      }
     }
   }
   if (copy_stream == stream) return;  // the caller looks at the status word when it waits for its stream
@@ -1180,12 +1193,7 @@ void RefreshSession::refresh_after_solve_new(bool foreground) {
     auto reserved_offset =
         CopyTo1DReuse(__offs_buffer, table->ReserveOffsetFront((IdType)num_insert), gpu_ctx, low_pri_stream);
     CopyRowsIntoSlots(insert_keys_gpu->CPtr<uint32_t>(), reserved_offset->CPtr<uint32_t>(), num_insert, foreground,
-                      low_pri_stream, stage);
-    auto insert_table_keys =
-        RunConfig::key_map_mul == 0
-            ? insert_keys_gpu
-            : table->TableKeysToDevice(new_insert_keys, ctx->_eager_gpu_mem_allocator, gpu_ctx, stream);
-    table->InsertWithLoc(insert_table_keys, reserved_offset, local, stream);
+                      low_pri_stream, stage);  // waits for the copy stream: rows copied and published
     table->CheckStatus(stream, "refresh insert");
   }
   AnonymousBarrier::_refresh_instance->Wait();
@@ -1288,8 +1296,6 @@ void RefreshSession::refresh_on_device(ExtractSession *session, size_t num_cache
     // the slots taken are the lowest free ones: every bit up to the last of them is set now
     UGK_CALL(ugk_bitmap_set_through(table->SlotUsedBits(), capacity, slots->CPtr<uint32_t>() + (num_insert - 1),
                                     _status_handle->ptr<uint32_t>(), stream));
-    TensorPtr insert_keys = table->RowsToTableKeys(insert_rows, __insert_ids, alloc, gpu_ctx, stream);
-    table->InsertWithLoc(insert_keys, slots, local, stream);
   }
   uint32_t stw[9] = {0};  // [0] status bits, [8] rows taken from the stage so far
   UGK_CALL(ugk_memcpy_async(stw, _status_handle->ptr<uint32_t>(), sizeof(stw), stream));

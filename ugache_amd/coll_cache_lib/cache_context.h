@@ -290,13 +290,15 @@ class RefreshSession {
   // rows the refreshes of this session have taken from the stage instead of the host table so far (blocks)
   uint64_t RowsFromStage();
  private:
-  // copies the listed host rows into the listed cache slots (step 6): in one launch when in the foreground, in
-  // small throttled batches behind running lookups otherwise
+  // copies the listed host rows into the listed cache slots and publishes them in the table (step 6): in one launch
+  // each when in the foreground; behind running lookups in small throttled batches, every batch published as soon as
+  // it has arrived, so the hit rate climbs while the refresh runs instead of at its end
   void CopyRowsIntoSlots(const uint32_t *rows_dev, const uint32_t *slots_dev, size_t num_rows, bool foreground,
                          StreamHandle copy_stream, const ugk_stage_t *stage);
+  TensorPtr __publish_ids;  // table keys of the rows being published (sparse ids)
   TensorPtr __keys_buffer;
   TensorPtr __offs_buffer;
-  TensorPtr __evict_rows, __insert_rows, __free_slots, __evict_ids, __insert_ids, __evict_slots;
+  TensorPtr __evict_rows, __insert_rows, __free_slots, __evict_ids, __evict_slots;
   MemHandle _status_handle;
 };
 

@@ -215,6 +215,20 @@ TensorPtr CacheEntryManager::RowsToTableKeys(TensorPtr rows_dev, TensorPtr &buff
   return ids;
 }
 
+void CacheEntryManager::PublishRows(const uint32_t *rows_dev, const uint32_t *slots_dev, size_t n, int loc,
+                                    TensorPtr &id_buffer, const std::function<MemHandle(size_t)> &allocator,
+                                    Context ctx, StreamHandle stream) {
+  if (n == 0) return;
+  if (RunConfig::key_map_mul == 0) {
+    UGK_CALL(ugk_table_insert_u32(_table, rows_dev, slots_dev, 0, (uint32_t)loc, n, StatusPtr(this, stream), stream));
+    return;
+  }
+  TensorPtr ids = ReuseList(id_buffer, kI64, n, allocator, ctx);
+  UGK_CALL(ugk_rows_to_keys(rows_dev, n, RunConfig::key_map_mul, RunConfig::key_map_mask, ids->Ptr<int64_t>(), stream));
+  UGK_CALL(ugk_table_insert_i64(_table, ids->CPtr<int64_t>(), slots_dev, 0, (uint32_t)loc, n, StatusPtr(this, stream),
+                                stream));
+}
+
 void CacheEntryManager::EnsureDeviceLists(const std::function<MemHandle(size_t)> &allocator, Context ctx,
                                           StreamHandle stream) {
   const size_t row_words = (num_total_key + 63) / 64, slot_words = ((size_t)_cache_space_capacity + 63) / 64;

@@ -130,6 +130,9 @@ class CacheEntryManager {
   // device list of host rows -> device list of table keys (the rows themselves, or their ids in sparse-id mode)
   TensorPtr RowsToTableKeys(TensorPtr rows_dev, TensorPtr &buffer, const std::function<MemHandle(size_t)> &allocator,
                             Context ctx, StreamHandle stream);
+  // InsertWithLoc for device lists of host rows and their slots (raw pointers: parts of longer lists)
+  void PublishRows(const uint32_t *rows_dev, const uint32_t *slots_dev, size_t n, int loc, TensorPtr &id_buffer,
+                   const std::function<MemHandle(size_t)> &allocator, Context ctx, StreamHandle stream);
 
   // cuh:693-740 — keys of `inputs` satisfying cond, in input order (deterministic, unlike the reference's
   // thread-interleaved order)

@@ -156,7 +156,8 @@ __global__ __launch_bounds__(kBlock) void gather_staged_kernel(const u32x4 *__re
                                                                u32x4 *__restrict__ out, uint64_t out_rows, uint32_t vpr,
                                                                uint32_t lpr, ugk_stage_t stage, uint32_t *status,
                                                                uint32_t *staged, uint32_t *rest_rows,
-                                                               uint32_t *rest_dst, uint32_t *rest_count) {
+                                                               uint32_t *rest_dst, uint32_t *rest_count,
+                                                               uint32_t *done_count) {
   constexpr int UNROLL = 2;
   __shared__ uint32_t block_staged;
   if (threadIdx.x == 0) block_staged = 0;
@@ -190,6 +191,12 @@ __global__ __launch_bounds__(kBlock) void gather_staged_kernel(const u32x4 *__re
           rest_dst[at] = (uint32_t)d[u];
         }
         ok[u] = false;
+      }
+      if (done_count && filed && lane == 0) {
+        // copied here: listed from the back of the same lists, for a caller that publishes rows as they arrive
+        const uint32_t at = (uint32_t)n - 1u - atomicAdd(done_count, 1u);
+        rest_rows[at] = (uint32_t)s;
+        rest_dst[at] = (uint32_t)d[u];
       }
       src[u] = !ok[u] ? reinterpret_cast<const u32x4 *>(out) : filed ? stage_rows + h * vpr : host + s * vpr;
       if (filed && lane == 0) ++mine;
@@ -368,10 +375,12 @@ int ugk_gather_scatter_staged_u32(const void *host_dev, uint64_t host_rows, cons
                                   const uint32_t *dst_off_dev, size_t n, void *out_dev, uint64_t out_rows,
                                   size_t row_bytes, ugk_stage_t stage, unsigned max_blocks, uint32_t *status_dev,
                                   uint32_t *staged_dev, uint32_t *rest_rows_dev, uint32_t *rest_dst_dev,
-                                  uint32_t *rest_count_dev, void *stream) {
+                                  uint32_t *rest_count_dev, uint32_t *done_count_dev, void *stream) {
   if (n == 0) return 0;
   UGK_REQUIRE(rest_count_dev == nullptr || (rest_rows_dev && rest_dst_dev),
               "ugk_gather_scatter_staged_u32: a rest count without the two rest lists");
+  UGK_REQUIRE(done_count_dev == nullptr || rest_count_dev, "ugk_gather_scatter_staged_u32: a done count without rest lists");
+  UGK_REQUIRE(n <= 0xffffffffull, "ugk_gather_scatter_staged_u32: %zu rows do not fit 32-bit list positions", n);
   UGK_REQUIRE(host_dev && rows_dev && dst_off_dev && out_dev && status_dev, "ugk_gather_scatter_staged_u32: null pointer");
   UGK_REQUIRE(stage.rows_dev && stage.owner_dev && ((stage.mask + 1) & stage.mask) == 0,
               "ugk_gather_scatter_staged_u32: the stage needs buffers and a power of two of entries");
@@ -387,7 +396,7 @@ int ugk_gather_scatter_staged_u32(const void *host_dev, uint64_t host_rows, cons
   hipLaunchKernelGGL(gather_staged_kernel, dim3(grid), dim3(kBlock), 0, as_stream(stream),
                      reinterpret_cast<const u32x4 *>(host_dev), host_rows, rows_dev, dst_off_dev, n,
                      reinterpret_cast<u32x4 *>(out_dev), out_rows, vpr, lpr, stage, status_dev, staged_dev,
-                     rest_rows_dev, rest_dst_dev, rest_count_dev);
+                     rest_rows_dev, rest_dst_dev, rest_count_dev, done_count_dev);
   UGK_HIP(hipGetLastError());
   return 0;
 }

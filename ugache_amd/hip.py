@@ -107,7 +107,7 @@ SIGNATURES = {
     "ugk_extract_mix_staged_u32": [Table, _vp, _sz, _vp, _u64, _vp, _u64, _vp, _sz, _vp, _vp, _vp, _vp, _u32, Stage, _vp],
     "ugk_extract_mix_staged_i64": [Table, _vp, _sz, _vp, _u64, _vp, _u64, _vp, _sz, _vp, _vp, _vp, _vp, _u32, Stage, _vp],
     "ugk_gather_scatter_staged_u32": [_vp, _u64, _vp, _vp, _sz, _vp, _u64, _sz, Stage, C.c_uint, _vp, _vp, _vp, _vp,
-                                      _vp, _vp],
+                                      _vp, _vp, _vp],
     "ugk_dedup_workspace_bytes": [_sz],
     "ugk_dedup_u32": [_vp, _sz, _vp, _sz, _u32, _vp, _vp, _vp, _vp, _vp, _vp],
     "ugk_dedup_i64": [_vp, _sz, _vp, _sz, _u32, _vp, _vp, _vp, _vp, _vp, _vp],
