@@ -43,7 +43,7 @@ def make_config(num_total_item, pct, threads=8):
 def _fresh_cache(monkeypatch):
     for v in ("COLL_HASH_TABLE", "SAMGRAPH_COLL_CACHE_CONCURRENT_LINK_IMPL", "SAMGRAPH_COLL_CACHE_NO_GROUP",
               "COLL_DEDUP_KEYS", "COLL_DEDUP_MIN_KEYS", "COLL_GPU_RECORD", "COLL_GPU_RECORD_EVERY", "COLL_GPU_REFRESH",
-              "COLL_GPU_REFRESH_KEEP", "COLL_GPU_REFRESH_STABLE"):
+              "COLL_GPU_REFRESH_KEEP", "COLL_GPU_REFRESH_STABLE", "COLL_REFRESH_RATE_GBPS"):
         monkeypatch.delenv(v, raising=False)
     yield
     if torch.cuda.is_available():
@@ -504,6 +504,49 @@ def test_refresh_on_the_device_places_like_the_oracle(table_kind, foreground, ke
     cached, nid = expected_cached_set(np.concatenate(counted), n_item, pct)
     check_cached(cached)
     lookup(rng.integers(0, n_item, size=20_000), nid)
+
+
+def test_background_refresh_paced_by_a_rate_over_the_link(monkeypatch):
+    """COLL_REFRESH_RATE_GBPS: the throttled copy of a background refresh pauses after each batch for as long as keeps
+    it at that rate (instead of the fixed pause): same cached set, and the copy cannot have gone faster than asked"""
+    monkeypatch.setenv("COLL_REFRESH_BATCH_ROWS", "500")
+    monkeypatch.setenv("COLL_REFRESH_SLEEP_US", "1000000")  # would make this refresh take half a minute if it were used
+    monkeypatch.setenv("COLL_REFRESH_RATE_GBPS", "0.004")
+    rng = np.random.default_rng(78)
+    n_item, dim, pct = 50_000, 32, 0.2
+    co.config(make_config(n_item, pct))
+    co.coll_cache_record_init(0)
+    perm = rng.permutation(n_item)
+    s0 = perm[zipf_ranks(rng, 150_000, n_item, 1.05)]
+    co.coll_torch_record(0, torch.from_numpy(s0).to(torch.int32))
+    emb = co.coll_torch_create_emb_shm(0, n_item, dim, torch.float32)
+    table = fill_table(emb, rng)
+    co.coll_torch_init_t(0, 0, emb, pct)
+    old, _ = expected_cached_set(s0.astype(np.uint32), n_item, pct)
+    s1 = perm[::-1][zipf_ranks(rng, 150_000, n_item, 1.05)].copy()
+    co.coll_torch_record(0, torch.from_numpy(s1).to(torch.int32))
+    new, nid = expected_cached_set(s1.astype(np.uint32), n_item, pct)
+    n_coming = len(np.setdiff1d(new, old))
+    t = threading.Thread(target=co.coll_torch_refresh, args=(0, False))
+    t0 = time.perf_counter()
+    t.start()
+    keys = rng.integers(0, n_item, size=3_000)
+    want = ORC.gather(table, keys).tobytes()
+    while t.is_alive():
+        out = co.coll_torch_lookup_key_t_val_ret(0, torch.from_numpy(keys).cuda(), False)
+        assert out.cpu().numpy().tobytes() == want
+        time.sleep(0.002)
+    t.join()
+    took = time.perf_counter() - t0
+    # all batches but the last are followed by their pause: (n - 500) rows of 128 bytes at 4 MB/s
+    assert took >= 0.9 * (n_coming - 500) * dim * 4 / 0.004e9, (took, n_coming)
+    assert took < 20
+    got = np.zeros(len(new), np.uint32)
+    assert _basics.C_LIB_CTYPES.coll_cache_get_cached_keys(0, got.ctypes.data, len(got)) == len(new)
+    assert np.array_equal(got, new)
+    out = co.coll_torch_lookup_key_t_val_ret(0, torch.from_numpy(keys).cuda(), False)
+    assert out.cpu().numpy().tobytes() == want
+    assert _basics.last_group_offset(0)[1] == int((nid[keys] == 0).sum())
 
 
 @pytest.mark.parametrize("table_kind", ["FLAT", "HASH"])

@@ -1087,13 +1087,20 @@ void RefreshSession::CopyRowsIntoSlots(const uint32_t *rows_dev, const uint32_t 
     const size_t batch = std::max<size_t>(RunConfig::refresh_batch_rows, 1);
     for (size_t begin = 0; begin < num_rows; begin += batch) {
       const size_t cur = std::min(batch, num_rows - begin);
+      Timer t_batch;
       UGK_CALL(ugk_gather_scatter_u32(host, ctx->_num_total_nodes, rows_dev + begin, slots_dev + begin, cur, cache,
                                       ctx->_cache_space_capacity, ctx->_row_bytes, RunConfig::refresh_limit_block,
                                       status, nullptr, copy_stream));
       publish(rows_dev + begin, slots_dev + begin, cur);
       if (begin + batch < num_rows) {
         UGK_CALL(ugk_stream_sync(copy_stream));
-        usleep(RunConfig::refresh_sleep_us);
+        if (RunConfig::refresh_rate_gbps > 0) {
+          // a share of the link instead of a fixed pause: the batch should have taken bytes / rate
+          const double due_s = (double)cur * ctx->_row_bytes / (RunConfig::refresh_rate_gbps * 1e9) - t_batch.Passed();
+          if (due_s > 0) usleep((useconds_t)(due_s * 1e6));
+        } else {
+          usleep(RunConfig::refresh_sleep_us);
+        }
       }
     }
   }

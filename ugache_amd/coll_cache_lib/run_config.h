@@ -63,6 +63,9 @@ struct RunConfig {
   static size_t refresh_batch_rows;    // COLL_REFRESH_BATCH_ROWS, default 4092 (cache_context.cu:4057)
   static unsigned refresh_sleep_us;    // COLL_REFRESH_SLEEP_US, default 3000 (cache_context.cu:4069)
   static unsigned refresh_limit_block; // COLL_REFRESH_LIMIT_BLOCK, default 20 (cache_context.cu:4068)
+  // COLL_REFRESH_RATE_GBPS, default 0 = off: instead of the fixed sleep, a background refresh sleeps after each batch
+  // for as long as keeps its copy over the host link at this many GB/s on average
+  static double refresh_rate_gbps;
   static bool gpu_record;          // COLL_GPU_RECORD=1: every lookup counts its keys in device-side hotness counters
   static size_t gpu_record_every;  // COLL_GPU_RECORD_EVERY, default 1: ... only every n-th lookup
   // COLL_GPU_REFRESH=1 (with COLL_GPU_RECORD=1): a refresh whose hotness was all counted on the device ranks, places
