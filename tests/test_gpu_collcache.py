@@ -600,7 +600,7 @@ def test_rows_of_a_background_refresh_hit_as_they_arrive(table_kind, kind, monke
     assert out.cpu().numpy().tobytes() == want
     assert _basics.last_group_offset(0)[1] == len(coming)  # all of them cached in the end
     assert hits == sorted(hits), hits
-    assert hits[0] < len(coming) // 4 and any(len(coming) // 4 < h < len(coming) for h in hits), hits[::5]
+    assert hits[0] < len(coming) // 2 and any(len(coming) // 2 < h < len(coming) for h in hits), hits[::5]
     got = np.zeros(len(new), np.uint32)
     assert _basics.C_LIB_CTYPES.coll_cache_get_cached_keys(0, got.ctypes.data, len(got)) == len(new)
     assert np.array_equal(got, new)
