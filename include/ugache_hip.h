@@ -89,7 +89,7 @@ typedef struct {
 const char *ugk_last_error(void);
 /* version of this ABI; bumped on any signature change.  ugk_abi_version() is what the loaded library was built with:
  * a caller compiled against another UGK_ABI_VERSION must not go on. */
-#define UGK_ABI_VERSION 11
+#define UGK_ABI_VERSION 12
 int ugk_abi_version(void);
 
 /* ---- runtime plumbing: Device::{AllocDataSpace,FreeDataSpace,CopyDataFromTo,StreamSync,CreateStream}
@@ -361,6 +361,12 @@ int ugk_record_i64(const int64_t *keys_dev, size_t n, uint64_t key_inv, uint64_t
 int ugk_record_drain(uint32_t *counts_dev, uint64_t first_row, uint64_t num_rows, uint64_t *observed_dev,
                      uint64_t *entries_dev, uint32_t capacity, uint32_t *n_entries_dev, uint32_t *host_out,
                      void *stream);
+/* the way back: counts_dev[row] += count for the n words (count << 32) | row of entries_dev (rows need not be distinct),
+ * with the observed bit of every row whose counter leaves zero.  What a cache was built from (the ranking of a
+ * presample, FreqRecorder::Sort's list, freq_recorder.cc:275-281) thereby becomes the device-side counters' starting
+ * point.  A row outside [0, num_rows) sets UGK_ST_KEY_OUT_OF_RANGE and is skipped. */
+int ugk_record_restore(const uint64_t *entries_dev, size_t n, uint32_t *counts_dev, uint64_t num_rows,
+                       uint64_t *observed_dev, uint32_t *status_dev, void *stream);
 
 /* ---- re-placement on the device, from the counters of ugk_record_* ---------------------------------------------
  * Stands, for hotness counted on the device, for the host passes of a refresh: FreqRecorder::Sort

@@ -731,6 +731,22 @@ int ugk_record_i64(const int64_t *keys, size_t n, uint64_t key_inv, uint64_t key
                    uint64_t num_rows, uint64_t *observed, uint32_t *status, uint32_t *mirror, void *) {
   return record(keys, n, key_inv, key_mask, counts, num_rows, observed, status, mirror);
 }
+int ugk_record_restore(const uint64_t *entries, size_t n, uint32_t *counts, uint64_t num_rows, uint64_t *observed,
+                       uint32_t *status, void *) {
+  if (n == 0) return 0;
+  REQUIRE(entries && counts && status, "ugk_record_restore: null pointer");
+  for (size_t i = 0; i < n; ++i) {
+    const uint32_t row = (uint32_t)entries[i], cnt = (uint32_t)(entries[i] >> 32);
+    if (row >= num_rows) {
+      or_status(status, UGK_ST_KEY_OUT_OF_RANGE);
+      continue;
+    }
+    if (cnt == 0) continue;
+    const uint32_t before = __atomic_fetch_add(counts + row, cnt, __ATOMIC_RELAXED);
+    if (before == 0 && observed) __atomic_fetch_or(observed + (row >> 6), 1ull << (row & 63), __ATOMIC_RELAXED);
+  }
+  return 0;
+}
 int ugk_record_drain(uint32_t *counts, uint64_t first_row, uint64_t num_rows, uint64_t *observed, uint64_t *entries,
                      uint32_t capacity, uint32_t *n_entries, uint32_t *host_out, void *) {
   REQUIRE(counts && entries && n_entries && host_out && capacity, "ugk_record_drain: bad argument");

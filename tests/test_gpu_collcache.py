@@ -43,7 +43,8 @@ def make_config(num_total_item, pct, threads=8):
 def _fresh_cache(monkeypatch):
     for v in ("COLL_HASH_TABLE", "SAMGRAPH_COLL_CACHE_CONCURRENT_LINK_IMPL", "SAMGRAPH_COLL_CACHE_NO_GROUP",
               "COLL_DEDUP_KEYS", "COLL_DEDUP_MIN_KEYS", "COLL_GPU_RECORD", "COLL_GPU_RECORD_EVERY", "COLL_GPU_REFRESH",
-              "COLL_GPU_REFRESH_KEEP", "COLL_GPU_REFRESH_STABLE", "COLL_REFRESH_RATE_GBPS"):
+              "COLL_GPU_REFRESH_KEEP", "COLL_GPU_REFRESH_STABLE", "COLL_REFRESH_RATE_GBPS",
+              "COLL_GPU_RECORD_SEED"):
         monkeypatch.delenv(v, raising=False)
     yield
     if torch.cuda.is_available():
@@ -504,6 +505,53 @@ def test_refresh_on_the_device_places_like_the_oracle(table_kind, foreground, ke
     cached, nid = expected_cached_set(np.concatenate(counted), n_item, pct)
     check_cached(cached)
     lookup(rng.integers(0, n_item, size=20_000), nid)
+
+
+@pytest.mark.parametrize("table_kind", ["FLAT", "HASH"])
+@pytest.mark.parametrize("keep", [False, True])
+def test_device_side_counters_seeded_with_the_hotness_the_cache_was_built_from(table_kind, keep, monkeypatch):
+    """COLL_GPU_RECORD_SEED=1: the counters the lookups bump start from the ranking the build was given, so the first
+    refresh on the device places by the presample and the counted lookups together; afterwards they go on as configured
+    (kept: everything so far; otherwise the interval since the last refresh)"""
+    monkeypatch.setenv("COLL_HASH_TABLE", table_kind)
+    monkeypatch.setenv("COLL_GPU_RECORD", "1")
+    monkeypatch.setenv("COLL_GPU_REFRESH", "1")
+    monkeypatch.setenv("COLL_GPU_RECORD_SEED", "1")
+    if keep:
+        monkeypatch.setenv("COLL_GPU_REFRESH_KEEP", "1")
+    rng = np.random.default_rng(91)
+    n_item, dim, pct = 30_011, 16, 0.25
+    co.config(make_config(n_item, pct))
+    co.coll_cache_record_init(0)
+    perm = rng.permutation(n_item)
+    s0 = perm[zipf_ranks(rng, 120_000, n_item, 1.1)]
+    co.coll_torch_record(0, torch.from_numpy(s0).to(torch.int32))
+    emb = co.coll_torch_create_emb_shm(0, n_item, dim, torch.float32)
+    table = fill_table(emb, rng)
+    co.coll_torch_init_t(0, 0, emb, pct)
+    counted = [s0.astype(np.uint32)]
+    for rnd in range(3):
+        swap = rng.choice(n_item, n_item // 10, replace=False)
+        perm[swap] = perm[rng.permutation(swap)]
+        keys = perm[zipf_ranks(rng, 20_000, n_item, 1.1)]
+        out = co.coll_torch_lookup_key_t_val_ret(0, torch.from_numpy(keys).to(torch.int32).cuda(), False)
+        assert out.cpu().numpy().tobytes() == ORC.gather(table, keys.astype(np.int64)).tobytes()
+        counted.append(keys.astype(np.uint32))
+        co.coll_torch_refresh(0, True)
+        want, nid = expected_cached_set(np.concatenate(counted), n_item, pct)
+        if rnd == 0:  # without the seed the same refresh would have placed by the 20,000 counted keys alone
+            unseeded, _ = expected_cached_set(keys.astype(np.uint32), n_item, pct)
+            assert len(np.setdiff1d(want, unseeded)) > 1_000
+        got = np.zeros(len(want), np.uint32)
+        assert _basics.C_LIB_CTYPES.coll_cache_get_cached_keys(0, got.ctypes.data, len(got)) == len(want)
+        assert np.array_equal(got, want), rnd
+        if not keep:
+            counted.clear()
+        probe = rng.integers(0, n_item, size=5_000)
+        out = co.coll_torch_lookup_key_t_val_ret(0, torch.from_numpy(probe).to(torch.int32).cuda(), False)
+        assert out.cpu().numpy().tobytes() == ORC.gather(table, probe.astype(np.int64)).tobytes()
+        assert _basics.last_group_offset(0)[1] == int((nid[probe] == 0).sum())
+        counted.append(probe.astype(np.uint32))
 
 
 def test_background_refresh_paced_by_a_rate_over_the_link(monkeypatch):

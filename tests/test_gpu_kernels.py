@@ -1044,6 +1044,53 @@ def test_record_rejects_keys_without_a_row():
     assert to_np(counts, np.uint32)[:10].tolist() == [0, 0, 0, 2, 0, 0, 0, 0, 0, 0]
 
 
+@pytest.mark.parametrize("n_rows,n_entries", [(1, 1), (70, 500), (100_003, 250_000)])
+def test_restore_adds_counts_back_and_marks_the_rows_observed(n_rows, n_entries):
+    """ugk_record_restore is the way back of a drain: counts[row] += count for (count << 32 | row) words, rows may
+    repeat, zero counts change nothing, the observed bit follows "counter above zero"; against numpy add.at"""
+    rng = np.random.default_rng(n_rows)
+    before = (rng.integers(0, 4, size=n_rows) * (rng.random(n_rows) < 0.3)).astype(np.uint32)
+    rows = rng.integers(0, n_rows, size=n_entries).astype(np.uint64)
+    cnts = (rng.integers(0, 1000, size=n_entries) * (rng.random(n_entries) < 0.8)).astype(np.uint64)
+    words = (n_rows + 63) // 64
+    pad = np.zeros(words * 64, bool)
+    pad[:n_rows] = before > 0
+    counts = to_dev(before)
+    observed = to_dev(np.packbits(pad, bitorder="little").view(np.uint64))
+    st = dev_zeros_u32(1)
+    d_entries = to_dev((cnts << np.uint64(32)) | rows)
+    hip.call("ugk_record_restore", ptr(d_entries), n_entries, ptr(counts), n_rows, ptr(observed), ptr(st), None)
+    sync()
+    assert status_value(st) == 0
+    want = before.astype(np.uint64)
+    np.add.at(want, rows.astype(np.int64), cnts)
+    assert np.array_equal(to_np(counts, np.uint32)[:n_rows], want.astype(np.uint32))
+    bits = np.unpackbits(to_np(observed, np.uint8)[: words * 8], bitorder="little")
+    assert np.array_equal(bits[:n_rows].astype(bool), want > 0) and not bits[n_rows:].any()
+    # what a drain hands over, handed back: the counters are what they were
+    if n_rows > 1:
+        entries = dev_bytes(n_rows * 8)
+        n_out = dev_zeros_u32(1)
+        out = PinnedArray((2,), np.uint32)
+        try:
+            hip.call("ugk_record_drain", ptr(counts), 0, n_rows, ptr(observed), ptr(entries), n_rows, ptr(n_out),
+                     out.ptr, None)
+            sync()
+            k = int(out.array[0])
+            assert k == int((want > 0).sum()) and not to_np(counts, np.uint32)[:n_rows].any()
+            hip.call("ugk_record_restore", ptr(entries), k, ptr(counts), n_rows, ptr(observed), ptr(st), None)
+            sync()
+            assert np.array_equal(to_np(counts, np.uint32)[:n_rows], want.astype(np.uint32))
+        finally:
+            out.free()
+    # a row outside the table is flagged and skipped
+    bad = to_dev(np.array([(5 << 32) | n_rows], np.uint64))
+    hip.call("ugk_record_restore", ptr(bad), 1, ptr(counts), n_rows, None, ptr(st), None)
+    sync()
+    assert status_value(st) & hip.ST_KEY_OUT_OF_RANGE
+    assert np.array_equal(to_np(counts, np.uint32)[:n_rows], want.astype(np.uint32))
+
+
 @pytest.mark.parametrize("first,cnt", [(0, 1), (1, 1), (3, 2), (1, 3), (2, 7), (5, 64), (7, 257), (0, 0)])
 def test_drain_of_short_and_unaligned_row_ranges(first, cnt):
     total = 300

@@ -431,6 +431,30 @@ void ExtractSession::PlaceOnDevice(size_t num_cached, uint64_t *in_new_bits, uin
   UGK_CALL(ugk_stream_wait_event(stream, _ev_placed));
 }
 
+void ExtractSession::SeedHotness(const FreqEntry *entries, size_t num_entries) {
+  CHECK_NOTNULL(_hot_counts) << "seeding needs the device-side hotness counters (COLL_GPU_RECORD=1)";
+  if (num_entries == 0) return;
+  CHECK_NOTNULL(entries);
+  UGK_CALL(ugk_set_device(_cache_ctx->_trainer_ctx.device_id));
+  static_assert(sizeof(FreqEntry) == sizeof(uint64_t), "an entry is one (count << 32 | row) word");
+  const size_t cap = _hot_entries->nbytes() / sizeof(uint64_t);
+  std::lock_guard<std::mutex> guard(_drain_mu);
+  uint64_t *dev_list = _hot_entries->ptr<uint64_t>();
+  auto *host_list = _hot_entries_host->ptr<FreqEntry>();
+  for (size_t first = 0; first < num_entries; first += cap) {
+    const size_t cur = std::min(cap, num_entries - first);
+    memcpy(host_list, entries + first, cur * sizeof(FreqEntry));  // pinned staging: the drain's own
+    UGK_CALL(ugk_memcpy_async(dev_list, host_list, cur * sizeof(uint64_t), _record_stream));
+    UGK_CALL(ugk_record_restore(dev_list, cur, _hot_counts->ptr<uint32_t>(), _cache_ctx->_num_total_nodes,
+                                ObservedBits(), _status, _record_stream));
+    UGK_CALL(ugk_stream_sync(_record_stream));
+  }
+  uint32_t st = 0;
+  UGK_CALL(ugk_memcpy_async(&st, _status, sizeof(st), _record_stream));
+  UGK_CALL(ugk_stream_sync(_record_stream));
+  CHECK_EQ(st, 0u) << "seeding the hotness counters: a row is outside num_total_item=" << _cache_ctx->_num_total_nodes;
+}
+
 size_t ExtractSession::DrainHotness(FreqRecorder *recorder) {
   CHECK_NOTNULL(recorder);
   if (!_hot_counts) return 0;

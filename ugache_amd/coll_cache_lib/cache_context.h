@@ -256,6 +256,8 @@ class ExtractSession {
   // reset_counts: the next interval starts from zero, as after DrainHotness.  keep_bits (may be null): rows that
   // win ties at the last count that gets in (ugk_rank_place_keep).
   bool CountsOnDevice() const { return _hot_counts != nullptr; }
+  // adds counts known on the host (entries with distinct or repeated rows) to the device-side counters
+  void SeedHotness(const FreqEntry *entries, size_t num_entries);
   int DeviceId() const { return _cache_ctx->_trainer_ctx.device_id; }
   // what a foreground refresh may read rows from besides the host table (null: nothing)
   const ugk_stage_t *StageForRefresh(bool foreground, StreamHandle stream);

@@ -141,6 +141,10 @@ void coll_cache_init(int replica_id, size_t key_space_size, std::function<MemHan
   if (need_rank) freq_rank = CombineAndRank(replica_id);
   _coll_cache->build_v2(replica_id, freq_rank, (IdType)key_space_size, allocator, cpu_data, dtype, dim,
                         cache_percentage, stream);
+  // COLL_GPU_RECORD_SEED: the counters the lookups bump start from what this cache was ranked by
+  auto session = _coll_cache->session(replica_id);
+  if (RunConfig::gpu_record_seed && freq_rank && session && session->CountsOnDevice())
+    session->SeedHotness(freq_rank->buf, freq_rank->entries.size());
   LOG(INFO) << "coll cache has been initialized successfully";
 }
 

@@ -42,6 +42,7 @@ size_t RunConfig::gpu_record_every = 1;
 bool RunConfig::gpu_refresh = false;
 bool RunConfig::gpu_refresh_keep = false;
 bool RunConfig::gpu_refresh_stable = false;
+bool RunConfig::gpu_record_seed = false;
 size_t RunConfig::miss_stage_rows = 0;
 unsigned RunConfig::spin_wait_us = 5000;
 bool RunConfig::kernel_events = false;
@@ -87,6 +88,7 @@ void RunConfig::LoadConfigFromEnv() {
   gpu_refresh = false;
   gpu_refresh_keep = false;
   gpu_refresh_stable = false;
+  gpu_record_seed = false;
   miss_stage_rows = 0;
   spin_wait_us = 5000;
   kernel_events = false;
@@ -123,6 +125,7 @@ void RunConfig::LoadConfigFromEnv() {
   if (GetEnv("COLL_GPU_REFRESH") != "") gpu_refresh = GetEnv("COLL_GPU_REFRESH") != "0";
   if (GetEnv("COLL_GPU_REFRESH_KEEP") != "") gpu_refresh_keep = GetEnv("COLL_GPU_REFRESH_KEEP") != "0";
   if (GetEnv("COLL_GPU_REFRESH_STABLE") != "") gpu_refresh_stable = GetEnv("COLL_GPU_REFRESH_STABLE") != "0";
+  if (GetEnv("COLL_GPU_RECORD_SEED") != "") gpu_record_seed = GetEnv("COLL_GPU_RECORD_SEED") != "0";
   if (GetEnv("COLL_SPIN_WAIT") != "") spin_wait_us = (unsigned)std::stoul(GetEnv("COLL_SPIN_WAIT"));
   if (GetEnv("COLL_MISS_STAGE_ROWS") != "") miss_stage_rows = (size_t)std::stoull(GetEnv("COLL_MISS_STAGE_ROWS"));
   if (GetEnv("COLL_KERNEL_EVENTS") != "") kernel_events = GetEnv("COLL_KERNEL_EVENTS") != "0";

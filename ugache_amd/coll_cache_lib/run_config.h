@@ -77,6 +77,10 @@ struct RunConfig {
   // COLL_GPU_REFRESH_STABLE=1: among rows whose counts tie at the last count that gets in, such a refresh prefers the
   // rows cached now, so it moves no row that the counters do not tell apart from the one it would replace
   static bool gpu_refresh_stable;
+  // COLL_GPU_RECORD_SEED=1: the device-side counters start from the hotness the cache was built from (the ranking
+  // handed to the build) instead of from zero, so the first refreshes on the device weigh what the lookups counted
+  // against what the build knew
+  static bool gpu_record_seed;
   // COLL_MISS_STAGE_ROWS=n (0 = off): the fused extraction also files the rows it takes from the host table in a
   // direct-mapped set of n (rounded up to a power of two) rows in HBM, and a foreground refresh takes the rows it inserts
   // from there when it finds them instead of over the host link again

@@ -134,6 +134,23 @@ __device__ __forceinline__ uint32_t nonzeros(const u32x4 &c) {
   return (c.x != 0) + (c.y != 0) + (c.z != 0) + (c.w != 0);
 }
 
+// the way back of a drain: counts handed over as (count << 32 | row) words are added to the counters
+__global__ __launch_bounds__(kBlock) void restore_kernel(const unsigned long long *__restrict__ entries, size_t n,
+                                                         uint32_t *counts, uint64_t num_rows,
+                                                         unsigned long long *observed, uint32_t *status) {
+  for (size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x; i < n; i += (size_t)gridDim.x * kBlock) {
+    const unsigned long long e = entries[i];
+    const uint32_t row = (uint32_t)e, cnt = (uint32_t)(e >> 32);
+    if (row >= num_rows) {
+      atomicOr(status, UGK_ST_KEY_OUT_OF_RANGE);
+      continue;
+    }
+    if (cnt == 0) continue;
+    const uint32_t before = atomicAdd(counts + row, cnt);
+    if (before == 0 && observed) atomicOr(observed + (row >> 6), 1ull << (row & 63));  // the counter leaves zero
+  }
+}
+
 __global__ __launch_bounds__(kBlock) void drain_kernel(uint32_t *counts, uint64_t num_rows, uint64_t first_row,
                                                        unsigned long long *observed, unsigned long long *entries,
                                                        uint32_t capacity, uint32_t *n_entries) {
@@ -245,6 +262,19 @@ int ugk_record_i64(const int64_t *keys_dev, size_t n, uint64_t key_inv, uint64_t
                    void *stream) {
   return record<int64_t>(keys_dev, n, key_inv, key_mask, counts_dev, num_rows, observed_dev, status_dev, host_mirror,
                          stream);
+}
+
+int ugk_record_restore(const uint64_t *entries_dev, size_t n, uint32_t *counts_dev, uint64_t num_rows,
+                       uint64_t *observed_dev, uint32_t *status_dev, void *stream) {
+  if (n == 0) return 0;
+  UGK_REQUIRE(entries_dev && counts_dev && status_dev, "ugk_record_restore: null pointer");
+  UGK_REQUIRE(num_rows <= 0xffffffffull, "ugk_record_restore: rows must fit 32 bits");
+  const unsigned grid = clamp_grid((n + kBlock - 1) / kBlock, 0);
+  hipLaunchKernelGGL(restore_kernel, dim3(grid), dim3(kBlock), 0, as_stream(stream),
+                     reinterpret_cast<const unsigned long long *>(entries_dev), n, counts_dev, num_rows,
+                     reinterpret_cast<unsigned long long *>(observed_dev), status_dev);
+  UGK_HIP(hipGetLastError());
+  return 0;
 }
 
 int ugk_record_drain(uint32_t *counts_dev, uint64_t first_row, uint64_t num_rows, uint64_t *observed_dev,

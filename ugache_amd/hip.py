@@ -116,6 +116,7 @@ SIGNATURES = {
     "ugk_record_i64": [_vp, _sz, _u64, _u64, _vp, _u64, _vp, _vp, _vp, _vp],
     "ugk_record_drain": [_vp, _u64, _u64, _vp, _vp, _u32, _vp, _vp, _vp],
     "ugk_rank_workspace_bytes": [],
+    "ugk_record_restore": [_vp, _sz, _vp, _u64, _vp, _vp, _vp],
     "ugk_rank_place": [_vp, _u64, _u64, _vp, _vp, _vp, _vp, C.c_int, _vp],
     "ugk_rank_place_keep": [_vp, _u64, _u64, _vp, _vp, _vp, _vp, _vp, C.c_int, _vp],
     "ugk_rank_threshold": [_vp, _vp, _vp],
