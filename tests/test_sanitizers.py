@@ -29,6 +29,9 @@ def _run(exe, table, refresh, steps):
     env["COLL_MISS_STAGE_ROWS"] = "4096"  # lookups file the rows they fetch from the host, foreground refreshes read them
     if table == "HASH":  # refreshes on the device keep cached rows that tie (the second placement path)
         env["COLL_GPU_REFRESH_STABLE"] = "1"
+    else:  # the device-side counters start from the build's ranking, and the background copy is paced by a rate
+        env["COLL_GPU_RECORD_SEED"] = "1"
+        env["COLL_REFRESH_RATE_GBPS"] = "0.5"
     env["ASAN_OPTIONS"] = "detect_leaks=1:abort_on_error=0"
     env["UBSAN_OPTIONS"] = "print_stacktrace=1:halt_on_error=1"
     env["TSAN_OPTIONS"] = "halt_on_error=0:second_deadlock_stack=1"
