@@ -183,20 +183,32 @@ __global__ __launch_bounds__(kBlock) void gather_staged_kernel(const u32x4 *__re
       const uint64_t h = fmix64(s) & stage.mask;
       const unsigned long long cur = stage.owner_dev[h];
       const bool filed = ok[u] && (cur >> 32) != 0 && (uint32_t)cur == (uint32_t)s;
-      if (rest_count && ok[u] && !filed) {
-        // left for the caller's own (throttled) copy over the host link: listed, not copied
-        if (lane == 0) {
-          const uint32_t at = atomicAdd(rest_count, 1u);
+      if (rest_count) {
+        // Rows the stage does not hold are left for the caller's own (throttled) copy over the host link: listed, not
+        // copied.  With done_count the rows that are copied here are listed too, from the back of the same lists, for
+        // a caller that publishes rows as they arrive.  One atomic per wavefront and list: the first lane of every
+        // row that goes on a list takes its place from a ballot.
+        const bool lead = lane == 0 && ok[u];
+        const unsigned long long to_rest = __ballot(lead && !filed);
+        const unsigned long long to_done = __ballot(lead && filed && done_count != nullptr);
+        const unsigned long long below = (1ull << lane_id()) - 1ull;
+        uint32_t rest_base = 0, done_base = 0;
+        if (lane_id() == 0) {
+          if (to_rest) rest_base = atomicAdd(rest_count, (uint32_t)__popcll(to_rest));
+          if (to_done) done_base = atomicAdd(done_count, (uint32_t)__popcll(to_done));
+        }
+        rest_base = __shfl(rest_base, 0);
+        done_base = __shfl(done_base, 0);
+        if (lead && !filed) {
+          const uint32_t at = rest_base + (uint32_t)__popcll(to_rest & below);
+          rest_rows[at] = (uint32_t)s;
+          rest_dst[at] = (uint32_t)d[u];
+        } else if (lead && filed && done_count) {
+          const uint32_t at = (uint32_t)n - 1u - (done_base + (uint32_t)__popcll(to_done & below));
           rest_rows[at] = (uint32_t)s;
           rest_dst[at] = (uint32_t)d[u];
         }
-        ok[u] = false;
-      }
-      if (done_count && filed && lane == 0) {
-        // copied here: listed from the back of the same lists, for a caller that publishes rows as they arrive
-        const uint32_t at = (uint32_t)n - 1u - atomicAdd(done_count, 1u);
-        rest_rows[at] = (uint32_t)s;
-        rest_dst[at] = (uint32_t)d[u];
+        if (!filed) ok[u] = false;
       }
       src[u] = !ok[u] ? reinterpret_cast<const u32x4 *>(out) : filed ? stage_rows + h * vpr : host + s * vpr;
       if (filed && lane == 0) ++mine;
