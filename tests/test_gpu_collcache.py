@@ -599,10 +599,12 @@ def test_background_refresh_paced_by_a_rate_over_the_link(monkeypatch):
 
 @pytest.mark.parametrize("table_kind", ["FLAT", "HASH"])
 @pytest.mark.parametrize("kind", ["host", "device", "device_staged"])
-def test_rows_of_a_background_refresh_hit_as_they_arrive(table_kind, kind, monkeypatch):
+@pytest.mark.parametrize("dim", [32, 16])
+def test_rows_of_a_background_refresh_hit_as_they_arrive(table_kind, kind, dim, monkeypatch):
     """a background refresh copies its rows in throttled batches and publishes every batch behind its copy: lookups of
     the rows that come in, run beside the refresh, find more and more of them in the cache (never fewer), some of them
-    long before the refresh ends, and always return table[keys]"""
+    long before the refresh ends, and always return table[keys].  Rows of 64 bytes share their 128-byte line with a
+    neighbour: those are published only once the lookups in flight at the end of their copy have finished."""
     monkeypatch.setenv("COLL_HASH_TABLE", table_kind)
     monkeypatch.setenv("COLL_REFRESH_SLEEP_US", "4000")
     monkeypatch.setenv("COLL_REFRESH_BATCH_ROWS", "200")
@@ -612,7 +614,7 @@ def test_rows_of_a_background_refresh_hit_as_they_arrive(table_kind, kind, monke
     if kind == "device_staged":
         monkeypatch.setenv("COLL_MISS_STAGE_ROWS", "2048")
     rng = np.random.default_rng(77)
-    n_item, dim, pct = 50_000, 32, 0.2
+    n_item, pct = 50_000, 0.2
     co.config(make_config(n_item, pct))
     co.coll_cache_record_init(0)
     perm = rng.permutation(n_item)

@@ -1068,8 +1068,19 @@ void RefreshSession::CopyRowsIntoSlots(const uint32_t *rows_dev, const uint32_t 
   void *cache = ctx->_device_cache_data[ctx->_local_location_id];
   // [0] error bits, [8] rows taken from the stage so far, [9] rows left for the link, [10] rows taken this time
   uint32_t *status = _status_handle->ptr<uint32_t>();
+  // Rows that do not fill whole 128-byte lines share a line with the slot next door.  A lookup kernel that runs while
+  // the copy does may hold such a line in the L2 of its XCD from reading the neighbour — the L2s of different XCDs only
+  // agree at kernel boundaries — and would read the stale half once the table names the new row.  Those rows are
+  // published only after every lookup that was in flight when their copy completed has finished.
+  const bool rows_share_lines = ctx->_row_bytes % 128 != 0 || reinterpret_cast<uintptr_t>(cache) % 128 != 0;
+  auto session = ctx->_coll_cache ? ctx->_coll_cache->session(local) : nullptr;
   // the rows of a list, or of a part of one, become visible to lookups: behind their copy on the same stream
   auto publish = [&](const uint32_t *rows, const uint32_t *slots, size_t n) {
+    if (n == 0) return;
+    if (!foreground && rows_share_lines && session) {
+      UGK_CALL(ugk_stream_sync(copy_stream));
+      session->WaitForLookupsInFlight(false, 20.0);
+    }
     table->PublishRows(rows, slots, n, local, __publish_ids, ctx->_eager_gpu_mem_allocator, gpu_ctx, copy_stream);
   };
   if (foreground) {
