@@ -115,10 +115,11 @@ def parse_args():
     ap.add_argument("--calibrate", action="store_true",
                     help="also run 5 plain device copies of 1 GiB (ugk_copy_rows) so a counter run has a kernel of "
                          "known traffic next to the gather")
-    ap.add_argument("--probe", default=None, choices=["kpw", "row_span", "cu_mask"],
+    ap.add_argument("--probe", default=None, choices=["kpw", "row_span", "cu_mask", "small_batch"],
                     help="instead of a workload, run one of the stand-alone measurements behind the launch rules "
                          "(ugache_amd/probes.py): keys per wavefront of the fused kernel, random rows over the host "
-                         "link by span, host-link gather confined to a few compute units; prints one JSON line")
+                         "link by span, host-link gather confined to a few compute units, serving-sized batches through "
+                         "the library; prints one JSON line")
     ap.add_argument("--quick", action="store_true", help="with --probe: a reduced sweep")
     args = ap.parse_args()
     if args.gpus != 1:

@@ -93,8 +93,10 @@ size_t coll_cache_lookup_unique_i64(int replica_id, const int64_t *key, size_t n
 /* Stream-ordered lookups (extension; the reference's lookup always blocks, facade.cc:74-88 and the synchronisations
  * of cache_context.cu:1199-1794).  coll_cache_lookup_async* enqueue the batch on `stream` and return: `output` is
  * complete for anything enqueued on the same stream afterwards, which is all a framework op needs; about 10 us of
- * blocking round trip per batch disappear.  `key` and `output` must stay valid until the work has run.  All
- * stream-ordered lookups of a replica, and its refreshes, must use one stream.  coll_cache_lookup_wait blocks until
+ * blocking round trip per batch disappear.  `key` and `output` must stay valid until the work has run.  The
+ * stream-ordered lookups of a replica that are in flight together must use one stream (they report through the same
+ * words); a refresh may run on any stream and in any thread: it waits for the lookups in flight wherever they were
+ * enqueued before it reuses a slot.  coll_cache_lookup_wait blocks until
  * everything enqueued so far has finished, aborts if a key was outside its table, and makes
  * coll_cache_last_group_offset describe the last batch; any blocking lookup does the same first.  No per-step profiler
  * values are logged for stream-ordered batches.  Such a call is kernel launches only (no synchronisation, no

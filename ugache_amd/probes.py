@@ -10,6 +10,9 @@ flagged an error (the parity tests check results).
             from its first S GiB: what small rows reach over the host link, and how that depends on the span
   cu_mask   a host-link gather on a side stream next to an HBM gather on the main stream: side stream plain or
             confined to 8 / 16 / 32 compute units (ugk_stream_create_cu_masked), grid capped to 32 - 256 workgroups
+  small_batch  serving-sized batches (1,024 - 131,072 keys that all hit) through the library: microseconds per blocking
+            coll_cache_lookup_i64 and per stream-ordered coll_cache_lookup_async_i64, without a table (the whole table
+            cached) and through the table of a half-cached key space (host clock around 2,000 calls)
 """
 import ctypes as C
 import json
@@ -221,7 +224,56 @@ def probe_cu_mask(hip, torch, note, quick=False):
                    "launched together, one event pair around each; the last of 4 rounds", "rows": res}
 
 
-PROBES = {"kpw": probe_kpw, "row_span": probe_row_span, "cu_mask": probe_cu_mask}
+def probe_small_batch(hip, torch, note, quick=False):
+    import collcache.torch as co
+    from collcache.torch.c_lib import _basics
+
+    Cl = _basics.C_LIB_CTYPES
+    rows, dim, calls = 2_000_000, 128, (300 if quick else 2000)
+    sizes = (1024, 65536) if quick else (1024, 8192, 26624, 65536, 131072)
+    stream = C.c_void_p(torch.cuda.current_stream().cuda_stream)
+    out_rows = []
+    for pct, label in ((1.0, "no table: the whole table cached"), (0.5, "flat table of a half-cached key space")):
+        co.config({"cache_percentage": pct, "_cache_policy": co.kCollCacheAsymmLink, "num_device": 1,
+                   "num_global_step_per_epoch": 10, "num_epoch": 1, "num_total_item": rows, "omp_thread_num": 8})
+        co.coll_cache_record_init(0)
+        # rows [0, rows / 2) are the hot ones: every key of the timed batches hits
+        co.coll_torch_record(0, torch.arange(0, rows // 2, dtype=torch.int32))
+        emb = co.coll_torch_create_emb_shm(0, rows, dim, torch.float32)
+        emb.normal_(generator=torch.Generator().manual_seed(1))
+        co.coll_torch_init_t(0, 0, emb, pct)
+        for n in sizes:
+            keys = torch.randint(0, rows // 2, (8, n), device="cuda", dtype=torch.int64)
+            ptrs = [keys[i].data_ptr() for i in range(8)]
+            out = torch.empty((n, dim), dtype=torch.float32, device="cuda")
+            torch.cuda.synchronize()
+            for i in range(20):
+                Cl.coll_cache_lookup_i64(0, ptrs[i % 8], n, out.data_ptr(), stream)
+            t0 = time.perf_counter()
+            for i in range(calls):
+                Cl.coll_cache_lookup_i64(0, ptrs[i % 8], n, out.data_ptr(), stream)
+            blocking = (time.perf_counter() - t0) / calls * 1e6
+            assert torch.equal(out.cpu(), emb[keys[(calls - 1) % 8].cpu()])
+            assert _basics.last_group_offset(0)[1] == n  # every key was served from HBM
+            for i in range(20):
+                Cl.coll_cache_lookup_async_i64(0, ptrs[i % 8], n, out.data_ptr(), stream)
+            Cl.coll_cache_lookup_wait(0, stream)
+            t0 = time.perf_counter()
+            for i in range(calls):
+                Cl.coll_cache_lookup_async_i64(0, ptrs[i % 8], n, out.data_ptr(), stream)
+            Cl.coll_cache_lookup_wait(0, stream)
+            ordered = (time.perf_counter() - t0) / calls * 1e6
+            out_rows.append({"path": label, "keys": n, "us_per_blocking_call": round(blocking, 2),
+                             "us_per_stream_ordered_call": round(ordered, 2)})
+            note("small_batch %s, %d keys: blocking %.1f us, stream-ordered %.1f us" % (label, n, blocking, ordered))
+            del keys, out
+        co.coll_torch_shutdown()
+    return {"probe": "small_batch", "table_rows": rows, "row_bytes": dim * 4, "calls_timed": calls,
+            "how": "coll_cache_lookup_i64 / coll_cache_lookup_async_i64 (+ one coll_cache_lookup_wait) over 8 cycled "
+                   "batches of uniformly random keys that all hit, host clock around the calls", "rows": out_rows}
+
+
+PROBES = {"kpw": probe_kpw, "row_span": probe_row_span, "cu_mask": probe_cu_mask, "small_batch": probe_small_batch}
 
 
 def run(name, quick=False):
