@@ -1404,10 +1404,12 @@ def test_counting_every_third_lookup_on_the_device(impl, monkeypatch):
 
 @pytest.mark.parametrize("table_kind", ["FLAT", "HASH"])
 @pytest.mark.parametrize("stage", [0, 8192])
-def test_lookups_stay_exact_while_the_device_refreshes_under_them(table_kind, stage, monkeypatch):
+@pytest.mark.parametrize("dim", [32, 12])
+def test_lookups_stay_exact_while_the_device_refreshes_under_them(table_kind, stage, dim, monkeypatch):
     """a thread refreshes back to back on the device (background mode, hotness accumulating from the very lookups that
     run beside it) while the caller looks keys up: every output is table[keys], and when the dust settles the cache
-    holds exactly its share of rows in exactly that many slots"""
+    holds exactly its share of rows in exactly that many slots.  Rows of 128 bytes fill their lines; rows of 48 bytes
+    share them with their neighbours, and are published only behind the lookups in flight."""
     monkeypatch.setenv("COLL_HASH_TABLE", table_kind)
     monkeypatch.setenv("COLL_GPU_RECORD", "1")
     monkeypatch.setenv("COLL_GPU_REFRESH", "1")
@@ -1418,7 +1420,7 @@ def test_lookups_stay_exact_while_the_device_refreshes_under_them(table_kind, st
     if stage:  # the refreshes read the stage of missed rows the lookups beside them have been switched away from
         monkeypatch.setenv("COLL_MISS_STAGE_ROWS", str(stage))
     rng = np.random.default_rng(91)
-    n_item, dim, pct = 60_000, 32, 0.15
+    n_item, pct = 60_000, 0.15
     co.config(make_config(n_item, pct))
     co.coll_cache_record_init(0)
     perm = rng.permutation(n_item)
