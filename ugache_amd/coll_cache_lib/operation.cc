@@ -336,7 +336,7 @@ class RecordWorker {
   // at process exit without coll_cache_shutdown: the thread ends, the stream, event and staging memory are left to
   // the runtime, which may be half gone by then
   ~RecordWorker() { Stop(/*release=*/false); }
-  /// hands the first `bytes` bytes of `key` (device memory, `key_bytes` per key) to the thread
+  /// hands the first `num` keys of `key` (device memory, `key_bytes` bytes each) to the thread
   void Post(int replica_id, int device, const void *key, size_t num, int key_bytes, StreamHandle stream) {
     Start(device);
     UGK_CALL(ugk_event_record(_keys_ready, stream));
@@ -419,7 +419,7 @@ class RecordWorker {
   StreamHandle _stream = nullptr;
   void *_keys_ready = nullptr;
   void *_staging = nullptr;  // pinned
-  // durations of the latest batches, for the log line at the end
+  // durations of the first 4096 batches, for the log line at the end
   static void Sample(std::vector<double> &v, double s) {
     if (v.size() < 4096) v.push_back(s);
   }
