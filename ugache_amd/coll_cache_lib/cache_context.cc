@@ -1317,7 +1317,10 @@ void RefreshSession::refresh_on_device(ExtractSession *session, size_t num_cache
   const double wait_s = t_phase.Passed();
   t_phase.Reset();
 
-  // Step 6: the first free slots, ascending, take the new rows, ascending; then the keys are published
+  // Step 6: the first free slots, ascending, take the new rows, ascending; then the keys are published.  (A foreground
+  // refresh that returned here and left copy, publication and the slot bitmap's update running on the copy stream
+  // beside the caller's next lookup was measured: the call got 0.15 ms shorter, a whole step no shorter, because that
+  // lookup holds every wavefront slot of the chip while it waits for the host link.)
   const size_t num_free_expected = table->_num_free + num_evicted;
   volatile uint32_t *n_free_word = nullptr;
   if (num_insert > 0) {
