@@ -90,6 +90,29 @@ size_t coll_cache_lookup_unique(int replica_id, const uint32_t *key, size_t num_
                                 uint32_t *inverse_out, StreamHandle stream);
 size_t coll_cache_lookup_unique_i64(int replica_id, const int64_t *key, size_t num_keys, void *output,
                                     uint32_t *inverse_out, StreamHandle stream);
+/* Lookup and per-sample combination of a multi-hot feature in one call (extension; what the TF2 sparse layer does in
+ * three steps, python_tf2/collcache_tf2/collcache_tf2/core/sparse_lookup_layer.py:196-265: look the ids up, gather,
+ * embedding_lookup_sparse).  Segment r = key[seg_off[r] .. seg_off[r + 1]); output[r, :] = sum of weights[j] x row(key[j])
+ * over the segment (weights NULL: 1), as it is (combiner 0 "sum"), divided by the sum of the weights (1 "mean") or by
+ * the root of the sum of their squares (2 "sqrtn"); a zero denominator or an empty segment gives a zero row.  Elements
+ * are fp32 (elem_bytes 4) or fp16 (elem_bytes 2: the rows of a table configured as half), added in fp32 in the order of
+ * the ids.  key, seg_off (num_rows + 1 ascending int64 offsets, the last one num_keys), weights: device memory;
+ * output: device [num_rows, dim], caller-allocated; blocking, like coll_cache_lookup.  Rows must be a multiple of 16
+ * bytes and at most 4096 bytes long.  coll_cache_last_group_offset afterwards counts keys, not output rows. */
+void coll_cache_lookup_pooled(int replica_id, const uint32_t *key, const int64_t *seg_off, const float *weights,
+                              size_t num_rows, size_t num_keys, int combiner, int elem_bytes, void *output,
+                              StreamHandle stream);
+void coll_cache_lookup_pooled_i64(int replica_id, const int64_t *key, const int64_t *seg_off, const float *weights,
+                                  size_t num_rows, size_t num_keys, int combiner, int elem_bytes, void *output,
+                                  StreamHandle stream);
+/* the same as one step of the serving loop (coll_cache_forward*: a prefix of the keys recorded, a background refresh
+ * at the configured step) */
+void coll_cache_forward_pooled(int replica_id, const uint32_t *key, const int64_t *seg_off, const float *weights,
+                               size_t num_rows, size_t num_keys, int combiner, int elem_bytes, void *output,
+                               StreamHandle stream);
+void coll_cache_forward_pooled_i64(int replica_id, const int64_t *key, const int64_t *seg_off, const float *weights,
+                                   size_t num_rows, size_t num_keys, int combiner, int elem_bytes, void *output,
+                                   StreamHandle stream);
 /* Stream-ordered lookups (extension; the reference's lookup always blocks, facade.cc:74-88 and the synchronisations
  * of cache_context.cu:1199-1794).  coll_cache_lookup_async* enqueue the batch on `stream` and return: `output` is
  * complete for anything enqueued on the same stream afterwards, which is all a framework op needs; about 10 us of

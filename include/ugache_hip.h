@@ -89,7 +89,7 @@ typedef struct {
 const char *ugk_last_error(void);
 /* version of this ABI; bumped on any signature change.  ugk_abi_version() is what the loaded library was built with:
  * a caller compiled against another UGK_ABI_VERSION must not go on. */
-#define UGK_ABI_VERSION 12
+#define UGK_ABI_VERSION 13
 int ugk_abi_version(void);
 
 /* ---- runtime plumbing: Device::{AllocDataSpace,FreeDataSpace,CopyDataFromTo,StreamSync,CreateStream}
@@ -263,6 +263,33 @@ int ugk_extract_mix_i64(ugk_table_t t, const int64_t *keys_dev, size_t n, const 
                         const void *host_dev, uint64_t host_rows, void *out_dev, size_t row_bytes,
                         uint32_t *status_dev, uint32_t *host_mirror, uint64_t *group_counts_host,
                         uint32_t *num_groups_host, uint32_t others_hint, void *stream);
+
+/* ---- pooled extraction: lookup + per-sample combination of a multi-hot feature in one kernel ---------------------
+ * The reference's sparse layer looks the distinct ids up and hands the rows to embedding_lookup_sparse
+ * (python_tf2/collcache_tf2/collcache_tf2/core/sparse_lookup_layer.py:196-265: unique -> lookup -> gather -> weighted
+ * segment sum / mean / sqrtn).  Here the rows of segment r, ids_dev[seg_off_dev[r] .. seg_off_dev[r + 1]), are read
+ * from where they live (table t, cache_dev, host_dev as for ugk_extract_mix_*; t.kind 0 = no table: row = id, read from
+ * host_dev, which may be HBM) and combined on the way:
+ *   out[r, :] = sum_j w_j x_j                                   combiner 0 (sum)
+ *             = sum_j w_j x_j / sum_j w_j                       combiner 1 (mean)
+ *             = sum_j w_j x_j / sqrt(sum_j w_j^2)               combiner 2 (sqrtn)
+ * with w_j = weights_dev[j] (1 when weights_dev is NULL), a zero denominator giving a zero row (div_no_nan), an empty
+ * segment a zero row.  Elements are fp32 (elem_bytes 4) or fp16 (2) and are added in fp32 in the order of the ids, one
+ * fused multiply-add each; the output has the element type of the rows.  The nnz x row_bytes intermediate of a lookup
+ * followed by a segment sum is never written.  seg_off_dev: n_rows + 1 ascending offsets into ids_dev, the last one
+ * nnz.  row_bytes: a multiple of 16, at most 4096.  Status, host mirror and the per-workgroup count words are those of
+ * ugk_extract_mix_* (the counts are of ids, not of output rows).  An id without a row sets UGK_ST_KEY_OUT_OF_RANGE and
+ * adds nothing. */
+int ugk_extract_pool_u32(ugk_table_t t, const uint32_t *ids_dev, const int64_t *seg_off_dev, const float *weights_dev,
+                         size_t n_rows, uint64_t nnz, int combiner, int elem_bytes, const void *cache_dev,
+                         uint64_t cache_rows, const void *host_dev, uint64_t host_rows, void *out_dev, size_t row_bytes,
+                         uint32_t *status_dev, uint32_t *host_mirror, uint64_t *group_counts_host,
+                         uint32_t *num_groups_host, void *stream);
+int ugk_extract_pool_i64(ugk_table_t t, const int64_t *ids_dev, const int64_t *seg_off_dev, const float *weights_dev,
+                         size_t n_rows, uint64_t nnz, int combiner, int elem_bytes, const void *cache_dev,
+                         uint64_t cache_rows, const void *host_dev, uint64_t host_rows, void *out_dev, size_t row_bytes,
+                         uint32_t *status_dev, uint32_t *host_mirror, uint64_t *group_counts_host,
+                         uint32_t *num_groups_host, void *stream);
 
 /* ---- rows that crossed the host link once, kept where a refresh finds them ---------------------------------------
  * The rows a refresh inserts (RefreshSession::refresh_after_solve_new, cache_context.cu:4054-4090: rows copied host ->

@@ -332,6 +332,26 @@ static inline uint64_t mix64(uint64_t x) {
   return x;
 }
 
+int orc_pool_f64(const double *table, size_t num_rows_table, size_t dim, const int64_t *ids, const int64_t *seg_off,
+                 const double *weights, size_t n_rows, int combiner, double *out) {
+  for (size_t r = 0; r < n_rows; ++r) {
+    double *o = out + r * dim;
+    double den = 0.0;
+    for (size_t c = 0; c < dim; ++c) o[c] = 0.0;
+    for (int64_t j = seg_off[r]; j < seg_off[r + 1]; ++j) {
+      if (ids[j] < 0 || (uint64_t)ids[j] >= num_rows_table) return 1;
+      const double w = weights ? weights[j] : 1.0;
+      const double *x = table + (size_t)ids[j] * dim;
+      for (size_t c = 0; c < dim; ++c) o[c] += w * x[c];
+      den += combiner == 2 ? w * w : w;
+    }
+    if (combiner == 0) continue;
+    if (combiner == 2) den = sqrt(den);
+    for (size_t c = 0; c < dim; ++c) o[c] = den != 0.0 ? o[c] / den : 0.0;
+  }
+  return 0;
+}
+
 size_t orc_dedup_i64(const int64_t *keys, size_t n, int64_t *unique, uint32_t *inverse) {
   size_t cap = 16;
   while (cap < 2 * n) cap <<= 1;

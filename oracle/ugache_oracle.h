@@ -22,6 +22,7 @@
  *   orc_rep_solve, orc_cache_capacity – closed forms on hand-worked cases
  *   orc_refresh_plan     – Python set algebra and free-list conservation
  *   orc_dedup            – numpy.unique(return_inverse=True)
+ *   orc_pool_f64         – numpy.add.at over float64 rows, and hand-worked segments
  * No function here is "parity unpinned".
  */
 #ifndef UGACHE_ORACLE_H_
@@ -141,6 +142,14 @@ int orc_refresh_plan(const uint32_t *old_block, const uint32_t *new_block, uint3
 /* caller-side dedup (python_tf2/collcache_tf2/collcache_tf2/core/sparse_lookup_layer.py:197 array_ops.unique):
  * unique keys in first-occurrence order and inverse[i] = position of keys[i] in unique.  Returns #unique. */
 size_t orc_dedup_i64(const int64_t *keys, size_t n, int64_t *unique, uint32_t *inverse);
+
+/* The per-sample combination that follows a sparse lookup (embedding_lookup_sparse as called by
+ * python_tf2/collcache_tf2/collcache_tf2/core/sparse_lookup_layer.py:196-265), in double precision:
+ * out[r, :] = sum over j in [seg_off[r], seg_off[r + 1]) of w_j * table[ids[j], :] (w_j = 1 when weights is NULL),
+ * divided by sum w_j (combiner 1, "mean") or sqrt(sum w_j^2) (combiner 2, "sqrtn"); a zero denominator gives a zero
+ * row (div_no_nan).  table: [num_rows_table, dim] doubles.  Returns non-zero if an id is out of range. */
+int orc_pool_f64(const double *table, size_t num_rows_table, size_t dim, const int64_t *ids, const int64_t *seg_off,
+                 const double *weights, size_t n_rows, int combiner, double *out);
 
 /* ---- CPU baseline leg (bench.py only): the same gather as orc_gather_*, OpenMP over keys ---- */
 int orc_omp_threads(void);

@@ -352,6 +352,104 @@ int extract_mix(ugk_table_t t, const K *keys, size_t n, const void *cache, uint6
   return 0;
 }
 
+// fp16 <-> fp32 without compiler support for _Float16 in every build: the bit patterns by hand
+inline float half_to_float(uint16_t h) {
+  const uint32_t sign = (uint32_t)(h >> 15) << 31, exp = (h >> 10) & 31u, man = h & 1023u;
+  uint32_t bits;
+  if (exp == 0) {
+    if (man == 0) bits = sign;
+    else {
+      int e = -1;
+      uint32_t m = man;
+      do { ++e; m <<= 1; } while (!(m & 1024u));
+      bits = sign | ((uint32_t)(127 - 15 - e) << 23) | ((m & 1023u) << 13);
+    }
+  } else if (exp == 31) bits = sign | 0x7f800000u | (man << 13);
+  else bits = sign | ((exp + 112u) << 23) | (man << 13);
+  float f;
+  memcpy(&f, &bits, 4);
+  return f;
+}
+inline uint16_t float_to_half(float f) {  // round to nearest even
+  uint32_t x;
+  memcpy(&x, &f, 4);
+  const uint32_t sign = (x >> 16) & 0x8000u;
+  x &= 0x7fffffffu;
+  if (x >= 0x7f800000u) return (uint16_t)(sign | 0x7c00u | (x > 0x7f800000u ? 0x200u : 0));
+  if (x >= 0x477ff000u) return (uint16_t)(sign | 0x7c00u);  // rounds to infinity
+  if (x < 0x33000001u) return (uint16_t)sign;               // rounds to zero
+  int e = (int)(x >> 23) - 127;
+  uint32_t m = (x & 0x7fffffu) | 0x800000u;
+  int shift = e < -14 ? 13 + (-14 - e) : 13;
+  uint32_t half_m = m >> shift, rest = m & ((1u << shift) - 1), mid = 1u << (shift - 1);
+  if (rest > mid || (rest == mid && (half_m & 1u))) ++half_m;
+  const uint32_t half_e = e < -14 ? 0 : (uint32_t)(e + 15);
+  return (uint16_t)(sign | ((half_e << 10) + (half_m - (e < -14 ? 0 : 1024u))));
+}
+
+template <typename K>
+int extract_pool(ugk_table_t t, const K *ids, const int64_t *seg_off, const float *weights, size_t n_rows,
+                 uint64_t nnz, int combiner, int elem_bytes, const void *cache, uint64_t cache_rows, const void *host,
+                 uint64_t host_rows, void *out, size_t rb, uint32_t *status, uint32_t *mirror, uint64_t *counts,
+                 uint32_t *num_groups) {
+  if (num_groups) *num_groups = 0;
+  if (n_rows == 0) return 0;
+  REQUIRE(seg_off && out && status && (nnz == 0 || ids), "ugk_extract_pool: null pointer");
+  REQUIRE(combiner >= 0 && combiner <= 2 && (elem_bytes == 2 || elem_bytes == 4), "ugk_extract_pool: bad argument");
+  REQUIRE(rb > 0 && rb % 16 == 0 && rb <= 4096, "ugk_extract_pool: rows of %zu bytes", rb);
+  if (t.kind != 0 && check_table(t, "ugk_extract_pool")) return 1;
+  const size_t dim = rb / elem_bytes;
+  uint64_t local = 0, others = 0;
+  std::vector<float> acc(dim);
+  for (size_t r = 0; r < n_rows; ++r) {
+    std::fill(acc.begin(), acc.end(), 0.f);
+    float wsum = 0.f;
+    for (int64_t j = seg_off[r]; j < seg_off[r + 1]; ++j) {
+      const uint64_t key = k64(ids[j]);
+      const Found f = t.kind ? lookup(t, key) : Found{false, 0, 0};
+      const char *row = nullptr;
+      bool from_cache = false;
+      if (f.hit && f.loc == UGK_LOC_LOCAL && f.off < cache_rows) {
+        row = (const char *)cache + (size_t)f.off * rb;
+        from_cache = true;
+      } else if (f.hit && f.loc == UGK_LOC_HOST && f.off < host_rows) {
+        row = (const char *)host + (size_t)f.off * rb;
+      } else if (!f.hit && fallback_row(t, key) < host_rows) {
+        row = (const char *)host + fallback_row(t, key) * rb;
+      } else {
+        or_status(status, UGK_ST_KEY_OUT_OF_RANGE, mirror);
+      }
+      if (from_cache) ++local;
+      else ++others;
+      if (!row) continue;
+      const float w = weights ? weights[j] : 1.f;
+      wsum += combiner == 2 ? w * w : w;
+      for (size_t c = 0; c < dim; ++c) {
+        float x;
+        if (elem_bytes == 4) memcpy(&x, row + c * 4, 4);
+        else {
+          uint16_t h;
+          memcpy(&h, row + c * 2, 2);
+          x = half_to_float(h);
+        }
+        acc[c] = std::fma(w, x, acc[c]);
+      }
+    }
+    const float denom = combiner == 1 ? wsum : combiner == 2 ? std::sqrt(wsum) : 1.f;
+    for (size_t c = 0; c < dim; ++c) {
+      const float y = denom != 0.f ? acc[c] / denom : 0.f;
+      if (elem_bytes == 4) memcpy((char *)out + (r * dim + c) * 4, &y, 4);
+      else {
+        const uint16_t h = float_to_half(y);
+        memcpy((char *)out + (r * dim + c) * 2, &h, 2);
+      }
+    }
+  }
+  if (counts) counts[0] = (others << 32) | local;
+  if (num_groups) *num_groups = 1;
+  return 0;
+}
+
 template <typename K>
 int dedup(const K *keys, size_t n, K *unique_out, uint32_t *inverse, uint32_t *rep, uint32_t *n_unique,
           uint32_t *n_unique_host) {
@@ -651,6 +749,21 @@ int ugk_extract_mix_i64(ugk_table_t t, const int64_t *keys, size_t n, const void
                         const void *host, uint64_t host_rows, void *out, size_t rb, uint32_t *status, uint32_t *mirror,
                         uint64_t *counts, uint32_t *num_groups, uint32_t, void *) {
   return extract_mix(t, keys, n, cache, cache_rows, host, host_rows, out, rb, status, mirror, counts, num_groups);
+}
+
+int ugk_extract_pool_u32(ugk_table_t t, const uint32_t *ids, const int64_t *seg_off, const float *weights, size_t n_rows,
+                         uint64_t nnz, int combiner, int elem_bytes, const void *cache, uint64_t cache_rows,
+                         const void *host, uint64_t host_rows, void *out, size_t rb, uint32_t *status, uint32_t *mirror,
+                         uint64_t *counts, uint32_t *num_groups, void *) {
+  return extract_pool(t, ids, seg_off, weights, n_rows, nnz, combiner, elem_bytes, cache, cache_rows, host, host_rows,
+                      out, rb, status, mirror, counts, num_groups);
+}
+int ugk_extract_pool_i64(ugk_table_t t, const int64_t *ids, const int64_t *seg_off, const float *weights, size_t n_rows,
+                         uint64_t nnz, int combiner, int elem_bytes, const void *cache, uint64_t cache_rows,
+                         const void *host, uint64_t host_rows, void *out, size_t rb, uint32_t *status, uint32_t *mirror,
+                         uint64_t *counts, uint32_t *num_groups, void *) {
+  return extract_pool(t, ids, seg_off, weights, n_rows, nnz, combiner, elem_bytes, cache, cache_rows, host, host_rows,
+                      out, rb, status, mirror, counts, num_groups);
 }
 
 int ugk_extract_mix_staged_u32(ugk_table_t t, const uint32_t *keys, size_t n, const void *cache, uint64_t cache_rows,

@@ -1362,6 +1362,16 @@ def test_serving_stack_from_a_ps_config_file(tmp_path):
                                               emb_vec_dtype=torch.float32, unique_in_library=True)
                 got2 = fused(sp_ids, weights, combiner=combiner).cpu().numpy()
                 assert np.allclose(got2, want, rtol=1e-5, atol=1e-5 * np.abs(want).max())
+                # ... and with lookup and combination in one kernel of the library (one serving step each)
+                pooled = hps.SparseLookupLayer(model_name="dlrm", table_id=0, emb_vec_size=dim,
+                                               emb_vec_dtype=torch.float32, fused=True)
+                before = _basics.info(0)["lookups"]
+                got3 = pooled(sp_ids, weights, combiner=combiner).cpu().numpy()
+                assert _basics.info(0)["lookups"] == before + 1
+                assert np.allclose(got3, want, rtol=1e-5, atol=1e-5 * np.abs(want).max())
+                assert np.allclose(got3, ORC.pool(rows, ids, np.concatenate([[0], np.cumsum(lens)]),
+                                                  None if weights is None else w, combiner or "mean"),
+                                   rtol=1e-5, atol=1e-5 * np.abs(want).max())
         with pytest.raises(ValueError):
             sparse(sp_ids, None, combiner="max")
         hps.SetStepProfileValue(profile_type=kLogL1FeatureBytes, value=123.0)
@@ -1369,6 +1379,56 @@ def test_serving_stack_from_a_ps_config_file(tmp_path):
         hps.Report()
     finally:
         hps.Shutdown()
+
+
+@pytest.mark.parametrize("pct,table_kind", [(1.0, "FLAT"), (0.0, "FLAT"), (0.3, "FLAT"), (0.3, "HASH")])
+@pytest.mark.parametrize("dtype,dim", [(torch.float32, 32), (torch.float16, 64), (torch.float32, 100)])
+@pytest.mark.parametrize("kdtype", [torch.int32, torch.int64])
+def test_pooled_lookup_through_the_library(pct, table_kind, dtype, dim, kdtype, monkeypatch):
+    """coll_torch_lookup_pooled (coll_cache_lookup_pooled*): lookup and combination of ragged, weighted segments in one
+    call, against the oracle's float64 combination of the same rows; the group sizes count the ids by source, and the
+    ids are counted as hotness like those of any lookup.  Tolerance: 1e-5 of the magnitude of the terms (fp32 sums of
+    at most 40 terms), plus fp16's rounding of the result where the table is fp16."""
+    monkeypatch.setenv("COLL_HASH_TABLE", table_kind)
+    monkeypatch.setenv("COLL_GPU_RECORD", "1")
+    rng = np.random.default_rng(int(pct * 10) + dim)
+    n_item = 30_000
+    co.config(make_config(n_item, pct))
+    co.coll_cache_record_init(0)
+    perm = rng.permutation(n_item)
+    s0 = perm[zipf_ranks(rng, 100_000, n_item, 1.05)]
+    co.coll_torch_record(0, torch.from_numpy(s0).to(torch.int32))
+    emb = co.coll_torch_create_emb_shm(0, n_item, dim, dtype)
+    emb.copy_(torch.from_numpy(rng.standard_normal((n_item, dim)).astype(np.float32)).to(dtype))
+    table = emb.float().numpy().astype(np.float64)
+    co.coll_torch_init_t(0, 0, emb, pct)
+    _, nid = expected_cached_set(s0.astype(np.uint32), n_item, pct) if 0 < pct < 1 else (None, None)
+    counted = []
+    for n_rows in (1, 64, 5_000):
+        lens = rng.choice([0, 1, 3, 8, 40], size=n_rows, p=[0.05, 0.35, 0.3, 0.25, 0.05])
+        off = np.concatenate([[0], np.cumsum(lens)]).astype(np.int64)
+        ids = perm[zipf_ranks(rng, int(off[-1]), n_item, 1.05)] if off[-1] else np.zeros(0, np.int64)
+        w = rng.uniform(0.1, 2.0, size=len(ids)).astype(np.float32)
+        t_ids, t_off, t_w = torch.from_numpy(ids).to(kdtype).cuda(), torch.from_numpy(off).cuda(), torch.from_numpy(w).cuda()
+        for combiner in ("sum", "mean", "sqrtn"):
+            for weights in (None, t_w):
+                got = co.coll_torch_lookup_pooled(0, t_ids, t_off, weights, combiner)
+                counted.append(ids.astype(np.uint32))
+                assert tuple(got.shape) == (n_rows, dim) and got.dtype == dtype
+                want = ORC.pool(table, ids, off, None if weights is None else w, combiner)
+                mag = ORC.pool(np.abs(table), ids, off, None if weights is None else w, combiner)
+                bound = 1e-5 * mag + (1e-3 * np.abs(want) + 2.0 ** -25 if dtype == torch.float16 else 0.0) + 1e-30
+                assert (np.abs(got.float().cpu().numpy().astype(np.float64) - want) <= bound).all(), (n_rows, combiner)
+                n_local = len(ids) if pct == 1.0 else 0 if pct == 0.0 else int((nid[ids] == 0).sum())
+                assert _basics.last_group_offset(0) == [0, n_local, len(ids)]
+    if not 0 < pct < 1:  # no ranking was needed to build: what was recorded up front is still waiting in the recorder
+        counted.append(s0.astype(np.uint32))
+    want_k, want_c = ORC.freq_rank(np.concatenate(counted))
+    got_k, got_c = np.zeros(n_item, np.uint32), np.zeros(n_item, np.uint32)
+    m = _basics.C_LIB_CTYPES.coll_cache_rank_hotness(0, got_k.ctypes.data, got_c.ctypes.data, n_item)
+    assert m == len(want_k) and np.array_equal(got_k[:m], want_k) and np.array_equal(got_c[:m], want_c)
+    if dim == 100 and dtype == torch.float32:  # 400-byte rows: a multiple of 16 bytes, but not of whole lane groups
+        assert co.c_lib.pooled_lookup_supported()
 
 
 @pytest.mark.parametrize("impl", ["", "SMMaskPhase"])

@@ -574,6 +574,156 @@ def test_extract_mix_at_every_launch_shape(kind, rb):
         mirror.free()
 
 
+def _pool_reference(table_f64, ids, seg_off, weights, combiner):
+    """embedding_lookup_sparse in float64: weighted sum of every segment's rows, divided by the sum of the weights
+    (mean) or the root of the sum of their squares (sqrtn); a zero denominator and an empty segment give a zero row"""
+    n_rows = len(seg_off) - 1
+    w = np.ones(len(ids), np.float64) if weights is None else weights.astype(np.float64)
+    out = np.zeros((n_rows, table_f64.shape[1]), np.float64)
+    seg = np.repeat(np.arange(n_rows), np.diff(seg_off))
+    np.add.at(out, seg, table_f64[ids] * w[:, None])
+    if combiner == 0:
+        return out
+    den = np.zeros(n_rows, np.float64)
+    np.add.at(den, seg, w if combiner == 1 else w * w)
+    if combiner == 2:
+        den = np.sqrt(den)
+    safe = np.where(den != 0, den, 1.0)
+    return np.where(den[:, None] != 0, out / safe[:, None], 0.0)
+
+
+@pytest.mark.parametrize("kind", ["none", "flat", "hash"])
+@pytest.mark.parametrize("dim,etype", [(4, np.float32), (32, np.float32), (128, np.float32), (512, np.float32),
+                                       (1024, np.float32), (8, np.float16), (64, np.float16), (256, np.float16),
+                                       (2048, np.float16)])
+def test_pooled_extraction_matches_a_float64_segment_sum(kind, dim, etype):
+    """ugk_extract_pool_*: rows looked up and combined per segment in one kernel (sum, mean, sqrtn; with and without
+    weights, negative and zero ones among them; segments that are empty, single, longer than a lane group).  fp32
+    rows within 1e-5 of the magnitude of the terms that were added (sum of |w x|, over the denominator), fp16 rows
+    within 1e-3 of the result on top (the output is rounded to fp16); the counts are those of the ids by source, as for
+    the plain fused extraction."""
+    rng = np.random.default_rng(dim + len(kind))
+    nkeys = 20_000
+    rb = dim * np.dtype(etype).itemsize
+    host = rng.standard_normal((nkeys, dim)).astype(etype)
+    host_bytes = host.view(np.uint8).reshape(nkeys, rb)
+    if kind == "none":  # no table: the id is the row, the "host" table may be anywhere (here HBM)
+        tb = hip.table(0, None, 0)
+        cached = np.zeros(0, np.int64)
+        mem = None
+    else:
+        cached = rng.choice(nkeys, nkeys * 3 // 4, replace=False).astype(np.int64)
+        if kind == "flat":
+            mem, tb = _make_flat(nkeys)
+        else:
+            mem, tb, _ = _make_hash(len(cached))
+    slots = rng.permutation(len(cached)).astype(np.uint32)
+    cache = np.zeros((max(len(cached), 1), rb), np.uint8)
+    if len(cached):
+        cache[slots] = host_bytes[cached]
+        assert _insert(tb, cached, slots) == 0
+    is_cached = np.zeros(nkeys, bool)
+    is_cached[cached] = True
+    pin = pinned_from(host_bytes)
+    mirror = pinned_from(np.zeros(4, np.uint32))
+    words = PinnedArray((hip.lib().ugk_extract_mix_max_groups(),), np.uint64)
+    try:
+        st = dev_zeros_u32(1)
+        d_cache = to_dev(cache)
+        f64 = host.astype(np.float64)
+        for n_rows in (1, 7, 3_000):
+            lens = rng.choice([0, 1, 2, 5, 9, 40, 70], size=n_rows, p=[0.05, 0.3, 0.2, 0.2, 0.15, 0.07, 0.03])
+            seg_off = np.concatenate([[0], np.cumsum(lens)]).astype(np.int64)
+            nnz = int(seg_off[-1])
+            ids = rng.integers(0, nkeys, size=max(nnz, 1)).astype(np.int64)[:nnz]
+            wts = rng.standard_normal(nnz).astype(np.float32)
+            wts[rng.random(nnz) < 0.1] = 0.0
+            d_ids, d_off, d_w = to_dev(ids if nnz else np.zeros(1, np.int64)), to_dev(seg_off), to_dev(wts if nnz else np.zeros(1, np.float32))
+            for combiner in (0, 1, 2):
+                for weights in (None, wts):
+                    out = dev_bytes(n_rows * rb, fill=0x7F)
+                    groups = C.c_uint32(0)
+                    hip.call("ugk_extract_pool_i64", tb, ptr(d_ids), ptr(d_off), None if weights is None else ptr(d_w),
+                             n_rows, nnz, combiner, np.dtype(etype).itemsize, ptr(d_cache), len(cached), pin.ptr, nkeys,
+                             ptr(out), rb, ptr(st), mirror.ptr, words.ptr, C.byref(groups), None)
+                    sync()
+                    assert status_value(st) == 0
+                    w = words.array[:groups.value]
+                    n_local = int(is_cached[ids].sum())
+                    assert [int((w & np.uint64(0xFFFFFFFF)).sum()), int((w >> np.uint64(32)).sum())] == [n_local, nnz - n_local]
+                    got = to_np(out)[: n_rows * rb].view(etype).reshape(n_rows, dim).astype(np.float64)
+                    want = _pool_reference(f64, ids, seg_off, weights, combiner)
+                    # fp32 adds of n terms are off by at most n 2^-24 of the terms' magnitudes; an fp16 output is
+                    # rounded to 11 bits on top.  (A mean over signed weights that nearly cancel is large and still
+                    # as accurate as its terms.)
+                    absw = None if weights is None else np.abs(wts)
+                    mag = _pool_reference(np.abs(f64), ids, seg_off, absw, 0)
+                    if combiner:
+                        den = _pool_reference(np.ones((nkeys, 1)), ids, seg_off,
+                                              weights if combiner == 1 or weights is None else wts * wts, 0)
+                        den = np.abs(den) if combiner == 1 else np.sqrt(den)
+                        mag = np.where(den != 0, mag / np.where(den != 0, den, 1.0), 0.0)
+                        if combiner == 1 and weights is not None:
+                            # the sum of signed weights is itself a rounded sum: its relative error is that of its
+                            # terms' magnitudes over what is left of them
+                            sum_abs = _pool_reference(np.ones((nkeys, 1)), ids, seg_off, absw, 0)
+                            mag = mag + np.abs(want) * np.where(den != 0, sum_abs / np.where(den != 0, den, 1.0), 0.0)
+                    # (fp16 results below 2^-14 are subnormal: steps of 2^-24 whatever their size)
+                    bound = 1e-5 * mag + (1e-3 * np.abs(want) + 2.0 ** -25 if etype == np.float16 else 0.0) + 1e-30
+                    if etype == np.float16:  # a mean over weights that nearly cancel may leave fp16's range
+                        big = np.abs(want) > 6.0e4
+                        assert np.isinf(got[big & (np.abs(want) > 6.6e4)]).all()
+                        got, want = np.where(big, 0.0, got), np.where(big, 0.0, want)
+                    worst = np.unravel_index(np.argmax(np.abs(got - want) - bound), got.shape)
+                    assert (np.abs(got - want) <= bound).all(), "%s dim %d rows %d combiner %d weights %s: [%d, %d] got %r " \
+                        "want %r bound %r ids %d" % (kind, dim, n_rows, combiner, weights is not None, worst[0], worst[1],
+                                                    float(got[worst]), float(want[worst]), float(bound[worst]),
+                                                    int(lens[worst[0]]))
+    finally:
+        sync()
+        pin.free()
+        mirror.free()
+        words.free()
+
+
+def test_pooled_extraction_hand_worked():
+    # rows r = [r, 10 r]; segments {1, 2}, {3}, {}, {4, 4} with weights 1 2 | 3 | | 1 -1
+    host = np.array([[r, 10 * r, 0, 0] for r in range(6)], np.float32)
+    pin = pinned_from(host.view(np.uint8).reshape(6, 16))
+    try:
+        ids, off = to_dev(np.array([1, 2, 3, 4, 4], np.int64)), to_dev(np.array([0, 2, 3, 3, 5], np.int64))
+        wts = to_dev(np.array([1, 2, 3, 1, -1], np.float32))
+        st = dev_zeros_u32(1)
+        cache = dev_bytes(16)
+
+        def run(combiner, w):
+            out = dev_bytes(4 * 16, fill=0x55)
+            hip.call("ugk_extract_pool_i64", hip.table(0, None, 0), ptr(ids), ptr(off), w, 4, 5, combiner, 4, ptr(cache), 0,
+                     pin.ptr, 6, ptr(out), 16, ptr(st), None, None, None, None)
+            sync()
+            assert status_value(st) == 0
+            return to_np(out)[:64].view(np.float32).reshape(4, 4)[:, :2].tolist()
+
+        assert run(0, None) == [[3, 30], [3, 30], [0, 0], [8, 80]]
+        assert run(0, ptr(wts)) == [[5, 50], [9, 90], [0, 0], [0, 0]]
+        assert run(1, None) == [[1.5, 15], [3, 30], [0, 0], [4, 40]]
+        assert run(1, ptr(wts)) == [[5 / 3, 50 / 3], [3, 30], [0, 0], [0, 0]] or \
+            np.allclose(run(1, ptr(wts)), [[5 / 3, 50 / 3], [3, 30], [0, 0], [0, 0]], rtol=1e-6)  # weights cancel: 0 / 0 -> 0
+        got = run(2, ptr(wts))
+        assert np.allclose(got, [[5 / 5 ** 0.5, 50 / 5 ** 0.5], [3, 30], [0, 0], [0, 0]], rtol=1e-6)
+        # an id without a row flags the launch and adds nothing
+        bad = to_dev(np.array([1, 77, 3, 4, 4], np.int64))
+        out = dev_bytes(4 * 16)
+        hip.call("ugk_extract_pool_i64", hip.table(0, None, 0), ptr(bad), ptr(off), None, 4, 5, 0, 4, ptr(cache), 0, pin.ptr,
+                 6, ptr(out), 16, ptr(st), None, None, None, None)
+        sync()
+        assert status_value(st) & hip.ST_KEY_OUT_OF_RANGE
+        assert to_np(out)[:64].view(np.float32).reshape(4, 4)[0, :2].tolist() == [1, 10]
+    finally:
+        sync()
+        pin.free()
+
+
 def _fmix64(x):
     x = np.asarray(x, np.uint64).copy()
     x ^= x >> np.uint64(33)

@@ -400,6 +400,44 @@ def test_dedup_matches_numpy_unique():
         assert np.array_equal(uniq, keys[np.sort(first)])  # first-occurrence order
 
 
+def test_pool_hand_worked_and_against_numpy():
+    """orc_pool_f64 against the definition of embedding_lookup_sparse's combiners: hand-worked segments (an empty one,
+    weights that cancel), then numpy.add.at over random ragged segments"""
+    table = np.array([[r, 10.0 * r] for r in range(6)])
+    ids, off = np.array([1, 2, 3, 4, 4]), np.array([0, 2, 3, 3, 5])
+    w = np.array([1.0, 2.0, 3.0, 1.0, -1.0])
+    assert ORC.pool(table, ids, off, None, "sum").tolist() == [[3, 30], [3, 30], [0, 0], [8, 80]]
+    assert ORC.pool(table, ids, off, w, "sum").tolist() == [[5, 50], [9, 90], [0, 0], [0, 0]]
+    assert ORC.pool(table, ids, off, None, "mean").tolist() == [[1.5, 15], [3, 30], [0, 0], [4, 40]]
+    assert np.allclose(ORC.pool(table, ids, off, w, "mean"), [[5 / 3, 50 / 3], [3, 30], [0, 0], [0, 0]], rtol=1e-15)
+    assert np.allclose(ORC.pool(table, ids, off, w, "sqrtn"),
+                       [[5 / 5 ** 0.5, 50 / 5 ** 0.5], [3, 30], [0, 0], [0, 0]], rtol=1e-15)
+    assert np.allclose(ORC.pool(table, ids, off, None, "sqrtn"),
+                       [[3 / 2 ** 0.5, 30 / 2 ** 0.5], [3, 30], [0, 0], [8 / 2 ** 0.5, 80 / 2 ** 0.5]], rtol=1e-15)
+    with pytest.raises(IndexError):
+        ORC.pool(table, np.array([1, 6]), np.array([0, 2]), None, "sum")
+    rng = np.random.default_rng(23)
+    table = rng.standard_normal((500, 7))
+    lens = rng.integers(0, 9, size=300)
+    off = np.concatenate([[0], np.cumsum(lens)])
+    ids = rng.integers(0, 500, size=off[-1])
+    w = rng.random(off[-1]) + 0.1
+    seg = np.repeat(np.arange(300), lens)
+    for weights in (None, w):
+        ww = np.ones(len(ids)) if weights is None else weights
+        total = np.zeros((300, 7))
+        np.add.at(total, seg, table[ids] * ww[:, None])
+        den1, den2 = np.zeros(300), np.zeros(300)
+        np.add.at(den1, seg, ww)
+        np.add.at(den2, seg, ww * ww)
+        assert np.allclose(ORC.pool(table, ids, off, weights, 0), total, rtol=1e-13, atol=1e-13)
+        safe = lambda d: np.where(d != 0, d, 1.0)[:, None]
+        assert np.allclose(ORC.pool(table, ids, off, weights, 1), np.where(den1[:, None] != 0, total / safe(den1), 0),
+                           rtol=1e-13, atol=1e-13)
+        assert np.allclose(ORC.pool(table, ids, off, weights, 2),
+                           np.where(den2[:, None] != 0, total / safe(np.sqrt(den2)), 0), rtol=1e-13, atol=1e-13)
+
+
 def test_oracle_reproduces_the_committed_golden_case():
     """tests/golden/extract_small.json was written by brute-force Python loops (tests/golden/make_fixtures.py), not
     by the oracle: ranking, placement, capacity and the gather must all land on it"""

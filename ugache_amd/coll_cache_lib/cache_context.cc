@@ -540,6 +540,21 @@ static int ExtractMix(ugk_table_t t, const Id64Type *keys, size_t n, const void 
                              s);
 }
 
+static int ExtractPool(ugk_table_t t, const IdType *ids, const int64_t *seg_off, const float *w, size_t n_rows,
+                       uint64_t nnz, int combiner, int elem_bytes, const void *cache, uint64_t cache_rows,
+                       const void *host, uint64_t host_rows, void *out, size_t rb, uint32_t *st, uint32_t *mirror,
+                       uint64_t *counts, uint32_t *groups, StreamHandle s) {
+  return ugk_extract_pool_u32(t, ids, seg_off, w, n_rows, nnz, combiner, elem_bytes, cache, cache_rows, host, host_rows,
+                              out, rb, st, mirror, counts, groups, s);
+}
+static int ExtractPool(ugk_table_t t, const Id64Type *ids, const int64_t *seg_off, const float *w, size_t n_rows,
+                       uint64_t nnz, int combiner, int elem_bytes, const void *cache, uint64_t cache_rows,
+                       const void *host, uint64_t host_rows, void *out, size_t rb, uint32_t *st, uint32_t *mirror,
+                       uint64_t *counts, uint32_t *groups, StreamHandle s) {
+  return ugk_extract_pool_i64(t, ids, seg_off, w, n_rows, nnz, combiner, elem_bytes, cache, cache_rows, host, host_rows,
+                              out, rb, st, mirror, counts, groups, s);
+}
+
 static int NonLocalFlags(ugk_table_t t, const IdType *keys, size_t n, uint64_t *flags, StreamHandle s) {
   return ugk_nonlocal_flags_u32(t, keys, n, flags, s);
 }
@@ -1010,6 +1025,84 @@ void ExtractSession::Wait(StreamHandle stream) {
   _group_offset[2] = (uint32_t)_async_last_nodes;
   _cache_ctx->progress.fetch_add(_async_pending);
   _async_pending = 0;
+}
+
+template <typename KeyT>
+void ExtractSession::ExtractPooledImpl(const KeyT *nodes, const int64_t *seg_off, const float *weights,
+                                       size_t num_rows, size_t num_nodes, int combiner, int elem_bytes, void *output,
+                                       StreamHandle stream, uint64_t task_key) {
+  CacheContext *ctx = _cache_ctx.get();
+  auto profiler = ctx->_coll_cache ? ctx->_coll_cache->_profiler : nullptr;
+  const size_t rb = ctx->_row_bytes;
+  InFlight in_flight(this);  // from before the kernel reads the table until the output is complete
+  Wait(stream);
+  _group_offset[0] = 0;
+  if (num_rows == 0) {
+    _group_offset[1] = _group_offset[2] = 0;
+    ctx->progress.fetch_add(1);
+    return;
+  }
+  CHECK_NOTNULL(seg_off);
+  CHECK_NOTNULL(output);
+  CHECK(num_nodes == 0 || nodes != nullptr);
+  CHECK(combiner >= 0 && combiner <= 2) << "combiner is 0 (sum), 1 (mean) or 2 (sqrtn)";
+  CHECK(elem_bytes == 2 || elem_bytes == 4) << "rows are combined as fp16 or fp32 elements";
+  CHECK(rb % 16 == 0 && rb <= 4096 && rb % elem_bytes == 0)
+      << "pooled lookups take rows of a multiple of 16 bytes up to 4096, not " << rb;
+  NoteOutput(output, num_rows * rb);
+  // without a table the id is the row and everything comes from the one source there is (HBM for a full cache, the
+  // host table for none); otherwise the table decides per id, as in the fused extraction
+  ugk_table_t table{};
+  const void *cache = nullptr, *host = nullptr;
+  uint64_t cache_rows = 0;
+  const bool direct = ctx->IsDirectMapping();
+  if (direct) {
+    table.kind = 0;
+    host = ctx->_device_cache_data[0];
+  } else {
+    table = ctx->_new_hash_table->Table();
+    cache = ctx->_device_cache_data[ctx->_local_location_id];
+    host = ctx->_device_cache_data[ctx->_cpu_location_id];
+    cache_rows = ctx->_cache_space_capacity;
+  }
+  CHECK((((uintptr_t)cache | (uintptr_t)host | (uintptr_t)output) & 15u) == 0) << "pooled lookup: misaligned buffer";
+  void *keys_ready = RecordBegin(stream);
+  Timer t_host;
+  UGK_CALL(ExtractPool(table, nodes, seg_off, weights, num_rows, num_nodes, combiner, elem_bytes, cache, cache_rows,
+                       host, ctx->_num_total_nodes, output, rb, _status, _host_mirror, _mix_counts->ptr<uint64_t>(),
+                       &_mix_groups, stream));
+  if (num_nodes) RecordLaunch(nodes, num_nodes, keys_ready);
+  WaitForBatch(stream);
+  const double host_time = t_host.Passed();
+  JoinRecordOnHost();
+  CheckStatusWord(stream);
+  SumMixCounts();
+  uint32_t n_local = _host_mirror[kMirGroupSizes + UGK_LOC_LOCAL], n_miss = _host_mirror[kMirGroupSizes + UGK_LOC_HOST];
+  CHECK_EQ((size_t)n_local + n_miss, num_nodes);
+  if (direct && ctx->_cpu_location_id == -1) std::swap(n_local, n_miss);  // the one source is the HBM copy
+  _group_offset[1] = n_local;
+  _group_offset[2] = (uint32_t)num_nodes;
+  if (profiler && task_key != 0xffffffffffffffffull) {
+    profiler->LogStep(task_key, kLogL1FeatureBytes, (double)num_nodes * rb);
+    profiler->LogStep(task_key, kLogL1MissBytes, (double)n_miss * rb);
+    profiler->LogStep(task_key, kLogL3CacheCombineCacheTime, host_time);
+    profiler->LogEpochAdd(task_key, kLogEpochFeatureBytes, (double)num_nodes * rb);
+    profiler->LogEpochAdd(task_key, kLogEpochMissBytes, (double)n_miss * rb);
+  }
+  ctx->progress.fetch_add(1);
+}
+
+void ExtractSession::ExtractPooled(const IdType *nodes, const int64_t *seg_off, const float *weights, size_t num_rows,
+                                   size_t num_nodes, int combiner, int elem_bytes, void *output, StreamHandle stream,
+                                   uint64_t task_key) {
+  ExtractPooledImpl<IdType>(nodes, seg_off, weights, num_rows, num_nodes, combiner, elem_bytes, output, stream, task_key);
+}
+
+void ExtractSession::ExtractPooled64(const Id64Type *nodes, const int64_t *seg_off, const float *weights,
+                                     size_t num_rows, size_t num_nodes, int combiner, int elem_bytes, void *output,
+                                     StreamHandle stream, uint64_t task_key) {
+  ExtractPooledImpl<Id64Type>(nodes, seg_off, weights, num_rows, num_nodes, combiner, elem_bytes, output, stream,
+                              task_key);
 }
 
 void ExtractSession::ExtractFeat(const IdType *nodes, const size_t num_nodes, void *output, StreamHandle stream,

@@ -193,6 +193,10 @@ class ExtractSession {
   template <typename KeyT>
   size_t ExtractUniqueImpl(const KeyT *nodes, size_t num_nodes, void *output, uint32_t *inverse_out,
                            StreamHandle stream, uint64_t task_key);
+  template <typename KeyT>
+  void ExtractPooledImpl(const KeyT *nodes, const int64_t *seg_off, const float *weights, size_t num_rows,
+                         size_t num_nodes, int combiner, int elem_bytes, void *output, StreamHandle stream,
+                         uint64_t task_key);
   // Where the outputs of the last lookups went.  A caller that hands the same buffer over every time (the reference's
   // adapter does, adapter.cc:204-237) finds its rows in the memory-side cache; one that rotates over more buffers than
   // that cache holds is better served by streaming stores, and the kernels are told so (ugk_set_output_hint).
@@ -220,6 +224,18 @@ class ExtractSession {
   // same for 64-bit keys (dense ids below num_total_item); an extension over the reference
   void ExtractFeat64(const Id64Type *nodes, const size_t num_nodes, void *output, StreamHandle stream,
                      uint64_t task_key);
+  // Lookup and per-sample combination of a multi-hot feature in one kernel (an extension; embedding_lookup_sparse
+  // behind the TF2 sparse layer, sparse_lookup_layer.py:196-265): output[r, :] = the rows of the ids
+  // nodes[seg_off[r] .. seg_off[r + 1]) times their weights (null: 1), summed (combiner 0), divided by the sum of the
+  // weights (1) or by the root of the sum of their squares (2); elements are fp32 (elem_bytes 4) or fp16 (2), added in
+  // fp32.  nodes, seg_off (num_rows + 1 int64 offsets), weights: device pointers; output: device [num_rows, dim];
+  // blocking.  Rows must be multiples of 16 bytes of at most 4096.  The group sizes afterwards count ids.
+  void ExtractPooled(const IdType *nodes, const int64_t *seg_off, const float *weights, size_t num_rows,
+                     size_t num_nodes, int combiner, int elem_bytes, void *output, StreamHandle stream,
+                     uint64_t task_key);
+  void ExtractPooled64(const Id64Type *nodes, const int64_t *seg_off, const float *weights, size_t num_rows,
+                       size_t num_nodes, int combiner, int elem_bytes, void *output, StreamHandle stream,
+                       uint64_t task_key);
   // The distinct keys of the batch looked up once (an extension; the "unique -> lookup -> gather(idx)" of the TF2
   // layer, sparse_lookup_layer.py:196-209, with the unique inside): output[u, :] = row of the u-th distinct key
   // (in order of first claim, not sorted), inverse_out[i] = which distinct key position i holds, so that

@@ -26,6 +26,26 @@ void CollCache::lookup64(int replica_id, const Id64Type *nodes, const size_t num
   _profiler->LogStep(step_key, common::kLogL2CacheCopyTime, t.Passed());
 }
 
+void CollCache::lookup_pooled(int replica_id, const IdType *nodes, const int64_t *seg_off, const float *weights,
+                              size_t num_rows, size_t num_nodes, int combiner, int elem_bytes, void *output,
+                              StreamHandle stream, uint64_t step_key) {
+  Timer t;
+  CHECK_LT((size_t)replica_id, _session_list.size());
+  _session_list[replica_id]->ExtractPooled(nodes, seg_off, weights, num_rows, num_nodes, combiner, elem_bytes, output,
+                                           stream, step_key);
+  _profiler->LogStep(step_key, common::kLogL2CacheCopyTime, t.Passed());
+}
+
+void CollCache::lookup_pooled64(int replica_id, const Id64Type *nodes, const int64_t *seg_off, const float *weights,
+                                size_t num_rows, size_t num_nodes, int combiner, int elem_bytes, void *output,
+                                StreamHandle stream, uint64_t step_key) {
+  Timer t;
+  CHECK_LT((size_t)replica_id, _session_list.size());
+  _session_list[replica_id]->ExtractPooled64(nodes, seg_off, weights, num_rows, num_nodes, combiner, elem_bytes,
+                                             output, stream, step_key);
+  _profiler->LogStep(step_key, common::kLogL2CacheCopyTime, t.Passed());
+}
+
 size_t CollCache::lookup_unique(int replica_id, const IdType *nodes, size_t num_nodes, void *output,
                                 uint32_t *inverse_out, StreamHandle stream, uint64_t step_key) {
   Timer t;

@@ -56,6 +56,13 @@ class CollCache : public std::enable_shared_from_this<CollCache> {
   void lookup64(int replica_id, const Id64Type *nodes, const size_t num_nodes, void *output, StreamHandle stream,
                 uint64_t step_key);
   // distinct keys looked up once: rows of the distinct keys + which of them every position holds (extension)
+  // lookup + per-sample combination of a multi-hot feature (ExtractSession::ExtractPooled)
+  void lookup_pooled(int replica_id, const IdType *nodes, const int64_t *seg_off, const float *weights, size_t num_rows,
+                     size_t num_nodes, int combiner, int elem_bytes, void *output, StreamHandle stream,
+                     uint64_t step_key);
+  void lookup_pooled64(int replica_id, const Id64Type *nodes, const int64_t *seg_off, const float *weights,
+                       size_t num_rows, size_t num_nodes, int combiner, int elem_bytes, void *output,
+                       StreamHandle stream, uint64_t step_key);
   size_t lookup_unique(int replica_id, const IdType *nodes, size_t num_nodes, void *output, uint32_t *inverse_out,
                        StreamHandle stream, uint64_t step_key);
   size_t lookup_unique64(int replica_id, const Id64Type *nodes, size_t num_nodes, void *output, uint32_t *inverse_out,

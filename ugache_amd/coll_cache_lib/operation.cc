@@ -223,6 +223,26 @@ void coll_cache_lookup_i64(int replica_id, const int64_t *key, size_t num_keys, 
   _coll_cache->lookup64(replica_id, key, num_keys, output, stream, step_key);
 }
 
+void coll_cache_lookup_pooled(int replica_id, const uint32_t *key, const int64_t *seg_off, const float *weights,
+                              size_t num_rows, size_t num_keys, int combiner, int elem_bytes, void *output,
+                              StreamHandle stream) {
+  CHECK_NOTNULL(_coll_cache);
+  const uint64_t step_key = steps[replica_id] * RunConfig::num_device + replica_id;
+  steps[replica_id]++;
+  _coll_cache->lookup_pooled(replica_id, key, seg_off, weights, num_rows, num_keys, combiner, elem_bytes, output, stream,
+                             step_key);
+}
+
+void coll_cache_lookup_pooled_i64(int replica_id, const int64_t *key, const int64_t *seg_off, const float *weights,
+                                  size_t num_rows, size_t num_keys, int combiner, int elem_bytes, void *output,
+                                  StreamHandle stream) {
+  CHECK_NOTNULL(_coll_cache);
+  const uint64_t step_key = steps[replica_id] * RunConfig::num_device + replica_id;
+  steps[replica_id]++;
+  _coll_cache->lookup_pooled64(replica_id, key, seg_off, weights, num_rows, num_keys, combiner, elem_bytes, output,
+                               stream, step_key);
+}
+
 size_t coll_cache_lookup_unique(int replica_id, const uint32_t *key, size_t num_keys, void *output,
                                 uint32_t *inverse_out, StreamHandle stream) {
   CHECK_NOTNULL(_coll_cache);
@@ -451,8 +471,9 @@ void ForwardJoin() {
   if (_forward.refresh_thread.joinable()) _forward.refresh_thread.join();
 }
 
-template <typename KeyT>
-void ForwardStep(int replica_id, const KeyT *key, size_t num_keys, void *output, StreamHandle stream) {
+// lookup(step_key): the extraction of the step — the plain lookup, or the pooled one
+template <typename KeyT, typename LookupFn>
+void ForwardStep(int replica_id, const KeyT *key, size_t num_keys, StreamHandle stream, const LookupFn &lookup) {
   CHECK_NOTNULL(_coll_cache);
   CHECK_EQ(replica_id, 0);
   ForwardState &fw = _forward;
@@ -465,10 +486,7 @@ void ForwardStep(int replica_id, const KeyT *key, size_t num_keys, void *output,
   }
   const uint64_t step_key = steps[replica_id] * RunConfig::num_device + replica_id;
   steps[replica_id]++;
-  if (sizeof(KeyT) == 8)
-    _coll_cache->lookup64(replica_id, reinterpret_cast<const Id64Type *>(key), num_keys, output, stream, step_key);
-  else
-    _coll_cache->lookup(replica_id, reinterpret_cast<const IdType *>(key), num_keys, output, stream, step_key);
+  lookup(step_key);
   if (RunConfig::gpu_record)
     session->SetRecordLimit(SIZE_MAX);
   else if (num_record > 0)
@@ -505,11 +523,33 @@ void coll_cache_forward_config(int enable_refresh, uint64_t refresh_iter, double
 }
 
 void coll_cache_forward(int replica_id, uint32_t *key, size_t num_keys, void *output, StreamHandle stream) {
-  ForwardStep<IdType>(replica_id, key, num_keys, output, stream);
+  ForwardStep<IdType>(replica_id, key, num_keys, stream, [&](uint64_t step_key) {
+    _coll_cache->lookup(replica_id, key, num_keys, output, stream, step_key);
+  });
 }
 
 void coll_cache_forward_i64(int replica_id, const int64_t *key, size_t num_keys, void *output, StreamHandle stream) {
-  ForwardStep<Id64Type>(replica_id, key, num_keys, output, stream);
+  ForwardStep<Id64Type>(replica_id, key, num_keys, stream, [&](uint64_t step_key) {
+    _coll_cache->lookup64(replica_id, key, num_keys, output, stream, step_key);
+  });
+}
+
+void coll_cache_forward_pooled(int replica_id, const uint32_t *key, const int64_t *seg_off, const float *weights,
+                               size_t num_rows, size_t num_keys, int combiner, int elem_bytes, void *output,
+                               StreamHandle stream) {
+  ForwardStep<IdType>(replica_id, key, num_keys, stream, [&](uint64_t step_key) {
+    _coll_cache->lookup_pooled(replica_id, key, seg_off, weights, num_rows, num_keys, combiner, elem_bytes, output,
+                               stream, step_key);
+  });
+}
+
+void coll_cache_forward_pooled_i64(int replica_id, const int64_t *key, const int64_t *seg_off, const float *weights,
+                                   size_t num_rows, size_t num_keys, int combiner, int elem_bytes, void *output,
+                                   StreamHandle stream) {
+  ForwardStep<Id64Type>(replica_id, key, num_keys, stream, [&](uint64_t step_key) {
+    _coll_cache->lookup_pooled64(replica_id, key, seg_off, weights, num_rows, num_keys, combiner, elem_bytes, output,
+                                 stream, step_key);
+  });
 }
 
 int coll_cache_forward_refresh_ongoing(void) { return _forward.refresh_ongoing.load() ? 1 : 0; }

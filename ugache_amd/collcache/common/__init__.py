@@ -130,6 +130,18 @@ C_API = {
                                                    ctypes.c_void_p, ctypes.c_void_p]),
     "coll_cache_lookup_unique_i64": (ctypes.c_size_t, [ctypes.c_int, ctypes.c_void_p, ctypes.c_size_t,
                                                        ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p]),
+    "coll_cache_lookup_pooled": (None, [ctypes.c_int, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p,
+                                        ctypes.c_size_t, ctypes.c_size_t, ctypes.c_int, ctypes.c_int, ctypes.c_void_p,
+                                        ctypes.c_void_p]),
+    "coll_cache_lookup_pooled_i64": (None, [ctypes.c_int, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p,
+                                            ctypes.c_size_t, ctypes.c_size_t, ctypes.c_int, ctypes.c_int,
+                                            ctypes.c_void_p, ctypes.c_void_p]),
+    "coll_cache_forward_pooled": (None, [ctypes.c_int, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p,
+                                         ctypes.c_size_t, ctypes.c_size_t, ctypes.c_int, ctypes.c_int, ctypes.c_void_p,
+                                         ctypes.c_void_p]),
+    "coll_cache_forward_pooled_i64": (None, [ctypes.c_int, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p,
+                                             ctypes.c_size_t, ctypes.c_size_t, ctypes.c_int, ctypes.c_int,
+                                             ctypes.c_void_p, ctypes.c_void_p]),
     "coll_cache_lookup_async": (None, [ctypes.c_int, ctypes.c_void_p, ctypes.c_size_t, ctypes.c_void_p,
                                        ctypes.c_void_p]),
     "coll_cache_lookup_async_i64": (None, [ctypes.c_int, ctypes.c_void_p, ctypes.c_size_t, ctypes.c_void_p,

@@ -167,6 +167,47 @@ def coll_torch_lookup_unique(local_id, keys):
     return out[: found[0]], inverse
 
 
+COMBINERS = {"sum": 0, "mean": 1, "sqrtn": 2}
+
+
+def pooled_lookup_supported():
+    """whether coll_torch_lookup_pooled can take the rows of the table that was built (a multiple of 16 bytes, at
+    most 4096; fp32 or fp16 elements)"""
+    elem = 2 if _State.external_dtype == torch.float16 else 4
+    row_bytes = _State.external_feat_dim * elem
+    return _State.external_dtype in (torch.float32, torch.float16) and row_bytes % 16 == 0 and 0 < row_bytes <= 4096
+
+
+def coll_torch_lookup_pooled(local_id, ids, seg_off, weights=None, combiner="sum", serving_step=False):
+    """lookup and per-sample combination of a multi-hot feature in one kernel (extension): segment r is
+    ids[seg_off[r] : seg_off[r + 1]]; returns a new [len(seg_off) - 1, dim] tensor whose row r is the weighted sum of
+    the segment's embeddings ("sum"), divided by the sum of the weights ("mean") or by the root of the sum of their
+    squares ("sqrtn") — embedding_lookup_sparse without the [len(ids), dim] intermediate.  ids: GPU int32 / int64;
+    seg_off: GPU int64, ascending, seg_off[0] == 0 and seg_off[-1] == len(ids); weights: GPU float32 or None.
+    serving_step: the call is one step of the serving loop (as coll_torch_forward is for a plain lookup)."""
+    dev = _State.dev_id.get(local_id, 0)
+    if not pooled_lookup_supported():
+        raise ValueError("pooled lookups need rows of a multiple of 16 bytes, at most 4096, of fp32 or fp16 elements")
+    if ids.dtype not in (torch.int32, torch.int64, torch.uint32) or not ids.is_cuda:
+        raise TypeError("ids must be a GPU tensor of int32 / uint32 or int64")
+    if seg_off.dtype != torch.int64 or not seg_off.is_cuda or seg_off.dim() != 1 or seg_off.numel() < 1:
+        raise TypeError("seg_off must be a one-dimensional GPU int64 tensor of num_rows + 1 offsets")
+    if weights is not None and (weights.dtype != torch.float32 or not weights.is_cuda or weights.numel() != ids.numel()):
+        raise TypeError("weights must be a GPU float32 tensor with one weight per id")
+    ids, seg_off = ids.contiguous().reshape(-1), seg_off.contiguous()
+    weights = None if weights is None else weights.contiguous().reshape(-1)
+    n_rows = seg_off.numel() - 1
+    out = torch.empty((n_rows, _State.external_feat_dim), dtype=_State.external_dtype, device="cuda:%d" % dev)
+    if serving_step:
+        fn = _C.coll_cache_forward_pooled_i64 if ids.dtype == torch.int64 else _C.coll_cache_forward_pooled
+    else:
+        fn = _C.coll_cache_lookup_pooled_i64 if ids.dtype == torch.int64 else _C.coll_cache_lookup_pooled
+    fn(local_id, ids.data_ptr() if ids.numel() else None, seg_off.data_ptr(),
+       None if weights is None else weights.data_ptr(), n_rows, ids.numel(), COMBINERS[combiner],
+       2 if _State.external_dtype == torch.float16 else 4, out.data_ptr(), _stream_handle(dev))
+    return out
+
+
 def coll_torch_lookup_async(local_id, keys, pad_to_8=True):
     """stream-ordered form of coll_torch_lookup_key_t_val_ret: the batch is enqueued on torch's current stream and
     the call returns without waiting, like any torch op; the returned view of the reused buffer is valid for work

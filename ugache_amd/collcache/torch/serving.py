@@ -25,6 +25,7 @@ import sys
 import torch
 
 from . import adapter as _adapter
+from . import c_lib as _c_lib
 from ..common import _basics
 
 # the share of every batch whose hotness the serving loop records (lookup_manager.cc:295-300: the first 5 %)
@@ -198,6 +199,9 @@ class SparseLookupLayer(torch.nn.Module):
         self.lookup = LookupLayer(model_name, table_id, emb_vec_size, emb_vec_dtype)
         self.emb_vec_size = emb_vec_size
         self.unique_in_library = bool(kwargs.get("unique_in_library", False))
+        # fused=True: lookup and combination in one kernel of the library (coll_torch_lookup_pooled) wherever that
+        # kernel can take the call (no max_norm, rows it supports); the steps below otherwise
+        self.fused = bool(kwargs.get("fused", False))
 
     def forward(self, sp_ids, sp_weights=None, name=None, combiner=None, max_norm=None):
         if combiner is None:
@@ -211,6 +215,14 @@ class SparseLookupLayer(torch.nn.Module):
         # entries as given (row-major order is the caller's contract); coalesce() would merge duplicate positions
         segment_ids = sp_ids._indices()[0]
         ids = sp_ids._values()
+        if self.fused and max_norm is None and _c_lib.pooled_lookup_supported():
+            self.lookup.check(ids)
+            num_rows = int(sp_ids.shape[0])
+            counts = torch.bincount(segment_ids, minlength=num_rows)
+            seg_off = torch.zeros(num_rows + 1, dtype=torch.int64, device=ids.device)
+            torch.cumsum(counts, 0, out=seg_off[1:])
+            weights = None if sp_weights is None else sp_weights._values().float()
+            return _adapter.coll_torch_lookup_pooled(0, ids, seg_off, weights, combiner, serving_step=True)
         if self.unique_in_library:  # unique + lookup in one call, the unique by the library's GPU hash set
             self.lookup.check(ids)
             emb_unique, idx = _adapter.coll_torch_lookup_unique(0, ids)
