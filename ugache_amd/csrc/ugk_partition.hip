@@ -815,9 +815,18 @@ __global__ __launch_bounds__(kBlock) void extract_pool_kernel(ugk_table_t t, con
 template <typename K, int KIND, typename E>
 int extract_pool_lpr(ugk_table_t t, const K *ids, const long long *seg_off, const float *weights, size_t n_rows,
                      const void *cache, uint64_t cache_rows, const void *host, uint64_t host_rows, void *out,
-                     uint32_t vpr, int combiner, uint32_t *status, uint32_t *host_mirror, uint64_t *counts,
-                     uint32_t *num_groups, hipStream_t st) {
-  const int lpr = vpr <= 8 ? 8 : vpr <= 32 * kPoolChunks ? 32 : 64;
+                     uint32_t vpr, uint64_t nnz, int combiner, uint32_t *status, uint32_t *host_mirror,
+                     uint64_t *counts, uint32_t *num_groups, hipStream_t st) {
+  // Lanes per output row.  A lane group walks its row's ids a few at a time, so what keeps memory busy is the number
+  // of rows a wavefront works on at once: rows of up to 512 bytes go to 8 lanes of up to four chunks each (eight rows
+  // per wavefront; with 32 lanes and two rows per wavefront 262,144 samples of one id took 138 us instead of 83 us, and
+  // 65,536 samples of 16 ids 123 us instead of 112 us), rows of up to 2 KB to 32 lanes, longer ones to 64.
+  (void)nnz;
+  int lpr = vpr <= 8 * kPoolChunks ? 8 : vpr <= 32 * kPoolChunks ? 32 : 64;
+  if (const char *forced = getenv("UGK_POOL_LPR")) {  // for sweeps; never a byte of the result depends on it
+    const int v = atoi(forced);
+    if ((v == 8 || v == 32 || v == 64) && vpr <= (uint32_t)v * kPoolChunks) lpr = v;
+  }
   const size_t rows_per_group = (size_t)(kWave / lpr) * kWavesPerBlock;
   const unsigned grid = clamp_grid((n_rows + rows_per_group - 1) / rows_per_group, 0);
   if (num_groups) *num_groups = grid;
@@ -862,10 +871,11 @@ int extract_pool(ugk_table_t t, const K *ids, const int64_t *seg_off, const floa
   hipStream_t st = as_stream(stream);
 #define UGK_POOL_KIND(KIND)                                                                                          \
   (elem_bytes == 4 ? extract_pool_lpr<K, KIND, float>(t, ids, so, weights, n_rows, cache, cache_rows, host, host_rows, \
-                                                      out, vpr, combiner, status, host_mirror, counts, num_groups, st) \
+                                                      out, vpr, nnz, combiner, status, host_mirror, counts,           \
+                                                      num_groups, st)                                                 \
                    : extract_pool_lpr<K, KIND, __half>(t, ids, so, weights, n_rows, cache, cache_rows, host,          \
-                                                       host_rows, out, vpr, combiner, status, host_mirror, counts,    \
-                                                       num_groups, st))
+                                                       host_rows, out, vpr, nnz, combiner, status, host_mirror,       \
+                                                       counts, num_groups, st))
   if (t.kind == 0) return UGK_POOL_KIND(0);
   if (t.kind == 1) return UGK_POOL_KIND(1);
   return UGK_POOL_KIND(2);

@@ -13,6 +13,9 @@ flagged an error (the parity tests check results).
   small_batch  serving-sized batches (1,024 - 131,072 keys that all hit) through the library: microseconds per blocking
             coll_cache_lookup_i64 and per stream-ordered coll_cache_lookup_async_i64, without a table (the whole table
             cached) and through the table of a half-cached key space (host clock around 2,000 calls)
+  pooled    a multi-hot feature through the library: lookup + weighted combination per sample in one call
+            (coll_torch_lookup_pooled) against the lookup of all ids followed by torch's index_add_ segment sum, and
+            against unique -> lookup -> index_select -> index_add_ (the reference's sparse layer), by ids per sample
 """
 import ctypes as C
 import json
@@ -273,7 +276,70 @@ def probe_small_batch(hip, torch, note, quick=False):
                    "batches of uniformly random keys that all hit, host clock around the calls", "rows": out_rows}
 
 
-PROBES = {"kpw": probe_kpw, "row_span": probe_row_span, "cu_mask": probe_cu_mask, "small_batch": probe_small_batch}
+def probe_pooled(hip, torch, note, quick=False):
+    import collcache.torch as co
+
+    rows, dim, calls = 10_000_000, 128, (20 if quick else 50)
+    out_rows = []
+    for pct, label in ((1.0, "whole table cached"), (0.5, "half of the rows cached, every id a hit")):
+        co.config({"cache_percentage": pct, "_cache_policy": co.kCollCacheAsymmLink, "num_device": 1,
+                   "num_global_step_per_epoch": 10, "num_epoch": 1, "num_total_item": rows, "omp_thread_num": 8})
+        co.coll_cache_record_init(0)
+        co.coll_torch_record(0, torch.arange(0, rows // 2, dtype=torch.int32))
+        emb = co.coll_torch_create_emb_shm(0, rows, dim, torch.float32)
+        emb.normal_(generator=torch.Generator().manual_seed(1))
+        co.coll_torch_init_t(0, 0, emb, pct)
+        for per_sample, zipf in ((1, 0.0), (4, 0.0), (16, 0.0), (16, 1.05)) if not quick else ((8, 0.0),):
+            n_samples = 262_144 if per_sample <= 4 else 65_536
+            nnz = n_samples * per_sample
+            if zipf:  # duplicates among the ids, as a skewed multi-hot feature has them
+                u = torch.rand(nnz, device="cuda", dtype=torch.float64)
+                h = float(rows // 2)
+                ids = (((h ** (1 - zipf) - 1) * u + 1) ** (1 / (1 - zipf))).long().clamp_(1, rows // 2) - 1
+            else:
+                ids = torch.randint(0, rows // 2, (nnz,), device="cuda", dtype=torch.int64)
+            seg_off = torch.arange(0, nnz + 1, per_sample, device="cuda", dtype=torch.int64)
+            seg = torch.arange(n_samples, device="cuda").repeat_interleave(per_sample)
+            w = torch.rand(nnz, device="cuda", dtype=torch.float32) + 0.5
+
+            def fused():
+                return co.coll_torch_lookup_pooled(0, ids, seg_off, w, "sum")
+
+            def lookup_then_sum():
+                e = co.coll_torch_lookup_key_t_val_ret(0, ids, False)
+                out = torch.zeros((n_samples, dim), dtype=torch.float32, device="cuda")
+                return out.index_add_(0, seg, e * w.unsqueeze(1))
+
+            def unique_lookup_sum():
+                uq, inv = torch.unique(ids, return_inverse=True)
+                e = co.coll_torch_lookup_key_t_val_ret(0, uq, False).index_select(0, inv)
+                out = torch.zeros((n_samples, dim), dtype=torch.float32, device="cuda")
+                return out.index_add_(0, seg, e * w.unsqueeze(1))
+
+            ref = lookup_then_sum()
+            assert torch.allclose(fused(), ref, rtol=1e-4, atol=1e-4) and torch.allclose(unique_lookup_sum(), ref, rtol=1e-4, atol=1e-4)
+            res = {}
+            for name, fn in (("fused", fused), ("lookup_then_sum", lookup_then_sum), ("unique_lookup_sum", unique_lookup_sum)):
+                for _ in range(3):
+                    fn()
+                torch.cuda.synchronize()
+                t0 = time.perf_counter()
+                for _ in range(calls):
+                    fn()
+                torch.cuda.synchronize()
+                res[name] = round((time.perf_counter() - t0) / calls * 1e6, 1)
+            moved = nnz * dim * 4 + n_samples * dim * 4 + nnz * 12
+            out_rows.append({"cache": label, "samples": n_samples, "ids_per_sample": per_sample, "zipf": zipf,
+                             "us_per_call": res, "fused_GBps_of_rows_read_and_written": round(moved / res["fused"] / 1e3, 1)})
+            note("pooled %s, %d x %d ids (zipf %.2f): %s" % (label, n_samples, per_sample, zipf, res))
+            del ids, seg, w, ref
+        co.coll_torch_shutdown()
+    return {"probe": "pooled", "table_rows": rows, "row_bytes": dim * 4, "calls_timed": calls,
+            "how": "weighted sum per sample of fp32 rows; host clock around the calls, one synchronisation at the end; "
+                   "the unfused forms use the library's plain lookup and torch ops", "rows": out_rows}
+
+
+PROBES = {"pooled": probe_pooled, "kpw": probe_kpw, "row_span": probe_row_span, "cu_mask": probe_cu_mask, "small_batch": probe_small_batch}
 
 
 def run(name, quick=False):
