@@ -11,6 +11,7 @@
 #include <algorithm>
 #include <atomic>
 #include <cstdint>
+#include <cmath>
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
@@ -132,6 +133,33 @@ int main(int argc, char **argv) {
       auto k = skewed_keys(g, 3000, 9000 + (uint64_t)step * 53);
       coll_cache_forward(0, k.data(), k.size(), out.data(), nullptr);
       bad_rows += check_rows(table, out.data(), k.data(), k.size());
+    }
+    // 5. pooled lookups (segments of ids combined per sample), plain and as steps of the serving loop
+    for (int step = 0; step < 6; ++step) {
+      auto k = skewed_keys(g, 2000, 20000 + (uint64_t)step * 31);
+      std::vector<int64_t> off(1, 0);
+      while ((size_t)off.back() < k.size()) off.push_back(std::min<int64_t>((int64_t)k.size(), off.back() + (int64_t)(g() % 6)));
+      std::vector<float> w(k.size());
+      for (auto &x : w) x = 0.5f + (float)(g() % 100) / 100.f;
+      const size_t n_rows = off.size() - 1;
+      const int combiner = step % 3;
+      if (step < 3)
+        coll_cache_lookup_pooled(0, k.data(), off.data(), step == 1 ? nullptr : w.data(), n_rows, k.size(), combiner, 4,
+                                 out.data(), nullptr);
+      else
+        coll_cache_forward_pooled(0, k.data(), off.data(), w.data(), n_rows, k.size(), combiner, 4, out.data(), nullptr);
+      for (size_t r = 0; r < n_rows; ++r)
+        for (size_t c = 0; c < kDim; ++c) {
+          double sum = 0, den = 0;
+          for (int64_t j = off[r]; j < off[r + 1]; ++j) {
+            const double wj = step == 1 ? 1.0 : w[j];
+            sum += wj * table[(size_t)k[j] * kDim + c];
+            den += combiner == 2 ? wj * wj : wj;
+          }
+          if (combiner == 2) den = std::sqrt(den);
+          const double want = combiner == 0 ? sum : den != 0 ? sum / den : 0.0;
+          if (std::fabs(out[r * kDim + c] - want) > 1e-4 * (1.0 + std::fabs(want))) ++bad_rows;
+        }
     }
     const uint64_t done = coll_cache_forward_join();
     uint64_t info[8];
