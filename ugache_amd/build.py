@@ -20,11 +20,12 @@ INCLUDE = os.path.join(ROOT, "include")
 HIP_LIB = os.path.join(PKG, "libugache_hip.so")
 HOST_LIB = os.path.join(PKG, "libcoll_cache.so")
 
-HIP_SOURCES = ["ugk_runtime.hip", "ugk_gather.hip", "ugk_table.hip", "ugk_partition.hip", "ugk_hotness.hip",
-               "ugk_refresh.hip"]
+HIP_SOURCES = ["ugk_runtime.hip", "ugk_gather.hip", "ugk_table.hip", "ugk_partition.hip", "ugk_pool.hip",
+               "ugk_hotness.hip", "ugk_refresh.hip"]
+OBJ_DIR = os.path.join(PKG, "_build")
 
 HIPCC_FLAGS = [
-    "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-shared",
+    "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC",
     # packed FP32 instructions are kept out of every code object of this library
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
     "-Wall", "-Wno-unused-function",
@@ -46,11 +47,23 @@ def hipcc_path():
     raise RuntimeError("hipcc not found")
 
 
+def _compile_all(jobs):
+    """jobs: (command, object file) pairs, run side by side (the long ones first); -> the object files"""
+    from concurrent.futures import ThreadPoolExecutor
+    os.makedirs(OBJ_DIR, exist_ok=True)
+    with ThreadPoolExecutor(max_workers=min(8, max(len(jobs), 1))) as pool:
+        outs = list(pool.map(lambda j: _run(j[0]), jobs))
+    return [j[1] for j in jobs], "\n".join(o for o in outs if o.strip())
+
+
 def build_hip(verbose=False):
-    cmd = [hipcc_path()] + HIPCC_FLAGS + ["-I", INCLUDE, "-I", CSRC]
-    cmd += [os.path.join(CSRC, s) for s in HIP_SOURCES]
-    cmd += ["-o", HIP_LIB]
-    out = _run(cmd)
+    base = [hipcc_path()] + HIPCC_FLAGS + ["-I", INCLUDE, "-I", CSRC]
+    jobs = []
+    for s in HIP_SOURCES:
+        obj = os.path.join(OBJ_DIR, s + ".o")
+        jobs.append((base + ["-c", os.path.join(CSRC, s), "-o", obj], obj))
+    objs, out = _compile_all(jobs)
+    out += _run([hipcc_path(), "--offload-arch=gfx950", "-shared", "-fPIC"] + objs + ["-o", HIP_LIB])
     if verbose and out.strip():
         print(out)
     return HIP_LIB
@@ -66,11 +79,15 @@ def build_host(verbose=False):
     srcs = host_sources()
     if not srcs:
         return None
-    cmd = ["g++", "-O2", "-g", "-std=c++17", "-fPIC", "-shared", "-fopenmp", "-pthread", "-Wall", "-Wextra",
-           "-Wno-unused-parameter", "-I", INCLUDE, "-I", PKG]
-    cmd += srcs
-    cmd += ["-o", HOST_LIB, "-L", PKG, "-lugache_hip", "-Wl,-rpath,$ORIGIN", "-Wl,--no-undefined"]
-    out = _run(cmd)
+    base = ["g++", "-O2", "-g", "-std=c++17", "-fPIC", "-fopenmp", "-pthread", "-Wall", "-Wextra",
+            "-Wno-unused-parameter", "-I", INCLUDE, "-I", PKG]
+    jobs = []
+    for s in srcs:
+        obj = os.path.join(OBJ_DIR, os.path.basename(s) + ".o")
+        jobs.append((base + ["-c", s, "-o", obj], obj))
+    objs, out = _compile_all(jobs)
+    out += _run(["g++", "-shared", "-fopenmp", "-pthread"] + objs +
+                ["-o", HOST_LIB, "-L", PKG, "-lugache_hip", "-Wl,-rpath,$ORIGIN", "-Wl,--no-undefined"])
     if verbose and out.strip():
         print(out)
     return HOST_LIB

@@ -1,0 +1,249 @@
+// Pooled extraction: the lookup of a multi-hot feature and its per-sample combination in one kernel
+// (ugk_extract_pool_*).
+#include <hip/hip_fp16.h>
+
+#include <cstdlib>
+
+#include "ugk_internal.h"
+#include "ugk_mix.cuh"
+#include "ugk_table.cuh"
+
+namespace ugk {
+namespace {
+
+// ---- pooled extraction -------------------------------------------------------------------------------------
+// out[r, :] = combine_j( w_j * row(ids[j]) ) over the ids j of segment r = [seg_off[r], seg_off[r + 1]): the lookup of
+// a multi-hot feature and the per-sample combination that follows it (embedding_lookup_sparse behind
+// python_tf2/collcache_tf2/collcache_tf2/core/sparse_lookup_layer.py:196-265) in one pass, so that the nnz x row_bytes
+// intermediate of a lookup followed by a segment sum is never written or read back.  A group of LPR lanes owns an
+// output row: its lanes resolve LPR of the row's ids at a time (the table lookup is the fused extraction's), then
+// every id's row is read once, 16 bytes per lane and chunk, and added in fp32 in the order of the ids.
+template <typename E>
+struct PoolElem;
+template <>
+struct PoolElem<float> {
+  static constexpr int kPerChunk = 4;
+  static __device__ __forceinline__ void unpack(const u32x4 &v, float *x) {
+    x[0] = __uint_as_float(v.x), x[1] = __uint_as_float(v.y), x[2] = __uint_as_float(v.z), x[3] = __uint_as_float(v.w);
+  }
+  static __device__ __forceinline__ u32x4 pack(const float *x) {
+    return u32x4{__float_as_uint(x[0]), __float_as_uint(x[1]), __float_as_uint(x[2]), __float_as_uint(x[3])};
+  }
+};
+template <>
+struct PoolElem<__half> {
+  static constexpr int kPerChunk = 8;
+  static __device__ __forceinline__ void unpack(const u32x4 &v, float *x) {
+    const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      x[2 * k] = __half2float(__ushort_as_half((unsigned short)(w[k] & 0xffffu)));
+      x[2 * k + 1] = __half2float(__ushort_as_half((unsigned short)(w[k] >> 16)));
+    }
+  }
+  static __device__ __forceinline__ u32x4 pack(const float *x) {
+    uint32_t w[4];
+#pragma unroll
+    for (int k = 0; k < 4; ++k)
+      w[k] = (uint32_t)__half_as_ushort(__float2half(x[2 * k])) |
+             ((uint32_t)__half_as_ushort(__float2half(x[2 * k + 1])) << 16);
+    return u32x4{w[0], w[1], w[2], w[3]};
+  }
+};
+
+constexpr int kPoolChunks = 4;  // 16-byte chunks of a row a lane may own: rows of up to LPR x 64 bytes
+
+template <typename K, int KIND, int LPR, typename E>
+__global__ __launch_bounds__(kBlock) void extract_pool_kernel(ugk_table_t t, const K *__restrict__ ids,
+                                                              const long long *__restrict__ seg_off,
+                                                              const float *__restrict__ weights, size_t n_rows,
+                                                              const u32x4 *__restrict__ cache, uint64_t cache_rows,
+                                                              const u32x4 *__restrict__ host, uint64_t host_rows,
+                                                              u32x4 *__restrict__ out, uint32_t vpr, int combiner,
+                                                              uint32_t *status, uint32_t *host_mirror,
+                                                              unsigned long long *counts) {
+  constexpr int RPW = kWave / LPR;  // output rows per wavefront and pass
+  constexpr int EPC = PoolElem<E>::kPerChunk;
+  constexpr int U = 4;  // rows in flight per lane group
+  static_assert(LPR % U == 0, "ids are taken in rounds of U");
+  __shared__ uint32_t block_tot[2];
+  if (threadIdx.x < 2) block_tot[threadIdx.x] = 0;
+  __syncthreads();
+  uint32_t wave_local = 0, wave_host = 0;
+  const int lane = (int)lane_id();
+  const int sub = lane % LPR, rg = lane / LPR;
+  const size_t wave_global = (size_t)blockIdx.x * kWavesPerBlock + threadIdx.x / kWave;
+  const size_t n_waves = (size_t)gridDim.x * kWavesPerBlock;
+  for (size_t row0 = wave_global * RPW; row0 < n_rows; row0 += n_waves * RPW) {  // wavefront-uniform
+    const size_t r = row0 + rg;
+    const bool row_ok = r < n_rows;
+    const long long beg = row_ok ? seg_off[r] : 0, end = row_ok ? seg_off[r + 1] : 0;
+    float acc[kPoolChunks][EPC];
+#pragma unroll
+    for (int c = 0; c < kPoolChunks; ++c)
+#pragma unroll
+      for (int e = 0; e < EPC; ++e) acc[c][e] = 0.f;
+    float wsum = 0.f;  // this lane's share of the row's sum of weights (or of their squares)
+    for (long long j0 = beg; __ballot(j0 < end) != 0ull; j0 += LPR) {  // until every group of the wavefront is through
+      const long long j = j0 + sub;
+      const bool active = j < end;
+      const uint64_t key = active ? key_to_u64<K>(ids[j]) : 0;
+      const Found f = table_lookup<KIND>(t, key, active);
+      const MixRow row = mix_resolve(t, key, active, f, cache, cache_rows, host, host_rows, out, vpr, status, host_mirror);
+      if (counts) {
+        wave_local += __popcll(__ballot(row.from_cache));
+        wave_host += __popcll(__ballot(active && !row.from_cache));
+      }
+      const bool use = active && row.has_row;  // a key without a row adds nothing (the launch is flagged)
+      const float w = use ? (weights ? weights[j] : 1.f) : 0.f;
+      wsum += combiner == 2 ? w * w : w;
+      for (int s0 = 0; s0 < LPR; s0 += U) {
+        if (__ballot(active && sub >= s0) == 0ull) break;  // no group has an id left in this round
+        grow_t p[U];
+        float wv[U];
+        bool ok[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+          const int src = rg * LPR + s0 + u;
+          p[u] = reinterpret_cast<grow_t>(shfl64(row.bits, src));
+          wv[u] = __shfl(w, src);
+          ok[u] = __shfl((int)use, src) != 0;
+        }
+#pragma unroll
+        for (int c = 0; c < kPoolChunks; ++c) {
+          const uint32_t col = (uint32_t)c * LPR + sub;
+          if (col < vpr) {
+            u32x4 v[U];
+#pragma unroll
+            for (int u = 0; u < U; ++u) v[u] = __builtin_nontemporal_load(p[u] + col);
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+              float x[EPC];
+              PoolElem<E>::unpack(v[u], x);
+              if (ok[u]) {
+#pragma unroll
+                for (int e = 0; e < EPC; ++e) acc[c][e] = fmaf(wv[u], x[e], acc[c][e]);
+              }
+            }
+          }
+        }
+      }
+    }
+    // the row's denominator: every lane of the group holds a share
+#pragma unroll
+    for (int d = LPR / 2; d > 0; d >>= 1) wsum += __shfl_xor(wsum, d);
+    const float denom = combiner == 1 ? wsum : combiner == 2 ? sqrtf(wsum) : 1.f;
+    if (row_ok) {
+#pragma unroll
+      for (int c = 0; c < kPoolChunks; ++c) {
+        const uint32_t col = (uint32_t)c * LPR + sub;
+        if (col < vpr) {
+          float y[EPC];
+#pragma unroll
+          for (int e = 0; e < EPC; ++e) y[e] = denom != 0.f ? acc[c][e] / denom : 0.f;  // div_no_nan
+          out[r * vpr + col] = PoolElem<E>::pack(y);
+        }
+      }
+    }
+  }
+  if (counts) mix_leave_counts(block_tot, wave_local, wave_host, counts);
+}
+
+template <typename K, int KIND, typename E>
+int extract_pool_lpr(ugk_table_t t, const K *ids, const long long *seg_off, const float *weights, size_t n_rows,
+                     const void *cache, uint64_t cache_rows, const void *host, uint64_t host_rows, void *out,
+                     uint32_t vpr, uint64_t nnz, int combiner, uint32_t *status, uint32_t *host_mirror,
+                     uint64_t *counts, uint32_t *num_groups, hipStream_t st) {
+  // Lanes per output row.  A lane group walks its row's ids a few at a time, so what keeps memory busy is the number
+  // of rows a wavefront works on at once: rows of up to 512 bytes go to 8 lanes of up to four chunks each (eight rows
+  // per wavefront; with 32 lanes and two rows per wavefront 262,144 samples of one id took 138 us instead of 83 us, and
+  // 65,536 samples of 16 ids 123 us instead of 112 us), rows of up to 2 KB to 32 lanes, longer ones to 64.
+  (void)nnz;
+  int lpr = vpr <= 8 * kPoolChunks ? 8 : vpr <= 32 * kPoolChunks ? 32 : 64;
+  if (const char *forced = getenv("UGK_POOL_LPR")) {  // for sweeps; never a byte of the result depends on it
+    const int v = atoi(forced);
+    if ((v == 8 || v == 32 || v == 64) && vpr <= (uint32_t)v * kPoolChunks) lpr = v;
+  }
+  const size_t rows_per_group = (size_t)(kWave / lpr) * kWavesPerBlock;
+  const unsigned grid = clamp_grid((n_rows + rows_per_group - 1) / rows_per_group, 0);
+  if (num_groups) *num_groups = grid;
+#define UGK_POOL(L)                                                                                                 \
+  hipLaunchKernelGGL((extract_pool_kernel<K, KIND, L, E>), dim3(grid), dim3(kBlock), 0, st, t, ids, seg_off, weights, \
+                     n_rows, (const u32x4 *)cache, cache_rows, (const u32x4 *)host, host_rows, (u32x4 *)out, vpr,   \
+                     combiner, status, host_mirror, reinterpret_cast<unsigned long long *>(counts))
+  if (lpr == 8) UGK_POOL(8);
+  else if (lpr == 32) UGK_POOL(32);
+  else UGK_POOL(64);
+#undef UGK_POOL
+  UGK_HIP(hipGetLastError());
+  return 0;
+}
+
+template <typename K>
+int extract_pool(ugk_table_t t, const K *ids, const int64_t *seg_off, const float *weights, size_t n_rows, uint64_t nnz,
+                 int combiner, int elem_bytes, const void *cache, uint64_t cache_rows, const void *host,
+                 uint64_t host_rows, void *out, size_t row_bytes, uint32_t *status, uint32_t *host_mirror,
+                 uint64_t *counts, uint32_t *num_groups, void *stream) {
+  if (num_groups) *num_groups = 0;
+  if (n_rows == 0) return 0;
+  UGK_REQUIRE(seg_off && out && status, "ugk_extract_pool: null offsets, output or status");
+  UGK_REQUIRE(nnz == 0 || ids, "ugk_extract_pool: null ids");
+  UGK_REQUIRE((uintptr_t)counts % 8 == 0, "ugk_extract_pool: the count words must be 8-byte aligned");
+  UGK_REQUIRE(combiner >= 0 && combiner <= 2, "ugk_extract_pool: combiner %d is not sum(0), mean(1) or sqrtn(2)", combiner);
+  UGK_REQUIRE(elem_bytes == 4 || elem_bytes == 2, "ugk_extract_pool: elements of %d bytes are not fp32 or fp16", elem_bytes);
+  UGK_REQUIRE(t.kind == 0 || t.kind == 1 || t.kind == 2, "ugk_extract_pool: table kind %d", t.kind);
+  if (t.kind != 0) UGK_REQUIRE(t.table && t.size, "ugk_extract_pool: empty table");
+  if (t.kind == 2)
+    UGK_REQUIRE(t.size % 8 == 0 && (uintptr_t)t.table % 128 == 0,
+                "ugk_extract_pool: hash table must be 128-byte aligned with a multiple of 8 buckets");
+  UGK_REQUIRE(cache_rows == 0 || cache, "ugk_extract_pool: null cache with %llu rows", (unsigned long long)cache_rows);
+  UGK_REQUIRE(host_rows == 0 || host, "ugk_extract_pool: null host table with %llu rows", (unsigned long long)host_rows);
+  const uintptr_t align = (uintptr_t)cache | (uintptr_t)host | (uintptr_t)out | (uintptr_t)row_bytes;
+  UGK_REQUIRE(row_bytes > 0 && align % 16 == 0,
+              "ugk_extract_pool: rows and buffers must be multiples of 16 bytes (row_bytes=%zu)", row_bytes);
+  const uint32_t vpr = (uint32_t)(row_bytes / 16);
+  UGK_REQUIRE(vpr <= (uint32_t)kWave * kPoolChunks, "ugk_extract_pool: rows of %zu bytes exceed %d", row_bytes,
+              kWave * kPoolChunks * 16);
+  const long long *so = reinterpret_cast<const long long *>(seg_off);
+  hipStream_t st = as_stream(stream);
+#define UGK_POOL_KIND(KIND)                                                                                          \
+  (elem_bytes == 4 ? extract_pool_lpr<K, KIND, float>(t, ids, so, weights, n_rows, cache, cache_rows, host, host_rows, \
+                                                      out, vpr, nnz, combiner, status, host_mirror, counts,           \
+                                                      num_groups, st)                                                 \
+                   : extract_pool_lpr<K, KIND, __half>(t, ids, so, weights, n_rows, cache, cache_rows, host,          \
+                                                       host_rows, out, vpr, nnz, combiner, status, host_mirror,       \
+                                                       counts, num_groups, st))
+  if (t.kind == 0) return UGK_POOL_KIND(0);
+  if (t.kind == 1) return UGK_POOL_KIND(1);
+  return UGK_POOL_KIND(2);
+#undef UGK_POOL_KIND
+}
+
+}  // namespace
+}  // namespace ugk
+
+using namespace ugk;
+
+extern "C" {
+
+int ugk_extract_pool_u32(ugk_table_t t, const uint32_t *ids_dev, const int64_t *seg_off_dev, const float *weights_dev,
+                         size_t n_rows, uint64_t nnz, int combiner, int elem_bytes, const void *cache_dev,
+                         uint64_t cache_rows, const void *host_dev, uint64_t host_rows, void *out_dev, size_t row_bytes,
+                         uint32_t *status_dev, uint32_t *host_mirror, uint64_t *group_counts_host,
+                         uint32_t *num_groups_host, void *stream) {
+  return extract_pool<uint32_t>(t, ids_dev, seg_off_dev, weights_dev, n_rows, nnz, combiner, elem_bytes, cache_dev,
+                                cache_rows, host_dev, host_rows, out_dev, row_bytes, status_dev, host_mirror,
+                                group_counts_host, num_groups_host, stream);
+}
+
+int ugk_extract_pool_i64(ugk_table_t t, const int64_t *ids_dev, const int64_t *seg_off_dev, const float *weights_dev,
+                         size_t n_rows, uint64_t nnz, int combiner, int elem_bytes, const void *cache_dev,
+                         uint64_t cache_rows, const void *host_dev, uint64_t host_rows, void *out_dev, size_t row_bytes,
+                         uint32_t *status_dev, uint32_t *host_mirror, uint64_t *group_counts_host,
+                         uint32_t *num_groups_host, void *stream) {
+  return extract_pool<int64_t>(t, ids_dev, seg_off_dev, weights_dev, n_rows, nnz, combiner, elem_bytes, cache_dev,
+                               cache_rows, host_dev, host_rows, out_dev, row_bytes, status_dev, host_mirror,
+                               group_counts_host, num_groups_host, stream);
+}
+
+}  // extern "C"
