@@ -32,6 +32,7 @@ extern "C" {
 #define UGK_ST_TABLE_FULL 0x2u       /* hash insert found no free bucket */
 #define UGK_ST_DUP_KEY 0x4u          /* insert of a key that is already present (the reference asserts) */
 #define UGK_ST_EVICT_ABSENT 0x8u     /* evict of a key that is not present */
+#define UGK_ST_BAD_SEGMENT 0x10u     /* pooled extraction: offsets that leave [0, nnz] or run backwards: row of zeros */
 
 /* ---- locations (cache_context.cu:2421-2422: GPUs are 0..G-1, the host is G; here G = 1) ---------- */
 #define UGK_LOC_LOCAL 0u
@@ -279,7 +280,8 @@ int ugk_extract_mix_i64(ugk_table_t t, const int64_t *keys_dev, size_t n, const 
  * followed by a segment sum is never written.  seg_off_dev: n_rows + 1 ascending offsets into ids_dev, the last one
  * nnz.  row_bytes: a multiple of 16, at most 4096.  Status, host mirror and the per-workgroup count words are those of
  * ugk_extract_mix_* (the counts are of ids, not of output rows).  An id without a row sets UGK_ST_KEY_OUT_OF_RANGE and
- * adds nothing. */
+ * adds nothing; a segment whose offsets leave [0, nnz] or run backwards sets UGK_ST_BAD_SEGMENT, reads no id and
+ * gives a zero row. */
 int ugk_extract_pool_u32(ugk_table_t t, const uint32_t *ids_dev, const int64_t *seg_off_dev, const float *weights_dev,
                          size_t n_rows, uint64_t nnz, int combiner, int elem_bytes, const void *cache_dev,
                          uint64_t cache_rows, const void *host_dev, uint64_t host_rows, void *out_dev, size_t row_bytes,

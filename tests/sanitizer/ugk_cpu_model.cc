@@ -404,7 +404,12 @@ int extract_pool(ugk_table_t t, const K *ids, const int64_t *seg_off, const floa
   for (size_t r = 0; r < n_rows; ++r) {
     std::fill(acc.begin(), acc.end(), 0.f);
     float wsum = 0.f;
-    for (int64_t j = seg_off[r]; j < seg_off[r + 1]; ++j) {
+    int64_t beg = seg_off[r], end = seg_off[r + 1];
+    if (beg < 0 || end > (int64_t)nnz || end < beg) {
+      or_status(status, UGK_ST_BAD_SEGMENT, mirror);
+      beg = end = 0;
+    }
+    for (int64_t j = beg; j < end; ++j) {
       const uint64_t key = k64(ids[j]);
       const Found f = t.kind ? lookup(t, key) : Found{false, 0, 0};
       const char *row = nullptr;

@@ -127,3 +127,24 @@ def test_a_process_that_never_calls_shutdown_still_exits_cleanly(gpu_record):
     """, env={"COLL_GPU_RECORD": gpu_record, "COLL_REFRESH_SLEEP_US": "20000"})
     assert "forwards ok" in p.stdout, p.stderr[-2000:]
     assert p.returncode == 0, p.stderr[-2000:]
+
+
+def test_pooled_lookup_with_offsets_beyond_the_ids_aborts_with_a_message():
+    p = run("""
+        n = 5000
+        co.config(cfg(n, 0.3)); co.coll_cache_record_init(0)
+        co.coll_torch_record(0, torch.arange(0, n, 3, dtype=torch.int32))
+        emb = co.coll_torch_create_emb_shm(0, n, 32, torch.float32); emb.normal_()
+        co.coll_torch_init_t(0, 0, emb, 0.3)
+        ids = torch.arange(40, dtype=torch.int64, device="cuda")
+        off = torch.arange(0, 41, 4, dtype=torch.int64, device="cuda")
+        good = co.coll_torch_lookup_pooled(0, ids, off)
+        assert torch.allclose(good.cpu(), emb[:40].reshape(10, 4, 32).sum(1), atol=1e-5)
+        print("good lookup ok", flush=True)
+        off[-1] = 4000
+        co.coll_torch_lookup_pooled(0, ids, off)
+        print("survived")
+    """)
+    assert "good lookup ok" in p.stdout and "survived" not in p.stdout, p.stderr[-2000:]
+    assert p.returncode == -6, p.stderr[-2000:]
+    assert "offsets of a pooled lookup" in p.stderr

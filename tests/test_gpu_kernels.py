@@ -719,6 +719,23 @@ def test_pooled_extraction_hand_worked():
         sync()
         assert status_value(st) & hip.ST_KEY_OUT_OF_RANGE
         assert to_np(out)[:64].view(np.float32).reshape(4, 4)[0, :2].tolist() == [1, 10]
+        # offsets that leave the ids (beyond nnz, negative, running backwards) flag the launch, read nothing and
+        # give rows of zeros; the other rows are unharmed
+        key = np.array([1, 2, 3, 4, 4])
+        for broken in ([0, 2, 3, 3, 9], [0, 2, 3, 3, 1 << 40], [0, 2, -7, 3, 5], [0, 4, 3, 3, 5]):
+            st.zero_()
+            boff = to_dev(np.array(broken, np.int64))
+            out = dev_bytes(4 * 16, fill=0x55)
+            hip.call("ugk_extract_pool_i64", hip.table(0, None, 0), ptr(ids), ptr(boff), None, 4, 5, 0, 4, ptr(cache), 0,
+                     pin.ptr, 6, ptr(out), 16, ptr(st), None, None, None, None)
+            sync()
+            assert status_value(st) == hip.ST_BAD_SEGMENT, broken
+            want = []
+            for r in range(4):
+                b, e = broken[r], broken[r + 1]
+                s = float(key[b:e].sum()) if 0 <= b <= e <= 5 else 0.0
+                want.append([s, 10 * s])
+            assert to_np(out)[:64].view(np.float32).reshape(4, 4)[:, :2].tolist() == want, broken
     finally:
         sync()
         pin.free()

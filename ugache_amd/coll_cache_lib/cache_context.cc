@@ -320,9 +320,14 @@ void ExtractSession::CheckStatusWord(StreamHandle stream) const {
   uint32_t st = 0;
   UGK_CALL(ugk_memcpy_async(&st, _status, sizeof(st), stream));
   UGK_CALL(ugk_stream_sync(stream));
-  CHECK_EQ(st, 0u) << "extraction kernels reported status 0x" << std::hex << st
-                   << ": a key is outside the table it has to be read from (num_total_item="
-                   << std::dec << _cache_ctx->_num_total_nodes << ")";
+  CHECK_EQ(st, 0u) << "extraction kernels reported status 0x" << std::hex << st << std::dec
+                   << ((st & UGK_ST_KEY_OUT_OF_RANGE)
+                           ? ": a key is outside the table it has to be read from (num_total_item=" +
+                                 std::to_string(_cache_ctx->_num_total_nodes) + ")"
+                           : "")
+                   << ((st & UGK_ST_BAD_SEGMENT)
+                           ? ": the offsets of a pooled lookup leave the list of ids or run backwards"
+                           : "");
 }
 
 static int GatherDirect(const void *src, uint64_t rows, const IdType *keys, size_t n, void *out, size_t rb,

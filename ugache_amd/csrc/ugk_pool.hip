@@ -57,7 +57,8 @@ template <typename K, int KIND, int LPR, typename E>
 __global__ __launch_bounds__(kBlock) void extract_pool_kernel(ugk_table_t t, const K *__restrict__ ids,
                                                               const long long *__restrict__ seg_off,
                                                               const float *__restrict__ weights, size_t n_rows,
-                                                              const u32x4 *__restrict__ cache, uint64_t cache_rows,
+                                                              long long nnz, const u32x4 *__restrict__ cache,
+                                                              uint64_t cache_rows,
                                                               const u32x4 *__restrict__ host, uint64_t host_rows,
                                                               u32x4 *__restrict__ out, uint32_t vpr, int combiner,
                                                               uint32_t *status, uint32_t *host_mirror,
@@ -77,7 +78,14 @@ __global__ __launch_bounds__(kBlock) void extract_pool_kernel(ugk_table_t t, con
   for (size_t row0 = wave_global * RPW; row0 < n_rows; row0 += n_waves * RPW) {  // wavefront-uniform
     const size_t r = row0 + rg;
     const bool row_ok = r < n_rows;
-    const long long beg = row_ok ? seg_off[r] : 0, end = row_ok ? seg_off[r + 1] : 0;
+    long long beg = row_ok ? seg_off[r] : 0, end = row_ok ? seg_off[r + 1] : 0;
+    if (beg < 0 || end > nnz || end < beg) {  // a segment outside the ids: nothing is read for it, its row is zeros
+      if (sub == 0) {
+        atomicOr(status, UGK_ST_BAD_SEGMENT);
+        if (host_mirror) host_mirror[0] = UGK_ST_BAD_SEGMENT;
+      }
+      beg = end = 0;
+    }
     float acc[kPoolChunks][EPC];
 #pragma unroll
     for (int c = 0; c < kPoolChunks; ++c)
@@ -158,7 +166,6 @@ int extract_pool_lpr(ugk_table_t t, const K *ids, const long long *seg_off, cons
   // of rows a wavefront works on at once: rows of up to 512 bytes go to 8 lanes of up to four chunks each (eight rows
   // per wavefront; with 32 lanes and two rows per wavefront 262,144 samples of one id took 138 us instead of 83 us, and
   // 65,536 samples of 16 ids 123 us instead of 112 us), rows of up to 2 KB to 32 lanes, longer ones to 64.
-  (void)nnz;
   int lpr = vpr <= 8 * kPoolChunks ? 8 : vpr <= 32 * kPoolChunks ? 32 : 64;
   if (const char *forced = getenv("UGK_POOL_LPR")) {  // for sweeps; never a byte of the result depends on it
     const int v = atoi(forced);
@@ -169,8 +176,8 @@ int extract_pool_lpr(ugk_table_t t, const K *ids, const long long *seg_off, cons
   if (num_groups) *num_groups = grid;
 #define UGK_POOL(L)                                                                                                 \
   hipLaunchKernelGGL((extract_pool_kernel<K, KIND, L, E>), dim3(grid), dim3(kBlock), 0, st, t, ids, seg_off, weights, \
-                     n_rows, (const u32x4 *)cache, cache_rows, (const u32x4 *)host, host_rows, (u32x4 *)out, vpr,   \
-                     combiner, status, host_mirror, reinterpret_cast<unsigned long long *>(counts))
+                     n_rows, (long long)nnz, (const u32x4 *)cache, cache_rows, (const u32x4 *)host, host_rows,      \
+                     (u32x4 *)out, vpr, combiner, status, host_mirror, reinterpret_cast<unsigned long long *>(counts))
   if (lpr == 8) UGK_POOL(8);
   else if (lpr == 32) UGK_POOL(32);
   else UGK_POOL(64);
@@ -188,6 +195,7 @@ int extract_pool(ugk_table_t t, const K *ids, const int64_t *seg_off, const floa
   if (n_rows == 0) return 0;
   UGK_REQUIRE(seg_off && out && status, "ugk_extract_pool: null offsets, output or status");
   UGK_REQUIRE(nnz == 0 || ids, "ugk_extract_pool: null ids");
+  UGK_REQUIRE(nnz <= (uint64_t)INT64_MAX, "ugk_extract_pool: %llu ids", (unsigned long long)nnz);
   UGK_REQUIRE((uintptr_t)counts % 8 == 0, "ugk_extract_pool: the count words must be 8-byte aligned");
   UGK_REQUIRE(combiner >= 0 && combiner <= 2, "ugk_extract_pool: combiner %d is not sum(0), mean(1) or sqrtn(2)", combiner);
   UGK_REQUIRE(elem_bytes == 4 || elem_bytes == 2, "ugk_extract_pool: elements of %d bytes are not fp32 or fp16", elem_bytes);
