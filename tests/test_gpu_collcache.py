@@ -1404,8 +1404,12 @@ def test_pooled_lookup_through_the_library(pct, table_kind, dtype, dim, kdtype, 
     co.coll_torch_init_t(0, 0, emb, pct)
     _, nid = expected_cached_set(s0.astype(np.uint32), n_item, pct) if 0 < pct < 1 else (None, None)
     counted = []
-    for n_rows in (1, 64, 5_000):
+    # (the last batch is one of mostly one id per sample, large enough for the launch to give a lane group four
+    # output rows by itself)
+    for n_rows in (1, 64, 5_000, 70_000):
         lens = rng.choice([0, 1, 3, 8, 40], size=n_rows, p=[0.05, 0.35, 0.3, 0.25, 0.05])
+        if n_rows == 70_000:
+            lens = rng.choice([0, 1, 2, 5], size=n_rows, p=[0.1, 0.8, 0.08, 0.02])
         off = np.concatenate([[0], np.cumsum(lens)]).astype(np.int64)
         ids = perm[zipf_ranks(rng, int(off[-1]), n_item, 1.05)] if off[-1] else np.zeros(0, np.int64)
         w = rng.uniform(0.1, 2.0, size=len(ids)).astype(np.float32)

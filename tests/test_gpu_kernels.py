@@ -596,12 +596,16 @@ def _pool_reference(table_f64, ids, seg_off, weights, combiner):
 @pytest.mark.parametrize("dim,etype", [(4, np.float32), (32, np.float32), (128, np.float32), (512, np.float32),
                                        (1024, np.float32), (8, np.float16), (64, np.float16), (256, np.float16),
                                        (2048, np.float16)])
-def test_pooled_extraction_matches_a_float64_segment_sum(kind, dim, etype):
+@pytest.mark.parametrize("rows_per_group", ["", "3", "8"])
+def test_pooled_extraction_matches_a_float64_segment_sum(kind, dim, etype, rows_per_group, monkeypatch):
     """ugk_extract_pool_*: rows looked up and combined per segment in one kernel (sum, mean, sqrtn; with and without
-    weights, negative and zero ones among them; segments that are empty, single, longer than a lane group).  fp32
+    weights, negative and zero ones among them; segments that are empty, single, longer than a lane group; three
+    or eight output rows per lane group and pass, or as many as the launch picks by itself: one for these).  fp32
     rows within 1e-5 of the magnitude of the terms that were added (sum of |w x|, over the denominator), fp16 rows
     within 1e-3 of the result on top (the output is rounded to fp16); the counts are those of the ids by source, as for
     the plain fused extraction."""
+    if rows_per_group:
+        monkeypatch.setenv("UGK_POOL_ROWS", rows_per_group)
     rng = np.random.default_rng(dim + len(kind))
     nkeys = 20_000
     rb = dim * np.dtype(etype).itemsize
@@ -686,7 +690,10 @@ def test_pooled_extraction_matches_a_float64_segment_sum(kind, dim, etype):
         words.free()
 
 
-def test_pooled_extraction_hand_worked():
+@pytest.mark.parametrize("rows_per_group", ["", "2", "8"])
+def test_pooled_extraction_hand_worked(rows_per_group, monkeypatch):
+    if rows_per_group:
+        monkeypatch.setenv("UGK_POOL_ROWS", rows_per_group)
     # rows r = [r, 10 r]; segments {1, 2}, {3}, {}, {4, 4} with weights 1 2 | 3 | | 1 -1
     host = np.array([[r, 10 * r, 0, 0] for r in range(6)], np.float32)
     pin = pinned_from(host.view(np.uint8).reshape(6, 16))

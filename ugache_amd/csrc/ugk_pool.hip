@@ -157,30 +157,211 @@ __global__ __launch_bounds__(kBlock) void extract_pool_kernel(ugk_table_t t, con
   if (counts) mix_leave_counts(block_tot, wave_local, wave_host, counts);
 }
 
+constexpr int kPoolMaxRows = 8;  // output rows a lane group may own per pass
+
+// The same for short segments.  A lane group owns `rows_per_group` consecutive output rows per pass and walks their
+// ids as one list: position f of the list is id seg_beg[k] + (f - seg_start[k]) of the group's row k, the last k whose
+// seg_start is <= f.  The lanes resolve LPR positions at a time; the rows behind them are then read U at a time
+// whatever segments they belong to and added in the order of the list, an output row being written when the list
+// moves on to a later one.  What keeps memory busy is then the number of ids, not the shape of the segments: with one
+// row per group a sample of one or two ids leaves most of the group's lookups and loads unused (262,144 samples of
+// one id: 84 us per call with one row per group, 70 us with four).  The bookkeeping costs registers (three
+// wavefronts per SIMD instead of four), which is why samples of more ids stay with the kernel above (65,536 samples
+// of 16 ids: 121 us here, 114 us there).
+template <typename K, int KIND, int LPR, typename E>
+__global__ __launch_bounds__(kBlock) void extract_pool_rows_kernel(ugk_table_t t, const K *__restrict__ ids,
+                                                              const long long *__restrict__ seg_off,
+                                                              const float *__restrict__ weights, size_t n_rows,
+                                                              long long nnz, int rows_per_group,
+                                                              const u32x4 *__restrict__ cache, uint64_t cache_rows,
+                                                              const u32x4 *__restrict__ host, uint64_t host_rows,
+                                                              u32x4 *__restrict__ out, uint32_t vpr, int combiner,
+                                                              uint32_t *status, uint32_t *host_mirror,
+                                                              unsigned long long *counts) {
+  constexpr int RPW = kWave / LPR;  // lane groups per wavefront
+  constexpr int EPC = PoolElem<E>::kPerChunk;
+  constexpr int U = 4;  // rows in flight per lane group
+  static_assert(LPR % U == 0 && LPR >= kPoolMaxRows, "ids are taken in rounds of U; a lane per owned row");
+  __shared__ uint32_t block_tot[2];
+  __shared__ long long seg_beg[kWavesPerBlock][RPW][kPoolMaxRows];    // first id of the group's row k
+  __shared__ uint32_t seg_start[kWavesPerBlock][RPW][kPoolMaxRows];   // its first position in the group's list
+  if (threadIdx.x < 2) block_tot[threadIdx.x] = 0;
+  __syncthreads();
+  uint32_t wave_local = 0, wave_host = 0;
+  const int lane = (int)lane_id();
+  const int sub = lane % LPR, rg = lane / LPR, wv_in_block = (int)(threadIdx.x / kWave);
+  const size_t wave_global = (size_t)blockIdx.x * kWavesPerBlock + wv_in_block;
+  const size_t n_waves = (size_t)gridDim.x * kWavesPerBlock;
+  const size_t rows_per_wave = (size_t)RPW * rows_per_group;
+  long long *my_beg = seg_beg[wv_in_block][rg];
+  uint32_t *my_start = seg_start[wv_in_block][rg];
+  for (size_t row0 = wave_global * rows_per_wave; row0 < n_rows; row0 += n_waves * rows_per_wave) {  // wavefront-uniform
+    const size_t g0 = row0 + (size_t)rg * rows_per_group;  // the group's first row
+    const int n_own = g0 < n_rows ? (int)min((size_t)rows_per_group, n_rows - g0) : 0;
+    long long beg = 0;
+    uint32_t len = 0;
+    if (sub < n_own) {
+      const long long b = seg_off[g0 + sub], e = seg_off[g0 + sub + 1];
+      // a segment outside the ids (or one of 2^28 ids and more: the list of a group is counted in 32 bits): nothing
+      // is read for it, its row is zeros
+      if (b < 0 || e > nnz || e < b || e - b >= (1ll << 28)) {
+        atomicOr(status, UGK_ST_BAD_SEGMENT);
+        if (host_mirror) host_mirror[0] = UGK_ST_BAD_SEGMENT;
+      } else {
+        beg = b, len = (uint32_t)(e - b);
+      }
+    }
+    uint32_t incl = len;  // inclusive prefix over the group's rows (lanes past the owned rows add nothing)
+#pragma unroll
+    for (int d = 1; d < kPoolMaxRows; d <<= 1) {
+      const uint32_t up = (uint32_t)__shfl_up((int)incl, d, LPR);
+      if (sub >= d) incl += up;
+    }
+    const uint32_t total = (uint32_t)__shfl((int)incl, rg * LPR + kPoolMaxRows - 1);  // ids of the group this pass
+    if (sub < kPoolMaxRows) my_beg[sub] = beg, my_start[sub] = incl - len;
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    float acc[kPoolChunks][EPC];
+#pragma unroll
+    for (int c = 0; c < kPoolChunks; ++c)
+#pragma unroll
+      for (int e = 0; e < EPC; ++e) acc[c][e] = 0.f;
+    int cur = 0;       // the owned row the accumulators belong to
+    float wsum = 0.f;  // its sum of weights (or of their squares) so far
+    // one chunk of an owned row is complete: divide (div_no_nan), write, start the next row
+    auto flush = [&](int c, uint32_t col, int k, float ws) {
+      const float denom = combiner == 1 ? ws : combiner == 2 ? sqrtf(ws) : 1.f;
+      float y[EPC];
+#pragma unroll
+      for (int e = 0; e < EPC; ++e) y[e] = denom != 0.f ? acc[c][e] / denom : 0.f, acc[c][e] = 0.f;
+      out[(g0 + k) * vpr + col] = PoolElem<E>::pack(y);
+    };
+    for (uint32_t f0 = 0; __ballot(f0 < total) != 0ull; f0 += LPR) {  // until every group of the wavefront is through
+      const uint32_t f = f0 + sub;
+      const bool active = f < total;
+      int k = 0;
+      if (rows_per_group > 1) {
+#pragma unroll
+        for (int q = 1; q < kPoolMaxRows; ++q) k += my_start[q] <= f ? 1 : 0;  // rows past the owned ones start at total
+      }
+      const long long j = active ? my_beg[k] + (long long)(f - my_start[k]) : 0;
+      const uint64_t key = active ? key_to_u64<K>(ids[j]) : 0;
+      const Found fd = table_lookup<KIND>(t, key, active);
+      const MixRow row = mix_resolve(t, key, active, fd, cache, cache_rows, host, host_rows, out, vpr, status, host_mirror);
+      if (counts) {
+        wave_local += __popcll(__ballot(row.from_cache));
+        wave_host += __popcll(__ballot(active && !row.from_cache));
+      }
+      const bool use = active && row.has_row;  // a key without a row adds nothing (the launch is flagged)
+      const float w = use ? (weights ? weights[j] : 1.f) : 0.f;
+      const int meta = active ? (k | (use ? 0x100 : 0) | 0x200) : 0;  // owned row, "adds something", "is an id"
+      for (int s0 = 0; s0 < LPR; s0 += U) {
+        if (__ballot(active && sub >= s0) == 0ull) break;  // no group has an id left in this round
+        grow_t p[U];
+        float wv[U];
+        int m[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+          const int src = rg * LPR + s0 + u;
+          p[u] = reinterpret_cast<grow_t>(shfl64(row.bits, src));
+          wv[u] = __shfl(w, src);
+          m[u] = __shfl(meta, src);
+        }
+#pragma unroll
+        for (int c = 0; c < kPoolChunks; ++c) {
+          const uint32_t col = (uint32_t)c * LPR + sub;
+          if (col < vpr) {
+            u32x4 v[U];
+#pragma unroll
+            for (int u = 0; u < U; ++u) v[u] = __builtin_nontemporal_load(p[u] + col);
+            int cc = cur;  // every chunk walks the same ids from the same state
+            float ws = wsum;
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+              float x[EPC];
+              PoolElem<E>::unpack(v[u], x);
+              if (m[u] & 0x200) {
+                for (const int ku = m[u] & 0xff; cc < ku; ++cc, ws = 0.f) flush(c, col, cc, ws);
+                if (m[u] & 0x100) {
+#pragma unroll
+                  for (int e = 0; e < EPC; ++e) acc[c][e] = fmaf(wv[u], x[e], acc[c][e]);
+                  ws += combiner == 2 ? wv[u] * wv[u] : wv[u];
+                }
+              }
+            }
+          }
+        }
+        // the state after these ids, for the lanes of every chunk alike (a lane may own no chunk at all)
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+          if (m[u] & 0x200) {
+            if (cur < (m[u] & 0xff)) cur = m[u] & 0xff, wsum = 0.f;
+            if (m[u] & 0x100) wsum += combiner == 2 ? wv[u] * wv[u] : wv[u];
+          }
+        }
+      }
+    }
+    // the row the list ended in, and the empty ones behind it
+#pragma unroll
+    for (int c = 0; c < kPoolChunks; ++c) {
+      const uint32_t col = (uint32_t)c * LPR + sub;
+      if (col < vpr) {
+        float ws = wsum;
+        for (int cc = cur; cc < n_own; ++cc, ws = 0.f) flush(c, col, cc, ws);
+      }
+    }
+    __builtin_amdgcn_wave_barrier();  // the next pass rewrites the group's list
+  }
+  if (counts) mix_leave_counts(block_tot, wave_local, wave_host, counts);
+}
+
 template <typename K, int KIND, typename E>
 int extract_pool_lpr(ugk_table_t t, const K *ids, const long long *seg_off, const float *weights, size_t n_rows,
                      const void *cache, uint64_t cache_rows, const void *host, uint64_t host_rows, void *out,
                      uint32_t vpr, uint64_t nnz, int combiner, uint32_t *status, uint32_t *host_mirror,
                      uint64_t *counts, uint32_t *num_groups, hipStream_t st) {
-  // Lanes per output row.  A lane group walks its row's ids a few at a time, so what keeps memory busy is the number
-  // of rows a wavefront works on at once: rows of up to 512 bytes go to 8 lanes of up to four chunks each (eight rows
-  // per wavefront; with 32 lanes and two rows per wavefront 262,144 samples of one id took 138 us instead of 83 us, and
-  // 65,536 samples of 16 ids 123 us instead of 112 us), rows of up to 2 KB to 32 lanes, longer ones to 64.
+  // Lanes per output row: rows of up to 512 bytes go to 8 lanes of up to four chunks each (eight lane groups per
+  // wavefront; with 32 lanes and two groups 65,536 samples of 16 ids took 123 us instead of 112 us), rows of up to
+  // 2 KB to 32 lanes, longer ones to 64.
   int lpr = vpr <= 8 * kPoolChunks ? 8 : vpr <= 32 * kPoolChunks ? 32 : 64;
   if (const char *forced = getenv("UGK_POOL_LPR")) {  // for sweeps; never a byte of the result depends on it
     const int v = atoi(forced);
     if ((v == 8 || v == 32 || v == 64) && vpr <= (uint32_t)v * kPoolChunks) lpr = v;
   }
-  const size_t rows_per_group = (size_t)(kWave / lpr) * kWavesPerBlock;
-  const unsigned grid = clamp_grid((n_rows + rows_per_group - 1) / rows_per_group, 0);
+  // Output rows per lane group and pass.  One row each (extract_pool_kernel) is the faster kernel from two ids per
+  // sample on (it needs fewer registers: four wavefronts per SIMD instead of three; at two ids the two are level);
+  // for samples of mostly one id a group takes four rows as one list (extract_pool_rows_kernel), as long as the
+  // launch still has wavefronts for every CU.
+  const int groups_per_wave = kWave / lpr;
+  int rows = n_rows && nnz <= (uint64_t)n_rows + n_rows / 2 ? 4 : 1;
+  const size_t enough_waves = (size_t)cu_count() * 8;
+  while (rows > 1 && n_rows / ((size_t)rows * groups_per_wave) < enough_waves) rows /= 2;
+  if (const char *forced = getenv("UGK_POOL_ROWS")) {  // for sweeps, like the one above
+    const int v = atoi(forced);
+    if (v >= 1 && v <= kPoolMaxRows) rows = v;
+  }
+  const size_t rows_per_block = (size_t)rows * groups_per_wave * kWavesPerBlock;
+  const unsigned grid = clamp_grid((n_rows + rows_per_block - 1) / rows_per_block, 0);
   if (num_groups) *num_groups = grid;
-#define UGK_POOL(L)                                                                                                 \
-  hipLaunchKernelGGL((extract_pool_kernel<K, KIND, L, E>), dim3(grid), dim3(kBlock), 0, st, t, ids, seg_off, weights, \
-                     n_rows, (long long)nnz, (const u32x4 *)cache, cache_rows, (const u32x4 *)host, host_rows,      \
-                     (u32x4 *)out, vpr, combiner, status, host_mirror, reinterpret_cast<unsigned long long *>(counts))
-  if (lpr == 8) UGK_POOL(8);
-  else if (lpr == 32) UGK_POOL(32);
-  else UGK_POOL(64);
+#define UGK_POOL(L)                                                                                                    \
+  if (rows == 1)                                                                                                       \
+    hipLaunchKernelGGL((extract_pool_kernel<K, KIND, L, E>), dim3(grid), dim3(kBlock), 0, st, t, ids, seg_off,         \
+                       weights, n_rows, (long long)nnz, (const u32x4 *)cache, cache_rows, (const u32x4 *)host,         \
+                       host_rows, (u32x4 *)out, vpr, combiner, status, host_mirror,                                    \
+                       reinterpret_cast<unsigned long long *>(counts));                                                \
+  else                                                                                                                 \
+    hipLaunchKernelGGL((extract_pool_rows_kernel<K, KIND, L, E>), dim3(grid), dim3(kBlock), 0, st, t, ids, seg_off,    \
+                       weights, n_rows, (long long)nnz, rows, (const u32x4 *)cache, cache_rows, (const u32x4 *)host,   \
+                       host_rows, (u32x4 *)out, vpr, combiner, status, host_mirror,                                    \
+                       reinterpret_cast<unsigned long long *>(counts))
+  if (lpr == 8) {
+    UGK_POOL(8);
+  } else if (lpr == 32) {
+    UGK_POOL(32);
+  } else {
+    UGK_POOL(64);
+  }
 #undef UGK_POOL
   UGK_HIP(hipGetLastError());
   return 0;

@@ -311,7 +311,7 @@ def probe_pooled(hip, torch, note, quick=False):
         emb = co.coll_torch_create_emb_shm(0, rows, dim, torch.float32)
         emb.normal_(generator=torch.Generator().manual_seed(1))
         co.coll_torch_init_t(0, 0, emb, pct)
-        for per_sample, zipf in ((1, 0.0), (4, 0.0), (16, 0.0), (16, 1.05)) if not quick else ((8, 0.0),):
+        for per_sample, zipf in ((1, 0.0), (2, 0.0), (4, 0.0), (16, 0.0), (16, 1.05)) if not quick else ((8, 0.0),):
             n_samples = 262_144 if per_sample <= 4 else 65_536
             nnz = n_samples * per_sample
             if zipf:  # duplicates among the ids, as a skewed multi-hot feature has them
