@@ -123,12 +123,22 @@ void coll_cache_forward_pooled_i64(int replica_id, const int64_t *key, const int
  * everything enqueued so far has finished, aborts if a key was outside its table, and makes
  * coll_cache_last_group_offset describe the last batch; any blocking lookup does the same first.  No per-step profiler
  * values are logged for stream-ordered batches.  Such a call is kernel launches only (no synchronisation, no
- * allocation, no memset), so it may be recorded into a HIP graph by a caller that captures its stream.  Batches the
+ * allocation, no memset), so it may be recorded into a HIP graph by a caller that captures its stream; a lookup that
+ * is being recorded is not counted by the device-side hotness counters (the counting runs on a stream of the library,
+ * which stays out of the caller's graph).  Batches the
  * one-kernel paths cannot take (COLL_DEDUP_KEYS, a factored
  * SAMGRAPH_COLL_CACHE_CONCURRENT_LINK_IMPL, rows not multiples of 16 bytes with a partial cache) block as usual. */
 void coll_cache_lookup_async(int replica_id, const uint32_t *key, size_t num_keys, void *output, StreamHandle stream);
 void coll_cache_lookup_async_i64(int replica_id, const int64_t *key, size_t num_keys, void *output,
                                  StreamHandle stream);
+/* The pooled lookup in the same stream-ordered form (no counterpart in the reference either): enqueued and left, the
+ * group sizes (of ids) and the status arrive with coll_cache_lookup_wait. */
+void coll_cache_lookup_pooled_async(int replica_id, const uint32_t *key, const int64_t *seg_off, const float *weights,
+                                    size_t num_rows, size_t num_keys, int combiner, int elem_bytes, void *output,
+                                    StreamHandle stream);
+void coll_cache_lookup_pooled_async_i64(int replica_id, const int64_t *key, const int64_t *seg_off,
+                                        const float *weights, size_t num_rows, size_t num_keys, int combiner,
+                                        int elem_bytes, void *output, StreamHandle stream);
 void coll_cache_lookup_wait(int replica_id, StreamHandle stream);
 /* Sparse-id mode (extension; call after coll_cache_config and before recording or building): the caller's id of
  * host row r is (r * mul) mod 2^bits with mul odd, so 64-bit hashed ids from a 2^bits space address a dense host table

@@ -90,7 +90,7 @@ typedef struct {
 const char *ugk_last_error(void);
 /* version of this ABI; bumped on any signature change.  ugk_abi_version() is what the loaded library was built with:
  * a caller compiled against another UGK_ABI_VERSION must not go on. */
-#define UGK_ABI_VERSION 13
+#define UGK_ABI_VERSION 14
 int ugk_abi_version(void);
 
 /* ---- runtime plumbing: Device::{AllocDataSpace,FreeDataSpace,CopyDataFromTo,StreamSync,CreateStream}
@@ -113,6 +113,8 @@ int ugk_stream_create(void **stream);
 int ugk_stream_create_cu_masked(void **stream, int num_cus);
 int ugk_stream_destroy(void *stream);
 int ugk_stream_sync(void *stream);
+/* *capturing = 1 while work enqueued on `stream` is being recorded into a HIP graph instead of being run, else 0 */
+int ugk_stream_is_capturing(void *stream, int *capturing);
 /* ugk_stream_sync for callers that wait for short launches: enqueues a one-lane kernel that writes `value` into
  * *ticket_host (pinned host word from ugk_host_malloc) behind everything already enqueued on `stream`, and polls that
  * word from the host for up to spin_us microseconds before it falls back to waiting for the stream.  The word changes a

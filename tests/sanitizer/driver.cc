@@ -134,8 +134,8 @@ int main(int argc, char **argv) {
       coll_cache_forward(0, k.data(), k.size(), out.data(), nullptr);
       bad_rows += check_rows(table, out.data(), k.data(), k.size());
     }
-    // 5. pooled lookups (segments of ids combined per sample), plain and as steps of the serving loop
-    for (int step = 0; step < 6; ++step) {
+    // 5. pooled lookups (segments of ids combined per sample): plain, as steps of the serving loop, stream-ordered
+    for (int step = 0; step < 8; ++step) {
       auto k = skewed_keys(g, 2000, 20000 + (uint64_t)step * 31);
       std::vector<int64_t> off(1, 0);
       while ((size_t)off.back() < k.size()) off.push_back(std::min<int64_t>((int64_t)k.size(), off.back() + (int64_t)(g() % 6)));
@@ -146,8 +146,13 @@ int main(int argc, char **argv) {
       if (step < 3)
         coll_cache_lookup_pooled(0, k.data(), off.data(), step == 1 ? nullptr : w.data(), n_rows, k.size(), combiner, 4,
                                  out.data(), nullptr);
-      else
+      else if (step < 6)
         coll_cache_forward_pooled(0, k.data(), off.data(), w.data(), n_rows, k.size(), combiner, 4, out.data(), nullptr);
+      else {
+        coll_cache_lookup_pooled_async(0, k.data(), off.data(), w.data(), n_rows, k.size(), combiner, 4, out.data(),
+                                       nullptr);
+        coll_cache_lookup_wait(0, nullptr);
+      }
       for (size_t r = 0; r < n_rows; ++r)
         for (size_t c = 0; c < kDim; ++c) {
           double sum = 0, den = 0;

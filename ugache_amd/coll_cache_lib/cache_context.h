@@ -176,6 +176,7 @@ class ExtractSession {
   }
   size_t _async_pending = 0;       // stream-ordered lookups enqueued since the last Wait()
   size_t _async_last_nodes = 0;    // size of the last of them
+  bool _async_swap_counts = false;  // the last of them counted ids read from HBM as "from the host table"
   // What a refresh has to see finished before it reuses the slots of evicted rows: blocking lookups are counted when
   // they start and when they end, the streams stream-ordered lookups were enqueued on are remembered (normally one).
   struct InFlight;
@@ -197,6 +198,12 @@ class ExtractSession {
   void ExtractPooledImpl(const KeyT *nodes, const int64_t *seg_off, const float *weights, size_t num_rows,
                          size_t num_nodes, int combiner, int elem_bytes, void *output, StreamHandle stream,
                          uint64_t task_key);
+  template <typename KeyT>
+  bool LaunchPooled(const KeyT *nodes, const int64_t *seg_off, const float *weights, size_t num_rows, size_t num_nodes,
+                    int combiner, int elem_bytes, void *output, StreamHandle stream);
+  template <typename KeyT>
+  void ExtractPooledAsyncImpl(const KeyT *nodes, const int64_t *seg_off, const float *weights, size_t num_rows,
+                              size_t num_nodes, int combiner, int elem_bytes, void *output, StreamHandle stream);
   // Where the outputs of the last lookups went.  A caller that hands the same buffer over every time (the reference's
   // adapter does, adapter.cc:204-237) finds its rows in the memory-side cache; one that rotates over more buffers than
   // that cache holds is better served by streaming stores, and the kernels are told so (ugk_set_output_hint).
@@ -236,6 +243,12 @@ class ExtractSession {
   void ExtractPooled64(const Id64Type *nodes, const int64_t *seg_off, const float *weights, size_t num_rows,
                        size_t num_nodes, int combiner, int elem_bytes, void *output, StreamHandle stream,
                        uint64_t task_key);
+  // the same enqueued on `stream` without waiting (kernel launches only); Wait() completes it like a stream-ordered
+  // plain lookup: status checked, group sizes of the last batch made available
+  void ExtractPooledAsync(const IdType *nodes, const int64_t *seg_off, const float *weights, size_t num_rows,
+                          size_t num_nodes, int combiner, int elem_bytes, void *output, StreamHandle stream);
+  void ExtractPooledAsync64(const Id64Type *nodes, const int64_t *seg_off, const float *weights, size_t num_rows,
+                            size_t num_nodes, int combiner, int elem_bytes, void *output, StreamHandle stream);
   // The distinct keys of the batch looked up once (an extension; the "unique -> lookup -> gather(idx)" of the TF2
   // layer, sparse_lookup_layer.py:196-209, with the unique inside): output[u, :] = row of the u-th distinct key
   // (in order of first claim, not sorted), inverse_out[i] = which distinct key position i holds, so that

@@ -120,6 +120,18 @@ class CollCache : public std::enable_shared_from_this<CollCache> {
   void lookup_async64(int replica_id, const Id64Type *nodes, size_t num_nodes, void *output, StreamHandle stream) {
     _session_list.at(replica_id)->ExtractFeatAsync64(nodes, num_nodes, output, stream);
   }
+  void lookup_pooled_async(int replica_id, const IdType *nodes, const int64_t *seg_off, const float *weights,
+                           size_t num_rows, size_t num_nodes, int combiner, int elem_bytes, void *output,
+                           StreamHandle stream) {
+    _session_list.at(replica_id)->ExtractPooledAsync(nodes, seg_off, weights, num_rows, num_nodes, combiner, elem_bytes,
+                                                     output, stream);
+  }
+  void lookup_pooled_async64(int replica_id, const Id64Type *nodes, const int64_t *seg_off, const float *weights,
+                             size_t num_rows, size_t num_nodes, int combiner, int elem_bytes, void *output,
+                             StreamHandle stream) {
+    _session_list.at(replica_id)->ExtractPooledAsync64(nodes, seg_off, weights, num_rows, num_nodes, combiner,
+                                                       elem_bytes, output, stream);
+  }
   void lookup_wait(int replica_id, StreamHandle stream) { _session_list.at(replica_id)->Wait(stream); }
   std::shared_ptr<ExtractSession> session(int replica_id) { return _session_list.at(replica_id); }
   TensorPtr nid_to_block() { return _nid_to_block; }

@@ -273,6 +273,24 @@ void coll_cache_lookup_async_i64(int replica_id, const int64_t *key, size_t num_
   _coll_cache->lookup_async64(replica_id, key, num_keys, output, stream);
 }
 
+void coll_cache_lookup_pooled_async(int replica_id, const uint32_t *key, const int64_t *seg_off, const float *weights,
+                                    size_t num_rows, size_t num_keys, int combiner, int elem_bytes, void *output,
+                                    StreamHandle stream) {
+  CHECK_NOTNULL(_coll_cache);
+  steps[replica_id]++;
+  _coll_cache->lookup_pooled_async(replica_id, key, seg_off, weights, num_rows, num_keys, combiner, elem_bytes, output,
+                                   stream);
+}
+
+void coll_cache_lookup_pooled_async_i64(int replica_id, const int64_t *key, const int64_t *seg_off,
+                                        const float *weights, size_t num_rows, size_t num_keys, int combiner,
+                                        int elem_bytes, void *output, StreamHandle stream) {
+  CHECK_NOTNULL(_coll_cache);
+  steps[replica_id]++;
+  _coll_cache->lookup_pooled_async64(replica_id, key, seg_off, weights, num_rows, num_keys, combiner, elem_bytes,
+                                     output, stream);
+}
+
 void coll_cache_lookup_wait(int replica_id, StreamHandle stream) {
   CHECK_NOTNULL(_coll_cache);
   _coll_cache->lookup_wait(replica_id, stream);

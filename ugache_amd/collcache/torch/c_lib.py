@@ -178,13 +178,17 @@ def pooled_lookup_supported():
     return _State.external_dtype in (torch.float32, torch.float16) and row_bytes % 16 == 0 and 0 < row_bytes <= 4096
 
 
-def coll_torch_lookup_pooled(local_id, ids, seg_off, weights=None, combiner="sum", serving_step=False):
+def coll_torch_lookup_pooled(local_id, ids, seg_off, weights=None, combiner="sum", serving_step=False,
+                             stream_ordered=False):
     """lookup and per-sample combination of a multi-hot feature in one kernel (extension): segment r is
     ids[seg_off[r] : seg_off[r + 1]]; returns a new [len(seg_off) - 1, dim] tensor whose row r is the weighted sum of
     the segment's embeddings ("sum"), divided by the sum of the weights ("mean") or by the root of the sum of their
     squares ("sqrtn") — embedding_lookup_sparse without the [len(ids), dim] intermediate.  ids: GPU int32 / int64;
     seg_off: GPU int64, ascending, seg_off[0] == 0 and seg_off[-1] == len(ids); weights: GPU float32 or None.
-    serving_step: the call is one step of the serving loop (as coll_torch_forward is for a plain lookup)."""
+    serving_step: the call is one step of the serving loop (as coll_torch_forward is for a plain lookup).
+    stream_ordered: the call is enqueued on torch's current stream and returns without waiting, like any torch op
+    (as coll_torch_lookup_async is for a plain lookup; `ids`, `seg_off` and `weights` must stay alive until the work has
+    run; coll_torch_lookup_wait reports a bad id or offset and makes the group sizes available)."""
     dev = _State.dev_id.get(local_id, 0)
     if not pooled_lookup_supported():
         raise ValueError("pooled lookups need rows of a multiple of 16 bytes, at most 4096, of fp32 or fp16 elements")
@@ -198,8 +202,12 @@ def coll_torch_lookup_pooled(local_id, ids, seg_off, weights=None, combiner="sum
     weights = None if weights is None else weights.contiguous().reshape(-1)
     n_rows = seg_off.numel() - 1
     out = torch.empty((n_rows, _State.external_feat_dim), dtype=_State.external_dtype, device="cuda:%d" % dev)
+    if serving_step and stream_ordered:
+        raise ValueError("a step of the serving loop blocks: serving_step and stream_ordered exclude each other")
     if serving_step:
         fn = _C.coll_cache_forward_pooled_i64 if ids.dtype == torch.int64 else _C.coll_cache_forward_pooled
+    elif stream_ordered:
+        fn = _C.coll_cache_lookup_pooled_async_i64 if ids.dtype == torch.int64 else _C.coll_cache_lookup_pooled_async
     else:
         fn = _C.coll_cache_lookup_pooled_i64 if ids.dtype == torch.int64 else _C.coll_cache_lookup_pooled
     fn(local_id, ids.data_ptr() if ids.numel() else None, seg_off.data_ptr(),

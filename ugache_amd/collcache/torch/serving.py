@@ -202,6 +202,9 @@ class SparseLookupLayer(torch.nn.Module):
         # fused=True: lookup and combination in one kernel of the library (coll_torch_lookup_pooled) wherever that
         # kernel can take the call (no max_norm, rows it supports); the steps below otherwise
         self.fused = bool(kwargs.get("fused", False))
+        # stream_ordered=True (with fused): the call is enqueued on torch's current stream like any torch op instead of
+        # being a blocking step of the serving loop
+        self.stream_ordered = bool(kwargs.get("stream_ordered", False))
 
     def forward(self, sp_ids, sp_weights=None, name=None, combiner=None, max_norm=None):
         if combiner is None:
@@ -222,7 +225,9 @@ class SparseLookupLayer(torch.nn.Module):
             seg_off = torch.zeros(num_rows + 1, dtype=torch.int64, device=ids.device)
             torch.cumsum(counts, 0, out=seg_off[1:])
             weights = None if sp_weights is None else sp_weights._values().float()
-            return _adapter.coll_torch_lookup_pooled(0, ids, seg_off, weights, combiner, serving_step=True)
+            return _adapter.coll_torch_lookup_pooled(0, ids, seg_off, weights, combiner,
+                                                     serving_step=not self.stream_ordered,
+                                                     stream_ordered=self.stream_ordered)
         if self.unique_in_library:  # unique + lookup in one call, the unique by the library's GPU hash set
             self.lookup.check(ids)
             emb_unique, idx = _adapter.coll_torch_lookup_unique(0, ids)

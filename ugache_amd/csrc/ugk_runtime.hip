@@ -193,6 +193,14 @@ int ugk_stream_sync(void *stream) {
   return 0;
 }
 
+int ugk_stream_is_capturing(void *stream, int *capturing) {
+  UGK_REQUIRE(capturing, "ugk_stream_is_capturing: null output");
+  hipStreamCaptureStatus st = hipStreamCaptureStatusNone;
+  UGK_HIP(hipStreamIsCapturing(as_stream(stream), &st));
+  *capturing = st != hipStreamCaptureStatusNone;
+  return 0;
+}
+
 namespace {
 __global__ void ticket_kernel(volatile uint32_t *word, uint32_t value) { *word = value; }
 }  // namespace

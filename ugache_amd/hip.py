@@ -65,6 +65,7 @@ SIGNATURES = {
     "ugk_stream_create_cu_masked": [C.POINTER(_vp), _i],
     "ugk_stream_destroy": [_vp],
     "ugk_stream_sync": [_vp],
+    "ugk_stream_is_capturing": [_vp, _vp],
     "ugk_stream_sync_ticket": [_vp, _vp, _u32, C.c_uint],
     "ugk_device_sync": [],
     "ugk_event_create": [C.POINTER(_vp)],

@@ -327,6 +327,9 @@ def probe_pooled(hip, torch, note, quick=False):
             def fused():
                 return co.coll_torch_lookup_pooled(0, ids, seg_off, w, "sum")
 
+            def fused_stream_ordered():
+                return co.coll_torch_lookup_pooled(0, ids, seg_off, w, "sum", stream_ordered=True)
+
             def lookup_then_sum():
                 e = co.coll_torch_lookup_key_t_val_ret(0, ids, False)
                 out = torch.zeros((n_samples, dim), dtype=torch.float32, device="cuda")
@@ -341,7 +344,9 @@ def probe_pooled(hip, torch, note, quick=False):
             ref = lookup_then_sum()
             assert torch.allclose(fused(), ref, rtol=1e-4, atol=1e-4) and torch.allclose(unique_lookup_sum(), ref, rtol=1e-4, atol=1e-4)
             res = {}
-            for name, fn in (("fused", fused), ("lookup_then_sum", lookup_then_sum), ("unique_lookup_sum", unique_lookup_sum)):
+            assert torch.equal(fused_stream_ordered(), fused())
+            for name, fn in (("fused", fused), ("fused_stream_ordered", fused_stream_ordered),
+                             ("lookup_then_sum", lookup_then_sum), ("unique_lookup_sum", unique_lookup_sum)):
                 for _ in range(3):
                     fn()
                 torch.cuda.synchronize()
@@ -350,6 +355,7 @@ def probe_pooled(hip, torch, note, quick=False):
                     fn()
                 torch.cuda.synchronize()
                 res[name] = round((time.perf_counter() - t0) / calls * 1e6, 1)
+                co.coll_torch_lookup_wait(0)
             moved = nnz * dim * 4 + n_samples * dim * 4 + nnz * 12
             out_rows.append({"cache": label, "samples": n_samples, "ids_per_sample": per_sample, "zipf": zipf,
                              "us_per_call": res, "fused_GBps_of_rows_read_and_written": round(moved / res["fused"] / 1e3, 1)})
