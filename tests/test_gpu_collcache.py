@@ -1010,6 +1010,35 @@ def test_random_configurations_are_exact(case, monkeypatch):
         keys = rng.integers(0, n_item, size=5_000)
         out = co.coll_torch_lookup_key_t_val_ret(0, torch.from_numpy(keys).to(kdtype).cuda(), False)
         assert out.cpu().numpy().tobytes() == ORC.gather(table, keys.astype(np.int64)).tobytes()
+    if co.c_lib.pooled_lookup_supported():
+        # the same cache through the pooled lookup, blocking and stream-ordered.  The table holds random bit patterns:
+        # elements whose terms are not finite, or so large that an fp32 sum (or an fp16 result) may overflow, are left
+        # out of the comparison; the others are within 1e-5 of the magnitude of their terms (fp16 rounding on top)
+        with np.errstate(all="ignore"):
+            vals = emb.float().numpy().astype(np.float64)
+        n_rows = int(rng.integers(1, 4_000))
+        lens = rng.choice([0, 1, 2, 5, 30], size=n_rows, p=[0.1, 0.5, 0.2, 0.15, 0.05])
+        off = np.concatenate([[0], np.cumsum(lens)]).astype(np.int64)
+        ids = perm[zipf_ranks(rng, int(off[-1]), n_item, case["zipf"])] if off[-1] else np.zeros(0, np.int64)
+        w = rng.uniform(0.1, 2.0, size=len(ids)).astype(np.float32)
+        t_ids, t_off, t_w = torch.from_numpy(ids).to(kdtype).cuda(), torch.from_numpy(off).cuda(), torch.from_numpy(w).cuda()
+        combiner = ("sum", "mean", "sqrtn")[case["seed"] % 3]
+        with np.errstate(all="ignore"):
+            want = ORC.pool(vals, ids, off, w, combiner)
+            mag_sum = ORC.pool(np.abs(vals), ids, off, w, "sum")
+            mag = ORC.pool(np.abs(vals), ids, off, w, combiner)
+        ok = np.isfinite(mag_sum) & (mag_sum < 1e36) & (mag < (6.0e4 if fdtype == torch.float16 else 1e36))
+        bound = 1e-5 * np.where(ok, mag, 0.0) + (1e-3 * np.abs(np.where(ok, want, 0.0)) + 2.0 ** -25
+                                                 if fdtype == torch.float16 else 0.0) + 1e-30
+        for stream_ordered in (False, True):
+            got = co.coll_torch_lookup_pooled(0, t_ids, t_off, t_w, combiner, stream_ordered=stream_ordered)
+            if stream_ordered:
+                co.coll_torch_lookup_wait(0)
+            assert _basics.last_group_offset(0)[2] == len(ids)
+            got = got.float().cpu().numpy().astype(np.float64)
+            assert got.shape == (n_rows, dim)
+            bad = ok & ~(np.abs(got - np.where(ok, want, 0.0)) <= bound)
+            assert not bad.any(), ("pooled", stream_ordered, combiner, int(bad.sum()))
 
 
 @pytest.mark.parametrize("device", [False, True])
