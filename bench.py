@@ -477,9 +477,11 @@ def run_mixed(args):
     for _ in range(spec["presample"]):
         co.coll_torch_record(0, ids_of(make_batch()).cpu())
     note("hotness of %d presample batches recorded" % spec["presample"])
+    t_build = time.perf_counter()
     co.coll_torch_init_t(0, 0, emb, pct)
+    build_s = time.perf_counter() - t_build
     info_cache = _basics.info(0)
-    note("cache built: %d rows cached" % info_cache["cached_rows"])
+    note("cache built in %.3f s: %d rows cached" % (build_s, info_cache["cached_rows"]))
 
     rows_pool = torch.stack([make_batch() for _ in range(pool)])
     keys_pool = ids_of(rows_pool)
@@ -773,6 +775,12 @@ def run_mixed(args):
         "dtype": "u8", "data": "synthetic",
         "refresh": refresh, "refresh_each_step": each_step, "under_concurrent_refresh": under_refresh,
         "serving_loop": serving,
+        # ranking of the presample, placement, the cached rows copied host -> HBM and their keys put into the table
+        "cache_build": {"seconds": build_s, "rows_filled": info_cache["cached_rows"],
+                        "bytes_filled": info_cache["cached_rows"] * row_bytes,
+                        "fill_GBps_over_the_whole_build": info_cache["cached_rows"] * row_bytes / build_s / 1e9,
+                        "frac_of_measured_link": info_cache["cached_rows"] * row_bytes / build_s / 1e9 / link_gbps
+                        if link_gbps > 0 else None},
         "config": {"workload": args.workload, "table_rows": rows, "row_bytes": row_bytes, "keys_per_batch": n_keys,
                    "key_dtype": "int64", "sparse_ids": sparse, "cache_percentage": pct, "cached_rows": info_cache["cached_rows"],
                    "cache_capacity_rows": info_cache["capacity_rows"], "table_kind": info_cache["table_kind"],
@@ -900,7 +908,7 @@ def random_row_ceiling(hip, torch, emb, rows, row_bytes, dev, stream, note):
 # what a leg contributes to the default line: enough to recompute both halves of the metric
 LEG_KEYS = ("value", "unit", "ms_per_step", "ms_per_step_spread", "steps", "warmup", "config", "hit_rate",
             "effective_extraction_GBps", "parity", "stages_us", "roofline", "host_link", "cpu_baseline", "gpu_over_cpu",
-            "refresh", "refresh_each_step", "setup_seconds", "stream_ordered")
+            "refresh", "refresh_each_step", "setup_seconds", "stream_ordered", "cache_build")
 DEFAULT_LEGS = ("c3_gnn_100Mx128xfp32_1M_i64_zipf0.9_cache25pct", "c5_hash_500Mx64xfp16_1M_i64_zipf1.05_cache50M")
 
 
