@@ -139,6 +139,12 @@ void coll_cache_lookup_pooled_async(int replica_id, const uint32_t *key, const i
 void coll_cache_lookup_pooled_async_i64(int replica_id, const int64_t *key, const int64_t *seg_off,
                                         const float *weights, size_t num_rows, size_t num_keys, int combiner,
                                         int elem_bytes, void *output, StreamHandle stream);
+/* The seg_off a pooled lookup takes, made on the device from the row of every entry of a sparse feature in row-major
+ * order (extension; the indices[:, 0] of the SparseTensor of sparse_lookup_layer.py:196-265): seg_off[r] = number of
+ * entries whose row is below r, r = 0 .. num_rows (num_rows + 1 device words).  One kernel on `stream`, no wait.
+ * Entries out of order or outside [0, num_rows) make the next lookup's status check abort with a message. */
+void coll_cache_segment_offsets(int replica_id, const int64_t *sorted_rows, size_t num_entries, size_t num_rows,
+                                int64_t *seg_off, StreamHandle stream);
 void coll_cache_lookup_wait(int replica_id, StreamHandle stream);
 /* Sparse-id mode (extension; call after coll_cache_config and before recording or building): the caller's id of
  * host row r is (r * mul) mod 2^bits with mul odd, so 64-bit hashed ids from a 2^bits space address a dense host table

@@ -90,7 +90,7 @@ typedef struct {
 const char *ugk_last_error(void);
 /* version of this ABI; bumped on any signature change.  ugk_abi_version() is what the loaded library was built with:
  * a caller compiled against another UGK_ABI_VERSION must not go on. */
-#define UGK_ABI_VERSION 14
+#define UGK_ABI_VERSION 15
 int ugk_abi_version(void);
 
 /* ---- runtime plumbing: Device::{AllocDataSpace,FreeDataSpace,CopyDataFromTo,StreamSync,CreateStream}
@@ -284,6 +284,13 @@ int ugk_extract_mix_i64(ugk_table_t t, const int64_t *keys_dev, size_t n, const 
  * ugk_extract_mix_* (the counts are of ids, not of output rows).  An id without a row sets UGK_ST_KEY_OUT_OF_RANGE and
  * adds nothing; a segment whose offsets leave [0, nnz] or run backwards sets UGK_ST_BAD_SEGMENT, reads no id and
  * gives a zero row. */
+/* The offsets ugk_extract_pool_* takes, from the row of every entry of a sparse feature in row-major order (the
+ * indices[:, 0] of the SparseTensor of sparse_lookup_layer.py:196-265): seg_off_dev[r] = number of entries whose row is
+ * below r, for r = 0 .. n_rows (n_rows + 1 words; rows without an entry get empty segments).  One launch, no
+ * synchronisation.  Entries that are out of order or outside [0, n_rows) set UGK_ST_BAD_SEGMENT (status_dev and
+ * host_mirror may be NULL) and leave words of seg_off_dev unwritten. */
+int ugk_segment_offsets_i64(const int64_t *sorted_rows_dev, size_t nnz, size_t n_rows, int64_t *seg_off_dev,
+                            uint32_t *status_dev, uint32_t *host_mirror, void *stream);
 int ugk_extract_pool_u32(ugk_table_t t, const uint32_t *ids_dev, const int64_t *seg_off_dev, const float *weights_dev,
                          size_t n_rows, uint64_t nnz, int combiner, int elem_bytes, const void *cache_dev,
                          uint64_t cache_rows, const void *host_dev, uint64_t host_rows, void *out_dev, size_t row_bytes,

@@ -149,7 +149,13 @@ int main(int argc, char **argv) {
       else if (step < 6)
         coll_cache_forward_pooled(0, k.data(), off.data(), w.data(), n_rows, k.size(), combiner, 4, out.data(), nullptr);
       else {
-        coll_cache_lookup_pooled_async(0, k.data(), off.data(), w.data(), n_rows, k.size(), combiner, 4, out.data(),
+        // the offsets made by the library from the row of every id
+        std::vector<int64_t> row_of(k.size()), made(off.size(), -1);
+        for (size_t r = 0; r < n_rows; ++r)
+          for (int64_t j = off[r]; j < off[r + 1]; ++j) row_of[j] = (int64_t)r;
+        coll_cache_segment_offsets(0, row_of.data(), row_of.size(), n_rows, made.data(), nullptr);
+        if (made != off) ++bad_rows;
+        coll_cache_lookup_pooled_async(0, k.data(), made.data(), w.data(), n_rows, k.size(), combiner, 4, out.data(),
                                        nullptr);
         coll_cache_lookup_wait(0, nullptr);
       }

@@ -760,6 +760,21 @@ int ugk_extract_mix_i64(ugk_table_t t, const int64_t *keys, size_t n, const void
   return extract_mix(t, keys, n, cache, cache_rows, host, host_rows, out, rb, status, mirror, counts, num_groups);
 }
 
+int ugk_segment_offsets_i64(const int64_t *rows, size_t nnz, size_t n_rows, int64_t *seg_off, uint32_t *status,
+                            uint32_t *mirror, void *) {
+  REQUIRE(seg_off && (nnz == 0 || rows), "ugk_segment_offsets: null pointer");
+  for (size_t i = 0; i <= nnz; ++i) {
+    const int64_t prev = i == 0 ? -1 : rows[i - 1];
+    const int64_t cur = i == nnz ? (int64_t)n_rows : rows[i];
+    if (cur < prev || cur < 0 || (i > 0 && prev < 0) || (i < nnz && cur >= (int64_t)n_rows) || prev >= (int64_t)n_rows) {
+      if (status) or_status(status, UGK_ST_BAD_SEGMENT, mirror);
+      continue;
+    }
+    for (int64_t r = prev + 1; r <= cur; ++r) seg_off[r] = (int64_t)i;
+  }
+  return 0;
+}
+
 int ugk_extract_pool_u32(ugk_table_t t, const uint32_t *ids, const int64_t *seg_off, const float *weights, size_t n_rows,
                          uint64_t nnz, int combiner, int elem_bytes, const void *cache, uint64_t cache_rows,
                          const void *host, uint64_t host_rows, void *out, size_t rb, uint32_t *status, uint32_t *mirror,

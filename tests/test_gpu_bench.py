@@ -42,6 +42,8 @@ def test_mixed_workload_line_with_the_serving_loop():
     _check_contract(d, 12, 3)
     link = d["host_link"]
     assert 0 < link["frac"] <= 1.05 and link["achieved"] > 0
+    b = d["cache_build"]
+    assert b["seconds"] > 0 and b["rows_filled"] == d["config"]["cached_rows"] and b["bytes_filled"] == b["rows_filled"] * 512
     s = d["serving_loop"]
     assert s["steps"] == 12 and s["ms_per_step"] > 0 and s["refreshes_completed"] >= 1
     assert sum(s["steps_of_each"]) == 12 and s["hotness_recorded_on"] == "host"

@@ -748,6 +748,31 @@ def test_pooled_extraction_hand_worked(rows_per_group, monkeypatch):
         pin.free()
 
 
+@pytest.mark.parametrize("n_rows,nnz", [(1, 0), (1, 1), (5, 0), (7, 3), (1000, 1000), (5000, 60_000), (300_000, 40_000)])
+def test_segment_offsets_match_searchsorted(n_rows, nnz):
+    """ugk_segment_offsets_i64: seg_off[r] = number of entries whose row is below r (rows without an entry among them)"""
+    rng = np.random.default_rng(n_rows + nnz)
+    rows = np.sort(rng.integers(0, n_rows, size=nnz)).astype(np.int64)
+    st = dev_zeros_u32(1)
+    d_rows = to_dev(rows if nnz else np.zeros(1, np.int64))
+    out = to_dev(np.full(n_rows + 1, -7, np.int64))
+    hip.call("ugk_segment_offsets_i64", ptr(d_rows), nnz, n_rows, ptr(out), ptr(st), None, None)
+    sync()
+    assert status_value(st) == 0
+    assert np.array_equal(to_np(out), np.searchsorted(rows, np.arange(n_rows + 1), side="left"))
+
+
+@pytest.mark.parametrize("bad", [[0, 2, 1, 3], [0, 1, 2, 9], [-1, 0, 1, 2], [3, 2, 1, 0], [0, 1, 2, 1 << 40]])
+def test_segment_offsets_flag_rows_out_of_order_or_range(bad):
+    st = dev_zeros_u32(1)
+    out = to_dev(np.full(6, -7, np.int64))
+    hip.call("ugk_segment_offsets_i64", ptr(to_dev(np.array(bad, np.int64))), 4, 5, ptr(out), ptr(st), None, None)
+    sync()
+    assert status_value(st) == hip.ST_BAD_SEGMENT
+    got = to_np(out)
+    assert ((got == -7) | ((got >= 0) & (got <= 4))).all()  # nothing written but offsets into the entries
+
+
 def _fmix64(x):
     x = np.asarray(x, np.uint64).copy()
     x ^= x >> np.uint64(33)

@@ -326,7 +326,8 @@ void ExtractSession::CheckStatusWord(StreamHandle stream) const {
                                  std::to_string(_cache_ctx->_num_total_nodes) + ")"
                            : "")
                    << ((st & UGK_ST_BAD_SEGMENT)
-                           ? ": the offsets of a pooled lookup leave the list of ids or run backwards"
+                           ? ": the offsets of a pooled lookup leave the list of ids or run backwards (or the rows "
+                             "they were made from are not in ascending order inside [0, num_rows))"
                            : "");
 }
 
@@ -1115,6 +1116,13 @@ void ExtractSession::ExtractPooledImpl(const KeyT *nodes, const int64_t *seg_off
     profiler->LogEpochAdd(task_key, kLogEpochMissBytes, (double)n_miss * rb);
   }
   ctx->progress.fetch_add(1);
+}
+
+void ExtractSession::SegmentOffsets(const int64_t *sorted_rows, size_t num_entries, size_t num_rows, int64_t *seg_off,
+                                    StreamHandle stream) {
+  CHECK_NOTNULL(seg_off);
+  CHECK(num_entries == 0 || sorted_rows != nullptr);
+  UGK_CALL(ugk_segment_offsets_i64(sorted_rows, num_entries, num_rows, seg_off, _status, _host_mirror, stream));
 }
 
 // the stream-ordered form: kernel launches only, completed by Wait() like a stream-ordered plain lookup

@@ -243,6 +243,11 @@ class ExtractSession {
   void ExtractPooled64(const Id64Type *nodes, const int64_t *seg_off, const float *weights, size_t num_rows,
                        size_t num_nodes, int combiner, int elem_bytes, void *output, StreamHandle stream,
                        uint64_t task_key);
+  // The offsets a pooled lookup takes, from the row of every entry of a sparse feature in row-major order:
+  // seg_off[r] = entries whose row is below r, r = 0 .. num_rows.  One launch on `stream`, no wait; entries out of
+  // order or outside [0, num_rows) are reported by the next lookup's status check.
+  void SegmentOffsets(const int64_t *sorted_rows, size_t num_entries, size_t num_rows, int64_t *seg_off,
+                      StreamHandle stream);
   // the same enqueued on `stream` without waiting (kernel launches only); Wait() completes it like a stream-ordered
   // plain lookup: status checked, group sizes of the last batch made available
   void ExtractPooledAsync(const IdType *nodes, const int64_t *seg_off, const float *weights, size_t num_rows,

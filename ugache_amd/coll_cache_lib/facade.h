@@ -132,6 +132,10 @@ class CollCache : public std::enable_shared_from_this<CollCache> {
     _session_list.at(replica_id)->ExtractPooledAsync64(nodes, seg_off, weights, num_rows, num_nodes, combiner,
                                                        elem_bytes, output, stream);
   }
+  void segment_offsets(int replica_id, const int64_t *sorted_rows, size_t num_entries, size_t num_rows,
+                       int64_t *seg_off, StreamHandle stream) {
+    _session_list.at(replica_id)->SegmentOffsets(sorted_rows, num_entries, num_rows, seg_off, stream);
+  }
   void lookup_wait(int replica_id, StreamHandle stream) { _session_list.at(replica_id)->Wait(stream); }
   std::shared_ptr<ExtractSession> session(int replica_id) { return _session_list.at(replica_id); }
   TensorPtr nid_to_block() { return _nid_to_block; }

@@ -291,6 +291,12 @@ void coll_cache_lookup_pooled_async_i64(int replica_id, const int64_t *key, cons
                                      output, stream);
 }
 
+void coll_cache_segment_offsets(int replica_id, const int64_t *sorted_rows, size_t num_entries, size_t num_rows,
+                                int64_t *seg_off, StreamHandle stream) {
+  CHECK_NOTNULL(_coll_cache);
+  _coll_cache->segment_offsets(replica_id, sorted_rows, num_entries, num_rows, seg_off, stream);
+}
+
 void coll_cache_lookup_wait(int replica_id, StreamHandle stream) {
   CHECK_NOTNULL(_coll_cache);
   _coll_cache->lookup_wait(replica_id, stream);

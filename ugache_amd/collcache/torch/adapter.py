@@ -40,6 +40,7 @@ def coll_torch_create_emb_shm(replica_id, n_keys, dim, dtype, fname=""):
 # what this build adds to the reference's surface
 coll_torch_lookup_unique = c_lib.coll_torch_lookup_unique
 coll_torch_lookup_pooled = c_lib.coll_torch_lookup_pooled
+coll_torch_segment_offsets = c_lib.coll_torch_segment_offsets
 coll_torch_lookup_async = c_lib.coll_torch_lookup_async
 coll_torch_lookup_wait = c_lib.coll_torch_lookup_wait
 coll_torch_forward_config = c_lib.coll_torch_forward_config

@@ -216,6 +216,21 @@ def coll_torch_lookup_pooled(local_id, ids, seg_off, weights=None, combiner="sum
     return out
 
 
+def coll_torch_segment_offsets(local_id, rows, num_rows):
+    """the seg_off coll_torch_lookup_pooled takes, from the row of every entry of a sparse feature in row-major order
+    (extension): a new GPU int64 tensor of num_rows + 1 offsets, seg_off[r] = number of entries whose row is below r.
+    One kernel on torch's current stream, no synchronisation (torch.bincount + cumsum make the same numbers and wait
+    for the device on the way).  rows: GPU int64, ascending, inside [0, num_rows)."""
+    if rows.dtype != torch.int64 or not rows.is_cuda:
+        raise TypeError("rows must be a GPU int64 tensor")
+    dev = _State.dev_id.get(local_id, 0)
+    rows = rows.contiguous().reshape(-1)
+    seg_off = torch.empty(int(num_rows) + 1, dtype=torch.int64, device=rows.device)
+    _C.coll_cache_segment_offsets(local_id, rows.data_ptr() if rows.numel() else None, rows.numel(), int(num_rows),
+                                  seg_off.data_ptr(), _stream_handle(dev))
+    return seg_off
+
+
 def coll_torch_lookup_async(local_id, keys, pad_to_8=True):
     """stream-ordered form of coll_torch_lookup_key_t_val_ret: the batch is enqueued on torch's current stream and
     the call returns without waiting, like any torch op; the returned view of the reused buffer is valid for work

@@ -221,9 +221,7 @@ class SparseLookupLayer(torch.nn.Module):
         if self.fused and max_norm is None and _c_lib.pooled_lookup_supported():
             self.lookup.check(ids)
             num_rows = int(sp_ids.shape[0])
-            counts = torch.bincount(segment_ids, minlength=num_rows)
-            seg_off = torch.zeros(num_rows + 1, dtype=torch.int64, device=ids.device)
-            torch.cumsum(counts, 0, out=seg_off[1:])
+            seg_off = _adapter.coll_torch_segment_offsets(0, segment_ids, num_rows)
             weights = None if sp_weights is None else sp_weights._values().float()
             return _adapter.coll_torch_lookup_pooled(0, ids, seg_off, weights, combiner,
                                                      serving_step=not self.stream_ordered,

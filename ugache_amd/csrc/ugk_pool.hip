@@ -367,6 +367,24 @@ int extract_pool_lpr(ugk_table_t t, const K *ids, const long long *seg_off, cons
   return 0;
 }
 
+// seg_off[r] = the number of entries whose row is below r: thread i writes the offsets of the rows that begin between
+// entry i - 1 and entry i (one when every row has an entry, several across rows without one)
+__global__ __launch_bounds__(kBlock) void segment_offsets_kernel(const long long *__restrict__ rows, size_t nnz,
+                                                                 size_t n_rows, long long *__restrict__ seg_off,
+                                                                 uint32_t *status, uint32_t *host_mirror) {
+  for (size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x; i <= nnz; i += (size_t)gridDim.x * kBlock) {
+    const long long prev = i == 0 ? -1 : rows[i - 1];
+    const long long cur = i == nnz ? (long long)n_rows : rows[i];
+    // entries out of order or outside [0, n_rows): flagged; what is written stays inside seg_off
+    if (cur < prev || cur < 0 || (i > 0 && prev < 0) || (i < nnz && cur >= (long long)n_rows) || prev >= (long long)n_rows) {
+      if (status) atomicOr(status, UGK_ST_BAD_SEGMENT);
+      if (host_mirror) host_mirror[0] = UGK_ST_BAD_SEGMENT;
+      continue;
+    }
+    for (long long r = prev + 1; r <= cur; ++r) seg_off[r] = (long long)i;
+  }
+}
+
 template <typename K>
 int extract_pool(ugk_table_t t, const K *ids, const int64_t *seg_off, const float *weights, size_t n_rows, uint64_t nnz,
                  int combiner, int elem_bytes, const void *cache, uint64_t cache_rows, const void *host,
@@ -414,6 +432,19 @@ int extract_pool(ugk_table_t t, const K *ids, const int64_t *seg_off, const floa
 using namespace ugk;
 
 extern "C" {
+
+int ugk_segment_offsets_i64(const int64_t *sorted_rows_dev, size_t nnz, size_t n_rows, int64_t *seg_off_dev,
+                            uint32_t *status_dev, uint32_t *host_mirror, void *stream) {
+  UGK_REQUIRE(seg_off_dev, "ugk_segment_offsets: null output");
+  UGK_REQUIRE(nnz == 0 || sorted_rows_dev, "ugk_segment_offsets: null rows");
+  UGK_REQUIRE(nnz < ((uint64_t)1 << 62) && n_rows < ((uint64_t)1 << 62), "ugk_segment_offsets: sizes out of range");
+  const unsigned grid = clamp_grid((nnz + 1 + kBlock - 1) / kBlock, 0);
+  hipLaunchKernelGGL(segment_offsets_kernel, dim3(grid), dim3(kBlock), 0, as_stream(stream),
+                     reinterpret_cast<const long long *>(sorted_rows_dev), nnz, n_rows,
+                     reinterpret_cast<long long *>(seg_off_dev), status_dev, host_mirror);
+  UGK_HIP(hipGetLastError());
+  return 0;
+}
 
 int ugk_extract_pool_u32(ugk_table_t t, const uint32_t *ids_dev, const int64_t *seg_off_dev, const float *weights_dev,
                          size_t n_rows, uint64_t nnz, int combiner, int elem_bytes, const void *cache_dev,

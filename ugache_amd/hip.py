@@ -106,6 +106,7 @@ SIGNATURES = {
     "ugk_extract_mix_max_groups": [],
     "ugk_extract_mix_u32": [Table, _vp, _sz, _vp, _u64, _vp, _u64, _vp, _sz, _vp, _vp, _vp, _vp, _u32, _vp],
     "ugk_extract_mix_i64": [Table, _vp, _sz, _vp, _u64, _vp, _u64, _vp, _sz, _vp, _vp, _vp, _vp, _u32, _vp],
+    "ugk_segment_offsets_i64": [_vp, _sz, _sz, _vp, _vp, _vp, _vp],
     "ugk_extract_pool_u32": [Table, _vp, _vp, _vp, _sz, _u64, C.c_int, C.c_int, _vp, _u64, _vp, _u64, _vp, _sz, _vp, _vp,
                              _vp, _vp, _vp],
     "ugk_extract_pool_i64": [Table, _vp, _vp, _vp, _sz, _u64, C.c_int, C.c_int, _vp, _u64, _vp, _u64, _vp, _sz, _vp, _vp,
