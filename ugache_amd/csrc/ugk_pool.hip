@@ -202,8 +202,8 @@ __global__ __launch_bounds__(kBlock) void extract_pool_rows_kernel(ugk_table_t t
     uint32_t len = 0;
     if (sub < n_own) {
       const long long b = seg_off[g0 + sub], e = seg_off[g0 + sub + 1];
-      // a segment outside the ids (or one of 2^28 ids and more: the list of a group is counted in 32 bits): nothing
-      // is read for it, its row is zeros
+      // a segment outside the ids: nothing is read for it, its row is zeros.  (The list of a group is counted in 32
+      // bits; the launcher keeps batches of 2^28 ids and more away from this kernel, so the last test never fires.)
       if (b < 0 || e > nnz || e < b || e - b >= (1ll << 28)) {
         atomicOr(status, UGK_ST_BAD_SEGMENT);
         if (host_mirror) host_mirror[0] = UGK_ST_BAD_SEGMENT;
@@ -341,6 +341,7 @@ int extract_pool_lpr(ugk_table_t t, const K *ids, const long long *seg_off, cons
     const int v = atoi(forced);
     if (v >= 1 && v <= kPoolMaxRows) rows = v;
   }
+  if (nnz >= ((uint64_t)1 << 28)) rows = 1;  // the list of a group is counted in 32 bits
   const size_t rows_per_block = (size_t)rows * groups_per_wave * kWavesPerBlock;
   const unsigned grid = clamp_grid((n_rows + rows_per_block - 1) / rows_per_block, 0);
   if (num_groups) *num_groups = grid;
