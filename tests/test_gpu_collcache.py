@@ -1401,6 +1401,12 @@ def test_serving_stack_from_a_ps_config_file(tmp_path):
                 assert np.allclose(got3, ORC.pool(rows, ids, np.concatenate([[0], np.cumsum(lens)]),
                                                   None if weights is None else w, combiner or "mean"),
                                    rtol=1e-5, atol=1e-5 * np.abs(want).max())
+                # ... enqueued like any torch op instead of being a blocking serving step: the same kernel, same bytes
+                ordered = hps.SparseLookupLayer(model_name="dlrm", table_id=0, emb_vec_size=dim,
+                                                emb_vec_dtype=torch.float32, fused=True, stream_ordered=True)
+                got4 = ordered(sp_ids, weights, combiner=combiner)
+                co.coll_torch_lookup_wait(0)
+                assert got4.cpu().numpy().tobytes() == got3.tobytes()
         with pytest.raises(ValueError):
             sparse(sp_ids, None, combiner="max")
         hps.SetStepProfileValue(profile_type=kLogL1FeatureBytes, value=123.0)

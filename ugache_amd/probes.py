@@ -16,6 +16,10 @@ flagged an error (the parity tests check results).
   pooled    a multi-hot feature through the library: lookup + weighted combination per sample in one call
             (coll_torch_lookup_pooled) against the lookup of all ids followed by torch's index_add_ segment sum, and
             against unique -> lookup -> index_select -> index_add_ (the reference's sparse layer), by ids per sample
+  sparse_layer  the serving stack's SparseLookupLayer end to end (a ps_config file and a model directory written to a
+            temporary folder, Config -> record_hotness -> Init -> layer calls): the reference's steps (unique, lookup,
+            gather, weighted segment sum), the same with the unique inside the library, and lookup + combination in
+            one kernel as a blocking serving step and enqueued like a torch op
 """
 import ctypes as C
 import json
@@ -367,7 +371,73 @@ def probe_pooled(hip, torch, note, quick=False):
                    "the unfused forms use the library's plain lookup and torch ops", "rows": out_rows}
 
 
-PROBES = {"pooled": probe_pooled, "kpw": probe_kpw, "row_span": probe_row_span, "cu_mask": probe_cu_mask, "small_batch": probe_small_batch}
+def probe_sparse_layer(hip, torch, note, quick=False):
+    import shutil
+    import tempfile
+
+    import numpy as np
+
+    import collcache.torch as co
+    import collcache.torch.serving as hps
+
+    rng = np.random.default_rng(1)
+    n_item, dim, calls = (200_000 if quick else 2_000_000), 128, (5 if quick else 30)
+    folder = tempfile.mkdtemp(prefix="ugache_probe_")
+    out_rows = []
+    try:
+        model = os.path.join(folder, "m.model")
+        os.mkdir(model)
+        np.arange(n_item, dtype=np.int64).tofile(os.path.join(model, "key"))
+        rng.standard_normal((n_item, dim), dtype=np.float32).tofile(os.path.join(model, "emb_vector"))
+        cfg = {"iteration_per_epoch": 1000000, "epoch": 1, "coll_cache_enable_refresh": False,
+               "models": [{"model": "dlrm", "sparse_files": [model], "gpucacheper": 0.5, "max_batch_size": 65536,
+                           "deployed_device_list": [0], "maxnum_catfeature_query_per_table_per_sample": [16],
+                           "embedding_vecsize_per_table": [dim], "max_vocabulary_size": [n_item]}]}
+        path = os.path.join(folder, "ps_config.json")
+        with open(path, "w") as f:
+            json.dump(cfg, f)
+        hps.Config(ps_config_file=path)
+        hps.record_hotness(torch.arange(0, n_item // 2, device="cuda"))  # the rows every timed id hits
+        hps.Init(ps_config_file=path, global_batch_size=65536)
+        forms = (("reference_steps", {}), ("unique_in_library", {"unique_in_library": True}),
+                 ("fused_serving_step", {"fused": True}), ("fused_stream_ordered", {"fused": True, "stream_ordered": True}))
+        for n_rows, per in ((65536, 16), (262144, 1), (262144, 4)) if not quick else ((4096, 4),):
+            nnz = n_rows * per
+            seg = torch.arange(n_rows, device="cuda").repeat_interleave(per)
+            col = torch.arange(per, device="cuda").repeat(n_rows)
+            ids = torch.randint(0, n_item // 2, (nnz,), device="cuda")
+            w = torch.rand(nnz, device="cuda") + 0.5
+            ind = torch.stack([seg, col])
+            sp_ids = torch.sparse_coo_tensor(ind, ids, (n_rows, per))
+            sp_w = torch.sparse_coo_tensor(ind, w, (n_rows, per))
+            res, ref = {}, None
+            for name, kw in forms:
+                layer = hps.SparseLookupLayer(model_name="dlrm", table_id=0, emb_vec_size=dim,
+                                              emb_vec_dtype=torch.float32, **kw)
+                got = layer(sp_ids, sp_w, combiner="sum")
+                co.coll_torch_lookup_wait(0)
+                ref = got if ref is None else ref
+                assert torch.allclose(got, ref, rtol=1e-4, atol=1e-4)
+                for _ in range(3):
+                    layer(sp_ids, sp_w, combiner="sum")
+                torch.cuda.synchronize()
+                t0 = time.perf_counter()
+                for _ in range(calls):
+                    layer(sp_ids, sp_w, combiner="sum")
+                torch.cuda.synchronize()
+                res[name] = round((time.perf_counter() - t0) / calls * 1e6, 1)
+                co.coll_torch_lookup_wait(0)
+            out_rows.append({"samples": n_rows, "ids_per_sample": per, "us_per_layer_call": res})
+            note("sparse_layer %d x %d ids: %s" % (n_rows, per, res))
+        hps.Shutdown()
+    finally:
+        shutil.rmtree(folder, ignore_errors=True)
+    return {"probe": "sparse_layer", "table_rows": n_item, "row_bytes": dim * 4, "cache": "half of the rows, every id a hit",
+            "calls_timed": calls, "how": "SparseLookupLayer(sp_ids, sp_weights, combiner='sum') on sparse COO inputs; "
+            "host clock around the calls, one synchronisation at the end", "rows": out_rows}
+
+
+PROBES = {"sparse_layer": probe_sparse_layer, "pooled": probe_pooled, "kpw": probe_kpw, "row_span": probe_row_span, "cu_mask": probe_cu_mask, "small_batch": probe_small_batch}
 
 
 def run(name, quick=False):
