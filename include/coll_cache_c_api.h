@@ -203,6 +203,22 @@ uint32_t coll_cache_place_recorded(int replica_id, uint32_t num_node, double cac
 void coll_cache_forward_config(int enable_refresh, uint64_t refresh_iter, double record_fraction, int periodic);
 void coll_cache_forward(int replica_id, uint32_t *key, size_t num_keys, void *output, StreamHandle stream);
 void coll_cache_forward_i64(int replica_id, const int64_t *key, size_t num_keys, void *output, StreamHandle stream);
+/* A serving step that does not block (no counterpart in the reference: LookupManager::forward returns when the
+ * lookup has): the lookup is enqueued on `stream` like coll_cache_lookup_async* / coll_cache_lookup_pooled_async* and
+ * completed by coll_cache_lookup_wait; the prefix is recorded and the refresh started as in any step.  That needs the
+ * hotness to be counted on the device (COLL_GPU_RECORD=1) or nothing to record (no refresh configured, a
+ * record_fraction of 0): a step whose prefix is counted on the host blocks like coll_cache_forward*, because the
+ * prefix is copied out of the caller's key buffer while the step knows that buffer to be alive. */
+void coll_cache_forward_async(int replica_id, const uint32_t *key, size_t num_keys, void *output,
+                              StreamHandle stream);
+void coll_cache_forward_async_i64(int replica_id, const int64_t *key, size_t num_keys, void *output,
+                                  StreamHandle stream);
+void coll_cache_forward_pooled_async(int replica_id, const uint32_t *key, const int64_t *seg_off,
+                                     const float *weights, size_t num_rows, size_t num_keys, int combiner,
+                                     int elem_bytes, void *output, StreamHandle stream);
+void coll_cache_forward_pooled_async_i64(int replica_id, const int64_t *key, const int64_t *seg_off,
+                                         const float *weights, size_t num_rows, size_t num_keys, int combiner,
+                                         int elem_bytes, void *output, StreamHandle stream);
 /* 1 while a background refresh started by coll_cache_forward runs */
 int coll_cache_forward_refresh_ongoing(void);
 /* waits for it; returns the number of refreshes coll_cache_forward has completed so far */

@@ -131,7 +131,12 @@ int main(int argc, char **argv) {
     coll_cache_forward_config(1, 7, 0.25, 1);
     for (int step = 0; step < std::max(steps / 2, 24); ++step) {
       auto k = skewed_keys(g, 3000, 9000 + (uint64_t)step * 53);
-      coll_cache_forward(0, k.data(), k.size(), out.data(), nullptr);
+      if (step % 3 == 2) {  // a step that is enqueued and left (it blocks where the prefix is counted on the host)
+        coll_cache_forward_async(0, k.data(), k.size(), out.data(), nullptr);
+        coll_cache_lookup_wait(0, nullptr);
+      } else {
+        coll_cache_forward(0, k.data(), k.size(), out.data(), nullptr);
+      }
       bad_rows += check_rows(table, out.data(), k.data(), k.size());
     }
     // 5. pooled lookups (segments of ids combined per sample): plain, as steps of the serving loop, stream-ordered

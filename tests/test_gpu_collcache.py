@@ -789,11 +789,14 @@ def test_hotness_counted_on_the_device_ranks_like_the_host_recorder(pct, impl, d
     assert _basics.C_LIB_CTYPES.coll_cache_rank_hotness(0, None, None, 0) == 0  # drained
 
 
+@pytest.mark.parametrize("stream_ordered", [False, True])
 @pytest.mark.parametrize("gpu_record", [False, True, "and_refresh"])
 @pytest.mark.parametrize("kdtype", [torch.int32, torch.int64])
-def test_serving_loop_records_a_prefix_and_refreshes_in_the_background(gpu_record, kdtype, monkeypatch):
+def test_serving_loop_records_a_prefix_and_refreshes_in_the_background(gpu_record, kdtype, stream_ordered, monkeypatch):
     """LookupManager::forward re-expressed (lookup_manager.cc:158-213): every step records the first share of its
-    batch, looks the batch up, and at step refresh_iter starts a background refresh from what was recorded."""
+    batch, looks the batch up, and at step refresh_iter starts a background refresh from what was recorded.
+    stream_ordered: the steps are enqueued and left (coll_cache_forward_async*; with the hotness counted on the host
+    they block all the same) and must record, look up and refresh exactly like the blocking ones."""
     if gpu_record:
         monkeypatch.setenv("COLL_GPU_RECORD", "1")
     if gpu_record == "and_refresh":  # the background refresh is computed on the device as well
@@ -815,7 +818,10 @@ def test_serving_loop_records_a_prefix_and_refreshes_in_the_background(gpu_recor
     for step in range(7):
         n = 40_000 + 1000 * step
         keys = perm2[zipf_ranks(rng, n, n_item, 1.1)]
-        out = co.coll_torch_forward(0, torch.from_numpy(keys).to(kdtype).cuda(), False)
+        keys_dev = torch.from_numpy(keys).to(kdtype).cuda()
+        out = co.coll_torch_forward(0, keys_dev, False, stream_ordered=stream_ordered)
+        if stream_ordered:
+            co.coll_torch_lookup_wait(0)
         assert out.cpu().numpy().tobytes() == ORC.gather(table, keys.astype(np.int64)).tobytes()
         recorded.append(keys[: int(n * frac)])
         if step < 3:

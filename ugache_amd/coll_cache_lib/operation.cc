@@ -495,9 +495,12 @@ void ForwardJoin() {
   if (_forward.refresh_thread.joinable()) _forward.refresh_thread.join();
 }
 
-// lookup(step_key): the extraction of the step — the plain lookup, or the pooled one
+// lookup(step_key, ordered): the extraction of the step — the plain lookup, or the pooled one; blocking, or
+// (ordered) enqueued on the caller's stream and left.  A step whose recorded prefix is counted on the host blocks
+// whatever the caller asked for: the prefix is copied out of the caller's buffer while the step knows it to be alive.
 template <typename KeyT, typename LookupFn>
-void ForwardStep(int replica_id, const KeyT *key, size_t num_keys, StreamHandle stream, const LookupFn &lookup) {
+void ForwardStep(int replica_id, const KeyT *key, size_t num_keys, StreamHandle stream, bool stream_ordered,
+                 const LookupFn &lookup) {
   CHECK_NOTNULL(_coll_cache);
   CHECK_EQ(replica_id, 0);
   ForwardState &fw = _forward;
@@ -510,7 +513,7 @@ void ForwardStep(int replica_id, const KeyT *key, size_t num_keys, StreamHandle 
   }
   const uint64_t step_key = steps[replica_id] * RunConfig::num_device + replica_id;
   steps[replica_id]++;
-  lookup(step_key);
+  lookup(step_key, stream_ordered && (RunConfig::gpu_record || num_record == 0));
   if (RunConfig::gpu_record)
     session->SetRecordLimit(SIZE_MAX);
   else if (num_record > 0)
@@ -547,21 +550,41 @@ void coll_cache_forward_config(int enable_refresh, uint64_t refresh_iter, double
 }
 
 void coll_cache_forward(int replica_id, uint32_t *key, size_t num_keys, void *output, StreamHandle stream) {
-  ForwardStep<IdType>(replica_id, key, num_keys, stream, [&](uint64_t step_key) {
+  ForwardStep<IdType>(replica_id, key, num_keys, stream, false, [&](uint64_t step_key, bool) {
     _coll_cache->lookup(replica_id, key, num_keys, output, stream, step_key);
   });
 }
 
 void coll_cache_forward_i64(int replica_id, const int64_t *key, size_t num_keys, void *output, StreamHandle stream) {
-  ForwardStep<Id64Type>(replica_id, key, num_keys, stream, [&](uint64_t step_key) {
+  ForwardStep<Id64Type>(replica_id, key, num_keys, stream, false, [&](uint64_t step_key, bool) {
     _coll_cache->lookup64(replica_id, key, num_keys, output, stream, step_key);
+  });
+}
+
+void coll_cache_forward_async(int replica_id, const uint32_t *key, size_t num_keys, void *output,
+                              StreamHandle stream) {
+  ForwardStep<IdType>(replica_id, key, num_keys, stream, true, [&](uint64_t step_key, bool ordered) {
+    if (ordered)
+      _coll_cache->lookup_async(replica_id, key, num_keys, output, stream);
+    else
+      _coll_cache->lookup(replica_id, key, num_keys, output, stream, step_key);
+  });
+}
+
+void coll_cache_forward_async_i64(int replica_id, const int64_t *key, size_t num_keys, void *output,
+                                  StreamHandle stream) {
+  ForwardStep<Id64Type>(replica_id, key, num_keys, stream, true, [&](uint64_t step_key, bool ordered) {
+    if (ordered)
+      _coll_cache->lookup_async64(replica_id, key, num_keys, output, stream);
+    else
+      _coll_cache->lookup64(replica_id, key, num_keys, output, stream, step_key);
   });
 }
 
 void coll_cache_forward_pooled(int replica_id, const uint32_t *key, const int64_t *seg_off, const float *weights,
                                size_t num_rows, size_t num_keys, int combiner, int elem_bytes, void *output,
                                StreamHandle stream) {
-  ForwardStep<IdType>(replica_id, key, num_keys, stream, [&](uint64_t step_key) {
+  ForwardStep<IdType>(replica_id, key, num_keys, stream, false, [&](uint64_t step_key, bool) {
     _coll_cache->lookup_pooled(replica_id, key, seg_off, weights, num_rows, num_keys, combiner, elem_bytes, output,
                                stream, step_key);
   });
@@ -570,9 +593,35 @@ void coll_cache_forward_pooled(int replica_id, const uint32_t *key, const int64_
 void coll_cache_forward_pooled_i64(int replica_id, const int64_t *key, const int64_t *seg_off, const float *weights,
                                    size_t num_rows, size_t num_keys, int combiner, int elem_bytes, void *output,
                                    StreamHandle stream) {
-  ForwardStep<Id64Type>(replica_id, key, num_keys, stream, [&](uint64_t step_key) {
+  ForwardStep<Id64Type>(replica_id, key, num_keys, stream, false, [&](uint64_t step_key, bool) {
     _coll_cache->lookup_pooled64(replica_id, key, seg_off, weights, num_rows, num_keys, combiner, elem_bytes, output,
                                  stream, step_key);
+  });
+}
+
+void coll_cache_forward_pooled_async(int replica_id, const uint32_t *key, const int64_t *seg_off,
+                                     const float *weights, size_t num_rows, size_t num_keys, int combiner,
+                                     int elem_bytes, void *output, StreamHandle stream) {
+  ForwardStep<IdType>(replica_id, key, num_keys, stream, true, [&](uint64_t step_key, bool ordered) {
+    if (ordered)
+      _coll_cache->lookup_pooled_async(replica_id, key, seg_off, weights, num_rows, num_keys, combiner, elem_bytes,
+                                       output, stream);
+    else
+      _coll_cache->lookup_pooled(replica_id, key, seg_off, weights, num_rows, num_keys, combiner, elem_bytes, output,
+                                 stream, step_key);
+  });
+}
+
+void coll_cache_forward_pooled_async_i64(int replica_id, const int64_t *key, const int64_t *seg_off,
+                                         const float *weights, size_t num_rows, size_t num_keys, int combiner,
+                                         int elem_bytes, void *output, StreamHandle stream) {
+  ForwardStep<Id64Type>(replica_id, key, num_keys, stream, true, [&](uint64_t step_key, bool ordered) {
+    if (ordered)
+      _coll_cache->lookup_pooled_async64(replica_id, key, seg_off, weights, num_rows, num_keys, combiner, elem_bytes,
+                                         output, stream);
+    else
+      _coll_cache->lookup_pooled64(replica_id, key, seg_off, weights, num_rows, num_keys, combiner, elem_bytes,
+                                   output, stream, step_key);
   });
 }
 

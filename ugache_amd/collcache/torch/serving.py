@@ -163,6 +163,9 @@ class LookupLayer(torch.nn.Module):
         self.table_id = table_id
         self.emb_vec_size = emb_vec_size
         self.emb_vec_dtype = emb_vec_dtype
+        # stream_ordered=True (extension): the step is enqueued on torch's current stream like any torch op (it still
+        # blocks while the hotness of its prefix is counted on the host, i.e. without COLL_GPU_RECORD=1)
+        self.stream_ordered = bool(kwargs.get("stream_ordered", False))
 
     def check(self, inputs):
         """the configuration's say on a batch of keys (model, table, width, key type, size)"""
@@ -182,7 +185,7 @@ class LookupLayer(torch.nn.Module):
 
     def forward(self, inputs):
         self.check(inputs)
-        emb = _adapter.coll_torch_forward(0, inputs.reshape(-1), False)
+        emb = _adapter.coll_torch_forward(0, inputs.reshape(-1), False, stream_ordered=self.stream_ordered)
         return emb.reshape(tuple(inputs.shape) + (self.emb_vec_size,))
 
 
@@ -202,8 +205,8 @@ class SparseLookupLayer(torch.nn.Module):
         # fused=True: lookup and combination in one kernel of the library (coll_torch_lookup_pooled) wherever that
         # kernel can take the call (no max_norm, rows it supports); the steps below otherwise
         self.fused = bool(kwargs.get("fused", False))
-        # stream_ordered=True (with fused): the call is enqueued on torch's current stream like any torch op instead of
-        # being a blocking step of the serving loop
+        # stream_ordered=True (with fused): the step is enqueued on torch's current stream like any torch op (it still
+        # blocks while the hotness of its prefix is counted on the host, i.e. without COLL_GPU_RECORD=1)
         self.stream_ordered = bool(kwargs.get("stream_ordered", False))
 
     def forward(self, sp_ids, sp_weights=None, name=None, combiner=None, max_norm=None):
@@ -223,8 +226,7 @@ class SparseLookupLayer(torch.nn.Module):
             num_rows = int(sp_ids.shape[0])
             seg_off = _adapter.coll_torch_segment_offsets(0, segment_ids, num_rows)
             weights = None if sp_weights is None else sp_weights._values().float()
-            return _adapter.coll_torch_lookup_pooled(0, ids, seg_off, weights, combiner,
-                                                     serving_step=not self.stream_ordered,
+            return _adapter.coll_torch_lookup_pooled(0, ids, seg_off, weights, combiner, serving_step=True,
                                                      stream_ordered=self.stream_ordered)
         if self.unique_in_library:  # unique + lookup in one call, the unique by the library's GPU hash set
             self.lookup.check(ids)
