@@ -75,8 +75,12 @@ __device__ __forceinline__ void store_off_meta(ugk_bucket_t *b, uint32_t off, ui
 // first never-used bucket), but only once the whole sequence up to that never-used bucket has been seen not to hold the
 // key already: a tombstone in front of a live copy of the key must not hide it.  With tombstones piling up between
 // rebuilds that walk is tens of buckets long, which one lane per key did as a chain of dependent 16-byte loads (462 k
-// keys into a 71 M-bucket table with 13 % tombstones: 207 us).  Keys of one launch are distinct, so the only contest is
-// for buckets; a group that loses one starts its walk again.
+// keys into a 71 M-bucket table with 13 % tombstones: 207 us; the groups: 87 us).  One lane per key reading a whole
+// line per step (eight loads in flight) was measured too: 99 us for the insert, 75 instead of 88 us for the evict
+// below — what is left is a device-scope atomic per key (the CAS here, the slot bitmap there): a kernel that does
+// little else than one such atomic per key takes 44 us for the same 462 k keys, whatever walk comes in front of it.
+// Keys of one launch are distinct,
+// so the only contest is for buckets; a group that loses one starts its walk again.
 template <typename K>
 __global__ __launch_bounds__(kBlock) void hash_insert_kernel(ugk_bucket_t *table, uint64_t nb, const K *keys,
                                                              const uint32_t *offs, uint32_t seq_base, uint32_t loc,
