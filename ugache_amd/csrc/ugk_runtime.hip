@@ -196,7 +196,14 @@ int ugk_stream_sync(void *stream) {
 int ugk_stream_is_capturing(void *stream, int *capturing) {
   UGK_REQUIRE(capturing, "ugk_stream_is_capturing: null output");
   hipStreamCaptureStatus st = hipStreamCaptureStatusNone;
-  UGK_HIP(hipStreamIsCapturing(as_stream(stream), &st));
+  if (hipStreamIsCapturing(as_stream(stream), &st) != hipSuccess) {
+    // the query itself is refused where it would touch a capture (the default stream while another stream of the
+    // process records in global mode): then work enqueued here would be refused too, which is what "capturing" means
+    // to the callers
+    (void)hipGetLastError();
+    *capturing = 1;
+    return 0;
+  }
   *capturing = st != hipStreamCaptureStatusNone;
   return 0;
 }
