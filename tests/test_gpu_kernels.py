@@ -748,7 +748,8 @@ def test_pooled_extraction_hand_worked(rows_per_group, monkeypatch):
         pin.free()
 
 
-@pytest.mark.parametrize("n_rows,nnz", [(1, 0), (1, 1), (5, 0), (7, 3), (1000, 1000), (5000, 60_000), (300_000, 40_000)])
+@pytest.mark.parametrize("n_rows,nnz", [(1, 0), (1, 1), (5, 0), (7, 3), (1000, 1000), (5000, 60_000), (300_000, 40_000),
+                                        (3_000_000, 5), (1_000_000, 0), (200, 129)])
 def test_segment_offsets_match_searchsorted(n_rows, nnz):
     """ugk_segment_offsets_i64: seg_off[r] = number of entries whose row is below r (rows without an entry among them)"""
     rng = np.random.default_rng(n_rows + nnz)

@@ -368,21 +368,36 @@ int extract_pool_lpr(ugk_table_t t, const K *ids, const long long *seg_off, cons
   return 0;
 }
 
-// seg_off[r] = the number of entries whose row is below r: thread i writes the offsets of the rows that begin between
-// entry i - 1 and entry i (one when every row has an entry, several across rows without one)
+// seg_off[r] = the number of entries whose row is below r: lane i owns the offsets of the rows that begin between
+// entry i - 1 and entry i.  That is one offset where every row has an entry, which the lane writes itself; a run of
+// rows without entries is written by the whole wavefront, 64 offsets a step.
 __global__ __launch_bounds__(kBlock) void segment_offsets_kernel(const long long *__restrict__ rows, size_t nnz,
                                                                  size_t n_rows, long long *__restrict__ seg_off,
                                                                  uint32_t *status, uint32_t *host_mirror) {
-  for (size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x; i <= nnz; i += (size_t)gridDim.x * kBlock) {
-    const long long prev = i == 0 ? -1 : rows[i - 1];
-    const long long cur = i == nnz ? (long long)n_rows : rows[i];
-    // entries out of order or outside [0, n_rows): flagged; what is written stays inside seg_off
-    if (cur < prev || cur < 0 || (i > 0 && prev < 0) || (i < nnz && cur >= (long long)n_rows) || prev >= (long long)n_rows) {
-      if (status) atomicOr(status, UGK_ST_BAD_SEGMENT);
-      if (host_mirror) host_mirror[0] = UGK_ST_BAD_SEGMENT;
-      continue;
+  const size_t stride = (size_t)gridDim.x * kBlock;
+  const int lane = (int)lane_id();
+  for (size_t base = (size_t)blockIdx.x * kBlock + threadIdx.x - lane; base <= nnz; base += stride) {  // wavefront-uniform
+    const size_t i = base + lane;
+    long long prev = 0, cur = -1;  // an empty run for the lanes past the end
+    if (i <= nnz) {
+      prev = i == 0 ? -1 : rows[i - 1];
+      cur = i == nnz ? (long long)n_rows : rows[i];
+      // entries out of order or outside [0, n_rows): flagged; what is written stays inside seg_off
+      if (cur < prev || cur < 0 || (i > 0 && prev < 0) || (i < nnz && cur >= (long long)n_rows) ||
+          prev >= (long long)n_rows) {
+        if (status) atomicOr(status, UGK_ST_BAD_SEGMENT);
+        if (host_mirror) host_mirror[0] = UGK_ST_BAD_SEGMENT;
+        prev = 0, cur = -1;
+      }
     }
-    for (long long r = prev + 1; r <= cur; ++r) seg_off[r] = (long long)i;
+    const long long first = prev + 1, count = cur - prev;  // rows first .. first + count - 1 begin at entry i
+    if (count == 1) seg_off[first] = (long long)i;
+    for (unsigned long long runs = __ballot(count > 1); runs != 0ull; runs &= runs - 1ull) {
+      const int src = __ffsll((long long)runs) - 1;
+      const long long f = (long long)shfl64((uint64_t)first, src), c = (long long)shfl64((uint64_t)count, src);
+      const long long at = (long long)(base + src);
+      for (long long r = lane; r < c; r += kWave) seg_off[f + r] = at;
+    }
   }
 }
 
