@@ -279,6 +279,30 @@ def test_fp16_table_and_small_rows():
     assert out[:10_001].cpu().numpy().tobytes() == ORC.gather(table, q.astype(np.int64)).tobytes()
 
 
+@pytest.mark.parametrize("pct", [1.0, 0.2, 0.0])
+def test_bfloat16_table_is_looked_up_as_its_bytes(pct):
+    """a bfloat16 table (an extension: the reference's adapter knows float32 and float16) moves through the library as
+    two-byte elements; lookups return bfloat16 and the table's bytes.  The pooled lookup does not combine bfloat16."""
+    rng = np.random.default_rng(19)
+    n_item, dim = 20_000, 48
+    co.config(make_config(n_item, pct))
+    co.coll_cache_record_init(0)
+    co.coll_torch_record(0, torch.from_numpy(rng.integers(0, n_item, size=60_000)).to(torch.int32))
+    emb = co.coll_torch_create_emb_shm(0, n_item, dim, torch.bfloat16)
+    raw = emb.view(torch.int16).numpy()
+    raw[...] = rng.integers(-32768, 32768, size=raw.shape, dtype=np.int16)
+    co.coll_torch_init_t(0, 0, emb, pct)
+    q = rng.integers(0, n_item, size=9_999)
+    keys = torch.from_numpy(q).cuda()
+    out = co.coll_torch_lookup_key_t_val_ret(0, keys, False)
+    assert out.dtype == torch.bfloat16 and out.shape == (len(q), dim)
+    assert out.view(torch.int16).cpu().numpy().tobytes() == raw[q].tobytes()
+    a = co.coll_torch_lookup_async(0, keys, False).clone()
+    co.coll_torch_lookup_wait(0)
+    assert a.view(torch.int16).cpu().numpy().tobytes() == raw[q].tobytes()
+    assert not co.c_lib.pooled_lookup_supported()
+
+
 @pytest.mark.parametrize("dim,dtype", [(3, torch.float32), (5, torch.float16), (1, torch.float32), (7, torch.float32)])
 @pytest.mark.parametrize("pct", [0.2, 1.0, 0.0])
 def test_rows_that_are_not_multiples_of_16_bytes(dim, dtype, pct):

@@ -61,13 +61,15 @@ def _stream_handle(dev_id):
     return ctypes.c_void_p(torch.cuda.current_stream(dev_id).cuda_stream)
 
 
-def _setup_dims(dim, use_fp16):
+def _setup_dims(dim, use_fp16, dtype=None):
+    """use_fp16: elements of two bytes (the reference's flag, adapter.cc:126-190); dtype says which two-byte type the
+    lookups return (float16 unless the table is bfloat16, which the library moves as the same bytes)"""
     _State.external_feat_dim = dim
     if use_fp16:
         if dim % 2 != 0:
             sys.stderr.write("dimension must be even\n")
             os.abort()
-        _State.external_dtype = torch.float16
+        _State.external_dtype = dtype if dtype is not None else torch.float16
         _State.internal_feat_dim = dim // 2
     else:
         _State.external_dtype = torch.float32
@@ -79,11 +81,11 @@ def coll_torch_init_t(replica_id, dev_id, emb, cache_percentage):
     torch.cuda.set_device(dev_id)
     _State.dev_id[replica_id] = dev_id
     alloc, release = _make_allocator(dev_id)
-    use_fp16 = emb.dtype == torch.float16
+    use_fp16 = emb.dtype in (torch.float16, torch.bfloat16)  # two-byte elements: the same bytes to the library
     if not use_fp16 and emb.dtype != torch.float32:
-        raise TypeError("embedding table must be float32 or float16, got %s" % emb.dtype)
+        raise TypeError("embedding table must be float32, float16 or bfloat16, got %s" % emb.dtype)
     dim = emb.size(1)
-    _setup_dims(dim, use_fp16)
+    _setup_dims(dim, use_fp16, emb.dtype if use_fp16 else None)
     info_keys = emb.size(0)
     _C.coll_cache_init_c(replica_id, info_keys, alloc, release, None, emb.data_ptr(), kF16 if use_fp16 else kF32, dim,
                          float(cache_percentage), _stream_handle(dev_id))
@@ -131,7 +133,7 @@ def _lookup_into_reused_buffer(local_id, keys, pad_to_8, fn32, fn64):
             _State.batch_emb_reuse = torch.empty((max(max_num_keys, 1) * _State.internal_feat_dim * 4,),
                                                  dtype=torch.int8, device="cuda:%d" % dev)
             _State.out_views.clear()  # they pointed into the old buffer
-        elem = 2 if _State.external_dtype == torch.float16 else 4
+        elem = 4 if _State.external_dtype == torch.float32 else 2
         tensor = _State.batch_emb_reuse[: padded_len * _State.external_feat_dim * elem].view(
             _State.external_dtype).view(padded_len, _State.external_feat_dim)
         if len(_State.out_views) < 64:
@@ -173,7 +175,7 @@ COMBINERS = {"sum": 0, "mean": 1, "sqrtn": 2}
 def pooled_lookup_supported():
     """whether coll_torch_lookup_pooled can take the rows of the table that was built (a multiple of 16 bytes, at
     most 4096; fp32 or fp16 elements)"""
-    elem = 2 if _State.external_dtype == torch.float16 else 4
+    elem = 4 if _State.external_dtype == torch.float32 else 2
     row_bytes = _State.external_feat_dim * elem
     return _State.external_dtype in (torch.float32, torch.float16) and row_bytes % 16 == 0 and 0 < row_bytes <= 4096
 
@@ -282,7 +284,7 @@ def coll_torch_record(local_id, keys):
         _C.coll_cache_record(local_id, keys.data_ptr(), keys.numel())
 
 
-_ELEM = {torch.float32: 4, torch.float16: 2, torch.float64: 8, torch.int32: 4, torch.int64: 8, torch.uint8: 1,
+_ELEM = {torch.float32: 4, torch.float16: 2, torch.bfloat16: 2, torch.float64: 8, torch.int32: 4, torch.int64: 8, torch.uint8: 1,
          torch.int8: 1}
 
 
