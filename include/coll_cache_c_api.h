@@ -95,7 +95,8 @@ size_t coll_cache_lookup_unique_i64(int replica_id, const int64_t *key, size_t n
  * embedding_lookup_sparse).  Segment r = key[seg_off[r] .. seg_off[r + 1]); output[r, :] = sum of weights[j] x row(key[j])
  * over the segment (weights NULL: 1), as it is (combiner 0 "sum"), divided by the sum of the weights (1 "mean") or by
  * the root of the sum of their squares (2 "sqrtn"); a zero denominator or an empty segment gives a zero row.  Elements
- * are fp32 (elem_bytes 4) or fp16 (elem_bytes 2: the rows of a table configured as half), added in fp32 in the order of
+ * are fp32 (elem_bytes 4), fp16 (elem_bytes 2: the rows of a table configured as half) or bfloat16 (elem_bytes 0x102,
+ * UGK_ELEM_BF16 of ugache_hip.h: such a table is configured as half too), added in fp32 in the order of
  * the ids.  key, seg_off (num_rows + 1 ascending int64 offsets, the last one num_keys), weights: device memory;
  * output: device [num_rows, dim], caller-allocated; blocking, like coll_cache_lookup.  Rows must be a multiple of 16
  * bytes and at most 4096 bytes long.  coll_cache_last_group_offset afterwards counts keys, not output rows. */

@@ -34,6 +34,9 @@ extern "C" {
 #define UGK_ST_EVICT_ABSENT 0x8u     /* evict of a key that is not present */
 #define UGK_ST_BAD_SEGMENT 0x10u     /* pooled extraction: offsets that leave [0, nnz] or run backwards: row of zeros */
 
+/* element code of the pooled extraction for bfloat16 rows (fp32 and fp16 are named by their size, 4 and 2) */
+#define UGK_ELEM_BF16 0x102
+
 /* ---- locations (cache_context.cu:2421-2422: GPUs are 0..G-1, the host is G; here G = 1) ---------- */
 #define UGK_LOC_LOCAL 0u
 #define UGK_LOC_HOST 1u
@@ -90,7 +93,7 @@ typedef struct {
 const char *ugk_last_error(void);
 /* version of this ABI; bumped on any signature change.  ugk_abi_version() is what the loaded library was built with:
  * a caller compiled against another UGK_ABI_VERSION must not go on. */
-#define UGK_ABI_VERSION 15
+#define UGK_ABI_VERSION 16
 int ugk_abi_version(void);
 
 /* ---- runtime plumbing: Device::{AllocDataSpace,FreeDataSpace,CopyDataFromTo,StreamSync,CreateStream}
@@ -277,7 +280,8 @@ int ugk_extract_mix_i64(ugk_table_t t, const int64_t *keys_dev, size_t n, const 
  *             = sum_j w_j x_j / sum_j w_j                       combiner 1 (mean)
  *             = sum_j w_j x_j / sqrt(sum_j w_j^2)               combiner 2 (sqrtn)
  * with w_j = weights_dev[j] (1 when weights_dev is NULL), a zero denominator giving a zero row (div_no_nan), an empty
- * segment a zero row.  Elements are fp32 (elem_bytes 4) or fp16 (2) and are added in fp32 in the order of the ids, one
+ * segment a zero row.  Elements are fp32 (elem_bytes 4), fp16 (2) or bfloat16 (UGK_ELEM_BF16: two bytes as well) and
+ * are added in fp32 in the order of the ids, one
  * fused multiply-add each; the output has the element type of the rows.  The nnz x row_bytes intermediate of a lookup
  * followed by a segment sum is never written.  seg_off_dev: n_rows + 1 ascending offsets into ids_dev, the last one
  * nnz.  row_bytes: a multiple of 16, at most 4096.  Status, host mirror and the per-workgroup count words are those of

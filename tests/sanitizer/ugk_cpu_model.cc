@@ -395,7 +395,10 @@ int extract_pool(ugk_table_t t, const K *ids, const int64_t *seg_off, const floa
   if (num_groups) *num_groups = 0;
   if (n_rows == 0) return 0;
   REQUIRE(seg_off && out && status && (nnz == 0 || ids), "ugk_extract_pool: null pointer");
-  REQUIRE(combiner >= 0 && combiner <= 2 && (elem_bytes == 2 || elem_bytes == 4), "ugk_extract_pool: bad argument");
+  REQUIRE(combiner >= 0 && combiner <= 2 && (elem_bytes == 2 || elem_bytes == 4 || elem_bytes == UGK_ELEM_BF16),
+          "ugk_extract_pool: bad argument");
+  const bool bf16 = elem_bytes == UGK_ELEM_BF16;
+  elem_bytes &= 0xf;
   REQUIRE(rb > 0 && rb % 16 == 0 && rb <= 4096, "ugk_extract_pool: rows of %zu bytes", rb);
   if (t.kind != 0 && check_table(t, "ugk_extract_pool")) return 1;
   const size_t dim = rb / elem_bytes;
@@ -435,7 +438,12 @@ int extract_pool(ugk_table_t t, const K *ids, const int64_t *seg_off, const floa
         else {
           uint16_t h;
           memcpy(&h, row + c * 2, 2);
-          x = half_to_float(h);
+          if (bf16) {
+            const uint32_t u = (uint32_t)h << 16;
+            memcpy(&x, &u, 4);
+          } else {
+            x = half_to_float(h);
+          }
         }
         acc[c] = std::fma(w, x, acc[c]);
       }
@@ -445,7 +453,15 @@ int extract_pool(ugk_table_t t, const K *ids, const int64_t *seg_off, const floa
       const float y = denom != 0.f ? acc[c] / denom : 0.f;
       if (elem_bytes == 4) memcpy((char *)out + (r * dim + c) * 4, &y, 4);
       else {
-        const uint16_t h = float_to_half(y);
+        uint16_t h;
+        if (bf16) {
+          uint32_t u;
+          memcpy(&u, &y, 4);
+          h = (u & 0x7fffffffu) > 0x7f800000u ? (uint16_t)((u >> 16) | 0x40u)
+                                              : (uint16_t)((u + 0x7fffu + ((u >> 16) & 1u)) >> 16);
+        } else {
+          h = float_to_half(y);
+        }
         memcpy((char *)out + (r * dim + c) * 2, &h, 2);
       }
     }

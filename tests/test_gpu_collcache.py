@@ -282,7 +282,8 @@ def test_fp16_table_and_small_rows():
 @pytest.mark.parametrize("pct", [1.0, 0.2, 0.0])
 def test_bfloat16_table_is_looked_up_as_its_bytes(pct):
     """a bfloat16 table (an extension: the reference's adapter knows float32 and float16) moves through the library as
-    two-byte elements; lookups return bfloat16 and the table's bytes.  The pooled lookup does not combine bfloat16."""
+    two-byte elements; lookups return bfloat16 and the table's bytes.  The pooled lookup adds bfloat16 rows in fp32 and
+    rounds the result to bfloat16 (8 bits: 2^-8 of the result on top of 1e-5 of the terms' magnitude)."""
     rng = np.random.default_rng(19)
     n_item, dim = 20_000, 48
     co.config(make_config(n_item, pct))
@@ -300,7 +301,25 @@ def test_bfloat16_table_is_looked_up_as_its_bytes(pct):
     a = co.coll_torch_lookup_async(0, keys, False).clone()
     co.coll_torch_lookup_wait(0)
     assert a.view(torch.int16).cpu().numpy().tobytes() == raw[q].tobytes()
-    assert not co.c_lib.pooled_lookup_supported()
+    assert co.c_lib.pooled_lookup_supported()
+    vals = (raw.astype(np.int64) & 0xffff).astype(np.uint32) << np.uint32(16)
+    with np.errstate(all="ignore"):
+        vals = vals.view(np.float32).astype(np.float64)
+    lens = rng.choice([0, 1, 3, 8], size=2_000)
+    off = np.concatenate([[0], np.cumsum(lens)]).astype(np.int64)
+    ids = rng.integers(0, n_item, size=int(off[-1]))
+    w = rng.uniform(0.1, 2.0, size=len(ids)).astype(np.float32)
+    got = co.coll_torch_lookup_pooled(0, torch.from_numpy(ids).cuda(), torch.from_numpy(off).cuda(),
+                                      torch.from_numpy(w).cuda(), "mean")
+    assert got.dtype == torch.bfloat16
+    with np.errstate(all="ignore"):
+        want = ORC.pool(vals, ids, off, w, "mean")
+        mag_sum = ORC.pool(np.abs(vals), ids, off, w, "sum")
+        mag = ORC.pool(np.abs(vals), ids, off, w, "mean")
+    ok = np.isfinite(mag_sum) & (mag_sum < 1e36)  # random bit patterns: NaNs, infinities and sums that overflow aside
+    bound = 1e-5 * np.where(ok, mag, 0.0) + 2.0 ** -8 * np.abs(np.where(ok, want, 0.0)) + 1e-37
+    got64 = got.float().cpu().numpy().astype(np.float64)
+    assert not (ok & ~(np.abs(got64 - np.where(ok, want, 0.0)) <= bound)).any()
 
 
 @pytest.mark.parametrize("dim,dtype", [(3, torch.float32), (5, torch.float16), (1, torch.float32), (7, torch.float32)])

@@ -592,11 +592,25 @@ def _pool_reference(table_f64, ids, seg_off, weights, combiner):
     return np.where(den[:, None] != 0, out / safe[:, None], 0.0)
 
 
+def _bf16_bits(a32):
+    """float32 values cut to bfloat16 bit patterns (uint16)"""
+    return (np.ascontiguousarray(a32, np.float32).view(np.uint32) >> np.uint32(16)).astype(np.uint16)
+
+
+def _bf16_values(bits):
+    return (bits.astype(np.uint32) << np.uint32(16)).view(np.float32)
+
+
+_POOL_SHAPES = [(4, np.float32), (32, np.float32), (128, np.float32), (512, np.float32), (1024, np.float32),
+                (8, np.float16), (64, np.float16), (256, np.float16), (2048, np.float16), (64, "bf16"), (256, "bf16")]
+# every shape with the rows per lane group the launch picks, some of them with three and eight rows forced
+_POOL_CASES = [(d, e, "") for d, e in _POOL_SHAPES] + [
+    (d, e, r) for r in ("3", "8") for d, e in [(32, np.float32), (512, np.float32), (64, np.float16), (2048, np.float16),
+                                               (64, "bf16")]]
+
+
 @pytest.mark.parametrize("kind", ["none", "flat", "hash"])
-@pytest.mark.parametrize("dim,etype", [(4, np.float32), (32, np.float32), (128, np.float32), (512, np.float32),
-                                       (1024, np.float32), (8, np.float16), (64, np.float16), (256, np.float16),
-                                       (2048, np.float16)])
-@pytest.mark.parametrize("rows_per_group", ["", "3", "8"])
+@pytest.mark.parametrize("dim,etype,rows_per_group", _POOL_CASES)
 def test_pooled_extraction_matches_a_float64_segment_sum(kind, dim, etype, rows_per_group, monkeypatch):
     """ugk_extract_pool_*: rows looked up and combined per segment in one kernel (sum, mean, sqrtn; with and without
     weights, negative and zero ones among them; segments that are empty, single, longer than a lane group; three
@@ -608,9 +622,17 @@ def test_pooled_extraction_matches_a_float64_segment_sum(kind, dim, etype, rows_
         monkeypatch.setenv("UGK_POOL_ROWS", rows_per_group)
     rng = np.random.default_rng(dim + len(kind))
     nkeys = 20_000
-    rb = dim * np.dtype(etype).itemsize
-    host = rng.standard_normal((nkeys, dim)).astype(etype)
-    host_bytes = host.view(np.uint8).reshape(nkeys, rb)
+    bf16 = isinstance(etype, str)
+    esize = 2 if bf16 else np.dtype(etype).itemsize
+    ecode = hip.ELEM_BF16 if bf16 else esize
+    rb = dim * esize
+    if bf16:  # numpy has no bfloat16: the table is its bit patterns, the values are those patterns widened
+        host_bits = _bf16_bits(rng.standard_normal((nkeys, dim)))
+        host = _bf16_values(host_bits)
+        host_bytes = host_bits.view(np.uint8).reshape(nkeys, rb)
+    else:
+        host = rng.standard_normal((nkeys, dim)).astype(etype)
+        host_bytes = host.view(np.uint8).reshape(nkeys, rb)
     if kind == "none":  # no table: the id is the row, the "host" table may be anywhere (here HBM)
         tb = hip.table(0, None, 0)
         cached = np.zeros(0, np.int64)
@@ -648,14 +670,17 @@ def test_pooled_extraction_matches_a_float64_segment_sum(kind, dim, etype, rows_
                     out = dev_bytes(n_rows * rb, fill=0x7F)
                     groups = C.c_uint32(0)
                     hip.call("ugk_extract_pool_i64", tb, ptr(d_ids), ptr(d_off), None if weights is None else ptr(d_w),
-                             n_rows, nnz, combiner, np.dtype(etype).itemsize, ptr(d_cache), len(cached), pin.ptr, nkeys,
+                             n_rows, nnz, combiner, ecode, ptr(d_cache), len(cached), pin.ptr, nkeys,
                              ptr(out), rb, ptr(st), mirror.ptr, words.ptr, C.byref(groups), None)
                     sync()
                     assert status_value(st) == 0
                     w = words.array[:groups.value]
                     n_local = int(is_cached[ids].sum())
                     assert [int((w & np.uint64(0xFFFFFFFF)).sum()), int((w >> np.uint64(32)).sum())] == [n_local, nnz - n_local]
-                    got = to_np(out)[: n_rows * rb].view(etype).reshape(n_rows, dim).astype(np.float64)
+                    if bf16:
+                        got = _bf16_values(to_np(out)[: n_rows * rb].view(np.uint16)).reshape(n_rows, dim).astype(np.float64)
+                    else:
+                        got = to_np(out)[: n_rows * rb].view(etype).reshape(n_rows, dim).astype(np.float64)
                     want = _pool_reference(f64, ids, seg_off, weights, combiner)
                     # fp32 adds of n terms are off by at most n 2^-24 of the terms' magnitudes; an fp16 output is
                     # rounded to 11 bits on top.  (A mean over signed weights that nearly cancel is large and still
@@ -674,6 +699,8 @@ def test_pooled_extraction_matches_a_float64_segment_sum(kind, dim, etype, rows_
                             mag = mag + np.abs(want) * np.where(den != 0, sum_abs / np.where(den != 0, den, 1.0), 0.0)
                     # (fp16 results below 2^-14 are subnormal: steps of 2^-24 whatever their size)
                     bound = 1e-5 * mag + (1e-3 * np.abs(want) + 2.0 ** -25 if etype == np.float16 else 0.0) + 1e-30
+                    if bf16:  # a bfloat16 result is rounded to 8 bits
+                        bound = bound + 2.0 ** -8 * np.abs(want)
                     if etype == np.float16:  # a mean over weights that nearly cancel may leave fp16's range
                         big = np.abs(want) > 6.0e4
                         assert np.isinf(got[big & (np.abs(want) > 6.6e4)]).all()

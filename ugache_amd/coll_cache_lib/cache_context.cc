@@ -1052,8 +1052,9 @@ bool ExtractSession::LaunchPooled(const KeyT *nodes, const int64_t *seg_off, con
   CHECK_NOTNULL(output);
   CHECK(num_nodes == 0 || nodes != nullptr);
   CHECK(combiner >= 0 && combiner <= 2) << "combiner is 0 (sum), 1 (mean) or 2 (sqrtn)";
-  CHECK(elem_bytes == 2 || elem_bytes == 4) << "rows are combined as fp16 or fp32 elements";
-  CHECK(rb % 16 == 0 && rb <= 4096 && rb % elem_bytes == 0)
+  CHECK(elem_bytes == 2 || elem_bytes == 4 || elem_bytes == UGK_ELEM_BF16)
+      << "rows are combined as fp32 (4), fp16 (2) or bfloat16 (UGK_ELEM_BF16) elements";
+  CHECK(rb % 16 == 0 && rb <= 4096 && rb % (elem_bytes & 0xf) == 0)
       << "pooled lookups take rows of a multiple of 16 bytes up to 4096, not " << rb;
   NoteOutput(output, num_rows * rb);
   // without a table the id is the row and everything comes from the one source there is (HBM for a full cache, the

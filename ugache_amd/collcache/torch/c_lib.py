@@ -174,10 +174,14 @@ COMBINERS = {"sum": 0, "mean": 1, "sqrtn": 2}
 
 def pooled_lookup_supported():
     """whether coll_torch_lookup_pooled can take the rows of the table that was built (a multiple of 16 bytes, at
-    most 4096; fp32 or fp16 elements)"""
+    most 4096; fp32, fp16 or bfloat16 elements)"""
     elem = 4 if _State.external_dtype == torch.float32 else 2
     row_bytes = _State.external_feat_dim * elem
-    return _State.external_dtype in (torch.float32, torch.float16) and row_bytes % 16 == 0 and 0 < row_bytes <= 4096
+    return _State.external_dtype in _POOL_ELEM and row_bytes % 16 == 0 and 0 < row_bytes <= 4096
+
+
+# element codes of the pooled lookup: the size for fp32 and fp16, UGK_ELEM_BF16 for bfloat16
+_POOL_ELEM = {torch.float32: 4, torch.float16: 2, torch.bfloat16: 0x102}
 
 
 def coll_torch_lookup_pooled(local_id, ids, seg_off, weights=None, combiner="sum", serving_step=False,
@@ -194,7 +198,8 @@ def coll_torch_lookup_pooled(local_id, ids, seg_off, weights=None, combiner="sum
     run; coll_torch_lookup_wait reports a bad id or offset and makes the group sizes available)."""
     dev = _State.dev_id.get(local_id, 0)
     if not pooled_lookup_supported():
-        raise ValueError("pooled lookups need rows of a multiple of 16 bytes, at most 4096, of fp32 or fp16 elements")
+        raise ValueError("pooled lookups need rows of a multiple of 16 bytes, at most 4096, of fp32, fp16 or bfloat16 "
+                         "elements")
     if ids.dtype not in (torch.int32, torch.int64, torch.uint32) or not ids.is_cuda:
         raise TypeError("ids must be a GPU tensor of int32 / uint32 or int64")
     if seg_off.dtype != torch.int64 or not seg_off.is_cuda or seg_off.dim() != 1 or seg_off.numel() < 1:
@@ -216,7 +221,7 @@ def coll_torch_lookup_pooled(local_id, ids, seg_off, weights=None, combiner="sum
         fn = _C.coll_cache_lookup_pooled_i64 if ids.dtype == torch.int64 else _C.coll_cache_lookup_pooled
     fn(local_id, ids.data_ptr() if ids.numel() else None, seg_off.data_ptr(),
        None if weights is None else weights.data_ptr(), n_rows, ids.numel(), COMBINERS[combiner],
-       2 if _State.external_dtype == torch.float16 else 4, out.data_ptr(), _stream_handle(dev))
+       _POOL_ELEM[_State.external_dtype], out.data_ptr(), _stream_handle(dev))
     return out
 
 

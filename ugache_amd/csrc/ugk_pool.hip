@@ -18,35 +18,56 @@ namespace {
 // intermediate of a lookup followed by a segment sum is never written or read back.  A group of LPR lanes owns an
 // output row: its lanes resolve LPR of the row's ids at a time (the table lookup is the fused extraction's), then
 // every id's row is read once, 16 bytes per lane and chunk, and added in fp32 in the order of the ids.
+// the elements of a 16-byte chunk as floats and back.  `bf16` picks between the two two-byte formats at run time (a
+// wavefront-uniform branch), so that bfloat16 rows cost no kernels of their own.
 template <typename E>
 struct PoolElem;
 template <>
 struct PoolElem<float> {
   static constexpr int kPerChunk = 4;
-  static __device__ __forceinline__ void unpack(const u32x4 &v, float *x) {
+  static __device__ __forceinline__ void unpack(const u32x4 &v, float *x, bool) {
     x[0] = __uint_as_float(v.x), x[1] = __uint_as_float(v.y), x[2] = __uint_as_float(v.z), x[3] = __uint_as_float(v.w);
   }
-  static __device__ __forceinline__ u32x4 pack(const float *x) {
+  static __device__ __forceinline__ u32x4 pack(const float *x, bool) {
     return u32x4{__float_as_uint(x[0]), __float_as_uint(x[1]), __float_as_uint(x[2]), __float_as_uint(x[3])};
   }
 };
+// round to nearest even; NaN stays NaN
+__device__ __forceinline__ uint32_t float_to_bf16_bits(float f) {
+  const uint32_t u = __float_as_uint(f);
+  if ((u & 0x7fffffffu) > 0x7f800000u) return (u >> 16) | 0x40u;
+  return (u + 0x7fffu + ((u >> 16) & 1u)) >> 16;
+}
 template <>
 struct PoolElem<__half> {
   static constexpr int kPerChunk = 8;
-  static __device__ __forceinline__ void unpack(const u32x4 &v, float *x) {
+  static __device__ __forceinline__ void unpack(const u32x4 &v, float *x, bool bf16) {
     const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+    if (bf16) {
 #pragma unroll
-    for (int k = 0; k < 4; ++k) {
-      x[2 * k] = __half2float(__ushort_as_half((unsigned short)(w[k] & 0xffffu)));
-      x[2 * k + 1] = __half2float(__ushort_as_half((unsigned short)(w[k] >> 16)));
+      for (int k = 0; k < 4; ++k) {
+        x[2 * k] = __uint_as_float(w[k] << 16);
+        x[2 * k + 1] = __uint_as_float(w[k] & 0xffff0000u);
+      }
+    } else {
+#pragma unroll
+      for (int k = 0; k < 4; ++k) {
+        x[2 * k] = __half2float(__ushort_as_half((unsigned short)(w[k] & 0xffffu)));
+        x[2 * k + 1] = __half2float(__ushort_as_half((unsigned short)(w[k] >> 16)));
+      }
     }
   }
-  static __device__ __forceinline__ u32x4 pack(const float *x) {
+  static __device__ __forceinline__ u32x4 pack(const float *x, bool bf16) {
     uint32_t w[4];
+    if (bf16) {
 #pragma unroll
-    for (int k = 0; k < 4; ++k)
-      w[k] = (uint32_t)__half_as_ushort(__float2half(x[2 * k])) |
-             ((uint32_t)__half_as_ushort(__float2half(x[2 * k + 1])) << 16);
+      for (int k = 0; k < 4; ++k) w[k] = float_to_bf16_bits(x[2 * k]) | (float_to_bf16_bits(x[2 * k + 1]) << 16);
+    } else {
+#pragma unroll
+      for (int k = 0; k < 4; ++k)
+        w[k] = (uint32_t)__half_as_ushort(__float2half(x[2 * k])) |
+               ((uint32_t)__half_as_ushort(__float2half(x[2 * k + 1])) << 16);
+    }
     return u32x4{w[0], w[1], w[2], w[3]};
   }
 };
@@ -60,7 +81,7 @@ __global__ __launch_bounds__(kBlock) void extract_pool_kernel(ugk_table_t t, con
                                                               long long nnz, const u32x4 *__restrict__ cache,
                                                               uint64_t cache_rows,
                                                               const u32x4 *__restrict__ host, uint64_t host_rows,
-                                                              u32x4 *__restrict__ out, uint32_t vpr, int combiner,
+                                                              u32x4 *__restrict__ out, uint32_t vpr, int combiner, bool bf16,
                                                               uint32_t *status, uint32_t *host_mirror,
                                                               unsigned long long *counts) {
   constexpr int RPW = kWave / LPR;  // output rows per wavefront and pass
@@ -127,7 +148,7 @@ __global__ __launch_bounds__(kBlock) void extract_pool_kernel(ugk_table_t t, con
 #pragma unroll
             for (int u = 0; u < U; ++u) {
               float x[EPC];
-              PoolElem<E>::unpack(v[u], x);
+              PoolElem<E>::unpack(v[u], x, bf16);
               if (ok[u]) {
 #pragma unroll
                 for (int e = 0; e < EPC; ++e) acc[c][e] = fmaf(wv[u], x[e], acc[c][e]);
@@ -149,7 +170,7 @@ __global__ __launch_bounds__(kBlock) void extract_pool_kernel(ugk_table_t t, con
           float y[EPC];
 #pragma unroll
           for (int e = 0; e < EPC; ++e) y[e] = denom != 0.f ? acc[c][e] / denom : 0.f;  // div_no_nan
-          out[r * vpr + col] = PoolElem<E>::pack(y);
+          out[r * vpr + col] = PoolElem<E>::pack(y, bf16);
         }
       }
     }
@@ -175,7 +196,7 @@ __global__ __launch_bounds__(kBlock) void extract_pool_rows_kernel(ugk_table_t t
                                                               long long nnz, int rows_per_group,
                                                               const u32x4 *__restrict__ cache, uint64_t cache_rows,
                                                               const u32x4 *__restrict__ host, uint64_t host_rows,
-                                                              u32x4 *__restrict__ out, uint32_t vpr, int combiner,
+                                                              u32x4 *__restrict__ out, uint32_t vpr, int combiner, bool bf16,
                                                               uint32_t *status, uint32_t *host_mirror,
                                                               unsigned long long *counts) {
   constexpr int RPW = kWave / LPR;  // lane groups per wavefront
@@ -235,7 +256,7 @@ __global__ __launch_bounds__(kBlock) void extract_pool_rows_kernel(ugk_table_t t
       float y[EPC];
 #pragma unroll
       for (int e = 0; e < EPC; ++e) y[e] = denom != 0.f ? acc[c][e] / denom : 0.f, acc[c][e] = 0.f;
-      out[(g0 + k) * vpr + col] = PoolElem<E>::pack(y);
+      out[(g0 + k) * vpr + col] = PoolElem<E>::pack(y, bf16);
     };
     for (uint32_t f0 = 0; __ballot(f0 < total) != 0ull; f0 += LPR) {  // until every group of the wavefront is through
       const uint32_t f = f0 + sub;
@@ -280,7 +301,7 @@ __global__ __launch_bounds__(kBlock) void extract_pool_rows_kernel(ugk_table_t t
 #pragma unroll
             for (int u = 0; u < U; ++u) {
               float x[EPC];
-              PoolElem<E>::unpack(v[u], x);
+              PoolElem<E>::unpack(v[u], x, bf16);
               if (m[u] & 0x200) {
                 for (const int ku = m[u] & 0xff; cc < ku; ++cc, ws = 0.f) flush(c, col, cc, ws);
                 if (m[u] & 0x100) {
@@ -319,7 +340,7 @@ __global__ __launch_bounds__(kBlock) void extract_pool_rows_kernel(ugk_table_t t
 template <typename K, int KIND, typename E>
 int extract_pool_lpr(ugk_table_t t, const K *ids, const long long *seg_off, const float *weights, size_t n_rows,
                      const void *cache, uint64_t cache_rows, const void *host, uint64_t host_rows, void *out,
-                     uint32_t vpr, uint64_t nnz, int combiner, uint32_t *status, uint32_t *host_mirror,
+                     uint32_t vpr, uint64_t nnz, int combiner, bool bf16, uint32_t *status, uint32_t *host_mirror,
                      uint64_t *counts, uint32_t *num_groups, hipStream_t st) {
   // Lanes per output row: rows of up to 512 bytes go to 8 lanes of up to four chunks each (eight lane groups per
   // wavefront; with 32 lanes and two groups 65,536 samples of 16 ids took 123 us instead of 112 us), rows of up to
@@ -349,12 +370,12 @@ int extract_pool_lpr(ugk_table_t t, const K *ids, const long long *seg_off, cons
   if (rows == 1)                                                                                                       \
     hipLaunchKernelGGL((extract_pool_kernel<K, KIND, L, E>), dim3(grid), dim3(kBlock), 0, st, t, ids, seg_off,         \
                        weights, n_rows, (long long)nnz, (const u32x4 *)cache, cache_rows, (const u32x4 *)host,         \
-                       host_rows, (u32x4 *)out, vpr, combiner, status, host_mirror,                                    \
+                       host_rows, (u32x4 *)out, vpr, combiner, bf16, status, host_mirror,                              \
                        reinterpret_cast<unsigned long long *>(counts));                                                \
   else                                                                                                                 \
     hipLaunchKernelGGL((extract_pool_rows_kernel<K, KIND, L, E>), dim3(grid), dim3(kBlock), 0, st, t, ids, seg_off,    \
                        weights, n_rows, (long long)nnz, rows, (const u32x4 *)cache, cache_rows, (const u32x4 *)host,   \
-                       host_rows, (u32x4 *)out, vpr, combiner, status, host_mirror,                                    \
+                       host_rows, (u32x4 *)out, vpr, combiner, bf16, status, host_mirror,                              \
                        reinterpret_cast<unsigned long long *>(counts))
   if (lpr == 8) {
     UGK_POOL(8);
@@ -413,7 +434,9 @@ int extract_pool(ugk_table_t t, const K *ids, const int64_t *seg_off, const floa
   UGK_REQUIRE(nnz <= (uint64_t)INT64_MAX, "ugk_extract_pool: %llu ids", (unsigned long long)nnz);
   UGK_REQUIRE((uintptr_t)counts % 8 == 0, "ugk_extract_pool: the count words must be 8-byte aligned");
   UGK_REQUIRE(combiner >= 0 && combiner <= 2, "ugk_extract_pool: combiner %d is not sum(0), mean(1) or sqrtn(2)", combiner);
-  UGK_REQUIRE(elem_bytes == 4 || elem_bytes == 2, "ugk_extract_pool: elements of %d bytes are not fp32 or fp16", elem_bytes);
+  UGK_REQUIRE(elem_bytes == 4 || elem_bytes == 2 || elem_bytes == UGK_ELEM_BF16,
+              "ugk_extract_pool: element code %d is not fp32 (4), fp16 (2) or bfloat16 (UGK_ELEM_BF16)", elem_bytes);
+  const bool bf16 = elem_bytes == UGK_ELEM_BF16;
   UGK_REQUIRE(t.kind == 0 || t.kind == 1 || t.kind == 2, "ugk_extract_pool: table kind %d", t.kind);
   if (t.kind != 0) UGK_REQUIRE(t.table && t.size, "ugk_extract_pool: empty table");
   if (t.kind == 2)
@@ -431,10 +454,10 @@ int extract_pool(ugk_table_t t, const K *ids, const int64_t *seg_off, const floa
   hipStream_t st = as_stream(stream);
 #define UGK_POOL_KIND(KIND)                                                                                          \
   (elem_bytes == 4 ? extract_pool_lpr<K, KIND, float>(t, ids, so, weights, n_rows, cache, cache_rows, host, host_rows, \
-                                                      out, vpr, nnz, combiner, status, host_mirror, counts,           \
+                                                      out, vpr, nnz, combiner, false, status, host_mirror, counts,    \
                                                       num_groups, st)                                                 \
                    : extract_pool_lpr<K, KIND, __half>(t, ids, so, weights, n_rows, cache, cache_rows, host,          \
-                                                       host_rows, out, vpr, nnz, combiner, status, host_mirror,       \
+                                                       host_rows, out, vpr, nnz, combiner, bf16, status, host_mirror, \
                                                        counts, num_groups, st))
   if (t.kind == 0) return UGK_POOL_KIND(0);
   if (t.kind == 1) return UGK_POOL_KIND(1);

@@ -14,6 +14,7 @@ ST_TABLE_FULL = 0x2
 ST_DUP_KEY = 0x4
 ST_EVICT_ABSENT = 0x8
 ST_BAD_SEGMENT = 0x10
+ELEM_BF16 = 0x102
 
 LOC_LOCAL = 0
 LOC_HOST = 1
