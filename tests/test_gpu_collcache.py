@@ -41,7 +41,7 @@ def make_config(num_total_item, pct, threads=8):
 
 @pytest.fixture(autouse=True)
 def _fresh_cache(monkeypatch):
-    for v in ("COLL_HASH_TABLE", "SAMGRAPH_COLL_CACHE_CONCURRENT_LINK_IMPL", "SAMGRAPH_COLL_CACHE_NO_GROUP",
+    for v in ("COLL_HASH_TABLE", "COLL_RECORD_INLINE_BYTES", "SAMGRAPH_COLL_CACHE_CONCURRENT_LINK_IMPL", "SAMGRAPH_COLL_CACHE_NO_GROUP",
               "COLL_DEDUP_KEYS", "COLL_DEDUP_MIN_KEYS", "COLL_GPU_RECORD", "COLL_GPU_RECORD_EVERY", "COLL_GPU_REFRESH",
               "COLL_GPU_REFRESH_KEEP", "COLL_GPU_REFRESH_STABLE", "COLL_REFRESH_RATE_GBPS",
               "COLL_GPU_RECORD_SEED"):
@@ -844,6 +844,8 @@ def test_serving_loop_records_a_prefix_and_refreshes_in_the_background(gpu_recor
         monkeypatch.setenv("COLL_GPU_RECORD", "1")
     if gpu_record == "and_refresh":  # the background refresh is computed on the device as well
         monkeypatch.setenv("COLL_GPU_REFRESH", "1")
+    if stream_ordered:  # ... and the prefixes counted on the host are counted by the step itself, not by the thread
+        monkeypatch.setenv("COLL_RECORD_INLINE_BYTES", str(1 << 20))
     monkeypatch.setenv("COLL_REFRESH_SLEEP_US", "100")
     rng = np.random.default_rng(44)
     n_item, dim, pct, frac = 30_000, 32, 0.2, 0.5

@@ -32,6 +32,7 @@ def _run(exe, table, refresh, steps):
     else:  # the device-side counters start from the build's ranking, and the background copy is paced by a rate
         env["COLL_GPU_RECORD_SEED"] = "1"
         env["COLL_REFRESH_RATE_GBPS"] = "0.5"
+        env["COLL_RECORD_INLINE_BYTES"] = "0"  # every recorded prefix goes through the recorder's thread
     env["ASAN_OPTIONS"] = "detect_leaks=1:abort_on_error=0"
     env["UBSAN_OPTIONS"] = "print_stacktrace=1:halt_on_error=1"
     env["TSAN_OPTIONS"] = "halt_on_error=0:second_deadlock_stack=1"

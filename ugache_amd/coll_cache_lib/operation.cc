@@ -485,6 +485,12 @@ struct ForwardState {
   std::atomic<bool> refresh_ongoing{false};
   std::atomic<uint64_t> refreshes_done{0};
   RecordWorker recorder;  // the host-record path
+  // A small recorded prefix does not go through the recorder's thread: a copy kernel in front of the lookup, on the
+  // lookup's stream, leaves it in this pinned buffer, and the step counts it itself once the blocking lookup has
+  // returned.  Waking the thread and waiting for it cost a serving-sized batch more than its whole lookup
+  // (1,024 keys: 55 us per step against 12 us for the lookup alone).
+  void *inline_prefix = nullptr;
+  size_t inline_prefix_bytes = 0;
   ~ForwardState() {
     if (refresh_thread.joinable()) refresh_thread.join();  // a process that exits without coll_cache_shutdown
   }
@@ -506,18 +512,32 @@ void ForwardStep(int replica_id, const KeyT *key, size_t num_keys, StreamHandle 
   ForwardState &fw = _forward;
   auto session = _coll_cache->session(replica_id);
   const size_t num_record = fw.enable_refresh ? (size_t)(num_keys * fw.record_fraction) : 0;
+  const size_t record_bytes = num_record * sizeof(KeyT);
+  const bool inline_prefix = !RunConfig::gpu_record && num_record > 0 &&
+                             record_bytes <= RunConfig::record_inline_bytes &&
+                             reinterpret_cast<uintptr_t>(key) % 16 == 0;
   if (RunConfig::gpu_record) {
     session->SetRecordLimit(num_record);  // counted by the lookup itself
+  } else if (inline_prefix) {
+    if (fw.inline_prefix_bytes < RunConfig::record_inline_bytes) {
+      if (fw.inline_prefix) UGK_CALL(ugk_host_free(fw.inline_prefix));
+      UGK_CALL(ugk_host_malloc(&fw.inline_prefix, RunConfig::record_inline_bytes));
+      fw.inline_prefix_bytes = RunConfig::record_inline_bytes;
+    }
+    UGK_CALL(ugk_copy_rows(fw.inline_prefix, key, record_bytes, stream));  // complete when the lookup behind it is
   } else if (num_record > 0) {
     fw.recorder.Post(replica_id, session->DeviceId(), key, num_record, sizeof(KeyT), stream);  // counted while the lookup runs
   }
   const uint64_t step_key = steps[replica_id] * RunConfig::num_device + replica_id;
   steps[replica_id]++;
   lookup(step_key, stream_ordered && (RunConfig::gpu_record || num_record == 0));
-  if (RunConfig::gpu_record)
+  if (RunConfig::gpu_record) {
     session->SetRecordLimit(SIZE_MAX);
-  else if (num_record > 0)
+  } else if (inline_prefix) {
+    _freq_recorder[replica_id]->Record(static_cast<const KeyT *>(fw.inline_prefix), num_record);
+  } else if (num_record > 0) {
     fw.recorder.Wait();
+  }
   const bool due = fw.enable_refresh && fw.refresh_iter > 0 &&
                    (fw.periodic ? (fw.step > 0 && fw.step % fw.refresh_iter == 0) : fw.step == fw.refresh_iter);
   if (due) {
@@ -735,6 +755,11 @@ uint32_t coll_cache_place_recorded(int replica_id, uint32_t num_node, double cac
 void coll_cache_shutdown(void) {
   ForwardJoin();
   _forward.recorder.Stop();
+  if (_forward.inline_prefix) {
+    UGK_CALL(ugk_host_free(_forward.inline_prefix));
+    _forward.inline_prefix = nullptr;
+    _forward.inline_prefix_bytes = 0;
+  }
   _forward.enable_refresh = false;
   _forward.step = 0;
   _forward.refreshes_done.store(0);

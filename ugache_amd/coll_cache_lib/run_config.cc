@@ -1,5 +1,6 @@
 #include "run_config.h"
 
+#include <algorithm>
 #include <cstdlib>
 
 #include "logging.h"
@@ -36,6 +37,7 @@ size_t RunConfig::refresh_batch_rows = 4092;
 unsigned RunConfig::refresh_sleep_us = 3000;
 unsigned RunConfig::refresh_limit_block = 20;
 double RunConfig::refresh_rate_gbps = 0;
+size_t RunConfig::record_inline_bytes = 64 << 10;
 double RunConfig::hash_rebuild_tombstone_frac = 0.15;
 bool RunConfig::gpu_record = false;
 size_t RunConfig::gpu_record_every = 1;
@@ -79,6 +81,7 @@ void RunConfig::LoadConfigFromEnv() {
   refresh_sleep_us = 3000;
   refresh_limit_block = 20;
   refresh_rate_gbps = 0;
+  record_inline_bytes = 64 << 10;
   refresher_omp_thread_num = 8;
   hash_rebuild_tombstone_frac = 0.15;
   dedup_keys = false;
@@ -121,6 +124,8 @@ void RunConfig::LoadConfigFromEnv() {
   if (GetEnv("COLL_REFRESH_SLEEP_US") != "") refresh_sleep_us = std::stoul(GetEnv("COLL_REFRESH_SLEEP_US"));
   if (GetEnv("COLL_REFRESH_LIMIT_BLOCK") != "") refresh_limit_block = std::stoul(GetEnv("COLL_REFRESH_LIMIT_BLOCK"));
   if (GetEnv("COLL_REFRESH_RATE_GBPS") != "") refresh_rate_gbps = std::stod(GetEnv("COLL_REFRESH_RATE_GBPS"));
+  if (GetEnv("COLL_RECORD_INLINE_BYTES") != "")
+    record_inline_bytes = std::min<size_t>(std::stoul(GetEnv("COLL_RECORD_INLINE_BYTES")), (size_t)16 << 20);
   if (GetEnv("COLL_GPU_RECORD") != "") gpu_record = GetEnv("COLL_GPU_RECORD") != "0";
   if (GetEnv("COLL_GPU_REFRESH") != "") gpu_refresh = GetEnv("COLL_GPU_REFRESH") != "0";
   if (GetEnv("COLL_GPU_REFRESH_KEEP") != "") gpu_refresh_keep = GetEnv("COLL_GPU_REFRESH_KEEP") != "0";

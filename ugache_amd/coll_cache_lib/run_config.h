@@ -66,6 +66,9 @@ struct RunConfig {
   // COLL_REFRESH_RATE_GBPS, default 0 = off: instead of the fixed sleep, a background refresh sleeps after each batch
   // for as long as keeps its copy over the host link at this many GB/s on average
   static double refresh_rate_gbps;
+  // COLL_RECORD_INLINE_BYTES: a serving step counts a recorded prefix of up to this many bytes itself (a copy kernel in
+  // front of the lookup, counted after it) instead of handing it to the recorder's thread; 0 = always the thread
+  static size_t record_inline_bytes;
   static bool gpu_record;          // COLL_GPU_RECORD=1: every lookup counts its keys in device-side hotness counters
   static size_t gpu_record_every;  // COLL_GPU_RECORD_EVERY, default 1: ... only every n-th lookup
   // COLL_GPU_REFRESH=1 (with COLL_GPU_RECORD=1): a refresh whose hotness was all counted on the device ranks, places

@@ -296,6 +296,47 @@ def probe_small_batch(hip, torch, note, quick=False):
                  % (label, n, blocking, ordered, replayed))
             del keys, out, outs, graph
         co.coll_torch_shutdown()
+    # serving steps (a 5 % prefix recorded, a refresh configured but far away) at the same sizes: the prefix copied to
+    # the host and counted there by the recorder's thread (the default; such a step blocks whatever is asked for), or
+    # counted on the device, where a step can also be enqueued and left
+    for gpu_record in (False, True):
+        if gpu_record:
+            os.environ["COLL_GPU_RECORD"] = "1"
+        try:
+            co.config({"cache_percentage": 0.5, "_cache_policy": co.kCollCacheAsymmLink, "num_device": 1,
+                       "num_global_step_per_epoch": 10, "num_epoch": 1, "num_total_item": rows, "omp_thread_num": 8})
+            co.coll_cache_record_init(0)
+            co.coll_torch_record(0, torch.arange(0, rows // 2, dtype=torch.int32))
+            emb = co.coll_torch_create_emb_shm(0, rows, dim, torch.float32)
+            emb.normal_(generator=torch.Generator().manual_seed(1))
+            co.coll_torch_init_t(0, 0, emb, 0.5)
+            Cl.coll_cache_forward_config(1, 10 ** 12, 0.05, 0)
+            for n in sizes:
+                keys = torch.randint(0, rows // 2, (8, n), device="cuda", dtype=torch.int64)
+                ptrs = [keys[i].data_ptr() for i in range(8)]
+                out = torch.empty((n, dim), dtype=torch.float32, device="cuda")
+                torch.cuda.synchronize()
+                res = {}
+                for name, fn in (("blocking", Cl.coll_cache_forward_i64), ("stream_ordered", Cl.coll_cache_forward_async_i64)):
+                    for i in range(20):
+                        fn(0, ptrs[i % 8], n, out.data_ptr(), stream)
+                    Cl.coll_cache_lookup_wait(0, stream)
+                    t0 = time.perf_counter()
+                    for i in range(calls):
+                        fn(0, ptrs[i % 8], n, out.data_ptr(), stream)
+                    Cl.coll_cache_lookup_wait(0, stream)
+                    res[name] = round((time.perf_counter() - t0) / calls * 1e6, 2)
+                assert torch.equal(out.cpu(), emb[keys[(calls - 1) % 8].cpu()])
+                label = "serving step, prefix counted on the %s" % ("device" if gpu_record else "host")
+                out_rows.append({"path": label, "keys": n, "us_per_blocking_call": res["blocking"],
+                                 "us_per_stream_ordered_call": res["stream_ordered"]})
+                note("small_batch %s, %d keys: blocking %.1f us, stream-ordered %.1f us"
+                     % (label, n, res["blocking"], res["stream_ordered"]))
+                del keys, out
+            Cl.coll_cache_forward_config(0, 0, 0.0, 0)
+            co.coll_torch_shutdown()
+        finally:
+            os.environ.pop("COLL_GPU_RECORD", None)
     return {"probe": "small_batch", "table_rows": rows, "row_bytes": dim * 4, "calls_timed": calls,
             "how": "coll_cache_lookup_i64 / coll_cache_lookup_async_i64 (+ one coll_cache_lookup_wait) over 8 cycled "
                    "batches of uniformly random keys that all hit, host clock around the calls; the graph holds 26 "
