@@ -199,8 +199,10 @@ uint32_t coll_cache_place_recorded(int replica_id, uint32_t num_node, double cac
  * recorded, a prefix of the batch (the reference records the first 5 %: 0.05); periodic != 0 starts a refresh every
  * refresh_iter steps instead of once at step refresh_iter.
  * coll_cache_forward_*: one step = record the prefix (on the device when COLL_GPU_RECORD=1, else a copy of the prefix
- * to the host and coll_cache_record), blocking lookup, and at the configured step a refresh started on a background
- * thread (skipped with a log line while the previous one still runs).  output as in coll_cache_lookup. */
+ * to the host and coll_cache_record: by a thread of the library beside the lookup, or, for a prefix of up to
+ * COLL_RECORD_INLINE_BYTES = 64 KB, by a kernel in front of the lookup and the calling thread after it), blocking
+ * lookup, and at the configured step a refresh started on a background thread (skipped with a log line while the
+ * previous one still runs).  output as in coll_cache_lookup. */
 void coll_cache_forward_config(int enable_refresh, uint64_t refresh_iter, double record_fraction, int periodic);
 void coll_cache_forward(int replica_id, uint32_t *key, size_t num_keys, void *output, StreamHandle stream);
 void coll_cache_forward_i64(int replica_id, const int64_t *key, size_t num_keys, void *output, StreamHandle stream);
