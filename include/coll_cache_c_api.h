@@ -208,10 +208,12 @@ void coll_cache_forward(int replica_id, uint32_t *key, size_t num_keys, void *ou
 void coll_cache_forward_i64(int replica_id, const int64_t *key, size_t num_keys, void *output, StreamHandle stream);
 /* A serving step that does not block (no counterpart in the reference: LookupManager::forward returns when the
  * lookup has): the lookup is enqueued on `stream` like coll_cache_lookup_async* / coll_cache_lookup_pooled_async* and
- * completed by coll_cache_lookup_wait; the prefix is recorded and the refresh started as in any step.  That needs the
- * hotness to be counted on the device (COLL_GPU_RECORD=1) or nothing to record (no refresh configured, a
- * record_fraction of 0): a step whose prefix is counted on the host blocks like coll_cache_forward*, because the
- * prefix is copied out of the caller's key buffer while the step knows that buffer to be alive. */
+ * completed by coll_cache_lookup_wait; the prefix is recorded and the refresh started as in any step.  Where the
+ * hotness is counted on the host, a prefix of up to COLL_RECORD_INLINE_BYTES is copied into pinned memory by a kernel
+ * on `stream` and counted later — by a later step that finds the copy complete, or by whatever needs the counts (a
+ * ranking, coll_cache_lookup_wait, coll_cache_shutdown), which waits for it; a longer prefix makes the step block like
+ * coll_cache_forward*, because it is copied out of the caller's key buffer while the step knows that buffer to be
+ * alive.  A step that is being recorded into a HIP graph records no prefix. */
 void coll_cache_forward_async(int replica_id, const uint32_t *key, size_t num_keys, void *output,
                               StreamHandle stream);
 void coll_cache_forward_async_i64(int replica_id, const int64_t *key, size_t num_keys, void *output,

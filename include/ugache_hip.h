@@ -93,7 +93,7 @@ typedef struct {
 const char *ugk_last_error(void);
 /* version of this ABI; bumped on any signature change.  ugk_abi_version() is what the loaded library was built with:
  * a caller compiled against another UGK_ABI_VERSION must not go on. */
-#define UGK_ABI_VERSION 16
+#define UGK_ABI_VERSION 17
 int ugk_abi_version(void);
 
 /* ---- runtime plumbing: Device::{AllocDataSpace,FreeDataSpace,CopyDataFromTo,StreamSync,CreateStream}
@@ -130,6 +130,8 @@ int ugk_event_create(void **event);
 int ugk_event_destroy(void *event);
 int ugk_event_record(void *event, void *stream);
 int ugk_event_sync(void *event);
+/* *complete = 1 if the work in front of the event's last record has finished, else 0; never waits */
+int ugk_event_query(void *event, int *complete);
 int ugk_stream_wait_event(void *stream, void *event);
 int ugk_event_elapsed_ms(void *start, void *stop, float *ms);
 /* async copy, direction inferred from the pointers */

@@ -608,6 +608,10 @@ int ugk_event_record(void *event, void *) {
   return 0;
 }
 int ugk_event_sync(void *) { return 0; }
+int ugk_event_query(void *, int *complete) {
+  *complete = 1;
+  return 0;
+}
 int ugk_stream_wait_event(void *, void *) { return 0; }
 int ugk_event_elapsed_ms(void *start, void *stop, float *ms) {
   REQUIRE(start && stop && ms, "null event");

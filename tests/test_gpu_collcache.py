@@ -838,8 +838,9 @@ def test_hotness_counted_on_the_device_ranks_like_the_host_recorder(pct, impl, d
 def test_serving_loop_records_a_prefix_and_refreshes_in_the_background(gpu_record, kdtype, stream_ordered, monkeypatch):
     """LookupManager::forward re-expressed (lookup_manager.cc:158-213): every step records the first share of its
     batch, looks the batch up, and at step refresh_iter starts a background refresh from what was recorded.
-    stream_ordered: the steps are enqueued and left (coll_cache_forward_async*; with the hotness counted on the host
-    they block all the same) and must record, look up and refresh exactly like the blocking ones."""
+    stream_ordered: the steps are enqueued and left (coll_cache_forward_async*; a prefix counted on the host is counted
+    later, by a later step, the wait or the ranking) and must record, look up and refresh exactly like the blocking
+    ones."""
     if gpu_record:
         monkeypatch.setenv("COLL_GPU_RECORD", "1")
     if gpu_record == "and_refresh":  # the background refresh is computed on the device as well
@@ -887,6 +888,37 @@ def test_serving_loop_records_a_prefix_and_refreshes_in_the_background(gpu_recor
             assert _basics.last_group_offset(0)[1] == int((new_nid[keys] == 0).sum())
     assert co.coll_torch_forward_join() == 1  # not periodic: one refresh only
     # plain lookups count whole batches again
+    co.coll_torch_forward_config(False, 0, frac, False)
+
+
+@pytest.mark.parametrize("kdtype", [torch.int32, torch.int64])
+def test_stream_ordered_serving_steps_count_their_prefixes_later(kdtype):
+    """coll_cache_forward_async* with the hotness counted on the host: thirty steps enqueued back to back without a
+    wait (more than the library has buffers for waiting prefixes); every step's prefix has been counted once
+    coll_cache_lookup_wait returns, and the outputs are the table's rows."""
+    rng = np.random.default_rng(61)
+    n_item, dim, pct, frac = 20_000, 32, 0.3, 0.25
+    co.config(make_config(n_item, pct))
+    co.coll_cache_record_init(0)
+    co.coll_torch_record(0, torch.from_numpy(rng.integers(0, n_item, size=60_000)).to(kdtype))
+    emb = co.coll_torch_create_emb_shm(0, n_item, dim, torch.float32)
+    table = fill_table(emb, rng)
+    co.coll_torch_init_t(0, 0, emb, pct)
+    co.coll_torch_forward_config(True, 10 ** 9, frac, False)
+    alive, recorded, outs = [], [], []
+    for step in range(30):
+        n = 4_000 + 16 * step
+        keys = rng.integers(0, n_item, size=n)
+        alive.append(torch.from_numpy(keys).to(kdtype).cuda())
+        outs.append((keys, co.coll_torch_forward(0, alive[-1], False, stream_ordered=True).clone()))
+        recorded.append(keys[: int(n * frac)])
+    co.coll_torch_lookup_wait(0)
+    for keys, out in outs:
+        assert out.cpu().numpy().tobytes() == ORC.gather(table, keys.astype(np.int64)).tobytes()
+    want_k, want_c = ORC.freq_rank(np.concatenate(recorded).astype(np.uint32))
+    got_k, got_c = np.zeros(n_item, np.uint32), np.zeros(n_item, np.uint32)
+    m = _basics.C_LIB_CTYPES.coll_cache_rank_hotness(0, got_k.ctypes.data, got_c.ctypes.data, n_item)
+    assert m == len(want_k) and np.array_equal(got_k[:m], want_k) and np.array_equal(got_c[:m], want_c)
     co.coll_torch_forward_config(False, 0, frac, False)
 
 

@@ -99,9 +99,13 @@ void coll_cache_config_from_map(std::unordered_map<std::string, std::string> &co
   _coll_cache->_profiler = _profiler;
 }
 
+// prefixes that stream-ordered serving steps have copied out and not counted yet (defined with the serving loop)
+void CountPendingPrefixes(bool all);
+
 ContFreqBuf *CombineAndRank(int replica_id) {
   CHECK_LT((size_t)replica_id, _freq_recorder.size()) << "coll_cache_record_init was not called";
   CHECK_NOTNULL(_freq_recorder[replica_id]);
+  CountPendingPrefixes(/*all=*/true);
   // what the lookups counted on the device joins what coll_cache_record counted on the host
   if (_coll_cache && _coll_cache->num_replicas_built() > (size_t)replica_id && _coll_cache->session(replica_id)) {
     const size_t rows = _coll_cache->session(replica_id)->DrainHotness(_freq_recorder[replica_id].get());
@@ -300,6 +304,7 @@ void coll_cache_segment_offsets(int replica_id, const int64_t *sorted_rows, size
 void coll_cache_lookup_wait(int replica_id, StreamHandle stream) {
   CHECK_NOTNULL(_coll_cache);
   _coll_cache->lookup_wait(replica_id, stream);
+  CountPendingPrefixes(/*all=*/true);
 }
 
 void coll_cache_record(int replica_id, uint32_t *key, size_t num_keys) {
@@ -491,6 +496,19 @@ struct ForwardState {
   // (1,024 keys: 55 us per step against 12 us for the lookup alone).
   void *inline_prefix = nullptr;
   size_t inline_prefix_bytes = 0;
+  // A step that is enqueued and left cannot count its prefix when it returns: the copy kernel has not run yet.  Its
+  // prefix waits in one of a few pinned buffers, behind an event, until a later step (or whoever needs the counts: a
+  // ranking, coll_cache_lookup_wait, the shutdown) finds the event complete, or waits for it, and counts it.
+  struct PendingPrefix {
+    void *staging = nullptr;
+    void *copied = nullptr;  // event behind the copy kernel
+    size_t bytes = 0, num = 0;
+    int replica = 0, key_bytes = 4;
+  };
+  static constexpr size_t kPendingSlots = 8;
+  PendingPrefix pending[kPendingSlots];
+  size_t pending_head = 0, pending_tail = 0;  // [tail, head) wait to be counted
+  std::mutex pending_mu;                      // the steps' thread and a refresh thread that ranks
   ~ForwardState() {
     if (refresh_thread.joinable()) refresh_thread.join();  // a process that exits without coll_cache_shutdown
   }
@@ -499,6 +517,70 @@ ForwardState _forward;
 
 void ForwardJoin() {
   if (_forward.refresh_thread.joinable()) _forward.refresh_thread.join();
+}
+
+// caller holds pending_mu
+void CountPendingLocked(bool all) {
+  ForwardState &fw = _forward;
+  while (fw.pending_tail != fw.pending_head) {
+    ForwardState::PendingPrefix &p = fw.pending[fw.pending_tail % ForwardState::kPendingSlots];
+    if (all) {
+      UGK_CALL(ugk_event_sync(p.copied));
+    } else {
+      int complete = 0;
+      UGK_CALL(ugk_event_query(p.copied, &complete));
+      if (!complete) break;
+    }
+    if ((size_t)p.replica < _freq_recorder.size() && _freq_recorder[p.replica]) {
+      if (p.key_bytes == 8)
+        _freq_recorder[p.replica]->Record(static_cast<const Id64Type *>(p.staging), p.num);
+      else
+        _freq_recorder[p.replica]->Record(static_cast<const IdType *>(p.staging), p.num);
+    }
+    fw.pending_tail++;
+  }
+}
+
+void CountPendingPrefixes(bool all) {
+  std::lock_guard<std::mutex> g(_forward.pending_mu);
+  CountPendingLocked(all);
+}
+
+// the prefix of a stream-ordered step: a copy kernel on the caller's stream into the next pinned buffer, an event behind
+// it; counted later (CountPendingPrefixes)
+void PostPendingPrefix(int replica_id, const void *key, size_t num, int key_bytes, StreamHandle stream) {
+  ForwardState &fw = _forward;
+  std::lock_guard<std::mutex> g(fw.pending_mu);
+  CountPendingLocked(/*all=*/false);
+  if (fw.pending_head - fw.pending_tail == ForwardState::kPendingSlots) {  // every buffer waits: take the oldest
+    ForwardState::PendingPrefix &oldest = fw.pending[fw.pending_tail % ForwardState::kPendingSlots];
+    UGK_CALL(ugk_event_sync(oldest.copied));
+    CountPendingLocked(/*all=*/false);
+  }
+  ForwardState::PendingPrefix &p = fw.pending[fw.pending_head % ForwardState::kPendingSlots];
+  const size_t bytes = num * key_bytes;
+  if (p.bytes < bytes) {
+    if (p.staging) UGK_CALL(ugk_host_free(p.staging));
+    p.bytes = std::max(bytes, RunConfig::record_inline_bytes);
+    UGK_CALL(ugk_host_malloc(&p.staging, p.bytes));
+  }
+  if (p.copied == nullptr) UGK_CALL(ugk_event_create(&p.copied));
+  p.replica = replica_id, p.num = num, p.key_bytes = key_bytes;
+  UGK_CALL(ugk_copy_rows(p.staging, key, bytes, stream));
+  UGK_CALL(ugk_event_record(p.copied, stream));
+  fw.pending_head++;
+}
+
+void ReleasePendingPrefixes() {
+  ForwardState &fw = _forward;
+  std::lock_guard<std::mutex> g(fw.pending_mu);
+  CountPendingLocked(/*all=*/true);
+  for (auto &p : fw.pending) {
+    if (p.staging) UGK_CALL(ugk_host_free(p.staging));
+    if (p.copied) UGK_CALL(ugk_event_destroy(p.copied));
+    p = ForwardState::PendingPrefix();
+  }
+  fw.pending_head = fw.pending_tail = 0;
 }
 
 // lookup(step_key, ordered): the extraction of the step — the plain lookup, or the pooled one; blocking, or
@@ -513,11 +595,24 @@ void ForwardStep(int replica_id, const KeyT *key, size_t num_keys, StreamHandle 
   auto session = _coll_cache->session(replica_id);
   const size_t num_record = fw.enable_refresh ? (size_t)(num_keys * fw.record_fraction) : 0;
   const size_t record_bytes = num_record * sizeof(KeyT);
-  const bool inline_prefix = !RunConfig::gpu_record && num_record > 0 &&
-                             record_bytes <= RunConfig::record_inline_bytes &&
-                             reinterpret_cast<uintptr_t>(key) % 16 == 0;
+  const bool small_prefix = !RunConfig::gpu_record && num_record > 0 &&
+                            record_bytes <= RunConfig::record_inline_bytes &&
+                            reinterpret_cast<uintptr_t>(key) % 16 == 0;
+  // a small prefix of a step that is enqueued and left is counted later; a step that is being recorded into a HIP
+  // graph records nothing (the host cannot count what a replay copies)
+  bool deferred_prefix = false, skip_record = false;
+  if (stream_ordered && small_prefix) {
+    int capturing = 0;
+    UGK_CALL(ugk_stream_is_capturing(stream, &capturing));
+    skip_record = capturing != 0;
+    deferred_prefix = !skip_record;
+  }
+  const bool inline_prefix = small_prefix && !deferred_prefix && !skip_record;
   if (RunConfig::gpu_record) {
     session->SetRecordLimit(num_record);  // counted by the lookup itself
+  } else if (deferred_prefix) {
+    PostPendingPrefix(replica_id, key, num_record, (int)sizeof(KeyT), stream);
+  } else if (skip_record) {
   } else if (inline_prefix) {
     if (fw.inline_prefix_bytes < RunConfig::record_inline_bytes) {
       if (fw.inline_prefix) UGK_CALL(ugk_host_free(fw.inline_prefix));
@@ -530,9 +625,10 @@ void ForwardStep(int replica_id, const KeyT *key, size_t num_keys, StreamHandle 
   }
   const uint64_t step_key = steps[replica_id] * RunConfig::num_device + replica_id;
   steps[replica_id]++;
-  lookup(step_key, stream_ordered && (RunConfig::gpu_record || num_record == 0));
+  lookup(step_key, stream_ordered && (RunConfig::gpu_record || num_record == 0 || deferred_prefix || skip_record));
   if (RunConfig::gpu_record) {
     session->SetRecordLimit(SIZE_MAX);
+  } else if (deferred_prefix || skip_record) {
   } else if (inline_prefix) {
     _freq_recorder[replica_id]->Record(static_cast<const KeyT *>(fw.inline_prefix), num_record);
   } else if (num_record > 0) {
@@ -544,6 +640,7 @@ void ForwardStep(int replica_id, const KeyT *key, size_t num_keys, StreamHandle 
     if (!fw.refresh_ongoing.load()) {
       fw.refresh_ongoing.store(true);
       ForwardJoin();
+      CountPendingPrefixes(/*all=*/true);  // the refresh ranks what every step up to this one recorded
       fw.refresh_thread = std::thread([replica_id, stream]() {
         coll_cache_refresh(replica_id, stream, /*foreground=*/0);
         _forward.refreshes_done.fetch_add(1);
@@ -755,6 +852,7 @@ uint32_t coll_cache_place_recorded(int replica_id, uint32_t num_node, double cac
 void coll_cache_shutdown(void) {
   ForwardJoin();
   _forward.recorder.Stop();
+  ReleasePendingPrefixes();
   if (_forward.inline_prefix) {
     UGK_CALL(ugk_host_free(_forward.inline_prefix));
     _forward.inline_prefix = nullptr;

@@ -192,7 +192,7 @@ def coll_torch_lookup_pooled(local_id, ids, seg_off, weights=None, combiner="sum
     squares ("sqrtn") — embedding_lookup_sparse without the [len(ids), dim] intermediate.  ids: GPU int32 / int64;
     seg_off: GPU int64, ascending, seg_off[0] == 0 and seg_off[-1] == len(ids); weights: GPU float32 or None.
     serving_step: the call is one step of the serving loop (as coll_torch_forward is for a plain lookup; with
-    stream_ordered as well it blocks only if the step's prefix is counted on the host).
+    stream_ordered as well it blocks only if the step's prefix is counted on the host and exceeds 64 KB).
     stream_ordered: the call is enqueued on torch's current stream and returns without waiting, like any torch op
     (as coll_torch_lookup_async is for a plain lookup; `ids`, `seg_off` and `weights` must stay alive until the work has
     run; coll_torch_lookup_wait reports a bad id or offset and makes the group sizes available)."""
@@ -265,8 +265,9 @@ def coll_torch_forward(local_id, keys, pad_to_8=True, stream_ordered=False):
     """one serving step (LookupManager::forward, lookup_manager.cc:158-213): the hotness of a prefix of the batch is
     recorded, the keys are looked up, and at the configured step a refresh starts on a background thread.  Returns
     the same reused buffer view as coll_torch_lookup_key_t_val_ret.  stream_ordered (extension): the lookup is
-    enqueued on torch's current stream like coll_torch_lookup_async and the call returns without waiting; a step whose
-    prefix is counted on the host (COLL_GPU_RECORD unset, a refresh configured) blocks all the same."""
+    enqueued on torch's current stream like coll_torch_lookup_async and the call returns without waiting (a prefix
+    counted on the host is then counted by a later step or by coll_torch_lookup_wait; one beyond
+    COLL_RECORD_INLINE_BYTES = 64 KB makes the step block all the same)."""
     if stream_ordered:
         return _lookup_into_reused_buffer(local_id, keys, pad_to_8, _C.coll_cache_forward_async,
                                           _C.coll_cache_forward_async_i64)

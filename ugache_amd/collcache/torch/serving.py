@@ -163,8 +163,8 @@ class LookupLayer(torch.nn.Module):
         self.table_id = table_id
         self.emb_vec_size = emb_vec_size
         self.emb_vec_dtype = emb_vec_dtype
-        # stream_ordered=True (extension): the step is enqueued on torch's current stream like any torch op (it still
-        # blocks while the hotness of its prefix is counted on the host, i.e. without COLL_GPU_RECORD=1)
+        # stream_ordered=True (extension): the step is enqueued on torch's current stream like any torch op (only a
+        # recorded prefix beyond 64 KB that is counted on the host still makes it block)
         self.stream_ordered = bool(kwargs.get("stream_ordered", False))
 
     def check(self, inputs):
@@ -205,8 +205,8 @@ class SparseLookupLayer(torch.nn.Module):
         # fused=True: lookup and combination in one kernel of the library (coll_torch_lookup_pooled) wherever that
         # kernel can take the call (no max_norm, rows it supports); the steps below otherwise
         self.fused = bool(kwargs.get("fused", False))
-        # stream_ordered=True (with fused): the step is enqueued on torch's current stream like any torch op (it still
-        # blocks while the hotness of its prefix is counted on the host, i.e. without COLL_GPU_RECORD=1)
+        # stream_ordered=True (with fused): the step is enqueued on torch's current stream like any torch op (only a
+        # recorded prefix beyond 64 KB that is counted on the host still makes it block)
         self.stream_ordered = bool(kwargs.get("stream_ordered", False))
 
     def forward(self, sp_ids, sp_weights=None, name=None, combiner=None, max_norm=None):

@@ -261,6 +261,19 @@ int ugk_event_sync(void *event) {
   return 0;
 }
 
+int ugk_event_query(void *event, int *complete) {
+  UGK_REQUIRE(event && complete, "ugk_event_query: null pointer");
+  const hipError_t e = hipEventQuery(reinterpret_cast<hipEvent_t>(event));
+  if (e == hipErrorNotReady) {
+    (void)hipGetLastError();
+    *complete = 0;
+    return 0;
+  }
+  UGK_HIP(e);
+  *complete = 1;
+  return 0;
+}
+
 int ugk_stream_wait_event(void *stream, void *event) {
   UGK_HIP(hipStreamWaitEvent(as_stream(stream), reinterpret_cast<hipEvent_t>(event), 0));
   return 0;

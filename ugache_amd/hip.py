@@ -73,6 +73,7 @@ SIGNATURES = {
     "ugk_event_destroy": [_vp],
     "ugk_event_record": [_vp, _vp],
     "ugk_event_sync": [_vp],
+    "ugk_event_query": [_vp, _vp],
     "ugk_stream_wait_event": [_vp, _vp],
     "ugk_event_elapsed_ms": [_vp, _vp, C.POINTER(C.c_float)],
     "ugk_memcpy_async": [_vp, _vp, _sz, _vp],
