@@ -584,8 +584,9 @@ void ReleasePendingPrefixes() {
 }
 
 // lookup(step_key, ordered): the extraction of the step — the plain lookup, or the pooled one; blocking, or
-// (ordered) enqueued on the caller's stream and left.  A step whose recorded prefix is counted on the host blocks
-// whatever the caller asked for: the prefix is copied out of the caller's buffer while the step knows it to be alive.
+// (ordered) enqueued on the caller's stream and left.  A step whose recorded prefix this thread or the record thread
+// counts blocks whatever the caller asked for: the record thread copies the prefix out of the caller's buffer while
+// the step knows it to be alive.
 template <typename KeyT, typename LookupFn>
 void ForwardStep(int replica_id, const KeyT *key, size_t num_keys, StreamHandle stream, bool stream_ordered,
                  const LookupFn &lookup) {
@@ -595,44 +596,55 @@ void ForwardStep(int replica_id, const KeyT *key, size_t num_keys, StreamHandle 
   auto session = _coll_cache->session(replica_id);
   const size_t num_record = fw.enable_refresh ? (size_t)(num_keys * fw.record_fraction) : 0;
   const size_t record_bytes = num_record * sizeof(KeyT);
-  const bool small_prefix = !RunConfig::gpu_record && num_record > 0 &&
-                            record_bytes <= RunConfig::record_inline_bytes &&
-                            reinterpret_cast<uintptr_t>(key) % 16 == 0;
-  // a small prefix of a step that is enqueued and left is counted later; a step that is being recorded into a HIP
-  // graph records nothing (the host cannot count what a replay copies)
-  bool deferred_prefix = false, skip_record = false;
-  if (stream_ordered && small_prefix) {
-    int capturing = 0;
-    UGK_CALL(ugk_stream_is_capturing(stream, &capturing));
-    skip_record = capturing != 0;
-    deferred_prefix = !skip_record;
-  }
-  const bool inline_prefix = small_prefix && !deferred_prefix && !skip_record;
-  if (RunConfig::gpu_record) {
-    session->SetRecordLimit(num_record);  // counted by the lookup itself
-  } else if (deferred_prefix) {
-    PostPendingPrefix(replica_id, key, num_record, (int)sizeof(KeyT), stream);
-  } else if (skip_record) {
-  } else if (inline_prefix) {
-    if (fw.inline_prefix_bytes < RunConfig::record_inline_bytes) {
-      if (fw.inline_prefix) UGK_CALL(ugk_host_free(fw.inline_prefix));
-      UGK_CALL(ugk_host_malloc(&fw.inline_prefix, RunConfig::record_inline_bytes));
-      fw.inline_prefix_bytes = RunConfig::record_inline_bytes;
+  // who counts the prefix
+  enum class Prefix {
+    kNone,      // nothing to record
+    kDevice,    // the lookup itself, into the device-side counters
+    kThread,    // the record thread, from a copy it makes beside the lookup; the step waits for it
+    kInline,    // this thread after the blocking lookup, from a copy a kernel in front of the lookup makes
+    kDeferred,  // a later step (or the wait, or the ranking), from such a copy: the step is enqueued and left
+  } prefix = Prefix::kNone;
+  if (num_record > 0) {
+    const bool small = record_bytes <= RunConfig::record_inline_bytes && reinterpret_cast<uintptr_t>(key) % 16 == 0;
+    if (RunConfig::gpu_record) {
+      prefix = Prefix::kDevice;
+    } else if (small && stream_ordered) {
+      // a step that is being recorded into a HIP graph records nothing: the host cannot count what a replay copies
+      int capturing = 0;
+      UGK_CALL(ugk_stream_is_capturing(stream, &capturing));
+      prefix = capturing ? Prefix::kNone : Prefix::kDeferred;
+    } else {
+      prefix = small ? Prefix::kInline : Prefix::kThread;
     }
-    UGK_CALL(ugk_copy_rows(fw.inline_prefix, key, record_bytes, stream));  // complete when the lookup behind it is
-  } else if (num_record > 0) {
-    fw.recorder.Post(replica_id, session->DeviceId(), key, num_record, sizeof(KeyT), stream);  // counted while the lookup runs
+  }
+  switch (prefix) {
+    case Prefix::kDevice: session->SetRecordLimit(num_record); break;
+    case Prefix::kDeferred: PostPendingPrefix(replica_id, key, num_record, (int)sizeof(KeyT), stream); break;
+    case Prefix::kInline:
+      if (fw.inline_prefix_bytes < RunConfig::record_inline_bytes) {
+        if (fw.inline_prefix) UGK_CALL(ugk_host_free(fw.inline_prefix));
+        UGK_CALL(ugk_host_malloc(&fw.inline_prefix, RunConfig::record_inline_bytes));
+        fw.inline_prefix_bytes = RunConfig::record_inline_bytes;
+      }
+      UGK_CALL(ugk_copy_rows(fw.inline_prefix, key, record_bytes, stream));  // complete when the lookup behind it is
+      break;
+    case Prefix::kThread:
+      fw.recorder.Post(replica_id, session->DeviceId(), key, num_record, sizeof(KeyT), stream);
+      break;
+    case Prefix::kNone: break;
   }
   const uint64_t step_key = steps[replica_id] * RunConfig::num_device + replica_id;
   steps[replica_id]++;
-  lookup(step_key, stream_ordered && (RunConfig::gpu_record || num_record == 0 || deferred_prefix || skip_record));
-  if (RunConfig::gpu_record) {
-    session->SetRecordLimit(SIZE_MAX);
-  } else if (deferred_prefix || skip_record) {
-  } else if (inline_prefix) {
-    _freq_recorder[replica_id]->Record(static_cast<const KeyT *>(fw.inline_prefix), num_record);
-  } else if (num_record > 0) {
-    fw.recorder.Wait();
+  // the host's own counting (kInline, kThread) needs the lookup to have returned
+  lookup(step_key, stream_ordered && prefix != Prefix::kInline && prefix != Prefix::kThread);
+  switch (prefix) {
+    case Prefix::kDevice: session->SetRecordLimit(SIZE_MAX); break;
+    case Prefix::kInline:
+      _freq_recorder[replica_id]->Record(static_cast<const KeyT *>(fw.inline_prefix), num_record);
+      break;
+    case Prefix::kThread: fw.recorder.Wait(); break;
+    case Prefix::kDeferred:
+    case Prefix::kNone: break;
   }
   const bool due = fw.enable_refresh && fw.refresh_iter > 0 &&
                    (fw.periodic ? (fw.step > 0 && fw.step % fw.refresh_iter == 0) : fw.step == fw.refresh_iter);
