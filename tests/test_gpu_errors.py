@@ -123,6 +123,10 @@ def test_a_process_that_never_calls_shutdown_still_exits_cleanly(gpu_record):
             keys = torch.from_numpy((rng.zipf(1.1, 20000) + step * 1000) % n).to(torch.int64).cuda()
             out = co.coll_torch_forward(0, keys)
             assert torch.equal(out.cpu(), emb[keys.cpu()])
+        # ... nor wait for the steps it enqueued last, whose prefixes nobody has counted yet
+        kept = [torch.from_numpy(rng.integers(0, n, 4000)).cuda() for _ in range(3)]
+        for keys in kept:
+            co.coll_torch_forward(0, keys, stream_ordered=True)
         print("forwards ok", flush=True)
     """, env={"COLL_GPU_RECORD": gpu_record, "COLL_REFRESH_SLEEP_US": "20000"})
     assert "forwards ok" in p.stdout, p.stderr[-2000:]
