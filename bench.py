@@ -117,7 +117,7 @@ def parse_args():
                          "known traffic next to the gather")
     ap.add_argument("--probe", default=None, choices=["kpw", "row_span", "cu_mask", "small_batch", "pooled", "sparse_layer"],
                     help="instead of a workload, run one of the stand-alone measurements behind the launch rules "
-                         "(ugache_amd/probes.py): keys per wavefront of the fused kernel, random rows over the host "
+                         "(bench_probes.py): keys per wavefront of the fused kernel, random rows over the host "
                          "link by span, host-link gather confined to a few compute units, serving-sized batches through "
                          "the library; prints one JSON line")
     ap.add_argument("--quick", action="store_true", help="with --probe: a reduced sweep")
@@ -972,9 +972,9 @@ def main():
     global _REAL_STDOUT
     args = parse_args()
     if args.probe:
-        from ugache_amd import probes
+        import bench_probes
 
-        probes.run(args.probe, args.quick)
+        bench_probes.run(args.probe, args.quick)
         return
     if args.workload is None:
         return run_default(args)

@@ -32,7 +32,7 @@ extern "C" {
 #define UGK_ST_TABLE_FULL 0x2u       /* hash insert found no free bucket */
 #define UGK_ST_DUP_KEY 0x4u          /* insert of a key that is already present (the reference asserts) */
 #define UGK_ST_EVICT_ABSENT 0x8u     /* evict of a key that is not present */
-#define UGK_ST_BAD_SEGMENT 0x10u     /* pooled extraction: offsets that leave [0, nnz] or run backwards: row of zeros */
+#define UGK_ST_BAD_SEGMENT 0x10u     /* pooled extraction: offsets that leave [0, nnz], run backwards or do not span [0, nnz] */
 
 /* element code of the pooled extraction for bfloat16 rows (fp32 and fp16 are named by their size, 4 and 2) */
 #define UGK_ELEM_BF16 0x102
@@ -93,7 +93,7 @@ typedef struct {
 const char *ugk_last_error(void);
 /* version of this ABI; bumped on any signature change.  ugk_abi_version() is what the loaded library was built with:
  * a caller compiled against another UGK_ABI_VERSION must not go on. */
-#define UGK_ABI_VERSION 17
+#define UGK_ABI_VERSION 18
 int ugk_abi_version(void);
 
 /* ---- runtime plumbing: Device::{AllocDataSpace,FreeDataSpace,CopyDataFromTo,StreamSync,CreateStream}
@@ -116,7 +116,10 @@ int ugk_stream_create(void **stream);
 int ugk_stream_create_cu_masked(void **stream, int num_cus);
 int ugk_stream_destroy(void *stream);
 int ugk_stream_sync(void *stream);
-/* *capturing = 1 while work enqueued on `stream` is being recorded into a HIP graph instead of being run, else 0 */
+/* *capturing = 1 while work enqueued on `stream` is being recorded into a HIP graph instead of being run, 0 when it
+ * runs, UGK_CAPTURE_QUERY_REFUSED when the runtime refuses the question (the legacy default stream while another
+ * stream of the process records in global mode: work enqueued on `stream` would be refused as well) */
+#define UGK_CAPTURE_QUERY_REFUSED 2
 int ugk_stream_is_capturing(void *stream, int *capturing);
 /* ugk_stream_sync for callers that wait for short launches: enqueues a one-lane kernel that writes `value` into
  * *ticket_host (pinned host word from ugk_host_malloc) behind everything already enqueued on `stream`, and polls that
@@ -289,7 +292,8 @@ int ugk_extract_mix_i64(ugk_table_t t, const int64_t *keys_dev, size_t n, const 
  * nnz.  row_bytes: a multiple of 16, at most 4096.  Status, host mirror and the per-workgroup count words are those of
  * ugk_extract_mix_* (the counts are of ids, not of output rows).  An id without a row sets UGK_ST_KEY_OUT_OF_RANGE and
  * adds nothing; a segment whose offsets leave [0, nnz] or run backwards sets UGK_ST_BAD_SEGMENT, reads no id and
- * gives a zero row. */
+ * gives a zero row; offsets that do not begin at 0 or do not end at nnz set the same bit (the rows are computed as the
+ * offsets say, but the counts of ids per source then do not add up to nnz). */
 /* The offsets ugk_extract_pool_* takes, from the row of every entry of a sparse feature in row-major order (the
  * indices[:, 0] of the SparseTensor of sparse_lookup_layer.py:196-265): seg_off_dev[r] = number of entries whose row is
  * below r, for r = 0 .. n_rows (n_rows + 1 words; rows without an entry get empty segments).  One launch, no
@@ -325,7 +329,10 @@ int ugk_extract_pool_i64(ugk_table_t t, const int64_t *ids_dev, const int64_t *s
  * in its table before the rest has arrived.  Results are the same
  * bytes with and without a stage: the host table does not change under a cache.  An entry is only consistent at launch
  * boundaries, so the staged gather must not read a stage that an extraction in flight writes (a caller with lookups
- * running beside its refreshes keeps two stages and reads the one the lookups have been switched away from).
+ * running beside its refreshes keeps two stages and reads the one the lookups have been switched away from).  For the
+ * same reason two staged extractions that may run at the same time (launches on different streams with nothing that
+ * orders them) must not share a stage: both could claim one entry and interleave the 16-byte stores of two different
+ * rows under an owner word that names one of them.  Launches on one stream are ordered and may share it.
  * rows_dev: (mask + 1) x row_bytes bytes; owner_dev: mask + 1 words, zero-filled once; host rows must fit 32 bits. */
 typedef struct {
   void *rows_dev;
@@ -375,7 +382,8 @@ int ugk_dedup_i64(const int64_t *keys_dev, size_t n, void *workspace_dev, size_t
  * hipMalloc / hipFree and no allocating library call; *n_unique_dev is cleared by the call (an output, not an in/out).
  * key_bytes: 4 (uint32 keys) or 8 (int64 keys).  n may not exceed UGK_DEDUP_STATIC_MAX_KEYS: larger batches are
  * refused with an error.  All calls on one GPU share that GPU's array: calls that overlap in time on one GPU (different
- * streams, or threads) race and give wrong results; calls ordered one after the other, on any streams, are fine. */
+ * streams, or threads) race and give wrong results; calls ordered one after the other, on any streams, are fine.
+ * The first call on a device looks the array's address up (hipGetSymbolAddress): make that call outside a capture. */
 #define UGK_DEDUP_STATIC_MAX_KEYS (1u << 20)
 int ugk_dedup_static(const void *keys_dev, uint32_t key_bytes, size_t n, void *unique_out_dev,
                      uint32_t *inverse_out_dev, uint32_t *rep_out_dev, uint32_t *n_unique_dev, uint32_t *n_unique_host,

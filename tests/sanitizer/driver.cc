@@ -3,7 +3,11 @@
 // AddressSanitizer / UBSan and ThreadSanitizer:
 //   build -> blocking lookups on one thread  ||  hotness records + background refreshes on another
 //         -> stream-ordered lookups on one stream  ||  a refresh on another stream
-//         -> the serving loop (coll_cache_forward) with its own background refresh thread -> shutdown,
+//         -> the serving loop (coll_cache_forward) with its own background refresh thread
+//         -> stream-ordered lookups that a caller records into a graph on a stream of its own, a refresh on that stream,
+//            the shutdown while the graph still lives (the model lists every call that breaks a rule of such a capture
+//            or ties an object of the library to the caller's graph)
+//         -> shutdown,
 // once per table kind and per refresh kind (host lists / device bitmaps).  Every looked-up row is compared with the
 // host table, so a refresh that reused a slot too early is also seen as a wrong row.
 //
@@ -20,6 +24,8 @@
 #include <vector>
 
 #include "coll_cache_c_api.h"
+#include "ugache_hip.h"
+#include "ugk_cpu_model.h"
 
 namespace {
 
@@ -177,6 +183,72 @@ int main(int argc, char **argv) {
           if (std::fabs(out[r * kDim + c] - want) > 1e-4 * (1.0 + std::fabs(want))) ++bad_rows;
         }
     }
+    // 6. a caller records stream-ordered lookups, plain and pooled, and a serving step into a graph on its own stream.
+    //    With the hotness counted on the device the lookups count inside that graph; nothing of the library but kernels
+    //    on the caller's stream may take part in the capture.
+    void *caller_stream = nullptr;
+    std::vector<void *> extra_streams;
+    int graph = 0;
+    {
+      if (ugk_stream_create(&caller_stream) != 0) return 1;
+      const uint32_t marked = 4242;  // a key every captured batch holds 64 times
+      auto k = skewed_keys(g, 2048, 31000);
+      for (size_t i = 0; i < 64; ++i) k[i * 7] = marked;
+      std::vector<int64_t> off(1, 0);
+      while ((size_t)off.back() < k.size()) off.push_back(std::min<int64_t>((int64_t)k.size(), off.back() + 4));
+      std::vector<float> pooled((off.size() - 1) * kDim), plain(k.size() * kDim), step_out(k.size() * kDim);
+      coll_cache_lookup_wait(0, nullptr);
+      coll_cache_forward_join();  // the foreground refresh below must not meet one of the serving loop's
+      if (ugk_model_capture_begin(caller_stream) != 0) return 1;
+      coll_cache_lookup_async(0, k.data(), k.size(), plain.data(), caller_stream);
+      coll_cache_lookup_pooled_async(0, k.data(), off.data(), nullptr, off.size() - 1, k.size(), 0, 4, pooled.data(),
+                                     caller_stream);
+      coll_cache_forward_async(0, k.data(), k.size(), step_out.data(), caller_stream);
+      if (ugk_model_capture_end(caller_stream, &graph) != 0) return 1;
+      coll_cache_lookup_wait(0, caller_stream);
+      bad_rows += check_rows(table, plain.data(), k.data(), k.size());
+      bad_rows += check_rows(table, step_out.data(), k.data(), k.size());
+      for (size_t r = 0; r + 1 < off.size(); ++r)
+        for (size_t c = 0; c < kDim; ++c) {
+          double sum = 0;
+          for (int64_t j = off[r]; j < off[r + 1]; ++j) sum += table[(size_t)k[j] * kDim + c];
+          if (std::fabs(pooled[r * kDim + c] - sum) > 1e-4 * (1.0 + std::fabs(sum))) ++bad_rows;
+        }
+      // an eager lookup and a foreground refresh on the stream the graph was recorded on
+      coll_cache_lookup_async(0, k.data(), k.size(), plain.data(), caller_stream);
+      coll_cache_lookup_wait(0, caller_stream);
+      coll_cache_refresh(0, caller_stream, /*foreground=*/1);
+      coll_cache_lookup(0, k.data(), k.size(), plain.data(), caller_stream);
+      bad_rows += check_rows(table, plain.data(), k.data(), k.size());
+      if (on_device) {
+        // the two plain lookups and the pooled one counted every key, the serving step its recorded quarter: the marked
+        // key was counted at least 3 x 64 times by launches inside the capture
+        coll_cache_lookup_async(0, k.data(), k.size(), plain.data(), caller_stream);  // counted eagerly: 64 more
+        coll_cache_lookup_wait(0, caller_stream);
+        std::vector<uint32_t> rk(kRows), rc(kRows);
+        const size_t n = coll_cache_rank_hotness(0, rk.data(), rc.data(), kRows);
+        uint32_t seen = 0;
+        for (size_t i = 0; i < n; ++i)
+          if (rk[i] == marked) seen = rc[i];
+        if (seen < 64) {
+          fprintf(stderr, "the marked key was counted %u times after the refresh, 64 expected from the last lookup\n", seen);
+          return 1;
+        }
+      }
+      // stream-ordered lookups on two streams with no wait between them: the second must not file rows in the stage the
+      // first may still be writing (the model reports two unordered writers of one stage)
+      void *second_stream = nullptr;
+      if (ugk_stream_create(&second_stream) != 0) return 1;
+      coll_cache_lookup_async(0, k.data(), k.size(), plain.data(), caller_stream);
+      coll_cache_lookup_async(0, k.data(), k.size(), step_out.data(), second_stream);
+      coll_cache_lookup_wait(0, second_stream);
+      coll_cache_lookup_wait(0, caller_stream);
+      bad_rows += check_rows(table, plain.data(), k.data(), k.size());
+      bad_rows += check_rows(table, step_out.data(), k.data(), k.size());
+      coll_cache_refresh(0, caller_stream, /*foreground=*/1);  // also waits for, and forgets nothing of, both streams
+      extra_streams.push_back(second_stream);
+      if (round == 1) ugk_model_graph_destroy(graph);  // round 0 shuts down while the caller still holds its graph
+    }
     const uint64_t done = coll_cache_forward_join();
     uint64_t info[8];
     coll_cache_get_info(0, info);
@@ -190,6 +262,15 @@ int main(int argc, char **argv) {
     }
     coll_cache_shutdown();
     coll_cache_free_host_table(table);
+    ugk_model_graph_destroy(graph);
+    ugk_stream_destroy(caller_stream);
+    for (void *st : extra_streams) ugk_stream_destroy(st);
+    char text[4096];
+    if (const size_t broken = ugk_model_violations(text, sizeof(text))) {
+      fprintf(stderr, "%zu calls broke a rule that the model of the kernel layer checks:\n%s", broken, text);
+      return 1;
+    }
+    ugk_model_reset();
   }
   if (bad_rows) {
     fprintf(stderr, "%ld looked-up rows differ from the host table\n", bad_rows);

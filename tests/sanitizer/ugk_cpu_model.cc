@@ -23,6 +23,7 @@
 #include <cstring>
 #include <map>
 #include <mutex>
+#include <string>
 #include <unordered_map>
 #include <vector>
 
@@ -411,6 +412,8 @@ int extract_pool(ugk_table_t t, const K *ids, const int64_t *seg_off, const floa
     if (beg < 0 || end > (int64_t)nnz || end < beg) {
       or_status(status, UGK_ST_BAD_SEGMENT, mirror);
       beg = end = 0;
+    } else if ((r == 0 && beg != 0) || (r + 1 == n_rows && end != (int64_t)nnz)) {
+      or_status(status, UGK_ST_BAD_SEGMENT, mirror);  // the ids are not covered from the first to the last
     }
     for (int64_t j = beg; j < end; ++j) {
       const uint64_t key = k64(ids[j]);
@@ -522,11 +525,129 @@ uint64_t bm_word(const uint64_t *a, const uint64_t *b, int invert_a, uint64_t nb
   return m;
 }
 
+// ---- streams, events and the rules of recording a stream into a graph -----------------------------------------------
+// Work enqueued on a stream still runs at once (see the top of the file), also while the stream "captures": what the
+// model adds is the bookkeeping the runtime keeps for a capture, so that a sequence of calls that the runtime refuses,
+// or that leaves objects of the library tied to a graph the caller owns, is reported here, on the CPU:
+//   - an event recorded on a capturing stream is a captured event; a stream that waits for one joins the capture;
+//   - a captured event cannot be waited for, queried or timed on the host; a capturing stream cannot be waited for, nor
+//     can the device while any stream captures; memory cannot be allocated or freed meanwhile (global capture mode);
+//   - a capturing stream cannot wait for an event recorded outside the capture;
+//   - a stream that joined has to be joined back before the capture ends;
+//   - a stream or event that took part in a capture must not be destroyed while the recorded graph lives, and -- the
+//     rule of the library itself -- only the caller's stream takes part in the caller's capture: an event recorded or a
+//     second stream joined while capturing is reported even where the runtime would accept it.
+struct Stream {
+  int capture = 0;      // id of the capture this stream records into, 0: runs its work
+  bool origin = false;  // the capture was begun on this stream
+  void *join_event = nullptr;  // joined stream: the last event recorded on it
+  bool joined_back = true;
+};
 struct Event {
   std::chrono::steady_clock::time_point at;
+  int captured_in = 0;  // id of the capture its last record went into, 0: recorded on a running stream
+  Stream *recorded_on = nullptr;
 };
+struct Graph {
+  std::vector<Stream *> streams;
+  std::vector<void *> events;
+  bool alive = true;
+};
+std::mutex g_rt_mu;  // guards everything below and the fields of every Stream and Event
+Stream g_null_stream;
+int g_capture_active = 0, g_capture_next = 1;
+std::map<int, Graph> g_graphs;
+std::vector<std::string> g_violations;
+// which stream last filed rows in a stage (keyed by its owner words) and whether the host has waited for it since
+std::map<const void *, std::pair<Stream *, bool>> g_stage_writers;
+
+Stream *as_stream(void *s) { return s ? static_cast<Stream *>(s) : &g_null_stream; }
+void violation(const char *fmt, ...) {
+  char buf[256];
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(buf, sizeof(buf), fmt, ap);
+  va_end(ap);
+  g_violations.emplace_back(buf);
+}
+// caller holds g_rt_mu: the host has waited for `s` (null: for every stream)
+void note_stream_idle(Stream *s) {
+  for (auto &kv : g_stage_writers)
+    if (s == nullptr || kv.second.first == s) kv.second.second = false;
+}
+void note_staged_launch(const ugk_stage_t &stage, void *stream) {
+  std::lock_guard<std::mutex> g(g_rt_mu);
+  auto &w = g_stage_writers[stage.owner_dev];
+  if (w.second && w.first != as_stream(stream))
+    violation("two extractions on different streams, with no wait between them, file rows in one stage");
+  w = {as_stream(stream), true};
+}
+// caller holds g_rt_mu
+void note_host_wait(const char *what) {
+  if (g_capture_active) violation("%s while a stream records into a graph", what);
+}
+bool referenced_by_live_graph(const void *obj) {
+  for (auto &kv : g_graphs) {
+    if (!kv.second.alive) continue;
+    for (auto *s : kv.second.streams)
+      if (s == obj) return true;
+    for (auto *e : kv.second.events)
+      if (e == obj) return true;
+  }
+  return false;
+}
 
 }  // namespace
+
+// hooks of the model itself (declared in ugk_cpu_model.h): the driver plays the caller that records a graph
+extern "C" {
+int ugk_model_capture_begin(void *stream) {
+  std::lock_guard<std::mutex> g(g_rt_mu);
+  Stream *s = as_stream(stream);
+  REQUIRE(g_capture_active == 0 && s->capture == 0, "ugk_model_capture_begin: a capture is active already");
+  g_capture_active = s->capture = g_capture_next++;
+  s->origin = true;
+  g_graphs[g_capture_active].streams.push_back(s);
+  return 0;
+}
+int ugk_model_capture_end(void *stream, int *graph_id) {
+  std::lock_guard<std::mutex> g(g_rt_mu);
+  Stream *s = as_stream(stream);
+  REQUIRE(s->origin && s->capture == g_capture_active && g_capture_active != 0,
+          "ugk_model_capture_end: no capture was begun on this stream");
+  Graph &graph = g_graphs[g_capture_active];
+  for (Stream *m : graph.streams) {
+    if (m != s && !m->joined_back) violation("a stream that joined the capture was not joined back before its end");
+    m->capture = 0;
+    m->origin = false;
+    m->join_event = nullptr;
+    m->joined_back = true;
+  }
+  if (graph_id) *graph_id = g_capture_active;
+  g_capture_active = 0;
+  return 0;
+}
+void ugk_model_graph_destroy(int graph_id) {
+  std::lock_guard<std::mutex> g(g_rt_mu);
+  auto it = g_graphs.find(graph_id);
+  if (it != g_graphs.end()) it->second.alive = false;
+}
+size_t ugk_model_violations(char *text, size_t capacity) {
+  std::lock_guard<std::mutex> g(g_rt_mu);
+  if (text && capacity) {
+    std::string all;
+    for (auto &v : g_violations) all += v + "\n";
+    snprintf(text, capacity, "%s", all.c_str());
+  }
+  return g_violations.size();
+}
+void ugk_model_reset(void) {
+  std::lock_guard<std::mutex> g(g_rt_mu);
+  g_violations.clear();
+  g_graphs.clear();
+  g_stage_writers.clear();
+}
+}
 
 extern "C" {
 
@@ -557,10 +678,26 @@ int ugk_mem_info(size_t *free_bytes, size_t *total_bytes) {
   if (total_bytes) *total_bytes = 64ull << 30;
   return 0;
 }
-int ugk_malloc(void **ptr, size_t nbytes) { return alloc_block(ptr, nbytes, 2); }
-int ugk_free(void *ptr) { return free_block(ptr, 2); }
-int ugk_host_malloc(void **ptr, size_t nbytes) { return alloc_block(ptr, nbytes, 1); }
-int ugk_host_free(void *ptr) { return free_block(ptr, 1); }
+static void note_allocation(const char *what) {
+  std::lock_guard<std::mutex> g(g_rt_mu);
+  if (g_capture_active) violation("%s while a stream records into a graph", what);
+}
+int ugk_malloc(void **ptr, size_t nbytes) {
+  note_allocation("device memory allocated");
+  return alloc_block(ptr, nbytes, 2);
+}
+int ugk_free(void *ptr) {
+  if (ptr) note_allocation("device memory freed");
+  return free_block(ptr, 2);
+}
+int ugk_host_malloc(void **ptr, size_t nbytes) {
+  note_allocation("pinned memory allocated");
+  return alloc_block(ptr, nbytes, 1);
+}
+int ugk_host_free(void *ptr) {
+  if (ptr) note_allocation("pinned memory freed");
+  return free_block(ptr, 1);
+}
 int ugk_pointer_kind(const void *ptr, int *kind) {
   std::lock_guard<std::mutex> g(g_mem_mu);
   *kind = 0;
@@ -572,49 +709,124 @@ int ugk_pointer_kind(const void *ptr, int *kind) {
   return 0;
 }
 int ugk_stream_create(void **stream) {
-  *stream = malloc(8);
-  return *stream ? 0 : fail("out of memory");
+  *stream = new Stream;
+  return 0;
 }
 int ugk_stream_create_cu_masked(void **stream, int num_cus) {
   REQUIRE(num_cus > 0, "ugk_stream_create_cu_masked: %d compute units", num_cus);
   return ugk_stream_create(stream);
 }
 int ugk_stream_destroy(void *stream) {
-  free(stream);
+  if (!stream) return 0;
+  {
+    std::lock_guard<std::mutex> g(g_rt_mu);
+    if (as_stream(stream)->capture) violation("a stream was destroyed while it records into a graph");
+    if (referenced_by_live_graph(stream)) violation("a stream that took part in a capture was destroyed while the graph lives");
+    for (auto &kv : g_graphs)
+      for (auto &m : kv.second.streams)
+        if (m == stream) m = nullptr;
+  }
+  delete static_cast<Stream *>(stream);
   return 0;
 }
-int ugk_stream_sync(void *) { return 0; }
-int ugk_stream_is_capturing(void *, int *capturing) {
-  *capturing = 0;
+int ugk_stream_sync(void *stream) {
+  std::lock_guard<std::mutex> g(g_rt_mu);
+  if (as_stream(stream)->capture) violation("the host waited for a stream that records into a graph");
+  note_stream_idle(as_stream(stream));
   return 0;
 }
-int ugk_stream_sync_ticket(void *, uint32_t *ticket_host, uint32_t value, unsigned) {
+int ugk_stream_is_capturing(void *stream, int *capturing) {
+  std::lock_guard<std::mutex> g(g_rt_mu);
+  *capturing = as_stream(stream)->capture != 0;
+  return 0;
+}
+int ugk_stream_sync_ticket(void *stream, uint32_t *ticket_host, uint32_t value, unsigned) {
   REQUIRE(ticket_host, "ugk_stream_sync_ticket: null ticket word");
+  {
+    std::lock_guard<std::mutex> g(g_rt_mu);
+    if (as_stream(stream)->capture) violation("the host waited for a ticket on a stream that records into a graph");
+    note_stream_idle(as_stream(stream));
+  }
   *ticket_host = value;
   return 0;
 }
-int ugk_device_sync(void) { return 0; }
+int ugk_device_sync(void) {
+  std::lock_guard<std::mutex> g(g_rt_mu);
+  note_host_wait("the host waited for the device");
+  note_stream_idle(nullptr);
+  return 0;
+}
 int ugk_event_create(void **event) {
   *event = new Event{std::chrono::steady_clock::now()};
   return 0;
 }
 int ugk_event_destroy(void *event) {
+  if (!event) return 0;
+  {
+    std::lock_guard<std::mutex> g(g_rt_mu);
+    if (referenced_by_live_graph(event)) violation("an event that was recorded into a capture was destroyed while the graph lives");
+    for (auto &kv : g_graphs)
+      for (auto &e : kv.second.events)
+        if (e == event) e = nullptr;
+  }
   delete static_cast<Event *>(event);
   return 0;
 }
-int ugk_event_record(void *event, void *) {
+int ugk_event_record(void *event, void *stream) {
   REQUIRE(event, "null event");
-  static_cast<Event *>(event)->at = std::chrono::steady_clock::now();
+  std::lock_guard<std::mutex> g(g_rt_mu);
+  Event *e = static_cast<Event *>(event);
+  Stream *s = as_stream(stream);
+  e->at = std::chrono::steady_clock::now();
+  e->captured_in = s->capture;
+  e->recorded_on = s;
+  if (s->capture) {
+    violation("an event was recorded on a stream that records into a graph: it belongs to the caller's capture now");
+    g_graphs[s->capture].events.push_back(event);
+    if (!s->origin) s->join_event = event;
+  }
   return 0;
 }
-int ugk_event_sync(void *) { return 0; }
-int ugk_event_query(void *, int *complete) {
+int ugk_event_sync(void *event) {
+  REQUIRE(event, "null event");
+  std::lock_guard<std::mutex> g(g_rt_mu);
+  if (static_cast<Event *>(event)->captured_in) violation("the host waited for a captured event");
+  return 0;
+}
+int ugk_event_query(void *event, int *complete) {
+  REQUIRE(event && complete, "null pointer");
+  std::lock_guard<std::mutex> g(g_rt_mu);
+  if (static_cast<Event *>(event)->captured_in) violation("the host queried a captured event");
   *complete = 1;
   return 0;
 }
-int ugk_stream_wait_event(void *, void *) { return 0; }
+int ugk_stream_wait_event(void *stream, void *event) {
+  REQUIRE(event, "null event");
+  std::lock_guard<std::mutex> g(g_rt_mu);
+  Event *e = static_cast<Event *>(event);
+  Stream *s = as_stream(stream);
+  const bool live_capture = e->captured_in != 0 && e->captured_in == g_capture_active;
+  if (live_capture && s->capture == 0) {
+    // the waiting stream joins the capture the event belongs to
+    violation("a second stream joined the caller's capture by waiting for a captured event");
+    s->capture = e->captured_in;
+    s->joined_back = false;
+    g_graphs[s->capture].streams.push_back(s);
+  } else if (live_capture && s->capture == e->captured_in) {
+    Stream *from = e->recorded_on;
+    if (from && from != s && !from->origin && from->join_event == event) from->joined_back = true;
+  } else if (s->capture != 0 && !live_capture) {
+    violation("a stream that records into a graph waited for an event recorded outside the capture");
+  } else if (e->captured_in != 0) {
+    violation("a stream waited for a captured event of a capture that has ended");
+  }
+  return 0;
+}
 int ugk_event_elapsed_ms(void *start, void *stop, float *ms) {
   REQUIRE(start && stop && ms, "null event");
+  std::lock_guard<std::mutex> g(g_rt_mu);
+  if (static_cast<Event *>(start)->captured_in || static_cast<Event *>(stop)->captured_in)
+    violation("the time between captured events was asked for");
   *ms = std::chrono::duration<float, std::milli>(static_cast<Event *>(stop)->at - static_cast<Event *>(start)->at)
             .count();
   return 0;
@@ -813,16 +1025,18 @@ int ugk_extract_pool_i64(ugk_table_t t, const int64_t *ids, const int64_t *seg_o
 int ugk_extract_mix_staged_u32(ugk_table_t t, const uint32_t *keys, size_t n, const void *cache, uint64_t cache_rows,
                                const void *host, uint64_t host_rows, void *out, size_t rb, uint32_t *status,
                                uint32_t *mirror, uint64_t *counts, uint32_t *num_groups, uint32_t, ugk_stage_t stage,
-                               void *) {
+                               void *stream) {
   REQUIRE(stage.rows_dev && stage.owner_dev && stage.epoch, "ugk_extract_mix_staged: bad stage");
+  note_staged_launch(stage, stream);
   return extract_mix(t, keys, n, cache, cache_rows, host, host_rows, out, rb, status, mirror, counts, num_groups,
                      &stage);
 }
 int ugk_extract_mix_staged_i64(ugk_table_t t, const int64_t *keys, size_t n, const void *cache, uint64_t cache_rows,
                                const void *host, uint64_t host_rows, void *out, size_t rb, uint32_t *status,
                                uint32_t *mirror, uint64_t *counts, uint32_t *num_groups, uint32_t, ugk_stage_t stage,
-                               void *) {
+                               void *stream) {
   REQUIRE(stage.rows_dev && stage.owner_dev && stage.epoch, "ugk_extract_mix_staged: bad stage");
+  note_staged_launch(stage, stream);
   return extract_mix(t, keys, n, cache, cache_rows, host, host_rows, out, rb, status, mirror, counts, num_groups,
                      &stage);
 }

@@ -1596,32 +1596,71 @@ def test_stream_ordered_pooled_lookups(pct, table_kind, kdtype, monkeypatch):
     assert m == len(want_k) and np.array_equal(got_k[:m], want_k) and np.array_equal(got_c[:m], want_c)
 
 
-@pytest.mark.skip(reason="a run of this combination (a stream-ordered pooled lookup recorded into a graph while the "
-                         "session counted hotness on its own stream) passed its comparisons and then did not return "
-                         "from coll_cache_shutdown; the cause is not established.  Since then a lookup that is being "
-                         "recorded into a graph is not counted, and the combination stays off the GPU")
-def test_stream_ordered_pooled_lookup_recorded_into_a_graph_with_device_counters(monkeypatch):
+@pytest.mark.parametrize("pooled,pct", [(True, 1.0), (False, 1.0), (False, 0.25)])
+def test_stream_ordered_lookup_recorded_into_a_graph_with_device_counters(pooled, pct, monkeypatch):
+    """COLL_GPU_RECORD=1 and a stream-ordered lookup (pooled or plain) that the caller records into a graph: the
+    counting is one more kernel of that graph on the caller's stream -- no stream and no event of the session takes part
+    in the capture -- so every replay gives the eager result and counts the keys it read; the ranking drained afterwards
+    equals the oracle's ranking of the eager batches plus one batch per replay.  The graph is destroyed before the
+    shutdown in one case and outlives it in the others."""
     monkeypatch.setenv("COLL_GPU_RECORD", "1")
     rng = np.random.default_rng(78)
-    n_item, dim = 30_000, 32
-    co.config(make_config(n_item, 1.0))
+    n_item, dim, n = 30_000, 32, 4000
+    co.config(make_config(n_item, pct))
     co.coll_cache_record_init(0)
+    s0 = rng.integers(0, n_item, size=60_000)
+    if pct < 1.0:
+        co.coll_torch_record(0, torch.from_numpy(s0).to(torch.int32))
     emb = co.coll_torch_create_emb_shm(0, n_item, dim, torch.float32)
     emb.copy_(torch.from_numpy(rng.standard_normal((n_item, dim)).astype(np.float32)))
-    co.coll_torch_init_t(0, 0, emb, 1.0)
-    off = np.arange(0, 4001, 4, dtype=np.int64)
-    t_ids, t_off = torch.from_numpy(rng.integers(0, n_item, size=4000)).cuda(), torch.from_numpy(off).cuda()
-    want = co.coll_torch_lookup_pooled(0, t_ids, t_off, None, "mean").cpu()
-    result = torch.zeros_like(want, device="cuda")
+    co.coll_torch_init_t(0, 0, emb, pct)
+    t_ids = torch.zeros(n, dtype=torch.int64, device="cuda")
+    t_off = torch.from_numpy(np.arange(0, n + 1, 4, dtype=np.int64)).cuda()
+
+    def lookup(stream_ordered):
+        if pooled:
+            return co.coll_torch_lookup_pooled(0, t_ids, t_off, None, "mean", stream_ordered=stream_ordered)
+        return co.coll_torch_lookup_async(0, t_ids, False) if stream_ordered else \
+            co.coll_torch_lookup_key_t_val_ret(0, t_ids, False)
+
+    counted = []
+    first = rng.integers(0, n_item, size=n)
+    t_ids.copy_(torch.from_numpy(first))
+    warm = lookup(True)  # outside the capture: reused buffers get allocated here
+    co.coll_torch_lookup_wait(0)
+    counted.append(first.astype(np.uint32))
+    result = torch.zeros_like(warm)
     g = torch.cuda.CUDAGraph()
     with torch.cuda.graph(g):
-        result.copy_(co.coll_torch_lookup_pooled(0, t_ids, t_off, None, "mean", stream_ordered=True))
+        result.copy_(lookup(True))  # recorded, not run: nothing is counted here
     for it in range(3):
+        q = rng.integers(0, n_item, size=n)
+        t_ids.copy_(torch.from_numpy(q))
         result.zero_()
         g.replay()
         torch.cuda.synchronize()
-        assert result.cpu().numpy().tobytes() == want.numpy().tobytes(), it
+        counted.append(q.astype(np.uint32))
+        eager = lookup(False)  # eager work between the replays, counted on the session's own stream
+        counted.append(q.astype(np.uint32))
+        assert result.cpu().numpy().tobytes() == eager.cpu().numpy().tobytes(), it
     co.coll_torch_lookup_wait(0)
+    if pct == 1.0 and pooled:
+        del g  # the caller lets go of its graph before the shutdown; the other cases keep it beyond
+    want_k, want_c = ORC.freq_rank(np.concatenate(counted))
+    got_k, got_c = np.zeros(n_item, np.uint32), np.zeros(n_item, np.uint32)
+    m = _basics.C_LIB_CTYPES.coll_cache_rank_hotness(0, got_k.ctypes.data, got_c.ctypes.data, n_item)
+    assert m == len(want_k) and np.array_equal(got_k[:m], want_k) and np.array_equal(got_c[:m], want_c)
+    if pct < 1.0:  # a refresh on the device-side counts of replays and eager lookups, then one more replay
+        q = rng.integers(0, n_item // 8, size=n)
+        t_ids.copy_(torch.from_numpy(q))
+        for _ in range(3):
+            g.replay()
+        torch.cuda.synchronize()
+        co.coll_torch_refresh(0, True)
+        g.replay()
+        torch.cuda.synchronize()
+        assert result.cpu().numpy().tobytes() == lookup(False).cpu().numpy().tobytes()
+    co.coll_torch_shutdown()  # with the graph alive (unless deleted above); the fixture's second shutdown finds nothing
 
 
 @pytest.mark.parametrize("impl", ["", "SMMaskPhase"])

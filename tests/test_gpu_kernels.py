@@ -756,7 +756,10 @@ def test_pooled_extraction_hand_worked(rows_per_group, monkeypatch):
         # offsets that leave the ids (beyond nnz, negative, running backwards) flag the launch, read nothing and
         # give rows of zeros; the other rows are unharmed
         key = np.array([1, 2, 3, 4, 4])
-        for broken in ([0, 2, 3, 3, 9], [0, 2, 3, 3, 1 << 40], [0, 2, -7, 3, 5], [0, 4, 3, 3, 5]):
+        # offsets that stay inside the ids but do not begin at 0 or end at nnz flag the launch as well: the rows are what
+        # the offsets say, the per-source counts of ids would not add up to nnz
+        for broken in ([0, 2, 3, 3, 9], [0, 2, 3, 3, 1 << 40], [0, 2, -7, 3, 5], [0, 4, 3, 3, 5], [1, 2, 3, 3, 5],
+                       [0, 2, 3, 3, 4]):
             st.zero_()
             boff = to_dev(np.array(broken, np.int64))
             out = dev_bytes(4 * 16, fill=0x55)

@@ -90,6 +90,22 @@ def test_static_scratch_dedup_matches_the_workspace_one(kdtype):
     hip.call("ugk_dedup_static", None, 8, 0, None, None, None, ptr(nu), None, None)
     sync()
     assert int(nu.cpu()[0]) == 0
+    # ... also in the pinned word that mirrors it, which still holds the count of the batch before
+    from gpu_util import PinnedArray
+    host_word = PinnedArray((4,), np.uint32)
+    try:
+        keys = to_dev(np.array([5, 5, 9], kdtype))
+        uniq, inv = dev_bytes(3 * 8), dev_zeros_u32(3)
+        hip.call("ugk_dedup_static", ptr(keys), keys.element_size(), 3, ptr(uniq), ptr(inv), None, ptr(nu),
+                 host_word.ptr, None)
+        sync()
+        assert int(host_word.array[0]) == 2
+        hip.call("ugk_dedup_static", None, 8, 0, None, None, None, ptr(nu), host_word.ptr, None)
+        sync()
+        assert int(host_word.array[0]) == 0 and int(nu.cpu()[0]) == 0
+    finally:
+        sync()
+        host_word.free()
 
 
 def test_static_scratch_dedup_refuses_what_does_not_fit():

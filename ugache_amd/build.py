@@ -93,14 +93,9 @@ def build_host(verbose=False):
     return HOST_LIB
 
 
-def build_oracle():
-    _run(["make", "-B", "-C", os.path.join(ROOT, "oracle")])
-
-
 def build_all(verbose=False):
     build_hip(verbose)
     build_host(verbose)
-    build_oracle()
 
 
 if __name__ == "__main__":

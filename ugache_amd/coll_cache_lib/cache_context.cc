@@ -326,8 +326,9 @@ void ExtractSession::CheckStatusWord(StreamHandle stream) const {
                                  std::to_string(_cache_ctx->_num_total_nodes) + ")"
                            : "")
                    << ((st & UGK_ST_BAD_SEGMENT)
-                           ? ": the offsets of a pooled lookup leave the list of ids or run backwards (or the rows "
-                             "they were made from are not in ascending order inside [0, num_rows))"
+                           ? ": the offsets of a pooled lookup leave the list of ids, run backwards or do not span "
+                             "it from 0 to the number of ids (or the rows they were made from are not in ascending "
+                             "order inside [0, num_rows))"
                            : "");
 }
 
@@ -380,27 +381,50 @@ static int Record(const Id64Type *keys, size_t n, uint64_t mul, uint64_t mask, u
 // the caller's stream wait for it before the lookup returns (the keys belong to the caller again after that).
 // RecordBegin marks that point and says whether this lookup is counted at all; the extraction kernels are launched
 // next, and only then RecordLaunch enqueues the counting: its handful of API calls then run while the GPU already
-// works on the batch instead of in front of it.
-void *ExtractSession::RecordBegin(StreamHandle stream) {
+// works on the batch instead of in front of it.  A lookup that the caller is recording into a HIP graph is counted
+// by a record kernel on the caller's own stream instead (RecordPlan in the header says why).
+ExtractSession::RecordPlan ExtractSession::RecordBegin(StreamHandle stream) {
   _record_pending = false;
-  if (!_hot_counts) return nullptr;
-  // A lookup that a caller records into a HIP graph is not counted: the counting runs on a stream of this session,
-  // which would become part of the caller's graph.
+  RecordPlan plan;
+  if (!_hot_counts) return plan;
   int capturing = 0;
   UGK_CALL(ugk_stream_is_capturing(stream, &capturing));
-  if (capturing) return nullptr;
-  if ((_num_lookups++ % RunConfig::gpu_record_every) != 0) return nullptr;
+  if (capturing == UGK_CAPTURE_QUERY_REFUSED) {
+    // the runtime refuses the query where the stream may not be used at all (the legacy default stream while another
+    // stream of the process records a graph): nothing is counted, and the launch that follows reports the misuse
+    if (!_capture_query_refused_logged)
+      LOG(WARNING) << "the capture state of the lookup's stream cannot be queried; this lookup is not counted";
+    _capture_query_refused_logged = true;
+    return plan;
+  }
+  if ((_num_lookups++ % RunConfig::gpu_record_every) != 0) return plan;
+  if (capturing) {
+    // A lookup that the caller records into a HIP graph: the record stream and the events of this session stay out of
+    // that graph (see RecordPlan).  Every replay counts the keys the replayed lookup reads.
+    plan.kind = RecordPlan::kCallersStream;
+    plan.stream = stream;
+    _counted_on_callers_stream.store(true);
+    return plan;
+  }
   UGK_CALL(ugk_event_record(_ev_rec_begin, stream));
-  return _ev_rec_begin;
+  plan.kind = RecordPlan::kRecordStream;
+  plan.after = _ev_rec_begin;
+  return plan;
 }
 
 template <typename KeyT>
-void ExtractSession::RecordLaunch(const KeyT *nodes, size_t num_nodes, void *after) {
-  if (after == nullptr) return;
+void ExtractSession::RecordLaunch(const KeyT *nodes, size_t num_nodes, const RecordPlan &plan) {
+  if (plan.kind == RecordPlan::kNone) return;
   num_nodes = std::min(num_nodes, _record_limit);
   if (num_nodes == 0) return;
+  if (plan.kind == RecordPlan::kCallersStream) {
+    // in stream order behind the extraction, nothing to join
+    UGK_CALL(Record(nodes, num_nodes, RunConfig::key_map_inv, RunConfig::key_map_mask, _hot_counts->ptr<uint32_t>(),
+                    _cache_ctx->_num_total_nodes, ObservedBits(), _status, _host_mirror, plan.stream));
+    return;
+  }
   std::lock_guard<std::mutex> guard(_enqueue_mu);  // not in the middle of a placement's passes
-  UGK_CALL(ugk_stream_wait_event(_record_stream, after));
+  UGK_CALL(ugk_stream_wait_event(_record_stream, plan.after));
   UGK_CALL(Record(nodes, num_nodes, RunConfig::key_map_inv, RunConfig::key_map_mask, _hot_counts->ptr<uint32_t>(),
                   _cache_ctx->_num_total_nodes, ObservedBits(), _status, _host_mirror, _record_stream));
   UGK_CALL(ugk_event_record(_ev_rec_done, _record_stream));
@@ -413,7 +437,10 @@ void ExtractSession::RecordKeys(const KeyT *nodes, size_t num_nodes, StreamHandl
   _record_pending = false;
   if (!_hot_counts || (_num_lookups++ % RunConfig::gpu_record_every) != 0) return;
   (void)stream;
-  RecordLaunch(nodes, num_nodes, after);
+  RecordPlan plan;
+  plan.kind = RecordPlan::kRecordStream;
+  plan.after = after;
+  RecordLaunch(nodes, num_nodes, plan);
 }
 
 void ExtractSession::JoinRecord(StreamHandle stream) {
@@ -437,6 +464,13 @@ void ExtractSession::PlaceOnDevice(size_t num_cached, uint64_t *in_new_bits, uin
   const size_t rows = _cache_ctx->_num_total_nodes;
   std::lock_guard<std::mutex> no_drain(_drain_mu);
   std::lock_guard<std::mutex> guard(_enqueue_mu);
+  if (_counted_on_callers_stream.load()) {
+    // replays of a graph that counts run on the caller's stream, not on the record stream: the passes below start
+    // behind whatever that stream holds at this point (a refresh that shares the stream of the replays, the usual
+    // case, is thereby ordered against all of them; replays launched from elsewhere while the passes run are not)
+    UGK_CALL(ugk_event_record(_ev_placed, stream));
+    UGK_CALL(ugk_stream_wait_event(_record_stream, _ev_placed));
+  }
   UGK_CALL(ugk_rank_place_keep(_hot_counts->ptr<uint32_t>(), rows, num_cached, rank_ws, in_new_bits, scratch_bits,
                                ObservedBits(), keep_bits, reset_counts ? 1 : 0, _record_stream));
   UGK_CALL(ugk_event_record(_ev_placed, _record_stream));
@@ -711,7 +745,7 @@ void ExtractSession::ExtractFeatImpl(const KeyT *nodes, size_t num_nodes, void *
     // the logged combine time: a host timer around launch and wait, as in the reference (Timer around Combine + StreamSync,
     // cache_context.cu:1206-1216, 1312-1315), or with COLL_KERNEL_EVENTS=1 the kernel's duration from an event pair on its
     // stream, which costs 1.9 us per step
-    void *keys_ready = RecordBegin(stream);
+    const RecordPlan keys_ready = RecordBegin(stream);
     const bool events = RunConfig::kernel_events;
     Timer t_host;
     if (events) UGK_CALL(ugk_event_record(_ev_t[0], stream));
@@ -774,7 +808,7 @@ void ExtractSession::ExtractFeatImpl(const KeyT *nodes, size_t num_nodes, void *
     // host link is busy from the first wavefront on, with no classify pass and no cross-stream hand-off in front of
     // it, and since the link bounds a mixed batch it does not matter that host loads spread over the chip slow the
     // HBM loads next to them.
-    void *keys_ready = RecordBegin(stream);
+    const RecordPlan keys_ready = RecordBegin(stream);
     const bool events = RunConfig::kernel_events;
     Timer t_host;
     if (events) UGK_CALL(ugk_event_record(_ev_t[0], stream));
@@ -783,7 +817,7 @@ void ExtractSession::ExtractFeatImpl(const KeyT *nodes, size_t num_nodes, void *
     // from outside the cache), not guessed from the previous batch.
     const uint32_t hint = skip_local ? (uint32_t)num_nodes : UGK_HINT_UNKNOWN;
     UGK_CALL(ExtractMix(table, nodes, num_nodes, cache, cache_rows, host, host_rows, output, rb, _status,
-                        _host_mirror, _mix_counts->ptr<uint64_t>(), &_mix_groups, hint, NextStage(), stream));
+                        _host_mirror, _mix_counts->ptr<uint64_t>(), &_mix_groups, hint, NextStage(stream, false), stream));
     if (events) UGK_CALL(ugk_event_record(_ev_t[1], stream));
     RecordLaunch(input_nodes, num_input, keys_ready);
     WaitForBatch(stream);
@@ -917,7 +951,7 @@ void ExtractSession::ExtractFeatAsyncImpl(const KeyT *nodes, size_t num_nodes, v
   InFlight enqueueing(this);
   if (ctx->IsDirectMapping() && !dedup) {
     const bool from_host = ctx->_cpu_location_id != -1;
-    void *keys_ready = RecordBegin(stream);
+    const RecordPlan keys_ready = RecordBegin(stream);
     UGK_CALL(GatherDirect(ctx->_device_cache_data[0], ctx->_num_total_nodes, nodes, num_nodes, output, rb,
                           from_host ? _cpu_blocks : 0, _status, _host_mirror, stream));
     RecordLaunch(nodes, num_nodes, keys_ready);
@@ -931,12 +965,12 @@ void ExtractSession::ExtractFeatAsyncImpl(const KeyT *nodes, size_t num_nodes, v
              (((uintptr_t)ctx->_device_cache_data[ctx->_local_location_id] |
                (uintptr_t)ctx->_device_cache_data[ctx->_cpu_location_id] | (uintptr_t)output | (uintptr_t)rb) &
               15u) == 0) {
-    void *keys_ready = RecordBegin(stream);
+    const RecordPlan keys_ready = RecordBegin(stream);
     UGK_CALL(ExtractMix(ctx->_new_hash_table->Table(), nodes, num_nodes,
                         ctx->_device_cache_data[ctx->_local_location_id], ctx->_cache_space_capacity,
                         ctx->_device_cache_data[ctx->_cpu_location_id], ctx->_num_total_nodes, output, rb, _status,
-                        _host_mirror, _mix_counts->ptr<uint64_t>(), &_mix_groups, UGK_HINT_UNKNOWN, NextStage(),
-                        stream));
+                        _host_mirror, _mix_counts->ptr<uint64_t>(), &_mix_groups, UGK_HINT_UNKNOWN,
+                        NextStage(stream, true), stream));
     RecordLaunch(nodes, num_nodes, keys_ready);
     JoinRecord(stream);
     _async_last_fused = true;
@@ -1029,6 +1063,7 @@ void ExtractSession::WaitForLookupsInFlight(bool foreground, double timeout_s) {
 void ExtractSession::Wait(StreamHandle stream) {
   if (_async_pending == 0) return;
   UGK_CALL(ugk_stream_sync(stream));
+  if (stream == _stage_writer) _stage_writer_busy = false;
   CheckStatusWord(stream);
   if (_async_last_fused) SumMixCounts();
   uint32_t n_local = _host_mirror[kMirGroupSizes + UGK_LOC_LOCAL], n_miss = _host_mirror[kMirGroupSizes + UGK_LOC_HOST];
@@ -1073,7 +1108,7 @@ bool ExtractSession::LaunchPooled(const KeyT *nodes, const int64_t *seg_off, con
     cache_rows = ctx->_cache_space_capacity;
   }
   CHECK((((uintptr_t)cache | (uintptr_t)host | (uintptr_t)output) & 15u) == 0) << "pooled lookup: misaligned buffer";
-  void *keys_ready = RecordBegin(stream);
+  const RecordPlan keys_ready = RecordBegin(stream);
   UGK_CALL(ExtractPool(table, nodes, seg_off, weights, num_rows, num_nodes, combiner, elem_bytes, cache, cache_rows,
                        host, ctx->_num_total_nodes, output, rb, _status, _host_mirror, _mix_counts->ptr<uint64_t>(),
                        &_mix_groups, stream));
@@ -1239,10 +1274,11 @@ void RefreshSession::CopyRowsIntoSlots(const uint32_t *rows_dev, const uint32_t 
     table->PublishRows(rows, slots, n, local, __publish_ids, ctx->_eager_gpu_mem_allocator, gpu_ctx, copy_stream);
   };
   if (foreground) {
-    // Nothing runs beside a foreground refresh: one launch copies every row, from the stage where it holds it (most of
-    // the rows a refresh brings in were missed by the last few lookups, which filed them in HBM) or from the host
-    // table, on a capped grid: rows of 512 bytes and more cross the link faster from 128 workgroups than from as many
-    // as the rows would fill (56.9 against 52.7 GB/s).  One more launch publishes them.
+    // Nothing runs beside a foreground refresh: one launch copies every row.  Without a stage all of them cross the host
+    // link, on a capped grid: rows of 512 bytes and more cross it faster from 128 workgroups than from as many as the
+    // rows would fill (56.9 against 52.7 GB/s).  With a stage most rows are read from HBM (they were missed by the last
+    // few lookups, which filed them there), which wants the whole chip, so that launch is not capped and the few rows
+    // the stage does not hold cross the link at the lower of the two rates.  One more launch publishes them.
     if (stage)
       UGK_CALL(ugk_gather_scatter_staged_u32(host, ctx->_num_total_nodes, rows_dev, slots_dev, num_rows, cache,
                                              ctx->_cache_space_capacity, ctx->_row_bytes, *stage, 0, status, status + 8,

@@ -143,9 +143,21 @@ class ExtractSession {
   static constexpr size_t kHotDrainRows = 32u << 20;  // rows per drain step = capacity of the entry list
   template <typename KeyT>
   void RecordKeys(const KeyT *nodes, size_t num_nodes, StreamHandle stream, void *after);
-  void *RecordBegin(StreamHandle stream);
+  // How the keys of the lookup that is being enqueued get counted on the device: not at all, by a record kernel on
+  // the session's record stream behind the event `after` (which the caller's stream has recorded), or by a record
+  // kernel on the caller's own stream.  The last is for a lookup that the caller is recording into a HIP graph: no
+  // stream and no event of the session may become part of a graph that the caller owns, replays and destroys when it
+  // likes, so there the counting is one more kernel node of that graph, behind the extraction.
+  struct RecordPlan {
+    enum Kind { kNone, kRecordStream, kCallersStream } kind = kNone;
+    void *after = nullptr;
+    StreamHandle stream = nullptr;
+  };
+  RecordPlan RecordBegin(StreamHandle stream);
   template <typename KeyT>
-  void RecordLaunch(const KeyT *nodes, size_t num_nodes, void *after);
+  void RecordLaunch(const KeyT *nodes, size_t num_nodes, const RecordPlan &plan);
+  bool _capture_query_refused_logged = false;
+  std::atomic<bool> _counted_on_callers_stream{false};  // some lookup was recorded into a graph together with its counting
 
   MemHandle _mix_counts;           // pinned: one word per workgroup of the fused kernel, its two row counts
   uint32_t _mix_groups = 0;        // workgroups of the last fused launch
@@ -167,8 +179,17 @@ class ExtractSession {
   void AllocStage(int which, StreamHandle stream);
   // Called after the lookup has counted itself in flight (InFlight): a refresh that switched the stages before it
   // sampled that count then either sees this lookup in the count or this lookup sees the switch.
-  const ugk_stage_t *NextStage() {
+  // Rows are filed by the launches of one stream at a time: launches on one stream run one after the other, launches
+  // on two streams may overlap, and two overlapping launches could both claim an entry and mix the bytes of two rows
+  // in it.  A lookup on another stream than the last one that filed rows gets no stage while that one may still run
+  // (a stream-ordered lookup that has not been waited for); a blocking lookup has finished when it returns.
+  StreamHandle _stage_writer = nullptr;
+  bool _stage_writer_busy = false;
+  const ugk_stage_t *NextStage(StreamHandle stream, bool stream_ordered) {
     if (_stage_entries == 0) return nullptr;
+    if (_stage_writer_busy && stream != _stage_writer) return nullptr;
+    _stage_writer = stream;
+    _stage_writer_busy = stream_ordered;
     _stage_launch = _stages[_stage_active.load()];
     if (++_stage_epoch == 0) _stage_epoch = 1;
     _stage_launch.epoch = _stage_epoch;

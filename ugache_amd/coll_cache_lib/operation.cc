@@ -604,15 +604,19 @@ void ForwardStep(int replica_id, const KeyT *key, size_t num_keys, StreamHandle 
     kInline,    // this thread after the blocking lookup, from a copy a kernel in front of the lookup makes
     kDeferred,  // a later step (or the wait, or the ranking), from such a copy: the step is enqueued and left
   } prefix = Prefix::kNone;
+  // A step that the caller is recording into a HIP graph is not a step of the loop: it runs when the caller replays
+  // it.  Its prefix is counted where the device counts (the counting is part of the recorded lookup); the host cannot
+  // count what a replay copies.  It starts no refresh either: the refresh thread would wait for a stream that records.
+  int capturing = 0;
+  if (stream_ordered) UGK_CALL(ugk_stream_is_capturing(stream, &capturing));
   if (num_record > 0) {
     const bool small = record_bytes <= RunConfig::record_inline_bytes && reinterpret_cast<uintptr_t>(key) % 16 == 0;
     if (RunConfig::gpu_record) {
       prefix = Prefix::kDevice;
+    } else if (capturing) {
+      prefix = Prefix::kNone;
     } else if (small && stream_ordered) {
-      // a step that is being recorded into a HIP graph records nothing: the host cannot count what a replay copies
-      int capturing = 0;
-      UGK_CALL(ugk_stream_is_capturing(stream, &capturing));
-      prefix = capturing ? Prefix::kNone : Prefix::kDeferred;
+      prefix = Prefix::kDeferred;
     } else {
       prefix = small ? Prefix::kInline : Prefix::kThread;
     }
@@ -646,6 +650,7 @@ void ForwardStep(int replica_id, const KeyT *key, size_t num_keys, StreamHandle 
     case Prefix::kDeferred:
     case Prefix::kNone: break;
   }
+  if (capturing) return;
   const bool due = fw.enable_refresh && fw.refresh_iter > 0 &&
                    (fw.periodic ? (fw.step > 0 && fw.step % fw.refresh_iter == 0) : fw.step == fw.refresh_iter);
   if (due) {

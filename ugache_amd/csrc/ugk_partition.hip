@@ -409,10 +409,11 @@ __global__ __launch_bounds__(kBlock) void static_wrap_kernel(const uint32_t *epo
   for (size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x; i < cap; i += (size_t)gridDim.x * kBlock) slots[i] = 0ull;
 }
 
-__global__ void static_epoch_kernel(uint32_t *epoch, uint32_t *n_unique) {
+__global__ void static_epoch_kernel(uint32_t *epoch, uint32_t *n_unique, uint32_t *n_unique_host) {
   const uint32_t e = *epoch;
   *epoch = e == 0xffffffffu ? 1u : e + 1u;
   *n_unique = 0u;
+  if (n_unique_host) *n_unique_host = 0u;  // an empty batch launches nothing else; a full one overwrites it
 }
 
 size_t dedup_capacity(size_t n) {
@@ -766,7 +767,8 @@ int ugk_dedup_static(const void *keys_dev, uint32_t key_bytes, size_t n, void *u
   hipLaunchKernelGGL(static_wrap_kernel, dim3(clamp_grid(1024, 0)), dim3(kBlock), 0, as_stream(stream),
                      epoch_dev, reinterpret_cast<unsigned long long *>(ws), cap);
   UGK_HIP(hipGetLastError());
-  hipLaunchKernelGGL(static_epoch_kernel, dim3(1), dim3(1), 0, as_stream(stream), epoch_dev, n_unique_dev);
+  hipLaunchKernelGGL(static_epoch_kernel, dim3(1), dim3(1), 0, as_stream(stream), epoch_dev, n_unique_dev,
+                     n_unique_host);
   UGK_HIP(hipGetLastError());
   if (n == 0) return 0;
   if (key_bytes == 4)

@@ -106,6 +106,11 @@ __global__ __launch_bounds__(kBlock) void extract_pool_kernel(ugk_table_t t, con
         if (host_mirror) host_mirror[0] = UGK_ST_BAD_SEGMENT;
       }
       beg = end = 0;
+    } else if (row_ok && sub == 0 && ((r == 0 && beg != 0) || (r + 1 == n_rows && end != nnz))) {
+      // the offsets do not cover the ids from the first to the last (neighbouring segments share their boundary word,
+      // so the two ends are all that can be wrong): the per-source id counts would not add up to nnz
+      atomicOr(status, UGK_ST_BAD_SEGMENT);
+      if (host_mirror) host_mirror[0] = UGK_ST_BAD_SEGMENT;
     }
     float acc[kPoolChunks][EPC];
 #pragma unroll
@@ -230,6 +235,10 @@ __global__ __launch_bounds__(kBlock) void extract_pool_rows_kernel(ugk_table_t t
         if (host_mirror) host_mirror[0] = UGK_ST_BAD_SEGMENT;
       } else {
         beg = b, len = (uint32_t)(e - b);
+        if ((g0 + sub == 0 && b != 0) || (g0 + sub + 1 == n_rows && e != nnz)) {  // the ids are not covered end to end
+          atomicOr(status, UGK_ST_BAD_SEGMENT);
+          if (host_mirror) host_mirror[0] = UGK_ST_BAD_SEGMENT;
+        }
       }
     }
     uint32_t incl = len;  // inclusive prefix over the group's rows (lanes past the owned rows add nothing)

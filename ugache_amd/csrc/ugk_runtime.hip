@@ -198,13 +198,12 @@ int ugk_stream_is_capturing(void *stream, int *capturing) {
   hipStreamCaptureStatus st = hipStreamCaptureStatusNone;
   if (hipStreamIsCapturing(as_stream(stream), &st) != hipSuccess) {
     // the query itself is refused where it would touch a capture (the default stream while another stream of the
-    // process records in global mode): then work enqueued here would be refused too, which is what "capturing" means
-    // to the callers
+    // process records in global mode): work enqueued here would be refused too, and the caller is told so
     (void)hipGetLastError();
-    *capturing = 1;
+    *capturing = UGK_CAPTURE_QUERY_REFUSED;
     return 0;
   }
-  *capturing = st != hipStreamCaptureStatusNone;
+  *capturing = st != hipStreamCaptureStatusNone ? 1 : 0;
   return 0;
 }
 
