@@ -16,6 +16,11 @@ flagged an error (the parity tests check results).
   pooled    a multi-hot feature through the library: lookup + weighted combination per sample in one call
             (coll_torch_lookup_pooled) against the lookup of all ids followed by torch's index_add_ segment sum, and
             against unique -> lookup -> index_select -> index_add_ (the reference's sparse layer), by ids per sample
+  link_latency  what bounds rows of 128 bytes read out of pinned host memory: (a) the latency of one dependent read, from a
+            single lane that follows a chain of links scattered over the first S GiB of a 60 GiB allocation (and over
+            HBM for comparison); (b) the rate of independent row reads by the number of bytes in flight (workgroups x
+            loads in flight per lane), which shows where the link stops answering faster; (c) where the allocation's
+            pages live (/proc/self/numa_maps).  Kernels: bench_probes_kernels.hip (libbench_probes.so)
   sparse_layer  the serving stack's SparseLookupLayer end to end (a ps_config file and a model directory written to a
             temporary folder, Config -> record_hotness -> Init -> layer calls): the reference's steps (unique, lookup,
             gather, weighted segment sum), the same with the unique inside the library, and lookup + combination in
@@ -478,13 +483,142 @@ def probe_sparse_layer(hip, torch, note, quick=False):
             "host clock around the calls, one synchronisation at the end", "rows": out_rows}
 
 
-PROBES = {"sparse_layer": probe_sparse_layer, "pooled": probe_pooled, "kpw": probe_kpw, "row_span": probe_row_span, "cu_mask": probe_cu_mask, "small_batch": probe_small_batch}
+def _probe_lib():
+    """libbench_probes.so, built beside this file by __graft_entry__.build() from bench_probes_kernels.hip"""
+    path = os.path.join(os.path.dirname(os.path.abspath(__file__)), "libbench_probes.so")
+    if not os.path.exists(path):
+        sys.exit("probe link_latency needs libbench_probes.so: run `python __graft_entry__.py` first")
+    lib = C.CDLL(path)
+    lib.bp_last_error.restype = C.c_char_p
+    lib.bp_chase.argtypes = [C.c_void_p, C.c_uint64, C.c_uint64, C.c_uint64, C.c_void_p, C.c_void_p]
+    lib.bp_rows_inflight.argtypes = [C.c_void_p, C.c_uint32, C.c_void_p, C.c_size_t, C.c_int, C.c_uint, C.c_void_p,
+                                     C.c_void_p]
+
+    def call(name, *args):
+        if getattr(lib, name)(*args) != 0:
+            sys.exit("probe link_latency: %s" % lib.bp_last_error().decode())
+    return call
+
+
+def _numa_placement(addr):
+    """the /proc/self/numa_maps line of the mapping that holds `addr`: policy, pages per node, page size"""
+    try:
+        best = None
+        with open("/proc/self/numa_maps") as f:
+            for line in f:
+                start = int(line.split()[0], 16)
+                if start <= addr and (best is None or start > best[0]):
+                    best = (start, line.strip())
+        online = open("/sys/devices/system/node/online").read().strip()
+        fields = best[1].split() if best else []
+        return {"mapping_start": hex(best[0]) if best else None, "policy": fields[1] if len(fields) > 1 else None,
+                "pages_by_node": {f.split("=")[0]: int(f.split("=")[1]) for f in fields if f[0] == "N" and "=" in f},
+                "kernelpagesize_kB": next((int(f.split("=")[1]) for f in fields if f.startswith("kernelpagesize_kB=")), None),
+                "nodes_online": online}
+    except Exception as e:  # the file is not there in every container
+        return {"error": str(e)}
+
+
+def probe_link_latency(hip, torch, note, quick=False):
+    import numpy as np
+    call = _probe_lib()
+    GiB = 1 << 30
+    total = (8 if quick else 60) * GiB
+    stream = C.c_void_p()
+    hip.call("ugk_stream_create", C.byref(stream))
+    t0 = time.perf_counter()
+    host = _pinned(hip, total)
+    # contents: ascending words written by the device (all-zero lines could be moved faster than real rows)
+    chunk = 1 << 30
+    for off in range(0, total, chunk):
+        hip.call("ugk_arange_u32", host.value + off, (off // 4) & 0xffffffff, chunk // 4, stream)
+    hip.call("ugk_stream_sync", stream)
+    note("pinned and filled %d GiB in %.1f s" % (total // GiB, time.perf_counter() - t0))
+    placement = _numa_placement(host.value)
+    note("placement of the allocation: %s" % placement)
+    host_bytes = (C.c_uint8 * total).from_address(host.value)
+    host_lines = np.frombuffer(host_bytes, dtype=np.uint64).reshape(-1, 16)  # 128-byte lines, link in word 0
+    rng = np.random.default_rng(7)
+    last = torch.zeros(2, dtype=torch.int64, device="cuda")
+    spans = (1, 4, 8) if quick else (1, 4, 16, 32, 60)
+    hops = 20_000
+    scrub = np.empty(256 << 20, np.uint8)  # written after the chain, so that its lines leave the CPU's caches
+
+    def chase(base_ptr, write_links, n_lines):
+        nodes = rng.choice(n_lines, size=hops, replace=False).astype(np.uint64)
+        write_links(nodes, np.roll(nodes, -1))
+        scrub[:] = 1
+        out = []
+        for rep in range(3):
+            a, b = _event(hip), _event(hip)
+            hip.call("ugk_event_record", a, stream)
+            call("bp_chase", base_ptr, 128, int(nodes[0]), hops, last.data_ptr(), stream)
+            hip.call("ugk_event_record", b, stream)
+            hip.call("ugk_event_sync", b)
+            out.append(_elapsed_us(hip, a, b) / hops)
+            hip.call("ugk_event_destroy", a)
+            hip.call("ugk_event_destroy", b)
+        assert int(last[0].item()) == int(nodes[0])  # the chain is a cycle of `hops` links
+        return out
+
+    def host_links(nodes, nxt):
+        host_lines[nodes, 0] = nxt
+
+    latency = []
+    for span in spans:
+        us = chase(host, host_links, span * GiB // 128)
+        latency.append({"span_GiB": span, "us_per_dependent_read": [round(x, 3) for x in us]})
+        note("pinned host memory, links over the first %d GiB: %s us per dependent read" % (span, latency[-1]["us_per_dependent_read"]))
+    dev_lines = torch.zeros(((2 if quick else 8) * GiB // 128, 16), dtype=torch.int64, device="cuda")
+
+    def dev_links(nodes, nxt):
+        dev_lines[torch.from_numpy(nodes.astype(np.int64)).cuda(), 0] = torch.from_numpy(nxt.astype(np.int64)).cuda()
+        torch.cuda.synchronize()
+
+    hbm_us = chase(dev_lines.data_ptr(), dev_links, dev_lines.shape[0])
+    note("HBM, links over %d GiB: %s us per dependent read" % (dev_lines.numel() * 8 // GiB, [round(x, 3) for x in hbm_us]))
+    del dev_lines
+
+    # (b) independent reads by bytes in flight
+    n_rows = 1 << 20
+    g = torch.Generator(device="cuda").manual_seed(1)
+    grids = (8, 64, 512, 2048) if quick else (4, 8, 16, 32, 64, 128, 256, 512, 1024, 2048, 4096, 8192)
+    sink = torch.zeros(max(grids) * 256, dtype=torch.int32, device="cuda")
+    sweep = []
+    for rb in (128, 512):
+        for span in (spans[-1],) if quick else (16, spans[-1]):
+            rows = torch.randint(0, span * GiB // rb, (4, n_rows), generator=g, device="cuda", dtype=torch.int64).to(torch.int32)
+            for unroll in (1, 2, 4, 8, 16):
+                by_grid = {}
+                for grid in grids:
+                    def go(i):
+                        call("bp_rows_inflight", host, rb, rows[i % 4].data_ptr(), n_rows, unroll, grid, sink.data_ptr(), stream)
+                    us = _timed(hip, stream, go, 3, warm=1)
+                    by_grid[str(grid)] = round(n_rows * rb / us / 1e3, 2)
+                sweep.append({"row_bytes": rb, "span_GiB": span, "loads_in_flight_per_lane": unroll,
+                              "KiB_in_flight_per_workgroup": unroll * 4, "GBps_by_workgroups": by_grid})
+                note("rows of %d B over %d GiB, %2d loads per lane in flight: %s GB/s by workgroups" % (rb, span, unroll, by_grid))
+            del rows
+    hip.call("ugk_host_free", host)
+    return {"probe": "link_latency", "allocation_GiB": total // GiB, "placement": placement,
+            "dependent_reads": {"hops": hops, "line_bytes": 128, "pinned_host": latency,
+                                "hbm_us_per_dependent_read": [round(x, 3) for x in hbm_us],
+                                "how": "one lane follows a cycle of 20,000 links at random 128-byte lines of the first "
+                                       "S GiB; 3 passes over the same cycle (the lines are not cached on the device: "
+                                       "the passes agree); microseconds per link"},
+            "independent_reads": {"rows_per_launch": n_rows, "rows": sweep,
+                                  "how": "bp_rows_inflight: a grid of W workgroups of 256 lanes reads 2^20 listed rows, "
+                                         "U 16-byte loads in flight per lane, nothing written; bytes in flight = "
+                                         "min(W, resident workgroups) x 256 x U x 16; 2 HIP events around 3 launches"}}
+
+
+PROBES = {"link_latency": probe_link_latency, "sparse_layer": probe_sparse_layer, "pooled": probe_pooled, "kpw": probe_kpw, "row_span": probe_row_span, "cu_mask": probe_cu_mask, "small_batch": probe_small_batch}
 
 
 def run(name, quick=False):
     import torch
 
-    from . import hip
+    from ugache_amd import hip
 
     if not torch.cuda.is_available():
         sys.exit("probes need a GPU")
