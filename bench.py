@@ -37,7 +37,9 @@ HBM_PEAK_GBPS = 8000.0  # MI355X published HBM3E bandwidth
 # profiles/gather_kernel_c2_all_hit.md (each counter scaled by its reading for a 1 GiB copy kernel)
 MEASURED_TRAFFIC_BYTES = {"c2_all_hit_10Mx128xfp32_262144_u32_uniform": 270_530_000,
                           # fused kernel; includes the 126 MB of rows that reach the L2 over the host link
-                          "c3_gnn_100Mx128xfp32_1M_i64_zipf0.9_cache25pct": 1_137_700_000}
+                          "c3_gnn_100Mx128xfp32_1M_i64_zipf0.9_cache25pct": 1_137_700_000,
+                          # fused kernel over the hash table (profiles/extract_mix_kernel_mixed_c1_c3_c4_c5.md)
+                          "c5_hash_500Mx64xfp16_1M_i64_zipf1.05_cache50M": 311_000_000}
 
 ALL_HIT = {
     # name: (rows, dim, keys per batch)
@@ -211,6 +213,50 @@ def cpu_baseline(orc, table_np, keys_host, n_keys, row_bytes, seconds):
             break
     el = time.perf_counter() - t0
     return n_keys * n_cpu / el, n_cpu, el, lib.orc_omp_threads()
+
+
+def cpu_baseline_lookup_and_gather(orc, table_np, cached_rows, keys_host, key_inv, key_mask, n_keys, row_bytes, seconds,
+                                   gpu_batch0):
+    """The CPU form of the whole mixed-source step: per key, id -> row, lookup in a flat host array of the row space,
+    then a copy of the row from a host-side copy of the cached rows or from the host table, OpenMP over keys
+    (orc_extract_flat_i64_omp).  The cache copy and the flat array are built here, untimed, from the rows the GPU
+    cache holds (slot = position in that list).  The output of the first batch is compared with the GPU's.
+    Returns (keys/s, batches, elapsed, threads)."""
+    import numpy as np
+
+    rows = table_np.shape[0]
+    lib = orc.lib
+    cached_rows = np.ascontiguousarray(cached_rows, np.uint32)
+    flat = np.full(rows, 0xFFFFFFFF, np.uint32)
+    flat[cached_rows] = np.arange(len(cached_rows), dtype=np.uint32)
+    cache_copy = np.empty((max(len(cached_rows), 1), row_bytes), np.uint8)
+    if len(cached_rows):
+        assert lib.orc_gather_u32_omp(table_np.ctypes.data, rows, cached_rows, len(cached_rows), cache_copy.ctypes.data,
+                                      row_bytes) == 0
+    cpu_out = np.empty((n_keys, row_bytes), np.uint8)
+    counts = np.zeros(2, np.uint64)
+    pool = len(keys_host)
+
+    def cpu_step(i):
+        rc = lib.orc_extract_flat_i64_omp(flat.ctypes.data, rows, ctypes.c_uint64(key_inv), ctypes.c_uint64(key_mask),
+                                          keys_host[i % pool].ctypes.data, n_keys, cache_copy.ctypes.data,
+                                          len(cache_copy), table_np.ctypes.data, cpu_out.ctypes.data, row_bytes,
+                                          counts.ctypes.data)
+        assert rc == 0
+
+    cpu_step(0)
+    if cpu_out.tobytes() != gpu_batch0:
+        sys.exit("bench.py: the CPU baseline's output differs from the GPU's for the same batch")
+    split0 = counts.tolist()
+    t0 = time.perf_counter()
+    n_cpu = 0
+    while True:
+        cpu_step(n_cpu)
+        n_cpu += 1
+        if time.perf_counter() - t0 >= seconds or n_cpu >= 100000:
+            break
+    el = time.perf_counter() - t0
+    return n_keys * n_cpu / el, n_cpu, el, lib.orc_omp_threads(), split0
 
 
 def fill_table_from_device(emb, dev, seed):
@@ -526,6 +572,15 @@ def run_mixed(args):
                                                 out, stream, torch, W, K)
     note("stream-ordered leg done: %.3f ms/step" % (so_step_s * 1e3))
 
+    if args.calibrate:  # a kernel of known traffic beside the extraction kernel, for counter runs
+        cal_src = torch.empty(1 << 30, dtype=torch.uint8, device=dev)
+        cal_dst = torch.empty(1 << 30, dtype=torch.uint8, device=dev)
+        torch.cuda.synchronize()
+        for _ in range(5):
+            hip.call("ugk_copy_rows", cal_dst.data_ptr(), cal_src.data_ptr(), 1 << 30, stream)
+        torch.cuda.synchronize()
+        del cal_src, cal_dst
+
     orc = Oracle()
     table_np = emb.numpy().view(np.uint8).reshape(rows, row_bytes)
     rows_host = rows_pool.cpu().numpy()
@@ -582,14 +637,30 @@ def run_mixed(args):
         stages = {"classify_partition": t_idx * 1e6, "host_gather": t_miss * 1e6, "hbm_gather": t_hit * 1e6}
     achieved = hit_alg / t_hit / 1e9 if t_hit > 0 else 0.0
 
-    miss_alone = miss_stream_alone(C, _basics, step, stream, torch, W, K, pool, rows_host, table_np, orc, out,
+    # (with deduplication the group sizes count distinct keys, the skip-local extraction every key: the plain leg of
+    # the same workload carries this figure)
+    miss_alone = None if args.dedup else miss_stream_alone(C, _basics, step, stream, torch, W, K, pool, rows_host, table_np, orc, out,
                                    row_bytes, link_gbps, kLogL1MissBytes, kLogL3CacheCombineCacheTime,
                                    kLogL3CacheCombineMissTime, args.workload, note)
     ceiling = random_row_ceiling(hip, torch, emb, rows, row_bytes, dev, stream, note)
 
-    # the CPU baseline gathers by row number (it is spared the id -> row translation of sparse-id mode)
+    # The CPU baseline, two ways, each for half the budget.  (i) the whole step as the CPU would do it: id -> row, lookup
+    # in a flat host array, per-row source (a host-side copy of the cached rows, or the host table), copy; its first
+    # batch is compared with the GPU's output.  (ii) a plain gather by row number out of the host table, spared the
+    # lookup and the id -> row translation: the fastest the CPU can be on these batches.
     keys_host = rows_host
-    cpu_kps, n_cpu, cpu_el, cores = cpu_baseline(orc, table_np, keys_host, n_keys, row_bytes, args.cpu_seconds)
+    cached_now = np.zeros(info_cache["cached_rows"], np.uint32)
+    C.coll_cache_get_cached_keys(0, cached_now.ctypes.data, len(cached_now))
+    ids_host = np.ascontiguousarray(keys_pool.cpu().numpy())
+    step(0)
+    torch.cuda.synchronize()
+    gpu_batch0 = out.cpu().numpy().tobytes()
+    key_inv = pow(KEY_MUL, -1, 1 << KEY_BITS) if sparse else 0
+    cpu8_kps, n_cpu8, cpu8_el, cores, cpu_split = cpu_baseline_lookup_and_gather(
+        orc, table_np, cached_now, ids_host, key_inv, (1 << KEY_BITS) - 1 if sparse else 0, n_keys, row_bytes,
+        args.cpu_seconds / 2, gpu_batch0)
+    note("CPU lookup + gather: %.1f M keys/s on %d threads" % (cpu8_kps / 1e6, cores))
+    cpu_kps, n_cpu, cpu_el, cores = cpu_baseline(orc, table_np, keys_host, n_keys, row_bytes, args.cpu_seconds / 2)
     uniq = float(np.mean([len(np.unique(keys_host[i])) for i in range(min(pool, 4))]))
 
     refresh = None
@@ -791,7 +862,7 @@ def run_mixed(args):
         "parity": "bit-exact vs CPU oracle: every one of the %d pooled batches, after the timed region" % n_checked,
         "device": info["name"] + " " + info["arch"],
         "stages_us": stages,
-        "hit_rate": n_hit / n_keys,
+        "hit_rate": n_hit / (n_hit + n_miss),  # over the keys that were extracted (the distinct ones with --dedup)
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                      "frac": achieved / HBM_PEAK_GBPS,
                      "traffic": MEASURED_TRAFFIC_BYTES.get(args.workload) if fused else None,
@@ -805,12 +876,19 @@ def run_mixed(args):
                       "frac_of_row_ceiling": ((miss_bytes / t_link / 1e9) / ceiling["best_GBps"]
                                               if t_link > 0 and ceiling["best_GBps"] > 0 else None),
                       "miss_stream_alone": miss_alone},
-        "cpu_baseline": {"value": cpu_kps, "unit": "keys/s", "cores": cores, "kind": "port",
-                         "sample": "%d batches of %d keys from the same pool, %.1f s, OpenMP gather over keys by row "
-                                   "number out of the whole host table (no lookup or classify step: the fastest the "
-                                   "CPU path can be)" % (n_cpu, n_keys, cpu_el),
-                         "effective_GBps": n_keys * row_bytes * n_cpu / cpu_el / 1e9},
-        "gpu_over_cpu": keys_per_s / cpu_kps,
+        "cpu_baseline": {"value": cpu8_kps, "unit": "keys/s", "cores": cores, "kind": "port",
+                         "sample": "%d batches of %d keys from the same pool, %.1f s: per key id -> row, lookup in a "
+                                   "flat host array, copy of the row from a host-side copy of the cached rows or from "
+                                   "the host table, OpenMP over keys; first batch byte-equal to the GPU's output"
+                                   % (n_cpu8, n_keys, cpu8_el),
+                         "effective_GBps": n_keys * row_bytes * n_cpu8 / cpu8_el / 1e9,
+                         "rows_from_cache_copy_first_batch": cpu_split[0],
+                         "gather_by_row_number": {
+                             "value": cpu_kps, "unit": "keys/s", "cores": cores,
+                             "sample": "%d batches, %.1f s, OpenMP gather by row number out of the whole host table "
+                                       "(no lookup, no id -> row step: the fastest the CPU can be)" % (n_cpu, cpu_el)}},
+        "gpu_over_cpu": keys_per_s / cpu8_kps,
+        "gpu_over_cpu_gather_by_row_number": keys_per_s / cpu_kps,
         "setup_seconds": setup_s,
         "stream_ordered": {"keys_per_s": n_keys / so_step_s, "ms_per_step": so_step_s * 1e3,
                            "entry_point": "coll_cache_lookup_async_i64 (extension: enqueue only, one wait after the K "
@@ -909,7 +987,18 @@ def random_row_ceiling(hip, torch, emb, rows, row_bytes, dev, stream, note):
 LEG_KEYS = ("value", "unit", "ms_per_step", "ms_per_step_spread", "steps", "warmup", "config", "hit_rate",
             "effective_extraction_GBps", "parity", "stages_us", "roofline", "host_link", "cpu_baseline", "gpu_over_cpu",
             "refresh", "refresh_each_step", "setup_seconds", "stream_ordered", "cache_build")
-DEFAULT_LEGS = ("c3_gnn_100Mx128xfp32_1M_i64_zipf0.9_cache25pct", "c5_hash_500Mx64xfp16_1M_i64_zipf1.05_cache50M")
+# (short name, workload, extra options, what it is)
+DEFAULT_LEGS = (
+    ("c3", "c3_gnn_100Mx128xfp32_1M_i64_zipf0.9_cache25pct", (), "configuration 3, every key extracted (default)"),
+    ("c3_dedup", "c3_gnn_100Mx128xfp32_1M_i64_zipf0.9_cache25pct", ("--dedup",),
+     "configuration 3 as BASELINE words it: distinct keys extracted once, duplicates re-expanded (COLL_DEDUP_KEYS=1)"),
+    ("c4_half", "c4_dlr_half_26x4Mx128xfp32_212992_i64_zipf1.2_cache20GB", (),
+     "configuration 4 at half its rows per field: the box pins 64 GiB, the full 106 GB cannot be pinned"),
+    ("c1", "c1_cpu_ref_1Mx128xfp32_65536_i64_zipf1.1_cache10pct", (), "configuration 1's shape on the GPU"),
+    ("c5", "c5_hash_500Mx64xfp16_1M_i64_zipf1.05_cache50M", (), "configuration 5, lookups and one host-side refresh"),
+    ("c5_device_refresh", "c5_hash_500Mx64xfp16_1M_i64_zipf1.05_cache50M", ("--device-refresh",),
+     "configuration 5 with a refresh after every step, counted, ranked and placed on the device"),
+)
 
 
 def run_child(workload, args, cpu_seconds, extra=()):
@@ -937,25 +1026,43 @@ def run_default(args):
     result, err = run_child(main_name, args, args.cpu_seconds)
     if result is None:
         sys.exit("bench.py: the all-hit configuration failed: %s" % err)
-    legs = {}
+    legs, summary = {}, {}
     if not args.no_legs:
-        for name in DEFAULT_LEGS:
-            leg, err = run_child(name, args, min(args.cpu_seconds, 5.0))
+        for short, name, extra, what in DEFAULT_LEGS:
+            leg, err = run_child(name, args, 0.5 if "--device-refresh" in extra else min(args.cpu_seconds, 4.0), extra=extra)
             if leg is None:
                 # a leg that cannot report (a parity failure ends it without a number) takes the whole line with it
-                sys.exit("bench.py: leg %s failed: %s" % (name, err))
-            legs[name] = {k: leg[k] for k in LEG_KEYS if k in leg}
-        # config 5's "a refresh with every step": the same workload with the hotness counted and the cache re-placed on
-        # the device (COLL_GPU_RECORD=1 COLL_GPU_REFRESH=1), 1 % of the cache replaced per step
-        name = DEFAULT_LEGS[-1]
-        leg, err = run_child(name, args, 0.5, extra=("--device-refresh",))
-        if leg is None:
-            sys.exit("bench.py: leg %s --device-refresh failed: %s" % (name, err))
-        legs[name + "+device_refresh"] = {k: leg[k] for k in LEG_KEYS if k in leg and k != "cpu_baseline"}
+                sys.exit("bench.py: leg %s (%s %s) failed: %s" % (short, name, " ".join(extra), err))
+            legs[short] = {k: leg[k] for k in LEG_KEYS if k in leg}
+            legs[short]["what"] = what
+            hl = leg.get("host_link") or {}
+            summary[short] = {"ms_per_step": leg["ms_per_step"], "keys_per_s": leg["value"], "hit_rate": leg.get("hit_rate"),
+                              "host_link_GBps": hl.get("achieved"), "host_link_frac": hl.get("frac"),
+                              "frac_of_row_ceiling": hl.get("frac_of_row_ceiling"),
+                              "cpu_keys_per_s": leg["cpu_baseline"]["value"], "cpu_cores": leg["cpu_baseline"]["cores"],
+                              "gpu_over_cpu": leg.get("gpu_over_cpu"), "parity": "bit-exact, every pooled batch"}
+            if leg.get("refresh_each_step"):
+                summary[short]["refresh_each_step_ms"] = leg["refresh_each_step"]["ms_per_step"]
+                summary[short]["refresh_ms"] = leg["refresh_each_step"]["refresh_ms"]
+            if leg.get("cache_build"):
+                summary[short]["build_frac_of_link"] = leg["cache_build"]["frac_of_measured_link"]
     result["legs"] = legs
-    result["legs_note"] = ("each leg is the same bench.py with --workload <name>, run after the top-level workload in "
-                           "a process of its own, same --steps and --warmup; value / roofline / cpu_baseline at the top "
-                           "level are the all-hit configuration's alone")
+    result["legs_note"] = ("each leg is the same bench.py with --workload <name> (and the options named), run after the "
+                           "top-level workload in a process of its own, same --steps and --warmup; value / roofline / "
+                           "cpu_baseline at the top level are the all-hit configuration's alone")
+    # The figures of the other configurations once more in short form, at the top level and inside `roofline` (a
+    # reader that keeps only the objects of the contract keeps these)
+    large = result.get("all_hit_large_output") or {}
+    short_keys = {"c2_frac_output_1M_keys": (large.get("keys_1M") or {}).get("frac_of_hbm_peak"),
+                  "c2_frac_outputs_rotated_1GiB": (large.get("outputs_rotated") or {}).get("frac_of_hbm_peak")}
+    for short, sm in summary.items():
+        short_keys[short + "_ms_per_step"] = sm["ms_per_step"]
+        short_keys[short + "_host_link_frac"] = sm["host_link_frac"]
+        short_keys[short + "_gpu_over_cpu"] = sm["gpu_over_cpu"]
+    result.update(short_keys)
+    result["roofline"]["other_configs"] = dict(summary, **{"c2_large_output": {
+        "frac_output_1M_keys": short_keys["c2_frac_output_1M_keys"],
+        "frac_outputs_rotated_1GiB": short_keys["c2_frac_outputs_rotated_1GiB"]}})
     emit(result)
 
 

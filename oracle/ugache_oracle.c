@@ -417,3 +417,39 @@ int orc_gather_i64_omp(const void *table, size_t num_rows, const int64_t *keys, 
   }
   return bad ? -1 : 0;
 }
+
+/* The CPU form of the whole mixed-source step, one pass per key: id -> row (identity, or the inverse of the sparse-id
+ * map), flat-table lookup (LookupHelper over the flat table, cache_hashtable.cuh:233-237, 480-503), source chosen per
+ * row and copied (DataIterMixLoc, cache_context.cu:137-159, 195-231).  count_out[0] / [1] = rows taken from the cache
+ * copy / from the host table. */
+int orc_extract_flat_i64_omp(const uint32_t *flat, size_t num_rows, uint64_t key_inv, uint64_t key_mask,
+                             const int64_t *keys, size_t n, const void *cache, size_t cache_rows, const void *host_table,
+                             void *out, size_t row_bytes, uint64_t count_out[2]) {
+  int bad = 0;
+  uint64_t n_local = 0, n_host = 0;
+#pragma omp parallel for schedule(static) reduction(| : bad) reduction(+ : n_local, n_host)
+  for (size_t i = 0; i < n; i++) {
+    uint64_t row = (uint64_t)keys[i];
+    if (key_inv != 0) row = row <= key_mask ? (row * key_inv) & key_mask : ~(uint64_t)0;
+    if (row >= num_rows) {
+      bad |= 1;
+      continue;
+    }
+    const uint32_t v = flat[row];
+    const char *src;
+    if (v != ORC_EMPTY_POS && orc_loc(v) == 0) {
+      if (orc_off(v) >= cache_rows) {
+        bad |= 1;
+        continue;
+      }
+      src = (const char *)cache + (size_t)orc_off(v) * row_bytes;
+      n_local++;
+    } else {
+      src = (const char *)host_table + (size_t)row * row_bytes;
+      n_host++;
+    }
+    memcpy((char *)out + i * row_bytes, src, row_bytes);
+  }
+  if (count_out) count_out[0] = n_local, count_out[1] = n_host;
+  return bad ? -1 : 0;
+}

@@ -23,6 +23,8 @@
  *   orc_refresh_plan     – Python set algebra and free-list conservation
  *   orc_dedup            – numpy.unique(return_inverse=True)
  *   orc_pool_f64         – numpy.add.at over float64 rows, and hand-worked segments
+ *   orc_extract_flat_i64_omp – numpy.where / numpy.take over a cache copy that differs from the host rows, a
+ *                              brute-force modular inverse for the sparse ids
  * No function here is "parity unpinned".
  */
 #ifndef UGACHE_ORACLE_H_
@@ -157,6 +159,15 @@ int orc_gather_u32_omp(const void *table, size_t num_rows, const uint32_t *keys,
                        size_t row_bytes);
 int orc_gather_i64_omp(const void *table, size_t num_rows, const int64_t *keys, size_t n, void *out,
                        size_t row_bytes);
+
+/* the mixed-source step of the CPU baseline: per key, id -> row (row = key when key_inv == 0, else
+ * (key * key_inv) & key_mask), lookup in the flat table of the whole row space (ORC_EMPTY_POS or a packed
+ * (location, slot) with location 0 = the cache copy), then memcpy of the row from the cache copy or from the host
+ * table; OpenMP over keys.  count_out (may be NULL): rows taken from the cache copy / from the host table.
+ * Returns -1 if a key has no row or a slot lies outside the cache copy. */
+int orc_extract_flat_i64_omp(const uint32_t *flat, size_t num_rows, uint64_t key_inv, uint64_t key_mask,
+                             const int64_t *keys, size_t n, const void *cache, size_t cache_rows, const void *host_table,
+                             void *out, size_t row_bytes, uint64_t count_out[2]);
 
 #ifdef __cplusplus
 }

@@ -81,6 +81,8 @@ def load():
     lib.orc_gather_u32_omp.argtypes = [vp, sz, u32p, sz, vp, sz]
     lib.orc_gather_i64_omp.restype = C.c_int
     lib.orc_gather_i64_omp.argtypes = [vp, sz, i64p, sz, vp, sz]
+    lib.orc_extract_flat_i64_omp.restype = C.c_int
+    lib.orc_extract_flat_i64_omp.argtypes = [vp, sz, C.c_uint64, C.c_uint64, vp, sz, vp, sz, vp, vp, sz, vp]
     return lib
 
 
@@ -104,6 +106,21 @@ class Oracle:
         if rc != 0:
             raise IndexError("key out of range")
         return out
+
+    def extract_flat(self, flat, keys, cache, host_table, key_inv=0, key_mask=0):
+        """the CPU baseline's mixed-source step; returns (rows, [n from the cache copy, n from the host table])"""
+        host_table = np.ascontiguousarray(host_table)
+        cache = np.ascontiguousarray(cache)
+        rb = host_table.strides[0]
+        out = np.empty((len(keys),) + host_table.shape[1:], dtype=host_table.dtype)
+        counts = np.zeros(2, np.uint64)
+        rc = self.lib.orc_extract_flat_i64_omp(_ptr(np.ascontiguousarray(flat, np.uint32)), host_table.shape[0],
+                                               C.c_uint64(key_inv), C.c_uint64(key_mask),
+                                               _ptr(np.ascontiguousarray(keys, np.int64)), len(keys), _ptr(cache),
+                                               cache.shape[0], _ptr(host_table), _ptr(out), rb, _ptr(counts))
+        if rc != 0:
+            raise IndexError("key without a row, or slot outside the cache copy")
+        return out, counts.tolist()
 
     # --- tables -------------------------------------------------------------------------------
     def simple_table(self, n_entries):

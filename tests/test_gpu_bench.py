@@ -42,6 +42,11 @@ def test_mixed_workload_line_with_the_serving_loop():
     _check_contract(d, 12, 3)
     link = d["host_link"]
     assert 0 < link["frac"] <= 1.05 and link["achieved"] > 0
+    # the CPU leg both ways: the whole step (lookup + per-row source + copy) and a plain gather by row number
+    c = d["cpu_baseline"]
+    assert c["gather_by_row_number"]["value"] > 0 and c["gather_by_row_number"]["cores"] == c["cores"]
+    assert 0 < c["rows_from_cache_copy_first_batch"] < 262_144
+    assert abs(d["gpu_over_cpu"] - d["value"] / c["value"]) < 1e-6 * d["gpu_over_cpu"]
     b = d["cache_build"]
     assert b["seconds"] > 0 and b["rows_filled"] == d["config"]["cached_rows"] and b["bytes_filled"] == b["rows_filled"] * 512
     s = d["serving_loop"]

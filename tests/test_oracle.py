@@ -457,3 +457,53 @@ def test_oracle_reproduces_the_committed_golden_case():
     keys = np.array(g["lookup_keys"], np.int64)
     assert ORC.gather(table, keys).tolist() == g["expected_output"]
     assert [0, int((nid[keys] == 0).sum()), len(keys)] == g["expected_group_offset"]
+
+
+def test_extract_flat_picks_the_source_per_row_like_numpy_where():
+    """orc_extract_flat_i64_omp (the mixed-source step of bench.py's CPU leg): a row comes from the cache copy exactly
+    when the flat table names a slot for it, from the host table otherwise.  The cache copy holds different bytes from
+    the host rows here, so a wrong source, a wrong slot or a transposed argument shows; slots are a permutation, so
+    slot != position in the list of cached rows.  Sparse ids: the row of an id by a brute-force search for the
+    multiplier's inverse instead of a formula."""
+    rng = np.random.default_rng(21)
+    n_rows, rb, n_cached = 3000, 48, 700
+    host = rng.integers(0, 256, size=(n_rows, rb), dtype=np.uint8)
+    cached_rows = rng.choice(n_rows, n_cached, replace=False)
+    slots = rng.permutation(n_cached + 50)[:n_cached]
+    cache = rng.integers(0, 256, size=(n_cached + 50, rb), dtype=np.uint8)  # NOT the host rows
+    flat = np.full(n_rows, 0xFFFFFFFF, np.uint32)
+    flat[cached_rows] = slots  # location 0 in the top four bits
+    keys = rng.integers(0, n_rows, size=5000)
+    slot_of = np.full(n_rows, -1, np.int64)
+    slot_of[cached_rows] = slots
+    want = np.where((slot_of[keys] >= 0)[:, None], cache[np.maximum(slot_of[keys], 0)], host[keys])
+    got, counts = ORC.extract_flat(flat, keys, cache, host)
+    assert got.tobytes() == want.tobytes()
+    assert counts == [int((slot_of[keys] >= 0).sum()), int((slot_of[keys] < 0).sum())]
+    # a table entry of another location than 0 reads from the host table
+    flat2 = flat.copy()
+    flat2[cached_rows[:10]] = (1 << 28) + 5
+    slot2 = slot_of.copy()
+    slot2[cached_rows[:10]] = -1
+    want2 = np.where((slot2[keys] >= 0)[:, None], cache[np.maximum(slot2[keys], 0)], host[keys])
+    assert ORC.extract_flat(flat2, keys, cache, host)[0].tobytes() == want2.tobytes()
+    # sparse ids: id = (row * mul) mod 2^bits; the inverse found by search on a small modulus
+    bits, mul = 12, 0x9E3779B97F4A7C15 & 0xFFF | 1
+    mask = (1 << bits) - 1
+    inv = next(x for x in range(1, 1 << bits, 2) if (x * mul) & mask == 1)
+    rows_b = rng.integers(0, n_rows, size=2000)
+    ids = (rows_b * mul) & mask
+    got3, _ = ORC.extract_flat(flat, ids, cache, host, key_inv=inv, key_mask=mask)
+    want3 = np.where((slot_of[rows_b] >= 0)[:, None], cache[np.maximum(slot_of[rows_b], 0)], host[rows_b])
+    assert got3.tobytes() == want3.tobytes()
+    # keys without a row, and a slot outside the cache copy, are refused
+    with pytest.raises(IndexError):
+        ORC.extract_flat(flat, np.array([n_rows]), cache, host)
+    with pytest.raises(IndexError):
+        ORC.extract_flat(flat, np.array([-1]), cache, host)
+    with pytest.raises(IndexError):
+        ORC.extract_flat(flat, np.array([mask + 1]), cache, host, key_inv=inv, key_mask=mask)
+    flat3 = flat.copy()
+    flat3[cached_rows[0]] = len(cache)
+    with pytest.raises(IndexError):
+        ORC.extract_flat(flat3, np.array([cached_rows[0]]), cache, host)

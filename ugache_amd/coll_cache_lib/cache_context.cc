@@ -764,7 +764,11 @@ void ExtractSession::ExtractFeatImpl(const KeyT *nodes, size_t num_nodes, void *
     JoinRecordOnHost();
     CheckStatusWord(stream);
     float combine_ms = 0;
-    if (events) UGK_CALL(ugk_event_elapsed_ms(_ev_t[0], _ev_t[1], &combine_ms));
+    if (events) {
+      // the ticket behind the batch can turn up before the runtime has seen the event in front of it complete
+      UGK_CALL(ugk_event_sync(_ev_t[1]));
+      UGK_CALL(ugk_event_elapsed_ms(_ev_t[0], _ev_t[1], &combine_ms));
+    }
     const double combine_time = events ? combine_ms * 1e-3 : host_time;
     _group_offset[1] = from_host ? 0 : (uint32_t)num_nodes;
     _group_offset[2] = (uint32_t)num_nodes;
@@ -829,7 +833,10 @@ void ExtractSession::ExtractFeatImpl(const KeyT *nodes, size_t num_nodes, void *
                    n_miss = _host_mirror[kMirGroupSizes + UGK_LOC_HOST];
     CHECK_EQ((size_t)n_local + n_miss, num_nodes);
     float mix_ms = (float)(host_time * 1e3);
-    if (events) UGK_CALL(ugk_event_elapsed_ms(_ev_t[0], _ev_t[1], &mix_ms));
+    if (events) {
+      UGK_CALL(ugk_event_sync(_ev_t[1]));  // see the direct-mapping branch
+      UGK_CALL(ugk_event_elapsed_ms(_ev_t[0], _ev_t[1], &mix_ms));
+    }
     _group_offset[1] = n_local;
     _group_offset[2] = (uint32_t)num_nodes;
     if (profiler && task_key != 0xffffffffffffffffull) {
