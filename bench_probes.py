@@ -92,7 +92,9 @@ def probe_kpw(hip, torch, note, quick=False):
                 hip.call("ugk_fill_u32", mem.data_ptr(), hip.EMPTY_U32, rows, stream)
                 tb = hip.table(hip.TABLE_FLAT, mem.data_ptr(), rows)
             else:
-                nb = hip.lib().ugk_hash_buckets_for(ncache, 0.7)
+                # (BENCH_PROBE_HASH_LOAD: the same sweep over a sparser table, to see what the keys that need a second
+                # line cost)
+                nb = hip.lib().ugk_hash_buckets_for(ncache, float(os.environ.get("BENCH_PROBE_HASH_LOAD", "0.7")))
                 mem = torch.empty(nb * 16 + 128, dtype=torch.uint8, device="cuda")
                 base = (mem.data_ptr() + 127) // 128 * 128
                 hip.call("ugk_hash_init", base, nb, stream)

@@ -124,9 +124,10 @@ void coll_cache_forward_pooled_i64(int replica_id, const int64_t *key, const int
  * everything enqueued so far has finished, aborts if a key was outside its table, and makes
  * coll_cache_last_group_offset describe the last batch; any blocking lookup does the same first.  No per-step profiler
  * values are logged for stream-ordered batches.  Such a call is kernel launches only (no synchronisation, no
- * allocation, no memset), so it may be recorded into a HIP graph by a caller that captures its stream; a lookup that
- * is being recorded is not counted by the device-side hotness counters (the counting runs on a stream of the library,
- * which stays out of the caller's graph).  Batches the
+ * allocation, no memset), so it may be recorded into a HIP graph by a caller that captures its stream; while a stream
+ * records, the library enqueues kernels on that stream and nothing else, and with the hotness counted on the device
+ * (COLL_GPU_RECORD=1) the counting is one more kernel of the recorded lookup, so every replay counts the keys it
+ * reads.  Batches the
  * one-kernel paths cannot take (COLL_DEDUP_KEYS, a factored
  * SAMGRAPH_COLL_CACHE_CONCURRENT_LINK_IMPL, rows not multiples of 16 bytes with a partial cache) block as usual. */
 void coll_cache_lookup_async(int replica_id, const uint32_t *key, size_t num_keys, void *output, StreamHandle stream);
@@ -140,6 +141,11 @@ void coll_cache_lookup_pooled_async(int replica_id, const uint32_t *key, const i
 void coll_cache_lookup_pooled_async_i64(int replica_id, const int64_t *key, const int64_t *seg_off,
                                         const float *weights, size_t num_rows, size_t num_keys, int combiner,
                                         int elem_bytes, void *output, StreamHandle stream);
+/* The max_norm of the sparse layer (python_tf2/collcache_tf2/collcache_tf2/core/sparse_lookup_layer.py:95-140, handed to
+ * embedding_lookup_sparse): the pooled lookups of the replica that follow clip every looked-up row to this l2 norm
+ * before it is weighted, x * max_norm / max(||x||_2, max_norm), inside the same kernel.  0 (the default) turns it
+ * off.  No counterpart as an entry point in the reference, where TensorFlow clips. */
+void coll_cache_set_pooled_max_norm(int replica_id, float max_norm);
 /* The seg_off a pooled lookup takes, made on the device from the row of every entry of a sparse feature in row-major
  * order (extension; the indices[:, 0] of the SparseTensor of sparse_lookup_layer.py:196-265): seg_off[r] = number of
  * entries whose row is below r, r = 0 .. num_rows (num_rows + 1 device words).  One kernel on `stream`, no wait.

@@ -312,6 +312,22 @@ int ugk_extract_pool_i64(ugk_table_t t, const int64_t *ids_dev, const int64_t *s
                          uint32_t *status_dev, uint32_t *host_mirror, uint64_t *group_counts_host,
                          uint32_t *num_groups_host, void *stream);
 
+/* The same with every looked-up row clipped to the l2 norm max_norm before it is weighted (the max_norm of the sparse
+ * layer, sparse_lookup_layer.py:95-140: x * max_norm / max(||x||_2, max_norm), norms summed in fp32); max_norm = 0:
+ * no clipping, exactly ugk_extract_pool_*. */
+int ugk_extract_pool_clip_u32(ugk_table_t t, const uint32_t *ids_dev, const int64_t *seg_off_dev,
+                              const float *weights_dev, size_t n_rows, uint64_t nnz, int combiner, int elem_bytes,
+                              float max_norm, const void *cache_dev, uint64_t cache_rows, const void *host_dev,
+                              uint64_t host_rows, void *out_dev, size_t row_bytes, uint32_t *status_dev,
+                              uint32_t *host_mirror, uint64_t *group_counts_host, uint32_t *num_groups_host,
+                              void *stream);
+int ugk_extract_pool_clip_i64(ugk_table_t t, const int64_t *ids_dev, const int64_t *seg_off_dev,
+                              const float *weights_dev, size_t n_rows, uint64_t nnz, int combiner, int elem_bytes,
+                              float max_norm, const void *cache_dev, uint64_t cache_rows, const void *host_dev,
+                              uint64_t host_rows, void *out_dev, size_t row_bytes, uint32_t *status_dev,
+                              uint32_t *host_mirror, uint64_t *group_counts_host, uint32_t *num_groups_host,
+                              void *stream);
+
 /* ---- rows that crossed the host link once, kept where a refresh finds them ---------------------------------------
  * The rows a refresh inserts (RefreshSession::refresh_after_solve_new, cache_context.cu:4054-4090: rows copied host ->
  * HBM in throttled batches) are rows recent lookups missed, i.e. rows that have just crossed the host link into some

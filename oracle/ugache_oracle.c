@@ -334,16 +334,31 @@ static inline uint64_t mix64(uint64_t x) {
 
 int orc_pool_f64(const double *table, size_t num_rows_table, size_t dim, const int64_t *ids, const int64_t *seg_off,
                  const double *weights, size_t n_rows, int combiner, double *out) {
+  return orc_pool_clip_f64(table, num_rows_table, dim, ids, seg_off, weights, n_rows, combiner, 0.0, out);
+}
+
+/* with max_norm > 0 every looked-up row is first clipped to that l2 norm (clip_by_norm over axis 1, applied to the
+ * embeddings before they are weighted: sparse_lookup_layer.py:95-140 hands max_norm to embedding_lookup_sparse):
+ * x * max_norm / max(||x||, max_norm) */
+int orc_pool_clip_f64(const double *table, size_t num_rows_table, size_t dim, const int64_t *ids,
+                      const int64_t *seg_off, const double *weights, size_t n_rows, int combiner, double max_norm,
+                      double *out) {
   for (size_t r = 0; r < n_rows; ++r) {
     double *o = out + r * dim;
     double den = 0.0;
     for (size_t c = 0; c < dim; ++c) o[c] = 0.0;
     for (int64_t j = seg_off[r]; j < seg_off[r + 1]; ++j) {
       if (ids[j] < 0 || (uint64_t)ids[j] >= num_rows_table) return 1;
-      const double w = weights ? weights[j] : 1.0;
+      double w = weights ? weights[j] : 1.0;
       const double *x = table + (size_t)ids[j] * dim;
+      den += combiner == 2 ? w * w : w; /* the denominator is made of the weights alone */
+      if (max_norm > 0.0) {
+        double ss = 0.0;
+        for (size_t c = 0; c < dim; ++c) ss += x[c] * x[c];
+        const double norm = sqrt(ss);
+        w *= max_norm / (norm > max_norm ? norm : max_norm);
+      }
       for (size_t c = 0; c < dim; ++c) o[c] += w * x[c];
-      den += combiner == 2 ? w * w : w;
     }
     if (combiner == 0) continue;
     if (combiner == 2) den = sqrt(den);

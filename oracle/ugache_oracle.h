@@ -23,6 +23,7 @@
  *   orc_refresh_plan     – Python set algebra and free-list conservation
  *   orc_dedup            – numpy.unique(return_inverse=True)
  *   orc_pool_f64         – numpy.add.at over float64 rows, and hand-worked segments
+ *   orc_pool_clip_f64    – hand-worked rows on either side of the norm (3-4-5 triangles), numpy.linalg.norm
  *   orc_extract_flat_i64_omp – numpy.where / numpy.take over a cache copy that differs from the host rows, a
  *                              brute-force modular inverse for the sparse ids
  * No function here is "parity unpinned".
@@ -152,6 +153,13 @@ size_t orc_dedup_i64(const int64_t *keys, size_t n, int64_t *unique, uint32_t *i
  * row (div_no_nan).  table: [num_rows_table, dim] doubles.  Returns non-zero if an id is out of range. */
 int orc_pool_f64(const double *table, size_t num_rows_table, size_t dim, const int64_t *ids, const int64_t *seg_off,
                  const double *weights, size_t n_rows, int combiner, double *out);
+
+/* the same with every looked-up row clipped to the l2 norm max_norm before it is weighted (max_norm <= 0: no clipping):
+ * x * max_norm / max(||x||_2, max_norm), the clip_by_norm that embedding_lookup_sparse applies when the layer is given
+ * max_norm (sparse_lookup_layer.py:95-140, 264) */
+int orc_pool_clip_f64(const double *table, size_t num_rows_table, size_t dim, const int64_t *ids,
+                      const int64_t *seg_off, const double *weights, size_t n_rows, int combiner, double max_norm,
+                      double *out);
 
 /* ---- CPU baseline leg (bench.py only): the same gather as orc_gather_*, OpenMP over keys ---- */
 int orc_omp_threads(void);

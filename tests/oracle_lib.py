@@ -76,6 +76,8 @@ def load():
     f64p = np.ctypeslib.ndpointer(np.float64, flags="C_CONTIGUOUS")
     lib.orc_pool_f64.restype = C.c_int
     lib.orc_pool_f64.argtypes = [f64p, sz, sz, i64p, i64p, vp, sz, C.c_int, f64p]
+    lib.orc_pool_clip_f64.restype = C.c_int
+    lib.orc_pool_clip_f64.argtypes = [f64p, sz, sz, i64p, i64p, vp, sz, C.c_int, C.c_double, f64p]
     lib.orc_omp_threads.restype = C.c_int
     lib.orc_gather_u32_omp.restype = C.c_int
     lib.orc_gather_u32_omp.argtypes = [vp, sz, u32p, sz, vp, sz]
@@ -206,8 +208,9 @@ class Oracle:
         return uniq[:nu].copy(), inv
 
     # --- pooled lookup ------------------------------------------------------------------------
-    def pool(self, table, ids, seg_off, weights, combiner):
-        """float64 combination of the rows of every segment; combiner: "sum" / "mean" / "sqrtn" or 0 / 1 / 2"""
+    def pool(self, table, ids, seg_off, weights, combiner, max_norm=None):
+        """float64 combination of the rows of every segment; combiner: "sum" / "mean" / "sqrtn" or 0 / 1 / 2;
+        max_norm: every row clipped to that l2 norm before it is weighted"""
         combiner = {"sum": 0, "mean": 1, "sqrtn": 2}.get(combiner, combiner)
         t = np.ascontiguousarray(table, dtype=np.float64)
         ids = np.ascontiguousarray(ids, dtype=np.int64)
@@ -216,8 +219,8 @@ class Oracle:
         out = np.empty((len(seg_off) - 1, t.shape[1]), np.float64)
         if len(ids) == 0:
             ids = np.zeros(1, np.int64)
-        rc = self.lib.orc_pool_f64(t, t.shape[0], t.shape[1], ids, seg_off, None if w is None else w.ctypes.data,
-                                   len(seg_off) - 1, combiner, out)
+        rc = self.lib.orc_pool_clip_f64(t, t.shape[0], t.shape[1], ids, seg_off, None if w is None else w.ctypes.data,
+                                        len(seg_off) - 1, combiner, float(max_norm or 0.0), out)
         if rc != 0:
             raise IndexError("id out of range")
         return out

@@ -392,10 +392,11 @@ template <typename K>
 int extract_pool(ugk_table_t t, const K *ids, const int64_t *seg_off, const float *weights, size_t n_rows,
                  uint64_t nnz, int combiner, int elem_bytes, const void *cache, uint64_t cache_rows, const void *host,
                  uint64_t host_rows, void *out, size_t rb, uint32_t *status, uint32_t *mirror, uint64_t *counts,
-                 uint32_t *num_groups) {
+                 uint32_t *num_groups, float max_norm = 0.f) {
   if (num_groups) *num_groups = 0;
   if (n_rows == 0) return 0;
   REQUIRE(seg_off && out && status && (nnz == 0 || ids), "ugk_extract_pool: null pointer");
+  REQUIRE(max_norm >= 0.f, "ugk_extract_pool: negative max_norm");
   REQUIRE(combiner >= 0 && combiner <= 2 && (elem_bytes == 2 || elem_bytes == 4 || elem_bytes == UGK_ELEM_BF16),
           "ugk_extract_pool: bad argument");
   const bool bf16 = elem_bytes == UGK_ELEM_BF16;
@@ -433,9 +434,9 @@ int extract_pool(ugk_table_t t, const K *ids, const int64_t *seg_off, const floa
       if (from_cache) ++local;
       else ++others;
       if (!row) continue;
-      const float w = weights ? weights[j] : 1.f;
+      float w = weights ? weights[j] : 1.f;
       wsum += combiner == 2 ? w * w : w;
-      for (size_t c = 0; c < dim; ++c) {
+      auto element = [&](size_t c) {
         float x;
         if (elem_bytes == 4) memcpy(&x, row + c * 4, 4);
         else {
@@ -448,8 +449,14 @@ int extract_pool(ugk_table_t t, const K *ids, const int64_t *seg_off, const floa
             x = half_to_float(h);
           }
         }
-        acc[c] = std::fma(w, x, acc[c]);
+        return x;
+      };
+      if (max_norm > 0.f) {  // the row clipped to that l2 norm before it is weighted
+        float ss = 0.f;
+        for (size_t c = 0; c < dim; ++c) ss = std::fma(element(c), element(c), ss);
+        w *= max_norm / std::max(std::sqrt(ss), max_norm);
       }
+      for (size_t c = 0; c < dim; ++c) acc[c] = std::fma(w, element(c), acc[c]);
     }
     const float denom = combiner == 1 ? wsum : combiner == 2 ? std::sqrt(wsum) : 1.f;
     for (size_t c = 0; c < dim; ++c) {
@@ -1020,6 +1027,23 @@ int ugk_extract_pool_i64(ugk_table_t t, const int64_t *ids, const int64_t *seg_o
                          uint64_t *counts, uint32_t *num_groups, void *) {
   return extract_pool(t, ids, seg_off, weights, n_rows, nnz, combiner, elem_bytes, cache, cache_rows, host, host_rows,
                       out, rb, status, mirror, counts, num_groups);
+}
+
+int ugk_extract_pool_clip_u32(ugk_table_t t, const uint32_t *ids, const int64_t *seg_off, const float *weights,
+                              size_t n_rows, uint64_t nnz, int combiner, int elem_bytes, float max_norm,
+                              const void *cache, uint64_t cache_rows, const void *host, uint64_t host_rows, void *out,
+                              size_t rb, uint32_t *status, uint32_t *mirror, uint64_t *counts, uint32_t *num_groups,
+                              void *) {
+  return extract_pool(t, ids, seg_off, weights, n_rows, nnz, combiner, elem_bytes, cache, cache_rows, host, host_rows,
+                      out, rb, status, mirror, counts, num_groups, max_norm);
+}
+int ugk_extract_pool_clip_i64(ugk_table_t t, const int64_t *ids, const int64_t *seg_off, const float *weights,
+                              size_t n_rows, uint64_t nnz, int combiner, int elem_bytes, float max_norm,
+                              const void *cache, uint64_t cache_rows, const void *host, uint64_t host_rows, void *out,
+                              size_t rb, uint32_t *status, uint32_t *mirror, uint64_t *counts, uint32_t *num_groups,
+                              void *) {
+  return extract_pool(t, ids, seg_off, weights, n_rows, nnz, combiner, elem_bytes, cache, cache_rows, host, host_rows,
+                      out, rb, status, mirror, counts, num_groups, max_norm);
 }
 
 int ugk_extract_mix_staged_u32(ugk_table_t t, const uint32_t *keys, size_t n, const void *cache, uint64_t cache_rows,

@@ -1490,8 +1490,27 @@ def test_serving_stack_from_a_ps_config_file(tmp_path):
                 got4 = ordered(sp_ids, weights, combiner=combiner)
                 co.coll_torch_lookup_wait(0)
                 assert got4.cpu().numpy().tobytes() == got3.tobytes()
+        # max_norm: every embedding clipped to that l2 norm before it is weighted -- the steps of the reference
+        # (torch ops here), and lookup + clipping + combination in one kernel, both against the oracle
+        norms = np.linalg.norm(rows.astype(np.float64), axis=1)
+        for max_norm in (float(np.median(norms)), float(norms.max() * 2)):
+            for combiner in ("sum", "mean", "sqrtn"):
+                want = ORC.pool(rows, ids, np.concatenate([[0], np.cumsum(lens)]), w, combiner, max_norm=max_norm)
+                tol = 1e-5 * np.abs(want).max()
+                got = sparse(sp_ids, sp_w, combiner=combiner, max_norm=max_norm).cpu().numpy()
+                assert np.allclose(got, want, rtol=1e-5, atol=tol)
+                before = _basics.info(0)["lookups"]
+                got5 = pooled(sp_ids, sp_w, combiner=combiner, max_norm=max_norm).cpu().numpy()
+                assert _basics.info(0)["lookups"] == before + 1  # one fused serving step, not the unfused steps
+                assert np.allclose(got5, want, rtol=1e-5, atol=tol)
+                # the clipping does not stick to the lookups that follow
+                plain = pooled(sp_ids, sp_w, combiner=combiner).cpu().numpy()
+                assert np.allclose(plain, ORC.pool(rows, ids, np.concatenate([[0], np.cumsum(lens)]), w, combiner),
+                                   rtol=1e-5, atol=tol)
         with pytest.raises(ValueError):
             sparse(sp_ids, None, combiner="max")
+        with pytest.raises(ValueError):
+            pooled(sp_ids, None, combiner="sum", max_norm=-1.0)
         hps.SetStepProfileValue(profile_type=kLogL1FeatureBytes, value=123.0)
         assert _basics.step_value(hps._last_step_key(), kLogL1FeatureBytes) == 123.0
         hps.Report()

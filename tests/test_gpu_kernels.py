@@ -778,6 +778,86 @@ def test_pooled_extraction_hand_worked(rows_per_group, monkeypatch):
         pin.free()
 
 
+@pytest.mark.parametrize("kind", ["none", "flat", "hash"])
+@pytest.mark.parametrize("dim,etype", [(4, np.float32), (32, np.float32), (100, np.float32), (128, np.float32),
+                                       (512, np.float32), (1024, np.float32), (64, np.float16), (2048, np.float16),
+                                       (64, "bf16")])
+def test_pooled_extraction_with_max_norm_matches_the_oracle(kind, dim, etype):
+    """ugk_extract_pool_clip_*: every looked-up row is clipped to the l2 norm max_norm before it is weighted, in the
+    same kernel; against the oracle's float64 statement (orc_pool_clip_f64) on rows whose norms lie on both sides of
+    max_norm.  Tolerance as for the plain pooled extraction: 1e-5 of the magnitude of the terms (the norm is a fp32
+    sum of up to 2048 squares, good to a few 1e-7 relative), fp16 / bf16 outputs rounded on top.  max_norm = 0 is
+    the plain kernel, bit for bit."""
+    rng = np.random.default_rng(dim + 3 * len(kind))
+    nkeys = 8_000
+    bf16 = isinstance(etype, str)
+    esize = 2 if bf16 else np.dtype(etype).itemsize
+    ecode = hip.ELEM_BF16 if bf16 else esize
+    rb = dim * esize
+    scale = rng.uniform(0.05, 3.0, size=(nkeys, 1)) / np.sqrt(dim)  # row norms between 0.05 and 3
+    vals = rng.standard_normal((nkeys, dim)) * scale
+    vals[:50] = 0.0  # rows of zeros have norm 0 and stay zeros
+    if bf16:
+        host_bits = _bf16_bits(vals)
+        host = _bf16_values(host_bits)
+        host_bytes = host_bits.view(np.uint8).reshape(nkeys, rb)
+    else:
+        host = vals.astype(etype)
+        host_bytes = host.view(np.uint8).reshape(nkeys, rb)
+    if kind == "none":
+        tb, cached, mem = hip.table(0, None, 0), np.zeros(0, np.int64), None
+    else:
+        cached = rng.choice(nkeys, nkeys // 2, replace=False).astype(np.int64)
+        mem, tb = _make_flat(nkeys) if kind == "flat" else _make_hash(len(cached))[:2]
+    slots = rng.permutation(len(cached)).astype(np.uint32)
+    cache = np.zeros((max(len(cached), 1), rb), np.uint8)
+    if len(cached):
+        cache[slots] = host_bytes[cached]
+        assert _insert(tb, cached, slots) == 0
+    pin = pinned_from(host_bytes)
+    try:
+        st = dev_zeros_u32(1)
+        d_cache = to_dev(cache)
+        f64 = host.astype(np.float64)
+        n_rows = 2_000
+        lens = rng.choice([0, 1, 2, 5, 9, 40], size=n_rows, p=[0.05, 0.3, 0.25, 0.2, 0.15, 0.05])
+        seg_off = np.concatenate([[0], np.cumsum(lens)]).astype(np.int64)
+        nnz = int(seg_off[-1])
+        ids = rng.integers(0, nkeys, size=nnz).astype(np.int64)
+        wts = rng.uniform(0.1, 2.0, size=nnz).astype(np.float32)
+        d_ids, d_off, d_w = to_dev(ids), to_dev(seg_off), to_dev(wts)
+
+        def run(entry, *norm):
+            out = dev_bytes(n_rows * rb, fill=0x7F)
+            hip.call(entry, tb, ptr(d_ids), ptr(d_off), ptr(d_w), n_rows, nnz, combiner, ecode, *norm, ptr(d_cache),
+                     len(cached), pin.ptr, nkeys, ptr(out), rb, ptr(st), None, None, None, None)
+            sync()
+            assert status_value(st) == 0
+            return to_np(out)[: n_rows * rb]
+
+        for combiner in (0, 1, 2):
+            assert run("ugk_extract_pool_clip_i64", 0.0).tobytes() == run("ugk_extract_pool_i64").tobytes()
+            for max_norm in (0.4, 1.5, 100.0):
+                raw = run("ugk_extract_pool_clip_i64", max_norm)
+                got = (_bf16_values(raw.view(np.uint16)) if bf16 else raw.view(etype)).reshape(n_rows, dim).astype(np.float64)
+                want = ORC.pool(f64, ids, seg_off, wts, combiner, max_norm=max_norm)
+                mag = ORC.pool(np.abs(f64), ids, seg_off, wts, combiner, max_norm=max_norm)
+                tol = 1e-5 * mag + 1e-30
+                if esize == 2:
+                    tol = tol + (2.0 ** -8 if bf16 else 1e-3) * np.abs(want) + 2.0 ** -24
+                assert (np.abs(got - want) <= tol).all(), (combiner, max_norm, float(np.abs(got - want).max()))
+                if max_norm == 100.0:  # beyond every row's norm: nothing is clipped
+                    plain = ORC.pool(f64, ids, seg_off, wts, combiner)
+                    assert (np.abs(got - plain) <= tol).all()
+        with pytest.raises(hip.UgkError, match="max_norm"):
+            hip.call("ugk_extract_pool_clip_i64", tb, ptr(d_ids), ptr(d_off), None, n_rows, nnz, 0, ecode, -1.0,
+                     ptr(d_cache), len(cached), pin.ptr, nkeys, ptr(dev_bytes(n_rows * rb)), rb, ptr(st), None, None,
+                     None, None)
+    finally:
+        sync()
+        pin.free()
+
+
 @pytest.mark.parametrize("n_rows,nnz", [(1, 0), (1, 1), (5, 0), (7, 3), (1000, 1000), (5000, 60_000), (300_000, 40_000),
                                         (3_000_000, 5), (1_000_000, 0), (200, 129)])
 def test_segment_offsets_match_searchsorted(n_rows, nnz):

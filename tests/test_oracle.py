@@ -507,3 +507,42 @@ def test_extract_flat_picks_the_source_per_row_like_numpy_where():
     flat3[cached_rows[0]] = len(cache)
     with pytest.raises(IndexError):
         ORC.extract_flat(flat3, np.array([cached_rows[0]]), cache, host)
+
+
+def test_pool_with_max_norm_on_hand_worked_rows_and_against_numpy():
+    """orc_pool_clip_f64: every looked-up row is clipped to the l2 norm max_norm before it is weighted.  Hand-worked:
+    (3, 4) has norm 5, so max_norm 2.5 halves it and max_norm 10 leaves it alone; (0.6, 0.8) has norm 1 and is never
+    touched; a zero row stays zero.  The denominator of mean / sqrtn is made of the weights alone."""
+    table = np.array([[3.0, 4.0], [0.6, 0.8], [0.0, 0.0], [-6.0, 8.0]])
+    ids = np.array([0, 1, 2, 3, 0])
+    off = np.array([0, 2, 3, 5])
+    w = np.array([1.0, 2.0, 5.0, 1.0, 3.0])
+    got = ORC.pool(table, ids, off, None, "sum", max_norm=2.5)
+    assert np.allclose(got, [[1.5 + 0.6, 2.0 + 0.8], [0, 0], [-1.5 + 1.5, 2.0 + 2.0]], rtol=0, atol=1e-15)
+    got = ORC.pool(table, ids, off, w, "sum", max_norm=2.5)
+    assert np.allclose(got, [[1.5 + 1.2, 2.0 + 1.6], [0, 0], [-1.5 + 4.5, 2.0 + 6.0]], rtol=0, atol=1e-15)
+    got = ORC.pool(table, ids, off, w, "mean", max_norm=2.5)  # divided by 3, 5 and 4: the weights, not the clipped ones
+    assert np.allclose(got, [[2.7 / 3, 3.6 / 3], [0, 0], [3.0 / 4, 8.0 / 4]], rtol=0, atol=1e-15)
+    got = ORC.pool(table, ids, off, w, "sqrtn", max_norm=2.5)
+    assert np.allclose(got, [[2.7 / 5 ** 0.5, 3.6 / 5 ** 0.5], [0, 0], [3.0 / 10 ** 0.5, 8.0 / 10 ** 0.5]], atol=1e-15)
+    assert np.array_equal(ORC.pool(table, ids, off, w, "sum", max_norm=10.0), ORC.pool(table, ids, off, w, "sum"))
+    assert np.array_equal(ORC.pool(table, ids, off, w, "sum", max_norm=None), ORC.pool(table, ids, off, w, "sum"))
+    # against numpy on random segments
+    rng = np.random.default_rng(12)
+    table = rng.standard_normal((400, 9)) * rng.uniform(0.1, 4.0, size=(400, 1))
+    lens = rng.integers(0, 7, size=200)
+    off = np.concatenate([[0], np.cumsum(lens)])
+    ids = rng.integers(0, 400, size=off[-1])
+    w = rng.random(off[-1]) + 0.1
+    seg = np.repeat(np.arange(200), lens)
+    for max_norm in (0.5, 3.0):
+        norms = np.linalg.norm(table, axis=1, keepdims=True)
+        clipped = table * (max_norm / np.maximum(norms, max_norm))
+        assert (np.linalg.norm(clipped, axis=1) <= max_norm * (1 + 1e-12)).all()
+        total = np.zeros((200, 9))
+        np.add.at(total, seg, clipped[ids] * w[:, None])
+        den = np.zeros(200)
+        np.add.at(den, seg, w)
+        assert np.allclose(ORC.pool(table, ids, off, w, 0, max_norm=max_norm), total, rtol=1e-13, atol=1e-13)
+        want = np.where(den[:, None] != 0, total / np.where(den != 0, den, 1.0)[:, None], 0)
+        assert np.allclose(ORC.pool(table, ids, off, w, 1, max_norm=max_norm), want, rtol=1e-13, atol=1e-13)

@@ -104,6 +104,7 @@ void CacheContext::build_with_advise_new_hash(int location_id, std::shared_ptr<C
                                             coll_cache_ptr->_block_density, num_total_nodes, keys_for_each_source,
                                             (int)RunConfig::num_device);
   const size_t num_cached_nodes = keys_for_each_source[location_id]->NumItem();
+  const double detect_s = t.Passed();
   _new_hash_table->_remote_keys = Tensor::Empty(kI32, {0}, CPU_CLIB(), "");
   const size_t num_cpu_nodes = num_total_nodes - num_cached_nodes;
 
@@ -138,6 +139,7 @@ void CacheContext::build_with_advise_new_hash(int location_id, std::shared_ptr<C
     _new_hash_table->CreateHash(_eager_gpu_mem_allocator, std::max<size_t>(_cache_space_capacity, 1), stream);
   }
 
+  const double alloc_s = t.Passed() - detect_s;
   // 4. fill: rows of the cached keys host -> HBM in list order, slot = position in the list
   if (num_cached_nodes > 0) {
     auto cache_node_list = Tensor::CopyToExternal(keys_for_each_source[location_id], _eager_gpu_mem_allocator,
@@ -159,6 +161,7 @@ void CacheContext::build_with_advise_new_hash(int location_id, std::shared_ptr<C
     _new_hash_table->CheckStatus(stream, "cache fill");
   }
   UGK_CALL(ugk_stream_sync(stream));
+  const double fill_s = t.Passed() - detect_s - alloc_s;
 
   // 5. bookkeeping for refresh: cached key list and free slots [n_cached, capacity) (cache_context.cu:2577-2585)
   _new_hash_table->_cached_keys = keys_for_each_source[location_id];
@@ -177,7 +180,8 @@ void CacheContext::build_with_advise_new_hash(int location_id, std::shared_ptr<C
   LOG(INFO) << "Asymm Coll cache (policy: " << (int)RunConfig::cache_policy << ") | local " << num_cached_nodes
             << " / " << num_total_nodes << " nodes ( " << ToPercentage(num_cached_nodes / (double)num_total_nodes)
             << "~" << ToPercentage(cache_percentage) << ") | cpu " << num_cpu_nodes << " / " << num_total_nodes
-            << " | " << ToReadableSize(_cache_nbytes) << " | " << t.Passed() << " secs";
+            << " | " << ToReadableSize(_cache_nbytes) << " | " << t.Passed() << " secs (key list " << detect_s
+            << ", cache space + table " << alloc_s << ", rows + table insert " << fill_s << ")";
   std::cout << "test_result:init:feat_nbytes=" << num_total_nodes * _row_bytes << "\n";
   std::cout << "test_result:init:cache_nbytes=" << _cache_nbytes << "\n";
 }
@@ -587,18 +591,18 @@ static int ExtractMix(ugk_table_t t, const Id64Type *keys, size_t n, const void 
 }
 
 static int ExtractPool(ugk_table_t t, const IdType *ids, const int64_t *seg_off, const float *w, size_t n_rows,
-                       uint64_t nnz, int combiner, int elem_bytes, const void *cache, uint64_t cache_rows,
-                       const void *host, uint64_t host_rows, void *out, size_t rb, uint32_t *st, uint32_t *mirror,
-                       uint64_t *counts, uint32_t *groups, StreamHandle s) {
-  return ugk_extract_pool_u32(t, ids, seg_off, w, n_rows, nnz, combiner, elem_bytes, cache, cache_rows, host, host_rows,
-                              out, rb, st, mirror, counts, groups, s);
+                       uint64_t nnz, int combiner, int elem_bytes, float max_norm, const void *cache,
+                       uint64_t cache_rows, const void *host, uint64_t host_rows, void *out, size_t rb, uint32_t *st,
+                       uint32_t *mirror, uint64_t *counts, uint32_t *groups, StreamHandle s) {
+  return ugk_extract_pool_clip_u32(t, ids, seg_off, w, n_rows, nnz, combiner, elem_bytes, max_norm, cache, cache_rows,
+                                   host, host_rows, out, rb, st, mirror, counts, groups, s);
 }
 static int ExtractPool(ugk_table_t t, const Id64Type *ids, const int64_t *seg_off, const float *w, size_t n_rows,
-                       uint64_t nnz, int combiner, int elem_bytes, const void *cache, uint64_t cache_rows,
-                       const void *host, uint64_t host_rows, void *out, size_t rb, uint32_t *st, uint32_t *mirror,
-                       uint64_t *counts, uint32_t *groups, StreamHandle s) {
-  return ugk_extract_pool_i64(t, ids, seg_off, w, n_rows, nnz, combiner, elem_bytes, cache, cache_rows, host, host_rows,
-                              out, rb, st, mirror, counts, groups, s);
+                       uint64_t nnz, int combiner, int elem_bytes, float max_norm, const void *cache,
+                       uint64_t cache_rows, const void *host, uint64_t host_rows, void *out, size_t rb, uint32_t *st,
+                       uint32_t *mirror, uint64_t *counts, uint32_t *groups, StreamHandle s) {
+  return ugk_extract_pool_clip_i64(t, ids, seg_off, w, n_rows, nnz, combiner, elem_bytes, max_norm, cache, cache_rows,
+                                   host, host_rows, out, rb, st, mirror, counts, groups, s);
 }
 
 static int NonLocalFlags(ugk_table_t t, const IdType *keys, size_t n, uint64_t *flags, StreamHandle s) {
@@ -1116,9 +1120,9 @@ bool ExtractSession::LaunchPooled(const KeyT *nodes, const int64_t *seg_off, con
   }
   CHECK((((uintptr_t)cache | (uintptr_t)host | (uintptr_t)output) & 15u) == 0) << "pooled lookup: misaligned buffer";
   const RecordPlan keys_ready = RecordBegin(stream);
-  UGK_CALL(ExtractPool(table, nodes, seg_off, weights, num_rows, num_nodes, combiner, elem_bytes, cache, cache_rows,
-                       host, ctx->_num_total_nodes, output, rb, _status, _host_mirror, _mix_counts->ptr<uint64_t>(),
-                       &_mix_groups, stream));
+  UGK_CALL(ExtractPool(table, nodes, seg_off, weights, num_rows, num_nodes, combiner, elem_bytes, _pool_max_norm, cache,
+                       cache_rows, host, ctx->_num_total_nodes, output, rb, _status, _host_mirror,
+                       _mix_counts->ptr<uint64_t>(), &_mix_groups, stream));
   if (num_nodes) RecordLaunch(nodes, num_nodes, keys_ready);
   return direct && ctx->_cpu_location_id == -1;
 }

@@ -321,6 +321,14 @@ class ExtractSession {
   // the device-side counting of the following lookups covers only the first `num_keys` keys of a batch
   // (the recorded prefix of LookupManager's record thread); SIZE_MAX, the default: the whole batch
   void SetRecordLimit(size_t num_keys) { _record_limit = num_keys; }
+  // the pooled lookups that follow clip every looked-up row to this l2 norm before it is weighted (the max_norm of
+  // the sparse layer, sparse_lookup_layer.py:95-140); 0, the default: no clipping
+  void SetPooledMaxNorm(float max_norm) { _pool_max_norm = max_norm; }
+
+ private:
+  float _pool_max_norm = 0.f;
+
+ public:
 };
 
 class RefreshSession {

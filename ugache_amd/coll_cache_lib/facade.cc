@@ -147,7 +147,9 @@ void CollCache::build_common(int replica_id, std::function<void()> solve, IdType
   RunConfig::solver_omp_thread_num_per_gpu = std::max<int>(1, RunConfig::omp_thread_num / (int)RunConfig::num_device);
 
   const bool need_solver = (cache_percentage != 0 && cache_percentage != 1);
+  Timer t_solve;
   if (need_solver) solve();
+  LOG(INFO) << "build: placement " << t_solve.Passed() << " s";
   this->_replica_barrier->Wait();
 
   auto cache_ctx = std::make_shared<CacheContext>(_replica_barrier);

@@ -142,14 +142,17 @@ void coll_cache_init(int replica_id, size_t key_space_size, std::function<MemHan
   NormalizeHalf(dtype, dim);
   ContFreqBuf *freq_rank = nullptr;
   const bool need_rank = cache_percentage != 0 && cache_percentage != 1;
+  Timer t_rank;
   if (need_rank) freq_rank = CombineAndRank(replica_id);
+  LOG(INFO) << "build: ranking " << t_rank.Passed() << " s";
+  Timer t_build;
   _coll_cache->build_v2(replica_id, freq_rank, (IdType)key_space_size, allocator, cpu_data, dtype, dim,
                         cache_percentage, stream);
   // COLL_GPU_RECORD_SEED: the counters the lookups bump start from what this cache was ranked by
   auto session = _coll_cache->session(replica_id);
   if (RunConfig::gpu_record_seed && freq_rank && session && session->CountsOnDevice())
     session->SeedHotness(freq_rank->buf, freq_rank->entries.size());
-  LOG(INFO) << "coll cache has been initialized successfully";
+  LOG(INFO) << "coll cache has been initialized successfully: build_v2 " << t_build.Passed() << " s";
 }
 
 extern "C" {
@@ -293,6 +296,12 @@ void coll_cache_lookup_pooled_async_i64(int replica_id, const int64_t *key, cons
   steps[replica_id]++;
   _coll_cache->lookup_pooled_async64(replica_id, key, seg_off, weights, num_rows, num_keys, combiner, elem_bytes,
                                      output, stream);
+}
+
+void coll_cache_set_pooled_max_norm(int replica_id, float max_norm) {
+  CHECK_NOTNULL(_coll_cache);
+  CHECK(max_norm >= 0.f) << "max_norm is an l2 norm (0 turns the clipping off), not " << max_norm;
+  _coll_cache->session(replica_id)->SetPooledMaxNorm(max_norm);
 }
 
 void coll_cache_segment_offsets(int replica_id, const int64_t *sorted_rows, size_t num_entries, size_t num_rows,

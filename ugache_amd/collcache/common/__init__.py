@@ -148,6 +148,7 @@ C_API = {
     "coll_cache_lookup_pooled_async_i64": (None, [ctypes.c_int, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p,
                                                   ctypes.c_size_t, ctypes.c_size_t, ctypes.c_int, ctypes.c_int,
                                                   ctypes.c_void_p, ctypes.c_void_p]),
+    "coll_cache_set_pooled_max_norm": (None, [ctypes.c_int, ctypes.c_float]),
     "coll_cache_segment_offsets": (None, [ctypes.c_int, ctypes.c_void_p, ctypes.c_size_t, ctypes.c_size_t,
                                           ctypes.c_void_p, ctypes.c_void_p]),
     "coll_cache_forward_pooled": (None, [ctypes.c_int, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p,

@@ -185,7 +185,7 @@ _POOL_ELEM = {torch.float32: 4, torch.float16: 2, torch.bfloat16: 0x102}
 
 
 def coll_torch_lookup_pooled(local_id, ids, seg_off, weights=None, combiner="sum", serving_step=False,
-                             stream_ordered=False):
+                             stream_ordered=False, max_norm=None):
     """lookup and per-sample combination of a multi-hot feature in one kernel (extension): segment r is
     ids[seg_off[r] : seg_off[r + 1]]; returns a new [len(seg_off) - 1, dim] tensor whose row r is the weighted sum of
     the segment's embeddings ("sum"), divided by the sum of the weights ("mean") or by the root of the sum of their
@@ -195,8 +195,11 @@ def coll_torch_lookup_pooled(local_id, ids, seg_off, weights=None, combiner="sum
     stream_ordered as well it blocks only if the step's prefix is counted on the host and exceeds 64 KB).
     stream_ordered: the call is enqueued on torch's current stream and returns without waiting, like any torch op
     (as coll_torch_lookup_async is for a plain lookup; `ids`, `seg_off` and `weights` must stay alive until the work has
-    run; coll_torch_lookup_wait reports a bad id or offset and makes the group sizes available)."""
+    run; coll_torch_lookup_wait reports a bad id or offset and makes the group sizes available).
+    max_norm: every looked-up embedding is clipped to this l2 norm before it is weighted (the layer's max_norm)."""
     dev = _State.dev_id.get(local_id, 0)
+    if max_norm is not None and not float(max_norm) > 0:
+        raise ValueError("max_norm must be a positive l2 norm or None, got %r" % (max_norm,))
     if not pooled_lookup_supported():
         raise ValueError("pooled lookups need rows of a multiple of 16 bytes, at most 4096, of fp32, fp16 or bfloat16 "
                          "elements")
@@ -219,9 +222,15 @@ def coll_torch_lookup_pooled(local_id, ids, seg_off, weights=None, combiner="sum
         fn = _C.coll_cache_lookup_pooled_async_i64 if ids.dtype == torch.int64 else _C.coll_cache_lookup_pooled_async
     else:
         fn = _C.coll_cache_lookup_pooled_i64 if ids.dtype == torch.int64 else _C.coll_cache_lookup_pooled
-    fn(local_id, ids.data_ptr() if ids.numel() else None, seg_off.data_ptr(),
-       None if weights is None else weights.data_ptr(), n_rows, ids.numel(), COMBINERS[combiner],
-       _POOL_ELEM[_State.external_dtype], out.data_ptr(), _stream_handle(dev))
+    if max_norm is not None:
+        _C.coll_cache_set_pooled_max_norm(local_id, float(max_norm))
+    try:
+        fn(local_id, ids.data_ptr() if ids.numel() else None, seg_off.data_ptr(),
+           None if weights is None else weights.data_ptr(), n_rows, ids.numel(), COMBINERS[combiner],
+           _POOL_ELEM[_State.external_dtype], out.data_ptr(), _stream_handle(dev))
+    finally:
+        if max_norm is not None:  # the launch has taken it: the lookups that follow are not clipped
+            _C.coll_cache_set_pooled_max_norm(local_id, 0.0)
     return out
 
 

@@ -202,8 +202,8 @@ class SparseLookupLayer(torch.nn.Module):
         self.lookup = LookupLayer(model_name, table_id, emb_vec_size, emb_vec_dtype)
         self.emb_vec_size = emb_vec_size
         self.unique_in_library = bool(kwargs.get("unique_in_library", False))
-        # fused=True: lookup and combination in one kernel of the library (coll_torch_lookup_pooled) wherever that
-        # kernel can take the call (no max_norm, rows it supports); the steps below otherwise
+        # fused=True: lookup, clipping to max_norm and combination in one kernel of the library
+        # (coll_torch_lookup_pooled) wherever that kernel can take the rows; the steps below otherwise
         self.fused = bool(kwargs.get("fused", False))
         # stream_ordered=True (with fused): the step is enqueued on torch's current stream like any torch op (only a
         # recorded prefix beyond 64 KB that is counted on the host still makes it block)
@@ -221,13 +221,15 @@ class SparseLookupLayer(torch.nn.Module):
         # entries as given (row-major order is the caller's contract); coalesce() would merge duplicate positions
         segment_ids = sp_ids._indices()[0]
         ids = sp_ids._values()
-        if self.fused and max_norm is None and _c_lib.pooled_lookup_supported():
+        if max_norm is not None and not float(max_norm) > 0:
+            raise ValueError("max_norm must be a positive l2 norm or None, got %r" % (max_norm,))
+        if self.fused and _c_lib.pooled_lookup_supported():
             self.lookup.check(ids)
             num_rows = int(sp_ids.shape[0])
             seg_off = _adapter.coll_torch_segment_offsets(0, segment_ids, num_rows)
             weights = None if sp_weights is None else sp_weights._values().float()
             return _adapter.coll_torch_lookup_pooled(0, ids, seg_off, weights, combiner, serving_step=True,
-                                                     stream_ordered=self.stream_ordered)
+                                                     stream_ordered=self.stream_ordered, max_norm=max_norm)
         if self.unique_in_library:  # unique + lookup in one call, the unique by the library's GPU hash set
             self.lookup.check(ids)
             emb_unique, idx = _adapter.coll_torch_lookup_unique(0, ids)

@@ -241,7 +241,9 @@ __global__ __launch_bounds__(kBlock) void extract_mix_kernel(ugk_table_t t, cons
     const bool active = lane < KPW && i < n;
     const uint64_t key = active ? key_to_u64<K>(keys[i]) : 0;
     // a full wavefront of keys probes its eight home lines in one go (see hash_probe_home)
-    const Found f = table_lookup<KIND, KPW == kWave ? 1 : 2>(t, key, active);
+    // (fewer keys: their home lines in one go as well, and only the rounds of the probe that have keys to serve)
+    constexpr int ROUNDS = KPW >= 8 ? KPW / 8 : 1;
+    const Found f = table_lookup<KIND, (KPW == kWave || ROUNDS < 8) ? 1 : 2, ROUNDS>(t, key, active);
     const MixRow row = mix_resolve(t, key, active, f, cache, cache_rows, host, host_rows, out, vpr, status, host_mirror);
     if (counts) {
       // rows from the cache, and all others (host rows, and rows skipped for a key without a row: the launch is

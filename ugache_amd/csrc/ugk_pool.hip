@@ -74,7 +74,11 @@ struct PoolElem<__half> {
 
 constexpr int kPoolChunks = 4;  // 16-byte chunks of a row a lane may own: rows of up to LPR x 64 bytes
 
-template <typename K, int KIND, int LPR, typename E>
+// CLIP: every looked-up row is clipped to the l2 norm max_norm before it is weighted (clip_by_norm over the row:
+// x * max_norm / max(||x||, max_norm)).  The whole row has to be seen before any of it can be added, so the chunks of
+// the U rows in flight are held in registers (up to 64 more than without), the squares summed per row over the lanes
+// of the group, and the row's weight scaled; a kernel of its own, so that the plain combination keeps its registers.
+template <typename K, int KIND, int LPR, typename E, bool CLIP>
 __global__ __launch_bounds__(kBlock) void extract_pool_kernel(ugk_table_t t, const K *__restrict__ ids,
                                                               const long long *__restrict__ seg_off,
                                                               const float *__restrict__ weights, size_t n_rows,
@@ -82,7 +86,7 @@ __global__ __launch_bounds__(kBlock) void extract_pool_kernel(ugk_table_t t, con
                                                               uint64_t cache_rows,
                                                               const u32x4 *__restrict__ host, uint64_t host_rows,
                                                               u32x4 *__restrict__ out, uint32_t vpr, int combiner, bool bf16,
-                                                              uint32_t *status, uint32_t *host_mirror,
+                                                              float max_norm, uint32_t *status, uint32_t *host_mirror,
                                                               unsigned long long *counts) {
   constexpr int RPW = kWave / LPR;  // output rows per wavefront and pass
   constexpr int EPC = PoolElem<E>::kPerChunk;
@@ -143,20 +147,61 @@ __global__ __launch_bounds__(kBlock) void extract_pool_kernel(ugk_table_t t, con
           wv[u] = __shfl(w, src);
           ok[u] = __shfl((int)use, src) != 0;
         }
+        if constexpr (CLIP) {
+          u32x4 v[kPoolChunks][U];
+          float ss[U];
 #pragma unroll
-        for (int c = 0; c < kPoolChunks; ++c) {
-          const uint32_t col = (uint32_t)c * LPR + sub;
-          if (col < vpr) {
-            u32x4 v[U];
+          for (int u = 0; u < U; ++u) ss[u] = 0.f;
 #pragma unroll
-            for (int u = 0; u < U; ++u) v[u] = __builtin_nontemporal_load(p[u] + col);
+          for (int c = 0; c < kPoolChunks; ++c) {
+            const uint32_t col = (uint32_t)c * LPR + sub;
+#pragma unroll
+            for (int u = 0; u < U; ++u) v[c][u] = col < vpr ? __builtin_nontemporal_load(p[u] + col) : u32x4{0, 0, 0, 0};
+          }
+#pragma unroll
+          for (int c = 0; c < kPoolChunks; ++c) {
 #pragma unroll
             for (int u = 0; u < U; ++u) {
               float x[EPC];
-              PoolElem<E>::unpack(v[u], x, bf16);
+              PoolElem<E>::unpack(v[c][u], x, bf16);  // a chunk past the row's end is zeros in either two-byte format
+#pragma unroll
+              for (int e = 0; e < EPC; ++e) ss[u] = fmaf(x[e], x[e], ss[u]);
+            }
+          }
+#pragma unroll
+          for (int u = 0; u < U; ++u) {
+#pragma unroll
+            for (int d = LPR / 2; d > 0; d >>= 1) ss[u] += __shfl_xor(ss[u], d);
+            wv[u] *= max_norm / fmaxf(sqrtf(ss[u]), max_norm);
+          }
+#pragma unroll
+          for (int c = 0; c < kPoolChunks; ++c) {
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+              float x[EPC];
+              PoolElem<E>::unpack(v[c][u], x, bf16);
               if (ok[u]) {
 #pragma unroll
                 for (int e = 0; e < EPC; ++e) acc[c][e] = fmaf(wv[u], x[e], acc[c][e]);
+              }
+            }
+          }
+        } else {
+#pragma unroll
+          for (int c = 0; c < kPoolChunks; ++c) {
+            const uint32_t col = (uint32_t)c * LPR + sub;
+            if (col < vpr) {
+              u32x4 v[U];
+#pragma unroll
+              for (int u = 0; u < U; ++u) v[u] = __builtin_nontemporal_load(p[u] + col);
+#pragma unroll
+              for (int u = 0; u < U; ++u) {
+                float x[EPC];
+                PoolElem<E>::unpack(v[u], x, bf16);
+                if (ok[u]) {
+#pragma unroll
+                  for (int e = 0; e < EPC; ++e) acc[c][e] = fmaf(wv[u], x[e], acc[c][e]);
+                }
               }
             }
           }
@@ -349,8 +394,8 @@ __global__ __launch_bounds__(kBlock) void extract_pool_rows_kernel(ugk_table_t t
 template <typename K, int KIND, typename E>
 int extract_pool_lpr(ugk_table_t t, const K *ids, const long long *seg_off, const float *weights, size_t n_rows,
                      const void *cache, uint64_t cache_rows, const void *host, uint64_t host_rows, void *out,
-                     uint32_t vpr, uint64_t nnz, int combiner, bool bf16, uint32_t *status, uint32_t *host_mirror,
-                     uint64_t *counts, uint32_t *num_groups, hipStream_t st) {
+                     uint32_t vpr, uint64_t nnz, int combiner, bool bf16, float max_norm, uint32_t *status,
+                     uint32_t *host_mirror, uint64_t *counts, uint32_t *num_groups, hipStream_t st) {
   // Lanes per output row: rows of up to 512 bytes go to 8 lanes of up to four chunks each (eight lane groups per
   // wavefront; with 32 lanes and two groups 65,536 samples of 16 ids took 123 us instead of 112 us), rows of up to
   // 2 KB to 32 lanes, longer ones to 64.
@@ -372,14 +417,21 @@ int extract_pool_lpr(ugk_table_t t, const K *ids, const long long *seg_off, cons
     if (v >= 1 && v <= kPoolMaxRows) rows = v;
   }
   if (nnz >= ((uint64_t)1 << 28)) rows = 1;  // the list of a group is counted in 32 bits
+  const bool clip = max_norm > 0.f;
+  if (clip) rows = 1;  // clipping lives in the kernel of one output row per lane group
   const size_t rows_per_block = (size_t)rows * groups_per_wave * kWavesPerBlock;
   const unsigned grid = clamp_grid((n_rows + rows_per_block - 1) / rows_per_block, 0);
   if (num_groups) *num_groups = grid;
 #define UGK_POOL(L)                                                                                                    \
-  if (rows == 1)                                                                                                       \
-    hipLaunchKernelGGL((extract_pool_kernel<K, KIND, L, E>), dim3(grid), dim3(kBlock), 0, st, t, ids, seg_off,         \
+  if (clip)                                                                                                            \
+    hipLaunchKernelGGL((extract_pool_kernel<K, KIND, L, E, true>), dim3(grid), dim3(kBlock), 0, st, t, ids, seg_off,   \
                        weights, n_rows, (long long)nnz, (const u32x4 *)cache, cache_rows, (const u32x4 *)host,         \
-                       host_rows, (u32x4 *)out, vpr, combiner, bf16, status, host_mirror,                              \
+                       host_rows, (u32x4 *)out, vpr, combiner, bf16, max_norm, status, host_mirror,                    \
+                       reinterpret_cast<unsigned long long *>(counts));                                                \
+  else if (rows == 1)                                                                                                  \
+    hipLaunchKernelGGL((extract_pool_kernel<K, KIND, L, E, false>), dim3(grid), dim3(kBlock), 0, st, t, ids, seg_off,  \
+                       weights, n_rows, (long long)nnz, (const u32x4 *)cache, cache_rows, (const u32x4 *)host,         \
+                       host_rows, (u32x4 *)out, vpr, combiner, bf16, 0.f, status, host_mirror,                         \
                        reinterpret_cast<unsigned long long *>(counts));                                                \
   else                                                                                                                 \
     hipLaunchKernelGGL((extract_pool_rows_kernel<K, KIND, L, E>), dim3(grid), dim3(kBlock), 0, st, t, ids, seg_off,    \
@@ -434,11 +486,12 @@ __global__ __launch_bounds__(kBlock) void segment_offsets_kernel(const long long
 template <typename K>
 int extract_pool(ugk_table_t t, const K *ids, const int64_t *seg_off, const float *weights, size_t n_rows, uint64_t nnz,
                  int combiner, int elem_bytes, const void *cache, uint64_t cache_rows, const void *host,
-                 uint64_t host_rows, void *out, size_t row_bytes, uint32_t *status, uint32_t *host_mirror,
-                 uint64_t *counts, uint32_t *num_groups, void *stream) {
+                 uint64_t host_rows, void *out, size_t row_bytes, float max_norm, uint32_t *status,
+                 uint32_t *host_mirror, uint64_t *counts, uint32_t *num_groups, void *stream) {
   if (num_groups) *num_groups = 0;
   if (n_rows == 0) return 0;
   UGK_REQUIRE(seg_off && out && status, "ugk_extract_pool: null offsets, output or status");
+  UGK_REQUIRE(max_norm >= 0.f, "ugk_extract_pool: max_norm %g is not a norm (0 = no clipping)", (double)max_norm);
   UGK_REQUIRE(nnz == 0 || ids, "ugk_extract_pool: null ids");
   UGK_REQUIRE(nnz <= (uint64_t)INT64_MAX, "ugk_extract_pool: %llu ids", (unsigned long long)nnz);
   UGK_REQUIRE((uintptr_t)counts % 8 == 0, "ugk_extract_pool: the count words must be 8-byte aligned");
@@ -463,11 +516,11 @@ int extract_pool(ugk_table_t t, const K *ids, const int64_t *seg_off, const floa
   hipStream_t st = as_stream(stream);
 #define UGK_POOL_KIND(KIND)                                                                                          \
   (elem_bytes == 4 ? extract_pool_lpr<K, KIND, float>(t, ids, so, weights, n_rows, cache, cache_rows, host, host_rows, \
-                                                      out, vpr, nnz, combiner, false, status, host_mirror, counts,    \
-                                                      num_groups, st)                                                 \
+                                                      out, vpr, nnz, combiner, false, max_norm, status, host_mirror,  \
+                                                      counts, num_groups, st)                                         \
                    : extract_pool_lpr<K, KIND, __half>(t, ids, so, weights, n_rows, cache, cache_rows, host,          \
-                                                       host_rows, out, vpr, nnz, combiner, bf16, status, host_mirror, \
-                                                       counts, num_groups, st))
+                                                       host_rows, out, vpr, nnz, combiner, bf16, max_norm, status,    \
+                                                       host_mirror, counts, num_groups, st))
   if (t.kind == 0) return UGK_POOL_KIND(0);
   if (t.kind == 1) return UGK_POOL_KIND(1);
   return UGK_POOL_KIND(2);
@@ -500,7 +553,7 @@ int ugk_extract_pool_u32(ugk_table_t t, const uint32_t *ids_dev, const int64_t *
                          uint32_t *status_dev, uint32_t *host_mirror, uint64_t *group_counts_host,
                          uint32_t *num_groups_host, void *stream) {
   return extract_pool<uint32_t>(t, ids_dev, seg_off_dev, weights_dev, n_rows, nnz, combiner, elem_bytes, cache_dev,
-                                cache_rows, host_dev, host_rows, out_dev, row_bytes, status_dev, host_mirror,
+                                cache_rows, host_dev, host_rows, out_dev, row_bytes, 0.f, status_dev, host_mirror,
                                 group_counts_host, num_groups_host, stream);
 }
 
@@ -510,7 +563,29 @@ int ugk_extract_pool_i64(ugk_table_t t, const int64_t *ids_dev, const int64_t *s
                          uint32_t *status_dev, uint32_t *host_mirror, uint64_t *group_counts_host,
                          uint32_t *num_groups_host, void *stream) {
   return extract_pool<int64_t>(t, ids_dev, seg_off_dev, weights_dev, n_rows, nnz, combiner, elem_bytes, cache_dev,
-                               cache_rows, host_dev, host_rows, out_dev, row_bytes, status_dev, host_mirror,
+                               cache_rows, host_dev, host_rows, out_dev, row_bytes, 0.f, status_dev, host_mirror,
+                               group_counts_host, num_groups_host, stream);
+}
+
+int ugk_extract_pool_clip_u32(ugk_table_t t, const uint32_t *ids_dev, const int64_t *seg_off_dev,
+                              const float *weights_dev, size_t n_rows, uint64_t nnz, int combiner, int elem_bytes,
+                              float max_norm, const void *cache_dev, uint64_t cache_rows, const void *host_dev,
+                              uint64_t host_rows, void *out_dev, size_t row_bytes, uint32_t *status_dev,
+                              uint32_t *host_mirror, uint64_t *group_counts_host, uint32_t *num_groups_host,
+                              void *stream) {
+  return extract_pool<uint32_t>(t, ids_dev, seg_off_dev, weights_dev, n_rows, nnz, combiner, elem_bytes, cache_dev,
+                                cache_rows, host_dev, host_rows, out_dev, row_bytes, max_norm, status_dev, host_mirror,
+                                group_counts_host, num_groups_host, stream);
+}
+
+int ugk_extract_pool_clip_i64(ugk_table_t t, const int64_t *ids_dev, const int64_t *seg_off_dev,
+                              const float *weights_dev, size_t n_rows, uint64_t nnz, int combiner, int elem_bytes,
+                              float max_norm, const void *cache_dev, uint64_t cache_rows, const void *host_dev,
+                              uint64_t host_rows, void *out_dev, size_t row_bytes, uint32_t *status_dev,
+                              uint32_t *host_mirror, uint64_t *group_counts_host, uint32_t *num_groups_host,
+                              void *stream) {
+  return extract_pool<int64_t>(t, ids_dev, seg_off_dev, weights_dev, n_rows, nnz, combiner, elem_bytes, cache_dev,
+                               cache_rows, host_dev, host_rows, out_dev, row_bytes, max_norm, status_dev, host_mirror,
                                group_counts_host, num_groups_host, stream);
 }
 

@@ -81,10 +81,13 @@ struct HashProbe {
 // PASSES = 2: two passes of four rounds, the four line loads of a pass in flight together; PASSES = 1: all eight
 // rounds in flight at once, which saves a round trip to memory per wavefront and costs about 30 more vector
 // registers (fewer wavefronts per SIMD: taken where the launch does not fill them all anyway).
-template <int PASSES>
+// ROUNDS: a caller whose keys sit in lanes 0 .. 8 * ROUNDS - 1 only (a wavefront that resolves fewer than 64 keys at a
+// time) runs that many rounds; the shuffles and ballots of a round cost the same whether its lanes hold keys or not.
+template <int PASSES, int ROUNDS = 8>
 __device__ __forceinline__ HashProbe hash_probe_home(const ugk_bucket_t *table, uint64_t nb, uint64_t key,
                                                      bool active) {
-  constexpr int PER = 8 / PASSES;  // rounds whose loads are in flight together
+  static_assert(ROUNDS >= 1 && ROUNDS <= 8 && ROUNDS % PASSES == 0, "whole passes of rounds");
+  constexpr int PER = ROUNDS / PASSES;  // rounds whose loads are in flight together
   HashProbe p{Found{false, 0, 0}, 0, false};
   const int lane = (int)lane_id();
   const int grp = lane >> 3, sub = lane & 7;
@@ -210,17 +213,18 @@ __device__ __forceinline__ Found hash_probe_rest(const ugk_bucket_t *table, uint
   return f;
 }
 
-template <int PASSES = 2>
+template <int PASSES = 2, int ROUNDS = 8>
 __device__ __forceinline__ Found hash_lookup_wave(const ugk_bucket_t *table, uint64_t nb, uint64_t key, bool active) {
-  return hash_probe_rest(table, nb, key, hash_probe_home<PASSES>(table, nb, key, active));
+  return hash_probe_rest(table, nb, key, hash_probe_home<PASSES, ROUNDS>(table, nb, key, active));
 }
 
-// Table lookup dispatch.  KIND is ugk_table_t::kind.  All lanes of the wavefront must call it.
-template <int KIND, int PASSES = 2>
+// Table lookup dispatch.  KIND is ugk_table_t::kind.  All lanes of the wavefront must call it; with ROUNDS < 8 only
+// lanes 0 .. 8 * ROUNDS - 1 may be active.
+template <int KIND, int PASSES = 2, int ROUNDS = 8>
 __device__ __forceinline__ Found table_lookup(const ugk_table_t &t, uint64_t key, bool active) {
   if (KIND == 1) return flat_lookup(reinterpret_cast<const uint32_t *>(t.table), t.size, key, active);
   if (KIND == 2)
-    return hash_lookup_wave<PASSES>(reinterpret_cast<const ugk_bucket_t *>(t.table), t.size, key, active);
+    return hash_lookup_wave<PASSES, ROUNDS>(reinterpret_cast<const ugk_bucket_t *>(t.table), t.size, key, active);
   return Found{false, 0, 0};
 }
 

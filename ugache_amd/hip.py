@@ -113,6 +113,10 @@ SIGNATURES = {
                              _vp, _vp, _vp],
     "ugk_extract_pool_i64": [Table, _vp, _vp, _vp, _sz, _u64, C.c_int, C.c_int, _vp, _u64, _vp, _u64, _vp, _sz, _vp, _vp,
                              _vp, _vp, _vp],
+    "ugk_extract_pool_clip_u32": [Table, _vp, _vp, _vp, _sz, _u64, C.c_int, C.c_int, C.c_float, _vp, _u64, _vp, _u64,
+                                  _vp, _sz, _vp, _vp, _vp, _vp, _vp],
+    "ugk_extract_pool_clip_i64": [Table, _vp, _vp, _vp, _sz, _u64, C.c_int, C.c_int, C.c_float, _vp, _u64, _vp, _u64,
+                                  _vp, _sz, _vp, _vp, _vp, _vp, _vp],
     "ugk_extract_mix_staged_u32": [Table, _vp, _sz, _vp, _u64, _vp, _u64, _vp, _sz, _vp, _vp, _vp, _vp, _u32, Stage, _vp],
     "ugk_extract_mix_staged_i64": [Table, _vp, _sz, _vp, _u64, _vp, _u64, _vp, _sz, _vp, _vp, _vp, _vp, _u32, Stage, _vp],
     "ugk_gather_scatter_staged_u32": [_vp, _u64, _vp, _vp, _sz, _vp, _u64, _sz, Stage, C.c_uint, _vp, _vp, _vp, _vp,
