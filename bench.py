@@ -601,7 +601,7 @@ def run_mixed(args):
         n_hit, n_miss = float(g[1]), float(g[2] - g[1])
         miss_bytes = n_miss * row_bytes
     fused = t_miss == 0.0 and t_idx == 0.0  # one kernel did lookup and both gathers: its time is logged as t_hit
-    entry = 128 if info_cache["table_kind"] == 2 else 4  # bytes of table read per key: a bucket line / a flat word
+    entry = 128 if info_cache["table_kind"] >= 2 else 4  # bytes of table read per key: a line of entries / a flat word
     per_launch_pair_us = t_hit * 1e6
     if fused and not args.dedup:
         # one kernel per step: its average duration over the K back-to-back launches of the stream-ordered leg (two

@@ -84,13 +84,20 @@ def probe_kpw(hip, torch, note, quick=False):
     cases = ((512, 1),) if quick else ((512, 1), (512, 10), (128, 1), (128, 10))
     out_rows = []
     saved = os.environ.get("UGK_MIX_KPW")
-    for kind in ("flat", "hash"):
+    # (BENCH_PROBE_TABLES: a comma-separated subset, to time one table without the others' allocations before it)
+    for kind in os.environ.get("BENCH_PROBE_TABLES", "flat,hash,hash8").split(","):
         for rb, miss_pct in cases:
             ncache = int(rows * (1 - miss_pct / 100))
             if kind == "flat":
                 mem = torch.empty(rows, dtype=torch.int32, device="cuda")
                 hip.call("ugk_fill_u32", mem.data_ptr(), hip.EMPTY_U32, rows, stream)
                 tb = hip.table(hip.TABLE_FLAT, mem.data_ptr(), rows)
+            elif kind == "hash8":  # 8-byte entries keyed by the row, sixteen to a line
+                ne = hip.lib().ugk_hash32_entries_for(ncache, float(os.environ.get("BENCH_PROBE_HASH_LOAD", "0.7")))
+                mem = torch.empty(ne * 8 + 128, dtype=torch.uint8, device="cuda")
+                base = (mem.data_ptr() + 127) // 128 * 128
+                tb = hip.table(hip.TABLE_HASH32, base, ne)
+                hip.call("ugk_table_init", tb, stream)
             else:
                 # (BENCH_PROBE_HASH_LOAD: the same sweep over a sparser table, to see what the keys that need a second
                 # line cost)
@@ -127,6 +134,7 @@ def probe_kpw(hip, torch, note, quick=False):
             _check_status(torch, st, "kpw")
             hip.call("ugk_host_free", host)
             del cache, mem, cached
+            torch.cuda.empty_cache()  # every case allocates afresh: a table in recycled blocks has timed up to 1.7x slower
     if saved is None:
         os.environ.pop("UGK_MIX_KPW", None)
     else:

@@ -68,12 +68,21 @@ typedef struct {
  * kind 0: none (direct mapping, cache_context.h:309-317 IsDirectMapping)
  * kind 1: flat  — uint32 per key of the key space, (loc << 28) + off, 0xffffffff = absent
  *                 (DeviceFlatHashTable, cache_hashtable.cuh:224-251)
- * kind 2: hash  — ugk_bucket_t[size], linear probing (replaces DeviceSimpleHashTable, cuh:154-222) */
+ * kind 2: hash  — ugk_bucket_t[size], linear probing (replaces DeviceSimpleHashTable, cuh:154-222)
+ * kind 3: compact hash — uint64[size] (size a multiple of 16, 128-byte aligned), one word per entry: low half the ROW
+ *                 of the host table the key stands for (the key itself when fb_mul == 0, else (key * fb_mul) & fb_mask:
+ *                 a bijection, so 32 bits identify the key), high half (loc << 28) + off as in the flat table; all ones
+ *                 = never used, low half 0xfffffffe = evicted.  Same 8-byte entry as BucketO2N (cache_hashtable.h:44-49)
+ *                 with sixteen of them probed per 128-byte line; needs rows below 0xfffffffe and slots below 2^28.
+ *                 Every ugk_* call that takes a table takes the caller's keys for it, whatever the kind. */
+#define UGK_TABLE_FLAT 1
+#define UGK_TABLE_HASH 2
+#define UGK_TABLE_HASH32 3
 typedef struct {
   int32_t kind;
   int32_t reserved;
   void *table;
-  uint64_t size; /* flat: number of keys; hash: number of buckets */
+  uint64_t size; /* flat: number of keys; hash: number of buckets (kind 3: of 8-byte entries) */
   /* host row of a key the table does not hold: key itself when fb_mul == 0 (the reference's CPUFallback,
    * cache_hashtable.cuh:388-395), else (key * fb_mul) & fb_mask — the inverse of an odd-multiplier bijection on
    * 2^k ids, which lets sparse hashed ids address a dense host table without a second table */
@@ -196,6 +205,11 @@ int ugk_gather_idx(const void *src_dev, uint64_t src_rows, const ugk_idx_t *idx_
 /* number of buckets for n entries at the given load factor (replaces TableSize, cache_hashtable.cu:222-225) */
 size_t ugk_hash_buckets_for(size_t n_entries, double load_factor);
 int ugk_hash_init(ugk_bucket_t *table_dev, size_t nbuckets, void *stream);
+/* the same for a table of any kind: entries of a compact table (kind 3) for n keys at the given load factor, a multiple
+ * of 16; every entry of `t` set to "never used" / "absent"; the census of ugk_hash_census for kind 2 or 3 */
+size_t ugk_hash32_entries_for(size_t n_entries, double load_factor);
+int ugk_table_init(ugk_table_t t, void *stream);
+int ugk_table_census(ugk_table_t t, uint64_t *census_dev, void *stream);
 /* insert_hashmap_unique + InsertWithLoc / InsertSeqOffWithLoc (cache_hashtable.cu:249-268;
  * cache_hashtable.cuh:601-608): value = (loc, offs ? offs[i] : seq_base + i).  Keys must be unique and absent. */
 int ugk_table_insert_u32(ugk_table_t t, const uint32_t *keys_dev, const uint32_t *offs_dev, uint32_t seq_base,

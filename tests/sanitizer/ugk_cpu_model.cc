@@ -99,6 +99,12 @@ uint64_t fallback_row(const ugk_table_t &t, uint64_t key) {
   return key <= t.fb_mask ? ((key * t.fb_mul) & t.fb_mask) : ~0ull;
 }
 
+constexpr uint32_t kH32Tomb = 0xfffffffeu;
+constexpr uint64_t kH32EmptyWord = ~0ull, kH32TombWord = 0x00000000fffffffeull;
+uint64_t h32_home(uint64_t row, uint64_t nentries) {
+  return (uint64_t)(((unsigned __int128)fmix64(row) * (nentries >> 4)) >> 64) << 4;
+}
+
 struct Found {
   bool hit;
   uint32_t loc, off;
@@ -124,12 +130,29 @@ Found lookup(const ugk_table_t &t, uint64_t key) {
       if (cur == UGK_HASH_EMPTY) return f;
       if (++pos == t.size) pos = 0;
     }
+  } else if (t.kind == 3) {
+    // 8-byte entries {row, (loc << 28) + off}, keyed by the row the key stands for; probing starts at a 16-entry line
+    const uint64_t row = fallback_row(t, key);
+    if (row >= kH32Tomb) return f;
+    const uint64_t *w = reinterpret_cast<const uint64_t *>(t.table);
+    uint64_t pos = h32_home(row, t.size);
+    for (uint64_t step = 0; step < t.size; ++step) {
+      const uint64_t cur = ld(w + pos);
+      if ((uint32_t)cur == (uint32_t)row) {
+        const uint32_t v = (uint32_t)(cur >> 32);
+        return Found{true, (v >> 28) & 0xfu, v & 0x0fffffffu};
+      }
+      if (cur == kH32EmptyWord) return f;
+      if (++pos == t.size) pos = 0;
+    }
   }
   return f;
 }
 int check_table(const ugk_table_t &t, const char *who) {
-  REQUIRE(t.kind == 1 || t.kind == 2, "%s: table kind %d is not flat(1) or hash(2)", who, t.kind);
+  REQUIRE(t.kind >= 1 && t.kind <= 3, "%s: table kind %d is not flat(1), hash(2) or compact hash(3)", who, t.kind);
   REQUIRE(t.table && t.size, "%s: empty table", who);
+  if (t.kind == 2) REQUIRE(t.size % 8 == 0 && (uintptr_t)t.table % 128 == 0, "%s: hash table layout", who);
+  if (t.kind == 3) REQUIRE(t.size % 16 == 0 && (uintptr_t)t.table % 128 == 0, "%s: compact hash table layout", who);
   return 0;
 }
 
@@ -180,6 +203,38 @@ int table_insert(ugk_table_t t, const K *keys, const uint32_t *offs, uint32_t se
       const uint32_t old = __atomic_exchange_n(reinterpret_cast<uint32_t *>(t.table) + key, (loc << 28) + off,
                                                __ATOMIC_ACQ_REL);
       if (old != UGK_EMPTY_U32) or_status(status, UGK_ST_DUP_KEY);
+      continue;
+    }
+    if (t.kind == 3) {
+      const uint64_t row = fallback_row(t, key);
+      if (row >= kH32Tomb || off > 0x0fffffffu) {
+        or_status(status, UGK_ST_KEY_OUT_OF_RANGE);
+        continue;
+      }
+      uint64_t *w = reinterpret_cast<uint64_t *>(t.table);
+      uint64_t pos = h32_home(row, t.size), first_tomb = ~0ull;
+      bool dup = false;
+      for (uint64_t step = 0; step < t.size; ++step) {
+        const uint64_t cur = ld(w + pos);
+        if ((uint32_t)cur == (uint32_t)row) {
+          dup = true;
+          break;
+        }
+        if (cur == kH32EmptyWord) break;
+        if (cur == kH32TombWord && first_tomb == ~0ull) first_tomb = pos;
+        if (++pos == t.size) pos = 0;
+      }
+      if (dup) {
+        or_status(status, UGK_ST_DUP_KEY);
+        continue;
+      }
+      const uint64_t target = first_tomb != ~0ull ? first_tomb : pos;
+      const uint64_t cur = ld(w + target);
+      if (cur != kH32EmptyWord && cur != kH32TombWord) {
+        or_status(status, UGK_ST_TABLE_FULL);
+        continue;
+      }
+      st(w + target, ((uint64_t)(((loc & 0xfu) << 28) + off) << 32) | (uint32_t)row);  // row and value appear together
       continue;
     }
     if (key >= UGK_HASH_TOMB) {
@@ -236,6 +291,25 @@ int table_evict(ugk_table_t t, const K *keys, size_t n, uint32_t *status, uint64
           __atomic_exchange_n(reinterpret_cast<uint32_t *>(t.table) + key, UGK_EMPTY_U32, __ATOMIC_ACQ_REL);
       if (old == UGK_EMPTY_U32) or_status(status, UGK_ST_EVICT_ABSENT);
       else release(old & 0x0fffffffu);
+      continue;
+    }
+    if (t.kind == 3) {
+      const uint64_t row = fallback_row(t, key);
+      uint64_t *w = reinterpret_cast<uint64_t *>(t.table);
+      uint64_t pos = row < kH32Tomb ? h32_home(row, t.size) : 0;
+      bool gone = false;
+      for (uint64_t step = 0; step < t.size && row < kH32Tomb; ++step) {
+        const uint64_t cur = ld(w + pos);
+        if ((uint32_t)cur == (uint32_t)row) {
+          release((uint32_t)(cur >> 32) & 0x0fffffffu);
+          st(w + pos, kH32TombWord);
+          gone = true;
+          break;
+        }
+        if (cur == kH32EmptyWord) break;
+        if (++pos == t.size) pos = 0;
+      }
+      if (!gone) or_status(status, UGK_ST_EVICT_ABSENT);
       continue;
     }
     ugk_bucket_t *b = reinterpret_cast<ugk_bucket_t *>(t.table);
@@ -954,6 +1028,39 @@ int ugk_hash_census(const ugk_bucket_t *table, size_t nbuckets, uint64_t *census
     const uint64_t k = ld(&table[i].key);
     if (k == UGK_HASH_EMPTY) ++empty;
     else if (k == UGK_HASH_TOMB) ++tomb;
+    else ++occ;
+  }
+  census[0] = occ;
+  census[1] = tomb;
+  census[2] = empty;
+  return 0;
+}
+
+size_t ugk_hash32_entries_for(size_t n_entries, double load_factor) {
+  if (!(load_factor > 0.0) || load_factor > 0.95) load_factor = 0.7;
+  size_t ne = (size_t)std::ceil((double)n_entries / load_factor) + 1;
+  if (ne < 64) ne = 64;
+  return (ne + 15) / 16 * 16;
+}
+int ugk_table_init(ugk_table_t t, void *stream) {
+  if (check_table(t, "ugk_table_init")) return 1;
+  if (t.kind == 1) return ugk_fill_u32(static_cast<uint32_t *>(t.table), UGK_EMPTY_U32, t.size, stream);
+  if (t.kind == 2) return ugk_hash_init(static_cast<ugk_bucket_t *>(t.table), t.size, stream);
+  uint64_t *w = static_cast<uint64_t *>(t.table);
+  for (size_t i = 0; i < t.size; ++i) st(w + i, kH32EmptyWord);
+  return 0;
+}
+int ugk_table_census(ugk_table_t t, uint64_t *census, void *stream) {
+  if (check_table(t, "ugk_table_census")) return 1;
+  REQUIRE(t.kind == 2 || t.kind == 3, "ugk_table_census: a flat table has no buckets to count");
+  REQUIRE(census, "ugk_table_census: null output");
+  if (t.kind == 2) return ugk_hash_census(static_cast<const ugk_bucket_t *>(t.table), t.size, census, stream);
+  uint64_t occ = 0, tomb = 0, empty = 0;
+  const uint64_t *w = static_cast<const uint64_t *>(t.table);
+  for (size_t i = 0; i < t.size; ++i) {
+    const uint32_t k = (uint32_t)ld(w + i);
+    if (k == 0xffffffffu) ++empty;
+    else if (k == kH32Tomb) ++tomb;
     else ++occ;
   }
   census[0] = occ;

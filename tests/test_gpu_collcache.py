@@ -151,7 +151,7 @@ def test_build_of_every_replica_with_an_allocator_builder(pct):
         assert handed_out
 
 
-@pytest.mark.parametrize("table_kind", ["FLAT", "HASH"])
+@pytest.mark.parametrize("table_kind", ["FLAT", "HASH", "HASH16"])
 @pytest.mark.parametrize("impl", ["", "SMMaskPhase", "DIRECT", "NONE"])
 @pytest.mark.parametrize("kdtype", [torch.int32, torch.int64])
 def test_partial_cache_matches_oracle(table_kind, impl, kdtype, monkeypatch):
@@ -174,7 +174,7 @@ def test_partial_cache_matches_oracle(table_kind, impl, kdtype, monkeypatch):
 
     want_cached, nid = expected_cached_set(np.concatenate(stream).astype(np.uint32), n_item, pct)
     info = _basics.info(0)
-    assert info["table_kind"] == (1 if table_kind == "FLAT" else 2)
+    assert info["table_kind"] == {"FLAT": 1, "HASH": 3, "HASH16": 2}[table_kind]  # HASH: 8-byte entries when they fit
     assert info["capacity_rows"] == ORC.lib.orc_cache_capacity(n_item, pct)
     assert info["cached_rows"] == len(want_cached) == int(n_item * (pct * 100 / 100.0))
     assert info["free_slots"] == info["capacity_rows"] - info["cached_rows"]
@@ -397,7 +397,7 @@ def test_raw_model_directory_and_mock_table(tmp_path):
     assert tuple(mock.shape) == (1000, 16) and not mock.any()
 
 
-@pytest.mark.parametrize("table_kind", ["FLAT", "HASH"])
+@pytest.mark.parametrize("table_kind", ["FLAT", "HASH", "HASH16"])
 @pytest.mark.parametrize("foreground", [True, False])
 @pytest.mark.parametrize("impl", ["", "SMMaskPhase"])
 def test_refresh_evicts_and_inserts_like_the_oracle(table_kind, foreground, impl, monkeypatch):
@@ -456,7 +456,7 @@ def test_refresh_evicts_and_inserts_like_the_oracle(table_kind, foreground, impl
         old_cached = new_cached
 
 
-@pytest.mark.parametrize("table_kind", ["FLAT", "HASH"])
+@pytest.mark.parametrize("table_kind", ["FLAT", "HASH", "HASH16"])
 @pytest.mark.parametrize("foreground", [True, False])
 @pytest.mark.parametrize("keep", [False, True])
 @pytest.mark.parametrize("stage", [0, 16384])
@@ -1036,7 +1036,7 @@ def _random_case(seed):
     dims = [1, 2, 3, 4, 8, 12, 16, 31, 32, 64, 100, 128, 256, 300]
     return dict(seed=seed, n_item=int(r.integers(1, 60_000)), dim=int(r.choice(dims)),
                 pct=float(r.choice([0.0, 0.01, 0.1, 0.37, 0.9, 0.999, 1.0])),
-                table_kind=str(r.choice(["FLAT", "HASH"])), impl=str(r.choice(["", "SMMaskPhase", "NONE"])),
+                table_kind=str(r.choice(["FLAT", "HASH", "HASH16"])), impl=str(r.choice(["", "SMMaskPhase", "NONE"])),
                 i64=bool(r.integers(0, 2)), dedup=bool(r.integers(0, 4) == 0), gpu_record=bool(r.integers(0, 4) == 0),
                 zipf=float(r.choice([0.6, 1.05, 1.4])), half=bool(r.integers(0, 3) == 0),
                 stage=int(r.choice([0, 0, 1024])))
@@ -1167,7 +1167,7 @@ def test_refresh_of_a_table_too_small_for_spare_slots(device, monkeypatch):
 def _random_refresh_case(seed):
     r = np.random.default_rng(5000 + seed)
     return dict(seed=seed, n_item=int(r.integers(130, 90_000)), dim=int(r.choice([4, 16, 32, 64, 100])),
-                pct=float(r.choice([0.01, 0.1, 0.37, 0.9, 0.99])), table_kind=str(r.choice(["FLAT", "HASH"])),
+                pct=float(r.choice([0.01, 0.1, 0.37, 0.9, 0.99])), table_kind=str(r.choice(["FLAT", "HASH", "HASH16"])),
                 keep=bool(r.integers(0, 2)), sparse=bool(r.integers(0, 3) == 0), zipf=float(r.choice([0.6, 1.05, 1.4])),
                 rounds=int(r.integers(2, 5)), stream_ordered=bool(r.integers(0, 3) == 0),
                 stage=int(r.choice([0, 256, 65536])), stable=bool(r.integers(0, 3) == 0))
@@ -1363,7 +1363,7 @@ def test_sparse_ids_hash_table_with_refresh_each_step(gpu_record, monkeypatch):
     table = fill_table(emb, rng)
     co.coll_torch_init_t(0, 0, emb, pct)
     info = _basics.info(0)
-    assert info["table_kind"] == 2 and info["row_bytes"] == 128
+    assert info["table_kind"] == 3 and info["row_bytes"] == 128  # sparse ids: the 8-byte entries, keyed by the row
     cached, nid = expected_cached_set(np.concatenate(s0).astype(np.uint32), n_item, pct)
     cap = info["capacity_rows"]
     assert info["cached_rows"] == len(cached)
@@ -1518,7 +1518,7 @@ def test_serving_stack_from_a_ps_config_file(tmp_path):
         hps.Shutdown()
 
 
-@pytest.mark.parametrize("pct,table_kind", [(1.0, "FLAT"), (0.0, "FLAT"), (0.3, "FLAT"), (0.3, "HASH")])
+@pytest.mark.parametrize("pct,table_kind", [(1.0, "FLAT"), (0.0, "FLAT"), (0.3, "FLAT"), (0.3, "HASH"), (0.3, "HASH16")])
 @pytest.mark.parametrize("dtype,dim", [(torch.float32, 32), (torch.float16, 64), (torch.float32, 100)])
 @pytest.mark.parametrize("kdtype", [torch.int32, torch.int64])
 def test_pooled_lookup_through_the_library(pct, table_kind, dtype, dim, kdtype, monkeypatch):
@@ -1572,7 +1572,7 @@ def test_pooled_lookup_through_the_library(pct, table_kind, dtype, dim, kdtype, 
         assert co.c_lib.pooled_lookup_supported()
 
 
-@pytest.mark.parametrize("pct,table_kind", [(1.0, "FLAT"), (0.0, "FLAT"), (0.3, "FLAT"), (0.3, "HASH")])
+@pytest.mark.parametrize("pct,table_kind", [(1.0, "FLAT"), (0.0, "FLAT"), (0.3, "FLAT"), (0.3, "HASH"), (0.3, "HASH16")])
 @pytest.mark.parametrize("kdtype", [torch.int32, torch.int64])
 def test_stream_ordered_pooled_lookups(pct, table_kind, kdtype, monkeypatch):
     """coll_torch_lookup_pooled(stream_ordered=True) (coll_cache_lookup_pooled_async*): several batches enqueued back
@@ -1713,7 +1713,7 @@ def test_counting_every_third_lookup_on_the_device(impl, monkeypatch):
     assert np.array_equal(got_k[:m], want_k) and np.array_equal(got_c[:m], want_c)
 
 
-@pytest.mark.parametrize("table_kind", ["FLAT", "HASH"])
+@pytest.mark.parametrize("table_kind", ["FLAT", "HASH", "HASH16"])
 @pytest.mark.parametrize("stage", [0, 8192])
 @pytest.mark.parametrize("dim", [32, 12])
 def test_lookups_stay_exact_while_the_device_refreshes_under_them(table_kind, stage, dim, monkeypatch):

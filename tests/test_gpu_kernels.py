@@ -196,6 +196,17 @@ def _make_hash(n_entries, load=0.7):
     return t, hip.table(hip.TABLE_HASH, base, nb), nb
 
 
+def _make_hash32(n_entries, load=0.7, fb_mul=0, fb_mask=0):
+    """the compact hash table (kind 3): 8-byte entries, sixteen to a 128-byte line, keyed by the row a key stands for"""
+    ne = hip.lib().ugk_hash32_entries_for(n_entries, load)
+    assert ne % 16 == 0
+    t = dev_bytes(ne * 8 + 128)
+    base = (ptr(t) + 127) // 128 * 128
+    tb = hip.table(hip.TABLE_HASH32, base, ne, fb_mul, fb_mask)
+    hip.call("ugk_table_init", tb, None)
+    return t, tb, ne
+
+
 def _lookup(tb, keys_np, fallback=1):
     n = len(keys_np)
     loc = dev_zeros_u32(n)
@@ -364,6 +375,165 @@ def test_hash_table_dense_collisions_and_host_entries():
     assert loc[0] == 1
 
 
+# ---- the compact hash table (kind 3): keyed by the row a key stands for --------------------------------------------
+def _census(tb):
+    cen = torch.zeros(3, dtype=torch.int64, device="cuda")
+    hip.call("ugk_table_census", tb, cen.data_ptr(), None)
+    sync()
+    return cen.cpu().tolist()
+
+
+def _sparse_map(bits=40):
+    """an odd multiplier and its inverse modulo 2^bits: ids = (rows * mul) & mask, rows = (ids * inv) & mask"""
+    mask = (1 << bits) - 1
+    mul = (0x9E3779B97F4A7C15 | 1) & mask
+    return mul, pow(mul, -1, 1 << bits), mask
+
+
+@pytest.mark.parametrize("keys_are", ["u32", "i64_rows", "i64_sparse_ids"])
+@pytest.mark.parametrize("n", [10, 1000, 200_000])
+def test_compact_hash_table_against_dict_and_oracle_table(keys_are, n):
+    rng = np.random.default_rng(n + len(keys_are))
+    kdtype = np.uint32 if keys_are == "u32" else np.int64
+    row_space = 1 << 28 if keys_are == "u32" else 0xFFFFFFFE  # rows the table can hold: all below the tombstone mark
+    rows = np.unique(np.concatenate([rng.integers(0, row_space, size=n * 2), [row_space - 1, 0]]))
+    rng.shuffle(rows)
+    rows = rows[:n].astype(np.uint64)
+    n = len(rows)
+    fb_mul = inv = fb_mask = 0
+    if keys_are == "i64_sparse_ids":
+        mul, inv, fb_mask = _sparse_map()
+        fb_mul = inv  # the table turns an id back into its row
+        keys = ((rows * np.uint64(mul)) & np.uint64(fb_mask)).astype(np.int64)
+    else:
+        keys = rows.astype(kdtype)
+    offs = rng.integers(0, 1 << 28, size=n).astype(np.uint32)
+    mem, tb, ne = _make_hash32(n, fb_mul=fb_mul, fb_mask=fb_mask)
+    assert _census(tb) == [0, 0, ne]
+    assert _insert(tb, keys, offs, loc=0) == 0
+    absent_rows = np.setdiff1d(rng.integers(0, row_space, size=n).astype(np.uint64), rows)
+    absent = (((absent_rows * np.uint64(mul)) & np.uint64(fb_mask)).astype(np.int64)
+              if keys_are == "i64_sparse_ids" else absent_rows.astype(kdtype))
+    q = np.concatenate([keys, absent, keys[::-1][: n // 2]])
+    q_rows = np.concatenate([rows, absent_rows, rows[::-1][: n // 2]])
+    loc, off = _lookup(tb, q)
+    model = dict(zip(keys.tolist(), offs.tolist()))
+    want_loc = np.array([0 if int(k) in model else 1 for k in q], np.uint32)
+    want_off = np.array([model.get(int(k), int(r) & 0xFFFFFFFF) for k, r in zip(q, q_rows)], np.uint32)
+    assert np.array_equal(loc, want_loc) and np.array_equal(off, want_off)
+    if keys_are == "u32":
+        ot = ORC.simple_table(n)
+        ORC.simple_insert(ot, keys, offs)
+        want = ORC.lookup_src_dst(q.astype(np.uint32), simple=ot, fallback_loc=1)
+        assert np.array_equal(loc, want["src"] >> 28) and np.array_equal(off, want["src"] & 0x0FFFFFFF)
+    assert _census(tb) == [n, 0, ne - n]
+    ev = keys[: n // 2]
+    assert _evict(tb, ev) == 0
+    loc, off = _lookup(tb, keys)
+    assert (loc[: n // 2] == 1).all() and (loc[n // 2:] == 0).all()
+    assert np.array_equal(off[n // 2:], offs[n // 2:])
+    assert _census(tb) == [n - n // 2, n // 2, ne - n]
+    assert _evict(tb, ev[:1]) & hip.ST_EVICT_ABSENT
+    new_offs = (offs[: n // 2] ^ 0x5555).astype(np.uint32)
+    assert _insert(tb, ev, new_offs) == 0
+    loc, off = _lookup(tb, keys)
+    assert (loc == 0).all() and np.array_equal(off[: n // 2], new_offs)
+    assert _insert(tb, keys[:1], offs[:1]) & hip.ST_DUP_KEY
+    occ, tomb, empty = _census(tb)
+    assert occ == n and occ + tomb + empty == ne
+
+
+def test_compact_hash_table_refuses_what_its_entries_cannot_hold():
+    """a row at or above the tombstone mark, an id beyond the id space of the key map, an offset wider than 28 bits:
+    refused on insert with KEY_OUT_OF_RANGE, a miss on lookup, absent on evict"""
+    mem, tb, ne = _make_hash32(100)
+    for bad in (0xFFFFFFFE, 0xFFFFFFFF, 1 << 32, (1 << 40) + 5):
+        assert _insert(tb, np.array([bad], np.int64)) & hip.ST_KEY_OUT_OF_RANGE
+        loc, off = _lookup(tb, np.array([bad], np.int64), fallback=7)
+        assert loc[0] == 7 and off[0] == bad & 0xFFFFFFFF
+        assert _evict(tb, np.array([bad], np.int64)) & hip.ST_EVICT_ABSENT
+    assert _insert(tb, np.array([5], np.int64), np.array([1 << 28], np.uint32)) & hip.ST_KEY_OUT_OF_RANGE
+    assert _census(tb) == [0, 0, ne]
+    assert _insert(tb, np.array([0xFFFFFFFD, 5], np.int64), np.array([(1 << 28) - 1, 0], np.uint32), loc=3) == 0
+    loc, off = _lookup(tb, np.array([0xFFFFFFFD, 5, 6], np.int64), fallback=7)
+    assert loc.tolist() == [3, 3, 7] and off.tolist() == [(1 << 28) - 1, 0, 6]
+    mul, inv, mask = _sparse_map(20)
+    mem2, tb2, _ = _make_hash32(100, fb_mul=inv, fb_mask=mask)
+    assert _insert(tb2, np.array([mask + 1], np.int64)) & hip.ST_KEY_OUT_OF_RANGE  # no row stands behind this id
+    loc, off = _lookup(tb2, np.array([mask + 1], np.int64), fallback=7)
+    assert loc[0] == 7
+
+
+@pytest.mark.parametrize("load", [0.5, 0.7, 0.9])
+def test_compact_hash_table_under_churn_follows_a_dict(load):
+    """as test_hash_table_under_churn_follows_a_dict, on 8-byte entries: tombstones pile up between rounds, every
+    present key returns its latest value, every evicted or never-inserted key misses"""
+    rng = np.random.default_rng(int(load * 10) + 100)
+    n = 40_000
+    space = 0xFFFFFFFE
+    mem, tb, ne = _make_hash32(n, load=load)
+    model = {}
+    keys = np.unique(rng.integers(0, space, size=2 * n))[:n].astype(np.int64)
+    keys = rng.permutation(keys)
+    offs = rng.integers(0, 1 << 28, size=n).astype(np.uint32)
+    assert _insert(tb, keys, offs) == 0
+    model.update(zip(keys.tolist(), offs.tolist()))
+    gone = set()
+    for rnd in range(12):
+        present = np.fromiter(model.keys(), np.int64, len(model))
+        ev = rng.choice(present, n // 10, replace=False)
+        assert _evict(tb, ev) == 0
+        for k in ev.tolist():
+            del model[k]
+            gone.add(k)
+        fresh = np.setdiff1d(np.unique(rng.integers(0, space, size=n // 5)).astype(np.int64), present)[: n // 10]
+        back = np.array(list(gone)[: n // 50], np.int64)
+        ins = np.unique(np.concatenate([back, fresh]))
+        ins = rng.permutation(ins)[: n // 10]
+        ins_off = rng.integers(0, 1 << 28, size=len(ins)).astype(np.uint32)
+        st = _insert(tb, ins, ins_off, loc=rnd % 16)
+        assert st == 0, (rnd, st)
+        for k, o in zip(ins.tolist(), ins_off.tolist()):
+            model[k] = o | ((rnd % 16) << 28)
+            gone.discard(k)
+        present = np.fromiter(model.keys(), np.int64, len(model))
+        absent = np.array(list(gone)[:5000] + rng.integers(1 << 33, 1 << 42, size=1000).tolist(), np.int64)
+        loc, off = _lookup(tb, np.concatenate([present, absent]), fallback=99)
+        want = np.array([model[k] for k in present.tolist()], np.uint32)
+        assert (loc[len(present):] == 99).all(), rnd
+        assert np.array_equal(loc[: len(present)], want >> 28) and np.array_equal(off[: len(present)], want & 0x0FFFFFFF), rnd
+        occ, tomb, empty = _census(tb)
+        assert occ == len(model) and occ + tomb + empty == ne, rnd
+
+
+def test_compact_hash_table_dense_collisions_full_table_and_no_never_used_entry():
+    n = 50_000
+    keys = (np.arange(n, dtype=np.int64) * 7 + 3)
+    mem, tb, ne = _make_hash32(n, load=0.9)
+    half = n // 2
+    assert _insert(tb, keys[:half], seq_base=100, loc=hip.LOC_LOCAL) == 0
+    assert _insert(tb, keys[half:], seq_base=0, loc=hip.LOC_HOST) == 0
+    loc, off = _lookup(tb, keys, fallback=9)
+    assert (loc[:half] == 0).all() and (loc[half:] == 1).all()
+    assert np.array_equal(off[:half], 100 + np.arange(half, dtype=np.uint32))
+    assert np.array_equal(off[half:], np.arange(n - half, dtype=np.uint32))
+    loc, off = _lookup(tb, keys + 1, fallback=9)
+    assert (loc == 9).all()
+    # every entry taken: one more key does not fit, and a lookup of an absent key ends after one lap
+    mem2, tb2, ne2 = _make_hash32(10, load=0.9)
+    assert _insert(tb2, np.arange(ne2, dtype=np.int64)) == 0
+    assert _census(tb2) == [ne2, 0, 0]
+    assert _insert(tb2, np.array([ne2 + 5], np.int64)) & hip.ST_TABLE_FULL
+    loc, off = _lookup(tb2, np.array([10_000_000, 3], np.int64), fallback=1)
+    assert loc.tolist() == [1, 0] and off[1] == 3
+    # evicted entries are reused although no never-used entry is left
+    assert _evict(tb2, np.array([3, 17], np.int64)) == 0
+    assert _insert(tb2, np.array([1000, 1001], np.int64), np.array([7, 8], np.uint32)) == 0
+    assert _census(tb2) == [ne2, 0, 0]
+    loc, off = _lookup(tb2, np.array([1000, 1001, 3, 17, 4], np.int64), fallback=1)
+    assert loc.tolist() == [0, 0, 1, 1, 0] and off[:2].tolist() == [7, 8]
+
+
 # ------------------------------------------------------------------------------------------------------
 # classify + partition + factored gather
 # ------------------------------------------------------------------------------------------------------
@@ -381,7 +551,7 @@ def _classify(tb, keys_np, host_rows):
     return idx, counts, c, status_value(st), keys
 
 
-@pytest.mark.parametrize("mode", ["flat", "hash"])
+@pytest.mark.parametrize("mode", ["flat", "hash", "hash32"])
 @pytest.mark.parametrize("kdtype", [np.uint32, np.int64])
 @pytest.mark.parametrize("n", [0, 1, 1023, 1024, 1025, 70_001])
 def test_classify_partition_and_factored_gather(mode, kdtype, n):
@@ -395,7 +565,7 @@ def test_classify_partition_and_factored_gather(mode, kdtype, n):
     if mode == "flat":
         mem, tb = _make_flat(nkeys)
     else:
-        mem, tb, _ = _make_hash(len(cached))
+        mem, tb, _ = (_make_hash32 if mode == "hash32" else _make_hash)(len(cached))
     assert _insert(tb, cached.astype(kdtype)) == 0
     oflat = ORC.flat_table(nkeys)
     ORC.lib.orc_flat_insert(oflat, cached, np.arange(len(cached), dtype=np.uint32), len(cached))
@@ -532,7 +702,7 @@ def test_outputs_beyond_4_GiB():
         mirror.free()
 
 
-@pytest.mark.parametrize("kind", ["flat", "hash"])
+@pytest.mark.parametrize("kind", ["flat", "hash", "hash32"])
 @pytest.mark.parametrize("rb", [32, 128, 512, 2048])
 def test_extract_mix_at_every_launch_shape(kind, rb):
     """the fused kernel cuts a batch into wavefronts of 8, 16, 32 or 64 keys by the batch size, the table kind, the row
@@ -547,7 +717,7 @@ def test_extract_mix_at_every_launch_shape(kind, rb):
     if kind == "flat":
         mem, tb = _make_flat(nkeys)
     else:
-        mem, tb, _ = _make_hash(len(cached))
+        mem, tb, _ = (_make_hash32 if kind == "hash32" else _make_hash)(len(cached))
     assert _insert(tb, cached, slots) == 0
     is_cached = np.zeros(nkeys, bool)
     is_cached[cached] = True
@@ -609,7 +779,7 @@ _POOL_CASES = [(d, e, "") for d, e in _POOL_SHAPES] + [
                                                (64, "bf16")]]
 
 
-@pytest.mark.parametrize("kind", ["none", "flat", "hash"])
+@pytest.mark.parametrize("kind", ["none", "flat", "hash", "hash32"])
 @pytest.mark.parametrize("dim,etype,rows_per_group", _POOL_CASES)
 def test_pooled_extraction_matches_a_float64_segment_sum(kind, dim, etype, rows_per_group, monkeypatch):
     """ugk_extract_pool_*: rows looked up and combined per segment in one kernel (sum, mean, sqrtn; with and without
@@ -642,7 +812,7 @@ def test_pooled_extraction_matches_a_float64_segment_sum(kind, dim, etype, rows_
         if kind == "flat":
             mem, tb = _make_flat(nkeys)
         else:
-            mem, tb, _ = _make_hash(len(cached))
+            mem, tb, _ = (_make_hash32 if kind == "hash32" else _make_hash)(len(cached))
     slots = rng.permutation(len(cached)).astype(np.uint32)
     cache = np.zeros((max(len(cached), 1), rb), np.uint8)
     if len(cached):
@@ -778,7 +948,7 @@ def test_pooled_extraction_hand_worked(rows_per_group, monkeypatch):
         pin.free()
 
 
-@pytest.mark.parametrize("kind", ["none", "flat", "hash"])
+@pytest.mark.parametrize("kind", ["none", "flat", "hash", "hash32"])
 @pytest.mark.parametrize("dim,etype", [(4, np.float32), (32, np.float32), (100, np.float32), (128, np.float32),
                                        (512, np.float32), (1024, np.float32), (64, np.float16), (2048, np.float16),
                                        (64, "bf16")])
@@ -808,7 +978,7 @@ def test_pooled_extraction_with_max_norm_matches_the_oracle(kind, dim, etype):
         tb, cached, mem = hip.table(0, None, 0), np.zeros(0, np.int64), None
     else:
         cached = rng.choice(nkeys, nkeys // 2, replace=False).astype(np.int64)
-        mem, tb = _make_flat(nkeys) if kind == "flat" else _make_hash(len(cached))[:2]
+        mem, tb = _make_flat(nkeys) if kind == "flat" else (_make_hash32 if kind == "hash32" else _make_hash)(len(cached))[:2]
     slots = rng.permutation(len(cached)).astype(np.uint32)
     cache = np.zeros((max(len(cached), 1), rb), np.uint8)
     if len(cached):
@@ -894,7 +1064,7 @@ def _fmix64(x):
     return x
 
 
-@pytest.mark.parametrize("kind", ["flat", "hash"])
+@pytest.mark.parametrize("kind", ["flat", "hash", "hash32"])
 @pytest.mark.parametrize("rb", [64, 128, 512])
 def test_rows_from_the_host_are_filed_in_the_stage_and_found_there(kind, rb):
     """ugk_extract_mix_staged_*: same output and group sizes as the plain extraction; afterwards every owner word with a
@@ -911,7 +1081,7 @@ def test_rows_from_the_host_are_filed_in_the_stage_and_found_there(kind, rb):
     if kind == "flat":
         mem, tb = _make_flat(nkeys)
     else:
-        mem, tb, _ = _make_hash(len(cached))
+        mem, tb, _ = (_make_hash32 if kind == "hash32" else _make_hash)(len(cached))
     assert _insert(tb, cached, slots) == 0
     is_cached = np.zeros(nkeys, bool)
     is_cached[cached] = True
@@ -1181,7 +1351,7 @@ def test_dedup_of_small_and_large_batches_sharing_one_workspace(kdtype):
                  ptr(dev_zeros_u32(n)), None, ptr(dev_zeros_u32(1)), None, None)
 
 
-@pytest.mark.parametrize("mode", ["flat", "hash"])
+@pytest.mark.parametrize("mode", ["flat", "hash", "hash32"])
 @pytest.mark.parametrize("kdtype", [np.uint32, np.int64])
 @pytest.mark.parametrize("n", [1, 63, 64, 65, 4097, 200_000])
 def test_nonlocal_flags_and_stable_selection(mode, kdtype, n):
@@ -1196,7 +1366,7 @@ def test_nonlocal_flags_and_stable_selection(mode, kdtype, n):
     if mode == "flat":
         mem, tb = _make_flat(nkeys)
     else:
-        mem, tb, _ = _make_hash(20_000)
+        mem, tb, _ = (_make_hash32 if mode == "hash32" else _make_hash)(20_000)
     assert _insert(tb, local) == 0
     assert _insert(tb, on_host, offs_np=on_host.astype(np.uint32), loc=1) == 0
     keys = rng.integers(0, nkeys, size=n).astype(kdtype)

@@ -147,7 +147,7 @@ def test_config5_sparse_ids_hash_table_full_size(refresh_on, monkeypatch):
         words[r0 : r0 + len(r)].copy_(((r.unsqueeze(1) * words_per_row + col) & 0xffffffff).to(torch.int32))
     co.coll_torch_init_t(0, 0, emb, pct)
     info = _basics.info(0)
-    assert info["table_kind"] == 2 and info["row_bytes"] == 128 and info["key_space"] == n_item
+    assert info["table_kind"] == 3 and info["row_bytes"] == 128 and info["key_space"] == n_item
     assert info["cached_rows"] == num_cached
     assert info["capacity_rows"] == ORC.lib.orc_cache_capacity(n_item, pct)
     cached, n_obs = top_rows(pre, n_item, num_cached)

@@ -27,7 +27,7 @@ def _run(exe, table, refresh, steps):
     env = dict(os.environ)
     env["COLL_HASH_REBUILD_FRAC"] = "0.02"  # a few hundred evictions already rebuild the open-addressing table
     env["COLL_MISS_STAGE_ROWS"] = "4096"  # lookups file the rows they fetch from the host, foreground refreshes read them
-    if table == "HASH":  # refreshes on the device keep cached rows that tie (the second placement path)
+    if table.startswith("HASH"):  # refreshes on the device keep cached rows that tie (the second placement path)
         env["COLL_GPU_REFRESH_STABLE"] = "1"
     else:  # the device-side counters start from the build's ranking, and the background copy is paced by a rate
         env["COLL_GPU_RECORD_SEED"] = "1"
@@ -43,18 +43,18 @@ def _run(exe, table, refresh, steps):
 
 
 @pytest.mark.parametrize("refresh", ["host", "device"])
-@pytest.mark.parametrize("table", ["FLAT", "HASH"])
+@pytest.mark.parametrize("table", ["FLAT", "HASH", "HASH16"])
 def test_host_library_under_asan_and_ubsan(drivers, table, refresh):
     rc, out = _run(drivers["asan"], table, refresh, 150)
     assert "AddressSanitizer" not in out and "runtime error" not in out and "LeakSanitizer" not in out, out[-6000:]
     assert rc == 0 and out.rstrip().endswith("OK"), out[-3000:]
-    if table == "HASH":  # the table swap of a rebuild ran beside the lookups
+    if table.startswith("HASH"):  # the table swap of a rebuild ran beside the lookups
         rebuilds = [int(l.split(" table rebuilds")[0].split()[-1]) for l in out.splitlines() if " table rebuilds" in l]
         assert rebuilds and max(rebuilds) > 0, out[-3000:]
 
 
 @pytest.mark.parametrize("refresh", ["host", "device"])
-@pytest.mark.parametrize("table", ["FLAT", "HASH"])
+@pytest.mark.parametrize("table", ["FLAT", "HASH", "HASH16"])
 def test_host_library_under_tsan(drivers, table, refresh):
     rc, out = _run(drivers["tsan"], table, refresh, 30)
     assert "ThreadSanitizer" not in out, out[-8000:]

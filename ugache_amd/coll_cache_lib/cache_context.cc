@@ -121,7 +121,7 @@ void CacheContext::build_with_advise_new_hash(int location_id, std::shared_ptr<C
   bool use_flat = TableSize(std::max<size_t>(num_cached_nodes, 2)) > num_total_nodes / 2 ||
                   num_total_nodes * sizeof(IdType) <= ((size_t)256 << 20);
   if (RunConfig::force_table_kind == 1) use_flat = true;
-  if (RunConfig::force_table_kind == 2) use_flat = false;
+  if (RunConfig::force_table_kind >= 2) use_flat = false;
   if (RunConfig::key_map_mul != 0) {
     CHECK(RunConfig::force_table_kind != 1) << "sparse ids cannot index a flat table";
     use_flat = false;
@@ -136,7 +136,8 @@ void CacheContext::build_with_advise_new_hash(int location_id, std::shared_ptr<C
   if (use_flat) {
     _new_hash_table->CreateFlat(_eager_gpu_mem_allocator, num_total_nodes, stream);
   } else {
-    _new_hash_table->CreateHash(_eager_gpu_mem_allocator, std::max<size_t>(_cache_space_capacity, 1), stream);
+    _new_hash_table->CreateHash(_eager_gpu_mem_allocator, std::max<size_t>(_cache_space_capacity, 1), num_total_nodes,
+                                stream);
   }
 
   const double alloc_s = t.Passed() - detect_s;

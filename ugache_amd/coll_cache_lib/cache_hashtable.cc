@@ -27,16 +27,36 @@ void CacheEntryManager::CreateFlat(const std::function<MemHandle(size_t)> &alloc
   RunConfig::use_flat_hashtable = true;
 }
 
+namespace {
+size_t HashEntryBytes(int kind) { return kind == 3 ? sizeof(uint64_t) : sizeof(ugk_bucket_t); }
+size_t HashEntriesFor(int kind, size_t num_entries) {
+  return kind == 3 ? ugk_hash32_entries_for(num_entries, RunConfig::hash_load_factor)
+                   : ugk_hash_buckets_for(num_entries, RunConfig::hash_load_factor);
+}
+}  // namespace
+
+bool CacheEntryManager::CompactHashFits(size_t num_slots, size_t num_host_rows) {
+  // an 8-byte entry names its key by the host row (below 0xfffffffe: the two values above mark never-used and evicted
+  // entries) and packs the slot into 28 bits beside the 4-bit location
+  return num_host_rows <= 0xfffffffeull && num_slots <= ((size_t)1 << 28);
+}
+
 void CacheEntryManager::CreateHash(const std::function<MemHandle(size_t)> &allocator, size_t num_entries,
-                                   StreamHandle stream) {
-  const size_t nb = ugk_hash_buckets_for(num_entries, RunConfig::hash_load_factor);
-  LOG(INFO) << "open-addressing lookup table for " << num_entries << " entries: " << nb << " buckets, "
-            << ToReadableSize(nb * sizeof(ugk_bucket_t));
-  _table_handle = allocator(nb * sizeof(ugk_bucket_t) + 128);
+                                   size_t num_host_rows, StreamHandle stream) {
+  int kind = CompactHashFits(num_entries, num_host_rows) ? 3 : 2;
+  if (RunConfig::force_table_kind == 16) kind = 2;
+  if (RunConfig::force_table_kind == 8) {
+    CHECK(kind == 3) << "COLL_HASH_TABLE=HASH8: 8-byte entries hold rows below 0xfffffffe and 2^28 slots; this cache has "
+                     << num_host_rows << " rows and " << num_entries << " slots";
+  }
+  const size_t ne = HashEntriesFor(kind, num_entries);
+  LOG(INFO) << "open-addressing lookup table for " << num_entries << " entries: " << ne << " entries of "
+            << HashEntryBytes(kind) << " bytes, " << ToReadableSize(ne * HashEntryBytes(kind));
+  _table_handle = allocator(ne * HashEntryBytes(kind) + 128);
   CHECK_NOTNULL(_table_handle);
   void *base = Align128(_table_handle->ptr());
-  _table = {2, 0, base, nb, RunConfig::key_map_inv, RunConfig::key_map_mask};
-  UGK_CALL(ugk_hash_init(static_cast<ugk_bucket_t *>(base), nb, stream));
+  _table = {kind, 0, base, ne, RunConfig::key_map_inv, RunConfig::key_map_mask};
+  UGK_CALL(ugk_table_init(_table, stream));
   RunConfig::use_flat_hashtable = false;
 }
 
@@ -88,7 +108,7 @@ void CacheEntryManager::Evict(TensorPtr keys_to_evict, StreamHandle stream) {
   else
     UGK_CALL(ugk_table_evict_u32(_table, keys_to_evict->CPtr<uint32_t>(), keys_to_evict->NumItem(),
                                  StatusPtr(this, stream), stream));
-  if (_table.kind == 2) _num_tombstones += keys_to_evict->NumItem();
+  if (_table.kind >= 2) _num_tombstones += keys_to_evict->NumItem();
 }
 
 void CacheEntryManager::EvictRelease(TensorPtr keys_to_evict, StreamHandle stream) {
@@ -98,18 +118,18 @@ void CacheEntryManager::EvictRelease(TensorPtr keys_to_evict, StreamHandle strea
   else
     UGK_CALL(ugk_table_evict_release_u32(_table, keys_to_evict->CPtr<uint32_t>(), keys_to_evict->NumItem(),
                                          SlotUsedBits(), _cache_space_capacity, StatusPtr(this, stream), stream));
-  if (_table.kind == 2) _num_tombstones += keys_to_evict->NumItem();
+  if (_table.kind >= 2) _num_tombstones += keys_to_evict->NumItem();
 }
 
 bool CacheEntryManager::MaybeRebuild(const std::function<MemHandle(size_t)> &allocator, Context ctx, int loc,
                                      StreamHandle stream, const std::function<void()> &wait_for_lookups) {
-  if (_table.kind != 2) return false;
+  if (_table.kind < 2) return false;
   const double limit = RunConfig::hash_rebuild_tombstone_frac * (double)_table.size;
   if ((double)_num_tombstones <= limit) return false;
   // _num_tombstones counts evictions; inserts reuse tombstones they pass, so look before rebuilding
   uint64_t *census_dev = reinterpret_cast<uint64_t *>(StatusPtr(this, stream) + 16);
   uint64_t census[3] = {0, 0, 0};
-  UGK_CALL(ugk_hash_census(static_cast<const ugk_bucket_t *>(_table.table), _table.size, census_dev, stream));
+  UGK_CALL(ugk_table_census(_table, census_dev, stream));
   UGK_CALL(ugk_memcpy_async(census, census_dev, sizeof(census), stream));
   UGK_CALL(ugk_stream_sync(stream));
   _num_tombstones = census[1];
@@ -124,16 +144,16 @@ bool CacheEntryManager::MaybeRebuild(const std::function<MemHandle(size_t)> &all
     n = _cached_keys->NumItem();
     keys = TableKeysToDevice(_cached_keys, allocator, ctx, stream);
   }
-  LOG(INFO) << "rebuilding the lookup table: " << _num_tombstones << " tombstones in " << _table.size << " buckets, "
+  LOG(INFO) << "rebuilding the lookup table: " << _num_tombstones << " tombstones in " << _table.size << " entries, "
             << n << " live keys";
   offs = Tensor::EmptyExternal(kI32, {n}, allocator, ctx, "");
   if (n > 0) LookupOffset(keys, offs, stream);
   // the keys go into a second table; the one in use keeps serving lookups until the swap
-  MemHandle fresh_handle = allocator(_table.size * sizeof(ugk_bucket_t) + 128);
+  MemHandle fresh_handle = allocator(_table.size * HashEntryBytes(_table.kind) + 128);
   CHECK_NOTNULL(fresh_handle);
   ugk_table_t fresh = _table;
   fresh.table = Align128(fresh_handle->ptr());
-  UGK_CALL(ugk_hash_init(static_cast<ugk_bucket_t *>(fresh.table), fresh.size, stream));
+  UGK_CALL(ugk_table_init(fresh, stream));
   if (n > 0) {
     if (keys->Type() == kI64)
       UGK_CALL(ugk_table_insert_i64(fresh, keys->CPtr<int64_t>(), offs->CPtr<uint32_t>(), 0, (uint32_t)loc, n,

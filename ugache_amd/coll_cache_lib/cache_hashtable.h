@@ -57,7 +57,11 @@ class CacheEntryManager {
 
   // allocate and clear the table (FlatHashTable / SimpleHashTable ctors, cache_hashtable.cu:432-457, 588-607)
   void CreateFlat(const std::function<MemHandle(size_t)> &allocator, size_t num_keys, StreamHandle stream);
-  void CreateHash(const std::function<MemHandle(size_t)> &allocator, size_t num_entries, StreamHandle stream);
+  // 8-byte entries keyed by the host row when `num_entries` slots and `num_host_rows` rows fit them, else 16-byte
+  // buckets keyed by the id (COLL_HASH_TABLE=HASH16 / HASH8 force one)
+  void CreateHash(const std::function<MemHandle(size_t)> &allocator, size_t num_entries, size_t num_host_rows,
+                  StreamHandle stream);
+  static bool CompactHashFits(size_t num_slots, size_t num_host_rows);
 
   // Device copy of a host list of row numbers in the form the table is keyed by: the uint32 row numbers
   // themselves, or — in sparse-id mode — the int64 caller-side ids of those rows.

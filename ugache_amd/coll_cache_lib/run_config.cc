@@ -118,7 +118,9 @@ void RunConfig::LoadConfigFromEnv() {
   const std::string tbl = GetEnv("COLL_HASH_TABLE");
   if (tbl == "FLAT") force_table_kind = 1;
   else if (tbl == "HASH") force_table_kind = 2;
-  else if (tbl != "") LOG(FATAL) << "COLL_HASH_TABLE must be FLAT or HASH, got " << tbl;
+  else if (tbl == "HASH16") force_table_kind = 16;
+  else if (tbl == "HASH8") force_table_kind = 8;
+  else if (tbl != "") LOG(FATAL) << "COLL_HASH_TABLE must be FLAT, HASH, HASH16 or HASH8, got " << tbl;
   if (GetEnv("COLL_REFRESH_THREADS") != "") refresher_omp_thread_num = std::max(1, std::stoi(GetEnv("COLL_REFRESH_THREADS")));
   if (GetEnv("COLL_REFRESH_BATCH_ROWS") != "") refresh_batch_rows = std::stoul(GetEnv("COLL_REFRESH_BATCH_ROWS"));
   if (GetEnv("COLL_REFRESH_SLEEP_US") != "") refresh_sleep_us = std::stoul(GetEnv("COLL_REFRESH_SLEEP_US"));

@@ -59,7 +59,8 @@ struct RunConfig {
   static coll_cache::AsymmLinkDesc coll_cache_link_desc;
   // knobs of this implementation
   static double hash_load_factor;      // COLL_HASH_LOAD_FACTOR, default 0.7
-  static int force_table_kind;         // COLL_HASH_TABLE=FLAT|HASH -> 1|2, 0 = decide by size
+  static int force_table_kind;         // COLL_HASH_TABLE=FLAT|HASH|HASH16|HASH8 -> 1|2|16|8, 0 = decide by size;
+                                       // HASH picks the entry width itself, HASH16 / HASH8 name it (bytes)
   static size_t refresh_batch_rows;    // COLL_REFRESH_BATCH_ROWS, default 4092 (cache_context.cu:4057)
   static unsigned refresh_sleep_us;    // COLL_REFRESH_SLEEP_US, default 3000 (cache_context.cu:4069)
   static unsigned refresh_limit_block; // COLL_REFRESH_LIMIT_BLOCK, default 20 (cache_context.cu:4068)

@@ -430,11 +430,11 @@ int classify(ugk_table_t t, const K *keys, size_t n, uint64_t host_rows, const u
   UGK_REQUIRE(counts && status, "ugk_classify: null counters or status");
   UGK_REQUIRE(n <= 0xffffffffull, "ugk_classify: batch of %zu keys exceeds 2^32", n);
   UGK_REQUIRE((uintptr_t)counts % 8 == 0, "ugk_classify: the two counters must share an 8-byte aligned word");
-  UGK_REQUIRE(t.kind == 1 || t.kind == 2, "ugk_classify: table kind %d is not flat(1) or hash(2)", t.kind);
+  UGK_REQUIRE(t.kind >= 1 && t.kind <= 3, "ugk_classify: table kind %d is not flat(1), hash(2) or compact hash(3)", t.kind);
   UGK_REQUIRE(t.table && t.size, "ugk_classify: empty table");
-  if (t.kind == 2)
-    UGK_REQUIRE(t.size % 8 == 0 && (uintptr_t)t.table % 128 == 0,
-                "ugk_classify: hash table must be 128-byte aligned with a multiple of 8 buckets");
+  if (t.kind >= 2)
+    UGK_REQUIRE(t.size % (t.kind == 2 ? 8 : 16) == 0 && (uintptr_t)t.table % 128 == 0,
+                "ugk_classify: hash table must be 128-byte aligned with whole 128-byte lines of buckets");
   UGK_REQUIRE(n == 0 || (keys && idx), "ugk_classify: null keys or index list");
   // n == 0 still launches one block so that next_counts is cleared
   const int items = items_for(n);
@@ -445,8 +445,10 @@ int classify(ugk_table_t t, const K *keys, size_t n, uint64_t host_rows, const u
                      n, host_rows, dst_map, idx, counts, next_counts, status, host_mirror)
   if (t.kind == 1 && items == 1) UGK_GO(1, 1);
   else if (t.kind == 1) UGK_GO(1, kItems);
-  else if (items == 1) UGK_GO(2, 1);
-  else UGK_GO(2, kItems);
+  else if (t.kind == 2 && items == 1) UGK_GO(2, 1);
+  else if (t.kind == 2) UGK_GO(2, kItems);
+  else if (items == 1) UGK_GO(3, 1);
+  else UGK_GO(3, kItems);
 #undef UGK_GO
   UGK_HIP(hipGetLastError());
   return 0;
@@ -457,17 +459,20 @@ int nonlocal_flags(ugk_table_t t, const K *keys, size_t n, uint64_t *flags, void
   if (n == 0) return 0;
   UGK_REQUIRE(keys && flags, "ugk_nonlocal_flags: null keys or bitmap");
   UGK_REQUIRE((uintptr_t)flags % 8 == 0, "ugk_nonlocal_flags: the bitmap must be 8-byte aligned");
-  UGK_REQUIRE(t.kind == 1 || t.kind == 2, "ugk_nonlocal_flags: table kind %d is not flat(1) or hash(2)", t.kind);
+  UGK_REQUIRE(t.kind >= 1 && t.kind <= 3, "ugk_nonlocal_flags: table kind %d is not flat(1), hash(2) or compact hash(3)", t.kind);
   UGK_REQUIRE(t.table && t.size, "ugk_nonlocal_flags: empty table");
-  if (t.kind == 2)
-    UGK_REQUIRE(t.size % 8 == 0 && (uintptr_t)t.table % 128 == 0,
-                "ugk_nonlocal_flags: hash table must be 128-byte aligned with a multiple of 8 buckets");
+  if (t.kind >= 2)
+    UGK_REQUIRE(t.size % (t.kind == 2 ? 8 : 16) == 0 && (uintptr_t)t.table % 128 == 0,
+                "ugk_nonlocal_flags: hash table must be 128-byte aligned with whole 128-byte lines of buckets");
   const unsigned grid = clamp_grid((n + kBlock - 1) / kBlock, 0);
   if (t.kind == 1)
     hipLaunchKernelGGL((nonlocal_flags_kernel<K, 1>), dim3(grid), dim3(kBlock), 0, as_stream(stream), t, keys, n,
                        reinterpret_cast<unsigned long long *>(flags));
-  else
+  else if (t.kind == 2)
     hipLaunchKernelGGL((nonlocal_flags_kernel<K, 2>), dim3(grid), dim3(kBlock), 0, as_stream(stream), t, keys, n,
+                       reinterpret_cast<unsigned long long *>(flags));
+  else
+    hipLaunchKernelGGL((nonlocal_flags_kernel<K, 3>), dim3(grid), dim3(kBlock), 0, as_stream(stream), t, keys, n,
                        reinterpret_cast<unsigned long long *>(flags));
   UGK_HIP(hipGetLastError());
   return 0;
@@ -597,11 +602,11 @@ int extract_mix(ugk_table_t t, const K *keys, size_t n, const void *cache, uint6
   UGK_REQUIRE(keys && out && status, "ugk_extract_mix: null keys, output or status");
   UGK_REQUIRE((uintptr_t)counts % 8 == 0, "ugk_extract_mix: the count words must be 8-byte aligned");
   UGK_REQUIRE(n <= 0xffffffffull, "ugk_extract_mix: batch of %zu keys exceeds 2^32", n);
-  UGK_REQUIRE(t.kind == 1 || t.kind == 2, "ugk_extract_mix: table kind %d is not flat(1) or hash(2)", t.kind);
+  UGK_REQUIRE(t.kind >= 1 && t.kind <= 3, "ugk_extract_mix: table kind %d is not flat(1), hash(2) or compact hash(3)", t.kind);
   UGK_REQUIRE(t.table && t.size, "ugk_extract_mix: empty table");
-  if (t.kind == 2)
-    UGK_REQUIRE(t.size % 8 == 0 && (uintptr_t)t.table % 128 == 0,
-                "ugk_extract_mix: hash table must be 128-byte aligned with a multiple of 8 buckets");
+  if (t.kind >= 2)
+    UGK_REQUIRE(t.size % (t.kind == 2 ? 8 : 16) == 0 && (uintptr_t)t.table % 128 == 0,
+                "ugk_extract_mix: hash table must be 128-byte aligned with whole 128-byte lines of buckets");
   UGK_REQUIRE(cache_rows == 0 || cache, "ugk_extract_mix: null cache with %llu rows", (unsigned long long)cache_rows);
   UGK_REQUIRE(host_rows == 0 || host, "ugk_extract_mix: null host table with %llu rows",
               (unsigned long long)host_rows);
@@ -619,7 +624,10 @@ int extract_mix(ugk_table_t t, const K *keys, size_t n, const void *cache, uint6
   if (t.kind == 1)
     return extract_mix_lpr<K, 1>(t, keys, n, cache, cache_rows, host, host_rows, out, vpr, status, host_mirror,
                                  counts, num_groups, others_hint, stage, as_stream(stream));
-  return extract_mix_lpr<K, 2>(t, keys, n, cache, cache_rows, host, host_rows, out, vpr, status, host_mirror,
+  if (t.kind == 2)
+    return extract_mix_lpr<K, 2>(t, keys, n, cache, cache_rows, host, host_rows, out, vpr, status, host_mirror,
+                                 counts, num_groups, others_hint, stage, as_stream(stream));
+  return extract_mix_lpr<K, 3>(t, keys, n, cache, cache_rows, host, host_rows, out, vpr, status, host_mirror,
                                counts, num_groups, others_hint, stage, as_stream(stream));
 }
 

@@ -499,11 +499,11 @@ int extract_pool(ugk_table_t t, const K *ids, const int64_t *seg_off, const floa
   UGK_REQUIRE(elem_bytes == 4 || elem_bytes == 2 || elem_bytes == UGK_ELEM_BF16,
               "ugk_extract_pool: element code %d is not fp32 (4), fp16 (2) or bfloat16 (UGK_ELEM_BF16)", elem_bytes);
   const bool bf16 = elem_bytes == UGK_ELEM_BF16;
-  UGK_REQUIRE(t.kind == 0 || t.kind == 1 || t.kind == 2, "ugk_extract_pool: table kind %d", t.kind);
+  UGK_REQUIRE(t.kind >= 0 && t.kind <= 3, "ugk_extract_pool: table kind %d", t.kind);
   if (t.kind != 0) UGK_REQUIRE(t.table && t.size, "ugk_extract_pool: empty table");
-  if (t.kind == 2)
-    UGK_REQUIRE(t.size % 8 == 0 && (uintptr_t)t.table % 128 == 0,
-                "ugk_extract_pool: hash table must be 128-byte aligned with a multiple of 8 buckets");
+  if (t.kind >= 2)
+    UGK_REQUIRE(t.size % (t.kind == 2 ? 8 : 16) == 0 && (uintptr_t)t.table % 128 == 0,
+                "ugk_extract_pool: hash table must be 128-byte aligned with whole 128-byte lines of buckets");
   UGK_REQUIRE(cache_rows == 0 || cache, "ugk_extract_pool: null cache with %llu rows", (unsigned long long)cache_rows);
   UGK_REQUIRE(host_rows == 0 || host, "ugk_extract_pool: null host table with %llu rows", (unsigned long long)host_rows);
   const uintptr_t align = (uintptr_t)cache | (uintptr_t)host | (uintptr_t)out | (uintptr_t)row_bytes;
@@ -523,7 +523,8 @@ int extract_pool(ugk_table_t t, const K *ids, const int64_t *seg_off, const floa
                                                        host_mirror, counts, num_groups, st))
   if (t.kind == 0) return UGK_POOL_KIND(0);
   if (t.kind == 1) return UGK_POOL_KIND(1);
-  return UGK_POOL_KIND(2);
+  if (t.kind == 2) return UGK_POOL_KIND(2);
+  return UGK_POOL_KIND(3);
 #undef UGK_POOL_KIND
 }
 

@@ -10,6 +10,15 @@
 //               insert or an evict therefore reads as a miss, which is always correct because the host
 //               table holds every row.
 //
+// compact hash table (kind 3): uint64[nentries] (nentries a multiple of 16, base 128-byte aligned), one word per entry:
+//               low half = the ROW of the host table the key stands for (the key itself for dense ids, the inverse of
+//               the sparse-id map otherwise: a bijection, so the 32-bit row identifies the key exactly), high half =
+//               (loc << 28) + off as in the flat table.  Sixteen entries fill a 128-byte line, so at load 0.7 about
+//               one key in a hundred is not settled by its home line (one in thirteen with the 16-byte buckets), and
+//               the second, dependent round of a lookup all but disappears.  An entry appears and disappears whole
+//               (one 8-byte word), so there is no "present, not yet valid" state.  0xffffffff_ffffffff = never used,
+//               key half 0xfffffffe = tombstone; rows from 0xfffffffe on cannot be stored.
+//
 // Lookup is wavefront-cooperative: an 8-lane group reads one 128-byte line (eight adjacent buckets) of one key's
 // probe sequence per step and a wavefront ballot decides match / never-used / continue.  Step 1 reads the
 // home line of all 64 keys of the wavefront in eight rounds whose loads are independent of each other (all in
@@ -68,6 +77,14 @@ __device__ __forceinline__ Found flat_lookup(const uint32_t *table, uint64_t nke
   }
   return f;
 }
+
+// host row of a key that is not in the table
+__device__ __forceinline__ uint64_t fallback_row(const ugk_table_t &t, uint64_t key) {
+  if (t.fb_mul == 0) return key;
+  return key <= t.fb_mask ? ((key * t.fb_mul) & t.fb_mask) : ~0ull;  // ids beyond the id space have no row
+}
+// the row a compact table (kind 3) stores a key under
+__device__ __forceinline__ uint64_t h32_row(const ugk_table_t &t, uint64_t key) { return fallback_row(t, key); }
 
 // Wavefront-cooperative hash lookup in two steps.  All 64 lanes of the wavefront must call both (inactive lanes pass
 // active = false).
@@ -213,6 +230,142 @@ __device__ __forceinline__ Found hash_probe_rest(const ugk_bucket_t *table, uint
   return f;
 }
 
+// ---- the compact table (kind 3) -----------------------------------------------------------------------------------
+constexpr uint32_t kH32Empty = 0xffffffffu, kH32Tomb = 0xfffffffeu;
+constexpr uint64_t kH32EmptyWord = ~0ull, kH32TombWord = 0x00000000fffffffeull;
+
+__device__ __forceinline__ uint64_t h32_home(uint64_t row, uint64_t nentries) {
+  return __umul64hi(fmix64(row), nentries >> 4) << 4;
+}
+
+// bit i of `even` to bit 2i, bit i of `odd` to bit 2i + 1: the sixteen entries of a line in their order, from the two
+// per-lane predicates of an 8-lane group
+__device__ __forceinline__ uint32_t h32_interleave(uint32_t even, uint32_t odd) {
+  auto spread = [](uint32_t b) {
+    b = (b | (b << 4)) & 0x0f0fu;
+    b = (b | (b << 2)) & 0x3333u;
+    return (b | (b << 1)) & 0x5555u;
+  };
+  return spread(even & 0xffu) | (spread(odd & 0xffu) << 1);
+}
+
+struct H32Line {
+  bool found, done;
+  uint32_t val;  // group-uniform
+};
+
+// what one 128-byte line says about `row`: every lane of the 8-lane group passes the 16 bytes it read (entries
+// 2 * sub and 2 * sub + 1); act is group-uniform.  All 64 lanes call it.
+__device__ __forceinline__ H32Line h32_examine(const u32x4 &raw, uint32_t row, bool act, int grp) {
+  const uint32_t m = h32_interleave((uint32_t)(__ballot(act && raw.x == row) >> (grp * 8)),
+                                    (uint32_t)(__ballot(act && raw.z == row) >> (grp * 8)));
+  const uint32_t e = h32_interleave((uint32_t)(__ballot(act && raw.x == kH32Empty) >> (grp * 8)),
+                                    (uint32_t)(__ballot(act && raw.z == kH32Empty) >> (grp * 8)));
+  const int fm = m ? (__ffs(m) - 1) : 16;
+  const int fe = e ? (__ffs(e) - 1) : 16;
+  H32Line r;
+  r.found = fm < fe;  // a key sits in front of the first never-used entry of its probe sequence
+  r.done = r.found || fe < 16;
+  const int hit_lane = grp * 8 + (r.found ? (fm >> 1) : 0);
+  const uint32_t vy = __shfl(raw.y, hit_lane), vw = __shfl(raw.w, hit_lane);
+  r.val = (fm & 1) ? vw : vy;
+  return r;
+}
+
+template <int PASSES, int ROUNDS = 8>
+__device__ __forceinline__ HashProbe h32_probe_home(const uint64_t *table, uint64_t n, uint64_t row, bool active) {
+  static_assert(ROUNDS >= 1 && ROUNDS <= 8 && ROUNDS % PASSES == 0, "whole passes of rounds");
+  constexpr int PER = ROUNDS / PASSES;
+  HashProbe p{Found{false, 0, 0}, 0, false};
+  const int lane = (int)lane_id();
+  const int grp = lane >> 3, sub = lane & 7;
+  const uint64_t home = active ? h32_home(row, n) : 0;
+#pragma unroll
+  for (int pass = 0; pass < PASSES; ++pass) {
+    u32x4 raw[PER];
+    uint32_t kk[PER];
+    bool act[PER];
+#pragma unroll
+    for (int q = 0; q < PER; ++q) {
+      const int owner = (pass * PER + q) * 8 + grp;
+      kk[q] = __shfl((uint32_t)row, owner);
+      const uint64_t hb = shfl64(home, owner);
+      act[q] = __shfl((int)active, owner) != 0;
+      raw[q] = u32x4{kH32Empty, kH32Empty, kH32Empty, kH32Empty};  // reads as never-used entries
+      if (act[q]) raw[q] = reinterpret_cast<const u32x4 *>(table + hb)[sub];
+    }
+#pragma unroll
+    for (int q = 0; q < PER; ++q) {
+      const int r = pass * PER + q;
+      const H32Line line = h32_examine(raw[q], kk[q], act[q], grp);
+      const uint32_t g_flags = (line.done ? 1u : 0u) | (line.found ? 2u : 0u);
+      const int from = (lane & 7) * 8;  // the owner of this round's key served by group g is lane 8r + g
+      const uint32_t r_flags = __shfl(g_flags, from);
+      const uint32_t r_val = __shfl(line.val, from);
+      if ((lane >> 3) == r && active) {
+        if (r_flags & 1u) {
+          if (r_flags & 2u) {
+            p.f.hit = true;
+            p.f.loc = (r_val >> 28) & 0xfu;
+            p.f.off = r_val & 0x0fffffffu;
+          }
+        } else {
+          p.pending = true;
+        }
+      }
+    }
+  }
+  p.next_win = home + 16 >= n ? 0 : home + 16;
+  return p;
+}
+
+__device__ __forceinline__ Found h32_probe_rest(const uint64_t *table, uint64_t n, uint64_t row, HashProbe p) {
+  Found f = p.f;
+  bool pending = p.pending;
+  uint64_t pend = __ballot(pending);
+  if (pend == 0) return f;
+  const int lane = (int)lane_id();
+  const int grp = lane >> 3, sub = lane & 7;
+  uint64_t win = p.next_win;
+  uint64_t steps = 0;
+  const uint64_t max_steps = n / 16 + 1;  // a full lap: give up (table without a never-used entry)
+  while (pend) {
+    // the g-th 8-lane group serves the g-th pending lane
+    const int rank = __popcll(pend & ((1ull << lane) - 1ull));
+    uint64_t m = pend;
+    for (int i = 0; i < grp; ++i) m &= m - 1;
+    const int src = m ? (__ffsll((unsigned long long)m) - 1) : -1;
+    const bool gactive = src >= 0;
+    const int from = gactive ? src : lane;
+    const uint32_t k = __shfl((uint32_t)row, from);
+    const uint64_t w = shfl64(win, from);
+    u32x4 raw{kH32Empty, kH32Empty, kH32Empty, kH32Empty};
+    if (gactive) raw = reinterpret_cast<const u32x4 *>(table + w)[sub];
+    const H32Line line = h32_examine(raw, k, gactive, grp);
+    const uint32_t g_flags = (line.done ? 1u : 0u) | (line.found ? 2u : 0u);
+    const bool served = pending && rank < 8;
+    const int back = served ? rank * 8 : lane;
+    const uint32_t r_flags = __shfl(g_flags, back);
+    const uint32_t r_val = __shfl(line.val, back);
+    if (served) {
+      if (r_flags & 1u) {
+        pending = false;
+        if (r_flags & 2u) {
+          f.hit = true;
+          f.loc = (r_val >> 28) & 0xfu;
+          f.off = r_val & 0x0fffffffu;
+        }
+      } else {
+        win += 16;
+        if (win >= n) win = 0;
+        if (++steps > max_steps) pending = false;
+      }
+    }
+    pend = __ballot(pending);
+  }
+  return f;
+}
+
 template <int PASSES = 2, int ROUNDS = 8>
 __device__ __forceinline__ Found hash_lookup_wave(const ugk_bucket_t *table, uint64_t nb, uint64_t key, bool active) {
   return hash_probe_rest(table, nb, key, hash_probe_home<PASSES, ROUNDS>(table, nb, key, active));
@@ -225,6 +378,13 @@ __device__ __forceinline__ Found table_lookup(const ugk_table_t &t, uint64_t key
   if (KIND == 1) return flat_lookup(reinterpret_cast<const uint32_t *>(t.table), t.size, key, active);
   if (KIND == 2)
     return hash_lookup_wave<PASSES, ROUNDS>(reinterpret_cast<const ugk_bucket_t *>(t.table), t.size, key, active);
+  if (KIND == 3) {
+    // keyed by the row the key stands for; a key without a storable row is in no table
+    const uint64_t row = active ? h32_row(t, key) : 0;
+    const bool probe = active && row < kH32Tomb;
+    const uint64_t *table = reinterpret_cast<const uint64_t *>(t.table);
+    return h32_probe_rest(table, t.size, row, h32_probe_home<PASSES, ROUNDS>(table, t.size, row, probe));
+  }
   return Found{false, 0, 0};
 }
 
@@ -239,11 +399,6 @@ __device__ __forceinline__ uint64_t key_to_u64<int64_t>(int64_t k) {
   return (uint64_t)k;
 }
 
-// host row of a key that is not in the table
-__device__ __forceinline__ uint64_t fallback_row(const ugk_table_t &t, uint64_t key) {
-  if (t.fb_mul == 0) return key;
-  return key <= t.fb_mask ? ((key * t.fb_mul) & t.fb_mask) : ~0ull;  // ids beyond the id space have no row
-}
 
 // keys that collide with the two reserved bucket states cannot live in the hash table
 __device__ __forceinline__ bool key_is_reserved(uint64_t k) { return k >= UGK_HASH_TOMB; }

@@ -187,6 +187,148 @@ __global__ __launch_bounds__(kBlock) void hash_evict_kernel(ugk_bucket_t *table,
   }
 }
 
+// ---- the compact table (kind 3): one 8-byte word per entry, sixteen to a line ------------------------------------
+__global__ __launch_bounds__(kBlock) void h32_init_kernel(unsigned long long *table, size_t n) {
+  for (size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x; i < n; i += (size_t)gridDim.x * kBlock)
+    table[i] = kH32EmptyWord;
+}
+
+// Insert, eight keys per wavefront, as hash_insert_kernel: an 8-lane group walks one key's probe sequence a line
+// (sixteen entries, two per lane) at a time up to the first never-used entry, so that a tombstone in front of a live
+// copy of the key cannot hide it, and claims the first reusable entry with one compare-and-swap on the whole word:
+// row and value appear together.
+template <typename K>
+__global__ __launch_bounds__(kBlock) void h32_insert_kernel(ugk_table_t t, const K *keys, const uint32_t *offs,
+                                                            uint32_t seq_base, uint32_t loc, size_t n,
+                                                            uint32_t *status) {
+  constexpr uint64_t kNone = ~0ull;
+  unsigned long long *table = reinterpret_cast<unsigned long long *>(t.table);
+  const uint64_t ne = t.size;
+  const int lane = (int)lane_id();
+  const int grp = lane >> 3, sub = lane & 7;
+  const size_t wave = ((size_t)blockIdx.x * kBlock + threadIdx.x) / kWave;
+  const size_t n_waves = (size_t)gridDim.x * (kBlock / kWave);
+  const uint64_t lines = ne >> 4;
+  for (size_t i0 = wave * 8; i0 < n; i0 += n_waves * 8) {  // wavefront-uniform: every ballot below sees all 64 lanes
+    const size_t i = i0 + grp;
+    const bool active = i < n;
+    const uint64_t row = active ? h32_row(t, key_to_u64<K>(keys[i])) : 0;
+    const uint32_t off = active ? (offs ? offs[i] : seq_base + (uint32_t)i) : 0;
+    bool done = !active;
+    if (active && (row >= kH32Tomb || off > 0x0fffffffu)) {
+      if (sub == 0) atomicOr(status, UGK_ST_KEY_OUT_OF_RANGE);
+      done = true;
+    }
+    const uint32_t r32 = (uint32_t)row;
+    const uint64_t home = done ? 0 : h32_home(row, ne);
+    uint64_t win = home, first_tomb = kNone, steps = 0;
+    while (__ballot(!done)) {
+      uint32_t k0 = 0, k1 = 0;  // read as some other key
+      if (!done) {
+        k0 = (uint32_t)__atomic_load_n(table + win + 2 * sub, __ATOMIC_RELAXED);
+        k1 = (uint32_t)__atomic_load_n(table + win + 2 * sub + 1, __ATOMIC_RELAXED);
+      }
+      const int sh = grp * 8;
+      const uint32_t mb = h32_interleave((uint32_t)(__ballot(!done && k0 == r32) >> sh),
+                                         (uint32_t)(__ballot(!done && k1 == r32) >> sh));
+      const uint32_t eb = h32_interleave((uint32_t)(__ballot(!done && k0 == kH32Empty) >> sh),
+                                         (uint32_t)(__ballot(!done && k1 == kH32Empty) >> sh));
+      const uint32_t tb = h32_interleave((uint32_t)(__ballot(!done && k0 == kH32Tomb) >> sh),
+                                         (uint32_t)(__ballot(!done && k1 == kH32Tomb) >> sh));
+      int action = 0;  // 0 walk on, 1 the key is there already, 2 claim `target`
+      uint64_t target = 0, expect = 0;
+      if (!done) {
+        const int fe = eb ? (__ffs(eb) - 1) : 16;
+        const uint32_t in_front = fe < 16 ? ((1u << fe) - 1u) : 0xffffu;  // entries in front of the first never-used one
+        if (mb & in_front) {
+          action = 1;
+        } else {
+          if (first_tomb == kNone && (tb & in_front)) first_tomb = win + (uint64_t)(__ffs(tb & in_front) - 1);
+          const bool lap_done = steps >= lines && first_tomb != kNone;  // no never-used entry at all: take the tombstone
+          if (fe < 16 || lap_done) {
+            action = 2;
+            target = first_tomb != kNone ? first_tomb : win + (uint64_t)fe;
+            expect = first_tomb != kNone ? kH32TombWord : kH32EmptyWord;
+          }
+        }
+      }
+      uint64_t seen = 0;
+      if (action == 2 && sub == 0)
+        seen = atomicCAS(table + target, (unsigned long long)expect,
+                         ((unsigned long long)(((loc & 0xfu) << 28) + off) << 32) | r32);
+      seen = shfl64(seen, grp * 8);
+      if (action == 1) {
+        if (sub == 0) atomicOr(status, UGK_ST_DUP_KEY);
+        done = true;
+      } else if (action == 2) {
+        if (seen == expect) {
+          done = true;
+        } else {  // another key of this launch took it: walk again from the start (rare)
+          win = home;
+          first_tomb = kNone;
+          steps = 0;
+        }
+      } else if (!done) {
+        win += 16;
+        if (win >= ne) win = 0;
+        if (++steps > 2 * lines + 2) {
+          if (sub == 0) atomicOr(status, UGK_ST_TABLE_FULL);
+          done = true;
+        }
+      }
+    }
+  }
+}
+
+template <typename K>
+__global__ __launch_bounds__(kBlock) void h32_evict_kernel(ugk_table_t t, const K *keys, size_t n,
+                                                           unsigned long long *slot_bits, uint64_t nslots,
+                                                           uint32_t *status) {
+  unsigned long long *table = reinterpret_cast<unsigned long long *>(t.table);
+  const uint64_t ne = t.size;
+  for (size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x; i < n; i += (size_t)gridDim.x * kBlock) {
+    const uint64_t row = h32_row(t, key_to_u64<K>(keys[i]));
+    bool done = row >= kH32Tomb;
+    if (done) atomicOr(status, UGK_ST_EVICT_ABSENT);
+    uint64_t pos = done ? 0 : h32_home(row, ne);
+    for (uint64_t step = 0; step < ne && !done; ++step) {
+      const unsigned long long w = __atomic_load_n(table + pos, __ATOMIC_RELAXED);
+      if ((uint32_t)w == (uint32_t)row) {
+        if (slot_bits) release_slot(slot_bits, nslots, (uint32_t)(w >> 32) & 0x0fffffffu, status);
+        // the entry leaves whole: a concurrent lookup sees the key there (its slot keeps the row until a later lookup
+        // has passed) or gone
+        __atomic_store_n(table + pos, kH32TombWord, __ATOMIC_RELAXED);
+        done = true;
+      } else if (w == kH32EmptyWord) {
+        atomicOr(status, UGK_ST_EVICT_ABSENT);
+        done = true;
+      } else if (++pos == ne) {
+        pos = 0;
+      }
+    }
+    if (!done) atomicOr(status, UGK_ST_EVICT_ABSENT);
+  }
+}
+
+__global__ __launch_bounds__(kBlock) void h32_census_kernel(const unsigned long long *table, size_t n,
+                                                            unsigned long long *census) {
+  unsigned long long occ = 0, tomb = 0, empty = 0;
+  for (size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x; i < n; i += (size_t)gridDim.x * kBlock) {
+    const uint32_t k = (uint32_t)table[i];
+    if (k == kH32Empty) ++empty;
+    else if (k == kH32Tomb) ++tomb;
+    else ++occ;
+  }
+  __shared__ unsigned long long red[3];
+  if (threadIdx.x < 3) red[threadIdx.x] = 0;
+  __syncthreads();
+  atomicAdd(&red[0], occ);
+  atomicAdd(&red[1], tomb);
+  atomicAdd(&red[2], empty);
+  __syncthreads();
+  if (threadIdx.x < 3) atomicAdd(census + threadIdx.x, red[threadIdx.x]);
+}
+
 template <typename K, int KIND>
 __global__ __launch_bounds__(kBlock) void lookup_kernel(ugk_table_t t, const K *keys, size_t n, uint32_t fallback_loc,
                                                         uint32_t *loc_out, uint32_t *off_out) {
@@ -223,10 +365,15 @@ __global__ __launch_bounds__(kBlock) void census_kernel(const ugk_bucket_t *tabl
 }
 
 int check_table(const ugk_table_t &t, const char *who) {
-  UGK_REQUIRE(t.kind == 1 || t.kind == 2, "%s: table kind %d is not flat(1) or hash(2)", who, t.kind);
+  UGK_REQUIRE(t.kind >= 1 && t.kind <= 3, "%s: table kind %d is not flat(1), hash(2) or compact hash(3)", who, t.kind);
   UGK_REQUIRE(t.table != nullptr && t.size > 0, "%s: empty table", who);
   if (t.kind == 2) {
     UGK_REQUIRE(t.size % 8 == 0, "%s: hash table needs a multiple of 8 buckets, got %llu", who,
+                (unsigned long long)t.size);
+    UGK_REQUIRE((uintptr_t)t.table % 128 == 0, "%s: hash table must be 128-byte aligned", who);
+  }
+  if (t.kind == 3) {
+    UGK_REQUIRE(t.size % 16 == 0, "%s: compact hash table needs a multiple of 16 entries, got %llu", who,
                 (unsigned long long)t.size);
     UGK_REQUIRE((uintptr_t)t.table % 128 == 0, "%s: hash table must be 128-byte aligned", who);
   }
@@ -244,9 +391,12 @@ int table_insert(ugk_table_t t, const K *keys, const uint32_t *offs, uint32_t se
   if (t.kind == 1)
     hipLaunchKernelGGL(flat_insert_kernel<K>, dim3(grid), dim3(kBlock), 0, as_stream(stream), (uint32_t *)t.table,
                        t.size, keys, offs, seq_base, loc, n, status);
-  else
+  else if (t.kind == 2)
     hipLaunchKernelGGL(hash_insert_kernel<K>, dim3(clamp_grid((n + 31) / 32, 0)), dim3(kBlock), 0, as_stream(stream),
                        (ugk_bucket_t *)t.table, t.size, keys, offs, seq_base, loc, n, status);
+  else
+    hipLaunchKernelGGL(h32_insert_kernel<K>, dim3(clamp_grid((n + 31) / 32, 0)), dim3(kBlock), 0, as_stream(stream),
+                       t, keys, offs, seq_base, loc, n, status);
   UGK_HIP(hipGetLastError());
   return 0;
 }
@@ -262,9 +412,12 @@ int table_evict(ugk_table_t t, const K *keys, size_t n, uint64_t *slot_bits_dev,
   if (t.kind == 1)
     hipLaunchKernelGGL(flat_evict_kernel<K>, dim3(grid), dim3(kBlock), 0, as_stream(stream), (uint32_t *)t.table,
                        t.size, keys, n, slot_bits, nslots, status);
-  else
+  else if (t.kind == 2)
     hipLaunchKernelGGL(hash_evict_kernel<K>, dim3(grid), dim3(kBlock), 0, as_stream(stream), (ugk_bucket_t *)t.table,
                        t.size, keys, n, slot_bits, nslots, status);
+  else
+    hipLaunchKernelGGL(h32_evict_kernel<K>, dim3(grid), dim3(kBlock), 0, as_stream(stream), t, keys, n, slot_bits,
+                       nslots, status);
   UGK_HIP(hipGetLastError());
   return 0;
 }
@@ -279,8 +432,11 @@ int table_lookup_host(ugk_table_t t, const K *keys, size_t n, uint32_t fallback_
   if (t.kind == 1)
     hipLaunchKernelGGL((lookup_kernel<K, 1>), dim3(grid), dim3(kBlock), 0, as_stream(stream), t, keys, n,
                        fallback_loc, loc_out, off_out);
-  else
+  else if (t.kind == 2)
     hipLaunchKernelGGL((lookup_kernel<K, 2>), dim3(grid), dim3(kBlock), 0, as_stream(stream), t, keys, n,
+                       fallback_loc, loc_out, off_out);
+  else
+    hipLaunchKernelGGL((lookup_kernel<K, 3>), dim3(grid), dim3(kBlock), 0, as_stream(stream), t, keys, n,
                        fallback_loc, loc_out, off_out);
   UGK_HIP(hipGetLastError());
   return 0;
@@ -298,6 +454,38 @@ size_t ugk_hash_buckets_for(size_t n_entries, double load_factor) {
   size_t nb = (size_t)std::ceil((double)n_entries / load_factor) + 1;
   if (nb < 64) nb = 64;
   return (nb + 7) / 8 * 8;
+}
+
+size_t ugk_hash32_entries_for(size_t n_entries, double load_factor) {
+  if (!(load_factor > 0.0) || load_factor > 0.95) load_factor = 0.7;
+  size_t ne = (size_t)std::ceil((double)n_entries / load_factor) + 1;
+  if (ne < 64) ne = 64;
+  return (ne + 15) / 16 * 16;
+}
+
+int ugk_table_init(ugk_table_t t, void *stream) {
+  if (check_table(t, "ugk_table_init")) return 1;
+  if (t.kind == 1) return ugk_fill_u32(static_cast<uint32_t *>(t.table), UGK_EMPTY_U32, t.size, stream);
+  if (t.kind == 2) return ugk_hash_init(static_cast<ugk_bucket_t *>(t.table), t.size, stream);
+  const unsigned grid = clamp_grid((t.size + kBlock - 1) / kBlock, 0);
+  hipLaunchKernelGGL(h32_init_kernel, dim3(grid), dim3(kBlock), 0, as_stream(stream),
+                     static_cast<unsigned long long *>(t.table), t.size);
+  UGK_HIP(hipGetLastError());
+  return 0;
+}
+
+int ugk_table_census(ugk_table_t t, uint64_t *census_dev, void *stream) {
+  if (check_table(t, "ugk_table_census")) return 1;
+  UGK_REQUIRE(t.kind == 2 || t.kind == 3, "ugk_table_census: a flat table has no buckets to count");
+  UGK_REQUIRE(census_dev, "ugk_table_census: null output");
+  if (t.kind == 2) return ugk_hash_census(static_cast<const ugk_bucket_t *>(t.table), t.size, census_dev, stream);
+  if (ugk_fill_u32(reinterpret_cast<uint32_t *>(census_dev), 0u, 6, stream)) return 1;
+  const unsigned grid = clamp_grid((t.size + kBlock - 1) / kBlock, 0);
+  hipLaunchKernelGGL(h32_census_kernel, dim3(grid), dim3(kBlock), 0, as_stream(stream),
+                     static_cast<const unsigned long long *>(t.table), t.size,
+                     reinterpret_cast<unsigned long long *>(census_dev));
+  UGK_HIP(hipGetLastError());
+  return 0;
 }
 
 int ugk_hash_init(ugk_bucket_t *table_dev, size_t nbuckets, void *stream) {

@@ -24,6 +24,7 @@ HINT_UNKNOWN = 0xFFFFFFFF
 TABLE_NONE = 0
 TABLE_FLAT = 1
 TABLE_HASH = 2
+TABLE_HASH32 = 3
 
 
 class UgkError(RuntimeError):
@@ -90,6 +91,9 @@ SIGNATURES = {
     "ugk_gather_idx": [_vp, _u64, _vp, _sz, _vp, _sz, C.c_uint, _vp, _vp],
     "ugk_hash_buckets_for": [_sz, C.c_double],
     "ugk_hash_init": [_vp, _sz, _vp],
+    "ugk_hash32_entries_for": [_sz, C.c_double],
+    "ugk_table_init": [Table, _vp],
+    "ugk_table_census": [Table, _vp, _vp],
     "ugk_table_insert_u32": [Table, _vp, _vp, _u32, _u32, _sz, _vp, _vp],
     "ugk_table_insert_i64": [Table, _vp, _vp, _u32, _u32, _sz, _vp, _vp],
     "ugk_table_evict_u32": [Table, _vp, _sz, _vp, _vp],
@@ -141,7 +145,7 @@ SIGNATURES = {
     "ugk_rows_to_keys": [_vp, _sz, _u64, _u64, _vp, _vp],
     "ugk_last_error": [],
 }
-_RESTYPES = {"ugk_extract_mix_max_groups": C.c_uint, "ugk_hash_buckets_for": _sz, "ugk_dedup_workspace_bytes": _sz, "ugk_rank_workspace_bytes": _sz,
+_RESTYPES = {"ugk_extract_mix_max_groups": C.c_uint, "ugk_hash_buckets_for": _sz, "ugk_hash32_entries_for": _sz, "ugk_dedup_workspace_bytes": _sz, "ugk_rank_workspace_bytes": _sz,
              "ugk_bitmap_workspace_bytes": _sz, "ugk_last_error": C.c_char_p}
 _NO_CHECK = set(_RESTYPES) | {"ugk_abi_version"}
 
