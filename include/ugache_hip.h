@@ -33,6 +33,7 @@ extern "C" {
 #define UGK_ST_DUP_KEY 0x4u          /* insert of a key that is already present (the reference asserts) */
 #define UGK_ST_EVICT_ABSENT 0x8u     /* evict of a key that is not present */
 #define UGK_ST_BAD_SEGMENT 0x10u     /* pooled extraction: offsets that leave [0, nnz], run backwards or do not span [0, nnz] */
+#define UGK_ST_PLACE_PROMISE 0x20u   /* ugk_rank_place_observed: k or more rows were observed; nothing was placed */
 
 /* element code of the pooled extraction for bfloat16 rows (fp32 and fp16 are named by their size, 4 and 2) */
 #define UGK_ELEM_BF16 0x102
@@ -102,7 +103,7 @@ typedef struct {
 const char *ugk_last_error(void);
 /* version of this ABI; bumped on any signature change.  ugk_abi_version() is what the loaded library was built with:
  * a caller compiled against another UGK_ABI_VERSION must not go on. */
-#define UGK_ABI_VERSION 18
+#define UGK_ABI_VERSION 19
 int ugk_abi_version(void);
 
 /* ---- runtime plumbing: Device::{AllocDataSpace,FreeDataSpace,CopyDataFromTo,StreamSync,CreateStream}
@@ -471,6 +472,16 @@ int ugk_record_restore(const uint64_t *entries_dev, size_t n, uint32_t *counts_d
  * or wider than the set of rows observed so far, otherwise trades its never-counted rows for the lowest-numbered
  * ones).  keep_dev is read only and may not be one of the two output bitmaps; ugk_rank_threshold reports the last row
  * taken from the group that was cut.
+ * ugk_rank_place_observed: the placement for a caller that knows that fewer than k rows were observed (say, the rows
+ * observed at the last placement plus the keys counted since stay below k), 0 < k < num_rows: in_new = every observed
+ * row and the lowest k - |observed| never-observed rows, what ugk_rank_place computes in that case, in five launches
+ * over the bitmaps and none over the counters.  If k or more rows turn out to be observed, UGK_ST_PLACE_PROMISE is set
+ * in *status_dev and in_new_dev is left as it was.  cached_dev (may be NULL; then evict_ws_dev, insert_ws_dev and
+ * totals_host may be NULL too): the rows cached now; the rows that leave (cached & ~in_new) and that come in
+ * (in_new & ~cached) are counted in the same pass: evict_ws_dev / insert_ws_dev (ugk_bitmap_workspace_bytes() each)
+ * are left as ugk_bitmap_count(cached, in_new) / ugk_bitmap_count(in_new, cached) would leave them, ready for
+ * ugk_bitmap_emit, and totals_host (three pinned words) receives [0] rows leaving, [1] rows coming in, [2] rows
+ * observed (before a reset).
  * ugk_rank_threshold: copies the rank of the k-th best row of the last ugk_rank_place to the host (blocking; for tests
  * and logs; all ones for k == 0, zero for k >= num_rows). */
 size_t ugk_rank_workspace_bytes(void);
@@ -479,6 +490,9 @@ int ugk_rank_place(uint32_t *counts_dev, uint64_t num_rows, uint64_t k, void *ws
 int ugk_rank_place_keep(uint32_t *counts_dev, uint64_t num_rows, uint64_t k, void *ws_dev, uint64_t *in_new_dev,
                         uint64_t *scratch_bitmap_dev, uint64_t *observed_dev, const uint64_t *keep_dev,
                         int reset_counts, void *stream);
+int ugk_rank_place_observed(uint32_t *counts_dev, uint64_t num_rows, uint64_t k, void *ws_dev, uint64_t *in_new_dev,
+                            uint64_t *observed_dev, int reset_counts, const uint64_t *cached_dev, void *evict_ws_dev,
+                            void *insert_ws_dev, uint32_t *totals_host, uint32_t *status_dev, void *stream);
 int ugk_rank_threshold(const void *ws_dev, uint64_t *threshold_host, void *stream);
 /* Ordered compaction over bitmaps.  The set S = { p < nbits : bit p of m is set }, m = (invert_a ? ~a : a) & ~b
  * (b_dev may be NULL).  ugk_bitmap_count writes |S| to *total_host (pinned host word, may be NULL) and leaves the

@@ -1316,6 +1316,52 @@ int ugk_rank_place_keep(uint32_t *counts, uint64_t num_rows, uint64_t k, void *w
   *static_cast<uint64_t *>(ws) = k == 0 ? ~0ull : k >= num_rows ? 0ull : ((uint64_t)th_count << 32) | th_tie;
   return 0;
 }
+int ugk_rank_place_observed(uint32_t *counts, uint64_t num_rows, uint64_t k, void *ws, uint64_t *in_new,
+                            uint64_t *observed, int reset_counts, const uint64_t *cached, void *evict_ws,
+                            void *insert_ws, uint32_t *totals_host, uint32_t *status, void *) {
+  REQUIRE(counts && ws && in_new && observed && status, "ugk_rank_place_observed: null pointer");
+  REQUIRE(num_rows > 0 && num_rows < 0xffffffffull, "ugk_rank_place_observed: rows do not fit 32 bits");
+  REQUIRE(k > 0 && k < num_rows, "ugk_rank_place_observed: k outside (0, rows)");
+  REQUIRE(in_new != observed && cached != in_new, "ugk_rank_place_observed: output bitmap is an input bitmap");
+  REQUIRE(!cached || (evict_ws && insert_ws && totals_host && evict_ws != insert_ws),
+          "ugk_rank_place_observed: counting what changes needs two workspaces and the host words");
+  const uint64_t n_words = (num_rows + 63) / 64;
+  uint64_t seen = 0;
+  for (uint64_t w = 0; w < n_words; ++w) seen += __builtin_popcountll(ld(observed + w));
+  if (totals_host) totals_host[2] = (uint32_t)seen;
+  if (seen >= k) {
+    or_status(status, UGK_ST_PLACE_PROMISE);
+    if (cached) totals_host[0] = totals_host[1] = 0;
+    return 0;
+  }
+  uint64_t need = k - seen, last_row = 0;
+  uint32_t leaving = 0, coming = 0;
+  for (uint64_t w = 0; w < n_words; ++w) {
+    const uint64_t obs = ld(observed + w);
+    uint64_t m = obs;
+    for (uint64_t r = w * 64; r < std::min(num_rows, w * 64 + 64) && need; ++r)
+      if (!((obs >> (r & 63)) & 1)) {
+        m |= 1ull << (r & 63);
+        last_row = r;
+        --need;
+      }
+    in_new[w] = m;
+    if (cached) {
+      leaving += __builtin_popcountll(ld(cached + w) & ~m);
+      coming += __builtin_popcountll(m & ~ld(cached + w));
+    }
+  }
+  if (cached) {
+    *static_cast<uint32_t *>(evict_ws) = totals_host[0] = leaving;
+    *static_cast<uint32_t *>(insert_ws) = totals_host[1] = coming;
+  }
+  if (reset_counts) {
+    for (uint64_t r = 0; r < num_rows; ++r) st(counts + r, 0u);
+    for (uint64_t w = 0; w < n_words; ++w) st(observed + w, (uint64_t)0);
+  }
+  *static_cast<uint64_t *>(ws) = 0xffffffffull - last_row;
+  return 0;
+}
 int ugk_rank_threshold(const void *ws, uint64_t *threshold_host, void *) {
   *threshold_host = *static_cast<const uint64_t *>(ws);
   return 0;

@@ -168,6 +168,97 @@ def test_rank_place_on_the_committed_golden_case():
     assert th == (fx["rank_counts_observed"][k - 1] << 32) | last
 
 
+def _place_observed(counts, k, reset, cached=None):
+    """ugk_rank_place_observed -> (membership bits or None when the promise was refused, status word, counters afterwards,
+    lists of the rows that leave and come in when `cached` is given, the observed count the host was told)"""
+    n = len(counts)
+    words = (n + 63) // 64
+    d_counts = to_dev(counts)
+    ws = dev_bytes(hip.lib().ugk_rank_workspace_bytes())
+    bitmap = dev_bytes(words * 8, fill=0xA5)
+    pad = np.zeros(words * 64, bool)
+    pad[:n] = counts > 0
+    observed = to_dev(np.packbits(pad, bitorder="little").view(np.uint64))
+    st = dev_zeros_u32(1)
+    totals = PinnedArray((4,), np.uint32)
+    try:
+        totals.array[...] = 0xFFFFFFFF
+        d_cached = ws_out = ws_in = None
+        if cached is not None:
+            cpad = np.zeros(words * 64, bool)
+            cpad[:n] = cached
+            d_cached = to_dev(np.packbits(cpad, bitorder="little").view(np.uint64))
+            ws_out = dev_bytes(hip.lib().ugk_bitmap_workspace_bytes())
+            ws_in = dev_bytes(hip.lib().ugk_bitmap_workspace_bytes())
+        hip.call("ugk_rank_place_observed", ptr(d_counts), n, k, ptr(ws), ptr(bitmap), ptr(observed), reset,
+                 ptr(d_cached), ptr(ws_out), ptr(ws_in), totals.ptr, ptr(st), None)
+        status = status_value(st)
+        seen = int(totals.array[2])
+        if status & hip.ST_PLACE_PROMISE:
+            assert np.array_equal(to_np(bitmap)[: words * 8], np.full(words * 8, 0xA5, np.uint8))  # left as it was
+            return None, status, to_np(d_counts, np.uint32)[:n], None, None, seen
+        th = C.c_uint64(0)
+        hip.call("ugk_rank_threshold", ptr(ws), C.byref(th), None)
+        bits = np.unpackbits(to_np(bitmap)[: words * 8], bitorder="little")
+        assert not bits[n:].any()
+        left = np.unpackbits(to_np(observed, np.uint8)[: words * 8], bitorder="little")[:n].astype(bool)
+        assert np.array_equal(left, (counts > 0) & (reset == 0))
+        leaving = coming = None
+        if cached is not None:
+            n_out, n_in = int(totals.array[0]), int(totals.array[1])
+            out_l, in_l = dev_zeros_u32(max(n_out, 1)), dev_zeros_u32(max(n_in, 1))
+            hip.call("ugk_bitmap_emit", ptr(d_cached), ptr(bitmap), 0, n, ptr(ws_out), ptr(out_l), n_out, None)
+            hip.call("ugk_bitmap_emit", ptr(bitmap), ptr(d_cached), 0, n, ptr(ws_in), ptr(in_l), n_in, None)
+            sync()
+            leaving, coming = to_np(out_l, np.uint32)[:n_out], to_np(in_l, np.uint32)[:n_in]
+        return bits[:n].astype(bool), (status, th.value), to_np(d_counts, np.uint32)[:n], leaving, coming, seen
+    finally:
+        totals.free()
+
+
+@pytest.mark.parametrize("kind", ["zipf", "zero", "ties"])
+@pytest.mark.parametrize("n", [2, 3, 63, 64, 65, 1000, 100_003, 2_000_001, 40_000_000])
+def test_rank_place_observed_is_rank_place_where_few_rows_were_observed(kind, n):
+    """every observed row and the lowest never-observed ones, as ugk_rank_place and a full sort give them; the rows
+    that leave and come in against a cached set, counted on the way, as flatnonzero gives them; k at or below the
+    number of observed rows is refused"""
+    rng = np.random.default_rng(n * 13 + len(kind))
+    if n < 40_000_000:
+        counts = _counts(rng, n, kind)
+    else:  # sparse: whole chunks and blocks without an observed row
+        counts = np.zeros(n, np.uint32)
+        counts[rng.integers(0, n, size=300_000)] = 3
+        counts[n // 2: n // 2 + 100_000] = 1
+    ranks = ranks_of(counts)
+    order = np.sort(ranks)[::-1]
+    observed = int((counts > 0).sum())
+    ks = sorted({observed + 1, observed + 2, (observed + n) // 2, n - 1} - {0, n})
+    ks = [k for k in ks if observed < k < n]
+    for k in ks:
+        want = ranks >= order[k - 1]
+        cached = np.zeros(n, bool)
+        cached[rng.permutation(n)[: max(k - 1, 0)] if n < 3_000_000 else slice(0, k - 1)] = True
+        for reset in (0, 1):
+            got, (status, th), left, leaving, coming, seen = _place_observed(counts, k, reset, cached)
+            assert status == 0 and seen == observed
+            assert th == int(order[k - 1]), (kind, n, k)
+            assert np.array_equal(got, want), (kind, n, k, reset)
+            assert np.array_equal(left, counts if reset == 0 else np.zeros(n, np.uint32))
+            assert np.array_equal(leaving, np.flatnonzero(cached & ~want).astype(np.uint32))
+            assert np.array_equal(coming, np.flatnonzero(want & ~cached).astype(np.uint32))
+        if n <= 100_003:
+            plain, _, _ = _place(counts, k, 0, with_observed=True)
+            assert np.array_equal(plain, want)
+            got, (status, _), _, leaving, coming, _ = _place_observed(counts, k, 0, None)  # no diff asked for
+            assert status == 0 and np.array_equal(got, want) and leaving is None
+    for k in sorted({1, observed // 2, observed} - {0}):
+        if k >= n or k > observed:
+            continue
+        got, status, left, _, _, seen = _place_observed(counts, k, 1, np.zeros(n, bool))
+        assert got is None and status == hip.ST_PLACE_PROMISE and seen == observed
+        assert np.array_equal(left, counts)  # nothing was reset either
+
+
 def _bits(rng, nbits, density):
     words = (nbits + 63) // 64
     b = rng.random(words * 64) < density

@@ -429,6 +429,7 @@ void ExtractSession::RecordLaunch(const KeyT *nodes, size_t num_nodes, const Rec
     return;
   }
   std::lock_guard<std::mutex> guard(_enqueue_mu);  // not in the middle of a placement's passes
+  _keys_counted_since += num_nodes;
   UGK_CALL(ugk_stream_wait_event(_record_stream, plan.after));
   UGK_CALL(Record(nodes, num_nodes, RunConfig::key_map_inv, RunConfig::key_map_mask, _hot_counts->ptr<uint32_t>(),
                   _cache_ctx->_num_total_nodes, ObservedBits(), _status, _host_mirror, _record_stream));
@@ -462,24 +463,52 @@ void ExtractSession::JoinRecordOnHost() {
   _record_pending = false;
 }
 
-void ExtractSession::PlaceOnDevice(size_t num_cached, uint64_t *in_new_bits, uint64_t *scratch_bits,
-                                   const uint64_t *keep_bits, void *rank_ws,
-                                   bool reset_counts, StreamHandle stream) {
+bool ExtractSession::PlaceOnDevice(size_t num_cached, uint64_t *in_new_bits, uint64_t *scratch_bits,
+                                   const uint64_t *keep_bits, void *rank_ws, bool reset_counts, const DiffCount *diff,
+                                   StreamHandle stream) {
   CHECK_NOTNULL(_hot_counts) << "placement on the device needs the device-side hotness counters (COLL_GPU_RECORD=1)";
   const size_t rows = _cache_ctx->_num_total_nodes;
   std::lock_guard<std::mutex> no_drain(_drain_mu);
   std::lock_guard<std::mutex> guard(_enqueue_mu);
-  if (_counted_on_callers_stream.load()) {
+  const bool replays_count = _counted_on_callers_stream.load();
+  if (replays_count) {
     // replays of a graph that counts run on the caller's stream, not on the record stream: the passes below start
     // behind whatever that stream holds at this point (a refresh that shares the stream of the replays, the usual
     // case, is thereby ordered against all of them; replays launched from elsewhere while the passes run are not)
     UGK_CALL(ugk_event_record(_ev_placed, stream));
     UGK_CALL(ugk_stream_wait_event(_record_stream, _ev_placed));
   }
-  UGK_CALL(ugk_rank_place_keep(_hot_counts->ptr<uint32_t>(), rows, num_cached, rank_ws, in_new_bits, scratch_bits,
-                               ObservedBits(), keep_bits, reset_counts ? 1 : 0, _record_stream));
+  // every counting launch enqueued so far is in this sum, and on the record stream in front of the passes
+  const uint64_t counted = _keys_counted_since.exchange(0);
+  const uint64_t bound = _observed_known == UINT64_MAX ? UINT64_MAX : _observed_known + counted;
+  if (_observed_known != UINT64_MAX) _observed_known = bound;  // stands until the placement's own count is read
+  const bool few_observed = diff != nullptr && keep_bits == nullptr && !replays_count && ObservedBits() != nullptr &&
+                            num_cached > 0 && num_cached < rows && bound < num_cached;
+  if (few_observed) {
+    UGK_CALL(ugk_rank_place_observed(_hot_counts->ptr<uint32_t>(), rows, num_cached, rank_ws, in_new_bits,
+                                     ObservedBits(), reset_counts ? 1 : 0, diff->cached_bits, diff->evict_ws,
+                                     diff->insert_ws, diff->totals_host, diff->status_dev, _record_stream));
+  } else {
+    UGK_CALL(ugk_rank_place_keep(_hot_counts->ptr<uint32_t>(), rows, num_cached, rank_ws, in_new_bits, scratch_bits,
+                                 ObservedBits(), keep_bits, reset_counts ? 1 : 0, _record_stream));
+    // how many rows are observed now: what lets the next placement skip the counters
+    if (diff && !reset_counts && ObservedBits())
+      UGK_CALL(ugk_bitmap_count(ObservedBits(), nullptr, 0, rows, diff->evict_ws, diff->totals_host + 2,
+                                _record_stream));
+  }
+  _observed_word = diff && ObservedBits() ? diff->totals_host + 2 : nullptr;
+  _placement_reset = reset_counts;
   UGK_CALL(ugk_event_record(_ev_placed, _record_stream));
   UGK_CALL(ugk_stream_wait_event(stream, _ev_placed));
+  return few_observed;
+}
+
+void ExtractSession::PlacementWaitedFor() {
+  std::lock_guard<std::mutex> guard(_enqueue_mu);
+  if (_placement_reset) _observed_known = 0;  // keys counted while the passes ran are in _keys_counted_since
+  else if (_observed_word) _observed_known = *_observed_word;
+  else _observed_known = UINT64_MAX;
+  _observed_word = nullptr;
 }
 
 void ExtractSession::SeedHotness(const FreqEntry *entries, size_t num_entries) {
@@ -490,6 +519,7 @@ void ExtractSession::SeedHotness(const FreqEntry *entries, size_t num_entries) {
   static_assert(sizeof(FreqEntry) == sizeof(uint64_t), "an entry is one (count << 32 | row) word");
   const size_t cap = _hot_entries->nbytes() / sizeof(uint64_t);
   std::lock_guard<std::mutex> guard(_drain_mu);
+  _keys_counted_since += num_entries;
   uint64_t *dev_list = _hot_entries->ptr<uint64_t>();
   auto *host_list = _hot_entries_host->ptr<FreqEntry>();
   for (size_t first = 0; first < num_entries; first += cap) {
@@ -532,6 +562,10 @@ size_t ExtractSession::DrainHotness(FreqRecorder *recorder) {
     UGK_CALL(ugk_stream_sync(_record_stream));
     recorder->AddEntries(host_list, got);
     moved += got;
+  }
+  {
+    std::lock_guard<std::mutex> placed(_enqueue_mu);
+    _observed_known = 0;  // every counter was handed over; what is counted from here on is in _keys_counted_since
   }
   return moved;
 }
@@ -1485,12 +1519,20 @@ void RefreshSession::refresh_on_device(ExtractSession *session, size_t num_cache
   // Steps 1-3: the new placement as a bitmap, then evict = cached & ~new and insert = new & ~cached, ascending.  Both
   // sets are counted before the one wait that tells the host their sizes.
   // COLL_GPU_REFRESH_STABLE: rows that tie at the last count that gets in stay where they are (cached or not)
-  session->PlaceOnDevice(num_cached, table->InNewBits(), table->_dev_scratch_bits->ptr<uint64_t>(),
-                         RunConfig::gpu_refresh_stable ? table->InCacheBits() : nullptr, table->_dev_rank_ws->ptr(),
-                         !RunConfig::gpu_refresh_keep, stream);
-  volatile uint32_t *n_evict_word = table->CountBits(table->InCacheBits(), table->InNewBits(), false, num_rows, 0, stream);
-  volatile uint32_t *n_insert_word = table->CountBits(table->InNewBits(), table->InCacheBits(), false, num_rows, 1, stream);
+  // (a placement that knows that fewer rows were observed than the cache holds counts both sets on its way)
+  const ExtractSession::DiffCount diff = {table->InCacheBits(), table->_dev_bm_ws->ptr(), table->_dev_bm_ws2->ptr(),
+                                          table->DevWords() + 8, _status_handle->ptr<uint32_t>()};
+  const bool counted = session->PlaceOnDevice(
+      num_cached, table->InNewBits(), table->_dev_scratch_bits->ptr<uint64_t>(),
+      RunConfig::gpu_refresh_stable ? table->InCacheBits() : nullptr, table->_dev_rank_ws->ptr(),
+      !RunConfig::gpu_refresh_keep, &diff, stream);
+  volatile uint32_t *n_evict_word = table->DevWords() + 8, *n_insert_word = table->DevWords() + 9;
+  if (!counted) {
+    n_evict_word = table->CountBits(table->InCacheBits(), table->InNewBits(), false, num_rows, 0, stream);
+    n_insert_word = table->CountBits(table->InNewBits(), table->InCacheBits(), false, num_rows, 1, stream);
+  }
   UGK_CALL(ugk_stream_sync(stream));
+  session->PlacementWaitedFor();
   const size_t num_evicted = *n_evict_word, num_insert = *n_insert_word;
   TensorPtr evict_rows = table->EmitBits(table->InCacheBits(), table->InNewBits(), false, num_rows, 0, num_evicted,
                                          __evict_rows, alloc, gpu_ctx, stream);
@@ -1548,7 +1590,8 @@ void RefreshSession::refresh_on_device(ExtractSession *session, size_t num_cache
   uint32_t stw[9] = {0};  // [0] status bits, [8] rows taken from the stage so far
   UGK_CALL(ugk_memcpy_async(stw, _status_handle->ptr<uint32_t>(), sizeof(stw), stream));
   table->CheckStatus(stream, "refresh on the device");  // waits for the stream
-  CHECK_EQ(stw[0], 0u) << "refresh on the device: a listed row or slot is outside its table or bitmap";
+  CHECK_EQ(stw[0], 0u) << "refresh on the device: a listed row or slot is outside its table or bitmap (1), or the "
+                          "placement found more observed rows than the host's bound allows (0x20)";
   const uint32_t from_stage = stw[8] - _rows_from_stage;
   _rows_from_stage = stw[8];
   if (n_free_word) CHECK_EQ((size_t)*n_free_word, num_free_expected);
@@ -1564,7 +1607,8 @@ void RefreshSession::refresh_on_device(ExtractSession *session, size_t num_cache
   const bool rebuilt = table->MaybeRebuild(alloc, gpu_ctx, local, stream, [&]() {
     session->WaitForLookupsInFlight(foreground, 20.0);
   });
-  LOG(INFO) << "refresh on the device: bitmaps " << sync_s << " s, placement + key lists " << place_s << " s, evict "
+  LOG(INFO) << "refresh on the device: bitmaps " << sync_s << " s, placement"
+            << (counted ? " (from the observed rows alone)" : "") << " + key lists " << place_s << " s, evict "
             << evict_s << " s, wait for a lookup " << wait_s << " s, row copy + insert " << insert_s
             << " s (" << from_stage << " of " << num_insert << " rows from the stage), table rebuild "
             << (rebuilt ? t_phase.Passed() : 0.0) << " s";

@@ -158,6 +158,11 @@ class ExtractSession {
   void RecordLaunch(const KeyT *nodes, size_t num_nodes, const RecordPlan &plan);
   bool _capture_query_refused_logged = false;
   std::atomic<bool> _counted_on_callers_stream{false};  // some lookup was recorded into a graph together with its counting
+  // bound on the rows observed (counter above zero): what the last placement saw plus every key counted since
+  std::atomic<uint64_t> _keys_counted_since{0};
+  uint64_t _observed_known = UINT64_MAX;        // UINT64_MAX: no placement has looked yet
+  const uint32_t *_observed_word = nullptr;     // pinned word the placement in flight writes the count to
+  bool _placement_reset = false;
 
   MemHandle _mix_counts;           // pinned: one word per workgroup of the fused kernel, its two row counts
   uint32_t _mix_groups = 0;        // workgroups of the last fused launch
@@ -316,8 +321,21 @@ class ExtractSession {
   int DeviceId() const { return _cache_ctx->_trainer_ctx.device_id; }
   // what a foreground refresh may read rows from besides the host table (null: nothing)
   const ugk_stage_t *StageForRefresh(bool foreground, StreamHandle stream);
-  void PlaceOnDevice(size_t num_cached, uint64_t *in_new_bits, uint64_t *scratch_bits, const uint64_t *keep_bits,
-                     void *rank_ws, bool reset_counts, StreamHandle stream);
+  // What changes, counted on the way when the placement can tell (DiffCount non-null and the return value true): the
+  // two workspaces are left ready for ugk_bitmap_emit and totals_host[0..1] (pinned) receive the rows that leave and
+  // that come in once `stream` has been waited for.  That is the case when fewer rows can have been observed than the
+  // cache holds (the rows observed at the last placement plus the keys counted since stay below num_cached, no tie
+  // rule, no counting inside a caller's graph): then no pass over the counters is made either.
+  struct DiffCount {
+    const uint64_t *cached_bits;
+    void *evict_ws, *insert_ws;
+    uint32_t *totals_host;  // three pinned words; [2] receives the rows observed
+    uint32_t *status_dev;
+  };
+  bool PlaceOnDevice(size_t num_cached, uint64_t *in_new_bits, uint64_t *scratch_bits, const uint64_t *keep_bits,
+                     void *rank_ws, bool reset_counts, const DiffCount *diff, StreamHandle stream);
+  // after `stream` has been waited for: the host learns how many rows the placement saw observed
+  void PlacementWaitedFor();
   // the device-side counting of the following lookups covers only the first `num_keys` keys of a batch
   // (the recorded prefix of LookupManager's record thread); SIZE_MAX, the default: the whole batch
   void SetRecordLimit(size_t num_keys) { _record_limit = num_keys; }

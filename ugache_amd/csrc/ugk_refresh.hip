@@ -330,6 +330,135 @@ __global__ __launch_bounds__(kBlock) void rank_combine_kernel(const RankWs *ws, 
   }
 }
 
+// ---- the placement when the caller knows that fewer rows were observed than are wanted ----------------------------
+// One workgroup, after `observed` was counted and scanned into ws->bm: checks the caller's promise and finds the last
+// needed never-observed row, the (remaining - 1)-th clear bit of `observed` in ascending order (clear bits in front of
+// chunk c = its first bit number - set bits in front of it).
+__global__ __launch_bounds__(kBlock) void rank_locate_unobserved_kernel(RankWs *ws, const unsigned long long *observed,
+                                                                        uint64_t nbits, uint64_t per_chunk,
+                                                                        uint32_t *status, uint32_t *observed_host) {
+  __shared__ uint32_t chunk_of;
+  const int tid = threadIdx.x;
+  const uint32_t total = ws->bm.total;
+  const unsigned long long want = ws->remaining;
+  if (tid == 0 && observed_host) *observed_host = total;
+  if (total >= want) {  // uniform: the promise does not hold, nothing is placed
+    if (tid == 0) atomicOr(status, UGK_ST_PLACE_PROMISE);
+    return;
+  }
+  const uint64_t index = want - total - 1;  // among the clear bits, from 0
+  const uint64_t chunk_bits = per_chunk * 64;
+  auto clear_before = [&](int c) -> uint64_t {  // c in [0, kBmChunks]
+    if (c >= kBmChunks) return nbits - total;
+    const uint64_t first = (uint64_t)c * chunk_bits;
+    return (first < nbits ? first : nbits) - ws->bm.base[c];
+  };
+  constexpr int kPer = kBmChunks / kBlock;
+  for (int j = 0; j < kPer; ++j) {
+    const int c = tid * kPer + j;
+    if (clear_before(c) <= index && index < clear_before(c + 1)) chunk_of = (uint32_t)c;  // exactly one chunk holds it
+  }
+  __syncthreads();
+  if (tid >= kWave) return;
+  const uint32_t c = chunk_of;
+  const uint64_t n_words = (nbits + 63) / 64;
+  const uint64_t begin = (uint64_t)c * per_chunk, end = min(n_words, begin + per_chunk);
+  uint64_t skip = index - clear_before((int)c);  // clear bits of the chunk below the wanted one
+  for (uint64_t w0 = begin; w0 < end; w0 += kWave) {
+    const uint64_t w = w0 + tid;
+    unsigned long long m = 0ull;
+    if (w < end) {
+      m = ~observed[w];
+      if (nbits - w * 64 < 64) m &= (1ull << (nbits - w * 64)) - 1ull;
+    }
+    const uint32_t mine = __popcll(m);
+    uint32_t incl = mine;
+#pragma unroll
+    for (int s = 1; s < kWave; s <<= 1) {
+      const uint32_t up = __shfl_up(incl, s);
+      if (tid >= s) incl += up;
+    }
+    const uint32_t all = __shfl(incl, kWave - 1);
+    if (skip < all) {  // in this group of words; wavefront-uniform
+      if (incl - mine <= skip && skip < incl) {
+        uint32_t drop = (uint32_t)skip - (incl - mine);
+        while (drop--) m &= m - 1;
+        const uint32_t row = (uint32_t)(w * 64 + __builtin_ctzll(m));
+        ws->last_row = row;
+        ws->threshold = rank_of(0u, row);
+        ws->remaining = want - total;
+        ws->from_bitmap = 1;
+        ws->settled = 1;
+      }
+      return;
+    }
+    skip -= all;
+  }
+}
+
+// in_new = observed | (never observed, up to last_row); with `cached`, the rows that leave (cached & ~in_new) and come
+// in (in_new & ~cached) are counted per 64-word block and per chunk on the way, as bitmap_count_kernel would.  One
+// wavefront per chunk.
+__global__ __launch_bounds__(kBlock) void rank_combine_observed_kernel(uint32_t *counts, uint64_t nbits,
+                                                                       uint64_t per_chunk, const RankWs *ws,
+                                                                       unsigned long long *observed,
+                                                                       unsigned long long *in_new,
+                                                                       const unsigned long long *cached,
+                                                                       BmWs *evict_ws, BmWs *insert_ws,
+                                                                       int reset_counts) {
+  if (!ws->from_bitmap) return;
+  const uint64_t wl = ws->last_row >> 6;
+  const unsigned bl = ws->last_row & 63u;
+  const int lane = (int)lane_id();
+  const uint64_t n_words = (nbits + 63) / 64;
+  const uint64_t wave = ((uint64_t)blockIdx.x * kBlock + threadIdx.x) / kWave;
+  const uint64_t n_waves = (uint64_t)gridDim.x * (kBlock / kWave);
+  for (uint64_t chunk = wave; chunk < (uint64_t)kBmChunks; chunk += n_waves) {
+    const uint64_t begin = chunk * per_chunk, end = min(n_words, begin + per_chunk);
+    uint32_t out_sum = 0, in_sum = 0;
+    for (uint64_t w0 = begin; w0 < end; w0 += kWave) {
+      const uint64_t w = w0 + lane;
+      uint32_t leaving = 0, coming = 0;
+      if (w < end) {
+        unsigned long long obs = observed[w];
+        unsigned long long upto = w < wl ? ~0ull : (w == wl ? (bl == 63 ? ~0ull : (1ull << (bl + 1)) - 1ull) : 0ull);
+        if (nbits - w * 64 < 64) upto &= (1ull << (nbits - w * 64)) - 1ull;
+        const unsigned long long nw = obs | (~obs & upto);
+        in_new[w] = nw;
+        if (cached) {
+          const unsigned long long c = cached[w];
+          leaving = __popcll(c & ~nw);
+          coming = __popcll(nw & ~c);
+        }
+        if (reset_counts) {
+          observed[w] = 0;
+          while (obs) {
+            counts[w * 64 + __builtin_ctzll(obs)] = 0;
+            obs &= obs - 1;
+          }
+        }
+      }
+      if (cached) {  // uniform
+#pragma unroll
+        for (int d = kWave / 2; d > 0; d >>= 1) {
+          leaving += __shfl_xor(leaving, d);
+          coming += __shfl_xor(coming, d);
+        }
+        if (lane == 0) {
+          evict_ws->block[w0 / kWave] = leaving;  // chunks begin on block boundaries
+          insert_ws->block[w0 / kWave] = coming;
+        }
+        out_sum += leaving;
+        in_sum += coming;
+      }
+    }
+    if (cached && lane == 0) {
+      evict_ws->base[chunk] = out_sum;
+      insert_ws->base[chunk] = in_sum;
+    }
+  }
+}
+
 // every row, or none: bitmap of n set (or clear) bits, counters reset on request
 __global__ __launch_bounds__(kBlock) void rank_fill_kernel(uint32_t *counts, uint64_t n, unsigned long long *bitmap,
                                                            int all, int reset_counts, RankWs *ws,
@@ -387,8 +516,7 @@ __global__ __launch_bounds__(kBlock) void bitmap_count_kernel(const unsigned lon
   }
 }
 
-__global__ __launch_bounds__(kBlock) void bitmap_scan_kernel(BmWs *ws, uint32_t *total_host, const RankWs *gate) {
-  if (gate && gate->keep_mode != 2) return;
+__device__ __forceinline__ void scan_chunks(BmWs *ws, uint32_t *total_host) {
   constexpr int kPer = kBmChunks / kBlock;  // 32 chunks per thread
   __shared__ uint32_t part[kBlock];
   const int tid = threadIdx.x;
@@ -412,6 +540,22 @@ __global__ __launch_bounds__(kBlock) void bitmap_scan_kernel(BmWs *ws, uint32_t 
     ws->total = part[tid];
     if (total_host) *total_host = part[tid];
   }
+}
+
+__global__ __launch_bounds__(kBlock) void bitmap_scan_kernel(BmWs *ws, uint32_t *total_host, const RankWs *gate) {
+  if (gate && gate->keep_mode != 2) return;
+  scan_chunks(ws, total_host);
+}
+
+// two workspaces in one launch (one workgroup each), totals to totals_host[0] and [1]; gate: a placement that must have
+// taken the observed-rows path
+__global__ __launch_bounds__(kBlock) void bitmap_scan2_kernel(BmWs *a, BmWs *b, uint32_t *totals_host,
+                                                              const RankWs *gate) {
+  if (!gate->from_bitmap) {
+    if (threadIdx.x == 0) totals_host[blockIdx.x] = 0;
+    return;
+  }
+  scan_chunks(blockIdx.x == 0 ? a : b, totals_host + blockIdx.x);
 }
 
 __global__ __launch_bounds__(kBlock) void bitmap_emit_kernel(const unsigned long long *a, const unsigned long long *b,
@@ -572,6 +716,43 @@ int ugk_rank_place_keep(uint32_t *counts_dev, uint64_t num_rows, uint64_t k, voi
   hipLaunchKernelGGL(rank_locate_kernel, dim3(1), dim3(kBlock), 0, st, ws, eq, keep, num_rows, per_chunk);
   hipLaunchKernelGGL(rank_combine_kernel, dim3(word_grid), dim3(kBlock), 0, st, ws, in_new, eq, keep, n_words,
                      reset_counts ? observed : (unsigned long long *)nullptr);
+  UGK_HIP(hipGetLastError());
+  return 0;
+}
+
+int ugk_rank_place_observed(uint32_t *counts_dev, uint64_t num_rows, uint64_t k, void *ws_dev, uint64_t *in_new_dev,
+                            uint64_t *observed_dev, int reset_counts, const uint64_t *cached_dev, void *evict_ws_dev,
+                            void *insert_ws_dev, uint32_t *totals_host, uint32_t *status_dev, void *stream) {
+  UGK_REQUIRE(counts_dev && ws_dev && in_new_dev && observed_dev && status_dev, "ugk_rank_place_observed: null pointer");
+  UGK_REQUIRE(num_rows > 0 && num_rows < 0xffffffffull, "ugk_rank_place_observed: %llu rows do not fit 32 bits",
+              (unsigned long long)num_rows);
+  UGK_REQUIRE(k > 0 && k < num_rows, "ugk_rank_place_observed: k = %llu is not inside (0, %llu)",
+              (unsigned long long)k, (unsigned long long)num_rows);
+  UGK_REQUIRE(in_new_dev != observed_dev && cached_dev != in_new_dev,
+              "ugk_rank_place_observed: the output bitmap is one of the input bitmaps");
+  UGK_REQUIRE(!cached_dev || (evict_ws_dev && insert_ws_dev && totals_host && evict_ws_dev != insert_ws_dev),
+              "ugk_rank_place_observed: counting what changes needs two workspaces and the host words");
+  RankWs *ws = static_cast<RankWs *>(ws_dev);
+  hipStream_t st = as_stream(stream);
+  unsigned long long *observed = reinterpret_cast<unsigned long long *>(observed_dev);
+  const unsigned long long *none = nullptr;
+  const RankWs *no_gate = nullptr;
+  const uint64_t n_words = (num_rows + 63) / 64;
+  const uint64_t per_chunk = bm_words_per_chunk(n_words);
+  const unsigned bm_grid = clamp_grid((kBmChunks + (kBlock / kWave) - 1) / (kBlock / kWave), (unsigned)cu_count() * 8u);
+  hipLaunchKernelGGL(rank_init_kernel, dim3(1), dim3(kBlock), 0, st, ws, (unsigned long long)k);
+  hipLaunchKernelGGL(bitmap_count_kernel, dim3(bm_grid), dim3(kBlock), 0, st, observed, none, 0, num_rows, per_chunk,
+                     &ws->bm, no_gate);
+  hipLaunchKernelGGL(bitmap_scan_kernel, dim3(1), dim3(kBlock), 0, st, &ws->bm, (uint32_t *)nullptr, no_gate);
+  hipLaunchKernelGGL(rank_locate_unobserved_kernel, dim3(1), dim3(kBlock), 0, st, ws, observed, num_rows, per_chunk,
+                     status_dev, totals_host ? totals_host + 2 : (uint32_t *)nullptr);
+  hipLaunchKernelGGL(rank_combine_observed_kernel, dim3(bm_grid), dim3(kBlock), 0, st, counts_dev, num_rows, per_chunk,
+                     (const RankWs *)ws, observed, reinterpret_cast<unsigned long long *>(in_new_dev),
+                     reinterpret_cast<const unsigned long long *>(cached_dev), static_cast<BmWs *>(evict_ws_dev),
+                     static_cast<BmWs *>(insert_ws_dev), reset_counts);
+  if (cached_dev)
+    hipLaunchKernelGGL(bitmap_scan2_kernel, dim3(2), dim3(kBlock), 0, st, static_cast<BmWs *>(evict_ws_dev),
+                       static_cast<BmWs *>(insert_ws_dev), totals_host, (const RankWs *)ws);
   UGK_HIP(hipGetLastError());
   return 0;
 }

@@ -280,33 +280,60 @@ __global__ __launch_bounds__(kBlock) void h32_insert_kernel(ugk_table_t t, const
   }
 }
 
+// Evict, eight keys per wavefront: an 8-lane group reads its key's probe sequence a line at a time; the lane that holds
+// the key's entry stores the tombstone word and releases the slot.  A live key sits in front of the first never-used
+// entry of its sequence (inserts only ever take entries in front of it, evictions leave tombstones), so a line with
+// the key in it settles the walk whatever else it holds, and one without the key but with a never-used entry ends it.
 template <typename K>
 __global__ __launch_bounds__(kBlock) void h32_evict_kernel(ugk_table_t t, const K *keys, size_t n,
                                                            unsigned long long *slot_bits, uint64_t nslots,
                                                            uint32_t *status) {
   unsigned long long *table = reinterpret_cast<unsigned long long *>(t.table);
   const uint64_t ne = t.size;
-  for (size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x; i < n; i += (size_t)gridDim.x * kBlock) {
-    const uint64_t row = h32_row(t, key_to_u64<K>(keys[i]));
-    bool done = row >= kH32Tomb;
-    if (done) atomicOr(status, UGK_ST_EVICT_ABSENT);
-    uint64_t pos = done ? 0 : h32_home(row, ne);
-    for (uint64_t step = 0; step < ne && !done; ++step) {
-      const unsigned long long w = __atomic_load_n(table + pos, __ATOMIC_RELAXED);
-      if ((uint32_t)w == (uint32_t)row) {
-        if (slot_bits) release_slot(slot_bits, nslots, (uint32_t)(w >> 32) & 0x0fffffffu, status);
-        // the entry leaves whole: a concurrent lookup sees the key there (its slot keeps the row until a later lookup
-        // has passed) or gone
-        __atomic_store_n(table + pos, kH32TombWord, __ATOMIC_RELAXED);
-        done = true;
-      } else if (w == kH32EmptyWord) {
-        atomicOr(status, UGK_ST_EVICT_ABSENT);
-        done = true;
-      } else if (++pos == ne) {
-        pos = 0;
+  const int lane = (int)lane_id();
+  const int grp = lane >> 3, sub = lane & 7;
+  const size_t wave = ((size_t)blockIdx.x * kBlock + threadIdx.x) / kWave;
+  const size_t n_waves = (size_t)gridDim.x * (kBlock / kWave);
+  const uint64_t lines = ne >> 4;
+  for (size_t i0 = wave * 8; i0 < n; i0 += n_waves * 8) {  // wavefront-uniform: every ballot below sees all 64 lanes
+    const size_t i = i0 + grp;
+    const bool active = i < n;
+    const uint64_t row = active ? h32_row(t, key_to_u64<K>(keys[i])) : 0;
+    bool done = !active;
+    if (active && row >= kH32Tomb) {  // no entry can hold it
+      if (sub == 0) atomicOr(status, UGK_ST_EVICT_ABSENT);
+      done = true;
+    }
+    const uint32_t r32 = (uint32_t)row;
+    uint64_t win = done ? 0 : h32_home(row, ne), steps = 0;
+    while (__ballot(!done)) {
+      unsigned long long w0 = 0, w1 = 0;  // read as some other key
+      if (!done) {
+        w0 = __atomic_load_n(table + win + 2 * sub, __ATOMIC_RELAXED);
+        w1 = __atomic_load_n(table + win + 2 * sub + 1, __ATOMIC_RELAXED);
+      }
+      const bool m0 = !done && (uint32_t)w0 == r32, m1 = !done && (uint32_t)w1 == r32;
+      const int sh = grp * 8;
+      const uint32_t hit = (uint32_t)(__ballot(m0 || m1) >> sh) & 0xffu;
+      const uint32_t never = (uint32_t)(__ballot(!done && (w0 == kH32EmptyWord || w1 == kH32EmptyWord)) >> sh) & 0xffu;
+      if (!done) {
+        if (hit) {
+          if (m0 || m1) {
+            if (slot_bits) release_slot(slot_bits, nslots, (uint32_t)((m0 ? w0 : w1) >> 32) & 0x0fffffffu, status);
+            // the entry leaves whole: a concurrent lookup sees the key there (its slot keeps the row until a later
+            // lookup has passed) or gone
+            __atomic_store_n(table + win + 2 * sub + (m0 ? 0 : 1), kH32TombWord, __ATOMIC_RELAXED);
+          }
+          done = true;
+        } else if (never || ++steps > lines) {
+          if (sub == 0) atomicOr(status, UGK_ST_EVICT_ABSENT);
+          done = true;
+        } else {
+          win += 16;
+          if (win >= ne) win = 0;
+        }
       }
     }
-    if (!done) atomicOr(status, UGK_ST_EVICT_ABSENT);
   }
 }
 
@@ -416,8 +443,8 @@ int table_evict(ugk_table_t t, const K *keys, size_t n, uint64_t *slot_bits_dev,
     hipLaunchKernelGGL(hash_evict_kernel<K>, dim3(grid), dim3(kBlock), 0, as_stream(stream), (ugk_bucket_t *)t.table,
                        t.size, keys, n, slot_bits, nslots, status);
   else
-    hipLaunchKernelGGL(h32_evict_kernel<K>, dim3(grid), dim3(kBlock), 0, as_stream(stream), t, keys, n, slot_bits,
-                       nslots, status);
+    hipLaunchKernelGGL(h32_evict_kernel<K>, dim3(clamp_grid((n + 31) / 32, 0)), dim3(kBlock), 0, as_stream(stream), t,
+                       keys, n, slot_bits, nslots, status);
   UGK_HIP(hipGetLastError());
   return 0;
 }

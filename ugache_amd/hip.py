@@ -14,6 +14,7 @@ ST_TABLE_FULL = 0x2
 ST_DUP_KEY = 0x4
 ST_EVICT_ABSENT = 0x8
 ST_BAD_SEGMENT = 0x10
+ST_PLACE_PROMISE = 0x20
 ELEM_BF16 = 0x102
 
 LOC_LOCAL = 0
@@ -136,6 +137,7 @@ SIGNATURES = {
     "ugk_record_restore": [_vp, _sz, _vp, _u64, _vp, _vp, _vp],
     "ugk_rank_place": [_vp, _u64, _u64, _vp, _vp, _vp, _vp, C.c_int, _vp],
     "ugk_rank_place_keep": [_vp, _u64, _u64, _vp, _vp, _vp, _vp, _vp, C.c_int, _vp],
+    "ugk_rank_place_observed": [_vp, _u64, _u64, _vp, _vp, _vp, C.c_int, _vp, _vp, _vp, _vp, _vp, _vp],
     "ugk_rank_threshold": [_vp, _vp, _vp],
     "ugk_bitmap_workspace_bytes": [],
     "ugk_bitmap_count": [_vp, _vp, C.c_int, _u64, _vp, _vp, _vp],
