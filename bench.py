@@ -108,7 +108,7 @@ def parse_args():
                     help="mixed workloads: COLL_GPU_RECORD=1 COLL_GPU_REFRESH=1 COLL_GPU_REFRESH_KEEP=1; after the "
                          "timed steps, time steps that each end with a refresh computed on the device from the "
                          "accumulated hotness, with 1 %% of the cache replaced per step")
-    ap.add_argument("--stage-rows", type=int, default=1 << 22,
+    ap.add_argument("--stage-rows", type=int, default=1 << 24,
                     help="with --device-refresh: entries of the set of recently missed rows kept in HBM "
                          "(COLL_MISS_STAGE_ROWS; 0 = none, every inserted row crosses the host link again)")
     ap.add_argument("--serving", action="store_true",

@@ -150,7 +150,8 @@ void CacheContext::build_with_advise_new_hash(int location_id, std::shared_ptr<C
     UGK_CALL(ugk_gather_direct_u32(cpu_data, num_total_nodes, cache_node_list->CPtr<uint32_t>(), num_cached_nodes,
                                    _device_cache_data[_local_location_id], _row_bytes, 0, st->ptr<uint32_t>(),
                                    nullptr, stream));
-    auto table_keys = RunConfig::key_map_mul == 0
+    // (8-byte entries are keyed by the row: no id list)
+    auto table_keys = RunConfig::key_map_mul == 0 || _new_hash_table->_table.kind == 3
                           ? cache_node_list
                           : _new_hash_table->TableKeysToDevice(keys_for_each_source[location_id],
                                                                _eager_gpu_mem_allocator, _trainer_ctx, stream);
@@ -1082,7 +1083,7 @@ void ExtractSession::NoteAsyncStream(StreamHandle stream) {
   _async_any = true;
 }
 
-void ExtractSession::WaitForLookupsInFlight(bool foreground, double timeout_s) {
+void ExtractSession::WaitForLookupsInFlight(bool foreground, double timeout_s, const StreamHandle *ordered_on) {
   if (!foreground) {
     // A lookup counts itself before it reads the table: one that is not counted yet starts after the evictions (or the
     // table swap) have completed.  Blocking lookups stay counted until their output is complete, stream-ordered ones
@@ -1103,7 +1104,8 @@ void ExtractSession::WaitForLookupsInFlight(bool foreground, double timeout_s) {
     std::lock_guard<std::mutex> guard(_async_mu);
     streams = _async_streams;
   }
-  for (StreamHandle s : streams) UGK_CALL(ugk_stream_sync(s));
+  for (StreamHandle s : streams)
+    if (ordered_on == nullptr || s != *ordered_on) UGK_CALL(ugk_stream_sync(s));
 }
 
 void ExtractSession::Wait(StreamHandle stream) {
@@ -1289,9 +1291,9 @@ TensorPtr RefreshSession::CopyTo1DReuse(TensorPtr &preserved_buffer, TensorPtr s
 // cache_context.cu:4045-4052.  The reference waits until `progress` has moved by one (or 20 s have passed); here the
 // session knows which lookups are in flight, on whichever stream, so the wait is for exactly those and an idle cache
 // is not waited for at all.
-void RefreshSession::WaitForOneLookup(ExtractSession *session, bool foreground) {
+void RefreshSession::WaitForOneLookup(ExtractSession *session, bool foreground, const StreamHandle *ordered_on) {
   AnonymousBarrier::_refresh_instance->Wait();
-  if (session) session->WaitForLookupsInFlight(foreground, 20.0);
+  if (session) session->WaitForLookupsInFlight(foreground, 20.0, ordered_on);
 }
 
 void RefreshSession::CopyRowsIntoSlots(const uint32_t *rows_dev, const uint32_t *slots_dev, size_t num_rows,
@@ -1332,6 +1334,8 @@ void RefreshSession::CopyRowsIntoSlots(const uint32_t *rows_dev, const uint32_t 
     else
       UGK_CALL(ugk_gather_scatter_u32(host, ctx->_num_total_nodes, rows_dev, slots_dev, num_rows, cache,
                                       ctx->_cache_space_capacity, ctx->_row_bytes, 128, status, nullptr, copy_stream));
+    // (Publishing beside the copy, on the second stream, instead of behind it was measured at config 5: the step
+    // "row copy + insert" went from 0.245 to 0.318 ms.)
     publish(rows_dev, slots_dev, num_rows);
   } else {
     if (stage) {
@@ -1558,7 +1562,8 @@ void RefreshSession::refresh_on_device(ExtractSession *session, size_t num_cache
   t_phase.Reset();
 
   // Step 5: let one more lookup finish, so that no gather in flight still reads a slot about to be reused
-  WaitForOneLookup(session, foreground);
+  // (a foreground refresh copies on its own stream: lookups enqueued there are in front of the copy as it is)
+  WaitForOneLookup(session, foreground, foreground ? &stream : nullptr);
   const double wait_s = t_phase.Passed();
   t_phase.Reset();
 

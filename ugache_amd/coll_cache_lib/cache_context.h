@@ -304,7 +304,9 @@ class ExtractSession {
   // each stream they went to; the streams must still exist, so call Wait() before destroying one) and, unless
   // `foreground` says that no lookup runs beside the refresh, the blocking ones that had started (bounded by
   // `timeout_s`).  Lookups that start later see the evicted keys as misses and read the host table.
-  void WaitForLookupsInFlight(bool foreground, double timeout_s);
+  // ordered_on (may be null): a stream the caller enqueues everything that follows on; lookups enqueued there are
+  // ordered in front of it already and are not waited for on the host
+  void WaitForLookupsInFlight(bool foreground, double timeout_s, const StreamHandle *ordered_on = nullptr);
   // {0, #local, n} of the last lookup — the reference's group_offset (cache_context.cu:825-847)
   const uint32_t *LastGroupOffset() const { return _group_offset; }
   // moves what the lookups have counted on the device since the last call into `recorder` (FreqRecorder::Record's
@@ -366,7 +368,7 @@ class RefreshSession {
   TensorPtr Empty1DReuse(TensorPtr &preserved_buffer, DataType dtype, std::vector<size_t> shape, Context ctx);
   TensorPtr CopyTo1DReuse(TensorPtr &preserved_buffer, TensorPtr src, Context ctx, StreamHandle stream);
   // step 5: lets one more lookup finish, so that no gather in flight still reads a slot about to be reused
-  void WaitForOneLookup(ExtractSession *session, bool foreground);
+  void WaitForOneLookup(ExtractSession *session, bool foreground, const StreamHandle *ordered_on = nullptr);
   uint32_t _rows_from_stage = 0;  // what status word 8 read after the last refresh on the device
   TensorPtr __rest_rows, __rest_slots;  // rows a background refresh did not find in the stage
  public:

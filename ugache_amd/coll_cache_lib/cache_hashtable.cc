@@ -62,7 +62,8 @@ void CacheEntryManager::CreateHash(const std::function<MemHandle(size_t)> &alloc
 
 TensorPtr CacheEntryManager::TableKeysToDevice(TensorPtr host_rows, const std::function<MemHandle(size_t)> &allocator,
                                                Context ctx, StreamHandle stream) {
-  if (RunConfig::key_map_mul == 0) return Tensor::CopyToExternal(host_rows, allocator, ctx, stream);
+  // (8-byte entries are keyed by the row: the list is the key list)
+  if (RunConfig::key_map_mul == 0 || _table.kind == 3) return Tensor::CopyToExternal(host_rows, allocator, ctx, stream);
   const size_t n = host_rows->NumItem();
   TensorPtr ids = Tensor::Empty(kI64, {n}, CPU_CLIB(), "");
   const IdType *rows = host_rows->CPtr<IdType>();
@@ -78,7 +79,7 @@ void CacheEntryManager::LookupOffset(TensorPtr keys, TensorPtr off, StreamHandle
     UGK_CALL(ugk_table_lookup_i64(_table, keys->CPtr<int64_t>(), keys->NumItem(), (uint32_t)cpu_location_id, nullptr,
                                   off->Ptr<uint32_t>(), stream));
   else
-    UGK_CALL(ugk_table_lookup_u32(_table, keys->CPtr<uint32_t>(), keys->NumItem(), (uint32_t)cpu_location_id, nullptr,
+    UGK_CALL(ugk_table_lookup_u32(RowView(), keys->CPtr<uint32_t>(), keys->NumItem(), (uint32_t)cpu_location_id, nullptr,
                                   off->Ptr<uint32_t>(), stream));
 }
 
@@ -88,7 +89,7 @@ void CacheEntryManager::InsertWithLoc(TensorPtr keys, TensorPtr off, int loc, St
     UGK_CALL(ugk_table_insert_i64(_table, keys->CPtr<int64_t>(), off->CPtr<uint32_t>(), 0, (uint32_t)loc,
                                   keys->NumItem(), StatusPtr(this, stream), stream));
   else
-    UGK_CALL(ugk_table_insert_u32(_table, keys->CPtr<uint32_t>(), off->CPtr<uint32_t>(), 0, (uint32_t)loc,
+    UGK_CALL(ugk_table_insert_u32(RowView(), keys->CPtr<uint32_t>(), off->CPtr<uint32_t>(), 0, (uint32_t)loc,
                                   keys->NumItem(), StatusPtr(this, stream), stream));
 }
 
@@ -97,7 +98,7 @@ void CacheEntryManager::InsertSeqOffWithLoc(TensorPtr keys, int loc, StreamHandl
     UGK_CALL(ugk_table_insert_i64(_table, keys->CPtr<int64_t>(), nullptr, 0, (uint32_t)loc, keys->NumItem(),
                                   StatusPtr(this, stream), stream));
   else
-    UGK_CALL(ugk_table_insert_u32(_table, keys->CPtr<uint32_t>(), nullptr, 0, (uint32_t)loc, keys->NumItem(),
+    UGK_CALL(ugk_table_insert_u32(RowView(), keys->CPtr<uint32_t>(), nullptr, 0, (uint32_t)loc, keys->NumItem(),
                                   StatusPtr(this, stream), stream));
 }
 
@@ -106,7 +107,7 @@ void CacheEntryManager::Evict(TensorPtr keys_to_evict, StreamHandle stream) {
     UGK_CALL(ugk_table_evict_i64(_table, keys_to_evict->CPtr<int64_t>(), keys_to_evict->NumItem(),
                                  StatusPtr(this, stream), stream));
   else
-    UGK_CALL(ugk_table_evict_u32(_table, keys_to_evict->CPtr<uint32_t>(), keys_to_evict->NumItem(),
+    UGK_CALL(ugk_table_evict_u32(RowView(), keys_to_evict->CPtr<uint32_t>(), keys_to_evict->NumItem(),
                                  StatusPtr(this, stream), stream));
   if (_table.kind >= 2) _num_tombstones += keys_to_evict->NumItem();
 }
@@ -116,7 +117,7 @@ void CacheEntryManager::EvictRelease(TensorPtr keys_to_evict, StreamHandle strea
     UGK_CALL(ugk_table_evict_release_i64(_table, keys_to_evict->CPtr<int64_t>(), keys_to_evict->NumItem(),
                                          SlotUsedBits(), _cache_space_capacity, StatusPtr(this, stream), stream));
   else
-    UGK_CALL(ugk_table_evict_release_u32(_table, keys_to_evict->CPtr<uint32_t>(), keys_to_evict->NumItem(),
+    UGK_CALL(ugk_table_evict_release_u32(RowView(), keys_to_evict->CPtr<uint32_t>(), keys_to_evict->NumItem(),
                                          SlotUsedBits(), _cache_space_capacity, StatusPtr(this, stream), stream));
   if (_table.kind >= 2) _num_tombstones += keys_to_evict->NumItem();
 }
@@ -154,12 +155,14 @@ bool CacheEntryManager::MaybeRebuild(const std::function<MemHandle(size_t)> &all
   ugk_table_t fresh = _table;
   fresh.table = Align128(fresh_handle->ptr());
   UGK_CALL(ugk_table_init(fresh, stream));
+  ugk_table_t fresh_rows = fresh;  // as 32-bit row numbers address it (RowView)
+  if (fresh_rows.kind == 3) fresh_rows.fb_mul = fresh_rows.fb_mask = 0;
   if (n > 0) {
     if (keys->Type() == kI64)
       UGK_CALL(ugk_table_insert_i64(fresh, keys->CPtr<int64_t>(), offs->CPtr<uint32_t>(), 0, (uint32_t)loc, n,
                                     StatusPtr(this, stream), stream));
     else
-      UGK_CALL(ugk_table_insert_u32(fresh, keys->CPtr<uint32_t>(), offs->CPtr<uint32_t>(), 0, (uint32_t)loc, n,
+      UGK_CALL(ugk_table_insert_u32(fresh_rows, keys->CPtr<uint32_t>(), offs->CPtr<uint32_t>(), 0, (uint32_t)loc, n,
                                     StatusPtr(this, stream), stream));
   }
   CheckStatus(stream, "table rebuild");  // waits for the stream: the new table is complete
@@ -227,7 +230,7 @@ TensorPtr CacheEntryManager::EmitBits(const uint64_t *a, const uint64_t *b, bool
 TensorPtr CacheEntryManager::RowsToTableKeys(TensorPtr rows_dev, TensorPtr &buffer,
                                              const std::function<MemHandle(size_t)> &allocator, Context ctx,
                                              StreamHandle stream) {
-  if (RunConfig::key_map_mul == 0) return rows_dev;
+  if (RunConfig::key_map_mul == 0 || _table.kind == 3) return rows_dev;  // 8-byte entries are keyed by the row
   const size_t n = rows_dev->NumItem();
   TensorPtr ids = ReuseList(buffer, kI64, n, allocator, ctx);
   UGK_CALL(ugk_rows_to_keys(rows_dev->CPtr<uint32_t>(), n, RunConfig::key_map_mul, RunConfig::key_map_mask,
@@ -239,8 +242,8 @@ void CacheEntryManager::PublishRows(const uint32_t *rows_dev, const uint32_t *sl
                                     TensorPtr &id_buffer, const std::function<MemHandle(size_t)> &allocator,
                                     Context ctx, StreamHandle stream) {
   if (n == 0) return;
-  if (RunConfig::key_map_mul == 0) {
-    UGK_CALL(ugk_table_insert_u32(_table, rows_dev, slots_dev, 0, (uint32_t)loc, n, StatusPtr(this, stream), stream));
+  if (RunConfig::key_map_mul == 0 || _table.kind == 3) {
+    UGK_CALL(ugk_table_insert_u32(RowView(), rows_dev, slots_dev, 0, (uint32_t)loc, n, StatusPtr(this, stream), stream));
     return;
   }
   TensorPtr ids = ReuseList(id_buffer, kI64, n, allocator, ctx);

@@ -113,6 +113,13 @@ class CacheEntryManager {
   uint64_t *InNewBits() const { return _dev_in_new->ptr<uint64_t>(); }
   uint64_t *SlotUsedBits() const { return _dev_slot_used->ptr<uint64_t>(); }
   uint32_t *DevWords() const { return _dev_words->ptr<uint32_t>(); }
+  // the table as 32-bit row numbers address it: a compact table stores its keys by the row, so with sparse ids the
+  // lists of rows a refresh works on need no translation into ids
+  ugk_table_t RowView() const {
+    ugk_table_t t = _table;
+    if (t.kind == 3) t.fb_mul = t.fb_mask = 0;
+    return t;
+  }
   // bitmaps from the host lists (allocates them on first use)
   void EnsureDeviceLists(const std::function<MemHandle(size_t)> &allocator, Context ctx, StreamHandle stream);
   // host lists from the bitmaps: cached rows ascending, free slots ascending

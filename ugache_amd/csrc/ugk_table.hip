@@ -316,10 +316,35 @@ __global__ __launch_bounds__(kBlock) void h32_evict_kernel(ugk_table_t t, const 
       const int sh = grp * 8;
       const uint32_t hit = (uint32_t)(__ballot(m0 || m1) >> sh) & 0xffu;
       const uint32_t never = (uint32_t)(__ballot(!done && (w0 == kH32EmptyWord || w1 == kH32EmptyWord)) >> sh) & 0xffu;
+      // The slots of the keys found in this step leave the slot bitmap.  Neighbouring keys of an evict list often hold
+      // neighbouring slots (a refresh evicts runs of rows that went in together), whose bits share a word: the lanes
+      // of the wavefront that hold a found entry merge their bits per word first, one atomic per word.
+      const bool mine = !done && (m0 || m1);
+      if (slot_bits) {
+        const uint32_t slot = (uint32_t)((m0 ? w0 : w1) >> 32) & 0x0fffffffu;
+        bool todo = mine;
+        if (mine && slot >= nslots) {
+          atomicOr(status, UGK_ST_KEY_OUT_OF_RANGE);
+          todo = false;
+        }
+        unsigned long long left = __ballot(todo);
+        while (left) {  // wavefront-uniform: at most eight lanes hold an entry
+          const int lead = __ffsll(left) - 1;
+          const uint32_t word = __shfl(slot >> 6, lead);
+          const bool same = todo && (slot >> 6) == word;
+          const unsigned long long group = __ballot(same);
+          unsigned long long bits = 0;
+          for (unsigned long long g = group; g; g &= g - 1) {
+            const int l = __ffsll(g) - 1;
+            bits |= 1ull << (__shfl(slot, l) & 63u);
+          }
+          if (lane == lead) atomicAnd(slot_bits + word, ~bits);
+          left &= ~group;
+        }
+      }
       if (!done) {
         if (hit) {
-          if (m0 || m1) {
-            if (slot_bits) release_slot(slot_bits, nslots, (uint32_t)((m0 ? w0 : w1) >> 32) & 0x0fffffffu, status);
+          if (mine) {
             // the entry leaves whole: a concurrent lookup sees the key there (its slot keeps the row until a later
             // lookup has passed) or gone
             __atomic_store_n(table + win + 2 * sub + (m0 ? 0 : 1), kH32TombWord, __ATOMIC_RELAXED);
