@@ -476,7 +476,8 @@ int ugk_record_restore(const uint64_t *entries_dev, size_t n, uint32_t *counts_d
  * observed at the last placement plus the keys counted since stay below k), 0 < k < num_rows: in_new = every observed
  * row and the lowest k - |observed| never-observed rows, what ugk_rank_place computes in that case, in five launches
  * over the bitmaps and none over the counters.  If k or more rows turn out to be observed, UGK_ST_PLACE_PROMISE is set
- * in *status_dev and in_new_dev is left as it was.  cached_dev (may be NULL; then evict_ws_dev, insert_ws_dev and
+ * in *status_dev and in_new_dev is left as it was.  counts_dev may be NULL when reset_counts is 0 (only the bitmap is
+ * read then: "observed" can be any set of rows that are in for sure).  cached_dev (may be NULL; then evict_ws_dev, insert_ws_dev and
  * totals_host may be NULL too): the rows cached now; the rows that leave (cached & ~in_new) and that come in
  * (in_new & ~cached) are counted in the same pass: evict_ws_dev / insert_ws_dev (ugk_bitmap_workspace_bytes() each)
  * are left as ugk_bitmap_count(cached, in_new) / ugk_bitmap_count(in_new, cached) would leave them, ready for

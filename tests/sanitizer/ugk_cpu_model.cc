@@ -1319,7 +1319,8 @@ int ugk_rank_place_keep(uint32_t *counts, uint64_t num_rows, uint64_t k, void *w
 int ugk_rank_place_observed(uint32_t *counts, uint64_t num_rows, uint64_t k, void *ws, uint64_t *in_new,
                             uint64_t *observed, int reset_counts, const uint64_t *cached, void *evict_ws,
                             void *insert_ws, uint32_t *totals_host, uint32_t *status, void *) {
-  REQUIRE(counts && ws && in_new && observed && status, "ugk_rank_place_observed: null pointer");
+  REQUIRE(ws && in_new && observed && status, "ugk_rank_place_observed: null pointer");
+  REQUIRE(counts || !reset_counts, "ugk_rank_place_observed: counters to reset, but no counters");
   REQUIRE(num_rows > 0 && num_rows < 0xffffffffull, "ugk_rank_place_observed: rows do not fit 32 bits");
   REQUIRE(k > 0 && k < num_rows, "ugk_rank_place_observed: k outside (0, rows)");
   REQUIRE(in_new != observed && cached != in_new, "ugk_rank_place_observed: output bitmap is an input bitmap");

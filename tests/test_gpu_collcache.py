@@ -44,7 +44,7 @@ def _fresh_cache(monkeypatch):
     for v in ("COLL_HASH_TABLE", "COLL_RECORD_INLINE_BYTES", "SAMGRAPH_COLL_CACHE_CONCURRENT_LINK_IMPL", "SAMGRAPH_COLL_CACHE_NO_GROUP",
               "COLL_DEDUP_KEYS", "COLL_DEDUP_MIN_KEYS", "COLL_GPU_RECORD", "COLL_GPU_RECORD_EVERY", "COLL_GPU_REFRESH",
               "COLL_GPU_REFRESH_KEEP", "COLL_GPU_REFRESH_STABLE", "COLL_REFRESH_RATE_GBPS",
-              "COLL_GPU_RECORD_SEED"):
+              "COLL_GPU_RECORD_SEED", "COLL_DEVICE_KEY_LIST"):
         monkeypatch.delenv(v, raising=False)
     yield
     if torch.cuda.is_available():
@@ -191,6 +191,91 @@ def test_partial_cache_matches_oracle(table_kind, impl, kdtype, monkeypatch):
         assert _basics.last_group_offset(0) == [0, n_local, n]
     step = _basics.info(0)["lookups"] - 1
     assert _basics.step_value(step, kLogL1MissBytes) == (n - n_local) * dim * 4
+
+
+@pytest.mark.parametrize("key_list", ["device", "host"])
+@pytest.mark.parametrize("table_kind,sparse", [("FLAT", False), ("HASH", False), ("HASH", True), ("HASH16", True)])
+@pytest.mark.parametrize("pct", [0.003, 0.1, 0.7])
+def test_key_list_of_a_build_made_on_the_device_or_on_the_host(key_list, table_kind, sparse, pct, monkeypatch):
+    """The ascending list of cached rows comes from a bitmap on the device (the default) or from the key -> block
+    array on the host (COLL_DEVICE_KEY_LIST=0): the same cached set either way, the oracle's, with fewer rows observed
+    than the cache holds (0.7: the lowest never-observed rows fill it up), with more (0.003, 0.1: the best-ranked
+    ones), and a refresh through the host afterwards starts from the right list."""
+    monkeypatch.setenv("COLL_HASH_TABLE", table_kind)
+    monkeypatch.setenv("COLL_DEVICE_KEY_LIST", "1" if key_list == "device" else "0")
+    rng = np.random.default_rng(int(pct * 1000) + len(table_kind))
+    n_item, dim = 70_003, 32
+    MUL, BITS = 0x9E3779B97F4A7C15, 40
+
+    def ids_of(rows):
+        if not sparse:
+            return torch.from_numpy(rows.astype(np.int64))
+        return torch.from_numpy(((rows.astype(np.uint64) * np.uint64(MUL)) & np.uint64((1 << BITS) - 1)).astype(np.int64))
+
+    co.config(make_config(n_item, pct))
+    if sparse:
+        _basics.set_key_map(MUL, BITS)
+    co.coll_cache_record_init(0)
+    perm = rng.permutation(n_item)
+    s0 = perm[zipf_ranks(rng, 60_000, n_item, 1.05)]
+    co.coll_torch_record(0, ids_of(s0))
+    emb = co.coll_torch_create_emb_shm(0, n_item, dim, torch.float32)
+    table = fill_table(emb, rng)
+    co.coll_torch_init_t(0, 0, emb, pct)
+
+    def check(stream_u32):
+        want, nid = expected_cached_set(stream_u32, n_item, pct)
+        got = np.zeros(len(want), np.uint32)
+        assert _basics.C_LIB_CTYPES.coll_cache_get_cached_keys(0, got.ctypes.data, len(got)) == len(want)
+        assert np.array_equal(got, want)
+        rows = rng.integers(0, n_item, size=20_001)
+        out = co.coll_torch_lookup_key_t_val_ret(0, ids_of(rows).cuda(), False)
+        assert out.cpu().numpy().tobytes() == ORC.gather(table, rows).tobytes()
+        assert _basics.last_group_offset(0)[1] == int((nid[rows] == 0).sum())
+
+    observed = len(np.unique(s0))
+    assert (observed > int(n_item * pct)) == (pct < 0.5)  # both sides of "more observed than cached" are covered
+    check(s0.astype(np.uint32))
+    s1 = perm[::-1][zipf_ranks(rng, 60_000, n_item, 1.05)]  # the other end of the table turns hot
+    co.coll_torch_record(0, ids_of(s1))
+    co.coll_torch_refresh(0, True)
+    check(s1.astype(np.uint32))
+
+
+@pytest.mark.parametrize("key_list", ["device", "host"])
+@pytest.mark.parametrize("table_kind", ["FLAT", "HASH"])
+def test_build_from_an_explicit_rank_list(key_list, table_kind, monkeypatch):
+    """coll_cache_init_ranked_c (the build_v2 overload with a rank list and a frequency list over all keys,
+    facade.h:56-60): the first K keys of the list are the cached set, whatever order they come in"""
+    from collcache.torch import c_lib  # the module `co` wraps: one _State
+    monkeypatch.setenv("COLL_HASH_TABLE", table_kind)
+    monkeypatch.setenv("COLL_DEVICE_KEY_LIST", "1" if key_list == "device" else "0")
+    rng = np.random.default_rng(31)
+    n_item, dim, pct = 40_001, 16, 0.25
+    co.config(make_config(n_item, pct))
+    rank_keys = rng.permutation(n_item).astype(np.uint32)
+    rank_freq = np.sort(rng.integers(0, 1000, size=n_item).astype(np.uint32))[::-1].copy()
+    emb = co.coll_torch_create_emb_shm(0, n_item, dim, torch.float32)
+    table = fill_table(emb, rng)
+    torch.cuda.set_device(0)
+    c_lib._State.dev_id[0] = 0
+    alloc, release = c_lib._make_allocator(0)
+    c_lib._setup_dims(dim, False)
+    _basics.C_LIB_CTYPES.coll_cache_init_ranked_c(0, n_item, rank_keys.ctypes.data, rank_freq.ctypes.data, alloc, release,
+                                                  None, emb.data_ptr(), c_lib.kF32, dim, float(pct),
+                                                  c_lib._stream_handle(0))
+    c_lib._State.host_tables.append(emb)
+    k = int(n_item * (pct * 100 / 100.0))
+    want = np.sort(rank_keys[:k])
+    nid, nc = ORC.rep_solve(rank_keys, n_item, pct * 100)
+    assert nc == k and np.array_equal(np.nonzero(nid == 0)[0].astype(np.uint32), want)
+    got = np.zeros(k, np.uint32)
+    assert _basics.C_LIB_CTYPES.coll_cache_get_cached_keys(0, got.ctypes.data, k) == k
+    assert np.array_equal(got, want)
+    keys = rng.integers(0, n_item, size=30_000)
+    out = co.coll_torch_lookup_key_t_val_ret(0, torch.from_numpy(keys).cuda(), False)
+    assert out.cpu().numpy().tobytes() == ORC.gather(table, keys).tobytes()
+    assert _basics.last_group_offset(0) == [0, int((nid[keys] == 0).sum()), len(keys)]
 
 
 @pytest.mark.parametrize("pct", [0.0, 0.1, 1.0])
@@ -1039,7 +1124,7 @@ def _random_case(seed):
                 table_kind=str(r.choice(["FLAT", "HASH", "HASH16"])), impl=str(r.choice(["", "SMMaskPhase", "NONE"])),
                 i64=bool(r.integers(0, 2)), dedup=bool(r.integers(0, 4) == 0), gpu_record=bool(r.integers(0, 4) == 0),
                 zipf=float(r.choice([0.6, 1.05, 1.4])), half=bool(r.integers(0, 3) == 0),
-                stage=int(r.choice([0, 0, 1024])))
+                stage=int(r.choice([0, 0, 1024])), host_list=bool(seed % 3 == 0))
 
 
 # UGACHE_TEST_SEEDS widens the two seeded sweeps of this file for an occasional longer run
@@ -1061,6 +1146,8 @@ def test_random_configurations_are_exact(case, monkeypatch):
         monkeypatch.setenv("COLL_GPU_RECORD", "1")
     if case["stage"]:
         monkeypatch.setenv("COLL_MISS_STAGE_ROWS", str(case["stage"]))
+    if case["host_list"]:  # the key -> block array and its scans on the host, instead of the bitmap on the device
+        monkeypatch.setenv("COLL_DEVICE_KEY_LIST", "0")
     rng = np.random.default_rng(case["seed"])
     n_item, dim, pct = case["n_item"], case["dim"], case["pct"]
     kdtype = torch.int64 if case["i64"] else torch.int32
@@ -1170,7 +1257,7 @@ def _random_refresh_case(seed):
                 pct=float(r.choice([0.01, 0.1, 0.37, 0.9, 0.99])), table_kind=str(r.choice(["FLAT", "HASH", "HASH16"])),
                 keep=bool(r.integers(0, 2)), sparse=bool(r.integers(0, 3) == 0), zipf=float(r.choice([0.6, 1.05, 1.4])),
                 rounds=int(r.integers(2, 5)), stream_ordered=bool(r.integers(0, 3) == 0),
-                stage=int(r.choice([0, 256, 65536])), stable=bool(r.integers(0, 3) == 0))
+                stage=int(r.choice([0, 256, 65536])), stable=bool(r.integers(0, 3) == 0), host_list=bool(seed % 3 == 1))
 
 
 @pytest.mark.parametrize("case", [_random_refresh_case(i) for i in range(max(24, _SEEDS // 2))],
@@ -1191,6 +1278,8 @@ def test_random_sequences_of_refreshes_on_the_device(case, monkeypatch):
         monkeypatch.setenv("COLL_GPU_REFRESH_KEEP", "1")
     if case["stable"]:
         monkeypatch.setenv("COLL_GPU_REFRESH_STABLE", "1")
+    if case["host_list"]:
+        monkeypatch.setenv("COLL_DEVICE_KEY_LIST", "0")
     rng = np.random.default_rng(case["seed"])
     n_item, dim, pct = case["n_item"], case["dim"], case["pct"]
     MUL, BITS = 0x9E3779B97F4A7C15, 40

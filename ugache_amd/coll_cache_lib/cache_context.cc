@@ -71,6 +71,50 @@ void CacheContext::build_full_cache(int location_id, std::shared_ptr<CollCache> 
   std::cout << "test_result:init:cache_nbytes=" << _cache_nbytes << "\n";
 }
 
+// the ascending list of the rows a placement caches, made on the device: bit r of a bitmap over the key space = row r
+// is cached (the ranked rows that are cached, then the lowest `num_extra` rows that are not among them), compacted in
+// order.  Waits for `stream`: the list is complete on return.
+TensorPtr CacheContext::KeyListOnDevice(TensorPtr top_rows, size_t num_extra, size_t num_rows, StreamHandle stream) {
+  CHECK_NOTNULL(top_rows);
+  const size_t num_top = top_rows->NumItem(), num_cached = num_top + num_extra;
+  CHECK_LT(num_cached, num_rows);
+  if (num_cached == 0) return Tensor::EmptyExternal(kI32, {0}, _eager_gpu_mem_allocator, _trainer_ctx, "");
+  const size_t words = (num_rows + 63) / 64;
+  MemHandle ranked = _eager_gpu_mem_allocator(words * 8), placed = num_extra ? _eager_gpu_mem_allocator(words * 8) : nullptr;
+  MemHandle bm_ws = _eager_gpu_mem_allocator(ugk_bitmap_workspace_bytes());
+  MemHandle rank_ws = num_extra ? _eager_gpu_mem_allocator(ugk_rank_workspace_bytes()) : nullptr;
+  MemHandle st = _eager_gpu_mem_allocator(256);
+  MemHandle total = PinnedHostAlloc(64);
+  UGK_CALL(ugk_fill_u32(ranked->ptr<uint32_t>(), 0, words * 2, stream));
+  UGK_CALL(ugk_fill_u32(st->ptr<uint32_t>(), 0, 1, stream));
+  if (num_top > 0) {
+    TensorPtr top_dev = Tensor::CopyToExternal(top_rows, _eager_gpu_mem_allocator, _trainer_ctx, stream);
+    UGK_CALL(ugk_bitmap_update(ranked->ptr<uint64_t>(), num_rows, top_dev->CPtr<uint32_t>(), num_top, 1,
+                               st->ptr<uint32_t>(), stream));
+    UGK_CALL(ugk_stream_sync(stream));  // top_dev goes out of scope
+  }
+  const uint64_t *cached = ranked->ptr<uint64_t>();
+  if (num_extra > 0) {
+    // every ranked row is cached and the lowest rows that were not ranked fill the rest: the placement of a cache that
+    // is larger than the set of observed rows
+    UGK_CALL(ugk_rank_place_observed(nullptr, num_rows, num_cached, rank_ws->ptr(), placed->ptr<uint64_t>(),
+                                     ranked->ptr<uint64_t>(), 0, nullptr, nullptr, nullptr, nullptr,
+                                     st->ptr<uint32_t>(), stream));
+    cached = placed->ptr<uint64_t>();
+  }
+  UGK_CALL(ugk_bitmap_count(cached, nullptr, 0, num_rows, bm_ws->ptr(), total->ptr<uint32_t>(), stream));
+  uint32_t status = 0;
+  UGK_CALL(ugk_memcpy_async(&status, st->ptr(), sizeof(status), stream));
+  UGK_CALL(ugk_stream_sync(stream));
+  CHECK_EQ(status, 0u) << "key list on the device: a ranked key is outside the key space (1) or the ranked keys are "
+                          "not distinct (0x20)";
+  CHECK_EQ((size_t)*total->ptr<uint32_t>(), num_cached) << "key list on the device: the ranked keys are not distinct";
+  TensorPtr list = Tensor::EmptyExternal(kI32, {num_cached}, _eager_gpu_mem_allocator, _trainer_ctx, "");
+  UGK_CALL(ugk_bitmap_emit(cached, nullptr, 0, num_rows, bm_ws->ptr(), list->Ptr<uint32_t>(), num_cached, stream));
+  UGK_CALL(ugk_stream_sync(stream));  // the bitmaps go out of scope
+  return list;
+}
+
 // cache_context.cu:2414-2599 — partial cache: frequency-ranked fill + lookup table
 void CacheContext::build_with_advise_new_hash(int location_id, std::shared_ptr<CollCache> coll_cache_ptr,
                                               void *cpu_data, DataType dtype, size_t dim, Context gpu_ctx,
@@ -82,10 +126,18 @@ void CacheContext::build_with_advise_new_hash(int location_id, std::shared_ptr<C
   CHECK_EQ(_cpu_location_id, kCpuLoc);
   CHECK_EQ(location_id, kLocalLoc);
   _local_location_id = location_id;
-  CHECK_NOTNULL(coll_cache_ptr->_nid_to_block);
+  CHECK(coll_cache_ptr->HasPartialPlacement());
   CHECK_NOTNULL(coll_cache_ptr->_block_access_advise);
   CHECK_NOTNULL(coll_cache_ptr->_block_density);
-  const size_t num_total_nodes = coll_cache_ptr->_nid_to_block->Shape()[0];
+  // The solver may have left the key -> block array unwritten and handed over what it placed from (the ranked keys
+  // that are cached + how many never-observed keys fill the rest): then the ascending list of cached rows is made on
+  // the device, from a bitmap of the key space, and no pass over per-key arrays of the whole key space runs on the
+  // host.  Bitmap positions are 32-bit.
+  if (coll_cache_ptr->_nid_to_block == nullptr && coll_cache_ptr->_placed_num_node >= 0xffffffffu)
+    coll_cache_ptr->EnsureNidToBlock();
+  const bool list_on_device = coll_cache_ptr->_nid_to_block == nullptr;
+  const size_t num_total_nodes =
+      list_on_device ? (size_t)coll_cache_ptr->_placed_num_node : coll_cache_ptr->_nid_to_block->Shape()[0];
   _num_total_nodes = num_total_nodes;
   Timer t;
 
@@ -100,10 +152,17 @@ void CacheContext::build_with_advise_new_hash(int location_id, std::shared_ptr<C
   TensorPtr advise_line = Tensor::FromBlob(
       coll_cache_ptr->_block_access_advise->Ptr<uint8_t>() + (size_t)location_id * num_block, kU8, {num_block},
       CPU_CLIB(), "advise_line");
-  CacheEntryManager::DetectKeysForAllSource(coll_cache_ptr->_nid_to_block, advise_line, location_id,
-                                            coll_cache_ptr->_block_density, num_total_nodes, keys_for_each_source,
-                                            (int)RunConfig::num_device);
-  const size_t num_cached_nodes = keys_for_each_source[location_id]->NumItem();
+  TensorPtr cache_node_list;  // on the device, ascending
+  if (list_on_device) {
+    cache_node_list = KeyListOnDevice(coll_cache_ptr->_placed_top_rows, coll_cache_ptr->_placed_extra,
+                                      num_total_nodes, stream);
+  } else {
+    CacheEntryManager::DetectKeysForAllSource(coll_cache_ptr->_nid_to_block, advise_line, location_id,
+                                              coll_cache_ptr->_block_density, num_total_nodes, keys_for_each_source,
+                                              (int)RunConfig::num_device);
+  }
+  const size_t num_cached_nodes =
+      list_on_device ? cache_node_list->NumItem() : keys_for_each_source[location_id]->NumItem();
   const double detect_s = t.Passed();
   _new_hash_table->_remote_keys = Tensor::Empty(kI32, {0}, CPU_CLIB(), "");
   const size_t num_cpu_nodes = num_total_nodes - num_cached_nodes;
@@ -141,21 +200,37 @@ void CacheContext::build_with_advise_new_hash(int location_id, std::shared_ptr<C
   }
 
   const double alloc_s = t.Passed() - detect_s;
-  // 4. fill: rows of the cached keys host -> HBM in list order, slot = position in the list
+  // 4. fill: rows of the cached keys host -> HBM in list order, slot = position in the list.  The copy is bound by
+  //    the host link; the host's copy of a list that was made on the device comes back beside it, on a second stream.
+  //    (The table insert beside the copy as well, instead of behind it, was measured at 500M rows / 50M cached: the
+  //    step went from 0.140 to 0.178 s, the link-bound copy kernel loses more than the insert takes.)
+  if (list_on_device) keys_for_each_source[location_id] = Tensor::Empty(kI32, {num_cached_nodes}, CPU_CLIB(), "");
   if (num_cached_nodes > 0) {
-    auto cache_node_list = Tensor::CopyToExternal(keys_for_each_source[location_id], _eager_gpu_mem_allocator,
-                                                  _trainer_ctx, stream);
+    if (!list_on_device)
+      cache_node_list = Tensor::CopyToExternal(keys_for_each_source[location_id], _eager_gpu_mem_allocator,
+                                               _trainer_ctx, stream);
     MemHandle st = _eager_gpu_mem_allocator(256);
     UGK_CALL(ugk_fill_u32(st->ptr<uint32_t>(), 0, 1, stream));
     UGK_CALL(ugk_gather_direct_u32(cpu_data, num_total_nodes, cache_node_list->CPtr<uint32_t>(), num_cached_nodes,
                                    _device_cache_data[_local_location_id], _row_bytes, 0, st->ptr<uint32_t>(),
                                    nullptr, stream));
     // (8-byte entries are keyed by the row: no id list)
-    auto table_keys = RunConfig::key_map_mul == 0 || _new_hash_table->_table.kind == 3
-                          ? cache_node_list
+    TensorPtr id_buffer;
+    auto table_keys = RunConfig::key_map_mul == 0 || _new_hash_table->_table.kind == 3 ? cache_node_list
+                      : list_on_device
+                          ? _new_hash_table->RowsToTableKeys(cache_node_list, id_buffer, _eager_gpu_mem_allocator,
+                                                             _trainer_ctx, stream)
                           : _new_hash_table->TableKeysToDevice(keys_for_each_source[location_id],
                                                                _eager_gpu_mem_allocator, _trainer_ctx, stream);
     _new_hash_table->InsertSeqOffWithLoc(table_keys, location_id, stream);
+    if (list_on_device) {  // what a refresh through the host compares the next placement with
+      StreamHandle beside = nullptr;
+      UGK_CALL(ugk_stream_create(&beside));
+      UGK_CALL(ugk_memcpy_async(keys_for_each_source[location_id]->MutableData(), cache_node_list->Data(),
+                                num_cached_nodes * sizeof(IdType), beside));
+      UGK_CALL(ugk_stream_sync(beside));
+      UGK_CALL(ugk_stream_destroy(beside));
+    }
     uint32_t fill_status = 0;
     UGK_CALL(ugk_memcpy_async(&fill_status, st->ptr(), sizeof(fill_status), stream));
     UGK_CALL(ugk_stream_sync(stream));

@@ -85,9 +85,28 @@ void CheckPolicy() {
 }
 }  // namespace
 
+void CollCache::take_solution(coll_cache::FreqRankSolver &solver, IdType num_node) {
+  _block_placement = solver.block_placement;
+  _block_access_advise = solver.block_access_from;
+  _block_density = solver.block_density_tensor;
+  _placed_top_rows = solver.defer_nid_to_block ? solver.top_rows : nullptr;
+  _placed_extra = solver.defer_nid_to_block ? solver.num_extra : 0;
+  _placed_num_node = num_node;
+}
+
+TensorPtr CollCache::EnsureNidToBlock() {
+  if (_nid_to_block == nullptr && _placed_top_rows != nullptr) {
+    _nid_to_block = Tensor::Empty(kI32, {(size_t)_placed_num_node}, CPU_CLIB(), "nid_to_block");
+    coll_cache::FreqRankSolver::Materialize(_placed_top_rows->CPtr<IdType>(), _placed_top_rows->NumItem(),
+                                            _placed_extra, _placed_num_node, _nid_to_block->Ptr<IdType>());
+    _placed_top_rows = nullptr;
+  }
+  return _nid_to_block;
+}
+
 // facade.cc:93-160
 void CollCache::solve_impl_master(IdType *ranking_nodes_list_ptr, IdType *ranking_nodes_freq_list_ptr,
-                                  IdType num_node) {
+                                  IdType num_node, bool defer) {
   CheckPolicy();
   std::vector<int> trainer_to_stream(RunConfig::num_device, 0);
   std::vector<coll_cache::PerT> trainer_cache_percent(RunConfig::num_device, RunConfig::cache_percentage * 100);
@@ -96,28 +115,26 @@ void CollCache::solve_impl_master(IdType *ranking_nodes_list_ptr, IdType *rankin
   auto ranking_nodes_freq_list = Tensor::FromBlob(ranking_nodes_freq_list_ptr, kI32, {1, (size_t)num_node},
                                                   CPU(CPU_FOREIGN), "ranking_nodes_freq_list");
   coll_cache::FreqRankSolver solver;
-  _nid_to_block = Tensor::Empty(kI32, {(size_t)num_node}, CPU_CLIB(), "nid_to_block");
+  solver.defer_nid_to_block = defer;
+  _nid_to_block = defer ? nullptr : Tensor::Empty(kI32, {(size_t)num_node}, CPU_CLIB(), "nid_to_block");
   solver.Build(ranking_nodes_list, ranking_nodes_freq_list, trainer_to_stream, num_node, _nid_to_block);
   solver.Solve(trainer_to_stream, trainer_cache_percent, "BIN", RunConfig::coll_cache_hyperparam_T_local,
                RunConfig::coll_cache_hyperparam_T_cpu);
-  _block_placement = solver.block_placement;
-  _block_access_advise = solver.block_access_from;
-  _block_density = solver.block_density_tensor;
+  take_solution(solver, num_node);
 }
 
 // facade.cc:161-236
-void CollCache::solve_impl_master(ContFreqBuf *freq_rank, IdType num_node) {
+void CollCache::solve_impl_master(ContFreqBuf *freq_rank, IdType num_node, bool defer) {
   CheckPolicy();
   std::vector<int> trainer_to_stream(RunConfig::num_device, 0);
   std::vector<coll_cache::PerT> trainer_cache_percent(RunConfig::num_device, RunConfig::cache_percentage * 100);
   coll_cache::FreqRankSolver solver;
-  _nid_to_block = Tensor::Empty(kI32, {(size_t)num_node}, CPU_CLIB(), "nid_to_block");
+  solver.defer_nid_to_block = defer;
+  _nid_to_block = defer ? nullptr : Tensor::Empty(kI32, {(size_t)num_node}, CPU_CLIB(), "nid_to_block");
   solver.BuildSingleStream(freq_rank, trainer_to_stream, num_node, _nid_to_block);
   solver.Solve(trainer_to_stream, trainer_cache_percent, "BIN", RunConfig::coll_cache_hyperparam_T_local,
                RunConfig::coll_cache_hyperparam_T_cpu);
-  _block_placement = solver.block_placement;
-  _block_access_advise = solver.block_access_from;
-  _block_density = solver.block_density_tensor;
+  take_solution(solver, num_node);
 }
 
 void CollCache::build_common(int replica_id, std::function<void()> solve, IdType num_node,
@@ -175,8 +192,9 @@ void CollCache::build_common(int replica_id, std::function<void()> solve, IdType
 void CollCache::build(std::function<std::function<MemHandle(size_t)>(int)> allocator_builder, void *cpu_data,
                       DataType dtype, size_t dim, double cache_percentage, StreamHandle stream) {
   const bool partial = cache_percentage != 0 && cache_percentage != 1;
-  CHECK(!partial || (_nid_to_block != nullptr && _block_access_advise != nullptr))
+  CHECK(!partial || (HasPartialPlacement() && _block_access_advise != nullptr))
       << "CollCache::build places nothing itself: a partial cache needs the placement of an earlier build_v2 / refresh";
+  if (partial) EnsureNidToBlock();
   const IdType num_node = partial ? (IdType)_nid_to_block->Shape()[0] : (IdType)RunConfig::num_total_item;
   for (size_t replica_id = 0; replica_id < RunConfig::num_device; replica_id++)
     build_common((int)replica_id, []() {}, num_node, allocator_builder((int)replica_id), cpu_data, dtype, dim,
@@ -189,7 +207,8 @@ void CollCache::build_v2(int replica_id, IdType *ranking_nodes_list_ptr, IdType 
                          DataType dtype, size_t dim, double cache_percentage, StreamHandle stream) {
   build_common(
       replica_id,
-      [&]() { solve_impl_master(ranking_nodes_list_ptr, ranking_nodes_freq_list_ptr, num_node); }, num_node,
+      [&]() { solve_impl_master(ranking_nodes_list_ptr, ranking_nodes_freq_list_ptr, num_node, RunConfig::device_key_list); },
+      num_node,
       gpu_mem_allocator, cpu_data, dtype, dim, cache_percentage, stream);
 }
 
@@ -198,8 +217,8 @@ void CollCache::build_v2(int replica_id, ContFreqBuf *freq_rank, IdType num_node
                          std::function<MemHandle(size_t)> gpu_mem_allocator, void *cpu_data, DataType dtype,
                          size_t dim, double cache_percentage, StreamHandle stream) {
   build_common(
-      replica_id, [&]() { solve_impl_master(freq_rank, num_node); }, num_node, gpu_mem_allocator, cpu_data, dtype,
-      dim, cache_percentage, stream);
+      replica_id, [&]() { solve_impl_master(freq_rank, num_node, RunConfig::device_key_list); }, num_node,
+      gpu_mem_allocator, cpu_data, dtype, dim, cache_percentage, stream);
 }
 
 void CollCache::preserve_old_solution() {
@@ -211,13 +230,14 @@ void CollCache::preserve_old_solution() {
   this->_block_density = nullptr;
   this->_block_placement = nullptr;
   this->_nid_to_block = nullptr;
+  this->_placed_top_rows = nullptr;
 }
 
 // facade.cc:383-428
 void CollCache::refresh(int replica_id, IdType *ranking_nodes_list_ptr, IdType *ranking_nodes_freq_list_ptr,
                         StreamHandle stream, bool foreground) {
   CHECK_EQ(replica_id, 0);
-  CHECK_NOTNULL(_nid_to_block) << "refresh needs a cache built with 0 < cache_percentage < 1";
+  CHECK(HasPartialPlacement()) << "refresh needs a cache built with 0 < cache_percentage < 1";
   AnonymousBarrier::_refresh_instance->Wait();
   preserve_old_solution();
   solve_impl_master(ranking_nodes_list_ptr, ranking_nodes_freq_list_ptr, (IdType)RunConfig::num_total_item);
@@ -230,7 +250,7 @@ void CollCache::refresh(int replica_id, IdType *ranking_nodes_list_ptr, IdType *
 // facade.cc:513-557
 void CollCache::refresh(int replica_id, ContFreqBuf *freq_rank, StreamHandle stream, bool foreground) {
   CHECK_EQ(replica_id, 0);
-  CHECK_NOTNULL(_nid_to_block) << "refresh needs a cache built with 0 < cache_percentage < 1";
+  CHECK(HasPartialPlacement()) << "refresh needs a cache built with 0 < cache_percentage < 1";
   AnonymousBarrier::_refresh_instance->Wait();
   Timer t_solve;
   preserve_old_solution();
@@ -246,7 +266,7 @@ void CollCache::refresh(int replica_id, ContFreqBuf *freq_rank, StreamHandle str
 
 void CollCache::refresh_on_device(int replica_id, StreamHandle stream, bool foreground) {
   CHECK_EQ(replica_id, 0);
-  CHECK_NOTNULL(_nid_to_block) << "refresh needs a cache built with 0 < cache_percentage < 1";
+  CHECK(HasPartialPlacement()) << "refresh needs a cache built with 0 < cache_percentage < 1";
   CheckPolicy();
   AnonymousBarrier::_refresh_instance->Wait();
   Timer t_apply;

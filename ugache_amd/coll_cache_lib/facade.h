@@ -9,6 +9,7 @@
 #include "cache_context.h"
 #include "common.h"
 #include "freq_recorder.h"
+#include "placement.h"
 #include "profiler.h"
 
 namespace coll_cache_lib {
@@ -33,8 +34,18 @@ class CollCache : public std::enable_shared_from_this<CollCache> {
   std::vector<std::shared_ptr<CacheContext>> _cache_ctx_list;
   std::vector<std::shared_ptr<ExtractSession>> _session_list;
   std::vector<std::shared_ptr<RefreshSession>> _refresh_session_list;
-  void solve_impl_master(IdType *ranking_nodes_list_ptr, IdType *ranking_nodes_freq_list_ptr, IdType num_node);
-  void solve_impl_master(ContFreqBuf *freq_rank, IdType num_node);
+  // defer: the key -> block array is left unwritten and the placement kept as _placed_top_rows / _placed_extra
+  // (FreqRankSolver::defer_nid_to_block): the build that follows makes its key list on the device from them
+  void solve_impl_master(IdType *ranking_nodes_list_ptr, IdType *ranking_nodes_freq_list_ptr, IdType num_node,
+                         bool defer = false);
+  void solve_impl_master(ContFreqBuf *freq_rank, IdType num_node, bool defer = false);
+  void take_solution(coll_cache::FreqRankSolver &solver, IdType num_node);
+  TensorPtr _placed_top_rows;  // set while _nid_to_block is deferred
+  size_t _placed_extra = 0;
+  IdType _placed_num_node = 0;
+  // the key -> block array of the placement in force, written out on first use when the solver deferred it
+  TensorPtr EnsureNidToBlock();
+  bool HasPartialPlacement() const { return _nid_to_block != nullptr || _placed_top_rows != nullptr; }
   void preserve_old_solution();
   void build_common(int replica_id, std::function<void()> solve, IdType num_node,
                     std::function<MemHandle(size_t)> gpu_mem_allocator, void *cpu_data, DataType dtype, size_t dim,
@@ -138,7 +149,7 @@ class CollCache : public std::enable_shared_from_this<CollCache> {
   }
   void lookup_wait(int replica_id, StreamHandle stream) { _session_list.at(replica_id)->Wait(stream); }
   std::shared_ptr<ExtractSession> session(int replica_id) { return _session_list.at(replica_id); }
-  TensorPtr nid_to_block() { return _nid_to_block; }
+  TensorPtr nid_to_block() { return EnsureNidToBlock(); }
 };
 
 }  // namespace coll_cache_lib

@@ -42,6 +42,18 @@ void ContFreqBuf::sort_desc() {
   buf = entries.data();
 }
 
+void ContFreqBuf::select_top(size_t k) {
+  // every rank word is distinct (the key sits in its low half), so the k best entries are one set
+  uint64_t *w = reinterpret_cast<uint64_t *>(entries.data());
+  if (k == 0 || k >= entries.size()) return;
+#ifdef _OPENMP
+  __gnu_parallel::nth_element(w, w + k, w + entries.size(), std::greater<uint64_t>());
+#else
+  std::nth_element(w, w + k, w + entries.size(), std::greater<uint64_t>());
+#endif
+  buf = entries.data();
+}
+
 void ContFreqBuf::GetLegacyFreqRank(LegacyFreqBuf *output, size_t total_num_node) const {
   output->rank_vec.resize(total_num_node);
   output->freq_vec.assign(total_num_node, 0);
@@ -189,6 +201,32 @@ void FreqRecorder::LocalCombineToShared() {
   }
   CntT *shared = _shared;
   const size_t n = _num_nodes;
+  if (!_shared_dirty && _direct.empty()) {
+    // Nothing waits in the shared array: the counted keys leave the drained array as entries at once, in one pass
+    // over it instead of three over arrays of the whole key space (add into the shared array, count its non-zero
+    // keys, list them).  Ascending key order whatever the thread count, as GlobalCombine lists them.
+    const int nthr = ScanThreads();
+    const size_t chunk = (n + nthr - 1) / nthr;
+    std::vector<std::vector<FreqEntry>> part(nthr);
+#pragma omp parallel for num_threads(nthr) schedule(static, 1)
+    for (int t = 0; t < nthr; t++) {
+      const size_t lo = std::min(n, chunk * t), hi = std::min(n, chunk * (t + 1));
+      auto &mine = part[t];
+      for (size_t k = lo; k < hi; k++)
+        if (drained[k]) {
+          mine.push_back({(IdType)k, drained[k]});
+          drained[k] = 0;
+        }
+    }
+    std::vector<size_t> first(nthr + 1, 0);
+    for (int t = 0; t < nthr; t++) first[t + 1] = first[t] + part[t].size();
+    _direct.resize(first[nthr]);
+#pragma omp parallel for num_threads(nthr) schedule(static, 1)
+    for (int t = 0; t < nthr; t++)
+      if (!part[t].empty()) memcpy(_direct.data() + first[t], part[t].data(), part[t].size() * sizeof(FreqEntry));
+    return;
+  }
+  if (!_direct.empty()) ScatterHandedOver(_direct, shared);  // an earlier round still waits as a list: both add up
   _shared_dirty = true;
 #pragma omp parallel for num_threads(ScanThreads())
   for (size_t i = 0; i < n; i++) {
@@ -208,6 +246,17 @@ void FreqRecorder::GlobalCombine() {
   }
   auto &e = global_cont_freq_buf->entries;
   e.clear();
+  if (!_direct.empty()) {
+    if (!_shared_dirty && handed_over.empty()) {  // what LocalCombineToShared listed is the list
+      e.swap(_direct);
+      _direct.clear();
+      global_cont_freq_buf->buf = e.data();
+      LOG(INFO) << "freq recorder global combine: " << e.size() << " distinct keys";
+      return;
+    }
+    ScatterHandedOver(_direct, _shared);  // keys may repeat across the lists: they add up in the array
+    _shared_dirty = true;
+  }
   if (!_shared_dirty) {
     // only handed-over entries (distinct keys): they are the list, whatever their order — Sort() follows
     const size_t n_nodes = _num_nodes;
@@ -246,6 +295,8 @@ void FreqRecorder::GlobalCombine() {
   global_cont_freq_buf->buf = e.data();
   LOG(INFO) << "freq recorder global combine: " << e.size() << " distinct keys";
 }
+
+void FreqRecorder::SelectTop(size_t k) { global_cont_freq_buf->select_top(k); }
 
 void FreqRecorder::Sort() {
   global_cont_freq_buf->sort_desc();

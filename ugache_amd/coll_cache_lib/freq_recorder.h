@@ -39,6 +39,9 @@ struct ContFreqBuf {
   // (the reference appends them in a thread-dependent order, freq_recorder.cc:305-333)
   void GetLegacyFreqRank(LegacyFreqBuf *output, size_t total_num_node) const;
   void sort_desc();
+  // the k best-ranked entries in front (in no particular order), the rest behind them: what a placement of k keys
+  // needs of the order, in linear time; k >= size() leaves the list as it is
+  void select_top(size_t k);
 };
 
 class FreqRecorder {
@@ -56,12 +59,13 @@ class FreqRecorder {
   void LocalCombineToShared();
   void GlobalCombine();
   void Sort();
+  void SelectTop(size_t k);
   inline size_t NumNodes() const { return _num_nodes; }
   // true when counts wait here for the next ranking (recorded on the host, or handed over from the device)
   bool HasCounts() {
     std::lock_guard<std::mutex> combine(_combine_mu);
     std::lock_guard<std::mutex> g(_mu);
-    return _live_dirty || _shared_dirty || !_handed_over.empty();
+    return _live_dirty || _shared_dirty || !_handed_over.empty() || !_direct.empty();
   }
   ContFreqBuf *global_cont_freq_buf;
 
@@ -74,6 +78,8 @@ class FreqRecorder {
   CntT *_shared = nullptr;  // counts handed over by LocalCombineToShared
   bool _live_dirty = false, _shared_dirty = false;  // the array holds a non-zero counter
   std::vector<FreqEntry> _handed_over;              // entries of the open hand-over, not in the arrays
+  std::vector<FreqEntry> _direct;                   // what LocalCombineToShared listed straight from the counters
+                                                    // (ascending, distinct keys), not in the shared array
   void ScatterHandedOver(std::vector<FreqEntry> &list, CntT *into);
   // _mu guards what recording touches (_live, _live_dirty, _handed_over) and is held for one batch at most;
   // _combine_mu guards the rest (_spare, _shared, _shared_dirty, the ranked list) for the length of a scan of the

@@ -102,7 +102,9 @@ void coll_cache_config_from_map(std::unordered_map<std::string, std::string> &co
 // prefixes that stream-ordered serving steps have copied out and not counted yet (defined with the serving loop)
 void CountPendingPrefixes(bool all);
 
-ContFreqBuf *CombineAndRank(int replica_id) {
+// top_k: SIZE_MAX for the full rank order; else the placement that follows caches top_k keys and needs only to know
+// which entries are the top_k best (FreqRankSolver reads the list as "the first top_k entries are cached")
+ContFreqBuf *CombineAndRank(int replica_id, size_t top_k = SIZE_MAX) {
   CHECK_LT((size_t)replica_id, _freq_recorder.size()) << "coll_cache_record_init was not called";
   CHECK_NOTNULL(_freq_recorder[replica_id]);
   CountPendingPrefixes(/*all=*/true);
@@ -116,7 +118,8 @@ ContFreqBuf *CombineAndRank(int replica_id) {
   ContFreqBuf *freq_rank = nullptr;
   if (replica_id == 0) {
     _freq_recorder[0]->GlobalCombine();
-    _freq_recorder[0]->Sort();
+    if (top_k == SIZE_MAX) _freq_recorder[0]->Sort();
+    else _freq_recorder[0]->SelectTop(top_k);
     freq_rank = _freq_recorder[0]->global_cont_freq_buf;
   }
   return freq_rank;
@@ -143,7 +146,9 @@ void coll_cache_init(int replica_id, size_t key_space_size, std::function<MemHan
   ContFreqBuf *freq_rank = nullptr;
   const bool need_rank = cache_percentage != 0 && cache_percentage != 1;
   Timer t_rank;
-  if (need_rank) freq_rank = CombineAndRank(replica_id);
+  if (need_rank)
+    freq_rank = CombineAndRank(
+        replica_id, coll_cache::FreqRankSolver::NumCachedNodes((IdType)key_space_size, cache_percentage * 100));
   LOG(INFO) << "build: ranking " << t_rank.Passed() << " s";
   Timer t_build;
   _coll_cache->build_v2(replica_id, freq_rank, (IdType)key_space_size, allocator, cpu_data, dtype, dim,
@@ -375,7 +380,9 @@ void coll_cache_refresh(int replica_id, StreamHandle stream, int foreground) {
     if (_profiler) _profiler->SetRefreshDuration(t_rank.Passed());
     return;
   }
-  ContFreqBuf *freq_rank = CombineAndRank(replica_id);
+  ContFreqBuf *freq_rank = CombineAndRank(
+      replica_id, coll_cache::FreqRankSolver::NumCachedNodes((IdType)RunConfig::num_total_item,
+                                                             RunConfig::cache_percentage * 100));
   LOG(INFO) << "refresh: ranking " << t_rank.Passed() << " s";
   _coll_cache->refresh(replica_id, freq_rank, stream, foreground != 0);
   if (_profiler) _profiler->SetRefreshDuration(t_rank.Passed());

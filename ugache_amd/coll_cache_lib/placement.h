@@ -47,6 +47,17 @@ class FreqRankSolver : public CollCacheSolver {
   // how many of num_node keys a cache of `percent` % holds (optimal_solver_class.cc:1878)
   static IdType NumCachedNodes(IdType num_node, PerT percent) { return (IdType)(num_node * (percent / (double)100)); }
 
+  // Set before Solve: the key -> block array (4 bytes per key of the key space) is not written.  The placement is
+  // described by what it was computed from instead: top_rows, the cached keys that were ranked (observed entries, or
+  // the head of a full rank list), and num_extra, how many never-observed keys, lowest first, fill the rest of the
+  // cache.  A build on one GPU turns that into its key list on the device (CacheContext::build), and Materialize
+  // writes the array out for whoever still wants it.
+  bool defer_nid_to_block = false;
+  TensorPtr top_rows;  // u32 [n], distinct keys
+  size_t num_extra = 0;
+  static void Materialize(const IdType *top_rows, size_t num_top, size_t num_extra, IdType num_node,
+                          IdType *nid_to_block);
+
  private:
   TensorPtr _rank_keys;  // u32 [num_node]   (Build)
   TensorPtr _rank_freq;  // u32 [num_node]   (Build)

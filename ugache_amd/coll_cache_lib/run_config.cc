@@ -33,6 +33,7 @@ double RunConfig::coll_cache_hyperparam_T_cpu = 8000.0 / 50.0;
 coll_cache::AsymmLinkDesc RunConfig::coll_cache_link_desc;
 double RunConfig::hash_load_factor = 0.7;
 int RunConfig::force_table_kind = 0;
+bool RunConfig::device_key_list = true;
 size_t RunConfig::refresh_batch_rows = 4092;
 unsigned RunConfig::refresh_sleep_us = 3000;
 unsigned RunConfig::refresh_limit_block = 20;
@@ -77,6 +78,7 @@ void RunConfig::LoadConfigFromEnv() {
   coll_cache_scale_nb = 16;
   hash_load_factor = 0.7;
   force_table_kind = 0;
+  device_key_list = true;
   refresh_batch_rows = 4092;
   refresh_sleep_us = 3000;
   refresh_limit_block = 20;
@@ -115,6 +117,7 @@ void RunConfig::LoadConfigFromEnv() {
   }
   if (GetEnv("COLL_CACHE_SCALE") != "") coll_cache_scale_nb = std::stoul(GetEnv("COLL_CACHE_SCALE"));
   if (GetEnv("COLL_HASH_LOAD_FACTOR") != "") hash_load_factor = std::stod(GetEnv("COLL_HASH_LOAD_FACTOR"));
+  if (GetEnv("COLL_DEVICE_KEY_LIST") != "") device_key_list = GetEnv("COLL_DEVICE_KEY_LIST") != "0";
   const std::string tbl = GetEnv("COLL_HASH_TABLE");
   if (tbl == "FLAT") force_table_kind = 1;
   else if (tbl == "HASH") force_table_kind = 2;

@@ -723,7 +723,8 @@ int ugk_rank_place_keep(uint32_t *counts_dev, uint64_t num_rows, uint64_t k, voi
 int ugk_rank_place_observed(uint32_t *counts_dev, uint64_t num_rows, uint64_t k, void *ws_dev, uint64_t *in_new_dev,
                             uint64_t *observed_dev, int reset_counts, const uint64_t *cached_dev, void *evict_ws_dev,
                             void *insert_ws_dev, uint32_t *totals_host, uint32_t *status_dev, void *stream) {
-  UGK_REQUIRE(counts_dev && ws_dev && in_new_dev && observed_dev && status_dev, "ugk_rank_place_observed: null pointer");
+  UGK_REQUIRE(ws_dev && in_new_dev && observed_dev && status_dev, "ugk_rank_place_observed: null pointer");
+  UGK_REQUIRE(counts_dev || !reset_counts, "ugk_rank_place_observed: counters to reset, but no counters");
   UGK_REQUIRE(num_rows > 0 && num_rows < 0xffffffffull, "ugk_rank_place_observed: %llu rows do not fit 32 bits",
               (unsigned long long)num_rows);
   UGK_REQUIRE(k > 0 && k < num_rows, "ugk_rank_place_observed: k = %llu is not inside (0, %llu)",
