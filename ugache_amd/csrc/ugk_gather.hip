@@ -147,6 +147,7 @@ __global__ __launch_bounds__(kBlock) void replicate_kernel(V *out, uint32_t vpr,
   }
 }
 
+constexpr int kStagedUnroll = 4;  // rows a lane group keeps in flight in gather_staged_kernel
 // Rows out of the host table, or out of the stage where it holds them (refresh inserts: most of the rows a refresh
 // brings in were missed by the last few lookups and are filed there).  Lanes per row chosen at run time: this runs at
 // refresh time, on some hundred thousand rows.
@@ -158,7 +159,7 @@ __global__ __launch_bounds__(kBlock) void gather_staged_kernel(const u32x4 *__re
                                                                uint32_t *staged, uint32_t *rest_rows,
                                                                uint32_t *rest_dst, uint32_t *rest_count,
                                                                uint32_t *done_count) {
-  constexpr int UNROLL = 2;
+  constexpr int UNROLL = kStagedUnroll;
   __shared__ uint32_t block_staged;
   if (threadIdx.x == 0) block_staged = 0;
   __syncthreads();
@@ -403,7 +404,7 @@ int ugk_gather_scatter_staged_u32(const void *host_dev, uint64_t host_rows, cons
   const uint32_t vpr = (uint32_t)(row_bytes / 16);
   uint32_t lpr = 1;
   while (lpr < vpr && lpr < 64) lpr <<= 1;
-  const size_t per_iter = (size_t)(kBlock / lpr) * 2;
+  const size_t per_iter = (size_t)(kBlock / lpr) * kStagedUnroll;
   const unsigned grid = clamp_grid((n + per_iter - 1) / per_iter, max_blocks);
   hipLaunchKernelGGL(gather_staged_kernel, dim3(grid), dim3(kBlock), 0, as_stream(stream),
                      reinterpret_cast<const u32x4 *>(host_dev), host_rows, rows_dev, dst_off_dev, n,
