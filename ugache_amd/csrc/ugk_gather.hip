@@ -147,7 +147,7 @@ __global__ __launch_bounds__(kBlock) void replicate_kernel(V *out, uint32_t vpr,
   }
 }
 
-constexpr int kStagedUnroll = 4;  // rows a lane group keeps in flight in gather_staged_kernel
+constexpr int kStagedUnroll = 8;  // rows a lane group keeps in flight in gather_staged_kernel
 // Rows out of the host table, or out of the stage where it holds them (refresh inserts: most of the rows a refresh
 // brings in were missed by the last few lookups and are filed there).  Lanes per row chosen at run time: this runs at
 // refresh time, on some hundred thousand rows.
