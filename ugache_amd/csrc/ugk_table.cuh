@@ -239,7 +239,7 @@ __device__ __forceinline__ uint64_t h32_home(uint64_t row, uint64_t nentries) {
 }
 
 // bit i of `even` to bit 2i, bit i of `odd` to bit 2i + 1: the sixteen entries of a line in their order, from the two
-// per-lane predicates of an 8-lane group
+// per-lane predicates of an 8-lane group (what the insert orders tombstones and never-used entries by)
 __device__ __forceinline__ uint32_t h32_interleave(uint32_t even, uint32_t odd) {
   auto spread = [](uint32_t b) {
     b = (b | (b << 4)) & 0x0f0fu;
@@ -255,20 +255,22 @@ struct H32Line {
 };
 
 // what one 128-byte line says about `row`: every lane of the 8-lane group passes the 16 bytes it read (entries
-// 2 * sub and 2 * sub + 1); act is group-uniform.  All 64 lanes call it.
+// 2 * sub and 2 * sub + 1); act is group-uniform.  All 64 lanes call it.  No order among the entries is needed:
+// every probe sequence enters a line at its first entry, inserts take the first reusable entry and evictions leave
+// tombstones, so the never-used entries of a line are its tail and a live key sits in front of them — a line that
+// holds the key settles the lookup, one without it but with a never-used entry ends it.
+// (Measured at 262,144 keys / 99 % hits: 51.6 us against 53.0 us with the entries' order worked out from four ballots;
+// a probe that also sends the home line's number instead of its address and lets the key's lane fetch the value
+// straight from the lane that holds the entry, three permutes per round instead of seven: 53.5 us.)
 __device__ __forceinline__ H32Line h32_examine(const u32x4 &raw, uint32_t row, bool act, int grp) {
-  const uint32_t m = h32_interleave((uint32_t)(__ballot(act && raw.x == row) >> (grp * 8)),
-                                    (uint32_t)(__ballot(act && raw.z == row) >> (grp * 8)));
-  const uint32_t e = h32_interleave((uint32_t)(__ballot(act && raw.x == kH32Empty) >> (grp * 8)),
-                                    (uint32_t)(__ballot(act && raw.z == kH32Empty) >> (grp * 8)));
-  const int fm = m ? (__ffs(m) - 1) : 16;
-  const int fe = e ? (__ffs(e) - 1) : 16;
+  const bool first = act && raw.x == row, second = act && raw.z == row;
+  const uint32_t m = (uint32_t)(__ballot(first || second) >> (grp * 8)) & 0xffu;
+  const uint32_t e = (uint32_t)(__ballot(act && (raw.x == kH32Empty || raw.z == kH32Empty)) >> (grp * 8)) & 0xffu;
   H32Line r;
-  r.found = fm < fe;  // a key sits in front of the first never-used entry of its probe sequence
-  r.done = r.found || fe < 16;
-  const int hit_lane = grp * 8 + (r.found ? (fm >> 1) : 0);
-  const uint32_t vy = __shfl(raw.y, hit_lane), vw = __shfl(raw.w, hit_lane);
-  r.val = (fm & 1) ? vw : vy;
+  r.found = m != 0;
+  r.done = r.found || e != 0;
+  const uint32_t mine = first ? raw.y : raw.w;
+  r.val = __shfl(mine, grp * 8 + (m ? __ffs(m) - 1 : 0));
   return r;
 }
 

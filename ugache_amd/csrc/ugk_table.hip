@@ -429,7 +429,8 @@ int check_table(const ugk_table_t &t, const char *who) {
     UGK_REQUIRE((uintptr_t)t.table % 128 == 0, "%s: hash table must be 128-byte aligned", who);
   }
   if (t.kind == 3) {
-    UGK_REQUIRE(t.size % 16 == 0, "%s: compact hash table needs a multiple of 16 entries, got %llu", who,
+    UGK_REQUIRE(t.size % 16 == 0 && (t.size >> 4) <= 0xffffffffull,
+                "%s: compact hash table needs a multiple of 16 entries and at most 2^32 lines, got %llu", who,
                 (unsigned long long)t.size);
     UGK_REQUIRE((uintptr_t)t.table % 128 == 0, "%s: hash table must be 128-byte aligned", who);
   }
