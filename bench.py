@@ -38,8 +38,8 @@ HBM_PEAK_GBPS = 8000.0  # MI355X published HBM3E bandwidth
 MEASURED_TRAFFIC_BYTES = {"c2_all_hit_10Mx128xfp32_262144_u32_uniform": 270_530_000,
                           # fused kernel; includes the 126 MB of rows that reach the L2 over the host link
                           "c3_gnn_100Mx128xfp32_1M_i64_zipf0.9_cache25pct": 1_137_700_000,
-                          # fused kernel over the hash table (profiles/extract_mix_kernel_mixed_c1_c3_c4_c5.md)
-                          "c5_hash_500Mx64xfp16_1M_i64_zipf1.05_cache50M": 311_000_000}
+                          # fused kernel over the compact hash table (profiles/extract_mix_kernel_mixed_c1_c3_c4_c5.md)
+                          "c5_hash_500Mx64xfp16_1M_i64_zipf1.05_cache50M": 301_400_000}
 
 ALL_HIT = {
     # name: (rows, dim, keys per batch)

@@ -107,6 +107,7 @@ def probe_kpw(hip, torch, note, quick=False):
                 hip.call("ugk_hash_init", base, nb, stream)
                 tb = hip.table(hip.TABLE_HASH, base, nb)
             cached = torch.arange(ncache, dtype=torch.int64, device="cuda")
+            torch.cuda.synchronize()  # torch made the key list on its own stream; the insert reads it on this one
             hip.call("ugk_table_insert_i64", tb, cached.data_ptr(), None, 0, hip.LOC_LOCAL, ncache, st.data_ptr(), stream)
             cache = torch.randint(0, 2 ** 31 - 1, (ncache, rb // 4), dtype=torch.int32, device="cuda")
             host = _pinned(hip, rows * rb)
@@ -134,7 +135,7 @@ def probe_kpw(hip, torch, note, quick=False):
             _check_status(torch, st, "kpw")
             hip.call("ugk_host_free", host)
             del cache, mem, cached
-            torch.cuda.empty_cache()  # every case allocates afresh: a table in recycled blocks has timed up to 1.7x slower
+            torch.cuda.empty_cache()
     if saved is None:
         os.environ.pop("UGK_MIX_KPW", None)
     else:
