@@ -201,10 +201,9 @@ void CacheContext::build_with_advise_new_hash(int location_id, std::shared_ptr<C
 
   const double alloc_s = t.Passed() - detect_s;
   // 4. fill: rows of the cached keys host -> HBM in list order, slot = position in the list.  The copy is bound by
-  //    the host link; the host's copy of a list that was made on the device comes back beside it, on a second stream.
-  //    (The table insert beside the copy as well, instead of behind it, was measured at 500M rows / 50M cached: the
-  //    step went from 0.140 to 0.178 s, the link-bound copy kernel loses more than the insert takes.)
-  if (list_on_device) keys_for_each_source[location_id] = Tensor::Empty(kI32, {num_cached_nodes}, CPU_CLIB(), "");
+  //    the host link.  (The table insert beside the copy, on a second stream, instead of behind it, was measured at
+  //    500M rows / 50M cached: the step went from 0.140 to 0.178 s, the link-bound copy kernel loses more than the
+  //    insert takes.)
   if (num_cached_nodes > 0) {
     if (!list_on_device)
       cache_node_list = Tensor::CopyToExternal(keys_for_each_source[location_id], _eager_gpu_mem_allocator,
@@ -223,14 +222,6 @@ void CacheContext::build_with_advise_new_hash(int location_id, std::shared_ptr<C
                           : _new_hash_table->TableKeysToDevice(keys_for_each_source[location_id],
                                                                _eager_gpu_mem_allocator, _trainer_ctx, stream);
     _new_hash_table->InsertSeqOffWithLoc(table_keys, location_id, stream);
-    if (list_on_device) {  // what a refresh through the host compares the next placement with
-      StreamHandle beside = nullptr;
-      UGK_CALL(ugk_stream_create(&beside));
-      UGK_CALL(ugk_memcpy_async(keys_for_each_source[location_id]->MutableData(), cache_node_list->Data(),
-                                num_cached_nodes * sizeof(IdType), beside));
-      UGK_CALL(ugk_stream_sync(beside));
-      UGK_CALL(ugk_stream_destroy(beside));
-    }
     uint32_t fill_status = 0;
     UGK_CALL(ugk_memcpy_async(&fill_status, st->ptr(), sizeof(fill_status), stream));
     UGK_CALL(ugk_stream_sync(stream));
@@ -241,7 +232,9 @@ void CacheContext::build_with_advise_new_hash(int location_id, std::shared_ptr<C
   const double fill_s = t.Passed() - detect_s - alloc_s;
 
   // 5. bookkeeping for refresh: cached key list and free slots [n_cached, capacity) (cache_context.cu:2577-2585)
-  _new_hash_table->_cached_keys = keys_for_each_source[location_id];
+  // (a list made on the device stays there until the host asks for it: CacheEntryManager::HostCachedKeys)
+  if (list_on_device) _new_hash_table->_cached_keys_on_device = cache_node_list;
+  else _new_hash_table->_cached_keys = keys_for_each_source[location_id];
   _new_hash_table->_cache_space_capacity = (IdType)_cache_space_capacity;
   _new_hash_table->cpu_location_id = _cpu_location_id;
   _new_hash_table->num_total_key = num_total_nodes;
@@ -1507,6 +1500,7 @@ void RefreshSession::refresh_after_solve_new(bool foreground) {
   // (DetectKeysWithCond over the other placement's nid_to_block in the reference, cache_context.cu:3975-4003).
   // Both lists are ascending (DetectKeysForAllSource), so the two differences are merges.
   const IdType *new_keys = key_list_of_each_src[local]->CPtr<IdType>();
+  table->HostCachedKeys(stream);
   const IdType *old_keys = table->_cached_keys->CPtr<IdType>();
   const size_t num_old_local_key = table->_cached_keys->NumItem();
   TensorPtr new_insert_keys = CacheEntryManager::SortedDifference(new_keys, num_new_local_key, old_keys, num_old_local_key);
@@ -1559,6 +1553,7 @@ void RefreshSession::refresh_after_solve_new(bool foreground) {
   insert_s = t_phase.Passed();
   t_phase.Reset();
   table->_cached_keys = key_list_of_each_src[local];
+  table->_cached_keys_on_device = nullptr;
   table->_dev_lists_valid = false;  // the host lists hold the truth now
   ctx->_cache_nodes = num_new_local_key;
   const bool rebuilt = table->MaybeRebuild(ctx->_eager_gpu_mem_allocator, gpu_ctx, local, stream, [&]() {
@@ -1683,6 +1678,7 @@ void RefreshSession::refresh_on_device(ExtractSession *session, size_t num_cache
   table->_num_cached = num_preserved_key + num_insert;
   table->_num_free = capacity - table->_num_cached;
   table->_host_lists_valid = false;  // the bitmaps hold the truth now
+  table->_cached_keys_on_device = nullptr;
   ctx->_cache_nodes = table->_num_cached;
   const bool rebuilt = table->MaybeRebuild(alloc, gpu_ctx, local, stream, [&]() {
     session->WaitForLookupsInFlight(foreground, 20.0);

@@ -60,6 +60,20 @@ void CacheEntryManager::CreateHash(const std::function<MemHandle(size_t)> &alloc
   RunConfig::use_flat_hashtable = false;
 }
 
+TensorPtr CacheEntryManager::HostCachedKeys(StreamHandle stream) {
+  if (_cached_keys_on_device) {
+    const size_t n = _cached_keys_on_device->NumItem();
+    _cached_keys = Tensor::Empty(kI32, {n}, CPU_CLIB(), "cached_keys");
+    if (n) {
+      UGK_CALL(ugk_set_device(_device_id));
+      UGK_CALL(ugk_memcpy_async(_cached_keys->MutableData(), _cached_keys_on_device->Data(), n * sizeof(IdType), stream));
+      UGK_CALL(ugk_stream_sync(stream));
+    }
+    _cached_keys_on_device = nullptr;
+  }
+  return _cached_keys;
+}
+
 TensorPtr CacheEntryManager::TableKeysToDevice(TensorPtr host_rows, const std::function<MemHandle(size_t)> &allocator,
                                                Context ctx, StreamHandle stream) {
   // (8-byte entries are keyed by the row: the list is the key list)
@@ -142,8 +156,13 @@ bool CacheEntryManager::MaybeRebuild(const std::function<MemHandle(size_t)> &all
                                  ctx, stream, &n);
     keys = RowsToTableKeys(rows, key_buffer, allocator, ctx, stream);
   } else {
-    n = _cached_keys->NumItem();
-    keys = TableKeysToDevice(_cached_keys, allocator, ctx, stream);
+    if (_cached_keys_on_device) {  // the list of the build is still on the device
+      n = _cached_keys_on_device->NumItem();
+      keys = RowsToTableKeys(_cached_keys_on_device, key_buffer, allocator, ctx, stream);
+    } else {
+      n = _cached_keys->NumItem();
+      keys = TableKeysToDevice(_cached_keys, allocator, ctx, stream);
+    }
   }
   LOG(INFO) << "rebuilding the lookup table: " << _num_tombstones << " tombstones in " << _table.size << " entries, "
             << n << " live keys";
@@ -270,11 +289,14 @@ void CacheEntryManager::EnsureDeviceLists(const std::function<MemHandle(size_t)>
   CHECK(_host_lists_valid);
   UGK_CALL(ugk_fill_u32(_dev_in_cache->ptr<uint32_t>(), 0, row_words * 2, stream));
   UGK_CALL(ugk_fill_u32(_dev_slot_used->ptr<uint32_t>(), 0, std::max<size_t>(slot_words, 1) * 2, stream));
-  const size_t n = _cached_keys->NumItem();
+  const size_t n = NumCached();
   if (n > 0) {
-    TensorPtr rows = ReuseList(_dev_list_buffer, kI32, n, allocator, ctx);
-    UGK_CALL(ugk_memcpy_async(rows->MutableData(), _cached_keys->Data(), n * sizeof(IdType), stream));
-    UGK_CALL(ugk_stream_sync(stream));  // the source is pageable host memory
+    TensorPtr rows = _cached_keys_on_device;  // the list of the build, if it is still on the device
+    if (!rows) {
+      rows = ReuseList(_dev_list_buffer, kI32, n, allocator, ctx);
+      UGK_CALL(ugk_memcpy_async(rows->MutableData(), _cached_keys->Data(), n * sizeof(IdType), stream));
+      UGK_CALL(ugk_stream_sync(stream));  // the source is pageable host memory
+    }
     uint32_t *status = StatusPtr(this, stream);
     UGK_CALL(ugk_bitmap_update(InCacheBits(), num_total_key, rows->CPtr<uint32_t>(), n, 1, status, stream));
     TensorPtr key_buffer;
@@ -292,7 +314,11 @@ void CacheEntryManager::EnsureDeviceLists(const std::function<MemHandle(size_t)>
 
 void CacheEntryManager::EnsureHostLists(const std::function<MemHandle(size_t)> &allocator, Context ctx,
                                         StreamHandle stream) {
-  if (_host_lists_valid) return;
+  if (_host_lists_valid) {
+    HostCachedKeys(stream);
+    return;
+  }
+  _cached_keys_on_device = nullptr;  // superseded by what the bitmaps say
   CHECK(_dev_lists_valid);
   UGK_CALL(ugk_set_device(_device_id));
   size_t n_cached = 0, n_free = 0;

@@ -36,6 +36,11 @@ inline size_t TableSize(const size_t num, const size_t scale = 2) {
 class CacheEntryManager {
  public:
   TensorPtr _cached_keys;   // host, u32: keys currently cached on this GPU
+  // A build that made its key list on the device leaves the list there; the host's copy is fetched when something asks
+  // for it (a refresh through the host, a table rebuild from the host's list, coll_cache_get_cached_keys).  While it
+  // waits here _cached_keys is null and _host_lists_valid stays true: the list is the host's, just not copied yet.
+  TensorPtr _cached_keys_on_device;
+  TensorPtr HostCachedKeys(StreamHandle stream);
   TensorPtr _remote_keys;   // always empty with one GPU
   TensorPtr _free_offsets;  // host, u32: free cache slots, allocation sized for the whole capacity
   ugk_table_t _table = {0, 0, nullptr, 0, 0, 0};
@@ -107,7 +112,11 @@ class CacheEntryManager {
   bool _dev_lists_valid = false;
   bool _host_lists_valid = true;
   size_t _num_cached = 0, _num_free = 0;  // valid when the host lists are not
-  size_t NumCached() const { return _host_lists_valid ? (_cached_keys ? _cached_keys->NumItem() : 0) : _num_cached; }
+  size_t NumCached() const {
+    if (!_host_lists_valid) return _num_cached;
+    if (_cached_keys_on_device) return _cached_keys_on_device->NumItem();
+    return _cached_keys ? _cached_keys->NumItem() : 0;
+  }
   size_t NumFree() const { return _host_lists_valid ? (_free_offsets ? _free_offsets->NumItem() : 0) : _num_free; }
   uint64_t *InCacheBits() const { return _dev_in_cache->ptr<uint64_t>(); }
   uint64_t *InNewBits() const { return _dev_in_new->ptr<uint64_t>(); }

@@ -159,7 +159,7 @@ void FreqRecorder::Record(const KeyT *input, size_t num_inputs) {
 template void FreqRecorder::Record<Id64Type>(const Id64Type *input, size_t num_inputs);
 template void FreqRecorder::Record<IdType>(const IdType *input, size_t num_inputs);
 
-void FreqRecorder::ScatterHandedOver(std::vector<FreqEntry> &list, CntT *into) {
+void FreqRecorder::ScatterHandedOver(FreqEntryList &list, CntT *into) {
   const size_t n = list.size(), n_nodes = _num_nodes;
   const FreqEntry *e = list.data();
   bool bad = false;
@@ -202,28 +202,43 @@ void FreqRecorder::LocalCombineToShared() {
   CntT *shared = _shared;
   const size_t n = _num_nodes;
   if (!_shared_dirty && _direct.empty()) {
-    // Nothing waits in the shared array: the counted keys leave the drained array as entries at once, in one pass
-    // over it instead of three over arrays of the whole key space (add into the shared array, count its non-zero
-    // keys, list them).  Ascending key order whatever the thread count, as GlobalCombine lists them.
+    // Nothing waits in the shared array: the counted keys leave the drained array as entries at once (count, size the
+    // list, fill), instead of being added into the shared array, which was then counted and listed in two more passes
+    // over the whole key space.  Ascending key order whatever the thread count, as GlobalCombine lists them.  Most
+    // counters are zero: sixteen of them (one 64-byte line) are looked at as eight words first.
+    static_assert(sizeof(CntT) == 4, "sixteen counters to a 64-byte line");
+    typedef uint64_t __attribute__((may_alias)) Word;
     const int nthr = ScanThreads();
-    const size_t chunk = (n + nthr - 1) / nthr;
-    std::vector<std::vector<FreqEntry>> part(nthr);
+    const size_t chunk = ((n + nthr - 1) / nthr + 15) / 16 * 16;  // whole lines per thread
+    auto for_each_counted = [&](size_t lo, size_t hi, auto &&fn) {
+      size_t k = lo;
+      for (; k + 16 <= hi; k += 16) {
+        const Word *w = reinterpret_cast<const Word *>(drained + k);
+        if ((w[0] | w[1] | w[2] | w[3] | w[4] | w[5] | w[6] | w[7]) == 0) continue;
+        for (size_t j = k; j < k + 16; j++)
+          if (drained[j]) fn(j);
+      }
+      for (; k < hi; k++)
+        if (drained[k]) fn(k);
+    };
+    std::vector<size_t> first(nthr + 1, 0);
 #pragma omp parallel for num_threads(nthr) schedule(static, 1)
     for (int t = 0; t < nthr; t++) {
-      const size_t lo = std::min(n, chunk * t), hi = std::min(n, chunk * (t + 1));
-      auto &mine = part[t];
-      for (size_t k = lo; k < hi; k++)
-        if (drained[k]) {
-          mine.push_back({(IdType)k, drained[k]});
-          drained[k] = 0;
-        }
+      size_t c = 0;
+      for_each_counted(std::min(n, chunk * t), std::min(n, chunk * (t + 1)), [&](size_t) { c++; });
+      first[t + 1] = c;
     }
-    std::vector<size_t> first(nthr + 1, 0);
-    for (int t = 0; t < nthr; t++) first[t + 1] = first[t] + part[t].size();
-    _direct.resize(first[nthr]);
+    for (int t = 0; t < nthr; t++) first[t + 1] += first[t];
+    _direct.resize(first[nthr]);  // not zeroed (FreqEntryList)
+    FreqEntry *out = _direct.data();
 #pragma omp parallel for num_threads(nthr) schedule(static, 1)
-    for (int t = 0; t < nthr; t++)
-      if (!part[t].empty()) memcpy(_direct.data() + first[t], part[t].data(), part[t].size() * sizeof(FreqEntry));
+    for (int t = 0; t < nthr; t++) {
+      size_t pos = first[t];
+      for_each_counted(std::min(n, chunk * t), std::min(n, chunk * (t + 1)), [&](size_t k) {
+        out[pos++] = {(IdType)k, drained[k]};
+        drained[k] = 0;
+      });
+    }
     return;
   }
   if (!_direct.empty()) ScatterHandedOver(_direct, shared);  // an earlier round still waits as a list: both add up
@@ -239,7 +254,7 @@ void FreqRecorder::LocalCombineToShared() {
 
 void FreqRecorder::GlobalCombine() {
   std::lock_guard<std::mutex> combine(_combine_mu);
-  std::vector<FreqEntry> handed_over;
+  FreqEntryList handed_over;
   {
     std::lock_guard<std::mutex> g(_mu);
     handed_over.swap(_handed_over);

@@ -7,7 +7,9 @@
 #pragma once
 
 #include <cstdint>
+#include <memory>
 #include <mutex>
+#include <utility>
 #include <vector>
 
 #include "common.h"
@@ -24,13 +26,33 @@ struct FreqEntry {
 };
 static_assert(sizeof(FreqEntry) == 8, "FreqEntry is sorted as one 64-bit word");
 
+// a vector whose resize() leaves new elements as they are: lists of tens of millions of entries are sized first and
+// filled by many threads afterwards, and zeroing them in between on one thread would cost as much as the fill
+template <typename T>
+struct DefaultInitAllocator : std::allocator<T> {
+  template <typename U>
+  struct rebind {
+    using other = DefaultInitAllocator<U>;
+  };
+  using std::allocator<T>::allocator;
+  template <typename U>
+  void construct(U *p) noexcept {
+    ::new (static_cast<void *>(p)) U;
+  }
+  template <typename U, typename... Args>
+  void construct(U *p, Args &&...args) {
+    ::new (static_cast<void *>(p)) U(std::forward<Args>(args)...);
+  }
+};
+using FreqEntryList = std::vector<FreqEntry, DefaultInitAllocator<FreqEntry>>;
+
 struct LegacyFreqBuf {
   std::vector<uint32_t> rank_vec, freq_vec;
 };
 
 // Distinct observed keys with their counts; after FreqRecorder::Sort() in rank order.
 struct ContFreqBuf {
-  std::vector<FreqEntry> entries;
+  FreqEntryList entries;
   FreqEntry *buf = nullptr;  // == entries.data()
   size_t size() const { return entries.size(); }
   void add(const IdType &key, const CntT &cnt);  // linear probe over `entries`; for small hand-built buffers
@@ -77,10 +99,10 @@ class FreqRecorder {
   CntT *_spare = nullptr;   // all zero: takes the place of _live when LocalCombineToShared drains it
   CntT *_shared = nullptr;  // counts handed over by LocalCombineToShared
   bool _live_dirty = false, _shared_dirty = false;  // the array holds a non-zero counter
-  std::vector<FreqEntry> _handed_over;              // entries of the open hand-over, not in the arrays
-  std::vector<FreqEntry> _direct;                   // what LocalCombineToShared listed straight from the counters
+  FreqEntryList _handed_over;                      // entries of the open hand-over, not in the arrays
+  FreqEntryList _direct;                           // what LocalCombineToShared listed straight from the counters
                                                     // (ascending, distinct keys), not in the shared array
-  void ScatterHandedOver(std::vector<FreqEntry> &list, CntT *into);
+  void ScatterHandedOver(FreqEntryList &list, CntT *into);
   // _mu guards what recording touches (_live, _live_dirty, _handed_over) and is held for one batch at most;
   // _combine_mu guards the rest (_spare, _shared, _shared_dirty, the ranked list) for the length of a scan of the
   // key space.  Where both are held, _combine_mu is taken first.

@@ -824,7 +824,7 @@ size_t coll_cache_get_cached_keys(int replica_id, uint32_t *out, size_t capacity
   CHECK_NOTNULL(_coll_cache);
   _coll_cache->cache_ctx(replica_id)->SyncHostLists();
   auto mgr = _coll_cache->cache_ctx(replica_id)->EntryManager();
-  if (!mgr || !mgr->_cached_keys) return 0;
+  if (!mgr || !mgr->_cached_keys) return 0;  // (SyncHostLists has fetched a list the build left on the device)
   const size_t n = mgr->_cached_keys->NumItem();
   if (out) memcpy(out, mgr->_cached_keys->Data(), std::min(n, capacity) * sizeof(uint32_t));
   return n;
