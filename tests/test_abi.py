@@ -135,6 +135,23 @@ def test_c_lib_module_of_the_torch_binding():
         assert callable(getattr(co, name)) and getattr(co, name) is not fn
 
 
+def test_compiled_c_lib_module_is_built_and_has_the_six_entry_points():
+    """collcache.torch.c_lib_native: the extension module of PYBIND11_MODULE(c_lib, m) (adapter.cc:274-281) built by
+    python -m ugache_amd.build, linked against libcoll_cache.so; importing it needs no GPU"""
+    pytest.importorskip("torch")
+    sys.path.insert(0, os.path.join(ROOT, "ugache_amd"))
+    import importlib
+    native = importlib.import_module("collcache.torch.c_lib_native")
+    assert native.__file__.endswith(".so")
+    for name in ("coll_torch_init", "coll_torch_init_t", "coll_torch_test", "coll_torch_record",
+                 "coll_torch_lookup_key_t_val_ret", "coll_torch_create_emb_shm"):
+        assert callable(getattr(native, name)), name
+    # pybind11 puts the C++ signature into the docstring
+    doc = native.coll_torch_lookup_key_t_val_ret.__doc__
+    assert doc.startswith("coll_torch_lookup_key_t_val_ret(arg0:") and "arg1: object, arg2: bool) -> object" in doc
+    assert "fname: str = ''" in native.coll_torch_create_emb_shm.__doc__
+
+
 def test_serving_module_has_the_tf2_bindings_entry_points():
     """collcache.torch.serving carries the names the reference's inference scripts call on collcache_tf2
     (python_tf2/collcache_tf2/collcache_tf2/core/initialize.py:33-39, 79, 129, 292; core/lookup_layer.py:22;

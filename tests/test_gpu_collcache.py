@@ -242,6 +242,46 @@ def test_key_list_of_a_build_made_on_the_device_or_on_the_host(key_list, table_k
     check(s1.astype(np.uint32))
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16])
+@pytest.mark.parametrize("kdtype", [torch.int32, torch.int64])
+def test_compiled_c_lib_module_end_to_end(dtype, kdtype, tmp_path):
+    """collcache.torch.c_lib_native, the pybind11 form of the reference's c_lib (adapter.cc:274-281), in the reference's
+    call order: create_emb_shm (from a file) -> record -> init_t -> lookup; same bytes as the oracle's gather, the
+    output a padded view of a reused buffer, coll_torch_test an uninitialised tensor of the output's shape"""
+    import importlib
+    native = importlib.import_module("collcache.torch.c_lib_native")
+    rng = np.random.default_rng(77)
+    n_item, dim, pct = 30_000, 64, 0.2
+    co.config(make_config(n_item, pct))
+    co.coll_cache_record_init(0)
+    np_dtype = np.float32 if dtype == torch.float32 else np.float16
+    table = rng.standard_normal((n_item, dim)).astype(np_dtype)
+    fname = str(tmp_path / "feat.bin")
+    table.tofile(fname)
+    try:
+        emb = native.coll_torch_create_emb_shm(0, n_item, dim, dtype, fname)
+        assert tuple(emb.shape) == (n_item, dim) and emb.dtype == dtype and emb.numpy().tobytes() == table.tobytes()
+        perm = rng.permutation(n_item)
+        s0 = perm[zipf_ranks(rng, 50_000, n_item, 1.1)]
+        native.coll_torch_record(0, torch.from_numpy(s0).to(kdtype))
+        native.coll_torch_init_t(0, 0, emb, pct)
+        want_cached, nid = expected_cached_set(s0.astype(np.uint32), n_item, pct)
+        assert _basics.info(0)["cached_rows"] == len(want_cached)
+        for n in (1, 13, 4097):
+            keys = perm[zipf_ranks(rng, n, n_item, 1.1)]
+            kt = torch.from_numpy(keys).to(kdtype).cuda()
+            out = native.coll_torch_lookup_key_t_val_ret(0, kt, True)
+            assert tuple(out.shape) == ((n + 7) // 8 * 8, dim) and out.dtype == dtype and out.is_cuda
+            assert out[:n].cpu().numpy().tobytes() == table[keys].tobytes()
+            assert _basics.last_group_offset(0) == [0, int((nid[keys] == 0).sum()), n]
+            out2 = native.coll_torch_lookup_key_t_val_ret(0, kt, False)
+            assert tuple(out2.shape) == (n, dim) and out2.data_ptr() == out.data_ptr()  # the reused buffer
+            blank = native.coll_torch_test(0, kt)
+            assert tuple(blank.shape) == (n, dim) and blank.dtype == torch.float32 and blank.is_cuda
+    finally:
+        native.coll_torch_shutdown()
+
+
 @pytest.mark.parametrize("key_list", ["device", "host"])
 @pytest.mark.parametrize("table_kind", ["FLAT", "HASH"])
 def test_build_from_an_explicit_rank_list(key_list, table_kind, monkeypatch):

@@ -4,7 +4,10 @@
   libcoll_cache.so  — host C++ mirror of the reference's coll_cache_lib facade + extern "C" shim (g++),
                       linked against libugache_hip.so; it never includes a HIP header.
 
-Both are built in-tree next to this file.  `python -m ugache_amd.build` rebuilds everything.
+  collcache/torch/c_lib_native.*.so — the compiled form of collcache.torch.c_lib (pybind11, g++), linked against
+                      libcoll_cache.so.
+
+All are built in-tree.  `python -m ugache_amd.build` rebuilds everything.
 """
 import os
 import shutil
@@ -93,11 +96,31 @@ def build_host(verbose=False):
     return HOST_LIB
 
 
+def native_c_lib_path():
+    import sysconfig
+    return os.path.join(PKG, "collcache", "torch", "c_lib_native" + sysconfig.get_config_var("EXT_SUFFIX"))
+
+
+def build_native_c_lib(verbose=False):
+    """the pybind11 extension module collcache.torch.c_lib_native over libcoll_cache.so"""
+    import sysconfig
+
+    import pybind11
+    src = os.path.join(PKG, "collcache", "torch", "c_lib_native.cc")
+    out = _run(["g++", "-O2", "-std=c++17", "-fPIC", "-shared", "-fvisibility=hidden", "-Wall",
+                "-I", pybind11.get_include(), "-I", sysconfig.get_paths()["include"], "-I", INCLUDE, src,
+                "-o", native_c_lib_path(), "-L", PKG, "-lcoll_cache", "-Wl,-rpath,$ORIGIN/../.."])
+    if verbose and out.strip():
+        print(out)
+    return native_c_lib_path()
+
+
 def build_all(verbose=False):
     build_hip(verbose)
     build_host(verbose)
+    build_native_c_lib(verbose)
 
 
 if __name__ == "__main__":
     build_all(verbose=True)
-    print("built:", HIP_LIB, HOST_LIB if os.path.exists(HOST_LIB) else "(no host lib yet)")
+    print("built:", HIP_LIB, HOST_LIB if os.path.exists(HOST_LIB) else "(no host lib yet)", native_c_lib_path())
