@@ -103,7 +103,7 @@ typedef struct {
 const char *ugk_last_error(void);
 /* version of this ABI; bumped on any signature change.  ugk_abi_version() is what the loaded library was built with:
  * a caller compiled against another UGK_ABI_VERSION must not go on. */
-#define UGK_ABI_VERSION 19
+#define UGK_ABI_VERSION 20
 int ugk_abi_version(void);
 
 /* ---- runtime plumbing: Device::{AllocDataSpace,FreeDataSpace,CopyDataFromTo,StreamSync,CreateStream}
@@ -138,6 +138,13 @@ int ugk_stream_is_capturing(void *stream, int *capturing);
  * wait).  `value` must differ from what the word holds (a counter).  What kernels enqueued before the ticket wrote into
  * pinned host memory is visible once the ticket is. */
 int ugk_stream_sync_ticket(void *stream, uint32_t *ticket_host, uint32_t value, unsigned spin_us);
+/* The same wait with a few device words brought along: one launch behind everything enqueued on `stream` copies
+ * a_dev[0 .. n_a) and b_dev[0 .. n_b) (either may be NULL with a count of 0; n_a + n_b <= 63) to dst_host[1 ...] and
+ * then writes `value` to dst_host[0]; the host polls dst_host[0] as above.  dst_host: pinned host words from
+ * ugk_host_malloc, 1 + n_a + n_b of them.  For status words at the end of a sequence of launches: one launch and no
+ * copy call, where a copy into pageable memory and a wait for the stream take two calls into the runtime. */
+int ugk_words_to_host_ticket(const uint32_t *a_dev, unsigned n_a, const uint32_t *b_dev, unsigned n_b,
+                             uint32_t *dst_host, uint32_t value, unsigned spin_us, void *stream);
 int ugk_device_sync(void);
 int ugk_event_create(void **event);
 int ugk_event_destroy(void *event);
@@ -474,7 +481,7 @@ int ugk_record_restore(const uint64_t *entries_dev, size_t n, uint32_t *counts_d
  * taken from the group that was cut.
  * ugk_rank_place_observed: the placement for a caller that knows that fewer than k rows were observed (say, the rows
  * observed at the last placement plus the keys counted since stay below k), 0 < k < num_rows: in_new = every observed
- * row and the lowest k - |observed| never-observed rows, what ugk_rank_place computes in that case, in five launches
+ * row and the lowest k - |observed| never-observed rows, what ugk_rank_place computes in that case, in four launches
  * over the bitmaps and none over the counters.  If k or more rows turn out to be observed, UGK_ST_PLACE_PROMISE is set
  * in *status_dev and in_new_dev is left as it was.  counts_dev may be NULL when reset_counts is 0 (only the bitmap is
  * read then: "observed" can be any set of rows that are in for sure).  cached_dev (may be NULL; then evict_ws_dev, insert_ws_dev and
@@ -506,6 +513,12 @@ int ugk_bitmap_count(const uint64_t *a_dev, const uint64_t *b_dev, int invert_a,
                      uint32_t *total_host, void *stream);
 int ugk_bitmap_emit(const uint64_t *a_dev, const uint64_t *b_dev, int invert_a, uint64_t nbits, const void *ws_dev,
                     uint32_t *out_dev, uint64_t max_out, void *stream);
+/* both differences of two bitmaps in one pass: a & ~b to out_ab_dev and b & ~a to out_ba_dev, each exactly what
+ * ugk_bitmap_emit(a, b, 0, ...) / ugk_bitmap_emit(b, a, 0, ...) writes, from the workspaces ugk_bitmap_count(a, b) and
+ * ugk_bitmap_count(b, a) (or ugk_rank_place_observed) left.  A list with a maximum of 0 is not written. */
+int ugk_bitmap_emit_diff(const uint64_t *a_dev, const uint64_t *b_dev, uint64_t nbits, const void *ws_ab_dev,
+                         const void *ws_ba_dev, uint32_t *out_ab_dev, uint64_t max_ab, uint32_t *out_ba_dev,
+                         uint64_t max_ba, void *stream);
 /* sets (set != 0) or clears the bits listed in idx_dev; a position >= nbits flags UGK_ST_KEY_OUT_OF_RANGE */
 int ugk_bitmap_update(uint64_t *bitmap_dev, uint64_t nbits, const uint32_t *idx_dev, size_t n, int set,
                       uint32_t *status_dev, void *stream);

@@ -831,6 +831,19 @@ int ugk_stream_sync_ticket(void *stream, uint32_t *ticket_host, uint32_t value, 
   *ticket_host = value;
   return 0;
 }
+int ugk_words_to_host_ticket(const uint32_t *a, unsigned n_a, const uint32_t *b, unsigned n_b, uint32_t *dst,
+                             uint32_t value, unsigned, void *stream) {
+  REQUIRE(dst && (a || n_a == 0) && (b || n_b == 0) && n_a + n_b <= 63u, "ugk_words_to_host_ticket: bad argument");
+  {
+    std::lock_guard<std::mutex> g(g_rt_mu);
+    if (as_stream(stream)->capture) violation("the host waited for a ticket on a stream that records into a graph");
+    note_stream_idle(as_stream(stream));
+  }
+  for (unsigned i = 0; i < n_a; ++i) dst[1 + i] = a[i];
+  for (unsigned i = 0; i < n_b; ++i) dst[1 + n_a + i] = b[i];
+  dst[0] = value;
+  return 0;
+}
 int ugk_device_sync(void) {
   std::lock_guard<std::mutex> g(g_rt_mu);
   note_host_wait("the host waited for the device");
@@ -1391,6 +1404,12 @@ int ugk_bitmap_emit(const uint64_t *a, const uint64_t *b, int invert_a, uint64_t
     }
   }
   return 0;
+}
+int ugk_bitmap_emit_diff(const uint64_t *a, const uint64_t *b, uint64_t nbits, const void *ws_ab, const void *ws_ba,
+                         uint32_t *out_ab, uint64_t max_ab, uint32_t *out_ba, uint64_t max_ba, void *stream) {
+  REQUIRE(a && b && ws_ab && ws_ba, "ugk_bitmap_emit_diff: null pointer");
+  if (int rc = ugk_bitmap_emit(a, b, 0, nbits, ws_ab, out_ab, max_ab, stream)) return rc;
+  return ugk_bitmap_emit(b, a, 0, nbits, ws_ba, out_ba, max_ba, stream);
 }
 int ugk_bitmap_update(uint64_t *bitmap, uint64_t nbits, const uint32_t *idx, size_t n, int set, uint32_t *status,
                       void *) {

@@ -154,6 +154,46 @@ def test_wait_on_a_ticket_behind_the_launch(spin_us):
         word.free()
 
 
+@pytest.mark.parametrize("spin_us", [0, 1, 1_000_000])
+def test_words_brought_to_the_host_with_the_ticket(spin_us):
+    """ugk_words_to_host_ticket: device words written by a launch in front of it arrive with the ticket, whichever way
+    the wait ends; either source may be absent"""
+    rng = np.random.default_rng(11)
+    table = _rand_table(rng, 20_000, 512)
+    keys = rng.integers(0, 20_000, size=300_000).astype(np.uint32)
+    d_table, d_keys = to_dev(table), to_dev(keys)
+    out = dev_bytes(len(keys) * 512, fill=0)
+    st = dev_zeros_u32(1)
+    extra = to_dev(np.arange(100, 130, dtype=np.uint32))
+    dst = PinnedArray((64,), np.uint32)
+    try:
+        dst.array[...] = 0
+        stream = C.c_void_p()
+        hip.call("ugk_stream_create", C.byref(stream))
+        sync()
+        bad = keys.copy()
+        bad[12345] = 20_000  # a key outside the table: the gather flags it in its status word
+        d_bad = to_dev(bad)
+        for ticket, (k_dev, n_b) in zip((1, 2, 0xFFFFFFFF), ((d_keys, 30), (d_bad, 7), (d_keys, 0))):
+            st.zero_()
+            sync()
+            hip.call("ugk_gather_direct_u32", ptr(d_table), 20_000, ptr(k_dev), len(keys), ptr(out), 512, 4, ptr(st), None,
+                     stream)  # 4 workgroups: a launch of a few hundred microseconds
+            hip.call("ugk_words_to_host_ticket", ptr(st), 1, ptr(extra) if n_b else None, n_b, dst.ptr, ticket, spin_us,
+                     stream)
+            assert int(dst.array[0]) == ticket
+            assert int(dst.array[1]) == (hip.ST_KEY_OUT_OF_RANGE if k_dev is d_bad else 0)
+            assert dst.array[2: 2 + n_b].tolist() == list(range(100, 100 + n_b))
+        hip.call("ugk_words_to_host_ticket", None, 0, ptr(extra), 3, dst.ptr, 77, spin_us, stream)
+        assert dst.array[:4].tolist() == [77, 100, 101, 102]
+        with pytest.raises(hip.UgkError):
+            hip.call("ugk_words_to_host_ticket", ptr(st), 34, ptr(extra), 30, dst.ptr, 78, spin_us, stream)
+        hip.call("ugk_stream_destroy", stream)
+    finally:
+        sync()
+        dst.free()
+
+
 def test_gather_full_size_all_hit_closed_form():
     """10M x 128 fp32 table resident in HBM, 262144 uniform uint32 keys (the all-hit configuration).
     table[r, c] is a closed form of (r, c), so out[i, c] can be checked without a host copy of the table."""

@@ -211,6 +211,13 @@ def _place_observed(counts, k, reset, cached=None):
             hip.call("ugk_bitmap_emit", ptr(bitmap), ptr(d_cached), 0, n, ptr(ws_in), ptr(in_l), n_in, None)
             sync()
             leaving, coming = to_np(out_l, np.uint32)[:n_out], to_np(in_l, np.uint32)[:n_in]
+            # both lists in one launch from the same two workspaces
+            out_2, in_2 = dev_zeros_u32(max(n_out, 1)), dev_zeros_u32(max(n_in, 1))
+            hip.call("ugk_bitmap_emit_diff", ptr(d_cached), ptr(bitmap), n, ptr(ws_out), ptr(ws_in), ptr(out_2), n_out,
+                     ptr(in_2), n_in, None)
+            sync()
+            assert np.array_equal(to_np(out_2, np.uint32)[:n_out], leaving)
+            assert np.array_equal(to_np(in_2, np.uint32)[:n_in], coming)
         return bits[:n].astype(bool), (status, th.value), to_np(d_counts, np.uint32)[:n], leaving, coming, seen
     finally:
         totals.free()
@@ -298,6 +305,60 @@ def test_bitmap_compaction_matches_flatnonzero(nbits, mode):
             lim = min(max_out, len(want))
             assert np.array_equal(got[:lim], want[:lim])
             assert (got[lim: lim + 8] == 0xFFFFFFFF).all()  # nothing written beyond the limit
+    finally:
+        sync()
+        total.free()
+
+
+@pytest.mark.parametrize("nbits", [1, 64, 65, 4097, 1_000_003, 40_000_000])
+@pytest.mark.parametrize("shape", ["dense", "sparse", "run", "same"])
+def test_bitmap_emit_diff_writes_both_lists_as_two_emits_would(nbits, shape):
+    """a & ~b and b & ~a from one launch = flatnonzero of each, for bitmaps that differ everywhere, in a few places, in
+    one contiguous run (what a refresh of never-observed filler rows looks like) and nowhere; limits below the sizes
+    cut the lists and nothing is written behind them; a limit of 0 with a null list skips that side"""
+    rng = np.random.default_rng(nbits % 977 + len(shape))
+    a_w, a = _bits(rng, nbits, 0.3)
+    if shape == "dense":
+        b_w, b = _bits(rng, nbits, 0.5)
+    else:
+        b = a.copy()
+        if shape == "sparse":
+            flip = rng.integers(0, nbits, size=max(nbits // 1000, 1))
+            b[flip] = ~b[flip]
+        elif shape == "run":
+            lo = nbits // 3
+            b[lo: lo + max(nbits // 50, 1)] = True
+            a[lo: lo + max(nbits // 50, 1)] = False
+            a[-(nbits // 7 + 1):] = True
+            b[-(nbits // 7 + 1):] = False
+            a_w = np.packbits(a, bitorder="little").view(np.uint64)
+        b_w = np.packbits(b, bitorder="little").view(np.uint64)
+    valid = np.zeros(len(a), bool)
+    valid[:nbits] = True
+    want_ab = np.flatnonzero(a & ~b & valid).astype(np.uint32)
+    want_ba = np.flatnonzero(b & ~a & valid).astype(np.uint32)
+    d_a, d_b = to_dev(a_w), to_dev(b_w)
+    ws_ab = dev_bytes(hip.lib().ugk_bitmap_workspace_bytes())
+    ws_ba = dev_bytes(hip.lib().ugk_bitmap_workspace_bytes())
+    total = PinnedArray((4,), np.uint32)
+    try:
+        total.array[...] = 0xFFFFFFFF
+        hip.call("ugk_bitmap_count", ptr(d_a), ptr(d_b), 0, nbits, ptr(ws_ab), total.ptr, None)
+        hip.call("ugk_bitmap_count", ptr(d_b), ptr(d_a), 0, nbits, ptr(ws_ba), total.ptr + 4, None)
+        sync()
+        assert (int(total.array[0]), int(total.array[1])) == (len(want_ab), len(want_ba))
+        for cut_ab, cut_ba in ((1.0, 1.0), (0.5, 1.0), (1.0, 0.0), (0.0, 0.3)):
+            max_ab, max_ba = int(len(want_ab) * cut_ab), int(len(want_ba) * cut_ba)
+            out_ab, out_ba = dev_zeros_u32(len(want_ab) + 8), dev_zeros_u32(len(want_ba) + 8)
+            out_ab.fill_(-1)
+            out_ba.fill_(-1)
+            hip.call("ugk_bitmap_emit_diff", ptr(d_a), ptr(d_b), nbits, ptr(ws_ab), ptr(ws_ba),
+                     ptr(out_ab) if max_ab else None, max_ab, ptr(out_ba) if max_ba else None, max_ba, None)
+            sync()
+            got_ab, got_ba = to_np(out_ab, np.uint32), to_np(out_ba, np.uint32)
+            assert np.array_equal(got_ab[:max_ab], want_ab[:max_ab]), (nbits, shape, cut_ab)
+            assert np.array_equal(got_ba[:max_ba], want_ba[:max_ba]), (nbits, shape, cut_ba)
+            assert (got_ab[max_ab: max_ab + 8] == 0xFFFFFFFF).all() and (got_ba[max_ba: max_ba + 8] == 0xFFFFFFFF).all()
     finally:
         sync()
         total.free()

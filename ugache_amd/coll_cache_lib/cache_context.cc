@@ -1605,13 +1605,12 @@ void RefreshSession::refresh_on_device(ExtractSession *session, size_t num_cache
     n_evict_word = table->CountBits(table->InCacheBits(), table->InNewBits(), false, num_rows, 0, stream);
     n_insert_word = table->CountBits(table->InNewBits(), table->InCacheBits(), false, num_rows, 1, stream);
   }
-  UGK_CALL(ugk_stream_sync(stream));
+  table->WaitByTicket(stream);
   session->PlacementWaitedFor();
   const size_t num_evicted = *n_evict_word, num_insert = *n_insert_word;
-  TensorPtr evict_rows = table->EmitBits(table->InCacheBits(), table->InNewBits(), false, num_rows, 0, num_evicted,
-                                         __evict_rows, alloc, gpu_ctx, stream);
-  TensorPtr insert_rows = table->EmitBits(table->InNewBits(), table->InCacheBits(), false, num_rows, 1, num_insert,
-                                          __insert_rows, alloc, gpu_ctx, stream);
+  TensorPtr evict_rows, insert_rows;  // both lists in one pass over the two bitmaps
+  table->EmitDiff(table->InCacheBits(), table->InNewBits(), num_rows, num_evicted, num_insert, __evict_rows,
+                  __insert_rows, &evict_rows, &insert_rows, alloc, gpu_ctx, stream);
   const size_t num_old = table->_num_cached;
   CHECK_LE(num_evicted, num_old);
   const size_t num_preserved_key = num_old - num_evicted;
@@ -1663,8 +1662,11 @@ void RefreshSession::refresh_on_device(ExtractSession *session, size_t num_cache
                                     _status_handle->ptr<uint32_t>(), stream));
   }
   uint32_t stw[9] = {0};  // [0] status bits, [8] rows taken from the stage so far
-  UGK_CALL(ugk_memcpy_async(stw, _status_handle->ptr<uint32_t>(), sizeof(stw), stream));
-  table->CheckStatus(stream, "refresh on the device");  // waits for the stream
+  // one launch brings the table's status word and these nine to the host, one wait by ticket ends the refresh
+  const uint32_t table_status = table->StatusAndWords(_status_handle->ptr<uint32_t>(), 9, stw, stream);
+  CHECK_EQ(table_status, 0u) << "refresh on the device: table maintenance kernel reported status 0x" << std::hex
+                             << table_status
+                             << " (1 key out of range, 2 table full, 4 duplicate key, 8 evict of absent key)";
   CHECK_EQ(stw[0], 0u) << "refresh on the device: a listed row or slot is outside its table or bitmap (1), or the "
                           "placement found more observed rows than the host's bound allows (0x20)";
   const uint32_t from_stage = stw[8] - _rows_from_stage;

@@ -246,6 +246,40 @@ TensorPtr CacheEntryManager::EmitBits(const uint64_t *a, const uint64_t *b, bool
   return list;
 }
 
+void CacheEntryManager::EmitDiff(const uint64_t *a, const uint64_t *b, uint64_t nbits, size_t n_ab, size_t n_ba,
+                                 TensorPtr &buffer_ab, TensorPtr &buffer_ba, TensorPtr *list_ab, TensorPtr *list_ba,
+                                 const std::function<MemHandle(size_t)> &allocator, Context ctx, StreamHandle stream) {
+  *list_ab = ReuseList(buffer_ab, kI32, n_ab, allocator, ctx);
+  *list_ba = ReuseList(buffer_ba, kI32, n_ba, allocator, ctx);
+  UGK_CALL(ugk_bitmap_emit_diff(a, b, nbits, _dev_bm_ws->ptr(), _dev_bm_ws2->ptr(),
+                                n_ab ? (*list_ab)->Ptr<uint32_t>() : nullptr, n_ab,
+                                n_ba ? (*list_ba)->Ptr<uint32_t>() : nullptr, n_ba, stream));
+}
+
+// pinned words of the table (64): [0] CompactBits' total, [8..10] the counts of a refresh, [16] the ticket of
+// WaitByTicket, [32] the ticket of StatusAndWords and [33 ...] its words
+void CacheEntryManager::WaitByTicket(StreamHandle stream) {
+  CHECK(_dev_words) << "the table's pinned words come with its device lists";
+  if (RunConfig::spin_wait_us == 0) {
+    UGK_CALL(ugk_stream_sync(stream));
+    return;
+  }
+  if (++_ticket == 0) _ticket = 1;
+  UGK_CALL(ugk_stream_sync_ticket(stream, DevWords() + 16, _ticket, RunConfig::spin_wait_us));
+}
+
+uint32_t CacheEntryManager::StatusAndWords(const uint32_t *extra_dev, unsigned n_extra, uint32_t *extra_out,
+                                           StreamHandle stream) {
+  CHECK_LE(n_extra, 30u);
+  CHECK(_dev_words) << "the table's pinned words come with its device lists";
+  if (++_ticket == 0) _ticket = 1;
+  uint32_t *dst = DevWords() + 32;
+  UGK_CALL(ugk_words_to_host_ticket(StatusPtr(this, stream), 1, extra_dev, n_extra, dst, _ticket,
+                                    RunConfig::spin_wait_us, stream));
+  for (unsigned i = 0; i < n_extra; ++i) extra_out[i] = dst[2 + i];
+  return dst[1];
+}
+
 TensorPtr CacheEntryManager::RowsToTableKeys(TensorPtr rows_dev, TensorPtr &buffer,
                                              const std::function<MemHandle(size_t)> &allocator, Context ctx,
                                              StreamHandle stream) {

@@ -108,6 +108,7 @@ class CacheEntryManager {
   MemHandle _dev_rank_ws, _dev_bm_ws;    // workspaces of ugk_rank_* / ugk_bitmap_*
   MemHandle _dev_bm_ws2;                 // a second one, so that two compactions can be counted before one wait
   MemHandle _dev_words;                  // pinned host words the kernels report counts in
+  uint32_t _ticket = 0;                  // last value written behind a stream for WaitByTicket / StatusAndWords
   TensorPtr _dev_list_buffer;            // scratch list for bringing either side up to date
   bool _dev_lists_valid = false;
   bool _host_lists_valid = true;
@@ -147,6 +148,16 @@ class CacheEntryManager {
   TensorPtr EmitBits(const uint64_t *a, const uint64_t *b, bool invert_a, uint64_t nbits, int which, size_t n,
                      TensorPtr &buffer, const std::function<MemHandle(size_t)> &allocator, Context ctx,
                      StreamHandle stream);
+  // both differences of two bitmaps in one launch, counted as sets 0 (a & ~b) and 1 (b & ~a): the first n_ab and n_ba
+  // elements into lists taken from the two buffers
+  void EmitDiff(const uint64_t *a, const uint64_t *b, uint64_t nbits, size_t n_ab, size_t n_ba, TensorPtr &buffer_ab,
+                TensorPtr &buffer_ba, TensorPtr *list_ab, TensorPtr *list_ba,
+                const std::function<MemHandle(size_t)> &allocator, Context ctx, StreamHandle stream);
+  // waits for `stream` by a ticket in the table's pinned words (spin_us == 0: by the runtime)
+  void WaitByTicket(StreamHandle stream);
+  // status words of the table's kernels and n_extra more device words (<= 30), brought to the host by one launch and
+  // one wait by ticket; returns the table's status word, the extra words land in extra_out
+  uint32_t StatusAndWords(const uint32_t *extra_dev, unsigned n_extra, uint32_t *extra_out, StreamHandle stream);
   // device list of host rows -> device list of table keys (the rows themselves, or their ids in sparse-id mode)
   TensorPtr RowsToTableKeys(TensorPtr rows_dev, TensorPtr &buffer, const std::function<MemHandle(size_t)> &allocator,
                             Context ctx, StreamHandle stream);

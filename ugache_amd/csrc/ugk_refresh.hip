@@ -330,17 +330,31 @@ __global__ __launch_bounds__(kBlock) void rank_combine_kernel(const RankWs *ws, 
   }
 }
 
+__device__ __forceinline__ void scan_chunks(BmWs *ws, uint32_t *total_host);  // with the bitmap kernels below
+
 // ---- the placement when the caller knows that fewer rows were observed than are wanted ----------------------------
-// One workgroup, after `observed` was counted and scanned into ws->bm: checks the caller's promise and finds the last
-// needed never-observed row, the (remaining - 1)-th clear bit of `observed` in ascending order (clear bits in front of
-// chunk c = its first bit number - set bits in front of it).
+// One workgroup, after `observed` was counted into ws->bm: scans the chunk counts, checks the caller's promise and
+// finds the last needed never-observed row, the (want - observed rows - 1)-th clear bit of `observed`, ascending (clear
+// bits in front of chunk c = its first bit number - set bits in front of it).  Three dependent reads after the scan:
+// the chunk offsets, the block counts of the one chunk, the 64 words of the one block.
 __global__ __launch_bounds__(kBlock) void rank_locate_unobserved_kernel(RankWs *ws, const unsigned long long *observed,
                                                                         uint64_t nbits, uint64_t per_chunk,
-                                                                        uint32_t *status, uint32_t *observed_host) {
+                                                                        unsigned long long want, uint32_t *status,
+                                                                        uint32_t *observed_host) {
   __shared__ uint32_t chunk_of;
   const int tid = threadIdx.x;
+  if (tid == 0) {  // what rank_init_kernel sets, for the readers of a placement (the histogram is not used here)
+    ws->threshold = 0;
+    ws->remaining = want;
+    ws->count_t = 0;
+    ws->settled = 0;
+    ws->last_row = 0;
+    ws->from_bitmap = 0;
+    ws->keep_mode = 0;
+  }
+  scan_chunks(&ws->bm, nullptr);
+  __syncthreads();
   const uint32_t total = ws->bm.total;
-  const unsigned long long want = ws->remaining;
   if (tid == 0 && observed_host) *observed_host = total;
   if (total >= want) {  // uniform: the promise does not hold, nothing is placed
     if (tid == 0) atomicOr(status, UGK_ST_PLACE_PROMISE);
@@ -354,24 +368,31 @@ __global__ __launch_bounds__(kBlock) void rank_locate_unobserved_kernel(RankWs *
     return (first < nbits ? first : nbits) - ws->bm.base[c];
   };
   constexpr int kPer = kBmChunks / kBlock;
+  uint64_t lo = clear_before(tid * kPer);
   for (int j = 0; j < kPer; ++j) {
     const int c = tid * kPer + j;
-    if (clear_before(c) <= index && index < clear_before(c + 1)) chunk_of = (uint32_t)c;  // exactly one chunk holds it
+    const uint64_t hi = clear_before(c + 1);
+    if (lo <= index && index < hi) chunk_of = (uint32_t)c;  // exactly one chunk holds it
+    lo = hi;
   }
   __syncthreads();
   if (tid >= kWave) return;
   const uint32_t c = chunk_of;
   const uint64_t n_words = (nbits + 63) / 64;
-  const uint64_t begin = (uint64_t)c * per_chunk, end = min(n_words, begin + per_chunk);
+  const uint64_t n_blocks = (n_words + kWave - 1) / kWave;
+  const uint64_t blocks_per_chunk = per_chunk / kWave, first_blk = (uint64_t)c * blocks_per_chunk;
+  constexpr uint64_t kBlockBits = (uint64_t)kWave * 64;
   uint64_t skip = index - clear_before((int)c);  // clear bits of the chunk below the wanted one
-  for (uint64_t w0 = begin; w0 < end; w0 += kWave) {
-    const uint64_t w = w0 + tid;
-    unsigned long long m = 0ull;
-    if (w < end) {
-      m = ~observed[w];
-      if (nbits - w * 64 < 64) m &= (1ull << (nbits - w * 64)) - 1ull;
+  // the block: a lane per block of the chunk
+  uint64_t blk = 0;
+  bool found = false;
+  for (uint64_t b0 = 0; b0 < blocks_per_chunk && !found; b0 += kWave) {
+    const uint64_t b = first_blk + b0 + tid;
+    uint32_t mine = 0;
+    if (b0 + tid < blocks_per_chunk && b < n_blocks) {
+      const uint64_t bits = min(nbits - b * kBlockBits, kBlockBits);
+      mine = (uint32_t)bits - ws->bm.block[b];
     }
-    const uint32_t mine = __popcll(m);
     uint32_t incl = mine;
 #pragma unroll
     for (int s = 1; s < kWave; s <<= 1) {
@@ -379,20 +400,40 @@ __global__ __launch_bounds__(kBlock) void rank_locate_unobserved_kernel(RankWs *
       if (tid >= s) incl += up;
     }
     const uint32_t all = __shfl(incl, kWave - 1);
-    if (skip < all) {  // in this group of words; wavefront-uniform
-      if (incl - mine <= skip && skip < incl) {
-        uint32_t drop = (uint32_t)skip - (incl - mine);
-        while (drop--) m &= m - 1;
-        const uint32_t row = (uint32_t)(w * 64 + __builtin_ctzll(m));
-        ws->last_row = row;
-        ws->threshold = rank_of(0u, row);
-        ws->remaining = want - total;
-        ws->from_bitmap = 1;
-        ws->settled = 1;
-      }
-      return;
+    if (skip < all) {  // wavefront-uniform
+      const unsigned long long holds = __ballot(incl - mine <= skip && skip < incl);
+      const int src = __builtin_ctzll(holds);
+      blk = first_blk + b0 + src;
+      skip -= __shfl(incl - mine, src);
+      found = true;
+    } else {
+      skip -= all;
     }
-    skip -= all;
+  }
+  if (!found) return;  // cannot be: the chunk holds the bit
+  // the word and the bit: a lane per word of the block
+  const uint64_t w = blk * kWave + tid;
+  unsigned long long m = 0ull;
+  if (w < n_words) {
+    m = ~observed[w];
+    if (nbits - w * 64 < 64) m &= (1ull << (nbits - w * 64)) - 1ull;
+  }
+  const uint32_t mine = __popcll(m);
+  uint32_t incl = mine;
+#pragma unroll
+  for (int s = 1; s < kWave; s <<= 1) {
+    const uint32_t up = __shfl_up(incl, s);
+    if (tid >= s) incl += up;
+  }
+  if (incl - mine <= skip && skip < incl) {
+    uint32_t drop = (uint32_t)skip - (incl - mine);
+    while (drop--) m &= m - 1;
+    const uint32_t row = (uint32_t)(w * 64 + __builtin_ctzll(m));
+    ws->last_row = row;
+    ws->threshold = rank_of(0u, row);
+    ws->remaining = want - total;
+    ws->from_bitmap = 1;
+    ws->settled = 1;
   }
 }
 
@@ -596,6 +637,72 @@ __global__ __launch_bounds__(kBlock) void bitmap_emit_kernel(const unsigned long
   }
 }
 
+// Both differences of two bitmaps in one pass, a & ~b -> out_ab and b & ~a -> out_ba, each list as bitmap_emit_kernel
+// writes it from its own counts (ws_ab, ws_ba).  The small arrays of counts are read before it is known whether the
+// block holds anything, the two words of the bitmaps only when it does: two dependent reads per block.
+__device__ __forceinline__ void emit_word(unsigned long long m, uint64_t pos0, uint64_t w, int lane, uint32_t *out,
+                                          uint64_t max_out) {
+  const uint32_t mine = __popcll(m);
+  uint32_t incl = mine;
+#pragma unroll
+  for (int s = 1; s < kWave; s <<= 1) {
+    const uint32_t up = __shfl_up(incl, s);
+    if (lane >= s) incl += up;
+  }
+  uint64_t pos = pos0 + incl - mine;
+  while (m) {
+    const int bit = __builtin_ctzll(m);
+    m &= m - 1;
+    if (pos < max_out) out[pos] = (uint32_t)(w * 64 + bit);
+    ++pos;
+  }
+}
+
+__global__ __launch_bounds__(kBlock) void bitmap_emit_diff_kernel(const unsigned long long *a,
+                                                                  const unsigned long long *b, uint64_t nbits,
+                                                                  uint64_t per_chunk, const BmWs *ws_ab,
+                                                                  const BmWs *ws_ba, uint32_t *out_ab, uint64_t max_ab,
+                                                                  uint32_t *out_ba, uint64_t max_ba) {
+  const int lane = (int)lane_id();
+  const uint64_t n_words = (nbits + 63) / 64;
+  const uint64_t n_blocks = (n_words + kWave - 1) / kWave;
+  const uint64_t wave = ((uint64_t)blockIdx.x * kBlock + threadIdx.x) / kWave;
+  const uint64_t n_waves = (uint64_t)gridDim.x * (kBlock / kWave);
+  const uint64_t blocks_per_chunk = per_chunk / kWave;
+  for (uint64_t blk = wave; blk < n_blocks; blk += n_waves) {
+    const uint32_t n_ab = ws_ab->block[blk], n_ba = ws_ba->block[blk];
+    const uint64_t chunk = blk / blocks_per_chunk, first = chunk * blocks_per_chunk;
+    uint32_t before_ab = 0, before_ba = 0;
+    for (uint64_t q = first + lane; q < blk; q += kWave) {
+      before_ab += ws_ab->block[q];
+      before_ba += ws_ba->block[q];
+    }
+    const uint64_t base_ab = ws_ab->base[chunk], base_ba = ws_ba->base[chunk];
+    if ((n_ab | n_ba) == 0) continue;  // wavefront-uniform
+#pragma unroll
+    for (int d = kWave / 2; d > 0; d >>= 1) {
+      before_ab += __shfl_xor(before_ab, d);
+      before_ba += __shfl_xor(before_ba, d);
+    }
+    const uint64_t pos_ab = base_ab + before_ab, pos_ba = base_ba + before_ba;
+    const bool do_ab = n_ab != 0 && pos_ab < max_ab, do_ba = n_ba != 0 && pos_ba < max_ba;
+    if (!do_ab && !do_ba) continue;
+    const uint64_t w = blk * kWave + lane;
+    unsigned long long wa = 0ull, wb = 0ull;
+    if (w < n_words) {
+      wa = a[w];
+      wb = b[w];
+      if (nbits - w * 64 < 64) {  // the last, partial word
+        const unsigned long long valid = (1ull << (nbits - w * 64)) - 1ull;
+        wa &= valid;
+        wb &= valid;
+      }
+    }
+    if (do_ab) emit_word(wa & ~wb, pos_ab, w, lane, out_ab, max_ab);
+    if (do_ba) emit_word(wb & ~wa, pos_ba, w, lane, out_ba, max_ba);
+  }
+}
+
 __global__ __launch_bounds__(kBlock) void bitmap_update_kernel(unsigned long long *bitmap, uint64_t nbits,
                                                                const uint32_t *idx, size_t n, int set,
                                                                uint32_t *status) {
@@ -741,12 +848,10 @@ int ugk_rank_place_observed(uint32_t *counts_dev, uint64_t num_rows, uint64_t k,
   const uint64_t n_words = (num_rows + 63) / 64;
   const uint64_t per_chunk = bm_words_per_chunk(n_words);
   const unsigned bm_grid = clamp_grid((kBmChunks + (kBlock / kWave) - 1) / (kBlock / kWave), (unsigned)cu_count() * 8u);
-  hipLaunchKernelGGL(rank_init_kernel, dim3(1), dim3(kBlock), 0, st, ws, (unsigned long long)k);
   hipLaunchKernelGGL(bitmap_count_kernel, dim3(bm_grid), dim3(kBlock), 0, st, observed, none, 0, num_rows, per_chunk,
                      &ws->bm, no_gate);
-  hipLaunchKernelGGL(bitmap_scan_kernel, dim3(1), dim3(kBlock), 0, st, &ws->bm, (uint32_t *)nullptr, no_gate);
   hipLaunchKernelGGL(rank_locate_unobserved_kernel, dim3(1), dim3(kBlock), 0, st, ws, observed, num_rows, per_chunk,
-                     status_dev, totals_host ? totals_host + 2 : (uint32_t *)nullptr);
+                     (unsigned long long)k, status_dev, totals_host ? totals_host + 2 : (uint32_t *)nullptr);
   hipLaunchKernelGGL(rank_combine_observed_kernel, dim3(bm_grid), dim3(kBlock), 0, st, counts_dev, num_rows, per_chunk,
                      (const RankWs *)ws, observed, reinterpret_cast<unsigned long long *>(in_new_dev),
                      reinterpret_cast<const unsigned long long *>(cached_dev), static_cast<BmWs *>(evict_ws_dev),
@@ -801,6 +906,27 @@ int ugk_bitmap_emit(const uint64_t *a_dev, const uint64_t *b_dev, int invert_a, 
                      reinterpret_cast<const unsigned long long *>(a_dev),
                      reinterpret_cast<const unsigned long long *>(b_dev), invert_a ? kBmInvertA : 0, nbits,
                      per_chunk, static_cast<const BmWs *>(ws_dev), out_dev, max_out);
+  UGK_HIP(hipGetLastError());
+  return 0;
+}
+
+int ugk_bitmap_emit_diff(const uint64_t *a_dev, const uint64_t *b_dev, uint64_t nbits, const void *ws_ab_dev,
+                         const void *ws_ba_dev, uint32_t *out_ab_dev, uint64_t max_ab, uint32_t *out_ba_dev,
+                         uint64_t max_ba, void *stream) {
+  UGK_REQUIRE(a_dev && b_dev && ws_ab_dev && ws_ba_dev, "ugk_bitmap_emit_diff: null pointer");
+  UGK_REQUIRE(nbits > 0 && nbits <= 0xffffffffull, "ugk_bitmap_emit_diff: %llu bits do not fit 32-bit positions",
+              (unsigned long long)nbits);
+  if (max_ab == 0 && max_ba == 0) return 0;
+  UGK_REQUIRE((out_ab_dev || max_ab == 0) && (out_ba_dev || max_ba == 0), "ugk_bitmap_emit_diff: null output list");
+  const uint64_t n_words = (nbits + 63) / 64;
+  const uint64_t per_chunk = bm_words_per_chunk(n_words);
+  const uint64_t n_blocks = (n_words + kWave - 1) / kWave;
+  const unsigned grid = clamp_grid((n_blocks + (kBlock / kWave) - 1) / (kBlock / kWave), 0);
+  hipLaunchKernelGGL(bitmap_emit_diff_kernel, dim3(grid), dim3(kBlock), 0, as_stream(stream),
+                     reinterpret_cast<const unsigned long long *>(a_dev),
+                     reinterpret_cast<const unsigned long long *>(b_dev), nbits, per_chunk,
+                     static_cast<const BmWs *>(ws_ab_dev), static_cast<const BmWs *>(ws_ba_dev), out_ab_dev, max_ab,
+                     out_ba_dev, max_ba);
   UGK_HIP(hipGetLastError());
   return 0;
 }

@@ -2,6 +2,7 @@
 #include <cstdlib>
 #include <cstring>
 
+#include <atomic>
 #include <chrono>
 
 #include "ugk_internal.h"
@@ -209,6 +210,20 @@ int ugk_stream_is_capturing(void *stream, int *capturing) {
 
 namespace {
 __global__ void ticket_kernel(volatile uint32_t *word, uint32_t value) { *word = value; }
+
+// one wavefront: n_a + n_b device words to dst[1 ...], then the ticket to dst[0]
+__global__ void words_ticket_kernel(const uint32_t *a, unsigned n_a, const uint32_t *b, unsigned n_b,
+                                    volatile uint32_t *dst, uint32_t value) {
+  const unsigned lane = threadIdx.x;
+  if (lane < n_a) dst[1 + lane] = a[lane];
+  else if (lane < n_a + n_b) dst[1 + lane] = b[lane - n_a];
+  __threadfence_system();
+  __syncthreads();
+  if (lane == 0) {
+    __threadfence_system();
+    dst[0] = value;
+  }
+}
 }  // namespace
 
 int ugk_stream_sync_ticket(void *stream, uint32_t *ticket_host, uint32_t value, unsigned spin_us) {
@@ -229,6 +244,28 @@ int ugk_stream_sync_ticket(void *stream, uint32_t *ticket_host, uint32_t value, 
   // microseconds the poll saved
   if (*word == value) return 0;
   UGK_HIP(hipStreamSynchronize(as_stream(stream)));
+  return 0;
+}
+
+int ugk_words_to_host_ticket(const uint32_t *a_dev, unsigned n_a, const uint32_t *b_dev, unsigned n_b,
+                             uint32_t *dst_host, uint32_t value, unsigned spin_us, void *stream) {
+  UGK_REQUIRE(dst_host, "ugk_words_to_host_ticket: null destination");
+  UGK_REQUIRE((a_dev || n_a == 0) && (b_dev || n_b == 0), "ugk_words_to_host_ticket: null source");
+  UGK_REQUIRE(n_a + n_b <= 63u, "ugk_words_to_host_ticket: %u words, at most 63 fit one launch", n_a + n_b);
+  hipLaunchKernelGGL(words_ticket_kernel, dim3(1), dim3(64), 0, as_stream(stream), a_dev, n_a, b_dev, n_b, dst_host,
+                     value);
+  UGK_HIP(hipGetLastError());
+  volatile uint32_t *word = dst_host;
+  const auto t0 = std::chrono::steady_clock::now();
+  unsigned polls = 0;
+  while (*word != value) {
+    if ((++polls & 63u) == 0 &&
+        std::chrono::duration_cast<std::chrono::microseconds>(std::chrono::steady_clock::now() - t0).count() >=
+            (long long)spin_us)
+      break;
+  }
+  if (*word != value) UGK_HIP(hipStreamSynchronize(as_stream(stream)));
+  std::atomic_thread_fence(std::memory_order_acquire);
   return 0;
 }
 

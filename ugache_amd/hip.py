@@ -70,6 +70,7 @@ SIGNATURES = {
     "ugk_stream_sync": [_vp],
     "ugk_stream_is_capturing": [_vp, _vp],
     "ugk_stream_sync_ticket": [_vp, _vp, _u32, C.c_uint],
+    "ugk_words_to_host_ticket": [_vp, C.c_uint, _vp, C.c_uint, _vp, _u32, C.c_uint, _vp],
     "ugk_device_sync": [],
     "ugk_event_create": [C.POINTER(_vp)],
     "ugk_event_destroy": [_vp],
@@ -142,6 +143,7 @@ SIGNATURES = {
     "ugk_bitmap_workspace_bytes": [],
     "ugk_bitmap_count": [_vp, _vp, C.c_int, _u64, _vp, _vp, _vp],
     "ugk_bitmap_emit": [_vp, _vp, C.c_int, _u64, _vp, _vp, _u64, _vp],
+    "ugk_bitmap_emit_diff": [_vp, _vp, _u64, _vp, _vp, _vp, _u64, _vp, _u64, _vp],
     "ugk_bitmap_update": [_vp, _u64, _vp, _sz, C.c_int, _vp, _vp],
     "ugk_bitmap_set_through": [_vp, _u64, _vp, _vp, _vp],
     "ugk_rows_to_keys": [_vp, _sz, _u64, _u64, _vp, _vp],
