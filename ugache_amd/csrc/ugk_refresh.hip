@@ -599,6 +599,48 @@ __global__ __launch_bounds__(kBlock) void bitmap_scan2_kernel(BmWs *a, BmWs *b, 
   scan_chunks(blockIdx.x == 0 ? a : b, totals_host + blockIdx.x);
 }
 
+// The set bits of one 64-word block, a lane per word on entry (m), to out[pos0 ...] in ascending order; n_set: how
+// many there are (wavefront-uniform).  A block with few bits: every lane walks the bits of its own word (a step or
+// two).  A block with many: the wavefront takes the non-zero words one at a time, a lane per bit, one store of
+// consecutive positions per word and at most 64 of them (a lane per word would store at 64 scattered places per step,
+// 64 steps for a block of all ones: a contiguous run of rows that leave the cache kept a handful of wavefronts busy
+// long after the rest had finished; for blocks with a few bits the word-at-a-time form is the slower one, 51 against
+// 37 us over 122 k blocks with four bits each).
+constexpr uint32_t kEmitDense = 2 * kWave;
+__device__ __forceinline__ void emit_word(unsigned long long m, uint32_t n_set, uint64_t pos0, uint64_t w, int lane,
+                                          uint32_t *out, uint64_t max_out) {
+  const uint32_t mine = __popcll(m);
+  uint32_t incl = mine;
+#pragma unroll
+  for (int s = 1; s < kWave; s <<= 1) {
+    const uint32_t up = __shfl_up(incl, s);
+    if (lane >= s) incl += up;
+  }
+  const uint32_t excl = incl - mine;
+  if (n_set <= kEmitDense) {
+    uint64_t pos = pos0 + excl;
+    while (m) {
+      const int bit = __builtin_ctzll(m);
+      m &= m - 1;
+      if (pos < max_out) out[pos] = (uint32_t)(w * 64 + bit);
+      ++pos;
+    }
+    return;
+  }
+  const uint64_t w_first = w - (uint64_t)lane;
+  const unsigned long long below = (1ull << lane) - 1ull;
+  unsigned long long todo = __ballot(m != 0ull);
+  while (todo) {  // wavefront-uniform
+    const int src = __builtin_ctzll(todo);
+    todo &= todo - 1;
+    const unsigned long long word =
+        ((unsigned long long)(uint32_t)__builtin_amdgcn_readlane((int)(uint32_t)(m >> 32), src) << 32) |
+        (uint32_t)__builtin_amdgcn_readlane((int)(uint32_t)m, src);
+    const uint64_t pos = pos0 + (uint32_t)__builtin_amdgcn_readlane((int)excl, src) + __popcll(word & below);
+    if (((word >> lane) & 1ull) && pos < max_out) out[pos] = (uint32_t)((w_first + src) * 64 + lane);
+  }
+}
+
 __global__ __launch_bounds__(kBlock) void bitmap_emit_kernel(const unsigned long long *a, const unsigned long long *b,
                                                              int flags, uint64_t nbits, uint64_t per_chunk,
                                                              const BmWs *ws, uint32_t *out, uint64_t max_out) {
@@ -609,7 +651,8 @@ __global__ __launch_bounds__(kBlock) void bitmap_emit_kernel(const unsigned long
   const uint64_t n_waves = (uint64_t)gridDim.x * (kBlock / kWave);
   const uint64_t blocks_per_chunk = per_chunk / kWave;
   for (uint64_t blk = wave; blk < n_blocks; blk += n_waves) {
-    if (ws->block[blk] == 0) continue;  // wavefront-uniform
+    const uint32_t n_here = ws->block[blk];
+    if (n_here == 0) continue;  // wavefront-uniform
     // where the block's elements go: its chunk's offset plus the counts of the chunk's earlier blocks
     const uint64_t chunk = blk / blocks_per_chunk, first = chunk * blocks_per_chunk;
     uint32_t before = 0;
@@ -620,44 +663,14 @@ __global__ __launch_bounds__(kBlock) void bitmap_emit_kernel(const unsigned long
     if (pos0 >= max_out) continue;
     const uint64_t w = blk * kWave + lane;
     unsigned long long m = w < n_words ? bm_word(a, b, flags, nbits, w) : 0ull;
-    const uint32_t mine = __popcll(m);
-    uint32_t incl = mine;
-#pragma unroll
-    for (int s = 1; s < kWave; s <<= 1) {
-      const uint32_t up = __shfl_up(incl, s);
-      if (lane >= s) incl += up;
-    }
-    uint64_t pos = pos0 + incl - mine;
-    while (m) {
-      const int bit = __builtin_ctzll(m);
-      m &= m - 1;
-      if (pos < max_out) out[pos] = (uint32_t)(w * 64 + bit);
-      ++pos;
-    }
+    emit_word(m, n_here, pos0, w, lane, out, max_out);
   }
 }
 
 // Both differences of two bitmaps in one pass, a & ~b -> out_ab and b & ~a -> out_ba, each list as bitmap_emit_kernel
 // writes it from its own counts (ws_ab, ws_ba).  The small arrays of counts are read before it is known whether the
 // block holds anything, the two words of the bitmaps only when it does: two dependent reads per block.
-__device__ __forceinline__ void emit_word(unsigned long long m, uint64_t pos0, uint64_t w, int lane, uint32_t *out,
-                                          uint64_t max_out) {
-  const uint32_t mine = __popcll(m);
-  uint32_t incl = mine;
-#pragma unroll
-  for (int s = 1; s < kWave; s <<= 1) {
-    const uint32_t up = __shfl_up(incl, s);
-    if (lane >= s) incl += up;
-  }
-  uint64_t pos = pos0 + incl - mine;
-  while (m) {
-    const int bit = __builtin_ctzll(m);
-    m &= m - 1;
-    if (pos < max_out) out[pos] = (uint32_t)(w * 64 + bit);
-    ++pos;
-  }
-}
-
+constexpr int kDiffBlocks = 1;  // consecutive blocks per wavefront and round
 __global__ __launch_bounds__(kBlock) void bitmap_emit_diff_kernel(const unsigned long long *a,
                                                                   const unsigned long long *b, uint64_t nbits,
                                                                   uint64_t per_chunk, const BmWs *ws_ab,
@@ -666,40 +679,76 @@ __global__ __launch_bounds__(kBlock) void bitmap_emit_diff_kernel(const unsigned
   const int lane = (int)lane_id();
   const uint64_t n_words = (nbits + 63) / 64;
   const uint64_t n_blocks = (n_words + kWave - 1) / kWave;
+  const uint64_t n_groups = (n_blocks + kDiffBlocks - 1) / kDiffBlocks;
   const uint64_t wave = ((uint64_t)blockIdx.x * kBlock + threadIdx.x) / kWave;
   const uint64_t n_waves = (uint64_t)gridDim.x * (kBlock / kWave);
   const uint64_t blocks_per_chunk = per_chunk / kWave;
-  for (uint64_t blk = wave; blk < n_blocks; blk += n_waves) {
-    const uint32_t n_ab = ws_ab->block[blk], n_ba = ws_ba->block[blk];
-    const uint64_t chunk = blk / blocks_per_chunk, first = chunk * blocks_per_chunk;
+  for (uint64_t grp = wave; grp < n_groups; grp += n_waves) {
+    const uint64_t blk0 = grp * kDiffBlocks;
+    // first round, all of it asked for at once: the counts of the group's blocks, the counts in front of its first
+    // block inside that block's chunk, the chunk offsets
+    uint32_t n_ab[kDiffBlocks], n_ba[kDiffBlocks];
+    uint64_t base_ab[kDiffBlocks], base_ba[kDiffBlocks];
+#pragma unroll
+    for (int j = 0; j < kDiffBlocks; ++j) {
+      const uint64_t blk = min(blk0 + j, n_blocks - 1);
+      const bool valid = blk0 + j < n_blocks;
+      n_ab[j] = valid ? ws_ab->block[blk] : 0u;
+      n_ba[j] = valid ? ws_ba->block[blk] : 0u;
+      base_ab[j] = ws_ab->base[blk / blocks_per_chunk];
+      base_ba[j] = ws_ba->base[blk / blocks_per_chunk];
+    }
     uint32_t before_ab = 0, before_ba = 0;
-    for (uint64_t q = first + lane; q < blk; q += kWave) {
+    for (uint64_t q = blk0 / blocks_per_chunk * blocks_per_chunk + lane; q < blk0; q += kWave) {
       before_ab += ws_ab->block[q];
       before_ba += ws_ba->block[q];
     }
-    const uint64_t base_ab = ws_ab->base[chunk], base_ba = ws_ba->base[chunk];
-    if ((n_ab | n_ba) == 0) continue;  // wavefront-uniform
+    uint32_t any = 0;
+#pragma unroll
+    for (int j = 0; j < kDiffBlocks; ++j) any |= n_ab[j] | n_ba[j];
+    if (any == 0) continue;  // wavefront-uniform
 #pragma unroll
     for (int d = kWave / 2; d > 0; d >>= 1) {
       before_ab += __shfl_xor(before_ab, d);
       before_ba += __shfl_xor(before_ba, d);
     }
-    const uint64_t pos_ab = base_ab + before_ab, pos_ba = base_ba + before_ba;
-    const bool do_ab = n_ab != 0 && pos_ab < max_ab, do_ba = n_ba != 0 && pos_ba < max_ba;
-    if (!do_ab && !do_ba) continue;
-    const uint64_t w = blk * kWave + lane;
-    unsigned long long wa = 0ull, wb = 0ull;
-    if (w < n_words) {
-      wa = a[w];
-      wb = b[w];
-      if (nbits - w * 64 < 64) {  // the last, partial word
-        const unsigned long long valid = (1ull << (nbits - w * 64)) - 1ull;
-        wa &= valid;
-        wb &= valid;
+    // where each block's elements go: its chunk's offset plus the counts of the chunk's earlier blocks
+    uint64_t pos_ab[kDiffBlocks], pos_ba[kDiffBlocks];
+#pragma unroll
+    for (int j = 0; j < kDiffBlocks; ++j) {
+      if (j > 0) {
+        const bool new_chunk = (blk0 + j) % blocks_per_chunk == 0;
+        before_ab = new_chunk ? 0u : before_ab + n_ab[j - 1];
+        before_ba = new_chunk ? 0u : before_ba + n_ba[j - 1];
+      }
+      pos_ab[j] = base_ab[j] + before_ab;
+      pos_ba[j] = base_ba[j] + before_ba;
+    }
+    // second round: the words of the blocks that hold anything that is still wanted
+    unsigned long long wa[kDiffBlocks], wb[kDiffBlocks];
+    bool do_ab[kDiffBlocks], do_ba[kDiffBlocks];
+#pragma unroll
+    for (int j = 0; j < kDiffBlocks; ++j) {
+      do_ab[j] = n_ab[j] != 0 && pos_ab[j] < max_ab;
+      do_ba[j] = n_ba[j] != 0 && pos_ba[j] < max_ba;
+      const uint64_t w = (blk0 + j) * kWave + lane;
+      wa[j] = wb[j] = 0ull;
+      if ((do_ab[j] || do_ba[j]) && w < n_words) {
+        wa[j] = a[w];
+        wb[j] = b[w];
+        if (nbits - w * 64 < 64) {  // the last, partial word
+          const unsigned long long valid = (1ull << (nbits - w * 64)) - 1ull;
+          wa[j] &= valid;
+          wb[j] &= valid;
+        }
       }
     }
-    if (do_ab) emit_word(wa & ~wb, pos_ab, w, lane, out_ab, max_ab);
-    if (do_ba) emit_word(wb & ~wa, pos_ba, w, lane, out_ba, max_ba);
+#pragma unroll
+    for (int j = 0; j < kDiffBlocks; ++j) {
+      const uint64_t w = (blk0 + j) * kWave + lane;
+      if (do_ab[j]) emit_word(wa[j] & ~wb[j], n_ab[j], pos_ab[j], w, lane, out_ab, max_ab);
+      if (do_ba[j]) emit_word(wb[j] & ~wa[j], n_ba[j], pos_ba[j], w, lane, out_ba, max_ba);
+    }
   }
 }
 
@@ -920,8 +969,8 @@ int ugk_bitmap_emit_diff(const uint64_t *a_dev, const uint64_t *b_dev, uint64_t 
   UGK_REQUIRE((out_ab_dev || max_ab == 0) && (out_ba_dev || max_ba == 0), "ugk_bitmap_emit_diff: null output list");
   const uint64_t n_words = (nbits + 63) / 64;
   const uint64_t per_chunk = bm_words_per_chunk(n_words);
-  const uint64_t n_blocks = (n_words + kWave - 1) / kWave;
-  const unsigned grid = clamp_grid((n_blocks + (kBlock / kWave) - 1) / (kBlock / kWave), 0);
+  const uint64_t n_groups = ((n_words + kWave - 1) / kWave + kDiffBlocks - 1) / kDiffBlocks;
+  const unsigned grid = clamp_grid((n_groups + (kBlock / kWave) - 1) / (kBlock / kWave), 0);
   hipLaunchKernelGGL(bitmap_emit_diff_kernel, dim3(grid), dim3(kBlock), 0, as_stream(stream),
                      reinterpret_cast<const unsigned long long *>(a_dev),
                      reinterpret_cast<const unsigned long long *>(b_dev), nbits, per_chunk,
