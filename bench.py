@@ -117,7 +117,7 @@ def parse_args():
     ap.add_argument("--calibrate", action="store_true",
                     help="also run 5 plain device copies of 1 GiB (ugk_copy_rows) so a counter run has a kernel of "
                          "known traffic next to the gather")
-    ap.add_argument("--probe", default=None, choices=["kpw", "row_span", "link_latency", "rw_ceiling", "cu_mask", "small_batch", "pooled", "sparse_layer"],
+    ap.add_argument("--probe", default=None, choices=["kpw", "row_span", "link_latency", "rw_ceiling", "placement", "cu_mask", "small_batch", "pooled", "sparse_layer"],
                     help="instead of a workload, run one of the stand-alone measurements behind the launch rules "
                          "(bench_probes.py): keys per wavefront of the fused kernel, random rows over the host "
                          "link by span, host-link gather confined to a few compute units, serving-sized batches through "

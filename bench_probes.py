@@ -21,6 +21,9 @@ flagged an error (the parity tests check results).
             HBM for comparison); (b) the rate of independent row reads by the number of bytes in flight (workgroups x
             loads in flight per lane), which shows where the link stops answering faster; (c) where the allocation's
             pages live (/proc/self/numa_maps).  Kernels: bench_probes_kernels.hip (libbench_probes.so)
+  placement  the placement of a refresh on the device alone on the chip at config 5's size (500 M counters, some 57 M
+            above zero, 50 M and 20 M rows wanted): counters kept (one pass when the last placement's threshold still
+            holds, two when it does not) and counters reset (two passes)
   rw_ceiling  what the two sides of the all-hit gather reach alone on its own shapes: random 512-byte rows read and
             nothing written, a buffer written and nothing read, a plain copy, the gather itself; with an output that
             stays in the memory-side cache and with one that cannot
@@ -32,6 +35,7 @@ flagged an error (the parity tests check results).
 import ctypes as C
 import json
 import os
+import math
 import sys
 import time
 
@@ -670,7 +674,75 @@ def probe_rw_ceiling(hip, torch, note, quick=False):
             "sizes": res}
 
 
-PROBES = {"rw_ceiling": probe_rw_ceiling, "link_latency": probe_link_latency, "sparse_layer": probe_sparse_layer, "pooled": probe_pooled, "kpw": probe_kpw, "row_span": probe_row_span, "cu_mask": probe_cu_mask, "small_batch": probe_small_batch}
+def probe_placement(hip, torch, note, quick=False):
+    """The placement of a refresh on the device, alone on the chip, at config 5's size: 500 M counters of which some
+    57 M are above zero (Zipf 1.05 over the rows, 200 M draws), K = 50 M and 20 M rows wanted.  ugk_rank_place with the
+    counters kept (the first pass splits by the last placement's threshold on its way: timed with a workspace that has
+    seen the same placement, and with one whose guess is wrong), with the counters reset after every placement (two
+    passes), and ugk_rank_place_observed where it applies (K above the number of observed rows)."""
+    stream = C.c_void_p()
+    hip.call("ugk_stream_create", C.byref(stream))
+    rows = 100_000_000 if quick else 500_000_000
+    words = (rows + 63) // 64
+    g = torch.Generator(device="cuda").manual_seed(5)
+    counts = torch.zeros(rows, dtype=torch.int32, device="cuda")
+    draws = 40_000_000 if quick else 200_000_000
+    for _ in range(draws // 20_000_000):
+        u = torch.rand(20_000_000, generator=g, device="cuda", dtype=torch.float64)
+        r = (torch.exp(u * math.log(rows)) - 1).clamp_(0, rows - 1).to(torch.int64)  # log-uniform: ~ Zipf 1
+        r = (r * 2654435761) % rows  # hot rows spread over the key space
+        counts.index_add_(0, r, torch.ones_like(r, dtype=torch.int32))
+        del u, r
+    observed_n = int((counts > 0).sum().item())
+    saved = counts.clone()
+    # the observed-rows bitmap as the record kernel keeps it (bit r = counter r above zero), packed with torch
+    pad = torch.zeros(words * 64, dtype=torch.bool, device="cuda")
+    pad[:rows] = counts > 0
+    weights = torch.ones(64, dtype=torch.int64, device="cuda") << torch.arange(64, device="cuda", dtype=torch.int64)
+    obs_words = (pad.view(words, 64).to(torch.int64) * weights).sum(dim=1)  # bit 63 is the sign bit of the same word
+    del pad
+    ws = torch.zeros(hip.lib().ugk_rank_workspace_bytes() // 4 + 8, dtype=torch.int32, device="cuda")
+    in_new = torch.empty(words, dtype=torch.int64, device="cuda")
+    scratch = torch.empty(words, dtype=torch.int64, device="cuda")
+    torch.cuda.synchronize()
+    reps = 5 if quick else 10
+    res = {"rows": rows, "rows_observed": observed_n}
+    for k in (rows // 10, rows // 25):
+        r = {}
+
+        def place(reset, observed):
+            hip.call("ugk_rank_place", counts.data_ptr(), rows, k, ws.data_ptr(), in_new.data_ptr(), scratch.data_ptr(),
+                     obs_words.data_ptr() if observed else None, reset, stream)
+
+        us = _timed(hip, stream, lambda i: place(0, False), reps)
+        r["counters_kept_guess_right"] = round(us, 1)
+        other = rows // 3
+
+        def place_after_another(i):
+            hip.call("ugk_rank_place", counts.data_ptr(), rows, other if i % 2 == 0 else k, ws.data_ptr(),
+                     in_new.data_ptr(), scratch.data_ptr(), None, 0, stream)
+
+        us2 = _timed(hip, stream, place_after_another, 2 * reps, warm=2)
+        r["counters_kept_alternating_with_another_k_per_pair"] = round(2 * us2, 1)
+
+        def place_reset(i):
+            hip.call("ugk_copy_rows", counts.data_ptr(), saved.data_ptr(), rows * 4, stream)
+            place(1, False)
+
+        us_copy = _timed(hip, stream, lambda i: hip.call("ugk_copy_rows", counts.data_ptr(), saved.data_ptr(), rows * 4,
+                                                         stream), reps)
+        us3 = _timed(hip, stream, place_reset, reps)
+        r["counters_reset_two_passes"] = round(us3 - us_copy, 1)
+        hip.call("ugk_copy_rows", counts.data_ptr(), saved.data_ptr(), rows * 4, stream)
+        us4 = _timed(hip, stream, lambda i: place(0, True), reps)
+        r["counters_kept_with_observed_bitmap"] = round(us4, 1)
+        res["k=%d" % k] = r
+        note("k=%d: %s" % (k, r))
+    return {"probe": "placement", "launches_timed": reps, "unit": "us per placement, 2 HIP events around the launches",
+            "sizes": res}
+
+
+PROBES = {"placement": probe_placement, "rw_ceiling": probe_rw_ceiling, "link_latency": probe_link_latency, "sparse_layer": probe_sparse_layer, "pooled": probe_pooled, "kpw": probe_kpw, "row_span": probe_row_span, "cu_mask": probe_cu_mask, "small_batch": probe_small_batch}
 
 
 def run(name, quick=False):

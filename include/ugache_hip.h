@@ -468,6 +468,10 @@ int ugk_record_restore(const uint64_t *entries_dev, size_t n, uint32_t *counts_d
  * ugk_rank_place: bit r of in_new_dev (ceil(num_rows / 64) words, every word written) = row r is one of the k
  * best-ranked rows of [0, num_rows) (k == 0: no row; k >= num_rows: every row).  Two streaming passes over the
  * counters (five when the k-th best count is 2047 or more) and a few launches over bitmaps; no host round trip.
+ * With reset_counts == 0 the first pass also splits the rows by the k-th best count of the placement that used ws_dev
+ * last, and when that count still is the k-th best (counters that are kept only grow, it moves slowly) the second
+ * pass is skipped: one pass over the counters, 0.47 against 0.87 ms at 500 M rows.  The result does not depend on
+ * what ws_dev held; give the placements of one cache one workspace.
  * counts_dev must be 16-byte aligned; num_rows < 2^32 - 1; ws_dev: ugk_rank_workspace_bytes() bytes, 8-byte aligned;
  * scratch_bitmap_dev: as large as in_new_dev, overwritten.  With reset_counts != 0 the counters (and observed_dev)
  * are zeroed on the way.  observed_dev (may be NULL): the bitmap ugk_record_* keeps; when fewer rows were observed

@@ -36,13 +36,15 @@ def _counts(rng, n, kind):
     raise AssertionError(kind)
 
 
-def _place(counts, k, reset, with_observed=False, keep=None):
+def _place(counts, k, reset, with_observed=False, keep=None, ws=None):
     """-> membership bits of the k best rows, the rank threshold, the counters afterwards.
-    keep (bool per row, optional): rows that win ties at the k-th count (ugk_rank_place_keep)"""
+    keep (bool per row, optional): rows that win ties at the k-th count (ugk_rank_place_keep);
+    ws (optional): a workspace that earlier placements have used"""
     n = len(counts)
     words = (n + 63) // 64
     d_counts = to_dev(counts)
-    ws = dev_bytes(hip.lib().ugk_rank_workspace_bytes())
+    if ws is None:
+        ws = dev_bytes(hip.lib().ugk_rank_workspace_bytes())
     bitmap = dev_bytes(words * 8, fill=0xA5)
     scratch = dev_bytes(words * 8, fill=0x5A)
     observed = None
@@ -92,6 +94,42 @@ def test_rank_place_matches_a_full_sort(kind, n):
                 assert th == int(order[k - 1]), (kind, n, k, with_observed)
             assert np.array_equal(got, want), (kind, n, k, reset, with_observed)
             assert np.array_equal(left, counts if reset == 0 else np.zeros(n, np.uint32))
+
+
+@pytest.mark.parametrize("kind", ["zipf", "ties", "saturated"])
+@pytest.mark.parametrize("n", [65, 1000, 100_003, 2_000_001])
+def test_placements_that_share_a_workspace(kind, n):
+    """With the counters kept, the first pass over them splits by the threshold count of the placement before (left in
+    the workspace) and the second pass is skipped when that guess holds.  A sequence of placements in one workspace -
+    the same one again (guess right), counters grown a little (mostly right), another k (wrong), counters grown a lot
+    (wrong), a placement with a reset in between (two passes, as before) - gives what a full sort gives every time."""
+    rng = np.random.default_rng(n * 3 + len(kind))
+    counts = _counts(rng, n, kind)
+    ws = dev_bytes(hip.lib().ugk_rank_workspace_bytes(), fill=0xC3)  # whatever the memory held: a guess like any other
+    observed = int((counts > 0).sum())
+    k0 = max(1, min(observed // 2, n - 1))
+    steps = [("same", k0), ("same", k0), ("grow_a_little", k0), ("same", max(1, k0 // 3)), ("grow_a_lot", k0),
+             ("reset", k0), ("same", k0), ("same", min(n - 1, max(1, observed + 1)))]
+    for what, k in steps:
+        if what == "grow_a_little":
+            counts = counts.copy()
+            counts[rng.integers(0, n, size=max(n // 200, 1))] += 1
+        elif what == "grow_a_lot":
+            counts = (counts + rng.integers(0, 4, size=n)).astype(np.uint32)
+        ranks = ranks_of(counts)
+        order = np.sort(ranks)[::-1]
+        want = ranks >= order[k - 1]
+        for keep in (None, rng.random(n) < 0.5):
+            if keep is not None:
+                rows = np.arange(n, dtype=np.int64)
+                best = np.lexsort((np.where(counts > 0, rows, -rows), keep, counts))[::-1]
+                want_k = np.zeros(n, bool)
+                want_k[best[:k]] = True
+            got, th, left = _place(counts, k, 1 if what == "reset" else 0, with_observed=(n % 2 == 1), keep=keep, ws=ws)
+            assert np.array_equal(got, want if keep is None else want_k), (kind, n, what, k, keep is not None)
+            if keep is None:
+                assert th == int(order[k - 1])
+            assert np.array_equal(left, np.zeros(n, np.uint32) if what == "reset" else counts)
 
 
 def test_rank_place_picks_the_hotter_rows_and_breaks_ties_towards_larger_rows():
