@@ -1603,13 +1603,79 @@ void RefreshSession::refresh_on_device(ExtractSession *session, size_t num_cache
       num_cached, table->InNewBits(), table->_dev_scratch_bits->ptr<uint64_t>(),
       RunConfig::gpu_refresh_stable ? table->InCacheBits() : nullptr, table->_dev_rank_ws->ptr(),
       !RunConfig::gpu_refresh_keep, &diff, stream);
-  volatile uint32_t *n_evict_word = table->DevWords() + 8, *n_insert_word = table->DevWords() + 9;
-  if (!counted) {
-    n_evict_word = table->CountBits(table->InCacheBits(), table->InNewBits(), false, num_rows, 0, stream);
-    n_insert_word = table->CountBits(table->InNewBits(), table->InCacheBits(), false, num_rows, 1, stream);
+  if (!counted) {  // into the same two pinned words
+    table->CountBits(table->InCacheBits(), table->InNewBits(), false, num_rows, 0, stream);
+    table->CountBits(table->InNewBits(), table->InCacheBits(), false, num_rows, 1, stream);
   }
+  ApplyPlacedBits(session, num_cached, foreground, stage, true,
+                  counted ? "placement (from the observed rows alone)" : "placement", sync_s, t_phase);
+}
+
+// A refresh whose placement the host has ranked (FreqRecorder + solver: the default) applied like one computed on the
+// device.  The placement arrives as what it was computed from: the ranked rows that are cached and how many of the
+// lowest other rows fill the rest.  Their bits make the bitmap of rows cached after the refresh; what leaves and what
+// comes in are its differences with the bitmap of rows cached now.  No array over the key space is written or
+// scanned on the host (config 5: 2 GB written by the solver and read by the key-list scan, 0.45 s of a 0.48 s
+// refresh).
+void RefreshSession::refresh_from_ranked_rows(ExtractSession *session, TensorPtr top_rows, size_t num_extra,
+                                              bool foreground) {
+  CacheContext *ctx = _cache_ctx.get();
+  auto table = ctx->_new_hash_table;
+  CHECK_NOTNULL(table) << "refresh needs a partial cache (0 < cache_percentage < 1)";
+  CHECK_NOTNULL(top_rows);
+  const Context gpu_ctx = ctx->_trainer_ctx;
+  const auto &alloc = ctx->_eager_gpu_mem_allocator;
+  const size_t num_rows = ctx->_num_total_nodes;
+  const size_t num_top = top_rows->NumItem(), num_cached = num_top + num_extra;
+  CHECK_LE(num_cached, (size_t)ctx->_cache_space_capacity) << "cache space can not hold refreshed new cache";
+  CHECK_LT(num_cached, num_rows);
+  UGK_CALL(ugk_set_device(gpu_ctx.device_id));
+  if (low_pri_stream == nullptr) UGK_CALL(ugk_stream_create(&low_pri_stream));
+  if (!_status_handle) {
+    _status_handle = EagerGPUAlloc(gpu_ctx.device_id, 256);
+    UGK_CALL(ugk_fill_u32(_status_handle->ptr<uint32_t>(), 0, 64, stream));
+  }
+  const ugk_stage_t *stage = session ? session->StageForRefresh(foreground, stream) : nullptr;
+  Timer t_phase;
+  table->EnsureDeviceLists(alloc, gpu_ctx, stream);
+  const double sync_s = t_phase.Passed();
+  t_phase.Reset();
+  const size_t words = (num_rows + 63) / 64;
+  // the ranked rows' bits: straight into the new bitmap when they are all of it, else into the scratch bitmap, from
+  // which the placement adds the lowest rows that are not among them
+  uint64_t *ranked_bits = num_extra ? table->_dev_scratch_bits->ptr<uint64_t>() : table->InNewBits();
+  UGK_CALL(ugk_fill_u32(reinterpret_cast<uint32_t *>(ranked_bits), 0, words * 2, stream));
+  if (num_top > 0) {
+    TensorPtr top_dev = CopyTo1DReuse(__ranked_rows, top_rows, gpu_ctx, stream);
+    UGK_CALL(ugk_bitmap_update(ranked_bits, num_rows, top_dev->CPtr<uint32_t>(), num_top, 1,
+                               _status_handle->ptr<uint32_t>(), stream));
+  }
+  if (num_extra > 0) {
+    UGK_CALL(ugk_rank_place_observed(nullptr, num_rows, num_cached, table->_dev_rank_ws->ptr(), table->InNewBits(),
+                                     ranked_bits, 0, table->InCacheBits(), table->_dev_bm_ws->ptr(),
+                                     table->_dev_bm_ws2->ptr(), table->DevWords() + 8,
+                                     _status_handle->ptr<uint32_t>(), stream));
+  } else {
+    table->CountBits(table->InCacheBits(), table->InNewBits(), false, num_rows, 0, stream);
+    table->CountBits(table->InNewBits(), table->InCacheBits(), false, num_rows, 1, stream);
+  }
+  ApplyPlacedBits(session, num_cached, foreground, stage, false, "placement ranked on the host", sync_s, t_phase);
+}
+
+// The second half of a refresh whose new placement stands in the table's bitmap of rows cached after it, with the two
+// counts (rows that leave, rows that come in) on their way into the pinned words 8 and 9: waits for the counts, lists
+// evict = cached & ~new and insert = new & ~cached, then steps 4 - 6 of refresh_after_solve_new on device lists.
+void RefreshSession::ApplyPlacedBits(ExtractSession *session, size_t num_cached, bool foreground,
+                                     const ugk_stage_t *stage, bool placed_from_counters, const char *how,
+                                     double sync_s, Timer &t_phase) {
+  CacheContext *ctx = _cache_ctx.get();
+  auto table = ctx->_new_hash_table;
+  const Context gpu_ctx = ctx->_trainer_ctx;
+  const auto &alloc = ctx->_eager_gpu_mem_allocator;
+  const size_t num_rows = ctx->_num_total_nodes, capacity = ctx->_cache_space_capacity;
+  volatile uint32_t *n_evict_word = table->DevWords() + 8, *n_insert_word = table->DevWords() + 9;
   table->WaitByTicket(stream);
-  session->PlacementWaitedFor();
+  if (placed_from_counters) session->PlacementWaitedFor();
   const size_t num_evicted = *n_evict_word, num_insert = *n_insert_word;
   TensorPtr evict_rows, insert_rows;  // both lists in one pass over the two bitmaps
   table->EmitDiff(table->InCacheBits(), table->InNewBits(), num_rows, num_evicted, num_insert, __evict_rows,
@@ -1685,11 +1751,10 @@ void RefreshSession::refresh_on_device(ExtractSession *session, size_t num_cache
   table->_host_lists_valid = false;  // the bitmaps hold the truth now
   table->_cached_keys_on_device = nullptr;
   ctx->_cache_nodes = table->_num_cached;
-  const bool rebuilt = table->MaybeRebuild(alloc, gpu_ctx, local, stream, [&]() {
-    session->WaitForLookupsInFlight(foreground, 20.0);
+  const bool rebuilt = table->MaybeRebuild(alloc, gpu_ctx, ctx->_local_location_id, stream, [&]() {
+    if (session) session->WaitForLookupsInFlight(foreground, 20.0);
   });
-  LOG(INFO) << "refresh on the device: bitmaps " << sync_s << " s, placement"
-            << (counted ? " (from the observed rows alone)" : "") << " + key lists " << place_s << " s, evict "
+  LOG(INFO) << "refresh on the device: bitmaps " << sync_s << " s, " << how << " + key lists " << place_s << " s, evict "
             << evict_s << " s, wait for a lookup " << wait_s << " s, row copy + insert " << insert_s
             << " s (" << from_stage << " of " << num_insert << " rows from the stage), table rebuild "
             << (rebuilt ? t_phase.Passed() : 0.0) << " s";

@@ -20,6 +20,7 @@
 #include "freq_recorder.h"
 #include "profiler.h"
 #include "run_config.h"
+#include "timer.h"
 #include "ugache_hip.h"
 
 namespace coll_cache_lib {
@@ -362,10 +363,15 @@ class RefreshSession {
   // `session`, evict = cached & ~new and insert = new & ~cached as bitmap compactions, free slots from the slot bitmap;
   // then the same evict / wait / copy / insert steps as refresh_after_solve_new (cache_context.cu:3944-4107).
   void refresh_on_device(ExtractSession *session, size_t num_cached, bool foreground);
+  // A placement ranked on the host, given as the ranked rows that are cached (distinct) plus `num_extra` of the lowest
+  // other rows, applied through the same bitmaps and device lists (session may be null: no lookups to wait for).
+  void refresh_from_ranked_rows(ExtractSession *session, TensorPtr top_rows, size_t num_extra, bool foreground);
   ~RefreshSession();
 
  private:
   void refresh_after_solve_new(bool foreground);
+  void ApplyPlacedBits(ExtractSession *session, size_t num_cached, bool foreground, const ugk_stage_t *stage,
+                       bool placed_from_counters, const char *how, double sync_s, common::Timer &t_phase);
   TensorPtr Empty1DReuse(TensorPtr &preserved_buffer, DataType dtype, std::vector<size_t> shape, Context ctx);
   TensorPtr CopyTo1DReuse(TensorPtr &preserved_buffer, TensorPtr src, Context ctx, StreamHandle stream);
   // step 5: lets one more lookup finish, so that no gather in flight still reads a slot about to be reused
@@ -385,6 +391,7 @@ class RefreshSession {
   TensorPtr __keys_buffer;
   TensorPtr __offs_buffer;
   TensorPtr __evict_rows, __insert_rows, __free_slots, __evict_ids, __evict_slots;
+  TensorPtr __ranked_rows;  // device copy of the rows a host-ranked placement caches
   MemHandle _status_handle;
 };
 

@@ -240,11 +240,22 @@ void CollCache::refresh(int replica_id, IdType *ranking_nodes_list_ptr, IdType *
   CHECK(HasPartialPlacement()) << "refresh needs a cache built with 0 < cache_percentage < 1";
   AnonymousBarrier::_refresh_instance->Wait();
   preserve_old_solution();
-  solve_impl_master(ranking_nodes_list_ptr, ranking_nodes_freq_list_ptr, (IdType)RunConfig::num_total_item);
+  solve_impl_master(ranking_nodes_list_ptr, ranking_nodes_freq_list_ptr, (IdType)RunConfig::num_total_item,
+                    RunConfig::device_key_list);
   AnonymousBarrier::_refresh_instance->Wait();
-  this->_refresh_session_list[replica_id]->stream = stream;
-  this->_refresh_session_list[replica_id]->refresh_after_solve_main(foreground);
+  apply_solution(replica_id, stream, foreground);
   AnonymousBarrier::_refresh_instance->Wait();
+}
+
+// The new placement replaces the old one in the cache.  By default (COLL_DEVICE_KEY_LIST) the solver has left the
+// key -> block array unwritten and the placement goes to the device as the rows it was computed from.
+void CollCache::apply_solution(int replica_id, StreamHandle stream, bool foreground) {
+  auto &refresher = this->_refresh_session_list[replica_id];
+  refresher->stream = stream;
+  if (_placed_top_rows != nullptr)
+    refresher->refresh_from_ranked_rows(_session_list[replica_id].get(), _placed_top_rows, _placed_extra, foreground);
+  else
+    refresher->refresh_after_solve_main(foreground);
 }
 
 // facade.cc:513-557
@@ -254,12 +265,11 @@ void CollCache::refresh(int replica_id, ContFreqBuf *freq_rank, StreamHandle str
   AnonymousBarrier::_refresh_instance->Wait();
   Timer t_solve;
   preserve_old_solution();
-  solve_impl_master(freq_rank, (IdType)RunConfig::num_total_item);
+  solve_impl_master(freq_rank, (IdType)RunConfig::num_total_item, RunConfig::device_key_list);
   const double solve_s = t_solve.Passed();
   AnonymousBarrier::_refresh_instance->Wait();
   Timer t_apply;
-  this->_refresh_session_list[replica_id]->stream = stream;
-  this->_refresh_session_list[replica_id]->refresh_after_solve_main(foreground);
+  apply_solution(replica_id, stream, foreground);
   AnonymousBarrier::_refresh_instance->Wait();
   LOG(INFO) << "refresh: placement " << solve_s << " s, evict + insert " << t_apply.Passed() << " s";
 }

@@ -47,6 +47,7 @@ class CollCache : public std::enable_shared_from_this<CollCache> {
   TensorPtr EnsureNidToBlock();
   bool HasPartialPlacement() const { return _nid_to_block != nullptr || _placed_top_rows != nullptr; }
   void preserve_old_solution();
+  void apply_solution(int replica_id, StreamHandle stream, bool foreground);
   void build_common(int replica_id, std::function<void()> solve, IdType num_node,
                     std::function<MemHandle(size_t)> gpu_mem_allocator, void *cpu_data, DataType dtype, size_t dim,
                     double cache_percentage, StreamHandle stream);
