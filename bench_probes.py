@@ -634,42 +634,46 @@ def probe_rw_ceiling(hip, torch, note, quick=False):
     """What the two sides of the all-hit gather reach alone, on its own shapes: random 512-byte rows of a 5.12 GB table
     read and nothing written (bp_rows_inflight), a buffer written and nothing read (ugk_fill_u32), a plain copy
     (ugk_copy_rows), and the gather itself (ugk_gather_direct_u32) -- each with an output that stays in the 256 MB
-    memory-side cache (134 MB, rewritten every launch) and with one that cannot (1 GiB)."""
+    memory-side cache (134 MB, rewritten every launch) and with one that cannot (1 GiB).  Then the same for random
+    128-byte rows of a 6.4 GB table (configuration 5's cache), 1 M rows per launch."""
     call = _probe_lib()
     stream = C.c_void_p()
     hip.call("ugk_stream_create", C.byref(stream))
-    rows, rb = 10_000_000, 512
-    table = torch.empty(rows * rb // 4, dtype=torch.int32, device="cuda")
-    hip.call("ugk_arange_u32", table.data_ptr(), 1, table.numel(), stream)
     g = torch.Generator(device="cuda").manual_seed(3)
     st = torch.zeros(4, dtype=torch.int32, device="cuda")
     res = {}
     reps = 10 if quick else 30
-    for n in (262_144, 2_097_152):
-        nbytes = n * rb
-        keys = torch.randint(0, rows, (4, n), generator=g, device="cuda", dtype=torch.int32)
-        out = torch.empty(nbytes // 4, dtype=torch.int32, device="cuda")
-        src = torch.empty(nbytes // 4, dtype=torch.int32, device="cuda")
-        sink = torch.zeros(8192 * 256, dtype=torch.int32, device="cuda")
-        torch.cuda.synchronize()
-        r = {}
-        us = min(_timed(hip, stream, lambda i, u=u, w=w: call("bp_rows_inflight", table.data_ptr(), rb, keys[i % 4].data_ptr(),
-                                                              n, u, w, sink.data_ptr(), stream), reps)
-                 for u in (2, 4, 8) for w in (2048, 8192))
-        r["random_rows_read_only"] = {"us": round(us, 2), "TBps": round(nbytes / us / 1e6, 3)}
-        us = _timed(hip, stream, lambda i: hip.call("ugk_fill_u32", out.data_ptr(), i + 1, nbytes // 4, stream), reps)
-        r["write_only"] = {"us": round(us, 2), "TBps": round(nbytes / us / 1e6, 3)}
-        us = _timed(hip, stream, lambda i: hip.call("ugk_copy_rows", out.data_ptr(), src.data_ptr(), nbytes, stream), reps)
-        r["plain_copy"] = {"us": round(us, 2), "TBps_read_plus_written": round(2 * nbytes / us / 1e6, 3)}
-        us = _timed(hip, stream, lambda i: hip.call("ugk_gather_direct_u32", table.data_ptr(), rows, keys[i % 4].data_ptr(), n,
-                                                    out.data_ptr(), rb, 0, st.data_ptr(), None, stream), reps)
-        r["gather"] = {"us": round(us, 2), "TBps_read_plus_written": round((2 * nbytes + 4 * n) / us / 1e6, 3)}
-        res["%d rows of 512 B (%d MB out)" % (n, nbytes >> 20)] = r
-        note("%d rows: %s" % (n, r))
-        del keys, out, src, sink
+    for rows, rb, sizes in ((10_000_000, 512, (262_144, 2_097_152)), (50_000_000, 128, (1_048_576,))):
+        table = torch.empty(rows * rb // 4, dtype=torch.int32, device="cuda")
+        hip.call("ugk_arange_u32", table.data_ptr(), 1, table.numel(), stream)
+        for n in sizes:
+            nbytes = n * rb
+            keys = torch.randint(0, rows, (4, n), generator=g, device="cuda", dtype=torch.int32)
+            out = torch.empty(nbytes // 4, dtype=torch.int32, device="cuda")
+            src = torch.empty(nbytes // 4, dtype=torch.int32, device="cuda")
+            sink = torch.zeros(8192 * 256, dtype=torch.int32, device="cuda")
+            torch.cuda.synchronize()
+            r = {}
+            us = min(_timed(hip, stream, lambda i, u=u, w=w: call("bp_rows_inflight", table.data_ptr(), rb,
+                                                                  keys[i % 4].data_ptr(), n, u, w, sink.data_ptr(), stream),
+                            reps)
+                     for u in (2, 4, 8) for w in (2048, 8192))
+            r["random_rows_read_only"] = {"us": round(us, 2), "TBps": round(nbytes / us / 1e6, 3)}
+            us = _timed(hip, stream, lambda i: hip.call("ugk_fill_u32", out.data_ptr(), i + 1, nbytes // 4, stream), reps)
+            r["write_only"] = {"us": round(us, 2), "TBps": round(nbytes / us / 1e6, 3)}
+            us = _timed(hip, stream, lambda i: hip.call("ugk_copy_rows", out.data_ptr(), src.data_ptr(), nbytes, stream), reps)
+            r["plain_copy"] = {"us": round(us, 2), "TBps_read_plus_written": round(2 * nbytes / us / 1e6, 3)}
+            us = _timed(hip, stream, lambda i: hip.call("ugk_gather_direct_u32", table.data_ptr(), rows, keys[i % 4].data_ptr(),
+                                                        n, out.data_ptr(), rb, 0, st.data_ptr(), None, stream), reps)
+            r["gather"] = {"us": round(us, 2), "TBps_read_plus_written": round((2 * nbytes + 4 * n) / us / 1e6, 3)}
+            res["%d rows of %d B (%d MB out)" % (n, rb, nbytes >> 20)] = r
+            note("%d rows of %d B: %s" % (n, rb, r))
+            del keys, out, src, sink
+            torch.cuda.empty_cache()
+        del table
         torch.cuda.empty_cache()
     _check_status(torch, st, "rw_ceiling")
-    return {"probe": "rw_ceiling", "table": "10 M rows of 512 bytes in HBM", "launches_timed": reps,
+    return {"probe": "rw_ceiling", "tables": "10 M rows of 512 bytes, 50 M rows of 128 bytes, in HBM", "launches_timed": reps,
             "how": "2 HIP events around the launches; read-only: best of 2, 4, 8 loads per lane x 2048, 8192 workgroups",
             "sizes": res}
 
