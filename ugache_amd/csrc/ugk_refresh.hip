@@ -208,7 +208,11 @@ __global__ __launch_bounds__(kBlock) void rank_split_kernel(uint32_t *counts, ui
         my_gt = above;
         my_eq = equal;
       }
-      if (reset_counts && row < n && c[k] != 0) counts[row] = 0;
+      // a group of 64 counters with any of them above zero is cleared as a whole: two full lines written, where the
+      // counters above zero alone would be partial writes that the memory side turns into a read and a write each
+      // (500 M counters, 43 M of them above zero: the placement takes 1.13 ms this way and took 1.67 ms the other)
+      const bool any_counted = __ballot(row < n && c[k] != 0) != 0ull;
+      if (reset_counts && any_counted && row < n) counts[row] = 0;
     }
     if (lane < kMarkWords && w0 + lane < n_words) {
       gt[w0 + lane] = my_gt;
