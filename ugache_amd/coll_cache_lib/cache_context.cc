@@ -201,7 +201,9 @@ void CacheContext::build_with_advise_new_hash(int location_id, std::shared_ptr<C
 
   const double alloc_s = t.Passed() - detect_s;
   // 4. fill: rows of the cached keys host -> HBM in list order, slot = position in the list.  The copy is bound by
-  //    the host link.  (The table insert beside the copy, on a second stream, instead of behind it, was measured at
+  //    the host link, which answers a grid of 128 workgroups a little faster than one that fills the chip (12.8 GB of
+  //    512-byte rows: 0.235 against 0.243 s; 6.4 GB of 128-byte rows: 0.131 against 0.137 s; 64 and 1,024 workgroups
+  //    are no better than the full grid).  (The table insert beside the copy, on a second stream, instead of behind it, was measured at
   //    500M rows / 50M cached: the step went from 0.140 to 0.178 s, the link-bound copy kernel loses more than the
   //    insert takes.)
   if (num_cached_nodes > 0) {
@@ -211,8 +213,9 @@ void CacheContext::build_with_advise_new_hash(int location_id, std::shared_ptr<C
     MemHandle st = _eager_gpu_mem_allocator(256);
     UGK_CALL(ugk_fill_u32(st->ptr<uint32_t>(), 0, 1, stream));
     UGK_CALL(ugk_gather_direct_u32(cpu_data, num_total_nodes, cache_node_list->CPtr<uint32_t>(), num_cached_nodes,
-                                   _device_cache_data[_local_location_id], _row_bytes, 0, st->ptr<uint32_t>(),
-                                   nullptr, stream));
+                                   _device_cache_data[_local_location_id], _row_bytes,
+                                   PointerKind(cpu_data) == 1 ? RunConfig::fill_limit_block : 0u,  // 2: a table in HBM
+                                   st->ptr<uint32_t>(), nullptr, stream));
     // (8-byte entries are keyed by the row: no id list)
     TensorPtr id_buffer;
     auto table_keys = RunConfig::key_map_mul == 0 || _new_hash_table->_table.kind == 3 ? cache_node_list

@@ -34,6 +34,7 @@ coll_cache::AsymmLinkDesc RunConfig::coll_cache_link_desc;
 double RunConfig::hash_load_factor = 0.7;
 int RunConfig::force_table_kind = 0;
 bool RunConfig::device_key_list = true;
+unsigned RunConfig::fill_limit_block = 128;
 size_t RunConfig::refresh_batch_rows = 4092;
 unsigned RunConfig::refresh_sleep_us = 3000;
 unsigned RunConfig::refresh_limit_block = 20;
@@ -79,6 +80,7 @@ void RunConfig::LoadConfigFromEnv() {
   hash_load_factor = 0.7;
   force_table_kind = 0;
   device_key_list = true;
+  fill_limit_block = 128;
   refresh_batch_rows = 4092;
   refresh_sleep_us = 3000;
   refresh_limit_block = 20;
@@ -118,6 +120,7 @@ void RunConfig::LoadConfigFromEnv() {
   if (GetEnv("COLL_CACHE_SCALE") != "") coll_cache_scale_nb = std::stoul(GetEnv("COLL_CACHE_SCALE"));
   if (GetEnv("COLL_HASH_LOAD_FACTOR") != "") hash_load_factor = std::stod(GetEnv("COLL_HASH_LOAD_FACTOR"));
   if (GetEnv("COLL_DEVICE_KEY_LIST") != "") device_key_list = GetEnv("COLL_DEVICE_KEY_LIST") != "0";
+  if (GetEnv("COLL_FILL_LIMIT_BLOCK") != "") fill_limit_block = (unsigned)std::stoul(GetEnv("COLL_FILL_LIMIT_BLOCK"));
   const std::string tbl = GetEnv("COLL_HASH_TABLE");
   if (tbl == "FLAT") force_table_kind = 1;
   else if (tbl == "HASH") force_table_kind = 2;

@@ -61,6 +61,8 @@ struct RunConfig {
   static bool device_key_list;         // COLL_DEVICE_KEY_LIST, default 1: a build gets its ascending list of cached
                                        // rows from a bitmap on the device instead of from a key -> block array
                                        // over the whole key space on the host
+  static unsigned fill_limit_block;    // COLL_FILL_LIMIT_BLOCK, default 128: workgroups of a build's row copy over the
+                                       // host link (0: as many as the rows fill)
   static double hash_load_factor;      // COLL_HASH_LOAD_FACTOR, default 0.7
   static int force_table_kind;         // COLL_HASH_TABLE=FLAT|HASH|HASH16|HASH8 -> 1|2|16|8, 0 = decide by size;
                                        // HASH picks the entry width itself, HASH16 / HASH8 name it (bytes)
