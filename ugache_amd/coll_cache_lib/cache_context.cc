@@ -74,7 +74,8 @@ void CacheContext::build_full_cache(int location_id, std::shared_ptr<CollCache> 
 // the ascending list of the rows a placement caches, made on the device: bit r of a bitmap over the key space = row r
 // is cached (the ranked rows that are cached, then the lowest `num_extra` rows that are not among them), compacted in
 // order.  Waits for `stream`: the list is complete on return.
-TensorPtr CacheContext::KeyListOnDevice(TensorPtr top_rows, size_t num_extra, size_t num_rows, StreamHandle stream) {
+TensorPtr CacheContext::KeyListOnDevice(TensorPtr top_rows, size_t num_extra, size_t num_rows, StreamHandle stream,
+                                        MemHandle *bits_out) {
   CHECK_NOTNULL(top_rows);
   const size_t num_top = top_rows->NumItem(), num_cached = num_top + num_extra;
   CHECK_LT(num_cached, num_rows);
@@ -112,6 +113,7 @@ TensorPtr CacheContext::KeyListOnDevice(TensorPtr top_rows, size_t num_extra, si
   TensorPtr list = Tensor::EmptyExternal(kI32, {num_cached}, _eager_gpu_mem_allocator, _trainer_ctx, "");
   UGK_CALL(ugk_bitmap_emit(cached, nullptr, 0, num_rows, bm_ws->ptr(), list->Ptr<uint32_t>(), num_cached, stream));
   UGK_CALL(ugk_stream_sync(stream));  // the bitmaps go out of scope
+  if (bits_out) *bits_out = num_extra > 0 ? placed : ranked;
   return list;
 }
 
@@ -154,8 +156,11 @@ void CacheContext::build_with_advise_new_hash(int location_id, std::shared_ptr<C
       CPU_CLIB(), "advise_line");
   TensorPtr cache_node_list;  // on the device, ascending
   if (list_on_device) {
+    // the bitmap the list comes from is what the first refresh needs to know of this placement: the table keeps it
+    MemHandle cached_bits;
     cache_node_list = KeyListOnDevice(coll_cache_ptr->_placed_top_rows, coll_cache_ptr->_placed_extra,
-                                      num_total_nodes, stream);
+                                      num_total_nodes, stream, &cached_bits);
+    _new_hash_table->AdoptBuildBits(cached_bits);
   } else {
     CacheEntryManager::DetectKeysForAllSource(coll_cache_ptr->_nid_to_block, advise_line, location_id,
                                               coll_cache_ptr->_block_density, num_total_nodes, keys_for_each_source,
@@ -1489,6 +1494,7 @@ void RefreshSession::refresh_after_solve_new(bool foreground) {
   const ugk_stage_t *stage = nullptr;
   if (auto s0 = coll_cache->session(ctx->_local_location_id)) stage = s0->StageForRefresh(foreground, stream);
   table->EnsureHostLists(ctx->_eager_gpu_mem_allocator, gpu_ctx, stream);  // after a refresh on the device
+  table->DropBuildBits();  // this refresh goes through the host's lists
   // Step 1: key list of the new placement
   Timer t_phase;
   double detect_s = 0, evict_s = 0, wait_s = 0, insert_s = 0;

@@ -66,7 +66,9 @@ class CacheContext {
                       size_t dim, Context gpu_ctx, StreamHandle stream = nullptr);
   void build_full_cache(int location_id, std::shared_ptr<CollCache> coll_cache_ptr, void *cpu_data, DataType dtype,
                         size_t dim, Context gpu_ctx, size_t num_total_nodes, StreamHandle stream = nullptr);
-  TensorPtr KeyListOnDevice(TensorPtr top_rows, size_t num_extra, size_t num_rows, StreamHandle stream);
+  // bits_out (optional): receives the bitmap the list was compacted from (bit r = row r is cached)
+  TensorPtr KeyListOnDevice(TensorPtr top_rows, size_t num_extra, size_t num_rows, StreamHandle stream,
+                            MemHandle *bits_out = nullptr);
   void build_with_advise_new_hash(int location_id, std::shared_ptr<CollCache> coll_cache_ptr, void *cpu_data,
                                   DataType dtype, size_t dim, Context gpu_ctx, double cache_percentage,
                                   StreamHandle stream = nullptr);

@@ -308,8 +308,8 @@ void CacheEntryManager::PublishRows(const uint32_t *rows_dev, const uint32_t *sl
 void CacheEntryManager::EnsureDeviceLists(const std::function<MemHandle(size_t)> &allocator, Context ctx,
                                           StreamHandle stream) {
   const size_t row_words = (num_total_key + 63) / 64, slot_words = ((size_t)_cache_space_capacity + 63) / 64;
-  if (!_dev_in_cache) {
-    _dev_in_cache = EagerGPUAlloc(_device_id, row_words * 8);
+  if (!_dev_words) {
+    if (!_dev_in_cache) _dev_in_cache = EagerGPUAlloc(_device_id, row_words * 8);  // else: the build's bitmap
     _dev_in_new = EagerGPUAlloc(_device_id, row_words * 8);
     _dev_scratch_bits = EagerGPUAlloc(_device_id, row_words * 8);
     _dev_slot_used = EagerGPUAlloc(_device_id, std::max<size_t>(slot_words, 1) * 8);
@@ -321,9 +321,25 @@ void CacheEntryManager::EnsureDeviceLists(const std::function<MemHandle(size_t)>
   }
   if (_dev_lists_valid) return;
   CHECK(_host_lists_valid);
-  UGK_CALL(ugk_fill_u32(_dev_in_cache->ptr<uint32_t>(), 0, row_words * 2, stream));
-  UGK_CALL(ugk_fill_u32(_dev_slot_used->ptr<uint32_t>(), 0, std::max<size_t>(slot_words, 1) * 2, stream));
   const size_t n = NumCached();
+  UGK_CALL(ugk_fill_u32(_dev_slot_used->ptr<uint32_t>(), 0, std::max<size_t>(slot_words, 1) * 2, stream));
+  if (_build_bits_fresh) {
+    // nothing has changed the cache since the build: its bitmap stands, its rows sit in slots 0 .. n - 1
+    _build_bits_fresh = false;
+    CHECK_EQ(_free_offsets->NumItem() + n, (size_t)_cache_space_capacity);
+    if (n > 0) {
+      uint32_t *status = StatusPtr(this, stream);
+      uint32_t *last = status + 32;  // a device word for the position of the last slot taken
+      UGK_CALL(ugk_fill_u32(last, (uint32_t)(n - 1), 1, stream));
+      UGK_CALL(ugk_bitmap_set_through(SlotUsedBits(), _cache_space_capacity, last, status, stream));
+      CheckStatus(stream, "placement bitmaps");
+    }
+    _num_cached = n;
+    _num_free = _free_offsets->NumItem();
+    _dev_lists_valid = true;
+    return;
+  }
+  UGK_CALL(ugk_fill_u32(_dev_in_cache->ptr<uint32_t>(), 0, row_words * 2, stream));
   if (n > 0) {
     TensorPtr rows = _cached_keys_on_device;  // the list of the build, if it is still on the device
     if (!rows) {

@@ -108,6 +108,7 @@ class CacheEntryManager {
   MemHandle _dev_rank_ws, _dev_bm_ws;    // workspaces of ugk_rank_* / ugk_bitmap_*
   MemHandle _dev_bm_ws2;                 // a second one, so that two compactions can be counted before one wait
   MemHandle _dev_words;                  // pinned host words the kernels report counts in
+  bool _build_bits_fresh = false;        // _dev_in_cache came from the build and nothing has changed the cache since
   uint32_t _ticket = 0;                  // last value written behind a stream for WaitByTicket / StatusAndWords
   TensorPtr _dev_list_buffer;            // scratch list for bringing either side up to date
   bool _dev_lists_valid = false;
@@ -148,6 +149,16 @@ class CacheEntryManager {
   TensorPtr EmitBits(const uint64_t *a, const uint64_t *b, bool invert_a, uint64_t nbits, int which, size_t n,
                      TensorPtr &buffer, const std::function<MemHandle(size_t)> &allocator, Context ctx,
                      StreamHandle stream);
+  // A build that made its key list from a bitmap on the device hands the bitmap over: until a refresh changes the
+  // cache it is the bitmap of cached rows, and the slots taken are 0 .. cached - 1 (the build fills them in list
+  // order), so the first refresh finds both bitmaps without a pass over the key list and a lookup of every key.
+  void AdoptBuildBits(MemHandle bits) {
+    if (!_dev_in_cache) {
+      _dev_in_cache = bits;
+      _build_bits_fresh = bits != nullptr;
+    }
+  }
+  void DropBuildBits() { _build_bits_fresh = false; }
   // both differences of two bitmaps in one launch, counted as sets 0 (a & ~b) and 1 (b & ~a): the first n_ab and n_ba
   // elements into lists taken from the two buffers
   void EmitDiff(const uint64_t *a, const uint64_t *b, uint64_t nbits, size_t n_ab, size_t n_ba, TensorPtr &buffer_ab,
