@@ -103,7 +103,7 @@ typedef struct {
 const char *ugk_last_error(void);
 /* version of this ABI; bumped on any signature change.  ugk_abi_version() is what the loaded library was built with:
  * a caller compiled against another UGK_ABI_VERSION must not go on. */
-#define UGK_ABI_VERSION 20
+#define UGK_ABI_VERSION 21
 int ugk_abi_version(void);
 
 /* ---- runtime plumbing: Device::{AllocDataSpace,FreeDataSpace,CopyDataFromTo,StreamSync,CreateStream}
@@ -145,6 +145,11 @@ int ugk_stream_sync_ticket(void *stream, uint32_t *ticket_host, uint32_t value, 
  * copy call, where a copy into pageable memory and a wait for the stream take two calls into the runtime. */
 int ugk_words_to_host_ticket(const uint32_t *a_dev, unsigned n_a, const uint32_t *b_dev, unsigned n_b,
                              uint32_t *dst_host, uint32_t value, unsigned spin_us, void *stream);
+/* The first launch of a kernel of one of this library's source files loads that file's code object onto the current
+ * device, which takes 5 - 11 ms each the first time (a first gather of 51 MB: 12.4 ms, the second 0.9 ms).  This call
+ * launches an empty kernel of every file on a stream of its own and waits for them, so that no later call pays; a
+ * host library can make it from a helper thread while it is busy on the CPU. */
+int ugk_preload_kernels(void);
 int ugk_device_sync(void);
 int ugk_event_create(void **event);
 int ugk_event_destroy(void *event);

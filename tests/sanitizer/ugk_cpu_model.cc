@@ -844,6 +844,7 @@ int ugk_words_to_host_ticket(const uint32_t *a, unsigned n_a, const uint32_t *b,
   dst[0] = value;
   return 0;
 }
+int ugk_preload_kernels(void) { return 0; }
 int ugk_device_sync(void) {
   std::lock_guard<std::mutex> g(g_rt_mu);
   note_host_wait("the host waited for the device");

@@ -154,6 +154,15 @@ def test_wait_on_a_ticket_behind_the_launch(spin_us):
         word.free()
 
 
+def test_preload_launches_an_empty_kernel_of_every_source_file():
+    """ugk_preload_kernels: returns once its empty launches have run; any number of times, beside other work"""
+    d = to_dev(np.arange(1000, dtype=np.uint32))
+    for _ in range(3):
+        hip.call("ugk_preload_kernels")
+    sync()
+    assert np.array_equal(to_np(d, np.uint32)[:1000], np.arange(1000, dtype=np.uint32))
+
+
 @pytest.mark.parametrize("spin_us", [0, 1, 1_000_000])
 def test_words_brought_to_the_host_with_the_ticket(spin_us):
     """ugk_words_to_host_ticket: device words written by a launch in front of it arrive with the ticket, whichever way

@@ -208,9 +208,10 @@ void CacheContext::build_with_advise_new_hash(int location_id, std::shared_ptr<C
   // 4. fill: rows of the cached keys host -> HBM in list order, slot = position in the list.  The copy is bound by
   //    the host link, which answers a grid of 128 workgroups a little faster than one that fills the chip (12.8 GB of
   //    512-byte rows: 0.235 against 0.243 s; 6.4 GB of 128-byte rows: 0.131 against 0.137 s; 64 and 1,024 workgroups
-  //    are no better than the full grid).  (The table insert beside the copy, on a second stream, instead of behind it, was measured at
-  //    500M rows / 50M cached: the step went from 0.140 to 0.178 s, the link-bound copy kernel loses more than the
-  //    insert takes.)
+  //    are no better than the full grid).  (The table insert beside the copy, on a second stream, instead of behind
+  //    it, was measured at 500M rows / 50M cached: the step went from 0.140 to 0.178 s, the link-bound copy kernel
+  //    loses more than the insert takes.)
+  double rows_s = 0;
   if (num_cached_nodes > 0) {
     if (!list_on_device)
       cache_node_list = Tensor::CopyToExternal(keys_for_each_source[location_id], _eager_gpu_mem_allocator,
@@ -221,6 +222,10 @@ void CacheContext::build_with_advise_new_hash(int location_id, std::shared_ptr<C
                                    _device_cache_data[_local_location_id], _row_bytes,
                                    PointerKind(cpu_data) == 1 ? RunConfig::fill_limit_block : 0u,  // 2: a table in HBM
                                    st->ptr<uint32_t>(), nullptr, stream));
+    if (common::MinLogLevel() <= common::LogLevel::INFO) {  // the two parts of the step timed apart: one more wait
+      UGK_CALL(ugk_stream_sync(stream));
+      rows_s = t.Passed() - detect_s - alloc_s;
+    }
     // (8-byte entries are keyed by the row: no id list)
     TensorPtr id_buffer;
     auto table_keys = RunConfig::key_map_mul == 0 || _new_hash_table->_table.kind == 3 ? cache_node_list
@@ -259,7 +264,8 @@ void CacheContext::build_with_advise_new_hash(int location_id, std::shared_ptr<C
             << " / " << num_total_nodes << " nodes ( " << ToPercentage(num_cached_nodes / (double)num_total_nodes)
             << "~" << ToPercentage(cache_percentage) << ") | cpu " << num_cpu_nodes << " / " << num_total_nodes
             << " | " << ToReadableSize(_cache_nbytes) << " | " << t.Passed() << " secs (key list " << detect_s
-            << ", cache space + table " << alloc_s << ", rows + table insert " << fill_s << ")";
+            << ", cache space + table " << alloc_s << ", rows + table insert " << fill_s << ", of which rows "
+            << rows_s << ")";
   std::cout << "test_result:init:feat_nbytes=" << num_total_nodes * _row_bytes << "\n";
   std::cout << "test_result:init:cache_nbytes=" << _cache_nbytes << "\n";
 }

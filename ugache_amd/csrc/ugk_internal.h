@@ -53,4 +53,12 @@ bool nt_store_for(size_t out_bytes);
 
 __device__ __forceinline__ unsigned lane_id() { return __lane_id(); }
 
+// one per source file with kernels: launches an empty kernel of that file on `stream`
+void preload_gather(hipStream_t stream);
+void preload_hotness(hipStream_t stream);
+void preload_partition(hipStream_t stream);
+void preload_pool(hipStream_t stream);
+void preload_refresh(hipStream_t stream);
+void preload_table(hipStream_t stream);
+
 }  // namespace ugk

@@ -210,6 +210,7 @@ int ugk_stream_is_capturing(void *stream, int *capturing) {
 
 namespace {
 __global__ void ticket_kernel(volatile uint32_t *word, uint32_t value) { *word = value; }
+__global__ void preload_runtime_kernel() {}
 
 // one wavefront: n_a + n_b device words to dst[1 ...], then the ticket to dst[0]
 __global__ void words_ticket_kernel(const uint32_t *a, unsigned n_a, const uint32_t *b, unsigned n_b,
@@ -266,6 +267,24 @@ int ugk_words_to_host_ticket(const uint32_t *a_dev, unsigned n_a, const uint32_t
   }
   if (*word != value) UGK_HIP(hipStreamSynchronize(as_stream(stream)));
   std::atomic_thread_fence(std::memory_order_acquire);
+  return 0;
+}
+
+int ugk_preload_kernels(void) {
+  hipStream_t st;
+  UGK_HIP(hipStreamCreateWithFlags(&st, hipStreamNonBlocking));
+  hipLaunchKernelGGL(preload_runtime_kernel, dim3(1), dim3(1), 0, st);  // this file's own
+  ugk::preload_gather(st);
+  ugk::preload_hotness(st);
+  ugk::preload_partition(st);
+  ugk::preload_pool(st);
+  ugk::preload_refresh(st);
+  ugk::preload_table(st);
+  const hipError_t launched = hipGetLastError();
+  const hipError_t waited = hipStreamSynchronize(st);
+  (void)hipStreamDestroy(st);
+  UGK_HIP(launched);
+  UGK_HIP(waited);
   return 0;
 }
 

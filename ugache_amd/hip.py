@@ -71,6 +71,7 @@ SIGNATURES = {
     "ugk_stream_is_capturing": [_vp, _vp],
     "ugk_stream_sync_ticket": [_vp, _vp, _u32, C.c_uint],
     "ugk_words_to_host_ticket": [_vp, C.c_uint, _vp, C.c_uint, _vp, _u32, C.c_uint, _vp],
+    "ugk_preload_kernels": [],
     "ugk_device_sync": [],
     "ugk_event_create": [C.POINTER(_vp)],
     "ugk_event_destroy": [_vp],
