@@ -33,6 +33,8 @@ def _run(exe, table, refresh, steps):
         env["COLL_GPU_RECORD_SEED"] = "1"
         env["COLL_REFRESH_RATE_GBPS"] = "0.5"
         env["COLL_RECORD_INLINE_BYTES"] = "0"  # every recorded prefix goes through the recorder's thread
+    if table == "HASH16" and refresh == "host":  # build and refresh through the host's key -> block array and key lists
+        env["COLL_DEVICE_KEY_LIST"] = "0"
     env["ASAN_OPTIONS"] = "detect_leaks=1:abort_on_error=0"
     env["UBSAN_OPTIONS"] = "print_stacktrace=1:halt_on_error=1"
     env["TSAN_OPTIONS"] = "halt_on_error=0:second_deadlock_stack=1"
