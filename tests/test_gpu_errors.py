@@ -133,6 +133,30 @@ def test_a_process_that_never_calls_shutdown_still_exits_cleanly(gpu_record):
     assert p.returncode == 0, p.stderr[-2000:]
 
 
+@pytest.mark.parametrize("preload", ["1", "0"])
+def test_a_process_that_configures_and_ends_at_once_exits_cleanly(preload):
+    """coll_cache_config starts a helper thread that loads the kernels onto the device; a process that ends right
+    behind the call (no build, no shutdown), one that shuts down right behind it, and one that configures again
+    afterwards all end with status 0"""
+    for body in ("""
+        co.config(cfg(1000, 0.2))
+        print("configured", flush=True)
+    """, """
+        co.config(cfg(1000, 0.2))
+        co.coll_torch_shutdown()
+        co.config(cfg(2000, 0.5)); co.coll_cache_record_init(0)
+        co.coll_torch_record(0, torch.arange(0, 2000, 3, dtype=torch.int32))
+        emb = co.coll_torch_create_emb_shm(0, 2000, 32, torch.float32); emb.normal_()
+        co.coll_torch_init_t(0, 0, emb, 0.5)
+        keys = torch.arange(0, 2000, 7, dtype=torch.int64, device="cuda")
+        assert torch.equal(co.coll_torch_lookup_key_t_val_ret(0, keys, False).cpu(), emb[keys.cpu()])
+        print("configured", flush=True)
+    """):
+        p = run(body, env={"COLL_PRELOAD_KERNELS": preload})
+        assert "configured" in p.stdout, p.stderr[-2000:]
+        assert p.returncode == 0, p.stderr[-2000:]
+
+
 def test_pooled_lookup_with_offsets_beyond_the_ids_aborts_with_a_message():
     p = run("""
         n = 5000
