@@ -103,7 +103,7 @@ typedef struct {
 const char *ugk_last_error(void);
 /* version of this ABI; bumped on any signature change.  ugk_abi_version() is what the loaded library was built with:
  * a caller compiled against another UGK_ABI_VERSION must not go on. */
-#define UGK_ABI_VERSION 21
+#define UGK_ABI_VERSION 22
 int ugk_abi_version(void);
 
 /* ---- runtime plumbing: Device::{AllocDataSpace,FreeDataSpace,CopyDataFromTo,StreamSync,CreateStream}
@@ -522,6 +522,10 @@ int ugk_bitmap_count(const uint64_t *a_dev, const uint64_t *b_dev, int invert_a,
                      uint32_t *total_host, void *stream);
 int ugk_bitmap_emit(const uint64_t *a_dev, const uint64_t *b_dev, int invert_a, uint64_t nbits, const void *ws_dev,
                     uint32_t *out_dev, uint64_t max_out, void *stream);
+/* ugk_bitmap_count(a, b, 0, ..., ws_ab) and ugk_bitmap_count(b, a, 0, ..., ws_ba) in one pass over the two bitmaps:
+ * totals_host (two pinned words, may be NULL) receives [0] |a & ~b| and [1] |b & ~a| */
+int ugk_bitmap_count_diff(const uint64_t *a_dev, const uint64_t *b_dev, uint64_t nbits, void *ws_ab_dev,
+                          void *ws_ba_dev, uint32_t *totals_host, void *stream);
 /* both differences of two bitmaps in one pass: a & ~b to out_ab_dev and b & ~a to out_ba_dev, each exactly what
  * ugk_bitmap_emit(a, b, 0, ...) / ugk_bitmap_emit(b, a, 0, ...) writes, from the workspaces ugk_bitmap_count(a, b) and
  * ugk_bitmap_count(b, a) (or ugk_rank_place_observed) left.  A list with a maximum of 0 is not written. */

@@ -1406,6 +1406,12 @@ int ugk_bitmap_emit(const uint64_t *a, const uint64_t *b, int invert_a, uint64_t
   }
   return 0;
 }
+int ugk_bitmap_count_diff(const uint64_t *a, const uint64_t *b, uint64_t nbits, void *ws_ab, void *ws_ba,
+                          uint32_t *totals_host, void *stream) {
+  REQUIRE(a && b && ws_ab && ws_ba && ws_ab != ws_ba, "ugk_bitmap_count_diff: bad argument");
+  if (int rc = ugk_bitmap_count(a, b, 0, nbits, ws_ab, totals_host, stream)) return rc;
+  return ugk_bitmap_count(b, a, 0, nbits, ws_ba, totals_host ? totals_host + 1 : nullptr, stream);
+}
 int ugk_bitmap_emit_diff(const uint64_t *a, const uint64_t *b, uint64_t nbits, const void *ws_ab, const void *ws_ba,
                          uint32_t *out_ab, uint64_t max_ab, uint32_t *out_ba, uint64_t max_ba, void *stream) {
   REQUIRE(a && b && ws_ab && ws_ba, "ugk_bitmap_emit_diff: null pointer");

@@ -1618,10 +1618,7 @@ void RefreshSession::refresh_on_device(ExtractSession *session, size_t num_cache
       num_cached, table->InNewBits(), table->_dev_scratch_bits->ptr<uint64_t>(),
       RunConfig::gpu_refresh_stable ? table->InCacheBits() : nullptr, table->_dev_rank_ws->ptr(),
       !RunConfig::gpu_refresh_keep, &diff, stream);
-  if (!counted) {  // into the same two pinned words
-    table->CountBits(table->InCacheBits(), table->InNewBits(), false, num_rows, 0, stream);
-    table->CountBits(table->InNewBits(), table->InCacheBits(), false, num_rows, 1, stream);
-  }
+  if (!counted) table->CountDiff(table->InCacheBits(), table->InNewBits(), num_rows, stream);  // the same pinned words
   ApplyPlacedBits(session, num_cached, foreground, stage, true,
                   counted ? "placement (from the observed rows alone)" : "placement", sync_s, t_phase);
 }
@@ -1671,8 +1668,7 @@ void RefreshSession::refresh_from_ranked_rows(ExtractSession *session, TensorPtr
                                      table->_dev_bm_ws2->ptr(), table->DevWords() + 8,
                                      _status_handle->ptr<uint32_t>(), stream));
   } else {
-    table->CountBits(table->InCacheBits(), table->InNewBits(), false, num_rows, 0, stream);
-    table->CountBits(table->InNewBits(), table->InCacheBits(), false, num_rows, 1, stream);
+    table->CountDiff(table->InCacheBits(), table->InNewBits(), num_rows, stream);
   }
   ApplyPlacedBits(session, num_cached, foreground, stage, false, "placement ranked on the host", sync_s, t_phase);
 }

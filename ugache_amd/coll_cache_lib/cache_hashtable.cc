@@ -246,6 +246,10 @@ TensorPtr CacheEntryManager::EmitBits(const uint64_t *a, const uint64_t *b, bool
   return list;
 }
 
+void CacheEntryManager::CountDiff(const uint64_t *a, const uint64_t *b, uint64_t nbits, StreamHandle stream) {
+  UGK_CALL(ugk_bitmap_count_diff(a, b, nbits, _dev_bm_ws->ptr(), _dev_bm_ws2->ptr(), DevWords() + 8, stream));
+}
+
 void CacheEntryManager::EmitDiff(const uint64_t *a, const uint64_t *b, uint64_t nbits, size_t n_ab, size_t n_ba,
                                  TensorPtr &buffer_ab, TensorPtr &buffer_ba, TensorPtr *list_ab, TensorPtr *list_ba,
                                  const std::function<MemHandle(size_t)> &allocator, Context ctx, StreamHandle stream) {

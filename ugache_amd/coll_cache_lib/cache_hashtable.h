@@ -159,6 +159,9 @@ class CacheEntryManager {
     }
   }
   void DropBuildBits() { _build_bits_fresh = false; }
+  // the counts of both differences of two bitmaps (sets 0 = a & ~b and 1 = b & ~a) from one pass, into the pinned
+  // words CountBits would write
+  void CountDiff(const uint64_t *a, const uint64_t *b, uint64_t nbits, StreamHandle stream);
   // both differences of two bitmaps in one launch, counted as sets 0 (a & ~b) and 1 (b & ~a): the first n_ab and n_ba
   // elements into lists taken from the two buffers
   void EmitDiff(const uint64_t *a, const uint64_t *b, uint64_t nbits, size_t n_ab, size_t n_ba, TensorPtr &buffer_ab,

@@ -625,6 +625,50 @@ __global__ __launch_bounds__(kBlock) void bitmap_count_kernel(const unsigned lon
   }
 }
 
+// bitmap_count_kernel for a & ~b and b & ~a at once: the two bitmaps are read once, both workspaces are left as two
+// counts would leave them
+__global__ __launch_bounds__(kBlock) void bitmap_count_diff_kernel(const unsigned long long *a,
+                                                                   const unsigned long long *b, uint64_t nbits,
+                                                                   uint64_t per_chunk, BmWs *ws_ab, BmWs *ws_ba) {
+  const int lane = (int)lane_id();
+  const uint64_t n_words = (nbits + 63) / 64;
+  const uint64_t wave = ((uint64_t)blockIdx.x * kBlock + threadIdx.x) / kWave;
+  const uint64_t n_waves = (uint64_t)gridDim.x * (kBlock / kWave);
+  for (uint64_t chunk = wave; chunk < (uint64_t)kBmChunks; chunk += n_waves) {
+    const uint64_t begin = chunk * per_chunk, end = min(n_words, begin + per_chunk);
+    uint32_t sum_ab = 0, sum_ba = 0;
+    for (uint64_t w0 = begin; w0 < end; w0 += kWave) {
+      const uint64_t w = w0 + lane;
+      uint32_t n_ab = 0, n_ba = 0;
+      if (w < end) {
+        unsigned long long wa = a[w], wb = b[w];
+        if (nbits - w * 64 < 64) {  // the last, partial word
+          const unsigned long long valid = (1ull << (nbits - w * 64)) - 1ull;
+          wa &= valid;
+          wb &= valid;
+        }
+        n_ab = __popcll(wa & ~wb);
+        n_ba = __popcll(wb & ~wa);
+      }
+#pragma unroll
+      for (int d = kWave / 2; d > 0; d >>= 1) {
+        n_ab += __shfl_xor(n_ab, d);
+        n_ba += __shfl_xor(n_ba, d);
+      }
+      if (lane == 0) {
+        ws_ab->block[w0 / kWave] = n_ab;  // chunks begin on block boundaries
+        ws_ba->block[w0 / kWave] = n_ba;
+      }
+      sum_ab += n_ab;
+      sum_ba += n_ba;
+    }
+    if (lane == 0) {
+      ws_ab->base[chunk] = sum_ab;
+      ws_ba->base[chunk] = sum_ba;
+    }
+  }
+}
+
 __device__ __forceinline__ void scan_chunks(BmWs *ws, uint32_t *total_host) {
   constexpr int kPer = kBmChunks / kBlock;  // 32 chunks per thread
   __shared__ uint32_t part[kBlock];
@@ -660,11 +704,11 @@ __global__ __launch_bounds__(kBlock) void bitmap_scan_kernel(BmWs *ws, uint32_t 
 // taken the observed-rows path
 __global__ __launch_bounds__(kBlock) void bitmap_scan2_kernel(BmWs *a, BmWs *b, uint32_t *totals_host,
                                                               const RankWs *gate) {
-  if (!gate->from_bitmap) {
+  if (gate && !gate->from_bitmap) {
     if (threadIdx.x == 0) totals_host[blockIdx.x] = 0;
     return;
   }
-  scan_chunks(blockIdx.x == 0 ? a : b, totals_host + blockIdx.x);
+  scan_chunks(blockIdx.x == 0 ? a : b, totals_host ? totals_host + blockIdx.x : (uint32_t *)nullptr);
 }
 
 // The set bits of one 64-word block, a lane per word on entry (m), to out[pos0 ...] in ascending order; n_set: how
@@ -1018,6 +1062,24 @@ int ugk_bitmap_count(const uint64_t *a_dev, const uint64_t *b_dev, int invert_a,
                      per_chunk, static_cast<BmWs *>(ws_dev), (const RankWs *)nullptr);
   hipLaunchKernelGGL(bitmap_scan_kernel, dim3(1), dim3(kBlock), 0, as_stream(stream), static_cast<BmWs *>(ws_dev),
                      total_host, (const RankWs *)nullptr);
+  UGK_HIP(hipGetLastError());
+  return 0;
+}
+
+int ugk_bitmap_count_diff(const uint64_t *a_dev, const uint64_t *b_dev, uint64_t nbits, void *ws_ab_dev,
+                          void *ws_ba_dev, uint32_t *totals_host, void *stream) {
+  UGK_REQUIRE(a_dev && b_dev && ws_ab_dev && ws_ba_dev && ws_ab_dev != ws_ba_dev,
+              "ugk_bitmap_count_diff: null pointer, or one workspace for both counts");
+  UGK_REQUIRE(nbits > 0 && nbits <= 0xffffffffull, "ugk_bitmap_count_diff: %llu bits do not fit 32-bit positions",
+              (unsigned long long)nbits);
+  const uint64_t per_chunk = bm_words_per_chunk((nbits + 63) / 64);
+  const unsigned grid = clamp_grid((kBmChunks + (kBlock / kWave) - 1) / (kBlock / kWave), (unsigned)cu_count() * 8u);
+  hipLaunchKernelGGL(bitmap_count_diff_kernel, dim3(grid), dim3(kBlock), 0, as_stream(stream),
+                     reinterpret_cast<const unsigned long long *>(a_dev),
+                     reinterpret_cast<const unsigned long long *>(b_dev), nbits, per_chunk,
+                     static_cast<BmWs *>(ws_ab_dev), static_cast<BmWs *>(ws_ba_dev));
+  hipLaunchKernelGGL(bitmap_scan2_kernel, dim3(2), dim3(kBlock), 0, as_stream(stream), static_cast<BmWs *>(ws_ab_dev),
+                     static_cast<BmWs *>(ws_ba_dev), totals_host, (const RankWs *)nullptr);
   UGK_HIP(hipGetLastError());
   return 0;
 }

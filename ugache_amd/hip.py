@@ -144,6 +144,7 @@ SIGNATURES = {
     "ugk_bitmap_workspace_bytes": [],
     "ugk_bitmap_count": [_vp, _vp, C.c_int, _u64, _vp, _vp, _vp],
     "ugk_bitmap_emit": [_vp, _vp, C.c_int, _u64, _vp, _vp, _u64, _vp],
+    "ugk_bitmap_count_diff": [_vp, _vp, _u64, _vp, _vp, _vp, _vp],
     "ugk_bitmap_emit_diff": [_vp, _vp, _u64, _vp, _vp, _vp, _u64, _vp, _u64, _vp],
     "ugk_bitmap_update": [_vp, _u64, _vp, _sz, C.c_int, _vp, _vp],
     "ugk_bitmap_set_through": [_vp, _u64, _vp, _vp, _vp],
