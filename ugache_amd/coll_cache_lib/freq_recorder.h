@@ -101,6 +101,7 @@ class FreqRecorder {
   bool _live_dirty = false, _shared_dirty = false;  // the array holds a non-zero counter
   FreqEntryList _handed_over;                      // entries of the open hand-over, not in the arrays
   FreqEntryList _direct;                           // what LocalCombineToShared listed straight from the counters
+  size_t _last_listed = 0;                         // how many keys the last such listing found (sizes the next one's lists)
                                                     // (ascending, distinct keys), not in the shared array
   void ScatterHandedOver(FreqEntryList &list, CntT *into);
   // _mu guards what recording touches (_live, _live_dirty, _handed_over) and is held for one batch at most;
